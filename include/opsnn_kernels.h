@@ -1,0 +1,109 @@
+/*
+ * Thin C ABI over the gfx950 HIP kernels of the quantized-matmul path: plain
+ * pointers, sizes and type codes, no tensor objects.  The aclnn entry points
+ * (include/aclnnop/*.h) are built on exactly these calls; a host that already
+ * owns device buffers and a HIP stream can call them directly.
+ *
+ * These launchers have no single counterpart in the reference: together they
+ * stand where the reference has host tiling plus device kernels --
+ *   opsnnQmmInt8        <- quant_batch_matmul_v3 K-C/K-T/T-C kernel
+ *                          (matmul/quant_batch_matmul_v3/op_kernel/arch35/qbmm_mix_online_dynamic.h:387-388, 648-736)
+ *   opsnnQmmBlockScale  <- per-tile kernel (matmul/common/cmct/epilogue/block_epilogue_pertile.h:502-642)
+ *   opsnnQmmMx          <- MX kernel (matmul/common/cmct/block/block_mmad_mx.h)
+ *   opsnnWqmm           <- weight_quant_batch_matmul_v2 arch35 kernels
+ *                          (matmul/weight_quant_batch_matmul_v2/op_kernel/arch35/n_first/basic_block_vf_nd.h:139-148)
+ *   opsnnTranspose*     <- the reference's ND->NZ weight relayout (offline weight pre-pack)
+ *
+ * All functions return 0 on success, a negative value for an argument the
+ * kernels cannot take (nothing launched), or a positive hipError_t.
+ * Type codes are the aclDataType values.  `stream` is a hipStream_t.
+ * Every launcher is asynchronous on `stream`.
+ */
+#ifndef OPSNN_KERNELS_H_
+#define OPSNN_KERNELS_H_
+#include <stdint.h>
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define OPSNN_API __attribute__((visibility("default")))
+
+/* A matrix operand: element (r, c) of batch b lives at element index
+ * b*batch_stride + r*row_stride + c*col_stride (strides in elements, also for 4-bit types). */
+typedef struct {
+    const void* ptr;
+    int64_t row_stride;
+    int64_t col_stride;
+    int64_t batch_stride;
+} OpsnnMat;
+
+typedef struct {
+    int64_t M, N, K, batch;
+    OpsnnMat x1;          /* logical [M, K] */
+    OpsnnMat x2;          /* logical [K, N] */
+    int x1_dtype, x2_dtype;
+    void* out;            /* [batch, M, N] dense */
+    int out_dtype;        /* BF16 / FLOAT16 / FLOAT / INT32 */
+    const void* x1_scale; /* see each launcher */
+    const void* x2_scale;
+    int x2_scale_dtype;   /* FLOAT or BF16 */
+    int64_t x2_scale_len; /* 1 or N */
+    const void* bias;     /* [N] or NULL */
+    int bias_dtype;       /* INT32 / BF16 / FLOAT16 / FLOAT */
+    int64_t bias_batch_stride;
+    /* block-scale and MX modes */
+    int64_t gsM, gsN, gsK;
+    /* block mode: x1_scale_mat is logical [ceil(M/gsM), ceil(K/gsK)], x2_scale_mat logical [ceil(K/gsK), ceil(N/gsN)].
+     * MX mode: the e8m0 byte for row r (m or n) and 32-wide K block kb is
+     *          ptr[r*row_stride + (kb/2)*col_stride + kb%2]  (the reference stores K scales in pairs). */
+    OpsnnMat x1_scale_mat;
+    OpsnnMat x2_scale_mat;
+    void* workspace;       /* opsnnQmmWorkspace() bytes, or NULL if that is 0 */
+    int force_variant;     /* 0 = selector decides; >0 pins a kernel variant (tuning and tests) */
+} OpsnnQmmArgs;
+
+/* int8 x int8 -> int32, then  out = fp32(acc + int32 bias) * x2_scale[n] * x1_scale[m] + float bias.
+ * x1_scale: fp32 [M] or NULL. */
+OPSNN_API int opsnnQmmInt8(const OpsnnQmmArgs* a, void* stream);
+/* fp8 x fp8 with fp32 block scales: out = sum_kb (x1_kb @ x2_kb) * (s1[m/gsM,kb] * s2[kb,n/gsN]). */
+OPSNN_API int opsnnQmmBlockScale(const OpsnnQmmArgs* a, void* stream);
+/* MX: fp4/fp8 operands, e8m0 scale per 32 K. out = (x1*s1) @ (x2*s2) + fp32 bias. */
+OPSNN_API int opsnnQmmMx(const OpsnnQmmArgs* a, void* stream);
+/* Device workspace bytes a launcher needs for these arguments (0 if none). */
+OPSNN_API uint64_t opsnnQmmWorkspace(const OpsnnQmmArgs* a, int mode);
+
+typedef struct {
+    int64_t M, N, K;
+    const void* x;        /* [M, K] dense, FLOAT16 or BF16 */
+    int x_dtype;
+    OpsnnMat w;           /* logical [K, N]; INT8 / INT4 / FLOAT8_E4M3FN / FLOAT4_E2M1 */
+    int w_dtype;
+    OpsnnMat scale;       /* logical [G, N] with G = 1 or ceil(K/group); x's dtype, or FLOAT8_E8M0 */
+    int scale_dtype;
+    int64_t scale_n;      /* N, or 1 for per-tensor */
+    const void* offset;   /* same layout as scale, or NULL */
+    int64_t group;        /* 0 = per-channel / per-tensor */
+    const void* bias;     /* [N] or NULL */
+    int bias_dtype;
+    void* y;              /* [M, N] dense, x's dtype */
+    void* workspace;      /* opsnnWqmmWorkspace() bytes, or NULL if that is 0 */
+    int force_variant;
+} OpsnnWqmmArgs;
+
+/* y = x @ T(T(w + offset) * scale) + bias, T = rounding through x's dtype. */
+OPSNN_API int opsnnWqmm(const OpsnnWqmmArgs* a, void* stream);
+OPSNN_API uint64_t opsnnWqmmWorkspace(const OpsnnWqmmArgs* a);
+
+/* dst[c, r] = src[r, c] for a dense [rows, cols] matrix of 8-bit elements (batched). */
+OPSNN_API int opsnnTranspose8(const void* src, void* dst, int64_t rows, int64_t cols, int64_t batch, void* stream);
+/* Same for 4-bit elements packed two per byte along the last axis (low nibble = even index);
+ * rows and cols must be even. */
+OPSNN_API int opsnnTranspose4(const void* src, void* dst, int64_t rows, int64_t cols, int64_t batch, void* stream);
+
+/* Device properties the selector uses. */
+OPSNN_API int opsnnDeviceInfo(int* cu_count, int* clock_khz, int64_t* hbm_bytes, char* arch, int arch_len);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

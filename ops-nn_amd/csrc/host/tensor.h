@@ -1,0 +1,87 @@
+// Internal definitions behind the opaque aclTensor / aclOpExecutor handles.
+#pragma once
+#include <cstdarg>
+#include <cstdint>
+#include <string>
+#include <vector>
+
+#include "acl/acl.h"
+#include "opsnn_kernels.h"
+
+struct aclTensor {
+    std::vector<int64_t> view;     // view shape, in elements
+    std::vector<int64_t> strides;  // in elements
+    int64_t offset = 0;            // in elements
+    aclDataType dtype = ACL_DT_UNDEFINED;
+    aclFormat format = ACL_FORMAT_ND;
+    std::vector<int64_t> storage;  // storage shape
+    void* data = nullptr;
+};
+
+namespace opsnn {
+
+constexpr uint32_t kExecutorMagic = 0x51454D4Du;
+
+enum class OpKind { None, QmmInt8, QmmBlockScale, QmmMx, Wqmm };
+
+// What phase 1 decided; phase 2 only fills in workspace/stream and launches.
+struct aclOpExecutorImpl {
+    uint32_t magic = kExecutorMagic;
+    OpKind kind = OpKind::None;     // None: nothing to launch (empty output)
+    OpsnnQmmArgs qmm{};
+    OpsnnWqmmArgs wqmm{};
+    uint64_t workspace_size = 0;
+    const char* api = "";
+};
+
+// Thread-local last-error text (aclGetRecentErrMsg).
+void set_error(const char* fmt, ...) __attribute__((format(printf, 1, 2)));
+void clear_error();
+bool log_enabled();
+
+inline bool is_4bit(aclDataType d) { return d == ACL_INT4 || d == ACL_FLOAT4_E2M1 || d == ACL_FLOAT4_E1M2; }
+inline int dtype_bits(aclDataType d)
+{
+    switch (d) {
+        case ACL_FLOAT: case ACL_INT32: case ACL_UINT32: return 32;
+        case ACL_FLOAT16: case ACL_BF16: case ACL_INT16: case ACL_UINT16: return 16;
+        case ACL_INT8: case ACL_UINT8: case ACL_BOOL: case ACL_HIFLOAT8: case ACL_FLOAT8_E5M2:
+        case ACL_FLOAT8_E4M3FN: case ACL_FLOAT8_E8M0: return 8;
+        case ACL_INT64: case ACL_UINT64: case ACL_DOUBLE: case ACL_COMPLEX64: return 64;
+        case ACL_INT4: case ACL_FLOAT4_E2M1: case ACL_FLOAT4_E1M2: return 4;
+        default: return 0;
+    }
+}
+const char* dtype_name(aclDataType d);
+std::string shape_str(const std::vector<int64_t>& s);
+
+// A lightweight copy of a tensor's view that the checks may rewrite (swap dims, re-tag dtype).
+struct TView {
+    std::vector<int64_t> shape, strides;
+    int64_t offset = 0;
+    aclDataType dtype = ACL_DT_UNDEFINED;
+    aclFormat format = ACL_FORMAT_ND;
+    std::vector<int64_t> storage;
+    void* data = nullptr;
+    bool present = false;
+    int64_t rank() const { return (int64_t)shape.size(); }
+    int64_t dim(int64_t i) const { return shape[(size_t)(i < 0 ? i + rank() : i)]; }
+    int64_t stride(int64_t i) const { return strides[(size_t)(i < 0 ? i + rank() : i)]; }
+    int64_t numel() const { int64_t n = 1; for (auto d : shape) n *= d; return n; }
+    bool empty() const { return numel() == 0; }
+    // address of element offset `off` (in elements) from the storage base
+    const void* ptr_at(int64_t off) const
+    {
+        if (!data) return nullptr;
+        return (const char*)data + ((offset + off) * dtype_bits(dtype)) / 8;
+    }
+};
+TView make_view(const aclTensor* t);
+bool is_contiguous(const TView& v);
+// Last two dims transposed: stride[-2]==1, stride[-1]==shape[-2], dense batch strides, not both extents 1.
+bool is_transposed_last2(const TView& v);
+void swap_last2(TView& v);
+
+}  // namespace opsnn
+
+struct aclOpExecutor : opsnn::aclOpExecutorImpl {};

@@ -1,0 +1,138 @@
+// Shared device helpers for the gfx950 quantized-matmul kernels.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace opsnn {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v8i __attribute__((ext_vector_type(8)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+typedef _Float16 v8h __attribute__((ext_vector_type(8)));
+typedef _Float16 v2h __attribute__((ext_vector_type(2)));
+typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
+typedef unsigned short v4us __attribute__((ext_vector_type(4)));
+
+// Element type codes: the aclDataType values.
+enum : int {
+    DT_F32 = 0, DT_F16 = 1, DT_I8 = 2, DT_I32 = 3, DT_BF16 = 27, DT_I4 = 29,
+    DT_E5M2 = 35, DT_E4M3 = 36, DT_E8M0 = 37, DT_E2M1 = 40
+};
+
+__device__ __forceinline__ uint32_t f2u(float f) { return __builtin_bit_cast(uint32_t, f); }
+__device__ __forceinline__ float u2f(uint32_t u) { return __builtin_bit_cast(float, u); }
+
+// fp32 -> bf16 bits, round to nearest even, NaN kept quiet.
+__device__ __forceinline__ uint16_t bf16_bits(float f)
+{
+    uint32_t u = f2u(f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x0040u);
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return (uint16_t)(u >> 16);
+}
+__device__ __forceinline__ float bf16_to_f32(uint16_t h) { return u2f((uint32_t)h << 16); }
+__device__ __forceinline__ uint16_t f16_bits(float f)
+{
+    _Float16 h = (_Float16)f;  // v_cvt_f16_f32: round to nearest even
+    return __builtin_bit_cast(uint16_t, h);
+}
+__device__ __forceinline__ float f16_to_f32(uint16_t b) { return (float)__builtin_bit_cast(_Float16, b); }
+
+// Round an fp32 value to the 16-bit output type and return its bits.
+template <int DT>
+__device__ __forceinline__ uint16_t to_b16(float f)
+{
+    if constexpr (DT == DT_BF16) return bf16_bits(f);
+    else return f16_bits(f);
+}
+
+__device__ __forceinline__ float load_scalar_as_f32(const void* p, int dt, int64_t i)
+{
+    switch (dt) {
+        case DT_F32: return ((const float*)p)[i];
+        case DT_BF16: return bf16_to_f32(((const uint16_t*)p)[i]);
+        case DT_F16: return f16_to_f32(((const uint16_t*)p)[i]);
+        case DT_I32: return (float)((const int32_t*)p)[i];
+        default: return 0.0f;
+    }
+}
+
+__device__ __forceinline__ float e4m3_to_f32(uint32_t b)
+{
+    uint32_t e = (b >> 3) & 0xfu, m = b & 7u;
+    float v;
+    if (e == 15u && m == 7u) v = u2f(0x7fc00000u);
+    else if (e == 0u) v = (float)m * 0.001953125f;
+    else v = u2f(((e + 120u) << 23) | (m << 20));
+    return (b & 0x80u) ? -v : v;
+}
+__device__ __forceinline__ float e5m2_to_f32(uint32_t b)
+{
+    // e5m2 is the upper byte of an IEEE binary16
+    return f16_to_f32((uint16_t)(b << 8));
+}
+__device__ __forceinline__ float e2m1_to_f32(uint32_t c)
+{
+    uint32_t e = (c >> 1) & 3u, m = c & 1u;
+    float v = (e == 0u) ? 0.5f * (float)m : u2f(((e + 126u) << 23) | (m << 22));
+    return (c & 8u) ? -v : v;
+}
+__device__ __forceinline__ float e8m0_to_f32(uint32_t b)
+{
+    if (b == 0xffu) return u2f(0x7fc00000u);
+    if (b == 0u) return u2f(0x00400000u);
+    return u2f(b << 23);
+}
+
+// Decode element i of a dense buffer of 8-bit or 4-bit quantised values.
+__device__ __forceinline__ float load_q_as_f32(const void* p, int dt, int64_t i)
+{
+    switch (dt) {
+        case DT_I8: return (float)((const int8_t*)p)[i];
+        case DT_E4M3: return e4m3_to_f32(((const uint8_t*)p)[i]);
+        case DT_E5M2: return e5m2_to_f32(((const uint8_t*)p)[i]);
+        case DT_I4: {
+            uint32_t b = ((const uint8_t*)p)[i >> 1];
+            int v = (int)((i & 1) ? (b >> 4) : (b & 15u));
+            return (float)(v >= 8 ? v - 16 : v);
+        }
+        case DT_E2M1: {
+            uint32_t b = ((const uint8_t*)p)[i >> 1];
+            return e2m1_to_f32((i & 1) ? (b >> 4) : (b & 15u));
+        }
+        default: return 0.0f;
+    }
+}
+
+__device__ __forceinline__ void store_f32_as(void* p, int dt, int64_t i, float v)
+{
+    switch (dt) {
+        case DT_F32: ((float*)p)[i] = v; break;
+        case DT_BF16: ((uint16_t*)p)[i] = bf16_bits(v); break;
+        case DT_F16: ((uint16_t*)p)[i] = f16_bits(v); break;
+        default: break;
+    }
+}
+
+// 16-byte asynchronous copy global -> LDS.  `lds` must be wave-uniform; lane l lands at lds + 16*l.
+__device__ __forceinline__ void async_copy16(const void* g, void* lds)
+{
+    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)g,
+                                     (__attribute__((address_space(3))) void*)lds, 16, 0, 0);
+}
+
+// Workgroup ids are dealt round-robin over the 8 XCDs; give each XCD (own L2) a contiguous
+// range of logical tile ids so that neighbouring tiles share operand panels in one L2.
+__device__ __forceinline__ uint32_t xcd_remap(uint32_t wg, uint32_t total)
+{
+    const uint32_t X = 8;
+    uint32_t per = total / X, rem = total % X;
+    uint32_t xcd = wg % X, idx = wg / X;
+    // the first `rem` XCDs own per+1 tiles
+    uint32_t base = xcd * per + (xcd < rem ? xcd : rem);
+    return base + idx;
+}
+
+}  // namespace opsnn

@@ -1,0 +1,79 @@
+// Launcher entry points for the block-scale, MX and weight-only paths, and workspace sizing.
+// Each launcher first offers the call to the MFMA kernel family for that mode; whatever that family
+// does not take (odd shapes, strided layouts, rarely used dtype pairs) runs on the plain kernels.
+#include "common.hip.h"
+#include "launch.h"
+
+namespace opsnn {
+int launch_blockscale_plain(const OpsnnQmmArgs& a, hipStream_t st);
+int launch_mx_plain(const OpsnnQmmArgs& a, hipStream_t st);
+int launch_wqmm_plain(const OpsnnWqmmArgs& a, hipStream_t st);
+// Return OPSNN_NOT_TAKEN when the arguments are outside what the fast kernels handle.
+int launch_blockscale_mfma(const OpsnnQmmArgs& a, hipStream_t st);
+int launch_mx_mfma(const OpsnnQmmArgs& a, hipStream_t st);
+int launch_wqmm_mfma(const OpsnnWqmmArgs& a, hipStream_t st);
+}  // namespace opsnn
+
+using namespace opsnn;
+
+static bool qmm_args_ok(const OpsnnQmmArgs* a)
+{
+    return a && a->x1.ptr && a->x2.ptr && a->out && a->M > 0 && a->N > 0 && a->K > 0 && a->batch > 0 && a->batch <= 65535;
+}
+
+extern "C" int opsnnQmmBlockScale(const OpsnnQmmArgs* a, void* stream)
+{
+    if (!qmm_args_ok(a) || !a->x1_scale_mat.ptr || !a->x2_scale_mat.ptr) return -1;
+    if (a->force_variant != OPSNN_VARIANT_PLAIN) {
+        int rc = launch_blockscale_mfma(*a, (hipStream_t)stream);
+        if (rc != OPSNN_NOT_TAKEN) return rc;
+        if (a->force_variant != 0) return -4;
+    }
+    return launch_blockscale_plain(*a, (hipStream_t)stream);
+}
+
+extern "C" int opsnnQmmMx(const OpsnnQmmArgs* a, void* stream)
+{
+    if (!qmm_args_ok(a) || !a->x1_scale_mat.ptr || !a->x2_scale_mat.ptr) return -1;
+    if (a->force_variant != OPSNN_VARIANT_PLAIN) {
+        int rc = launch_mx_mfma(*a, (hipStream_t)stream);
+        if (rc != OPSNN_NOT_TAKEN) return rc;
+        if (a->force_variant != 0) return -4;
+    }
+    return launch_mx_plain(*a, (hipStream_t)stream);
+}
+
+extern "C" int opsnnWqmm(const OpsnnWqmmArgs* a, void* stream)
+{
+    if (!a || !a->x || !a->w.ptr || !a->scale.ptr || !a->y || a->M <= 0 || a->N <= 0 || a->K <= 0) return -1;
+    if (a->force_variant != OPSNN_VARIANT_PLAIN) {
+        int rc = launch_wqmm_mfma(*a, (hipStream_t)stream);
+        if (rc != OPSNN_NOT_TAKEN) return rc;
+        if (a->force_variant != 0) return -4;
+    }
+    return launch_wqmm_plain(*a, (hipStream_t)stream);
+}
+
+// mode: 0 = int8 per-token/per-channel, 1 = block scale, 2 = MX.
+// The MFMA kernels stream a K-contiguous right operand ("x2 stored [N, K]").  An N-contiguous x2 is
+// first re-laid out into the workspace; callers who keep x2 in [N, K] form (transposeX2 = true or a
+// transposed view) need no workspace and skip that pass.
+extern "C" uint64_t opsnnQmmWorkspace(const OpsnnQmmArgs* a, int mode)
+{
+    (void)mode;
+    if (!a) return 0;
+    if (a->x2.row_stride == 1 || a->K == 1) return 0;           // already K-contiguous
+    if (a->x2.col_stride != 1 || a->x2.row_stride != a->N) return 0;  // not a dense [K, N]: plain kernel
+    uint64_t bits = (a->x2_dtype == DT_I4 || a->x2_dtype == DT_E2M1) ? 4 : 8;
+    uint64_t nb = a->x2.batch_stride == 0 ? 1 : (uint64_t)a->batch;
+    return ((uint64_t)a->N * (uint64_t)a->K * bits / 8) * nb;
+}
+
+extern "C" uint64_t opsnnWqmmWorkspace(const OpsnnWqmmArgs* a)
+{
+    if (!a) return 0;
+    if (a->w.row_stride == 1 || a->K == 1) return 0;
+    if (a->w.col_stride != 1 || a->w.row_stride != a->N) return 0;
+    uint64_t bits = (a->w_dtype == DT_I4 || a->w_dtype == DT_E2M1) ? 4 : 8;
+    return (uint64_t)a->N * (uint64_t)a->K * bits / 8;
+}

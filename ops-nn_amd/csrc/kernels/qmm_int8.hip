@@ -1,0 +1,333 @@
+// int8 x int8 -> int32 quantized matmul with the fused per-token / per-channel dequant epilogue
+// (K-C, K-T and dynamic T-C modes).  gfx950 only.
+//
+//   acc[m,n] = sum_k int32(x1[m,k]) * int32(x2[k,n])                 exact
+//   out[m,n] = cast( fp32(acc + int32 bias[n]) * x2Scale[n] * x1Scale[m] + float bias[n] )
+//
+// The multiplication order and the place of the bias follow the reference's golden
+// (matmul/quant_batch_matmul_v3/tests/assets/qbmmv3_kernel_golden.py:361-387) and its device epilogue
+// (matmul/quant_batch_matmul_v3/op_kernel/arch35/qbmm_mix_online_dynamic.h:648-736).
+//
+// Fast path: both operands K-contiguous ("x2 stored [N, K]"), 16-byte aligned rows.
+//   - 256x256 (or 128x128) output tile per workgroup, 4 waves, each wave owns a square quarter and
+//     drives v_mfma_i32_32x32x32_i8 with accumulators kept in registers for the whole K loop;
+//   - K tiles are copied global -> LDS asynchronously (16 B per lane, no register round trip),
+//     double buffered, one workgroup barrier per K tile;
+//   - LDS rows are XOR-swizzled in 16-byte chunks so the MFMA operand reads are bank-conflict free;
+//   - the MFMA is issued as x2-fragment x x1-fragment so every lane ends up with four consecutive n
+//     of one output row: scales and bias load as vectors and the 16-bit results leave as 8-byte stores.
+// Anything else (odd K, unaligned or strided operands) runs the plain strided kernel below.
+#include <type_traits>
+#include "common.hip.h"
+#include "launch.h"
+
+namespace opsnn {
+
+struct QmmI8Params {
+    const int8_t* a;  // x1
+    const int8_t* b;  // x2
+    int64_t a_rs, a_cs, a_bs;  // strides of logical [M,K]
+    int64_t b_rs, b_cs, b_bs;  // strides of logical [K,N]
+    void* out;
+    int64_t M, N, K;
+    const float* x1s;
+    const void* x2s;
+    int x2s_dt;
+    int64_t x2s_len;
+    const void* bias;
+    int bias_dt;
+    int64_t bias_bs;
+    int out_dt;
+};
+
+// ---------------------------------------------------------------------------------------------
+// Plain strided kernel: one thread per output element.  Any strides, any K.
+// ---------------------------------------------------------------------------------------------
+__global__ void qmm_i8_plain(QmmI8Params p)
+{
+    const int64_t nchunks = (p.N + blockDim.x - 1) / blockDim.x;
+    int64_t m = blockIdx.x / nchunks;
+    int64_t n = (blockIdx.x % nchunks) * (int64_t)blockDim.x + threadIdx.x;
+    int64_t bz = blockIdx.y;
+    if (n >= p.N) return;
+    const int8_t* a = p.a + bz * p.a_bs + m * p.a_rs;
+    const int8_t* b = p.b + bz * p.b_bs + n * p.b_cs;
+    int32_t acc = 0;
+    for (int64_t k = 0; k < p.K; k++) acc += (int32_t)a[k * p.a_cs] * (int32_t)b[k * p.b_rs];
+    int64_t o = (bz * p.M + m) * p.N + n;
+    if (p.out_dt == DT_I32) {
+        if (p.bias && p.bias_dt == DT_I32) acc += ((const int32_t*)p.bias)[bz * p.bias_bs + n];
+        ((int32_t*)p.out)[o] = acc;
+        return;
+    }
+    if (p.bias && p.bias_dt == DT_I32) acc += ((const int32_t*)p.bias)[bz * p.bias_bs + n];
+    float v = (float)acc;
+    v = v * load_scalar_as_f32(p.x2s, p.x2s_dt, p.x2s_len == 1 ? 0 : n);
+    if (p.x1s) v = v * p.x1s[m];
+    if (p.bias && p.bias_dt != DT_I32) v = v + load_scalar_as_f32(p.bias, p.bias_dt, bz * p.bias_bs + n);
+    store_f32_as(p.out, p.out_dt, o, v);
+}
+
+// ---------------------------------------------------------------------------------------------
+// MFMA kernel.
+// ---------------------------------------------------------------------------------------------
+__device__ __attribute__((aligned(16))) static const int8_t g_zero16[16] = {0};
+
+template <int BM, int BN, int BK, int OUT_DT>
+__global__ __launch_bounds__(256, 1) void qmm_i8_mfma(QmmI8Params p, int tiles_m, int tiles_n)
+{
+    constexpr int NT = 256;
+    constexpr int CPR = BK / 16;            // 16-byte chunks per LDS row
+    constexpr int TM = BM / 2, TN = BN / 2; // per-wave tile (2 x 2 waves)
+    constexpr int FM = TM / 32, FN = TN / 32;
+    constexpr int KS = BK / 32;             // MFMA K steps per tile
+    constexpr int A_BYTES = BM * BK, B_BYTES = BN * BK;
+    constexpr int STAGE = A_BYTES + B_BYTES;
+    constexpr int RPI = NT / CPR;           // tile rows covered by one copy instruction of the workgroup
+    constexpr int NA = BM / RPI, NB = BN / RPI;
+    static_assert(CPR == 8 || CPR == 4, "BK must be 64 or 128");
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+
+    // tile id: XCD-contiguous, m fastest so that one XCD works on few x2 panels at a time
+    const uint32_t t = xcd_remap(blockIdx.x, (uint32_t)(tiles_m * tiles_n));
+    const int tm = (int)(t % (uint32_t)tiles_m), tn = (int)(t / (uint32_t)tiles_m);
+    const int64_t m0 = (int64_t)tm * BM, n0 = (int64_t)tn * BN;
+    const int64_t bz = blockIdx.y;
+
+    const int64_t lda = p.a_rs, ldb = p.b_cs;
+    const int8_t* A = p.a + bz * p.a_bs + m0 * lda;
+    const int8_t* B = p.b + bz * p.b_bs + n0 * ldb;
+    const int64_t K = p.K;
+    const int KT = (int)((K + BK - 1) / BK);
+
+    // Async copies: copy instruction i of the workgroup fills LDS chunks [i*NT, (i+1)*NT), i.e. tile rows
+    // i*RPI .. i*RPI+RPI-1; this thread always handles row i*RPI + tid/CPR and the (swizzled) chunk below.
+    // Rows past the matrix edge are clamped to the last valid row: they only feed outputs that are never
+    // stored.  K chunks past the end must read as zero and are redirected to a zero page.
+    const int crow = tid / CPR;
+    const int cchunk = (tid % CPR) ^ (crow & (CPR - 1));
+    const int a_rows = (int)((p.M - m0) < BM ? (p.M - m0) : BM);   // valid rows of this tile
+    const int b_rows = (int)((p.N - n0) < BN ? (p.N - n0) : BN);
+    uint32_t a_off[NA], b_off[NB];
+#pragma unroll
+    for (int i = 0; i < NA; i++) {
+        int r = i * RPI + crow;
+        r = r < a_rows ? r : a_rows - 1;
+        a_off[i] = (uint32_t)(r * lda + cchunk * 16);
+    }
+#pragma unroll
+    for (int i = 0; i < NB; i++) {
+        int r = i * RPI + crow;
+        r = r < b_rows ? r : b_rows - 1;
+        b_off[i] = (uint32_t)(r * ldb + cchunk * 16);
+    }
+    const int8_t* const zero_page = g_zero16;
+
+    auto issue_tile = [&](int kt, int stage) {
+        char* sA = smem + stage * STAGE + wave * 1024;
+        char* sB = sA + A_BYTES;
+        const int64_t k0 = (int64_t)kt * BK;
+        const bool kok = (k0 + cchunk * 16) < K;
+        const int8_t* Ak = A + k0;
+        const int8_t* Bk = B + k0;
+#pragma unroll
+        for (int i = 0; i < NA; i++) {
+            const int8_t* g = Ak + a_off[i];
+            g = kok ? g : zero_page;
+            async_copy16(g, sA + i * NT * 16);
+        }
+#pragma unroll
+        for (int i = 0; i < NB; i++) {
+            const int8_t* g = Bk + b_off[i];
+            g = kok ? g : zero_page;
+            async_copy16(g, sB + i * NT * 16);
+        }
+    };
+
+    v16i acc[FN][FM];
+#pragma unroll
+    for (int i = 0; i < FN; i++)
+#pragma unroll
+        for (int j = 0; j < FM; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[i][j][r] = 0;
+
+    const int frow = lane & 31;   // row inside a 32-row fragment
+    const int fkc = lane >> 5;    // which 16-byte half of the 32-byte K step
+    const int swz = fkc ^ (frow & (CPR - 1));
+    const int a_rowbase = (wm * TM + frow) * BK;
+    const int b_rowbase = A_BYTES + (wn * TN + frow) * BK;
+
+    v4i fa[2][FM], fb[2][FN];
+    auto load_frags = [&](int stage, int s, int buf) {
+        const char* base = smem + stage * STAGE + (((2 * s) ^ swz) << 4);
+#pragma unroll
+        for (int j = 0; j < FM; j++) fa[buf][j] = *(const v4i*)(base + a_rowbase + j * 32 * BK);
+#pragma unroll
+        for (int i = 0; i < FN; i++) fb[buf][i] = *(const v4i*)(base + b_rowbase + i * 32 * BK);
+    };
+    auto mma = [&](int buf) {
+#pragma unroll
+        for (int i = 0; i < FN; i++)
+#pragma unroll
+            for (int j = 0; j < FM; j++)
+                acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fb[buf][i], fa[buf][j], acc[i][j], 0, 0, 0);
+    };
+
+    // Pipeline: the copy of tile kt+2 and the first operand reads of tile kt+1 are issued right after the
+    // single barrier of iteration kt, ahead of the last MFMA group of tile kt.
+    issue_tile(0, 0);
+    __syncthreads();
+    if (KT > 1) issue_tile(1, 1);
+    load_frags(0, 0, 0);
+
+    // One K tile.  ISSUE / PREFETCH are compile-time so the steady-state loop body has no branches.
+    auto k_tile = [&](int kt, auto issue, auto prefetch) {
+        const int st = kt & 1;
+#pragma unroll
+        for (int s = 0; s < KS - 1; s++) {
+            load_frags(st, s + 1, (s + 1) & 1);
+            mma(s & 1);
+        }
+        __syncthreads();  // tile kt+1 has landed; every wave holds its last operands of tile kt in registers
+        if constexpr (decltype(issue)::value) issue_tile(kt + 2, st);
+        if constexpr (decltype(prefetch)::value) load_frags(st ^ 1, 0, KS & 1);
+        mma((KS - 1) & 1);
+    };
+    using T = std::true_type;
+    using F = std::false_type;
+    int kt = 0;
+    for (; kt + 2 < KT; kt++) k_tile(kt, T{}, T{});
+    if (kt + 1 < KT) { k_tile(kt, F{}, T{}); kt++; }
+    k_tile(kt, F{}, F{});
+
+    // Epilogue.  acc[i][j][r]: n = n_base + 8*(r/4) + 4*(lane/32) + r%4,  m = m_base + lane%32.
+    // Scales and bias are first widened to fp32 in LDS (free after the last barrier), so the unrolled
+    // part below is branch-free: absent terms are the neutral elements 1.0f, 0 and -0.0f.
+    float* sS2 = (float*)smem;
+    float* sFb = sS2 + BN;
+    int32_t* sIb = (int32_t*)(sFb + BN);
+    float* sS1 = (float*)(sIb + BN);
+    {
+        const bool has_ib = p.bias && p.bias_dt == DT_I32;
+        const bool has_fb = p.bias && p.bias_dt != DT_I32;
+        for (int i = tid; i < BN; i += NT) {
+            int64_t n = n0 + i;
+            if (n >= p.N) n = p.N - 1;
+            sS2[i] = load_scalar_as_f32(p.x2s, p.x2s_dt, p.x2s_len == 1 ? 0 : n);
+            sFb[i] = has_fb ? load_scalar_as_f32(p.bias, p.bias_dt, bz * p.bias_bs + n) : -0.0f;
+            sIb[i] = has_ib ? ((const int32_t*)p.bias)[bz * p.bias_bs + n] : 0;
+        }
+        for (int i = tid; i < BM; i += NT) {
+            int64_t m = m0 + i;
+            if (m >= p.M) m = p.M - 1;
+            sS1[i] = p.x1s ? p.x1s[m] : 1.0f;
+        }
+    }
+    __syncthreads();
+    uint16_t* out = (uint16_t*)p.out + bz * p.M * p.N;
+    const bool vec_ok = (p.N % 4) == 0;
+#pragma unroll
+    for (int j = 0; j < FM; j++) {
+        const int ml = wm * TM + j * 32 + frow;
+        const int64_t m = m0 + ml;
+        const float s1 = sS1[ml];
+#pragma unroll
+        for (int i = 0; i < FN; i++) {
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+                const int nl = wn * TN + i * 32 + 8 * q + 4 * fkc;
+                const int64_t n = n0 + nl;
+                const v4f s2 = *(const v4f*)(sS2 + nl);
+                const v4f fb = *(const v4f*)(sFb + nl);
+                const v4i ib = *(const v4i*)(sIb + nl);
+                v4us o;
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    float v = (float)(acc[i][j][q * 4 + e] + ib[e]);
+                    v = v * s2[e];
+                    v = v * s1;
+                    v = v + fb[e];
+                    o[e] = to_b16<OUT_DT>(v);
+                }
+                if (m < p.M) {
+                    if (vec_ok && n + 3 < p.N) {
+                        *(v4us*)(out + m * p.N + n) = o;
+                    } else {
+#pragma unroll
+                        for (int e = 0; e < 4; e++)
+                            if (n + e < p.N) out[m * p.N + n + e] = o[e];
+                    }
+                }
+            }
+        }
+    }
+}
+
+template <int BM, int BN, int BK>
+static int launch_mfma(const QmmI8Params& p, int64_t batch, hipStream_t st)
+{
+    int tiles_m = (int)((p.M + BM - 1) / BM), tiles_n = (int)((p.N + BN - 1) / BN);
+    dim3 grid((unsigned)(tiles_m * tiles_n), (unsigned)batch);
+    size_t lds = 2 * (size_t)(BM + BN) * BK;
+    hipError_t e;
+    if (p.out_dt == DT_BF16) {
+        auto k = qmm_i8_mfma<BM, BN, BK, DT_BF16>;
+        e = hipFuncSetAttribute((const void*)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return (int)e;
+        hipLaunchKernelGGL(k, grid, dim3(256), lds, st, p, tiles_m, tiles_n);
+    } else {
+        auto k = qmm_i8_mfma<BM, BN, BK, DT_F16>;
+        e = hipFuncSetAttribute((const void*)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return (int)e;
+        hipLaunchKernelGGL(k, grid, dim3(256), lds, st, p, tiles_m, tiles_n);
+    }
+    return (int)hipGetLastError();
+}
+
+}  // namespace opsnn
+
+using namespace opsnn;
+
+extern "C" int opsnnQmmInt8(const OpsnnQmmArgs* a, void* stream)
+{
+    if (!a || !a->x1.ptr || !a->x2.ptr || !a->out || !a->x2_scale) return -1;
+    if (a->x1_dtype != DT_I8 || a->x2_dtype != DT_I8) return -2;
+    if (a->M <= 0 || a->N <= 0 || a->K <= 0 || a->batch <= 0) return -3;
+    hipStream_t st = (hipStream_t)stream;
+    QmmI8Params p;
+    p.a = (const int8_t*)a->x1.ptr; p.a_rs = a->x1.row_stride; p.a_cs = a->x1.col_stride; p.a_bs = a->x1.batch_stride;
+    p.b = (const int8_t*)a->x2.ptr; p.b_rs = a->x2.row_stride; p.b_cs = a->x2.col_stride; p.b_bs = a->x2.batch_stride;
+    p.out = a->out; p.M = a->M; p.N = a->N; p.K = a->K;
+    p.x1s = (const float*)a->x1_scale; p.x2s = a->x2_scale; p.x2s_dt = a->x2_scale_dtype; p.x2s_len = a->x2_scale_len;
+    p.bias = a->bias; p.bias_dt = a->bias_dtype; p.bias_bs = a->bias_batch_stride; p.out_dt = a->out_dtype;
+
+    // x2 stored N-major ([K, N] rows): relayout into the workspace as [N, K] first.
+    bool b_kmajor = (p.b_rs == 1);
+    bool a_kmajor = (p.a_cs == 1);
+    bool b16 = (p.out_dt == DT_BF16 || p.out_dt == DT_F16);
+    int variant = a->force_variant;
+    bool want_fast = b16 && a_kmajor && variant != OPSNN_VARIANT_PLAIN && p.M * p.N >= 64 * 64 && (p.K % 16) == 0 &&
+                     (p.a_rs % 16) == 0 && ((uintptr_t)p.a % 16) == 0 && (p.a_bs % 16) == 0;
+    if (want_fast && !b_kmajor && p.b_cs == 1 && a->workspace && p.b_rs == p.N && (p.b_bs == 0 || p.b_bs == p.K * p.N)) {
+        int64_t nb = p.b_bs == 0 ? 1 : a->batch;
+        int rc = opsnnTranspose8(p.b, a->workspace, p.K, p.N, nb, stream);
+        if (rc != 0) return rc;
+        p.b = (const int8_t*)a->workspace; p.b_rs = 1; p.b_cs = p.K; p.b_bs = p.b_bs == 0 ? 0 : p.K * p.N;
+        b_kmajor = true;
+    }
+    bool fast = want_fast && b_kmajor && (p.b_cs % 16) == 0 && ((uintptr_t)p.b % 16) == 0 && (p.b_bs % 16) == 0;
+    if (fast) {
+        if (variant == OPSNN_VARIANT_I8_128 || (variant == 0 && (p.M <= 128 || p.N <= 128 || p.M * p.N < 256 * 256 * 64)))
+            return launch_mfma<128, 128, 128>(p, a->batch, st);
+        return launch_mfma<256, 256, 128>(p, a->batch, st);
+    }
+    dim3 block(256), grid((unsigned)(((p.N + 255) / 256) * p.M), (unsigned)a->batch);
+    hipLaunchKernelGGL(qmm_i8_plain, grid, block, 0, st, p);
+    return (int)hipGetLastError();
+}

@@ -1,0 +1,530 @@
+/*
+ * CPU oracle for the quantized-matmul path -- TEST INFRASTRUCTURE ONLY.
+ *
+ * A plain-C restatement of the reference's numpy golden functions.  Only the
+ * test-suite, the smoke check and the benchmark's CPU-baseline leg may link or
+ * call this file; the product library never does.
+ *
+ * Each function cites the golden it follows (paths relative to the reference
+ * tree, under matmul/):
+ *   G3  = quant_batch_matmul_v3/tests/assets/qbmmv3_kernel_golden.py
+ *   GW  = weight_quant_batch_matmul_v2/tests/assets/wqbmmv2_kernel_golden.py
+ *   GU  = common/tests/st/arch35/matmul_golden_util.py
+ *   GQ  = common/tests/st/arch35/matmul_quant_util.py
+ *
+ * Arithmetic conventions shared with the golden: every float operation is a
+ * separately rounded fp32 operation (this file is compiled with
+ * -ffp-contract=off so the compiler cannot fuse a*b+c), casts to 16-bit types
+ * round to nearest even, int8 x int8 accumulates exactly in int32.  The one
+ * thing the golden leaves open is the summation order inside np.matmul (BLAS);
+ * here it is ascending k.
+ *
+ * Pinning status (tests/test_oracle_*.py):
+ *   codecs ............ pinned (exhaustive tables vs OCP definitions, torch CPU dtypes, reference constants)
+ *   orc_qmm_int8_acc .. pinned (brute force, closed forms, identity operands)
+ *   orc_qmm_pertoken .. pinned (float64 recomputation, operation-order cases, all-ones example)
+ *   orc_qmm_perblock .. pinned (reduces to pertoken formula with one K block; power-of-two scales exact; float64)
+ *   orc_qmm_mx ........ pinned (power-of-two products are exact: equals integer arithmetic; float64)
+ *   orc_wqbmm ......... pinned (hand-computed double-rounding cases; group==K equals per-channel; float64)
+ *   hifloat8 .......... not implemented (decoder lives only in an absent third-party package): parity unpinned
+ */
+#include <math.h>
+#include <stdint.h>
+#include <stdlib.h>
+#include <string.h>
+
+#include "oracle.h"
+
+#define CLONES __attribute__((target_clones("avx512f", "avx2", "default")))
+
+/* ------------------------------------------------------------------------- */
+/* Codecs                                                                     */
+/* ------------------------------------------------------------------------- */
+
+static inline uint32_t f2u(float f) { uint32_t u; memcpy(&u, &f, 4); return u; }
+static inline float u2f(uint32_t u) { float f; memcpy(&f, &u, 4); return f; }
+
+/* fp32 -> bf16, round to nearest even; NaN stays NaN (quiet). */
+uint16_t orc_bf16_from_f32(float f)
+{
+    uint32_t u = f2u(f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x0040u);
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return (uint16_t)(u >> 16);
+}
+float orc_bf16_to_f32(uint16_t h) { return u2f((uint32_t)h << 16); }
+
+/* fp32 -> fp16 (IEEE binary16), round to nearest even, gradual underflow, overflow to inf. */
+uint16_t orc_f16_from_f32(float f)
+{
+    uint32_t u = f2u(f);
+    uint32_t sign = (u >> 16) & 0x8000u;
+    uint32_t a = u & 0x7fffffffu;
+    if (a > 0x7f800000u) return (uint16_t)(sign | 0x7e00u);
+    if (a >= 0x47800000u) { /* >= 65536: inf; [65520, 65536) also rounds to inf below */
+        return (uint16_t)(sign | 0x7c00u);
+    }
+    if (a < 0x38800000u) { /* below the smallest normal 2^-14: subnormal result */
+        if (a < 0x33000000u) return (uint16_t)sign; /* < 2^-25 rounds to zero (2^-25 itself ties to even = 0) */
+        uint32_t e = a >> 23;                 /* biased fp32 exponent, 102..112 */
+        uint32_t m = (a & 0x7fffffu) | 0x800000u;
+        uint32_t shift = 126u - e;            /* 14..24: value = m * 2^(e-150); half ulp16sub = 2^-24 */
+        uint32_t q = m >> shift;
+        uint32_t rem = m & ((1u << shift) - 1u);
+        uint32_t half = 1u << (shift - 1u);
+        if (rem > half || (rem == half && (q & 1u))) q++;
+        return (uint16_t)(sign | q);
+    }
+    uint32_t r = a + 0xfffu + ((a >> 13) & 1u);
+    r = (r - 0x38000000u) >> 13;
+    if (r >= 0x7c00u) r = 0x7c00u;
+    return (uint16_t)(sign | r);
+}
+float orc_f16_to_f32(uint16_t h)
+{
+    uint32_t sign = ((uint32_t)h & 0x8000u) << 16;
+    uint32_t e = (h >> 10) & 0x1fu;
+    uint32_t m = h & 0x3ffu;
+    if (e == 0) {
+        if (m == 0) return u2f(sign);
+        float v = (float)m * 5.9604644775390625e-08f; /* 2^-24 */
+        return sign ? -v : v;
+    }
+    if (e == 31) return u2f(sign | 0x7f800000u | (m << 13));
+    return u2f(sign | ((e + 112u) << 23) | (m << 13));
+}
+
+/* OCP FP8 E4M3 (fn): bias 7, no inf, NaN = S.1111.111, max 448. */
+float orc_e4m3_to_f32(uint8_t b)
+{
+    uint32_t e = (b >> 3) & 0xfu, m = b & 7u;
+    float v;
+    if (e == 15 && m == 7) return u2f(0x7fc00000u | ((uint32_t)(b & 0x80u) << 24));
+    if (e == 0) v = (float)m * 0.001953125f; /* 2^-9 */
+    else v = ldexpf((float)(8 + m), (int)e - 10);
+    return (b & 0x80u) ? -v : v;
+}
+/* OCP FP8 E5M2: bias 15, IEEE-like inf/NaN. */
+float orc_e5m2_to_f32(uint8_t b)
+{
+    uint32_t e = (b >> 2) & 0x1fu, m = b & 3u;
+    float v;
+    if (e == 31) return u2f(((uint32_t)(b & 0x80u) << 24) | 0x7f800000u | (m ? 0x400000u : 0u));
+    if (e == 0) v = (float)m * 1.52587890625e-05f; /* 2^-16 */
+    else v = ldexpf((float)(4 + m), (int)e - 17);
+    return (b & 0x80u) ? -v : v;
+}
+/* fp32 -> e4m3fn, round to nearest even; magnitudes that round above 448 and NaN give NaN (0x7f). */
+uint8_t orc_e4m3_from_f32(float f)
+{
+    uint32_t u = f2u(f);
+    uint8_t sign = (uint8_t)((u >> 24) & 0x80u);
+    float a = fabsf(f);
+    if (!(a == a)) return (uint8_t)(sign | 0x7f);
+    if (a >= 480.0f) return (uint8_t)(sign | 0x7f); /* 464 is the tie between 448 and the absent 480: stays 448 */
+    if (a < 0.0009765625f) return sign;              /* < 2^-10 -> 0 (tie at 2^-10 goes to even = 0) */
+    int e;
+    (void)frexpf(a, &e);                             /* a = fr * 2^e, fr in [0.5,1) */
+    int exp = e - 1;                                 /* a in [2^exp, 2^(exp+1)) */
+    if (exp < -6) exp = -6;                          /* subnormal quantum 2^-9 */
+    float q = ldexpf(1.0f, exp - 3);
+    float n = a / q;                                 /* exact: power-of-two division */
+    float r = nearbyintf(n);                         /* default rounding mode = nearest even */
+    float v = r * q;
+    if (v > 448.0f) return (uint8_t)(sign | 0x7e);   /* 464 case rounds to 448 */
+    /* encode v */
+    if (v < 0.015625f) return (uint8_t)(sign | (uint8_t)(v * 512.0f));
+    int e2;
+    float fr = frexpf(v, &e2);
+    uint32_t mant = (uint32_t)(fr * 16.0f) - 8u;
+    return (uint8_t)(sign | (uint8_t)(((e2 - 1 + 7) << 3) | mant));
+}
+
+/* FP4 E2M1 value table (GQ:329-346): codes 0..7 = {0,.5,1,1.5,2,3,4,6}, bit 3 = sign. */
+static const float kE2M1[16] = {0.0f, 0.5f, 1.0f, 1.5f, 2.0f, 3.0f, 4.0f, 6.0f,
+                                -0.0f, -0.5f, -1.0f, -1.5f, -2.0f, -3.0f, -4.0f, -6.0f};
+float orc_e2m1_to_f32(uint8_t code) { return kE2M1[code & 15u]; }
+/* E8M0: 2^(b-127); 0xFF = NaN. */
+float orc_e8m0_to_f32(uint8_t b)
+{
+    if (b == 0xffu) return u2f(0x7fc00000u);
+    if (b == 0) return u2f(0x00400000u); /* 2^-127, an fp32 subnormal */
+    return u2f((uint32_t)b << 23);
+}
+
+void orc_vec_f32_to_bf16(const float* in, uint16_t* out, size_t n) { for (size_t i = 0; i < n; i++) out[i] = orc_bf16_from_f32(in[i]); }
+void orc_vec_bf16_to_f32(const uint16_t* in, float* out, size_t n) { for (size_t i = 0; i < n; i++) out[i] = orc_bf16_to_f32(in[i]); }
+void orc_vec_f32_to_f16(const float* in, uint16_t* out, size_t n) { for (size_t i = 0; i < n; i++) out[i] = orc_f16_from_f32(in[i]); }
+void orc_vec_f16_to_f32(const uint16_t* in, float* out, size_t n) { for (size_t i = 0; i < n; i++) out[i] = orc_f16_to_f32(in[i]); }
+void orc_vec_f32_to_e4m3(const float* in, uint8_t* out, size_t n) { for (size_t i = 0; i < n; i++) out[i] = orc_e4m3_from_f32(in[i]); }
+void orc_vec_e4m3_to_f32(const uint8_t* in, float* out, size_t n) { for (size_t i = 0; i < n; i++) out[i] = orc_e4m3_to_f32(in[i]); }
+void orc_vec_e5m2_to_f32(const uint8_t* in, float* out, size_t n) { for (size_t i = 0; i < n; i++) out[i] = orc_e5m2_to_f32(in[i]); }
+void orc_vec_e8m0_to_f32(const uint8_t* in, float* out, size_t n) { for (size_t i = 0; i < n; i++) out[i] = orc_e8m0_to_f32(in[i]); }
+
+/* groupSize = gsK | gsN << 16 | gsM << 32, zero fields read as 1 (GQ:179-191). */
+void orc_unpack_groupsize(int64_t gs, int64_t* gsM, int64_t* gsN, int64_t* gsK)
+{
+    *gsM = (gs >> 32) & 0xffff; *gsN = (gs >> 16) & 0xffff; *gsK = gs & 0xffff;
+    if (*gsM == 0) *gsM = 1;
+    if (*gsN == 0) *gsN = 1;
+    if (*gsK == 0) *gsK = 1;
+}
+
+/* Eight int4 values per int32, element i in bits 4i..4i+3 (GQ:228-273, 349-394). */
+void orc_pack_int4_to_int32(const int8_t* in, int32_t* out, size_t n_packed)
+{
+    for (size_t i = 0; i < n_packed; i++) {
+        uint32_t w = 0;
+        for (int j = 0; j < 8; j++) w |= ((uint32_t)in[i * 8 + j] & 0xfu) << (4 * j);
+        out[i] = (int32_t)w;
+    }
+}
+void orc_unpack_int32_to_int4(const int32_t* in, int8_t* out, size_t n_packed)
+{
+    for (size_t i = 0; i < n_packed; i++) {
+        uint32_t w = (uint32_t)in[i];
+        for (int j = 0; j < 8; j++) {
+            int v = (int)((w >> (4 * j)) & 0xfu);
+            out[i * 8 + j] = (int8_t)(v >= 8 ? v - 16 : v);
+        }
+    }
+}
+
+static size_t dtype_bits(int dt)
+{
+    switch (dt) {
+        case ORC_F32: case ORC_I32: return 32;
+        case ORC_F16: case ORC_BF16: return 16;
+        case ORC_I8: case ORC_E4M3: case ORC_E5M2: case ORC_E8M0: return 8;
+        case ORC_I4: case ORC_E2M1: return 4;
+        default: return 0;
+    }
+}
+
+/* Decode element i of a dense buffer to fp32 (every supported type converts exactly). */
+static inline float load_as_f32(const void* p, int dt, size_t i)
+{
+    switch (dt) {
+        case ORC_F32: return ((const float*)p)[i];
+        case ORC_I32: return (float)((const int32_t*)p)[i];
+        case ORC_F16: return orc_f16_to_f32(((const uint16_t*)p)[i]);
+        case ORC_BF16: return orc_bf16_to_f32(((const uint16_t*)p)[i]);
+        case ORC_I8: return (float)((const int8_t*)p)[i];
+        case ORC_E4M3: return orc_e4m3_to_f32(((const uint8_t*)p)[i]);
+        case ORC_E5M2: return orc_e5m2_to_f32(((const uint8_t*)p)[i]);
+        case ORC_E8M0: return orc_e8m0_to_f32(((const uint8_t*)p)[i]);
+        case ORC_I4: {
+            uint8_t b = ((const uint8_t*)p)[i >> 1];
+            int v = (i & 1) ? (b >> 4) : (b & 15);
+            return (float)(v >= 8 ? v - 16 : v);
+        }
+        case ORC_E2M1: {
+            uint8_t b = ((const uint8_t*)p)[i >> 1];
+            return kE2M1[(i & 1) ? (b >> 4) : (b & 15)];
+        }
+        default: return NAN;
+    }
+}
+
+/* cast_output_dtype (GU:68-73): fp32 -> y dtype, RNE. */
+static inline void store_from_f32(void* p, int dt, size_t i, float v)
+{
+    switch (dt) {
+        case ORC_F32: ((float*)p)[i] = v; break;
+        case ORC_F16: ((uint16_t*)p)[i] = orc_f16_from_f32(v); break;
+        case ORC_BF16: ((uint16_t*)p)[i] = orc_bf16_from_f32(v); break;
+        default: break;
+    }
+}
+
+/* Storage [rows, cols] (row-major, sub-byte types packed along cols) -> fp32 [R, C]
+ * where (R, C) = (cols, rows) if transpose else (rows, cols). */
+static float* decode_matrix(const void* src, int dt, int64_t rows, int64_t cols, int transpose)
+{
+    float* dst = (float*)malloc(sizeof(float) * (size_t)rows * (size_t)cols);
+    if (!dst) return NULL;
+#pragma omp parallel for schedule(static)
+    for (int64_t r = 0; r < rows; r++)
+        for (int64_t c = 0; c < cols; c++) {
+            float v = load_as_f32(src, dt, (size_t)(r * cols + c));
+            if (transpose) dst[c * rows + r] = v; else dst[r * cols + c] = v;
+        }
+    return dst;
+}
+
+/* ------------------------------------------------------------------------- */
+/* Contractions                                                               */
+/* ------------------------------------------------------------------------- */
+
+/* C[M,N] (+)= A[M,K(lda)] @ B[K,N(ldb)], fp32, ascending k, product and sum rounded separately. */
+CLONES static void sgemm_tile(const float* A, int64_t lda, const float* B, int64_t ldb, float* C, int64_t ldc,
+                              int64_t m0, int64_t m1, int64_t n0, int64_t n1, int64_t K)
+{
+    for (int64_t m = m0; m < m1; m++) {
+        float* c = C + m * ldc;
+        for (int64_t k = 0; k < K; k++) {
+            float a = A[m * lda + k];
+            const float* b = B + k * ldb;
+            for (int64_t n = n0; n < n1; n++) c[n] = c[n] + a * b[n];
+        }
+    }
+}
+
+static void sgemm_acc(const float* A, int64_t lda, const float* B, int64_t ldb, float* C, int64_t ldc, int64_t M,
+                      int64_t N, int64_t K)
+{
+    const int64_t TM = 8, TN = 512;
+    int64_t mt = (M + TM - 1) / TM, nt = (N + TN - 1) / TN;
+#pragma omp parallel for collapse(2) schedule(dynamic)
+    for (int64_t i = 0; i < mt; i++)
+        for (int64_t j = 0; j < nt; j++) {
+            int64_t m1 = (i + 1) * TM < M ? (i + 1) * TM : M;
+            int64_t n1 = (j + 1) * TN < N ? (j + 1) * TN : N;
+            sgemm_tile(A, lda, B, ldb, C, ldc, i * TM, m1, j * TN, n1, K);
+        }
+}
+
+CLONES static void igemm_tile(const int8_t* A, int64_t lda, const int8_t* B, int64_t ldb, int32_t* C, int64_t ldc,
+                              int64_t m0, int64_t m1, int64_t n0, int64_t n1, int64_t K)
+{
+    for (int64_t m = m0; m < m1; m++) {
+        int32_t* c = C + m * ldc;
+        for (int64_t k = 0; k < K; k++) {
+            int32_t a = A[m * lda + k];
+            const int8_t* b = B + k * ldb;
+            for (int64_t n = n0; n < n1; n++) c[n] += a * (int32_t)b[n];
+        }
+    }
+}
+
+/*
+ * acc[M,N] = int32(x1) @ int32(x2)   (G3:614-634: both operands widened to int32, np.matmul).
+ * x1 storage is [M,K] (or [K,M] if tA), x2 storage is [K,N] (or [N,K] if tB), int8.
+ */
+int orc_qmm_int8_acc(const int8_t* x1, const int8_t* x2, int64_t M, int64_t K, int64_t N, int tA, int tB,
+                     int32_t* acc)
+{
+    int8_t* a = (int8_t*)x1;
+    int8_t* b = (int8_t*)x2;
+    if (tA) {
+        a = (int8_t*)malloc((size_t)M * K);
+        if (!a) return -1;
+        for (int64_t k = 0; k < K; k++) for (int64_t m = 0; m < M; m++) a[m * K + k] = x1[k * M + m];
+    }
+    if (tB) {
+        b = (int8_t*)malloc((size_t)N * K);
+        if (!b) return -1;
+#pragma omp parallel for schedule(static)
+        for (int64_t n = 0; n < N; n++) for (int64_t k = 0; k < K; k++) b[k * N + n] = x2[n * K + k];
+    }
+    memset(acc, 0, sizeof(int32_t) * (size_t)M * N);
+    const int64_t TM = 8, TN = 1024;
+    int64_t mt = (M + TM - 1) / TM, nt = (N + TN - 1) / TN;
+#pragma omp parallel for collapse(2) schedule(dynamic)
+    for (int64_t i = 0; i < mt; i++)
+        for (int64_t j = 0; j < nt; j++) {
+            int64_t m1 = (i + 1) * TM < M ? (i + 1) * TM : M;
+            int64_t n1 = (j + 1) * TN < N ? (j + 1) * TN : N;
+            igemm_tile(a, K, b, N, acc, N, i * TM, m1, j * TN, n1, K);
+        }
+    if (tA) free(a);
+    if (tB) free(b);
+    return 0;
+}
+
+/*
+ * compute_pertoken (G3:361-387), K-C / K-T modes.
+ *   out = acc (+ int32 bias, integer domain)
+ *   out = fp32(out) * x2Scale[n] * x1Scale[m]        -- evaluated left to right
+ *   out = out + fp32(bias) for a float bias           -- after scaling (both golden branches agree)
+ *   y   = cast(out)
+ * x2s_len is 1 (K-T) or N (K-C).  x1s may be NULL (then treated as absent: T-C dynamic path of
+ * compute_tc G3:390-475 without scale truncation, i.e. bf16/fp32 scale with float bias).
+ */
+int orc_qmm_pertoken_epilogue(const int32_t* acc, int64_t M, int64_t N, const float* x1s, const float* x2s,
+                              int64_t x2s_len, const void* bias, int bias_dt, int y_dt, void* y)
+{
+#pragma omp parallel for schedule(static)
+    for (int64_t m = 0; m < M; m++)
+        for (int64_t n = 0; n < N; n++) {
+            int32_t a = acc[m * N + n];
+            if (bias && bias_dt == ORC_I32) a += ((const int32_t*)bias)[n];
+            float o = (float)a;
+            o = o * x2s[x2s_len == 1 ? 0 : n];
+            if (x1s) o = o * x1s[m];
+            if (bias && bias_dt != ORC_I32) o = o + load_as_f32(bias, bias_dt, (size_t)n);
+            store_from_f32(y, y_dt, (size_t)(m * N + n), o);
+        }
+    return 0;
+}
+
+int orc_qmm_pertoken(const int8_t* x1, const int8_t* x2, int64_t M, int64_t K, int64_t N, int tA, int tB,
+                     const float* x1s, const float* x2s, int64_t x2s_len, const void* bias, int bias_dt, int y_dt,
+                     void* y, int32_t* acc_out)
+{
+    int32_t* acc = acc_out ? acc_out : (int32_t*)malloc(sizeof(int32_t) * (size_t)M * N);
+    if (!acc) return -1;
+    int rc = orc_qmm_int8_acc(x1, x2, M, K, N, tA, tB, acc);
+    if (rc == 0) rc = orc_qmm_pertoken_epilogue(acc, M, N, x1s, x2s, x2s_len, bias, bias_dt, y_dt, y);
+    if (!acc_out) free(acc);
+    return rc;
+}
+
+/*
+ * compute_perblock (G3:237-358), G-B / B-B modes, one batch slice.
+ *   for kb in range(ceil(K/gsK)):
+ *       y += (fp32(x1[:, kb]) @ fp32(x2[kb, :])) * (x1Scale[m/gsM, kb] * x2Scale[kb, n/gsN])
+ *   y (+ fp32 bias);  cast
+ * Scale storage follows the operand's transposition (G3:276-286): x1s is [ceil(M/gsM), KB]
+ * (or [KB, ceil(M/gsM)] if tA); x2s is [KB, ceil(N/gsN)] (or [ceil(N/gsN), KB] if tB).
+ */
+int orc_qmm_perblock(const void* x1, const void* x2, int dt1, int dt2, int64_t M, int64_t K, int64_t N, int tA,
+                     int tB, const float* x1s, const float* x2s, int64_t gsM, int64_t gsN, int64_t gsK,
+                     const float* bias, int y_dt, void* y)
+{
+    float* a = tA ? decode_matrix(x1, dt1, K, M, 1) : decode_matrix(x1, dt1, M, K, 0);
+    float* b = tB ? decode_matrix(x2, dt2, N, K, 1) : decode_matrix(x2, dt2, K, N, 0);
+    float* acc = (float*)calloc((size_t)M * N, sizeof(float));
+    float* part = (float*)malloc(sizeof(float) * (size_t)M * N);
+    if (!a || !b || !acc || !part) return -1;
+    int64_t KB = (K + gsK - 1) / gsK, MB = (M + gsM - 1) / gsM, NB = (N + gsN - 1) / gsN;
+    for (int64_t kb = 0; kb < KB; kb++) {
+        int64_t k0 = kb * gsK, k1 = (kb + 1) * gsK < K ? (kb + 1) * gsK : K;
+        memset(part, 0, sizeof(float) * (size_t)M * N);
+        sgemm_acc(a + k0, K, b + k0 * N, N, part, N, M, N, k1 - k0);
+#pragma omp parallel for schedule(static)
+        for (int64_t m = 0; m < M; m++) {
+            float s1 = tA ? x1s[kb * MB + m / gsM] : x1s[(m / gsM) * KB + kb];
+            for (int64_t n = 0; n < N; n++) {
+                float s2 = tB ? x2s[(n / gsN) * KB + kb] : x2s[kb * NB + n / gsN];
+                float sc = s1 * s2;
+                acc[m * N + n] = acc[m * N + n] + part[m * N + n] * sc;
+            }
+        }
+    }
+    for (int64_t m = 0; m < M; m++)
+        for (int64_t n = 0; n < N; n++) {
+            float o = acc[m * N + n];
+            if (bias) o = o + bias[n];
+            store_from_f32(y, y_dt, (size_t)(m * N + n), o);
+        }
+    free(a); free(b); free(acc); free(part);
+    return 0;
+}
+
+/*
+ * compute_mx (G3:153-234), MX (G-G) mode, one batch slice.
+ *   x1f = fp32(x1) * repeat32(x1Scale),  x2f = fp32(x2) * repeat32(x2Scale)   (K zero-padded to the scale extent)
+ *   y = x1f @ x2f (+ fp32 bias);  cast
+ * Scale storage (e8m0 bytes): x1s [M, KS, 2] (or [KS, M, 2] if tA); x2s [KS, N, 2] (or [N, KS, 2] if tB),
+ * KS = ceil(K/64); the scale for 32-wide K block kb is entry [.., kb/2, .., kb%2] (G3:171-197).
+ * If ceil(K/32) is odd the last (pad) scale is dropped (G3:199-202).
+ */
+int orc_qmm_mx(const void* x1, const void* x2, int dt1, int dt2, int64_t M, int64_t K, int64_t N, int tA, int tB,
+               const uint8_t* x1s, const uint8_t* x2s, const float* bias, int y_dt, void* y)
+{
+    float* a = tA ? decode_matrix(x1, dt1, K, M, 1) : decode_matrix(x1, dt1, M, K, 0);
+    float* b = tB ? decode_matrix(x2, dt2, N, K, 1) : decode_matrix(x2, dt2, K, N, 0);
+    float* acc = (float*)calloc((size_t)M * N, sizeof(float));
+    if (!a || !b || !acc) return -1;
+    int64_t KS = (K + 63) / 64;
+#pragma omp parallel for schedule(static)
+    for (int64_t m = 0; m < M; m++)
+        for (int64_t k = 0; k < K; k++) {
+            int64_t kb = k / 32;
+            uint8_t s = tA ? x1s[((kb / 2) * M + m) * 2 + (kb & 1)] : x1s[(m * KS + kb / 2) * 2 + (kb & 1)];
+            a[m * K + k] = a[m * K + k] * orc_e8m0_to_f32(s);
+        }
+#pragma omp parallel for schedule(static)
+    for (int64_t k = 0; k < K; k++)
+        for (int64_t n = 0; n < N; n++) {
+            int64_t kb = k / 32;
+            uint8_t s = tB ? x2s[(n * KS + kb / 2) * 2 + (kb & 1)] : x2s[((kb / 2) * N + n) * 2 + (kb & 1)];
+            b[k * N + n] = b[k * N + n] * orc_e8m0_to_f32(s);
+        }
+    sgemm_acc(a, K, b, N, acc, N, M, N, K);
+    for (int64_t m = 0; m < M; m++)
+        for (int64_t n = 0; n < N; n++) {
+            float o = acc[m * N + n];
+            if (bias) o = o + bias[n];
+            store_from_f32(y, y_dt, (size_t)(m * N + n), o);
+        }
+    free(a); free(b); free(acc);
+    return 0;
+}
+
+/* truncate (GU:235-239): round an fp32 value through the intermediate 16-bit type. */
+static inline float trunc_to(float v, int dt)
+{
+    if (dt == ORC_F16) return orc_f16_to_f32(orc_f16_from_f32(v));
+    if (dt == ORC_BF16) return orc_bf16_to_f32(orc_bf16_from_f32(v));
+    return v;
+}
+
+/*
+ * wqbmm_kernel_compute (GW:106-196) for the T / C / G / MX antiquant modes.
+ *   per-tensor / per-channel (_compute_tc, GW:199-239) and per-group (_compute_pergroup, GW:242-297):
+ *       w = T(T(w + offset) * scale)      with offset
+ *       w = T(w * scale)                  without offset            T = round through x's dtype
+ *   MX (_compute_mx, GW:300-352): w = T(fp4 * T16(2^e)) per 32 K (the scale is first rounded through
+ *       fp16 when x is fp16)
+ *   y = fp32(x) @ w  (+ fp32(bias));  if x is bf16 round through bf16;  cast to x's dtype
+ *   (matmul_and_finalize / finalize, GW:85-103).
+ *
+ * weight storage: [K, N] (or [N, K] if tW), sub-byte packed along the storage's last axis.
+ * scale/offset storage: [G, N] (or [N, G] if tW) with G = 1 or ceil(K/group); a scale with
+ * scale_n == 1 is per-tensor.  scale_dt is x's dtype or ORC_E8M0.
+ */
+int orc_wqbmm(const void* x, int x_dt, const void* w, int w_dt, int64_t M, int64_t K, int64_t N, int tW,
+              const void* scale, int scale_dt, int64_t scale_n, const void* offset, int64_t group,
+              const void* bias, int bias_dt, void* y)
+{
+    int inter = x_dt;
+    float* xf = decode_matrix(x, x_dt, M, K, 0);
+    float* wf = tW ? decode_matrix(w, w_dt, N, K, 1) : decode_matrix(w, w_dt, K, N, 0);
+    float* acc = (float*)calloc((size_t)M * N, sizeof(float));
+    if (!xf || !wf || !acc) return -1;
+    int mx = (scale_dt == ORC_E8M0);
+    int64_t g = mx ? 32 : (group > 0 ? group : K);
+    int64_t G = (K + g - 1) / g;
+    if (scale_n == 1 || (!mx && group <= 0)) G = 1, g = K;
+#pragma omp parallel for schedule(static)
+    for (int64_t k = 0; k < K; k++) {
+        int64_t gi = k / g;
+        for (int64_t n = 0; n < N; n++) {
+            int64_t sn = scale_n == 1 ? 0 : n;
+            size_t si = (size_t)(tW ? sn * G + gi : gi * scale_n + sn);
+            float s = load_as_f32(scale, scale_dt, si);
+            float v = wf[k * N + n];
+            if (inter == ORC_F16) v = trunc_to(v, ORC_F16); /* prepare_weight GW:53-62 (exact for every weight type) */
+            if (mx) {
+                if (inter == ORC_F16) s = trunc_to(s, ORC_F16);
+                v = trunc_to(v * s, inter);
+            } else if (offset) {
+                float o = trunc_to(load_as_f32(offset, x_dt, si), inter);
+                v = trunc_to(v + o, inter);
+                v = trunc_to(v * s, inter);
+            } else {
+                v = trunc_to(v * s, inter);
+            }
+            wf[k * N + n] = v;
+        }
+    }
+    sgemm_acc(xf, K, wf, N, acc, N, M, N, K);
+    for (int64_t m = 0; m < M; m++)
+        for (int64_t n = 0; n < N; n++) {
+            float o = acc[m * N + n];
+            if (bias) o = o + load_as_f32(bias, bias_dt, (size_t)n);
+            if (x_dt == ORC_BF16) o = trunc_to(o, ORC_BF16);
+            store_from_f32(y, x_dt, (size_t)(m * N + n), o);
+        }
+    free(xf); free(wf); free(acc);
+    return 0;
+}
+
+/* scale_generate (GQ:50-54): keep the upper 19 bits of an fp32 scale. */
+float orc_scale_generate(float s) { return u2f(f2u(s) & 0xFFFFE000u); }
+/* u64_to_deq_scale (GQ:129-135): the low 32 bits hold an fp32 scale, truncated as above. */
+float orc_u64_to_deq_scale(uint64_t v) { return u2f((uint32_t)v & 0xFFFFE000u); }
+
+size_t orc_dtype_bits(int dt) { return dtype_bits(dt); }

@@ -1,0 +1,62 @@
+/*
+ * CPU oracle for the quantized-matmul path -- TEST INFRASTRUCTURE ONLY
+ * (tests, the smoke check and the benchmark's CPU-baseline leg).  See oracle.c.
+ * Type codes equal the aclDataType values of include/acl/acl.h.
+ */
+#ifndef OPSNN_ORACLE_H_
+#define OPSNN_ORACLE_H_
+#include <stddef.h>
+#include <stdint.h>
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum {
+    ORC_F32 = 0, ORC_F16 = 1, ORC_I8 = 2, ORC_I32 = 3, ORC_BF16 = 27, ORC_I4 = 29,
+    ORC_E5M2 = 35, ORC_E4M3 = 36, ORC_E8M0 = 37, ORC_E2M1 = 40
+};
+
+uint16_t orc_bf16_from_f32(float f);
+float orc_bf16_to_f32(uint16_t h);
+uint16_t orc_f16_from_f32(float f);
+float orc_f16_to_f32(uint16_t h);
+float orc_e4m3_to_f32(uint8_t b);
+float orc_e5m2_to_f32(uint8_t b);
+uint8_t orc_e4m3_from_f32(float f);
+float orc_e2m1_to_f32(uint8_t code);
+float orc_e8m0_to_f32(uint8_t b);
+void orc_vec_f32_to_bf16(const float* in, uint16_t* out, size_t n);
+void orc_vec_bf16_to_f32(const uint16_t* in, float* out, size_t n);
+void orc_vec_f32_to_f16(const float* in, uint16_t* out, size_t n);
+void orc_vec_f16_to_f32(const uint16_t* in, float* out, size_t n);
+void orc_vec_f32_to_e4m3(const float* in, uint8_t* out, size_t n);
+void orc_vec_e4m3_to_f32(const uint8_t* in, float* out, size_t n);
+void orc_vec_e5m2_to_f32(const uint8_t* in, float* out, size_t n);
+void orc_vec_e8m0_to_f32(const uint8_t* in, float* out, size_t n);
+void orc_unpack_groupsize(int64_t gs, int64_t* gsM, int64_t* gsN, int64_t* gsK);
+void orc_pack_int4_to_int32(const int8_t* in, int32_t* out, size_t n_packed);
+void orc_unpack_int32_to_int4(const int32_t* in, int8_t* out, size_t n_packed);
+float orc_scale_generate(float s);
+float orc_u64_to_deq_scale(uint64_t v);
+size_t orc_dtype_bits(int dt);
+
+int orc_qmm_int8_acc(const int8_t* x1, const int8_t* x2, int64_t M, int64_t K, int64_t N, int tA, int tB,
+                     int32_t* acc);
+int orc_qmm_pertoken_epilogue(const int32_t* acc, int64_t M, int64_t N, const float* x1s, const float* x2s,
+                              int64_t x2s_len, const void* bias, int bias_dt, int y_dt, void* y);
+int orc_qmm_pertoken(const int8_t* x1, const int8_t* x2, int64_t M, int64_t K, int64_t N, int tA, int tB,
+                     const float* x1s, const float* x2s, int64_t x2s_len, const void* bias, int bias_dt, int y_dt,
+                     void* y, int32_t* acc_out);
+int orc_qmm_perblock(const void* x1, const void* x2, int dt1, int dt2, int64_t M, int64_t K, int64_t N, int tA,
+                     int tB, const float* x1s, const float* x2s, int64_t gsM, int64_t gsN, int64_t gsK,
+                     const float* bias, int y_dt, void* y);
+int orc_qmm_mx(const void* x1, const void* x2, int dt1, int dt2, int64_t M, int64_t K, int64_t N, int tA, int tB,
+               const uint8_t* x1s, const uint8_t* x2s, const float* bias, int y_dt, void* y);
+int orc_wqbmm(const void* x, int x_dt, const void* w, int w_dt, int64_t M, int64_t K, int64_t N, int tW,
+              const void* scale, int scale_dt, int64_t scale_n, const void* offset, int64_t group,
+              const void* bias, int bias_dt, void* y);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

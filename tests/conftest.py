@@ -1,0 +1,28 @@
+import os
+import sys
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+sys.path.insert(0, os.path.join(ROOT, "ops-nn_amd"))
+sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
+
+
+def pytest_configure(config):
+    config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu)")
+
+
+@pytest.fixture(scope="session")
+def opsnn():
+    import opsnn as m
+    m.lib()
+    return m
+
+
+@pytest.fixture(scope="session")
+def gpu(opsnn):
+    if not opsnn.gpu_available():
+        pytest.fail("this test is marked gpu but no HIP device is visible")
+    opsnn.check(opsnn.lib().aclInit(None), "aclInit")
+    opsnn.check(opsnn.lib().aclrtSetDevice(0), "aclrtSetDevice")
+    return opsnn

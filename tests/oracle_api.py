@@ -1,0 +1,147 @@
+"""ctypes access to oracle/liboracle.so (the CPU restatement of the reference goldens) plus numpy-side
+helpers for the narrow float formats.  Test infrastructure only."""
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+LIB = os.path.join(ROOT, "oracle", "liboracle.so")
+
+F32, F16, I8, I32, BF16, I4, E5M2, E4M3, E8M0, E2M1 = 0, 1, 2, 3, 27, 29, 35, 36, 37, 40
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB):
+            subprocess.run(["make", "-C", os.path.join(ROOT, "oracle")], check=True)
+        _lib = C.CDLL(LIB)
+        L = _lib
+        vp, i64, ci = C.c_void_p, C.c_int64, C.c_int
+        L.orc_qmm_int8_acc.argtypes = [vp, vp, i64, i64, i64, ci, ci, vp]
+        L.orc_qmm_pertoken_epilogue.argtypes = [vp, i64, i64, vp, vp, i64, vp, ci, ci, vp]
+        L.orc_qmm_pertoken.argtypes = [vp, vp, i64, i64, i64, ci, ci, vp, vp, i64, vp, ci, ci, vp, vp]
+        L.orc_qmm_perblock.argtypes = [vp, vp, ci, ci, i64, i64, i64, ci, ci, vp, vp, i64, i64, i64, vp, ci, vp]
+        L.orc_qmm_mx.argtypes = [vp, vp, ci, ci, i64, i64, i64, ci, ci, vp, vp, vp, ci, vp]
+        L.orc_wqbmm.argtypes = [vp, ci, vp, ci, i64, i64, i64, ci, vp, ci, i64, vp, i64, vp, ci, vp]
+        for n in ("orc_vec_f32_to_bf16", "orc_vec_bf16_to_f32", "orc_vec_f32_to_f16", "orc_vec_f16_to_f32",
+                  "orc_vec_f32_to_e4m3", "orc_vec_e4m3_to_f32", "orc_vec_e5m2_to_f32", "orc_vec_e8m0_to_f32"):
+            getattr(L, n).argtypes = [vp, vp, C.c_size_t]
+        L.orc_unpack_groupsize.argtypes = [i64, C.POINTER(i64), C.POINTER(i64), C.POINTER(i64)]
+        L.orc_pack_int4_to_int32.argtypes = [vp, vp, C.c_size_t]
+        L.orc_unpack_int32_to_int4.argtypes = [vp, vp, C.c_size_t]
+        L.orc_scale_generate.argtypes = [C.c_float]
+        L.orc_scale_generate.restype = C.c_float
+        L.orc_u64_to_deq_scale.argtypes = [C.c_uint64]
+        L.orc_u64_to_deq_scale.restype = C.c_float
+        L.orc_e2m1_to_f32.argtypes = [C.c_uint8]
+        L.orc_e2m1_to_f32.restype = C.c_float
+    return _lib
+
+
+def _p(a):
+    return a.ctypes.data if a is not None else None
+
+
+def _conv(name, src, out_dtype):
+    src = np.ascontiguousarray(src)
+    out = np.empty(src.shape, dtype=out_dtype)
+    getattr(lib(), name)(_p(src), _p(out), src.size)
+    return out
+
+
+def f32_to_bf16(a): return _conv("orc_vec_f32_to_bf16", np.asarray(a, np.float32), np.uint16)
+def bf16_to_f32(a): return _conv("orc_vec_bf16_to_f32", np.asarray(a, np.uint16), np.float32)
+def f32_to_f16(a): return _conv("orc_vec_f32_to_f16", np.asarray(a, np.float32), np.uint16)
+def f16_to_f32(a): return _conv("orc_vec_f16_to_f32", np.asarray(a, np.uint16), np.float32)
+def f32_to_e4m3(a): return _conv("orc_vec_f32_to_e4m3", np.asarray(a, np.float32), np.uint8)
+def e4m3_to_f32(a): return _conv("orc_vec_e4m3_to_f32", np.asarray(a, np.uint8), np.float32)
+def e5m2_to_f32(a): return _conv("orc_vec_e5m2_to_f32", np.asarray(a, np.uint8), np.float32)
+def e8m0_to_f32(a): return _conv("orc_vec_e8m0_to_f32", np.asarray(a, np.uint8), np.float32)
+
+
+E2M1_VALUES = np.array([0, .5, 1, 1.5, 2, 3, 4, 6, -0.0, -.5, -1, -1.5, -2, -3, -4, -6], np.float32)
+
+
+def pack_nibbles(codes):
+    """[.., C] values 0..15 -> [.., C/2] bytes, even index in the low nibble."""
+    codes = np.asarray(codes, np.uint8)
+    return (codes[..., 0::2] & 15) | ((codes[..., 1::2] & 15) << 4)
+
+
+def unpack_nibbles(b):
+    b = np.asarray(b, np.uint8)
+    out = np.empty(b.shape[:-1] + (b.shape[-1] * 2,), np.uint8)
+    out[..., 0::2] = b & 15
+    out[..., 1::2] = b >> 4
+    return out
+
+
+def b16_to_f32(bits, dt):
+    return bf16_to_f32(bits) if dt == BF16 else f16_to_f32(bits)
+
+
+def f32_to_b16(v, dt):
+    return f32_to_bf16(v) if dt == BF16 else f32_to_f16(v)
+
+
+def out_array(shape, dt):
+    return np.empty(shape, np.float32 if dt == F32 else (np.int32 if dt == I32 else np.uint16))
+
+
+def qmm_pertoken(x1, x2, M, K, N, tA, tB, x1s, x2s, bias, bias_dt, y_dt, want_acc=False):
+    y = out_array((M, N), y_dt)
+    acc = np.empty((M, N), np.int32) if want_acc else None
+    x2s = np.ascontiguousarray(x2s, np.float32)
+    rc = lib().orc_qmm_pertoken(_p(x1), _p(x2), M, K, N, int(tA), int(tB), _p(x1s), _p(x2s), x2s.size, _p(bias), bias_dt, y_dt,
+                                _p(y), _p(acc))
+    assert rc == 0
+    return (y, acc) if want_acc else y
+
+
+def qmm_int8_acc(x1, x2, M, K, N, tA=False, tB=False):
+    acc = np.empty((M, N), np.int32)
+    assert lib().orc_qmm_int8_acc(_p(x1), _p(x2), M, K, N, int(tA), int(tB), _p(acc)) == 0
+    return acc
+
+
+def qmm_perblock(x1, x2, dt1, dt2, M, K, N, tA, tB, x1s, x2s, gsM, gsN, gsK, bias, y_dt):
+    y = out_array((M, N), y_dt)
+    rc = lib().orc_qmm_perblock(_p(x1), _p(x2), dt1, dt2, M, K, N, int(tA), int(tB), _p(x1s), _p(x2s), gsM, gsN, gsK, _p(bias),
+                                y_dt, _p(y))
+    assert rc == 0
+    return y
+
+
+def qmm_mx(x1, x2, dt1, dt2, M, K, N, tA, tB, x1s, x2s, bias, y_dt):
+    y = out_array((M, N), y_dt)
+    rc = lib().orc_qmm_mx(_p(x1), _p(x2), dt1, dt2, M, K, N, int(tA), int(tB), _p(x1s), _p(x2s), _p(bias), y_dt, _p(y))
+    assert rc == 0
+    return y
+
+
+def wqbmm(x, x_dt, w, w_dt, M, K, N, tW, scale, scale_dt, scale_n, offset, group, bias, bias_dt):
+    y = np.empty((M, N), np.uint16)
+    rc = lib().orc_wqbmm(_p(x), x_dt, _p(w), w_dt, M, K, N, int(tW), _p(scale), scale_dt, scale_n, _p(offset), group, _p(bias),
+                         bias_dt, _p(y))
+    assert rc == 0
+    return y
+
+
+def rel_err_stats(got_f32, want_f32, floor=None):
+    """max and mean relative error with an absolute floor on the denominator."""
+    got = np.asarray(got_f32, np.float64)
+    want = np.asarray(want_f32, np.float64)
+    if floor is None:
+        floor = max(float(np.mean(np.abs(want))) * 1e-2, 1e-30)
+    rel = np.abs(got - want) / np.maximum(np.abs(want), floor)
+    return float(rel.max()), float(rel.mean())
+
+
+def isclose_fraction(got_f32, want_f32, rtol=1e-3, atol=1e-3):
+    """The reference's ST acceptance (matmul_golden_util.py:340-380): fraction of elements outside isclose."""
+    ok = np.isclose(got_f32, want_f32, rtol=rtol, atol=atol, equal_nan=True)
+    return 1.0 - ok.sum() / ok.size

@@ -1,0 +1,124 @@
+"""GPU parity: int8 x int8 per-token / per-channel quantized matmul (aclnnQuantMatmulV5, K-C / K-T / T-C).
+
+Bar: bit-exact.  The int32 accumulators are exact in any order, and the epilogue is a fixed sequence of
+separately rounded fp32 operations followed by one round-to-nearest-even cast, so the 16-bit outputs of the
+HIP kernels must equal the oracle's bit for bit (qbmmv3_kernel_golden.py:361-387).
+"""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+import cases
+import oracle_api as orc
+
+pytestmark = pytest.mark.gpu
+
+
+def _check_equal(got, want, what):
+    if not np.array_equal(got, want):
+        bad = np.argwhere(got != want)
+        raise AssertionError(f"{what}: {len(bad)} of {got.size} elements differ; first at {bad[0]}: "
+                             f"got {got[tuple(bad[0])]:#x} want {want[tuple(bad[0])]:#x}")
+
+
+@pytest.mark.parametrize("M,K,N,tB", [
+    (128, 256, 512, True),     # the reference's ST shape v3_kc_int8_fp32
+    (256, 512, 384, True),
+    (256, 512, 384, False),    # N-contiguous x2: re-laid out into the workspace first
+    (197, 960, 854, True),     # ragged M and N, K multiple of 16
+    (33, 77, 19, True),        # odd everything: plain kernel
+    (1, 4096, 128, True),      # M = 1
+    (300, 128, 260, False),
+])
+@pytest.mark.parametrize("out_dt,bias_dt", [("bf16", "bf16"), ("bf16", None), ("f16", "f32"), ("bf16", "i32"), ("f16", "f16")])
+def test_kc_matches_oracle(gpu, M, K, N, tB, out_dt, bias_dt):
+    m = gpu
+    dt = {"bf16": m.ACL_BF16, "f16": m.ACL_FLOAT16, "f32": m.ACL_FLOAT, "i32": m.ACL_INT32, None: None}
+    print(f"case int8 K-C M={M} K={K} N={N} tB={tB} out={out_dt} bias={bias_dt}", flush=True)
+    got, want, _ = cases.run_qmm_int8_case(m, orc, M, K, N, seed=M * 31 + N, out_dtype=dt[out_dt], bias_dtype=dt[bias_dt],
+                                           transpose_x2=tB)
+    _check_equal(got, want, "aclnnQuantMatmulV5 K-C")
+
+
+def test_kt_and_bf16_scale(gpu):
+    """K-T (one x2 scale) and a bf16 per-channel scale."""
+    m = gpu
+    for s2_len, s2_dt in [(1, m.ACL_FLOAT), (None, m.ACL_BF16)]:
+        print(f"case int8 x2s_len={s2_len} dtype={s2_dt}", flush=True)
+        got, want, _ = cases.run_qmm_int8_case(m, orc, 160, 320, 272, seed=5, out_dtype=m.ACL_BF16, bias_dtype=m.ACL_BF16,
+                                               transpose_x2=True, x2s_len=s2_len, x2s_dtype=s2_dt)
+        _check_equal(got, want, "K-T / bf16 scale")
+
+
+def test_transposed_view_equals_flag(gpu):
+    """x2 given as a strided (1, K) view with transposeX2 = false must equal transposeX2 = true on [N, K]."""
+    m = gpu
+    M, K, N = 128, 256, 192
+    inp = cases.make_qmm_int8_inputs(m, M, K, N, 3, m.ACL_BF16, True)
+    a = cases.run_qmm_int8_aclnn(m, inp, M, K, N, True, m.ACL_BF16)
+    b = cases.run_qmm_int8_aclnn(m, inp, M, K, N, True, m.ACL_BF16, x2_as_view=True)
+    want, _ = cases.oracle_qmm_int8(m, inp, M, K, N, True, m.ACL_BF16)
+    _check_equal(a, want, "flag form")
+    _check_equal(b, want, "view form")
+
+
+def test_batched(gpu):
+    m = gpu
+    print("case int8 batched", flush=True)
+    got, want, _ = cases.run_qmm_int8_case(m, orc, 130, 256, 140, seed=9, out_dtype=m.ACL_BF16, bias_dtype=m.ACL_FLOAT,
+                                           transpose_x2=True, batch=3)
+    _check_equal(got, want, "batched K-C")
+
+
+@pytest.mark.parametrize("variant", [1, 2, 3])
+def test_every_kernel_variant_and_int32_accumulators(gpu, variant):
+    """Each kernel variant (1 plain, 2 MFMA 256x256, 3 MFMA 128x128) through the thin launcher ABI.
+    With unit scales and no bias the fp32 epilogue is the identity on |acc| < 2^24, which exposes the raw
+    int32 accumulators: K = 512 keeps |acc| <= 512*127*127 < 2^24."""
+    m = gpu
+    M, K, N = 384, 512, 640
+    rng = np.random.default_rng(variant)
+    inp = dict(x1=cases.gen_int8(rng, (1, M, K)), x2=cases.gen_int8(rng, (1, N, K)), s1=np.ones(M, np.float32),
+               s2=np.ones(N, np.float32))
+    acc = orc.qmm_int8_acc(inp["x1"][0], inp["x2"][0], M, K, N, False, True)
+    d = {k: m.DeviceBuffer(host=v) for k, v in inp.items()}
+    out = m.DeviceBuffer(M * N * 2)
+    a = cases.qmm_args_int8(m, d, M, K, N, 1, True, out.ptr, m.ACL_FLOAT16, m.ACL_FLOAT, N, None, variant=variant)
+    print(f"case int8 variant {variant}", flush=True)
+    rc = m.lib().opsnnQmmInt8(C.byref(a), None)
+    assert rc == 0, rc
+    m.check(m.lib().aclrtSynchronizeDevice(), "sync")
+    got = orc.f16_to_f32(out.to_host(np.uint16, (M, N)))
+    # fp16 holds integers exactly only up to 2048; compare through the same rounding instead
+    want = orc.f16_to_f32(orc.f32_to_f16(acc.astype(np.float32)))
+    _check_equal(got.view(np.uint32), want.view(np.uint32), f"variant {variant}")
+    # and exactly, on the int32 output of the plain kernel
+    if variant == 1:
+        out32 = m.DeviceBuffer(M * N * 4)
+        a = cases.qmm_args_int8(m, d, M, K, N, 1, True, out32.ptr, m.ACL_INT32, m.ACL_FLOAT, N, None, variant=1)
+        assert m.lib().opsnnQmmInt8(C.byref(a), None) == 0
+        m.check(m.lib().aclrtSynchronizeDevice(), "sync")
+        _check_equal(out32.to_host(np.int32, (M, N)), acc, "int32 accumulators")
+
+
+def test_config2_full_size_on_sampled_rows(gpu):
+    """BASELINE config 2 at full size (M=2048, K=4096, N=11008, bf16 bias/out): every output row the oracle is
+    asked for (a seeded sample of 48 rows, first and last included) must be bit-identical."""
+    m = gpu
+    M, K, N = 2048, 4096, 11008
+    inp = cases.make_qmm_int8_inputs(m, M, K, N, 0, m.ACL_BF16, True)
+    print("case int8 config 2 full size", flush=True)
+    got = cases.run_qmm_int8_aclnn(m, inp, M, K, N, True, m.ACL_BF16)
+    rows = np.unique(np.concatenate([[0, M - 1, 255, 256], np.random.default_rng(1).integers(0, M, 44)]))
+    want, _ = cases.oracle_qmm_int8(m, inp, M, K, N, True, m.ACL_BF16, rows=rows)
+    _check_equal(got[0][rows], want[0], "config 2 sampled rows")
+    # size-independent property: the result is linear in x1Scale -- doubling a row's scale doubles that row exactly
+    inp2 = dict(inp)
+    inp2["s1"] = inp["s1"] * np.float32(2.0)
+    inp2["bias"] = None
+    inp2["bias_dtype"] = None
+    inp1 = dict(inp, bias=None, bias_dtype=None)
+    y1 = orc.bf16_to_f32(cases.run_qmm_int8_aclnn(m, inp1, M, K, N, True, m.ACL_BF16))
+    y2 = orc.bf16_to_f32(cases.run_qmm_int8_aclnn(m, inp2, M, K, N, True, m.ACL_BF16))
+    assert np.array_equal(y2, y1 * 2.0)
