@@ -294,6 +294,8 @@ static int launch_mfma(const QmmI8Params& p, int64_t batch, hipStream_t st)
 
 using namespace opsnn;
 
+extern "C" bool opsnn_force_plain();
+
 extern "C" int opsnnQmmInt8(const OpsnnQmmArgs* a, void* stream)
 {
     if (!a || !a->x1.ptr || !a->x2.ptr || !a->out || !a->x2_scale) return -1;
@@ -312,6 +314,7 @@ extern "C" int opsnnQmmInt8(const OpsnnQmmArgs* a, void* stream)
     bool a_kmajor = (p.a_cs == 1);
     bool b16 = (p.out_dt == DT_BF16 || p.out_dt == DT_F16);
     int variant = a->force_variant;
+    if (opsnn_force_plain()) variant = OPSNN_VARIANT_PLAIN;
     bool want_fast = b16 && a_kmajor && variant != OPSNN_VARIANT_PLAIN && p.M * p.N >= 64 * 64 && (p.K % 16) == 0 &&
                      (p.a_rs % 16) == 0 && ((uintptr_t)p.a % 16) == 0 && (p.a_bs % 16) == 0;
     if (want_fast && !b_kmajor && p.b_cs == 1 && a->workspace && p.b_rs == p.N && (p.b_bs == 0 || p.b_bs == p.K * p.N)) {

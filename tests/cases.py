@@ -120,3 +120,161 @@ def qmm_args_int8(m, d, M, K, N, batch, transpose_x2, out_ptr, out_dtype, s2_dty
     a.force_variant = variant
     a.workspace = ws.ptr if ws is not None else None
     return a
+
+
+# --------------------------------------------------------------------------------------------------
+# fp8 block scale (G-B / B-B)
+# --------------------------------------------------------------------------------------------------
+def gen_fp8(rng, shape):
+    v = np.clip(rng.normal(0.0, 1.0, size=shape), -448.0, 448.0).astype(np.float32)
+    return orc.f32_to_e4m3(v)
+
+
+def make_blockscale_inputs(m, M, K, N, seed, tB, gsM=1, batch=1):
+    rng = np.random.default_rng(seed)
+    KB, NB, MB = -(-K // 128), -(-N // 128), -(-M // gsM)
+    x1 = gen_fp8(rng, (batch, M, K))
+    x2 = gen_fp8(rng, (batch, N, K) if tB else (batch, K, N))
+    s1 = gen_scale(rng, batch * MB * KB).reshape(batch, MB, KB)
+    s2 = gen_scale(rng, batch * KB * NB).reshape((batch, NB, KB) if tB else (batch, KB, NB))
+    return dict(x1=x1, x2=x2, s1=s1, s2=s2, gsM=gsM)
+
+
+def oracle_blockscale(m, inp, M, K, N, tB, out_dtype, rows=None):
+    outs = []
+    gsM = inp["gsM"]
+    for b in range(inp["x1"].shape[0]):
+        x1, s1 = inp["x1"][b], inp["s1"][b]
+        Mr = M
+        if rows is not None:
+            assert gsM == 1
+            x1, s1, Mr = np.ascontiguousarray(x1[rows]), np.ascontiguousarray(s1[rows]), len(rows)
+        outs.append(orc.qmm_perblock(x1, inp["x2"][b], orc.E4M3, orc.E4M3, Mr, K, N, False, tB, s1,
+                                     np.ascontiguousarray(inp["s2"][b]), gsM, 128, 128, None, out_dtype))
+    return np.stack(outs)
+
+
+def run_blockscale_aclnn(m, inp, M, K, N, tB, out_dtype, group_size=None):
+    batch = inp["x1"].shape[0]
+    bshape = (batch,) if batch > 1 else ()
+    d = {k: m.DeviceBuffer(host=v) for k, v in inp.items() if isinstance(v, np.ndarray)}
+    out_np = orc.out_array((batch, M, N), out_dtype)
+    d_out = m.DeviceBuffer(out_np.nbytes)
+    d_out.fill(0xFF)
+    x1 = m.Tensor(bshape + (M, K), m.ACL_FLOAT8_E4M3FN, d["x1"])
+    x2 = m.Tensor(bshape + ((N, K) if tB else (K, N)), m.ACL_FLOAT8_E4M3FN, d["x2"])
+    s1 = m.Tensor(bshape + inp["s1"].shape[1:], m.ACL_FLOAT, d["s1"])
+    s2 = m.Tensor(bshape + inp["s2"].shape[1:], m.ACL_FLOAT, d["s2"])
+    out = m.Tensor(bshape + (M, N), out_dtype, d_out)
+    gs = (inp["gsM"] << 32) | (128 << 16) | 128 if group_size is None else group_size
+    ws = m.quant_matmul_v5(x1, x2, s1, s2, out, transpose_x2=tB, group_size=gs)
+    m.check(m.lib().aclrtSynchronizeDevice(), "sync")
+    del ws
+    return d_out.to_host(out_np.dtype, out_np.shape)
+
+
+# --------------------------------------------------------------------------------------------------
+# MX (fp4 / fp8 with e8m0 scales per 32 K)
+# --------------------------------------------------------------------------------------------------
+def make_mx_inputs(m, M, K, N, seed, tB, fp4=True, batch=1, exp_range=4):
+    rng = np.random.default_rng(seed)
+    KS = -(-K // 64)
+    if fp4:
+        c1 = rng.integers(0, 16, size=(batch, M, K), dtype=np.uint8)
+        c2 = rng.integers(0, 16, size=(batch, N, K) if tB else (batch, K, N), dtype=np.uint8)
+        x1, x2 = orc.pack_nibbles(c1), orc.pack_nibbles(c2)
+    else:
+        x1 = gen_fp8(rng, (batch, M, K))
+        x2 = gen_fp8(rng, (batch, N, K) if tB else (batch, K, N))
+    s1 = (127 + rng.integers(-exp_range, exp_range + 1, size=(batch, M, KS, 2))).astype(np.uint8)
+    s2 = (127 + rng.integers(-exp_range, exp_range + 1, size=(batch, N, KS, 2) if tB else (batch, KS, N, 2))).astype(np.uint8)
+    return dict(x1=x1, x2=x2, s1=s1, s2=s2, fp4=fp4)
+
+
+def oracle_mx(m, inp, M, K, N, tB, out_dtype, bias=None, rows=None):
+    dt = orc.E2M1 if inp["fp4"] else orc.E4M3
+    outs = []
+    for b in range(inp["x1"].shape[0]):
+        x1, s1, Mr = inp["x1"][b], inp["s1"][b], M
+        if rows is not None:
+            x1, s1, Mr = np.ascontiguousarray(x1[rows]), np.ascontiguousarray(s1[rows]), len(rows)
+        outs.append(orc.qmm_mx(x1, inp["x2"][b], dt, dt, Mr, K, N, False, tB, s1, np.ascontiguousarray(inp["s2"][b]), bias, out_dtype))
+    return np.stack(outs)
+
+
+def run_mx_aclnn(m, inp, M, K, N, tB, out_dtype, bias=None):
+    batch = inp["x1"].shape[0]
+    bshape = (batch,) if batch > 1 else ()
+    adt = m.ACL_FLOAT4_E2M1 if inp["fp4"] else m.ACL_FLOAT8_E4M3FN
+    d = {k: m.DeviceBuffer(host=v) for k, v in inp.items() if isinstance(v, np.ndarray)}
+    out_np = orc.out_array((batch, M, N), out_dtype)
+    d_out = m.DeviceBuffer(out_np.nbytes)
+    d_out.fill(0xFF)
+    x1 = m.Tensor(bshape + (M, K), adt, d["x1"])
+    x2 = m.Tensor(bshape + ((N, K) if tB else (K, N)), adt, d["x2"])
+    s1 = m.Tensor(bshape + inp["s1"].shape[1:], m.ACL_FLOAT8_E8M0, d["s1"])
+    s2 = m.Tensor(bshape + inp["s2"].shape[1:], m.ACL_FLOAT8_E8M0, d["s2"])
+    out = m.Tensor(bshape + (M, N), out_dtype, d_out)
+    d_bias = m.DeviceBuffer(host=bias) if bias is not None else None
+    t_bias = m.Tensor((N,), m.ACL_FLOAT, d_bias) if bias is not None else None
+    ws = m.quant_matmul_v5(x1, x2, s1, s2, out, bias=t_bias, transpose_x2=tB, group_size=(1 << 32) | (1 << 16) | 32)
+    m.check(m.lib().aclrtSynchronizeDevice(), "sync")
+    del ws
+    return d_out.to_host(out_np.dtype, out_np.shape)
+
+
+# --------------------------------------------------------------------------------------------------
+# weight-only (aclnnWeightQuantBatchMatmulV2)
+# --------------------------------------------------------------------------------------------------
+def make_wq_inputs(m, M, K, N, seed, x_dt, w_dt, group, tW, with_offset=True, bias_dt=None, scale_lo=0.005, scale_hi=0.02,
+                   per_tensor=False):
+    """x ~N(0,1) in x_dt; weight int8 [-127,127] or int4 [-8,7]; scale U(lo,hi), offset U(-1,1) in x_dt."""
+    rng = np.random.default_rng(seed)
+    x = orc.f32_to_b16(rng.normal(0, 1, size=(M, K)).astype(np.float32), x_dt)
+    wshape = (N, K) if tW else (K, N)
+    if w_dt == m.ACL_INT8:
+        w = rng.integers(-127, 128, size=wshape, dtype=np.int8)
+    elif w_dt == m.ACL_INT4:
+        w = orc.pack_nibbles((rng.integers(-8, 8, size=wshape) & 15).astype(np.uint8))
+    elif w_dt == m.ACL_FLOAT8_E4M3FN:
+        w = gen_fp8(rng, wshape)
+    else:
+        raise ValueError(w_dt)
+    G = -(-K // group) if group > 0 else 1
+    sshape = (1,) if per_tensor else ((N, G) if tW else (G, N))
+    scale = orc.f32_to_b16(rng.uniform(scale_lo, scale_hi, size=sshape).astype(np.float32), x_dt)
+    offset = orc.f32_to_b16(rng.uniform(-1, 1, size=sshape).astype(np.float32), x_dt) if with_offset else None
+    bias = gen_bias(rng, N, bias_dt, m)
+    return dict(x=x, w=w, scale=scale, offset=offset, bias=bias, bias_dt=bias_dt, x_dt=x_dt, w_dt=w_dt, group=group, tW=tW,
+                per_tensor=per_tensor)
+
+
+def oracle_wq(m, inp, M, K, N, rows=None):
+    x = inp["x"] if rows is None else np.ascontiguousarray(inp["x"][rows])
+    return orc.wqbmm(x, inp["x_dt"], inp["w"], inp["w_dt"], x.shape[0], K, N, inp["tW"], inp["scale"], inp["x_dt"],
+                     1 if inp["per_tensor"] else N, inp["offset"], inp["group"], inp["bias"], inp["bias_dt"] or 0)
+
+
+def run_wq_aclnn(m, inp, M, K, N, v3=False, scale_2d=None):
+    d = {k: m.DeviceBuffer(host=v) for k, v in inp.items() if isinstance(v, np.ndarray)}
+    d_y = m.DeviceBuffer(M * N * 2)
+    d_y.fill(0xFF)
+    tW, group = inp["tW"], inp["group"]
+    G = -(-K // group) if group > 0 else 1
+    x = m.Tensor((M, K), inp["x_dt"], d["x"])
+    # the weight view is always the logical [K, N]; [N, K] storage is expressed through strides (1, K)
+    w = m.Tensor((K, N), inp["w_dt"], d["w"], strides=(1, K) if tW else None)
+    if inp["per_tensor"]:
+        sshape, sst = (1,), None
+    elif group > 0 or scale_2d:
+        sshape, sst = (G, N), ((1, G) if tW else None)
+    else:
+        sshape, sst = (N,), None
+    sc = m.Tensor(sshape, inp["x_dt"], d["scale"], strides=sst)
+    off = m.Tensor(sshape, inp["x_dt"], d["offset"], strides=sst) if inp["offset"] is not None else None
+    bias = m.Tensor((N,), inp["bias_dt"], d["bias"]) if inp["bias"] is not None else None
+    y = m.Tensor((M, N), inp["x_dt"], d_y)
+    ws = m.weight_quant_batch_matmul(x, w, sc, y, offset=off, bias=bias, group_size=group, inner_precise=0 if v3 else None)
+    m.check(m.lib().aclrtSynchronizeDevice(), "sync")
+    del ws
+    return d_y.to_host(np.uint16, (M, N))

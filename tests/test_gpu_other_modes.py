@@ -1,0 +1,128 @@
+"""GPU parity for the fp8 block-scale, MX and weight-only paths.
+
+Two bars.  (1) The plain kernels evaluate the golden formulas operation by operation in ascending-k order, as
+the oracle does, so they must match it bit for bit.  (2) The MFMA kernels accumulate in another order (as the
+reference hardware and BLAS do); for them the bar is the one BASELINE states: max relative error <= 2^-7 and
+mean relative error <= 2^-10 against the fp32-accumulated oracle (denominator floored at 1 % of the mean
+magnitude), plus the reference's own acceptance rule (>= 99.9 % of elements within rtol = atol = 1e-3).
+"""
+import os
+
+import numpy as np
+import pytest
+
+import cases
+import oracle_api as orc
+
+pytestmark = pytest.mark.gpu
+
+MAX_REL, MEAN_REL = 2.0 ** -7, 2.0 ** -10
+
+
+def check_close(got_bits, want_bits, dt, what, exact=False):
+    if exact:
+        if not np.array_equal(got_bits, want_bits):
+            bad = np.argwhere(got_bits != want_bits)
+            raise AssertionError(f"{what}: {len(bad)} of {got_bits.size} differ, first at {bad[0]}")
+        return
+    got, want = orc.b16_to_f32(got_bits, dt), orc.b16_to_f32(want_bits, dt)
+    assert np.isfinite(got).all(), f"{what}: non-finite output"
+    mx, mean = orc.rel_err_stats(got, want)
+    frac = orc.isclose_fraction(got, want)
+    assert mx <= MAX_REL and mean <= MEAN_REL, f"{what}: max rel {mx:.3e} mean rel {mean:.3e}"
+    assert frac <= 1e-3, f"{what}: {frac:.2e} of elements outside rtol=atol=1e-3"
+
+
+def plain(flag):
+    """Route through the plain kernels (set) or let the selector choose (unset)."""
+    if flag:
+        os.environ["OPSNN_FORCE_PLAIN"] = "1"
+    else:
+        os.environ.pop("OPSNN_FORCE_PLAIN", None)
+
+
+@pytest.fixture(autouse=True)
+def _reset_env():
+    yield
+    os.environ.pop("OPSNN_FORCE_PLAIN", None)
+
+
+@pytest.mark.parametrize("use_plain", [True, False])
+@pytest.mark.parametrize("M,K,N,tB,gsM", [
+    (128, 512, 256, True, 1), (128, 512, 256, False, 1), (100, 300, 200, True, 1), (256, 384, 384, True, 128),
+    (130, 256, 130, False, 128), (1, 1024, 256, True, 1),
+])
+def test_fp8_blockscale(gpu, M, K, N, tB, gsM, use_plain):
+    m = gpu
+    print(f"case fp8 block M={M} K={K} N={N} tB={tB} gsM={gsM} plain={use_plain}", flush=True)
+    inp = cases.make_blockscale_inputs(m, M, K, N, M + N, tB, gsM)
+    want = cases.oracle_blockscale(m, inp, M, K, N, tB, m.ACL_BF16)
+    plain(use_plain)
+    got = cases.run_blockscale_aclnn(m, inp, M, K, N, tB, m.ACL_BF16)
+    check_close(got, want, orc.BF16, "fp8 block scale", exact=use_plain)
+
+
+def test_fp8_blockscale_group_size_inferred(gpu):
+    """groupSize 0 is inferred from the scale shapes (quant_matmul_checker.cpp:700-722)."""
+    m = gpu
+    inp = cases.make_blockscale_inputs(m, 128, 256, 256, 1, True, 1)
+    a = cases.run_blockscale_aclnn(m, inp, 128, 256, 256, True, m.ACL_BF16)
+    b = cases.run_blockscale_aclnn(m, inp, 128, 256, 256, True, m.ACL_BF16, group_size=0)
+    assert np.array_equal(a, b)
+
+
+@pytest.mark.parametrize("use_plain", [True, False])
+@pytest.mark.parametrize("M,K,N,tB,fp4", [
+    (128, 256, 256, True, True), (128, 256, 256, False, True), (197, 960, 854, True, True), (64, 128, 64, True, False),
+    (64, 320, 96, False, False), (33, 192, 50, True, True),
+])
+def test_mx(gpu, M, K, N, tB, fp4, use_plain):
+    m = gpu
+    print(f"case mx M={M} K={K} N={N} tB={tB} fp4={fp4} plain={use_plain}", flush=True)
+    inp = cases.make_mx_inputs(m, M, K, N, K + N, tB, fp4)
+    bias = np.random.default_rng(1).normal(0, 1, N).astype(np.float32)
+    want = cases.oracle_mx(m, inp, M, K, N, tB, m.ACL_BF16, bias)
+    plain(use_plain)
+    got = cases.run_mx_aclnn(m, inp, M, K, N, tB, m.ACL_BF16, bias)
+    check_close(got, want, orc.BF16, "mx", exact=use_plain)
+
+
+def test_mx_batched(gpu):
+    m = gpu
+    inp = cases.make_mx_inputs(m, 96, 256, 128, 4, True, True, batch=3)
+    want = cases.oracle_mx(m, inp, 96, 256, 128, True, m.ACL_BF16)
+    got = cases.run_mx_aclnn(m, inp, 96, 256, 128, True, m.ACL_BF16)
+    check_close(got, want, orc.BF16, "mx batched")
+
+
+@pytest.mark.parametrize("use_plain", [True, False])
+@pytest.mark.parametrize("M,K,N,x_dt,w_dt,group,tW,off,bias", [
+    (16, 512, 256, "bf16", "i8", 0, False, False, None),      # config 1 shape class
+    (16, 512, 256, "bf16", "i8", 0, True, True, "f32"),
+    (1, 1024, 512, "f16", "i4", 128, False, True, None),       # config 3 shape class
+    (16, 1024, 512, "f16", "i4", 128, True, True, "f16"),
+    (64, 512, 384, "f16", "i4", 128, True, True, None),
+    (256, 512, 256, "f16", "i4", 128, False, True, None),
+    (7, 320, 130, "bf16", "i4", 64, False, True, "bf16"),
+    (5, 256, 64, "f16", "i8", 32, True, False, None),
+    (33, 864, 212, "f16", "i4", 96, False, True, None),         # ragged groups (864 = 9 * 96)
+    (4, 256, 128, "bf16", "e4m3", 0, True, False, "bf16"),
+])
+def test_weight_only(gpu, M, K, N, x_dt, w_dt, group, tW, off, bias, use_plain):
+    m = gpu
+    dt = {"bf16": m.ACL_BF16, "f16": m.ACL_FLOAT16, "f32": m.ACL_FLOAT, "i8": m.ACL_INT8, "i4": m.ACL_INT4,
+          "e4m3": m.ACL_FLOAT8_E4M3FN, None: None}
+    print(f"case wq M={M} K={K} N={N} x={x_dt} w={w_dt} g={group} tW={tW} off={off} bias={bias} plain={use_plain}", flush=True)
+    inp = cases.make_wq_inputs(m, M, K, N, M * 7 + N, dt[x_dt], dt[w_dt], group, tW, off, dt[bias])
+    want = cases.oracle_wq(m, inp, M, K, N)
+    plain(use_plain)
+    got = cases.run_wq_aclnn(m, inp, M, K, N)
+    check_close(got, want, dt[x_dt], "weight-only", exact=use_plain)
+
+
+def test_weight_only_v3_and_per_tensor(gpu):
+    m = gpu
+    inp = cases.make_wq_inputs(m, 8, 256, 128, 2, m.ACL_FLOAT16, m.ACL_INT8, 0, False, True, None, per_tensor=True)
+    want = cases.oracle_wq(m, inp, 8, 256, 128)
+    got = cases.run_wq_aclnn(m, inp, 8, 256, 128, v3=True)
+    check_close(got, want, orc.F16, "per-tensor V3")
