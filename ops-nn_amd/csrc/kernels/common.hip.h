@@ -48,6 +48,27 @@ __device__ __forceinline__ uint16_t to_b16(float f)
     else return f16_bits(f);
 }
 
+// Four fp32 values -> four 16-bit floats (round to nearest even) using the packed hardware conversions.
+typedef __bf16 v2bf __attribute__((ext_vector_type(2)));
+typedef float v2f __attribute__((ext_vector_type(2)));
+template <int DT>
+__device__ __forceinline__ v4us pack4_b16(v4f v)
+{
+    if constexpr (DT == DT_BF16) {
+        v2f lo = {v[0], v[1]}, hi = {v[2], v[3]};
+        v2bf a = __builtin_convertvector(lo, v2bf), b = __builtin_convertvector(hi, v2bf);   // v_cvt_pk_bf16_f32
+        uint32_t ua = __builtin_bit_cast(uint32_t, a), ub = __builtin_bit_cast(uint32_t, b);
+        v4us o = {(unsigned short)(ua & 0xffffu), (unsigned short)(ua >> 16), (unsigned short)(ub & 0xffffu), (unsigned short)(ub >> 16)};
+        return o;
+    } else {
+        v2f lo = {v[0], v[1]}, hi = {v[2], v[3]};
+        v2h a = __builtin_convertvector(lo, v2h), b = __builtin_convertvector(hi, v2h);
+        uint32_t ua = __builtin_bit_cast(uint32_t, a), ub = __builtin_bit_cast(uint32_t, b);
+        v4us o = {(unsigned short)(ua & 0xffffu), (unsigned short)(ua >> 16), (unsigned short)(ub & 0xffffu), (unsigned short)(ub >> 16)};
+        return o;
+    }
+}
+
 __device__ __forceinline__ float load_scalar_as_f32(const void* p, int dt, int64_t i)
 {
     switch (dt) {

@@ -9,4 +9,7 @@ enum {
     OPSNN_VARIANT_PLAIN = 1,      // strided one-thread-per-output kernels (any shape)
     OPSNN_VARIANT_I8_256 = 2,     // int8 MFMA, 256x256 tile
     OPSNN_VARIANT_I8_128 = 3,     // int8 MFMA, 128x128 tile
+    OPSNN_VARIANT_I8_256x128_S3 = 4,  // int8 MFMA, 256x128 tile, BK 64, 3 stages, 2 workgroups per CU
+    OPSNN_VARIANT_I8_256_W8 = 5,  // int8 MFMA, 256x256 tile, 8 waves, BK 64, 4 stages
+    OPSNN_VARIANT_I8_256_S4 = 6,  // int8 MFMA, 256x256 tile, 4 waves, BK 64, 4 stages
 };

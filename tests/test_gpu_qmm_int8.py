@@ -71,9 +71,10 @@ def test_batched(gpu):
     _check_equal(got, want, "batched K-C")
 
 
-@pytest.mark.parametrize("variant", [1, 2, 3])
+@pytest.mark.parametrize("variant", [1, 2, 3, 4, 5, 6])
 def test_every_kernel_variant_and_int32_accumulators(gpu, variant):
-    """Each kernel variant (1 plain, 2 MFMA 256x256, 3 MFMA 128x128) through the thin launcher ABI.
+    """Each kernel variant (1 plain, 2 MFMA 256x256, 3 MFMA 128x128,
+    4 MFMA 256x128 three-stage, 5 MFMA 256x256 eight-wave) through the thin launcher ABI.
     With unit scales and no bias the fp32 epilogue is the identity on |acc| < 2^24, which exposes the raw
     int32 accumulators: K = 512 keeps |acc| <= 512*127*127 < 2^24."""
     m = gpu
