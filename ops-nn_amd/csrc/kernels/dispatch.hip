@@ -14,6 +14,7 @@ int launch_wqmm_plain(const OpsnnWqmmArgs& a, hipStream_t st);
 int launch_blockscale_mfma(const OpsnnQmmArgs& a, hipStream_t st);
 int launch_mx_mfma(const OpsnnQmmArgs& a, hipStream_t st);
 int launch_wqmm_mfma(const OpsnnWqmmArgs& a, hipStream_t st);
+uint64_t mx_workspace_bytes(const OpsnnQmmArgs& a);
 }  // namespace opsnn
 
 using namespace opsnn;
@@ -69,8 +70,8 @@ extern "C" int opsnnWqmm(const OpsnnWqmmArgs* a, void* stream)
 // transposed view) need no workspace and skip that pass.
 extern "C" uint64_t opsnnQmmWorkspace(const OpsnnQmmArgs* a, int mode)
 {
-    (void)mode;
     if (!a) return 0;
+    if (mode == 2) return mx_workspace_bytes(*a);
     if (a->x2.row_stride == 1 || a->K == 1) return 0;           // already K-contiguous
     if (a->x2.col_stride != 1 || a->x2.row_stride != a->N) return 0;  // not a dense [K, N]: plain kernel
     uint64_t bits = (a->x2_dtype == DT_I4 || a->x2_dtype == DT_E2M1) ? 4 : 8;

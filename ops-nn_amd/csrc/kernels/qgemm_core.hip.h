@@ -1,0 +1,446 @@
+// Shared tile-GEMM core for the 8-bit / 4-bit quantized matmuls on gfx950.
+//
+// One kernel template, specialised by MODE:
+//   MODE_I8     int8 x int8 -> int32 (v_mfma_i32_32x32x32_i8), per-token / per-channel dequant epilogue
+//   MODE_MXFP4  fp4 e2m1 x fp4 e2m1 with e8m0 scales per 32 K (v_mfma_scale_f32_32x32x64_f8f6f4), bias epilogue
+//   MODE_MXFP8  fp8 e4m3 x fp8 e4m3 with e8m0 scales per 32 K (same instruction, 8-bit formats)
+// Both operands are K-contiguous ("x2 stored [N, K]") with 16-byte aligned rows.  Everything is addressed in
+// BYTES of the packed operand rows, so int8 and fp4 share all data movement (32 bytes of K per row per MFMA)
+// and fp8 uses 64.
+//
+//   - BM x BN output tile per workgroup, WGM x WGN waves, each wave owns a (BM/WGM) x (BN/WGN) sub-tile of
+//     32x32 MFMA fragments with accumulators held in registers for the whole K loop;
+//   - K tiles of BK bytes are copied global -> LDS asynchronously (16 B per lane, no register round trip),
+//     STAGES deep; MX scale bytes ride along as 4-byte async copies;
+//   - LDS rows are XOR-swizzled in 16-byte chunks so the MFMA operand reads are bank-conflict free;
+//   - the MFMA is issued as x2-fragment x x1-fragment so every lane ends up with four consecutive n of one
+//     output row: epilogue vectors load as float4 and the 16-bit results leave as 8-byte stores.
+#pragma once
+#include <type_traits>
+
+#include "common.hip.h"
+
+namespace opsnn {
+
+enum : int { MODE_I8 = 0, MODE_MXFP4 = 1, MODE_MXFP8 = 2 };
+
+struct QgemmParams {
+    const int8_t* a;   // x1 rows, K-contiguous
+    const int8_t* b;   // x2 rows (one per n), K-contiguous
+    int64_t lda, ldb;  // row strides in bytes
+    int64_t a_bs, b_bs;  // batch strides in bytes (0 = broadcast)
+    void* out;         // [batch, M, N] dense, 16-bit floats
+    int64_t M, N, KB;  // KB = bytes of K per operand row
+    // MODE_I8 epilogue: out = cast(fp32(acc + ib[n]) * x2s[n] * x1s[m] + fb[n])
+    const float* x1s;
+    const void* x2s;
+    int x2s_dt;
+    int64_t x2s_len;
+    // bias: int32 / 16-bit / fp32 for MODE_I8, fp32 for the MX modes
+    const void* bias;
+    int bias_dt;
+    int64_t bias_bs;
+    // MX: one e8m0 byte per 32 K elements, K-contiguous per row
+    const uint8_t* sa;
+    const uint8_t* sb;
+    int64_t sa_rs, sb_rs, sa_bs, sb_bs;
+};
+
+__device__ __attribute__((aligned(16))) static const int8_t g_zero16[16] = {0};
+
+// s_waitcnt with only the vector-memory counter constrained (gfx9 encoding: vmcnt = imm[3:0] | imm[15:14] << 4).
+template <int N>
+__device__ __forceinline__ void wait_vmcnt()
+{
+    static_assert(N >= 0 && N < 64, "vmcnt range");
+    __builtin_amdgcn_s_waitcnt((N & 15) | (((N >> 4) & 3) << 14) | (7 << 4) | (15 << 8));
+}
+__device__ __forceinline__ void wait_lgkmcnt0() { __builtin_amdgcn_s_waitcnt(15 | (3 << 14) | (7 << 4) | (0 << 8)); }
+
+// 4-byte asynchronous copy global -> LDS; lane l lands at lds + 4*l.
+__device__ __forceinline__ void async_copy4(const void* g, void* lds)
+{
+    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)g,
+                                     (__attribute__((address_space(3))) void*)lds, 4, 0, 0);
+}
+
+template <int MODE, int BM, int BN, int BK, int WGM, int WGN, int STAGES, int MINWG, bool KTAIL, int OUT_DT>
+__global__ __launch_bounds__(WGM* WGN * 64, MINWG) void qgemm_kernel(QgemmParams p, int tiles_m, int tiles_n)
+{
+    constexpr bool MX = MODE != MODE_I8;
+    constexpr int NT = WGM * WGN * 64;
+    constexpr int CPR = BK / 16;                 // 16-byte chunks per LDS row
+    constexpr int RPW = 16 / CPR;                // rows per 256-byte LDS bank wrap
+    constexpr int TM = BM / WGM, TN = BN / WGN;  // per-wave tile
+    constexpr int FM = TM / 32, FN = TN / 32;
+    constexpr int KSTEP = MODE == MODE_MXFP8 ? 64 : 32;  // bytes of K per row per MFMA
+    constexpr int FREG = KSTEP / 8;                      // operand dwords per lane per fragment
+    constexpr int KS = BK / KSTEP;                       // MFMA K steps per tile
+    constexpr int SCB = MX ? BK / (MODE == MODE_MXFP8 ? 32 : 16) : 0;  // scale bytes per row per tile
+    constexpr int A_BYTES = BM * BK, B_BYTES = BN * BK;
+    constexpr int SC_BYTES = MX ? (BM + BN) * 4 : 0;
+    constexpr int STAGE = A_BYTES + B_BYTES + SC_BYTES;
+    constexpr int RPI = NT / CPR;                // tile rows covered by one copy instruction of the workgroup
+    constexpr int NA = BM / RPI, NB = BN / RPI;  // copy instructions per thread per tile
+    constexpr int NSC = MX ? (BM + BN) / NT : 0; // scale-copy instructions per thread per tile
+    constexpr int CPT = NA + NB + NSC;
+    static_assert(CPR == 8 || CPR == 4, "BK must be 64 or 128");
+    static_assert(BM % RPI == 0 && BN % RPI == 0, "tile rows must be a multiple of the rows one copy pass covers");
+    static_assert(STAGES >= 2 && STAGES * CPT < 64, "stage count");
+    static_assert(KS % 2 == 0, "operand double buffer parity");
+    static_assert(!MX || SCB == 4, "MX tiles carry exactly four scale bytes per row");
+    static_assert(!MX || (BM + BN) % NT == 0, "scale copy mapping");
+    static_assert(!MX || !KTAIL, "MX fast path takes whole K tiles only");
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave / WGN, wn = wave % WGN;
+
+    // tile id: XCD-contiguous, m fastest so that one XCD works on few x2 panels at a time
+    const uint32_t t = xcd_remap(blockIdx.x, (uint32_t)(tiles_m * tiles_n));
+    const int tm = (int)(t % (uint32_t)tiles_m), tn = (int)(t / (uint32_t)tiles_m);
+    const int64_t m0 = (int64_t)tm * BM, n0 = (int64_t)tn * BN;
+    const int64_t bz = blockIdx.y;
+
+    const int64_t lda = p.lda, ldb = p.ldb;
+    const int8_t* A = p.a + bz * p.a_bs + m0 * lda;
+    const int8_t* B = p.b + bz * p.b_bs + n0 * ldb;
+    const int64_t K = p.KB;
+    const int KT = (int)((K + BK - 1) / BK);
+
+    // LDS layout of one operand tile: row r holds CPR chunks of 16 bytes; logical chunk c is stored at position
+    // c ^ key(r), key(r) = (r / RPW) % CPR, so that 16 consecutive rows at one logical chunk hit 16 different
+    // 16-byte bank groups.
+    // Async copies: copy instruction i of the workgroup fills LDS chunks [i*NT, (i+1)*NT), i.e. tile rows
+    // i*RPI .. i*RPI+RPI-1; this thread always handles row i*RPI + tid/CPR and the chunk computed below.
+    // Rows past the matrix edge are clamped to the last valid row: they only feed outputs that are never stored.
+    const int crow = tid / CPR;
+    const int cchunk = (tid % CPR) ^ ((crow / RPW) & (CPR - 1));  // RPI is a multiple of RPW*CPR: same key for every i
+    const int a_rows = (int)((p.M - m0) < BM ? (p.M - m0) : BM);
+    const int b_rows = (int)((p.N - n0) < BN ? (p.N - n0) : BN);
+    uint32_t a_off[NA], b_off[NB];
+#pragma unroll
+    for (int i = 0; i < NA; i++) {
+        int r = i * RPI + crow;
+        r = r < a_rows ? r : a_rows - 1;
+        a_off[i] = (uint32_t)(r * lda + cchunk * 16);
+    }
+#pragma unroll
+    for (int i = 0; i < NB; i++) {
+        int r = i * RPI + crow;
+        r = r < b_rows ? r : b_rows - 1;
+        b_off[i] = (uint32_t)(r * ldb + cchunk * 16);
+    }
+    const int8_t* const zero_page = g_zero16;
+    // MX scales: scale-copy instruction i covers rows i*NT .. i*NT+NT-1 of the stacked [x1 rows; x2 rows] of the
+    // tile; each lane copies the four scale bytes one row needs for a K tile.
+    const uint8_t* sc_src[NSC > 0 ? NSC : 1];
+    if constexpr (MX) {
+#pragma unroll
+        for (int i = 0; i < NSC; i++) {
+            int r = i * NT + tid;
+            if (r < BM) {
+                int rr = r < a_rows ? r : a_rows - 1;
+                sc_src[i] = p.sa + bz * p.sa_bs + (m0 + rr) * p.sa_rs;
+            } else {
+                int rr = r - BM;
+                rr = rr < b_rows ? rr : b_rows - 1;
+                sc_src[i] = p.sb + bz * p.sb_bs + (n0 + rr) * p.sb_rs;
+            }
+        }
+    }
+
+    auto issue_tile = [&](int kt) {
+        char* sA = smem + (kt % STAGES) * STAGE + wave * 1024;
+        char* sB = sA + A_BYTES;
+        const int64_t k0 = (int64_t)kt * BK;
+        const int8_t* Ak = A + k0;
+        const int8_t* Bk = B + k0;
+        const bool kok = !KTAIL || (k0 + cchunk * 16) < K;
+#pragma unroll
+        for (int i = 0; i < NA; i++) {
+            const int8_t* g = Ak + a_off[i];
+            if constexpr (KTAIL) g = kok ? g : zero_page;
+            async_copy16(g, sA + i * NT * 16);
+        }
+#pragma unroll
+        for (int i = 0; i < NB; i++) {
+            const int8_t* g = Bk + b_off[i];
+            if constexpr (KTAIL) g = kok ? g : zero_page;
+            async_copy16(g, sB + i * NT * 16);
+        }
+        if constexpr (MX) {
+            char* sS = smem + (kt % STAGES) * STAGE + A_BYTES + B_BYTES + wave * 256;
+#pragma unroll
+            for (int i = 0; i < NSC; i++) async_copy4(sc_src[i] + (int64_t)kt * SCB, sS + i * NT * 4);
+        }
+    };
+
+    using Acc = std::conditional_t<MODE == MODE_I8, v16i, v16f>;
+    Acc acc[FN][FM];
+#pragma unroll
+    for (int i = 0; i < FN; i++)
+#pragma unroll
+        for (int j = 0; j < FM; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[i][j][r] = 0;
+
+    // Operand fragments, lane (row = lane%32, half = lane/32):
+    //   32-byte K steps (int8, fp4): the lane's four operand dwords are bytes [16*half, 16*half+16) of the step;
+    //   64-byte K steps (fp8): dwords 0-3 are bytes [16*half, +16) and dwords 4-7 bytes [32+16*half, +16) -- the
+    //   8-bit form of the instruction consumes K in two 32-element blocks, dwords 0-3 of all lanes first.  The
+    //   lane's scale byte belongs to block `half`, whichever registers hold that block's data.
+    const int frow = lane & 31;
+    const int fkc = lane >> 5;
+    const int key = (frow / RPW) & (CPR - 1);  // 32-row fragments start at multiples of RPW*CPR rows
+    const int swz = fkc ^ key;                 // KSTEP 32: chunk 2s + half
+    const int swz0 = fkc ^ key;                // KSTEP 64: chunks 4s + half and 4s + 2 + half (see load_frags)
+    const int swz1 = (2 + fkc) ^ key;
+    const int a_rowbase = (wm * TM + frow) * BK;
+    const int b_rowbase = A_BYTES + (wn * TN + frow) * BK;
+
+    typedef int frag_t __attribute__((ext_vector_type(FREG)));
+    frag_t fa[2][FM], fb[2][FN];
+    uint32_t sca[FM], scb[FN];  // MX: this lane's four scale bytes of the current tile, shifted down by its K half
+    (void)swz; (void)swz0; (void)swz1; (void)sca; (void)scb;
+
+    auto load_frags = [&](int kt, int s, int buf) {
+        const char* st = smem + (kt % STAGES) * STAGE;
+        if constexpr (KSTEP == 32) {
+            const char* base = st + (((2 * s) ^ swz) << 4);
+#pragma unroll
+            for (int j = 0; j < FM; j++) fa[buf][j] = *(const frag_t*)(base + a_rowbase + j * 32 * BK);
+#pragma unroll
+            for (int i = 0; i < FN; i++) fb[buf][i] = *(const frag_t*)(base + b_rowbase + i * 32 * BK);
+        } else {
+            const char* b0 = st + (((4 * s) ^ swz0) << 4);
+            const char* b1 = st + (((4 * s) ^ swz1) << 4);
+#pragma unroll
+            for (int j = 0; j < FM; j++) {
+                const v4i lo = *(const v4i*)(b0 + a_rowbase + j * 32 * BK), hi = *(const v4i*)(b1 + a_rowbase + j * 32 * BK);
+                fa[buf][j] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+            }
+#pragma unroll
+            for (int i = 0; i < FN; i++) {
+                const v4i lo = *(const v4i*)(b0 + b_rowbase + i * 32 * BK), hi = *(const v4i*)(b1 + b_rowbase + i * 32 * BK);
+                fb[buf][i] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+            }
+        }
+    };
+    // MX: the four scale bytes of a row cover the tile's K blocks 0..3 (32 elements each).  MFMA step s of a lane
+    // in K half h multiplies block 2s + h, i.e. byte 2s of the dword once it is shifted right by 8h.
+    auto load_scales = [&](int kt) {
+        if constexpr (MX) {
+            const char* sS = smem + (kt % STAGES) * STAGE + A_BYTES + B_BYTES;
+#pragma unroll
+            for (int j = 0; j < FM; j++) sca[j] = *(const uint32_t*)(sS + (wm * TM + j * 32 + frow) * 4) >> (8 * fkc);
+#pragma unroll
+            for (int i = 0; i < FN; i++) scb[i] = *(const uint32_t*)(sS + (BM + wn * TN + i * 32 + frow) * 4) >> (8 * fkc);
+        }
+    };
+    auto mma = [&](int buf, auto sidx) {
+        constexpr int S = decltype(sidx)::value;
+        (void)S;
+#pragma unroll
+        for (int i = 0; i < FN; i++)
+#pragma unroll
+            for (int j = 0; j < FM; j++) {
+                if constexpr (MODE == MODE_I8) {
+                    acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fb[buf][i], fa[buf][j], acc[i][j], 0, 0, 0);
+                } else if constexpr (MODE == MODE_MXFP4) {
+                    const v4i z = {0, 0, 0, 0};  // fp4 operands occupy the first four of the eight operand dwords
+                    const v8i bb = __builtin_shufflevector(fb[buf][i], z, 0, 1, 2, 3, 4, 5, 6, 7);
+                    const v8i aa = __builtin_shufflevector(fa[buf][j], z, 0, 1, 2, 3, 4, 5, 6, 7);
+                    acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(bb, aa, acc[i][j], 4, 4, 2 * S, (int)scb[i], 2 * S, (int)sca[j]);
+                } else {
+                    acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb[buf][i], fa[buf][j], acc[i][j], 0, 0, 2 * S, (int)scb[i], 2 * S, (int)sca[j]);
+                }
+            }
+    };
+    auto interleave = [&](bool with_copies) {
+        // (FM+FN) groups of {MFMAs, one LDS read (+ one async copy)}: memory instructions issue in the MFMA shadow
+#pragma unroll
+        for (int g = 0; g < FM + FN; g++) {
+            __builtin_amdgcn_sched_group_barrier(0x008, (FM * FN) / (FM + FN), 0);
+            __builtin_amdgcn_sched_group_barrier(0x100, KSTEP / 32, 0);
+            if (with_copies && g < CPT) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+        }
+    };
+
+    // Pipeline.  All STAGES stages are kept in flight.  The loop is rotated so that its single barrier sits in
+    // front of the LAST K step of a tile: on entry to iteration kt the operands of K step 0 are already in
+    // registers; K steps 0..KS-2 multiply while the operands of the following step are read; then
+    //   wait for this thread's copies of tile kt+1, barrier (tile kt+1 is complete in LDS and every wave has
+    //   finished reading tile kt, whose last operands now sit in registers),
+    //   start the copy of tile kt+STAGES into the freed stage, read K step 0 of tile kt+1, multiply the last step.
+#pragma unroll
+    for (int i = 0; i < STAGES; i++)
+        if (i < KT) issue_tile(i);
+    if (KT >= STAGES) wait_vmcnt<(STAGES - 1) * CPT>();
+    else wait_vmcnt<0>();
+    __builtin_amdgcn_s_barrier();
+    load_frags(0, 0, 0);
+    load_scales(0);
+
+    auto k_tile = [&](int kt, auto issue, auto next) {
+        constexpr bool ISSUE = decltype(issue)::value, NEXT = decltype(next)::value;
+        uint32_t sca_n[FM], scb_n[FN];
+        (void)sca_n; (void)scb_n;
+        if constexpr (KS >= 4) {
+            load_frags(kt, 1, 1);
+            mma(0, std::integral_constant<int, 0>{});
+            interleave(false);
+            load_frags(kt, 2, 0);
+            mma(1, std::integral_constant<int, 1>{});
+            interleave(false);
+            load_frags(kt, 3, 1);
+            mma(0, std::integral_constant<int, 2>{});
+            interleave(false);
+        } else {
+            load_frags(kt, 1, 1);
+            mma(0, std::integral_constant<int, 0>{});
+            interleave(false);
+        }
+        if constexpr (NEXT) {
+            if constexpr (ISSUE) wait_vmcnt<(STAGES - 2) * CPT>();
+            else wait_vmcnt<0>();
+        }
+        wait_lgkmcnt0();  // this wave's reads of the stage about to be recycled have retired
+        __builtin_amdgcn_s_barrier();
+        if constexpr (ISSUE) issue_tile(kt + STAGES);
+        if constexpr (NEXT) {
+            load_frags(kt + 1, 0, 0);
+            if constexpr (MX) {  // next tile's scales go to a second set: the last MFMA step still uses this tile's
+                const char* sS = smem + ((kt + 1) % STAGES) * STAGE + A_BYTES + B_BYTES;
+#pragma unroll
+                for (int j = 0; j < FM; j++) sca_n[j] = *(const uint32_t*)(sS + (wm * TM + j * 32 + frow) * 4) >> (8 * fkc);
+#pragma unroll
+                for (int i = 0; i < FN; i++) scb_n[i] = *(const uint32_t*)(sS + (BM + wn * TN + i * 32 + frow) * 4) >> (8 * fkc);
+            }
+        }
+        mma(1, std::integral_constant<int, KS - 1>{});
+        if constexpr (NEXT) interleave(ISSUE);
+        if constexpr (NEXT && MX) {
+#pragma unroll
+            for (int j = 0; j < FM; j++) sca[j] = sca_n[j];
+#pragma unroll
+            for (int i = 0; i < FN; i++) scb[i] = scb_n[i];
+        }
+    };
+    using T = std::true_type;
+    using F = std::false_type;
+    int kt = 0;
+    for (; kt + STAGES < KT; kt++) k_tile(kt, T{}, T{});
+    for (; kt + 1 < KT; kt++) k_tile(kt, F{}, T{});
+    k_tile(kt, F{}, F{});
+    __syncthreads();  // all operand reads done before LDS is reused below
+
+    // Epilogue.  acc[i][j][r]: n = n_base + 8*(r/4) + 4*(lane/32) + r%4,  m = m_base + lane%32.
+    // Per-row and per-column terms are first widened to fp32 in LDS, so the unrolled part is branch-free:
+    // absent terms are the neutral elements 1.0f, 0 and -0.0f.
+    float* sS2 = (float*)smem;
+    float* sFb = sS2 + BN;
+    int32_t* sIb = (int32_t*)(sFb + BN);
+    float* sS1 = (float*)(sIb + BN);
+    {
+        const bool has_ib = MODE == MODE_I8 && p.bias && p.bias_dt == DT_I32;
+        const bool has_fb = p.bias && p.bias_dt != DT_I32;
+        for (int i = tid; i < BN; i += NT) {
+            int64_t n = n0 + i;
+            if (n >= p.N) n = p.N - 1;
+            if constexpr (MODE == MODE_I8) {
+                sS2[i] = load_scalar_as_f32(p.x2s, p.x2s_dt, p.x2s_len == 1 ? 0 : n);
+                sIb[i] = has_ib ? ((const int32_t*)p.bias)[bz * p.bias_bs + n] : 0;
+            }
+            sFb[i] = has_fb ? load_scalar_as_f32(p.bias, p.bias_dt, bz * p.bias_bs + n) : -0.0f;
+        }
+        if constexpr (MODE == MODE_I8) {
+            for (int i = tid; i < BM; i += NT) {
+                int64_t m = m0 + i;
+                if (m >= p.M) m = p.M - 1;
+                sS1[i] = p.x1s ? p.x1s[m] : 1.0f;
+            }
+        }
+    }
+    __syncthreads();
+    uint16_t* out = (uint16_t*)p.out + bz * p.M * p.N;
+    const bool vec_ok = (p.N % 4) == 0;
+#pragma unroll
+    for (int j = 0; j < FM; j++) {
+        const int ml = wm * TM + j * 32 + frow;
+        const int64_t m = m0 + ml;
+        float s1 = 1.0f;
+        if constexpr (MODE == MODE_I8) s1 = sS1[ml];
+#pragma unroll
+        for (int i = 0; i < FN; i++) {
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+                const int nl = wn * TN + i * 32 + 8 * q + 4 * fkc;
+                const int64_t n = n0 + nl;
+                const v4f fbv = *(const v4f*)(sFb + nl);
+                v4f v;
+                if constexpr (MODE == MODE_I8) {
+                    const v4f s2 = *(const v4f*)(sS2 + nl);
+                    const v4i ib = *(const v4i*)(sIb + nl);
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        float tv = (float)(acc[i][j][q * 4 + e] + ib[e]);
+                        tv = tv * s2[e];
+                        tv = tv * s1;
+                        v[e] = tv + fbv[e];
+                    }
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 4; e++) v[e] = acc[i][j][q * 4 + e] + fbv[e];
+                }
+                const v4us o = pack4_b16<OUT_DT>(v);
+                if (m < p.M) {
+                    if (vec_ok && n + 3 < p.N) {
+                        *(v4us*)(out + m * p.N + n) = o;
+                    } else {
+#pragma unroll
+                        for (int e = 0; e < 4; e++)
+                            if (n + e < p.N) out[m * p.N + n + e] = o[e];
+                    }
+                }
+            }
+        }
+    }
+}
+
+template <int MODE, int BM, int BN, int BK, int WGM, int WGN, int STAGES, int MINWG, bool KTAIL, int OUT_DT>
+static int qgemm_launch_one(const QgemmParams& p, int64_t batch, hipStream_t st)
+{
+    constexpr bool MX = MODE != MODE_I8;
+    int tiles_m = (int)((p.M + BM - 1) / BM), tiles_n = (int)((p.N + BN - 1) / BN);
+    dim3 grid((unsigned)(tiles_m * tiles_n), (unsigned)batch);
+    size_t lds = (size_t)STAGES * ((BM + BN) * BK + (MX ? (BM + BN) * 4 : 0));
+    auto k = qgemm_kernel<MODE, BM, BN, BK, WGM, WGN, STAGES, MINWG, KTAIL, OUT_DT>;
+    static bool attr_set = false;  // per instantiation; benign if two threads both set it
+    if (!attr_set) {
+        hipError_t e = hipFuncSetAttribute((const void*)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return (int)e;
+        attr_set = true;
+    }
+    hipLaunchKernelGGL(k, grid, dim3(WGM * WGN * 64), lds, st, p, tiles_m, tiles_n);
+    return (int)hipGetLastError();
+}
+
+// Picks the K-tail and output-type instantiation.
+template <int MODE, int BM, int BN, int BK, int WGM, int WGN, int STAGES, int MINWG>
+static int qgemm_launch(const QgemmParams& p, int64_t batch, int out_dt, hipStream_t st)
+{
+    const bool bf = out_dt == DT_BF16;
+    if constexpr (MODE == MODE_I8) {
+        if ((p.KB % BK) != 0) {
+            return bf ? qgemm_launch_one<MODE, BM, BN, BK, WGM, WGN, STAGES, MINWG, true, DT_BF16>(p, batch, st)
+                      : qgemm_launch_one<MODE, BM, BN, BK, WGM, WGN, STAGES, MINWG, true, DT_F16>(p, batch, st);
+        }
+    }
+    return bf ? qgemm_launch_one<MODE, BM, BN, BK, WGM, WGN, STAGES, MINWG, false, DT_BF16>(p, batch, st)
+              : qgemm_launch_one<MODE, BM, BN, BK, WGM, WGN, STAGES, MINWG, false, DT_F16>(p, batch, st);
+}
+
+}  // namespace opsnn

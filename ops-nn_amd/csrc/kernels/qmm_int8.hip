@@ -8,19 +8,13 @@
 // (matmul/quant_batch_matmul_v3/tests/assets/qbmmv3_kernel_golden.py:361-387) and its device epilogue
 // (matmul/quant_batch_matmul_v3/op_kernel/arch35/qbmm_mix_online_dynamic.h:648-736).
 //
-// Fast path: both operands K-contiguous ("x2 stored [N, K]"), 16-byte aligned rows.
-//   - 256x256 (or 128x128) output tile per workgroup, 4 waves, each wave owns a square quarter and
-//     drives v_mfma_i32_32x32x32_i8 with accumulators kept in registers for the whole K loop;
-//   - K tiles are copied global -> LDS asynchronously (16 B per lane, no register round trip),
-//     double buffered, one workgroup barrier per K tile;
-//   - LDS rows are XOR-swizzled in 16-byte chunks so the MFMA operand reads are bank-conflict free;
-//   - the MFMA is issued as x2-fragment x x1-fragment so every lane ends up with four consecutive n
-//     of one output row: scales and bias load as vectors and the 16-bit results leave as 8-byte stores.
-// Anything else (odd K, unaligned or strided operands) runs the plain strided kernel below.
+// Fast path: both operands K-contiguous ("x2 stored [N, K]"), 16-byte aligned rows: the shared MFMA tile
+// kernel of qgemm_core.hip.h in MODE_I8.  Anything else (odd K, unaligned or strided operands, int32 or fp32
+// output) runs the plain strided kernel below.
 #include <cstdlib>
-#include <type_traits>
-#include "common.hip.h"
+
 #include "launch.h"
+#include "qgemm_core.hip.h"
 
 namespace opsnn {
 
@@ -69,304 +63,6 @@ __global__ void qmm_i8_plain(QmmI8Params p)
     store_f32_as(p.out, p.out_dt, o, v);
 }
 
-// ---------------------------------------------------------------------------------------------
-// MFMA kernel family.
-//   BM x BN output tile per workgroup, WGM x WGN waves, each wave owns a (BM/WGM) x (BN/WGN) sub-tile built from
-//   32x32x32 int8 MFMAs; BK bytes of K per pipeline stage, STAGES stages of LDS, MINWG workgroups per CU.
-//   KTAIL: K is not a multiple of BK (the last tile is zero-filled through a zero page).
-// ---------------------------------------------------------------------------------------------
-__device__ __attribute__((aligned(16))) static const int8_t g_zero16[16] = {0};
-
-#ifdef OPSNN_PROF
-// Build-time instrumentation (make PROF=1): per-workgroup phase timestamps in 10 ns ticks.
-__device__ unsigned long long g_prof[8 * 8192];
-#define PROF_MARK(slot)                                                                                  \
-    do {                                                                                                 \
-        if (threadIdx.x == 0 && blockIdx.x < 8192) g_prof[blockIdx.x * 8 + (slot)] = wall_clock64();      \
-    } while (0)
-#define PROF_ID()                                                                                        \
-    do {                                                                                                 \
-        if (threadIdx.x == 0 && blockIdx.x < 8192) g_prof[blockIdx.x * 8 + 7] = __builtin_amdgcn_s_getreg((4 << 0) | (0 << 6) | (31 << 11)); \
-    } while (0)
-#else
-#define PROF_MARK(slot)
-#define PROF_ID()
-#endif
-
-// s_waitcnt with only the vector-memory counter constrained (gfx9 encoding: vmcnt = imm[3:0] | imm[15:14] << 4).
-template <int N>
-__device__ __forceinline__ void wait_vmcnt()
-{
-    static_assert(N >= 0 && N < 64, "vmcnt range");
-    __builtin_amdgcn_s_waitcnt((N & 15) | (((N >> 4) & 3) << 14) | (7 << 4) | (15 << 8));
-}
-
-template <int BM, int BN, int BK, int WGM, int WGN, int STAGES, int MINWG, bool KTAIL, int OUT_DT>
-__global__ __launch_bounds__(WGM* WGN * 64, MINWG) void qmm_i8_mfma(QmmI8Params p, int tiles_m, int tiles_n)
-{
-    constexpr int NT = WGM * WGN * 64;
-    constexpr int CPR = BK / 16;                // 16-byte chunks per LDS row
-    constexpr int RPW = 16 / CPR;               // rows per 256-byte LDS bank wrap
-    constexpr int TM = BM / WGM, TN = BN / WGN; // per-wave tile
-    constexpr int FM = TM / 32, FN = TN / 32;
-    constexpr int KS = BK / 32;                 // MFMA K steps per tile
-    constexpr int A_BYTES = BM * BK, B_BYTES = BN * BK;
-    constexpr int STAGE = A_BYTES + B_BYTES;
-    constexpr int RPI = NT / CPR;               // tile rows covered by one copy instruction of the workgroup
-    constexpr int NA = BM / RPI, NB = BN / RPI; // copy instructions per thread per tile
-    constexpr int CPT = NA + NB;
-    static_assert(CPR == 8 || CPR == 4, "BK must be 64 or 128");
-    static_assert(BM % RPI == 0 && BN % RPI == 0, "tile rows must be a multiple of the rows one copy pass covers");
-    static_assert(STAGES >= 2 && STAGES * CPT < 64, "stage count");
-    extern __shared__ __attribute__((aligned(16))) char smem[];
-
-    PROF_MARK(0);
-    PROF_ID();
-    const int tid = threadIdx.x;
-    const int lane = tid & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int wm = wave / WGN, wn = wave % WGN;
-
-    // tile id: XCD-contiguous, m fastest so that one XCD works on few x2 panels at a time
-    const uint32_t t = xcd_remap(blockIdx.x, (uint32_t)(tiles_m * tiles_n));
-    const int tm = (int)(t % (uint32_t)tiles_m), tn = (int)(t / (uint32_t)tiles_m);
-    const int64_t m0 = (int64_t)tm * BM, n0 = (int64_t)tn * BN;
-    const int64_t bz = blockIdx.y;
-
-    const int64_t lda = p.a_rs, ldb = p.b_cs;
-    const int8_t* A = p.a + bz * p.a_bs + m0 * lda;
-    const int8_t* B = p.b + bz * p.b_bs + n0 * ldb;
-    const int64_t K = p.K;
-    const int KT = (int)((K + BK - 1) / BK);
-
-    // LDS layout of one operand tile: row r holds CPR chunks of 16 bytes; logical chunk c is stored at position
-    // c ^ key(r), key(r) = (r / RPW) % CPR, so that 16 consecutive rows at one logical chunk hit 16 different
-    // 16-byte bank groups.
-    // Async copies: copy instruction i of the workgroup fills LDS chunks [i*NT, (i+1)*NT), i.e. tile rows
-    // i*RPI .. i*RPI+RPI-1; this thread always handles row i*RPI + tid/CPR and the chunk computed below.
-    // Rows past the matrix edge are clamped to the last valid row: they only feed outputs that are never stored.
-    const int crow = tid / CPR;
-    const int cchunk = (tid % CPR) ^ ((crow / RPW) & (CPR - 1));   // RPI is a multiple of RPW*CPR: same key for every i
-    const int a_rows = (int)((p.M - m0) < BM ? (p.M - m0) : BM);
-    const int b_rows = (int)((p.N - n0) < BN ? (p.N - n0) : BN);
-    uint32_t a_off[NA], b_off[NB];
-#pragma unroll
-    for (int i = 0; i < NA; i++) {
-        int r = i * RPI + crow;
-        r = r < a_rows ? r : a_rows - 1;
-        a_off[i] = (uint32_t)(r * lda + cchunk * 16);
-    }
-#pragma unroll
-    for (int i = 0; i < NB; i++) {
-        int r = i * RPI + crow;
-        r = r < b_rows ? r : b_rows - 1;
-        b_off[i] = (uint32_t)(r * ldb + cchunk * 16);
-    }
-    const int8_t* const zero_page = g_zero16;
-
-    auto issue_tile = [&](int kt) {
-        char* sA = smem + (kt % STAGES) * STAGE + wave * 1024;
-        char* sB = sA + A_BYTES;
-        const int64_t k0 = (int64_t)kt * BK;
-        const int8_t* Ak = A + k0;
-        const int8_t* Bk = B + k0;
-        const bool kok = !KTAIL || (k0 + cchunk * 16) < K;
-#pragma unroll
-        for (int i = 0; i < NA; i++) {
-            const int8_t* g = Ak + a_off[i];
-            if constexpr (KTAIL) g = kok ? g : zero_page;
-            async_copy16(g, sA + i * NT * 16);
-        }
-#pragma unroll
-        for (int i = 0; i < NB; i++) {
-            const int8_t* g = Bk + b_off[i];
-            if constexpr (KTAIL) g = kok ? g : zero_page;
-            async_copy16(g, sB + i * NT * 16);
-        }
-    };
-
-    v16i acc[FN][FM];
-#pragma unroll
-    for (int i = 0; i < FN; i++)
-#pragma unroll
-        for (int j = 0; j < FM; j++)
-#pragma unroll
-            for (int r = 0; r < 16; r++) acc[i][j][r] = 0;
-
-    const int frow = lane & 31;   // row inside a 32-row fragment
-    const int fkc = lane >> 5;    // which 16-byte half of the 32-byte K step
-    const int swz = fkc ^ ((frow / RPW) & (CPR - 1));   // 32-row fragments start at multiples of RPW*CPR rows
-    const int a_rowbase = (wm * TM + frow) * BK;
-    const int b_rowbase = A_BYTES + (wn * TN + frow) * BK;
-
-    v4i fa[2][FM], fb[2][FN];
-    auto load_frags = [&](int kt, int s, int buf) {
-        const char* base = smem + (kt % STAGES) * STAGE + (((2 * s) ^ swz) << 4);
-#pragma unroll
-        for (int j = 0; j < FM; j++) fa[buf][j] = *(const v4i*)(base + a_rowbase + j * 32 * BK);
-#pragma unroll
-        for (int i = 0; i < FN; i++) fb[buf][i] = *(const v4i*)(base + b_rowbase + i * 32 * BK);
-    };
-    auto mma = [&](int buf) {
-#pragma unroll
-        for (int i = 0; i < FN; i++)
-#pragma unroll
-            for (int j = 0; j < FM; j++)
-                acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fb[buf][i], fa[buf][j], acc[i][j], 0, 0, 0);
-    };
-
-    // Pipeline.  All STAGES stages are kept in flight.  The loop is rotated so that its single barrier sits in
-    // front of the LAST K step of a tile: on entry to iteration kt the operands of K step 0 are already in
-    // registers; K steps 0..KS-2 multiply while the operands of the following step are read; then
-    //   wait for this thread's copies of tile kt+1, barrier (tile kt+1 is complete in LDS and every wave has
-    //   finished reading tile kt, whose last operands now sit in registers),
-    //   start the copy of tile kt+STAGES into the freed stage, read K step 0 of tile kt+1, multiply the last step.
-    // sched_group_barrier interleaves the LDS reads and copies between the MFMAs so that they issue in the
-    // shadow of the matrix pipe instead of in front of it.
-    static_assert(KS % 2 == 0, "operand double buffer parity");
-#pragma unroll
-    for (int i = 0; i < STAGES; i++)
-        if (i < KT) issue_tile(i);
-    if (KT >= STAGES) wait_vmcnt<(STAGES - 1) * CPT>();
-    else wait_vmcnt<0>();
-    __builtin_amdgcn_s_barrier();
-    PROF_MARK(1);
-    load_frags(0, 0, 0);
-
-    auto k_tile = [&](int kt, auto issue, auto next) {
-        constexpr bool ISSUE = decltype(issue)::value, NEXT = decltype(next)::value;
-#pragma unroll
-        for (int s = 0; s < KS - 1; s++) {
-            load_frags(kt, s + 1, (s + 1) & 1);
-            mma(s & 1);
-#pragma unroll
-            for (int g = 0; g < FM + FN; g++) {
-                __builtin_amdgcn_sched_group_barrier(0x008, (FM * FN) / (FM + FN), 0);   // MFMA
-                __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);                       // LDS read
-            }
-        }
-        if constexpr (NEXT) {
-            if constexpr (ISSUE) wait_vmcnt<(STAGES - 2) * CPT>();
-            else wait_vmcnt<0>();
-        }
-        __builtin_amdgcn_s_waitcnt((63 & 15) | (3 << 14) | (7 << 4) | (0 << 8));   // lgkmcnt(0): stage reads retired
-        __builtin_amdgcn_s_barrier();
-        if constexpr (ISSUE) issue_tile(kt + STAGES);
-        if constexpr (NEXT) load_frags(kt + 1, 0, 0);
-        mma((KS - 1) & 1);
-        if constexpr (NEXT) {
-#pragma unroll
-            for (int g = 0; g < FM + FN; g++) {
-                __builtin_amdgcn_sched_group_barrier(0x008, (FM * FN) / (FM + FN), 0);
-                __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-                if (ISSUE && g < CPT) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);  // copy
-            }
-        }
-    };
-    using T = std::true_type;
-    using F = std::false_type;
-    int kt = 0;
-    for (; kt + STAGES < KT; kt++) k_tile(kt, T{}, T{});
-    for (; kt + 1 < KT; kt++) k_tile(kt, F{}, T{});
-    k_tile(kt, F{}, F{});
-    PROF_MARK(2);
-    __syncthreads();   // all operand reads done before LDS is reused below
-
-    // Epilogue.  acc[i][j][r]: n = n_base + 8*(r/4) + 4*(lane/32) + r%4,  m = m_base + lane%32.
-    // Scales and bias are first widened to fp32 in LDS, so the unrolled part below is branch-free:
-    // absent terms are the neutral elements 1.0f, 0 and -0.0f.
-    float* sS2 = (float*)smem;
-    float* sFb = sS2 + BN;
-    int32_t* sIb = (int32_t*)(sFb + BN);
-    float* sS1 = (float*)(sIb + BN);
-    {
-        const bool has_ib = p.bias && p.bias_dt == DT_I32;
-        const bool has_fb = p.bias && p.bias_dt != DT_I32;
-        for (int i = tid; i < BN; i += NT) {
-            int64_t n = n0 + i;
-            if (n >= p.N) n = p.N - 1;
-            sS2[i] = load_scalar_as_f32(p.x2s, p.x2s_dt, p.x2s_len == 1 ? 0 : n);
-            sFb[i] = has_fb ? load_scalar_as_f32(p.bias, p.bias_dt, bz * p.bias_bs + n) : -0.0f;
-            sIb[i] = has_ib ? ((const int32_t*)p.bias)[bz * p.bias_bs + n] : 0;
-        }
-        for (int i = tid; i < BM; i += NT) {
-            int64_t m = m0 + i;
-            if (m >= p.M) m = p.M - 1;
-            sS1[i] = p.x1s ? p.x1s[m] : 1.0f;
-        }
-    }
-    __syncthreads();
-    PROF_MARK(4);
-    uint16_t* out = (uint16_t*)p.out + bz * p.M * p.N;
-    const bool vec_ok = (p.N % 4) == 0;
-#pragma unroll
-    for (int j = 0; j < FM; j++) {
-        const int ml = wm * TM + j * 32 + frow;
-        const int64_t m = m0 + ml;
-        const float s1 = sS1[ml];
-#pragma unroll
-        for (int i = 0; i < FN; i++) {
-#pragma unroll
-            for (int q = 0; q < 4; q++) {
-                const int nl = wn * TN + i * 32 + 8 * q + 4 * fkc;
-                const int64_t n = n0 + nl;
-                const v4f s2 = *(const v4f*)(sS2 + nl);
-                const v4f fb = *(const v4f*)(sFb + nl);
-                const v4i ib = *(const v4i*)(sIb + nl);
-                v4f v;
-#pragma unroll
-                for (int e = 0; e < 4; e++) {
-                    float t = (float)(acc[i][j][q * 4 + e] + ib[e]);
-                    t = t * s2[e];
-                    t = t * s1;
-                    v[e] = t + fb[e];
-                }
-                const v4us o = pack4_b16<OUT_DT>(v);
-                if (m < p.M) {
-                    if (vec_ok && n + 3 < p.N) {
-                        *(v4us*)(out + m * p.N + n) = o;
-                    } else {
-#pragma unroll
-                        for (int e = 0; e < 4; e++)
-                            if (n + e < p.N) out[m * p.N + n + e] = o[e];
-                    }
-                }
-            }
-        }
-    }
-    PROF_MARK(3);
-}
-
-template <int BM, int BN, int BK, int WGM, int WGN, int STAGES, int MINWG, bool KTAIL, int OUT_DT>
-static int launch_one(const QmmI8Params& p, int64_t batch, hipStream_t st)
-{
-    int tiles_m = (int)((p.M + BM - 1) / BM), tiles_n = (int)((p.N + BN - 1) / BN);
-    dim3 grid((unsigned)(tiles_m * tiles_n), (unsigned)batch);
-    size_t lds = (size_t)STAGES * (BM + BN) * BK;
-    auto k = qmm_i8_mfma<BM, BN, BK, WGM, WGN, STAGES, MINWG, KTAIL, OUT_DT>;
-    static bool attr_set = false;   // per instantiation; benign if two threads both set it
-    if (!attr_set) {
-        hipError_t e = hipFuncSetAttribute((const void*)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-        if (e != hipSuccess) return (int)e;
-        attr_set = true;
-    }
-    hipLaunchKernelGGL(k, grid, dim3(WGM * WGN * 64), lds, st, p, tiles_m, tiles_n);
-    return (int)hipGetLastError();
-}
-
-template <int BM, int BN, int BK, int WGM, int WGN, int STAGES, int MINWG>
-static int launch_mfma(const QmmI8Params& p, int64_t batch, hipStream_t st)
-{
-    const bool ktail = (p.K % BK) != 0;
-    const bool bf = p.out_dt == DT_BF16;
-    if (ktail) {
-        return bf ? launch_one<BM, BN, BK, WGM, WGN, STAGES, MINWG, true, DT_BF16>(p, batch, st)
-                  : launch_one<BM, BN, BK, WGM, WGN, STAGES, MINWG, true, DT_F16>(p, batch, st);
-    }
-    return bf ? launch_one<BM, BN, BK, WGM, WGN, STAGES, MINWG, false, DT_BF16>(p, batch, st)
-              : launch_one<BM, BN, BK, WGM, WGN, STAGES, MINWG, false, DT_F16>(p, batch, st);
-}
-
 }  // namespace opsnn
 
 using namespace opsnn;
@@ -407,25 +103,24 @@ extern "C" int opsnnQmmInt8(const OpsnnQmmArgs* a, void* stream)
     }
     bool fast = want_fast && b_kmajor && (p.b_cs % 16) == 0 && ((uintptr_t)p.b % 16) == 0 && (p.b_bs % 16) == 0;
     if (fast) {
+        QgemmParams g{};
+        g.a = p.a; g.b = p.b; g.lda = p.a_rs; g.ldb = p.b_cs; g.a_bs = p.a_bs; g.b_bs = p.b_bs;
+        g.out = p.out; g.M = p.M; g.N = p.N; g.KB = p.K;
+        g.x1s = p.x1s; g.x2s = p.x2s; g.x2s_dt = p.x2s_dt; g.x2s_len = p.x2s_len;
+        g.bias = p.bias; g.bias_dt = p.bias_dt; g.bias_bs = p.bias_bs;
         switch (variant) {
-            case OPSNN_VARIANT_I8_256: return launch_mfma<256, 256, 128, 2, 2, 2, 1>(p, a->batch, st);
-            case OPSNN_VARIANT_I8_128: return launch_mfma<128, 128, 128, 2, 2, 2, 1>(p, a->batch, st);
-            case OPSNN_VARIANT_I8_256x128_S3: return launch_mfma<256, 128, 64, 2, 2, 3, 2>(p, a->batch, st);
-            case OPSNN_VARIANT_I8_256_W8: return launch_mfma<256, 256, 64, 2, 4, 4, 1>(p, a->batch, st);
-            case OPSNN_VARIANT_I8_256_S4: return launch_mfma<256, 256, 64, 2, 2, 4, 1>(p, a->batch, st);
+            case OPSNN_VARIANT_I8_256: return qgemm_launch<MODE_I8, 256, 256, 128, 2, 2, 2, 1>(g, a->batch, p.out_dt, st);
+            case OPSNN_VARIANT_I8_128: return qgemm_launch<MODE_I8, 128, 128, 128, 2, 2, 2, 1>(g, a->batch, p.out_dt, st);
+            case OPSNN_VARIANT_I8_256x128_S3: return qgemm_launch<MODE_I8, 256, 128, 64, 2, 2, 3, 2>(g, a->batch, p.out_dt, st);
+            case OPSNN_VARIANT_I8_256_W8: return qgemm_launch<MODE_I8, 256, 256, 64, 2, 4, 4, 1>(g, a->batch, p.out_dt, st);
+            case OPSNN_VARIANT_I8_256_S4: return qgemm_launch<MODE_I8, 256, 256, 64, 2, 2, 4, 1>(g, a->batch, p.out_dt, st);
             default: break;
         }
-        if (p.M <= 128 || p.N <= 128 || p.M * p.N < 256 * 256 * 64) return launch_mfma<128, 128, 128, 2, 2, 2, 1>(p, a->batch, st);
-        return launch_mfma<256, 256, 128, 2, 2, 2, 1>(p, a->batch, st);
+        if (p.M <= 128 || p.N <= 128 || p.M * p.N < 256 * 256 * 64) return qgemm_launch<MODE_I8, 128, 128, 128, 2, 2, 2, 1>(g, a->batch, p.out_dt, st);
+        return qgemm_launch<MODE_I8, 256, 128, 64, 2, 2, 3, 2>(g, a->batch, p.out_dt, st);
     }
     dim3 block(256), grid((unsigned)(((p.N + 255) / 256) * p.M), (unsigned)a->batch);
     hipLaunchKernelGGL(qmm_i8_plain, grid, block, 0, st, p);
     return (int)hipGetLastError();
 }
 
-#ifdef OPSNN_PROF
-extern "C" __attribute__((visibility("default"))) int opsnnDebugReadProf(unsigned long long* host, int n)
-{
-    return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(opsnn::g_prof), sizeof(unsigned long long) * n, 0, hipMemcpyDeviceToHost);
-}
-#endif

@@ -1,0 +1,121 @@
+// MX quantized matmul: fp4 e2m1 (or fp8 e4m3) operands with one e8m0 scale per 32 K elements.
+//
+//   out[m,n] = cast( sum_k (x1[m,k] * 2^(s1[m,k/32]-127)) * (x2[k,n] * 2^(s2[k/32,n]-127)) + bias[n] )
+//
+// Formula and scale layouts: matmul/quant_batch_matmul_v3/tests/assets/qbmmv3_kernel_golden.py:153-234; the
+// device counterpart in the reference is the MX block-mmad (matmul/common/cmct/block/block_mmad_mx.h).
+// Here the contraction and the scaling are one instruction, v_mfma_scale_f32_32x32x64_f8f6f4: each lane hands
+// the matrix core its 32 K elements together with the e8m0 byte that scales exactly those 32 elements, so the
+// MX block size (32) and the hardware operand block coincide and no dequantised copy is ever formed.
+//
+// Fast path (qgemm_core.hip.h, MODE_MXFP4 / MODE_MXFP8): operands and scales K-contiguous, K % 128 == 0,
+// 16-bit output.  An N-contiguous x2 (data [K, N], scales [K/64, N, 2]) is first re-laid out into the
+// workspace; everything else runs the plain kernel.
+#include "launch.h"
+#include "qgemm_core.hip.h"
+
+namespace opsnn {
+
+// dst[c, r] = src[r, c] for 16-bit elements: the paired e8m0 scales [K/64, N, 2] -> [N, K/64, 2].
+__global__ __launch_bounds__(256) void transpose16_kernel(const uint16_t* __restrict__ src, uint16_t* __restrict__ dst,
+                                                          int64_t rows, int64_t cols)
+{
+    __shared__ uint16_t tile[32][33];
+    const int64_t bz = blockIdx.z;
+    src += bz * rows * cols;
+    dst += bz * rows * cols;
+    const int64_t r0 = (int64_t)blockIdx.y * 32, c0 = (int64_t)blockIdx.x * 32;
+    const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;
+    for (int i = ty; i < 32; i += 8) {
+        int64_t r = r0 + i, c = c0 + tx;
+        tile[i][tx] = (r < rows && c < cols) ? src[r * cols + c] : 0;
+    }
+    __syncthreads();
+    for (int i = ty; i < 32; i += 8) {
+        int64_t c = c0 + i, r = r0 + tx;
+        if (c < cols && r < rows) dst[c * rows + r] = tile[tx][i];
+    }
+}
+
+static inline uint64_t align_up(uint64_t v, uint64_t a) { return (v + a - 1) / a * a; }
+
+uint64_t mx_workspace_bytes(const OpsnnQmmArgs& a)
+{
+    if (a.x2.row_stride == 1 || a.K == 1) return 0;
+    if (a.x2.col_stride != 1 || a.x2.row_stride != a.N) return 0;
+    const uint64_t bits = a.x2_dtype == DT_E2M1 ? 4 : 8;
+    const uint64_t nb = a.x2.batch_stride == 0 ? 1 : (uint64_t)a.batch;
+    const uint64_t data = align_up((uint64_t)a.N * (uint64_t)a.K * bits / 8, 256) * nb;
+    const uint64_t ks = ((uint64_t)a.K + 63) / 64;
+    const uint64_t snb = a.x2_scale_mat.batch_stride == 0 ? 1 : (uint64_t)a.batch;
+    return data + align_up((uint64_t)a.N * ks * 2, 256) * snb;
+}
+
+int launch_mx_mfma(const OpsnnQmmArgs& a0, hipStream_t st)
+{
+    OpsnnQmmArgs a = a0;
+    const bool fp4 = a.x1_dtype == DT_E2M1 && a.x2_dtype == DT_E2M1;
+    const bool fp8 = a.x1_dtype == DT_E4M3 && a.x2_dtype == DT_E4M3;
+    if (!fp4 && !fp8) return OPSNN_NOT_TAKEN;
+    // The 8-bit forms of the matrix instruction sum their 64 products with a reduced-width aligner (measured:
+    // mean error 1e-5 of sum|terms| per instruction).  Chained over all of K that exceeds the 16-bit output's own
+    // rounding, so MXFP8 takes the MFMA path only on request (OPSNN_VARIANT_MX_FP8_MFMA) until it gains the
+    // per-128-K fp32 promotion the block-scale kernel has; fp4 products are exact in that datapath.
+    if (fp8 && a.force_variant != OPSNN_VARIANT_MX_FP8_MFMA && a.force_variant != OPSNN_VARIANT_MX_128) return OPSNN_NOT_TAKEN;
+    if (a.out_dtype != DT_BF16 && a.out_dtype != DT_F16) return OPSNN_NOT_TAKEN;
+    if (a.bias && a.bias_dtype != DT_F32) return OPSNN_NOT_TAKEN;
+    if (a.K % 128 != 0 || a.M * a.N < 64 * 64) return OPSNN_NOT_TAKEN;
+    const int64_t ks = a.K / 64;  // scale pairs per row
+    if (a.x1.col_stride != 1 || a.x1_scale_mat.col_stride != 2 || a.x1_scale_mat.row_stride != ks * 2) return OPSNN_NOT_TAKEN;
+    const int64_t epb = fp4 ? 2 : 1;  // elements per byte
+
+    if (a.x2.row_stride != 1) {
+        // x2 is [K, N] with N contiguous: re-lay data and scales out K-contiguous in the workspace
+        if (!a.workspace || a.x2.col_stride != 1 || a.x2.row_stride != a.N) return OPSNN_NOT_TAKEN;
+        if (a.x2_scale_mat.row_stride != 2 || a.x2_scale_mat.col_stride != a.N * 2) return OPSNN_NOT_TAKEN;
+        if (a.x2.batch_stride != 0 && a.x2.batch_stride != a.K * a.N) return OPSNN_NOT_TAKEN;
+        const int64_t nb = a.x2.batch_stride == 0 ? 1 : a.batch;
+        const int64_t snb = a.x2_scale_mat.batch_stride == 0 ? 1 : a.batch;
+        if (snb != 1 && a.x2_scale_mat.batch_stride != ks * a.N * 2) return OPSNN_NOT_TAKEN;
+        const uint64_t data_one = align_up((uint64_t)a.N * a.K / epb, 256);
+        char* wdata = (char*)a.workspace;
+        char* wscale = wdata + data_one * nb;
+        const uint64_t scale_one = align_up((uint64_t)a.N * ks * 2, 256);
+        for (int64_t b = 0; b < nb; b++) {  // per-batch because of the aligned pitch
+            const char* src = (const char*)a.x2.ptr + b * (a.K * a.N / epb);
+            int rc = fp4 ? opsnnTranspose4(src, wdata + b * data_one, a.K, a.N, 1, st) : opsnnTranspose8(src, wdata + b * data_one, a.K, a.N, 1, st);
+            if (rc != 0) return rc;
+        }
+        for (int64_t b = 0; b < snb; b++) {
+            dim3 grid((unsigned)((a.N + 31) / 32), (unsigned)((ks + 31) / 32), 1);
+            hipLaunchKernelGGL(transpose16_kernel, grid, dim3(256), 0, st,
+                               (const uint16_t*)((const char*)a.x2_scale_mat.ptr + b * (ks * a.N * 2)),
+                               (uint16_t*)(wscale + b * scale_one), ks, a.N);
+        }
+        a.x2.ptr = wdata; a.x2.row_stride = 1; a.x2.col_stride = a.K; a.x2.batch_stride = nb == 1 ? 0 : (int64_t)(data_one * epb);
+        a.x2_scale_mat.ptr = wscale; a.x2_scale_mat.row_stride = ks * 2; a.x2_scale_mat.col_stride = 2;
+        a.x2_scale_mat.batch_stride = snb == 1 ? 0 : (int64_t)scale_one;
+    }
+    if (a.x2_scale_mat.col_stride != 2 || a.x2_scale_mat.row_stride != ks * 2) return OPSNN_NOT_TAKEN;
+
+    QgemmParams g{};
+    g.a = (const int8_t*)a.x1.ptr; g.b = (const int8_t*)a.x2.ptr;
+    g.lda = a.x1.row_stride / epb; g.ldb = a.x2.col_stride / epb;
+    g.a_bs = a.x1.batch_stride / epb; g.b_bs = a.x2.batch_stride / epb;
+    g.out = a.out; g.M = a.M; g.N = a.N; g.KB = a.K / epb;
+    g.bias = a.bias; g.bias_dt = a.bias_dtype; g.bias_bs = a.bias_batch_stride;
+    g.sa = (const uint8_t*)a.x1_scale_mat.ptr; g.sb = (const uint8_t*)a.x2_scale_mat.ptr;
+    g.sa_rs = a.x1_scale_mat.row_stride; g.sb_rs = a.x2_scale_mat.row_stride;
+    g.sa_bs = a.x1_scale_mat.batch_stride; g.sb_bs = a.x2_scale_mat.batch_stride;
+    if (((uintptr_t)g.a | (uintptr_t)g.b | (uint64_t)g.lda | (uint64_t)g.ldb | (uint64_t)g.a_bs | (uint64_t)g.b_bs) % 16) return OPSNN_NOT_TAKEN;
+    if (((uintptr_t)g.sa | (uintptr_t)g.sb | (uint64_t)g.sa_rs | (uint64_t)g.sb_rs | (uint64_t)g.sa_bs | (uint64_t)g.sb_bs) % 4) return OPSNN_NOT_TAKEN;
+    const bool small = a.M <= 128 || a.N <= 128;
+    if (fp4) {
+        if (small || a.force_variant == OPSNN_VARIANT_MX_128) return qgemm_launch<MODE_MXFP4, 128, 128, 64, 2, 2, 4, 1>(g, a.batch, a.out_dtype, st);
+        return qgemm_launch<MODE_MXFP4, 256, 256, 64, 2, 2, 4, 1>(g, a.batch, a.out_dtype, st);
+    }
+    if (small || a.force_variant == OPSNN_VARIANT_MX_128) return qgemm_launch<MODE_MXFP8, 128, 128, 128, 2, 2, 2, 1>(g, a.batch, a.out_dtype, st);
+    return qgemm_launch<MODE_MXFP8, 256, 256, 128, 2, 2, 2, 1>(g, a.batch, a.out_dtype, st);
+}
+
+}  // namespace opsnn
