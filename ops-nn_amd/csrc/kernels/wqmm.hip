@@ -1,0 +1,336 @@
+// Weight-only quantized matmul for decode-shaped M (fp16 / bf16 activations, int4 / int8 weights).
+//
+//   y[m,n] = cast( sum_k x[m,k] * T(T(w[k,n] + offset[g,n]) * scale[g,n]) + bias[n] ),   g = k / group,
+//   T = rounding through x's dtype (both dequantisation steps are rounded, as the reference's vector unit does:
+//   matmul/weight_quant_batch_matmul_v2/op_kernel/arch35/n_first/basic_block_vf_nd.h:139-148; golden:
+//   matmul/weight_quant_batch_matmul_v2/tests/assets/wqbmmv2_kernel_golden.py:199-297).
+//
+// The path is bound by the weight stream from HBM, so the kernel is built around it:
+//   - the weight is consumed K-contiguous ("stored [N, K]"); every lane streams 16-byte pieces of one weight row
+//     straight from global memory into registers -- each weight byte is used by exactly one wave, so it never
+//     visits LDS -- with several pieces in flight per lane;
+//   - a wave owns 16 output columns for all of K.  A 16-byte piece holds 32 int4 (16 int8) consecutive k of one
+//     column; the four 16-lane groups of the wave take consecutive pieces, so one load instruction covers a
+//     [16 n] x [128 k] (int8: [64 k]) weight block that lies inside one quantisation group whenever the group
+//     size is a multiple of 128 (64);
+//   - dequantisation happens in registers in x's own arithmetic: for fp16 the nibbles are spliced into the
+//     mantissa of 1024.0 (exact), re-centred with one packed add or fma, then one packed fp16 add (offset) and
+//     one packed fp16 multiply (scale) perform exactly the two roundings of the formula; for bf16 the same steps
+//     run in fp32 with the hardware's round-to-nearest-even conversion to bf16 after each;
+//   - the contraction is v_mfma_f32_16x16x32_{f16,bf16} with the weight block as the row operand and x as the
+//     column operand (fp32 accumulation); for M = 1 fifteen of the sixteen columns are idle, which costs nothing
+//     because the matrix pipe is far from being the limit;
+//   - x is staged through LDS in K slabs shared by the workgroup's four waves, already permuted into the element
+//     order the nibble splicing produces, so no weight register ever needs a shuffle.
+// M > 64 is processed in row slabs of 64 (the weight is re-streamed per slab; such shapes are compute-bound).
+#include "launch.h"
+#include "qgemm_core.hip.h"
+
+namespace opsnn {
+
+int launch_wqmm_plain(const OpsnnWqmmArgs& a, hipStream_t st);
+
+struct WqParams {
+    const uint16_t* x;       // [M, K] dense 16-bit
+    const uint8_t* w;        // row n at w + n*ldw (bytes), K-contiguous
+    int64_t ldw;
+    const uint16_t* scale;   // element (g, n) at scale[g*s_rs + n*s_cs]
+    const uint16_t* offset;  // same layout, or null
+    int64_t s_rs, s_cs;
+    const void* bias;
+    int bias_dt;
+    uint16_t* y;             // [M, N]
+    int64_t M, N, K;
+    int64_t group;           // elements per group (K if per-channel)
+    int group_shift;         // log2(group) if it is a power of two, else -1
+    int64_t m_base, m_rows;  // row slab handled by this launch
+};
+
+typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ uint32_t u32(h2 v) { return __builtin_bit_cast(uint32_t, v); }
+
+// ---- fp16 dequantisation: 8 int4 of one dword -> 4 packed pairs in element order [0,4], [1,5], [2,6], [3,7] ----
+// q holds two's-complement nibbles; after xor 0x88888888 each nibble is w + 8 in 0..15.
+__device__ __forceinline__ void dequant_i4_f16(uint32_t q, h2 off, h2 sc, bool has_off, h2 (&out)[4])
+{
+    const uint32_t u = q ^ 0x88888888u;
+    const uint32_t u8 = u >> 8;
+    const h2 c1032 = {(_Float16)-1032.0f, (_Float16)-1032.0f};
+    const h2 c72 = {(_Float16)-72.0f, (_Float16)-72.0f};
+    const h2 r16 = {(_Float16)0.0625f, (_Float16)0.0625f};
+    h2 t0 = __builtin_bit_cast(h2, (u & 0x000F000Fu) | 0x64006400u);   // 1024 + (w+8)        elements 0, 4
+    h2 t1 = __builtin_bit_cast(h2, (u & 0x00F000F0u) | 0x64006400u);   // 1024 + 16*(w+8)     elements 1, 5
+    h2 t2 = __builtin_bit_cast(h2, (u8 & 0x000F000Fu) | 0x64006400u);  //                     elements 2, 6
+    h2 t3 = __builtin_bit_cast(h2, (u8 & 0x00F000F0u) | 0x64006400u);  //                     elements 3, 7
+    t0 = t0 + c1032;                                   // exact: w
+    t2 = t2 + c1032;
+    t1 = __builtin_elementwise_fma(t1, r16, c72);      // exact: (1024 + 16(w+8))/16 - 72 = w
+    t3 = __builtin_elementwise_fma(t3, r16, c72);
+    if (has_off) { t0 = t0 + off; t1 = t1 + off; t2 = t2 + off; t3 = t3 + off; }   // first rounding
+    out[0] = t0 * sc; out[1] = t1 * sc; out[2] = t2 * sc; out[3] = t3 * sc;         // second rounding
+}
+
+// ---- generic dequantisation of one weight to fp32 holding a value of x's dtype ----
+template <int XDT>
+__device__ __forceinline__ float round_x(float v)
+{
+    if constexpr (XDT == DT_F16) return (float)(_Float16)v;
+    else return bf16_to_f32(bf16_bits(v));
+}
+template <int XDT>
+__device__ __forceinline__ uint16_t bits_x(float v)
+{
+    if constexpr (XDT == DT_F16) return f16_bits(v);
+    else return bf16_bits(v);
+}
+template <int XDT>
+__device__ __forceinline__ float dequant_one(float w, float off, float sc, bool has_off)
+{
+    if (has_off) w = round_x<XDT>(w + off);
+    return round_x<XDT>(w * sc);
+}
+
+// MB: 16-row blocks of x handled per launch slab (1, 2 or 4).  WBITS: 4 or 8.
+template <int XDT, int WBITS, int MB>
+__global__ __launch_bounds__(256, 2) void wqmm_decode_kernel(WqParams p)
+{
+    constexpr int KPL = 128 / WBITS;          // k elements per 16-byte piece per lane: 32 (int4) or 16 (int8)
+    constexpr int KC = 4 * KPL;               // k per wave load instruction ("chunk"): 128 or 64
+    constexpr int STEPS = KC / 32;            // MFMA steps per chunk: 4 or 2
+    constexpr int KX = 1024 / MB;             // k per LDS slab of x
+    constexpr int CPS = KX / KC;              // chunks per slab
+    constexpr int ROWS = 16 * MB;
+    constexpr int XROW = KX * 2 + 16;         // padded LDS row pitch in bytes (conflict-free 16-byte reads)
+    constexpr int XSLAB = ROWS * XROW;
+    constexpr int PF = CPS < 8 ? CPS : 8;     // weight pieces in flight per lane
+    extern __shared__ __attribute__((aligned(16))) char sx[];   // 2 * XSLAB bytes
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int nrow = lane & 15, g = lane >> 4;
+    const int64_t n0 = ((int64_t)blockIdx.x * 4 + wave) * 16;
+    const bool n_ok = n0 < p.N;                       // whole wave idle past the edge (still joins barriers)
+    const int64_t n = (n0 + nrow) < p.N ? (n0 + nrow) : p.N - 1;
+    const bool has_off = p.offset != nullptr;
+    const int64_t K = p.K;
+    const int NSLAB = (int)((K + KX - 1) / KX);
+
+    const uint8_t* wrow = p.w + n * p.ldw;
+    const uint16_t* srow = p.scale + n * p.s_cs;
+    const uint16_t* orow = has_off ? p.offset + n * p.s_cs : nullptr;
+
+    // x staging: thread t copies 8 consecutive halves (16 bytes) per pass, permuted to the order [0,4,1,5,2,6,3,7]
+    // for int4 so that the pairs produced by the nibble splicing line up with natural pairs of x.
+    auto stage_x = [&](int slab, int buf) {
+        char* dst = sx + buf * XSLAB;
+        const int64_t k0 = (int64_t)slab * KX;
+        for (int idx = tid; idx < ROWS * (KX / 8); idx += 256) {
+            const int r = idx / (KX / 8), c = idx % (KX / 8);
+            const int64_t m = p.m_base + r, k = k0 + (int64_t)c * 8;
+            v4i v = {0, 0, 0, 0};
+            if (r < p.m_rows && k + 8 <= K) {
+                v = *(const v4i*)(p.x + m * K + k);
+            } else if (r < p.m_rows && k < K) {
+                uint16_t tmp[8];
+#pragma unroll
+                for (int e = 0; e < 8; e++) tmp[e] = (k + e < K) ? p.x[m * K + k + e] : (uint16_t)0;
+                v = *(const v4i*)tmp;
+            }
+            if constexpr (WBITS == 4) {
+                // halves h0..h7 -> [h0,h4,h1,h5,h2,h6,h3,h7]
+                const uint32_t a0 = (uint32_t)v[0], a1 = (uint32_t)v[1], a2 = (uint32_t)v[2], a3 = (uint32_t)v[3];
+                v4i o;
+                o[0] = (int)((a0 & 0xffffu) | (a2 << 16));          // h0, h4
+                o[1] = (int)((a0 >> 16) | (a2 & 0xffff0000u));      // h1, h5
+                o[2] = (int)((a1 & 0xffffu) | (a3 << 16));          // h2, h6
+                o[3] = (int)((a1 >> 16) | (a3 & 0xffff0000u));      // h3, h7
+                v = o;
+            }
+            *(v4i*)(dst + r * XROW + c * 16) = v;
+        }
+    };
+
+    v4f acc[MB];
+#pragma unroll
+    for (int b = 0; b < MB; b++) acc[b] = (v4f){0.0f, 0.0f, 0.0f, 0.0f};
+
+    // weight pieces with their group's scale and offset, prefetched in groups of PF ahead of their use
+    v4i wq[PF];
+    uint16_t sq[PF], oq[PF];
+    const int Ki = (int)K, groupi = (int)p.group;
+    auto load_w = [&](int slab, int c0) {
+#pragma unroll
+        for (int i = 0; i < PF; i++) {
+            const int k = slab * KX + (c0 + i) * KC + g * KPL;
+            // K is a multiple of KPL on this path; pieces past K read the row's last piece and are masked below
+            const int kk = k < Ki ? k : Ki - KPL;
+            wq[i] = n_ok ? *(const v4i*)(wrow + (int64_t)kk * WBITS / 8) : (v4i){0, 0, 0, 0};
+            const int gi = p.group_shift >= 0 ? (kk >> p.group_shift) : (kk / groupi);
+            sq[i] = srow[(int64_t)gi * p.s_rs];
+            oq[i] = has_off ? orow[(int64_t)gi * p.s_rs] : (uint16_t)0;
+        }
+    };
+
+    stage_x(0, 0);
+    load_w(0, 0);
+    __syncthreads();
+
+    for (int slab = 0; slab < NSLAB; slab++) {
+        const int buf = slab & 1;
+        if (slab + 1 < NSLAB) stage_x(slab + 1, buf ^ 1);
+        const char* xs = sx + buf * XSLAB;
+#pragma unroll
+        for (int c0 = 0; c0 < CPS; c0 += PF) {
+            v4i cur[PF];
+            uint16_t scur[PF], ocur[PF];
+#pragma unroll
+            for (int i = 0; i < PF; i++) { cur[i] = wq[i]; scur[i] = sq[i]; ocur[i] = oq[i]; }
+            // prefetch the next group of pieces (next part of this slab, or the start of the next slab)
+            if (c0 + PF < CPS) load_w(slab, c0 + PF);
+            else if (slab + 1 < NSLAB) load_w(slab + 1, 0);
+#pragma unroll
+            for (int i = 0; i < PF; i++) {
+                const int c = c0 + i;
+                const int k = slab * KX + c * KC + g * KPL;   // first k of this lane's piece
+                const bool live = k < Ki;
+                const uint16_t sb = scur[i], ob = ocur[i];
+#pragma unroll
+                for (int s = 0; s < STEPS; s++) {
+                    // operand A: this lane's 8 dequantised weights for MFMA step s
+                    v4i aop;
+                    if constexpr (XDT == DT_F16 && WBITS == 4) {
+                        const _Float16 sh = __builtin_bit_cast(_Float16, sb), oh = __builtin_bit_cast(_Float16, ob);
+                        h2 o4[4];
+                        dequant_i4_f16(live ? (uint32_t)cur[i][s] : 0x88888888u, (h2){oh, oh}, (h2){sh, sh}, has_off, o4);
+                        if (!live) { o4[0] = o4[1] = o4[2] = o4[3] = (h2){(_Float16)0.0f, (_Float16)0.0f}; }
+                        aop = (v4i){(int)u32(o4[0]), (int)u32(o4[1]), (int)u32(o4[2]), (int)u32(o4[3])};
+                    } else {
+                        float scf, off;
+                        if constexpr (XDT == DT_F16) { scf = f16_to_f32(sb); off = f16_to_f32(ob); }
+                        else { scf = bf16_to_f32(sb); off = bf16_to_f32(ob); }
+                        uint16_t e[8];
+                        if constexpr (WBITS == 4) {
+                            const uint32_t q = (uint32_t)cur[i][s];
+                            // element order [0,4,1,5,2,6,3,7] to match the staged x
+                            const int ord[8] = {0, 4, 1, 5, 2, 6, 3, 7};
+#pragma unroll
+                            for (int j = 0; j < 8; j++) {
+                                int v = (int)((q >> (4 * ord[j])) & 15u);
+                                v = v >= 8 ? v - 16 : v;
+                                e[j] = live ? bits_x<XDT>(dequant_one<XDT>((float)v, off, scf, has_off)) : (uint16_t)0;
+                            }
+                        } else {
+                            // int8: 16 bytes per piece, step s uses bytes 8s..8s+7 in natural order
+#pragma unroll
+                            for (int j = 0; j < 8; j++) {
+                                const uint32_t q = (uint32_t)cur[i][2 * s + (j >> 2)];
+                                const int v = (int)(int8_t)((q >> (8 * (j & 3))) & 0xffu);
+                                e[j] = live ? bits_x<XDT>(dequant_one<XDT>((float)v, off, scf, has_off)) : (uint16_t)0;
+                            }
+                        }
+                        aop = (v4i){(int)(e[0] | ((uint32_t)e[1] << 16)), (int)(e[2] | ((uint32_t)e[3] << 16)),
+                                    (int)(e[4] | ((uint32_t)e[5] << 16)), (int)(e[6] | ((uint32_t)e[7] << 16))};
+                    }
+                    // operand B: x[m = 16b + nrow][k = chunk + g*KPL + 8s + 0..7] (already permuted for int4)
+                    const int kofs = (c * KC + g * KPL + 8 * s) * 2;
+#pragma unroll
+                    for (int b = 0; b < MB; b++) {
+                        const v4i bop = *(const v4i*)(xs + (16 * b + nrow) * XROW + kofs);
+                        if constexpr (XDT == DT_F16) {
+                            acc[b] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(v8h, aop), __builtin_bit_cast(v8h, bop), acc[b], 0, 0, 0);
+                        } else {
+                            acc[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf, aop), __builtin_bit_cast(v8bf, bop), acc[b], 0, 0, 0);
+                        }
+                    }
+                }
+            }
+        }
+        __syncthreads();
+    }
+
+    // D'[row = weight row n][col = x row m]: lane holds col m = lane%16, rows n = 4*(lane/16) + i
+    if (!n_ok) return;
+#pragma unroll
+    for (int b = 0; b < MB; b++) {
+        const int r = 16 * b + nrow;
+        if (r >= p.m_rows) continue;
+        const int64_t m = p.m_base + r;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const int64_t nn = n0 + 4 * g + i;
+            if (nn >= p.N) continue;
+            float v = acc[b][i];
+            if (p.bias) v = v + load_scalar_as_f32(p.bias, p.bias_dt, nn);
+            if constexpr (XDT == DT_BF16) v = bf16_to_f32(bf16_bits(v));   // the golden rounds bf16 results twice (a no-op)
+            p.y[m * p.N + nn] = bits_x<XDT>(v);
+        }
+    }
+}
+
+template <int XDT, int WBITS, int MB>
+static int launch_decode(const WqParams& p, unsigned grid, hipStream_t st)
+{
+    constexpr int KX = 1024 / MB;
+    const size_t lds = 2 * (size_t)(16 * MB) * (KX * 2 + 16);
+    auto k = wqmm_decode_kernel<XDT, WBITS, MB>;
+    static bool attr_set = false;
+    if (!attr_set) {
+        hipError_t e = hipFuncSetAttribute((const void*)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return (int)e;
+        attr_set = true;
+    }
+    hipLaunchKernelGGL(k, dim3(grid), dim3(256), lds, st, p);
+    return (int)hipGetLastError();
+}
+
+template <int XDT, int WBITS>
+static int launch_slabs(WqParams p, hipStream_t st)
+{
+    const unsigned grid = (unsigned)((p.N + 63) / 64);
+    for (int64_t m0 = 0; m0 < p.M; m0 += 64) {
+        p.m_base = m0;
+        p.m_rows = (p.M - m0) < 64 ? (p.M - m0) : 64;
+        int rc;
+        if (p.m_rows <= 16) rc = launch_decode<XDT, WBITS, 1>(p, grid, st);
+        else if (p.m_rows <= 32) rc = launch_decode<XDT, WBITS, 2>(p, grid, st);
+        else rc = launch_decode<XDT, WBITS, 4>(p, grid, st);
+        if (rc != 0) return rc;
+    }
+    return 0;
+}
+
+int launch_wqmm_mfma(const OpsnnWqmmArgs& a0, hipStream_t st)
+{
+    OpsnnWqmmArgs a = a0;
+    if (a.x_dtype != DT_F16 && a.x_dtype != DT_BF16) return OPSNN_NOT_TAKEN;
+    if (a.w_dtype != DT_I4 && a.w_dtype != DT_I8) return OPSNN_NOT_TAKEN;
+    if (a.scale_dtype != a.x_dtype) return OPSNN_NOT_TAKEN;
+    const int wbits = a.w_dtype == DT_I4 ? 4 : 8;
+    const int64_t kpl = 128 / wbits;
+    if (a.K % kpl != 0 || a.K < kpl) return OPSNN_NOT_TAKEN;
+    const int64_t group = a.group > 0 ? a.group : a.K;
+    if (group % kpl != 0) return OPSNN_NOT_TAKEN;   // a lane's piece must lie inside one group
+    if (a.w.row_stride != 1) {
+        // weight is [K, N] with N contiguous: re-lay it out K-contiguous in the workspace
+        if (!a.workspace || a.w.col_stride != 1 || a.w.row_stride != a.N || a.K == 1) return OPSNN_NOT_TAKEN;
+        int rc = wbits == 4 ? opsnnTranspose4(a.w.ptr, a.workspace, a.K, a.N, 1, st) : opsnnTranspose8(a.w.ptr, a.workspace, a.K, a.N, 1, st);
+        if (rc != 0) return rc;
+        a.w.ptr = a.workspace; a.w.row_stride = 1; a.w.col_stride = a.K;
+    }
+    WqParams p{};
+    p.x = (const uint16_t*)a.x;
+    p.w = (const uint8_t*)a.w.ptr;
+    p.ldw = a.w.col_stride * wbits / 8;
+    p.scale = (const uint16_t*)a.scale.ptr; p.offset = (const uint16_t*)a.offset;
+    p.s_rs = a.scale.row_stride; p.s_cs = a.scale_n == 1 ? 0 : a.scale.col_stride;
+    p.bias = a.bias; p.bias_dt = a.bias_dtype;
+    p.y = (uint16_t*)a.y; p.M = a.M; p.N = a.N; p.K = a.K; p.group = group;
+    p.group_shift = (group & (group - 1)) == 0 ? __builtin_ctzll((unsigned long long)group) : -1;
+    if (a.K >= (1ll << 31) || a.N >= (1ll << 31)) return OPSNN_NOT_TAKEN;
+    if (((uintptr_t)p.w | (uint64_t)p.ldw) % 16 || ((uintptr_t)p.x % 16) || (a.K % 8)) return OPSNN_NOT_TAKEN;
+    if (a.x_dtype == DT_F16) return wbits == 4 ? launch_slabs<DT_F16, 4>(p, st) : launch_slabs<DT_F16, 8>(p, st);
+    return wbits == 4 ? launch_slabs<DT_BF16, 4>(p, st) : launch_slabs<DT_BF16, 8>(p, st);
+}
+
+}  // namespace opsnn
