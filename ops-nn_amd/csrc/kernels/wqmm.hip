@@ -92,53 +92,64 @@ __device__ __forceinline__ float dequant_one(float w, float off, float sc, bool 
 }
 
 // MB: 16-row blocks of x handled per launch slab (1, 2 or 4).  WBITS: 4 or 8.
-template <int XDT, int WBITS, int MB>
+// WK: waves of the workgroup that split K between them (1, 2 or 4); the other 4/WK waves take different column
+// blocks.  WK > 1 is for narrow N, where column blocks alone cannot fill the chip; partial sums meet in LDS and
+// are added in a fixed order.
+template <int XDT, int WBITS, int MB, int WK>
 __global__ __launch_bounds__(256, 2) void wqmm_decode_kernel(WqParams p)
 {
+    constexpr int WN = 4 / WK;
     constexpr int KPL = 128 / WBITS;          // k elements per 16-byte piece per lane: 32 (int4) or 16 (int8)
     constexpr int KC = 4 * KPL;               // k per wave load instruction ("chunk"): 128 or 64
     constexpr int STEPS = KC / 32;            // MFMA steps per chunk: 4 or 2
-    constexpr int KX = 1024 / MB;             // k per LDS slab of x
-    constexpr int CPS = KX / KC;              // chunks per slab
+    constexpr int PF = 8;                     // weight pieces in flight per lane = chunks per super-step
+    constexpr int KX = (PF * KC) / MB;        // k per LDS slab of x
+    constexpr int CPS = KX / KC;              // chunks per slab: 8, 4 or 2
     constexpr int ROWS = 16 * MB;
     constexpr int XROW = KX * 2 + 16;         // padded LDS row pitch in bytes (conflict-free 16-byte reads)
     constexpr int XSLAB = ROWS * XROW;
-    constexpr int PF = CPS < 8 ? CPS : 8;     // weight pieces in flight per lane
-    extern __shared__ __attribute__((aligned(16))) char sx[];   // 2 * XSLAB bytes
+    constexpr int XITEMS = ROWS * (KX / 8) / 256;   // 16-byte x pieces staged per thread per slab
+    static_assert(ROWS * (KX / 8) % 256 == 0, "x staging mapping");
+    extern __shared__ __attribute__((aligned(16))) char sx[];   // 2 * XSLAB bytes (reused for the K-split reduction)
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wn = wave / WK, wk = wave % WK;
     const int nrow = lane & 15, g = lane >> 4;
-    const int64_t n0 = ((int64_t)blockIdx.x * 4 + wave) * 16;
+    const int64_t n0 = ((int64_t)blockIdx.x * WN + wn) * 16;
     const bool n_ok = n0 < p.N;                       // whole wave idle past the edge (still joins barriers)
     const int64_t n = (n0 + nrow) < p.N ? (n0 + nrow) : p.N - 1;
     const bool has_off = p.offset != nullptr;
-    const int64_t K = p.K;
-    const int NSLAB = (int)((K + KX - 1) / KX);
+    const int Ki = (int)p.K, groupi = (int)p.group;
+    const int NSLAB = (Ki + KX - 1) / KX;
 
     const uint8_t* wrow = p.w + n * p.ldw;
     const uint16_t* srow = p.scale + n * p.s_cs;
     const uint16_t* orow = has_off ? p.offset + n * p.s_cs : nullptr;
 
-    // x staging: thread t copies 8 consecutive halves (16 bytes) per pass, permuted to the order [0,4,1,5,2,6,3,7]
-    // for int4 so that the pairs produced by the nibble splicing line up with natural pairs of x.
-    auto stage_x = [&](int slab, int buf) {
-        char* dst = sx + buf * XSLAB;
-        const int64_t k0 = (int64_t)slab * KX;
-        for (int idx = tid; idx < ROWS * (KX / 8); idx += 256) {
-            const int r = idx / (KX / 8), c = idx % (KX / 8);
-            const int64_t m = p.m_base + r, k = k0 + (int64_t)c * 8;
-            v4i v = {0, 0, 0, 0};
-            if (r < p.m_rows && k + 8 <= K) {
-                v = *(const v4i*)(p.x + m * K + k);
-            } else if (r < p.m_rows && k < K) {
-                uint16_t tmp[8];
+    // x staging: each thread moves XITEMS 16-byte pieces (8 consecutive halves) per slab; for int4 the halves are
+    // permuted to [0,4,1,5,2,6,3,7] so that the pairs produced by the nibble splicing line up with pairs of x.
+    v4i xreg[XITEMS];
+    auto load_x = [&](int slab) {
 #pragma unroll
-                for (int e = 0; e < 8; e++) tmp[e] = (k + e < K) ? p.x[m * K + k + e] : (uint16_t)0;
-                v = *(const v4i*)tmp;
-            }
+        for (int it = 0; it < XITEMS; it++) {
+            const int idx = it * 256 + tid;
+            const int r = idx / (KX / 8), c = idx % (KX / 8);
+            const int64_t m = p.m_base + r;
+            const int k = slab * KX + c * 8;
+            v4i v = {0, 0, 0, 0};
+            if (r < p.m_rows && k + 8 <= Ki) v = *(const v4i*)(p.x + m * p.K + k);   // K % 8 == 0 on this path
+            xreg[it] = v;
+        }
+    };
+    auto store_x = [&](int buf) {
+        char* dst = sx + buf * XSLAB;
+#pragma unroll
+        for (int it = 0; it < XITEMS; it++) {
+            const int idx = it * 256 + tid;
+            const int r = idx / (KX / 8), c = idx % (KX / 8);
+            v4i v = xreg[it];
             if constexpr (WBITS == 4) {
-                // halves h0..h7 -> [h0,h4,h1,h5,h2,h6,h3,h7]
                 const uint32_t a0 = (uint32_t)v[0], a1 = (uint32_t)v[1], a2 = (uint32_t)v[2], a3 = (uint32_t)v[3];
                 v4i o;
                 o[0] = (int)((a0 & 0xffffu) | (a2 << 16));          // h0, h4
@@ -155,15 +166,16 @@ __global__ __launch_bounds__(256, 2) void wqmm_decode_kernel(WqParams p)
 #pragma unroll
     for (int b = 0; b < MB; b++) acc[b] = (v4f){0.0f, 0.0f, 0.0f, 0.0f};
 
-    // weight pieces with their group's scale and offset, prefetched in groups of PF ahead of their use
+    // weight pieces with their group's scale and offset, fetched one super-step (PF chunks) ahead of their use;
+    // with WK > 1 a wave only touches the chunks c with c % WK == wk
     v4i wq[PF];
     uint16_t sq[PF], oq[PF];
-    const int Ki = (int)K, groupi = (int)p.group;
-    auto load_w = [&](int slab, int c0) {
+    auto load_w = [&](int c0) {
 #pragma unroll
         for (int i = 0; i < PF; i++) {
-            const int k = slab * KX + (c0 + i) * KC + g * KPL;
-            // K is a multiple of KPL on this path; pieces past K read the row's last piece and are masked below
+            if (WK > 1 && (i % WK) != wk) continue;
+            const int k = (c0 + i) * KC + g * KPL;
+            // K is a multiple of KPL on this path; pieces past K read the row's last piece and are masked when used
             const int kk = k < Ki ? k : Ki - KPL;
             wq[i] = n_ok ? *(const v4i*)(wrow + (int64_t)kk * WBITS / 8) : (v4i){0, 0, 0, 0};
             const int gi = p.group_shift >= 0 ? (kk >> p.group_shift) : (kk / groupi);
@@ -172,81 +184,104 @@ __global__ __launch_bounds__(256, 2) void wqmm_decode_kernel(WqParams p)
         }
     };
 
-    stage_x(0, 0);
-    load_w(0, 0);
-    __syncthreads();
+    const int NCHUNK = (Ki + KC - 1) / KC;
+    load_x(0);
+    load_w(0);
+    store_x(0);
+    if (NSLAB > 1) load_x(1);
 
-    for (int slab = 0; slab < NSLAB; slab++) {
-        const int buf = slab & 1;
-        if (slab + 1 < NSLAB) stage_x(slab + 1, buf ^ 1);
-        const char* xs = sx + buf * XSLAB;
+    for (int c0 = 0; c0 < NCHUNK; c0 += PF) {
+        v4i cur[PF];
+        uint16_t scur[PF], ocur[PF];
 #pragma unroll
-        for (int c0 = 0; c0 < CPS; c0 += PF) {
-            v4i cur[PF];
-            uint16_t scur[PF], ocur[PF];
+        for (int i = 0; i < PF; i++) { cur[i] = wq[i]; scur[i] = sq[i]; ocur[i] = oq[i]; }
+        if (c0 + PF < NCHUNK) load_w(c0 + PF);
 #pragma unroll
-            for (int i = 0; i < PF; i++) { cur[i] = wq[i]; scur[i] = sq[i]; ocur[i] = oq[i]; }
-            // prefetch the next group of pieces (next part of this slab, or the start of the next slab)
-            if (c0 + PF < CPS) load_w(slab, c0 + PF);
-            else if (slab + 1 < NSLAB) load_w(slab + 1, 0);
+        for (int i = 0; i < PF; i++) {
+            const int c = c0 + i;
+            if (i % CPS == 0) {
+                // slab boundary: every wave is done with the previous slab and sees the current one; the slab after
+                // it moves from registers to the buffer just vacated, and the one after that starts loading
+                const int slab = c / CPS;
+                __syncthreads();
+                if (slab + 1 < NSLAB) store_x((slab + 1) & 1);
+                if (slab + 2 < NSLAB) load_x(slab + 2);
+            }
+            if (WK > 1 && (i % WK) != wk) continue;
+            const int slab = c / CPS;
+            const char* xs = sx + (slab & 1) * XSLAB;
+            const int k = c * KC + g * KPL;   // first k of this lane's piece
+            const bool live = k < Ki;
+            const uint16_t sb = scur[i], ob = ocur[i];
 #pragma unroll
-            for (int i = 0; i < PF; i++) {
-                const int c = c0 + i;
-                const int k = slab * KX + c * KC + g * KPL;   // first k of this lane's piece
-                const bool live = k < Ki;
-                const uint16_t sb = scur[i], ob = ocur[i];
+            for (int s = 0; s < STEPS; s++) {
+                // operand A: this lane's 8 dequantised weights for MFMA step s
+                v4i aop;
+                if constexpr (XDT == DT_F16 && WBITS == 4) {
+                    const _Float16 sh = __builtin_bit_cast(_Float16, sb), oh = __builtin_bit_cast(_Float16, ob);
+                    h2 o4[4];
+                    dequant_i4_f16(live ? (uint32_t)cur[i][s] : 0x88888888u, (h2){oh, oh}, (h2){sh, sh}, has_off, o4);
+                    if (!live) { o4[0] = o4[1] = o4[2] = o4[3] = (h2){(_Float16)0.0f, (_Float16)0.0f}; }
+                    aop = (v4i){(int)u32(o4[0]), (int)u32(o4[1]), (int)u32(o4[2]), (int)u32(o4[3])};
+                } else {
+                    float scf, off;
+                    if constexpr (XDT == DT_F16) { scf = f16_to_f32(sb); off = f16_to_f32(ob); }
+                    else { scf = bf16_to_f32(sb); off = bf16_to_f32(ob); }
+                    uint16_t e[8];
+                    if constexpr (WBITS == 4) {
+                        const uint32_t q = (uint32_t)cur[i][s];
+                        const int ord[8] = {0, 4, 1, 5, 2, 6, 3, 7};   // element order of the staged x
 #pragma unroll
-                for (int s = 0; s < STEPS; s++) {
-                    // operand A: this lane's 8 dequantised weights for MFMA step s
-                    v4i aop;
-                    if constexpr (XDT == DT_F16 && WBITS == 4) {
-                        const _Float16 sh = __builtin_bit_cast(_Float16, sb), oh = __builtin_bit_cast(_Float16, ob);
-                        h2 o4[4];
-                        dequant_i4_f16(live ? (uint32_t)cur[i][s] : 0x88888888u, (h2){oh, oh}, (h2){sh, sh}, has_off, o4);
-                        if (!live) { o4[0] = o4[1] = o4[2] = o4[3] = (h2){(_Float16)0.0f, (_Float16)0.0f}; }
-                        aop = (v4i){(int)u32(o4[0]), (int)u32(o4[1]), (int)u32(o4[2]), (int)u32(o4[3])};
+                        for (int j = 0; j < 8; j++) {
+                            int v = (int)((q >> (4 * ord[j])) & 15u);
+                            v = v >= 8 ? v - 16 : v;
+                            e[j] = live ? bits_x<XDT>(dequant_one<XDT>((float)v, off, scf, has_off)) : (uint16_t)0;
+                        }
                     } else {
-                        float scf, off;
-                        if constexpr (XDT == DT_F16) { scf = f16_to_f32(sb); off = f16_to_f32(ob); }
-                        else { scf = bf16_to_f32(sb); off = bf16_to_f32(ob); }
-                        uint16_t e[8];
-                        if constexpr (WBITS == 4) {
-                            const uint32_t q = (uint32_t)cur[i][s];
-                            // element order [0,4,1,5,2,6,3,7] to match the staged x
-                            const int ord[8] = {0, 4, 1, 5, 2, 6, 3, 7};
+                        // int8: 16 bytes per piece, step s uses bytes 8s..8s+7 in natural order
 #pragma unroll
-                            for (int j = 0; j < 8; j++) {
-                                int v = (int)((q >> (4 * ord[j])) & 15u);
-                                v = v >= 8 ? v - 16 : v;
-                                e[j] = live ? bits_x<XDT>(dequant_one<XDT>((float)v, off, scf, has_off)) : (uint16_t)0;
-                            }
-                        } else {
-                            // int8: 16 bytes per piece, step s uses bytes 8s..8s+7 in natural order
-#pragma unroll
-                            for (int j = 0; j < 8; j++) {
-                                const uint32_t q = (uint32_t)cur[i][2 * s + (j >> 2)];
-                                const int v = (int)(int8_t)((q >> (8 * (j & 3))) & 0xffu);
-                                e[j] = live ? bits_x<XDT>(dequant_one<XDT>((float)v, off, scf, has_off)) : (uint16_t)0;
-                            }
+                        for (int j = 0; j < 8; j++) {
+                            const uint32_t q = (uint32_t)cur[i][2 * s + (j >> 2)];
+                            const int v = (int)(int8_t)((q >> (8 * (j & 3))) & 0xffu);
+                            e[j] = live ? bits_x<XDT>(dequant_one<XDT>((float)v, off, scf, has_off)) : (uint16_t)0;
                         }
-                        aop = (v4i){(int)(e[0] | ((uint32_t)e[1] << 16)), (int)(e[2] | ((uint32_t)e[3] << 16)),
-                                    (int)(e[4] | ((uint32_t)e[5] << 16)), (int)(e[6] | ((uint32_t)e[7] << 16))};
                     }
-                    // operand B: x[m = 16b + nrow][k = chunk + g*KPL + 8s + 0..7] (already permuted for int4)
-                    const int kofs = (c * KC + g * KPL + 8 * s) * 2;
+                    aop = (v4i){(int)(e[0] | ((uint32_t)e[1] << 16)), (int)(e[2] | ((uint32_t)e[3] << 16)),
+                                (int)(e[4] | ((uint32_t)e[5] << 16)), (int)(e[6] | ((uint32_t)e[7] << 16))};
+                }
+                // operand B: x[m = 16b + nrow][k = chunk + g*KPL + 8s + 0..7] (already permuted for int4)
+                const int kofs = ((c % CPS) * KC + g * KPL + 8 * s) * 2;
 #pragma unroll
-                    for (int b = 0; b < MB; b++) {
-                        const v4i bop = *(const v4i*)(xs + (16 * b + nrow) * XROW + kofs);
-                        if constexpr (XDT == DT_F16) {
-                            acc[b] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(v8h, aop), __builtin_bit_cast(v8h, bop), acc[b], 0, 0, 0);
-                        } else {
-                            acc[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf, aop), __builtin_bit_cast(v8bf, bop), acc[b], 0, 0, 0);
-                        }
+                for (int b = 0; b < MB; b++) {
+                    const v4i bop = *(const v4i*)(xs + (16 * b + nrow) * XROW + kofs);
+                    if constexpr (XDT == DT_F16) {
+                        acc[b] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(v8h, aop), __builtin_bit_cast(v8h, bop), acc[b], 0, 0, 0);
+                    } else {
+                        acc[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf, aop), __builtin_bit_cast(v8bf, bop), acc[b], 0, 0, 0);
                     }
                 }
             }
         }
+    }
+
+    if constexpr (WK > 1) {
+        // fixed-order reduction of the K-split partial sums: wave (wn, wk) parks its sums, wave (wn, 0) adds them
         __syncthreads();
+        float* red = (float*)sx;
+        if (wk > 0) {
+#pragma unroll
+            for (int b = 0; b < MB; b++)
+#pragma unroll
+                for (int i = 0; i < 4; i++) red[(((wn * (WK - 1) + (wk - 1)) * MB + b) * 4 + i) * 64 + lane] = acc[b][i];
+        }
+        __syncthreads();
+        if (wk > 0) return;
+#pragma unroll
+        for (int j = 0; j < WK - 1; j++)
+#pragma unroll
+            for (int b = 0; b < MB; b++)
+#pragma unroll
+                for (int i = 0; i < 4; i++) acc[b][i] = acc[b][i] + red[(((wn * (WK - 1) + j) * MB + b) * 4 + i) * 64 + lane];
     }
 
     // D'[row = weight row n][col = x row m]: lane holds col m = lane%16, rows n = 4*(lane/16) + i
@@ -256,24 +291,33 @@ __global__ __launch_bounds__(256, 2) void wqmm_decode_kernel(WqParams p)
         const int r = 16 * b + nrow;
         if (r >= p.m_rows) continue;
         const int64_t m = p.m_base + r;
+        float v[4];
 #pragma unroll
         for (int i = 0; i < 4; i++) {
             const int64_t nn = n0 + 4 * g + i;
-            if (nn >= p.N) continue;
-            float v = acc[b][i];
-            if (p.bias) v = v + load_scalar_as_f32(p.bias, p.bias_dt, nn);
-            if constexpr (XDT == DT_BF16) v = bf16_to_f32(bf16_bits(v));   // the golden rounds bf16 results twice (a no-op)
-            p.y[m * p.N + nn] = bits_x<XDT>(v);
+            v[i] = acc[b][i];
+            if (p.bias && nn < p.N) v[i] = v[i] + load_scalar_as_f32(p.bias, p.bias_dt, nn);
+            if constexpr (XDT == DT_BF16) v[i] = bf16_to_f32(bf16_bits(v[i]));   // the golden rounds bf16 results twice (a no-op)
+        }
+        const int64_t nn0 = n0 + 4 * g;
+        if (nn0 + 3 < p.N && (p.N % 4) == 0) {
+            const v4us o = {bits_x<XDT>(v[0]), bits_x<XDT>(v[1]), bits_x<XDT>(v[2]), bits_x<XDT>(v[3])};
+            *(v4us*)(p.y + m * p.N + nn0) = o;
+        } else {
+#pragma unroll
+            for (int i = 0; i < 4; i++)
+                if (nn0 + i < p.N) p.y[m * p.N + nn0 + i] = bits_x<XDT>(v[i]);
         }
     }
 }
 
-template <int XDT, int WBITS, int MB>
-static int launch_decode(const WqParams& p, unsigned grid, hipStream_t st)
+template <int XDT, int WBITS, int MB, int WK>
+static int launch_decode(const WqParams& p, hipStream_t st)
 {
-    constexpr int KX = 1024 / MB;
+    constexpr int KC = 4 * (128 / WBITS), KX = 8 * KC / MB, WN = 4 / WK;
     const size_t lds = 2 * (size_t)(16 * MB) * (KX * 2 + 16);
-    auto k = wqmm_decode_kernel<XDT, WBITS, MB>;
+    const unsigned grid = (unsigned)((p.N + 16 * WN - 1) / (16 * WN));
+    auto k = wqmm_decode_kernel<XDT, WBITS, MB, WK>;
     static bool attr_set = false;
     if (!attr_set) {
         hipError_t e = hipFuncSetAttribute((const void*)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
@@ -284,17 +328,27 @@ static int launch_decode(const WqParams& p, unsigned grid, hipStream_t st)
     return (int)hipGetLastError();
 }
 
+template <int XDT, int WBITS, int MB>
+static int launch_wk(const WqParams& p, hipStream_t st)
+{
+    // split K between the waves of a workgroup when column blocks alone would leave most of the chip idle
+    const int64_t nblocks = (p.N + 15) / 16;
+    static const int force = [] { const char* e = getenv("OPSNN_WQ_WK"); return e ? atoi(e) : 0; }();
+    const bool split = force ? force == 4 : (nblocks < 1024 && p.K >= 2048);
+    if (split) return launch_decode<XDT, WBITS, MB, 4>(p, st);
+    return launch_decode<XDT, WBITS, MB, 1>(p, st);
+}
+
 template <int XDT, int WBITS>
 static int launch_slabs(WqParams p, hipStream_t st)
 {
-    const unsigned grid = (unsigned)((p.N + 63) / 64);
     for (int64_t m0 = 0; m0 < p.M; m0 += 64) {
         p.m_base = m0;
         p.m_rows = (p.M - m0) < 64 ? (p.M - m0) : 64;
         int rc;
-        if (p.m_rows <= 16) rc = launch_decode<XDT, WBITS, 1>(p, grid, st);
-        else if (p.m_rows <= 32) rc = launch_decode<XDT, WBITS, 2>(p, grid, st);
-        else rc = launch_decode<XDT, WBITS, 4>(p, grid, st);
+        if (p.m_rows <= 16) rc = launch_wk<XDT, WBITS, 1>(p, st);
+        else if (p.m_rows <= 32) rc = launch_wk<XDT, WBITS, 2>(p, st);
+        else rc = launch_wk<XDT, WBITS, 4>(p, st);
         if (rc != 0) return rc;
     }
     return 0;
