@@ -51,6 +51,11 @@ __device__ __forceinline__ uint16_t to_b16(float f)
 // Four fp32 values -> four 16-bit floats (round to nearest even) using the packed hardware conversions.
 typedef __bf16 v2bf __attribute__((ext_vector_type(2)));
 typedef float v2f __attribute__((ext_vector_type(2)));
+// Two fp32 values -> packed bf16 pair (round to nearest even, v_cvt_pk_bf16_f32); element 0 in the low half.
+__device__ __forceinline__ uint32_t pack2_bf16(v2f v)
+{
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, v2bf));
+}
 template <int DT>
 __device__ __forceinline__ v4us pack4_b16(v4f v)
 {

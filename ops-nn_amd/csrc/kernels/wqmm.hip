@@ -23,73 +23,11 @@
 //   - x is staged through LDS in K slabs shared by the workgroup's four waves, already permuted into the element
 //     order the nibble splicing produces, so no weight register ever needs a shuffle.
 // M > 64 is processed in row slabs of 64 (the weight is re-streamed per slab; such shapes are compute-bound).
-#include "launch.h"
-#include "qgemm_core.hip.h"
+#include "wqmm_stream.hip.h"
 
 namespace opsnn {
 
 int launch_wqmm_plain(const OpsnnWqmmArgs& a, hipStream_t st);
-
-struct WqParams {
-    const uint16_t* x;       // [M, K] dense 16-bit
-    const uint8_t* w;        // row n at w + n*ldw (bytes), K-contiguous
-    int64_t ldw;
-    const uint16_t* scale;   // element (g, n) at scale[g*s_rs + n*s_cs]
-    const uint16_t* offset;  // same layout, or null
-    int64_t s_rs, s_cs;
-    const void* bias;
-    int bias_dt;
-    uint16_t* y;             // [M, N]
-    int64_t M, N, K;
-    int64_t group;           // elements per group (K if per-channel)
-    int group_shift;         // log2(group) if it is a power of two, else -1
-    int64_t m_base, m_rows;  // row slab handled by this launch
-};
-
-typedef _Float16 h2 __attribute__((ext_vector_type(2)));
-
-__device__ __forceinline__ uint32_t u32(h2 v) { return __builtin_bit_cast(uint32_t, v); }
-
-// ---- fp16 dequantisation: 8 int4 of one dword -> 4 packed pairs in element order [0,4], [1,5], [2,6], [3,7] ----
-// q holds two's-complement nibbles; after xor 0x88888888 each nibble is w + 8 in 0..15.
-__device__ __forceinline__ void dequant_i4_f16(uint32_t q, h2 off, h2 sc, bool has_off, h2 (&out)[4])
-{
-    const uint32_t u = q ^ 0x88888888u;
-    const uint32_t u8 = u >> 8;
-    const h2 c1032 = {(_Float16)-1032.0f, (_Float16)-1032.0f};
-    const h2 c72 = {(_Float16)-72.0f, (_Float16)-72.0f};
-    const h2 r16 = {(_Float16)0.0625f, (_Float16)0.0625f};
-    h2 t0 = __builtin_bit_cast(h2, (u & 0x000F000Fu) | 0x64006400u);   // 1024 + (w+8)        elements 0, 4
-    h2 t1 = __builtin_bit_cast(h2, (u & 0x00F000F0u) | 0x64006400u);   // 1024 + 16*(w+8)     elements 1, 5
-    h2 t2 = __builtin_bit_cast(h2, (u8 & 0x000F000Fu) | 0x64006400u);  //                     elements 2, 6
-    h2 t3 = __builtin_bit_cast(h2, (u8 & 0x00F000F0u) | 0x64006400u);  //                     elements 3, 7
-    t0 = t0 + c1032;                                   // exact: w
-    t2 = t2 + c1032;
-    t1 = __builtin_elementwise_fma(t1, r16, c72);      // exact: (1024 + 16(w+8))/16 - 72 = w
-    t3 = __builtin_elementwise_fma(t3, r16, c72);
-    if (has_off) { t0 = t0 + off; t1 = t1 + off; t2 = t2 + off; t3 = t3 + off; }   // first rounding
-    out[0] = t0 * sc; out[1] = t1 * sc; out[2] = t2 * sc; out[3] = t3 * sc;         // second rounding
-}
-
-// ---- generic dequantisation of one weight to fp32 holding a value of x's dtype ----
-template <int XDT>
-__device__ __forceinline__ float round_x(float v)
-{
-    if constexpr (XDT == DT_F16) return (float)(_Float16)v;
-    else return bf16_to_f32(bf16_bits(v));
-}
-template <int XDT>
-__device__ __forceinline__ uint16_t bits_x(float v)
-{
-    if constexpr (XDT == DT_F16) return f16_bits(v);
-    else return bf16_bits(v);
-}
-template <int XDT>
-__device__ __forceinline__ float dequant_one(float w, float off, float sc, bool has_off)
-{
-    if (has_off) w = round_x<XDT>(w + off);
-    return round_x<XDT>(w * sc);
-}
 
 // MB: 16-row blocks of x handled per launch slab (1, 2 or 4).  WBITS: 4 or 8.
 // WK: waves of the workgroup that split K between them (1, 2 or 4); the other 4/WK waves take different column
@@ -333,20 +271,50 @@ static int launch_wk(const WqParams& p, hipStream_t st)
 {
     // split K between the waves of a workgroup when column blocks alone would leave most of the chip idle
     const int64_t nblocks = (p.N + 15) / 16;
-    static const int force = [] { const char* e = getenv("OPSNN_WQ_WK"); return e ? atoi(e) : 0; }();
-    const bool split = force ? force == 4 : (nblocks < 1024 && p.K >= 2048);
-    if (split) return launch_decode<XDT, WBITS, MB, 4>(p, st);
+    if (nblocks < 1024 && p.K >= 2048) return launch_decode<XDT, WBITS, MB, 4>(p, st);
     return launch_decode<XDT, WBITS, MB, 1>(p, st);
+}
+
+template <> int launch_wq_stream<DT_F16, 4>(const WqParams&, const WqStreamOpts&, hipStream_t);
+template <> int launch_wq_stream<DT_F16, 8>(const WqParams&, const WqStreamOpts&, hipStream_t);
+template <> int launch_wq_stream<DT_BF16, 4>(const WqParams&, const WqStreamOpts&, hipStream_t);
+template <> int launch_wq_stream<DT_BF16, 8>(const WqParams&, const WqStreamOpts&, hipStream_t);
+
+// Can the streamlined kernel take this problem, and in which form?
+template <int WBITS>
+static bool stream_eligible(WqParams& p, WqStreamOpts& o)
+{
+    constexpr int64_t KC = 4 * (128 / WBITS);
+    static const bool off = [] { const char* e = getenv("OPSNN_WQ_GENERAL"); return e && e[0] == '1'; }();
+    if (off || p.K % KC != 0) return false;
+    const int64_t nch = p.K / KC;
+    if (p.group >= p.K) p.cpg_shift = 31;
+    else {
+        if (p.group % KC != 0) return false;
+        const int64_t cpg = p.group / KC;
+        if (cpg & (cpg - 1)) return false;
+        p.cpg_shift = __builtin_ctzll((unsigned long long)cpg);
+    }
+    o.has_off = p.offset != nullptr;
+    const int64_t nblocks = (p.N + 15) / 16;
+    o.ksplit = p.M <= 16 && nblocks < 1024 && nch % 4 == 0 && nch >= 8;
+    const int64_t ngroups = p.group >= p.K ? 1 : p.K / p.group;
+    o.vscale = !o.ksplit && p.group == KC && p.s_rs == 1 && p.s_cs % 8 == 0 && ngroups % 8 == 0 &&
+               (uintptr_t)p.scale % 16 == 0 && (!p.offset || (uintptr_t)p.offset % 16 == 0);
+    return true;
 }
 
 template <int XDT, int WBITS>
 static int launch_slabs(WqParams p, hipStream_t st)
 {
+    WqStreamOpts o{};
+    const bool stream = stream_eligible<WBITS>(p, o);
     for (int64_t m0 = 0; m0 < p.M; m0 += 64) {
         p.m_base = m0;
         p.m_rows = (p.M - m0) < 64 ? (p.M - m0) : 64;
         int rc;
-        if (p.m_rows <= 16) rc = launch_wk<XDT, WBITS, 1>(p, st);
+        if (stream) rc = launch_wq_stream<XDT, WBITS>(p, o, st);
+        else if (p.m_rows <= 16) rc = launch_wk<XDT, WBITS, 1>(p, st);
         else if (p.m_rows <= 32) rc = launch_wk<XDT, WBITS, 2>(p, st);
         else rc = launch_wk<XDT, WBITS, 4>(p, st);
         if (rc != 0) return rc;

@@ -1,0 +1,367 @@
+// Weight-only decode kernel, streamlined form: the shapes it takes are restricted so that the inner loop carries
+// nothing but the essential work -- per 8 weights of a lane: the dequantisation (18 packed-fp16 / integer
+// operations with an offset, 14 without), one 16-byte LDS read of x and one v_mfma_f32_16x16x32.
+//
+// Restrictions (the launcher checks them; anything else goes to the general kernel in wqmm.hip):
+//   K is a multiple of the chunk KC (128 int4 / 64 int8 weights: what one wave load instruction covers per row);
+//   the group size is a power-of-two multiple of KC, or the scale is per channel;
+//   VSCALE: group == KC, a row's scales contiguous and 16-byte aligned, K/group a multiple of 8 -- then one
+//           16-byte load per lane brings the scales of the next 8 chunks.
+//
+// Work split: a wave owns 16 weight rows (output columns).  WK = 1: the four waves of a workgroup take four row
+// blocks and all of K.  WK = 4: they take one row block and every fourth chunk each (narrow N), and their partial
+// sums meet in LDS in a fixed order.  Either way all four waves walk the same K slabs of x, staged once per
+// workgroup in LDS (only the rows that exist, plus one zero row that the idle MFMA columns read).
+//
+// Weight pieces are fetched 8 chunks ahead: the register that a chunk has just been consumed from is reloaded
+// with the chunk 8 further on, so 8 loads per lane are always in flight without a second register set.
+#pragma once
+#include "wqmm_common.hip.h"
+
+namespace opsnn {
+
+// ---- 8 consecutive-k weights of one lane -> MFMA row operand (8 values of x's dtype) ----
+// piece: the lane's 16-byte weight piece; s: which 8 of its weights (int4: dword s, element order
+// [0,4,1,5,2,6,3,7] matched by the staged x; int8: dwords 2s, 2s+1 in natural order).
+struct DqConst {
+    uint32_t mlo, mhi, clo, chi;   // int4 splice masks and exponent/sign constants, held in registers
+};
+__device__ __forceinline__ DqConst make_dq_const()
+{
+    DqConst c = {0x000F000Fu, 0x00F000F0u, 0x64086408u, 0x64806480u};
+    asm volatile("" : "+v"(c.mlo), "+v"(c.mhi), "+v"(c.clo), "+v"(c.chi));   // not literals: see dequant8
+    return c;
+}
+
+template <int XDT, int WBITS, bool HAS_OFF>
+__device__ __forceinline__ v4i dequant8(const v4i& piece, int s, uint16_t sb, uint16_t ob, const DqConst& dc)
+{
+    if constexpr (XDT == DT_F16) {
+        const _Float16 sh = __builtin_bit_cast(_Float16, sb), oh = __builtin_bit_cast(_Float16, ob);
+        const h2 sc = {sh, sh}, off = {oh, oh};
+        h2 t0, t1, t2, t3;
+        if constexpr (WBITS == 4) {
+            // (q & mask) ^ c flips each nibble's sign bit (w + 8 in 0..15) and sets the exponent of 1024.0 in one
+            // three-operand bit operation; the constants are kept in registers so that it stays one instruction
+            const uint32_t q = (uint32_t)piece[s], q8 = q >> 8;
+            const uint32_t mlo = dc.mlo, mhi = dc.mhi, clo = dc.clo, chi = dc.chi;
+            const h2 c1032 = {(_Float16)-1032.0f, (_Float16)-1032.0f};
+            const h2 c72 = {(_Float16)-72.0f, (_Float16)-72.0f};
+            const h2 r16 = {(_Float16)0.0625f, (_Float16)0.0625f};
+            t0 = __builtin_bit_cast(h2, (q & mlo) ^ clo);     // 1024 + (w+8): elements 0, 4
+            t1 = __builtin_bit_cast(h2, (q & mhi) ^ chi);     // 1024 + 16(w+8): elements 1, 5
+            t2 = __builtin_bit_cast(h2, (q8 & mlo) ^ clo);    // elements 2, 6
+            t3 = __builtin_bit_cast(h2, (q8 & mhi) ^ chi);    // elements 3, 7
+            t0 = t0 + c1032;                                // exact
+            t2 = t2 + c1032;
+            t1 = __builtin_elementwise_fma(t1, r16, c72);   // exact: (1024 + 16(w+8))/16 - 72
+            t3 = __builtin_elementwise_fma(t3, r16, c72);
+        } else {
+            // bytes become w + 128 in 0..255 and are spliced under the exponent byte of 1024.0
+            const uint32_t qa = (uint32_t)piece[2 * s] ^ 0x80808080u, qb = (uint32_t)piece[2 * s + 1] ^ 0x80808080u;
+            const uint32_t magic = 0x64646464u;
+            const h2 c1152 = {(_Float16)-1152.0f, (_Float16)-1152.0f};
+            t0 = __builtin_bit_cast(h2, __builtin_amdgcn_perm(magic, qa, 0x04010400u)) + c1152;   // elements 0, 1
+            t1 = __builtin_bit_cast(h2, __builtin_amdgcn_perm(magic, qa, 0x04030402u)) + c1152;   // elements 2, 3
+            t2 = __builtin_bit_cast(h2, __builtin_amdgcn_perm(magic, qb, 0x04010400u)) + c1152;   // elements 4, 5
+            t3 = __builtin_bit_cast(h2, __builtin_amdgcn_perm(magic, qb, 0x04030402u)) + c1152;   // elements 6, 7
+        }
+        if constexpr (HAS_OFF) { t0 = t0 + off; t1 = t1 + off; t2 = t2 + off; t3 = t3 + off; }   // first rounding
+        t0 = t0 * sc; t1 = t1 * sc; t2 = t2 * sc; t3 = t3 * sc;                                  // second rounding
+        return (v4i){(int)u32(t0), (int)u32(t1), (int)u32(t2), (int)u32(t3)};
+    } else {
+        // bf16: no packed bf16 arithmetic on this chip, so the two steps run in fp32 with a hardware
+        // round-to-nearest-even conversion to bf16 after each
+        const float scf = bf16_to_f32(sb), off = bf16_to_f32(ob);
+        float w[8];
+        if constexpr (WBITS == 4) {
+            const uint32_t q = (uint32_t)piece[s];
+            const int ord[8] = {0, 4, 1, 5, 2, 6, 3, 7};
+#pragma unroll
+            for (int j = 0; j < 8; j++) w[j] = (float)(((int)(q << (28 - 4 * ord[j]))) >> 28);
+        } else {
+#pragma unroll
+            for (int j = 0; j < 8; j++) w[j] = (float)(((int)((uint32_t)piece[2 * s + (j >> 2)] << (24 - 8 * (j & 3)))) >> 24);
+        }
+        v4i r;
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            float a = w[2 * j], b = w[2 * j + 1];
+            if constexpr (HAS_OFF) {
+                const v2f t = {a + off, b + off};
+                const uint32_t pk = pack2_bf16(t);
+                a = __builtin_bit_cast(float, pk << 16);
+                b = __builtin_bit_cast(float, pk & 0xffff0000u);
+            }
+            const v2f t = {a * scf, b * scf};
+            r[j] = (int)pack2_bf16(t);
+        }
+        return r;
+    }
+}
+
+template <int XDT, int WBITS, int MB, int WK, bool HAS_OFF, bool VSCALE>
+__global__ __launch_bounds__(256, 2) void wqmm_stream_kernel(WqParams p)
+{
+    static_assert(!(VSCALE && WK != 1), "vector scale loads need consecutive chunks per wave");
+    constexpr int WN = 4 / WK;
+    constexpr int KPL = 128 / WBITS;     // k per 16-byte piece: 32 or 16
+    constexpr int KC = 4 * KPL;          // k per chunk: 128 or 64 (64 bytes of a weight row either way)
+    constexpr int STEPS = KC / 32;       // MFMA steps per chunk: 4 or 2
+    constexpr int PF = 8;                // chunks per super-step = pieces in flight per lane
+    constexpr int KX = PF * KC / MB;     // k per LDS slab of x
+    constexpr int CPS = KX / KC;         // chunks per slab: 8, 4, 2
+    constexpr int CPSW = CPS / WK;       // of which this wave's
+    static_assert(CPSW >= 1, "a slab must hold at least one chunk per K-split wave");
+    constexpr int XROW = KX * 2 + 16;    // LDS row pitch (bytes); the pad makes the 16-byte reads conflict free
+    constexpr int XPR = KX / 8;          // 16-byte pieces per x row per slab
+    constexpr int XITEMS = 16 * MB * XPR / 256;
+    extern __shared__ __attribute__((aligned(16))) char sx[];
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wn = wave / WK, wk = wave % WK;
+    const int nrow = lane & 15, g = lane >> 4;
+    const int64_t n0 = ((int64_t)blockIdx.x * WN + wn) * 16;
+    const bool n_ok = n0 < p.N;
+    const int64_t n = (n0 + nrow) < p.N ? (n0 + nrow) : p.N - 1;   // rows past the edge recompute the last one
+    const int Ki = (int)p.K;
+    const int NCW = Ki / (KC * WK);      // this wave's chunks: chunk index = cw * WK + wk
+    const int NSLAB = (Ki + KX - 1) / KX;
+    const int rows = (int)p.m_rows;      // 1 .. 16*MB rows of x in this launch
+    const int xslab = (rows + 1) * XROW; // + the zero row
+
+    const uint8_t* wptr = p.w + n * p.ldw + g * 16 + wk * 64;
+    const uint16_t* srow = p.scale + n * p.s_cs;
+    const uint16_t* orow = HAS_OFF ? p.offset + n * p.s_cs : nullptr;
+
+    // ---- x staging ----
+    v4i xreg[XITEMS];
+    const int xtotal = rows * XPR;
+    auto load_x = [&](int slab) {
+#pragma unroll
+        for (int it = 0; it < XITEMS; it++) {
+            const int idx = it * 256 + tid;
+            if (it * 256 >= xtotal) break;
+            const int r = idx / XPR, c = idx % XPR;
+            const int k = slab * KX + c * 8;
+            v4i v = {0, 0, 0, 0};
+            if (idx < xtotal && k < Ki) v = *(const v4i*)(p.x + (p.m_base + r) * p.K + k);
+            xreg[it] = v;
+        }
+    };
+    auto store_x = [&](int buf) {
+        char* dst = sx + buf * xslab;
+#pragma unroll
+        for (int it = 0; it < XITEMS; it++) {
+            const int idx = it * 256 + tid;
+            if (it * 256 >= xtotal) break;
+            const int r = idx / XPR, c = idx % XPR;
+            v4i v = xreg[it];
+            if constexpr (WBITS == 4 && XDT == DT_F16) {
+                // halves [0..7] -> [0,4,1,5,2,6,3,7]: the order in which the nibble splicing yields pairs
+                const uint32_t a0 = (uint32_t)v[0], a1 = (uint32_t)v[1], a2 = (uint32_t)v[2], a3 = (uint32_t)v[3];
+                v = (v4i){(int)__builtin_amdgcn_perm(a2, a0, 0x05040100u), (int)__builtin_amdgcn_perm(a2, a0, 0x07060302u),
+                          (int)__builtin_amdgcn_perm(a3, a1, 0x05040100u), (int)__builtin_amdgcn_perm(a3, a1, 0x07060302u)};
+            } else if constexpr (WBITS == 4) {
+                const uint32_t a0 = (uint32_t)v[0], a1 = (uint32_t)v[1], a2 = (uint32_t)v[2], a3 = (uint32_t)v[3];
+                v = (v4i){(int)__builtin_amdgcn_perm(a2, a0, 0x05040100u), (int)__builtin_amdgcn_perm(a2, a0, 0x07060302u),
+                          (int)__builtin_amdgcn_perm(a3, a1, 0x05040100u), (int)__builtin_amdgcn_perm(a3, a1, 0x07060302u)};
+            }
+            if (idx < xtotal) *(v4i*)(dst + r * XROW + c * 16) = v;
+        }
+    };
+    // the zero row of both buffers
+    for (int i = tid; i < 2 * (XROW / 16); i += 256) {
+        const int buf = i / (XROW / 16), c = i % (XROW / 16);
+        *(v4i*)(sx + buf * xslab + rows * XROW + c * 16) = (v4i){0, 0, 0, 0};
+    }
+    // LDS byte offset of this lane's column operand inside a slab buffer, per 16-row block
+    int xoff[MB];
+#pragma unroll
+    for (int b = 0; b < MB; b++) {
+        const int r = 16 * b + nrow;
+        xoff[b] = (r < rows ? r : rows) * XROW + g * KPL * 2;
+    }
+
+    v4f acc[MB];
+#pragma unroll
+    for (int b = 0; b < MB; b++) acc[b] = (v4f){0.0f, 0.0f, 0.0f, 0.0f};
+    const DqConst dqc = make_dq_const();
+
+    // ---- weight / scale prefetch state ----
+    v4i wq[PF];
+    uint16_t sq[PF], oq[PF];   // !VSCALE: scale and offset of each chunk in flight
+    v4i sv, ov, svn, ovn;      // VSCALE: the 8 scales (offsets) of this and of the next super-step
+    sv = ov = svn = ovn = (v4i){0, 0, 0, 0};
+    auto group_of = [&](int cw) { return ((cw * WK + wk) >> p.cpg_shift); };   // cpg_shift = 31 for per-channel
+    auto fetch = [&](int j, int cw) {   // chunk cw of this wave into slot j
+        wq[j] = *(const v4i*)(wptr + (int64_t)cw * (WK * 64));
+        if constexpr (!VSCALE) {
+            const int64_t so = (int64_t)group_of(cw) * p.s_rs;
+            sq[j] = srow[so];
+            if constexpr (HAS_OFF) oq[j] = orow[so];
+        }
+    };
+#pragma unroll
+    for (int j = 0; j < PF; j++) fetch(j, j < NCW ? j : NCW - 1);
+    if constexpr (VSCALE) {
+        svn = *(const v4i*)srow;
+        if constexpr (HAS_OFF) ovn = *(const v4i*)orow;
+    }
+    load_x(0);
+    store_x(0);
+    if (NSLAB > 1) load_x(1);
+
+    // one super-step: this wave's chunks c0 .. c0+7.  TAIL: some of them may not exist and the refills are clamped.
+    auto superstep = [&](int c0, auto tail_tag) {
+        constexpr bool TAIL = decltype(tail_tag)::value;
+        if constexpr (VSCALE) {
+            sv = svn; ov = ovn;
+            if (c0 + PF < NCW) {
+                svn = *(const v4i*)(srow + c0 + PF);
+                if constexpr (HAS_OFF) ovn = *(const v4i*)(orow + c0 + PF);
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < PF; j++) {
+            const int cw = c0 + j;
+            if (j % CPSW == 0) {
+                // slab boundary: every wave has finished the previous slab and sees this one; the next slab moves
+                // from registers into the buffer just vacated and the one after it starts loading
+                const int slab = cw / CPSW;
+                if (!TAIL || slab < NSLAB) {
+                    __syncthreads();
+                    if (slab + 1 < NSLAB) store_x((slab + 1) & 1);
+                    if (slab + 2 < NSLAB) load_x(slab + 2);
+                }
+            }
+            if (TAIL && cw >= NCW) continue;
+            const int slab = cw / CPSW;
+            const char* xs = sx + (slab & 1) * xslab + ((cw % CPSW) * WK + wk) * (KC * 2);
+            uint16_t sb, ob = 0;
+            if constexpr (VSCALE) {
+                sb = (uint16_t)((uint32_t)sv[j / 2] >> (16 * (j % 2)));
+                if constexpr (HAS_OFF) ob = (uint16_t)((uint32_t)ov[j / 2] >> (16 * (j % 2)));
+            } else {
+                sb = sq[j];
+                if constexpr (HAS_OFF) ob = oq[j];
+            }
+#pragma unroll
+            for (int s = 0; s < STEPS; s++) {
+                const v4i aop = dequant8<XDT, WBITS, HAS_OFF>(wq[j], s, sb, ob, dqc);
+#pragma unroll
+                for (int b = 0; b < MB; b++) {
+                    const v4i bop = *(const v4i*)(xs + xoff[b] + 16 * s);
+                    if constexpr (XDT == DT_F16) {
+                        acc[b] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(v8h, aop), __builtin_bit_cast(v8h, bop), acc[b], 0, 0, 0);
+                    } else {
+                        acc[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf, aop), __builtin_bit_cast(v8bf, bop), acc[b], 0, 0, 0);
+                    }
+                }
+            }
+            // refill the slot with the chunk 8 further on
+            if constexpr (TAIL) {
+                const int nx = cw + PF;
+                fetch(j, nx < NCW ? nx : NCW - 1);
+            } else {
+                fetch(j, cw + PF);
+            }
+        }
+    };
+
+    int c0 = 0;
+    for (; c0 + 2 * PF <= NCW; c0 += PF) superstep(c0, std::false_type{});
+    for (; c0 < NCW; c0 += PF) superstep(c0, std::true_type{});
+
+    if constexpr (WK > 1) {
+        __syncthreads();
+        float* red = (float*)sx;
+        if (wk > 0) {
+#pragma unroll
+            for (int b = 0; b < MB; b++)
+#pragma unroll
+                for (int i = 0; i < 4; i++) red[(((wn * (WK - 1) + (wk - 1)) * MB + b) * 4 + i) * 64 + lane] = acc[b][i];
+        }
+        __syncthreads();
+        if (wk > 0) return;
+#pragma unroll
+        for (int j = 0; j < WK - 1; j++)
+#pragma unroll
+            for (int b = 0; b < MB; b++)
+#pragma unroll
+                for (int i = 0; i < 4; i++) acc[b][i] = acc[b][i] + red[(((wn * (WK - 1) + j) * MB + b) * 4 + i) * 64 + lane];
+    }
+
+    // D'[row = weight row n][col = x row m]: lane holds col m = lane%16, rows n = 4*(lane/16) + i
+    if (!n_ok) return;
+#pragma unroll
+    for (int b = 0; b < MB; b++) {
+        const int r = 16 * b + nrow;
+        if (r >= rows) continue;
+        const int64_t m = p.m_base + r;
+        float v[4];
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const int64_t nn = n0 + 4 * g + i;
+            v[i] = acc[b][i];
+            if (p.bias && nn < p.N) v[i] = v[i] + load_scalar_as_f32(p.bias, p.bias_dt, nn);
+            if constexpr (XDT == DT_BF16) v[i] = bf16_to_f32(bf16_bits(v[i]));   // the golden rounds bf16 results twice (a no-op)
+        }
+        const int64_t nn0 = n0 + 4 * g;
+        if (nn0 + 3 < p.N && (p.N % 4) == 0) {
+            const v4us o = {bits_x<XDT>(v[0]), bits_x<XDT>(v[1]), bits_x<XDT>(v[2]), bits_x<XDT>(v[3])};
+            *(v4us*)(p.y + m * p.N + nn0) = o;
+        } else {
+#pragma unroll
+            for (int i = 0; i < 4; i++)
+                if (nn0 + i < p.N) p.y[m * p.N + nn0 + i] = bits_x<XDT>(v[i]);
+        }
+    }
+}
+
+template <int XDT, int WBITS, int MB, int WK, bool HAS_OFF, bool VSCALE>
+static int launch_stream_one(const WqParams& p, hipStream_t st)
+{
+    constexpr int KC = 4 * (128 / WBITS), KX = 8 * KC / MB, WN = 4 / WK;
+    const size_t lds_x = 2 * (size_t)(p.m_rows + 1) * (KX * 2 + 16);
+    const size_t lds_red = WK > 1 ? (size_t)WN * (WK - 1) * MB * 4 * 64 * 4 : 0;
+    const size_t lds = lds_x > lds_red ? lds_x : lds_red;
+    const unsigned grid = (unsigned)((p.N + 16 * WN - 1) / (16 * WN));
+    auto k = wqmm_stream_kernel<XDT, WBITS, MB, WK, HAS_OFF, VSCALE>;
+    static bool attr_set = false;
+    if (!attr_set) {
+        constexpr size_t lds_max = 2 * (size_t)(16 * MB + 1) * (KX * 2 + 16);
+        hipError_t e = hipFuncSetAttribute((const void*)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_max);
+        if (e != hipSuccess) return (int)e;
+        attr_set = true;
+    }
+    hipLaunchKernelGGL(k, dim3(grid), dim3(256), lds, st, p);
+    return (int)hipGetLastError();
+}
+
+struct WqStreamOpts {
+    bool has_off, vscale, ksplit;
+};
+
+// One row slab (p.m_rows <= 64) of one dtype pair; defined once per pair in its own translation unit.
+template <int XDT, int WBITS>
+int launch_wq_stream(const WqParams& p, const WqStreamOpts& o, hipStream_t st);
+
+#define OPSNN_WQ_STREAM_DEFINE(XDT, WBITS)                                                                          \
+    template <int MB, int WK, bool VS>                                                                              \
+    static int wq_stream_off(const WqParams& p, bool has_off, hipStream_t st)                                       \
+    {                                                                                                               \
+        return has_off ? launch_stream_one<XDT, WBITS, MB, WK, true, VS>(p, st)                                     \
+                       : launch_stream_one<XDT, WBITS, MB, WK, false, VS>(p, st);                                   \
+    }                                                                                                               \
+    template <>                                                                                                     \
+    int launch_wq_stream<XDT, WBITS>(const WqParams& p, const WqStreamOpts& o, hipStream_t st)                      \
+    {                                                                                                               \
+        if (o.ksplit && p.m_rows <= 16) return wq_stream_off<1, 4, false>(p, o.has_off, st);                        \
+        if (p.m_rows <= 16) return o.vscale ? wq_stream_off<1, 1, true>(p, o.has_off, st) : wq_stream_off<1, 1, false>(p, o.has_off, st); \
+        if (p.m_rows <= 32) return o.vscale ? wq_stream_off<2, 1, true>(p, o.has_off, st) : wq_stream_off<2, 1, false>(p, o.has_off, st); \
+        return o.vscale ? wq_stream_off<4, 1, true>(p, o.has_off, st) : wq_stream_off<4, 1, false>(p, o.has_off, st); \
+    }
+
+}  // namespace opsnn

@@ -118,6 +118,23 @@ def test_mx_batched(gpu):
     (5, 256, 64, "f16", "i8", 32, True, False, None),
     (33, 864, 212, "f16", "i4", 96, False, True, None),         # ragged groups (864 = 9 * 96)
     (4, 256, 128, "bf16", "e4m3", 0, True, False, "bf16"),
+    # shapes the streamlined decode kernel takes: vector scale loads (group 128 int4, K/128 a multiple of 8) ...
+    (1, 2048, 528, "f16", "i4", 128, True, True, None),
+    (16, 3072, 272, "f16", "i4", 128, True, False, "f16"),
+    (32, 1024, 260, "f16", "i4", 128, True, True, None),
+    (64, 2048, 256, "f16", "i4", 128, True, True, "f16"),
+    (48, 1024, 256, "bf16", "i4", 128, True, True, None),
+    (16, 1024, 256, "f16", "i8", 64, True, True, None),
+    # ... scalar scale loads: wider groups, ragged chunk counts, N-contiguous weight, per-channel
+    (3, 1280, 144, "f16", "i4", 256, True, True, None),
+    (20, 1280, 144, "f16", "i4", 256, False, False, None),
+    (16, 1152, 8208, "f16", "i4", 128, True, True, None),       # 9 groups: not a multiple of 8; 513 row blocks
+    (9, 640, 96, "bf16", "i8", 128, True, True, "bf16"),
+    (64, 1024, 320, "bf16", "i8", 0, True, False, None),
+    # ... K split between the waves of a workgroup (narrow N, M <= 16)
+    (16, 4096, 256, "bf16", "i8", 0, True, False, None),
+    (1, 4096, 200, "f16", "i4", 128, True, True, "f16"),
+    (11, 2048, 64, "f16", "i8", 0, False, True, None),
 ])
 def test_weight_only(gpu, M, K, N, x_dt, w_dt, group, tW, off, bias, use_plain):
     m = gpu
