@@ -301,6 +301,11 @@ static bool stream_eligible(WqParams& p, WqStreamOpts& o)
     const int64_t ngroups = p.group >= p.K ? 1 : p.K / p.group;
     o.vscale = !o.ksplit && p.group == KC && p.s_rs == 1 && p.s_cs % 8 == 0 && ngroups % 8 == 0 &&
                (uintptr_t)p.scale % 16 == 0 && (!p.offset || (uintptr_t)p.offset % 16 == 0);
+    // few rows: x whole in LDS (<= 64 KB), K in four contiguous quarters per workgroup
+    static const bool no_resx = [] { const char* e = getenv("OPSNN_WQ_NO_RESX"); return e && e[0] == '1'; }();
+    o.resx = !no_resx && p.M <= 16 && nch % 4 == 0 && (p.M + 1) * (p.K * 2 + 16) <= 65536;
+    o.resx_vscale = o.resx && p.group == KC && p.s_rs == 1 && p.s_cs % 8 == 0 && (nch / 4) % 8 == 0 &&
+                    (uintptr_t)p.scale % 16 == 0 && (!p.offset || (uintptr_t)p.offset % 16 == 0);
     return true;
 }
 

@@ -17,6 +17,9 @@
 // with the chunk 8 further on, so 8 loads per lane are always in flight without a second register set.
 #pragma once
 #include "wqmm_common.hip.h"
+#ifndef WQ_ABL
+#define WQ_ABL 0
+#endif
 
 namespace opsnn {
 
@@ -108,8 +111,12 @@ __global__ __launch_bounds__(256, 2) void wqmm_stream_kernel(WqParams p)
     constexpr int KPL = 128 / WBITS;     // k per 16-byte piece: 32 or 16
     constexpr int KC = 4 * KPL;          // k per chunk: 128 or 64 (64 bytes of a weight row either way)
     constexpr int STEPS = KC / 32;       // MFMA steps per chunk: 4 or 2
-    constexpr int PF = 8;                // chunks per super-step = pieces in flight per lane
-    constexpr int KX = PF * KC / MB;     // k per LDS slab of x
+#ifdef WQ_PF
+    constexpr int PF = WQ_PF;
+#else
+    constexpr int PF = (MB == 1 && WK == 1) ? 16 : 8;   // chunks per super-step = pieces in flight per lane
+#endif
+    constexpr int KX = 8 * KC / MB;      // k per LDS slab of x
     constexpr int CPS = KX / KC;         // chunks per slab: 8, 4, 2
     constexpr int CPSW = CPS / WK;       // of which this wave's
     static_assert(CPSW >= 1, "a slab must hold at least one chunk per K-split wave");
@@ -192,8 +199,10 @@ __global__ __launch_bounds__(256, 2) void wqmm_stream_kernel(WqParams p)
     // ---- weight / scale prefetch state ----
     v4i wq[PF];
     uint16_t sq[PF], oq[PF];   // !VSCALE: scale and offset of each chunk in flight
-    v4i sv, ov, svn, ovn;      // VSCALE: the 8 scales (offsets) of this and of the next super-step
-    sv = ov = svn = ovn = (v4i){0, 0, 0, 0};
+    constexpr int SV = PF / 8; // VSCALE: the scales (offsets) of this and of the next super-step, 8 per register quad
+    v4i sv[SV], ov[SV], svn[SV], ovn[SV];
+#pragma unroll
+    for (int h = 0; h < SV; h++) sv[h] = ov[h] = svn[h] = ovn[h] = (v4i){0, 0, 0, 0};
     auto group_of = [&](int cw) { return ((cw * WK + wk) >> p.cpg_shift); };   // cpg_shift = 31 for per-channel
     auto fetch = [&](int j, int cw) {   // chunk cw of this wave into slot j
         wq[j] = *(const v4i*)(wptr + (int64_t)cw * (WK * 64));
@@ -206,8 +215,13 @@ __global__ __launch_bounds__(256, 2) void wqmm_stream_kernel(WqParams p)
 #pragma unroll
     for (int j = 0; j < PF; j++) fetch(j, j < NCW ? j : NCW - 1);
     if constexpr (VSCALE) {
-        svn = *(const v4i*)srow;
-        if constexpr (HAS_OFF) ovn = *(const v4i*)orow;
+#pragma unroll
+        for (int h = 0; h < SV; h++) {
+            if (8 * h < NCW) {
+                svn[h] = *(const v4i*)(srow + 8 * h);
+                if constexpr (HAS_OFF) ovn[h] = *(const v4i*)(orow + 8 * h);
+            }
+        }
     }
     load_x(0);
     store_x(0);
@@ -217,10 +231,13 @@ __global__ __launch_bounds__(256, 2) void wqmm_stream_kernel(WqParams p)
     auto superstep = [&](int c0, auto tail_tag) {
         constexpr bool TAIL = decltype(tail_tag)::value;
         if constexpr (VSCALE) {
-            sv = svn; ov = ovn;
-            if (c0 + PF < NCW) {
-                svn = *(const v4i*)(srow + c0 + PF);
-                if constexpr (HAS_OFF) ovn = *(const v4i*)(orow + c0 + PF);
+#pragma unroll
+            for (int h = 0; h < SV; h++) {
+                sv[h] = svn[h]; ov[h] = ovn[h];
+                if (c0 + PF + 8 * h < NCW) {
+                    svn[h] = *(const v4i*)(srow + c0 + PF + 8 * h);
+                    if constexpr (HAS_OFF) ovn[h] = *(const v4i*)(orow + c0 + PF + 8 * h);
+                }
             }
         }
 #pragma unroll
@@ -232,8 +249,10 @@ __global__ __launch_bounds__(256, 2) void wqmm_stream_kernel(WqParams p)
                 const int slab = cw / CPSW;
                 if (!TAIL || slab < NSLAB) {
                     __syncthreads();
+#if WQ_ABL != 5
                     if (slab + 1 < NSLAB) store_x((slab + 1) & 1);
                     if (slab + 2 < NSLAB) load_x(slab + 2);
+#endif
                 }
             }
             if (TAIL && cw >= NCW) continue;
@@ -241,17 +260,24 @@ __global__ __launch_bounds__(256, 2) void wqmm_stream_kernel(WqParams p)
             const char* xs = sx + (slab & 1) * xslab + ((cw % CPSW) * WK + wk) * (KC * 2);
             uint16_t sb, ob = 0;
             if constexpr (VSCALE) {
-                sb = (uint16_t)((uint32_t)sv[j / 2] >> (16 * (j % 2)));
-                if constexpr (HAS_OFF) ob = (uint16_t)((uint32_t)ov[j / 2] >> (16 * (j % 2)));
+                sb = (uint16_t)((uint32_t)sv[j / 8][(j % 8) / 2] >> (16 * (j % 2)));
+                if constexpr (HAS_OFF) ob = (uint16_t)((uint32_t)ov[j / 8][(j % 8) / 2] >> (16 * (j % 2)));
             } else {
                 sb = sq[j];
                 if constexpr (HAS_OFF) ob = oq[j];
             }
 #pragma unroll
             for (int s = 0; s < STEPS; s++) {
+#if WQ_ABL == 2
+                const v4i aop = wq[j] + (v4i){s, s, s, s};
+#else
                 const v4i aop = dequant8<XDT, WBITS, HAS_OFF>(wq[j], s, sb, ob, dqc);
+#endif
 #pragma unroll
                 for (int b = 0; b < MB; b++) {
+#if WQ_ABL == 3
+                    acc[b][0] += __builtin_bit_cast(float, aop[0] ^ aop[1] ^ aop[2] ^ aop[3]); continue;
+#endif
                     const v4i bop = *(const v4i*)(xs + xoff[b] + 16 * s);
                     if constexpr (XDT == DT_F16) {
                         acc[b] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(v8h, aop), __builtin_bit_cast(v8h, bop), acc[b], 0, 0, 0);
@@ -265,7 +291,9 @@ __global__ __launch_bounds__(256, 2) void wqmm_stream_kernel(WqParams p)
                 const int nx = cw + PF;
                 fetch(j, nx < NCW ? nx : NCW - 1);
             } else {
+#if WQ_ABL != 4
                 fetch(j, cw + PF);
+#endif
             }
         }
     };
@@ -320,6 +348,249 @@ __global__ __launch_bounds__(256, 2) void wqmm_stream_kernel(WqParams p)
     }
 }
 
+// ---- few rows of x (rows * K * 2 bytes fit in LDS): x is staged whole, once per workgroup ----
+// The four waves of a workgroup share one block of 16 weight rows at a time and take one contiguous quarter of K
+// each; partial sums meet in LDS in a fixed order.  A workgroup walks several row blocks (blockIdx.x, + gridDim.x,
+// ...) and its weight stream never stops: the refills issued while the last chunks of one row block are consumed
+// already fetch the first chunks of the next, so the memory latency is paid once per workgroup, not per row block.
+#ifndef WQ_RESX_PF
+#define WQ_RESX_PF 8
+#endif
+#ifndef WQ_RESX_OCC
+#define WQ_RESX_OCC 2
+#endif
+template <int XDT, int WBITS, bool HAS_OFF, bool VSCALE>
+__global__ __launch_bounds__(256, WQ_RESX_OCC) void wqmm_resx_kernel(WqParams p)
+{
+    constexpr int KPL = 128 / WBITS, KC = 4 * KPL, STEPS = KC / 32;
+    constexpr int PF = WQ_RESX_PF;
+    extern __shared__ __attribute__((aligned(16))) char sx[];
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wk = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int nrow = lane & 15, g = lane >> 4;
+    const int Ki = (int)p.K;
+    const int NCW = Ki / (KC * 4);       // chunks per wave and row block; wave wk owns chunks wk*NCW .. wk*NCW+NCW-1
+    const int cbase = wk * NCW;
+    const int rows = (int)p.m_rows;
+    const int xrow = Ki * 2 + 16;        // LDS row pitch in bytes
+    const int nblocks = (int)((p.N + 15) / 16);
+    float* red = (float*)(sx + (rows + 1) * xrow);   // [2][3 waves][4][64] partial sums, double buffered by row-block parity
+
+    // per-lane stream pointers of a row block (rows past the edge of N re-read the last row)
+    auto row_of = [&](int rb) { const int64_t n = (int64_t)rb * 16 + nrow; return n < p.N ? n : p.N - 1; };
+    auto wptr_of = [&](int rb) { return p.w + row_of(rb) * p.ldw + g * 16 + (int64_t)cbase * 64; };
+    int rb = blockIdx.x;
+    const uint8_t* wptr = wptr_of(rb);
+    const uint16_t* srow = p.scale + row_of(rb) * p.s_cs;
+    const uint16_t* orow = HAS_OFF ? p.offset + row_of(rb) * p.s_cs : nullptr;
+#ifdef WQ_DBG
+    const uint64_t t_start = __builtin_readcyclecounter();
+    const uint64_t w_start = wall_clock64();
+#endif
+
+    // x: rows * K/8 pieces of 16 bytes.  The first four pieces of every thread are requested before the weight stream
+    // starts (loads return in issue order, and these are cache hits that must not queue behind it) and are written to
+    // LDS after the weight requests have gone out; further pieces (more than one row of 8192) follow.
+    const int xpr = Ki / 8, xtotal = rows * xpr;
+    auto x_piece = [&](int idx) {
+        const int r = idx / xpr, c = idx - r * xpr;
+        return *(const v4i*)(p.x + (p.m_base + r) * p.K + c * 8);
+    };
+    auto x_store = [&](int idx, v4i v) {
+        const int r = idx / xpr, c = idx - r * xpr;
+        if constexpr (WBITS == 4) {
+            // halves [0..7] -> [0,4,1,5,2,6,3,7]: the order in which the nibble splicing yields pairs
+            const uint32_t a0 = (uint32_t)v[0], a1 = (uint32_t)v[1], a2 = (uint32_t)v[2], a3 = (uint32_t)v[3];
+            v = (v4i){(int)__builtin_amdgcn_perm(a2, a0, 0x05040100u), (int)__builtin_amdgcn_perm(a2, a0, 0x07060302u),
+                      (int)__builtin_amdgcn_perm(a3, a1, 0x05040100u), (int)__builtin_amdgcn_perm(a3, a1, 0x07060302u)};
+        }
+        *(v4i*)(sx + r * xrow + c * 16) = v;
+    };
+    v4i xfirst[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) xfirst[i] = x_piece((i * 256 + tid) < xtotal ? (i * 256 + tid) : 0);
+    // VSCALE: the 8 scales (offsets) of a super-step are loaded one super-step ahead, before that super-step's weight
+    // refills, so that waiting for them never drains the younger weight loads (loads complete in issue order)
+    constexpr int SV = PF / 8;   // register quads of 8 scales per super-step
+    static_assert(PF % 8 == 0, "a super-step holds whole quads of scales");
+    v4i sv[SV], ov[SV], svn[SV], ovn[SV];
+#pragma unroll
+    for (int h = 0; h < SV; h++) {
+        sv[h] = ov[h] = svn[h] = ovn[h] = (v4i){0, 0, 0, 0};
+        if constexpr (VSCALE) {
+            if (8 * h < NCW) {
+                svn[h] = *(const v4i*)(srow + cbase + 8 * h);
+                if constexpr (HAS_OFF) ovn[h] = *(const v4i*)(orow + cbase + 8 * h);
+            }
+        }
+    }
+    v4i wq[PF];
+    uint16_t sq[PF], oq[PF];
+    auto fetch = [&](int j, const uint8_t* wp, const uint16_t* sr, const uint16_t* orw, int cw) {
+        wq[j] = *(const v4i*)(wp + (int64_t)cw * 64);
+        if constexpr (!VSCALE) {
+            const int64_t so = (int64_t)((cbase + cw) >> p.cpg_shift) * p.s_rs;
+            sq[j] = sr[so];
+            if constexpr (HAS_OFF) oq[j] = orw[so];
+        }
+    };
+#pragma unroll
+    for (int j = 0; j < PF; j++) fetch(j, wptr, srow, orow, j < NCW ? j : NCW - 1);
+
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+        if (i * 256 + tid < xtotal) x_store(i * 256 + tid, xfirst[i]);
+    for (int idx = 1024 + tid; idx < xtotal; idx += 256) x_store(idx, x_piece(idx));
+    for (int c = tid; c < xrow / 16; c += 256) *(v4i*)(sx + rows * xrow + c * 16) = (v4i){0, 0, 0, 0};
+    const int xoff = (nrow < rows ? nrow : rows) * xrow + g * KPL * 2 + cbase * (KC * 2);
+    const DqConst dqc = make_dq_const();
+    __syncthreads();
+#ifdef WQ_DBG
+    const uint64_t t_loop = __builtin_readcyclecounter();
+#endif
+
+    for (int it = 0; rb < nblocks; it++) {
+        const int rb_next = rb + (int)gridDim.x;
+        const bool has_next = rb_next < nblocks;
+        const uint8_t* wptr_n = has_next ? wptr_of(rb_next) : wptr;
+        const uint16_t* srow_n = has_next ? p.scale + row_of(rb_next) * p.s_cs : srow;
+        const uint16_t* orow_n = HAS_OFF ? (has_next ? p.offset + row_of(rb_next) * p.s_cs : orow) : nullptr;
+        v4f acc = {0.0f, 0.0f, 0.0f, 0.0f};
+
+        // LAST: the refills of this super-step run past the row block's chunks into the next row block
+        auto superstep = [&](int c0, auto last_tag) {
+            constexpr bool LAST = decltype(last_tag)::value;
+            if constexpr (VSCALE) {
+#pragma unroll
+                for (int h = 0; h < SV; h++) {
+                    sv[h] = svn[h]; ov[h] = ovn[h];
+                    // the quad of chunks c0 + PF + 8h ..: in this row block, or wrapped into the next one
+                    const int cn = c0 + PF + 8 * h;
+                    if (!LAST || cn < NCW) {
+                        svn[h] = *(const v4i*)(srow + cbase + cn);
+                        if constexpr (HAS_OFF) ovn[h] = *(const v4i*)(orow + cbase + cn);
+                    } else if (cn - NCW < NCW) {
+                        svn[h] = *(const v4i*)(srow_n + cbase + cn - NCW);
+                        if constexpr (HAS_OFF) ovn[h] = *(const v4i*)(orow_n + cbase + cn - NCW);
+                    }
+                }
+            }
+#pragma unroll
+            for (int j = 0; j < PF; j++) {
+                const int cw = c0 + j;
+                if (LAST && cw >= NCW) continue;
+                const char* xs = sx + xoff + cw * (KC * 2);
+                uint16_t sb, ob = 0;
+                if constexpr (VSCALE) {
+                    sb = (uint16_t)((uint32_t)sv[j / 8][(j % 8) / 2] >> (16 * (j % 2)));
+                    if constexpr (HAS_OFF) ob = (uint16_t)((uint32_t)ov[j / 8][(j % 8) / 2] >> (16 * (j % 2)));
+                } else {
+                    sb = sq[j];
+                    if constexpr (HAS_OFF) ob = oq[j];
+                }
+#pragma unroll
+                for (int s = 0; s < STEPS; s++) {
+                    const v4i aop = dequant8<XDT, WBITS, HAS_OFF>(wq[j], s, sb, ob, dqc);
+                    const v4i bop = *(const v4i*)(xs + 16 * s);
+                    if constexpr (XDT == DT_F16) {
+                        acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(v8h, aop), __builtin_bit_cast(v8h, bop), acc, 0, 0, 0);
+                    } else {
+                        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf, aop), __builtin_bit_cast(v8bf, bop), acc, 0, 0, 0);
+                    }
+                }
+                if constexpr (LAST) {
+                    // slot j next holds chunk cw + PF of this row block, or, past its end, a chunk of the next one
+                    // (clamped when the stream ends: the value is then never used)
+                    const int nx = cw + PF;
+                    if (nx < NCW) fetch(j, wptr, srow, orow, nx);
+                    else fetch(j, wptr_n, srow_n, orow_n, (nx - NCW) < NCW ? (nx - NCW) : NCW - 1);
+                } else {
+                    fetch(j, wptr, srow, orow, cw + PF);
+                }
+            }
+        };
+        int c0 = 0;
+        for (; c0 + 2 * PF <= NCW; c0 += PF) superstep(c0, std::false_type{});
+        for (; c0 < NCW; c0 += PF) superstep(c0, std::true_type{});
+
+        // fixed-order reduction of the four K quarters (one barrier per row block; the buffer alternates)
+        float* rd = red + (it & 1) * (3 * 4 * 64);
+        if (wk > 0) {
+#pragma unroll
+            for (int i = 0; i < 4; i++) rd[((wk - 1) * 4 + i) * 64 + lane] = acc[i];
+        }
+        __syncthreads();
+        if (wk == 0) {
+#pragma unroll
+            for (int j = 0; j < 3; j++)
+#pragma unroll
+                for (int i = 0; i < 4; i++) acc[i] = acc[i] + rd[(j * 4 + i) * 64 + lane];
+            if (nrow < rows) {
+                const int64_t n0 = (int64_t)rb * 16;
+                const int64_t m = p.m_base + nrow;
+                float v[4];
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    const int64_t nn = n0 + 4 * g + i;
+                    v[i] = acc[i];
+#ifndef WQ_DBG
+                    if (p.bias && nn < p.N) v[i] = v[i] + load_scalar_as_f32(p.bias, p.bias_dt, nn);
+#endif
+                    if constexpr (XDT == DT_BF16) v[i] = bf16_to_f32(bf16_bits(v[i]));
+                }
+                const int64_t nn0 = n0 + 4 * g;
+                if (nn0 + 3 < p.N && (p.N % 4) == 0) {
+                    const v4us o = {bits_x<XDT>(v[0]), bits_x<XDT>(v[1]), bits_x<XDT>(v[2]), bits_x<XDT>(v[3])};
+                    *(v4us*)(p.y + m * p.N + nn0) = o;
+                } else {
+#pragma unroll
+                    for (int i = 0; i < 4; i++)
+                        if (nn0 + i < p.N) p.y[m * p.N + nn0 + i] = bits_x<XDT>(v[i]);
+                }
+            }
+        }
+        rb = rb_next; wptr = wptr_n; srow = srow_n; orow = orow_n;
+    }
+#ifdef WQ_DBG
+    {
+        const uint64_t t_end = __builtin_readcyclecounter();
+        if (lane == 0) {
+            uint64_t* d = (uint64_t*)p.bias + ((int64_t)blockIdx.x * 4 + wk) * 4;
+            d[0] = w_start; d[1] = t_loop - t_start; d[2] = t_end - t_loop; d[3] = wall_clock64();
+        }
+    }
+#endif
+}
+
+// Workgroups of the persistent kernel: two per CU (row blocks are dealt round-robin, so the workgroups i and
+// i + CUs, which share a CU, together get an even share), or one per row block when there are fewer than that.
+static inline unsigned resx_grid(int64_t nblocks)
+{
+    static const int cus = [] {
+        int d = 0, n = 0;
+        if (hipGetDevice(&d) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, d) != hipSuccess || n <= 0) n = 256;
+        return n;
+    }();
+    const int64_t g = 2 * (int64_t)cus;
+    return (unsigned)(nblocks < g ? nblocks : g);
+}
+
+template <int XDT, int WBITS, bool HAS_OFF, bool VSCALE>
+static int launch_resx_one(const WqParams& p, hipStream_t st)
+{
+    const size_t lds = (size_t)(p.m_rows + 1) * (p.K * 2 + 16) + 2 * 3 * 4 * 64 * 4;
+    auto k = wqmm_resx_kernel<XDT, WBITS, HAS_OFF, VSCALE>;
+    static bool attr_set = false;
+    if (!attr_set) {
+        hipError_t e = hipFuncSetAttribute((const void*)k, hipFuncAttributeMaxDynamicSharedMemorySize, 65536 + 8192);
+        if (e != hipSuccess) return (int)e;
+        attr_set = true;
+    }
+    hipLaunchKernelGGL(k, dim3(resx_grid((p.N + 15) / 16)), dim3(256), lds, st, p);
+    return (int)hipGetLastError();
+}
+
 template <int XDT, int WBITS, int MB, int WK, bool HAS_OFF, bool VSCALE>
 static int launch_stream_one(const WqParams& p, hipStream_t st)
 {
@@ -342,6 +613,7 @@ static int launch_stream_one(const WqParams& p, hipStream_t st)
 
 struct WqStreamOpts {
     bool has_off, vscale, ksplit;
+    bool resx, resx_vscale;   // whole-x-in-LDS kernel eligible, and with vector scale loads
 };
 
 // One row slab (p.m_rows <= 64) of one dtype pair; defined once per pair in its own translation unit.
@@ -358,6 +630,12 @@ int launch_wq_stream(const WqParams& p, const WqStreamOpts& o, hipStream_t st);
     template <>                                                                                                     \
     int launch_wq_stream<XDT, WBITS>(const WqParams& p, const WqStreamOpts& o, hipStream_t st)                      \
     {                                                                                                               \
+        if (o.resx) {                                                                                               \
+            if (o.resx_vscale) return o.has_off ? launch_resx_one<XDT, WBITS, true, true>(p, st)                    \
+                                                : launch_resx_one<XDT, WBITS, false, true>(p, st);                  \
+            return o.has_off ? launch_resx_one<XDT, WBITS, true, false>(p, st)                                      \
+                             : launch_resx_one<XDT, WBITS, false, false>(p, st);                                    \
+        }                                                                                                           \
         if (o.ksplit && p.m_rows <= 16) return wq_stream_off<1, 4, false>(p, o.has_off, st);                        \
         if (p.m_rows <= 16) return o.vscale ? wq_stream_off<1, 1, true>(p, o.has_off, st) : wq_stream_off<1, 1, false>(p, o.has_off, st); \
         if (p.m_rows <= 32) return o.vscale ? wq_stream_off<2, 1, true>(p, o.has_off, st) : wq_stream_off<2, 1, false>(p, o.has_off, st); \
