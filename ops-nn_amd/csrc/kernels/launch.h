@@ -12,6 +12,7 @@ enum {
     OPSNN_VARIANT_I8_256x128_S3 = 4,  // int8 MFMA, 256x128 tile, BK 64, 3 stages, 2 workgroups per CU
     OPSNN_VARIANT_I8_256_W8 = 5,  // int8 MFMA, 256x256 tile, 8 waves, BK 64, 4 stages
     OPSNN_VARIANT_I8_256_S4 = 6,  // int8 MFMA, 256x256 tile, 4 waves, BK 64, 4 stages
+    OPSNN_VARIANT_I8_256_W8_K128 = 7,  // int8 MFMA, 256x256 tile, 8 waves, BK 128, 2 stages
     OPSNN_VARIANT_MX_128 = 16,    // MX MFMA, 128x128 tile
     OPSNN_VARIANT_MX_FP8_MFMA = 17,  // MXFP8 on the MFMA path (reduced accumulation precision, see qmm_mx.hip)
 };

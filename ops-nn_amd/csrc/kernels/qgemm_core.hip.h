@@ -29,8 +29,9 @@ struct QgemmParams {
     const int8_t* b;   // x2 rows (one per n), K-contiguous
     int64_t lda, ldb;  // row strides in bytes
     int64_t a_bs, b_bs;  // batch strides in bytes (0 = broadcast)
-    void* out;         // [batch, M, N] dense, 16-bit floats
+    void* out;         // 16-bit floats; element (m, n) of batch b at out[(b*M + m)*ldc + n]
     int64_t M, N, KB;  // KB = bytes of K per operand row
+    int64_t ldc;       // output row pitch in elements (N, or wider when this launch covers a column range)
     // MODE_I8 epilogue: out = cast(fp32(acc + ib[n]) * x2s[n] * x1s[m] + fb[n])
     const float* x1s;
     const void* x2s;
@@ -365,8 +366,8 @@ __global__ __launch_bounds__(WGM* WGN * 64, MINWG) void qgemm_kernel(QgemmParams
         }
     }
     __syncthreads();
-    uint16_t* out = (uint16_t*)p.out + bz * p.M * p.N;
-    const bool vec_ok = (p.N % 4) == 0;
+    uint16_t* out = (uint16_t*)p.out + bz * p.M * p.ldc;
+    const bool vec_ok = (p.ldc % 4) == 0 && ((uintptr_t)p.out % 8) == 0;
 #pragma unroll
     for (int j = 0; j < FM; j++) {
         const int ml = wm * TM + j * 32 + frow;
@@ -398,11 +399,11 @@ __global__ __launch_bounds__(WGM* WGN * 64, MINWG) void qgemm_kernel(QgemmParams
                 const v4us o = pack4_b16<OUT_DT>(v);
                 if (m < p.M) {
                     if (vec_ok && n + 3 < p.N) {
-                        *(v4us*)(out + m * p.N + n) = o;
+                        *(v4us*)(out + m * p.ldc + n) = o;
                     } else {
 #pragma unroll
                         for (int e = 0; e < 4; e++)
-                            if (n + e < p.N) out[m * p.N + n + e] = o[e];
+                            if (n + e < p.N) out[m * p.ldc + n + e] = o[e];
                     }
                 }
             }

@@ -69,6 +69,16 @@ using namespace opsnn;
 
 extern "C" bool opsnn_force_plain();
 
+static int64_t cu_count()
+{
+    static const int n = [] {
+        int d = 0, c = 0;
+        if (hipGetDevice(&d) != hipSuccess || hipDeviceGetAttribute(&c, hipDeviceAttributeMultiprocessorCount, d) != hipSuccess || c <= 0) c = 256;
+        return c;
+    }();
+    return n;
+}
+
 extern "C" int opsnnQmmInt8(const OpsnnQmmArgs* a, void* stream)
 {
     if (!a || !a->x1.ptr || !a->x2.ptr || !a->out || !a->x2_scale) return -1;
@@ -105,7 +115,7 @@ extern "C" int opsnnQmmInt8(const OpsnnQmmArgs* a, void* stream)
     if (fast) {
         QgemmParams g{};
         g.a = p.a; g.b = p.b; g.lda = p.a_rs; g.ldb = p.b_cs; g.a_bs = p.a_bs; g.b_bs = p.b_bs;
-        g.out = p.out; g.M = p.M; g.N = p.N; g.KB = p.K;
+        g.out = p.out; g.M = p.M; g.N = p.N; g.ldc = p.N; g.KB = p.K;
         g.x1s = p.x1s; g.x2s = p.x2s; g.x2s_dt = p.x2s_dt; g.x2s_len = p.x2s_len;
         g.bias = p.bias; g.bias_dt = p.bias_dt; g.bias_bs = p.bias_bs;
         switch (variant) {
@@ -114,9 +124,33 @@ extern "C" int opsnnQmmInt8(const OpsnnQmmArgs* a, void* stream)
             case OPSNN_VARIANT_I8_256x128_S3: return qgemm_launch<MODE_I8, 256, 128, 64, 2, 2, 3, 2>(g, a->batch, p.out_dt, st);
             case OPSNN_VARIANT_I8_256_W8: return qgemm_launch<MODE_I8, 256, 256, 64, 2, 4, 4, 1>(g, a->batch, p.out_dt, st);
             case OPSNN_VARIANT_I8_256_S4: return qgemm_launch<MODE_I8, 256, 256, 64, 2, 2, 4, 1>(g, a->batch, p.out_dt, st);
+            case OPSNN_VARIANT_I8_256_W8_K128: return qgemm_launch<MODE_I8, 256, 256, 128, 2, 4, 2, 1>(g, a->batch, p.out_dt, st);
             default: break;
         }
         if (p.M <= 128 || p.N <= 128 || p.M * p.N < 256 * 256 * 64) return qgemm_launch<MODE_I8, 128, 128, 128, 2, 2, 2, 1>(g, a->batch, p.out_dt, st);
+        // Large shapes: 256x256 tiles, one per CU at a time, are the most economical in operand traffic, but only
+        // whole rounds of them keep every CU busy.  Columns that fill whole rounds go to that kernel; the remaining
+        // columns (less than one round) go to 128x128 tiles, two workgroups per CU, in a second launch.
+        const int64_t cus = cu_count();
+        const int64_t tm = (p.M + 255) / 256, tn = (p.N + 255) / 256;
+        if (p.K >= 1024 && tm * tn * a->batch >= cus && a->batch == 1) {
+            const int64_t rounds = tm * tn / cus;
+            const int64_t cols_a = rounds * cus / tm;            // column tiles in whole rounds
+            if (cols_a >= 1 && cols_a * tm * 8 >= rounds * cus * 7) {   // at least 7/8 of those rounds is filled
+                const int64_t na = cols_a * 256 < p.N ? cols_a * 256 : p.N;
+                QgemmParams ga = g;
+                ga.N = na;
+                int rc = qgemm_launch<MODE_I8, 256, 256, 128, 2, 4, 2, 1>(ga, 1, p.out_dt, st);
+                if (rc != 0 || na == p.N) return rc;
+                QgemmParams gb = g;
+                gb.N = p.N - na;
+                gb.b = g.b + na * g.ldb;
+                gb.out = (uint16_t*)g.out + na;
+                if (g.x2s_len != 1) gb.x2s = (const char*)g.x2s + na * (g.x2s_dt == DT_F32 ? 4 : 2);
+                if (g.bias) gb.bias = (const char*)g.bias + na * (g.bias_dt == DT_I32 || g.bias_dt == DT_F32 ? 4 : 2);
+                return qgemm_launch<MODE_I8, 128, 128, 128, 2, 2, 2, 1>(gb, 1, p.out_dt, st);
+            }
+        }
         return qgemm_launch<MODE_I8, 256, 128, 64, 2, 2, 3, 2>(g, a->batch, p.out_dt, st);
     }
     dim3 block(256), grid((unsigned)(((p.N + 255) / 256) * p.M), (unsigned)a->batch);

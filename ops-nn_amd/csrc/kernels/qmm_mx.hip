@@ -102,7 +102,7 @@ int launch_mx_mfma(const OpsnnQmmArgs& a0, hipStream_t st)
     g.a = (const int8_t*)a.x1.ptr; g.b = (const int8_t*)a.x2.ptr;
     g.lda = a.x1.row_stride / epb; g.ldb = a.x2.col_stride / epb;
     g.a_bs = a.x1.batch_stride / epb; g.b_bs = a.x2.batch_stride / epb;
-    g.out = a.out; g.M = a.M; g.N = a.N; g.KB = a.K / epb;
+    g.out = a.out; g.M = a.M; g.N = a.N; g.ldc = a.N; g.KB = a.K / epb;
     g.bias = a.bias; g.bias_dt = a.bias_dtype; g.bias_bs = a.bias_batch_stride;
     g.sa = (const uint8_t*)a.x1_scale_mat.ptr; g.sb = (const uint8_t*)a.x2_scale_mat.ptr;
     g.sa_rs = a.x1_scale_mat.row_stride; g.sb_rs = a.x2_scale_mat.row_stride;

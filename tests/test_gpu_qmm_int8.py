@@ -123,3 +123,19 @@ def test_config2_full_size_on_sampled_rows(gpu):
     y1 = orc.bf16_to_f32(cases.run_qmm_int8_aclnn(m, inp1, M, K, N, True, m.ACL_BF16))
     y2 = orc.bf16_to_f32(cases.run_qmm_int8_aclnn(m, inp2, M, K, N, True, m.ACL_BF16))
     assert np.array_equal(y2, y1 * 2.0)
+
+
+@pytest.mark.parametrize("s2_dt,bias_dt,out_dt", [("bf16", "i32", "bf16"), ("f32", "f16", "f16")])
+def test_column_split_launch(gpu, s2_dt, bias_dt, out_dt):
+    """A shape whose 256x256 tiles do not fill whole rounds of the chip is computed by two launches over two column
+    ranges (M=4096, N=4352: 16x16 tiles in the first, the last 256 columns in the second); scales, bias and output
+    of the second range start at a column offset.  Sampled rows must be bit-identical to the oracle."""
+    m = gpu
+    dt = {"bf16": m.ACL_BF16, "f16": m.ACL_FLOAT16, "f32": m.ACL_FLOAT, "i32": m.ACL_INT32}
+    M, K, N = 4096, 1024, 4352
+    print(f"case int8 column split s2={s2_dt} bias={bias_dt}", flush=True)
+    inp = cases.make_qmm_int8_inputs(m, M, K, N, 11, dt[bias_dt], True, x2s_dtype=dt[s2_dt])
+    got = cases.run_qmm_int8_aclnn(m, inp, M, K, N, True, dt[out_dt])
+    rows = np.unique(np.concatenate([[0, M - 1, 255, 256], np.random.default_rng(2).integers(0, M, 28)]))
+    want, _ = cases.oracle_qmm_int8(m, inp, M, K, N, True, dt[out_dt], rows=rows)
+    _check_equal(got[0][rows], want[0], "column split")
