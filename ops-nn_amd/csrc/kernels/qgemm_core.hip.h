@@ -367,19 +367,32 @@ __global__ __launch_bounds__(WGM* WGN * 64, MINWG) void qgemm_kernel(QgemmParams
     }
     __syncthreads();
     uint16_t* out = (uint16_t*)p.out + bz * p.M * p.ldc;
-    const bool vec_ok = (p.ldc % 4) == 0 && ((uintptr_t)p.out % 8) == 0;
+    // Results leave through LDS: a lane holds 4 consecutive columns of one row per register quad, which would make
+    // every store instruction touch 32 rows with 16 bytes each.  Instead each wave parks one 32-row block of its
+    // sub-tile in a private LDS patch (row pitch TN*2+16 bytes) and reads it back row-wise, so that a store
+    // instruction writes whole 128-byte lines (16 bytes per lane, TN/8 lanes per row).
+    typedef v4us __attribute__((may_alias)) v4us_a;   // the patch is written as 16-bit quads and read as dword quads
+    typedef v4i __attribute__((may_alias)) v4i_a;
+    constexpr int EP_PITCH = TN * 2 + 16;
+    constexpr int EP_BYTES = 32 * EP_PITCH;
+    constexpr int EP_BASE = (3 * BN + BM) * 4;
+    static_assert(EP_BASE + WGM * WGN * EP_BYTES <= STAGES * STAGE, "epilogue staging fits in the operand stages");
+    char* ep = smem + EP_BASE + wave * EP_BYTES;
+    constexpr int LPR = TN / 8;          // lanes per row when every lane moves 16 bytes
+    constexpr int RPI2 = 64 / LPR;       // rows per store instruction
+    const int er = lane / LPR, ec = lane % LPR;
+    const bool vec_ok = (p.ldc % 8) == 0 && ((uintptr_t)p.out % 16) == 0;
 #pragma unroll
     for (int j = 0; j < FM; j++) {
         const int ml = wm * TM + j * 32 + frow;
-        const int64_t m = m0 + ml;
         float s1 = 1.0f;
         if constexpr (MODE == MODE_I8) s1 = sS1[ml];
 #pragma unroll
         for (int i = 0; i < FN; i++) {
 #pragma unroll
             for (int q = 0; q < 4; q++) {
-                const int nl = wn * TN + i * 32 + 8 * q + 4 * fkc;
-                const int64_t n = n0 + nl;
+                const int nw = i * 32 + 8 * q + 4 * fkc;   // column inside the wave's sub-tile
+                const int nl = wn * TN + nw;
                 const v4f fbv = *(const v4f*)(sFb + nl);
                 v4f v;
                 if constexpr (MODE == MODE_I8) {
@@ -396,15 +409,24 @@ __global__ __launch_bounds__(WGM* WGN * 64, MINWG) void qgemm_kernel(QgemmParams
 #pragma unroll
                     for (int e = 0; e < 4; e++) v[e] = acc[i][j][q * 4 + e] + fbv[e];
                 }
-                const v4us o = pack4_b16<OUT_DT>(v);
-                if (m < p.M) {
-                    if (vec_ok && n + 3 < p.N) {
-                        *(v4us*)(out + m * p.ldc + n) = o;
-                    } else {
+                *(v4us_a*)(ep + frow * EP_PITCH + nw * 2) = pack4_b16<OUT_DT>(v);
+            }
+        }
+        // this wave's 32 x TN block is complete in its patch (LDS operations of one wave complete in order)
 #pragma unroll
-                        for (int e = 0; e < 4; e++)
-                            if (n + e < p.N) out[m * p.ldc + n + e] = o[e];
-                    }
+        for (int r = 0; r < 32 / RPI2; r++) {
+            const int row = r * RPI2 + er;
+            const v4i o = *(const v4i_a*)(ep + row * EP_PITCH + ec * 16);
+            const int64_t m = m0 + wm * TM + j * 32 + row;
+            const int64_t n = n0 + wn * TN + ec * 8;
+            if (m < p.M) {
+                if (vec_ok && n + 7 < p.N) {
+                    *(v4i*)(out + m * p.ldc + n) = o;
+                } else {
+                    const uint16_t* oe = (const uint16_t*)&o;
+#pragma unroll
+                    for (int e = 0; e < 8; e++)
+                        if (n + e < p.N) out[m * p.ldc + n + e] = oe[e];
                 }
             }
         }
