@@ -60,6 +60,7 @@ def _reset_env():
     (128, 512, 256, True, 1), (128, 512, 256, False, 1), (100, 300, 200, True, 1), (256, 384, 384, True, 128),
     (130, 256, 130, False, 128), (1, 1024, 256, True, 1),
     (512, 1024, 768, True, 1), (300, 512, 520, True, 1), (384, 2048, 512, False, 1), (256, 1024, 256, True, 128),
+    (700, 384, 520, True, 1), (640, 256, 264, False, 128),     # M >= 512: the eight-wave 256 x 256 tile, ragged edges
 ])
 def test_fp8_blockscale(gpu, M, K, N, tB, gsM, use_plain):
     m = gpu
