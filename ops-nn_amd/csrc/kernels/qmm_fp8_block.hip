@@ -102,16 +102,17 @@ __global__ __launch_bounds__(WGM * 128, 1) void qmm_fp8_block_kernel(Fp8BlkParam
         }
     }
 
-    auto issue_tile = [&](int kt) {
+    // copy instruction `idx` (0 .. CPT-1) of K tile kt: x1 rows, then x2 rows, then the scales
+    auto issue_piece = [&](int kt, int idx) {
         char* sA = smem + (kt % STAGES) * STAGE + wave * 1024;
         char* sB = sA + A_BYTES;
-        const int8_t* Ak = A + (int64_t)kt * BK;
-        const int8_t* Bk = B + (int64_t)kt * BK;
+        if (idx < NA) async_copy16(A + (int64_t)kt * BK + a_off[idx], sA + idx * NT * 16);
+        else if (idx < NA + NB) async_copy16(B + (int64_t)kt * BK + b_off[idx - NA], sB + (idx - NA) * NT * 16);
+        else async_copy4(sc_src + (int64_t)kt * sc_step, smem + (kt % STAGES) * STAGE + A_BYTES + B_BYTES + wave * 256);
+    };
+    auto issue_tile = [&](int kt) {
 #pragma unroll
-        for (int i = 0; i < NA; i++) async_copy16(Ak + a_off[i], sA + i * NT * 16);
-#pragma unroll
-        for (int i = 0; i < NB; i++) async_copy16(Bk + b_off[i], sB + i * NT * 16);
-        async_copy4(sc_src + (int64_t)kt * sc_step, smem + (kt % STAGES) * STAGE + A_BYTES + B_BYTES + wave * 256);
+        for (int idx = 0; idx < CPT; idx++) issue_piece(kt, idx);
     };
 
     v16f acc[FN][FM];
@@ -145,7 +146,7 @@ __global__ __launch_bounds__(WGM * 128, 1) void qmm_fp8_block_kernel(Fp8BlkParam
         if (kt + STAGES - 1 <= KT) wait_vmcnt<(STAGES - 2) * CPT>();
         else wait_vmcnt<0>();
         __builtin_amdgcn_s_barrier();
-        if (kt + STAGES - 1 < KT) issue_tile(kt + STAGES - 1);
+        if (kt + STAGES - 1 < KT) issue_tile(kt + STAGES - 1);   // into the stage freed by the barrier above
         const char* st = smem + (kt % STAGES) * STAGE;
         const float* sS = (const float*)(st + A_BYTES + B_BYTES);
         // x1 fragments of both K steps stay resident; x2 fragments stream through
