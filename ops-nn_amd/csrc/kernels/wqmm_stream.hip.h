@@ -17,9 +17,6 @@
 // with the chunk 8 further on, so 8 loads per lane are always in flight without a second register set.
 #pragma once
 #include "wqmm_common.hip.h"
-#ifndef WQ_ABL
-#define WQ_ABL 0
-#endif
 
 namespace opsnn {
 
@@ -103,26 +100,24 @@ __device__ __forceinline__ v4i dequant8(const v4i& piece, int s, uint16_t sb, ui
     }
 }
 
-template <int XDT, int WBITS, int MB, int WK, bool HAS_OFF, bool VSCALE>
-__global__ __launch_bounds__(256, 2) void wqmm_stream_kernel(WqParams p)
+// NW waves per workgroup (4 or 8) = WN row blocks x WK waves that split K chunk by chunk.
+template <int XDT, int WBITS, int MB, int NW, int WK, bool HAS_OFF, bool VSCALE>
+__global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(NW == 8 ? 4 : 2))) void wqmm_stream_kernel(WqParams p)
 {
-    static_assert(!(VSCALE && WK != 1), "vector scale loads need consecutive chunks per wave");
-    constexpr int WN = 4 / WK;
+    static_assert(!(VSCALE && WK > 2), "vector scale loads: a wave's chunks are consecutive (WK 1) or every other one (WK 2)");
+    constexpr int NT = NW * 64;
+    constexpr int WN = NW / WK;
     constexpr int KPL = 128 / WBITS;     // k per 16-byte piece: 32 or 16
     constexpr int KC = 4 * KPL;          // k per chunk: 128 or 64 (64 bytes of a weight row either way)
     constexpr int STEPS = KC / 32;       // MFMA steps per chunk: 4 or 2
-#ifdef WQ_PF
-    constexpr int PF = WQ_PF;
-#else
     constexpr int PF = (MB == 1 && WK == 1) ? 16 : 8;   // chunks per super-step = pieces in flight per lane
-#endif
     constexpr int KX = 8 * KC / MB;      // k per LDS slab of x
     constexpr int CPS = KX / KC;         // chunks per slab: 8, 4, 2
     constexpr int CPSW = CPS / WK;       // of which this wave's
     static_assert(CPSW >= 1, "a slab must hold at least one chunk per K-split wave");
     constexpr int XROW = KX * 2 + 16;    // LDS row pitch (bytes); the pad makes the 16-byte reads conflict free
     constexpr int XPR = KX / 8;          // 16-byte pieces per x row per slab
-    constexpr int XITEMS = 16 * MB * XPR / 256;
+    constexpr int XITEMS = 16 * MB * XPR / NT;
     extern __shared__ __attribute__((aligned(16))) char sx[];
 
     const int tid = threadIdx.x, lane = tid & 63;
@@ -148,8 +143,8 @@ __global__ __launch_bounds__(256, 2) void wqmm_stream_kernel(WqParams p)
     auto load_x = [&](int slab) {
 #pragma unroll
         for (int it = 0; it < XITEMS; it++) {
-            const int idx = it * 256 + tid;
-            if (it * 256 >= xtotal) break;
+            const int idx = it * NT + tid;
+            if (it * NT >= xtotal) break;
             const int r = idx / XPR, c = idx % XPR;
             const int k = slab * KX + c * 8;
             v4i v = {0, 0, 0, 0};
@@ -161,8 +156,8 @@ __global__ __launch_bounds__(256, 2) void wqmm_stream_kernel(WqParams p)
         char* dst = sx + buf * xslab;
 #pragma unroll
         for (int it = 0; it < XITEMS; it++) {
-            const int idx = it * 256 + tid;
-            if (it * 256 >= xtotal) break;
+            const int idx = it * NT + tid;
+            if (it * NT >= xtotal) break;
             const int r = idx / XPR, c = idx % XPR;
             v4i v = xreg[it];
             if constexpr (WBITS == 4 && XDT == DT_F16) {
@@ -179,7 +174,7 @@ __global__ __launch_bounds__(256, 2) void wqmm_stream_kernel(WqParams p)
         }
     };
     // the zero row of both buffers
-    for (int i = tid; i < 2 * (XROW / 16); i += 256) {
+    for (int i = tid; i < 2 * (XROW / 16); i += NT) {
         const int buf = i / (XROW / 16), c = i % (XROW / 16);
         *(v4i*)(sx + buf * xslab + rows * XROW + c * 16) = (v4i){0, 0, 0, 0};
     }
@@ -199,7 +194,7 @@ __global__ __launch_bounds__(256, 2) void wqmm_stream_kernel(WqParams p)
     // ---- weight / scale prefetch state ----
     v4i wq[PF];
     uint16_t sq[PF], oq[PF];   // !VSCALE: scale and offset of each chunk in flight
-    constexpr int SV = PF / 8; // VSCALE: the scales (offsets) of this and of the next super-step, 8 per register quad
+    constexpr int SV = PF * WK / 8;   // VSCALE: the scales (offsets) of the chunks a super-step spans, 8 per register quad
     v4i sv[SV], ov[SV], svn[SV], ovn[SV];
 #pragma unroll
     for (int h = 0; h < SV; h++) sv[h] = ov[h] = svn[h] = ovn[h] = (v4i){0, 0, 0, 0};
@@ -217,7 +212,7 @@ __global__ __launch_bounds__(256, 2) void wqmm_stream_kernel(WqParams p)
     if constexpr (VSCALE) {
 #pragma unroll
         for (int h = 0; h < SV; h++) {
-            if (8 * h < NCW) {
+            if (8 * h < NCW * WK) {
                 svn[h] = *(const v4i*)(srow + 8 * h);
                 if constexpr (HAS_OFF) ovn[h] = *(const v4i*)(orow + 8 * h);
             }
@@ -234,9 +229,9 @@ __global__ __launch_bounds__(256, 2) void wqmm_stream_kernel(WqParams p)
 #pragma unroll
             for (int h = 0; h < SV; h++) {
                 sv[h] = svn[h]; ov[h] = ovn[h];
-                if (c0 + PF + 8 * h < NCW) {
-                    svn[h] = *(const v4i*)(srow + c0 + PF + 8 * h);
-                    if constexpr (HAS_OFF) ovn[h] = *(const v4i*)(orow + c0 + PF + 8 * h);
+                if ((c0 + PF) * WK + 8 * h < NCW * WK) {
+                    svn[h] = *(const v4i*)(srow + (c0 + PF) * WK + 8 * h);
+                    if constexpr (HAS_OFF) ovn[h] = *(const v4i*)(orow + (c0 + PF) * WK + 8 * h);
                 }
             }
         }
@@ -249,10 +244,8 @@ __global__ __launch_bounds__(256, 2) void wqmm_stream_kernel(WqParams p)
                 const int slab = cw / CPSW;
                 if (!TAIL || slab < NSLAB) {
                     __syncthreads();
-#if WQ_ABL != 5
                     if (slab + 1 < NSLAB) store_x((slab + 1) & 1);
                     if (slab + 2 < NSLAB) load_x(slab + 2);
-#endif
                 }
             }
             if (TAIL && cw >= NCW) continue;
@@ -260,24 +253,23 @@ __global__ __launch_bounds__(256, 2) void wqmm_stream_kernel(WqParams p)
             const char* xs = sx + (slab & 1) * xslab + ((cw % CPSW) * WK + wk) * (KC * 2);
             uint16_t sb, ob = 0;
             if constexpr (VSCALE) {
-                sb = (uint16_t)((uint32_t)sv[j / 8][(j % 8) / 2] >> (16 * (j % 2)));
-                if constexpr (HAS_OFF) ob = (uint16_t)((uint32_t)ov[j / 8][(j % 8) / 2] >> (16 * (j % 2)));
+                // this wave's chunk j of the super-step is chunk j*WK + wk of the span the scale quads cover
+                if constexpr (WK == 1) {
+                    sb = (uint16_t)((uint32_t)sv[j / 8][(j % 8) / 2] >> (16 * (j % 2)));
+                    if constexpr (HAS_OFF) ob = (uint16_t)((uint32_t)ov[j / 8][(j % 8) / 2] >> (16 * (j % 2)));
+                } else {
+                    sb = (uint16_t)((uint32_t)sv[j / 4][j % 4] >> (16 * wk));
+                    if constexpr (HAS_OFF) ob = (uint16_t)((uint32_t)ov[j / 4][j % 4] >> (16 * wk));
+                }
             } else {
                 sb = sq[j];
                 if constexpr (HAS_OFF) ob = oq[j];
             }
 #pragma unroll
             for (int s = 0; s < STEPS; s++) {
-#if WQ_ABL == 2
-                const v4i aop = wq[j] + (v4i){s, s, s, s};
-#else
                 const v4i aop = dequant8<XDT, WBITS, HAS_OFF>(wq[j], s, sb, ob, dqc);
-#endif
 #pragma unroll
                 for (int b = 0; b < MB; b++) {
-#if WQ_ABL == 3
-                    acc[b][0] += __builtin_bit_cast(float, aop[0] ^ aop[1] ^ aop[2] ^ aop[3]); continue;
-#endif
                     const v4i bop = *(const v4i*)(xs + xoff[b] + 16 * s);
                     if constexpr (XDT == DT_F16) {
                         acc[b] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(v8h, aop), __builtin_bit_cast(v8h, bop), acc[b], 0, 0, 0);
@@ -291,9 +283,7 @@ __global__ __launch_bounds__(256, 2) void wqmm_stream_kernel(WqParams p)
                 const int nx = cw + PF;
                 fetch(j, nx < NCW ? nx : NCW - 1);
             } else {
-#if WQ_ABL != 4
                 fetch(j, cw + PF);
-#endif
             }
         }
     };
@@ -353,17 +343,11 @@ __global__ __launch_bounds__(256, 2) void wqmm_stream_kernel(WqParams p)
 // each; partial sums meet in LDS in a fixed order.  A workgroup walks several row blocks (blockIdx.x, + gridDim.x,
 // ...) and its weight stream never stops: the refills issued while the last chunks of one row block are consumed
 // already fetch the first chunks of the next, so the memory latency is paid once per workgroup, not per row block.
-#ifndef WQ_RESX_PF
-#define WQ_RESX_PF 8
-#endif
-#ifndef WQ_RESX_OCC
-#define WQ_RESX_OCC 2
-#endif
 template <int XDT, int WBITS, bool HAS_OFF, bool VSCALE>
-__global__ __launch_bounds__(256, WQ_RESX_OCC) void wqmm_resx_kernel(WqParams p)
+__global__ __launch_bounds__(256, 2) void wqmm_resx_kernel(WqParams p)
 {
     constexpr int KPL = 128 / WBITS, KC = 4 * KPL, STEPS = KC / 32;
-    constexpr int PF = WQ_RESX_PF;
+    constexpr int PF = 8;   // weight pieces in flight per lane
     extern __shared__ __attribute__((aligned(16))) char sx[];
 
     const int tid = threadIdx.x, lane = tid & 63;
@@ -384,10 +368,6 @@ __global__ __launch_bounds__(256, WQ_RESX_OCC) void wqmm_resx_kernel(WqParams p)
     const uint8_t* wptr = wptr_of(rb);
     const uint16_t* srow = p.scale + row_of(rb) * p.s_cs;
     const uint16_t* orow = HAS_OFF ? p.offset + row_of(rb) * p.s_cs : nullptr;
-#ifdef WQ_DBG
-    const uint64_t t_start = __builtin_readcyclecounter();
-    const uint64_t w_start = wall_clock64();
-#endif
 
     // x: rows * K/8 pieces of 16 bytes.  The first four pieces of every thread are requested before the weight stream
     // starts (loads return in issue order, and these are cache hits that must not queue behind it) and are written to
@@ -446,9 +426,6 @@ __global__ __launch_bounds__(256, WQ_RESX_OCC) void wqmm_resx_kernel(WqParams p)
     const int xoff = (nrow < rows ? nrow : rows) * xrow + g * KPL * 2 + cbase * (KC * 2);
     const DqConst dqc = make_dq_const();
     __syncthreads();
-#ifdef WQ_DBG
-    const uint64_t t_loop = __builtin_readcyclecounter();
-#endif
 
     for (int it = 0; rb < nblocks; it++) {
         const int rb_next = rb + (int)gridDim.x;
@@ -534,9 +511,7 @@ __global__ __launch_bounds__(256, WQ_RESX_OCC) void wqmm_resx_kernel(WqParams p)
                 for (int i = 0; i < 4; i++) {
                     const int64_t nn = n0 + 4 * g + i;
                     v[i] = acc[i];
-#ifndef WQ_DBG
                     if (p.bias && nn < p.N) v[i] = v[i] + load_scalar_as_f32(p.bias, p.bias_dt, nn);
-#endif
                     if constexpr (XDT == DT_BF16) v[i] = bf16_to_f32(bf16_bits(v[i]));
                 }
                 const int64_t nn0 = n0 + 4 * g;
@@ -552,15 +527,6 @@ __global__ __launch_bounds__(256, WQ_RESX_OCC) void wqmm_resx_kernel(WqParams p)
         }
         rb = rb_next; wptr = wptr_n; srow = srow_n; orow = orow_n;
     }
-#ifdef WQ_DBG
-    {
-        const uint64_t t_end = __builtin_readcyclecounter();
-        if (lane == 0) {
-            uint64_t* d = (uint64_t*)p.bias + ((int64_t)blockIdx.x * 4 + wk) * 4;
-            d[0] = w_start; d[1] = t_loop - t_start; d[2] = t_end - t_loop; d[3] = wall_clock64();
-        }
-    }
-#endif
 }
 
 // Workgroups of the persistent kernel: two per CU (row blocks are dealt round-robin, so the workgroups i and
@@ -591,15 +557,15 @@ static int launch_resx_one(const WqParams& p, hipStream_t st)
     return (int)hipGetLastError();
 }
 
-template <int XDT, int WBITS, int MB, int WK, bool HAS_OFF, bool VSCALE>
+template <int XDT, int WBITS, int MB, int NW, int WK, bool HAS_OFF, bool VSCALE>
 static int launch_stream_one(const WqParams& p, hipStream_t st)
 {
-    constexpr int KC = 4 * (128 / WBITS), KX = 8 * KC / MB, WN = 4 / WK;
+    constexpr int KC = 4 * (128 / WBITS), KX = 8 * KC / MB, WN = NW / WK;
     const size_t lds_x = 2 * (size_t)(p.m_rows + 1) * (KX * 2 + 16);
     const size_t lds_red = WK > 1 ? (size_t)WN * (WK - 1) * MB * 4 * 64 * 4 : 0;
     const size_t lds = lds_x > lds_red ? lds_x : lds_red;
     const unsigned grid = (unsigned)((p.N + 16 * WN - 1) / (16 * WN));
-    auto k = wqmm_stream_kernel<XDT, WBITS, MB, WK, HAS_OFF, VSCALE>;
+    auto k = wqmm_stream_kernel<XDT, WBITS, MB, NW, WK, HAS_OFF, VSCALE>;
     static bool attr_set = false;
     if (!attr_set) {
         constexpr size_t lds_max = 2 * (size_t)(16 * MB + 1) * (KX * 2 + 16);
@@ -607,7 +573,7 @@ static int launch_stream_one(const WqParams& p, hipStream_t st)
         if (e != hipSuccess) return (int)e;
         attr_set = true;
     }
-    hipLaunchKernelGGL(k, dim3(grid), dim3(256), lds, st, p);
+    hipLaunchKernelGGL(k, dim3(grid), dim3(NW * 64), lds, st, p);
     return (int)hipGetLastError();
 }
 
@@ -621,11 +587,16 @@ template <int XDT, int WBITS>
 int launch_wq_stream(const WqParams& p, const WqStreamOpts& o, hipStream_t st);
 
 #define OPSNN_WQ_STREAM_DEFINE(XDT, WBITS)                                                                          \
-    template <int MB, int WK, bool VS>                                                                              \
+    template <int MB, int NW, int WK, bool VS>                                                                      \
     static int wq_stream_off(const WqParams& p, bool has_off, hipStream_t st)                                       \
     {                                                                                                               \
-        return has_off ? launch_stream_one<XDT, WBITS, MB, WK, true, VS>(p, st)                                     \
-                       : launch_stream_one<XDT, WBITS, MB, WK, false, VS>(p, st);                                   \
+        return has_off ? launch_stream_one<XDT, WBITS, MB, NW, WK, true, VS>(p, st)                                 \
+                       : launch_stream_one<XDT, WBITS, MB, NW, WK, false, VS>(p, st);                               \
+    }                                                                                                               \
+    template <int MB>                                                                                               \
+    static int wq_stream_mb(const WqParams& p, const WqStreamOpts& o, hipStream_t st)                               \
+    {                                                                                                               \
+        return o.vscale ? wq_stream_off<MB, 4, 1, true>(p, o.has_off, st) : wq_stream_off<MB, 4, 1, false>(p, o.has_off, st); \
     }                                                                                                               \
     template <>                                                                                                     \
     int launch_wq_stream<XDT, WBITS>(const WqParams& p, const WqStreamOpts& o, hipStream_t st)                      \
@@ -636,10 +607,10 @@ int launch_wq_stream(const WqParams& p, const WqStreamOpts& o, hipStream_t st);
             return o.has_off ? launch_resx_one<XDT, WBITS, true, false>(p, st)                                      \
                              : launch_resx_one<XDT, WBITS, false, false>(p, st);                                    \
         }                                                                                                           \
-        if (o.ksplit && p.m_rows <= 16) return wq_stream_off<1, 4, false>(p, o.has_off, st);                        \
-        if (p.m_rows <= 16) return o.vscale ? wq_stream_off<1, 1, true>(p, o.has_off, st) : wq_stream_off<1, 1, false>(p, o.has_off, st); \
-        if (p.m_rows <= 32) return o.vscale ? wq_stream_off<2, 1, true>(p, o.has_off, st) : wq_stream_off<2, 1, false>(p, o.has_off, st); \
-        return o.vscale ? wq_stream_off<4, 1, true>(p, o.has_off, st) : wq_stream_off<4, 1, false>(p, o.has_off, st); \
+        if (o.ksplit && p.m_rows <= 16) return wq_stream_off<1, 4, 4, false>(p, o.has_off, st);                     \
+        if (p.m_rows <= 16) return wq_stream_mb<1>(p, o, st);                                                       \
+        if (p.m_rows <= 32) return wq_stream_mb<2>(p, o, st);                                                       \
+        return wq_stream_mb<4>(p, o, st);                                                                           \
     }
 
 }  // namespace opsnn
