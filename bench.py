@@ -88,7 +88,8 @@ def main():
         value, unit = gbps, "GB/s"
         roof = {"bound": "hbm", "achieved": wl.bytes / (dev_ms * 1e-3) / 1e9, "peak": PEAK_HBM, "unit": "GB/s"}
     roof["frac"] = roof["achieved"] / roof["peak"]
-    roof["traffic"] = None
+    key = (args.config, (args.m or 16) if args.config == 3 else None)
+    roof["traffic"] = bench_cases.MEASURED_TRAFFIC.get(key) if args.layout == "packed" and not args.cold else None
     roof["kernel"] = wl.kernel
     roof["kernel_ms"] = dev_ms
 
