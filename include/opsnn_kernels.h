@@ -8,6 +8,8 @@
  * stand where the reference has host tiling plus device kernels --
  *   opsnnQmmInt8        <- quant_batch_matmul_v3 K-C/K-T/T-C kernel
  *                          (matmul/quant_batch_matmul_v3/op_kernel/arch35/qbmm_mix_online_dynamic.h:387-388, 648-736)
+ *   opsnnQmmTc          <- the same kernel family's per-tensor / per-channel epilogues (fixpipe dequant and requant,
+ *                          matmul/quant_batch_matmul_v3/op_kernel/arch35/qbmm_cube_on_the_fly.h:159-162)
  *   opsnnQmmBlockScale  <- per-tile kernel (matmul/common/cmct/epilogue/block_epilogue_pertile.h:502-642)
  *   opsnnQmmMx          <- MX kernel (matmul/common/cmct/block/block_mmad_mx.h)
  *   opsnnWqmm           <- weight_quant_batch_matmul_v2 arch35 kernels
@@ -60,6 +62,10 @@ typedef struct {
     OpsnnMat x2_scale_mat;
     void* workspace;       /* opsnnQmmWorkspace() bytes, or NULL if that is 0 */
     int force_variant;     /* 0 = selector decides; >0 pins a kernel variant (tuning and tests) */
+    /* per-tensor / per-channel family (opsnnQmmTc) */
+    int64_t x1_scale_len;  /* 1: one fp32 scale for all of x1 ("double scale" with fp8 inputs); 0 if x1_scale is NULL */
+    const float* x2_offset;/* fp32 [1] or [N], int8 output only; NULL = take it from the packed 64-bit scale */
+    int64_t x2_offset_len;
 } OpsnnQmmArgs;
 
 /* int8 x int8 -> int32, then  out = fp32(acc + int32 bias) * x2_scale[n] * x1_scale[m] + float bias.
@@ -69,6 +75,12 @@ OPSNN_API int opsnnQmmInt8(const OpsnnQmmArgs* a, void* stream);
 OPSNN_API int opsnnQmmBlockScale(const OpsnnQmmArgs* a, void* stream);
 /* MX: fp4/fp8 operands, e8m0 scale per 32 K. out = (x1*s1) @ (x2*s2) + fp32 bias. */
 OPSNN_API int opsnnQmmMx(const OpsnnQmmArgs* a, void* stream);
+/* Per-tensor / per-channel scales (T-T, T-C): int8 or fp8 (e4m3, e5m2) operands;
+ *   x2_scale FLOAT / BF16 [1] or [N], or UINT64 [1] or [N] (fp32 scale in the low word, upper 19 bits kept; signed 9-bit
+ *   offset at bits 37..45); optional one-element x1_scale with fp8 inputs; out BF16 / FLOAT16 / FLOAT, INT32 (integer
+ *   sums + bias) or INT8 (requantised: clip(s9(s9(acc * scale)) + s9(offset))).
+ * Reference formulas: matmul/quant_batch_matmul_v3/tests/assets/qbmmv3_kernel_golden.py:390-513. */
+OPSNN_API int opsnnQmmTc(const OpsnnQmmArgs* a, void* stream);
 /* Device workspace bytes a launcher needs for these arguments (0 if none). */
 OPSNN_API uint64_t opsnnQmmWorkspace(const OpsnnQmmArgs* a, int mode);
 

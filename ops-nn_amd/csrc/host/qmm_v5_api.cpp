@@ -636,9 +636,24 @@ extern "C" aclnnStatus aclnnQuantMatmulV5GetWorkspaceSize(const aclTensor* x1, c
         if (c.tB) { a.x2_scale_mat.row_stride = 1; a.x2_scale_mat.col_stride = kb; }
         else { a.x2_scale_mat.row_stride = nb; a.x2_scale_mat.col_stride = 1; }
         a.x2_scale_mat.batch_stride = b2 == 1 ? 0 : nb * kb;
-    } else if (c.int8_in() && in_list(c.x2s.dtype, {ACL_FLOAT, ACL_BF16}) && in_list(c.out.dtype, {ACL_BF16, ACL_FLOAT16, ACL_INT32})) {
+    } else if (c.int8_in() && in_list(c.x2s.dtype, {ACL_FLOAT, ACL_BF16}) && in_list(c.out.dtype, {ACL_BF16, ACL_FLOAT16, ACL_INT32}) &&
+               !(!c.x1s.present && c.x2s.dim(0) == 1 && c.out.dtype != ACL_INT32 &&
+                 !(c.bias.present && in_list(c.bias.dtype, {ACL_BF16, ACL_FLOAT})))) {
+        // (the excluded case is the per-tensor scale that the reference truncates to 19 bits: it goes to the T-C kernel)
         ex->kind = OpKind::QmmInt8; mode = 0;
         a.x2_scale_len = c.x2s.dim(0);
+    } else if ((c.int8_in() && in_list(c.x2s.dtype, {ACL_FLOAT, ACL_BF16, ACL_UINT64}) &&
+                in_list(c.out.dtype, {ACL_BF16, ACL_FLOAT16, ACL_INT8, ACL_INT32}) && !c.x1s.present) ||
+               (c.fp8_in() && in_list(c.x2s.dtype, {ACL_FLOAT, ACL_BF16, ACL_UINT64}) && in_list(c.out.dtype, {ACL_BF16, ACL_FLOAT16, ACL_FLOAT}) &&
+                (!c.x1s.present || (c.x1s.dtype == ACL_FLOAT && c.x1s.rank() == 1 && c.x1s.dim(0) == 1)))) {
+        // per-tensor / per-channel family: qbmmv3_kernel_golden.py:390-513
+        ex->kind = OpKind::QmmTc; mode = 3;
+        a.x2_scale_len = c.x2s.dim(0);
+        a.x1_scale_len = c.x1s.present ? c.x1s.dim(0) : 0;
+        if (c.x2o.present) {
+            a.x2_offset = (const float*)c.x2o.ptr_at(0);
+            a.x2_offset_len = c.x2o.dim(0);
+        }
     } else {
         FAIL(ACLNN_ERR_INNER_TILING_ERROR, "%s: no kernel for x1 %s, x2 %s, x2Scale %s, out %s on this device yet", kApi,
              dtype_name(c.x1.dtype), dtype_name(c.x2.dtype), dtype_name(c.x2s.dtype), dtype_name(c.out.dtype));
@@ -667,6 +682,7 @@ extern "C" aclnnStatus aclnnQuantMatmulV5(void* workspace, uint64_t workspaceSiz
         case OpKind::QmmInt8: rc = opsnnQmmInt8(&ex->qmm, stream); break;
         case OpKind::QmmBlockScale: rc = opsnnQmmBlockScale(&ex->qmm, stream); break;
         case OpKind::QmmMx: rc = opsnnQmmMx(&ex->qmm, stream); break;
+        case OpKind::QmmTc: rc = opsnnQmmTc(&ex->qmm, stream); break;
         default: rc = -100; break;
     }
     if (rc != 0) FAIL(rc < 0 ? ACLNN_ERR_INNER_TILING_ERROR : ACLNN_ERR_RUNTIME_ERROR, "aclnnQuantMatmulV5: launch failed with code %d", rc);

@@ -9,6 +9,7 @@
 namespace opsnn {
 int launch_blockscale_plain(const OpsnnQmmArgs& a, hipStream_t st);
 int launch_mx_plain(const OpsnnQmmArgs& a, hipStream_t st);
+int launch_tc_plain(const OpsnnQmmArgs& a, hipStream_t st);
 int launch_wqmm_plain(const OpsnnWqmmArgs& a, hipStream_t st);
 // Return OPSNN_NOT_TAKEN when the arguments are outside what the fast kernels handle.
 int launch_blockscale_mfma(const OpsnnQmmArgs& a, hipStream_t st);
@@ -53,6 +54,21 @@ extern "C" int opsnnQmmMx(const OpsnnQmmArgs* a, void* stream)
     return launch_mx_plain(*a, (hipStream_t)stream);
 }
 
+// Per-tensor / per-channel family.  The per-token x per-channel int8 kernel already covers int8 operands with a
+// float scale and a 16-bit output when the scale needs no 19-bit truncation; everything else (64-bit packed scales,
+// int8 requantisation, fp8 operands, truncated scales) runs on the plain kernel.
+extern "C" int opsnnQmmTc(const OpsnnQmmArgs* a, void* stream)
+{
+    if (!qmm_args_ok(a) || !a->x2_scale) return -1;
+    const bool i8 = a->x1_dtype == DT_I8 && a->x2_dtype == DT_I8;
+    const bool f8 = (a->x1_dtype == DT_E4M3 || a->x1_dtype == DT_E5M2) && (a->x2_dtype == DT_E4M3 || a->x2_dtype == DT_E5M2);
+    if (!i8 && !f8) return -2;
+    if (a->x2_scale_len != 1 && a->x2_scale_len != a->N) return -2;
+    if (a->x1_scale && (a->x1_scale_len != 1 || !f8)) return -2;
+    if (a->out_dtype == DT_I8 || a->out_dtype == DT_I32) { if (!i8) return -2; }
+    return launch_tc_plain(*a, (hipStream_t)stream);
+}
+
 extern "C" int opsnnWqmm(const OpsnnWqmmArgs* a, void* stream)
 {
     if (!a || !a->x || !a->w.ptr || !a->scale.ptr || !a->y || a->M <= 0 || a->N <= 0 || a->K <= 0) return -1;
@@ -64,7 +80,7 @@ extern "C" int opsnnWqmm(const OpsnnWqmmArgs* a, void* stream)
     return launch_wqmm_plain(*a, (hipStream_t)stream);
 }
 
-// mode: 0 = int8 per-token/per-channel, 1 = block scale, 2 = MX.
+// mode: 0 = int8 per-token/per-channel, 1 = block scale, 2 = MX, 3 = per-tensor / per-channel family.
 // The MFMA kernels stream a K-contiguous right operand ("x2 stored [N, K]").  An N-contiguous x2 is
 // first re-laid out into the workspace; callers who keep x2 in [N, K] form (transposeX2 = true or a
 // transposed view) need no workspace and skip that pass.
@@ -72,6 +88,7 @@ extern "C" uint64_t opsnnQmmWorkspace(const OpsnnQmmArgs* a, int mode)
 {
     if (!a) return 0;
     if (mode == 2) return mx_workspace_bytes(*a);
+    if (mode == 3) return 0;   // per-tensor / per-channel family: strided kernel, no re-layout
     if (a->x2.row_stride == 1 || a->K == 1) return 0;           // already K-contiguous
     if (a->x2.col_stride != 1 || a->x2.row_stride != a->N) return 0;  // not a dense [K, N]: plain kernel
     uint64_t bits = (a->x2_dtype == DT_I4 || a->x2_dtype == DT_E2M1) ? 4 : 8;

@@ -70,6 +70,92 @@ __global__ void qmm_mx_plain(OpsnnQmmArgs a)
     store_f32_as(a.out, a.out_dtype, (bz * a.M + m) * a.N + n, acc);
 }
 
+// per-tensor / per-channel family: see opsnnQmmTc in opsnn_kernels.h and qbmmv3_kernel_golden.py:390-513
+__device__ __forceinline__ float trunc19(float s) { return u2f(f2u(s) & 0xFFFFE000u); }
+__device__ __forceinline__ float s9f(float v)
+{
+    const float r = __builtin_rintf(v);   // round half to even
+    return r < -256.0f ? -256.0f : (r > 255.0f ? 255.0f : r);
+}
+__global__ void qmm_tc_plain(OpsnnQmmArgs a)
+{
+    const int64_t nchunks = (a.N + blockDim.x - 1) / blockDim.x;
+    const int64_t m = blockIdx.x / nchunks;
+    const int64_t n = (blockIdx.x % nchunks) * (int64_t)blockDim.x + threadIdx.x;
+    const int64_t bz = blockIdx.y;
+    if (n >= a.N) return;
+    const bool is_int = a.x1_dtype == DT_I8;
+    const int64_t abase = bz * a.x1.batch_stride + m * a.x1.row_stride;
+    const int64_t bbase = bz * a.x2.batch_stride + n * a.x2.col_stride;
+    int32_t iacc = 0;
+    float facc = 0.0f;
+    if (is_int) {
+        const int8_t* x1 = (const int8_t*)a.x1.ptr;
+        const int8_t* x2 = (const int8_t*)a.x2.ptr;
+        for (int64_t k = 0; k < a.K; k++) iacc += (int32_t)x1[abase + k * a.x1.col_stride] * (int32_t)x2[bbase + k * a.x2.row_stride];
+    } else {
+        for (int64_t k = 0; k < a.K; k++) {
+            const float x = load_q_as_f32(a.x1.ptr, a.x1_dtype, abase + k * a.x1.col_stride);
+            const float w = load_q_as_f32(a.x2.ptr, a.x2_dtype, bbase + k * a.x2.row_stride);
+            facc = __fadd_rn(facc, __fmul_rn(x, w));
+        }
+    }
+    const int64_t si = a.x2_scale_len == 1 ? 0 : n;
+    const bool u64 = a.x2_scale_dtype == DT_U64;
+    const uint64_t packed = u64 ? ((const uint64_t*)a.x2_scale)[si] : 0;
+    const float s = u64 ? trunc19(u2f((uint32_t)packed)) : load_scalar_as_f32(a.x2_scale, a.x2_scale_dtype, si);
+    const int64_t bi = bz * a.bias_batch_stride + n;
+    const int64_t o_idx = (bz * a.M + m) * a.N + n;
+    const bool bias_i32 = a.bias && a.bias_dtype == DT_I32, bias_float = a.bias && a.bias_dtype != DT_I32;
+    if (a.out_dtype == DT_I8) {
+        int32_t v = iacc;
+        if (bias_i32) v += ((const int32_t*)a.bias)[bi];
+        float o = s9f(__fmul_rn((float)v, s));
+        bool has_off = a.x2_offset != nullptr || u64;
+        if (has_off) {
+            float off;
+            if (a.x2_offset) off = a.x2_offset[a.x2_offset_len == 1 ? 0 : n];
+            else {
+                int64_t raw = (int64_t)((packed >> 37) & 0x1FF);
+                if (raw & 0x100) raw -= 0x200;
+                off = (float)raw;
+            }
+            o = __fadd_rn(s9f(o), s9f(off));
+        }
+        o = o < -128.0f ? -128.0f : (o > 127.0f ? 127.0f : o);
+        ((int8_t*)a.out)[o_idx] = (int8_t)o;
+        return;
+    }
+    if (a.out_dtype == DT_I32) {
+        int32_t v = iacc;
+        if (bias_i32) v += ((const int32_t*)a.bias)[bi];
+        else if (bias_float) v = (int32_t)__fadd_rn((float)v, load_scalar_as_f32(a.bias, a.bias_dtype, bi));
+        ((int32_t*)a.out)[o_idx] = v;
+        return;
+    }
+    const bool pertoken = a.x1_scale != nullptr;
+    const bool do_scale_gen = is_int && a.x2_scale_len == 1 && !(a.bias && (a.bias_dtype == DT_BF16 || a.bias_dtype == DT_F32));
+    const bool is_bias_vec = bias_float && (is_int || pertoken);
+    float o;
+    if (is_int) {
+        int32_t v = iacc;
+        if (!is_bias_vec && bias_i32) v += ((const int32_t*)a.bias)[bi];
+        o = (float)v;
+    } else {
+        o = facc;
+    }
+    if (!is_bias_vec && bias_float) o = __fadd_rn(o, load_scalar_as_f32(a.bias, a.bias_dtype, bi));
+    if (pertoken) {
+        const float pt = ((const float*)a.x1_scale)[0];
+        if (a.x2_scale_len == 1 && !is_bias_vec) o = __fmul_rn(o, trunc19(__fmul_rn(s, pt)));
+        else o = __fmul_rn(__fmul_rn(o, do_scale_gen ? trunc19(s) : s), pt);
+    } else {
+        o = __fmul_rn(o, do_scale_gen ? trunc19(s) : s);
+    }
+    if (is_bias_vec) o = __fadd_rn(o, load_scalar_as_f32(a.bias, a.bias_dtype, bi));
+    store_f32_as(a.out, a.out_dtype, o_idx, o);
+}
+
 __device__ __forceinline__ float round_through(float v, int dt)
 {
     if (dt == DT_F16) return f16_to_f32(f16_bits(v));
@@ -113,6 +199,12 @@ int launch_blockscale_plain(const OpsnnQmmArgs& a, hipStream_t st)
 {
     dim3 block(256), grid((unsigned)(((a.N + 255) / 256) * a.M), (unsigned)a.batch);
     hipLaunchKernelGGL(qmm_blockscale_plain, grid, block, 0, st, a);
+    return (int)hipGetLastError();
+}
+int launch_tc_plain(const OpsnnQmmArgs& a, hipStream_t st)
+{
+    dim3 block(256), grid((unsigned)(((a.N + 255) / 256) * a.M), (unsigned)a.batch);
+    hipLaunchKernelGGL(qmm_tc_plain, grid, block, 0, st, a);
     return (int)hipGetLastError();
 }
 int launch_mx_plain(const OpsnnQmmArgs& a, hipStream_t st)

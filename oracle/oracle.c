@@ -23,6 +23,8 @@
  *   codecs ............ pinned (exhaustive tables vs OCP definitions, torch CPU dtypes, reference constants)
  *   orc_qmm_int8_acc .. pinned (brute force, closed forms, identity operands)
  *   orc_qmm_pertoken .. pinned (float64 recomputation, operation-order cases, all-ones example)
+ *   orc_qmm_tc ........ pinned (reduces to orc_qmm_pertoken with a constant row scale; hand-computed requant and
+ *                       19-bit truncation cases; uint64 packing constants of the reference's utility)
  *   orc_qmm_perblock .. pinned (reduces to pertoken formula with one K block; power-of-two scales exact; float64)
  *   orc_qmm_mx ........ pinned (power-of-two products are exact: equals integer arithmetic; float64)
  *   orc_wqbmm ......... pinned (hand-computed double-rounding cases; group==K equals per-channel; float64)
@@ -368,6 +370,113 @@ int orc_qmm_pertoken(const int8_t* x1, const int8_t* x2, int64_t M, int64_t K, i
     if (rc == 0) rc = orc_qmm_pertoken_epilogue(acc, M, N, x1s, x2s, x2s_len, bias, bias_dt, y_dt, y);
     if (!acc_out) free(acc);
     return rc;
+}
+
+/*
+ * compute_tc / compute_requant / compute_int32 (G3:390-506): the T-T / T-C family, one batch slice, with
+ *   the mode rules of determine_quant_mode (G3:62-145): a one-element per-token scale with fp8 inputs is the
+ *     "doublescale" form -- merged and truncated when x2Scale has one element too (T-T), multiplied separately
+ *     when it has N (T-C);
+ *   needs_scale_generate (GQ:62-72): int inputs, a one-element scale and a bias that is neither bf16 nor fp32 ->
+ *     the scale keeps its upper 19 bits;
+ *   is_bias_vec (G3:574-581): a float bias is added after the scaling for int inputs, and for fp8 inputs when a
+ *     per-token scale is present; otherwise before it (an int32 bias is added to the int32 sums);
+ *   the uint64 decoding of the aclnn-level golden (matmul/quant_batch_matmul_v4/tests/assets/
+ *     qbmmv4_aclnn_golden.py:276-316): scale = fp32 from the low word with the upper 19 bits kept, offset =
+ *     the x2Offset tensor if there is one, else the signed 9-bit field at bits 37..45.
+ * scale_dt: ORC_F32, ORC_BF16 or ORC_U64.  y_dt ORC_I8 -> requant, ORC_I32 -> integer sums, else cast of the scaled sum.
+ */
+static float s9(float v)   /* f32_2_s9 (GQ:57-59): round half to even, clip to [-256, 255] */
+{
+    float r = rintf(v);
+    return r < -256.0f ? -256.0f : (r > 255.0f ? 255.0f : r);
+}
+
+int orc_qmm_tc(const void* x1, const void* x2, int dt1, int dt2, int64_t M, int64_t K, int64_t N, int tA, int tB,
+               const void* scale, int scale_dt, int64_t scale_len, const float* pertoken, const float* offset,
+               int64_t offset_len, const void* bias, int bias_dt, int y_dt, void* y)
+{
+    const int is_int = dt1 == ORC_I8 || dt1 == ORC_I4;
+    const int bias_float = bias && bias_dt != ORC_I32;
+    float* sc = (float*)malloc(sizeof(float) * (size_t)scale_len);
+    float* dec_off = NULL;
+    if (!sc) return -1;
+    for (int64_t i = 0; i < scale_len; i++) {
+        if (scale_dt == ORC_U64) sc[i] = orc_u64_to_deq_scale(((const uint64_t*)scale)[i]);
+        else sc[i] = load_as_f32(scale, scale_dt, (size_t)i);
+    }
+    if (y_dt == ORC_I8 && !offset && scale_dt == ORC_U64) {
+        dec_off = (float*)malloc(sizeof(float) * (size_t)scale_len);
+        if (!dec_off) return -1;
+        for (int64_t i = 0; i < scale_len; i++) {
+            int64_t raw = (int64_t)((((const uint64_t*)scale)[i] >> 37) & 0x1FF);
+            if (raw & 0x100) raw -= 0x200;
+            dec_off[i] = (float)raw;
+        }
+        offset = dec_off; offset_len = scale_len;
+    }
+    int32_t* iacc = NULL;
+    float* facc = NULL;
+    if (is_int) {
+        iacc = (int32_t*)malloc(sizeof(int32_t) * (size_t)M * N);
+        if (!iacc || orc_qmm_int8_acc((const int8_t*)x1, (const int8_t*)x2, M, K, N, tA, tB, iacc) != 0) return -1;
+    } else {
+        float* a = tA ? decode_matrix(x1, dt1, K, M, 1) : decode_matrix(x1, dt1, M, K, 0);
+        float* b = tB ? decode_matrix(x2, dt2, N, K, 1) : decode_matrix(x2, dt2, K, N, 0);
+        facc = (float*)calloc((size_t)M * N, sizeof(float));
+        if (!a || !b || !facc) return -1;
+        sgemm_acc(a, K, b, N, facc, N, M, N, K);
+        free(a); free(b);
+    }
+    const int do_scale_gen = is_int && scale_len == 1 && !(bias && (bias_dt == ORC_BF16 || bias_dt == ORC_F32));
+    const int is_bias_vec = bias_float && (is_int || pertoken != NULL);
+    const int merge_trunc = pertoken != NULL && scale_len == 1;   /* T-T-doublescale */
+#pragma omp parallel for schedule(static)
+    for (int64_t m = 0; m < M; m++)
+        for (int64_t n = 0; n < N; n++) {
+            const size_t i = (size_t)(m * N + n);
+            const float s = sc[scale_len == 1 ? 0 : n];
+            if (y_dt == ORC_I8) {            /* compute_requant (G3:478-496) */
+                int32_t a = iacc[i];
+                if (bias && bias_dt == ORC_I32) a += ((const int32_t*)bias)[n];
+                float o = s9((float)a * s);
+                if (offset) o = s9(o) + s9(offset[offset_len == 1 ? 0 : n]);
+                o = o < -128.0f ? -128.0f : (o > 127.0f ? 127.0f : o);
+                ((int8_t*)y)[i] = (int8_t)o;
+                continue;
+            }
+            if (y_dt == ORC_I32) {           /* compute_int32 (G3:499-513) */
+                int32_t a = iacc[i];
+                if (bias && bias_dt == ORC_I32) ((int32_t*)y)[i] = a + ((const int32_t*)bias)[n];
+                else if (bias) ((int32_t*)y)[i] = (int32_t)((float)a + load_as_f32(bias, bias_dt, (size_t)n));
+                else ((int32_t*)y)[i] = a;
+                continue;
+            }
+            float o;                         /* compute_tc (G3:390-475) */
+            if (is_int) {
+                int32_t a = iacc[i];
+                if (!is_bias_vec && bias && bias_dt == ORC_I32) a += ((const int32_t*)bias)[n];
+                o = (float)a;
+            } else {
+                o = facc[i];
+            }
+            if (!is_bias_vec && bias_float) o = o + load_as_f32(bias, bias_dt, (size_t)n);
+            if (pertoken) {
+                if (merge_trunc && !is_bias_vec) {
+                    o = o * orc_scale_generate(s * pertoken[0]);
+                } else {
+                    const float s2 = do_scale_gen ? orc_scale_generate(s) : s;
+                    o = o * s2;
+                    o = o * pertoken[0];
+                }
+            } else {
+                o = o * (do_scale_gen ? orc_scale_generate(s) : s);
+            }
+            if (is_bias_vec) o = o + load_as_f32(bias, bias_dt, (size_t)n);
+            store_from_f32(y, y_dt, i, o);
+        }
+    free(sc); free(dec_off); free(iacc); free(facc);
+    return 0;
 }
 
 /*

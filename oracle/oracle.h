@@ -13,7 +13,7 @@ extern "C" {
 
 enum {
     ORC_F32 = 0, ORC_F16 = 1, ORC_I8 = 2, ORC_I32 = 3, ORC_BF16 = 27, ORC_I4 = 29,
-    ORC_E5M2 = 35, ORC_E4M3 = 36, ORC_E8M0 = 37, ORC_E2M1 = 40
+    ORC_E5M2 = 35, ORC_E4M3 = 36, ORC_E8M0 = 37, ORC_E2M1 = 40, ORC_U64 = 10
 };
 
 uint16_t orc_bf16_from_f32(float f);
@@ -47,6 +47,9 @@ int orc_qmm_pertoken_epilogue(const int32_t* acc, int64_t M, int64_t N, const fl
 int orc_qmm_pertoken(const int8_t* x1, const int8_t* x2, int64_t M, int64_t K, int64_t N, int tA, int tB,
                      const float* x1s, const float* x2s, int64_t x2s_len, const void* bias, int bias_dt, int y_dt,
                      void* y, int32_t* acc_out);
+int orc_qmm_tc(const void* x1, const void* x2, int dt1, int dt2, int64_t M, int64_t K, int64_t N, int tA, int tB,
+               const void* scale, int scale_dt, int64_t scale_len, const float* pertoken, const float* offset,
+               int64_t offset_len, const void* bias, int bias_dt, int y_dt, void* y);
 int orc_qmm_perblock(const void* x1, const void* x2, int dt1, int dt2, int64_t M, int64_t K, int64_t N, int tA,
                      int tB, const float* x1s, const float* x2s, int64_t gsM, int64_t gsN, int64_t gsK,
                      const float* bias, int y_dt, void* y);

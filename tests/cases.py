@@ -174,6 +174,58 @@ def run_blockscale_aclnn(m, inp, M, K, N, tB, out_dtype, group_size=None):
 
 
 # --------------------------------------------------------------------------------------------------
+# per-tensor / per-channel family (T-T, T-C; 64-bit packed scales, int8 requantisation, fp8 double scale)
+# --------------------------------------------------------------------------------------------------
+def make_tc_inputs(m, M, K, N, seed, in_dt, scale_dt, scale_len, bias_dt, tB, pertoken=False, offset_len=0, e5m2=False):
+    """in_dt: ACL_INT8 or an fp8 type; scale_dt: ACL_FLOAT / ACL_BF16 / ACL_UINT64; offset_len: 0 (none), 1 or N."""
+    rng = np.random.default_rng(seed)
+    if in_dt == m.ACL_INT8:
+        x1, x2 = gen_int8(rng, (M, K)), gen_int8(rng, (N, K) if tB else (K, N))
+    else:
+        x1, x2 = gen_fp8(rng, (M, K)), gen_fp8(rng, (N, K) if tB else (K, N))
+        if e5m2:   # any byte pattern below infinity is a finite e5m2 value
+            x1, x2 = (x1 & 0xBB).astype(np.uint8), (x2 & 0xBB).astype(np.uint8)
+    sf = gen_scale(rng, N if scale_len != 1 else 1, 1e-3, 1e-2) if in_dt == m.ACL_INT8 else gen_scale(rng, N if scale_len != 1 else 1, 0.05, 0.5)
+    if scale_dt == m.ACL_UINT64:
+        scale = orc.pack_u64_scale(sf)
+    elif scale_dt == m.ACL_BF16:
+        scale = orc.f32_to_bf16(sf)
+    else:
+        scale = sf
+    pt = gen_scale(rng, 1, 0.5, 2.0) if pertoken else None
+    off = rng.uniform(-20, 20, size=offset_len).astype(np.float32) if offset_len else None
+    bias = gen_bias(rng, N, bias_dt, m)
+    if bias_dt == m.ACL_INT32 and bias is not None:
+        bias = rng.integers(-3000, 3000, size=N).astype(np.int32)
+    return dict(x1=x1, x2=x2, scale=scale, scale_dt=scale_dt, pt=pt, off=off, bias=bias, bias_dt=bias_dt, in_dt=in_dt, tB=tB,
+                x2_dt=in_dt)
+
+
+def oracle_tc(m, inp, M, K, N, out_dt):
+    return orc.qmm_tc(inp["x1"], inp["x2"], inp["in_dt"], inp["x2_dt"], M, K, N, False, inp["tB"], inp["scale"], inp["scale_dt"],
+                      inp["pt"], inp["off"], inp["bias"], inp["bias_dt"] or 0, out_dt)
+
+
+def run_tc_aclnn(m, inp, M, K, N, out_dt):
+    d = {k: m.DeviceBuffer(host=v) for k, v in inp.items() if isinstance(v, np.ndarray)}
+    out_np = orc.out_array((M, N), out_dt)
+    d_out = m.DeviceBuffer(out_np.nbytes)
+    d_out.fill(0x7F)
+    tB = inp["tB"]
+    x1 = m.Tensor((M, K), inp["in_dt"], d["x1"])
+    x2 = m.Tensor((N, K) if tB else (K, N), inp["x2_dt"], d["x2"])
+    s2 = m.Tensor((inp["scale"].size,), inp["scale_dt"], d["scale"])
+    s1 = m.Tensor((1,), m.ACL_FLOAT, d["pt"]) if inp["pt"] is not None else None
+    off = m.Tensor((inp["off"].size,), m.ACL_FLOAT, d["off"]) if inp["off"] is not None else None
+    bias = m.Tensor((N,), inp["bias_dt"], d["bias"]) if inp["bias"] is not None else None
+    out = m.Tensor((M, N), out_dt, d_out)
+    ws = m.quant_matmul_v5(x1, x2, s1, s2, out, bias=bias, x2_offset=off, transpose_x2=tB)
+    m.check(m.lib().aclrtSynchronizeDevice(), "sync")
+    del ws
+    return d_out.to_host(out_np.dtype, out_np.shape)
+
+
+# --------------------------------------------------------------------------------------------------
 # MX (fp4 / fp8 with e8m0 scales per 32 K)
 # --------------------------------------------------------------------------------------------------
 def make_mx_inputs(m, M, K, N, seed, tB, fp4=True, batch=1, exp_range=4):

@@ -10,6 +10,7 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 LIB = os.path.join(ROOT, "oracle", "liboracle.so")
 
 F32, F16, I8, I32, BF16, I4, E5M2, E4M3, E8M0, E2M1 = 0, 1, 2, 3, 27, 29, 35, 36, 37, 40
+U64 = 10
 _lib = None
 
 
@@ -25,6 +26,7 @@ def lib():
         L.orc_qmm_pertoken_epilogue.argtypes = [vp, i64, i64, vp, vp, i64, vp, ci, ci, vp]
         L.orc_qmm_pertoken.argtypes = [vp, vp, i64, i64, i64, ci, ci, vp, vp, i64, vp, ci, ci, vp, vp]
         L.orc_qmm_perblock.argtypes = [vp, vp, ci, ci, i64, i64, i64, ci, ci, vp, vp, i64, i64, i64, vp, ci, vp]
+        L.orc_qmm_tc.argtypes = [vp, vp, ci, ci, i64, i64, i64, ci, ci, vp, ci, i64, vp, vp, i64, vp, ci, ci, vp]
         L.orc_qmm_mx.argtypes = [vp, vp, ci, ci, i64, i64, i64, ci, ci, vp, vp, vp, ci, vp]
         L.orc_wqbmm.argtypes = [vp, ci, vp, ci, i64, i64, i64, ci, vp, ci, i64, vp, i64, vp, ci, vp]
         for n in ("orc_vec_f32_to_bf16", "orc_vec_bf16_to_f32", "orc_vec_f32_to_f16", "orc_vec_f16_to_f32",
@@ -89,7 +91,7 @@ def f32_to_b16(v, dt):
 
 
 def out_array(shape, dt):
-    return np.empty(shape, np.float32 if dt == F32 else (np.int32 if dt == I32 else np.uint16))
+    return np.empty(shape, {F32: np.float32, I32: np.int32, I8: np.int8}.get(dt, np.uint16))
 
 
 def qmm_pertoken(x1, x2, M, K, N, tA, tB, x1s, x2s, bias, bias_dt, y_dt, want_acc=False):
@@ -114,6 +116,29 @@ def qmm_perblock(x1, x2, dt1, dt2, M, K, N, tA, tB, x1s, x2s, gsM, gsN, gsK, bia
                                 y_dt, _p(y))
     assert rc == 0
     return y
+
+
+def qmm_tc(x1, x2, dt1, dt2, M, K, N, tA, tB, scale, scale_dt, pertoken, offset, bias, bias_dt, y_dt):
+    """Per-tensor / per-channel family; scale is float32 / bf16 bits / uint64 words according to scale_dt."""
+    y = out_array((M, N), y_dt)
+    scale = np.ascontiguousarray(scale)
+    offset = None if offset is None else np.ascontiguousarray(offset, np.float32)
+    pertoken = None if pertoken is None else np.ascontiguousarray(pertoken, np.float32)
+    rc = lib().orc_qmm_tc(_p(x1), _p(x2), dt1, dt2, M, K, N, int(tA), int(tB), _p(scale), scale_dt, scale.size, _p(pertoken),
+                          _p(offset), 0 if offset is None else offset.size, _p(bias), bias_dt, y_dt, _p(y))
+    assert rc == 0
+    return y
+
+
+def pack_u64_scale(scale_f32, offset_f32=None):
+    """The 64-bit packed scale of the static modes: fp32 bits in the low word, bit 46 set, the offset as a signed
+    9-bit integer at bits 37..45 (layout read by u64_to_deq_scale / u64_to_offset, matmul_quant_util.py:129-158)."""
+    u = np.ascontiguousarray(scale_f32, np.float32).view(np.uint32).astype(np.uint64)
+    u |= np.uint64(1 << 46)
+    if offset_f32 is not None:
+        s9 = np.clip(np.rint(np.asarray(offset_f32, np.float32)), -256, 255).astype(np.int64)
+        u |= (s9.astype(np.uint64) & np.uint64(0x1FF)) << np.uint64(37)
+    return u
 
 
 def qmm_mx(x1, x2, dt1, dt2, M, K, N, tA, tB, x1s, x2s, bias, y_dt):

@@ -1,0 +1,163 @@
+"""Per-tensor / per-channel quantized matmul (T-T, T-C): 64-bit packed scales, int8 requantisation, int32 output,
+19-bit scale truncation, fp8 operands with the one-element per-token scale ("double scale").
+
+CPU part: the oracle's orc_qmm_tc is pinned by recomputing the reference formulas
+(matmul/quant_batch_matmul_v3/tests/assets/qbmmv3_kernel_golden.py:390-513) independently in numpy on small
+cases, by hand-computed requantisation values, and by the case that reduces to the per-token function.
+GPU part: the library through the aclnn C ABI must be bit-identical to the oracle for integer operands (exact
+int32 sums, the same fp32 operation order) and for fp8 operands too (the kernel sums in ascending k like the oracle).
+"""
+import numpy as np
+import pytest
+
+import cases
+import oracle_api as orc
+
+
+def trunc19(a):
+    return (np.asarray(a, np.float32).view(np.uint32) & np.uint32(0xFFFFE000)).view(np.float32)
+
+
+def s9(a):
+    return np.clip(np.round(np.asarray(a, np.float32)), -256, 255).astype(np.float32)
+
+
+def test_requant_hand_values():
+    # acc = 1*3 + 2*4 = 11; 11 * 0.5 = 5.5 -> 6 (half to even); offset 2.5 -> 2; 6 + 2 = 8
+    x1 = np.array([[1, 2]], np.int8); x2 = np.array([[3], [4]], np.int8)
+    sc = orc.pack_u64_scale(np.array([0.5], np.float32))
+    y = orc.qmm_tc(x1, x2, orc.I8, orc.I8, 1, 2, 1, False, False, sc, orc.U64, None, np.array([2.5], np.float32), None, 0, orc.I8)
+    assert y[0, 0] == 8
+    # 4.5 -> 4 (half to even); no offset tensor: the offset packed in the scale word is used (-3)
+    sc = orc.pack_u64_scale(np.array([4.5 / 11], np.float32), np.array([-3.0], np.float32))
+    y = orc.qmm_tc(x1, x2, orc.I8, orc.I8, 1, 2, 1, False, False, sc, orc.U64, None, None, None, 0, orc.I8)
+    want = np.float32(11) * trunc19(np.float32(4.5 / 11))
+    assert y[0, 0] == int(np.clip(s9(want) - 3, -128, 127))
+    # saturation: 11 * 100 -> s9 clips to 255, + 10 -> 265 -> int8 clips to 127; negative side to -128
+    sc = orc.pack_u64_scale(np.array([100.0, -100.0], np.float32))
+    x2b = np.array([[3, 3], [4, 4]], np.int8)
+    y = orc.qmm_tc(x1, x2b, orc.I8, orc.I8, 1, 2, 2, False, False, sc, orc.U64, None, np.array([10.0], np.float32), None, 0, orc.I8)
+    assert list(y[0]) == [127, -128]
+
+
+def test_packed_scale_layout():
+    # bit 46 set, fp32 bits low, offset field at 37..45 (two's complement 9 bits)
+    w = orc.pack_u64_scale(np.array([1.0], np.float32), np.array([-1.0], np.float32))[0]
+    assert int(w) & 0xFFFFFFFF == 0x3F800000 and (int(w) >> 46) & 1 == 1 and (int(w) >> 37) & 0x1FF == 0x1FF
+    assert orc.lib().orc_u64_to_deq_scale(int(w)) == 1.0
+    # a scale with low mantissa bits loses them: 0.1 = 0x3DCCCCCD -> 0x3DCCC000
+    w = orc.pack_u64_scale(np.array([0.1], np.float32))[0]
+    assert np.float32(orc.lib().orc_u64_to_deq_scale(int(w))).view(np.uint32) == 0x3DCCC000
+
+
+@pytest.mark.parametrize("scale_len,bias_dt,y_dt", [(1, "i32", "f16"), ("N", "i32", "f16"), (1, "f16", "f16"), (1, "bf16", "bf16"),
+                                                    ("N", None, "bf16"), (1, None, "i32"), ("N", "i32", "i32"), ("N", "i32", "i8")])
+def test_int8_formulas_against_numpy(scale_len, bias_dt, y_dt):
+    M, K, N = 7, 40, 12
+    rng = np.random.default_rng(5)
+    x1 = rng.integers(-127, 128, (M, K), dtype=np.int8); x2 = rng.integers(-127, 128, (K, N), dtype=np.int8)
+    sf = rng.uniform(1e-3, 1e-2, 1 if scale_len == 1 else N).astype(np.float32)
+    codes = {"i32": orc.I32, "f16": orc.F16, "bf16": orc.BF16, "i8": orc.I8, None: 0}
+    if bias_dt == "i32":
+        bias = rng.integers(-500, 500, N).astype(np.int32); bias_f = None
+    elif bias_dt is None:
+        bias = None
+    else:
+        bias_f = rng.normal(0, 1, N).astype(np.float32)
+        bias = orc.f32_to_b16(bias_f, codes[bias_dt]); bias_f = orc.b16_to_f32(bias, codes[bias_dt])
+    u64 = y_dt == "i8"
+    scale = orc.pack_u64_scale(sf) if u64 else sf
+    got = orc.qmm_tc(x1, x2, orc.I8, orc.I8, M, K, N, False, False, scale, orc.U64 if u64 else orc.F32, None, None, bias,
+                     codes[bias_dt], codes[y_dt])
+    acc = x1.astype(np.int32) @ x2.astype(np.int32)
+    if y_dt == "i32":
+        want = acc + bias if bias is not None else acc
+        assert np.array_equal(got, want)
+        return
+    if y_dt == "i8":
+        o = s9((acc + bias).astype(np.float32) * trunc19(sf))
+        want = np.clip(s9(o) + np.float32(0), -128, 127).astype(np.int8)   # offset field of the packed word is 0
+        assert np.array_equal(got, want)
+        return
+    # compute_tc: int32 bias before scaling; float bias after (int operands); a one-element scale is truncated to
+    # 19 bits unless the bias is bf16 / fp32
+    s = sf
+    if scale_len == 1 and bias_dt not in ("bf16",):
+        s = trunc19(sf)
+    o = (acc + bias if bias_dt == "i32" else acc).astype(np.float32) * s
+    if bias_dt in ("f16", "bf16"):
+        o = o + bias_f
+    want = orc.f32_to_b16(o.astype(np.float32), codes[y_dt])
+    assert np.array_equal(got, want)
+
+
+def test_tc_without_truncation_equals_pertoken_function():
+    # T-C with N scales and a float bias is the per-token formula with no row scale: the already pinned function
+    M, K, N = 9, 64, 20
+    rng = np.random.default_rng(6)
+    x1 = rng.integers(-127, 128, (M, K), dtype=np.int8); x2 = rng.integers(-127, 128, (N, K), dtype=np.int8)
+    sf = rng.uniform(1e-3, 1e-2, N).astype(np.float32)
+    bias = orc.f32_to_bf16(rng.normal(0, 1, N).astype(np.float32))
+    a = orc.qmm_tc(x1, x2, orc.I8, orc.I8, M, K, N, False, True, sf, orc.F32, None, None, bias, orc.BF16, orc.BF16)
+    b = orc.qmm_pertoken(x1, x2, M, K, N, False, True, None, sf, bias, orc.BF16, orc.BF16)
+    assert np.array_equal(a, b)
+
+
+@pytest.mark.parametrize("scale_len", [1, "N"])
+def test_fp8_double_scale_against_numpy(scale_len):
+    # fp8 operands, one-element per-token scale, fp32 bias (added after the scaling).  With a one-element x2 scale
+    # the bias-after form still multiplies separately (the merged, truncated product is the no-bias cube path).
+    M, K, N = 5, 32, 8
+    rng = np.random.default_rng(7)
+    x1 = orc.f32_to_e4m3(rng.normal(0, 1, (M, K)).astype(np.float32)); x2 = orc.f32_to_e4m3(rng.normal(0, 1, (K, N)).astype(np.float32))
+    sf = rng.uniform(0.05, 0.5, 1 if scale_len == 1 else N).astype(np.float32)
+    pt = np.array([1.37], np.float32)
+    bias = rng.normal(0, 1, N).astype(np.float32)
+    mm = np.zeros((M, N), np.float32)
+    a, b = orc.e4m3_to_f32(x1), orc.e4m3_to_f32(x2)
+    for k in range(K):   # ascending k, fp32
+        mm = (mm + a[:, k:k + 1] * b[k:k + 1, :]).astype(np.float32)
+    got = orc.qmm_tc(x1, x2, orc.E4M3, orc.E4M3, M, K, N, False, False, sf, orc.F32, pt, None, bias, orc.F32, orc.F16)
+    want = orc.f32_to_f16(((mm * sf).astype(np.float32) * pt[0]).astype(np.float32) + bias)
+    assert np.array_equal(got, want)
+    # without a bias and with a one-element x2 scale the two scales are merged and truncated to 19 bits
+    got = orc.qmm_tc(x1, x2, orc.E4M3, orc.E4M3, M, K, N, False, False, sf, orc.F32, pt, None, None, 0, orc.F32)
+    if scale_len == 1:
+        want = mm * trunc19(sf * pt[0])
+    else:
+        want = (mm * sf).astype(np.float32) * pt[0]
+    assert np.array_equal(got, want.astype(np.float32))
+
+
+GPU_CASES = [
+    # M, K, N, in, scale dtype, scale len, bias, out, tB, pertoken, offset len
+    (16, 32, 16, "i8", "u64", 1, "i32", "f16", False, False, 0),      # the reference's A8W8FP16_pertensor row
+    (16, 32, 16, "i8", "u64", "N", "i32", "f16", False, False, 0),    # A8W8FP16_perchannel
+    (16, 32, 16, "i8", "u64", 1, "i32", "i8", False, False, 1),       # A8W8C8_pertensor_offset
+    (16, 32, 16, "i8", "u64", "N", "i32", "i8", False, False, 1),     # A8W8C8_perchannel_offset
+    (33, 200, 70, "i8", "u64", "N", "i32", "i8", True, False, "N"),
+    (33, 200, 70, "i8", "u64", "N", None, "i8", False, False, 0),     # offset taken from the packed word (zero)
+    (40, 96, 50, "i8", "f32", 1, "i32", "bf16", True, False, 0),      # per-tensor float scale: 19-bit truncation
+    (40, 96, 50, "i8", "f32", 1, "f32", "bf16", True, False, 0),      # fp32 bias: no truncation of the scale
+    (40, 96, 50, "i8", "bf16", 1, None, "bf16", False, False, 0),
+    (40, 96, 50, "i8", "f32", "N", "i32", "i32", False, False, 0),
+    (16, 32, 16, "e4m3", "f32", "N", "f32", "f16", False, True, 0),   # FP8E4M3..dynamic_tc_bias_float
+    (16, 32, 16, "e5m2", "f32", "N", "f32", "bf16", False, True, 0),  # FP8E5M2..dynamic_tc_bias_float
+    (37, 160, 48, "e4m3", "f32", 1, None, "bf16", True, True, 0),     # both scales one element: merged and truncated
+    (37, 160, 48, "e4m3", "u64", "N", None, "f32", True, False, 0),   # T-C without a per-token scale: packed scale
+    (37, 160, 48, "e4m3", "u64", 1, "f32", "f16", False, False, 0),   # float bias before the scaling (no per-token scale)
+]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("M,K,N,in_dt,s_dt,s_len,bias_dt,out_dt,tB,pt,off_len", GPU_CASES)
+def test_gpu_matches_oracle(gpu, M, K, N, in_dt, s_dt, s_len, bias_dt, out_dt, tB, pt, off_len):
+    m = gpu
+    dt = {"i8": m.ACL_INT8, "e4m3": m.ACL_FLOAT8_E4M3FN, "e5m2": m.ACL_FLOAT8_E5M2, "u64": m.ACL_UINT64, "f32": m.ACL_FLOAT,
+          "bf16": m.ACL_BF16, "f16": m.ACL_FLOAT16, "i32": m.ACL_INT32, None: None}
+    print(f"case tc {M}x{K}x{N} in={in_dt} scale={s_dt}/{s_len} bias={bias_dt} out={out_dt} tB={tB} pt={pt} off={off_len}", flush=True)
+    inp = cases.make_tc_inputs(m, M, K, N, M + N, dt[in_dt], dt[s_dt], 1 if s_len == 1 else N, dt[bias_dt], tB, pertoken=pt,
+                               offset_len=N if off_len == "N" else off_len, e5m2=in_dt == "e5m2")
+    want = cases.oracle_tc(m, inp, M, K, N, dt[out_dt])
+    got = cases.run_tc_aclnn(m, inp, M, K, N, dt[out_dt])
+    assert np.array_equal(got, want), f"{int((got != want).sum())} of {got.size} outputs differ"
