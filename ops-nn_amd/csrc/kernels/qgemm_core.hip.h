@@ -17,6 +17,11 @@
 //     output row: epilogue vectors load as float4 and the 16-bit results leave as 8-byte stores.
 #pragma once
 #include <type_traits>
+// -DQG_DBG=1 adds per-wave timestamps (start, loop start/end, end) and the clocks spent waiting for copies and at the
+// barrier, written to QgemmParams::dbg (16 x 8 bytes per wave); for timing harnesses, never set in the library build.
+#ifndef QG_DBG
+#define QG_DBG 0
+#endif
 
 #include "common.hip.h"
 
@@ -45,6 +50,9 @@ struct QgemmParams {
     const uint8_t* sa;
     const uint8_t* sb;
     int64_t sa_rs, sb_rs, sa_bs, sb_bs;
+#if QG_DBG
+    unsigned long long* dbg;
+#endif
 };
 
 __device__ __attribute__((aligned(16))) static const int8_t g_zero16[16] = {0};
@@ -79,21 +87,32 @@ __global__ __launch_bounds__(WGM* WGN * 64, MINWG) void qgemm_kernel(QgemmParams
     constexpr int KS = BK / KSTEP;                       // MFMA K steps per tile
     constexpr int SCB = MX ? BK / (MODE == MODE_MXFP8 ? 32 : 16) : 0;  // scale bytes per row per tile
     constexpr int A_BYTES = BM * BK, B_BYTES = BN * BK;
-    constexpr int SC_BYTES = MX ? (BM + BN) * 4 : 0;
+    constexpr int SCW = MX ? SCB / 4 : 1;                // scale dwords per row per tile
+    // Eight scale bytes per row per tile (fp4, BK = 128): one 16-byte copy per row brings the scales of TWO K tiles
+    // (a 4-byte copy per row costs a whole cache-line request for 4 useful bytes, as many requests as the operands
+    // themselves); they live in a ring of two slots behind the operand stages.
+    constexpr bool SC16 = MX && SCB == 8;
+    constexpr int SC_BYTES = (MX && !SC16) ? (BM + BN) * SCB : 0;
     constexpr int STAGE = A_BYTES + B_BYTES + SC_BYTES;
+    constexpr int SC_RING = STAGES * STAGE;              // SC16: two slots of (BM + BN) * 16 bytes from here
     constexpr int RPI = NT / CPR;                // tile rows covered by one copy instruction of the workgroup
     constexpr int NA = BM / RPI, NB = BN / RPI;  // copy instructions per thread per tile
-    constexpr int NSC = MX ? (BM + BN) / NT : 0; // scale-copy instructions per thread per tile
-    constexpr int CPT = NA + NB + NSC;
+    constexpr int NSC = MX ? (SC16 ? (BM + BN) / NT : (BM + BN) * SCW / NT) : 0; // scale-copy instructions per thread (SC16: per tile pair)
+    constexpr int CPT = NA + NB + (SC16 ? 0 : NSC);     // copies per tile that the wait counts step by
     static_assert(CPR == 8 || CPR == 4, "BK must be 64 or 128");
     static_assert(BM % RPI == 0 && BN % RPI == 0, "tile rows must be a multiple of the rows one copy pass covers");
     static_assert(STAGES >= 2 && STAGES * CPT < 64, "stage count");
     static_assert(KS % 2 == 0, "operand double buffer parity");
-    static_assert(!MX || SCB == 4, "MX tiles carry exactly four scale bytes per row");
-    static_assert(!MX || (BM + BN) % NT == 0, "scale copy mapping");
+    static_assert(!MX || SCB == 4 || SCB == 8, "MX tiles carry four or eight scale bytes per row");
+    static_assert(!MX || (SC16 ? (BM + BN) % NT == 0 : ((BM + BN) * SCW) % NT == 0), "scale copy mapping");
+    static_assert(!SC16 || STAGES == 2, "paired scale copies are waited for with the two-stage counts");
     static_assert(!MX || !KTAIL, "MX fast path takes whole K tiles only");
     extern __shared__ __attribute__((aligned(16))) char smem[];
 
+#if QG_DBG
+    const unsigned long long dbg_t0 = wall_clock64();
+    unsigned long long dbg_vm = 0, dbg_bar = 0, dbg_n = 0;
+#endif
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -135,25 +154,27 @@ __global__ __launch_bounds__(WGM* WGN * 64, MINWG) void qgemm_kernel(QgemmParams
         b_off[i] = (uint32_t)(r * ldb + cchunk * 16);
     }
     const int8_t* const zero_page = g_zero16;
-    // MX scales: scale-copy instruction i covers rows i*NT .. i*NT+NT-1 of the stacked [x1 rows; x2 rows] of the
-    // tile; each lane copies the four scale bytes one row needs for a K tile.
+    // MX scales: the stacked [x1 rows; x2 rows] of the tile need SCW dwords of scale bytes each per K tile; copy
+    // number c = i*NT + tid moves dword c % SCW of stacked row c / SCW, so a row's scale bytes are contiguous in LDS.
     const uint8_t* sc_src[NSC > 0 ? NSC : 1];
     if constexpr (MX) {
 #pragma unroll
         for (int i = 0; i < NSC; i++) {
-            int r = i * NT + tid;
+            const int c = i * NT + tid;
+            const int r = SC16 ? c : c / SCW, part = SC16 ? 0 : c % SCW;
             if (r < BM) {
                 int rr = r < a_rows ? r : a_rows - 1;
-                sc_src[i] = p.sa + bz * p.sa_bs + (m0 + rr) * p.sa_rs;
+                sc_src[i] = p.sa + bz * p.sa_bs + (m0 + rr) * p.sa_rs + part * 4;
             } else {
                 int rr = r - BM;
                 rr = rr < b_rows ? rr : b_rows - 1;
-                sc_src[i] = p.sb + bz * p.sb_bs + (n0 + rr) * p.sb_rs;
+                sc_src[i] = p.sb + bz * p.sb_bs + (n0 + rr) * p.sb_rs + part * 4;
             }
         }
     }
 
-    auto issue_tile = [&](int kt) {
+    auto issue_tile = [&](int kt, auto with_scales) {   // with_scales: SC16 only, true for even tiles
+        (void)with_scales;
         char* sA = smem + (kt % STAGES) * STAGE + wave * 1024;
         char* sB = sA + A_BYTES;
         const int64_t k0 = (int64_t)kt * BK;
@@ -172,7 +193,13 @@ __global__ __launch_bounds__(WGM* WGN * 64, MINWG) void qgemm_kernel(QgemmParams
             if constexpr (KTAIL) g = kok ? g : zero_page;
             async_copy16(g, sB + i * NT * 16);
         }
-        if constexpr (MX) {
+        if constexpr (SC16) {
+            if constexpr (decltype(with_scales)::value) {   // scales of tiles kt and kt+1; the slot's last reader was tile kt-1
+                char* sS = smem + SC_RING + ((kt >> 1) & 1) * ((BM + BN) * 16) + wave * 1024;
+#pragma unroll
+                for (int i = 0; i < NSC; i++) async_copy16(sc_src[i] + (int64_t)(kt >> 1) * 16, sS + i * NT * 16);
+            }
+        } else if constexpr (MX) {
             char* sS = smem + (kt % STAGES) * STAGE + A_BYTES + B_BYTES + wave * 256;
 #pragma unroll
             for (int i = 0; i < NSC; i++) async_copy4(sc_src[i] + (int64_t)kt * SCB, sS + i * NT * 4);
@@ -204,7 +231,7 @@ __global__ __launch_bounds__(WGM* WGN * 64, MINWG) void qgemm_kernel(QgemmParams
 
     typedef int frag_t __attribute__((ext_vector_type(FREG)));
     frag_t fa[2][FM], fb[2][FN];
-    uint32_t sca[FM], scb[FN];  // MX: this lane's four scale bytes of the current tile, shifted down by its K half
+    uint32_t sca[FM][SCW], scb[FN][SCW];  // MX: this lane's scale bytes of the current tile, shifted down by its K half
     (void)swz; (void)swz0; (void)swz1; (void)sca; (void)scb;
 
     auto load_frags = [&](int kt, int s, int buf) {
@@ -230,15 +257,38 @@ __global__ __launch_bounds__(WGM* WGN * 64, MINWG) void qgemm_kernel(QgemmParams
             }
         }
     };
-    // MX: the four scale bytes of a row cover the tile's K blocks 0..3 (32 elements each).  MFMA step s of a lane
-    // in K half h multiplies block 2s + h, i.e. byte 2s of the dword once it is shifted right by 8h.
-    auto load_scales = [&](int kt) {
+    // MX: byte b of a row's scale bytes of a tile covers the tile's K block b (32 elements).  MFMA step s of a lane
+    // in K half h multiplies block 2s + h, i.e. byte 2(s % 2) of scale dword s / 2 once that dword is shifted right
+    // by 8h.  read_scales_raw fetches dword w of tile kt's scales for this lane's rows; shift_scales moves them into
+    // place.
+    auto read_scales_raw = [&](int kt, int w, uint32_t (&ra)[FM], uint32_t (&rb)[FN]) {
         if constexpr (MX) {
-            const char* sS = smem + (kt % STAGES) * STAGE + A_BYTES + B_BYTES;
+            const char* sS;
+            int pitch, off;
+            if constexpr (SC16) {
+                sS = smem + SC_RING + ((kt >> 1) & 1) * ((BM + BN) * 16);
+                pitch = 16; off = (kt & 1) * 8 + 4 * w;
+            } else {
+                sS = smem + (kt % STAGES) * STAGE + A_BYTES + B_BYTES;
+                pitch = SCB; off = 4 * w;
+            }
 #pragma unroll
-            for (int j = 0; j < FM; j++) sca[j] = *(const uint32_t*)(sS + (wm * TM + j * 32 + frow) * 4) >> (8 * fkc);
+            for (int j = 0; j < FM; j++) ra[j] = *(const uint32_t*)(sS + (wm * TM + j * 32 + frow) * pitch + off);
 #pragma unroll
-            for (int i = 0; i < FN; i++) scb[i] = *(const uint32_t*)(sS + (BM + wn * TN + i * 32 + frow) * 4) >> (8 * fkc);
+            for (int i = 0; i < FN; i++) rb[i] = *(const uint32_t*)(sS + (BM + wn * TN + i * 32 + frow) * pitch + off);
+        }
+    };
+    auto shift_scales = [&](int w, const uint32_t (&ra)[FM], const uint32_t (&rb)[FN]) {
+#pragma unroll
+        for (int j = 0; j < FM; j++) sca[j][w] = ra[j] >> (8 * fkc);
+#pragma unroll
+        for (int i = 0; i < FN; i++) scb[i][w] = rb[i] >> (8 * fkc);
+    };
+    auto load_scales = [&](int kt) {   // dword 0 of tile kt, ready to use
+        if constexpr (MX) {
+            uint32_t ra[FM], rb[FN];
+            read_scales_raw(kt, 0, ra, rb);
+            shift_scales(0, ra, rb);
         }
     };
     auto mma = [&](int buf, auto sidx) {
@@ -254,19 +304,21 @@ __global__ __launch_bounds__(WGM* WGN * 64, MINWG) void qgemm_kernel(QgemmParams
                     const v4i z = {0, 0, 0, 0};  // fp4 operands occupy the first four of the eight operand dwords
                     const v8i bb = __builtin_shufflevector(fb[buf][i], z, 0, 1, 2, 3, 4, 5, 6, 7);
                     const v8i aa = __builtin_shufflevector(fa[buf][j], z, 0, 1, 2, 3, 4, 5, 6, 7);
-                    acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(bb, aa, acc[i][j], 4, 4, 2 * S, (int)scb[i], 2 * S, (int)sca[j]);
+                    acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(bb, aa, acc[i][j], 4, 4, 2 * (S % 2), (int)scb[i][S / 2], 2 * (S % 2), (int)sca[j][S / 2]);
                 } else {
-                    acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb[buf][i], fa[buf][j], acc[i][j], 0, 0, 2 * S, (int)scb[i], 2 * S, (int)sca[j]);
+                    acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb[buf][i], fa[buf][j], acc[i][j], 0, 0, 2 * S, (int)scb[i][0], 2 * S, (int)sca[j][0]);
                 }
             }
     };
     auto interleave = [&](bool with_copies) {
-        // (FM+FN) groups of {MFMAs, one LDS read (+ one async copy)}: memory instructions issue in the MFMA shadow
+        // (FM+FN) groups of {MFMAs, one LDS read (+ async copies)}: memory instructions issue in the MFMA shadow
+        constexpr int NCOPY = NA + NB + NSC;
+        constexpr int CPG = (NCOPY + FM + FN - 1) / (FM + FN);
 #pragma unroll
         for (int g = 0; g < FM + FN; g++) {
             __builtin_amdgcn_sched_group_barrier(0x008, (FM * FN) / (FM + FN), 0);
             __builtin_amdgcn_sched_group_barrier(0x100, KSTEP / 32, 0);
-            if (with_copies && g < CPT) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+            if (with_copies) __builtin_amdgcn_sched_group_barrier(0x020, CPG, 0);
         }
     };
 
@@ -278,24 +330,42 @@ __global__ __launch_bounds__(WGM* WGN * 64, MINWG) void qgemm_kernel(QgemmParams
     //   start the copy of tile kt+STAGES into the freed stage, read K step 0 of tile kt+1, multiply the last step.
 #pragma unroll
     for (int i = 0; i < STAGES; i++)
-        if (i < KT) issue_tile(i);
+        if (i < KT) {
+            if (i % 2 == 0) issue_tile(i, std::true_type{});
+            else issue_tile(i, std::false_type{});
+        }
     if (KT >= STAGES) wait_vmcnt<(STAGES - 1) * CPT>();
     else wait_vmcnt<0>();
     __builtin_amdgcn_s_barrier();
+#if QG_DBG
+    const unsigned long long dbg_t1 = wall_clock64();
+    const unsigned long long dbg_c1 = clock64();
+#endif
     load_frags(0, 0, 0);
     load_scales(0);
 
-    auto k_tile = [&](int kt, auto issue, auto next) {
+    auto k_tile = [&](int kt, auto issue, auto next, auto even) {
         constexpr bool ISSUE = decltype(issue)::value, NEXT = decltype(next)::value;
-        uint32_t sca_n[FM], scb_n[FN];
-        (void)sca_n; (void)scb_n;
+        uint32_t ra[FM], rb[FN];   // raw scale dwords on their way in
+        (void)ra; (void)rb;
         if constexpr (KS >= 4) {
+            // SC16: scale dword 1 of this tile (K steps 2, 3) is fetched now, dword 0 of the next tile after the
+            // barrier below, each into the registers its predecessor has just stopped using
+            if constexpr (SC16) {
+                read_scales_raw(kt, 1, ra, rb);
+                __builtin_amdgcn_sched_barrier(0);
+            }
             load_frags(kt, 1, 1);
             mma(0, std::integral_constant<int, 0>{});
             interleave(false);
             load_frags(kt, 2, 0);
             mma(1, std::integral_constant<int, 1>{});
             interleave(false);
+            if constexpr (SC16) {
+                __builtin_amdgcn_sched_barrier(0);
+                shift_scales(1, ra, rb);
+                __builtin_amdgcn_sched_barrier(0);
+            }
             load_frags(kt, 3, 1);
             mma(0, std::integral_constant<int, 2>{});
             interleave(false);
@@ -304,39 +374,56 @@ __global__ __launch_bounds__(WGM* WGN * 64, MINWG) void qgemm_kernel(QgemmParams
             mma(0, std::integral_constant<int, 0>{});
             interleave(false);
         }
+#if QG_DBG
+        wait_lgkmcnt0();
+        const unsigned long long c0 = clock64();
+#endif
         if constexpr (NEXT) {
             if constexpr (ISSUE) wait_vmcnt<(STAGES - 2) * CPT>();
             else wait_vmcnt<0>();
         }
         wait_lgkmcnt0();  // this wave's reads of the stage about to be recycled have retired
+#if QG_DBG
+        const unsigned long long c1 = clock64();
+#endif
         __builtin_amdgcn_s_barrier();
-        if constexpr (ISSUE) issue_tile(kt + STAGES);
-        if constexpr (NEXT) {
-            load_frags(kt + 1, 0, 0);
-            if constexpr (MX) {  // next tile's scales go to a second set: the last MFMA step still uses this tile's
-                const char* sS = smem + ((kt + 1) % STAGES) * STAGE + A_BYTES + B_BYTES;
-#pragma unroll
-                for (int j = 0; j < FM; j++) sca_n[j] = *(const uint32_t*)(sS + (wm * TM + j * 32 + frow) * 4) >> (8 * fkc);
-#pragma unroll
-                for (int i = 0; i < FN; i++) scb_n[i] = *(const uint32_t*)(sS + (BM + wn * TN + i * 32 + frow) * 4) >> (8 * fkc);
-            }
+#if QG_DBG
+        const unsigned long long c2 = clock64();
+        dbg_vm += c1 - c0; dbg_bar += c2 - c1; dbg_n++;
+#endif
+        if constexpr (NEXT && MX) {
+            // the next tile's first scale dword is requested ahead of its operands (LDS returns in order) and moved
+            // into place only after this tile's last MFMAs, which still use the current ones, have been issued
+            read_scales_raw(kt + 1, 0, ra, rb);
+            __builtin_amdgcn_sched_barrier(0);
         }
+        if constexpr (ISSUE) issue_tile(kt + STAGES, even);
+        if constexpr (NEXT) load_frags(kt + 1, 0, 0);
         mma(1, std::integral_constant<int, KS - 1>{});
         if constexpr (NEXT) interleave(ISSUE);
         if constexpr (NEXT && MX) {
-#pragma unroll
-            for (int j = 0; j < FM; j++) sca[j] = sca_n[j];
-#pragma unroll
-            for (int i = 0; i < FN; i++) scb[i] = scb_n[i];
+            __builtin_amdgcn_sched_barrier(0);
+            shift_scales(0, ra, rb);
         }
     };
     using T = std::true_type;
     using F = std::false_type;
     int kt = 0;
-    for (; kt + STAGES < KT; kt++) k_tile(kt, T{}, T{});
-    for (; kt + 1 < KT; kt++) k_tile(kt, F{}, T{});
-    k_tile(kt, F{}, F{});
+    if constexpr (SC16) {   // KT is even: tiles go in pairs, the even one also starts the pair's scale copy
+        for (; kt + STAGES < KT; kt += 2) {
+            k_tile(kt, T{}, T{}, T{});
+            k_tile(kt + 1, T{}, T{}, F{});
+        }
+    } else {
+        for (; kt + STAGES < KT; kt++) k_tile(kt, T{}, T{}, F{});
+    }
+    for (; kt + 1 < KT; kt++) k_tile(kt, F{}, T{}, F{});
+    k_tile(kt, F{}, F{}, F{});
     __syncthreads();  // all operand reads done before LDS is reused below
+#if QG_DBG
+    const unsigned long long dbg_t2 = wall_clock64();
+    const unsigned long long dbg_c2 = clock64();
+#endif
 
     // Epilogue.  acc[i][j][r]: n = n_base + 8*(r/4) + 4*(lane/32) + r%4,  m = m_base + lane%32.
     // Per-row and per-column terms are first widened to fp32 in LDS, so the unrolled part is branch-free:
@@ -431,6 +518,17 @@ __global__ __launch_bounds__(WGM* WGN * 64, MINWG) void qgemm_kernel(QgemmParams
             }
         }
     }
+#if QG_DBG
+    {
+        const unsigned long long dbg_t3 = wall_clock64();
+        wait_vmcnt<0>();
+        const unsigned long long dbg_t4 = wall_clock64();
+        if (lane == 0 && p.dbg) {
+            unsigned long long* d = p.dbg + ((size_t)blockIdx.x * (WGM * WGN) + wave) * 16;
+            d[0] = dbg_t0; d[1] = dbg_t1; d[2] = dbg_t2; d[3] = dbg_t3; d[4] = dbg_t4; d[5] = dbg_vm; d[6] = dbg_bar; d[7] = dbg_n; d[8] = dbg_c2 - dbg_c1;
+        }
+    }
+#endif
 }
 
 template <int MODE, int BM, int BN, int BK, int WGM, int WGN, int STAGES, int MINWG, bool KTAIL, int OUT_DT>
@@ -439,7 +537,9 @@ static int qgemm_launch_one(const QgemmParams& p, int64_t batch, hipStream_t st)
     constexpr bool MX = MODE != MODE_I8;
     int tiles_m = (int)((p.M + BM - 1) / BM), tiles_n = (int)((p.N + BN - 1) / BN);
     dim3 grid((unsigned)(tiles_m * tiles_n), (unsigned)batch);
-    size_t lds = (size_t)STAGES * ((BM + BN) * BK + (MX ? (BM + BN) * 4 : 0));
+    constexpr int SCB = MX ? BK / (MODE == MODE_MXFP8 ? 32 : 16) : 0;   // scale bytes per row per tile
+    size_t lds = SCB == 8 ? (size_t)STAGES * (BM + BN) * BK + 2 * (BM + BN) * 16   // scales in their own ring of two slots
+                          : (size_t)STAGES * ((BM + BN) * BK + (BM + BN) * SCB);
     auto k = qgemm_kernel<MODE, BM, BN, BK, WGM, WGN, STAGES, MINWG, KTAIL, OUT_DT>;
     static bool attr_set = false;  // per instantiation; benign if two threads both set it
     if (!attr_set) {

@@ -9,7 +9,7 @@
 // MX block size (32) and the hardware operand block coincide and no dequantised copy is ever formed.
 //
 // Fast path (qgemm_core.hip.h, MODE_MXFP4 / MODE_MXFP8): operands and scales K-contiguous, K % 128 == 0,
-// 16-bit output.  An N-contiguous x2 (data [K, N], scales [K/64, N, 2]) is first re-laid out into the
+// 16-bit output (fp4 with K % 512 == 0 takes 256-element K tiles, otherwise 128-element ones).  An N-contiguous x2 (data [K, N], scales [K/64, N, 2]) is first re-laid out into the
 // workspace; everything else runs the plain kernel.
 #include "launch.h"
 #include "qgemm_core.hip.h"
@@ -112,6 +112,11 @@ int launch_mx_mfma(const OpsnnQmmArgs& a0, hipStream_t st)
     const bool small = a.M <= 128 || a.N <= 128;
     if (fp4) {
         if (small || a.force_variant == OPSNN_VARIANT_MX_128) return qgemm_launch<MODE_MXFP4, 128, 128, 64, 2, 2, 4, 1>(g, a.batch, a.out_dtype, st);
+        // K tiles of 128 bytes (256 elements) with the scales of two tiles per 16-byte copy: needs an even number of
+        // such tiles and 16-byte aligned scale rows
+        const bool sc16 = a.K % 512 == 0 &&
+                          (((uintptr_t)g.sa | (uintptr_t)g.sb | (uint64_t)g.sa_rs | (uint64_t)g.sb_rs | (uint64_t)g.sa_bs | (uint64_t)g.sb_bs) % 16) == 0;
+        if (sc16) return qgemm_launch<MODE_MXFP4, 256, 256, 128, 2, 4, 2, 1>(g, a.batch, a.out_dtype, st);
         return qgemm_launch<MODE_MXFP4, 256, 256, 64, 2, 2, 4, 1>(g, a.batch, a.out_dtype, st);
     }
     if (small || a.force_variant == OPSNN_VARIANT_MX_128) return qgemm_launch<MODE_MXFP8, 128, 128, 128, 2, 2, 2, 1>(g, a.batch, a.out_dtype, st);

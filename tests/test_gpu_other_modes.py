@@ -87,6 +87,8 @@ def test_fp8_blockscale_group_size_inferred(gpu):
     (64, 320, 96, False, False), (33, 192, 50, True, True),
     (512, 1024, 768, True, True), (300, 512, 260, True, True), (300, 512, 260, False, True), (256, 2048, 512, True, False),
     (260, 384, 300, False, False),
+    # fp4 with K % 512 == 0 takes 256-element K tiles (scales of two tiles per copy): odd and even pair counts, ragged edges
+    (260, 1536, 300, True, True), (512, 2048, 264, False, True), (384, 768, 256, True, True),
 ])
 def test_mx(gpu, M, K, N, tB, fp4, use_plain):
     m = gpu
@@ -99,11 +101,12 @@ def test_mx(gpu, M, K, N, tB, fp4, use_plain):
     check_close(got, want, orc.BF16, "mx", exact=use_plain)
 
 
-def test_mx_batched(gpu):
+@pytest.mark.parametrize("M,K,N,batch", [(96, 256, 128, 3), (256, 1024, 264, 2)])
+def test_mx_batched(gpu, M, K, N, batch):
     m = gpu
-    inp = cases.make_mx_inputs(m, 96, 256, 128, 4, True, True, batch=3)
-    want = cases.oracle_mx(m, inp, 96, 256, 128, True, m.ACL_BF16)
-    got = cases.run_mx_aclnn(m, inp, 96, 256, 128, True, m.ACL_BF16)
+    inp = cases.make_mx_inputs(m, M, K, N, 4, True, True, batch=batch)
+    want = cases.oracle_mx(m, inp, M, K, N, True, m.ACL_BF16)
+    got = cases.run_mx_aclnn(m, inp, M, K, N, True, m.ACL_BF16)
     check_close(got, want, orc.BF16, "mx batched")
 
 
