@@ -306,6 +306,10 @@ static bool stream_eligible(WqParams& p, WqStreamOpts& o)
     o.resx = !no_resx && p.M <= 16 && nch % 4 == 0 && (p.M + 1) * (p.K * 2 + 16) <= 65536;
     o.resx_vscale = o.resx && p.group == KC && p.s_rs == 1 && p.s_cs % 8 == 0 && (nch / 4) % 8 == 0 &&
                     (uintptr_t)p.scale % 16 == 0 && (!p.offset || (uintptr_t)p.offset % 16 == 0);
+    // more than 64 rows: two weight blocks per wave share every x fragment, up to 128 rows per pass over the weights
+    // (needs whole groups of chunks in flight and whole wave tiles of columns)
+    static const bool no_rows = [] { const char* e = getenv("OPSNN_WQ_NO_ROWS"); return e && e[0] == '1'; }();
+    o.rows = !no_rows && p.M > 64 && nch % 8 == 0 && p.N % 32 == 0 && p.N >= 256;
     return true;
 }
 
@@ -314,9 +318,15 @@ static int launch_slabs(WqParams p, hipStream_t st)
 {
     WqStreamOpts o{};
     const bool stream = stream_eligible<WBITS>(p, o);
-    for (int64_t m0 = 0; m0 < p.M; m0 += 64) {
+    // rows per launch: as many as one pass over the weights can serve, in equal slabs
+    int64_t slab = 64;
+    if (stream && o.rows) {
+        const int64_t passes = (p.M + 127) / 128;
+        slab = ((p.M + passes - 1) / passes + 15) / 16 * 16;
+    }
+    for (int64_t m0 = 0; m0 < p.M; m0 += slab) {
         p.m_base = m0;
-        p.m_rows = (p.M - m0) < 64 ? (p.M - m0) : 64;
+        p.m_rows = (p.M - m0) < slab ? (p.M - m0) : slab;
         int rc;
         if (stream) rc = launch_wq_stream<XDT, WBITS>(p, o, st);
         else if (p.m_rows <= 16) rc = launch_wk<XDT, WBITS, 1>(p, st);

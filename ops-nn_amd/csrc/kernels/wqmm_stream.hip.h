@@ -33,7 +33,9 @@ __device__ __forceinline__ DqConst make_dq_const()
     return c;
 }
 
-template <int XDT, int WBITS, bool HAS_OFF>
+// NATURAL: the 8 values leave in k order (one more byte permute per register for int4 x fp16) for kernels whose x
+// reaches LDS unpermuted.
+template <int XDT, int WBITS, bool HAS_OFF, bool NATURAL = false>
 __device__ __forceinline__ v4i dequant8(const v4i& piece, int s, uint16_t sb, uint16_t ob, const DqConst& dc)
 {
     if constexpr (XDT == DT_F16) {
@@ -68,6 +70,10 @@ __device__ __forceinline__ v4i dequant8(const v4i& piece, int s, uint16_t sb, ui
         }
         if constexpr (HAS_OFF) { t0 = t0 + off; t1 = t1 + off; t2 = t2 + off; t3 = t3 + off; }   // first rounding
         t0 = t0 * sc; t1 = t1 * sc; t2 = t2 * sc; t3 = t3 * sc;                                  // second rounding
+        if constexpr (NATURAL && WBITS == 4) {   // pairs (0,4) (1,5) (2,6) (3,7) -> (0,1) (2,3) (4,5) (6,7)
+            return (v4i){(int)__builtin_amdgcn_perm(u32(t1), u32(t0), 0x05040100u), (int)__builtin_amdgcn_perm(u32(t3), u32(t2), 0x05040100u),
+                         (int)__builtin_amdgcn_perm(u32(t1), u32(t0), 0x07060302u), (int)__builtin_amdgcn_perm(u32(t3), u32(t2), 0x07060302u)};
+        }
         return (v4i){(int)u32(t0), (int)u32(t1), (int)u32(t2), (int)u32(t3)};
     } else {
         // bf16: no packed bf16 arithmetic on this chip, so the two steps run in fp32 with a hardware
@@ -78,7 +84,7 @@ __device__ __forceinline__ v4i dequant8(const v4i& piece, int s, uint16_t sb, ui
             const uint32_t q = (uint32_t)piece[s];
             const int ord[8] = {0, 4, 1, 5, 2, 6, 3, 7};
 #pragma unroll
-            for (int j = 0; j < 8; j++) w[j] = (float)(((int)(q << (28 - 4 * ord[j]))) >> 28);
+            for (int j = 0; j < 8; j++) w[j] = (float)(((int)(q << (28 - 4 * (NATURAL ? j : ord[j])))) >> 28);
         } else {
 #pragma unroll
             for (int j = 0; j < 8; j++) w[j] = (float)(((int)((uint32_t)piece[2 * s + (j >> 2)] << (24 - 8 * (j & 3)))) >> 24);
@@ -338,6 +344,184 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(NW == 8
     }
 }
 
+// ---- many rows of x (65 .. 128 per launch): a wave owns NB blocks of 16 weight rows ----
+// With several 16-row blocks of x per weight block the loop stops being a stream: every MFMA needs an x fragment
+// from LDS, and with one weight block per wave that is one 1 KB LDS read per MFMA (16 clocks), four times what the
+// LDS delivers.  Here every x fragment read serves NB MFMAs (NB weight blocks of the same wave):
+//   per 32-k step and wave: NB dequantisations, MB LDS reads, MB * NB MFMAs (16x16x32).
+// Workgroup: 8 waves = WN column groups (16 * NB columns each) x WK waves that take every WK-th chunk of K; their
+// partial sums meet in LDS in a fixed order at the end.  A slab of x is the WK chunks the waves work on at the same
+// time, double-buffered, one barrier per slab.  x travels global -> LDS with 16-byte asynchronous copies (no
+// registers, no vector ALU work), so it sits in LDS in k order and the dequantisation delivers k order too
+// (dequant8<..., NATURAL>); rows are 16-byte-piece swizzled (piece ^ row % 16) instead of padded, because a copy
+// instruction fills 1 KB of consecutive LDS.  Rows of the slab that x does not have repeat its last row: they only
+// feed output rows that are never stored.
+// A wave's loads complete in issue order, so waiting for its x copies of the next slab also waits for every weight
+// load issued before them; with the weights PF = 2..4 chunks ahead and the x copies issued one slab ahead, first
+// thing after the barrier, that costs the weight stream at most the lookahead beyond one slab.
+// Scale and offset of a chunk travel with its weights (one 16-bit load each per row block).
+// The launcher guarantees: N % (16 * NB) == 0, (K / KC) % (WK * PF) == 0, group a power-of-two multiple of KC or
+// per channel, x rows 16-byte aligned.
+template <int XDT, int WBITS, int MB, int NB, int WN, int WK, bool HAS_OFF>
+__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void wqmm_rows_kernel(WqParams p)
+{
+    static_assert(WN * WK == 8, "eight waves");
+    constexpr int NT = 512;
+    constexpr int KPL = 128 / WBITS, KC = 4 * KPL, STEPS = KC / 32;
+    constexpr int PF = 8 / NB;           // of this wave's chunks in flight per row block (a chunk is 500 to 1000 clocks of MFMA work here)
+    constexpr int KX = WK * KC;          // k per slab
+    constexpr int XROW = KX * 2;         // LDS row pitch (bytes)
+    constexpr int XPR = KX / 8;          // 16-byte pieces per x row per slab
+    constexpr int XBUF = 16 * MB * XROW; // one slab buffer
+    constexpr int XITEMS = 16 * MB * XPR / NT;
+    constexpr int NBL = NB * (HAS_OFF ? 3 : 2);   // loads of one weight fetch
+    static_assert((16 * MB * XPR) % NT == 0 && XPR >= 16 && PF >= 2, "staging and prefetch shape");
+    extern __shared__ __attribute__((aligned(16))) char sx[];
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wn = wave / WK, wk = wave % WK;
+    const int nrow = lane & 15, g = lane >> 4;
+    int64_t n0 = ((int64_t)blockIdx.x * WN + wn) * (16 * NB);
+    const bool n_ok = n0 < p.N;
+    if (!n_ok) n0 = p.N - 16 * NB;       // a wave past the edge recomputes the last columns and stores nothing
+    const int Ki = (int)p.K;
+    const int NSLAB = Ki / KX;           // = chunks per wave
+    const int rows = (int)p.m_rows;
+
+    const uint8_t* wptr = p.w + (n0 + nrow) * p.ldw + g * 16 + wk * 64;
+    const int64_t wblk = 16 * p.ldw;     // bytes between the row blocks of a wave
+    const uint16_t* srow = p.scale + (n0 + nrow) * p.s_cs;
+    const uint16_t* orow = HAS_OFF ? p.offset + (n0 + nrow) * p.s_cs : nullptr;
+    const int64_t sblk = 16 * p.s_cs;
+
+    // x copies: instruction `it` of this thread fills LDS piece it*NT + tid of the buffer, i.e. position
+    // (it*NT + tid) % XPR of row (it*NT + tid) / XPR, with the row's piece position ^ (row % 16)
+    const uint16_t* xsrc[XITEMS];
+#pragma unroll
+    for (int it = 0; it < XITEMS; it++) {
+        const int L = it * NT + tid;
+        const int r = L / XPR, pos = L % XPR;
+        const int rr = r < rows ? r : rows - 1;
+        xsrc[it] = p.x + (p.m_base + rr) * p.K + (pos ^ (r & 15)) * 8;
+    }
+    auto issue_x = [&](int slab) {
+        char* dst = sx + (slab & 1) * XBUF + wave * 1024;
+#pragma unroll
+        for (int it = 0; it < XITEMS; it++) async_copy16(xsrc[it] + (int64_t)slab * KX, dst + it * NT * 16);
+    };
+    // LDS byte offset of this lane's column operand inside a buffer, per 16-row block of x, at K step 0 (the lane's
+    // weights cover k = g*KPL .. +KPL of the chunk, step s the 8 at 8s); step s is s pieces further on, which the
+    // swizzle turns into an exclusive-or with 16s
+    int xoff[MB];
+#pragma unroll
+    for (int b = 0; b < MB; b++) {
+        const int r = 16 * b + nrow;
+        xoff[b] = r * XROW + ((wk * (KC / 8) + g * (KPL / 8)) ^ (r & 15)) * 16;
+    }
+
+    v4f acc[NB][MB];
+#pragma unroll
+    for (int q = 0; q < NB; q++)
+#pragma unroll
+        for (int b = 0; b < MB; b++) acc[q][b] = (v4f){0.0f, 0.0f, 0.0f, 0.0f};
+    const DqConst dqc = make_dq_const();
+
+    v4i wq[PF][NB];
+    uint16_t sq[PF][NB], oq[PF][NB];
+    auto fetch = [&](int j, int cw) {   // chunk cw of this wave (chunk cw * WK + wk of the row) into slot j
+        const int64_t so = (int64_t)((cw * WK + wk) >> p.cpg_shift) * p.s_rs;
+#pragma unroll
+        for (int q = 0; q < NB; q++) {
+            wq[j][q] = *(const v4i*)(wptr + q * wblk + (int64_t)cw * (WK * 64));
+            sq[j][q] = srow[q * sblk + so];
+            if constexpr (HAS_OFF) oq[j][q] = orow[q * sblk + so];
+            else oq[j][q] = 0;
+        }
+    };
+#pragma unroll
+    for (int j = 0; j < PF; j++) fetch(j, j);
+    issue_x(0);
+    wait_vmcnt<0>();
+
+    for (int c0 = 0; c0 < NSLAB; c0 += PF) {
+#pragma unroll
+        for (int j = 0; j < PF; j++) {
+            const int cw = c0 + j;
+            // this thread's copies of slab cw have landed (only the weight fetch issued after them may be in flight)
+            if (cw > 0) wait_vmcnt<NBL>();
+            __syncthreads();   // slab cw is complete and visible; every wave has finished slab cw-1
+            if (cw + 1 < NSLAB) issue_x(cw + 1);
+            const char* xs = sx + (cw & 1) * XBUF;
+#pragma unroll
+            for (int s = 0; s < STEPS; s++) {
+                v4i aop[NB];
+#pragma unroll
+                for (int q = 0; q < NB; q++) aop[q] = dequant8<XDT, WBITS, HAS_OFF, true>(wq[j][q], s, sq[j][q], oq[j][q], dqc);
+#pragma unroll
+                for (int b = 0; b < MB; b++) {
+                    const v4i bop = *(const v4i*)(xs + (xoff[b] ^ (16 * s)));
+#pragma unroll
+                    for (int q = 0; q < NB; q++) {
+                        if constexpr (XDT == DT_F16) {
+                            acc[q][b] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(v8h, aop[q]), __builtin_bit_cast(v8h, bop), acc[q][b], 0, 0, 0);
+                        } else {
+                            acc[q][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf, aop[q]), __builtin_bit_cast(v8bf, bop), acc[q][b], 0, 0, 0);
+                        }
+                    }
+                }
+            }
+            const int nx = cw + PF;
+            fetch(j, nx < NSLAB ? nx : NSLAB - 1);   // past the end: a harmless reload of the last chunk
+        }
+    }
+
+    if constexpr (WK > 1) {
+        __syncthreads();   // x is no longer needed: its buffers take the partial sums
+        float* red = (float*)sx;
+        if (wk > 0) {
+#pragma unroll
+            for (int q = 0; q < NB; q++)
+#pragma unroll
+                for (int b = 0; b < MB; b++)
+#pragma unroll
+                    for (int i = 0; i < 4; i++) red[((((wn * (WK - 1) + (wk - 1)) * NB + q) * MB + b) * 4 + i) * 64 + lane] = acc[q][b][i];
+        }
+        __syncthreads();
+        if (wk > 0) return;
+#pragma unroll
+        for (int j = 0; j < WK - 1; j++)
+#pragma unroll
+            for (int q = 0; q < NB; q++)
+#pragma unroll
+                for (int b = 0; b < MB; b++)
+#pragma unroll
+                    for (int i = 0; i < 4; i++) acc[q][b][i] = acc[q][b][i] + red[((((wn * (WK - 1) + j) * NB + q) * MB + b) * 4 + i) * 64 + lane];
+    }
+
+    // D'[row = weight row n][col = x row m]: lane holds col m = lane%16, rows n = 4*(lane/16) + i
+    if (!n_ok) return;
+#pragma unroll
+    for (int q = 0; q < NB; q++) {
+#pragma unroll
+        for (int b = 0; b < MB; b++) {
+            const int r = 16 * b + nrow;
+            if (r >= rows) continue;
+            const int64_t m = p.m_base + r;
+            const int64_t nn0 = n0 + 16 * q + 4 * g;
+            float v[4];
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                v[i] = acc[q][b][i];
+                if (p.bias) v[i] = v[i] + load_scalar_as_f32(p.bias, p.bias_dt, nn0 + i);
+                if constexpr (XDT == DT_BF16) v[i] = bf16_to_f32(bf16_bits(v[i]));   // the golden rounds bf16 results twice (a no-op)
+            }
+            const v4us o = {bits_x<XDT>(v[0]), bits_x<XDT>(v[1]), bits_x<XDT>(v[2]), bits_x<XDT>(v[3])};
+            *(v4us*)(p.y + m * p.N + nn0) = o;   // N % 16 == 0 here: 8-byte aligned
+        }
+    }
+}
+
 // ---- few rows of x (rows * K * 2 bytes fit in LDS): x is staged whole, once per workgroup ----
 // The four waves of a workgroup share one block of 16 weight rows at a time and take one contiguous quarter of K
 // each; partial sums meet in LDS in a fixed order.  A workgroup walks several row blocks (blockIdx.x, + gridDim.x,
@@ -577,12 +761,32 @@ static int launch_stream_one(const WqParams& p, hipStream_t st)
     return (int)hipGetLastError();
 }
 
+template <int XDT, int WBITS, int MB, int NB, int WN, int WK, bool HAS_OFF>
+static int launch_rows_one(const WqParams& p, hipStream_t st)
+{
+    constexpr int KC = 4 * (128 / WBITS);
+    constexpr size_t lds_x = 2 * (size_t)(16 * MB) * (WK * KC * 2);
+    constexpr size_t lds_red = (size_t)WN * (WK - 1) * NB * MB * 4 * 64 * 4;
+    constexpr size_t lds = lds_x > lds_red ? lds_x : lds_red;
+    const unsigned grid = (unsigned)((p.N + 16 * NB * WN - 1) / (16 * NB * WN));
+    auto k = wqmm_rows_kernel<XDT, WBITS, MB, NB, WN, WK, HAS_OFF>;
+    static bool attr_set = false;
+    if (!attr_set) {
+        hipError_t e = hipFuncSetAttribute((const void*)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return (int)e;
+        attr_set = true;
+    }
+    hipLaunchKernelGGL(k, dim3(grid), dim3(512), lds, st, p);
+    return (int)hipGetLastError();
+}
+
 struct WqStreamOpts {
     bool has_off, vscale, ksplit;
+    bool rows;                // many-rows kernel eligible (row slabs of up to 128)
     bool resx, resx_vscale;   // whole-x-in-LDS kernel eligible, and with vector scale loads
 };
 
-// One row slab (p.m_rows <= 64) of one dtype pair; defined once per pair in its own translation unit.
+// One row slab (p.m_rows <= 64, or <= 128 with o.rows) of one dtype pair; defined once per pair in its own translation unit.
 template <int XDT, int WBITS>
 int launch_wq_stream(const WqParams& p, const WqStreamOpts& o, hipStream_t st);
 
@@ -607,6 +811,8 @@ int launch_wq_stream(const WqParams& p, const WqStreamOpts& o, hipStream_t st);
             return o.has_off ? launch_resx_one<XDT, WBITS, true, false>(p, st)                                      \
                              : launch_resx_one<XDT, WBITS, false, false>(p, st);                                    \
         }                                                                                                           \
+        if (o.rows && p.m_rows > 64) return o.has_off ? launch_rows_one<XDT, WBITS, 8, 2, 4, 2, true>(p, st)              \
+                                                      : launch_rows_one<XDT, WBITS, 8, 2, 4, 2, false>(p, st);            \
         if (o.ksplit && p.m_rows <= 16) return wq_stream_off<1, 4, 4, false>(p, o.has_off, st);                     \
         if (p.m_rows <= 16) return wq_stream_mb<1>(p, o, st);                                                       \
         if (p.m_rows <= 32) return wq_stream_mb<2>(p, o, st);                                                       \
