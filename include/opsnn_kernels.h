@@ -66,6 +66,10 @@ typedef struct {
     int64_t x1_scale_len;  /* 1: one fp32 scale for all of x1 ("double scale" with fp8 inputs); 0 if x1_scale is NULL */
     const float* x2_offset;/* fp32 [1] or [N], int8 output only; NULL = take it from the packed 64-bit scale */
     int64_t x2_offset_len;
+    /* K-group family (opsnnQmmGroup) */
+    const void* y_scale;   /* UINT64 [1] or [N]: fp32 scale in the low word, upper 19 bits kept */
+    int64_t y_scale_len;
+    OpsnnMat x2_offset_mat;/* FLOAT16, logical [ceil(K/gsK), N] */
 } OpsnnQmmArgs;
 
 /* int8 x int8 -> int32, then  out = fp32(acc + int32 bias) * x2_scale[n] * x1_scale[m] + float bias.
@@ -81,6 +85,14 @@ OPSNN_API int opsnnQmmMx(const OpsnnQmmArgs* a, void* stream);
  *   sums + bias) or INT8 (requantised: clip(s9(s9(acc * scale)) + s9(offset))).
  * Reference formulas: matmul/quant_batch_matmul_v3/tests/assets/qbmmv3_kernel_golden.py:390-513. */
 OPSNN_API int opsnnQmmTc(const OpsnnQmmArgs* a, void* stream);
+/* K-group modes of quant_batch_matmul_v4 (gsK = K elements per group):
+ *   fp8 e4m3 x fp4 e2m1 ("T-CG"): x2_scale_mat BF16 / FLOAT16 logical [ceil(K/gsK), N] (dtype in x2_scale_dtype);
+ *     w = e4m3(T16(T16(x2) * scale)); out = (x1 @ w) * deq(y_scale[n]) + fp32 bias;
+ *   int4 x int4 with offsets (gsK = 256): x1_scale fp32 [M], x2_scale_mat fp32 and x2_offset_mat fp16 logical
+ *     [ceil(K/256), N]; out = x1_scale[m] * sum_g (x1_g @ x2_g - rowsum(x1_g) * offset[g,n]) * scale[g,n].
+ * Reference formulas: matmul/quant_batch_matmul_v4/tests/assets/qbmmv4_kernel_golden.py:189-255, 328-395.
+ * (The MX fp8 x fp4 mode of that file runs through opsnnQmmMx and its int8 per-tile mode through opsnnQmmBlockScale.) */
+OPSNN_API int opsnnQmmGroup(const OpsnnQmmArgs* a, void* stream);
 /* Device workspace bytes a launcher needs for these arguments (0 if none). */
 OPSNN_API uint64_t opsnnQmmWorkspace(const OpsnnQmmArgs* a, int mode);
 

@@ -611,8 +611,22 @@ extern "C" aclnnStatus aclnnQuantMatmulV5GetWorkspaceSize(const aclTensor* x1, c
     a.gsM = (int64_t)(((uint64_t)c.groupSize >> 32) & kMask16);
 
     int mode = 0;
-    if (isA8W4F || (c.int8_in() && c.perblock()) || a4w4_pergroup_nonsym(c, (uint64_t)a.gsK)) {
-        FAIL(ACLNN_ERR_INNER_TILING_ERROR, "%s: this quant mode (fp8 x fp4, int8 per-block or int4 K-G) has no kernel on this device yet", kApi);
+    if (isA8W4F && !c.mx()) {
+        // fp8 x fp4 with a 16-bit scale per K group and a packed 64-bit output scale: qbmmv4_kernel_golden.py:189-255
+        if (c.x1.dtype != ACL_FLOAT8_E4M3FN)
+            FAIL(ACLNN_ERR_INNER_TILING_ERROR, "%s: fp8 x fp4 with group scales takes FLOAT8_E4M3FN x1 only on this device, got %s", kApi, dtype_name(c.x1.dtype));
+        ex->kind = OpKind::QmmGroup; mode = 0;
+        a.gsK = (int64_t)((uint64_t)c.groupSize & kMask16);
+        const int64_t G = ceil_div(c.K1, std::max<int64_t>(a.gsK, 1));
+        a.x2_scale_mat.ptr = c.x2s.ptr_at(0);
+        if (c.tB) { a.x2_scale_mat.row_stride = 1; a.x2_scale_mat.col_stride = G; }    // stored [N, G]
+        else { a.x2_scale_mat.row_stride = c.N; a.x2_scale_mat.col_stride = 1; }       // stored [G, N]
+        if (c.ys.present) { a.y_scale = c.ys.ptr_at(0); a.y_scale_len = c.ys.numel(); }
+    } else if (a4w4_pergroup_nonsym(c, (uint64_t)a.gsK)) {
+        // int4 x int4 with per-group scales and offsets: qbmmv4_kernel_golden.py:328-395
+        ex->kind = OpKind::QmmGroup; mode = 0;
+        a.x2_scale_mat.ptr = c.x2s.ptr_at(0); a.x2_scale_mat.row_stride = c.N; a.x2_scale_mat.col_stride = 1;
+        a.x2_offset_mat.ptr = c.x2o.ptr_at(0); a.x2_offset_mat.row_stride = c.N; a.x2_offset_mat.col_stride = 1;
     } else if (c.mx()) {
         ex->kind = OpKind::QmmMx; mode = 2;
         // scale byte of row r and 32-wide K block kb: ptr[r*row_stride + (kb/2)*col_stride + kb%2]
@@ -683,6 +697,7 @@ extern "C" aclnnStatus aclnnQuantMatmulV5(void* workspace, uint64_t workspaceSiz
         case OpKind::QmmBlockScale: rc = opsnnQmmBlockScale(&ex->qmm, stream); break;
         case OpKind::QmmMx: rc = opsnnQmmMx(&ex->qmm, stream); break;
         case OpKind::QmmTc: rc = opsnnQmmTc(&ex->qmm, stream); break;
+        case OpKind::QmmGroup: rc = opsnnQmmGroup(&ex->qmm, stream); break;
         default: rc = -100; break;
     }
     if (rc != 0) FAIL(rc < 0 ? ACLNN_ERR_INNER_TILING_ERROR : ACLNN_ERR_RUNTIME_ERROR, "aclnnQuantMatmulV5: launch failed with code %d", rc);

@@ -22,7 +22,7 @@ namespace opsnn {
 
 constexpr uint32_t kExecutorMagic = 0x51454D4Du;
 
-enum class OpKind { None, QmmInt8, QmmBlockScale, QmmMx, QmmTc, Wqmm };
+enum class OpKind { None, QmmInt8, QmmBlockScale, QmmMx, QmmTc, QmmGroup, Wqmm };
 
 // What phase 1 decided; phase 2 only fills in workspace/stream and launches.
 struct aclOpExecutorImpl {

@@ -10,6 +10,7 @@ namespace opsnn {
 int launch_blockscale_plain(const OpsnnQmmArgs& a, hipStream_t st);
 int launch_mx_plain(const OpsnnQmmArgs& a, hipStream_t st);
 int launch_tc_plain(const OpsnnQmmArgs& a, hipStream_t st);
+int launch_group_plain(const OpsnnQmmArgs& a, bool tcg, hipStream_t st);
 int launch_wqmm_plain(const OpsnnWqmmArgs& a, hipStream_t st);
 // Return OPSNN_NOT_TAKEN when the arguments are outside what the fast kernels handle.
 int launch_blockscale_mfma(const OpsnnQmmArgs& a, hipStream_t st);
@@ -67,6 +68,24 @@ extern "C" int opsnnQmmTc(const OpsnnQmmArgs* a, void* stream)
     if (a->x1_scale && (a->x1_scale_len != 1 || !f8)) return -2;
     if (a->out_dtype == DT_I8 || a->out_dtype == DT_I32) { if (!i8) return -2; }
     return launch_tc_plain(*a, (hipStream_t)stream);
+}
+
+extern "C" int opsnnQmmGroup(const OpsnnQmmArgs* a, void* stream)
+{
+    if (!qmm_args_ok(a) || a->batch != 1 || a->gsK <= 0 || !a->x2_scale_mat.ptr) return -1;
+    const bool tcg = a->x1_dtype == DT_E4M3 && a->x2_dtype == DT_E2M1;
+    const bool i4 = a->x1_dtype == DT_I4 && a->x2_dtype == DT_I4;
+    if (tcg) {
+        if (a->x2_scale_dtype != DT_BF16 && a->x2_scale_dtype != DT_F16) return -2;
+        if (a->y_scale && a->y_scale_len != 1 && a->y_scale_len != a->N) return -2;
+        if (a->bias && a->bias_dtype != DT_F32) return -2;
+    } else if (i4) {
+        if (!a->x1_scale || !a->x2_offset_mat.ptr || a->bias) return -2;
+    } else {
+        return -2;
+    }
+    if (a->out_dtype != DT_BF16 && a->out_dtype != DT_F16 && a->out_dtype != DT_F32) return -2;
+    return launch_group_plain(*a, tcg, (hipStream_t)stream);
 }
 
 extern "C" int opsnnWqmm(const OpsnnWqmmArgs* a, void* stream)

@@ -195,6 +195,75 @@ __global__ void wqmm_plain(OpsnnWqmmArgs a)
     store_f32_as(a.y, T, m * a.N + n, acc);
 }
 
+// K-group modes of quant_batch_matmul_v4: see opsnnQmmGroup in opsnn_kernels.h and qbmmv4_kernel_golden.py:189-255, 328-395
+// fp32 -> e4m3fn bits, round to nearest even; NaN and magnitudes that round above 448 give NaN
+__device__ __forceinline__ uint32_t f32_to_e4m3_bits(float f)
+{
+    const uint32_t u = f2u(f), sign = (u >> 24) & 0x80u, a = u & 0x7fffffffu;
+    if (a > 0x7f800000u || a >= 0x43f00000u) return sign | 0x7fu;     // NaN; >= 480
+    if (a < 0x3a800000u) return sign;                                  // < 2^-10 rounds to zero
+    int exp = (int)(a >> 23) - 127;
+    if (exp < -6) exp = -6;                                            // subnormal quantum 2^-9
+    const float q = u2f((uint32_t)(exp - 3 + 127) << 23);
+    const float v = __fmul_rn(__builtin_rintf(__fdiv_rn(u2f(a), q)), q);
+    if (v > 448.0f) return sign | 0x7eu;                               // 464 (the tie below the absent 480) rounds to 448
+    if (v < 0.015625f) return sign | (uint32_t)__fmul_rn(v, 512.0f);
+    const uint32_t vb = f2u(v);
+    return sign | ((((vb >> 23) - 127 + 7) << 3) | ((vb >> 20) & 7u));
+}
+__global__ void qmm_tcg_plain(OpsnnQmmArgs a)
+{
+    const int64_t nchunks = (a.N + blockDim.x - 1) / blockDim.x;
+    const int64_t m = blockIdx.x / nchunks;
+    const int64_t n = (blockIdx.x % nchunks) * (int64_t)blockDim.x + threadIdx.x;
+    if (n >= a.N) return;
+    const int64_t abase = m * a.x1.row_stride, bbase = n * a.x2.col_stride;
+    const int sdt = a.x2_scale_dtype;
+    float acc = 0.0f;
+    for (int64_t k = 0; k < a.K; k++) {
+        const float x = load_q_as_f32(a.x1.ptr, a.x1_dtype, abase + k * a.x1.col_stride);
+        const float w4 = load_q_as_f32(a.x2.ptr, a.x2_dtype, bbase + k * a.x2.row_stride);
+        const float sc = load_scalar_as_f32(a.x2_scale_mat.ptr, sdt, (k / a.gsK) * a.x2_scale_mat.row_stride + n * a.x2_scale_mat.col_stride);
+        const float mid = round_through(__fmul_rn(round_through(w4, sdt), sc), sdt);
+        const float w = e4m3_to_f32(f32_to_e4m3_bits(mid));
+        acc = __fadd_rn(acc, __fmul_rn(x, w));
+    }
+    if (a.y_scale) acc = __fmul_rn(acc, trunc19(u2f((uint32_t)((const uint64_t*)a.y_scale)[a.y_scale_len == 1 ? 0 : n])));
+    if (a.bias) acc = __fadd_rn(acc, load_scalar_as_f32(a.bias, a.bias_dtype, n));
+    store_f32_as(a.out, a.out_dtype, m * a.N + n, acc);
+}
+__global__ void qmm_i4_asym_plain(OpsnnQmmArgs a)
+{
+    const int64_t nchunks = (a.N + blockDim.x - 1) / blockDim.x;
+    const int64_t m = blockIdx.x / nchunks;
+    const int64_t n = (blockIdx.x % nchunks) * (int64_t)blockDim.x + threadIdx.x;
+    if (n >= a.N) return;
+    const int64_t abase = m * a.x1.row_stride, bbase = n * a.x2.col_stride;
+    const int64_t G = (a.K + a.gsK - 1) / a.gsK;
+    float out = 0.0f;
+    for (int64_t g = 0; g < G; g++) {
+        const int64_t k0 = g * a.gsK, k1 = (g + 1) * a.gsK < a.K ? (g + 1) * a.gsK : a.K;
+        int32_t mm = 0, rs = 0;
+        for (int64_t k = k0; k < k1; k++) {
+            const int32_t xa = (int32_t)load_q_as_f32(a.x1.ptr, DT_I4, abase + k * a.x1.col_stride);
+            const int32_t xb = (int32_t)load_q_as_f32(a.x2.ptr, DT_I4, bbase + k * a.x2.row_stride);
+            mm += xa * xb;
+            rs += xa;
+        }
+        const float off = __fmul_rn((float)rs, load_scalar_as_f32(a.x2_offset_mat.ptr, DT_F16, g * a.x2_offset_mat.row_stride + n * a.x2_offset_mat.col_stride));
+        const float sc = ((const float*)a.x2_scale_mat.ptr)[g * a.x2_scale_mat.row_stride + n * a.x2_scale_mat.col_stride];
+        out = __fadd_rn(out, __fmul_rn(__fsub_rn((float)mm, off), sc));
+    }
+    out = __fmul_rn(out, ((const float*)a.x1_scale)[m]);
+    store_f32_as(a.out, a.out_dtype, m * a.N + n, out);
+}
+int launch_group_plain(const OpsnnQmmArgs& a, bool tcg, hipStream_t st)
+{
+    dim3 block(256), grid((unsigned)(((a.N + 255) / 256) * a.M));
+    if (tcg) hipLaunchKernelGGL(qmm_tcg_plain, grid, block, 0, st, a);
+    else hipLaunchKernelGGL(qmm_i4_asym_plain, grid, block, 0, st, a);
+    return (int)hipGetLastError();
+}
 int launch_blockscale_plain(const OpsnnQmmArgs& a, hipStream_t st)
 {
     dim3 block(256), grid((unsigned)(((a.N + 255) / 256) * a.M), (unsigned)a.batch);

@@ -44,6 +44,7 @@ class OpsnnQmmArgs(C.Structure):
         ("x1_scale_mat", OpsnnMat), ("x2_scale_mat", OpsnnMat),
         ("workspace", C.c_void_p), ("force_variant", C.c_int),
         ("x1_scale_len", C.c_int64), ("x2_offset", C.c_void_p), ("x2_offset_len", C.c_int64),
+        ("y_scale", C.c_void_p), ("y_scale_len", C.c_int64), ("x2_offset_mat", OpsnnMat),
     ]
 
 
@@ -103,6 +104,7 @@ _SIGS = {
     "opsnnQmmBlockScale": (C.c_int, [C.POINTER(OpsnnQmmArgs), C.c_void_p]),
     "opsnnQmmMx": (C.c_int, [C.POINTER(OpsnnQmmArgs), C.c_void_p]),
     "opsnnQmmTc": (C.c_int, [C.POINTER(OpsnnQmmArgs), C.c_void_p]),
+    "opsnnQmmGroup": (C.c_int, [C.POINTER(OpsnnQmmArgs), C.c_void_p]),
     "opsnnQmmWorkspace": (C.c_uint64, [C.POINTER(OpsnnQmmArgs), C.c_int]),
     "opsnnWqmm": (C.c_int, [C.POINTER(OpsnnWqmmArgs), C.c_void_p]),
     "opsnnWqmmWorkspace": (C.c_uint64, [C.POINTER(OpsnnWqmmArgs)]),

@@ -11,6 +11,7 @@
  *   GW  = weight_quant_batch_matmul_v2/tests/assets/wqbmmv2_kernel_golden.py
  *   GU  = common/tests/st/arch35/matmul_golden_util.py
  *   GQ  = common/tests/st/arch35/matmul_quant_util.py
+ *   G4  = quant_batch_matmul_v4/tests/assets/qbmmv4_kernel_golden.py
  *
  * Arithmetic conventions shared with the golden: every float operation is a
  * separately rounded fp32 operation (this file is compiled with
@@ -26,7 +27,12 @@
  *   orc_qmm_tc ........ pinned (reduces to orc_qmm_pertoken with a constant row scale; hand-computed requant and
  *                       19-bit truncation cases; uint64 packing constants of the reference's utility)
  *   orc_qmm_perblock .. pinned (reduces to pertoken formula with one K block; power-of-two scales exact; float64)
- *   orc_qmm_mx ........ pinned (power-of-two products are exact: equals integer arithmetic; float64)
+ *   orc_qmm_mx ........ pinned (power-of-two products are exact: equals integer arithmetic; float64); also serves
+ *                       compute_mx of G4 (fp8 x fp4) and, with int8 operands, orc_qmm_perblock serves compute_per_tile
+ *   orc_qmm_tcg ....... pinned for in-range values (numpy recomputation with independent codecs; unit scale reduces to
+ *                       a plain fp32 matmul); fp32 -> fp8 overflow: parity unpinned (see the function)
+ *   orc_qmm_i4_asym ... pinned (numpy int64 / float32 recomputation; zero offset and one group reduce to the
+ *                       per-token formula)
  *   orc_wqbmm ......... pinned (hand-computed double-rounding cases; group==K equals per-channel; float64)
  *   hifloat8 .......... not implemented (decoder lives only in an absent third-party package): parity unpinned
  */
@@ -568,6 +574,78 @@ static inline float trunc_to(float v, int dt)
     if (dt == ORC_F16) return orc_f16_to_f32(orc_f16_from_f32(v));
     if (dt == ORC_BF16) return orc_bf16_to_f32(orc_bf16_from_f32(v));
     return v;
+}
+
+/*
+ * compute_t_cg (G4:189-255): fp8 x1, fp4 x2 with a 16-bit scale per `gs` K elements, 64-bit packed output scale.
+ *   w[k,n] = fp32( T8( fp32( T16( T16(x2[k,n]) * x2Scale[k/gs, n] ) ) ) )     T16 = the scale's dtype, T8 = x1's dtype
+ *   y = (fp32(x1) @ w) * deq(yScale[n]) (+ fp32 bias);  cast            deq = u64_to_deq_scale (GQ:129-135)
+ * x2 storage: [K, N] packed along N, or [N, K] packed along K if tB; x2Scale storage [K/gs, N], or [N, K/gs] if tB.
+ * Only x1 = e4m3 is implemented.  fp32 -> e4m3 follows orc_e4m3_from_f32 (magnitudes that round above 448 give
+ * NaN); the golden delegates that cast to a third-party package that is not available here, so its overflow
+ * behaviour is parity unpinned -- in-range values are pinned by the exhaustive codec tables.
+ */
+int orc_qmm_tcg(const uint8_t* x1, const uint8_t* x2, int64_t M, int64_t K, int64_t N, int tB, const uint16_t* x2s,
+                int s_dt, int64_t gs, const uint64_t* yscale, int64_t ylen, const float* bias, int y_dt, void* y)
+{
+    float* a = decode_matrix(x1, ORC_E4M3, M, K, 0);
+    float* b = tB ? decode_matrix(x2, ORC_E2M1, N, K, 1) : decode_matrix(x2, ORC_E2M1, K, N, 0);
+    float* acc = (float*)calloc((size_t)M * N, sizeof(float));
+    if (!a || !b || !acc) return -1;
+    const int64_t G = (K + gs - 1) / gs;
+#pragma omp parallel for schedule(static)
+    for (int64_t k = 0; k < K; k++)
+        for (int64_t n = 0; n < N; n++) {
+            const int64_t g = k / gs;
+            const float sc = load_as_f32(x2s, s_dt, (size_t)(tB ? n * G + g : g * N + n));
+            const float mid = trunc_to(trunc_to(b[k * N + n], s_dt) * sc, s_dt);
+            b[k * N + n] = orc_e4m3_to_f32(orc_e4m3_from_f32(mid));
+        }
+    sgemm_acc(a, K, b, N, acc, N, M, N, K);
+    for (int64_t m = 0; m < M; m++)
+        for (int64_t n = 0; n < N; n++) {
+            float o = acc[m * N + n];
+            if (yscale) o = o * orc_u64_to_deq_scale(yscale[ylen == 1 ? 0 : n]);
+            if (bias) o = o + bias[n];
+            store_from_f32(y, y_dt, (size_t)(m * N + n), o);
+        }
+    free(a); free(b); free(acc);
+    return 0;
+}
+
+/*
+ * compute_int4_asymmetrical (G4:328-395): int4 x int4, one fp32 scale and one fp16 offset per 256 K elements and
+ * column, one fp32 scale per row.
+ *   acc[m,n] = sum_g ( fp32(sum_{k in g} x1*x2) - fp32(sum_{k in g} x1) * fp32(x2Offset[g,n]) ) * x2Scale[g,n]
+ *   y = acc * x1Scale[m];  cast
+ * x1 storage [M, K] packed along K; x2 storage [K, N] packed along N, or [N, K] packed along K if tB;
+ * x2Scale / x2Offset storage [ceil(K/256), N] either way.  The integer sums are exact.
+ */
+int orc_qmm_i4_asym(const uint8_t* x1, const uint8_t* x2, int64_t M, int64_t K, int64_t N, int tB, const float* x1s,
+                    const float* x2s, const uint16_t* x2o, int y_dt, void* y)
+{
+    const int64_t GK = 256, G = (K + GK - 1) / GK;
+    float* a = decode_matrix(x1, ORC_I4, M, K, 0);
+    float* b = tB ? decode_matrix(x2, ORC_I4, N, K, 1) : decode_matrix(x2, ORC_I4, K, N, 0);
+    if (!a || !b) return -1;
+#pragma omp parallel for schedule(static)
+    for (int64_t m = 0; m < M; m++)
+        for (int64_t n = 0; n < N; n++) {
+            float out = 0.0f;
+            for (int64_t g = 0; g < G; g++) {
+                const int64_t k0 = g * GK, k1 = (g + 1) * GK < K ? (g + 1) * GK : K;
+                int32_t mm = 0, rs = 0;
+                for (int64_t k = k0; k < k1; k++) {
+                    mm += (int32_t)a[m * K + k] * (int32_t)b[k * N + n];
+                    rs += (int32_t)a[m * K + k];
+                }
+                const float off = (float)rs * orc_f16_to_f32(x2o[g * N + n]);
+                out = out + ((float)mm - off) * x2s[g * N + n];
+            }
+            store_from_f32(y, y_dt, (size_t)(m * N + n), out * x1s[m]);
+        }
+    free(a); free(b);
+    return 0;
 }
 
 /*

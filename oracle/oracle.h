@@ -55,6 +55,10 @@ int orc_qmm_perblock(const void* x1, const void* x2, int dt1, int dt2, int64_t M
                      const float* bias, int y_dt, void* y);
 int orc_qmm_mx(const void* x1, const void* x2, int dt1, int dt2, int64_t M, int64_t K, int64_t N, int tA, int tB,
                const uint8_t* x1s, const uint8_t* x2s, const float* bias, int y_dt, void* y);
+int orc_qmm_tcg(const uint8_t* x1, const uint8_t* x2, int64_t M, int64_t K, int64_t N, int tB, const uint16_t* x2s,
+                int s_dt, int64_t gs, const uint64_t* yscale, int64_t ylen, const float* bias, int y_dt, void* y);
+int orc_qmm_i4_asym(const uint8_t* x1, const uint8_t* x2, int64_t M, int64_t K, int64_t N, int tB, const float* x1s,
+                    const float* x2s, const uint16_t* x2o, int y_dt, void* y);
 int orc_wqbmm(const void* x, int x_dt, const void* w, int w_dt, int64_t M, int64_t K, int64_t N, int tW,
               const void* scale, int scale_dt, int64_t scale_n, const void* offset, int64_t group,
               const void* bias, int bias_dt, void* y);

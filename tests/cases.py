@@ -330,3 +330,134 @@ def run_wq_aclnn(m, inp, M, K, N, v3=False, scale_2d=None):
     m.check(m.lib().aclrtSynchronizeDevice(), "sync")
     del ws
     return d_y.to_host(np.uint16, (M, N))
+
+
+# --------------------------------------------------------------------------------------------------
+# K-group modes of quant_batch_matmul_v4: fp8 x fp4 MX, fp8 x fp4 with 16-bit group scales (T-CG), int8 per-tile,
+# int4 x int4 with per-group scales and offsets
+# --------------------------------------------------------------------------------------------------
+FP4_VALUES = np.array([0.0, 0.5, 1.0, 1.5, 2.0, 3.0, 4.0, 6.0, -0.0, -0.5, -1.0, -1.5, -2.0, -3.0, -4.0, -6.0], np.float32)
+
+
+def make_a8w4_mx_inputs(m, M, K, N, seed, tB):
+    rng = np.random.default_rng(seed)
+    KS = -(-K // 64)
+    x1 = gen_fp8(rng, (M, K))
+    x2 = orc.pack_nibbles(rng.integers(0, 16, size=(N, K) if tB else (K, N), dtype=np.uint8))
+    s1 = (127 + rng.integers(-3, 4, size=(M, KS, 2))).astype(np.uint8)
+    s2 = (127 + rng.integers(-3, 4, size=(N, KS, 2) if tB else (KS, N, 2))).astype(np.uint8)
+    bias = orc.f32_to_f16(rng.normal(0, 1, N).astype(np.float32))
+    return dict(x1=x1, x2=x2, s1=s1, s2=s2, bias=bias)
+
+
+def oracle_a8w4_mx(m, inp, M, K, N, tB, out_dt):
+    return orc.qmm_mx(inp["x1"], inp["x2"], orc.E4M3, orc.E2M1, M, K, N, False, tB, inp["s1"], inp["s2"], orc.f16_to_f32(inp["bias"]), out_dt)
+
+
+def run_a8w4_mx_aclnn(m, inp, M, K, N, tB, out_dt):
+    d = {k: m.DeviceBuffer(host=v) for k, v in inp.items()}
+    out_np = orc.out_array((M, N), out_dt)
+    d_out = m.DeviceBuffer(out_np.nbytes); d_out.fill(0xFF)
+    x1 = m.Tensor((M, K), m.ACL_FLOAT8_E4M3FN, d["x1"])
+    x2 = m.Tensor((N, K) if tB else (K, N), m.ACL_FLOAT4_E2M1, d["x2"])
+    s1 = m.Tensor(inp["s1"].shape, m.ACL_FLOAT8_E8M0, d["s1"])
+    s2 = m.Tensor(inp["s2"].shape, m.ACL_FLOAT8_E8M0, d["s2"])
+    bias = m.Tensor((1, N), m.ACL_FLOAT16, d["bias"])
+    out = m.Tensor((M, N), out_dt, d_out)
+    ws = m.quant_matmul_v5(x1, x2, s1, s2, out, bias=bias, transpose_x2=tB, group_size=32)
+    m.check(m.lib().aclrtSynchronizeDevice(), "sync")
+    del ws
+    return d_out.to_host(out_np.dtype, out_np.shape)
+
+
+def make_tcg_inputs(m, M, K, N, seed, s_dt):
+    """x2 stored [N, K] (the mode requires transposeX2), scales [N, K/32] in s_dt, yScale uint64 [1, N].
+    Scales stay below 64 so that 6 * scale fits e4m3 (the cast's overflow behaviour is not pinned)."""
+    rng = np.random.default_rng(seed)
+    x1 = gen_fp8(rng, (M, K))
+    x2 = orc.pack_nibbles(rng.integers(0, 16, size=(N, K), dtype=np.uint8))
+    sf = rng.uniform(0.05, 60.0, size=(N, K // 32)).astype(np.float32)
+    s2 = orc.f32_to_bf16(sf) if s_dt == m.ACL_BF16 else orc.f32_to_f16(sf)
+    ys = orc.pack_u64_scale(rng.uniform(1e-3, 1e-2, N).astype(np.float32)).reshape(1, N)
+    return dict(x1=x1, x2=x2, s2=s2, ys=ys, s_dt=s_dt)
+
+
+def oracle_tcg(m, inp, M, K, N, out_dt):
+    return orc.qmm_tcg(inp["x1"], inp["x2"], M, K, N, True, inp["s2"], inp["s_dt"], 32, inp["ys"], None, out_dt)
+
+
+def run_tcg_aclnn(m, inp, M, K, N, out_dt, ys_dt=None):
+    d = {k: m.DeviceBuffer(host=v) for k, v in inp.items() if isinstance(v, np.ndarray)}
+    out_np = orc.out_array((M, N), out_dt)
+    d_out = m.DeviceBuffer(out_np.nbytes); d_out.fill(0xFF)
+    x1 = m.Tensor((M, K), m.ACL_FLOAT8_E4M3FN, d["x1"])
+    x2 = m.Tensor((N, K), m.ACL_FLOAT4_E2M1, d["x2"])
+    s2 = m.Tensor((N, K // 32), inp["s_dt"], d["s2"])
+    ys = m.Tensor((1, N), ys_dt or m.ACL_UINT64, d["ys"])
+    out = m.Tensor((M, N), out_dt, d_out)
+    ws = m.quant_matmul_v5(x1, x2, None, s2, out, y_scale=ys, transpose_x2=True, group_size=32)
+    m.check(m.lib().aclrtSynchronizeDevice(), "sync")
+    del ws
+    return d_out.to_host(out_np.dtype, out_np.shape)
+
+
+def make_pertile_i8_inputs(m, M, K, N, seed, tB):
+    rng = np.random.default_rng(seed)
+    KB, NB = -(-K // 128), -(-N // 128)
+    x1, x2 = gen_int8(rng, (M, K)), gen_int8(rng, (N, K) if tB else (K, N))
+    s1 = gen_scale(rng, (M, KB), 1e-3, 1e-2)
+    s2 = gen_scale(rng, (NB, KB) if tB else (KB, NB), 1e-3, 1e-2)
+    bias = rng.normal(0, 1, N).astype(np.float32)
+    return dict(x1=x1, x2=x2, s1=s1, s2=s2, bias=bias)
+
+
+def oracle_pertile_i8(m, inp, M, K, N, tB, out_dt):
+    return orc.qmm_perblock(inp["x1"], inp["x2"], orc.I8, orc.I8, M, K, N, False, tB, inp["s1"], inp["s2"], 1, 128, 128, inp["bias"], out_dt)
+
+
+def run_pertile_i8_aclnn(m, inp, M, K, N, tB, out_dt):
+    d = {k: m.DeviceBuffer(host=v) for k, v in inp.items()}
+    out_np = orc.out_array((M, N), out_dt)
+    d_out = m.DeviceBuffer(out_np.nbytes); d_out.fill(0xFF)
+    x1 = m.Tensor((M, K), m.ACL_INT8, d["x1"])
+    x2 = m.Tensor((N, K) if tB else (K, N), m.ACL_INT8, d["x2"])
+    s1 = m.Tensor(inp["s1"].shape, m.ACL_FLOAT, d["s1"])
+    s2 = m.Tensor(inp["s2"].shape, m.ACL_FLOAT, d["s2"])
+    bias = m.Tensor((N,), m.ACL_FLOAT, d["bias"])
+    out = m.Tensor((M, N), out_dt, d_out)
+    ws = m.quant_matmul_v5(x1, x2, s1, s2, out, bias=bias, transpose_x2=tB, group_size=(1 << 32) | (128 << 16) | 128)
+    m.check(m.lib().aclrtSynchronizeDevice(), "sync")
+    del ws
+    return d_out.to_host(out_np.dtype, out_np.shape)
+
+
+def make_i4_asym_inputs(m, M, K, N, seed):
+    """x2 stored [N, K] (the mode requires transposeX2); scales fp32 and offsets fp16 [K/256, N]; x1Scale fp32 [M, 1]."""
+    rng = np.random.default_rng(seed)
+    x1 = orc.pack_nibbles(rng.integers(0, 16, size=(M, K), dtype=np.uint8))
+    x2 = orc.pack_nibbles(rng.integers(0, 16, size=(N, K), dtype=np.uint8))
+    G = -(-K // 256)
+    s1 = gen_scale(rng, (M, 1), 1e-2, 1e-1)
+    s2 = gen_scale(rng, (G, N), 1e-2, 1e-1)
+    off = orc.f32_to_f16(rng.uniform(-8, 8, size=(G, N)).astype(np.float32))
+    return dict(x1=x1, x2=x2, s1=s1, s2=s2, off=off)
+
+
+def oracle_i4_asym(m, inp, M, K, N, out_dt):
+    return orc.qmm_i4_asym(inp["x1"], inp["x2"], M, K, N, True, inp["s1"], inp["s2"], inp["off"], out_dt)
+
+
+def run_i4_asym_aclnn(m, inp, M, K, N, out_dt):
+    d = {k: m.DeviceBuffer(host=v) for k, v in inp.items()}
+    out_np = orc.out_array((M, N), out_dt)
+    d_out = m.DeviceBuffer(out_np.nbytes); d_out.fill(0xFF)
+    x1 = m.Tensor((M, K), m.ACL_INT4, d["x1"])
+    x2 = m.Tensor((N, K), m.ACL_INT4, d["x2"])
+    s1 = m.Tensor(inp["s1"].shape, m.ACL_FLOAT, d["s1"])
+    s2 = m.Tensor(inp["s2"].shape, m.ACL_FLOAT, d["s2"])
+    off = m.Tensor(inp["off"].shape, m.ACL_FLOAT16, d["off"])
+    out = m.Tensor((M, N), out_dt, d_out)
+    ws = m.quant_matmul_v5(x1, x2, s1, s2, out, x2_offset=off, transpose_x2=True, group_size=256)
+    m.check(m.lib().aclrtSynchronizeDevice(), "sync")
+    del ws
+    return d_out.to_host(out_np.dtype, out_np.shape)

@@ -29,6 +29,8 @@ def lib():
         L.orc_qmm_tc.argtypes = [vp, vp, ci, ci, i64, i64, i64, ci, ci, vp, ci, i64, vp, vp, i64, vp, ci, ci, vp]
         L.orc_qmm_mx.argtypes = [vp, vp, ci, ci, i64, i64, i64, ci, ci, vp, vp, vp, ci, vp]
         L.orc_wqbmm.argtypes = [vp, ci, vp, ci, i64, i64, i64, ci, vp, ci, i64, vp, i64, vp, ci, vp]
+        L.orc_qmm_tcg.argtypes = [vp, vp, i64, i64, i64, ci, vp, ci, i64, vp, i64, vp, ci, vp]
+        L.orc_qmm_i4_asym.argtypes = [vp, vp, i64, i64, i64, ci, vp, vp, vp, ci, vp]
         for n in ("orc_vec_f32_to_bf16", "orc_vec_bf16_to_f32", "orc_vec_f32_to_f16", "orc_vec_f16_to_f32",
                   "orc_vec_f32_to_e4m3", "orc_vec_e4m3_to_f32", "orc_vec_e5m2_to_f32", "orc_vec_e8m0_to_f32"):
             getattr(L, n).argtypes = [vp, vp, C.c_size_t]
@@ -144,6 +146,27 @@ def pack_u64_scale(scale_f32, offset_f32=None):
 def qmm_mx(x1, x2, dt1, dt2, M, K, N, tA, tB, x1s, x2s, bias, y_dt):
     y = out_array((M, N), y_dt)
     rc = lib().orc_qmm_mx(_p(x1), _p(x2), dt1, dt2, M, K, N, int(tA), int(tB), _p(x1s), _p(x2s), _p(bias), y_dt, _p(y))
+    assert rc == 0
+    return y
+
+
+def qmm_tcg(x1, x2, M, K, N, tB, x2s, s_dt, gs, yscale, bias, y_dt):
+    """fp8 e4m3 x fp4 with 16-bit group scales and a packed 64-bit output scale (compute_t_cg)."""
+    y = out_array((M, N), y_dt)
+    x2s = np.ascontiguousarray(x2s)
+    yscale = None if yscale is None else np.ascontiguousarray(yscale, np.uint64)
+    bias = None if bias is None else np.ascontiguousarray(bias, np.float32)
+    rc = lib().orc_qmm_tcg(_p(x1), _p(x2), M, K, N, int(tB), _p(x2s), s_dt, gs, _p(yscale), 0 if yscale is None else yscale.size,
+                           _p(bias), y_dt, _p(y))
+    assert rc == 0
+    return y
+
+
+def qmm_i4_asym(x1, x2, M, K, N, tB, x1s, x2s, x2o, y_dt):
+    """int4 x int4 with per-256-K scales and fp16 offsets (compute_int4_asymmetrical)."""
+    y = out_array((M, N), y_dt)
+    x1s = np.ascontiguousarray(x1s, np.float32); x2s = np.ascontiguousarray(x2s, np.float32); x2o = np.ascontiguousarray(x2o, np.uint16)
+    rc = lib().orc_qmm_i4_asym(_p(x1), _p(x2), M, K, N, int(tB), _p(x1s), _p(x2s), _p(x2o), y_dt, _p(y))
     assert rc == 0
     return y
 

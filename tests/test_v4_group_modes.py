@@ -1,0 +1,172 @@
+"""K-group modes of quant_batch_matmul_v4 behind aclnnQuantMatmulV5: fp8 x fp4 MX, fp8 x fp4 with 16-bit group
+scales and a packed output scale (T-CG), int8 per-tile, int4 x int4 with per-group scales and offsets.
+
+CPU part: the two new oracle functions are pinned by independent numpy recomputations of the reference formulas
+(matmul/quant_batch_matmul_v4/tests/assets/qbmmv4_kernel_golden.py:189-255, 328-395) and by special cases that
+reduce to plain matrix products; the MX and per-tile modes reuse oracle functions that are pinned elsewhere (int8
+per-tile partial sums are integers below 2^24, so the fp32 sums of the block-scale function are exact).
+GPU part: the library through the aclnn C ABI must be bit-identical to the oracle (plain kernels, same operation order).
+"""
+import numpy as np
+import pytest
+
+import cases
+import oracle_api as orc
+
+
+def fp4_decode(packed):
+    return cases.FP4_VALUES[orc.unpack_nibbles(packed)]
+
+
+def i4_decode(packed):
+    v = orc.unpack_nibbles(packed).astype(np.int32)
+    return np.where(v >= 8, v - 16, v)
+
+
+def matmul_ascending(a, b):
+    out = np.zeros((a.shape[0], b.shape[1]), np.float32)
+    for k in range(a.shape[1]):
+        out = (out + a[:, k:k + 1] * b[k:k + 1, :]).astype(np.float32)
+    return out
+
+
+@pytest.mark.parametrize("s_dt", ["bf16", "f16"])
+def test_tcg_against_numpy(s_dt):
+    M, K, N = 5, 64, 12
+    rng = np.random.default_rng(3)
+    x1 = orc.f32_to_e4m3(rng.normal(0, 1, (M, K)).astype(np.float32))
+    x2 = orc.pack_nibbles(rng.integers(0, 16, size=(N, K), dtype=np.uint8))
+    sf = rng.uniform(0.05, 60, (N, K // 32)).astype(np.float32)
+    to16, from16, code = (orc.f32_to_bf16, orc.bf16_to_f32, orc.BF16) if s_dt == "bf16" else (orc.f32_to_f16, orc.f16_to_f32, orc.F16)
+    s2 = to16(sf)
+    ysf = rng.uniform(1e-3, 1e-2, N).astype(np.float32)
+    ys = orc.pack_u64_scale(ysf)
+    bias = rng.normal(0, 1, N).astype(np.float32)
+    # w = e4m3(T16(fp4 * scale)); the fp4 values are exact in both 16-bit types
+    w = fp4_decode(x2).T                                         # [K, N]
+    sc = np.repeat(from16(s2).T, 32, axis=0)                     # [K, N]
+    mid = from16(to16((w * sc).astype(np.float32)))
+    wq = orc.e4m3_to_f32(orc.f32_to_e4m3(mid))
+    deq = (ysf.view(np.uint32) & np.uint32(0xFFFFE000)).view(np.float32)
+    want = orc.f32_to_f16(((matmul_ascending(orc.e4m3_to_f32(x1), wq) * deq).astype(np.float32) + bias).astype(np.float32))
+    got = orc.qmm_tcg(x1, x2, M, K, N, True, s2, code, 32, ys, bias, orc.F16)
+    assert np.array_equal(got, want)
+    # the untransposed storage gives the same result
+    x2_kn = orc.pack_nibbles(np.ascontiguousarray(orc.unpack_nibbles(x2).T))
+    s2_kn = np.ascontiguousarray(s2.T)
+    assert np.array_equal(orc.qmm_tcg(x1, x2_kn, M, K, N, False, s2_kn, code, 32, ys, bias, orc.F16), want)
+
+
+def test_tcg_unit_scales_is_a_plain_product():
+    # scale 1.0 and an output scale of 1.0: fp4 values survive both roundings, the result is x1 @ x2 in fp32
+    M, K, N = 4, 32, 8
+    rng = np.random.default_rng(4)
+    x1 = orc.f32_to_e4m3(rng.integers(-4, 5, (M, K)).astype(np.float32))
+    x2 = orc.pack_nibbles(rng.integers(0, 16, size=(N, K), dtype=np.uint8))
+    s2 = orc.f32_to_bf16(np.ones((N, 1), np.float32))
+    ys = orc.pack_u64_scale(np.ones(N, np.float32))
+    got = orc.qmm_tcg(x1, x2, M, K, N, True, s2, orc.BF16, 32, ys, None, orc.F32)
+    want = orc.e4m3_to_f32(x1).astype(np.float64) @ fp4_decode(x2).T.astype(np.float64)   # small half-integers: exact
+    assert np.array_equal(got.astype(np.float64), want)
+
+
+def test_i4_asym_against_numpy():
+    M, K, N = 6, 600, 10      # 600 = 2 full groups of 256 and a ragged third
+    rng = np.random.default_rng(5)
+    x1 = orc.pack_nibbles(rng.integers(0, 16, size=(M, K), dtype=np.uint8))
+    x2 = orc.pack_nibbles(rng.integers(0, 16, size=(N, K), dtype=np.uint8))
+    G = 3
+    s1 = rng.uniform(0.01, 0.1, (M, 1)).astype(np.float32)
+    s2 = rng.uniform(0.01, 0.1, (G, N)).astype(np.float32)
+    off = orc.f32_to_f16(rng.uniform(-8, 8, (G, N)).astype(np.float32))
+    a, b = i4_decode(x1).astype(np.int64), i4_decode(x2).T.astype(np.int64)
+    out = np.zeros((M, N), np.float32)
+    for g in range(G):
+        ks = slice(256 * g, min(256 * (g + 1), K))
+        mm = (a[:, ks] @ b[ks, :]).astype(np.float32)
+        rs = a[:, ks].sum(axis=1, keepdims=True).astype(np.float32)
+        o = (rs * orc.f16_to_f32(off[g:g + 1, :])).astype(np.float32)
+        out = (out + ((mm - o).astype(np.float32) * s2[g:g + 1, :]).astype(np.float32)).astype(np.float32)
+    want = orc.f32_to_bf16((out * s1).astype(np.float32))
+    assert np.array_equal(orc.qmm_i4_asym(x1, x2, M, K, N, True, s1, s2, off, orc.BF16), want)
+
+
+def test_i4_asym_without_offsets_is_the_per_token_formula():
+    # zero offsets, one group, power-of-two scales: out = (x1 @ x2) * s2[n] * s1[m] exactly, as in compute_pertoken
+    M, K, N = 5, 256, 7
+    rng = np.random.default_rng(6)
+    x1 = orc.pack_nibbles(rng.integers(0, 16, size=(M, K), dtype=np.uint8))
+    x2 = orc.pack_nibbles(rng.integers(0, 16, size=(N, K), dtype=np.uint8))
+    s1 = (2.0 ** rng.integers(-6, -1, (M, 1))).astype(np.float32)
+    s2 = (2.0 ** rng.integers(-6, -1, (1, N))).astype(np.float32)
+    off = np.zeros((1, N), np.uint16)
+    acc = i4_decode(x1).astype(np.int64) @ i4_decode(x2).T.astype(np.int64)
+    want = (acc.astype(np.float64) * s2.astype(np.float64) * s1.astype(np.float64)).astype(np.float32)
+    assert np.array_equal(orc.qmm_i4_asym(x1, x2, M, K, N, True, s1, s2, off, orc.F32), want)
+
+
+def test_pertile_i8_partial_sums_are_exact():
+    # the block-scale oracle sums int8 products in fp32; per 128-K tile they are integers below 2^24, so the result
+    # equals the int32-matmul formulation of compute_per_tile (qbmmv4_kernel_golden.py:258-325)
+    M, K, N = 4, 300, 140
+    rng = np.random.default_rng(7)
+    x1 = np.full((M, K), 127, np.int8); x2 = np.full((K, N), -127, np.int8)     # worst case magnitude
+    x1[1:] = rng.integers(-127, 128, (M - 1, K)); x2[:, 1:] = rng.integers(-127, 128, (K, N - 1))
+    s1 = rng.uniform(1e-3, 1e-2, (M, 3)).astype(np.float32); s2 = rng.uniform(1e-3, 1e-2, (3, 2)).astype(np.float32)
+    bias = rng.normal(0, 1, N).astype(np.float32)
+    out = np.zeros((M, N), np.float32)
+    for kb in range(3):
+        ks = slice(128 * kb, min(128 * (kb + 1), K))
+        mm = (x1[:, ks].astype(np.int32) @ x2[ks, :].astype(np.int32)).astype(np.float32)
+        sc = (s1[:, kb:kb + 1] * np.repeat(s2[kb:kb + 1, :], 128, axis=1)[:, :N]).astype(np.float32)
+        out = (out + (mm * sc).astype(np.float32)).astype(np.float32)
+    want = orc.f32_to_bf16((out + bias).astype(np.float32))
+    got = orc.qmm_perblock(x1, x2, orc.I8, orc.I8, M, K, N, False, False, s1, s2, 1, 128, 128, bias, orc.BF16)
+    assert np.array_equal(got, want)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("M,K,N,tB", [(16, 128, 128, True), (33, 192, 72, True), (20, 256, 64, True)])
+def test_gpu_a8w4_mx(gpu, M, K, N, tB):
+    m = gpu
+    print(f"case a8w4 mx {M}x{K}x{N} tB={tB}", flush=True)
+    inp = cases.make_a8w4_mx_inputs(m, M, K, N, M + N, tB)
+    want = cases.oracle_a8w4_mx(m, inp, M, K, N, tB, m.ACL_FLOAT16)
+    got = cases.run_a8w4_mx_aclnn(m, inp, M, K, N, tB, m.ACL_FLOAT16)
+    assert np.array_equal(got, want), f"{int((got != want).sum())} of {got.size} outputs differ"
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("M,K,N,s_dt,out_dt,ys_i64", [(16, 64, 16, "bf16", "f16", False), (16, 64, 16, "bf16", "f16", True),
+                                                      (37, 256, 50, "f16", "bf16", False), (9, 128, 130, "bf16", "bf16", False)])
+def test_gpu_tcg(gpu, M, K, N, s_dt, out_dt, ys_i64):
+    m = gpu
+    print(f"case tcg {M}x{K}x{N} scale={s_dt} out={out_dt} yscale int64={ys_i64}", flush=True)
+    dt = {"bf16": m.ACL_BF16, "f16": m.ACL_FLOAT16}
+    inp = cases.make_tcg_inputs(m, M, K, N, M + N, dt[s_dt])
+    want = cases.oracle_tcg(m, inp, M, K, N, dt[out_dt])
+    got = cases.run_tcg_aclnn(m, inp, M, K, N, dt[out_dt], m.ACL_INT64 if ys_i64 else None)
+    assert np.array_equal(got, want), f"{int((got != want).sum())} of {got.size} outputs differ"
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("M,K,N,tB", [(16, 256, 128, True), (40, 300, 200, False), (7, 128, 130, True)])
+def test_gpu_pertile_i8(gpu, M, K, N, tB):
+    m = gpu
+    print(f"case int8 per-tile {M}x{K}x{N} tB={tB}", flush=True)
+    inp = cases.make_pertile_i8_inputs(m, M, K, N, M + N, tB)
+    want = cases.oracle_pertile_i8(m, inp, M, K, N, tB, m.ACL_BF16)
+    got = cases.run_pertile_i8_aclnn(m, inp, M, K, N, tB, m.ACL_BF16)
+    assert np.array_equal(got, want), f"{int((got != want).sum())} of {got.size} outputs differ"
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("M,K,N,out_dt", [(9, 1024, 256, "bf16"), (9, 1024, 256, "f16"), (33, 2048, 512, "bf16")])
+def test_gpu_i4_asym(gpu, M, K, N, out_dt):
+    m = gpu
+    print(f"case int4 K-G {M}x{K}x{N} out={out_dt}", flush=True)
+    dt = {"bf16": m.ACL_BF16, "f16": m.ACL_FLOAT16}
+    inp = cases.make_i4_asym_inputs(m, M, K, N, M + N)
+    want = cases.oracle_i4_asym(m, inp, M, K, N, dt[out_dt])
+    got = cases.run_i4_asym_aclnn(m, inp, M, K, N, dt[out_dt])
+    assert np.array_equal(got, want), f"{int((got != want).sum())} of {got.size} outputs differ"
