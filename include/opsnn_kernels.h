@@ -48,7 +48,7 @@ typedef struct {
     int out_dtype;        /* BF16 / FLOAT16 / FLOAT / INT32 */
     const void* x1_scale; /* see each launcher */
     const void* x2_scale;
-    int x2_scale_dtype;   /* FLOAT or BF16 */
+    int x2_scale_dtype;   /* FLOAT or BF16 (opsnnQmmInt8, opsnnQmmTc: also UINT64) */
     int64_t x2_scale_len; /* 1 or N */
     const void* bias;     /* [N] or NULL */
     int bias_dtype;       /* INT32 / BF16 / FLOAT16 / FLOAT */
@@ -70,6 +70,9 @@ typedef struct {
     const void* y_scale;   /* UINT64 [1] or [N]: fp32 scale in the low word, upper 19 bits kept */
     int64_t y_scale_len;
     OpsnnMat x2_offset_mat;/* FLOAT16, logical [ceil(K/gsK), N] */
+    /* opsnnQmmInt8: keep only the upper 19 bits of x2_scale (the reference's scale truncation; always applied to
+     * UINT64 scale words, whose low 32 bits are the fp32 scale) */
+    int x2_scale_trunc;
 } OpsnnQmmArgs;
 
 /* int8 x int8 -> int32, then  out = fp32(acc + int32 bias) * x2_scale[n] * x1_scale[m] + float bias.

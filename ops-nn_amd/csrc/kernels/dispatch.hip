@@ -67,6 +67,17 @@ extern "C" int opsnnQmmTc(const OpsnnQmmArgs* a, void* stream)
     if (a->x2_scale_len != 1 && a->x2_scale_len != a->N) return -2;
     if (a->x1_scale && (a->x1_scale_len != 1 || !f8)) return -2;
     if (a->out_dtype == DT_I8 || a->out_dtype == DT_I32) { if (!i8) return -2; }
+    // int8 operands, 16-bit output, no per-token scale: out = fp32(acc + int32 bias) * scale' + float bias, where scale'
+    // is the scale with only its upper 19 bits kept for 64-bit words and for a one-element scale without a bf16 / fp32
+    // bias (qbmmv3_kernel_golden.py:403-475).  That is the per-token x per-channel formula with x1_scale = 1: the MFMA
+    // kernel computes it bit-identically.
+    if (i8 && !a->x1_scale && (a->out_dtype == DT_BF16 || a->out_dtype == DT_F16) && a->force_variant != OPSNN_VARIANT_PLAIN &&
+        !opsnn_force_plain()) {
+        OpsnnQmmArgs b = *a;
+        b.x2_scale_trunc = a->x2_scale_dtype == DT_U64 ||
+                           (a->x2_scale_len == 1 && !(a->bias && (a->bias_dtype == DT_BF16 || a->bias_dtype == DT_F32)));
+        return opsnnQmmInt8(&b, stream);
+    }
     return launch_tc_plain(*a, (hipStream_t)stream);
 }
 

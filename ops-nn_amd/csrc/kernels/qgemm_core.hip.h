@@ -39,9 +39,10 @@ struct QgemmParams {
     int64_t ldc;       // output row pitch in elements (N, or wider when this launch covers a column range)
     // MODE_I8 epilogue: out = cast(fp32(acc + ib[n]) * x2s[n] * x1s[m] + fb[n])
     const float* x1s;
-    const void* x2s;
+    const void* x2s;   // FLOAT / BF16, or UINT64 words whose low 32 bits are the fp32 scale
     int x2s_dt;
     int64_t x2s_len;
+    int x2s_trunc;     // keep only the upper 19 bits of the scale (always done for UINT64 words)
     // bias: int32 / 16-bit / fp32 for MODE_I8, fp32 for the MX modes
     const void* bias;
     int bias_dt;
@@ -439,7 +440,10 @@ __global__ __launch_bounds__(WGM* WGN * 64, MINWG) void qgemm_kernel(QgemmParams
             int64_t n = n0 + i;
             if (n >= p.N) n = p.N - 1;
             if constexpr (MODE == MODE_I8) {
-                sS2[i] = load_scalar_as_f32(p.x2s, p.x2s_dt, p.x2s_len == 1 ? 0 : n);
+                const int64_t si = p.x2s_len == 1 ? 0 : n;
+                float sv = p.x2s_dt == DT_U64 ? u2f((uint32_t)((const uint64_t*)p.x2s)[si]) : load_scalar_as_f32(p.x2s, p.x2s_dt, si);
+                if (p.x2s_trunc || p.x2s_dt == DT_U64) sv = u2f(f2u(sv) & 0xFFFFE000u);
+                sS2[i] = sv;
                 sIb[i] = has_ib ? ((const int32_t*)p.bias)[bz * p.bias_bs + n] : 0;
             }
             sFb[i] = has_fb ? load_scalar_as_f32(p.bias, p.bias_dt, bz * p.bias_bs + n) : -0.0f;

@@ -29,6 +29,7 @@ struct QmmI8Params {
     const void* x2s;
     int x2s_dt;
     int64_t x2s_len;
+    int x2s_trunc;
     const void* bias;
     int bias_dt;
     int64_t bias_bs;
@@ -57,7 +58,12 @@ __global__ void qmm_i8_plain(QmmI8Params p)
     }
     if (p.bias && p.bias_dt == DT_I32) acc += ((const int32_t*)p.bias)[bz * p.bias_bs + n];
     float v = (float)acc;
-    v = v * load_scalar_as_f32(p.x2s, p.x2s_dt, p.x2s_len == 1 ? 0 : n);
+    {
+        const int64_t si = p.x2s_len == 1 ? 0 : n;
+        float sv = p.x2s_dt == DT_U64 ? u2f((uint32_t)((const uint64_t*)p.x2s)[si]) : load_scalar_as_f32(p.x2s, p.x2s_dt, si);
+        if (p.x2s_trunc || p.x2s_dt == DT_U64) sv = u2f(f2u(sv) & 0xFFFFE000u);
+        v = v * sv;
+    }
     if (p.x1s) v = v * p.x1s[m];
     if (p.bias && p.bias_dt != DT_I32) v = v + load_scalar_as_f32(p.bias, p.bias_dt, bz * p.bias_bs + n);
     store_f32_as(p.out, p.out_dt, o, v);
@@ -89,7 +95,7 @@ extern "C" int opsnnQmmInt8(const OpsnnQmmArgs* a, void* stream)
     p.a = (const int8_t*)a->x1.ptr; p.a_rs = a->x1.row_stride; p.a_cs = a->x1.col_stride; p.a_bs = a->x1.batch_stride;
     p.b = (const int8_t*)a->x2.ptr; p.b_rs = a->x2.row_stride; p.b_cs = a->x2.col_stride; p.b_bs = a->x2.batch_stride;
     p.out = a->out; p.M = a->M; p.N = a->N; p.K = a->K;
-    p.x1s = (const float*)a->x1_scale; p.x2s = a->x2_scale; p.x2s_dt = a->x2_scale_dtype; p.x2s_len = a->x2_scale_len;
+    p.x1s = (const float*)a->x1_scale; p.x2s = a->x2_scale; p.x2s_dt = a->x2_scale_dtype; p.x2s_len = a->x2_scale_len; p.x2s_trunc = a->x2_scale_trunc;
     p.bias = a->bias; p.bias_dt = a->bias_dtype; p.bias_bs = a->bias_batch_stride; p.out_dt = a->out_dtype;
 
     // x2 stored N-major ([K, N] rows): relayout into the workspace as [N, K] first.
@@ -116,7 +122,7 @@ extern "C" int opsnnQmmInt8(const OpsnnQmmArgs* a, void* stream)
         QgemmParams g{};
         g.a = p.a; g.b = p.b; g.lda = p.a_rs; g.ldb = p.b_cs; g.a_bs = p.a_bs; g.b_bs = p.b_bs;
         g.out = p.out; g.M = p.M; g.N = p.N; g.ldc = p.N; g.KB = p.K;
-        g.x1s = p.x1s; g.x2s = p.x2s; g.x2s_dt = p.x2s_dt; g.x2s_len = p.x2s_len;
+        g.x1s = p.x1s; g.x2s = p.x2s; g.x2s_dt = p.x2s_dt; g.x2s_len = p.x2s_len; g.x2s_trunc = a->x2_scale_trunc;
         g.bias = p.bias; g.bias_dt = p.bias_dt; g.bias_bs = p.bias_bs;
         switch (variant) {
             case OPSNN_VARIANT_I8_256: return qgemm_launch<MODE_I8, 256, 256, 128, 2, 2, 2, 1>(g, a->batch, p.out_dt, st);
@@ -146,7 +152,7 @@ extern "C" int opsnnQmmInt8(const OpsnnQmmArgs* a, void* stream)
                 gb.N = p.N - na;
                 gb.b = g.b + na * g.ldb;
                 gb.out = (uint16_t*)g.out + na;
-                if (g.x2s_len != 1) gb.x2s = (const char*)g.x2s + na * (g.x2s_dt == DT_F32 ? 4 : 2);
+                if (g.x2s_len != 1) gb.x2s = (const char*)g.x2s + na * (g.x2s_dt == DT_U64 ? 8 : g.x2s_dt == DT_F32 ? 4 : 2);
                 if (g.bias) gb.bias = (const char*)g.bias + na * (g.bias_dt == DT_I32 || g.bias_dt == DT_F32 ? 4 : 2);
                 return qgemm_launch<MODE_I8, 128, 128, 128, 2, 2, 2, 1>(gb, 1, p.out_dt, st);
             }

@@ -44,7 +44,7 @@ class OpsnnQmmArgs(C.Structure):
         ("x1_scale_mat", OpsnnMat), ("x2_scale_mat", OpsnnMat),
         ("workspace", C.c_void_p), ("force_variant", C.c_int),
         ("x1_scale_len", C.c_int64), ("x2_offset", C.c_void_p), ("x2_offset_len", C.c_int64),
-        ("y_scale", C.c_void_p), ("y_scale_len", C.c_int64), ("x2_offset_mat", OpsnnMat),
+        ("y_scale", C.c_void_p), ("y_scale_len", C.c_int64), ("x2_offset_mat", OpsnnMat), ("x2_scale_trunc", C.c_int),
     ]
 
 

@@ -141,6 +141,12 @@ GPU_CASES = [
     (40, 96, 50, "i8", "f32", 1, "f32", "bf16", True, False, 0),      # fp32 bias: no truncation of the scale
     (40, 96, 50, "i8", "bf16", 1, None, "bf16", False, False, 0),
     (40, 96, 50, "i8", "f32", "N", "i32", "i32", False, False, 0),
+    # large enough for the MFMA tile kernel (int8 operands, 16-bit output), K-contiguous and N-contiguous x2
+    (128, 256, 192, "i8", "u64", "N", "i32", "f16", True, False, 0),
+    (100, 192, 136, "i8", "f32", 1, "i32", "bf16", True, False, 0),   # truncated per-tensor float scale
+    (128, 256, 192, "i8", "u64", 1, "i32", "bf16", False, False, 0),
+    (96, 320, 160, "i8", "f32", 1, "f32", "bf16", True, False, 0),    # fp32 bias: scale not truncated
+    (96, 320, 160, "i8", "bf16", "N", "bf16", "bf16", True, False, 0),
     (16, 32, 16, "e4m3", "f32", "N", "f32", "f16", False, True, 0),   # FP8E4M3..dynamic_tc_bias_float
     (16, 32, 16, "e5m2", "f32", "N", "f32", "bf16", False, True, 0),  # FP8E5M2..dynamic_tc_bias_float
     (37, 160, 48, "e4m3", "f32", 1, None, "bf16", True, True, 0),     # both scales one element: merged and truncated
