@@ -8,8 +8,9 @@
 // the matrix core its 32 K elements together with the e8m0 byte that scales exactly those 32 elements, so the
 // MX block size (32) and the hardware operand block coincide and no dequantised copy is ever formed.
 //
-// Fast path (qgemm_core.hip.h, MODE_MXFP4 / MODE_MXFP8): operands and scales K-contiguous, K % 128 == 0,
-// 16-bit output (fp4 with K % 512 == 0 takes 256-element K tiles, otherwise 128-element ones).  An N-contiguous x2 (data [K, N], scales [K/64, N, 2]) is first re-laid out into the
+// Fast paths: operands and scales K-contiguous, K % 128 == 0, 16-bit output.  fp4: qgemm_core.hip.h, MODE_MXFP4
+// (K % 512 == 0 takes 256-element K tiles, otherwise 128-element ones); fp8: the MX mode of the kernel in
+// qmm_fp8_block.hip.  An N-contiguous x2 (data [K, N], scales [K/64, N, 2]) is first re-laid out into the
 // workspace; everything else runs the plain kernel.
 #include "launch.h"
 #include "qgemm_core.hip.h"
@@ -51,17 +52,19 @@ uint64_t mx_workspace_bytes(const OpsnnQmmArgs& a)
     return data + align_up((uint64_t)a.N * ks * 2, 256) * snb;
 }
 
+int launch_mxfp8_mfma(const OpsnnQmmArgs& a, hipStream_t st);   // qmm_fp8_block.hip
+
 int launch_mx_mfma(const OpsnnQmmArgs& a0, hipStream_t st)
 {
     OpsnnQmmArgs a = a0;
     const bool fp4 = a.x1_dtype == DT_E2M1 && a.x2_dtype == DT_E2M1;
     const bool fp8 = a.x1_dtype == DT_E4M3 && a.x2_dtype == DT_E4M3;
     if (!fp4 && !fp8) return OPSNN_NOT_TAKEN;
-    // The 8-bit forms of the matrix instruction sum their 64 products with a reduced-width aligner (measured:
-    // mean error 1e-5 of sum|terms| per instruction).  Chained over all of K that exceeds the 16-bit output's own
-    // rounding, so MXFP8 takes the MFMA path only on request (OPSNN_VARIANT_MX_FP8_MFMA) until it gains the
-    // per-128-K fp32 promotion the block-scale kernel has; fp4 products are exact in that datapath.
-    if (fp8 && a.force_variant != OPSNN_VARIANT_MX_FP8_MFMA && a.force_variant != OPSNN_VARIANT_MX_128) return OPSNN_NOT_TAKEN;
+    // MXFP8 runs on the block kernel of qmm_fp8_block.hip in MX mode (16x16x128 instructions, 64 x 128 per wave, the
+    // pipeline tuned for the fp8 block-scale path); the 32x32x64 tile kernel stays available on request
+    // (OPSNN_VARIANT_MX_FP8_MFMA) for comparison.  The 8-bit forms of the matrix instruction sum their products with a
+    // reduced-width aligner (measured: mean error 1e-5 of sum|terms| per instruction); fp4 products are exact in that
+    // datapath.
     if (a.out_dtype != DT_BF16 && a.out_dtype != DT_F16) return OPSNN_NOT_TAKEN;
     if (a.bias && a.bias_dtype != DT_F32) return OPSNN_NOT_TAKEN;
     if (a.K % 128 != 0 || a.M * a.N < 64 * 64) return OPSNN_NOT_TAKEN;
@@ -119,8 +122,11 @@ int launch_mx_mfma(const OpsnnQmmArgs& a0, hipStream_t st)
         if (sc16) return qgemm_launch<MODE_MXFP4, 256, 256, 128, 2, 4, 2, 1>(g, a.batch, a.out_dtype, st);
         return qgemm_launch<MODE_MXFP4, 256, 256, 64, 2, 2, 4, 1>(g, a.batch, a.out_dtype, st);
     }
-    if (small || a.force_variant == OPSNN_VARIANT_MX_128) return qgemm_launch<MODE_MXFP8, 128, 128, 128, 2, 2, 2, 1>(g, a.batch, a.out_dtype, st);
-    return qgemm_launch<MODE_MXFP8, 256, 256, 128, 2, 2, 2, 1>(g, a.batch, a.out_dtype, st);
+    if (a.force_variant == OPSNN_VARIANT_MX_FP8_MFMA || a.force_variant == OPSNN_VARIANT_MX_128) {   // chained-K variants (tests)
+        if (small || a.force_variant == OPSNN_VARIANT_MX_128) return qgemm_launch<MODE_MXFP8, 128, 128, 128, 2, 2, 2, 1>(g, a.batch, a.out_dtype, st);
+        return qgemm_launch<MODE_MXFP8, 256, 256, 128, 2, 2, 2, 1>(g, a.batch, a.out_dtype, st);
+    }
+    return launch_mxfp8_mfma(a, st);
 }
 
 }  // namespace opsnn
