@@ -13,6 +13,8 @@ enum {
     OPSNN_VARIANT_I8_256_W8 = 5,  // int8 MFMA, 256x256 tile, 8 waves, BK 64, 4 stages
     OPSNN_VARIANT_I8_256_S4 = 6,  // int8 MFMA, 256x256 tile, 4 waves, BK 64, 4 stages
     OPSNN_VARIANT_I8_256_W8_K128 = 7,  // int8 MFMA, 256x256 tile, 8 waves, BK 128, 2 stages
+    OPSNN_VARIANT_I8_WIDE8 = 8,   // int8 MFMA, 4 waves with 128 x 16n sub-tiles, 256 x 32n tile, n = 8..11 (ids 8..11)
+    OPSNN_VARIANT_I8_WIDE11 = 11,
     OPSNN_VARIANT_MX_128 = 16,    // MX MFMA, 128x128 tile
     OPSNN_VARIANT_MX_FP8_MFMA = 17,  // MXFP8 on the MFMA path (reduced accumulation precision, see qmm_mx.hip)
 };

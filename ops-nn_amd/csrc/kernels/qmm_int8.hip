@@ -74,6 +74,9 @@ __global__ void qmm_i8_plain(QmmI8Params p)
 using namespace opsnn;
 
 extern "C" bool opsnn_force_plain();
+namespace opsnn {
+int launch_int8_wide(const QgemmParams& p, int fn, int64_t batch, int out_dt, hipStream_t st);   // qmm_int8_wide.hip
+}
 
 static int64_t cu_count()
 {
@@ -124,6 +127,10 @@ extern "C" int opsnnQmmInt8(const OpsnnQmmArgs* a, void* stream)
         g.out = p.out; g.M = p.M; g.N = p.N; g.ldc = p.N; g.KB = p.K;
         g.x1s = p.x1s; g.x2s = p.x2s; g.x2s_dt = p.x2s_dt; g.x2s_len = p.x2s_len; g.x2s_trunc = a->x2_scale_trunc;
         g.bias = p.bias; g.bias_dt = p.bias_dt; g.bias_bs = p.bias_bs;
+        if (variant >= OPSNN_VARIANT_I8_WIDE8 && variant <= OPSNN_VARIANT_I8_WIDE11) {
+            const int rc = launch_int8_wide(g, variant, a->batch, p.out_dt, st);
+            if (rc != OPSNN_NOT_TAKEN) return rc;
+        }
         switch (variant) {
             case OPSNN_VARIANT_I8_256: return qgemm_launch<MODE_I8, 256, 256, 128, 2, 2, 2, 1>(g, a->batch, p.out_dt, st);
             case OPSNN_VARIANT_I8_128: return qgemm_launch<MODE_I8, 128, 128, 128, 2, 2, 2, 1>(g, a->batch, p.out_dt, st);
@@ -139,10 +146,28 @@ extern "C" int opsnnQmmInt8(const OpsnnQmmArgs* a, void* stream)
         // columns (less than one round) go to 128x128 tiles, two workgroups per CU, in a second launch.
         const int64_t cus = cu_count();
         const int64_t tm = (p.M + 255) / 256, tn = (p.N + 255) / 256;
+        // Cost of a strategy in units of "one round of tiles, per 32 columns of tile width".  The four-wave kernel
+        // takes tiles of 256 x 32n columns, n = 8..11: the width whose tile count wastes the least of its last round
+        // wins (2048 x 11008: 256 tiles of 352 columns, one round, 11 units against 8 + 5 for the split below).
+        int64_t wide_cost = INT64_MAX;
+        int wide_fn = 0;
+        if (p.K % 128 == 0 && p.K >= 1024 && tm * tn * a->batch >= cus) {
+            for (int fn = 8; fn <= 11; fn++) {
+                const int64_t tiles = tm * ((p.N + 32 * fn - 1) / (32 * fn)) * a->batch;
+                const int64_t cost = (tiles + cus - 1) / cus * fn;
+                if (cost < wide_cost) { wide_cost = cost; wide_fn = fn; }
+            }
+        }
         if (p.K >= 1024 && tm * tn * a->batch >= cus && a->batch == 1) {
             const int64_t rounds = tm * tn / cus;
             const int64_t cols_a = rounds * cus / tm;            // column tiles in whole rounds
-            if (cols_a >= 1 && cols_a * tm * 8 >= rounds * cus * 7) {   // at least 7/8 of those rounds is filled
+            const bool split_ok = cols_a >= 1 && cols_a * tm * 8 >= rounds * cus * 7;   // at least 7/8 of those rounds is filled
+            const int64_t split_cost = split_ok ? rounds * 8 + (cols_a * 256 < p.N ? 5 : 0) : INT64_MAX;   // measured: the remainder launch costs 5/8 of a round
+            if (wide_fn && wide_cost <= split_cost) {
+                const int rc = launch_int8_wide(g, wide_fn, a->batch, p.out_dt, st);
+                if (rc != OPSNN_NOT_TAKEN) return rc;
+            }
+            if (split_ok) {
                 const int64_t na = cols_a * 256 < p.N ? cols_a * 256 : p.N;
                 QgemmParams ga = g;
                 ga.N = na;
@@ -156,6 +181,10 @@ extern "C" int opsnnQmmInt8(const OpsnnQmmArgs* a, void* stream)
                 if (g.bias) gb.bias = (const char*)g.bias + na * (g.bias_dt == DT_I32 || g.bias_dt == DT_F32 ? 4 : 2);
                 return qgemm_launch<MODE_I8, 128, 128, 128, 2, 2, 2, 1>(gb, 1, p.out_dt, st);
             }
+        }
+        if (wide_fn) {
+            const int rc = launch_int8_wide(g, wide_fn, a->batch, p.out_dt, st);
+            if (rc != OPSNN_NOT_TAKEN) return rc;
         }
         return qgemm_launch<MODE_I8, 256, 128, 64, 2, 2, 3, 2>(g, a->batch, p.out_dt, st);
     }

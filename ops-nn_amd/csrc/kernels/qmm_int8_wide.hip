@@ -1,0 +1,348 @@
+// int8 x int8 tile kernel with one wave per SIMD and a 256 x (32*FN) output tile, FN = 8..11.
+//
+// Why a second int8 tile kernel: a GEMM runs in rounds of one tile per CU, and with a fixed 256 x 256 tile a shape
+// such as 2048 x 11008 needs 1.34 rounds -- the last third of a round costs a whole one (or a second launch of small
+// tiles with its own prologue, epilogue and launch gap).  Here the tile WIDTH is a template parameter in steps of 32
+// columns, and the launcher picks the width whose tile count fills whole rounds: 11008 columns = 32 tiles of 352, times
+// 8 row tiles = 256 tiles = one round of 256 CUs.
+//
+// What makes a 256 x 352 tile possible is the register file: 256 x 352 int32 sums are 352 KB of the CU's 512 KB.  So the
+// workgroup is FOUR waves, one per SIMD, each with the SIMD's whole register file (512 registers per lane): a wave owns
+// 128 x (16*FN) outputs as 8 x FN fragments of 16 x 16 (v_mfma_i32_16x16x64_i8, two per 128-byte K tile and fragment
+// pair), i.e. up to 352 accumulator registers, 64 registers of x1 fragments held for the whole K tile, and the x2
+// fragments streaming through two sets of 8, each requested one fragment (16 MFMAs = 256 clocks) ahead.  A wave reads
+// (8 + FN) fragments from LDS for 16 * FN MFMAs -- less than half the LDS traffic per MFMA of the 8-wave kernels.
+//
+// With one wave per SIMD there is no partner wave to fill in while this one waits, so nothing may wait:
+//   - the loop is software-pipelined: the barrier sits in front of the last x2 fragment of a tile, and in the shadow of
+//     that fragment's 16 MFMAs the wave requests the next tile's first x2 fragment and its x1 fragments, each half of
+//     a fragment as soon as the last MFMA that reads the old half has been issued; the next tile then starts on the
+//     halves that came first (lgkmcnt counts, never "wait for everything");
+//   - the global -> LDS copies are written as inline assembly, because of what the compiler does with the builtin (see
+//     dma_copy16), and are spread over the first fragments of the tile instead of being issued in one burst;
+//   - two stages of (256 + 32*FN) x 128 bytes fill the LDS (155,648 of 163,840 bytes at FN = 11): the copies of tile
+//     kt+1 are issued during tile kt into the stage that the barrier at the end of tile kt-1 freed, and are waited
+//     for in front of the barrier at the end of tile kt.
+// Measured on 2048 x 4096 x 11008 (bf16 out): 90-92 us against 103 us for 256 x 256 tiles on 8192 columns plus a second
+// launch of 128 x 128 tiles on the remaining 2816; at 256 x 256 (FN = 8) it is level with the 8-wave kernel
+// (62-64 against 65 us on 2048 x 4096 x 8192, 540 against 560 us on 8192^3).
+//
+// Epilogue formula and its order of operations: the K-C / K-T golden, as in qgemm_core.hip.h
+// (matmul/quant_batch_matmul_v3/tests/assets/qbmmv3_kernel_golden.py): out = cast(fp32(acc + ib[n]) * x2s[n] * x1s[m] + fb[n]).
+#include "launch.h"
+#include "qgemm_core.hip.h"
+
+namespace opsnn {
+
+// acc += a (16 x 64 int8, rows = output columns) x b (64 x 16 int8), with the accumulator pinned to one register class.
+// The wave's sums outnumber the 256 accumulation registers; left to itself the compiler puts all of them in that class
+// and copies the overflow in and out around every instruction (244 copies per K tile at FN = 11).  Written out, the
+// first 64 fragments live in accumulation registers and the rest in ordinary vector registers, and nothing moves.
+// (The compiler does not see an MFMA here: dependent instructions are kept eight apart by the loop order, and the
+// epilogue waits out the write-to-read hazard itself.)
+template <bool AG>
+__device__ __forceinline__ void mfma_i8_16x16x64(v4i& c, const v4i a, const v4i b)
+{
+    if constexpr (AG) asm volatile("v_mfma_i32_16x16x64_i8 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+    else asm volatile("v_mfma_i32_16x16x64_i8 %0, %1, %2, %0" : "+v"(c) : "v"(a), "v"(b));
+}
+
+// 16-byte asynchronous copy global -> LDS, written out: lane l reads sbase + voff(l) and lands at lds_base + LDS_IMM + 16*l.
+// Through the builtin the compiler's wait-count pass sees an instruction that touches both memory paths and from then
+// on answers every dependency on an LDS read with a wait for ALL outstanding reads, including the ones issued a moment
+// ago for the next fragment; hidden from it, the pass counts exactly.  The copies' own completion is waited for
+// explicitly (vmcnt + barrier) wherever LDS is read.
+template <int LDS_IMM>
+__device__ __forceinline__ void dma_copy16(const int8_t* sbase, uint32_t voff, uint32_t lds_base)
+{
+    asm volatile("s_add_u32 m0, %0, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                 : : "s"(lds_base), "v"(voff), "s"(sbase), "n"(LDS_IMM) : "memory", "m0", "scc");
+}
+
+template <int FN, int OUT_DT>
+__global__ __launch_bounds__(256, 1) void qgemm_i8_wide_kernel(QgemmParams p, int tiles_m, int tiles_n)
+{
+    constexpr int NT = 256, BM = 256, TM = 128, FM = TM / 16, TN = 16 * FN, BN = 2 * TN, BK = 128, STAGES = 2;
+    constexpr int CPR = BK / 16, RPW = 16 / CPR;
+    constexpr int A_BYTES = BM * BK, B_BYTES = BN * BK, STAGE = A_BYTES + B_BYTES;
+    constexpr int RPI = NT / CPR;                 // 32 tile rows per copy instruction of the workgroup
+    constexpr int NA = BM / RPI, NB = BN / RPI;   // 8 and FN
+    constexpr int CPT = NA + NB;
+    static_assert(FN >= 2 && STAGES * CPT < 64, "copy counts must fit the wait counter");
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave >> 1, wn = wave & 1;
+
+    const uint32_t t = xcd_remap(blockIdx.x, (uint32_t)(tiles_m * tiles_n));
+    const int tm = (int)(t % (uint32_t)tiles_m), tn = (int)(t / (uint32_t)tiles_m);
+    const int64_t m0 = (int64_t)tm * BM, n0 = (int64_t)tn * BN;
+    const int64_t bz = blockIdx.y;
+    const int64_t lda = p.lda, ldb = p.ldb;
+    const int8_t* A = p.a + bz * p.a_bs + m0 * lda;
+    const int8_t* B = p.b + bz * p.b_bs + n0 * ldb;
+    const int KT = (int)(p.KB / BK);
+
+    // Copies: instruction i of the workgroup fills LDS chunks [i*NT, (i+1)*NT) of an operand, i.e. tile rows
+    // 32i .. 32i+31; this thread moves chunk (tid % 8) ^ key of row 32i + tid/8.  Rows past the matrix edge repeat the
+    // last valid row: they only feed outputs that are never stored.
+    const int crow = tid / CPR;
+    const int cchunk = (tid % CPR) ^ ((crow / RPW) & (CPR - 1));
+    const int a_rows = (int)((p.M - m0) < BM ? (p.M - m0) : BM);
+    const int b_rows = (int)((p.N - n0) < BN ? (p.N - n0) : BN);
+    uint32_t a_off[NA], b_off[NB];
+#pragma unroll
+    for (int i = 0; i < NA; i++) {
+        int r = i * RPI + crow;
+        r = r < a_rows ? r : a_rows - 1;
+        a_off[i] = (uint32_t)(r * lda + cchunk * 16);
+    }
+#pragma unroll
+    for (int i = 0; i < NB; i++) {
+        int r = i * RPI + crow;
+        r = r < b_rows ? r : b_rows - 1;
+        b_off[i] = (uint32_t)(r * ldb + cchunk * 16);
+    }
+    auto scalar_ptr = [](const int8_t* q) -> const int8_t* {   // a wave-uniform pointer, held in scalar registers
+        const uint64_t u = (uint64_t)q;
+        const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)u), hi = __builtin_amdgcn_readfirstlane((uint32_t)(u >> 32));
+        return (const int8_t*)(((uint64_t)hi << 32) | lo);
+    };
+    const uint32_t lds0 = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)smem) + wave * 1024;
+    auto issue_piece = [&](int kt, int stage, auto idx_c) {
+        constexpr int idx = decltype(idx_c)::value;
+        const uint32_t sS = lds0 + stage * STAGE;
+        if constexpr (idx < NA) dma_copy16<idx * NT * 16>(scalar_ptr(A + (int64_t)kt * BK), a_off[idx], sS);
+        else dma_copy16<A_BYTES + (idx - NA) * NT * 16>(scalar_ptr(B + (int64_t)kt * BK), b_off[idx - NA], sS);
+    };
+    auto for_copies = [&](auto&& f) {   // f(integral_constant<int, c>) for c = 0 .. CPT-1
+        [&]<int... C>(std::integer_sequence<int, C...>) { (f(std::integral_constant<int, C>{}), ...); }(std::make_integer_sequence<int, CPT>{});
+    };
+    auto issue_tile = [&](int kt) {
+        for_copies([&](auto c) { issue_piece(kt, kt % STAGES, c); });
+    };
+
+    v4i acc[FN][FM];
+#pragma unroll
+    for (int i = 0; i < FN; i++)
+#pragma unroll
+        for (int j = 0; j < FM; j++) acc[i][j] = v4i{0, 0, 0, 0};
+
+    // Operand fragment of the 16x16x64 instruction pair, lane (row = lane%16, q = lane/16): bytes [16q, 16q+16) of the
+    // row's 128 bytes of K for the first instruction, [64+16q, +16) for the second.  (K is the contraction index: any
+    // assignment of K to lanes is right as long as both operands use the same one.)
+    const int frow = lane & 15, fq = lane >> 4;
+    const int key = (frow / RPW) & (CPR - 1);
+    const int ch0 = (fq ^ key) << 4, ch1 = ((4 + fq) ^ key) << 4;
+    const int a_rowbase = (wm * TM + frow) * BK;
+    const int b_rowbase = A_BYTES + (wn * TN + frow) * BK;
+    auto load_lo = [&](const char* st, int rowbase) -> v4i { return *(const v4i*)(st + rowbase + ch0); };
+    auto load_hi = [&](const char* st, int rowbase) -> v4i { return *(const v4i*)(st + rowbase + ch1); };
+
+    // The copies of tile kt+1 are issued evenly over the first SPREAD fragments of tile kt (into the stage that the
+    // barrier at the end of tile kt-1 freed) and are waited for at the end of tile kt.  Issued in one burst they fill
+    // the memory pipeline's queue and the wave -- the only one on its SIMD -- stalls in front of its MFMAs:
+    // measured 102.6 us (burst behind the last fragment) against 90.4 us (spread) for 2048 x 4096 x 11008.
+    constexpr int SPREAD = 4;
+    static_assert(SPREAD <= FN, "the copies are issued within one tile");
+    issue_tile(0);
+    wait_vmcnt<0>();
+    __builtin_amdgcn_s_barrier();
+    // Fragments are kept as halves (lo: the first instruction's 64 bytes of K, hi: the second's), so that a half can be
+    // replaced as soon as its last reader has been issued.
+    // The x2 fragments alternate between fb[0] and fb[1]; fragment 0 of the NEXT tile is requested into fb[FN % 2].  For
+    // odd FN that is fb[1], and the tile starts by moving it to fb[0] (eight register moves per K tile).
+    v4i fal[FM], fah[FM], fbl[2], fbh[2];
+    fbl[FN & 1] = load_lo(smem, b_rowbase);
+    fbh[FN & 1] = load_hi(smem, b_rowbase);
+#pragma unroll
+    for (int j = 0; j < FM; j++) fal[j] = load_lo(smem, a_rowbase + j * 16 * BK);
+#pragma unroll
+    for (int j = 0; j < FM; j++) fah[j] = load_hi(smem, a_rowbase + j * 16 * BK);
+
+    for (int kt = 0; kt < KT; kt++) {
+        const char* st = smem + (kt & 1) * STAGE;
+        const char* stn = smem + ((kt + 1) & 1) * STAGE;
+        // past the end the copies repeat the last tile (into a stage nobody reads any more): no branches in the loop
+        const int ktc = kt + 1 < KT ? kt + 1 : KT - 1;
+        const int cstage = (kt + 1) & 1;
+        auto spread_copies = [&](int slot) {   // slot = index within the tile of the MFMA just issued
+            for_copies([&](auto c) {
+                if ((decltype(c)::value * SPREAD * 16) / CPT == slot) issue_piece(ktc, cstage, c);
+            });
+        };
+#pragma unroll
+        for (int i = 0; i < FN; i++) {
+            if (i + 1 < FN) {
+                if (i == 0) {
+                    // Outstanding, oldest first: this tile's first x2 fragment, the lo halves of its x1 fragments, their hi
+                    // halves.  The first eight instructions need all but the hi halves.
+                    __builtin_amdgcn_s_waitcnt(0xc07f | (FM << 8));
+                    if (FN & 1) { fbl[0] = fbl[1]; fbh[0] = fbh[1]; }
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+                fbl[(i + 1) & 1] = load_lo(st, b_rowbase + (i + 1) * 16 * BK);
+                fbh[(i + 1) & 1] = load_hi(st, b_rowbase + (i + 1) * 16 * BK);
+                __builtin_amdgcn_sched_barrier(0);
+                if (i > 0) __builtin_amdgcn_s_waitcnt(0xc07f | (2 << 8));   // lgkmcnt: all but the two reads just issued
+            } else {
+                // every read of tile kt by this wave has been issued; its own copies of tile kt+1 must have landed
+                wait_vmcnt<0>();
+                wait_lgkmcnt0();
+                __builtin_amdgcn_s_barrier();
+                __builtin_amdgcn_sched_barrier(0);
+                fbl[(i + 1) & 1] = load_lo(stn, b_rowbase);
+                fbh[(i + 1) & 1] = load_hi(stn, b_rowbase);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            const v4i blo = fbl[i & 1], bhi = fbh[i & 1];
+            // the two instructions of a fragment pair are eight instructions apart: no back-to-back dependent MFMAs
+#pragma unroll
+            for (int j = 0; j < FM; j++) {
+                if (i * FM + j < 64) mfma_i8_16x16x64<true>(acc[i][j], blo, fal[j]);
+                else mfma_i8_16x16x64<false>(acc[i][j], blo, fal[j]);
+                __builtin_amdgcn_sched_barrier(0);
+                spread_copies(i * 16 + j);
+                if (i == FN - 1) fal[j] = load_lo(stn, a_rowbase + j * 16 * BK);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            if (i == 0) {   // now the hi halves: all but the two reads issued at the top of the tile
+                __builtin_amdgcn_s_waitcnt(0xc07f | (2 << 8));
+                __builtin_amdgcn_sched_barrier(0);
+            }
+#pragma unroll
+            for (int j = 0; j < FM; j++) {
+                if (i * FM + j < 64) mfma_i8_16x16x64<true>(acc[i][j], bhi, fah[j]);
+                else mfma_i8_16x16x64<false>(acc[i][j], bhi, fah[j]);
+                __builtin_amdgcn_sched_barrier(0);
+                spread_copies(i * 16 + 8 + j);
+                if (i == FN - 1) {
+                    fah[j] = load_hi(stn, a_rowbase + j * 16 * BK);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            }
+        }
+    }
+    wait_lgkmcnt0();   // the reads and copies past the last tile land before LDS is reused
+    wait_vmcnt<0>();
+    asm volatile("s_nop 15\n\ts_nop 15");   // the last MFMAs' results must be written before ordinary instructions read them
+    __syncthreads();   // every wave is done with the operand stages
+
+    // Epilogue.  acc[i][j][r] is out[m = m_base + 16j + lane%16][n = n_base + 16i + 4*(lane/16) + r].  Per-row and
+    // per-column terms are first widened to fp32 in LDS (absent terms are the neutral elements 1.0f, 0 and -0.0f).
+    float* sS2 = (float*)smem;
+    float* sFb = sS2 + BN;
+    int32_t* sIb = (int32_t*)(sFb + BN);
+    float* sS1 = (float*)(sIb + BN);
+    {
+        const bool has_ib = p.bias && p.bias_dt == DT_I32;
+        const bool has_fb = p.bias && p.bias_dt != DT_I32;
+        for (int i = tid; i < BN; i += NT) {
+            int64_t n = n0 + i;
+            if (n >= p.N) n = p.N - 1;
+            const int64_t si = p.x2s_len == 1 ? 0 : n;
+            float sv = p.x2s_dt == DT_U64 ? u2f((uint32_t)((const uint64_t*)p.x2s)[si]) : load_scalar_as_f32(p.x2s, p.x2s_dt, si);
+            if (p.x2s_trunc || p.x2s_dt == DT_U64) sv = u2f(f2u(sv) & 0xFFFFE000u);
+            sS2[i] = sv;
+            sIb[i] = has_ib ? ((const int32_t*)p.bias)[bz * p.bias_bs + n] : 0;
+            sFb[i] = has_fb ? load_scalar_as_f32(p.bias, p.bias_dt, bz * p.bias_bs + n) : -0.0f;
+        }
+        for (int i = tid; i < BM; i += NT) {
+            int64_t m = m0 + i;
+            if (m >= p.M) m = p.M - 1;
+            sS1[i] = p.x1s ? p.x1s[m] : 1.0f;
+        }
+    }
+    __syncthreads();
+    // Results leave through LDS: each wave parks one 16 x TN block in a private patch and reads it back row-wise, so
+    // that a store instruction writes runs of whole rows (16 bytes per lane, TN/8 lanes per row).
+    typedef v4us __attribute__((may_alias)) v4us_a;
+    typedef v4i __attribute__((may_alias)) v4i_a;
+    constexpr int EP_PITCH = TN * 2 + 16;
+    constexpr int EP_BASE = (3 * BN + BM) * 4;
+    static_assert(EP_BASE + 4 * 16 * EP_PITCH <= STAGES * STAGE, "epilogue staging fits in the operand stages");
+    char* ep = smem + EP_BASE + wave * (16 * EP_PITCH);
+    constexpr int LPR = TN / 8;                     // lanes per row when every lane moves 16 bytes
+    constexpr int PASSES = (16 * LPR + 63) / 64;
+    uint16_t* out = (uint16_t*)p.out + bz * p.M * p.ldc;
+    const bool vec_ok = (p.ldc % 8) == 0 && ((uintptr_t)p.out % 16) == 0;
+#pragma unroll
+    for (int j = 0; j < FM; j++) {
+        const float s1 = sS1[wm * TM + j * 16 + frow];
+#pragma unroll
+        for (int i = 0; i < FN; i++) {
+            const int nw = i * 16 + 4 * fq;   // column inside the wave's sub-tile
+            const int nl = wn * TN + nw;
+            const v4f fbv = *(const v4f*)(sFb + nl);
+            const v4f s2 = *(const v4f*)(sS2 + nl);
+            const v4i ib = *(const v4i*)(sIb + nl);
+            v4f v;
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                float tv = (float)(acc[i][j][e] + ib[e]);
+                tv = tv * s2[e];
+                tv = tv * s1;
+                v[e] = tv + fbv[e];
+            }
+            *(v4us_a*)(ep + frow * EP_PITCH + nw * 2) = pack4_b16<OUT_DT>(v);
+        }
+        // this wave's 16 x TN block is complete in its patch (LDS operations of one wave complete in order)
+#pragma unroll
+        for (int r = 0; r < PASSES; r++) {
+            const int idx = r * 64 + lane;
+            const int row = idx / LPR, ec = idx % LPR;
+            if (idx < 16 * LPR) {
+                const v4i o = *(const v4i_a*)(ep + row * EP_PITCH + ec * 16);
+                const int64_t m = m0 + wm * TM + j * 16 + row;
+                const int64_t n = n0 + wn * TN + ec * 8;
+                if (m < p.M) {
+                    if (vec_ok && n + 7 < p.N) {
+                        *(v4i*)(out + m * p.ldc + n) = o;
+                    } else {
+                        const uint16_t* oe = (const uint16_t*)&o;
+#pragma unroll
+                        for (int e = 0; e < 8; e++)
+                            if (n + e < p.N) out[m * p.ldc + n + e] = oe[e];
+                    }
+                }
+            }
+        }
+    }
+}
+
+template <int FN, int OUT_DT>
+static int launch_wide_one(const QgemmParams& p, int64_t batch, hipStream_t st)
+{
+    constexpr int BM = 256, BN = 32 * FN, BK = 128;
+    const int tiles_m = (int)((p.M + BM - 1) / BM), tiles_n = (int)((p.N + BN - 1) / BN);
+    const size_t lds = (size_t)2 * (BM + BN) * BK;
+    auto k = qgemm_i8_wide_kernel<FN, OUT_DT>;
+    static bool attr_set = false;   // per instantiation; benign if two threads both set it
+    if (!attr_set) {
+        hipError_t e = hipFuncSetAttribute((const void*)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return (int)e;
+        attr_set = true;
+    }
+    hipLaunchKernelGGL(k, dim3((unsigned)(tiles_m * tiles_n), (unsigned)batch), dim3(256), lds, st, p, tiles_m, tiles_n);
+    return (int)hipGetLastError();
+}
+
+// Tile width 32 * fn columns, fn = 8..11.  Needs what the int8 fast path needs (K-contiguous 16-byte aligned operands,
+// 16-bit output) and K % 128 == 0.
+int launch_int8_wide(const QgemmParams& p, int fn, int64_t batch, int out_dt, hipStream_t st)
+{
+    if (p.KB % 128 != 0 || p.KB < 128) return OPSNN_NOT_TAKEN;
+    if (out_dt != DT_BF16 && out_dt != DT_F16) return OPSNN_NOT_TAKEN;
+    const bool bf = out_dt == DT_BF16;
+    switch (fn) {
+        case 8: return bf ? launch_wide_one<8, DT_BF16>(p, batch, st) : launch_wide_one<8, DT_F16>(p, batch, st);
+        case 9: return bf ? launch_wide_one<9, DT_BF16>(p, batch, st) : launch_wide_one<9, DT_F16>(p, batch, st);
+        case 10: return bf ? launch_wide_one<10, DT_BF16>(p, batch, st) : launch_wide_one<10, DT_F16>(p, batch, st);
+        case 11: return bf ? launch_wide_one<11, DT_BF16>(p, batch, st) : launch_wide_one<11, DT_F16>(p, batch, st);
+        default: return OPSNN_NOT_TAKEN;
+    }
+}
+
+}  // namespace opsnn

@@ -14,7 +14,7 @@ import oracle_api as orc
 # very same bench command, each scaled by what the counter reads for a byte transpose of known size; the runs and the
 # figures are in profiles/<kernel>_<workload>.txt.  Keyed by (config, M of the weight-only configs).
 MEASURED_TRAFFIC = {
-    (2, None): 135.3e6, (4, None): 824.0e6, (5, None): 1807.1e6,
+    (2, None): 102.0e6, (4, None): 824.0e6, (5, None): 1807.1e6,
     (3, 1): 67.2e6, (3, 16): 69.2e6, (1, None): 9.2e6,
 }
 
@@ -46,7 +46,7 @@ def _cores():
 class Config2(Workload):
     """aclnnQuantMatmulV5, int8 x int8, per-token x per-channel fp32 scales, bf16 bias and output."""
     peak_key, dtype = "int8", "int8"
-    kernel = "qgemm_kernel<int8, 256x256x128> on the columns that fill whole rounds + qgemm_kernel<int8, 128x128x128> on the rest (the two launches of one step, timed together)"
+    kernel = "qgemm_i8_wide_kernel<FN=11> (256 x 352 tiles, one round of 256 workgroups)"
 
     def __init__(self, m, args, M=2048, K=4096, N=11008):
         self.m, self.M, self.K, self.N = m, M, K, N
@@ -155,7 +155,7 @@ class Config4(Workload):
 class Config5(Workload):
     """aclnnQuantMatmulV5, MXFP4 (e2m1 with e8m0 scale per 32 K), batch 8, bf16 output."""
     peak_key, dtype = "fp4", "fp4_e2m1"
-    kernel = "qgemm_kernel<mxfp4, 256x256x64B>"
+    kernel = "qgemm_kernel<mxfp4, 256x256x128B>"
 
     def __init__(self, m, args, B=8, M=4096, K=8192, N=8192):
         self.m, self.B, self.M, self.K, self.N = m, B, M, K, N
@@ -218,7 +218,7 @@ class ConfigWQ(Workload):
             self.dtype, lo, hi = "f16 (int4 weights)", 0.005, 0.02
             name = "config3: aclnnWeightQuantBatchMatmulV2 W4A16 per-group(128) fp16 decode"
         self.M, self.K, self.N, self.group = M, K, N, group
-        self.kernel = "wqmm_resx_kernel" if (config == 3 and M <= 3) else "wqmm_stream_kernel"
+        self.kernel = "wqmm_resx_kernel" if (config == 3 and M <= 3) else ("wqmm_rows_kernel" if M > 64 else "wqmm_stream_kernel")
         self.inp = cases.make_wq_inputs(m, M, K, N, 0, x_dt, w_dt, group, self.packed, off, None, lo, hi)
         inp = self.inp
         self.ncopies = 1

@@ -71,10 +71,11 @@ def test_batched(gpu):
     _check_equal(got, want, "batched K-C")
 
 
-@pytest.mark.parametrize("variant", [1, 2, 3, 4, 5, 6])
+@pytest.mark.parametrize("variant", [1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11])
 def test_every_kernel_variant_and_int32_accumulators(gpu, variant):
     """Each kernel variant (1 plain, 2 MFMA 256x256, 3 MFMA 128x128,
-    4 MFMA 256x128 three-stage, 5 MFMA 256x256 eight-wave) through the thin launcher ABI.
+    4 MFMA 256x128 three-stage, 5-7 MFMA 256x256 eight-wave, 8-11 four-wave tiles of 256 x 32n columns) through the
+    thin launcher ABI.
     With unit scales and no bias the fp32 epilogue is the identity on |acc| < 2^24, which exposes the raw
     int32 accumulators: K = 512 keeps |acc| <= 512*127*127 < 2^24."""
     m = gpu
@@ -101,6 +102,31 @@ def test_every_kernel_variant_and_int32_accumulators(gpu, variant):
         assert m.lib().opsnnQmmInt8(C.byref(a), None) == 0
         m.check(m.lib().aclrtSynchronizeDevice(), "sync")
         _check_equal(out32.to_host(np.int32, (M, N)), acc, "int32 accumulators")
+
+
+@pytest.mark.parametrize("variant", [8, 9, 10, 11])
+@pytest.mark.parametrize("M,K,N,batch,bias_dt,out_dt", [
+    (300, 384, 1000, 1, "bf16", "bf16"),    # ragged rows and columns, three K tiles
+    (512, 128, 704, 1, "i32", "f16"),       # one K tile, int32 bias
+    (256, 1024, 352, 2, "f32", "bf16"),     # batched, one tile of 352 columns
+    (65, 256, 96, 1, None, "bf16"),         # far smaller than one tile
+])
+def test_wide_tile_variants_full_epilogue(gpu, variant, M, K, N, batch, bias_dt, out_dt):
+    """The four-wave kernel with 256 x 32n tiles (n = variant): per-token and per-channel scales, every bias type,
+    ragged edges and batches, bit-exact against the oracle."""
+    m = gpu
+    dt = {"bf16": m.ACL_BF16, "f16": m.ACL_FLOAT16, "f32": m.ACL_FLOAT, "i32": m.ACL_INT32, None: None}
+    print(f"case int8 wide variant {variant} M={M} K={K} N={N} batch={batch} bias={bias_dt} out={out_dt}", flush=True)
+    inp = cases.make_qmm_int8_inputs(m, M, K, N, variant * 7 + M, dt[bias_dt], True, batch=batch)
+    want, _ = cases.oracle_qmm_int8(m, inp, M, K, N, True, dt[out_dt])
+    d = {k: m.DeviceBuffer(host=v) for k, v in inp.items() if isinstance(v, np.ndarray)}
+    out = m.DeviceBuffer(batch * M * N * 2)
+    out.fill(0xFF)
+    a = cases.qmm_args_int8(m, d, M, K, N, batch, True, out.ptr, dt[out_dt], m.ACL_FLOAT, N, dt[bias_dt], variant=variant)
+    rc = m.lib().opsnnQmmInt8(C.byref(a), None)
+    assert rc == 0, rc
+    m.check(m.lib().aclrtSynchronizeDevice(), "sync")
+    _check_equal(out.to_host(np.uint16, (batch, M, N)), want, f"wide variant {variant}")
 
 
 def test_config2_full_size_on_sampled_rows(gpu):
