@@ -149,6 +149,18 @@ __device__ __forceinline__ void async_copy16(const void* g, void* lds)
                                      (__attribute__((address_space(3))) void*)lds, 16, 0, 0);
 }
 
+// The same copy written out.  Through the builtin the compiler's wait-count pass sees an instruction that touches both
+// memory paths, and while one is outstanding it answers every dependency on a global load or an LDS read with a wait
+// for ALL outstanding operations of that kind (vmcnt(0) / lgkmcnt(0)) -- which empties a prefetch ring of ordinary
+// global loads every time a copy is in flight.  Hidden from the pass, those loads are counted exactly; since the
+// hardware counter also counts the hidden copies, the computed waits are at worst stricter than needed, never laxer.
+// The caller waits for the copies themselves explicitly (wait_vmcnt + barrier before the LDS data is read).
+__device__ __forceinline__ void async_copy16_uncounted(const void* g, void* lds)
+{
+    const uint32_t l = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(const __attribute__((address_space(3))) void*)lds);
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" : : "s"(l), "v"(g) : "memory", "m0");
+}
+
 // Workgroup ids are dealt round-robin over the 8 XCDs; give each XCD (own L2) a contiguous
 // range of logical tile ids so that neighbouring tiles share operand panels in one L2.
 __device__ __forceinline__ uint32_t xcd_remap(uint32_t wg, uint32_t total)

@@ -408,7 +408,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void w
     auto issue_x = [&](int slab) {
         char* dst = sx + (slab & 1) * XBUF + wave * 1024;
 #pragma unroll
-        for (int it = 0; it < XITEMS; it++) async_copy16(xsrc[it] + (int64_t)slab * KX, dst + it * NT * 16);
+        for (int it = 0; it < XITEMS; it++) async_copy16_uncounted(xsrc[it] + (int64_t)slab * KX, dst + it * NT * 16);
     };
     // LDS byte offset of this lane's column operand inside a buffer, per 16-row block of x, at K step 0 (the lane's
     // weights cover k = g*KPL .. +KPL of the chunk, step s the 8 at 8s); step s is s pieces further on, which the
