@@ -306,10 +306,13 @@ static bool stream_eligible(WqParams& p, WqStreamOpts& o)
     o.resx = !no_resx && p.M <= 16 && nch % 4 == 0 && (p.M + 1) * (p.K * 2 + 16) <= 65536;
     o.resx_vscale = o.resx && p.group == KC && p.s_rs == 1 && p.s_cs % 8 == 0 && (nch / 4) % 8 == 0 &&
                     (uintptr_t)p.scale % 16 == 0 && (!p.offset || (uintptr_t)p.offset % 16 == 0);
-    // more than 64 rows: two weight blocks per wave share every x fragment, up to 128 rows per pass over the weights
+    // more than 48 rows: two weight blocks per wave share every x fragment, up to 128 rows per pass over the weights
     // (needs whole groups of chunks in flight and whole wave tiles of columns)
     static const bool no_rows = [] { const char* e = getenv("OPSNN_WQ_NO_ROWS"); return e && e[0] == '1'; }();
-    o.rows = !no_rows && p.M > 64 && nch % 8 == 0 && p.N % 32 == 0 && p.N >= 256;
+    // (measured on 8192 x 28672 int4: 16 rows 43 us on the streaming kernel against 55 on this one, 32 rows 53 / 68,
+    // 48 rows 69 / 70, 64 rows 82 / 70, 128 rows 105; OPSNN_WQ_ROWS_MIN moves the switch for tuning)
+    static const int rows_min = [] { const char* e = getenv("OPSNN_WQ_ROWS_MIN"); return e ? atoi(e) : 49; }();
+    o.rows = !no_rows && p.M >= rows_min && nch % 8 == 0 && p.N % 32 == 0 && p.N >= 256;
     return true;
 }
 

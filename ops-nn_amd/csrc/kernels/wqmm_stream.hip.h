@@ -786,7 +786,7 @@ struct WqStreamOpts {
     bool resx, resx_vscale;   // whole-x-in-LDS kernel eligible, and with vector scale loads
 };
 
-// One row slab (p.m_rows <= 64, or <= 128 with o.rows) of one dtype pair; defined once per pair in its own translation unit.
+// One row slab (p.m_rows <= 128 with o.rows, else <= 64) of one dtype pair; defined once per pair in its own translation unit.
 template <int XDT, int WBITS>
 int launch_wq_stream(const WqParams& p, const WqStreamOpts& o, hipStream_t st);
 
@@ -813,6 +813,8 @@ int launch_wq_stream(const WqParams& p, const WqStreamOpts& o, hipStream_t st);
         }                                                                                                           \
         if (o.rows && p.m_rows > 64) return o.has_off ? launch_rows_one<XDT, WBITS, 8, 2, 4, 2, true>(p, st)              \
                                                       : launch_rows_one<XDT, WBITS, 8, 2, 4, 2, false>(p, st);            \
+        if (o.rows) return o.has_off ? launch_rows_one<XDT, WBITS, 4, 2, 4, 2, true>(p, st)                               \
+                                     : launch_rows_one<XDT, WBITS, 4, 2, 4, 2, false>(p, st);                             \
         if (o.ksplit && p.m_rows <= 16) return wq_stream_off<1, 4, 4, false>(p, o.has_off, st);                     \
         if (p.m_rows <= 16) return wq_stream_mb<1>(p, o, st);                                                       \
         if (p.m_rows <= 32) return wq_stream_mb<2>(p, o, st);                                                       \

@@ -218,7 +218,7 @@ class ConfigWQ(Workload):
             self.dtype, lo, hi = "f16 (int4 weights)", 0.005, 0.02
             name = "config3: aclnnWeightQuantBatchMatmulV2 W4A16 per-group(128) fp16 decode"
         self.M, self.K, self.N, self.group = M, K, N, group
-        self.kernel = "wqmm_resx_kernel" if (config == 3 and M <= 3) else ("wqmm_rows_kernel" if M > 64 else "wqmm_stream_kernel")
+        self.kernel = "wqmm_resx_kernel" if (config == 3 and M <= 3) else ("wqmm_rows_kernel" if M > 48 else "wqmm_stream_kernel")
         self.inp = cases.make_wq_inputs(m, M, K, N, 0, x_dt, w_dt, group, self.packed, off, None, lo, hi)
         inp = self.inp
         self.ncopies = 1

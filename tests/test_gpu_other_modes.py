@@ -158,7 +158,9 @@ def test_mx_batched(gpu, M, K, N, batch):
     (16, 4096, 256, "bf16", "i8", 0, True, False, None),
     (1, 4096, 200, "f16", "i4", 128, True, True, "f16"),
     (11, 2048, 64, "f16", "i8", 0, False, True, None),
-    # ... many rows (several weight blocks per wave share each x fragment): 33..64 rows, 65..128, and two passes
+    # ... many rows (several weight blocks per wave share each x fragment): 49..64 rows, 65..128, and two passes
+    (50, 2048, 288, "bf16", "i4", 128, True, False, "bf16"),   # 49..64 rows: the 64-row instance, ragged row count
+    (64, 1024, 256, "f16", "i8", 64, True, True, None),
     (100, 2048, 512, "f16", "i4", 128, True, True, None),
     (128, 1024, 256, "f16", "i8", 64, True, True, "f16"),
     (200, 2048, 320, "bf16", "i4", 256, True, True, None),
