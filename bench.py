@@ -34,6 +34,8 @@ def main():
     ap.add_argument("--config", type=int, default=2)
     ap.add_argument("--m", type=int, default=None, help="M for config 3 (1, 16, 64 or 256)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--int8-range", type=int, default=None,
+                    help="config 2: operands uniform in [-R, R] (default: the full int8 range, the most power-hungry data)")
     ap.add_argument("--cold", action="store_true", help="rotate through weight copies larger than the 256 MB cache")
     ap.add_argument("--calib-copy", action="store_true",
                     help="also run a byte transpose of an 8192x8192 matrix (64 MiB read, 64 MiB written) three times "

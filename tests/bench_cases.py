@@ -52,9 +52,11 @@ class Config2(Workload):
         self.m, self.M, self.K, self.N = m, M, K, N
         self.packed = args.layout == "packed"
         self.inp = cases.make_qmm_int8_inputs(m, M, K, N, 0, m.ACL_BF16, self.packed)
-        if os.environ.get("OPSNN_BENCH_ZERO"):   # experiment: data-dependent power
-            self.inp["x1"][:] = 0
-            self.inp["x2"][:] = 0
+        r = getattr(args, "int8_range", None)
+        if r:   # operands uniform in [-r, r] instead of the full int8 range (the sustained clock depends on the data)
+            rng = np.random.default_rng(1)
+            self.inp["x1"] = rng.integers(-r, r + 1, size=self.inp["x1"].shape, dtype=np.int8)
+            self.inp["x2"] = rng.integers(-r, r + 1, size=self.inp["x2"].shape, dtype=np.int8)
         self.d = {k: m.DeviceBuffer(host=v) for k, v in self.inp.items() if isinstance(v, np.ndarray)}
         self.d_out = m.DeviceBuffer(M * N * 2)
         self.t_x1 = m.Tensor((M, K), m.ACL_INT8, self.d["x1"])
