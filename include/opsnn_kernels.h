@@ -63,7 +63,7 @@ typedef struct {
     void* workspace;       /* opsnnQmmWorkspace() bytes, or NULL if that is 0 */
     int force_variant;     /* 0 = selector decides; >0 pins a kernel variant (tuning and tests) */
     /* per-tensor / per-channel family (opsnnQmmTc) */
-    int64_t x1_scale_len;  /* 1: one fp32 scale for all of x1 ("double scale" with fp8 inputs); 0 if x1_scale is NULL */
+    int64_t x1_scale_len;  /* opsnnQmmTc: 1 = one fp32 scale for all of x1 ("double scale" with fp8 inputs), M = one per row (fp8 K-C / K-T); 0 if x1_scale is NULL */
     const float* x2_offset;/* fp32 [1] or [N], int8 output only; NULL = take it from the packed 64-bit scale */
     int64_t x2_offset_len;
     /* K-group family (opsnnQmmGroup) */

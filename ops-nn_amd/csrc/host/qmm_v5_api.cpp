@@ -659,7 +659,7 @@ extern "C" aclnnStatus aclnnQuantMatmulV5GetWorkspaceSize(const aclTensor* x1, c
     } else if ((c.int8_in() && in_list(c.x2s.dtype, {ACL_FLOAT, ACL_BF16, ACL_UINT64}) &&
                 in_list(c.out.dtype, {ACL_BF16, ACL_FLOAT16, ACL_INT8, ACL_INT32}) && !c.x1s.present) ||
                (c.fp8_in() && in_list(c.x2s.dtype, {ACL_FLOAT, ACL_BF16, ACL_UINT64}) && in_list(c.out.dtype, {ACL_BF16, ACL_FLOAT16, ACL_FLOAT}) &&
-                (!c.x1s.present || (c.x1s.dtype == ACL_FLOAT && c.x1s.rank() == 1 && c.x1s.dim(0) == 1)))) {
+                (!c.x1s.present || (c.x1s.dtype == ACL_FLOAT && c.x1s.rank() == 1 && (c.x1s.dim(0) == 1 || c.x1s.dim(0) == c.M))))) {
         // per-tensor / per-channel family: qbmmv3_kernel_golden.py:390-513
         ex->kind = OpKind::QmmTc; mode = 3;
         a.x2_scale_len = c.x2s.dim(0);

@@ -65,7 +65,7 @@ extern "C" int opsnnQmmTc(const OpsnnQmmArgs* a, void* stream)
     const bool f8 = (a->x1_dtype == DT_E4M3 || a->x1_dtype == DT_E5M2) && (a->x2_dtype == DT_E4M3 || a->x2_dtype == DT_E5M2);
     if (!i8 && !f8) return -2;
     if (a->x2_scale_len != 1 && a->x2_scale_len != a->N) return -2;
-    if (a->x1_scale && (a->x1_scale_len != 1 || !f8)) return -2;
+    if (a->x1_scale && ((a->x1_scale_len != 1 && a->x1_scale_len != a->M) || !f8)) return -2;
     if (a->out_dtype == DT_I8 || a->out_dtype == DT_I32) { if (!i8) return -2; }
     // int8 operands, 16-bit output, no per-token scale: out = fp32(acc + int32 bias) * scale' + float bias, where scale'
     // is the scale with only its upper 19 bits kept for 64-bit words and for a one-element scale without a bf16 / fp32

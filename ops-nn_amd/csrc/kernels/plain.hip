@@ -146,8 +146,9 @@ __global__ void qmm_tc_plain(OpsnnQmmArgs a)
     }
     if (!is_bias_vec && bias_float) o = __fadd_rn(o, load_scalar_as_f32(a.bias, a.bias_dtype, bi));
     if (pertoken) {
-        const float pt = ((const float*)a.x1_scale)[0];
-        if (a.x2_scale_len == 1 && !is_bias_vec) o = __fmul_rn(o, trunc19(__fmul_rn(s, pt)));
+        // one-element x1Scale: the double-scale modes; one per row: K-C / K-T (compute_pertoken, no truncation)
+        const float pt = ((const float*)a.x1_scale)[a.x1_scale_len == 1 ? 0 : m];
+        if (a.x1_scale_len == 1 && a.x2_scale_len == 1 && !is_bias_vec) o = __fmul_rn(o, trunc19(__fmul_rn(s, pt)));
         else o = __fmul_rn(__fmul_rn(o, do_scale_gen ? trunc19(s) : s), pt);
     } else {
         o = __fmul_rn(o, do_scale_gen ? trunc19(s) : s);

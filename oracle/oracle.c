@@ -26,6 +26,9 @@
  *   orc_qmm_pertoken .. pinned (float64 recomputation, operation-order cases, all-ones example)
  *   orc_qmm_tc ........ pinned (reduces to orc_qmm_pertoken with a constant row scale; hand-computed requant and
  *                       19-bit truncation cases; uint64 packing constants of the reference's utility)
+ *   orc_qmm_pertoken_f8 pinned (integer-valued fp8 operands: sums exact in any order, numpy float64/float32
+ *                       recomputation; reduces to orc_qmm_tc's double-scale branch when x1Scale is constant and no
+ *                       truncation applies)
  *   orc_qmm_perblock .. pinned (reduces to pertoken formula with one K block; power-of-two scales exact; float64)
  *   orc_qmm_mx ........ pinned (power-of-two products are exact: equals integer arithmetic; float64); also serves
  *                       compute_mx of G4 (fp8 x fp4) and, with int8 operands, orc_qmm_perblock serves compute_per_tile
@@ -482,6 +485,32 @@ int orc_qmm_tc(const void* x1, const void* x2, int dt1, int dt2, int64_t M, int6
             store_from_f32(y, y_dt, i, o);
         }
     free(sc); free(dec_off); free(iacc); free(facc);
+    return 0;
+}
+
+/*
+ * K-C / K-T with fp8 operands (G3:612-634 + compute_pertoken, G3:361-387): the matmul is done in fp32 on the decoded
+ * operands, then  y = (acc * x2Scale[n]) * x1Scale[m];  + fp32 bias;  cast.  No truncation of either scale, no
+ * integer bias (the checker admits FLOAT bias only for fp8 operands).
+ */
+int orc_qmm_pertoken_f8(const void* x1, const void* x2, int dt1, int dt2, int64_t M, int64_t K, int64_t N, int tA, int tB,
+                        const float* x1s, const float* x2s, int64_t x2s_len, const float* bias, int y_dt, void* y)
+{
+    float* a = tA ? decode_matrix(x1, dt1, K, M, 1) : decode_matrix(x1, dt1, M, K, 0);
+    float* b = tB ? decode_matrix(x2, dt2, N, K, 1) : decode_matrix(x2, dt2, K, N, 0);
+    float* acc = (float*)calloc((size_t)M * N, sizeof(float));
+    if (!a || !b || !acc) return -1;
+    sgemm_acc(a, K, b, N, acc, N, M, N, K);
+#pragma omp parallel for schedule(static)
+    for (int64_t m = 0; m < M; m++)
+        for (int64_t n = 0; n < N; n++) {
+            float o = acc[m * N + n];
+            o = o * x2s[x2s_len == 1 ? 0 : n];
+            o = o * x1s[m];
+            if (bias) o = o + bias[n];
+            store_from_f32(y, y_dt, (size_t)(m * N + n), o);
+        }
+    free(a); free(b); free(acc);
     return 0;
 }
 

@@ -50,6 +50,8 @@ int orc_qmm_pertoken(const int8_t* x1, const int8_t* x2, int64_t M, int64_t K, i
 int orc_qmm_tc(const void* x1, const void* x2, int dt1, int dt2, int64_t M, int64_t K, int64_t N, int tA, int tB,
                const void* scale, int scale_dt, int64_t scale_len, const float* pertoken, const float* offset,
                int64_t offset_len, const void* bias, int bias_dt, int y_dt, void* y);
+int orc_qmm_pertoken_f8(const void* x1, const void* x2, int dt1, int dt2, int64_t M, int64_t K, int64_t N, int tA, int tB,
+                        const float* x1s, const float* x2s, int64_t x2s_len, const float* bias, int y_dt, void* y);
 int orc_qmm_perblock(const void* x1, const void* x2, int dt1, int dt2, int64_t M, int64_t K, int64_t N, int tA,
                      int tB, const float* x1s, const float* x2s, int64_t gsM, int64_t gsN, int64_t gsK,
                      const float* bias, int y_dt, void* y);

@@ -192,7 +192,7 @@ def make_tc_inputs(m, M, K, N, seed, in_dt, scale_dt, scale_len, bias_dt, tB, pe
         scale = orc.f32_to_bf16(sf)
     else:
         scale = sf
-    pt = gen_scale(rng, 1, 0.5, 2.0) if pertoken else None
+    pt = gen_scale(rng, M if pertoken == "M" else 1, 0.5, 2.0) if pertoken else None   # "M": one scale per row (K-C / K-T)
     off = rng.uniform(-20, 20, size=offset_len).astype(np.float32) if offset_len else None
     bias = gen_bias(rng, N, bias_dt, m)
     if bias_dt == m.ACL_INT32 and bias is not None:
@@ -202,6 +202,9 @@ def make_tc_inputs(m, M, K, N, seed, in_dt, scale_dt, scale_len, bias_dt, tB, pe
 
 
 def oracle_tc(m, inp, M, K, N, out_dt):
+    if inp["pt"] is not None and inp["pt"].size > 1:   # fp8 with a per-row scale: compute_pertoken
+        return orc.qmm_pertoken_f8(inp["x1"], inp["x2"], inp["in_dt"], inp["x2_dt"], M, K, N, False, inp["tB"], inp["pt"],
+                                   inp["scale"], inp["bias"], out_dt)
     return orc.qmm_tc(inp["x1"], inp["x2"], inp["in_dt"], inp["x2_dt"], M, K, N, False, inp["tB"], inp["scale"], inp["scale_dt"],
                       inp["pt"], inp["off"], inp["bias"], inp["bias_dt"] or 0, out_dt)
 
@@ -215,7 +218,7 @@ def run_tc_aclnn(m, inp, M, K, N, out_dt):
     x1 = m.Tensor((M, K), inp["in_dt"], d["x1"])
     x2 = m.Tensor((N, K) if tB else (K, N), inp["x2_dt"], d["x2"])
     s2 = m.Tensor((inp["scale"].size,), inp["scale_dt"], d["scale"])
-    s1 = m.Tensor((1,), m.ACL_FLOAT, d["pt"]) if inp["pt"] is not None else None
+    s1 = m.Tensor((inp["pt"].size,), m.ACL_FLOAT, d["pt"]) if inp["pt"] is not None else None
     off = m.Tensor((inp["off"].size,), m.ACL_FLOAT, d["off"]) if inp["off"] is not None else None
     bias = m.Tensor((N,), inp["bias_dt"], d["bias"]) if inp["bias"] is not None else None
     out = m.Tensor((M, N), out_dt, d_out)

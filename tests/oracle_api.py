@@ -27,6 +27,7 @@ def lib():
         L.orc_qmm_pertoken.argtypes = [vp, vp, i64, i64, i64, ci, ci, vp, vp, i64, vp, ci, ci, vp, vp]
         L.orc_qmm_perblock.argtypes = [vp, vp, ci, ci, i64, i64, i64, ci, ci, vp, vp, i64, i64, i64, vp, ci, vp]
         L.orc_qmm_tc.argtypes = [vp, vp, ci, ci, i64, i64, i64, ci, ci, vp, ci, i64, vp, vp, i64, vp, ci, ci, vp]
+        L.orc_qmm_pertoken_f8.argtypes = [vp, vp, ci, ci, i64, i64, i64, ci, ci, vp, vp, i64, vp, ci, vp]
         L.orc_qmm_mx.argtypes = [vp, vp, ci, ci, i64, i64, i64, ci, ci, vp, vp, vp, ci, vp]
         L.orc_wqbmm.argtypes = [vp, ci, vp, ci, i64, i64, i64, ci, vp, ci, i64, vp, i64, vp, ci, vp]
         L.orc_qmm_tcg.argtypes = [vp, vp, i64, i64, i64, ci, vp, ci, i64, vp, i64, vp, ci, vp]
@@ -128,6 +129,16 @@ def qmm_tc(x1, x2, dt1, dt2, M, K, N, tA, tB, scale, scale_dt, pertoken, offset,
     pertoken = None if pertoken is None else np.ascontiguousarray(pertoken, np.float32)
     rc = lib().orc_qmm_tc(_p(x1), _p(x2), dt1, dt2, M, K, N, int(tA), int(tB), _p(scale), scale_dt, scale.size, _p(pertoken),
                           _p(offset), 0 if offset is None else offset.size, _p(bias), bias_dt, y_dt, _p(y))
+    assert rc == 0
+    return y
+
+
+def qmm_pertoken_f8(x1, x2, dt1, dt2, M, K, N, tA, tB, x1s, x2s, bias, y_dt):
+    """fp8 operands with one fp32 scale per row of x1 and one or N for x2 (K-C / K-T through compute_pertoken)."""
+    y = out_array((M, N), y_dt)
+    x1s = np.ascontiguousarray(x1s, np.float32); x2s = np.ascontiguousarray(x2s, np.float32)
+    bias = None if bias is None else np.ascontiguousarray(bias, np.float32)
+    rc = lib().orc_qmm_pertoken_f8(_p(x1), _p(x2), dt1, dt2, M, K, N, int(tA), int(tB), _p(x1s), _p(x2s), x2s.size, _p(bias), y_dt, _p(y))
     assert rc == 0
     return y
 

@@ -1,5 +1,5 @@
 """Per-tensor / per-channel quantized matmul (T-T, T-C): 64-bit packed scales, int8 requantisation, int32 output,
-19-bit scale truncation, fp8 operands with the one-element per-token scale ("double scale").
+19-bit scale truncation, fp8 operands with the one-element per-token scale ("double scale") or one scale per row (K-C).
 
 CPU part: the oracle's orc_qmm_tc is pinned by recomputing the reference formulas
 (matmul/quant_batch_matmul_v3/tests/assets/qbmmv3_kernel_golden.py:390-513) independently in numpy on small
@@ -129,6 +129,45 @@ def test_fp8_double_scale_against_numpy(scale_len):
     assert np.array_equal(got, want.astype(np.float32))
 
 
+def test_fp8_pertoken_against_numpy():
+    """fp8 operands with one scale per row of x1 (K-C) or additionally one for all of x2 (K-T): compute_pertoken on the
+    fp32 matmul, (acc * x2Scale) * x1Scale[m] + bias, nothing truncated (qbmmv3_kernel_golden.py:361-387, 612-634)."""
+    M, K, N = 6, 48, 10
+    rng = np.random.default_rng(11)
+    # integer-valued operands: every product and partial sum is an exact fp32 integer, so the summation order cannot matter
+    xi1 = rng.integers(-6, 7, (M, K)).astype(np.float32); xi2 = rng.integers(-6, 7, (K, N)).astype(np.float32)
+    x1, x2 = orc.f32_to_e4m3(xi1), orc.f32_to_e4m3(xi2)
+    assert np.array_equal(orc.e4m3_to_f32(x1), xi1)
+    mm = (xi1.astype(np.float64) @ xi2.astype(np.float64)).astype(np.float32)
+    s1 = rng.uniform(0.5, 2.0, M).astype(np.float32); bias = rng.normal(0, 1, N).astype(np.float32)
+    for s2 in (rng.uniform(0.05, 0.5, N).astype(np.float32), np.array([0.1], np.float32)):   # 0.1 has low mantissa bits: no truncation
+        want = ((mm * s2).astype(np.float32) * s1[:, None]).astype(np.float32)
+        got = orc.qmm_pertoken_f8(x1, x2, orc.E4M3, orc.E4M3, M, K, N, False, False, s1, s2, None, orc.F32)
+        assert np.array_equal(got, want)
+        got = orc.qmm_pertoken_f8(x1, x2, orc.E4M3, orc.E4M3, M, K, N, False, False, s1, s2, bias, orc.BF16)
+        assert np.array_equal(got, orc.f32_to_bf16((want + bias).astype(np.float32)))
+    # a transposed x2 is the same matrix; the multiplication order is (acc * s2) * s1, not acc * (s2 * s1)
+    s2 = rng.uniform(0.05, 0.5, N).astype(np.float32)
+    a = orc.qmm_pertoken_f8(x1, x2, orc.E4M3, orc.E4M3, M, K, N, False, False, s1, s2, None, orc.F32)
+    b = orc.qmm_pertoken_f8(x1, np.ascontiguousarray(x2.T), orc.E4M3, orc.E4M3, M, K, N, False, True, s1, s2, None, orc.F32)
+    assert np.array_equal(a, b)
+    other = mm * (s2[None, :] * s1[:, None]).astype(np.float32)
+    assert not np.array_equal(a, other.astype(np.float32))
+    # general fp8 values: ascending-k fp32 sums like every other float path of the oracle, and with a constant row scale
+    # the function equals the double-scale branch of orc_qmm_tc that multiplies separately (per-channel x2 scale)
+    y1 = orc.f32_to_e4m3(rng.normal(0, 1, (M, K)).astype(np.float32)); y2 = orc.f32_to_e4m3(rng.normal(0, 1, (K, N)).astype(np.float32))
+    acc = np.zeros((M, N), np.float32)
+    fa, fb = orc.e4m3_to_f32(y1), orc.e4m3_to_f32(y2)
+    for k in range(K):
+        acc = (acc + fa[:, k:k + 1] * fb[k:k + 1, :]).astype(np.float32)
+    got = orc.qmm_pertoken_f8(y1, y2, orc.E4M3, orc.E4M3, M, K, N, False, False, s1, s2, bias, orc.F32)
+    assert np.array_equal(got, (((acc * s2).astype(np.float32) * s1[:, None]).astype(np.float32) + bias).astype(np.float32))
+    const = np.full(M, 1.37, np.float32)
+    a = orc.qmm_pertoken_f8(y1, y2, orc.E4M3, orc.E4M3, M, K, N, False, False, const, s2, bias, orc.F16)
+    b = orc.qmm_tc(y1, y2, orc.E4M3, orc.E4M3, M, K, N, False, False, s2, orc.F32, const[:1], None, bias, orc.F32, orc.F16)
+    assert np.array_equal(a, b)
+
+
 GPU_CASES = [
     # M, K, N, in, scale dtype, scale len, bias, out, tB, pertoken, offset len
     (16, 32, 16, "i8", "u64", 1, "i32", "f16", False, False, 0),      # the reference's A8W8FP16_pertensor row
@@ -152,6 +191,10 @@ GPU_CASES = [
     (37, 160, 48, "e4m3", "f32", 1, None, "bf16", True, True, 0),     # both scales one element: merged and truncated
     (37, 160, 48, "e4m3", "u64", "N", None, "f32", True, False, 0),   # T-C without a per-token scale: packed scale
     (37, 160, 48, "e4m3", "u64", 1, "f32", "f16", False, False, 0),   # float bias before the scaling (no per-token scale)
+    # fp8 with one scale per row of x1: K-C and K-T (compute_pertoken on the fp32 matmul)
+    (37, 160, 48, "e4m3", "f32", "N", "f32", "bf16", True, "M", 0),
+    (37, 160, 48, "e4m3", "f32", 1, None, "f32", False, "M", 0),
+    (16, 64, 24, "e5m2", "f32", "N", "f32", "f16", False, "M", 0),
 ]
 
 
