@@ -14,6 +14,7 @@ int launch_group_plain(const OpsnnQmmArgs& a, bool tcg, hipStream_t st);
 int launch_wqmm_plain(const OpsnnWqmmArgs& a, hipStream_t st);
 // Return OPSNN_NOT_TAKEN when the arguments are outside what the fast kernels handle.
 int launch_blockscale_mfma(const OpsnnQmmArgs& a, hipStream_t st);
+int launch_fp8_rowcol_mfma(const OpsnnQmmArgs& a, hipStream_t st);
 int launch_mx_mfma(const OpsnnQmmArgs& a, hipStream_t st);
 int launch_wqmm_mfma(const OpsnnWqmmArgs& a, hipStream_t st);
 uint64_t mx_workspace_bytes(const OpsnnQmmArgs& a);
@@ -77,6 +78,12 @@ extern "C" int opsnnQmmTc(const OpsnnQmmArgs* a, void* stream)
         b.x2_scale_trunc = a->x2_scale_dtype == DT_U64 ||
                            (a->x2_scale_len == 1 && !(a->bias && (a->bias_dtype == DT_BF16 || a->bias_dtype == DT_F32)));
         return opsnnQmmInt8(&b, stream);
+    }
+    // fp8 e4m3 operands with a row scale and a column scale that are multiplied in separately (K-C, K-T, T-C with the
+    // one-element x1Scale): matrix-core kernel when the layout allows, else the plain kernel
+    if (f8 && a->x1_scale && a->force_variant != OPSNN_VARIANT_PLAIN && !opsnn_force_plain()) {
+        const int rc = launch_fp8_rowcol_mfma(*a, (hipStream_t)stream);
+        if (rc != OPSNN_NOT_TAKEN) return rc;
     }
     return launch_tc_plain(*a, (hipStream_t)stream);
 }

@@ -43,16 +43,23 @@ struct Fp8BlkParams {
     int64_t sa_rs, sb_rs, sa_bs, sb_bs;
     const float* bias;
     int64_t bias_bs;
+    // row / column scale mode (fp8 K-C, K-T and the double-scale modes that multiply separately):
+    // out = (sum * cs[n * cs_stride]) * rs[m * rs_stride] + bias[n]; strides 0 (one scale) or 1
+    const float* rs;
+    const float* cs;
+    int rs_stride, cs_stride;
 #if QG_DBG
     unsigned long long* dbg;   // timing harness only (see qgemm_core.hip.h)
 #endif
 };
 
-// MX = false: fp32 block scales folded in by the vector ALU.  MX = true (MXFP8): the e8m0 scales of the tile's four
-// 32-element blocks go into the instruction, which then accumulates straight into the running sums (no fold, no
-// partial-sum registers).  Measured against summing every 128 elements from zero and adding in fp32: the same error
-// (1.0 % of bf16 outputs one ulp off the exactly rounded result at K = 7168..16384, either way -- the error is made
-// inside the instruction, between blocks whose scales differ), 1.4x the speed.
+// Three modes of one kernel.  FP8_BLOCK: fp32 block scales folded in by the vector ALU (above).  FP8_MX (MXFP8): the
+// e8m0 scales of the tile's four 32-element blocks go into the instruction, which then accumulates straight into the
+// running sums (no fold, no partial-sum registers).  Measured against summing every 128 elements from zero and adding
+// in fp32: the same error (1.0 % of bf16 outputs one ulp off the exactly rounded result at K = 7168..16384, either way
+// -- the error is made inside the instruction, between blocks whose scales differ), 1.4x the speed.  FP8_ROWCOL: plain
+// fp8 products accumulated in the instruction, one fp32 scale per output row and one per column applied in the epilogue
+// (fp8 K-C / K-T and the double-scale modes that multiply separately; no scale copies at all).
 // a wave-uniform pointer, held in scalar registers
 __device__ __forceinline__ const int8_t* scalar_ptr(const int8_t* p)
 {
@@ -61,9 +68,14 @@ __device__ __forceinline__ const int8_t* scalar_ptr(const int8_t* p)
     return (const int8_t*)(((uint64_t)hi << 32) | lo);
 }
 
-template <int WGM, int STAGES, int OUT_DT, bool MX = false>
+enum : int { FP8_BLOCK = 0, FP8_MX = 1, FP8_ROWCOL = 2 };
+
+template <int WGM, int STAGES, int OUT_DT, int MODE = FP8_BLOCK>
 __global__ __launch_bounds__(WGM * 128, 1) void qmm_fp8_block_kernel(Fp8BlkParams p, int tiles_m, int tiles_n)
 {
+    constexpr bool MX = MODE == FP8_MX;        // e8m0 scales inside the instruction
+    constexpr bool RC = MODE == FP8_ROWCOL;    // plain fp8 products, one scale per row and per column in the epilogue
+    constexpr bool BLK = MODE == FP8_BLOCK;    // fp32 block scales folded in by the vector ALU
     static_assert(!MX || WGM == 4, "MX mode: one scale copy per thread covers the 256 + 256 rows of the tile");
     constexpr int BM = 64 * WGM, BN = 256, BK = 128, NT = WGM * 128;   // WGM x 2 waves of 64 x 128 each
     constexpr int CPR = BK / 16, RPW = 16 / CPR;
@@ -73,7 +85,7 @@ __global__ __launch_bounds__(WGM * 128, 1) void qmm_fp8_block_kernel(Fp8BlkParam
     constexpr int STAGE = A_BYTES + B_BYTES + SC_BYTES;
     constexpr int RPI = NT / CPR;                // rows per copy instruction of the workgroup
     constexpr int NA = BM / RPI, NB = BN / RPI;
-    constexpr int CPT = NA + NB + 1;
+    constexpr int CPT = NA + NB + (RC ? 0 : 1);   // operand copies and, unless the scales wait for the epilogue, one scale copy
     static_assert(STAGES * CPT < 64, "stage count");
     extern __shared__ __attribute__((aligned(16))) char smem[];
 
@@ -114,9 +126,10 @@ __global__ __launch_bounds__(WGM * 128, 1) void qmm_fp8_block_kernel(Fp8BlkParam
     }
     // Scale copy: lanes 0..BM-1 fetch s1 of tile row `tid`, lanes BM, BM+1 fetch s2 of the tile's two n blocks,
     // the rest re-fetch a valid word (their LDS slots are never read).
-    const float* sc_src;
-    int64_t sc_step;
-    if constexpr (MX) {   // the four scale bytes of tile row `tid` (x1 rows, then x2 rows) for one K tile
+    const float* sc_src = nullptr;
+    int64_t sc_step = 0;
+    if constexpr (RC) {
+    } else if constexpr (MX) {   // the four scale bytes of tile row `tid` (x1 rows, then x2 rows) for one K tile
         if (tid < BM) {
             const int r = tid < a_rows ? tid : a_rows - 1;
             sc_src = (const float*)(p.sa + bz * p.sa_bs + (m0 + r) * p.sa_rs);
@@ -213,7 +226,8 @@ __global__ __launch_bounds__(WGM * 128, 1) void qmm_fp8_block_kernel(Fp8BlkParam
     (void)sc; (void)s1raw; (void)s2raw; (void)sca; (void)saraw; (void)sbraw;
     v4f part[2][FM];
     auto read_scales = [&](const char* st) {
-        if constexpr (MX) {
+        if constexpr (RC) {
+        } else if constexpr (MX) {
             const uint32_t* sS = (const uint32_t*)(st + A_BYTES + B_BYTES);
 #pragma unroll
             for (int j = 0; j < FM; j++) saraw[j] = sS[wm * TM + j * 16 + frow];
@@ -288,6 +302,8 @@ __global__ __launch_bounds__(WGM * 128, 1) void qmm_fp8_block_kernel(Fp8BlkParam
             for (int j = 0; j < FM; j++) {
                 if constexpr (MX)   // the instruction applies both scales: accumulate in place, nothing to fold
                     acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(fb[i & 1], fa[j], acc[i][j], 0, 0, 0, (int)scb, 0, (int)sca[j]);
+                else if constexpr (RC)
+                    acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(fb[i & 1], fa[j], acc[i][j], 0, 0, 0, 0x7f7f7f7f, 0, 0x7f7f7f7f);
                 else
                     part[i & 1][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(fb[i & 1], fa[j], v4f{0.0f, 0.0f, 0.0f, 0.0f}, 0, 0, 0,
                                                                                       0x7f7f7f7f, 0, 0x7f7f7f7f);
@@ -298,7 +314,7 @@ __global__ __launch_bounds__(WGM * 128, 1) void qmm_fp8_block_kernel(Fp8BlkParam
                     for (int c = j * CPS; c < (j + 1) * CPS && c < CPT; c++) issue_piece(ktc, kt & 1, c);
                     __builtin_amdgcn_sched_barrier(0);
                 }
-                if constexpr (MX) {
+                if constexpr (!BLK) {
                 } else if (i > 0) {
 #pragma unroll
                     for (int r = 0; r < 4; r++) acc[i - 1][j][r] = __builtin_fmaf(part[(i - 1) & 1][j][r], sc[j], acc[i - 1][j][r]);
@@ -308,7 +324,7 @@ __global__ __launch_bounds__(WGM * 128, 1) void qmm_fp8_block_kernel(Fp8BlkParam
                 }
                 __builtin_amdgcn_sched_barrier(0);
             }
-            if (!MX && i == 0) {   // from here on this tile's scales
+            if (BLK && i == 0) {   // from here on this tile's scales
 #pragma unroll
                 for (int j = 0; j < FM; j++) sc[j] = s1raw[j] * s2raw;
                 __builtin_amdgcn_sched_barrier(0);
@@ -317,7 +333,7 @@ __global__ __launch_bounds__(WGM * 128, 1) void qmm_fp8_block_kernel(Fp8BlkParam
     }
 #pragma unroll
     for (int j = 0; j < FM; j++) {
-        if constexpr (!MX) {
+        if constexpr (BLK) {
 #pragma unroll
             for (int r = 0; r < 4; r++) acc[FN - 1][j][r] = __builtin_fmaf(part[1][j][r], sc[j], acc[FN - 1][j][r]);
         }
@@ -341,12 +357,29 @@ __global__ __launch_bounds__(WGM * 128, 1) void qmm_fp8_block_kernel(Fp8BlkParam
     uint16_t* out = (uint16_t*)p.out + bz * p.M * p.N;
     const bool vec_ok = (p.N % 8) == 0 && ((uintptr_t)p.out % 16) == 0;
     const int er = lane >> 4, ec = lane & 15;
+    float rs_j[FM];   // row / column scale mode: the scale of this lane's output row in each x1 fragment
+    (void)rs_j;
+    if constexpr (RC) {
+#pragma unroll
+        for (int j = 0; j < FM; j++) {
+            const int64_t mrow = m0 + wm * TM + j * 16 + frow;
+            rs_j[j] = p.rs[(mrow < p.M ? mrow : p.M - 1) * p.rs_stride];
+        }
+    }
 #pragma unroll
     for (int j = 0; j < FM; j++) {
 #pragma unroll
         for (int i = 0; i < FN; i++) {
             v4f v = acc[i][j];
-            if constexpr (MX) {
+            if constexpr (RC) {   // (sum * x2Scale[n]) * x1Scale[m], each product rounded, as compute_pertoken orders them
+                const int64_t nb = n0 + wn * TN + i * 16 + 4 * fq;
+#pragma unroll
+                for (int r = 0; r < 4; r++) {
+                    const float c = p.cs[(nb + r < p.N ? nb + r : p.N - 1) * p.cs_stride];
+                    v[r] = (v[r] * c) * rs_j[j];
+                }
+            }
+            if constexpr (MX || RC) {
                 if (p.bias) {
                     const int64_t nb = n0 + wn * TN + i * 16 + 4 * fq;
 #pragma unroll
@@ -386,14 +419,14 @@ __global__ __launch_bounds__(WGM * 128, 1) void qmm_fp8_block_kernel(Fp8BlkParam
 #endif
 }
 
-template <int WGM, int STAGES, int OUT_DT, bool MX = false>
+template <int WGM, int STAGES, int OUT_DT, int MODE = FP8_BLOCK>
 static int launch_fp8_block(const Fp8BlkParams& p, int64_t batch, hipStream_t st)
 {
     constexpr int BM = 64 * WGM;
     int tiles_m = (int)((p.M + BM - 1) / BM), tiles_n = (int)((p.N + 255) / 256);
     dim3 grid((unsigned)(tiles_m * tiles_n), (unsigned)batch);
     size_t lds = (size_t)STAGES * ((BM + 256) * 128 + WGM * 128 * 4);
-    auto k = qmm_fp8_block_kernel<WGM, STAGES, OUT_DT, MX>;
+    auto k = qmm_fp8_block_kernel<WGM, STAGES, OUT_DT, MODE>;
     static bool attr_set = false;
     if (!attr_set) {
         hipError_t e = hipFuncSetAttribute((const void*)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
@@ -421,9 +454,39 @@ int launch_mxfp8_mfma(const OpsnnQmmArgs& a, hipStream_t st)
     if (((uintptr_t)p.a | (uintptr_t)p.b | (uint64_t)p.lda | (uint64_t)p.ldb | (uint64_t)p.a_bs | (uint64_t)p.b_bs) % 16) return OPSNN_NOT_TAKEN;
     if (((uintptr_t)p.sa | (uintptr_t)p.sb | (uint64_t)p.sa_rs | (uint64_t)p.sb_rs | (uint64_t)p.sa_bs | (uint64_t)p.sb_bs) % 4) return OPSNN_NOT_TAKEN;
     if (a.bias && a.bias_dtype != DT_F32) return OPSNN_NOT_TAKEN;
-    if (a.out_dtype == DT_BF16) return launch_fp8_block<4, 2, DT_BF16, true>(p, a.batch, st);
-    if (a.out_dtype == DT_F16) return launch_fp8_block<4, 2, DT_F16, true>(p, a.batch, st);
+    if (a.out_dtype == DT_BF16) return launch_fp8_block<4, 2, DT_BF16, FP8_MX>(p, a.batch, st);
+    if (a.out_dtype == DT_F16) return launch_fp8_block<4, 2, DT_F16, FP8_MX>(p, a.batch, st);
     return OPSNN_NOT_TAKEN;
+}
+
+// fp8 e4m3 x e4m3 with one fp32 scale per row of x1 (or one for all of it) and one per column of x2 (or one):
+// K-C, K-T and the double-scale modes whose two scales are multiplied in separately
+// (qbmmv3_kernel_golden.py:361-387 and :432-441).  out = (sum * x2Scale[n]) * x1Scale[m] + fp32 bias.
+// Needs K-contiguous operands with K % 128 == 0 and a 16-bit output; anything else stays on the plain kernel.
+int launch_fp8_rowcol_mfma(const OpsnnQmmArgs& a, hipStream_t st)
+{
+    if (a.x1_dtype != DT_E4M3 || a.x2_dtype != DT_E4M3) return OPSNN_NOT_TAKEN;
+    if (a.out_dtype != DT_BF16 && a.out_dtype != DT_F16) return OPSNN_NOT_TAKEN;
+    if (!a.x1_scale || !a.x2_scale || a.x2_scale_dtype != DT_F32) return OPSNN_NOT_TAKEN;
+    if (a.x1_scale_len != 1 && a.x1_scale_len != a.M) return OPSNN_NOT_TAKEN;
+    if (a.x2_scale_len != 1 && a.x2_scale_len != a.N) return OPSNN_NOT_TAKEN;
+    if (a.x1_scale_len == 1 && a.x2_scale_len == 1 && !a.bias) return OPSNN_NOT_TAKEN;   // merged and truncated scale: plain kernel
+    if (a.bias && a.bias_dtype != DT_F32) return OPSNN_NOT_TAKEN;
+    if (a.K % 128 != 0 || a.M * a.N < 64 * 64 || a.x1.col_stride != 1 || a.x2.row_stride != 1) return OPSNN_NOT_TAKEN;
+    Fp8BlkParams p{};
+    p.a = (const int8_t*)a.x1.ptr; p.b = (const int8_t*)a.x2.ptr;
+    p.lda = a.x1.row_stride; p.ldb = a.x2.col_stride; p.a_bs = a.x1.batch_stride; p.b_bs = a.x2.batch_stride;
+    p.out = a.out; p.M = a.M; p.N = a.N; p.K = a.K; p.gsM = 1;
+    p.rs = (const float*)a.x1_scale; p.rs_stride = a.x1_scale_len == 1 ? 0 : 1;
+    p.cs = (const float*)a.x2_scale; p.cs_stride = a.x2_scale_len == 1 ? 0 : 1;
+    p.bias = (const float*)a.bias; p.bias_bs = a.bias_batch_stride;
+    if (((uintptr_t)p.a | (uintptr_t)p.b | (uint64_t)p.lda | (uint64_t)p.ldb | (uint64_t)p.a_bs | (uint64_t)p.b_bs) % 16) return OPSNN_NOT_TAKEN;
+    if (a.M >= 512) {
+        if (a.out_dtype == DT_BF16) return launch_fp8_block<4, 2, DT_BF16, FP8_ROWCOL>(p, a.batch, st);
+        return launch_fp8_block<4, 2, DT_F16, FP8_ROWCOL>(p, a.batch, st);
+    }
+    if (a.out_dtype == DT_BF16) return launch_fp8_block<2, 2, DT_BF16, FP8_ROWCOL>(p, a.batch, st);
+    return launch_fp8_block<2, 2, DT_F16, FP8_ROWCOL>(p, a.batch, st);
 }
 
 int launch_blockscale_mfma(const OpsnnQmmArgs& a0, hipStream_t st)
