@@ -39,6 +39,7 @@ struct QgemmParams {
     int64_t ldc;       // output row pitch in elements (N, or wider when this launch covers a column range)
     // MODE_I8 epilogue: out = cast(fp32(acc + ib[n]) * x2s[n] * x1s[m] + fb[n])
     const float* x1s;
+    int x1s_one;       // x1s is one scale for every row (honoured by the four-wave kernel only)
     const void* x2s;   // FLOAT / BF16, or UINT64 words whose low 32 bits are the fp32 scale
     int x2s_dt;
     int64_t x2s_len;

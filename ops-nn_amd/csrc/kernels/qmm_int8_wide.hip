@@ -1,4 +1,4 @@
-// int8 x int8 tile kernel with one wave per SIMD and a 256 x (32*FN) output tile, FN = 8..11.
+// int8 x int8 (and fp8 e4m3 x e4m3) tile kernel with one wave per SIMD and a 256 x (32*FN) output tile, FN = 8..11.
 //
 // Why a second int8 tile kernel: a GEMM runs in rounds of one tile per CU, and with a fixed 256 x 256 tile a shape
 // such as 2048 x 11008 needs 1.34 rounds -- the last third of a round costs a whole one (or a second launch of small
@@ -27,6 +27,10 @@
 // launch of 128 x 128 tiles on the remaining 2816; at 256 x 256 (FN = 8) it is level with the 8-wave kernel
 // (62-64 against 65 us on 2048 x 4096 x 8192, 540 against 560 us on 8192^3).
 //
+// F8 = true: the same kernel on fp8 e4m3 operands for the modes with one scale per row and per column (K-C, K-T,
+// separately multiplied double scale): one v_mfma_f32_16x16x128_f8f6f4 per fragment pair and K tile instead of two
+// int8 instructions, float sums, and the same epilogue without the integer bias.
+//
 // Epilogue formula and its order of operations: the K-C / K-T golden, as in qgemm_core.hip.h
 // (matmul/quant_batch_matmul_v3/tests/assets/qbmmv3_kernel_golden.py): out = cast(fp32(acc + ib[n]) * x2s[n] * x1s[m] + fb[n]).
 #include "launch.h"
@@ -52,6 +56,14 @@ __device__ __forceinline__ void mfma_i8_16x16x64(v4i& c, const v4i a, const v4i 
 // on answers every dependency on an LDS read with a wait for ALL outstanding reads, including the ones issued a moment
 // ago for the next fragment; hidden from it, the pass counts exactly.  The copies' own completion is waited for
 // explicitly (vmcnt + barrier) wherever LDS is read.
+// acc += a (16 x 128 fp8 e4m3) x b (128 x 16 fp8 e4m3), fp32 sums; see mfma_i8_16x16x64 for the register classes
+template <bool AG>
+__device__ __forceinline__ void mfma_f8_16x16x128(v4f& c, const v8i a, const v8i b)
+{
+    if constexpr (AG) asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+    else asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, %0" : "+v"(c) : "v"(a), "v"(b));
+}
+
 template <int LDS_IMM>
 __device__ __forceinline__ void dma_copy16(const int8_t* sbase, uint32_t voff, uint32_t lds_base)
 {
@@ -59,9 +71,10 @@ __device__ __forceinline__ void dma_copy16(const int8_t* sbase, uint32_t voff, u
                  : : "s"(lds_base), "v"(voff), "s"(sbase), "n"(LDS_IMM) : "memory", "m0", "scc");
 }
 
-template <int FN, int OUT_DT>
+template <int FN, int OUT_DT, bool F8 = false>
 __global__ __launch_bounds__(256, 1) void qgemm_i8_wide_kernel(QgemmParams p, int tiles_m, int tiles_n)
 {
+    constexpr int SLOTS = F8 ? 8 : 16;   // MFMAs per x2 fragment
     constexpr int NT = 256, BM = 256, TM = 128, FM = TM / 16, TN = 16 * FN, BN = 2 * TN, BK = 128, STAGES = 2;
     constexpr int CPR = BK / 16, RPW = 16 / CPR;
     constexpr int A_BYTES = BM * BK, B_BYTES = BN * BK, STAGE = A_BYTES + B_BYTES;
@@ -124,11 +137,12 @@ __global__ __launch_bounds__(256, 1) void qgemm_i8_wide_kernel(QgemmParams p, in
         for_copies([&](auto c) { issue_piece(kt, kt % STAGES, c); });
     };
 
-    v4i acc[FN][FM];
+    using acc_t = std::conditional_t<F8, v4f, v4i>;
+    acc_t acc[FN][FM];
 #pragma unroll
     for (int i = 0; i < FN; i++)
 #pragma unroll
-        for (int j = 0; j < FM; j++) acc[i][j] = v4i{0, 0, 0, 0};
+        for (int j = 0; j < FM; j++) acc[i][j] = acc_t{0, 0, 0, 0};
 
     // Operand fragment of the 16x16x64 instruction pair, lane (row = lane%16, q = lane/16): bytes [16q, 16q+16) of the
     // row's 128 bytes of K for the first instruction, [64+16q, +16) for the second.  (K is the contraction index: any
@@ -170,9 +184,49 @@ __global__ __launch_bounds__(256, 1) void qgemm_i8_wide_kernel(QgemmParams p, in
         const int cstage = (kt + 1) & 1;
         auto spread_copies = [&](int slot) {   // slot = index within the tile of the MFMA just issued
             for_copies([&](auto c) {
-                if ((decltype(c)::value * SPREAD * 16) / CPT == slot) issue_piece(ktc, cstage, c);
+                if ((decltype(c)::value * SPREAD * SLOTS) / CPT == slot) issue_piece(ktc, cstage, c);
             });
         };
+        if constexpr (F8) {
+#pragma unroll
+            for (int i = 0; i < FN; i++) {
+                if (i + 1 < FN) {
+                    if (i == 0) {   // one instruction reads both halves of a fragment: everything requested so far is needed now
+                        wait_lgkmcnt0();
+                        if (FN & 1) { fbl[0] = fbl[1]; fbh[0] = fbh[1]; }
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
+                    fbl[(i + 1) & 1] = load_lo(st, b_rowbase + (i + 1) * 16 * BK);
+                    fbh[(i + 1) & 1] = load_hi(st, b_rowbase + (i + 1) * 16 * BK);
+                    __builtin_amdgcn_sched_barrier(0);
+                    if (i > 0) __builtin_amdgcn_s_waitcnt(0xc07f | (2 << 8));
+                } else {
+                    wait_vmcnt<0>();
+                    wait_lgkmcnt0();
+                    __builtin_amdgcn_s_barrier();
+                    __builtin_amdgcn_sched_barrier(0);
+                    fbl[(i + 1) & 1] = load_lo(stn, b_rowbase);
+                    fbh[(i + 1) & 1] = load_hi(stn, b_rowbase);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+                const v8i b8 = __builtin_shufflevector(fbl[i & 1], fbh[i & 1], 0, 1, 2, 3, 4, 5, 6, 7);
+#pragma unroll
+                for (int j = 0; j < FM; j++) {
+                    const v8i a8 = __builtin_shufflevector(fal[j], fah[j], 0, 1, 2, 3, 4, 5, 6, 7);
+                    if constexpr (F8) {   // (the int8 instantiation never compiles this call)
+                        if (i * FM + j < 64) mfma_f8_16x16x128<true>(acc[i][j], b8, a8);
+                        else mfma_f8_16x16x128<false>(acc[i][j], b8, a8);
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+                    spread_copies(i * SLOTS + j);
+                    if (i == FN - 1) {
+                        fal[j] = load_lo(stn, a_rowbase + j * 16 * BK);
+                        fah[j] = load_hi(stn, a_rowbase + j * 16 * BK);
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            }
+        } else {
 #pragma unroll
         for (int i = 0; i < FN; i++) {
             if (i + 1 < FN) {
@@ -224,6 +278,7 @@ __global__ __launch_bounds__(256, 1) void qgemm_i8_wide_kernel(QgemmParams p, in
                 }
             }
         }
+        }
     }
     wait_lgkmcnt0();   // the reads and copies past the last tile land before LDS is reused
     wait_vmcnt<0>();
@@ -252,7 +307,7 @@ __global__ __launch_bounds__(256, 1) void qgemm_i8_wide_kernel(QgemmParams p, in
         for (int i = tid; i < BM; i += NT) {
             int64_t m = m0 + i;
             if (m >= p.M) m = p.M - 1;
-            sS1[i] = p.x1s ? p.x1s[m] : 1.0f;
+            sS1[i] = p.x1s ? p.x1s[p.x1s_one ? 0 : m] : 1.0f;
         }
     }
     __syncthreads();
@@ -281,7 +336,9 @@ __global__ __launch_bounds__(256, 1) void qgemm_i8_wide_kernel(QgemmParams p, in
             v4f v;
 #pragma unroll
             for (int e = 0; e < 4; e++) {
-                float tv = (float)(acc[i][j][e] + ib[e]);
+                float tv;
+                if constexpr (F8) tv = acc[i][j][e];
+                else tv = (float)(acc[i][j][e] + ib[e]);
                 tv = tv * s2[e];
                 tv = tv * s1;
                 v[e] = tv + fbv[e];
@@ -312,13 +369,13 @@ __global__ __launch_bounds__(256, 1) void qgemm_i8_wide_kernel(QgemmParams p, in
     }
 }
 
-template <int FN, int OUT_DT>
+template <int FN, int OUT_DT, bool F8 = false>
 static int launch_wide_one(const QgemmParams& p, int64_t batch, hipStream_t st)
 {
     constexpr int BM = 256, BN = 32 * FN, BK = 128;
     const int tiles_m = (int)((p.M + BM - 1) / BM), tiles_n = (int)((p.N + BN - 1) / BN);
     const size_t lds = (size_t)2 * (BM + BN) * BK;
-    auto k = qgemm_i8_wide_kernel<FN, OUT_DT>;
+    auto k = qgemm_i8_wide_kernel<FN, OUT_DT, F8>;
     static bool attr_set = false;   // per instantiation; benign if two threads both set it
     if (!attr_set) {
         hipError_t e = hipFuncSetAttribute((const void*)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
@@ -341,6 +398,25 @@ int launch_int8_wide(const QgemmParams& p, int fn, int64_t batch, int out_dt, hi
         case 9: return bf ? launch_wide_one<9, DT_BF16>(p, batch, st) : launch_wide_one<9, DT_F16>(p, batch, st);
         case 10: return bf ? launch_wide_one<10, DT_BF16>(p, batch, st) : launch_wide_one<10, DT_F16>(p, batch, st);
         case 11: return bf ? launch_wide_one<11, DT_BF16>(p, batch, st) : launch_wide_one<11, DT_F16>(p, batch, st);
+        default: return OPSNN_NOT_TAKEN;
+    }
+}
+
+}  // namespace opsnn
+
+namespace opsnn {
+
+// The fp8 e4m3 instantiation: p.x1s / p.x2s / fp32 bias as for int8 (x1s_one: one scale for all rows), no integer bias.
+int launch_f8_wide(const QgemmParams& p, int fn, int64_t batch, int out_dt, hipStream_t st)
+{
+    if (p.KB % 128 != 0 || p.KB < 128) return OPSNN_NOT_TAKEN;
+    if (out_dt != DT_BF16 && out_dt != DT_F16) return OPSNN_NOT_TAKEN;
+    const bool bf = out_dt == DT_BF16;
+    switch (fn) {
+        case 8: return bf ? launch_wide_one<8, DT_BF16, true>(p, batch, st) : launch_wide_one<8, DT_F16, true>(p, batch, st);
+        case 9: return bf ? launch_wide_one<9, DT_BF16, true>(p, batch, st) : launch_wide_one<9, DT_F16, true>(p, batch, st);
+        case 10: return bf ? launch_wide_one<10, DT_BF16, true>(p, batch, st) : launch_wide_one<10, DT_F16, true>(p, batch, st);
+        case 11: return bf ? launch_wide_one<11, DT_BF16, true>(p, batch, st) : launch_wide_one<11, DT_F16, true>(p, batch, st);
         default: return OPSNN_NOT_TAKEN;
     }
 }

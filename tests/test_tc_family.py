@@ -218,6 +218,10 @@ def test_gpu_matches_oracle(gpu, M, K, N, in_dt, s_dt, s_len, bias_dt, out_dt, t
     (640, 1024, 520, "N", False, "f16", "M"),     # 256-row tile instance
     (128, 256, 192, 1, True, "bf16", "M"),        # K-T
     (128, 512, 256, "N", True, "f16", True),      # one-element x1Scale with a per-channel x2Scale: multiplied separately
+    # enough tiles for the four-wave kernel with 256 x 32n tiles: 4 x 65 tiles of 256 x 256 would take 2 rounds of 256 CUs,
+    # 4 x 60 tiles of 256 x 288 one (ragged last column tile; one-element x1Scale in the second case)
+    (1000, 1024, 16600, "N", True, "bf16", "M"),
+    (1024, 1024, 16640, "N", False, "f16", True),
 ])
 def test_gpu_fp8_row_and_column_scales_on_the_matrix_cores(gpu, M, K, N, s_len, bias, out_dt, pt):
     """fp8 e4m3 K-C / K-T / T-C-double-scale on the MFMA kernel (K-contiguous x2, K % 128 == 0, 16-bit output).  The
