@@ -148,13 +148,13 @@ extern "C" int opsnnQmmInt8(const OpsnnQmmArgs* a, void* stream)
         const int64_t tm = (p.M + 255) / 256, tn = (p.N + 255) / 256;
         // Cost of a strategy in units of "one round of tiles, per 32 columns of tile width".  The four-wave kernel
         // takes tiles of 256 x 32n columns, n = 8..11: the width whose tile count wastes the least of its last round
-        // wins (2048 x 11008: 256 tiles of 352 columns, one round, 11 units against 8 + 5 for the split below).
+        // wins (2048 x 11008: 256 tiles of 352 columns, one round, 13 units against 10 + 6 for the split below).
         int64_t wide_cost = INT64_MAX;
         int wide_fn = 0;
         if (p.K % 128 == 0 && p.K >= 1024 && tm * tn * a->batch >= cus) {
             for (int fn = 8; fn <= 11; fn++) {
                 const int64_t tiles = tm * ((p.N + 32 * fn - 1) / (32 * fn)) * a->batch;
-                const int64_t cost = (tiles + cus - 1) / cus * fn;
+                const int64_t cost = (tiles + cus - 1) / cus * (fn + 2);   // + 2: what a tile costs beyond its width (8192^3: 3 rounds of 352 columns 495 us, 4 of 256 529 us)
                 if (cost < wide_cost) { wide_cost = cost; wide_fn = fn; }
             }
         }
@@ -162,7 +162,7 @@ extern "C" int opsnnQmmInt8(const OpsnnQmmArgs* a, void* stream)
             const int64_t rounds = tm * tn / cus;
             const int64_t cols_a = rounds * cus / tm;            // column tiles in whole rounds
             const bool split_ok = cols_a >= 1 && cols_a * tm * 8 >= rounds * cus * 7;   // at least 7/8 of those rounds is filled
-            const int64_t split_cost = split_ok ? rounds * 8 + (cols_a * 256 < p.N ? 5 : 0) : INT64_MAX;   // measured: the remainder launch costs 5/8 of a round
+            const int64_t split_cost = split_ok ? rounds * 10 + (cols_a * 256 < p.N ? 6 : 0) : INT64_MAX;   // measured: the remainder launch costs 5/8 of a round
             if (wide_fn && wide_cost <= split_cost) {
                 const int rc = launch_int8_wide(g, wide_fn, a->batch, p.out_dt, st);
                 if (rc != OPSNN_NOT_TAKEN) return rc;
