@@ -14,8 +14,8 @@ import oracle_api as orc
 # very same bench command, each scaled by what the counter reads for a byte transpose of known size; the runs and the
 # figures are in profiles/<kernel>_<workload>.txt.  Keyed by (config, M of the weight-only configs).
 MEASURED_TRAFFIC = {
-    (2, None): 101.9e6, (4, None): 824.5e6, (5, None): 1802.8e6,
-    (3, 1): 67.3e6, (3, 16): 69.2e6, (1, None): 9.2e6,
+    (2, None): 101.9e6, (4, None): 824.4e6, (5, None): 1802.2e6,
+    (3, 1): 67.2e6, (3, 16): 69.2e6, (1, None): 9.2e6,
 }
 
 
