@@ -151,7 +151,9 @@ extern "C" int opsnnQmmInt8(const OpsnnQmmArgs* a, void* stream)
         // wins (2048 x 11008: 256 tiles of 352 columns, one round, 13 units against 10 + 6 for the split below).
         int64_t wide_cost = INT64_MAX;
         int wide_fn = 0;
-        if (p.K % 128 == 0 && p.K >= 1024 && tm * tn * a->batch >= cus) {
+        // (from 24 K tiles up: with fewer the 8-wave kernels, whose second wave per SIMD covers prologue and epilogue,
+        // are ahead -- 8192 x 1024 x 8192: 96 against 114 us, 4096 x 2048 x 14336: 147 against 154; and from 3/4 of a round of 256 x 256 tiles up)
+        if (p.K % 128 == 0 && p.K >= 3072 && tm * tn * a->batch * 4 >= cus * 3) {
             for (int fn = 8; fn <= 11; fn++) {
                 const int64_t tiles = tm * ((p.N + 32 * fn - 1) / (32 * fn)) * a->batch;
                 const int64_t cost = (tiles + cus - 1) / cus * (fn + 2);   // + 2: what a tile costs beyond its width (8192^3: 3 rounds of 352 columns 495 us, 4 of 256 529 us)
