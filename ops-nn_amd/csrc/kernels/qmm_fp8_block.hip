@@ -490,7 +490,8 @@ int launch_fp8_rowcol_mfma(const OpsnnQmmArgs& a, hipStream_t st)
         int dev = 0, cus = 0;
         if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0) cus = 256;
         const int64_t tm = (a.M + 255) / 256, tn = (a.N + 255) / 256;
-        if (a.K >= 1024 && tm * tn * a.batch >= cus) {
+        static const bool no_wide = [] { const char* e = getenv("OPSNN_F8_NO_WIDE"); return e && e[0] == '1'; }();   // tuning aid
+        if (!no_wide && a.K >= 1024 && tm * tn * a.batch * 4 >= cus * 3) {
             const int64_t block_cost = (tm * tn * a.batch + cus - 1) / cus * 10;   // tile cost = width / 32 + 2, as for int8
             int64_t wide_cost = INT64_MAX;
             int wide_fn = 0;
