@@ -437,6 +437,8 @@ static int launch_fp8_block(const Fp8BlkParams& p, int64_t batch, hipStream_t st
     return (int)hipGetLastError();
 }
 
+int launch_mxfp8_wide(const QgemmParams& p, int fn, int64_t batch, int out_dt, hipStream_t st);   // qmm_int8_wide.hip
+
 // MXFP8 (e4m3 x e4m3, e8m0 scale per 32 K) on the same kernel in MX mode.  Operands and scales must be K-contiguous with
 // K % 128 == 0 (four scale bytes per row per K tile); out[m,n] = sum_k (x1 s1)(x2 s2) + fp32 bias.
 int launch_mxfp8_mfma(const OpsnnQmmArgs& a, hipStream_t st)
@@ -454,6 +456,38 @@ int launch_mxfp8_mfma(const OpsnnQmmArgs& a, hipStream_t st)
     if (((uintptr_t)p.a | (uintptr_t)p.b | (uint64_t)p.lda | (uint64_t)p.ldb | (uint64_t)p.a_bs | (uint64_t)p.b_bs) % 16) return OPSNN_NOT_TAKEN;
     if (((uintptr_t)p.sa | (uintptr_t)p.sb | (uint64_t)p.sa_rs | (uint64_t)p.sb_rs | (uint64_t)p.sa_bs | (uint64_t)p.sb_bs) % 4) return OPSNN_NOT_TAKEN;
     if (a.bias && a.bias_dtype != DT_F32) return OPSNN_NOT_TAKEN;
+    // Large problems: the four-wave kernel with the tile width that fills its rounds of CUs best, as for the row/column
+    // scale modes below (K % 512 == 0 and 16-byte aligned scale rows, else it declines).  OPSNN_MX8_WIDE = 8 or 9 forces that
+    // kernel with that width (tests, tuning), 0 forbids it.
+    {
+        int dev = 0, cus = 0;
+        if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0) cus = 256;
+        const char* e = getenv("OPSNN_MX8_WIDE");
+        const int forced = e ? atoi(e) : -1;
+        const int64_t tm = (a.M + 255) / 256, tn = (a.N + 255) / 256;
+        int wide_fn = 0;
+        if (forced >= 8 && forced <= 9) {
+            wide_fn = forced;
+        } else if (forced != 0 && a.K >= 1024 && tm * tn * a.batch * 4 >= (int64_t)cus * 3) {
+            const int64_t block_cost = (tm * tn * a.batch + cus - 1) / cus * 10;
+            int64_t wide_cost = INT64_MAX;
+            for (int fn = 8; fn <= 9; fn++) {   // wider tiles leave no room in LDS for the scale slots
+                const int64_t tiles = tm * ((a.N + 32 * fn - 1) / (32 * fn)) * a.batch;
+                const int64_t cost = (tiles + cus - 1) / cus * (fn + 2);
+                if (cost < wide_cost) { wide_cost = cost; wide_fn = fn; }
+            }
+            if (wide_cost > block_cost) wide_fn = 0;
+        }
+        if (wide_fn) {
+            QgemmParams g{};
+            g.a = p.a; g.b = p.b; g.lda = p.lda; g.ldb = p.ldb; g.a_bs = p.a_bs; g.b_bs = p.b_bs;
+            g.out = a.out; g.M = a.M; g.N = a.N; g.ldc = a.N; g.KB = a.K;
+            g.bias = a.bias; g.bias_dt = DT_F32; g.bias_bs = a.bias_batch_stride;
+            g.sa = p.sa; g.sb = p.sb; g.sa_rs = p.sa_rs; g.sb_rs = p.sb_rs; g.sa_bs = p.sa_bs; g.sb_bs = p.sb_bs;
+            const int rc = launch_mxfp8_wide(g, wide_fn, a.batch, a.out_dtype, st);
+            if (rc != OPSNN_NOT_TAKEN) return rc;
+        }
+    }
     if (a.out_dtype == DT_BF16) return launch_fp8_block<4, 2, DT_BF16, FP8_MX>(p, a.batch, st);
     if (a.out_dtype == DT_F16) return launch_fp8_block<4, 2, DT_F16, FP8_MX>(p, a.batch, st);
     return OPSNN_NOT_TAKEN;

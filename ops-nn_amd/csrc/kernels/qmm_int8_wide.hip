@@ -31,6 +31,13 @@
 // separately multiplied double scale): one v_mfma_f32_16x16x128_f8f6f4 per fragment pair and K tile instead of two
 // int8 instructions, float sums, and the same epilogue without the integer bias.
 //
+// MXS = true (with F8): MXFP8.  A K tile needs four e8m0 bytes per row; one 16-byte copy per row brings the scales of
+// FOUR tiles into one of two slots behind the operand stages (a 4-byte copy per row and tile costs a cache-line request
+// for four useful bytes -- as many requests as the operands themselves, and the kernel ran no faster than the 8-wave
+// one).  Each lane reads the dword of its row with its fragment and shifts its own block's byte down (lane group q
+// supplies the scale of block q, see qmm_fp8_block.hip), and the scaled form of the instruction applies them.  Needs
+// K % 512 == 0, 16-byte aligned scale rows and FN <= 9 (the slots must fit into LDS).
+//
 // Epilogue formula and its order of operations: the K-C / K-T golden, as in qgemm_core.hip.h
 // (matmul/quant_batch_matmul_v3/tests/assets/qbmmv3_kernel_golden.py): out = cast(fp32(acc + ib[n]) * x2s[n] * x1s[m] + fb[n]).
 #include "launch.h"
@@ -64,6 +71,20 @@ __device__ __forceinline__ void mfma_f8_16x16x128(v4f& c, const v8i a, const v8i
     else asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, %0" : "+v"(c) : "v"(a), "v"(b));
 }
 
+template <bool AG>
+__device__ __forceinline__ void mfma_f8_16x16x128_scaled(v4f& c, const v8i a, const v8i b, uint32_t sa, uint32_t sb)
+{
+    if constexpr (AG) asm volatile("v_mfma_scale_f32_16x16x128_f8f6f4 %0, %1, %2, %0, %3, %4 op_sel_hi:[0,0,0]" : "+a"(c) : "v"(a), "v"(b), "v"(sa), "v"(sb));
+    else asm volatile("v_mfma_scale_f32_16x16x128_f8f6f4 %0, %1, %2, %0, %3, %4 op_sel_hi:[0,0,0]" : "+v"(c) : "v"(a), "v"(b), "v"(sa), "v"(sb));
+}
+
+// the same copy with a 64-bit address per lane (dma_copy16 below: scalar base + 32-bit lane offset)
+template <int LDS_IMM>
+__device__ __forceinline__ void dma_copy16v(const void* g, uint32_t lds_base)
+{
+    asm volatile("s_add_u32 m0, %0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" : : "s"(lds_base), "v"(g), "n"(LDS_IMM) : "memory", "m0", "scc");
+}
+
 template <int LDS_IMM>
 __device__ __forceinline__ void dma_copy16(const int8_t* sbase, uint32_t voff, uint32_t lds_base)
 {
@@ -71,13 +92,17 @@ __device__ __forceinline__ void dma_copy16(const int8_t* sbase, uint32_t voff, u
                  : : "s"(lds_base), "v"(voff), "s"(sbase), "n"(LDS_IMM) : "memory", "m0", "scc");
 }
 
-template <int FN, int OUT_DT, bool F8 = false>
+template <int FN, int OUT_DT, bool F8 = false, bool MXS = false>
 __global__ __launch_bounds__(256, 1) void qgemm_i8_wide_kernel(QgemmParams p, int tiles_m, int tiles_n)
 {
+    static_assert(!MXS || F8, "block scales ride on the fp8 form");
     constexpr int SLOTS = F8 ? 8 : 16;   // MFMAs per x2 fragment
     constexpr int NT = 256, BM = 256, TM = 128, FM = TM / 16, TN = 16 * FN, BN = 2 * TN, BK = 128, STAGES = 2;
     constexpr int CPR = BK / 16, RPW = 16 / CPR;
+    constexpr int NSC = MXS ? (BM + BN + NT - 1) / NT : 0;   // scale copies per thread and four K tiles: 16 bytes per tile row
     constexpr int A_BYTES = BM * BK, B_BYTES = BN * BK, STAGE = A_BYTES + B_BYTES;
+    constexpr int SC_RING = 2 * STAGE, SC_SLOT = NSC * NT * 16;   // two scale slots behind the operand stages
+    static_assert(SC_RING + 2 * SC_SLOT <= 163840, "operand stages and scale slots must fit into LDS");
     constexpr int RPI = NT / CPR;                 // 32 tile rows per copy instruction of the workgroup
     constexpr int NA = BM / RPI, NB = BN / RPI;   // 8 and FN
     constexpr int CPT = NA + NB;
@@ -123,12 +148,38 @@ __global__ __launch_bounds__(256, 1) void qgemm_i8_wide_kernel(QgemmParams p, in
         const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)u), hi = __builtin_amdgcn_readfirstlane((uint32_t)(u >> 32));
         return (const int8_t*)(((uint64_t)hi << 32) | lo);
     };
-    const uint32_t lds0 = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)smem) + wave * 1024;
+    const uint32_t lds_raw = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)smem);
+    const uint32_t lds0 = lds_raw + wave * 1024;
+    // MXFP8: scale copy `c` of this thread moves 16 scale bytes (four K tiles) of tile row c*NT + tid (x1 rows, then x2
+    // rows; rows past the tile repeat its last one into padding that nobody reads)
+    const uint8_t* sc_src[NSC > 0 ? NSC : 1];
+    if constexpr (MXS) {
+#pragma unroll
+        for (int c = 0; c < NSC; c++) {
+            const int r = c * NT + tid;
+            if (r < BM) {
+                const int rr = r < a_rows ? r : a_rows - 1;
+                sc_src[c] = p.sa + bz * p.sa_bs + (m0 + rr) * p.sa_rs;
+            } else {
+                int rr = r - BM;
+                rr = rr < b_rows ? rr : b_rows - 1;
+                sc_src[c] = p.sb + bz * p.sb_bs + (n0 + rr) * p.sb_rs;
+            }
+        }
+    }
     auto issue_piece = [&](int kt, int stage, auto idx_c) {
         constexpr int idx = decltype(idx_c)::value;
         const uint32_t sS = lds0 + stage * STAGE;
         if constexpr (idx < NA) dma_copy16<idx * NT * 16>(scalar_ptr(A + (int64_t)kt * BK), a_off[idx], sS);
         else dma_copy16<A_BYTES + (idx - NA) * NT * 16>(scalar_ptr(B + (int64_t)kt * BK), b_off[idx - NA], sS);
+    };
+    auto issue_scales = [&](int group) {   // the scales of K tiles 4*group .. 4*group+3 into slot group % 2
+        if constexpr (MXS) {
+            const uint32_t slot = lds0 + SC_RING + (group & 1) * SC_SLOT;
+            [&]<int... C>(std::integer_sequence<int, C...>) {
+                (dma_copy16v<C * NT * 16>(sc_src[C] + (int64_t)group * 16, slot), ...);
+            }(std::make_integer_sequence<int, NSC>{});
+        }
     };
     auto for_copies = [&](auto&& f) {   // f(integral_constant<int, c>) for c = 0 .. CPT-1
         [&]<int... C>(std::integer_sequence<int, C...>) { (f(std::integral_constant<int, C>{}), ...); }(std::make_integer_sequence<int, CPT>{});
@@ -162,6 +213,7 @@ __global__ __launch_bounds__(256, 1) void qgemm_i8_wide_kernel(QgemmParams p, in
     constexpr int SPREAD = 4;
     static_assert(SPREAD <= FN, "the copies are issued within one tile");
     issue_tile(0);
+    issue_scales(0);
     wait_vmcnt<0>();
     __builtin_amdgcn_s_barrier();
     // Fragments are kept as halves (lo: the first instruction's 64 bytes of K, hi: the second's), so that a half can be
@@ -175,6 +227,19 @@ __global__ __launch_bounds__(256, 1) void qgemm_i8_wide_kernel(QgemmParams p, in
     for (int j = 0; j < FM; j++) fal[j] = load_lo(smem, a_rowbase + j * 16 * BK);
 #pragma unroll
     for (int j = 0; j < FM; j++) fah[j] = load_hi(smem, a_rowbase + j * 16 * BK);
+    // MXFP8: the scale dword of this lane's row in each x1 fragment (raw, then shifted to this lane's block) and in the
+    // x2 fragments (alternating like fb)
+    uint32_t sar[FM], sca[FM], sbr[2];
+    (void)sar; (void)sca; (void)sbr;
+    // the scale dword of K tile kt for tile row r: slot (kt / 4) % 2, 16 bytes per row, dword kt % 4
+    auto scale_base = [&](int kt) -> const char* { return smem + SC_RING + ((kt >> 2) & 1) * SC_SLOT + (kt & 3) * 4; };
+    auto a_scale = [&](const char* sb, int j) -> uint32_t { return *(const uint32_t*)(sb + (wm * TM + j * 16 + frow) * 16); };
+    auto b_scale = [&](const char* sb, int i) -> uint32_t { return *(const uint32_t*)(sb + (BM + wn * TN + i * 16 + frow) * 16); };
+    if constexpr (MXS) {
+        sbr[FN & 1] = b_scale(scale_base(0), 0);
+#pragma unroll
+        for (int j = 0; j < FM; j++) sar[j] = a_scale(scale_base(0), j);
+    }
 
     for (int kt = 0; kt < KT; kt++) {
         const char* st = smem + (kt & 1) * STAGE;
@@ -193,13 +258,21 @@ __global__ __launch_bounds__(256, 1) void qgemm_i8_wide_kernel(QgemmParams p, in
                 if (i + 1 < FN) {
                     if (i == 0) {   // one instruction reads both halves of a fragment: everything requested so far is needed now
                         wait_lgkmcnt0();
-                        if (FN & 1) { fbl[0] = fbl[1]; fbh[0] = fbh[1]; }
+                        if (FN & 1) {
+                            fbl[0] = fbl[1]; fbh[0] = fbh[1];
+                            if constexpr (MXS) sbr[0] = sbr[1];
+                        }
+                        if constexpr (MXS) {
+#pragma unroll
+                            for (int j = 0; j < FM; j++) sca[j] = sar[j] >> (8 * fq);
+                        }
                         __builtin_amdgcn_sched_barrier(0);
                     }
                     fbl[(i + 1) & 1] = load_lo(st, b_rowbase + (i + 1) * 16 * BK);
                     fbh[(i + 1) & 1] = load_hi(st, b_rowbase + (i + 1) * 16 * BK);
+                    if constexpr (MXS) sbr[(i + 1) & 1] = b_scale(scale_base(kt), i + 1);
                     __builtin_amdgcn_sched_barrier(0);
-                    if (i > 0) __builtin_amdgcn_s_waitcnt(0xc07f | (2 << 8));
+                    if (i > 0) __builtin_amdgcn_s_waitcnt(0xc07f | ((MXS ? 3 : 2) << 8));   // all but the reads just issued
                 } else {
                     wait_vmcnt<0>();
                     wait_lgkmcnt0();
@@ -207,21 +280,36 @@ __global__ __launch_bounds__(256, 1) void qgemm_i8_wide_kernel(QgemmParams p, in
                     __builtin_amdgcn_sched_barrier(0);
                     fbl[(i + 1) & 1] = load_lo(stn, b_rowbase);
                     fbh[(i + 1) & 1] = load_hi(stn, b_rowbase);
+                    if constexpr (MXS) sbr[(i + 1) & 1] = b_scale(scale_base(kt + 1), 0);
                 }
                 __builtin_amdgcn_sched_barrier(0);
                 const v8i b8 = __builtin_shufflevector(fbl[i & 1], fbh[i & 1], 0, 1, 2, 3, 4, 5, 6, 7);
+                uint32_t scb = 0;
+                if constexpr (MXS) {
+                    scb = sbr[i & 1] >> (8 * fq);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
 #pragma unroll
                 for (int j = 0; j < FM; j++) {
                     const v8i a8 = __builtin_shufflevector(fal[j], fah[j], 0, 1, 2, 3, 4, 5, 6, 7);
-                    if constexpr (F8) {   // (the int8 instantiation never compiles this call)
+                    if constexpr (MXS) {
+                        if (i * FM + j < 64) mfma_f8_16x16x128_scaled<true>(acc[i][j], b8, a8, scb, sca[j]);
+                        else mfma_f8_16x16x128_scaled<false>(acc[i][j], b8, a8, scb, sca[j]);
+                    } else if constexpr (F8) {   // (the int8 instantiation never compiles this call)
                         if (i * FM + j < 64) mfma_f8_16x16x128<true>(acc[i][j], b8, a8);
                         else mfma_f8_16x16x128<false>(acc[i][j], b8, a8);
                     }
                     __builtin_amdgcn_sched_barrier(0);
                     spread_copies(i * SLOTS + j);
+                    if constexpr (MXS) {
+                        // first tile of a group of four: fetch the next group's scales, if there is one (its slot's last
+                        // reader was the tile before this one)
+                        if (i == SPREAD && j == 0 && (kt & 3) == 0 && kt + 4 < KT) issue_scales((kt >> 2) + 1);
+                    }
                     if (i == FN - 1) {
                         fal[j] = load_lo(stn, a_rowbase + j * 16 * BK);
                         fah[j] = load_hi(stn, a_rowbase + j * 16 * BK);
+                        if constexpr (MXS) sar[j] = a_scale(scale_base(kt + 1), j);
                     }
                     __builtin_amdgcn_sched_barrier(0);
                 }
@@ -298,8 +386,11 @@ __global__ __launch_bounds__(256, 1) void qgemm_i8_wide_kernel(QgemmParams p, in
             int64_t n = n0 + i;
             if (n >= p.N) n = p.N - 1;
             const int64_t si = p.x2s_len == 1 ? 0 : n;
-            float sv = p.x2s_dt == DT_U64 ? u2f((uint32_t)((const uint64_t*)p.x2s)[si]) : load_scalar_as_f32(p.x2s, p.x2s_dt, si);
-            if (p.x2s_trunc || p.x2s_dt == DT_U64) sv = u2f(f2u(sv) & 0xFFFFE000u);
+            float sv = 1.0f;
+            if constexpr (!MXS) {
+                sv = p.x2s_dt == DT_U64 ? u2f((uint32_t)((const uint64_t*)p.x2s)[si]) : load_scalar_as_f32(p.x2s, p.x2s_dt, si);
+                if (p.x2s_trunc || p.x2s_dt == DT_U64) sv = u2f(f2u(sv) & 0xFFFFE000u);
+            }
             sS2[i] = sv;
             sIb[i] = has_ib ? ((const int32_t*)p.bias)[bz * p.bias_bs + n] : 0;
             sFb[i] = has_fb ? load_scalar_as_f32(p.bias, p.bias_dt, bz * p.bias_bs + n) : -0.0f;
@@ -369,13 +460,13 @@ __global__ __launch_bounds__(256, 1) void qgemm_i8_wide_kernel(QgemmParams p, in
     }
 }
 
-template <int FN, int OUT_DT, bool F8 = false>
+template <int FN, int OUT_DT, bool F8 = false, bool MXS = false>
 static int launch_wide_one(const QgemmParams& p, int64_t batch, hipStream_t st)
 {
     constexpr int BM = 256, BN = 32 * FN, BK = 128;
     const int tiles_m = (int)((p.M + BM - 1) / BM), tiles_n = (int)((p.N + BN - 1) / BN);
-    const size_t lds = (size_t)2 * (BM + BN) * BK;
-    auto k = qgemm_i8_wide_kernel<FN, OUT_DT, F8>;
+    const size_t lds = (size_t)2 * (BM + BN) * BK + (MXS ? (size_t)2 * ((BM + BN + 255) / 256) * 4096 : 0);
+    auto k = qgemm_i8_wide_kernel<FN, OUT_DT, F8, MXS>;
     static bool attr_set = false;   // per instantiation; benign if two threads both set it
     if (!attr_set) {
         hipError_t e = hipFuncSetAttribute((const void*)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
@@ -417,6 +508,25 @@ int launch_f8_wide(const QgemmParams& p, int fn, int64_t batch, int out_dt, hipS
         case 9: return bf ? launch_wide_one<9, DT_BF16, true>(p, batch, st) : launch_wide_one<9, DT_F16, true>(p, batch, st);
         case 10: return bf ? launch_wide_one<10, DT_BF16, true>(p, batch, st) : launch_wide_one<10, DT_F16, true>(p, batch, st);
         case 11: return bf ? launch_wide_one<11, DT_BF16, true>(p, batch, st) : launch_wide_one<11, DT_F16, true>(p, batch, st);
+        default: return OPSNN_NOT_TAKEN;
+    }
+}
+
+}  // namespace opsnn
+
+namespace opsnn {
+
+// MXFP8: p.sa / p.sb (one e8m0 byte per 32 K elements, K-contiguous per row, 16-byte aligned rows), fp32 bias,
+// K % 512 == 0, fn 8 or 9.
+int launch_mxfp8_wide(const QgemmParams& p, int fn, int64_t batch, int out_dt, hipStream_t st)
+{
+    if (p.KB % 512 != 0 || p.KB < 512 || !p.sa || !p.sb) return OPSNN_NOT_TAKEN;
+    if (((uintptr_t)p.sa | (uintptr_t)p.sb | (uint64_t)p.sa_rs | (uint64_t)p.sb_rs | (uint64_t)p.sa_bs | (uint64_t)p.sb_bs) % 16) return OPSNN_NOT_TAKEN;
+    if (out_dt != DT_BF16 && out_dt != DT_F16) return OPSNN_NOT_TAKEN;
+    const bool bf = out_dt == DT_BF16;
+    switch (fn) {
+        case 8: return bf ? launch_wide_one<8, DT_BF16, true, true>(p, batch, st) : launch_wide_one<8, DT_F16, true, true>(p, batch, st);
+        case 9: return bf ? launch_wide_one<9, DT_BF16, true, true>(p, batch, st) : launch_wide_one<9, DT_F16, true, true>(p, batch, st);
         default: return OPSNN_NOT_TAKEN;
     }
 }

@@ -120,6 +120,31 @@ def test_mx(gpu, M, K, N, tB, fp4, use_plain):
     check_close(got, want, orc.BF16, "mx", exact=use_plain, fp8_mfma=not fp4, abs_sum=abs_sum)
 
 
+@pytest.mark.parametrize("fn", [8, 9])
+@pytest.mark.parametrize("M,K,N,tB,batch,bias", [
+    (300, 512, 700, True, 1, True),      # one group of four K tiles, ragged rows and columns
+    (512, 2048, 288, True, 1, False),    # four groups (both scale slots reused), exactly one tile at n = 9
+    (260, 1536, 1000, False, 2, True),   # three groups, N-contiguous x2 (re-laid out first), batched
+])
+def test_mxfp8_on_the_four_wave_kernel(gpu, fn, M, K, N, tB, batch, bias):
+    """MXFP8 forced onto the one-wave-per-SIMD kernel with 256 x 32n tiles, n = 8 or 9 (it is chosen by itself only for
+    problems of at least 3/4 of a round of CUs with K % 512 == 0): the bar of the default MXFP8 kernel (backward-error
+    bound, see check_close)."""
+    m = gpu
+    print(f"case mxfp8 four-wave kernel n={fn} M={M} K={K} N={N} tB={tB} batch={batch} bias={bias}", flush=True)
+    inp = cases.make_mx_inputs(m, M, K, N, fn + M, tB, False, batch=batch)
+    b = np.random.default_rng(2).normal(0, 1, N).astype(np.float32) if bias else None
+    want = cases.oracle_mx(m, inp, M, K, N, tB, m.ACL_BF16, b)
+    pos = dict(inp, x1=inp["x1"] & 0x7F, x2=inp["x2"] & 0x7F)
+    abs_sum = orc.b16_to_f32(cases.oracle_mx(m, pos, M, K, N, tB, m.ACL_BF16), orc.BF16).astype(np.float64)
+    os.environ["OPSNN_MX8_WIDE"] = str(fn)
+    try:
+        got = cases.run_mx_aclnn(m, inp, M, K, N, tB, m.ACL_BF16, b)
+    finally:
+        os.environ.pop("OPSNN_MX8_WIDE", None)
+    check_close(got, want, orc.BF16, "mxfp8 four-wave", fp8_mfma=True, abs_sum=abs_sum)
+
+
 @pytest.mark.parametrize("M,K,N,batch", [(96, 256, 128, 3), (256, 1024, 264, 2)])
 def test_mx_batched(gpu, M, K, N, batch):
     m = gpu
