@@ -17,7 +17,8 @@
 //   - the loop is software-pipelined: the barrier sits in front of the last x2 fragment of a tile, and in the shadow of
 //     that fragment's 16 MFMAs the wave requests the next tile's first x2 fragment and its x1 fragments, each half of
 //     a fragment as soon as the last MFMA that reads the old half has been issued; the next tile then starts on the
-//     halves that came first (lgkmcnt counts, never "wait for everything");
+//     halves that came first (lgkmcnt counts, never "wait for everything"; the fp8 forms read whole fragments per
+//     instruction and do wait for all of them at the start of a tile);
 //   - the global -> LDS copies are written as inline assembly, because of what the compiler does with the builtin (see
 //     dma_copy16), and are spread over the first fragments of the tile instead of being issued in one burst;
 //   - two stages of (256 + 32*FN) x 128 bytes fill the LDS (155,648 of 163,840 bytes at FN = 11): the copies of tile
@@ -58,11 +59,6 @@ __device__ __forceinline__ void mfma_i8_16x16x64(v4i& c, const v4i a, const v4i 
     else asm volatile("v_mfma_i32_16x16x64_i8 %0, %1, %2, %0" : "+v"(c) : "v"(a), "v"(b));
 }
 
-// 16-byte asynchronous copy global -> LDS, written out: lane l reads sbase + voff(l) and lands at lds_base + LDS_IMM + 16*l.
-// Through the builtin the compiler's wait-count pass sees an instruction that touches both memory paths and from then
-// on answers every dependency on an LDS read with a wait for ALL outstanding reads, including the ones issued a moment
-// ago for the next fragment; hidden from it, the pass counts exactly.  The copies' own completion is waited for
-// explicitly (vmcnt + barrier) wherever LDS is read.
 // acc += a (16 x 128 fp8 e4m3) x b (128 x 16 fp8 e4m3), fp32 sums; see mfma_i8_16x16x64 for the register classes
 template <bool AG>
 __device__ __forceinline__ void mfma_f8_16x16x128(v4f& c, const v8i a, const v8i b)
@@ -71,6 +67,7 @@ __device__ __forceinline__ void mfma_f8_16x16x128(v4f& c, const v8i a, const v8i
     else asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, %0" : "+v"(c) : "v"(a), "v"(b));
 }
 
+// the scaled form: sa / sb hold, in their low byte, the e8m0 scale of this lane's 32-element block of a / b
 template <bool AG>
 __device__ __forceinline__ void mfma_f8_16x16x128_scaled(v4f& c, const v8i a, const v8i b, uint32_t sa, uint32_t sb)
 {
@@ -78,18 +75,23 @@ __device__ __forceinline__ void mfma_f8_16x16x128_scaled(v4f& c, const v8i a, co
     else asm volatile("v_mfma_scale_f32_16x16x128_f8f6f4 %0, %1, %2, %0, %3, %4 op_sel_hi:[0,0,0]" : "+v"(c) : "v"(a), "v"(b), "v"(sa), "v"(sb));
 }
 
-// the same copy with a 64-bit address per lane (dma_copy16 below: scalar base + 32-bit lane offset)
-template <int LDS_IMM>
-__device__ __forceinline__ void dma_copy16v(const void* g, uint32_t lds_base)
-{
-    asm volatile("s_add_u32 m0, %0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" : : "s"(lds_base), "v"(g), "n"(LDS_IMM) : "memory", "m0", "scc");
-}
-
+// 16-byte asynchronous copy global -> LDS, written out: lane l reads sbase + voff(l) and lands at lds_base + LDS_IMM + 16*l.
+// Through the builtin the compiler's wait-count pass sees an instruction that touches both memory paths and from then
+// on answers every dependency on an LDS read with a wait for ALL outstanding reads, including the ones issued a moment
+// ago for the next fragment; hidden from it, the pass counts exactly.  The copies' own completion is waited for
+// explicitly (vmcnt + barrier) wherever LDS is read.
 template <int LDS_IMM>
 __device__ __forceinline__ void dma_copy16(const int8_t* sbase, uint32_t voff, uint32_t lds_base)
 {
     asm volatile("s_add_u32 m0, %0, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
                  : : "s"(lds_base), "v"(voff), "s"(sbase), "n"(LDS_IMM) : "memory", "m0", "scc");
+}
+
+// the same copy with a 64-bit address per lane
+template <int LDS_IMM>
+__device__ __forceinline__ void dma_copy16v(const void* g, uint32_t lds_base)
+{
+    asm volatile("s_add_u32 m0, %0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" : : "s"(lds_base), "v"(g), "n"(LDS_IMM) : "memory", "m0", "scc");
 }
 
 template <int FN, int OUT_DT, bool F8 = false, bool MXS = false>
