@@ -41,7 +41,8 @@ struct Fp8BlkParams {
     const uint8_t* sa;
     const uint8_t* sb;
     int64_t sa_rs, sb_rs, sa_bs, sb_bs;
-    const float* bias;
+    const float* bias;   // FP8_MX_W4: elements of bias_dt (fp32 or 16-bit)
+    int bias_dt;
     int64_t bias_bs;
     // row / column scale mode (fp8 K-C, K-T and the double-scale modes that multiply separately):
     // out = (sum * cs[n * cs_stride]) * rs[m * rs_stride] + bias[n]; strides 0 (one scale) or 1
@@ -68,23 +69,26 @@ __device__ __forceinline__ const int8_t* scalar_ptr(const int8_t* p)
     return (const int8_t*)(((uint64_t)hi << 32) | lo);
 }
 
-enum : int { FP8_BLOCK = 0, FP8_MX = 1, FP8_ROWCOL = 2 };
+enum : int { FP8_BLOCK = 0, FP8_MX = 1, FP8_ROWCOL = 2, FP8_MX_W4 = 3 };
 
 template <int WGM, int STAGES, int OUT_DT, int MODE = FP8_BLOCK>
 __global__ __launch_bounds__(WGM * 128, 1) void qmm_fp8_block_kernel(Fp8BlkParams p, int tiles_m, int tiles_n)
 {
-    constexpr bool MX = MODE == FP8_MX;        // e8m0 scales inside the instruction
+    constexpr bool W4 = MODE == FP8_MX_W4;     // MX with fp4 e2m1 x2 (fp8 x fp4): x2 rows are 64 bytes per K tile
+    constexpr bool MX = MODE == FP8_MX || W4;  // e8m0 scales inside the instruction
     constexpr bool RC = MODE == FP8_ROWCOL;    // plain fp8 products, one scale per row and per column in the epilogue
     constexpr bool BLK = MODE == FP8_BLOCK;    // fp32 block scales folded in by the vector ALU
     static_assert(!MX || WGM == 4, "MX mode: one scale copy per thread covers the 256 + 256 rows of the tile");
     constexpr int BM = 64 * WGM, BN = 256, BK = 128, NT = WGM * 128;   // WGM x 2 waves of 64 x 128 each
     constexpr int CPR = BK / 16, RPW = 16 / CPR;
     constexpr int TM = 64, TN = 128, FM = TM / 16, FN = TN / 16;      // 4 x 8 fragments of 16 x 16 per wave
-    constexpr int A_BYTES = BM * BK, B_BYTES = BN * BK;
+    constexpr int BKB = W4 ? BK / 2 : BK;        // bytes of an x2 row per K tile
+    constexpr int CPRB = BKB / 16, RPWB = 16 / CPRB;
+    constexpr int A_BYTES = BM * BK, B_BYTES = BN * BKB;
     constexpr int SC_BYTES = NT * 4;             // BM s1 floats + 2 s2 floats, one 4-byte copy per lane
     constexpr int STAGE = A_BYTES + B_BYTES + SC_BYTES;
-    constexpr int RPI = NT / CPR;                // rows per copy instruction of the workgroup
-    constexpr int NA = BM / RPI, NB = BN / RPI;
+    constexpr int RPI = NT / CPR, RPIB = NT / CPRB;   // rows per copy instruction of the workgroup
+    constexpr int NA = BM / RPI, NB = BN / RPIB;
     constexpr int CPT = NA + NB + (RC ? 0 : 1);   // operand copies and, unless the scales wait for the epilogue, one scale copy
     static_assert(STAGES * CPT < 64, "stage count");
     extern __shared__ __attribute__((aligned(16))) char smem[];
@@ -118,11 +122,13 @@ __global__ __launch_bounds__(WGM * 128, 1) void qmm_fp8_block_kernel(Fp8BlkParam
         r = r < a_rows ? r : a_rows - 1;
         a_off[i] = (uint32_t)(r * lda + cchunk * 16);
     }
+    const int crowb = tid / CPRB;
+    const int cchunkb = (tid % CPRB) ^ ((crowb / RPWB) & (CPRB - 1));
 #pragma unroll
     for (int i = 0; i < NB; i++) {
-        int r = i * RPI + crow;
+        int r = i * RPIB + crowb;
         r = r < b_rows ? r : b_rows - 1;
-        b_off[i] = (uint32_t)(r * ldb + cchunk * 16);
+        b_off[i] = (uint32_t)(r * ldb + cchunkb * 16);
     }
     // Scale copy: lanes 0..BM-1 fetch s1 of tile row `tid`, lanes BM, BM+1 fetch s2 of the tile's two n blocks,
     // the rest re-fetch a valid word (their LDS slots are never read).
@@ -163,7 +169,7 @@ __global__ __launch_bounds__(WGM * 128, 1) void qmm_fp8_block_kernel(Fp8BlkParam
         char* sA = smem + stage * STAGE + wave * 1024;
         char* sB = sA + A_BYTES;
         const int8_t* Ak = scalar_ptr(A + (int64_t)kt * BK);
-        const int8_t* Bk = scalar_ptr(B + (int64_t)kt * BK);
+        const int8_t* Bk = scalar_ptr(B + (int64_t)kt * BKB);
         if (idx < NA) async_copy16(Ak + a_off[idx], sA + idx * NT * 16);
         else if (idx < NA + NB) async_copy16(Bk + b_off[idx - NA], sB + (idx - NA) * NT * 16);
         else async_copy4(sc_src + (int64_t)kt * sc_step, smem + stage * STAGE + A_BYTES + B_BYTES + wave * 256);
@@ -186,7 +192,7 @@ __global__ __launch_bounds__(WGM * 128, 1) void qmm_fp8_block_kernel(Fp8BlkParam
     const int key = (frow / RPW) & (CPR - 1);
     const int ch0 = ((2 * fq) ^ key) << 4, ch1 = ((2 * fq + 1) ^ key) << 4;
     const int a_rowbase = (wm * TM + frow) * BK;
-    const int b_rowbase = A_BYTES + (wn * TN + frow) * BK;
+    const int b_rowbase = A_BYTES + (wn * TN + frow) * BKB;
     // MX mode, where the position of K matters: the instruction takes registers 0..3 of lane group q as the 16 elements
     // [16q, 16q+16) of K and registers 4..7 as [64+16q, 64+16q+16), so the 32-element block b lies in lane groups
     // 2(b%2), 2(b%2)+1, register half b/2 -- and it is scaled by the scale byte that the lanes of GROUP b supply
@@ -196,6 +202,20 @@ __global__ __launch_bounds__(WGM * 128, 1) void qmm_fp8_block_kernel(Fp8BlkParam
         const v4i lo = *(const v4i*)(st + rowbase + (MX ? mx0 : ch0));
         const v4i hi = *(const v4i*)(st + rowbase + (MX ? mx1 : ch1));
         return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+    };
+    // fp4 x2 fragment (W4): a 4-bit operand is four registers, and lane group q holds the 32 CONSECUTIVE elements
+    // [32q, 32q+32) of K in them (block q, scaled by its own lanes' byte) -- unlike the 8-bit operand above, whose
+    // groups hold two runs of 16.  Measured with one-hot operands: the instruction pairs K indices, not lane groups.
+    // Rows are stored in four 16-byte pieces, piece c at position c ^ (row / 4) % 4.
+    const int keyb = (frow / RPWB) & (CPRB - 1);
+    const int w4off = (fq ^ keyb) << 4;
+    auto load_frag_b = [&](const char* st, int rowbase) -> v8i {
+        if constexpr (W4) {
+            const v4i lo = *(const v4i*)(st + rowbase + w4off);
+            return (v8i){lo[0], lo[1], lo[2], lo[3], 0, 0, 0, 0};
+        } else {
+            return load_frag(st, rowbase);
+        }
     };
 
     // Pipeline (two stages).  The loop is rotated: on entry to tile kt its x1 fragments, its first x2 fragment and its
@@ -246,7 +266,7 @@ __global__ __launch_bounds__(WGM * 128, 1) void qmm_fp8_block_kernel(Fp8BlkParam
         read_scales(st);
 #pragma unroll
         for (int j = 0; j < FM; j++) fa[j] = load_frag(st, a_rowbase + j * 16 * BK);
-        fb[0] = load_frag(st, b_rowbase);
+        fb[0] = load_frag_b(st, b_rowbase);
         if constexpr (MX) sbraw[0] = read_bscale(st, 0);
 #pragma unroll
         for (int j = 0; j < FM; j++) {
@@ -264,10 +284,10 @@ __global__ __launch_bounds__(WGM * 128, 1) void qmm_fp8_block_kernel(Fp8BlkParam
 #pragma unroll
         for (int i = 0; i < FN; i++) {
             if (i + 1 < FN) {
-                fb[(i + 1) & 1] = load_frag(st, b_rowbase + (i + 1) * 16 * BK);
+                fb[(i + 1) & 1] = load_frag_b(st, b_rowbase + (i + 1) * 16 * BKB);
                 if constexpr (MX) sbraw[(i + 1) & 1] = read_bscale(st, i + 1);
                 __builtin_amdgcn_sched_barrier(0);
-                __builtin_amdgcn_s_waitcnt(0xc07f | ((MX ? 3 : 2) << 8));   // lgkmcnt: all but the reads just issued
+                __builtin_amdgcn_s_waitcnt(0xc07f | ((MX && !W4 ? 3 : 2) << 8));   // lgkmcnt: all but the reads just issued
             } else {
 #if QG_DBG
                 wait_lgkmcnt0();
@@ -285,7 +305,7 @@ __global__ __launch_bounds__(WGM * 128, 1) void qmm_fp8_block_kernel(Fp8BlkParam
 #endif
                 __builtin_amdgcn_sched_barrier(0);
                 read_scales(stn);
-                fb[0] = load_frag(stn, b_rowbase);
+                fb[0] = load_frag_b(stn, b_rowbase);
                 if constexpr (MX) sbraw[0] = read_bscale(stn, 0);
             }
             __builtin_amdgcn_sched_barrier(0);
@@ -301,7 +321,7 @@ __global__ __launch_bounds__(WGM * 128, 1) void qmm_fp8_block_kernel(Fp8BlkParam
 #pragma unroll
             for (int j = 0; j < FM; j++) {
                 if constexpr (MX)   // the instruction applies both scales: accumulate in place, nothing to fold
-                    acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(fb[i & 1], fa[j], acc[i][j], 0, 0, 0, (int)scb, 0, (int)sca[j]);
+                    acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(fb[i & 1], fa[j], acc[i][j], W4 ? 4 : 0, 0, 0, (int)scb, 0, (int)sca[j]);
                 else if constexpr (RC)
                     acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(fb[i & 1], fa[j], acc[i][j], 0, 0, 0, 0x7f7f7f7f, 0, 0x7f7f7f7f);
                 else
@@ -383,7 +403,10 @@ __global__ __launch_bounds__(WGM * 128, 1) void qmm_fp8_block_kernel(Fp8BlkParam
                 if (p.bias) {
                     const int64_t nb = n0 + wn * TN + i * 16 + 4 * fq;
 #pragma unroll
-                    for (int r = 0; r < 4; r++) v[r] = v[r] + p.bias[bz * p.bias_bs + (nb + r < p.N ? nb + r : p.N - 1)];
+                    for (int r = 0; r < 4; r++) {
+                        const int64_t bi = bz * p.bias_bs + (nb + r < p.N ? nb + r : p.N - 1);
+                        v[r] = v[r] + (W4 ? load_scalar_as_f32(p.bias, p.bias_dt, bi) : p.bias[bi]);
+                    }
                 }
             }
             *(v4us_a*)(ep + frow * EP_PITCH + (i * 16 + 4 * fq) * 2) = pack4_b16<OUT_DT>(v);
@@ -425,7 +448,7 @@ static int launch_fp8_block(const Fp8BlkParams& p, int64_t batch, hipStream_t st
     constexpr int BM = 64 * WGM;
     int tiles_m = (int)((p.M + BM - 1) / BM), tiles_n = (int)((p.N + 255) / 256);
     dim3 grid((unsigned)(tiles_m * tiles_n), (unsigned)batch);
-    size_t lds = (size_t)STAGES * ((BM + 256) * 128 + WGM * 128 * 4);
+    size_t lds = (size_t)STAGES * (BM * 128 + 256 * (MODE == FP8_MX_W4 ? 64 : 128) + WGM * 128 * 4);
     auto k = qmm_fp8_block_kernel<WGM, STAGES, OUT_DT, MODE>;
     static bool attr_set = false;
     if (!attr_set) {
@@ -494,6 +517,32 @@ int launch_mxfp8_mfma(const OpsnnQmmArgs& a, hipStream_t st)
 }
 
 int launch_f8_wide(const QgemmParams& p, int fn, int64_t batch, int out_dt, hipStream_t st);   // qmm_int8_wide.hip
+
+// fp8 e4m3 x fp4 e2m1 with e8m0 scales per 32 K on both operands (compute_mx of quant_batch_matmul_v4,
+// qbmmv4_kernel_golden.py:119-186): the MX mode with a 4-bit x2.  x2 [N, K] K-contiguous (two elements per byte),
+// K % 128 == 0, bias fp32 or 16-bit.
+int launch_mx_a8w4_mfma(const OpsnnQmmArgs& a, hipStream_t st)
+{
+    if (a.x1_dtype != DT_E4M3 || a.x2_dtype != DT_E2M1) return OPSNN_NOT_TAKEN;
+    if (a.out_dtype != DT_BF16 && a.out_dtype != DT_F16) return OPSNN_NOT_TAKEN;
+    if (a.K % 128 != 0 || a.M * a.N < 64 * 64 || a.x1.col_stride != 1 || a.x2.row_stride != 1) return OPSNN_NOT_TAKEN;
+    if (a.x1_scale_mat.col_stride != 2 || a.x2_scale_mat.col_stride != 2) return OPSNN_NOT_TAKEN;
+    if (a.bias && a.bias_dtype != DT_F32 && a.bias_dtype != DT_BF16 && a.bias_dtype != DT_F16) return OPSNN_NOT_TAKEN;
+    Fp8BlkParams p{};
+    p.a = (const int8_t*)a.x1.ptr; p.b = (const int8_t*)a.x2.ptr;
+    p.lda = a.x1.row_stride; p.ldb = a.x2.col_stride / 2;   // bytes per x2 row
+    p.a_bs = a.x1.batch_stride; p.b_bs = a.x2.batch_stride / 2;
+    p.out = a.out; p.M = a.M; p.N = a.N; p.K = a.K; p.gsM = 1;
+    p.sa = (const uint8_t*)a.x1_scale_mat.ptr; p.sb = (const uint8_t*)a.x2_scale_mat.ptr;
+    p.sa_rs = a.x1_scale_mat.row_stride; p.sb_rs = a.x2_scale_mat.row_stride;
+    p.sa_bs = a.x1_scale_mat.batch_stride; p.sb_bs = a.x2_scale_mat.batch_stride;
+    p.bias = (const float*)a.bias; p.bias_dt = a.bias_dtype; p.bias_bs = a.bias_batch_stride;
+    if (a.x2.col_stride % 2) return OPSNN_NOT_TAKEN;
+    if (((uintptr_t)p.a | (uintptr_t)p.b | (uint64_t)p.lda | (uint64_t)p.ldb | (uint64_t)p.a_bs | (uint64_t)p.b_bs) % 16) return OPSNN_NOT_TAKEN;
+    if (((uintptr_t)p.sa | (uintptr_t)p.sb | (uint64_t)p.sa_rs | (uint64_t)p.sb_rs | (uint64_t)p.sa_bs | (uint64_t)p.sb_bs) % 4) return OPSNN_NOT_TAKEN;
+    if (a.out_dtype == DT_BF16) return launch_fp8_block<4, 2, DT_BF16, FP8_MX_W4>(p, a.batch, st);
+    return launch_fp8_block<4, 2, DT_F16, FP8_MX_W4>(p, a.batch, st);
+}
 
 // fp8 e4m3 x e4m3 with one fp32 scale per row of x1 (or one for all of it) and one per column of x2 (or one):
 // K-C, K-T and the double-scale modes whose two scales are multiplied in separately

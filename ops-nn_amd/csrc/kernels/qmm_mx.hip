@@ -53,12 +53,14 @@ uint64_t mx_workspace_bytes(const OpsnnQmmArgs& a)
 }
 
 int launch_mxfp8_mfma(const OpsnnQmmArgs& a, hipStream_t st);   // qmm_fp8_block.hip
+int launch_mx_a8w4_mfma(const OpsnnQmmArgs& a, hipStream_t st);   // qmm_fp8_block.hip
 
 int launch_mx_mfma(const OpsnnQmmArgs& a0, hipStream_t st)
 {
     OpsnnQmmArgs a = a0;
     const bool fp4 = a.x1_dtype == DT_E2M1 && a.x2_dtype == DT_E2M1;
     const bool fp8 = a.x1_dtype == DT_E4M3 && a.x2_dtype == DT_E4M3;
+    if (a.x1_dtype == DT_E4M3 && a.x2_dtype == DT_E2M1) return launch_mx_a8w4_mfma(a, st);   // fp8 x fp4: qmm_fp8_block.hip
     if (!fp4 && !fp8) return OPSNN_NOT_TAKEN;
     // MXFP8 runs on the block kernel of qmm_fp8_block.hip in MX mode (16x16x128 instructions, 64 x 128 per wave, the
     // pipeline tuned for the fp8 block-scale path); the 32x32x64 tile kernel stays available on request
