@@ -69,7 +69,7 @@ __device__ __forceinline__ const int8_t* scalar_ptr(const int8_t* p)
     return (const int8_t*)(((uint64_t)hi << 32) | lo);
 }
 
-enum : int { FP8_BLOCK = 0, FP8_MX = 1, FP8_ROWCOL = 2, FP8_MX_W4 = 3 };
+enum : int { FP8_BLOCK = 0, FP8_MX = 1, FP8_ROWCOL = 2, FP8_MX_W4 = 3, I8_BLOCK = 4 };
 
 template <int WGM, int STAGES, int OUT_DT, int MODE = FP8_BLOCK>
 __global__ __launch_bounds__(WGM * 128, 1) void qmm_fp8_block_kernel(Fp8BlkParams p, int tiles_m, int tiles_n)
@@ -77,7 +77,8 @@ __global__ __launch_bounds__(WGM * 128, 1) void qmm_fp8_block_kernel(Fp8BlkParam
     constexpr bool W4 = MODE == FP8_MX_W4;     // MX with fp4 e2m1 x2 (fp8 x fp4): x2 rows are 64 bytes per K tile
     constexpr bool MX = MODE == FP8_MX || W4;  // e8m0 scales inside the instruction
     constexpr bool RC = MODE == FP8_ROWCOL;    // plain fp8 products, one scale per row and per column in the epilogue
-    constexpr bool BLK = MODE == FP8_BLOCK;    // fp32 block scales folded in by the vector ALU
+    constexpr bool I8 = MODE == I8_BLOCK;      // int8 operands with the block scales of FP8_BLOCK ("per-tile" of quant_batch_matmul_v4)
+    constexpr bool BLK = MODE == FP8_BLOCK || I8;   // fp32 block scales folded in by the vector ALU
     static_assert(!MX || WGM == 4, "MX mode: one scale copy per thread covers the 256 + 256 rows of the tile");
     constexpr int BM = 64 * WGM, BN = 256, BK = 128, NT = WGM * 128;   // WGM x 2 waves of 64 x 128 each
     constexpr int CPR = BK / 16, RPW = 16 / CPR;
@@ -244,7 +245,8 @@ __global__ __launch_bounds__(WGM * 128, 1) void qmm_fp8_block_kernel(Fp8BlkParam
     float sc[FM], s1raw[FM], s2raw;          // block-scale mode
     uint32_t sca[FM], saraw[FM], sbraw[2];   // MX mode: this lane's scale byte sits in bits 0..7 once shifted by 8 * fq
     (void)sc; (void)s1raw; (void)s2raw; (void)sca; (void)saraw; (void)sbraw;
-    v4f part[2][FM];
+    using part_t = std::conditional_t<I8, v4i, v4f>;   // a block's partial sums: exact int32 for int8 operands
+    part_t part[2][FM];
     auto read_scales = [&](const char* st) {
         if constexpr (RC) {
         } else if constexpr (MX) {
@@ -271,7 +273,7 @@ __global__ __launch_bounds__(WGM * 128, 1) void qmm_fp8_block_kernel(Fp8BlkParam
 #pragma unroll
         for (int j = 0; j < FM; j++) {
             sc[j] = 0.0f;   // multiplies the zero partial sums in the first tile's first fragment
-            part[1][j] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
+            part[1][j] = part_t{0, 0, 0, 0};
         }
     }
     constexpr int CPS = (CPT + FM - 1) / FM;   // copies issued behind each of the last fragment's MFMAs
@@ -324,7 +326,12 @@ __global__ __launch_bounds__(WGM * 128, 1) void qmm_fp8_block_kernel(Fp8BlkParam
                     acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(fb[i & 1], fa[j], acc[i][j], W4 ? 4 : 0, 0, 0, (int)scb, 0, (int)sca[j]);
                 else if constexpr (RC)
                     acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(fb[i & 1], fa[j], acc[i][j], 0, 0, 0, 0x7f7f7f7f, 0, 0x7f7f7f7f);
-                else
+                else if constexpr (I8) {   // two 64-byte steps; the block's integer sum is exact
+                    const v4i t = __builtin_amdgcn_mfma_i32_16x16x64_i8(__builtin_shufflevector(fb[i & 1], fb[i & 1], 0, 1, 2, 3),
+                                                                        __builtin_shufflevector(fa[j], fa[j], 0, 1, 2, 3), v4i{0, 0, 0, 0}, 0, 0, 0);
+                    part[i & 1][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(__builtin_shufflevector(fb[i & 1], fb[i & 1], 4, 5, 6, 7),
+                                                                           __builtin_shufflevector(fa[j], fa[j], 4, 5, 6, 7), t, 0, 0, 0);
+                } else
                     part[i & 1][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(fb[i & 1], fa[j], v4f{0.0f, 0.0f, 0.0f, 0.0f}, 0, 0, 0,
                                                                                       0x7f7f7f7f, 0, 0x7f7f7f7f);
                 __builtin_amdgcn_sched_barrier(0);
@@ -337,10 +344,10 @@ __global__ __launch_bounds__(WGM * 128, 1) void qmm_fp8_block_kernel(Fp8BlkParam
                 if constexpr (!BLK) {
                 } else if (i > 0) {
 #pragma unroll
-                    for (int r = 0; r < 4; r++) acc[i - 1][j][r] = __builtin_fmaf(part[(i - 1) & 1][j][r], sc[j], acc[i - 1][j][r]);
+                    for (int r = 0; r < 4; r++) acc[i - 1][j][r] = __builtin_fmaf((float)part[(i - 1) & 1][j][r], sc[j], acc[i - 1][j][r]);
                 } else {   // the previous tile's last fragment, still with that tile's scales
 #pragma unroll
-                    for (int r = 0; r < 4; r++) acc[FN - 1][j][r] = __builtin_fmaf(part[1][j][r], sc[j], acc[FN - 1][j][r]);
+                    for (int r = 0; r < 4; r++) acc[FN - 1][j][r] = __builtin_fmaf((float)part[1][j][r], sc[j], acc[FN - 1][j][r]);
                 }
                 __builtin_amdgcn_sched_barrier(0);
             }
@@ -355,7 +362,7 @@ __global__ __launch_bounds__(WGM * 128, 1) void qmm_fp8_block_kernel(Fp8BlkParam
     for (int j = 0; j < FM; j++) {
         if constexpr (BLK) {
 #pragma unroll
-            for (int r = 0; r < 4; r++) acc[FN - 1][j][r] = __builtin_fmaf(part[1][j][r], sc[j], acc[FN - 1][j][r]);
+            for (int r = 0; r < 4; r++) acc[FN - 1][j][r] = __builtin_fmaf((float)part[1][j][r], sc[j], acc[FN - 1][j][r]);
         }
     }
     wait_lgkmcnt0();   // the reads and copies past the last tile land before LDS is reused
@@ -399,7 +406,7 @@ __global__ __launch_bounds__(WGM * 128, 1) void qmm_fp8_block_kernel(Fp8BlkParam
                     v[r] = (v[r] * c) * rs_j[j];
                 }
             }
-            if constexpr (MX || RC) {
+            if constexpr (MX || RC || I8) {
                 if (p.bias) {
                     const int64_t nb = n0 + wn * TN + i * 16 + 4 * fq;
 #pragma unroll
@@ -606,9 +613,10 @@ int launch_fp8_rowcol_mfma(const OpsnnQmmArgs& a, hipStream_t st)
 int launch_blockscale_mfma(const OpsnnQmmArgs& a0, hipStream_t st)
 {
     OpsnnQmmArgs a = a0;
-    if (a.x1_dtype != DT_E4M3 || a.x2_dtype != DT_E4M3) return OPSNN_NOT_TAKEN;
+    const bool i8 = a.x1_dtype == DT_I8 && a.x2_dtype == DT_I8;   // the per-tile mode of quant_batch_matmul_v4 (qbmmv4_kernel_golden.py:258-325)
+    if (!i8 && (a.x1_dtype != DT_E4M3 || a.x2_dtype != DT_E4M3)) return OPSNN_NOT_TAKEN;
     if (a.out_dtype != DT_BF16 && a.out_dtype != DT_F16) return OPSNN_NOT_TAKEN;
-    if (a.bias) return OPSNN_NOT_TAKEN;
+    if (a.bias && !(i8 && a.bias_dtype == DT_F32)) return OPSNN_NOT_TAKEN;
     if (a.gsK != 128 || a.gsN != 128 || (a.gsM != 1 && a.gsM != 128)) return OPSNN_NOT_TAKEN;
     if (a.K % 128 != 0 || a.M * a.N < 64 * 64 || a.x1.col_stride != 1) return OPSNN_NOT_TAKEN;
     if (a.x2.row_stride != 1) {
@@ -629,11 +637,16 @@ int launch_blockscale_mfma(const OpsnnQmmArgs& a0, hipStream_t st)
     p.s2 = (const float*)a.x2_scale_mat.ptr; p.s2_rs = a.x2_scale_mat.row_stride; p.s2_cs = a.x2_scale_mat.col_stride;
     p.s2_bs = a.x2_scale_mat.batch_stride;
     p.gsM = (int)a.gsM;
+    p.bias = (const float*)a.bias; p.bias_dt = DT_F32; p.bias_bs = a.bias_batch_stride;
     if (((uintptr_t)p.a | (uintptr_t)p.b | (uint64_t)p.lda | (uint64_t)p.ldb | (uint64_t)p.a_bs | (uint64_t)p.b_bs) % 16) return OPSNN_NOT_TAKEN;
     if (((uintptr_t)p.s1 | (uintptr_t)p.s2) % 4) return OPSNN_NOT_TAKEN;
     // 256 x 256 tiles (8 waves) halve the operand traffic per flop; 128 x 256 (4 waves) keeps small M efficient
     static const int ev = [] { const char* e = getenv("OPSNN_FP8_WGM"); return e ? atoi(e) : 0; }();
     const bool big = ev ? ev == 4 : a.M >= 512;
+    if (i8) {
+        if (big) return a.out_dtype == DT_BF16 ? launch_fp8_block<4, 2, DT_BF16, I8_BLOCK>(p, a.batch, st) : launch_fp8_block<4, 2, DT_F16, I8_BLOCK>(p, a.batch, st);
+        return a.out_dtype == DT_BF16 ? launch_fp8_block<2, 2, DT_BF16, I8_BLOCK>(p, a.batch, st) : launch_fp8_block<2, 2, DT_F16, I8_BLOCK>(p, a.batch, st);
+    }
     if (big) {
         if (a.out_dtype == DT_BF16) return launch_fp8_block<4, 2, DT_BF16>(p, a.batch, st);
         return launch_fp8_block<4, 2, DT_F16>(p, a.batch, st);

@@ -189,6 +189,31 @@ def test_gpu_pertile_i8(gpu, M, K, N, tB):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("M,K,N,tB", [(128, 256, 256, True), (300, 384, 260, True), (640, 1024, 520, False)])
+def test_gpu_pertile_i8_on_the_matrix_cores(gpu, M, K, N, tB):
+    """int8 per-tile with K % 128 == 0 and enough outputs runs on the block-scale kernel with int8 instructions: the
+    block sums are exact integers, the fold into the running sum is a fused multiply-add (one rounding where the oracle
+    has two), so the bar is max rel <= 2^-7 and mean rel <= 2^-10; forced onto the plain kernel the call is bit-identical."""
+    import os
+    m = gpu
+    print(f"case int8 per-tile mfma {M}x{K}x{N} tB={tB}", flush=True)
+    inp = cases.make_pertile_i8_inputs(m, M, K, N, M + N, tB)
+    want = cases.oracle_pertile_i8(m, inp, M, K, N, tB, m.ACL_BF16)
+    got = cases.run_pertile_i8_aclnn(m, inp, M, K, N, tB, m.ACL_BF16)
+    g, w = orc.b16_to_f32(got, orc.BF16), orc.b16_to_f32(want, orc.BF16)
+    assert np.isfinite(g).all()
+    mx, mean = orc.rel_err_stats(g, w)
+    assert mx <= 2.0 ** -7 and mean <= 2.0 ** -10, f"max rel {mx:.3e} mean rel {mean:.3e}"
+    assert orc.isclose_fraction(g, w) <= 1e-3
+    os.environ["OPSNN_FORCE_PLAIN"] = "1"
+    try:
+        exact = cases.run_pertile_i8_aclnn(m, inp, M, K, N, tB, m.ACL_BF16)
+    finally:
+        os.environ.pop("OPSNN_FORCE_PLAIN", None)
+    assert np.array_equal(exact, want)
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("M,K,N,out_dt", [(9, 1024, 256, "bf16"), (9, 1024, 256, "f16"), (33, 2048, 512, "bf16")])
 def test_gpu_i4_asym(gpu, M, K, N, out_dt):
     m = gpu
