@@ -96,7 +96,9 @@ OPSNN_API int opsnnQmmTc(const OpsnnQmmArgs* a, void* stream);
  * Reference formulas: matmul/quant_batch_matmul_v4/tests/assets/qbmmv4_kernel_golden.py:189-255, 328-395.
  * (The MX fp8 x fp4 mode of that file runs through opsnnQmmMx and its int8 per-tile mode through opsnnQmmBlockScale.) */
 OPSNN_API int opsnnQmmGroup(const OpsnnQmmArgs* a, void* stream);
-/* Device workspace bytes a launcher needs for these arguments (0 if none). */
+/* Device workspace bytes a launcher needs for these arguments (0 if none).  mode names the entry point the arguments
+ * are for: 0 opsnnQmmInt8, 1 opsnnQmmBlockScale, 2 opsnnQmmMx, 3 opsnnQmmTc, 4 opsnnQmmGroup (the fp8 x fp4 mode's
+ * re-quantised weight, N * K bytes plus the decoded output scale, when its matrix-core path applies). */
 OPSNN_API uint64_t opsnnQmmWorkspace(const OpsnnQmmArgs* a, int mode);
 
 typedef struct {

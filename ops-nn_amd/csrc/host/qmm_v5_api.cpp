@@ -615,7 +615,7 @@ extern "C" aclnnStatus aclnnQuantMatmulV5GetWorkspaceSize(const aclTensor* x1, c
         // fp8 x fp4 with a 16-bit scale per K group and a packed 64-bit output scale: qbmmv4_kernel_golden.py:189-255
         if (c.x1.dtype != ACL_FLOAT8_E4M3FN)
             FAIL(ACLNN_ERR_INNER_TILING_ERROR, "%s: fp8 x fp4 with group scales takes FLOAT8_E4M3FN x1 only on this device, got %s", kApi, dtype_name(c.x1.dtype));
-        ex->kind = OpKind::QmmGroup; mode = 0;
+        ex->kind = OpKind::QmmGroup; mode = 4;
         a.gsK = (int64_t)((uint64_t)c.groupSize & kMask16);
         const int64_t G = ceil_div(c.K1, std::max<int64_t>(a.gsK, 1));
         a.x2_scale_mat.ptr = c.x2s.ptr_at(0);
@@ -624,7 +624,7 @@ extern "C" aclnnStatus aclnnQuantMatmulV5GetWorkspaceSize(const aclTensor* x1, c
         if (c.ys.present) { a.y_scale = c.ys.ptr_at(0); a.y_scale_len = c.ys.numel(); }
     } else if (a4w4_pergroup_nonsym(c, (uint64_t)a.gsK)) {
         // int4 x int4 with per-group scales and offsets: qbmmv4_kernel_golden.py:328-395
-        ex->kind = OpKind::QmmGroup; mode = 0;
+        ex->kind = OpKind::QmmGroup; mode = 4;
         a.x2_scale_mat.ptr = c.x2s.ptr_at(0); a.x2_scale_mat.row_stride = c.N; a.x2_scale_mat.col_stride = 1;
         a.x2_offset_mat.ptr = c.x2o.ptr_at(0); a.x2_offset_mat.row_stride = c.N; a.x2_offset_mat.col_stride = 1;
     } else if (c.mx()) {

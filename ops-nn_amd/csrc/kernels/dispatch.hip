@@ -14,7 +14,9 @@ int launch_group_plain(const OpsnnQmmArgs& a, bool tcg, hipStream_t st);
 int launch_wqmm_plain(const OpsnnWqmmArgs& a, hipStream_t st);
 // Return OPSNN_NOT_TAKEN when the arguments are outside what the fast kernels handle.
 int launch_blockscale_mfma(const OpsnnQmmArgs& a, hipStream_t st);
-int launch_fp8_rowcol_mfma(const OpsnnQmmArgs& a, hipStream_t st);
+int launch_fp8_rowcol_mfma(const OpsnnQmmArgs& a, hipStream_t st, bool merged_scales_ok);
+int launch_tcg_mfma(const OpsnnQmmArgs& a, hipStream_t st);
+uint64_t tcg_workspace_bytes(const OpsnnQmmArgs& a);
 int launch_mx_mfma(const OpsnnQmmArgs& a, hipStream_t st);
 int launch_wqmm_mfma(const OpsnnWqmmArgs& a, hipStream_t st);
 uint64_t mx_workspace_bytes(const OpsnnQmmArgs& a);
@@ -82,7 +84,7 @@ extern "C" int opsnnQmmTc(const OpsnnQmmArgs* a, void* stream)
     // fp8 e4m3 operands with a row scale and a column scale that are multiplied in separately (K-C, K-T, T-C with the
     // one-element x1Scale): matrix-core kernel when the layout allows, else the plain kernel
     if (f8 && a->x1_scale && a->force_variant != OPSNN_VARIANT_PLAIN && !opsnn_force_plain()) {
-        const int rc = launch_fp8_rowcol_mfma(*a, (hipStream_t)stream);
+        const int rc = launch_fp8_rowcol_mfma(*a, (hipStream_t)stream, false);
         if (rc != OPSNN_NOT_TAKEN) return rc;
     }
     return launch_tc_plain(*a, (hipStream_t)stream);
@@ -103,6 +105,10 @@ extern "C" int opsnnQmmGroup(const OpsnnQmmArgs* a, void* stream)
         return -2;
     }
     if (a->out_dtype != DT_BF16 && a->out_dtype != DT_F16 && a->out_dtype != DT_F32) return -2;
+    if (tcg && a->force_variant != OPSNN_VARIANT_PLAIN && !opsnn_force_plain()) {
+        const int rc = launch_tcg_mfma(*a, (hipStream_t)stream);
+        if (rc != OPSNN_NOT_TAKEN) return rc;
+    }
     return launch_group_plain(*a, tcg, (hipStream_t)stream);
 }
 
@@ -117,7 +123,7 @@ extern "C" int opsnnWqmm(const OpsnnWqmmArgs* a, void* stream)
     return launch_wqmm_plain(*a, (hipStream_t)stream);
 }
 
-// mode: 0 = int8 per-token/per-channel, 1 = block scale, 2 = MX, 3 = per-tensor / per-channel family.
+// mode: 0 = int8 per-token/per-channel, 1 = block scale, 2 = MX, 3 = per-tensor / per-channel family, 4 = K-group modes.
 // The MFMA kernels stream a K-contiguous right operand ("x2 stored [N, K]").  An N-contiguous x2 is
 // first re-laid out into the workspace; callers who keep x2 in [N, K] form (transposeX2 = true or a
 // transposed view) need no workspace and skip that pass.
@@ -126,6 +132,7 @@ extern "C" uint64_t opsnnQmmWorkspace(const OpsnnQmmArgs* a, int mode)
     if (!a) return 0;
     if (mode == 2) return mx_workspace_bytes(*a);
     if (mode == 3) return 0;   // per-tensor / per-channel family: strided kernel, no re-layout
+    if (mode == 4) return tcg_workspace_bytes(*a);   // K-group modes: the re-quantised weight of the fp8 x fp4 group-scale mode
     if (a->x2.row_stride == 1 || a->K == 1) return 0;           // already K-contiguous
     if (a->x2.col_stride != 1 || a->x2.row_stride != a->N) return 0;  // not a dense [K, N]: plain kernel
     uint64_t bits = (a->x2_dtype == DT_I4 || a->x2_dtype == DT_E2M1) ? 4 : 8;

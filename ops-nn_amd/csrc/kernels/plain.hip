@@ -206,7 +206,8 @@ __device__ __forceinline__ uint32_t f32_to_e4m3_bits(float f)
     int exp = (int)(a >> 23) - 127;
     if (exp < -6) exp = -6;                                            // subnormal quantum 2^-9
     const float q = u2f((uint32_t)(exp - 3 + 127) << 23);
-    const float v = __fmul_rn(__builtin_rintf(__fdiv_rn(u2f(a), q)), q);
+    const float qinv = u2f((uint32_t)(127 + 3 - exp) << 23);           // 1 / q: both scalings are exact
+    const float v = __fmul_rn(__builtin_rintf(__fmul_rn(u2f(a), qinv)), q);
     if (v > 448.0f) return sign | 0x7eu;                               // 464 (the tie below the absent 480) rounds to 448
     if (v < 0.015625f) return sign | (uint32_t)__fmul_rn(v, 512.0f);
     const uint32_t vb = f2u(v);
@@ -233,6 +234,48 @@ __global__ void qmm_tcg_plain(OpsnnQmmArgs a)
     if (a.bias) acc = __fadd_rn(acc, load_scalar_as_f32(a.bias, a.bias_dtype, n));
     store_f32_as(a.out, a.out_dtype, m * a.N + n, acc);
 }
+// Prologue of the matrix-core path of the same mode: the re-quantised weight once, as e4m3 bytes [N, K] K-contiguous
+// (the per-element operation of the loop above, so the bytes are the oracle's), the decoded output scale per column
+// (1.0 when absent) and a 1.0 for the row scale.  x2 is [N, K] with two fp4 per byte, low nibble first; thread t turns
+// the 32 elements k0 .. k0+31 of row n (16 bytes in, 32 bytes out), t = n * K/32 + k0/32.  They share one scale
+// (gsK % 32 == 0), and every step of the operation is odd in the weight, so the thread converts the 8 magnitudes once
+// into a table of 8 bytes and each element is a table byte with the nibble's sign bit.
+__global__ __launch_bounds__(256) void tcg_requant_kernel(OpsnnQmmArgs a, uint8_t* w8, float* cs, float* one)
+{
+    const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t kq = a.K / 32;
+    if (t == 0) one[0] = 1.0f;
+    if (t < a.N) cs[t] = a.y_scale ? trunc19(u2f((uint32_t)((const uint64_t*)a.y_scale)[a.y_scale_len == 1 ? 0 : t])) : 1.0f;
+    if (t >= a.N * kq) return;
+    const int64_t n = t / kq, k0 = (t % kq) * 32;
+    const int sdt = a.x2_scale_dtype;
+    const float sc = load_scalar_as_f32(a.x2_scale_mat.ptr, sdt, (k0 / a.gsK) * a.x2_scale_mat.row_stride + n * a.x2_scale_mat.col_stride);
+    uint64_t table = 0;
+#pragma unroll
+    for (uint32_t v = 0; v < 8; v++) {
+        const float mid = round_through(__fmul_rn(round_through(e2m1_to_f32(v), sdt), sc), sdt);
+        table |= (uint64_t)(f32_to_e4m3_bits(mid) & 0x7fu) << (8 * v);
+    }
+    if (sc < 0.0f || f2u(sc) == 0x80000000u) table |= 0x8080808080808080ull;   // a negative scale turns every sign
+    const uint4 in = *(const uint4*)((const uint8_t*)a.x2.ptr + (n * a.K + k0) / 2);
+    const uint32_t words[4] = {in.x, in.y, in.z, in.w};
+    uint32_t o[8];
+#pragma unroll
+    for (int w = 0; w < 8; w++) {
+        const uint32_t nib = (words[w >> 1] >> (16 * (w & 1))) & 0xffffu;
+        uint32_t r = 0;
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            const uint32_t q = (nib >> (4 * e)) & 15u;
+            const uint32_t b = (uint32_t)(table >> (8 * (q & 7u))) & 0xffu;
+            r |= (b ^ ((q & 8u) << 4)) << (8 * e);
+        }
+        o[w] = r;
+    }
+    uint4* dst = (uint4*)(w8 + n * a.K + k0);
+    dst[0] = make_uint4(o[0], o[1], o[2], o[3]);
+    dst[1] = make_uint4(o[4], o[5], o[6], o[7]);
+}
 __global__ void qmm_i4_asym_plain(OpsnnQmmArgs a)
 {
     const int64_t nchunks = (a.N + blockDim.x - 1) / blockDim.x;
@@ -257,6 +300,35 @@ __global__ void qmm_i4_asym_plain(OpsnnQmmArgs a)
     }
     out = __fmul_rn(out, ((const float*)a.x1_scale)[m]);
     store_f32_as(a.out, a.out_dtype, m * a.N + n, out);
+}
+int launch_fp8_rowcol_mfma(const OpsnnQmmArgs& a, hipStream_t st, bool merged_scales_ok);   // qmm_fp8_block.hip
+
+static inline uint64_t align256(uint64_t v) { return (v + 255) / 256 * 256; }
+// Workspace of the matrix-core path of the fp8 x fp4 group-scale mode (0: the shape stays on the plain kernel).
+uint64_t tcg_workspace_bytes(const OpsnnQmmArgs& a)
+{
+    if (a.x1_dtype != DT_E4M3 || a.x2_dtype != DT_E2M1 || a.batch != 1) return 0;
+    if (a.K % 128 != 0 || a.gsK <= 0 || a.gsK % 32 != 0 || (uintptr_t)a.x2.ptr % 16 != 0 || a.M * a.N < 64 * 64) return 0;
+    if (a.x1.col_stride != 1 || a.x2.row_stride != 1 || a.x2.col_stride != a.K) return 0;
+    if (a.out_dtype != DT_BF16 && a.out_dtype != DT_F16) return 0;
+    if (a.bias && a.bias_dtype != DT_F32) return 0;
+    return align256((uint64_t)a.N * a.K) + align256((uint64_t)a.N * 4) + 256;
+}
+// Re-quantise x2 into the workspace, then the fp8 kernel with a column scale (the decoded output scale) and a unit row scale.
+int launch_tcg_mfma(const OpsnnQmmArgs& a, hipStream_t st)
+{
+    const uint64_t need = tcg_workspace_bytes(a);
+    if (!need || !a.workspace || (uintptr_t)a.workspace % 16 != 0) return OPSNN_NOT_TAKEN;
+    uint8_t* w8 = (uint8_t*)a.workspace;
+    float* cs = (float*)(w8 + align256((uint64_t)a.N * a.K));
+    float* one = (float*)((char*)cs + align256((uint64_t)a.N * 4));
+    const int64_t threads = a.N * (a.K / 32);   // >= N since K >= 128
+    hipLaunchKernelGGL(tcg_requant_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, st, a, w8, cs, one);
+    OpsnnQmmArgs b = a;
+    b.x2.ptr = w8; b.x2_dtype = DT_E4M3; b.x2.row_stride = 1; b.x2.col_stride = a.K; b.x2.batch_stride = 0;
+    b.x1_scale = one; b.x1_scale_len = 1;
+    b.x2_scale = cs; b.x2_scale_dtype = DT_F32; b.x2_scale_len = a.N;
+    return launch_fp8_rowcol_mfma(b, st, true);
 }
 int launch_group_plain(const OpsnnQmmArgs& a, bool tcg, hipStream_t st)
 {

@@ -555,14 +555,16 @@ int launch_mx_a8w4_mfma(const OpsnnQmmArgs& a, hipStream_t st)
 // K-C, K-T and the double-scale modes whose two scales are multiplied in separately
 // (qbmmv3_kernel_golden.py:361-387 and :432-441).  out = (sum * x2Scale[n]) * x1Scale[m] + fp32 bias.
 // Needs K-contiguous operands with K % 128 == 0 and a 16-bit output; anything else stays on the plain kernel.
-int launch_fp8_rowcol_mfma(const OpsnnQmmArgs& a, hipStream_t st)
+int launch_fp8_rowcol_mfma(const OpsnnQmmArgs& a, hipStream_t st, bool merged_scales_ok)
 {
     if (a.x1_dtype != DT_E4M3 || a.x2_dtype != DT_E4M3) return OPSNN_NOT_TAKEN;
     if (a.out_dtype != DT_BF16 && a.out_dtype != DT_F16) return OPSNN_NOT_TAKEN;
     if (!a.x1_scale || !a.x2_scale || a.x2_scale_dtype != DT_F32) return OPSNN_NOT_TAKEN;
     if (a.x1_scale_len != 1 && a.x1_scale_len != a.M) return OPSNN_NOT_TAKEN;
     if (a.x2_scale_len != 1 && a.x2_scale_len != a.N) return OPSNN_NOT_TAKEN;
-    if (a.x1_scale_len == 1 && a.x2_scale_len == 1 && !a.bias) return OPSNN_NOT_TAKEN;   // merged and truncated scale: plain kernel
+    // both scales one element and no bias is the double-scale mode whose scales are merged and truncated: plain kernel
+    // (callers whose scales are not that mode's say so)
+    if (!merged_scales_ok && a.x1_scale_len == 1 && a.x2_scale_len == 1 && !a.bias) return OPSNN_NOT_TAKEN;
     if (a.bias && a.bias_dtype != DT_F32) return OPSNN_NOT_TAKEN;
     if (a.K % 128 != 0 || a.M * a.N < 64 * 64 || a.x1.col_stride != 1 || a.x2.row_stride != 1) return OPSNN_NOT_TAKEN;
     Fp8BlkParams p{};
