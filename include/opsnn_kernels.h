@@ -129,6 +129,12 @@ OPSNN_API int opsnnTranspose8(const void* src, void* dst, int64_t rows, int64_t 
  * rows and cols must be even. */
 OPSNN_API int opsnnTranspose4(const void* src, void* dst, int64_t rows, int64_t cols, int64_t batch, void* stream);
 
+/* Weight pre-pack: `count` 4-bit values, one per 32-bit carrier element (int32: value & 0xF; fp32: the fp4 e2m1 code of
+ * the value, 0 for a value that is not one of the 16), into count / 2 bytes, low nibble = even index.  count even, src
+ * 16-byte and dst 8-byte aligned.  Device form of the host loop in
+ * matmul/convert_weight_to_int4_pack/op_host/op_api/aclnn_convert_weight_to_int4_pack.cpp:79-126. */
+OPSNN_API int opsnnPackB4(const void* src, int src_is_fp32, void* dst, int64_t count, void* stream);
+
 /* Device properties the selector uses. */
 OPSNN_API int opsnnDeviceInfo(int* cu_count, int* clock_khz, int64_t* hbm_bytes, char* arch, int arch_len);
 

@@ -100,6 +100,9 @@ _SIGS = {
     "aclnnWeightQuantBatchMatmulV3GetWorkspaceSize": (C.c_int32, [_T] * 7 + [C.c_int, C.c_int, _T, C.POINTER(C.c_uint64),
                                                                          C.POINTER(C.c_void_p)]),
     "aclnnWeightQuantBatchMatmulV3": (C.c_int32, [C.c_void_p, C.c_uint64, C.c_void_p, C.c_void_p]),
+    "aclnnConvertWeightToINT4PackGetWorkspaceSize": (C.c_int32, [_T, _T, C.POINTER(C.c_uint64), C.POINTER(C.c_void_p)]),
+    "aclnnConvertWeightToINT4Pack": (C.c_int32, [C.c_void_p, C.c_uint64, C.c_void_p, C.c_void_p]),
+    "opsnnPackB4": (C.c_int, [C.c_void_p, C.c_int, C.c_void_p, C.c_int64, C.c_void_p]),
     "opsnnQmmInt8": (C.c_int, [C.POINTER(OpsnnQmmArgs), C.c_void_p]),
     "opsnnQmmBlockScale": (C.c_int, [C.POINTER(OpsnnQmmArgs), C.c_void_p]),
     "opsnnQmmMx": (C.c_int, [C.POINTER(OpsnnQmmArgs), C.c_void_p]),
@@ -293,6 +296,15 @@ def weight_quant_batch_matmul(x, weight, scale, y, stream=None, **kw):
     run = lib().aclnnWeightQuantBatchMatmulV3 if v3 else lib().aclnnWeightQuantBatchMatmulV2
     check(run(wbuf.ptr if wbuf else None, ws, ex, stream.ptr if stream else None), "aclnnWeightQuantBatchMatmul")
     return wbuf
+
+
+def convert_weight_to_int4_pack(weight, weight_int4_pack):
+    """Both phases of aclnnConvertWeightToINT4Pack; returns the first phase's status (the second does nothing)."""
+    ws, ex = C.c_uint64(0), C.c_void_p()
+    rc = lib().aclnnConvertWeightToINT4PackGetWorkspaceSize(_h(weight), _h(weight_int4_pack), C.byref(ws), C.byref(ex))
+    if rc == 0:
+        check(lib().aclnnConvertWeightToINT4Pack(None, ws.value, ex, None), "aclnnConvertWeightToINT4Pack")
+    return rc
 
 
 def device_info():

@@ -37,6 +37,9 @@
  *   orc_qmm_i4_asym ... pinned (numpy int64 / float32 recomputation; zero offset and one group reduce to the
  *                       per-token formula)
  *   orc_wqbmm ......... pinned (hand-computed double-rounding cases; group==K equals per-channel; float64)
+ *   orc_convert_weight_b4 pinned (int32 carriers: equals the golden utility's int4 packing orc_pack_int4_to_int32; fp32
+ *                       carriers: the 16 fp4 values decode back through orc_e2m1_to_f32, off-table values hand-derived
+ *                       from the mask and the table of the cited lines)
  *   hifloat8 .......... not implemented (decoder lives only in an absent third-party package): parity unpinned
  */
 #include <math.h>
@@ -188,6 +191,30 @@ void orc_pack_int4_to_int32(const int8_t* in, int32_t* out, size_t n_packed)
         uint32_t w = 0;
         for (int j = 0; j < 8; j++) w |= ((uint32_t)in[i * 8 + j] & 0xfu) << (4 * j);
         out[i] = (int32_t)w;
+    }
+}
+/* aclnnConvertWeightToINT4Pack's host loop (convert_weight_to_int4_pack/op_host/op_api/
+ * aclnn_convert_weight_to_int4_pack.cpp:79-126): one 4-bit value per 32-bit carrier element, packed two per byte with
+ * the even element in the low nibble.  int32 carrier: the low four bits.  fp32 carrier: the bits are cut to sign,
+ * exponent and first mantissa bit (mask 0xFFC00000) and looked up in the table of the 16 fp4 e2m1 values (:43-63); a
+ * pattern that is not in the table gives code 0, sign included. */
+static uint32_t convert_fp32_bits_to_e2m1(uint32_t bits)
+{
+    static const uint32_t mag_bits[8] = {0x00000000u, 0x3F000000u, 0x3F800000u, 0x3FC00000u,
+                                         0x40000000u, 0x40400000u, 0x40800000u, 0x40C00000u};
+    const uint32_t cut = bits & 0xFFC00000u;
+    for (uint32_t c = 0; c < 8; c++) {
+        if (cut == mag_bits[c]) return c;
+        if (cut == (mag_bits[c] | 0x80000000u)) return c | 8u;
+    }
+    return 0u;
+}
+void orc_convert_weight_b4(const int32_t* w, int64_t count, int is_fp32, uint8_t* out)
+{
+    for (int64_t i = 0; i + 1 < count; i += 2) {
+        uint32_t a = (uint32_t)w[i], b = (uint32_t)w[i + 1];
+        if (is_fp32) { a = convert_fp32_bits_to_e2m1(a); b = convert_fp32_bits_to_e2m1(b); }
+        out[i / 2] = (uint8_t)(((b & 0xFu) << 4) | (a & 0xFu));
     }
 }
 void orc_unpack_int32_to_int4(const int32_t* in, int8_t* out, size_t n_packed)

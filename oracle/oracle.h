@@ -36,6 +36,7 @@ void orc_vec_e8m0_to_f32(const uint8_t* in, float* out, size_t n);
 void orc_unpack_groupsize(int64_t gs, int64_t* gsM, int64_t* gsN, int64_t* gsK);
 void orc_pack_int4_to_int32(const int8_t* in, int32_t* out, size_t n_packed);
 void orc_unpack_int32_to_int4(const int32_t* in, int8_t* out, size_t n_packed);
+void orc_convert_weight_b4(const int32_t* w, int64_t count, int is_fp32, uint8_t* out);
 float orc_scale_generate(float s);
 float orc_u64_to_deq_scale(uint64_t v);
 size_t orc_dtype_bits(int dt);

@@ -38,6 +38,8 @@ def lib():
         L.orc_unpack_groupsize.argtypes = [i64, C.POINTER(i64), C.POINTER(i64), C.POINTER(i64)]
         L.orc_pack_int4_to_int32.argtypes = [vp, vp, C.c_size_t]
         L.orc_unpack_int32_to_int4.argtypes = [vp, vp, C.c_size_t]
+        L.orc_convert_weight_b4.argtypes = [vp, i64, C.c_int, vp]
+        L.orc_convert_weight_b4.restype = None
         L.orc_scale_generate.argtypes = [C.c_float]
         L.orc_scale_generate.restype = C.c_float
         L.orc_u64_to_deq_scale.argtypes = [C.c_uint64]
@@ -69,6 +71,15 @@ def e8m0_to_f32(a): return _conv("orc_vec_e8m0_to_f32", np.asarray(a, np.uint8),
 
 
 E2M1_VALUES = np.array([0, .5, 1, 1.5, 2, 3, 4, 6, -0.0, -.5, -1, -1.5, -2, -3, -4, -6], np.float32)
+
+
+def convert_weight_b4(w):
+    """int32 or float32 carrier array (one 4-bit value per element) -> uint8 array with half the last dim."""
+    w = np.ascontiguousarray(w)
+    assert w.dtype in (np.int32, np.float32) and w.shape[-1] % 2 == 0
+    out = np.empty(w.shape[:-1] + (w.shape[-1] // 2,), np.uint8)
+    lib().orc_convert_weight_b4(w.ctypes.data, w.size, int(w.dtype == np.float32), out.ctypes.data)
+    return out
 
 
 def pack_nibbles(codes):

@@ -102,6 +102,7 @@ def test_library_exports_every_declared_symbol(opsnn):
     declared = _declared_symbols()
     assert {"aclnnQuantMatmulV5GetWorkspaceSize", "aclnnQuantMatmulV5", "aclnnWeightQuantBatchMatmulV2GetWorkspaceSize",
             "aclnnWeightQuantBatchMatmulV2", "aclnnWeightQuantBatchMatmulV3GetWorkspaceSize", "aclnnWeightQuantBatchMatmulV3",
+            "aclnnConvertWeightToINT4PackGetWorkspaceSize", "aclnnConvertWeightToINT4Pack", "opsnnPackB4",
             "opsnnQmmInt8", "opsnnWqmm", "aclCreateTensor"} <= declared
     missing = [n for n in sorted(declared) if not hasattr(lib, n)]
     assert not missing, f"declared in include/ but not exported by the library: {missing}"
