@@ -135,6 +135,22 @@ OPSNN_API int opsnnTranspose4(const void* src, void* dst, int64_t rows, int64_t 
  * matmul/convert_weight_to_int4_pack/op_host/op_api/aclnn_convert_weight_to_int4_pack.cpp:79-126. */
 OPSNN_API int opsnnPackB4(const void* src, int src_is_fp32, void* dst, int64_t count, void* stream);
 
+/* Dynamic per-token quantisation of x [rows, cols] (FLOAT16 / BF16, dense): per row a scale (and, when `offset` is not
+ * NULL, an offset: the asymmetric form) and the quantised row y in INT8, INT4 (two per byte, even column in the low nibble;
+ * cols even), FLOAT8_E4M3FN or FLOAT8_E5M2.  smooth: NULL or [cols] factors of x's dtype.  Formula:
+ * quant/dynamic_quant/tests/assets/golden.py:17-122 (pertoken).  A row without range (all zeros; asymmetric: constant)
+ * gets scale 0 and zeros.  force_variant: 0 automatic, 1 the register-resident kernel, 2 the two-pass kernel. */
+typedef struct {
+    const void* x; int x_dtype;
+    const void* smooth;
+    void* y; int y_dtype;
+    float* scale;
+    float* offset;
+    int64_t rows, cols;
+    int force_variant;
+} OpsnnDynQuantArgs;
+OPSNN_API int opsnnDynamicQuant(const OpsnnDynQuantArgs* a, void* stream);
+
 /* Device properties the selector uses. */
 OPSNN_API int opsnnDeviceInfo(int* cu_count, int* clock_khz, int64_t* hbm_bytes, char* arch, int arch_len);
 

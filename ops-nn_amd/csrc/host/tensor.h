@@ -22,7 +22,7 @@ namespace opsnn {
 
 constexpr uint32_t kExecutorMagic = 0x51454D4Du;
 
-enum class OpKind { None, QmmInt8, QmmBlockScale, QmmMx, QmmTc, QmmGroup, Wqmm };
+enum class OpKind { None, QmmInt8, QmmBlockScale, QmmMx, QmmTc, QmmGroup, Wqmm, DynQuant };
 
 // What phase 1 decided; phase 2 only fills in workspace/stream and launches.
 struct aclOpExecutorImpl {
@@ -30,6 +30,7 @@ struct aclOpExecutorImpl {
     OpKind kind = OpKind::None;     // None: nothing to launch (empty output)
     OpsnnQmmArgs qmm{};
     OpsnnWqmmArgs wqmm{};
+    OpsnnDynQuantArgs dynq{};
     uint64_t workspace_size = 0;
     const char* api = "";
 };

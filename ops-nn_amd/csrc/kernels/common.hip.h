@@ -94,6 +94,37 @@ __device__ __forceinline__ float e4m3_to_f32(uint32_t b)
     else v = u2f(((e + 120u) << 23) | (m << 20));
     return (b & 0x80u) ? -v : v;
 }
+// fp32 -> e4m3fn bits, round to nearest even; NaN and magnitudes that round above 448 give NaN
+__device__ __forceinline__ uint32_t f32_to_e4m3_bits(float f)
+{
+    const uint32_t u = f2u(f), sign = (u >> 24) & 0x80u, a = u & 0x7fffffffu;
+    if (a > 0x7f800000u || a >= 0x43f00000u) return sign | 0x7fu;     // NaN; >= 480
+    if (a < 0x3a800000u) return sign;                                  // < 2^-10 rounds to zero
+    int exp = (int)(a >> 23) - 127;
+    if (exp < -6) exp = -6;                                            // subnormal quantum 2^-9
+    const float q = u2f((uint32_t)(exp - 3 + 127) << 23);
+    const float qinv = u2f((uint32_t)(127 + 3 - exp) << 23);           // 1 / q: both scalings are exact
+    const float v = __fmul_rn(__builtin_rintf(__fmul_rn(u2f(a), qinv)), q);
+    if (v > 448.0f) return sign | 0x7eu;                               // 464 (the tie below the absent 480) rounds to 448
+    if (v < 0.015625f) return sign | (uint32_t)__fmul_rn(v, 512.0f);
+    const uint32_t vb = f2u(v);
+    return sign | ((((vb >> 23) - 127 + 7) << 3) | ((vb >> 20) & 7u));
+}
+// fp32 -> e5m2 bits, round to nearest even directly on the fp32 value; overflow gives infinity, NaN stays NaN
+__device__ __forceinline__ uint32_t f32_to_e5m2_bits(float f)
+{
+    const uint32_t u = f2u(f), sign = (u >> 24) & 0x80u, a = u & 0x7fffffffu;
+    if (a > 0x7f800000u) return sign | 0x7fu;
+    if (a >= 0x47700000u) return sign | 0x7cu;                         // >= 61440: the tie with the absent 65536 goes to infinity
+    if (a <= 0x37000000u) return sign;                                 // <= 2^-17 rounds to zero
+    int exp = (int)(a >> 23) - 127;
+    if (exp < -14) exp = -14;                                          // subnormal quantum 2^-16
+    const float q = u2f((uint32_t)(exp - 2 + 127) << 23), qinv = u2f((uint32_t)(127 + 2 - exp) << 23);
+    const float v = __fmul_rn(__builtin_rintf(__fmul_rn(u2f(a), qinv)), q);
+    if (v < 6.103515625e-05f) return sign | (uint32_t)__fmul_rn(v, 65536.0f);
+    const uint32_t vb = f2u(v);
+    return sign | ((((vb >> 23) - 127 + 15) << 2) | ((vb >> 21) & 3u));
+}
 __device__ __forceinline__ float e5m2_to_f32(uint32_t b)
 {
     // e5m2 is the upper byte of an IEEE binary16

@@ -1,0 +1,255 @@
+// Dynamic per-token quantisation: the activation quantizer that feeds the quantized matmuls
+// (aclnnDynamicQuant / aclnnDynamicQuantV2; formula quant/dynamic_quant/tests/assets/golden.py:17-122).
+//
+// Per row of x [rows, cols] (fp16 / bf16), every step a separately rounded fp32 operation:
+//   v = x * smooth                                  (optional, one factor per column)
+//   symmetric:   scale = max|v| * (1 / tmax);                           q = v / scale
+//   asymmetric:  scale = (max v - min v) * (1 / tmax2);  offset = tmax - max v / scale;  q = v / scale + offset
+//   y = int8 / int4: round half to even;  e4m3 / e5m2: the cast rounds
+// HBM-bound: 2 bytes read and 1 (or 1/2) written per element, one pass.  A row lives in registers between the reduction and
+// the quantisation: up to 8 pieces of 8 elements per thread, one wave per row up to 2048 columns (four rows per
+// workgroup, reduction by lane exchange only) and one workgroup per row up to 16384 (partial results of the four waves
+// through LDS).  Rows that are longer, or whose length is not a multiple of 8, take the two-pass kernel that reads x
+// twice (the second time from cache).
+#include "common.hip.h"
+#include "launch.h"
+
+namespace opsnn {
+
+struct DynQuantParams {
+    const uint16_t* x; const uint16_t* smooth; void* y; float* scale; float* offset;
+    int64_t rows, cols;
+    int y_dt; float tmax, rcp;   // rcp = 1 / tmax (symmetric) or 1 / tmax2
+};
+
+template <int X_DT>
+__device__ __forceinline__ float x_to_f32(uint32_t h)
+{
+    if constexpr (X_DT == DT_BF16) return u2f(h << 16);
+    else return f16_to_f32((uint16_t)h);
+}
+
+__device__ __forceinline__ float wave_max(float v)
+{
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o));
+    return v;
+}
+
+// How a row's elements are divided by its scale.  An IEEE division costs about a dozen instructions per element; with the
+// correctly rounded reciprocal r of the scale (one division per row), q0 = RN(v * r), e = v - q0 * scale (exact in a
+// fused multiply-add) and q = RN(q0 + e * r) give the correctly rounded quotient (Markstein's theorem) unless the scale's
+// mantissa is all ones or an intermediate leaves the normal range -- rows where that could happen keep the division.
+struct RowQuant {
+    float scale, offset, rcp;
+    bool ok;        // false: a row without range, its outputs are zeros
+    bool fast;      // the reciprocal form is exact for this row
+};
+
+template <int Y_DT, bool ASYM>
+__device__ __forceinline__ uint32_t quant_one(float v, const RowQuant& r)
+{
+    float q = 0.0f;
+    if (r.ok) {
+        if (r.fast) {
+            const float q0 = __fmul_rn(v, r.rcp);
+            q = __fmaf_rn(__fmaf_rn(-q0, r.scale, v), r.rcp, q0);
+        } else {
+            q = __fdiv_rn(v, r.scale);
+        }
+        if (ASYM) q = __fadd_rn(q, r.offset);
+    }
+    if constexpr (Y_DT == DT_E4M3) return f32_to_e4m3_bits(q);
+    else if constexpr (Y_DT == DT_E5M2) return f32_to_e5m2_bits(q);
+    else {
+        constexpr float lo = Y_DT == DT_I8 ? -128.0f : -8.0f, hi = Y_DT == DT_I8 ? 127.0f : 7.0f;
+        float t = __builtin_rintf(q);
+        t = (t == t) ? fminf(fmaxf(t, lo), hi) : 0.0f;
+        return (uint32_t)(int)t & (Y_DT == DT_I8 ? 0xffu : 0xfu);
+    }
+}
+
+// scale / offset of a row from its reduced extremes
+template <bool ASYM>
+__device__ __forceinline__ RowQuant row_params(const DynQuantParams& p, float amax, float vmax, float vmin)
+{
+    RowQuant r;
+    if (!ASYM) {
+        r.scale = __fmul_rn(amax, p.rcp);
+        r.offset = 0.0f;
+    } else {
+        r.scale = __fmul_rn(__fsub_rn(vmax, vmin), p.rcp);
+        r.offset = __fsub_rn(p.tmax, __fdiv_rn(vmax, r.scale));
+    }
+    r.ok = r.scale > 0.0f && r.scale < __builtin_inff();
+    if (!r.ok) r.offset = 0.0f;
+    r.rcp = __fdiv_rn(1.0f, r.scale);
+    // |v| <= max|v| = O(scale * tmax): with the scale in [2^-60, 2^60] and max|v| >= 2^-60 every product stays normal or
+    // rounds to a quotient far below the first rounding boundary (1/2, or 2^-17 for e5m2)
+    r.fast = r.ok && (f2u(r.scale) & 0x7fffffu) != 0x7fffffu && r.scale > 0x1p-60f && r.scale < 0x1p60f;
+    return r;
+}
+
+// TPR threads per row (64: one wave, 256: the workgroup), pieces of 8 elements held in registers.
+template <int X_DT, int Y_DT, bool ASYM, int TPR>
+__global__ __launch_bounds__(256) void dynamic_quant_rows_kernel(DynQuantParams p)
+{
+    constexpr int RPW = 256 / TPR;   // rows per workgroup
+    constexpr int MAXP = 8;
+    __shared__ float red[3][4];
+    const int t = threadIdx.x % TPR;
+    const int64_t row = (int64_t)blockIdx.x * RPW + threadIdx.x / TPR;
+    const bool live = row < p.rows;   // whole waves: TPR is a multiple of 64
+    const int64_t pieces = p.cols / 8;
+    const uint4* xr = (const uint4*)(p.x + (live ? row : 0) * p.cols);
+    uint4 buf[MAXP];
+    float amax = 0.0f, vmax = -__builtin_inff(), vmin = __builtin_inff();
+    auto element = [&](const uint4& xv, const uint4& sv, int e) {
+        const uint32_t w[4] = {xv.x, xv.y, xv.z, xv.w}, sw[4] = {sv.x, sv.y, sv.z, sv.w};
+        float v = x_to_f32<X_DT>((w[e >> 1] >> (16 * (e & 1))) & 0xffffu);
+        if (p.smooth) v = __fmul_rn(v, x_to_f32<X_DT>((sw[e >> 1] >> (16 * (e & 1))) & 0xffffu));
+        return v;
+    };
+#pragma unroll
+    for (int i = 0; i < MAXP; i++) {
+        const int64_t c = (int64_t)i * TPR + t;
+        if (live && c < pieces) {
+            buf[i] = xr[c];
+            uint4 sm = make_uint4(0, 0, 0, 0);
+            if (p.smooth) sm = ((const uint4*)p.smooth)[c];
+#pragma unroll
+            for (int e = 0; e < 8; e++) {
+                const float v = element(buf[i], sm, e);
+                if (ASYM) { vmax = fmaxf(vmax, v); vmin = fminf(vmin, v); }
+                else amax = fmaxf(amax, fabsf(v));
+            }
+        }
+    }
+    if (ASYM) { vmax = wave_max(vmax); vmin = -wave_max(-vmin); }
+    else amax = wave_max(amax);
+    if constexpr (TPR == 256) {
+        const int w = threadIdx.x >> 6;
+        if ((threadIdx.x & 63) == 0) { red[0][w] = amax; red[1][w] = vmax; red[2][w] = vmin; }
+        __syncthreads();
+        amax = fmaxf(fmaxf(red[0][0], red[0][1]), fmaxf(red[0][2], red[0][3]));
+        vmax = fmaxf(fmaxf(red[1][0], red[1][1]), fmaxf(red[1][2], red[1][3]));
+        vmin = fminf(fminf(red[2][0], red[2][1]), fminf(red[2][2], red[2][3]));
+    }
+    if (!live) return;
+    const RowQuant r = row_params<ASYM>(p, amax, vmax, vmin);
+    if (t == 0) {
+        p.scale[row] = r.scale;
+        if (ASYM) p.offset[row] = r.offset;
+    }
+#pragma unroll
+    for (int i = 0; i < MAXP; i++) {
+        const int64_t c = (int64_t)i * TPR + t;
+        if (c < pieces) {
+            uint4 sm = make_uint4(0, 0, 0, 0);
+            if (p.smooth) sm = ((const uint4*)p.smooth)[c];
+            uint32_t lo = 0, hi = 0;
+#pragma unroll
+            for (int e = 0; e < 8; e++) {
+                const uint32_t b = quant_one<Y_DT, ASYM>(element(buf[i], sm, e), r);
+                if (Y_DT == DT_I4) lo |= b << (4 * e);
+                else if (e < 4) lo |= b << (8 * e);
+                else hi |= b << (8 * (e - 4));
+            }
+            if (Y_DT == DT_I4) ((uint32_t*)p.y)[row * pieces + c] = lo;
+            else ((uint2*)p.y)[row * pieces + c] = make_uint2(lo, hi);
+        }
+    }
+}
+
+// Any row length: one workgroup per row, element-wise loads, x read twice.  int4 needs an even length (two per byte).
+template <int X_DT, int Y_DT, bool ASYM>
+__global__ __launch_bounds__(256) void dynamic_quant_two_pass_kernel(DynQuantParams p)
+{
+    __shared__ float red[3][4];
+    const int64_t row = blockIdx.x;
+    const uint16_t* xr = p.x + row * p.cols;
+    float amax = 0.0f, vmax = -__builtin_inff(), vmin = __builtin_inff();
+    auto element = [&](int64_t c) {
+        float v = x_to_f32<X_DT>(xr[c]);
+        if (p.smooth) v = __fmul_rn(v, x_to_f32<X_DT>(p.smooth[c]));
+        return v;
+    };
+    for (int64_t c = threadIdx.x; c < p.cols; c += 256) {
+        const float v = element(c);
+        amax = fmaxf(amax, fabsf(v));
+        vmax = fmaxf(vmax, v);
+        vmin = fminf(vmin, v);
+    }
+    amax = wave_max(amax); vmax = wave_max(vmax); vmin = -wave_max(-vmin);
+    const int w = threadIdx.x >> 6;
+    if ((threadIdx.x & 63) == 0) { red[0][w] = amax; red[1][w] = vmax; red[2][w] = vmin; }
+    __syncthreads();
+    amax = fmaxf(fmaxf(red[0][0], red[0][1]), fmaxf(red[0][2], red[0][3]));
+    vmax = fmaxf(fmaxf(red[1][0], red[1][1]), fmaxf(red[1][2], red[1][3]));
+    vmin = fminf(fminf(red[2][0], red[2][1]), fminf(red[2][2], red[2][3]));
+    const RowQuant r = row_params<ASYM>(p, amax, vmax, vmin);
+    if (threadIdx.x == 0) {
+        p.scale[row] = r.scale;
+        if (ASYM) p.offset[row] = r.offset;
+    }
+    if (Y_DT == DT_I4) {
+        uint8_t* yr = (uint8_t*)p.y + row * (p.cols / 2);
+        for (int64_t c = threadIdx.x; c < p.cols / 2; c += 256)
+            yr[c] = (uint8_t)(quant_one<Y_DT, ASYM>(element(2 * c), r) | (quant_one<Y_DT, ASYM>(element(2 * c + 1), r) << 4));
+    } else {
+        uint8_t* yr = (uint8_t*)p.y + row * p.cols;
+        for (int64_t c = threadIdx.x; c < p.cols; c += 256) yr[c] = (uint8_t)quant_one<Y_DT, ASYM>(element(c), r);
+    }
+}
+
+template <int X_DT, int Y_DT, bool ASYM>
+static int launch_dynamic_quant(const DynQuantParams& p, int variant, hipStream_t st)
+{
+    const bool vec = p.cols % 8 == 0 && p.cols <= 8 * 8 * 256 && (uintptr_t)p.x % 16 == 0 && (uintptr_t)p.y % 8 == 0 &&
+                     (!p.smooth || (uintptr_t)p.smooth % 16 == 0);
+    if (variant == 2 || !vec) {
+        if (variant == 1) return -4;
+        hipLaunchKernelGGL((dynamic_quant_two_pass_kernel<X_DT, Y_DT, ASYM>), dim3((unsigned)p.rows), dim3(256), 0, st, p);
+    } else if (p.cols <= 8 * 4 * 64) {
+        hipLaunchKernelGGL((dynamic_quant_rows_kernel<X_DT, Y_DT, ASYM, 64>), dim3((unsigned)((p.rows + 3) / 4)), dim3(256), 0, st, p);
+    } else {
+        hipLaunchKernelGGL((dynamic_quant_rows_kernel<X_DT, Y_DT, ASYM, 256>), dim3((unsigned)p.rows), dim3(256), 0, st, p);
+    }
+    return (int)hipGetLastError();
+}
+
+template <int X_DT>
+static int launch_dynamic_quant_x(const DynQuantParams& p, int variant, hipStream_t st)
+{
+    const bool asym = p.offset != nullptr;
+    switch (p.y_dt) {
+        case DT_I8: return asym ? launch_dynamic_quant<X_DT, DT_I8, true>(p, variant, st) : launch_dynamic_quant<X_DT, DT_I8, false>(p, variant, st);
+        case DT_I4: return asym ? launch_dynamic_quant<X_DT, DT_I4, true>(p, variant, st) : launch_dynamic_quant<X_DT, DT_I4, false>(p, variant, st);
+        case DT_E4M3: return asym ? launch_dynamic_quant<X_DT, DT_E4M3, true>(p, variant, st) : launch_dynamic_quant<X_DT, DT_E4M3, false>(p, variant, st);
+        case DT_E5M2: return asym ? launch_dynamic_quant<X_DT, DT_E5M2, true>(p, variant, st) : launch_dynamic_quant<X_DT, DT_E5M2, false>(p, variant, st);
+        default: return -2;
+    }
+}
+
+}  // namespace opsnn
+
+using namespace opsnn;
+
+extern "C" int opsnnDynamicQuant(const OpsnnDynQuantArgs* a, void* stream)
+{
+    if (!a || !a->x || !a->y || !a->scale || a->rows <= 0 || a->cols <= 0 || a->rows > 0x7fffffff) return -1;
+    if (a->x_dtype != DT_F16 && a->x_dtype != DT_BF16) return -2;
+    DynQuantParams p{};
+    switch (a->y_dtype) {
+        case DT_I8: p.tmax = 127.0f; p.rcp = 1.0f / (a->offset ? 255.0f : 127.0f); break;
+        case DT_I4: p.tmax = 7.0f; p.rcp = 1.0f / (a->offset ? 15.0f : 7.0f); break;
+        case DT_E4M3: p.tmax = 448.0f; p.rcp = 1.0f / (a->offset ? 896.0f : 448.0f); break;
+        case DT_E5M2: p.tmax = 57344.0f; p.rcp = 1.0f / (a->offset ? 114688.0f : 57344.0f); break;
+        default: return -2;
+    }
+    if (a->y_dtype == DT_I4 && (a->cols & 1)) return -2;
+    p.x = (const uint16_t*)a->x; p.smooth = (const uint16_t*)a->smooth; p.y = a->y; p.scale = a->scale; p.offset = a->offset;
+    p.rows = a->rows; p.cols = a->cols; p.y_dt = a->y_dtype;
+    if (a->x_dtype == DT_BF16) return launch_dynamic_quant_x<DT_BF16>(p, a->force_variant, (hipStream_t)stream);
+    return launch_dynamic_quant_x<DT_F16>(p, a->force_variant, (hipStream_t)stream);
+}

@@ -197,22 +197,6 @@ __global__ void wqmm_plain(OpsnnWqmmArgs a)
 }
 
 // K-group modes of quant_batch_matmul_v4: see opsnnQmmGroup in opsnn_kernels.h and qbmmv4_kernel_golden.py:189-255, 328-395
-// fp32 -> e4m3fn bits, round to nearest even; NaN and magnitudes that round above 448 give NaN
-__device__ __forceinline__ uint32_t f32_to_e4m3_bits(float f)
-{
-    const uint32_t u = f2u(f), sign = (u >> 24) & 0x80u, a = u & 0x7fffffffu;
-    if (a > 0x7f800000u || a >= 0x43f00000u) return sign | 0x7fu;     // NaN; >= 480
-    if (a < 0x3a800000u) return sign;                                  // < 2^-10 rounds to zero
-    int exp = (int)(a >> 23) - 127;
-    if (exp < -6) exp = -6;                                            // subnormal quantum 2^-9
-    const float q = u2f((uint32_t)(exp - 3 + 127) << 23);
-    const float qinv = u2f((uint32_t)(127 + 3 - exp) << 23);           // 1 / q: both scalings are exact
-    const float v = __fmul_rn(__builtin_rintf(__fmul_rn(u2f(a), qinv)), q);
-    if (v > 448.0f) return sign | 0x7eu;                               // 464 (the tie below the absent 480) rounds to 448
-    if (v < 0.015625f) return sign | (uint32_t)__fmul_rn(v, 512.0f);
-    const uint32_t vb = f2u(v);
-    return sign | ((((vb >> 23) - 127 + 7) << 3) | ((vb >> 20) & 7u));
-}
 __global__ void qmm_tcg_plain(OpsnnQmmArgs a)
 {
     const int64_t nchunks = (a.N + blockDim.x - 1) / blockDim.x;

@@ -60,6 +60,17 @@ class OpsnnWqmmArgs(C.Structure):
     ]
 
 
+class OpsnnDynQuantArgs(C.Structure):
+    _fields_ = [
+        ("x", C.c_void_p), ("x_dtype", C.c_int),
+        ("smooth", C.c_void_p),
+        ("y", C.c_void_p), ("y_dtype", C.c_int),
+        ("scale", C.c_void_p), ("offset", C.c_void_p),
+        ("rows", C.c_int64), ("cols", C.c_int64),
+        ("force_variant", C.c_int),
+    ]
+
+
 _T = C.c_void_p  # aclTensor*
 _SIGS = {
     "aclInit": (C.c_int, [C.c_char_p]),
@@ -102,6 +113,11 @@ _SIGS = {
     "aclnnWeightQuantBatchMatmulV3": (C.c_int32, [C.c_void_p, C.c_uint64, C.c_void_p, C.c_void_p]),
     "aclnnConvertWeightToINT4PackGetWorkspaceSize": (C.c_int32, [_T, _T, C.POINTER(C.c_uint64), C.POINTER(C.c_void_p)]),
     "aclnnConvertWeightToINT4Pack": (C.c_int32, [C.c_void_p, C.c_uint64, C.c_void_p, C.c_void_p]),
+    "aclnnDynamicQuantGetWorkspaceSize": (C.c_int32, [_T] * 4 + [C.POINTER(C.c_uint64), C.POINTER(C.c_void_p)]),
+    "aclnnDynamicQuant": (C.c_int32, [C.c_void_p, C.c_uint64, C.c_void_p, C.c_void_p]),
+    "aclnnDynamicQuantV2GetWorkspaceSize": (C.c_int32, [_T] * 3 + [C.c_int64] + [_T] * 3 + [C.POINTER(C.c_uint64), C.POINTER(C.c_void_p)]),
+    "aclnnDynamicQuantV2": (C.c_int32, [C.c_void_p, C.c_uint64, C.c_void_p, C.c_void_p]),
+    "opsnnDynamicQuant": (C.c_int, [C.POINTER(OpsnnDynQuantArgs), C.c_void_p]),
     "opsnnPackB4": (C.c_int, [C.c_void_p, C.c_int, C.c_void_p, C.c_int64, C.c_void_p]),
     "opsnnQmmInt8": (C.c_int, [C.POINTER(OpsnnQmmArgs), C.c_void_p]),
     "opsnnQmmBlockScale": (C.c_int, [C.POINTER(OpsnnQmmArgs), C.c_void_p]),
@@ -296,6 +312,26 @@ def weight_quant_batch_matmul(x, weight, scale, y, stream=None, **kw):
     run = lib().aclnnWeightQuantBatchMatmulV3 if v3 else lib().aclnnWeightQuantBatchMatmulV2
     check(run(wbuf.ptr if wbuf else None, ws, ex, stream.ptr if stream else None), "aclnnWeightQuantBatchMatmul")
     return wbuf
+
+
+def dynamic_quant_get_workspace(x, y, scale, *, smooth=None, offset=None, group_index=None, v2=False, dst_type=2):
+    """Phase 1 of aclnnDynamicQuant (or V2 when v2 / offset / group_index is given).  Returns (status, workspace, executor)."""
+    ws, ex = C.c_uint64(0), C.c_void_p()
+    if v2 or offset is not None or group_index is not None:
+        rc = lib().aclnnDynamicQuantV2GetWorkspaceSize(_h(x), _h(smooth), _h(group_index), dst_type, _h(y), _h(scale), _h(offset),
+                                                       C.byref(ws), C.byref(ex))
+    else:
+        rc = lib().aclnnDynamicQuantGetWorkspaceSize(_h(x), _h(smooth), _h(y), _h(scale), C.byref(ws), C.byref(ex))
+    return rc, ws.value, ex.value
+
+
+def dynamic_quant(x, y, scale, stream=None, **kw):
+    """Both phases; asynchronous on `stream`."""
+    v2 = kw.get("v2") or kw.get("offset") is not None or kw.get("group_index") is not None
+    rc, ws, ex = dynamic_quant_get_workspace(x, y, scale, **kw)
+    check(rc, "aclnnDynamicQuantGetWorkspaceSize")
+    run = lib().aclnnDynamicQuantV2 if v2 else lib().aclnnDynamicQuant
+    check(run(None, ws, ex, stream.ptr if stream else None), "aclnnDynamicQuant")
 
 
 def convert_weight_to_int4_pack(weight, weight_int4_pack):

@@ -12,6 +12,7 @@
  *   GU  = common/tests/st/arch35/matmul_golden_util.py
  *   GQ  = common/tests/st/arch35/matmul_quant_util.py
  *   G4  = quant_batch_matmul_v4/tests/assets/qbmmv4_kernel_golden.py
+ *   GD  = ../quant/dynamic_quant/tests/assets/golden.py
  *
  * Arithmetic conventions shared with the golden: every float operation is a
  * separately rounded fp32 operation (this file is compiled with
@@ -40,6 +41,11 @@
  *   orc_convert_weight_b4 pinned (int32 carriers: equals the golden utility's int4 packing orc_pack_int4_to_int32; fp32
  *                       carriers: the 16 fp4 values decode back through orc_e2m1_to_f32, off-table values hand-derived
  *                       from the mask and the table of the cited lines)
+ *   orc_dynamic_quant . pinned for rows with a non-zero range (known answers chosen so that division by the type
+ *                       maximum instead of multiplication by its reciprocal, round-half-away, or a 16-bit smooth
+ *                       product each fail; numpy float32 recomputation; dequantisation error <= scale / 2); a row of
+ *                       zeros (symmetric) or a constant row (asymmetric) divides by zero in the golden: parity unpinned,
+ *                       this file writes zeros there
  *   hifloat8 .......... not implemented (decoder lives only in an absent third-party package): parity unpinned
  */
 #include <math.h>
@@ -152,6 +158,29 @@ uint8_t orc_e4m3_from_f32(float f)
     float fr = frexpf(v, &e2);
     uint32_t mant = (uint32_t)(fr * 16.0f) - 8u;
     return (uint8_t)(sign | (uint8_t)(((e2 - 1 + 7) << 3) | mant));
+}
+
+/* fp32 -> e5m2, round to nearest even; overflow to infinity, NaN stays NaN.  e5m2 is binary16 cut to two mantissa
+ * bits, so the rounding is done directly on the fp32 value (not through binary16, which would round twice). */
+uint8_t orc_e5m2_from_f32(float f)
+{
+    uint32_t u = f2u(f);
+    uint8_t sign = (uint8_t)((u >> 24) & 0x80u);
+    float a = fabsf(f);
+    if (!(a == a)) return (uint8_t)(sign | 0x7f);
+    if (a >= 61440.0f) return (uint8_t)(sign | 0x7c);  /* the tie between 57344 and the absent 65536 goes to even = infinity */
+    if (a <= 7.62939453125e-06f) return sign;          /* <= 2^-17: the tie with the smallest subnormal 2^-16 goes to 0 */
+    int e;
+    (void)frexpf(a, &e);
+    int exp = e - 1;
+    if (exp < -14) exp = -14;                          /* subnormal quantum 2^-16 */
+    float q = ldexpf(1.0f, exp - 2);
+    float v = nearbyintf(a / q) * q;
+    if (v < 6.103515625e-05f) return (uint8_t)(sign | (uint8_t)(v * 65536.0f));
+    int e2;
+    float fr = frexpf(v, &e2);
+    uint32_t mant = (uint32_t)(fr * 8.0f) - 4u;
+    return (uint8_t)(sign | (uint8_t)(((e2 - 1 + 15) << 2) | mant));
 }
 
 /* FP4 E2M1 value table (GQ:329-346): codes 0..7 = {0,.5,1,1.5,2,3,4,6}, bit 3 = sign. */
@@ -771,3 +800,79 @@ float orc_scale_generate(float s) { return u2f(f2u(s) & 0xFFFFE000u); }
 float orc_u64_to_deq_scale(uint64_t v) { return u2f((uint32_t)v & 0xFFFFE000u); }
 
 size_t orc_dtype_bits(int dt) { return dtype_bits(dt); }
+
+/* ------------------------------------------------------------------------- */
+/* Dynamic per-token quantisation (the activation quantizer before the matmul) */
+/* ------------------------------------------------------------------------- */
+
+/* GD:17-122 (_dynamic_quant_common, quant_mode "pertoken", no group index).  Per row of x [rows, cols]:
+ *   v = fp32(x) * fp32(smooth)                      (smooth optional, one per column)
+ *   symmetric:   scale = max|v| * (1 / tmax);                        q = v / scale
+ *   asymmetric:  scale = (max v - min v) * (1 / tmax2);  offset = tmax - max v / scale;  q = v / scale + offset
+ *   y = integer types: round half to even, then the cast; fp8 types: the cast itself rounds
+ * with (tmax, tmax2) = (127, 255) int8, (7, 15) int4, (448, 896) e4m3, (57344, 114688) e5m2; 1 / tmax is an fp32 constant
+ * and every operation is a separately rounded fp32 operation.  int4 results are packed two per byte, even column low.
+ * A row whose scale is zero divides by zero in the golden (NaN through an integer cast): zeros are written instead. */
+int orc_dynamic_quant(const void* x, int x_dt, int64_t rows, int64_t cols, const void* smooth, int y_dt, int symmetric,
+                      void* y, float* scale_out, float* offset_out)
+{
+    float tmax, tmax2;
+    switch (y_dt) {
+        case ORC_I8: tmax = 127.0f; tmax2 = 255.0f; break;
+        case ORC_I4: tmax = 7.0f; tmax2 = 15.0f; break;
+        case ORC_E4M3: tmax = 448.0f; tmax2 = 896.0f; break;
+        case ORC_E5M2: tmax = 57344.0f; tmax2 = 114688.0f; break;
+        default: return -1;
+    }
+    if ((x_dt != ORC_F16 && x_dt != ORC_BF16) || rows < 0 || cols <= 0 || (y_dt == ORC_I4 && (cols & 1))) return -1;
+    if (!symmetric && !offset_out) return -1;
+    const float rcp = 1.0f / (symmetric ? tmax : tmax2);
+    float* v = (float*)malloc((size_t)cols * sizeof(float));
+    if (!v) return -2;
+    for (int64_t r = 0; r < rows; r++) {
+        float vmax = -INFINITY, vmin = INFINITY, amax = 0.0f;
+        for (int64_t c = 0; c < cols; c++) {
+            float e = load_as_f32(x, x_dt, (size_t)(r * cols + c));
+            if (smooth) e = e * load_as_f32(smooth, x_dt, (size_t)c);
+            v[c] = e;
+            if (e > vmax) vmax = e;
+            if (e < vmin) vmin = e;
+            if (fabsf(e) > amax) amax = fabsf(e);
+        }
+        float scale, offset = 0.0f;
+        if (symmetric) {
+            scale = amax * rcp;
+        } else {
+            scale = (vmax - vmin) * rcp;
+            offset = tmax - vmax / scale;
+        }
+        const int degenerate = !(scale > 0.0f) || !isfinite(scale);
+        scale_out[r] = scale;
+        if (!symmetric) offset_out[r] = degenerate ? 0.0f : offset;
+        for (int64_t c = 0; c < cols; c++) {
+            float q = 0.0f;
+            if (!degenerate) {
+                q = v[c] / scale;
+                if (!symmetric) q = q + offset;
+            }
+            const size_t i = (size_t)(r * cols + c);
+            if (y_dt == ORC_E4M3) ((uint8_t*)y)[i] = orc_e4m3_from_f32(q);
+            else if (y_dt == ORC_E5M2) ((uint8_t*)y)[i] = orc_e5m2_from_f32(q);
+            else {
+                float rq = nearbyintf(q);
+                const float lo = y_dt == ORC_I8 ? -128.0f : -8.0f, hi = y_dt == ORC_I8 ? 127.0f : 7.0f;
+                if (!(rq == rq)) rq = 0.0f;
+                if (rq < lo) rq = lo;
+                if (rq > hi) rq = hi;
+                const int iv = (int)rq;
+                if (y_dt == ORC_I8) ((int8_t*)y)[i] = (int8_t)iv;
+                else {
+                    uint8_t* b = (uint8_t*)y + (i >> 1);
+                    *b = (i & 1) ? (uint8_t)((*b & 0x0fu) | ((iv & 15) << 4)) : (uint8_t)((*b & 0xf0u) | (iv & 15));
+                }
+            }
+        }
+    }
+    free(v);
+    return 0;
+}

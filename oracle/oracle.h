@@ -23,6 +23,7 @@ float orc_f16_to_f32(uint16_t h);
 float orc_e4m3_to_f32(uint8_t b);
 float orc_e5m2_to_f32(uint8_t b);
 uint8_t orc_e4m3_from_f32(float f);
+uint8_t orc_e5m2_from_f32(float f);
 float orc_e2m1_to_f32(uint8_t code);
 float orc_e8m0_to_f32(uint8_t b);
 void orc_vec_f32_to_bf16(const float* in, uint16_t* out, size_t n);
@@ -62,6 +63,8 @@ int orc_qmm_tcg(const uint8_t* x1, const uint8_t* x2, int64_t M, int64_t K, int6
                 int s_dt, int64_t gs, const uint64_t* yscale, int64_t ylen, const float* bias, int y_dt, void* y);
 int orc_qmm_i4_asym(const uint8_t* x1, const uint8_t* x2, int64_t M, int64_t K, int64_t N, int tB, const float* x1s,
                     const float* x2s, const uint16_t* x2o, int y_dt, void* y);
+int orc_dynamic_quant(const void* x, int x_dt, int64_t rows, int64_t cols, const void* smooth, int y_dt, int symmetric,
+                      void* y, float* scale_out, float* offset_out);
 int orc_wqbmm(const void* x, int x_dt, const void* w, int w_dt, int64_t M, int64_t K, int64_t N, int tW,
               const void* scale, int scale_dt, int64_t scale_n, const void* offset, int64_t group,
               const void* bias, int bias_dt, void* y);

@@ -40,6 +40,10 @@ def lib():
         L.orc_unpack_int32_to_int4.argtypes = [vp, vp, C.c_size_t]
         L.orc_convert_weight_b4.argtypes = [vp, i64, C.c_int, vp]
         L.orc_convert_weight_b4.restype = None
+        L.orc_dynamic_quant.argtypes = [vp, C.c_int, i64, i64, vp, C.c_int, C.c_int, vp, vp, vp]
+        L.orc_dynamic_quant.restype = C.c_int
+        L.orc_e5m2_from_f32.argtypes = [C.c_float]
+        L.orc_e5m2_from_f32.restype = C.c_uint8
         L.orc_scale_generate.argtypes = [C.c_float]
         L.orc_scale_generate.restype = C.c_float
         L.orc_u64_to_deq_scale.argtypes = [C.c_uint64]
@@ -71,6 +75,21 @@ def e8m0_to_f32(a): return _conv("orc_vec_e8m0_to_f32", np.asarray(a, np.uint8),
 
 
 E2M1_VALUES = np.array([0, .5, 1, 1.5, 2, 3, 4, 6, -0.0, -.5, -1, -1.5, -2, -3, -4, -6], np.float32)
+
+
+def dynamic_quant(x, x_dt, y_dt, smooth=None, symmetric=True):
+    """x: uint16 bits [..., cols] of x_dt.  Returns (y bytes, scale[, offset]); int4 results are packed two per byte."""
+    x = np.ascontiguousarray(x, np.uint16)
+    cols = x.shape[-1]
+    rows = x.size // cols
+    y = np.zeros(x.shape[:-1] + ((cols // 2) if y_dt == I4 else cols,), np.uint8)
+    scale = np.zeros(x.shape[:-1], np.float32)
+    offset = np.zeros(x.shape[:-1], np.float32)
+    sm = None if smooth is None else np.ascontiguousarray(smooth, np.uint16)
+    rc = lib().orc_dynamic_quant(x.ctypes.data, x_dt, rows, cols, sm.ctypes.data if sm is not None else None, y_dt, int(symmetric),
+                                 y.ctypes.data, scale.ctypes.data, offset.ctypes.data)
+    assert rc == 0, rc
+    return (y, scale) if symmetric else (y, scale, offset)
 
 
 def convert_weight_b4(w):

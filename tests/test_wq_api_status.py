@@ -103,6 +103,8 @@ def test_library_exports_every_declared_symbol(opsnn):
     assert {"aclnnQuantMatmulV5GetWorkspaceSize", "aclnnQuantMatmulV5", "aclnnWeightQuantBatchMatmulV2GetWorkspaceSize",
             "aclnnWeightQuantBatchMatmulV2", "aclnnWeightQuantBatchMatmulV3GetWorkspaceSize", "aclnnWeightQuantBatchMatmulV3",
             "aclnnConvertWeightToINT4PackGetWorkspaceSize", "aclnnConvertWeightToINT4Pack", "opsnnPackB4",
+            "aclnnDynamicQuantGetWorkspaceSize", "aclnnDynamicQuant", "aclnnDynamicQuantV2GetWorkspaceSize", "aclnnDynamicQuantV2",
+            "opsnnDynamicQuant",
             "opsnnQmmInt8", "opsnnWqmm", "aclCreateTensor"} <= declared
     missing = [n for n in sorted(declared) if not hasattr(lib, n)]
     assert not missing, f"declared in include/ but not exported by the library: {missing}"
