@@ -151,6 +151,22 @@ typedef struct {
 } OpsnnDynQuantArgs;
 OPSNN_API int opsnnDynamicQuant(const OpsnnDynQuantArgs* a, void* stream);
 
+/* Dynamic block quantisation of x [batch, rows, cols] (FLOAT16 / BF16, dense) to FLOAT8_E4M3FN / FLOAT8_E5M2 with one
+ * fp32 scale per block of row_block x col_block elements, scale [batch, ceil(rows / row_block), ceil(cols / col_block)];
+ * min_scale >= 0 caps the scale at 1 / min_scale (0: no cap).  Formula:
+ * quant/dynamic_block_quant/tests/assets/golden.py:95-222.  force_variant: 0 automatic, 1 the lane-group kernel
+ * (row_block == 1, cols % 8 == 0), 2 the workgroup-per-block kernel. */
+typedef struct {
+    const void* x; int x_dtype;
+    void* y; int y_dtype;
+    float* scale;
+    int64_t batch, rows, cols;
+    int64_t row_block, col_block;
+    double min_scale;
+    int force_variant;
+} OpsnnBlockQuantArgs;
+OPSNN_API int opsnnDynamicBlockQuant(const OpsnnBlockQuantArgs* a, void* stream);
+
 /* Device properties the selector uses. */
 OPSNN_API int opsnnDeviceInfo(int* cu_count, int* clock_khz, int64_t* hbm_bytes, char* arch, int arch_len);
 

@@ -125,6 +125,16 @@ __device__ __forceinline__ uint32_t f32_to_e5m2_bits(float f)
     const uint32_t vb = f2u(v);
     return sign | ((((vb >> 23) - 127 + 15) << 2) | ((vb >> 21) & 3u));
 }
+// Two fp32 values -> two fp8 bytes (a in bits 0..7, b in bits 8..15) with the hardware conversion.  For every fp32 of
+// either sign up to the format's largest finite value (448 / 57344), zeros and subnormal results included, it returns
+// the byte of f32_to_e4m3_bits / f32_to_e5m2_bits (compared exhaustively on the device); callers clamp to that range and
+// handle NaN themselves.
+template <int Y_DT>
+__device__ __forceinline__ uint32_t cvt2_fp8_in_range(float a, float b)
+{
+    if constexpr (Y_DT == DT_E4M3) return (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(a, b, 0, false) & 0xffffu;
+    else return (uint32_t)__builtin_amdgcn_cvt_pk_bf8_f32(a, b, 0, false) & 0xffffu;
+}
 __device__ __forceinline__ float e5m2_to_f32(uint32_t b)
 {
     // e5m2 is the upper byte of an IEEE binary16

@@ -1,0 +1,202 @@
+// Dynamic block quantisation to fp8: the quantizer that produces the operands and the per-block scales of the block-scale
+// matmul (aclnnDynamicBlockQuant; formula quant/dynamic_block_quant/tests/assets/golden.py:95-222).
+//
+// x [batch, rows, cols] (fp16 / bf16) is cut into blocks of rb x cb.  Per block, every step a separately rounded fp32
+// operation:  amax = max|x| (infinities and NaN count as 0);  scale = amax / tmax, capped at 1 / min_scale;
+// q = x / scale (x itself where x is infinite or NaN), clipped to +-tmax;  q = rint(q * 1e8) / 1e8;  NaN -> +0;  y = fp8(q).
+// HBM-bound: 2 bytes read, 1 written per element.
+//   rb == 1, cols % 8 == 0: a block is cb / 8 lanes of one wave (8 elements per lane, held in registers between the
+//     reduction and the quantisation), a lane group of 8 / 16 / 32 lanes per block, reduced by lane exchange only.
+//   any other shape: one workgroup per block, two sweeps over the block (the second one hits in cache: a block is at
+//     most 512 x 256 x 2 bytes).
+// The two divisions per element (by the block's scale, by 1e8) are done with the correctly rounded reciprocal and one
+// exact residual step, which gives the correctly rounded quotient except for a divisor whose mantissa is all ones or
+// operands near the ends of the exponent range; blocks where that could be keep the division instruction.
+#include "common.hip.h"
+#include "launch.h"
+
+namespace opsnn {
+
+struct BlockQuantParams {
+    const uint16_t* x; uint8_t* y; float* scale;
+    int64_t batch, rows, cols, rb, cb, nrb, ncb;
+    float tmax, cap;   // cap = fp32(1 / min_scale), or +inf when min_scale == 0
+};
+
+template <int X_DT>
+__device__ __forceinline__ float bq_x_to_f32(uint32_t h)
+{
+    if constexpr (X_DT == DT_BF16) return u2f(h << 16);
+    else return f16_to_f32((uint16_t)h);
+}
+
+struct BlockScale { float scale, rcp; bool fast; };
+
+__device__ __forceinline__ BlockScale block_scale(const BlockQuantParams& p, float amax)
+{
+    BlockScale b;
+    b.scale = fminf(__fdiv_rn(amax, p.tmax), p.cap);
+    b.rcp = __fdiv_rn(1.0f, b.scale);
+    b.fast = (f2u(b.scale) & 0x7fffffu) != 0x7fffffu && b.scale > 0x1p-60f && b.scale < 0x1p60f;
+    return b;
+}
+
+// the value that is cast: finite, within +-tmax, never NaN
+__device__ __forceinline__ float block_quant_value(float v, const BlockScale& b, float tmax)
+{
+    const bool finite = fabsf(v) < __builtin_inff();   // false for NaN too
+    float q;
+    {
+        const float q0 = __fmul_rn(v, b.rcp);
+        q = __fmaf_rn(__fmaf_rn(-q0, b.scale, v), b.rcp, q0);
+    }
+    // with the scale in [2^-60, 2^60] and |v| above 2^-100 every intermediate is a normal number; a zero stays a zero
+    if (!(b.fast && (fabsf(v) > 0x1p-100f || v == 0.0f))) q = __fdiv_rn(v, b.scale);
+    if (!finite) q = v;
+    q = q > tmax ? tmax : q;       // comparisons are false for NaN: it passes through, as in numpy's clip
+    q = q < -tmax ? -tmax : q;
+    const float t = __builtin_rintf(__fmul_rn(q, 1e8f));
+    const float d0 = __fmul_rn(t, 1e-8f);   // 1e-8f is the correctly rounded reciprocal of 1e8f
+    q = __fmaf_rn(__fmaf_rn(-d0, 1e8f, t), 1e-8f, d0);
+    return (q == q) ? q : 0.0f;
+}
+template <int Y_DT>
+__device__ __forceinline__ uint32_t block_quant_one(float v, const BlockScale& b, float tmax)
+{
+    return cvt2_fp8_in_range<Y_DT>(block_quant_value(v, b, tmax), 0.0f) & 0xffu;
+}
+// eight elements -> eight bytes
+template <int Y_DT>
+__device__ __forceinline__ uint2 block_quant_eight(const float* v, const BlockScale& b, float tmax)
+{
+    uint32_t h[4];
+#pragma unroll
+    for (int e = 0; e < 4; e++) h[e] = cvt2_fp8_in_range<Y_DT>(block_quant_value(v[2 * e], b, tmax), block_quant_value(v[2 * e + 1], b, tmax));
+    return make_uint2(h[0] | (h[1] << 16), h[2] | (h[3] << 16));
+}
+
+// rb == 1: lane groups of G lanes, LPB = cb / 8 of them active, one (row, block) pair per group.
+template <int X_DT, int Y_DT, int G>
+__global__ __launch_bounds__(256) void block_quant_rows_kernel(BlockQuantParams p, int lpb)
+{
+    const int64_t group = ((int64_t)blockIdx.x * 256 + threadIdx.x) / G;
+    const int lane = threadIdx.x % G;
+    const int64_t total = p.batch * p.rows * p.ncb;
+    const bool live_group = group < total;
+    const int64_t row = live_group ? group / p.ncb : 0, bc = live_group ? group % p.ncb : 0;
+    const int64_t col = bc * p.cb + (int64_t)lane * 8;
+    const bool live = live_group && lane < lpb && col < p.cols;   // cols % 8 == 0: a piece is inside the row or outside
+    uint4 buf = make_uint4(0, 0, 0, 0);
+    if (live) buf = *(const uint4*)(p.x + row * p.cols + col);
+    const uint32_t w[4] = {buf.x, buf.y, buf.z, buf.w};
+    float v[8];
+    float amax = 0.0f;
+#pragma unroll
+    for (int e = 0; e < 8; e++) {
+        v[e] = bq_x_to_f32<X_DT>((w[e >> 1] >> (16 * (e & 1))) & 0xffffu);
+        const float a = fabsf(v[e]);
+        amax = fmaxf(amax, a < __builtin_inff() ? a : 0.0f);
+    }
+#pragma unroll
+    for (int o = G / 2; o > 0; o >>= 1) amax = fmaxf(amax, __shfl_xor(amax, o));
+    const BlockScale b = block_scale(p, amax);
+    if (live_group && lane == 0) p.scale[group] = b.scale;
+    if (!live) return;
+    *(uint2*)(p.y + row * p.cols + col) = block_quant_eight<Y_DT>(v, b, p.tmax);
+}
+
+// Any block shape: one workgroup per block, two sweeps.  VEC: cols % 8 == 0 (then every block row is a whole number of
+// 16-byte pieces, since cb % 8 == 0); otherwise element by element.
+template <int X_DT, int Y_DT, bool VEC>
+__global__ __launch_bounds__(256) void block_quant_tile_kernel(BlockQuantParams p)
+{
+    __shared__ float red[4];
+    const int64_t blk = blockIdx.x;
+    const int64_t bc = blk % p.ncb, br = (blk / p.ncb) % p.nrb, bt = blk / (p.ncb * p.nrb);
+    const int64_t r0 = br * p.rb, c0 = bc * p.cb;
+    const int64_t nr = (r0 + p.rb < p.rows ? p.rb : p.rows - r0), nc = (c0 + p.cb < p.cols ? p.cb : p.cols - c0);
+    const uint16_t* xb = p.x + (bt * p.rows + r0) * p.cols + c0;
+    uint8_t* yb = p.y + (bt * p.rows + r0) * p.cols + c0;
+    constexpr int W = VEC ? 8 : 1;
+    const int64_t ppr = nc / W, items = nr * ppr;   // pieces per block row
+    float amax = 0.0f;
+    for (int64_t i = threadIdx.x; i < items; i += 256) {
+        const int64_t o = (i / ppr) * p.cols + (i % ppr) * W;
+        if constexpr (VEC) {
+            const uint4 b = *(const uint4*)(xb + o);
+            const uint32_t w[4] = {b.x, b.y, b.z, b.w};
+#pragma unroll
+            for (int e = 0; e < 8; e++) {
+                const float a = fabsf(bq_x_to_f32<X_DT>((w[e >> 1] >> (16 * (e & 1))) & 0xffffu));
+                amax = fmaxf(amax, a < __builtin_inff() ? a : 0.0f);
+            }
+        } else {
+            const float a = fabsf(bq_x_to_f32<X_DT>(xb[o]));
+            amax = fmaxf(amax, a < __builtin_inff() ? a : 0.0f);
+        }
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) amax = fmaxf(amax, __shfl_xor(amax, o));
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = amax;
+    __syncthreads();
+    amax = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+    const BlockScale b = block_scale(p, amax);
+    if (threadIdx.x == 0) p.scale[blk] = b.scale;
+    for (int64_t i = threadIdx.x; i < items; i += 256) {
+        const int64_t o = (i / ppr) * p.cols + (i % ppr) * W;
+        if constexpr (VEC) {
+            const uint4 xv = *(const uint4*)(xb + o);
+            const uint32_t w[4] = {xv.x, xv.y, xv.z, xv.w};
+            float v[8];
+#pragma unroll
+            for (int e = 0; e < 8; e++) v[e] = bq_x_to_f32<X_DT>((w[e >> 1] >> (16 * (e & 1))) & 0xffffu);
+            *(uint2*)(yb + o) = block_quant_eight<Y_DT>(v, b, p.tmax);
+        } else {
+            yb[o] = (uint8_t)block_quant_one<Y_DT>(bq_x_to_f32<X_DT>(xb[o]), b, p.tmax);
+        }
+    }
+}
+
+template <int X_DT, int Y_DT>
+static int launch_block_quant(const BlockQuantParams& p, int variant, hipStream_t st)
+{
+    const bool rows_ok = p.rb == 1 && p.cols % 8 == 0 && p.cb % 8 == 0 && p.cb <= 256 && (uintptr_t)p.x % 16 == 0 && (uintptr_t)p.y % 8 == 0;
+    if (variant != 2 && rows_ok) {
+        const int lpb = (int)(p.cb / 8);
+        const int g = lpb <= 8 ? 8 : lpb <= 16 ? 16 : 32;
+        const int64_t groups = p.batch * p.rows * p.ncb;
+        const int64_t wgs = (groups * g + 255) / 256;
+        if (wgs > 0x7fffffff) return -1;
+        if (g == 8) hipLaunchKernelGGL((block_quant_rows_kernel<X_DT, Y_DT, 8>), dim3((unsigned)wgs), dim3(256), 0, st, p, lpb);
+        else if (g == 16) hipLaunchKernelGGL((block_quant_rows_kernel<X_DT, Y_DT, 16>), dim3((unsigned)wgs), dim3(256), 0, st, p, lpb);
+        else hipLaunchKernelGGL((block_quant_rows_kernel<X_DT, Y_DT, 32>), dim3((unsigned)wgs), dim3(256), 0, st, p, lpb);
+    } else {
+        if (variant == 1) return -4;
+        const int64_t blocks = p.batch * p.nrb * p.ncb;
+        if (blocks > 0x7fffffff) return -1;
+        const bool vec = p.cols % 8 == 0 && p.cb % 8 == 0 && (uintptr_t)p.x % 16 == 0 && (uintptr_t)p.y % 8 == 0;
+        if (vec) hipLaunchKernelGGL((block_quant_tile_kernel<X_DT, Y_DT, true>), dim3((unsigned)blocks), dim3(256), 0, st, p);
+        else hipLaunchKernelGGL((block_quant_tile_kernel<X_DT, Y_DT, false>), dim3((unsigned)blocks), dim3(256), 0, st, p);
+    }
+    return (int)hipGetLastError();
+}
+
+}  // namespace opsnn
+
+using namespace opsnn;
+
+extern "C" int opsnnDynamicBlockQuant(const OpsnnBlockQuantArgs* a, void* stream)
+{
+    if (!a || !a->x || !a->y || !a->scale || a->batch <= 0 || a->rows <= 0 || a->cols <= 0 || a->row_block <= 0 || a->col_block <= 0) return -1;
+    if ((a->x_dtype != DT_F16 && a->x_dtype != DT_BF16) || (a->y_dtype != DT_E4M3 && a->y_dtype != DT_E5M2) || !(a->min_scale >= 0)) return -2;
+    BlockQuantParams p{};
+    p.x = (const uint16_t*)a->x; p.y = (uint8_t*)a->y; p.scale = a->scale;
+    p.batch = a->batch; p.rows = a->rows; p.cols = a->cols; p.rb = a->row_block; p.cb = a->col_block;
+    p.nrb = (p.rows + p.rb - 1) / p.rb; p.ncb = (p.cols + p.cb - 1) / p.cb;
+    p.tmax = a->y_dtype == DT_E4M3 ? 448.0f : 57344.0f;
+    p.cap = a->min_scale != 0 ? (float)(1.0 / a->min_scale) : __builtin_inff();
+    const hipStream_t st = (hipStream_t)stream;
+    if (a->x_dtype == DT_BF16)
+        return a->y_dtype == DT_E4M3 ? launch_block_quant<DT_BF16, DT_E4M3>(p, a->force_variant, st) : launch_block_quant<DT_BF16, DT_E5M2>(p, a->force_variant, st);
+    return a->y_dtype == DT_E4M3 ? launch_block_quant<DT_F16, DT_E4M3>(p, a->force_variant, st) : launch_block_quant<DT_F16, DT_E5M2>(p, a->force_variant, st);
+}

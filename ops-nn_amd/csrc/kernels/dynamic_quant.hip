@@ -59,9 +59,12 @@ __device__ __forceinline__ uint32_t quant_one(float v, const RowQuant& r)
         }
         if (ASYM) q = __fadd_rn(q, r.offset);
     }
-    if constexpr (Y_DT == DT_E4M3) return f32_to_e4m3_bits(q);
-    else if constexpr (Y_DT == DT_E5M2) return f32_to_e5m2_bits(q);
-    else {
+    if constexpr (Y_DT == DT_E4M3 || Y_DT == DT_E5M2) {
+        // |q| <= tmax up to the rounding of the division: clamped, the hardware conversion is the software rounding
+        constexpr float tmax = Y_DT == DT_E4M3 ? 448.0f : 57344.0f;
+        if (!(q == q)) return ((f2u(q) >> 24) & 0x80u) | 0x7fu;
+        return cvt2_fp8_in_range<Y_DT>(fminf(fmaxf(q, -tmax), tmax), 0.0f) & 0xffu;
+    } else {
         constexpr float lo = Y_DT == DT_I8 ? -128.0f : -8.0f, hi = Y_DT == DT_I8 ? 127.0f : 7.0f;
         float t = __builtin_rintf(q);
         t = (t == t) ? fminf(fmaxf(t, lo), hi) : 0.0f;

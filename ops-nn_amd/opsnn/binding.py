@@ -71,6 +71,18 @@ class OpsnnDynQuantArgs(C.Structure):
     ]
 
 
+class OpsnnBlockQuantArgs(C.Structure):
+    _fields_ = [
+        ("x", C.c_void_p), ("x_dtype", C.c_int),
+        ("y", C.c_void_p), ("y_dtype", C.c_int),
+        ("scale", C.c_void_p),
+        ("batch", C.c_int64), ("rows", C.c_int64), ("cols", C.c_int64),
+        ("row_block", C.c_int64), ("col_block", C.c_int64),
+        ("min_scale", C.c_double),
+        ("force_variant", C.c_int),
+    ]
+
+
 _T = C.c_void_p  # aclTensor*
 _SIGS = {
     "aclInit": (C.c_int, [C.c_char_p]),
@@ -118,6 +130,10 @@ _SIGS = {
     "aclnnDynamicQuantV2GetWorkspaceSize": (C.c_int32, [_T] * 3 + [C.c_int64] + [_T] * 3 + [C.POINTER(C.c_uint64), C.POINTER(C.c_void_p)]),
     "aclnnDynamicQuantV2": (C.c_int32, [C.c_void_p, C.c_uint64, C.c_void_p, C.c_void_p]),
     "opsnnDynamicQuant": (C.c_int, [C.POINTER(OpsnnDynQuantArgs), C.c_void_p]),
+    "aclnnDynamicBlockQuantGetWorkspaceSize": (C.c_int32, [_T, C.c_double, C.c_char_p, C.c_int64, C.c_int64, C.c_int64, _T, _T,
+                                                          C.POINTER(C.c_uint64), C.POINTER(C.c_void_p)]),
+    "aclnnDynamicBlockQuant": (C.c_int32, [C.c_void_p, C.c_uint64, C.c_void_p, C.c_void_p]),
+    "opsnnDynamicBlockQuant": (C.c_int, [C.POINTER(OpsnnBlockQuantArgs), C.c_void_p]),
     "opsnnPackB4": (C.c_int, [C.c_void_p, C.c_int, C.c_void_p, C.c_int64, C.c_void_p]),
     "opsnnQmmInt8": (C.c_int, [C.POINTER(OpsnnQmmArgs), C.c_void_p]),
     "opsnnQmmBlockScale": (C.c_int, [C.POINTER(OpsnnQmmArgs), C.c_void_p]),
@@ -332,6 +348,20 @@ def dynamic_quant(x, y, scale, stream=None, **kw):
     check(rc, "aclnnDynamicQuantGetWorkspaceSize")
     run = lib().aclnnDynamicQuantV2 if v2 else lib().aclnnDynamicQuant
     check(run(None, ws, ex, stream.ptr if stream else None), "aclnnDynamicQuant")
+
+
+def dynamic_block_quant_get_workspace(x, y, scale, *, dst_type=None, row_block=1, col_block=128, min_scale=0.0, round_mode=b"rint"):
+    ws, ex = C.c_uint64(0), C.c_void_p()
+    dst = dst_type if dst_type is not None else (y.dtype if y is not None else 36)
+    rc = lib().aclnnDynamicBlockQuantGetWorkspaceSize(_h(x), min_scale, round_mode, dst, row_block, col_block, _h(y), _h(scale),
+                                                      C.byref(ws), C.byref(ex))
+    return rc, ws.value, ex.value
+
+
+def dynamic_block_quant(x, y, scale, stream=None, **kw):
+    rc, ws, ex = dynamic_block_quant_get_workspace(x, y, scale, **kw)
+    check(rc, "aclnnDynamicBlockQuantGetWorkspaceSize")
+    check(lib().aclnnDynamicBlockQuant(None, ws, ex, stream.ptr if stream else None), "aclnnDynamicBlockQuant")
 
 
 def convert_weight_to_int4_pack(weight, weight_int4_pack):

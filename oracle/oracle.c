@@ -46,6 +46,9 @@
  *                       product each fail; numpy float32 recomputation; dequantisation error <= scale / 2); a row of
  *                       zeros (symmetric) or a constant row (asymmetric) divides by zero in the golden: parity unpinned,
  *                       this file writes zeros there
+ *   orc_dynamic_block_quant pinned (numpy float32 recomputation with torch's fp8 casts; a block with max 448 has scale 1
+ *                       and returns x itself through the decimal rounding; min_scale cap and clipping by hand;
+ *                       infinities and NaN by the golden's stated rules)
  *   hifloat8 .......... not implemented (decoder lives only in an absent third-party package): parity unpinned
  */
 #include <math.h>
@@ -874,5 +877,48 @@ int orc_dynamic_quant(const void* x, int x_dt, int64_t rows, int64_t cols, const
         }
     }
     free(v);
+    return 0;
+}
+
+/* Dynamic block quantisation to fp8 (the activation / weight quantizer of the block-scale matmul).
+ * ../quant/dynamic_block_quant/tests/assets/golden.py:95-222, x [batch, rows, cols] in fp16 / bf16, blocks of rb x cb:
+ *   amax  = max over the block of |x|, infinities and NaN counted as 0
+ *   scale = fp32(amax / tmax), and min(scale, fp32(1 / min_scale)) when min_scale != 0   (tmax: 448 e4m3, 57344 e5m2)
+ *   q     = fp32(x) / scale;  where x is infinite or NaN, q = x;  q clipped to +-tmax
+ *   q     = rint(q * 1e8) / 1e8 in fp32  (numpy's round(q, 8) on a float32 array);  NaN -> +0
+ *   y     = fp8(q), round to nearest even
+ * scale_out is [batch, ceil(rows / rb), ceil(cols / cb)]. */
+int orc_dynamic_block_quant(const void* x, int x_dt, int64_t batch, int64_t rows, int64_t cols, int64_t rb, int64_t cb,
+                            double min_scale, int y_dt, uint8_t* y, float* scale_out)
+{
+    if ((x_dt != ORC_F16 && x_dt != ORC_BF16) || (y_dt != ORC_E4M3 && y_dt != ORC_E5M2)) return -1;
+    if (batch <= 0 || rows <= 0 || cols <= 0 || rb <= 0 || cb <= 0 || min_scale < 0) return -1;
+    const float tmax = y_dt == ORC_E4M3 ? 448.0f : 57344.0f;
+    const int64_t nrb = (rows + rb - 1) / rb, ncb = (cols + cb - 1) / cb;
+    for (int64_t b = 0; b < batch; b++)
+        for (int64_t br = 0; br < nrb; br++)
+            for (int64_t bc = 0; bc < ncb; bc++) {
+                const int64_t r1 = (br + 1) * rb < rows ? (br + 1) * rb : rows, c1 = (bc + 1) * cb < cols ? (bc + 1) * cb : cols;
+                float amax = 0.0f;
+                for (int64_t r = br * rb; r < r1; r++)
+                    for (int64_t c = bc * cb; c < c1; c++) {
+                        const float v = fabsf(load_as_f32(x, x_dt, (size_t)((b * rows + r) * cols + c)));
+                        if (isfinite(v) && v > amax) amax = v;
+                    }
+                float scale = amax / tmax;
+                if (min_scale != 0) { const float cap = (float)(1.0 / min_scale); if (cap < scale) scale = cap; }
+                scale_out[(b * nrb + br) * ncb + bc] = scale;
+                for (int64_t r = br * rb; r < r1; r++)
+                    for (int64_t c = bc * cb; c < c1; c++) {
+                        const size_t i = (size_t)((b * rows + r) * cols + c);
+                        const float v = load_as_f32(x, x_dt, i);
+                        float q = isfinite(v) ? v / scale : v;
+                        if (q > tmax) q = tmax;          /* np.clip leaves NaN alone, as these comparisons do */
+                        if (q < -tmax) q = -tmax;
+                        q = nearbyintf(q * 1e8f) / 1e8f;
+                        if (!(q == q)) q = 0.0f;
+                        y[i] = y_dt == ORC_E4M3 ? orc_e4m3_from_f32(q) : orc_e5m2_from_f32(q);
+                    }
+            }
     return 0;
 }

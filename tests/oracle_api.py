@@ -44,6 +44,8 @@ def lib():
         L.orc_dynamic_quant.restype = C.c_int
         L.orc_e5m2_from_f32.argtypes = [C.c_float]
         L.orc_e5m2_from_f32.restype = C.c_uint8
+        L.orc_dynamic_block_quant.argtypes = [vp, C.c_int, i64, i64, i64, i64, i64, C.c_double, C.c_int, vp, vp]
+        L.orc_dynamic_block_quant.restype = C.c_int
         L.orc_scale_generate.argtypes = [C.c_float]
         L.orc_scale_generate.restype = C.c_float
         L.orc_u64_to_deq_scale.argtypes = [C.c_uint64]
@@ -90,6 +92,18 @@ def dynamic_quant(x, x_dt, y_dt, smooth=None, symmetric=True):
                                  y.ctypes.data, scale.ctypes.data, offset.ctypes.data)
     assert rc == 0, rc
     return (y, scale) if symmetric else (y, scale, offset)
+
+
+def dynamic_block_quant(x, x_dt, y_dt, rb, cb, min_scale=0.0):
+    """x: uint16 bits [rows, cols] or [batch, rows, cols].  Returns (y bytes of x's shape, scale [.., ceil(rows/rb), ceil(cols/cb)])."""
+    x = np.ascontiguousarray(x, np.uint16)
+    rows, cols = x.shape[-2:]
+    batch = x.shape[0] if x.ndim == 3 else 1
+    y = np.zeros(x.shape, np.uint8)
+    scale = np.zeros(x.shape[:-2] + (-(-rows // rb), -(-cols // cb)), np.float32)
+    rc = lib().orc_dynamic_block_quant(x.ctypes.data, x_dt, batch, rows, cols, rb, cb, float(min_scale), y_dt, y.ctypes.data, scale.ctypes.data)
+    assert rc == 0, rc
+    return y, scale
 
 
 def convert_weight_b4(w):

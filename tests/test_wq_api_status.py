@@ -104,7 +104,7 @@ def test_library_exports_every_declared_symbol(opsnn):
             "aclnnWeightQuantBatchMatmulV2", "aclnnWeightQuantBatchMatmulV3GetWorkspaceSize", "aclnnWeightQuantBatchMatmulV3",
             "aclnnConvertWeightToINT4PackGetWorkspaceSize", "aclnnConvertWeightToINT4Pack", "opsnnPackB4",
             "aclnnDynamicQuantGetWorkspaceSize", "aclnnDynamicQuant", "aclnnDynamicQuantV2GetWorkspaceSize", "aclnnDynamicQuantV2",
-            "opsnnDynamicQuant",
+            "opsnnDynamicQuant", "aclnnDynamicBlockQuantGetWorkspaceSize", "aclnnDynamicBlockQuant", "opsnnDynamicBlockQuant",
             "opsnnQmmInt8", "opsnnWqmm", "aclCreateTensor"} <= declared
     missing = [n for n in sorted(declared) if not hasattr(lib, n)]
     assert not missing, f"declared in include/ but not exported by the library: {missing}"
