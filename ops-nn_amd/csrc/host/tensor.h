@@ -22,7 +22,7 @@ namespace opsnn {
 
 constexpr uint32_t kExecutorMagic = 0x51454D4Du;
 
-enum class OpKind { None, QmmInt8, QmmBlockScale, QmmMx, QmmTc, QmmGroup, Wqmm, DynQuant, BlockQuant };
+enum class OpKind { None, QmmInt8, QmmBlockScale, QmmMx, QmmTc, QmmGroup, Wqmm, DynQuant, BlockQuant, MxQuant };
 
 // What phase 1 decided; phase 2 only fills in workspace/stream and launches.
 struct aclOpExecutorImpl {
@@ -32,6 +32,7 @@ struct aclOpExecutorImpl {
     OpsnnWqmmArgs wqmm{};
     OpsnnDynQuantArgs dynq{};
     OpsnnBlockQuantArgs blkq{};
+    OpsnnMxQuantArgs mxq{};
     uint64_t workspace_size = 0;
     const char* api = "";
 };

@@ -1,0 +1,207 @@
+// Dynamic MX quantisation along the last axis: 16-bit activations / weights -> fp4 e2m1 or fp8 elements with one e8m0
+// scale per 32 elements, the operand format of the MX matmuls (aclnnDynamicMxQuant; formula
+// quant/dynamic_mx_quant/tests/assets/golden.py:140-153, 196-218, 263-330 with round mode "rint", scale algorithm 0).
+//
+// Per block of 32:  share_exp = floor(log2 max|x|) - emax, at least -127;  q = x * 2^-share_exp (exact);  y = q rounded to
+// nearest even on the element grid, saturated at the format's maximum;  scale byte = share_exp + 127.  A block that holds
+// an infinity or a NaN gets scale 0xFF and zeros.  Scale rows are padded to an even number of bytes with 0.
+// HBM-bound: 2 bytes read and 1 (fp8) or 1/2 (fp4) written per element.  A block is four lanes of a wave with 8 elements
+// each (one 16-byte load per lane), reduced by two lane exchanges; rows whose length is not a multiple of 8 take the
+// one-thread-per-block kernel.
+#include "common.hip.h"
+#include "launch.h"
+
+namespace opsnn {
+
+struct MxQuantParams {
+    const uint16_t* x; uint8_t* y; uint8_t* scale;
+    int64_t rows, cols, nblk, spitch;
+};
+
+template <int X_DT>
+__device__ __forceinline__ float mx_x_to_f32(uint32_t h)
+{
+    if constexpr (X_DT == DT_BF16) return u2f(h << 16);
+    else return f16_to_f32((uint16_t)h);
+}
+
+template <int Y_DT> struct MxFormat;
+template <> struct MxFormat<DT_E2M1> { static constexpr int emax = 2; static constexpr float tmax = 6.0f; };
+template <> struct MxFormat<DT_E4M3> { static constexpr int emax = 8; static constexpr float tmax = 448.0f; };
+template <> struct MxFormat<DT_E5M2> { static constexpr int emax = 15; static constexpr float tmax = 57344.0f; };
+
+// Shared exponent of a block from the bits of its largest magnitude (a finite, non-negative fp32).  floor(log2) of a
+// normal fp32 is its exponent field; a zero or subnormal maximum lands below the floor of -127 in any case.
+template <int Y_DT>
+__device__ __forceinline__ int mx_share_exp(float amax)
+{
+    const int e = (int)(f2u(amax) >> 23);
+    const int s = e - 127 - MxFormat<Y_DT>::emax;
+    return (e == 0 || s < -127) ? -127 : s;
+}
+
+// |q| < 8 rounded to nearest even on {0, .5, 1, 1.5, 2, 3, 4, 6} by the binade of q and saturated at 6 -> code with sign
+// bit.  The step is 2^(max(e, 0) - 1) for a in [2^e, 2^(e+1)); adding and subtracting 1.5 * 2^23 times the step rounds a to
+// a multiple of the step, ties to even.  For r >= 1 the code is r's exponent and first mantissa bit, (bits >> 22) - 252.
+__device__ __forceinline__ uint32_t mx_e2m1_code(float q)
+{
+    const uint32_t sign = (f2u(q) >> 28) & 8u;
+    const float a = fminf(fabsf(q), 6.0f);
+    const uint32_t e = f2u(a) >> 23;
+    const float c = u2f((((e > 127u ? e : 127u) + 22u) << 23) | 0x400000u);
+    const float r = __fsub_rn(__fadd_rn(a, c), c);
+    const uint32_t code = r < 1.0f ? (uint32_t)__fmul_rn(r, 2.0f) : (f2u(r) >> 22) - 252u;
+    return sign | code;
+}
+
+template <int Y_DT>
+__device__ __forceinline__ float mx_scaled(float v, float inv_scale, bool bad)
+{
+    const float q = __fmul_rn(v, inv_scale);   // a power of two: exact
+    return bad ? 0.0f : q;
+}
+
+// eight scaled elements -> their bytes (fp8: 8 bytes in lo/hi; fp4: 4 bytes in lo)
+template <int Y_DT>
+__device__ __forceinline__ uint2 mx_pack8(const float* q)
+{
+    if constexpr (Y_DT == DT_E2M1) {
+        // The hardware conversion (two values -> one byte, low nibble first) returns mx_e2m1_code's nibble for every fp32 of
+        // either sign up to 8 (compared exhaustively on the device, with a unit scale operand); |q| < 8 by construction.
+        uint32_t r = 0;
+        r = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(r, q[0], q[1], 1.0f, 0);
+        r = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(r, q[2], q[3], 1.0f, 1);
+        r = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(r, q[4], q[5], 1.0f, 2);
+        r = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(r, q[6], q[7], 1.0f, 3);
+        return make_uint2(r, 0);
+    } else {
+        constexpr float t = MxFormat<Y_DT>::tmax;
+        uint32_t h[4];
+#pragma unroll
+        for (int e = 0; e < 4; e++)
+            h[e] = cvt2_fp8_in_range<Y_DT>(fminf(fmaxf(q[2 * e], -t), t), fminf(fmaxf(q[2 * e + 1], -t), t));
+        return make_uint2(h[0] | (h[1] << 16), h[2] | (h[3] << 16));
+    }
+}
+
+// cols % 8 == 0: lane groups of four, one (row, block) pair per group
+template <int X_DT, int Y_DT>
+__global__ __launch_bounds__(256) void mx_quant_kernel(MxQuantParams p)
+{
+    const int64_t group = ((int64_t)blockIdx.x * 256 + threadIdx.x) / 4;
+    const int lane = threadIdx.x & 3;
+    const bool live_group = group < p.rows * p.nblk;
+    const int64_t row = live_group ? group / p.nblk : 0, blk = live_group ? group % p.nblk : 0;
+    const int64_t col = blk * 32 + lane * 8;
+    const bool live = live_group && col < p.cols;
+    uint4 buf = make_uint4(0, 0, 0, 0);   // the zero padding of a short last block
+    if (live) buf = *(const uint4*)(p.x + row * p.cols + col);
+    const uint32_t w[4] = {buf.x, buf.y, buf.z, buf.w};
+    float v[8];
+    float amax = 0.0f;
+    bool bad = false;
+#pragma unroll
+    for (int e = 0; e < 8; e++) {
+        v[e] = mx_x_to_f32<X_DT>((w[e >> 1] >> (16 * (e & 1))) & 0xffffu);
+        const float a = fabsf(v[e]);
+        bad |= !(a < __builtin_inff());   // infinity or NaN
+        amax = fmaxf(amax, a);
+    }
+    amax = fmaxf(amax, __shfl_xor(amax, 1));
+    amax = fmaxf(amax, __shfl_xor(amax, 2));
+    bad |= (bool)__shfl_xor((int)bad, 1);
+    bad |= (bool)__shfl_xor((int)bad, 2);
+    const int share = bad ? 0 : mx_share_exp<Y_DT>(amax);
+    if (live_group && lane == 0) {
+        p.scale[row * p.spitch + blk] = bad ? 0xFFu : (uint8_t)(share + 127);
+        if (blk == p.nblk - 1 && (p.nblk & 1)) p.scale[row * p.spitch + blk + 1] = 0;
+    }
+    if (!live) return;
+    // 2^-share: share is in [-127, 125]; 2^127 and 2^-125 are both normal numbers
+    const float inv_scale = u2f((uint32_t)(127 - share) << 23);
+    float q[8];
+#pragma unroll
+    for (int e = 0; e < 8; e++) q[e] = mx_scaled<Y_DT>(v[e], inv_scale, bad);
+    const uint2 out = mx_pack8<Y_DT>(q);
+    if constexpr (Y_DT == DT_E2M1) *(uint32_t*)(p.y + (row * p.cols + col) / 2) = out.x;
+    else *(uint2*)(p.y + row * p.cols + col) = out;
+}
+
+// any row length: one thread per block of 32
+template <int X_DT, int Y_DT>
+__global__ __launch_bounds__(256) void mx_quant_generic_kernel(MxQuantParams p)
+{
+    const int64_t g = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (g >= p.rows * p.nblk) return;
+    const int64_t row = g / p.nblk, blk = g % p.nblk;
+    const int64_t c0 = blk * 32, c1 = c0 + 32 < p.cols ? c0 + 32 : p.cols;
+    const uint16_t* xr = p.x + row * p.cols;
+    float amax = 0.0f;
+    bool bad = false;
+    for (int64_t c = c0; c < c1; c++) {
+        const float a = fabsf(mx_x_to_f32<X_DT>(xr[c]));
+        bad |= !(a < __builtin_inff());
+        amax = fmaxf(amax, a);
+    }
+    const int share = bad ? 0 : mx_share_exp<Y_DT>(amax);
+    p.scale[row * p.spitch + blk] = bad ? 0xFFu : (uint8_t)(share + 127);
+    if (blk == p.nblk - 1 && (p.nblk & 1)) p.scale[row * p.spitch + blk + 1] = 0;
+    const float inv_scale = u2f((uint32_t)(127 - share) << 23);
+    constexpr float t = MxFormat<Y_DT>::tmax;
+    for (int64_t c = c0; c < c1; c += 2) {   // pairs: an fp4 byte holds two columns (cols is even for fp4)
+        const float q0 = mx_scaled<Y_DT>(mx_x_to_f32<X_DT>(xr[c]), inv_scale, bad);
+        const float q1 = c + 1 < c1 ? mx_scaled<Y_DT>(mx_x_to_f32<X_DT>(xr[c + 1]), inv_scale, bad) : 0.0f;
+        if constexpr (Y_DT == DT_E2M1) {
+            p.y[(row * p.cols + c) / 2] = (uint8_t)(mx_e2m1_code(q0) | (mx_e2m1_code(q1) << 4));
+        } else {
+            const uint32_t h = cvt2_fp8_in_range<Y_DT>(fminf(fmaxf(q0, -t), t), fminf(fmaxf(q1, -t), t));
+            p.y[row * p.cols + c] = (uint8_t)h;
+            if (c + 1 < c1) p.y[row * p.cols + c + 1] = (uint8_t)(h >> 8);
+        }
+    }
+}
+
+template <int X_DT, int Y_DT>
+static int launch_mx_quant(const MxQuantParams& p, int variant, hipStream_t st)
+{
+    const bool vec = p.cols % 8 == 0 && (uintptr_t)p.x % 16 == 0 && (uintptr_t)p.y % 8 == 0;
+    const int64_t groups = p.rows * p.nblk;
+    if (variant != 2 && vec) {
+        const int64_t wgs = (groups * 4 + 255) / 256;
+        if (wgs > 0x7fffffff) return -1;
+        hipLaunchKernelGGL((mx_quant_kernel<X_DT, Y_DT>), dim3((unsigned)wgs), dim3(256), 0, st, p);
+    } else {
+        if (variant == 1) return -4;
+        const int64_t wgs = (groups + 255) / 256;
+        if (wgs > 0x7fffffff) return -1;
+        hipLaunchKernelGGL((mx_quant_generic_kernel<X_DT, Y_DT>), dim3((unsigned)wgs), dim3(256), 0, st, p);
+    }
+    return (int)hipGetLastError();
+}
+
+template <int X_DT>
+static int launch_mx_quant_x(const MxQuantParams& p, int y_dt, int variant, hipStream_t st)
+{
+    switch (y_dt) {
+        case DT_E2M1: return launch_mx_quant<X_DT, DT_E2M1>(p, variant, st);
+        case DT_E4M3: return launch_mx_quant<X_DT, DT_E4M3>(p, variant, st);
+        case DT_E5M2: return launch_mx_quant<X_DT, DT_E5M2>(p, variant, st);
+        default: return -2;
+    }
+}
+
+}  // namespace opsnn
+
+using namespace opsnn;
+
+extern "C" int opsnnDynamicMxQuant(const OpsnnMxQuantArgs* a, void* stream)
+{
+    if (!a || !a->x || !a->y || !a->scale || a->rows <= 0 || a->cols <= 0) return -1;
+    if (a->x_dtype != DT_F16 && a->x_dtype != DT_BF16) return -2;
+    if (a->y_dtype == DT_E2M1 && (a->cols & 1)) return -2;
+    MxQuantParams p{};
+    p.x = (const uint16_t*)a->x; p.y = (uint8_t*)a->y; p.scale = (uint8_t*)a->scale;
+    p.rows = a->rows; p.cols = a->cols; p.nblk = (a->cols + 31) / 32; p.spitch = (p.nblk + 1) / 2 * 2;
+    if (a->x_dtype == DT_BF16) return launch_mx_quant_x<DT_BF16>(p, a->y_dtype, a->force_variant, (hipStream_t)stream);
+    return launch_mx_quant_x<DT_F16>(p, a->y_dtype, a->force_variant, (hipStream_t)stream);
+}

@@ -83,6 +83,16 @@ class OpsnnBlockQuantArgs(C.Structure):
     ]
 
 
+class OpsnnMxQuantArgs(C.Structure):
+    _fields_ = [
+        ("x", C.c_void_p), ("x_dtype", C.c_int),
+        ("y", C.c_void_p), ("y_dtype", C.c_int),
+        ("scale", C.c_void_p),
+        ("rows", C.c_int64), ("cols", C.c_int64),
+        ("force_variant", C.c_int),
+    ]
+
+
 _T = C.c_void_p  # aclTensor*
 _SIGS = {
     "aclInit": (C.c_int, [C.c_char_p]),
@@ -134,6 +144,10 @@ _SIGS = {
                                                           C.POINTER(C.c_uint64), C.POINTER(C.c_void_p)]),
     "aclnnDynamicBlockQuant": (C.c_int32, [C.c_void_p, C.c_uint64, C.c_void_p, C.c_void_p]),
     "opsnnDynamicBlockQuant": (C.c_int, [C.POINTER(OpsnnBlockQuantArgs), C.c_void_p]),
+    "aclnnDynamicMxQuantGetWorkspaceSize": (C.c_int32, [_T, C.c_int64, C.c_char_p, C.c_int64, C.c_int64, C.c_int64, _T, _T,
+                                                       C.POINTER(C.c_uint64), C.POINTER(C.c_void_p)]),
+    "aclnnDynamicMxQuant": (C.c_int32, [C.c_void_p, C.c_uint64, C.c_void_p, C.c_void_p]),
+    "opsnnDynamicMxQuant": (C.c_int, [C.POINTER(OpsnnMxQuantArgs), C.c_void_p]),
     "opsnnPackB4": (C.c_int, [C.c_void_p, C.c_int, C.c_void_p, C.c_int64, C.c_void_p]),
     "opsnnQmmInt8": (C.c_int, [C.POINTER(OpsnnQmmArgs), C.c_void_p]),
     "opsnnQmmBlockScale": (C.c_int, [C.POINTER(OpsnnQmmArgs), C.c_void_p]),
@@ -362,6 +376,20 @@ def dynamic_block_quant(x, y, scale, stream=None, **kw):
     rc, ws, ex = dynamic_block_quant_get_workspace(x, y, scale, **kw)
     check(rc, "aclnnDynamicBlockQuantGetWorkspaceSize")
     check(lib().aclnnDynamicBlockQuant(None, ws, ex, stream.ptr if stream else None), "aclnnDynamicBlockQuant")
+
+
+def dynamic_mx_quant_get_workspace(x, y, scale, *, axis=-1, round_mode=b"rint", dst_type=None, blocksize=32, scale_alg=0):
+    ws, ex = C.c_uint64(0), C.c_void_p()
+    dst = dst_type if dst_type is not None else (y.dtype if y is not None else 40)
+    rc = lib().aclnnDynamicMxQuantGetWorkspaceSize(_h(x), axis, round_mode, dst, blocksize, scale_alg, _h(y), _h(scale),
+                                                   C.byref(ws), C.byref(ex))
+    return rc, ws.value, ex.value
+
+
+def dynamic_mx_quant(x, y, scale, stream=None, **kw):
+    rc, ws, ex = dynamic_mx_quant_get_workspace(x, y, scale, **kw)
+    check(rc, "aclnnDynamicMxQuantGetWorkspaceSize")
+    check(lib().aclnnDynamicMxQuant(None, ws, ex, stream.ptr if stream else None), "aclnnDynamicMxQuant")
 
 
 def convert_weight_to_int4_pack(weight, weight_int4_pack):

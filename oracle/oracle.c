@@ -49,6 +49,10 @@
  *   orc_dynamic_block_quant pinned (numpy float32 recomputation with torch's fp8 casts; a block with max 448 has scale 1
  *                       and returns x itself through the decimal rounding; min_scale cap and clipping by hand;
  *                       infinities and NaN by the golden's stated rules)
+ *   orc_dynamic_mx_quant pinned (the OCP MX definition: shared exponent = floor(log2 max) - emax and round-to-nearest-even
+ *                       onto the element grid with saturation, recomputed in numpy with torch's fp8 casts and a brute-force
+ *                       nearest-grid-point search for e2m1; known answers for ties, saturation and the scale bytes; dequantised
+ *                       values within half a grid step)
  *   hifloat8 .......... not implemented (decoder lives only in an absent third-party package): parity unpinned
  */
 #include <math.h>
@@ -920,5 +924,79 @@ int orc_dynamic_block_quant(const void* x, int x_dt, int64_t batch, int64_t rows
                         y[i] = y_dt == ORC_E4M3 ? orc_e4m3_from_f32(q) : orc_e5m2_from_f32(q);
                     }
             }
+    return 0;
+}
+
+/* Dynamic MX quantisation along the last axis (the quantizer of the MX matmuls).
+ * ../quant/dynamic_mx_quant/tests/assets/golden.py:140-153 (shared exponent), 196-218 (element rounding), 263-330 (driver),
+ * round mode "rint", scale algorithm 0, x [rows, cols] in fp16 / bf16, blocks of `block` elements (zero padded):
+ *   amax      = max|x| over the block
+ *   share_exp = floor(log2(amax)) - emax, -127 when amax == 0 or the result is lower; NaN when above 127 (amax infinite) or
+ *               when the block holds a NaN          (emax: 2 for e2m1, 8 for e4m3, 15 for e5m2)
+ *   q         = x / 2^share_exp                                                   (fp32; an exact scaling)
+ *   e         = max(floor(log2|q|), emin), emin = 0 / -6 / -14;  q = rint(q / 2^e * 2^m) / 2^m * 2^e, m = 1 / 3 / 2 mantissa bits
+ *   q clipped to +-tmax (6 / 448 / 57344); NaN -> 0;  y = the element code of q (exact: q is on the format's grid)
+ *   scale byte = share_exp + 127 (e8m0), 0xFF for NaN;  scale rows are padded to an even count with byte 0
+ * e2m1 codes are packed two per byte, even column in the low nibble.  scale_out is [rows, 2 * ceil(nblocks / 2)]. */
+static uint8_t e2m1_code_of(float v)   /* v on the e2m1 grid */
+{
+    const float a = fabsf(v);
+    uint8_t c = 0;
+    for (uint8_t i = 0; i < 8; i++) if (kE2M1[i] == a) c = i;
+    return (uint8_t)(c | (signbit(v) ? 8u : 0u));
+}
+int orc_dynamic_mx_quant(const void* x, int x_dt, int64_t rows, int64_t cols, int64_t block, int y_dt, uint8_t* y, uint8_t* scale_out)
+{
+    int emax, emin, mbits; float tmax;
+    switch (y_dt) {
+        case ORC_E2M1: emax = 2; emin = 0; mbits = 1; tmax = 6.0f; break;
+        case ORC_E4M3: emax = 8; emin = -6; mbits = 3; tmax = 448.0f; break;
+        case ORC_E5M2: emax = 15; emin = -14; mbits = 2; tmax = 57344.0f; break;
+        default: return -1;
+    }
+    if ((x_dt != ORC_F16 && x_dt != ORC_BF16) || rows <= 0 || cols <= 0 || block <= 0 || (y_dt == ORC_E2M1 && (cols & 1))) return -1;
+    const int64_t nblk = (cols + block - 1) / block, spitch = (nblk + 1) / 2 * 2;
+    for (int64_t r = 0; r < rows; r++) {
+        for (int64_t b = 0; b < spitch; b++) scale_out[r * spitch + b] = 0;
+        for (int64_t b = 0; b < nblk; b++) {
+            const int64_t c1 = (b + 1) * block < cols ? (b + 1) * block : cols;
+            float amax = 0.0f; int has_nan = 0;
+            for (int64_t c = b * block; c < c1; c++) {
+                const float a = fabsf(load_as_f32(x, x_dt, (size_t)(r * cols + c)));
+                if (a != a) has_nan = 1;
+                if (a > amax) amax = a;
+            }
+            float share;   /* an integer, or NaN */
+            if (has_nan) share = NAN;
+            else if (amax == 0.0f) share = -127.0f;
+            else {
+                share = floorf(log2f(amax)) - (float)emax;
+                if (share > 127.0f) share = NAN;
+                else if (share < -127.0f) share = -127.0f;
+            }
+            scale_out[r * spitch + b] = (share == share) ? (uint8_t)((int)share + 127) : 0xFFu;
+            for (int64_t c = b * block; c < c1; c++) {
+                const size_t i = (size_t)(r * cols + c);
+                float q = 0.0f;
+                if (share == share) {
+                    q = load_as_f32(x, x_dt, i) / ldexpf(1.0f, (int)share);
+                    float e = floorf(log2f(fabsf(q) + (q == 0.0f ? 1.0f : 0.0f)));
+                    if (e < (float)emin) e = (float)emin;
+                    const float pe = ldexpf(1.0f, (int)e), pm = ldexpf(1.0f, mbits);
+                    q = nearbyintf(q / pe * pm) / pm * pe;
+                    if (q > tmax) q = tmax;
+                    if (q < -tmax) q = -tmax;
+                    if (!(q == q)) q = 0.0f;
+                }
+                if (y_dt == ORC_E4M3) y[i] = orc_e4m3_from_f32(q);
+                else if (y_dt == ORC_E5M2) y[i] = orc_e5m2_from_f32(q);
+                else {
+                    const uint8_t code = e2m1_code_of(q);
+                    uint8_t* p = y + (i >> 1);
+                    *p = (i & 1) ? (uint8_t)((*p & 0x0fu) | (code << 4)) : (uint8_t)((*p & 0xf0u) | code);
+                }
+            }
+        }
+    }
     return 0;
 }

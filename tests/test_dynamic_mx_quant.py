@@ -1,0 +1,203 @@
+"""aclnnDynamicMxQuant (MX quantizer of the fp4 / fp8 MX matmuls): oracle pins, phase-1 status cases, device parity.
+
+The golden (quant/dynamic_mx_quant/tests/assets/golden.py:140-330) states the OCP MX conversion: shared exponent
+floor(log2 max|x|) - emax, elements rounded to nearest even on the element grid and saturated.  The pins recompute that from
+the definition -- torch's fp8 casts, and a brute-force nearest-grid-point search for e2m1 -- and add known answers.
+Device bar: bit-identical elements (the sign of a zero result aside) and scale bytes.
+"""
+import numpy as np
+import pytest
+
+import oracle_api as orc
+
+torch = pytest.importorskip("torch")
+EMAX = {orc.E2M1: 2, orc.E4M3: 8, orc.E5M2: 15}
+TMAX = {orc.E2M1: 6.0, orc.E4M3: 448.0, orc.E5M2: 57344.0}
+GRID4 = np.array([0.0, 0.5, 1.0, 1.5, 2.0, 3.0, 4.0, 6.0])
+
+
+def _codes(y, y_dt):
+    return orc.unpack_nibbles(y) if y_dt == orc.E2M1 else y
+
+
+def _definition(xf, y_dt):
+    """[rows, cols] float32 (cols % 32 == 0) -> (element codes, scale bytes) from the MX definition, in float64."""
+    rows, cols = xf.shape
+    blk = xf.reshape(rows, cols // 32, 32).astype(np.float64)
+    amax = np.abs(blk).max(axis=-1)
+    with np.errstate(divide="ignore"):
+        share = np.where(amax > 0, np.floor(np.log2(np.where(amax > 0, amax, 1.0))) - EMAX[y_dt], -127.0)
+    share = np.maximum(share, -127.0)
+    q = np.clip(blk / 2.0 ** share[..., None], -TMAX[y_dt], TMAX[y_dt]).reshape(rows, cols)
+    if y_dt == orc.E2M1:
+        # nearest grid point, ties to the even code (codes 0, 2, 4, 6 have a zero mantissa bit)
+        d = np.abs(np.abs(q)[..., None] - GRID4)
+        best = d.min(axis=-1, keepdims=True)
+        cand = d == best
+        code = np.where(cand.sum(-1) == 1, cand.argmax(-1), np.where(cand[..., ::2].any(-1), 2 * cand[..., ::2].argmax(-1), cand.argmax(-1)))
+        codes = (code | np.where(np.signbit(q), 8, 0)).astype(np.uint8)
+    else:
+        tdt = torch.float8_e4m3fn if y_dt == orc.E4M3 else torch.float8_e5m2
+        codes = torch.from_numpy(q.astype(np.float32)).to(tdt).view(torch.uint8).numpy()
+    return codes, (share + 127).astype(np.uint8)
+
+
+def _same_but_zero_sign(a, b, y_dt):
+    mag = 0x7 if y_dt == orc.E2M1 else 0x7f
+    z = ((a | b) & mag) == 0
+    return np.array_equal(a[~z], b[~z])
+
+
+# ------------------------------------------------------------------------------------------------ oracle pins (CPU)
+@pytest.mark.parametrize("x_dt", [orc.F16, orc.BF16])
+@pytest.mark.parametrize("y_dt", [orc.E2M1, orc.E4M3, orc.E5M2])
+def test_against_the_mx_definition(x_dt, y_dt):
+    rng = np.random.default_rng(y_dt)
+    shape = (48, 256)
+    xf = (rng.normal(0, 1, size=shape) * 2.0 ** rng.integers(-12, 12, size=(48, 8)).repeat(32, axis=1)).astype(np.float32)
+    xb = orc.f32_to_b16(xf, x_dt)
+    want_codes, want_scale = _definition(orc.b16_to_f32(xb, x_dt), y_dt)
+    y, s = orc.dynamic_mx_quant(xb, x_dt, y_dt)
+    assert np.array_equal(s.reshape(48, -1), want_scale)
+    assert _same_but_zero_sign(_codes(y, y_dt), want_codes, y_dt)
+
+
+def test_known_answers():
+    """Block max 6 -> share_exp 0, scale byte 127, and the fp4 ties go to even: 0.25 -> 0, 0.75 -> 1, 1.25 -> 1, 1.75 -> 2,
+    2.5 -> 2, 3.5 -> 4, 5 -> 4.  Block max 7 -> floor(log2 7) = 2, same scale, 7 saturates to 6.  Block max 448 * 2^-20 with e4m3:
+    byte 107.  A zero block: byte 0 and zeros.  An odd number of blocks pads the scale row with byte 0.  A block with an infinity
+    or a NaN: byte 0xFF and zeros."""
+    x = np.zeros((1, 96), np.float32)
+    x[0, :9] = [6.0, 0.25, 0.75, 1.25, 1.75, 2.5, 3.5, 5.0, -0.75]
+    x[0, 32:34] = [7.0, -7.0]
+    y, s = orc.dynamic_mx_quant(orc.f32_to_bf16(x), orc.BF16, orc.E2M1)
+    c = orc.unpack_nibbles(y)[0]
+    assert list(c[:9]) == [7, 0, 2, 2, 4, 4, 6, 6, 10] and list(c[32:34]) == [7, 15]
+    assert s.shape == (1, 2, 2) and list(s.reshape(-1)) == [127, 127, 0, 0]
+    x8 = np.zeros((2, 64), np.float32)
+    x8[0, 0] = 448.0 * 2.0 ** -20
+    x8[0, 32], x8[1, 5], x8[1, 40] = np.inf, np.nan, 3.0
+    y, s = orc.dynamic_mx_quant(orc.f32_to_bf16(x8), orc.BF16, orc.E4M3)
+    assert list(s.reshape(2, 2)[0]) == [107, 0xFF] and list(s.reshape(2, 2)[1]) == [0xFF, 127 + 1 - 8]
+    assert y[0, 0] == 0x7e and not (y[0, 32:] & 0x7f).any() and not (y[1, :32] & 0x7f).any()
+    assert y[1, 40] == orc.f32_to_e4m3(np.float32([3.0 * 2.0 ** 7]))[0]
+
+
+def test_dequantised_values_are_within_half_a_grid_step():
+    """Relative 2^-4 (half a step of three mantissa bits), or 2^-3 where the block maximum saturates: a block maximum in
+    (448, 512) * scale comes back as 448 * scale."""
+    rng = np.random.default_rng(9)
+    xb = orc.f32_to_bf16(rng.normal(0, 1, size=(64, 512)).astype(np.float32))
+    xf = orc.b16_to_f32(xb, orc.BF16).astype(np.float64)
+    y, s = orc.dynamic_mx_quant(xb, orc.BF16, orc.E4M3)
+    deq = orc.e4m3_to_f32(y).astype(np.float64) * np.repeat(2.0 ** (s.reshape(64, -1).astype(np.float64) - 127), 32, axis=1)
+    assert (np.abs(deq - xf) <= np.maximum(np.abs(xf) * 2.0 ** -3, 2.0 ** -9 * np.repeat(2.0 ** (s.reshape(64, -1).astype(np.float64) - 127), 32, axis=1))).all()
+
+
+# ------------------------------------------------------------------------------------------- status cases (no GPU)
+def _t(m, shape, dt):
+    return m.Tensor(shape, dt, None)
+
+
+def _status(m, x, y, sc, **kw):
+    rc, ws, ex = m.dynamic_mx_quant_get_workspace(x, y, sc, **kw)
+    if ex:
+        m.lib().aclDestroyAclOpExecutor(ex)
+    return rc
+
+
+def test_status_rules(opsnn):
+    """The documented rules (docs/aclnnDynamicMxQuant.md:99-260, 312-320) and its example call (:428-454: axis -1, rint,
+    dstType 36, blocksize 32)."""
+    m = opsnn
+    bad, null, not_run = m.ACLNN_ERR_PARAM_INVALID, m.ACLNN_ERR_PARAM_NULLPTR, 561002
+    f4, f8, e8 = m.ACL_FLOAT4_E2M1, m.ACL_FLOAT8_E4M3FN, m.ACL_FLOAT8_E8M0
+    x, y, sc = _t(m, (4, 6, 320), m.ACL_BF16), _t(m, (4, 6, 320), f8), _t(m, (4, 6, 5, 2), e8)
+    assert _status(m, x, y, sc) == 0 and _status(m, x, y, sc, round_mode=None) == 0
+    assert _status(m, x, _t(m, (4, 6, 320), f4), sc) == 0
+    assert _status(m, _t(m, (96,), m.ACL_FLOAT16), _t(m, (96,), m.ACL_FLOAT8_E5M2), _t(m, (2, 2), e8)) == 0
+    assert _status(m, None, y, sc) == null and _status(m, x, None, sc) == null and _status(m, x, y, None) == null
+    assert _status(m, _t(m, (4, 6, 320), m.ACL_INT8), y, sc) == bad
+    assert _status(m, x, y, sc, dst_type=35) == bad and _status(m, x, _t(m, (4, 6, 320), m.ACL_INT8), sc, dst_type=2) == bad
+    assert _status(m, x, y, _t(m, (4, 6, 5, 2), m.ACL_UINT8 if hasattr(m, "ACL_UINT8") else 4)) == bad
+    assert _status(m, x, y, sc, round_mode=b"floor") == bad and _status(m, x, y, sc, round_mode=b"up") == bad
+    assert _status(m, x, y, sc, blocksize=48) == bad and _status(m, x, y, sc, blocksize=2048) == bad and _status(m, x, y, sc, blocksize=0) == bad
+    assert _status(m, x, y, sc, scale_alg=2) == bad and _status(m, x, _t(m, (4, 6, 320), f4), sc, scale_alg=1) == bad
+    assert _status(m, x, y, sc, axis=3) == bad and _status(m, x, y, sc, axis=-4) == bad
+    assert _status(m, x, _t(m, (4, 6, 160), f8), sc) == bad
+    assert _status(m, _t(m, (4, 31), m.ACL_BF16), _t(m, (4, 31), f4), _t(m, (4, 1, 2), e8)) == bad     # fp4 needs an even last dim
+    assert _status(m, x, y, _t(m, (4, 6, 10), e8)) == bad and _status(m, x, y, _t(m, (4, 6, 6, 2), e8)) == bad
+    # accepted by the reference, no kernel here
+    assert _status(m, x, y, _t(m, (4, 1, 320, 2), e8), axis=1) == not_run
+    assert _status(m, x, y, _t(m, (4, 6, 3, 2), e8), blocksize=64) == not_run
+    assert _status(m, _t(m, (4, 6, 320), m.ACL_FLOAT), y, sc) == not_run
+    assert _status(m, x, _t(m, (4, 6, 320), m.ACL_FLOAT4_E1M2), sc) == not_run
+    assert _status(m, x, _t(m, (4, 6, 320), f4), sc, round_mode=b"floor") == not_run
+    assert _status(m, x, y, sc, scale_alg=1) == not_run
+
+
+# --------------------------------------------------------------------------------------------------- device parity
+ACL_OF = {orc.E2M1: "ACL_FLOAT4_E2M1", orc.E4M3: "ACL_FLOAT8_E4M3FN", orc.E5M2: "ACL_FLOAT8_E5M2"}
+
+
+def _run(m, xb, x_dt, y_dt):
+    cols = xb.shape[-1]
+    nblk = -(-cols // 32)
+    ybytes = xb.size // 2 if y_dt == orc.E2M1 else xb.size
+    sbytes = xb.size // cols * ((nblk + 1) // 2) * 2
+    d_x, d_y, d_s = m.DeviceBuffer(host=xb), m.DeviceBuffer(ybytes + 16), m.DeviceBuffer(sbytes + 16)
+    d_y.fill(0xEE); d_s.fill(0xEE)
+    adt = m.ACL_FLOAT16 if x_dt == orc.F16 else m.ACL_BF16
+    sshape = xb.shape[:-1] + ((nblk + 1) // 2, 2)
+    m.dynamic_mx_quant(m.Tensor(xb.shape, adt, d_x), m.Tensor(xb.shape, m.DTYPE_BY_NAME[ACL_OF[y_dt]], d_y), m.Tensor(sshape, m.ACL_FLOAT8_E8M0, d_s))
+    m.check(m.lib().aclrtSynchronizeDevice(), "sync")
+    gy, gs = d_y.to_host(np.uint8, (ybytes + 16,)), d_s.to_host(np.uint8, (sbytes + 16,))
+    assert (gy[ybytes:] == 0xEE).all() and (gs[sbytes:] == 0xEE).all(), "wrote past an output"
+    return gy[:ybytes], gs[:sbytes].reshape(sshape)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("shape", [(16, 64), (33, 1024), (4, 8192), (3, 5, 320), (7, 40), (6, 1000), (5, 30), (2, 3, 4, 96), (4096,)])
+@pytest.mark.parametrize("x_dt,y_dt", [(orc.BF16, orc.E2M1), (orc.F16, orc.E2M1), (orc.BF16, orc.E4M3), (orc.F16, orc.E5M2)])
+def test_gpu_mx_quant_is_bit_identical(gpu, shape, x_dt, y_dt):
+    m = gpu
+    print(f"case mx quant {shape} x={x_dt} y={y_dt}", flush=True)
+    rng = np.random.default_rng(sum(shape) + y_dt)
+    xf = (rng.normal(0, 1, size=shape) * 2.0 ** rng.integers(-14, 14, size=shape[:-1] + (1,))).astype(np.float32)
+    flat = xf.reshape(-1)
+    flat[:min(40, flat.size // 2)] = 0.0
+    flat[-1] = np.inf
+    if flat.size > 200:
+        flat[100] = np.nan
+    xb = orc.f32_to_b16(xf, x_dt)
+    want_y, want_s = orc.dynamic_mx_quant(xb, x_dt, y_dt)
+    gy, gs = _run(m, xb, x_dt, y_dt)
+    assert np.array_equal(gs, want_s), "scale bytes differ"
+    assert _same_but_zero_sign(_codes(gy, y_dt), _codes(want_y.reshape(-1), y_dt), y_dt)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("fp4", [True, False])
+def test_gpu_mx_quantised_operands_feed_the_mx_matmul(gpu, fp4):
+    """bf16 activation and weight -> aclnnDynamicMxQuant -> aclnnQuantMatmulV5 (MX mode): the operands and the [.., K/64, 2]
+    scale tensors are passed on as they come out; the product is the oracle's on the oracle's quantised operands (fp4
+    products are exact in the matrix core, so identical; fp8 to the MX kernel's bar)."""
+    import cases
+    m = gpu
+    M, K, N = 128, 512, 256
+    y_dt = orc.E2M1 if fp4 else orc.E4M3
+    rng = np.random.default_rng(12)
+    xb = orc.f32_to_bf16(rng.normal(0, 1, size=(M, K)).astype(np.float32))
+    wb = orc.f32_to_bf16(rng.normal(0, 0.05, size=(N, K)).astype(np.float32))
+    gx, sx = _run(m, xb, orc.BF16, y_dt)
+    gw, sw = _run(m, wb, orc.BF16, y_dt)
+    ox, osx = orc.dynamic_mx_quant(xb, orc.BF16, y_dt)
+    ow, osw = orc.dynamic_mx_quant(wb, orc.BF16, y_dt)
+    assert np.array_equal(sx, osx) and np.array_equal(sw, osw)
+    kb = K // 2 if fp4 else K
+    inp = dict(x1=gx.reshape(1, M, kb), x2=gw.reshape(1, N, kb), s1=sx[None], s2=sw[None], fp4=fp4)
+    want = cases.oracle_mx(m, dict(inp, x1=ox[None], x2=ow[None]), M, K, N, True, m.ACL_BF16)
+    got = cases.run_mx_aclnn(m, inp, M, K, N, True, m.ACL_BF16)
+    g, w = orc.b16_to_f32(got, orc.BF16), orc.b16_to_f32(want, orc.BF16)
+    mx, mean = orc.rel_err_stats(g, w)
+    assert mx <= 2.0 ** -7 and mean <= 2.0 ** -10, f"max rel {mx:.3e} mean rel {mean:.3e}"

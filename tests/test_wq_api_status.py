@@ -105,6 +105,7 @@ def test_library_exports_every_declared_symbol(opsnn):
             "aclnnConvertWeightToINT4PackGetWorkspaceSize", "aclnnConvertWeightToINT4Pack", "opsnnPackB4",
             "aclnnDynamicQuantGetWorkspaceSize", "aclnnDynamicQuant", "aclnnDynamicQuantV2GetWorkspaceSize", "aclnnDynamicQuantV2",
             "opsnnDynamicQuant", "aclnnDynamicBlockQuantGetWorkspaceSize", "aclnnDynamicBlockQuant", "opsnnDynamicBlockQuant",
+            "aclnnDynamicMxQuantGetWorkspaceSize", "aclnnDynamicMxQuant", "opsnnDynamicMxQuant",
             "opsnnQmmInt8", "opsnnWqmm", "aclCreateTensor"} <= declared
     missing = [n for n in sorted(declared) if not hasattr(lib, n)]
     assert not missing, f"declared in include/ but not exported by the library: {missing}"
