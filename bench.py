@@ -31,7 +31,8 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--config", type=int, default=2)
+    ap.add_argument("--config", type=int, default=2,
+                    help="1-5: the BASELINE configs; 6-9: the pre-pack / quantizer operators that prepare their tensors")
     ap.add_argument("--m", type=int, default=None, help="M for config 3 (1, 16, 64 or 256)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--int8-range", type=int, default=None,

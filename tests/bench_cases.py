@@ -16,6 +16,7 @@ import oracle_api as orc
 MEASURED_TRAFFIC = {
     (2, None): 101.9e6, (4, None): 824.4e6, (5, None): 1802.2e6,
     (3, 1): 67.2e6, (3, 16): 69.2e6, (1, None): 9.2e6,
+    (6, None): 583.0e6, (7, None): 132.4e6, (8, None): 391.5e6, (9, None): 406.1e6,
 }
 
 
@@ -270,7 +271,78 @@ class ConfigWQ(Workload):
                 "sample": f"the whole workload once (oracle/liboracle.so, OpenMP), {t:.2f} s"}
 
 
+class PrepOp(Workload):
+    """The operators either side of the matmuls, each on the tensor of the BASELINE config it prepares (HBM-bound):
+    6 aclnnConvertWeightToINT4Pack on config 3's weight; 7 aclnnDynamicQuant (int8) on config 2's activation, 8 batches of it;
+    8 aclnnDynamicBlockQuant (e4m3, 128 x 128) on config 4's weight; 9 aclnnDynamicMxQuant (e2m1) on config 5's activation."""
+    metric = "prep_op_bandwidth"
+    bound = "hbm"
+
+    def __init__(self, m, args, config):
+        self.m, self.op = m, config
+        rng = np.random.default_rng(0)
+        if config == 6:
+            K, N = 8192, 28672
+            self.host = rng.integers(-8, 8, size=(K, N)).astype(np.int32)
+            self.d_in, self.d_out = m.DeviceBuffer(host=self.host), m.DeviceBuffer(K * N // 2)
+            self.count = K * N
+            self.bytes = K * N * 4 + K * N // 2
+            self.kernel, self.dtype = "pack_b4_kernel", "u32"
+            self.config = {"workload": "aclnnConvertWeightToINT4Pack on config 3's weight", "K": K, "N": N}
+            return
+        rows, cols = {7: (8 * 2048, 4096), 8: (18432, 7168), 9: (8 * 4096, 8192)}[config]
+        self.rows, self.cols = rows, cols
+        self.xb = orc.f32_to_bf16(rng.normal(0, 1, size=(rows, cols)).astype(np.float32))
+        self.d_in = m.DeviceBuffer(host=self.xb)
+        x = m.Tensor((rows, cols), m.ACL_BF16, self.d_in)
+        if config == 7:
+            self.d_out, self.d_sc = m.DeviceBuffer(rows * cols), m.DeviceBuffer(rows * 4)
+            self.tensors = (x, m.Tensor((rows, cols), m.ACL_INT8, self.d_out), m.Tensor((rows,), m.ACL_FLOAT, self.d_sc))
+            self.bytes = rows * cols * 3 + rows * 4
+            self.kernel, self.dtype = "dynamic_quant_rows_kernel", "f32"
+            self.config = {"workload": "aclnnDynamicQuant (int8, per token) on 8 batches of config 2's activation", "rows": rows, "cols": cols}
+        elif config == 8:
+            self.d_out, self.d_sc = m.DeviceBuffer(rows * cols), m.DeviceBuffer(rows // 128 * (cols // 128) * 4)
+            self.tensors = (x, m.Tensor((rows, cols), m.ACL_FLOAT8_E4M3FN, self.d_out), m.Tensor((rows // 128, cols // 128), m.ACL_FLOAT, self.d_sc))
+            self.bytes = rows * cols * 3 + rows // 128 * (cols // 128) * 4
+            self.kernel, self.dtype = "block_quant_tile_kernel", "f32"
+            self.config = {"workload": "aclnnDynamicBlockQuant (e4m3, 128 x 128 blocks) on config 4's weight", "rows": rows, "cols": cols}
+        else:
+            self.d_out, self.d_sc = m.DeviceBuffer(rows * cols // 2), m.DeviceBuffer(rows * cols // 32)
+            self.tensors = (x, m.Tensor((rows, cols), m.ACL_FLOAT4_E2M1, self.d_out), m.Tensor((rows, cols // 64, 2), m.ACL_FLOAT8_E8M0, self.d_sc))
+            self.bytes = rows * cols * 2 + rows * cols // 2 + rows * cols // 32
+            self.kernel, self.dtype = "mx_quant_kernel", "f32"
+            self.config = {"workload": "aclnnDynamicMxQuant (e2m1, blocks of 32) on config 5's activation, all 8 batches", "rows": rows, "cols": cols}
+
+    def step(self, stream):
+        m = self.m
+        if self.op == 6:   # the aclnn entry point of this op works on the null stream and waits; the stream form is timed
+            m.check(m.lib().opsnnPackB4(self.d_in.ptr, 0, self.d_out.ptr, self.count, stream.ptr), "opsnnPackB4")
+        elif self.op == 7:
+            m.dynamic_quant(*self.tensors, stream=stream)
+        elif self.op == 8:
+            m.dynamic_block_quant(*self.tensors, stream=stream, row_block=128, col_block=128)
+        else:
+            m.dynamic_mx_quant(*self.tensors, stream=stream)
+
+    def cpu_baseline(self):
+        t0 = time.perf_counter()
+        if self.op == 6:
+            orc.convert_weight_b4(self.host)
+        elif self.op == 7:
+            orc.dynamic_quant(self.xb, orc.BF16, orc.I8)
+        elif self.op == 8:
+            orc.dynamic_block_quant(self.xb, orc.BF16, orc.E4M3, 128, 128)
+        else:
+            orc.dynamic_mx_quant(self.xb, orc.BF16, orc.E2M1)
+        t = time.perf_counter() - t0
+        return {"value": self.bytes / t / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
+                "sample": f"the whole workload once (oracle/liboracle.so, one thread), {t:.2f} s"}
+
+
 def make_workload(m, config, args):
+    if config in (6, 7, 8, 9):
+        return PrepOp(m, args, config)
     if config in (1, 3):
         return ConfigWQ(m, args, config)
     if config == 2:
