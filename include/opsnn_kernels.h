@@ -135,6 +135,14 @@ OPSNN_API int opsnnTranspose4(const void* src, void* dst, int64_t rows, int64_t 
  * matmul/convert_weight_to_int4_pack/op_host/op_api/aclnn_convert_weight_to_int4_pack.cpp:79-126. */
 OPSNN_API int opsnnPackB4(const void* src, int src_is_fp32, void* dst, int64_t count, void* stream);
 
+/* fp32 scale (and optional fp32 offset) -> the 64-bit packed quantisation parameter of the per-tensor / per-channel
+ * matmul modes: the scale cut to 19 bits in the low word (round_mode 0: truncated, 1: rounded to nearest even), the offset
+ * as a signed 9-bit integer at bits 37..45, bit 46 set.  A one-element scale or offset is broadcast; out has
+ * max(scale_len, offset_len) elements.  Device kernel of the reference: quant/trans_quant_param_v2/op_kernel/
+ * trans_quant_param_v2.h:224-300. */
+OPSNN_API int opsnnTransQuantParam(const float* scale, int64_t scale_len, const float* offset, int64_t offset_len, int round_mode,
+                                   uint64_t* out, void* stream);
+
 /* Dynamic per-token quantisation of x [rows, cols] (FLOAT16 / BF16, dense): per row a scale (and, when `offset` is not
  * NULL, an offset: the asymmetric form) and the quantised row y in INT8, INT4 (two per byte, even column in the low nibble;
  * cols even), FLOAT8_E4M3FN or FLOAT8_E5M2.  smooth: NULL or [cols] factors of x's dtype.  Formula:

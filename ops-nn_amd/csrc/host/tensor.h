@@ -22,7 +22,7 @@ namespace opsnn {
 
 constexpr uint32_t kExecutorMagic = 0x51454D4Du;
 
-enum class OpKind { None, QmmInt8, QmmBlockScale, QmmMx, QmmTc, QmmGroup, Wqmm, DynQuant, BlockQuant, MxQuant };
+enum class OpKind { None, QmmInt8, QmmBlockScale, QmmMx, QmmTc, QmmGroup, Wqmm, DynQuant, BlockQuant, MxQuant, TransQuantParam };
 
 // What phase 1 decided; phase 2 only fills in workspace/stream and launches.
 struct aclOpExecutorImpl {
@@ -33,6 +33,7 @@ struct aclOpExecutorImpl {
     OpsnnDynQuantArgs dynq{};
     OpsnnBlockQuantArgs blkq{};
     OpsnnMxQuantArgs mxq{};
+    struct { const float* scale; int64_t scale_len; const float* offset; int64_t offset_len; int round_mode; uint64_t* out; } tqp{};
     uint64_t workspace_size = 0;
     const char* api = "";
 };

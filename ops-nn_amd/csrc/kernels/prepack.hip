@@ -66,3 +66,60 @@ extern "C" int opsnnPackB4(const void* src, int src_is_fp32, void* dst, int64_t 
     else hipLaunchKernelGGL(pack_b4_kernel<false>, grid, block, 0, (hipStream_t)stream, (const uint32_t*)src, (uint8_t*)dst, count);
     return (int)hipGetLastError();
 }
+
+// ---------------------------------------------------------------------------------------------------------------------
+// aclnnTransQuantParamV2 / V3: fp32 scale (+ fp32 offset) -> the 64-bit packed quantisation parameter the per-tensor /
+// per-channel matmul modes take (quant/trans_quant_param_v2/op_kernel/trans_quant_param_v2.h:224-300):
+//   bits 0..31  the scale cut to sign, exponent and 10 mantissa bits -- truncated (round mode 0) or rounded to nearest
+//               even with the carry running into the exponent, zero for a subnormal, infinity / NaN kept (round mode 1)
+//   bits 37..45 rint(offset) clamped to [-256, 255] as a signed 9-bit field
+//   bit 46      set
+// A one-element scale or offset is broadcast; out has max(scale_len, offset_len) elements.
+namespace opsnn {
+
+__device__ __forceinline__ uint32_t scale_to_fp19(uint32_t u, int round_mode)
+{
+    if (round_mode == 0) return u & 0xFFFFE000u;
+    const uint32_t sign = u >> 31;
+    uint32_t exponent = (u >> 23) & 0xFFu, mant = (u & 0x7FFFFFu) >> 13;
+    const uint32_t round_bit = (u >> 12) & 1u, sticky = u & 0xFFFu;
+    uint32_t fp19;
+    if (exponent == 0u) fp19 = sign << 18;
+    else if (exponent == 255u) fp19 = (sign << 18) | (exponent << 10) | mant;
+    else {
+        if (round_bit && (sticky || (mant & 1u))) {
+            mant += 1u;
+            if (mant >= 1024u) { mant = 0u; exponent += 1u; }
+        }
+        fp19 = (sign << 18) | (exponent << 10) | mant;   // a carry out of exponent 254 gives 255 with mantissa 0: infinity
+    }
+    return fp19 << 13;
+}
+
+__global__ __launch_bounds__(256) void trans_quant_param_kernel(const float* __restrict__ scale, int64_t scale_len,
+                                                                const float* __restrict__ offset, int64_t offset_len, int round_mode,
+                                                                uint64_t* __restrict__ out, int64_t n)
+{
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n) return;
+    uint64_t v = (uint64_t)scale_to_fp19(f2u(scale[scale_len == 1 ? 0 : i]), round_mode) | (1ull << 46);
+    if (offset) {
+        float o = __builtin_rintf(offset[offset_len == 1 ? 0 : i]);
+        o = (o == o) ? fminf(fmaxf(o, -256.0f), 255.0f) : 0.0f;
+        v |= ((uint64_t)(int64_t)(int)o & 0x1FFull) << 37;
+    }
+    out[i] = v;
+}
+
+}  // namespace opsnn
+
+extern "C" int opsnnTransQuantParam(const float* scale, int64_t scale_len, const float* offset, int64_t offset_len, int round_mode,
+                                    uint64_t* out, void* stream)
+{
+    if (!scale || !out || scale_len <= 0 || (offset && offset_len <= 0) || (round_mode != 0 && round_mode != 1)) return -1;
+    const int64_t n = offset && offset_len > scale_len ? offset_len : scale_len;
+    if ((scale_len != 1 && scale_len != n) || (offset && offset_len != 1 && offset_len != n)) return -2;
+    hipLaunchKernelGGL(trans_quant_param_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, (hipStream_t)stream, scale, scale_len,
+                       offset, offset ? offset_len : 0, round_mode, out, n);
+    return (int)hipGetLastError();
+}

@@ -148,6 +148,11 @@ _SIGS = {
                                                        C.POINTER(C.c_uint64), C.POINTER(C.c_void_p)]),
     "aclnnDynamicMxQuant": (C.c_int32, [C.c_void_p, C.c_uint64, C.c_void_p, C.c_void_p]),
     "opsnnDynamicMxQuant": (C.c_int, [C.POINTER(OpsnnMxQuantArgs), C.c_void_p]),
+    "aclnnTransQuantParamV2GetWorkspaceSize": (C.c_int32, [_T, _T, _T, C.POINTER(C.c_uint64), C.POINTER(C.c_void_p)]),
+    "aclnnTransQuantParamV2": (C.c_int32, [C.c_void_p, C.c_uint64, C.c_void_p, C.c_void_p]),
+    "aclnnTransQuantParamV3GetWorkspaceSize": (C.c_int32, [_T, _T, C.c_int64, _T, C.POINTER(C.c_uint64), C.POINTER(C.c_void_p)]),
+    "aclnnTransQuantParamV3": (C.c_int32, [C.c_void_p, C.c_uint64, C.c_void_p, C.c_void_p]),
+    "opsnnTransQuantParam": (C.c_int, [C.c_void_p, C.c_int64, C.c_void_p, C.c_int64, C.c_int, C.c_void_p, C.c_void_p]),
     "opsnnPackB4": (C.c_int, [C.c_void_p, C.c_int, C.c_void_p, C.c_int64, C.c_void_p]),
     "opsnnQmmInt8": (C.c_int, [C.POINTER(OpsnnQmmArgs), C.c_void_p]),
     "opsnnQmmBlockScale": (C.c_int, [C.POINTER(OpsnnQmmArgs), C.c_void_p]),
@@ -390,6 +395,23 @@ def dynamic_mx_quant(x, y, scale, stream=None, **kw):
     rc, ws, ex = dynamic_mx_quant_get_workspace(x, y, scale, **kw)
     check(rc, "aclnnDynamicMxQuantGetWorkspaceSize")
     check(lib().aclnnDynamicMxQuant(None, ws, ex, stream.ptr if stream else None), "aclnnDynamicMxQuant")
+
+
+def trans_quant_param_get_workspace(scale, offset, out, round_mode=None):
+    """Phase 1 of aclnnTransQuantParamV2, or V3 when round_mode is given."""
+    ws, ex = C.c_uint64(0), C.c_void_p()
+    if round_mode is None:
+        rc = lib().aclnnTransQuantParamV2GetWorkspaceSize(_h(scale), _h(offset), _h(out), C.byref(ws), C.byref(ex))
+    else:
+        rc = lib().aclnnTransQuantParamV3GetWorkspaceSize(_h(scale), _h(offset), round_mode, _h(out), C.byref(ws), C.byref(ex))
+    return rc, ws.value, ex.value
+
+
+def trans_quant_param(scale, offset, out, round_mode=None, stream=None):
+    rc, ws, ex = trans_quant_param_get_workspace(scale, offset, out, round_mode)
+    check(rc, "aclnnTransQuantParamGetWorkspaceSize")
+    run = lib().aclnnTransQuantParamV2 if round_mode is None else lib().aclnnTransQuantParamV3
+    check(run(None, ws, ex, stream.ptr if stream else None), "aclnnTransQuantParam")
 
 
 def convert_weight_to_int4_pack(weight, weight_int4_pack):

@@ -53,6 +53,9 @@
  *                       onto the element grid with saturation, recomputed in numpy with torch's fp8 casts and a brute-force
  *                       nearest-grid-point search for e2m1; known answers for ties, saturation and the scale bytes; dequantised
  *                       values within half a grid step)
+ *   orc_trans_quant_param pinned (the packing utility of the matmul golden and the reference's system-test formula in numpy;
+ *                       its inverse orc_u64_to_deq_scale; hand-derived cases of the rounding mode: ties, carry into the
+ *                       exponent, overflow to infinity, subnormal)
  *   hifloat8 .......... not implemented (decoder lives only in an absent third-party package): parity unpinned
  */
 #include <math.h>
@@ -999,4 +1002,38 @@ int orc_dynamic_mx_quant(const void* x, int x_dt, int64_t rows, int64_t cols, in
         }
     }
     return 0;
+}
+
+/* aclnnTransQuantParamV2 / V3: the packed 64-bit quantisation parameter (../quant/trans_quant_param_v2/op_kernel/
+ * trans_quant_param_v2.h:224-300; the same layout GQ:129-158 reads back).  round_mode 0 keeps the upper 19 bits of the scale;
+ * round_mode 1 rounds the 23-bit mantissa to 10 bits, nearest even, the carry running into the exponent, a zero or subnormal
+ * scale becoming a signed zero and infinity / NaN keeping their (truncated) bits.  The offset is rint'ed, clamped to
+ * [-256, 255] and stored as 9 bits at bit 37; bit 46 is set.  One-element inputs are broadcast. */
+void orc_trans_quant_param(const float* scale, int64_t scale_len, const float* offset, int64_t offset_len, int round_mode, uint64_t* out)
+{
+    const int64_t n = (offset && offset_len > scale_len) ? offset_len : scale_len;
+    for (int64_t i = 0; i < n; i++) {
+        const uint32_t u = f2u(scale[scale_len == 1 ? 0 : i]);
+        uint32_t lo;
+        if (round_mode == 0) lo = u & 0xFFFFE000u;
+        else {
+            const uint32_t sign = u >> 31;
+            uint32_t e = (u >> 23) & 0xFFu, m = (u & 0x7FFFFFu) >> 13;
+            if (e == 0) { m = 0; }
+            else if (e != 255) {
+                const uint32_t rest = u & 0x1FFFu;               /* the 13 dropped bits */
+                if (rest > 0x1000u || (rest == 0x1000u && (m & 1u))) { m += 1; if (m == 1024u) { m = 0; e += 1; } }
+            }
+            lo = (sign << 31) | (e << 23) | (m << 13);
+        }
+        uint64_t v = (uint64_t)lo | (1ull << 46);
+        if (offset) {
+            float o = nearbyintf(offset[offset_len == 1 ? 0 : i]);
+            if (!(o == o)) o = 0.0f;
+            if (o < -256.0f) o = -256.0f;
+            if (o > 255.0f) o = 255.0f;
+            v |= ((uint64_t)(int64_t)(int)o & 0x1FFull) << 37;
+        }
+        out[i] = v;
+    }
 }

@@ -48,6 +48,8 @@ def lib():
         L.orc_dynamic_block_quant.restype = C.c_int
         L.orc_dynamic_mx_quant.argtypes = [vp, C.c_int, i64, i64, i64, C.c_int, vp, vp]
         L.orc_dynamic_mx_quant.restype = C.c_int
+        L.orc_trans_quant_param.argtypes = [vp, i64, vp, i64, C.c_int, vp]
+        L.orc_trans_quant_param.restype = None
         L.orc_scale_generate.argtypes = [C.c_float]
         L.orc_scale_generate.restype = C.c_float
         L.orc_u64_to_deq_scale.argtypes = [C.c_uint64]
@@ -119,6 +121,16 @@ def dynamic_mx_quant(x, x_dt, y_dt, block=32):
     rc = lib().orc_dynamic_mx_quant(x.ctypes.data, x_dt, rows, cols, block, y_dt, y.ctypes.data, scale.ctypes.data)
     assert rc == 0, rc
     return y, scale
+
+
+def trans_quant_param(scale, offset=None, round_mode=0):
+    scale = np.ascontiguousarray(scale, np.float32).reshape(-1)
+    off = None if offset is None else np.ascontiguousarray(offset, np.float32).reshape(-1)
+    n = max(scale.size, off.size if off is not None else 0)
+    out = np.zeros(n, np.uint64)
+    lib().orc_trans_quant_param(scale.ctypes.data, scale.size, off.ctypes.data if off is not None else None,
+                                off.size if off is not None else 0, round_mode, out.ctypes.data)
+    return out
 
 
 def convert_weight_b4(w):

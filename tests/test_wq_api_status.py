@@ -106,6 +106,8 @@ def test_library_exports_every_declared_symbol(opsnn):
             "aclnnDynamicQuantGetWorkspaceSize", "aclnnDynamicQuant", "aclnnDynamicQuantV2GetWorkspaceSize", "aclnnDynamicQuantV2",
             "opsnnDynamicQuant", "aclnnDynamicBlockQuantGetWorkspaceSize", "aclnnDynamicBlockQuant", "opsnnDynamicBlockQuant",
             "aclnnDynamicMxQuantGetWorkspaceSize", "aclnnDynamicMxQuant", "opsnnDynamicMxQuant",
+            "aclnnTransQuantParamV2GetWorkspaceSize", "aclnnTransQuantParamV2", "aclnnTransQuantParamV3GetWorkspaceSize",
+            "aclnnTransQuantParamV3", "opsnnTransQuantParam",
             "opsnnQmmInt8", "opsnnWqmm", "aclCreateTensor"} <= declared
     missing = [n for n in sorted(declared) if not hasattr(lib, n)]
     assert not missing, f"declared in include/ but not exported by the library: {missing}"
