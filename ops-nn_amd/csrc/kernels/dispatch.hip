@@ -58,9 +58,11 @@ extern "C" int opsnnQmmMx(const OpsnnQmmArgs* a, void* stream)
     return launch_mx_plain(*a, (hipStream_t)stream);
 }
 
-// Per-tensor / per-channel family.  The per-token x per-channel int8 kernel already covers int8 operands with a
-// float scale and a 16-bit output when the scale needs no 19-bit truncation; everything else (64-bit packed scales,
-// int8 requantisation, fp8 operands, truncated scales) runs on the plain kernel.
+// Per-tensor / per-channel family.  The int8 MFMA kernels cover int8 operands with a 16-bit, INT32 or INT8 output (the
+// latter two through their integer epilogue), the fp8 row/column-scale kernel covers e4m3 operands with separately
+// multiplied scales; the rest (e5m2 operands, merged and truncated double scales, fp32 output, odd layouts) runs on the
+// plain kernel.
+extern "C" __attribute__((visibility("hidden"))) int opsnn_qmm_int8_impl(const OpsnnQmmArgs* a, void* stream);   // qmm_int8.hip
 extern "C" int opsnnQmmTc(const OpsnnQmmArgs* a, void* stream)
 {
     if (!qmm_args_ok(a) || !a->x2_scale) return -1;
@@ -80,6 +82,15 @@ extern "C" int opsnnQmmTc(const OpsnnQmmArgs* a, void* stream)
         b.x2_scale_trunc = a->x2_scale_dtype == DT_U64 ||
                            (a->x2_scale_len == 1 && !(a->bias && (a->bias_dtype == DT_BF16 || a->bias_dtype == DT_F32)));
         return opsnnQmmInt8(&b, stream);
+    }
+    // int8 operands with an INT32 output (sums + int32 bias) or an INT8 output (requantised): integer epilogue of the MFMA
+    // kernel, bit-identical; a float bias with INT32 output stays on the plain kernel
+    if (i8 && !a->x1_scale && (a->out_dtype == DT_I32 || a->out_dtype == DT_I8) && (!a->bias || a->bias_dtype == DT_I32) &&
+        a->force_variant != OPSNN_VARIANT_PLAIN && !opsnn_force_plain()) {
+        OpsnnQmmArgs b = *a;
+        b.x2_scale_trunc = 0;   // UINT64 words are always truncated; a float scale is used as it is
+        const int rc = opsnn_qmm_int8_impl(&b, stream);
+        if (rc != OPSNN_NOT_TAKEN) return rc;
     }
     // fp8 e4m3 operands with a row scale and a column scale that are multiplied in separately (K-C, K-T, T-C with the
     // one-element x1Scale): matrix-core kernel when the layout allows, else the plain kernel
@@ -131,7 +142,8 @@ extern "C" uint64_t opsnnQmmWorkspace(const OpsnnQmmArgs* a, int mode)
 {
     if (!a) return 0;
     if (mode == 2) return mx_workspace_bytes(*a);
-    if (mode == 3) return 0;   // per-tensor / per-channel family: strided kernel, no re-layout
+    // per-tensor / per-channel family: int8 operands share the int8 kernels and their re-layout; fp8 needs none
+    if (mode == 3 && !(a->x1_dtype == DT_I8 && a->x2_dtype == DT_I8 && !a->x1_scale)) return 0;
     if (mode == 4) return tcg_workspace_bytes(*a);   // K-group modes: the re-quantised weight of the fp8 x fp4 group-scale mode
     if (a->x2.row_stride == 1 || a->K == 1) return 0;           // already K-contiguous
     if (a->x2.col_stride != 1 || a->x2.row_stride != a->N) return 0;  // not a dense [K, N]: plain kernel

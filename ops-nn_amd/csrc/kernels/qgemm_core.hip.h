@@ -44,6 +44,10 @@ struct QgemmParams {
     int x2s_dt;
     int64_t x2s_len;
     int x2s_trunc;     // keep only the upper 19 bits of the scale (always done for UINT64 words)
+    // integer outputs of MODE_I8 (OUT_DT INT32: acc + ib[n];  INT8: clip(s9(s9(fp32(acc + ib[n]) * x2s[n]) + s9(off[n])), the offset
+    // from x2off or, for UINT64 scale words, from their bits 37..45; s9 = round half to even, clamp to [-256, 255])
+    const float* x2off;
+    int64_t x2off_len;
     // bias: int32 / 16-bit / fp32 for MODE_I8, fp32 for the MX modes
     const void* bias;
     int bias_dt;
@@ -457,6 +461,78 @@ __global__ __launch_bounds__(WGM* WGN * 64, MINWG) void qgemm_kernel(QgemmParams
             }
         }
     }
+    if constexpr (OUT_DT == DT_I32 || OUT_DT == DT_I8) {
+        // Integer outputs leave straight from the registers: a lane holds four consecutive columns of one row per register
+        // quad, 16 bytes (INT32) or 4 bytes (INT8) per store.
+        static_assert(MODE == MODE_I8, "integer outputs belong to the int8 mode");
+        float* sOff = (float*)smem + 3 * BN + BM;
+        const bool has_off = p.x2off != nullptr || p.x2s_dt == DT_U64;
+        if (OUT_DT == DT_I8 && has_off) {
+            for (int i = tid; i < BN; i += NT) {
+                int64_t n = n0 + i;
+                if (n >= p.N) n = p.N - 1;
+                float off;
+                if (p.x2off) off = p.x2off[p.x2off_len == 1 ? 0 : n];
+                else {
+                    int raw = (int)((((const uint64_t*)p.x2s)[p.x2s_len == 1 ? 0 : n] >> 37) & 0x1FF);
+                    off = (float)(raw & 0x100 ? raw - 0x200 : raw);
+                }
+                const float r = __builtin_rintf(off);
+                sOff[i] = r < -256.0f ? -256.0f : (r > 255.0f ? 255.0f : r);
+            }
+        }
+        __syncthreads();
+        const bool vec_ok = (p.ldc % 4) == 0 && ((uintptr_t)p.out % 16) == 0;
+#pragma unroll
+        for (int j = 0; j < FM; j++) {
+            const int64_t m = m0 + wm * TM + j * 32 + frow;
+#pragma unroll
+            for (int i = 0; i < FN; i++) {
+#pragma unroll
+                for (int q = 0; q < 4; q++) {
+                    const int nl = wn * TN + i * 32 + 8 * q + 4 * fkc;
+                    const int64_t n = n0 + nl;
+                    const v4i ib = *(const v4i*)(sIb + nl);
+                    v4i o;
+                    if constexpr (OUT_DT == DT_I32) {
+#pragma unroll
+                        for (int e = 0; e < 4; e++) o[e] = acc[i][j][q * 4 + e] + ib[e];
+                        if (m < p.M) {
+                            int32_t* dst = (int32_t*)p.out + (bz * p.M + m) * p.ldc + n;
+                            if (vec_ok && n + 3 < p.N) *(v4i*)dst = o;
+                            else {
+#pragma unroll
+                                for (int e = 0; e < 4; e++)
+                                    if (n + e < p.N) dst[e] = o[e];
+                            }
+                        }
+                    } else {
+                        const v4f s2 = *(const v4f*)(sS2 + nl);
+                        uint32_t packed = 0;
+#pragma unroll
+                        for (int e = 0; e < 4; e++) {
+                            float t = __builtin_rintf((float)(acc[i][j][q * 4 + e] + ib[e]) * s2[e]);
+                            t = t < -256.0f ? -256.0f : (t > 255.0f ? 255.0f : t);
+                            if (has_off) t = t + sOff[nl + e];
+                            t = t < -128.0f ? -128.0f : (t > 127.0f ? 127.0f : t);
+                            o[e] = (int)t;
+                            packed |= ((uint32_t)o[e] & 0xffu) << (8 * e);
+                        }
+                        if (m < p.M) {
+                            int8_t* dst = (int8_t*)p.out + (bz * p.M + m) * p.ldc + n;
+                            if (vec_ok && n + 3 < p.N) *(uint32_t*)dst = packed;
+                            else {
+#pragma unroll
+                                for (int e = 0; e < 4; e++)
+                                    if (n + e < p.N) dst[e] = (int8_t)o[e];
+                            }
+                        }
+                    }
+                }
+            }
+        }
+        return;
+    }
     __syncthreads();
     uint16_t* out = (uint16_t*)p.out + bz * p.M * p.ldc;
     // Results leave through LDS: a lane holds 4 consecutive columns of one row per register quad, which would make
@@ -562,6 +638,7 @@ static int qgemm_launch(const QgemmParams& p, int64_t batch, int out_dt, hipStre
 {
     const bool bf = out_dt == DT_BF16;
     if constexpr (MODE == MODE_I8) {
+        if (out_dt == DT_I32 || out_dt == DT_I8) return -2;   // qgemm_launch_int
         if ((p.KB % BK) != 0) {
             return bf ? qgemm_launch_one<MODE, BM, BN, BK, WGM, WGN, STAGES, MINWG, true, DT_BF16>(p, batch, st)
                       : qgemm_launch_one<MODE, BM, BN, BK, WGM, WGN, STAGES, MINWG, true, DT_F16>(p, batch, st);
@@ -569,6 +646,20 @@ static int qgemm_launch(const QgemmParams& p, int64_t batch, int out_dt, hipStre
     }
     return bf ? qgemm_launch_one<MODE, BM, BN, BK, WGM, WGN, STAGES, MINWG, false, DT_BF16>(p, batch, st)
               : qgemm_launch_one<MODE, BM, BN, BK, WGM, WGN, STAGES, MINWG, false, DT_F16>(p, batch, st);
+}
+
+// MODE_I8 with an INT32 or INT8 output (instantiated only for the tile shapes the int8 launcher uses for them).
+template <int BM, int BN, int BK, int WGM, int WGN, int STAGES, int MINWG>
+static int qgemm_launch_int(const QgemmParams& p, int64_t batch, int out_dt, hipStream_t st)
+{
+    const bool tail = (p.KB % BK) != 0;
+    if (out_dt == DT_I32)
+        return tail ? qgemm_launch_one<MODE_I8, BM, BN, BK, WGM, WGN, STAGES, MINWG, true, DT_I32>(p, batch, st)
+                    : qgemm_launch_one<MODE_I8, BM, BN, BK, WGM, WGN, STAGES, MINWG, false, DT_I32>(p, batch, st);
+    if (out_dt == DT_I8)
+        return tail ? qgemm_launch_one<MODE_I8, BM, BN, BK, WGM, WGN, STAGES, MINWG, true, DT_I8>(p, batch, st)
+                    : qgemm_launch_one<MODE_I8, BM, BN, BK, WGM, WGN, STAGES, MINWG, false, DT_I8>(p, batch, st);
+    return -2;
 }
 
 }  // namespace opsnn

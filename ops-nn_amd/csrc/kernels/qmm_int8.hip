@@ -88,7 +88,14 @@ static int64_t cu_count()
     return n;
 }
 
+// OPSNN_NOT_TAKEN: an INT8 output was asked for and the shape does not fit the MFMA kernels (the caller falls back).
+extern "C" __attribute__((visibility("hidden"))) int opsnn_qmm_int8_impl(const OpsnnQmmArgs* a, void* stream);
 extern "C" int opsnnQmmInt8(const OpsnnQmmArgs* a, void* stream)
+{
+    const int rc = opsnn_qmm_int8_impl(a, stream);
+    return rc == OPSNN_NOT_TAKEN ? -2 : rc;
+}
+extern "C" int opsnn_qmm_int8_impl(const OpsnnQmmArgs* a, void* stream)
 {
     if (!a || !a->x1.ptr || !a->x2.ptr || !a->out || !a->x2_scale) return -1;
     if (a->x1_dtype != DT_I8 || a->x2_dtype != DT_I8) return -2;
@@ -104,7 +111,10 @@ extern "C" int opsnnQmmInt8(const OpsnnQmmArgs* a, void* stream)
     // x2 stored N-major ([K, N] rows): relayout into the workspace as [N, K] first.
     bool b_kmajor = (p.b_rs == 1);
     bool a_kmajor = (p.a_cs == 1);
-    bool b16 = (p.out_dt == DT_BF16 || p.out_dt == DT_F16);
+    // INT32 / INT8 outputs (the static-quantisation modes: no per-token scale; bias absent or INT32) run on the 8-wave tile
+    // kernels with an integer epilogue
+    const bool int_out = (p.out_dt == DT_I32 || p.out_dt == DT_I8) && !a->x1_scale && (!a->bias || a->bias_dtype == DT_I32);
+    bool b16 = (p.out_dt == DT_BF16 || p.out_dt == DT_F16) || int_out;
     int variant = a->force_variant;
     if (opsnn_force_plain()) variant = OPSNN_VARIANT_PLAIN;
     if (variant == 0) {  // tuning aid: OPSNN_I8_VARIANT pins a kernel variant for calls that do not ask for one
@@ -127,6 +137,11 @@ extern "C" int opsnnQmmInt8(const OpsnnQmmArgs* a, void* stream)
         g.out = p.out; g.M = p.M; g.N = p.N; g.ldc = p.N; g.KB = p.K;
         g.x1s = p.x1s; g.x2s = p.x2s; g.x2s_dt = p.x2s_dt; g.x2s_len = p.x2s_len; g.x2s_trunc = a->x2_scale_trunc;
         g.bias = p.bias; g.bias_dt = p.bias_dt; g.bias_bs = p.bias_bs;
+        if (int_out) {
+            g.x2off = a->x2_offset; g.x2off_len = a->x2_offset_len;
+            if (p.M <= 128 || p.N <= 128 || p.M * p.N < 256 * 256 * 64) return qgemm_launch_int<128, 128, 128, 2, 2, 2, 1>(g, a->batch, p.out_dt, st);
+            return qgemm_launch_int<256, 256, 128, 2, 4, 2, 1>(g, a->batch, p.out_dt, st);
+        }
         if (variant >= OPSNN_VARIANT_I8_WIDE8 && variant <= OPSNN_VARIANT_I8_WIDE11) {
             const int rc = launch_int8_wide(g, variant, a->batch, p.out_dt, st);
             if (rc != OPSNN_NOT_TAKEN) return rc;
@@ -190,6 +205,7 @@ extern "C" int opsnnQmmInt8(const OpsnnQmmArgs* a, void* stream)
         }
         return qgemm_launch<MODE_I8, 256, 128, 64, 2, 2, 3, 2>(g, a->batch, p.out_dt, st);
     }
+    if (p.out_dt == DT_I8) return OPSNN_NOT_TAKEN;   // the strided kernel below has no requantising epilogue
     dim3 block(256), grid((unsigned)(((p.N + 255) / 256) * p.M), (unsigned)a->batch);
     hipLaunchKernelGGL(qmm_i8_plain, grid, block, 0, st, p);
     return (int)hipGetLastError();

@@ -186,6 +186,15 @@ GPU_CASES = [
     (128, 256, 192, "i8", "u64", 1, "i32", "bf16", False, False, 0),
     (96, 320, 160, "i8", "f32", 1, "f32", "bf16", True, False, 0),    # fp32 bias: scale not truncated
     (96, 320, 160, "i8", "bf16", "N", "bf16", "bf16", True, False, 0),
+    # INT8 (requantised) and INT32 outputs on the MFMA kernel's integer epilogue: 128 x 128 and 256 x 256 tiles, K tails,
+    # ragged and odd N, N-contiguous x2 (re-laid out into the workspace), offsets from the tensor and from the packed word
+    (128, 256, 192, "i8", "u64", "N", "i32", "i8", True, False, "N"),
+    (300, 384, 260, "i8", "u64", 1, "i32", "i8", True, False, 1),
+    (300, 400, 260, "i8", "f32", "N", "i32", "i32", True, False, 0),
+    (300, 400, 261, "i8", "u64", "N", None, "i8", True, False, 0),
+    (640, 1024, 520, "i8", "f32", "N", None, "i32", False, False, 0),
+    (2048, 512, 2304, "i8", "u64", "N", "i32", "i8", True, False, "N"),
+    (2048, 528, 2301, "i8", "f32", "N", "i32", "i32", True, False, 0),
     (16, 32, 16, "e4m3", "f32", "N", "f32", "f16", False, True, 0),   # FP8E4M3..dynamic_tc_bias_float
     (16, 32, 16, "e5m2", "f32", "N", "f32", "bf16", False, True, 0),  # FP8E5M2..dynamic_tc_bias_float
     (37, 160, 48, "e4m3", "f32", 1, None, "bf16", True, True, 0),     # both scales one element: merged and truncated
