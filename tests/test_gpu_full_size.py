@@ -93,3 +93,57 @@ def test_config5_mxfp4_batched_full(gpu):
     # one more on every x1 exponent doubles every output exactly
     inp2 = dict(inp, s1=(inp["s1"] + 1).astype(np.uint8))
     _double_exactly(got, cases.run_mx_aclnn(m, inp2, M, K, N, True, m.ACL_BF16), m.ACL_BF16)
+
+
+# ---- the operators that prepare the configs' tensors, at the configs' sizes (bit-identical to the oracle) ----
+def test_prepack_of_config3_weight_full(gpu):
+    """8192 x 28672 int32 carriers -> packed int4: every byte against the oracle, and unpacking returns the carriers' nibbles."""
+    m = gpu
+    K, N = 8192, 28672
+    print("case pre-pack full size", flush=True)
+    w = np.random.default_rng(0).integers(-8, 8, size=(K, N)).astype(np.int32)
+    d_w, d_p = m.DeviceBuffer(host=w), m.DeviceBuffer(K * N // 2)
+    assert m.convert_weight_to_int4_pack(m.Tensor((K, N), m.ACL_INT32, d_w), m.Tensor((K, N // 8), m.ACL_INT32, d_p)) == 0, m.err_msg()
+    got = d_p.to_host(np.uint8, (K, N // 2))
+    assert np.array_equal(got, orc.convert_weight_b4(w))
+    assert np.array_equal(orc.unpack_nibbles(got[:64]), (w[:64] & 15).astype(np.uint8))
+
+
+def test_dynamic_quant_of_config2_activation_full(gpu):
+    from test_dynamic_quant import _run
+    m = gpu
+    print("case dynamic quant full size", flush=True)
+    xb = orc.f32_to_bf16(np.random.default_rng(1).normal(0, 1, size=(2048, 4096)).astype(np.float32))
+    want_y, want_s = orc.dynamic_quant(xb, orc.BF16, orc.I8)
+    gy, gs, _ = _run(m, xb, orc.BF16, orc.I8, None, True)
+    assert np.array_equal(gs, want_s) and np.array_equal(gy, want_y.reshape(-1))
+    assert (np.abs(gy.view(np.int8).reshape(2048, 4096)).max(axis=1) == 127).all()   # every row's largest magnitude maps to 127
+
+
+def test_block_quant_of_config4_operands_full(gpu):
+    from test_dynamic_block_quant import _run
+    m = gpu
+    print("case block quant full size", flush=True)
+    rng = np.random.default_rng(2)
+    for shape, rb in (((4096, 7168), 1), ((18432, 7168), 128)):
+        xb = orc.f32_to_bf16(rng.normal(0, 1, size=shape).astype(np.float32))
+        want_y, want_s = orc.dynamic_block_quant(xb, orc.BF16, orc.E4M3, rb, 128)
+        gy, gs = _run(m, xb, orc.BF16, orc.E4M3, rb, 128)
+        assert np.array_equal(gs.view(np.uint32), want_s.view(np.uint32))
+        z = ((gy | want_y) & 0x7f) == 0
+        assert np.array_equal(gy[~z], want_y[~z])
+        assert ((gy & 0x7f).reshape(shape[0] // rb, rb, shape[1] // 128, 128).max(axis=(1, 3)) == 0x7e).all()   # every block reaches 448
+
+
+def test_mx_quant_of_config5_activation_full(gpu):
+    from test_dynamic_mx_quant import _run
+    m = gpu
+    print("case mx quant full size", flush=True)
+    xb = orc.f32_to_bf16(np.random.default_rng(3).normal(0, 1, size=(4096, 8192)).astype(np.float32))   # one of the 8 batches
+    want_y, want_s = orc.dynamic_mx_quant(xb, orc.BF16, orc.E2M1)
+    gy, gs = _run(m, xb, orc.BF16, orc.E2M1)
+    assert np.array_equal(gs, want_s)
+    a, b = orc.unpack_nibbles(gy), orc.unpack_nibbles(want_y.reshape(-1))
+    z = ((a | b) & 7) == 0
+    assert np.array_equal(a[~z], b[~z])
+    assert ((a & 7).reshape(-1, 32).max(axis=1) >= 6).all()   # every block's maximum lands in the top binade (codes 4.0 or 6.0)
