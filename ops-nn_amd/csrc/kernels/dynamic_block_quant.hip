@@ -37,7 +37,8 @@ __device__ __forceinline__ BlockScale block_scale(const BlockQuantParams& p, flo
     BlockScale b;
     b.scale = fminf(__fdiv_rn(amax, p.tmax), p.cap);
     b.rcp = __fdiv_rn(1.0f, b.scale);
-    b.fast = (f2u(b.scale) & 0x7fffffu) != 0x7fffffu && b.scale > 0x1p-60f && b.scale < 0x1p60f;
+    // the quotients stay far from overflow (a capped scale under a huge bf16 maximum would not)
+    b.fast = (f2u(b.scale) & 0x7fffffu) != 0x7fffffu && b.scale > 0x1p-60f && b.scale < 0x1p60f && __fmul_rn(amax, b.rcp) < 0x1p100f;
     return b;
 }
 
@@ -53,12 +54,13 @@ __device__ __forceinline__ float block_quant_value(float v, const BlockScale& b,
     // with the scale in [2^-60, 2^60] and |v| above 2^-100 every intermediate is a normal number; a zero stays a zero
     if (!(b.fast && (fabsf(v) > 0x1p-100f || v == 0.0f))) q = __fdiv_rn(v, b.scale);
     if (!finite) q = v;
-    q = q > tmax ? tmax : q;       // comparisons are false for NaN: it passes through, as in numpy's clip
-    q = q < -tmax ? -tmax : q;
+    // NaN (a NaN input, or 0 / 0 in a block of zeros) passes numpy's clip and rounding and becomes +0 at the end: done first
+    // here, which leaves the clip a single median instruction
+    q = (q == q) ? q : 0.0f;
+    q = __builtin_amdgcn_fmed3f(q, -tmax, tmax);
     const float t = __builtin_rintf(__fmul_rn(q, 1e8f));
     const float d0 = __fmul_rn(t, 1e-8f);   // 1e-8f is the correctly rounded reciprocal of 1e8f
-    q = __fmaf_rn(__fmaf_rn(-d0, 1e8f, t), 1e-8f, d0);
-    return (q == q) ? q : 0.0f;
+    return __fmaf_rn(__fmaf_rn(-d0, 1e8f, t), 1e-8f, d0);
 }
 template <int Y_DT>
 __device__ __forceinline__ uint32_t block_quant_one(float v, const BlockScale& b, float tmax)
@@ -75,34 +77,46 @@ __device__ __forceinline__ uint2 block_quant_eight(const float* v, const BlockSc
     return make_uint2(h[0] | (h[1] << 16), h[2] | (h[3] << 16));
 }
 
-// rb == 1: lane groups of G lanes, LPB = cb / 8 of them active, one (row, block) pair per group.
-template <int X_DT, int Y_DT, int G>
-__global__ __launch_bounds__(256) void block_quant_rows_kernel(BlockQuantParams p, int lpb)
+// rb == 1: lane groups of G lanes, LPB = cb / 8 of them active.  A group takes NB (row, block) pairs, the pairs
+// g, g + ngroups, g + 2 ngroups, ... so that neighbouring groups read neighbouring blocks; all NB loads are issued
+// before the first is used.
+template <int X_DT, int Y_DT, int G, int NB>
+__global__ __launch_bounds__(256) void block_quant_rows_kernel(BlockQuantParams p, int lpb, int64_t ngroups)
 {
     const int64_t group = ((int64_t)blockIdx.x * 256 + threadIdx.x) / G;
     const int lane = threadIdx.x % G;
     const int64_t total = p.batch * p.rows * p.ncb;
-    const bool live_group = group < total;
-    const int64_t row = live_group ? group / p.ncb : 0, bc = live_group ? group % p.ncb : 0;
-    const int64_t col = bc * p.cb + (int64_t)lane * 8;
-    const bool live = live_group && lane < lpb && col < p.cols;   // cols % 8 == 0: a piece is inside the row or outside
-    uint4 buf = make_uint4(0, 0, 0, 0);
-    if (live) buf = *(const uint4*)(p.x + row * p.cols + col);
-    const uint32_t w[4] = {buf.x, buf.y, buf.z, buf.w};
-    float v[8];
-    float amax = 0.0f;
+    uint4 buf[NB];
+    int64_t at[NB];      // element offset of the lane's piece, -1 when there is none
+    bool live_pair[NB];
 #pragma unroll
-    for (int e = 0; e < 8; e++) {
-        v[e] = bq_x_to_f32<X_DT>((w[e >> 1] >> (16 * (e & 1))) & 0xffffu);
-        const float a = fabsf(v[e]);
-        amax = fmaxf(amax, a < __builtin_inff() ? a : 0.0f);
+    for (int i = 0; i < NB; i++) {
+        const int64_t pair = (int64_t)i * ngroups + group;
+        live_pair[i] = group < ngroups && pair < total;
+        const int64_t row = live_pair[i] ? pair / p.ncb : 0, bc = live_pair[i] ? pair % p.ncb : 0;
+        const int64_t col = bc * p.cb + (int64_t)lane * 8;
+        // cols % 8 == 0: a piece is inside the row or outside
+        at[i] = (live_pair[i] && lane < lpb && col < p.cols) ? row * p.cols + col : -1;
+        buf[i] = make_uint4(0, 0, 0, 0);
+        if (at[i] >= 0) buf[i] = *(const uint4*)(p.x + at[i]);
     }
 #pragma unroll
-    for (int o = G / 2; o > 0; o >>= 1) amax = fmaxf(amax, __shfl_xor(amax, o));
-    const BlockScale b = block_scale(p, amax);
-    if (live_group && lane == 0) p.scale[group] = b.scale;
-    if (!live) return;
-    *(uint2*)(p.y + row * p.cols + col) = block_quant_eight<Y_DT>(v, b, p.tmax);
+    for (int i = 0; i < NB; i++) {
+        const uint32_t w[4] = {buf[i].x, buf[i].y, buf[i].z, buf[i].w};
+        float v[8];
+        float amax = 0.0f;
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+            v[e] = bq_x_to_f32<X_DT>((w[e >> 1] >> (16 * (e & 1))) & 0xffffu);
+            const float a = fabsf(v[e]);
+            amax = fmaxf(amax, a < __builtin_inff() ? a : 0.0f);
+        }
+#pragma unroll
+        for (int o = G / 2; o > 0; o >>= 1) amax = fmaxf(amax, __shfl_xor(amax, o));
+        const BlockScale b = block_scale(p, amax);
+        if (live_pair[i] && lane == 0) p.scale[(int64_t)i * ngroups + group] = b.scale;
+        if (at[i] >= 0) *(uint2*)(p.y + at[i]) = block_quant_eight<Y_DT>(v, b, p.tmax);
+    }
 }
 
 // Any block shape: one workgroup per block, two sweeps.  VEC: cols % 8 == 0 (then every block row is a whole number of
@@ -118,10 +132,14 @@ __global__ __launch_bounds__(256) void block_quant_tile_kernel(BlockQuantParams 
     const uint16_t* xb = p.x + (bt * p.rows + r0) * p.cols + c0;
     uint8_t* yb = p.y + (bt * p.rows + r0) * p.cols + c0;
     constexpr int W = VEC ? 8 : 1;
-    const int64_t ppr = nc / W, items = nr * ppr;   // pieces per block row
+    // pieces per block row (at most 256) and rows: a thread's piece index advances by 256 = da rows + db pieces per
+    // step, kept as (row, piece) so that the loops carry no division
+    const int ppr = (int)(nc / W), rows_here = (int)nr;
+    const int da = 256 / ppr, db = 256 % ppr;
+    const int r_first = (int)threadIdx.x / ppr, c_first = (int)threadIdx.x % ppr;
     float amax = 0.0f;
-    for (int64_t i = threadIdx.x; i < items; i += 256) {
-        const int64_t o = (i / ppr) * p.cols + (i % ppr) * W;
+    for (int r = r_first, c = c_first; r < rows_here;) {
+        const int64_t o = (int64_t)r * p.cols + c * W;
         if constexpr (VEC) {
             const uint4 b = *(const uint4*)(xb + o);
             const uint32_t w[4] = {b.x, b.y, b.z, b.w};
@@ -134,6 +152,8 @@ __global__ __launch_bounds__(256) void block_quant_tile_kernel(BlockQuantParams 
             const float a = fabsf(bq_x_to_f32<X_DT>(xb[o]));
             amax = fmaxf(amax, a < __builtin_inff() ? a : 0.0f);
         }
+        r += da; c += db;
+        if (c >= ppr) { c -= ppr; r++; }
     }
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) amax = fmaxf(amax, __shfl_xor(amax, o));
@@ -142,8 +162,8 @@ __global__ __launch_bounds__(256) void block_quant_tile_kernel(BlockQuantParams 
     amax = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
     const BlockScale b = block_scale(p, amax);
     if (threadIdx.x == 0) p.scale[blk] = b.scale;
-    for (int64_t i = threadIdx.x; i < items; i += 256) {
-        const int64_t o = (i / ppr) * p.cols + (i % ppr) * W;
+    for (int r = r_first, c = c_first; r < rows_here;) {
+        const int64_t o = (int64_t)r * p.cols + c * W;
         if constexpr (VEC) {
             const uint4 xv = *(const uint4*)(xb + o);
             const uint32_t w[4] = {xv.x, xv.y, xv.z, xv.w};
@@ -154,6 +174,8 @@ __global__ __launch_bounds__(256) void block_quant_tile_kernel(BlockQuantParams 
         } else {
             yb[o] = (uint8_t)block_quant_one<Y_DT>(bq_x_to_f32<X_DT>(xb[o]), b, p.tmax);
         }
+        r += da; c += db;
+        if (c >= ppr) { c -= ppr; r++; }
     }
 }
 
@@ -164,12 +186,22 @@ static int launch_block_quant(const BlockQuantParams& p, int variant, hipStream_
     if (variant != 2 && rows_ok) {
         const int lpb = (int)(p.cb / 8);
         const int g = lpb <= 8 ? 8 : lpb <= 16 ? 16 : 32;
-        const int64_t groups = p.batch * p.rows * p.ncb;
+        const int64_t pairs = p.batch * p.rows * p.ncb;
+        // four pairs per group once that still leaves every SIMD eight waves
+        const int nb = pairs * g / 64 >= (int64_t)4 * 8 * 1024 ? 4 : 1;
+        const int64_t groups = (pairs + nb - 1) / nb;
         const int64_t wgs = (groups * g + 255) / 256;
         if (wgs > 0x7fffffff) return -1;
-        if (g == 8) hipLaunchKernelGGL((block_quant_rows_kernel<X_DT, Y_DT, 8>), dim3((unsigned)wgs), dim3(256), 0, st, p, lpb);
-        else if (g == 16) hipLaunchKernelGGL((block_quant_rows_kernel<X_DT, Y_DT, 16>), dim3((unsigned)wgs), dim3(256), 0, st, p, lpb);
-        else hipLaunchKernelGGL((block_quant_rows_kernel<X_DT, Y_DT, 32>), dim3((unsigned)wgs), dim3(256), 0, st, p, lpb);
+        auto go = [&](auto kernel) { hipLaunchKernelGGL(kernel, dim3((unsigned)wgs), dim3(256), 0, st, p, lpb, groups); };
+        if (nb == 4) {
+            if (g == 8) go(block_quant_rows_kernel<X_DT, Y_DT, 8, 4>);
+            else if (g == 16) go(block_quant_rows_kernel<X_DT, Y_DT, 16, 4>);
+            else go(block_quant_rows_kernel<X_DT, Y_DT, 32, 4>);
+        } else {
+            if (g == 8) go(block_quant_rows_kernel<X_DT, Y_DT, 8, 1>);
+            else if (g == 16) go(block_quant_rows_kernel<X_DT, Y_DT, 16, 1>);
+            else go(block_quant_rows_kernel<X_DT, Y_DT, 32, 1>);
+        }
     } else {
         if (variant == 1) return -4;
         const int64_t blocks = p.batch * p.nrb * p.ncb;
