@@ -4,11 +4,14 @@
 // calls, empty tensors :366-371, the INT32 carrier of INT4 :384-389) for the per-token mode on the reference's newest
 // SoC generation.  Phase 1 never touches tensor data and never calls HIP.
 #include <algorithm>
+#include <cstring>
 #include <initializer_list>
 #include <memory>
 
 #include "aclnnop/aclnn_dynamic_quant.h"
 #include "aclnnop/aclnn_dynamic_quant_v2.h"
+#include "aclnnop/aclnn_dynamic_quant_v3.h"
+#include "aclnnop/aclnn_dynamic_quant_v4.h"
 #include "tensor.h"
 
 using namespace opsnn;
@@ -24,13 +27,20 @@ namespace {
 
 bool in_list(aclDataType d, std::initializer_list<aclDataType> l) { return std::find(l.begin(), l.end(), d) != l.end(); }
 
-aclnnStatus get_workspace(const char* api, const aclTensor* x_, const aclTensor* smooth_, const aclTensor* group_,
-                          const aclTensor* y_, const aclTensor* scale_, const aclTensor* offset_, uint64_t* workspaceSize,
-                          aclOpExecutor** executor)
+aclnnStatus get_workspace(const char* api, const aclTensor* x_, const aclTensor* smooth_, const aclTensor* group_, bool symmetrical,
+                          const char* quantMode, float dstTypeMax, const aclTensor* y_, const aclTensor* scale_, const aclTensor* offset_,
+                          uint64_t* workspaceSize, aclOpExecutor** executor)
 {
     clear_error();
     if (!x_ || !y_ || !scale_) FAIL(ACLNN_ERR_PARAM_NULLPTR, "%s: x, yOut and scaleOut must not be null", api);   // :136-142
     if (!workspaceSize || !executor) FAIL(ACLNN_ERR_PARAM_NULLPTR, "%s: workspaceSize/executor is null", api);
+    // attributes :171-189
+    if (symmetrical && offset_) INVALID("%s: offsetOut must be null when isSymmetrical is true", api);
+    if (!symmetrical && !offset_) INVALID("%s: offsetOut must not be null when isSymmetrical is false", api);
+    if (!quantMode) FAIL(ACLNN_ERR_PARAM_NULLPTR, "%s: quantMode is null", api);
+    const bool pertensor = !std::strcmp(quantMode, "pertensor"), perchannel = !std::strcmp(quantMode, "perchannel");
+    if (!pertensor && !perchannel && std::strcmp(quantMode, "pertoken") != 0) INVALID("%s: quantMode must be pertensor, pertoken or perchannel, got %s", api, quantMode);
+    if (perchannel && group_) INVALID("%s: groupIndex must be null when quantMode is perchannel", api);
     const TView x = make_view(x_), sm = make_view(smooth_), gi = make_view(group_), y = make_view(y_), sc = make_view(scale_),
                 off = make_view(offset_);
     // dtypes :293-317
@@ -52,7 +62,8 @@ aclnnStatus get_workspace(const char* api, const aclTensor* x_, const aclTensor*
             if (gi.rank() != 1) INVALID("%s: groupIndex must have one dim", api);
         } else {
             if (sm.rank() != 1) INVALID("%s: smoothScales must have one dim, got %ld", api, (long)sm.rank());
-            if (sm.dim(0) != cols) INVALID("%s: smoothScales has %ld elements, the last dim of x is %ld", api, (long)sm.dim(0), (long)cols);
+            const int64_t want_len = perchannel ? x.dim(-2) : cols;
+            if (sm.dim(0) != want_len) INVALID("%s: smoothScales has %ld elements, %ld expected", api, (long)sm.dim(0), (long)want_len);
         }
     }
     if (y.dtype != ACL_INT32) {
@@ -65,7 +76,13 @@ aclnnStatus get_workspace(const char* api, const aclTensor* x_, const aclTensor*
             if (x.dim(i) != y.dim(i)) INVALID("%s: dim %ld of x (%ld) and yOut (%ld) differ", api, (long)i, (long)x.dim(i), (long)y.dim(i));
     }
     if (y.dtype == ACL_INT4 && cols % 2 != 0) INVALID("%s: the last dim of x must be even for an INT4 yOut, got %ld", api, (long)cols);
-    if (sc.rank() != x.rank() - 1 || !std::equal(sc.shape.begin(), sc.shape.end(), x.shape.begin()))
+    if (pertensor) {
+        if (sc.rank() != 1 || sc.dim(0) != 1) INVALID("%s: scaleOut must be [1] when quantMode is pertensor", api);
+    } else if (perchannel) {
+        std::vector<int64_t> want(x.shape.begin(), x.shape.end() - 2);
+        want.push_back(cols);
+        if (sc.shape != want) INVALID("%s: scaleOut %s must be %s when quantMode is perchannel", api, shape_str(sc.shape).c_str(), shape_str(want).c_str());
+    } else if (sc.rank() != x.rank() - 1 || !std::equal(sc.shape.begin(), sc.shape.end(), x.shape.begin()))
         INVALID("%s: scaleOut %s must have x's shape %s without the last dim", api, shape_str(sc.shape).c_str(), shape_str(x.shape).c_str());
     if (off.present && off.shape != sc.shape) INVALID("%s: offsetOut %s and scaleOut %s differ in shape", api, shape_str(off.shape).c_str(), shape_str(sc.shape).c_str());
 
@@ -79,6 +96,8 @@ aclnnStatus get_workspace(const char* api, const aclTensor* x_, const aclTensor*
         return ACLNN_SUCCESS;
     }
     // what this build does not run
+    if (pertensor || perchannel) FAIL(ACLNN_ERR_INNER_TILING_ERROR, "%s: quantMode %s has no kernel here (pertoken has)", api, quantMode);
+    if (dstTypeMax != 0.0f) FAIL(ACLNN_ERR_INNER_TILING_ERROR, "%s: a dstTypeMax other than 0 has no kernel here", api);
     if (gi.present) FAIL(ACLNN_ERR_INNER_TILING_ERROR, "%s: groupIndex (per-expert smooth scales) has no kernel here", api);
     if (y.dtype == ACL_HIFLOAT8) FAIL(ACLNN_ERR_INNER_TILING_ERROR, "%s: HIFLOAT8 output has no kernel on this device", api);
     if (!is_contiguous(x) || !is_contiguous(y) || !is_contiguous(sc) || (sm.present && !is_contiguous(sm)) || (off.present && !is_contiguous(off)))
@@ -119,8 +138,8 @@ extern "C" {
 aclnnStatus aclnnDynamicQuantGetWorkspaceSize(const aclTensor* x, const aclTensor* smoothScalesOptional, const aclTensor* yOut,
                                               const aclTensor* scaleOut, uint64_t* workspaceSize, aclOpExecutor** executor)
 {
-    return get_workspace("aclnnDynamicQuantGetWorkspaceSize", x, smoothScalesOptional, nullptr, yOut, scaleOut, nullptr, workspaceSize,
-                         executor);
+    return get_workspace("aclnnDynamicQuantGetWorkspaceSize", x, smoothScalesOptional, nullptr, true, "pertoken", 0.0f, yOut, scaleOut, nullptr,
+                         workspaceSize, executor);
 }
 
 aclnnStatus aclnnDynamicQuant(void*, uint64_t, aclOpExecutor* executor, aclrtStream stream) { return run("aclnnDynamicQuant", executor, stream); }
@@ -131,10 +150,34 @@ aclnnStatus aclnnDynamicQuantV2GetWorkspaceSize(const aclTensor* x, const aclTen
                                                 aclOpExecutor** executor)
 {
     (void)dstType;   // the reference takes the output type from yOut (:384-389); dstType only reaches its log
-    return get_workspace("aclnnDynamicQuantV2GetWorkspaceSize", x, smoothScalesOptional, groupIndexOptional, yOut, scaleOut, offsetOut,
-                         workspaceSize, executor);
+    return get_workspace("aclnnDynamicQuantV2GetWorkspaceSize", x, smoothScalesOptional, groupIndexOptional, offsetOut == nullptr, "pertoken", 0.0f,
+                         yOut, scaleOut, offsetOut, workspaceSize, executor);
 }
 
 aclnnStatus aclnnDynamicQuantV2(void*, uint64_t, aclOpExecutor* executor, aclrtStream stream) { return run("aclnnDynamicQuantV2", executor, stream); }
+
+aclnnStatus aclnnDynamicQuantV3GetWorkspaceSize(const aclTensor* x, const aclTensor* smoothScalesOptional, const aclTensor* groupIndexOptional,
+                                                int64_t dstType, bool isSymmetrical, const char* quantMode, const aclTensor* yOut,
+                                                const aclTensor* scaleOut, const aclTensor* offsetOut, uint64_t* workspaceSize,
+                                                aclOpExecutor** executor)
+{
+    (void)dstType;
+    return get_workspace("aclnnDynamicQuantV3GetWorkspaceSize", x, smoothScalesOptional, groupIndexOptional, isSymmetrical, quantMode, 0.0f, yOut,
+                         scaleOut, offsetOut, workspaceSize, executor);
+}
+
+aclnnStatus aclnnDynamicQuantV3(void*, uint64_t, aclOpExecutor* executor, aclrtStream stream) { return run("aclnnDynamicQuantV3", executor, stream); }
+
+aclnnStatus aclnnDynamicQuantV4GetWorkspaceSize(const aclTensor* x, const aclTensor* smoothScalesOptional, const aclTensor* groupIndexOptional,
+                                                int64_t dstType, bool isSymmetrical, const char* quantMode, float dstTypeMax,
+                                                const aclTensor* yOut, const aclTensor* scaleOut, const aclTensor* offsetOut,
+                                                uint64_t* workspaceSize, aclOpExecutor** executor)
+{
+    (void)dstType;
+    return get_workspace("aclnnDynamicQuantV4GetWorkspaceSize", x, smoothScalesOptional, groupIndexOptional, isSymmetrical, quantMode, dstTypeMax,
+                         yOut, scaleOut, offsetOut, workspaceSize, executor);
+}
+
+aclnnStatus aclnnDynamicQuantV4(void*, uint64_t, aclOpExecutor* executor, aclrtStream stream) { return run("aclnnDynamicQuantV4", executor, stream); }
 
 }  // extern "C"

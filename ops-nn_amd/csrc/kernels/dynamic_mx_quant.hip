@@ -84,47 +84,62 @@ __device__ __forceinline__ uint2 mx_pack8(const float* q)
     }
 }
 
-// cols % 8 == 0: lane groups of four, one (row, block) pair per group
-template <int X_DT, int Y_DT>
-__global__ __launch_bounds__(256) void mx_quant_kernel(MxQuantParams p)
+// cols % 8 == 0: lane groups of four.  A group takes NB (row, block) pairs, the pairs g, g + ngroups, g + 2 ngroups, ...
+// so that neighbouring groups read neighbouring blocks; all NB loads are issued before the first is used.
+template <int X_DT, int Y_DT, int NB>
+__global__ __launch_bounds__(256) void mx_quant_kernel(MxQuantParams p, int64_t ngroups)
 {
     const int64_t group = ((int64_t)blockIdx.x * 256 + threadIdx.x) / 4;
     const int lane = threadIdx.x & 3;
-    const bool live_group = group < p.rows * p.nblk;
-    const int64_t row = live_group ? group / p.nblk : 0, blk = live_group ? group % p.nblk : 0;
-    const int64_t col = blk * 32 + lane * 8;
-    const bool live = live_group && col < p.cols;
-    uint4 buf = make_uint4(0, 0, 0, 0);   // the zero padding of a short last block
-    if (live) buf = *(const uint4*)(p.x + row * p.cols + col);
-    const uint32_t w[4] = {buf.x, buf.y, buf.z, buf.w};
-    float v[8];
-    float amax = 0.0f;
-    bool bad = false;
+    const int64_t total = p.rows * p.nblk;
+    uint4 buf[NB];
+    int64_t at[NB];        // element offset of the lane's piece, -1 when it lies in the zero padding of a short last block
+    int64_t sidx[NB];      // index of the pair's scale byte, -1 for a pair that does not exist
+    bool pad_after[NB];    // the pair is the last block of a row with an odd number of blocks
 #pragma unroll
-    for (int e = 0; e < 8; e++) {
-        v[e] = mx_x_to_f32<X_DT>((w[e >> 1] >> (16 * (e & 1))) & 0xffffu);
-        const float a = fabsf(v[e]);
-        bad |= !(a < __builtin_inff());   // infinity or NaN
-        amax = fmaxf(amax, a);
+    for (int i = 0; i < NB; i++) {
+        const int64_t pair = (int64_t)i * ngroups + group;
+        const bool live_pair = group < ngroups && pair < total;
+        const int64_t row = live_pair ? pair / p.nblk : 0, blk = live_pair ? pair % p.nblk : 0;
+        const int64_t col = blk * 32 + lane * 8;
+        at[i] = (live_pair && col < p.cols) ? row * p.cols + col : -1;
+        sidx[i] = live_pair ? row * p.spitch + blk : -1;
+        pad_after[i] = blk == p.nblk - 1 && (p.nblk & 1);
+        buf[i] = make_uint4(0, 0, 0, 0);
+        if (at[i] >= 0) buf[i] = *(const uint4*)(p.x + at[i]);
     }
-    amax = fmaxf(amax, __shfl_xor(amax, 1));
-    amax = fmaxf(amax, __shfl_xor(amax, 2));
-    bad |= (bool)__shfl_xor((int)bad, 1);
-    bad |= (bool)__shfl_xor((int)bad, 2);
-    const int share = bad ? 0 : mx_share_exp<Y_DT>(amax);
-    if (live_group && lane == 0) {
-        p.scale[row * p.spitch + blk] = bad ? 0xFFu : (uint8_t)(share + 127);
-        if (blk == p.nblk - 1 && (p.nblk & 1)) p.scale[row * p.spitch + blk + 1] = 0;
-    }
-    if (!live) return;
-    // 2^-share: share is in [-127, 125]; 2^127 and 2^-125 are both normal numbers
-    const float inv_scale = u2f((uint32_t)(127 - share) << 23);
-    float q[8];
 #pragma unroll
-    for (int e = 0; e < 8; e++) q[e] = mx_scaled<Y_DT>(v[e], inv_scale, bad);
-    const uint2 out = mx_pack8<Y_DT>(q);
-    if constexpr (Y_DT == DT_E2M1) *(uint32_t*)(p.y + (row * p.cols + col) / 2) = out.x;
-    else *(uint2*)(p.y + row * p.cols + col) = out;
+    for (int i = 0; i < NB; i++) {
+        const uint32_t w[4] = {buf[i].x, buf[i].y, buf[i].z, buf[i].w};
+        float v[8];
+        float amax = 0.0f;
+        bool bad = false;
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+            v[e] = mx_x_to_f32<X_DT>((w[e >> 1] >> (16 * (e & 1))) & 0xffffu);
+            const float a = fabsf(v[e]);
+            bad |= !(a < __builtin_inff());   // infinity or NaN
+            amax = fmaxf(amax, a);
+        }
+        amax = fmaxf(amax, __shfl_xor(amax, 1));
+        amax = fmaxf(amax, __shfl_xor(amax, 2));
+        bad |= (bool)__shfl_xor((int)bad, 1);
+        bad |= (bool)__shfl_xor((int)bad, 2);
+        const int share = bad ? 0 : mx_share_exp<Y_DT>(amax);
+        if (sidx[i] >= 0 && lane == 0) {
+            p.scale[sidx[i]] = bad ? 0xFFu : (uint8_t)(share + 127);
+            if (pad_after[i]) p.scale[sidx[i] + 1] = 0;
+        }
+        if (at[i] < 0) continue;
+        // 2^-share: share is in [-127, 125]; 2^127 and 2^-125 are both normal numbers
+        const float inv_scale = u2f((uint32_t)(127 - share) << 23);
+        float q[8];
+#pragma unroll
+        for (int e = 0; e < 8; e++) q[e] = mx_scaled<Y_DT>(v[e], inv_scale, bad);
+        const uint2 out = mx_pack8<Y_DT>(q);
+        if constexpr (Y_DT == DT_E2M1) *(uint32_t*)(p.y + at[i] / 2) = out.x;
+        else *(uint2*)(p.y + at[i]) = out;
+    }
 }
 
 // any row length: one thread per block of 32
@@ -167,9 +182,13 @@ static int launch_mx_quant(const MxQuantParams& p, int variant, hipStream_t st)
     const bool vec = p.cols % 8 == 0 && (uintptr_t)p.x % 16 == 0 && (uintptr_t)p.y % 8 == 0;
     const int64_t groups = p.rows * p.nblk;
     if (variant != 2 && vec) {
-        const int64_t wgs = (groups * 4 + 255) / 256;
+        // four pairs per group once that still leaves every SIMD eight waves
+        const int nb = groups * 4 / 64 >= (int64_t)4 * 8 * 1024 ? 4 : 1;
+        const int64_t ngroups = (groups + nb - 1) / nb;
+        const int64_t wgs = (ngroups * 4 + 255) / 256;
         if (wgs > 0x7fffffff) return -1;
-        hipLaunchKernelGGL((mx_quant_kernel<X_DT, Y_DT>), dim3((unsigned)wgs), dim3(256), 0, st, p);
+        if (nb == 4) hipLaunchKernelGGL((mx_quant_kernel<X_DT, Y_DT, 4>), dim3((unsigned)wgs), dim3(256), 0, st, p, ngroups);
+        else hipLaunchKernelGGL((mx_quant_kernel<X_DT, Y_DT, 1>), dim3((unsigned)wgs), dim3(256), 0, st, p, ngroups);
     } else {
         if (variant == 1) return -4;
         const int64_t wgs = (groups + 255) / 256;

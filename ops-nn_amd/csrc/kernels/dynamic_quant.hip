@@ -67,7 +67,7 @@ __device__ __forceinline__ uint32_t quant_one(float v, const RowQuant& r)
     } else {
         constexpr float lo = Y_DT == DT_I8 ? -128.0f : -8.0f, hi = Y_DT == DT_I8 ? 127.0f : 7.0f;
         float t = __builtin_rintf(q);
-        t = (t == t) ? fminf(fmaxf(t, lo), hi) : 0.0f;
+        t = __builtin_amdgcn_fmed3f((t == t) ? t : 0.0f, lo, hi);
         return (uint32_t)(int)t & (Y_DT == DT_I8 ? 0xffu : 0xfu);
     }
 }

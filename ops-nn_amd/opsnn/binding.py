@@ -139,6 +139,10 @@ _SIGS = {
     "aclnnDynamicQuant": (C.c_int32, [C.c_void_p, C.c_uint64, C.c_void_p, C.c_void_p]),
     "aclnnDynamicQuantV2GetWorkspaceSize": (C.c_int32, [_T] * 3 + [C.c_int64] + [_T] * 3 + [C.POINTER(C.c_uint64), C.POINTER(C.c_void_p)]),
     "aclnnDynamicQuantV2": (C.c_int32, [C.c_void_p, C.c_uint64, C.c_void_p, C.c_void_p]),
+    "aclnnDynamicQuantV3GetWorkspaceSize": (C.c_int32, [_T] * 3 + [C.c_int64, C.c_bool, C.c_char_p] + [_T] * 3 + [C.POINTER(C.c_uint64), C.POINTER(C.c_void_p)]),
+    "aclnnDynamicQuantV3": (C.c_int32, [C.c_void_p, C.c_uint64, C.c_void_p, C.c_void_p]),
+    "aclnnDynamicQuantV4GetWorkspaceSize": (C.c_int32, [_T] * 3 + [C.c_int64, C.c_bool, C.c_char_p, C.c_float] + [_T] * 3 + [C.POINTER(C.c_uint64), C.POINTER(C.c_void_p)]),
+    "aclnnDynamicQuantV4": (C.c_int32, [C.c_void_p, C.c_uint64, C.c_void_p, C.c_void_p]),
     "opsnnDynamicQuant": (C.c_int, [C.POINTER(OpsnnDynQuantArgs), C.c_void_p]),
     "aclnnDynamicBlockQuantGetWorkspaceSize": (C.c_int32, [_T, C.c_double, C.c_char_p, C.c_int64, C.c_int64, C.c_int64, _T, _T,
                                                           C.POINTER(C.c_uint64), C.POINTER(C.c_void_p)]),
@@ -349,10 +353,20 @@ def weight_quant_batch_matmul(x, weight, scale, y, stream=None, **kw):
     return wbuf
 
 
-def dynamic_quant_get_workspace(x, y, scale, *, smooth=None, offset=None, group_index=None, v2=False, dst_type=2):
-    """Phase 1 of aclnnDynamicQuant (or V2 when v2 / offset / group_index is given).  Returns (status, workspace, executor)."""
+def dynamic_quant_get_workspace(x, y, scale, *, smooth=None, offset=None, group_index=None, v2=False, dst_type=2, quant_mode=None,
+                                is_symmetrical=None, dst_type_max=None):
+    """Phase 1 of aclnnDynamicQuant; V2 when v2 / offset / group_index is given; V3 when quant_mode is given; V4 when dst_type_max
+    is given too.  Returns (status, workspace, executor)."""
     ws, ex = C.c_uint64(0), C.c_void_p()
-    if v2 or offset is not None or group_index is not None:
+    if quant_mode is not None:
+        sym = (offset is None) if is_symmetrical is None else is_symmetrical
+        if dst_type_max is None:
+            rc = lib().aclnnDynamicQuantV3GetWorkspaceSize(_h(x), _h(smooth), _h(group_index), dst_type, sym, quant_mode, _h(y), _h(scale),
+                                                           _h(offset), C.byref(ws), C.byref(ex))
+        else:
+            rc = lib().aclnnDynamicQuantV4GetWorkspaceSize(_h(x), _h(smooth), _h(group_index), dst_type, sym, quant_mode, dst_type_max, _h(y),
+                                                           _h(scale), _h(offset), C.byref(ws), C.byref(ex))
+    elif v2 or offset is not None or group_index is not None:
         rc = lib().aclnnDynamicQuantV2GetWorkspaceSize(_h(x), _h(smooth), _h(group_index), dst_type, _h(y), _h(scale), _h(offset),
                                                        C.byref(ws), C.byref(ex))
     else:
@@ -366,6 +380,8 @@ def dynamic_quant(x, y, scale, stream=None, **kw):
     rc, ws, ex = dynamic_quant_get_workspace(x, y, scale, **kw)
     check(rc, "aclnnDynamicQuantGetWorkspaceSize")
     run = lib().aclnnDynamicQuantV2 if v2 else lib().aclnnDynamicQuant
+    if kw.get("quant_mode") is not None:
+        run = lib().aclnnDynamicQuantV4 if kw.get("dst_type_max") is not None else lib().aclnnDynamicQuantV3
     check(run(None, ws, ex, stream.ptr if stream else None), "aclnnDynamicQuant")
 
 

@@ -168,6 +168,31 @@ def test_status_rules_one_by_one(opsnn):
     assert _status(m, x, y, sc, smooth=_t(m, (2, 32), m.ACL_BF16), group_index=_t(m, (2,), m.ACL_INT32)) == 561002
 
 
+def test_v3_v4_attribute_rules(opsnn):
+    """aclnn_dynamic_quant.cpp:171-189 and the mode-dependent scale shapes :258-284; the modes other than pertoken pass the
+    checks and are then answered with 561002 here (quant/dynamic_quant/tests/ut/op_host/op_api/test_aclnn_dynamic_quant_v3.cpp:71-90
+    is the per-tensor shape of scale and offset)."""
+    m = opsnn
+    bad, not_run = m.ACLNN_ERR_PARAM_INVALID, 561002
+    x, y, sc, off = _t(m, (16, 32), m.ACL_BF16), _t(m, (16, 32), m.ACL_INT8), _t(m, (16,), m.ACL_FLOAT), _t(m, (16,), m.ACL_FLOAT)
+    assert _status(m, x, y, sc, quant_mode=b"pertoken") == 0
+    assert _status(m, x, y, sc, offset=off, quant_mode=b"pertoken") == 0
+    assert _status(m, x, y, sc, quant_mode=b"pertoken", dst_type_max=0.0) == 0
+    assert _status(m, x, y, sc, offset=off, quant_mode=b"pertoken", is_symmetrical=True) == bad
+    assert _status(m, x, y, sc, quant_mode=b"pertoken", is_symmetrical=False) == bad
+    assert _status(m, x, y, sc, quant_mode=b"perrow") == bad
+    one = _t(m, (1,), m.ACL_FLOAT)
+    assert _status(m, x, y, one, offset=_t(m, (1,), m.ACL_FLOAT), quant_mode=b"pertensor") == not_run
+    assert _status(m, x, y, sc, quant_mode=b"pertensor") == bad                                            # scale must be [1]
+    assert _status(m, x, y, _t(m, (32,), m.ACL_FLOAT), quant_mode=b"perchannel") == not_run
+    assert _status(m, x, y, sc, quant_mode=b"perchannel") == bad                                           # scale must be [32]
+    assert _status(m, x, y, _t(m, (32,), m.ACL_FLOAT), quant_mode=b"perchannel", smooth=_t(m, (16,), m.ACL_BF16)) == not_run
+    assert _status(m, x, y, _t(m, (32,), m.ACL_FLOAT), quant_mode=b"perchannel", smooth=_t(m, (32,), m.ACL_BF16)) == bad
+    assert _status(m, x, y, _t(m, (32,), m.ACL_FLOAT), quant_mode=b"perchannel", smooth=_t(m, (2, 32), m.ACL_BF16),
+                   group_index=_t(m, (2,), m.ACL_INT32)) == bad
+    assert _status(m, x, y, sc, quant_mode=b"pertoken", dst_type_max=100.0) == not_run
+
+
 # --------------------------------------------------------------------------------------------------- device parity
 ACL_OF = {orc.I8: "ACL_INT8", orc.I4: "ACL_INT4", orc.E4M3: "ACL_FLOAT8_E4M3FN", orc.E5M2: "ACL_FLOAT8_E5M2"}
 
@@ -257,3 +282,17 @@ def test_gpu_quantised_activation_feeds_the_int8_matmul(gpu):
     inp_dev = dict(inp, x1=d_q.to_host(np.int8, (1, M, K)), s1=d_s.to_host(np.float32, (M,)))
     got = cases.run_qmm_int8_aclnn(m, inp_dev, M, K, N, True, m.ACL_BF16)
     assert np.array_equal(got, want)
+
+
+@pytest.mark.gpu
+def test_gpu_v3_and_v4_pertoken_equal_v1(gpu):
+    m = gpu
+    rng = np.random.default_rng(6)
+    xb = orc.f32_to_b16(rng.normal(0, 1, size=(40, 512)).astype(np.float32), orc.F16)
+    want_y, want_s = orc.dynamic_quant(xb, orc.F16, orc.I8)
+    d_x = m.DeviceBuffer(host=xb)
+    for kw in (dict(quant_mode=b"pertoken"), dict(quant_mode=b"pertoken", dst_type_max=0.0)):
+        d_y, d_s = m.DeviceBuffer(xb.size), m.DeviceBuffer(40 * 4)
+        m.dynamic_quant(m.Tensor((40, 512), m.ACL_FLOAT16, d_x), m.Tensor((40, 512), m.ACL_INT8, d_y), m.Tensor((40,), m.ACL_FLOAT, d_s), **kw)
+        m.check(m.lib().aclrtSynchronizeDevice(), "sync")
+        assert np.array_equal(d_y.to_host(np.uint8, (40, 512)), want_y) and np.array_equal(d_s.to_host(np.float32, (40,)), want_s)

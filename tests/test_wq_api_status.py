@@ -104,6 +104,7 @@ def test_library_exports_every_declared_symbol(opsnn):
             "aclnnWeightQuantBatchMatmulV2", "aclnnWeightQuantBatchMatmulV3GetWorkspaceSize", "aclnnWeightQuantBatchMatmulV3",
             "aclnnConvertWeightToINT4PackGetWorkspaceSize", "aclnnConvertWeightToINT4Pack", "opsnnPackB4",
             "aclnnDynamicQuantGetWorkspaceSize", "aclnnDynamicQuant", "aclnnDynamicQuantV2GetWorkspaceSize", "aclnnDynamicQuantV2",
+            "aclnnDynamicQuantV3GetWorkspaceSize", "aclnnDynamicQuantV3", "aclnnDynamicQuantV4GetWorkspaceSize", "aclnnDynamicQuantV4",
             "opsnnDynamicQuant", "aclnnDynamicBlockQuantGetWorkspaceSize", "aclnnDynamicBlockQuant", "opsnnDynamicBlockQuant",
             "aclnnDynamicMxQuantGetWorkspaceSize", "aclnnDynamicMxQuant", "opsnnDynamicMxQuant",
             "aclnnTransQuantParamV2GetWorkspaceSize", "aclnnTransQuantParamV2", "aclnnTransQuantParamV3GetWorkspaceSize",
