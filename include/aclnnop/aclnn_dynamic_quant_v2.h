@@ -5,8 +5,8 @@
  *
  * Replaces quant/dynamic_quant_v2/op_host/op_api/aclnn_dynamic_quant_v2.h:23-33 (implementation:
  * quant/dynamic_quant/op_host/op_api/aclnn_dynamic_quant.cpp:478-490).  dstType is carried as in the reference, which
- * takes the output type from yOut.  groupIndexOptional (per-expert smooth scales) is answered with
- * ACLNN_ERR_INNER_TILING_ERROR here.
+ * takes the output type from yOut.  groupIndexOptional [experts] (INT32 / INT64, the row where each expert's rows end) selects the
+ * row of smoothScalesOptional [experts, x.shape[-1]] that a row of x is multiplied with; rows past the last end are left untouched.
  */
 #ifndef OPSNN_AMD_ACLNN_DYNAMIC_QUANT_V2_H_
 #define OPSNN_AMD_ACLNN_DYNAMIC_QUANT_V2_H_

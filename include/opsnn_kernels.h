@@ -146,7 +146,7 @@ OPSNN_API int opsnnTransQuantParam(const float* scale, int64_t scale_len, const 
 /* Dynamic per-token quantisation of x [rows, cols] (FLOAT16 / BF16, dense): per row a scale (and, when `offset` is not
  * NULL, an offset: the asymmetric form) and the quantised row y in INT8, INT4 (two per byte, even column in the low nibble;
  * cols even), FLOAT8_E4M3FN or FLOAT8_E5M2.  smooth: NULL or [cols] factors of x's dtype.  Formula:
- * quant/dynamic_quant/tests/assets/golden.py:17-122 (pertoken).  A row without range (all zeros; asymmetric: constant)
+ * quant/dynamic_quant/tests/assets/golden.py:17-122 (pertoken, with or without group_index).  A row without range (all zeros; asymmetric: constant)
  * gets scale 0 and zeros.  force_variant: 0 automatic, 1 the register-resident kernel, 2 the two-pass kernel. */
 typedef struct {
     const void* x; int x_dtype;
@@ -156,6 +156,10 @@ typedef struct {
     float* offset;
     int64_t rows, cols;
     int force_variant;
+    /* per-expert smooth factors: group_index[e] (INT32 or INT64, ascending) is the row where expert e's rows end, and smooth
+     * is then [groups, cols]; rows from group_index[groups - 1] on are left untouched.  NULL: one smooth row for all. */
+    const void* group_index; int group_index_dtype;
+    int64_t groups;
 } OpsnnDynQuantArgs;
 OPSNN_API int opsnnDynamicQuant(const OpsnnDynQuantArgs* a, void* stream);
 

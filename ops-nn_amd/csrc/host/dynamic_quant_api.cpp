@@ -60,6 +60,10 @@ aclnnStatus get_workspace(const char* api, const aclTensor* x_, const aclTensor*
     if (sm.present) {
         if (gi.present) {
             if (gi.rank() != 1) INVALID("%s: groupIndex must have one dim", api);
+            // documented (quant/dynamic_quant_v2/docs/aclnnDynamicQuantV2.md:156-166): smoothScales [experts <= 1024, x.shape[-1]]
+            if (sm.rank() != 2 || sm.dim(1) != cols || sm.dim(0) != gi.dim(0) || sm.dim(0) > 1024)
+                INVALID("%s: with groupIndex [%ld] smoothScales must be [%ld, %ld] (at most 1024 experts), got %s", api, (long)gi.dim(0),
+                        (long)gi.dim(0), (long)cols, shape_str(sm.shape).c_str());
         } else {
             if (sm.rank() != 1) INVALID("%s: smoothScales must have one dim, got %ld", api, (long)sm.rank());
             const int64_t want_len = perchannel ? x.dim(-2) : cols;
@@ -98,7 +102,8 @@ aclnnStatus get_workspace(const char* api, const aclTensor* x_, const aclTensor*
     // what this build does not run
     if (pertensor || perchannel) FAIL(ACLNN_ERR_INNER_TILING_ERROR, "%s: quantMode %s has no kernel here (pertoken has)", api, quantMode);
     if (dstTypeMax != 0.0f) FAIL(ACLNN_ERR_INNER_TILING_ERROR, "%s: a dstTypeMax other than 0 has no kernel here", api);
-    if (gi.present) FAIL(ACLNN_ERR_INNER_TILING_ERROR, "%s: groupIndex (per-expert smooth scales) has no kernel here", api);
+    if (gi.present && !sm.present) INVALID("%s: groupIndex needs smoothScales", api);
+    if (gi.present && (gi.empty() || !is_contiguous(gi))) INVALID("%s: groupIndex must be a non-empty contiguous tensor here", api);
     if (y.dtype == ACL_HIFLOAT8) FAIL(ACLNN_ERR_INNER_TILING_ERROR, "%s: HIFLOAT8 output has no kernel on this device", api);
     if (!is_contiguous(x) || !is_contiguous(y) || !is_contiguous(sc) || (sm.present && !is_contiguous(sm)) || (off.present && !is_contiguous(off)))
         INVALID("%s: tensors must be contiguous here", api);
@@ -112,6 +117,7 @@ aclnnStatus get_workspace(const char* api, const aclTensor* x_, const aclTensor*
     a.offset = off.present ? (float*)const_cast<void*>(off.ptr_at(0)) : nullptr;
     a.rows = x.numel() / cols; a.cols = cols;
     a.force_variant = 0;
+    if (gi.present) { a.group_index = gi.ptr_at(0); a.group_index_dtype = gi.dtype; a.groups = gi.dim(0); }
     *executor = ex.release();
     return ACLNN_SUCCESS;
 }

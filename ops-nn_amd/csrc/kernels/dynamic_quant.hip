@@ -20,7 +20,23 @@ struct DynQuantParams {
     const uint16_t* x; const uint16_t* smooth; void* y; float* scale; float* offset;
     int64_t rows, cols;
     int y_dt; float tmax, rcp;   // rcp = 1 / tmax (symmetric) or 1 / tmax2
+    const void* gi; int gi_i64; int64_t groups;   // per-expert smooth rows: expert e owns the rows below gi[e] that no earlier expert owns
 };
+
+// Smooth row of a row of x: p.smooth itself without experts; with experts the row of the first expert whose end lies
+// above `row` (binary search; the ends ascend), nullptr-equivalent -1 past the last end.
+__device__ __forceinline__ int64_t smooth_row_of(const DynQuantParams& p, int64_t row)
+{
+    if (!p.gi) return 0;
+    int64_t lo = 0, hi = p.groups;   // first e in [lo, hi) with end(e) > row
+    while (lo < hi) {
+        const int64_t mid = (lo + hi) >> 1;
+        const int64_t end = p.gi_i64 ? ((const int64_t*)p.gi)[mid] : (int64_t)((const int32_t*)p.gi)[mid];
+        if (end > row) hi = mid;
+        else lo = mid + 1;
+    }
+    return lo < p.groups ? lo : -1;
+}
 
 template <int X_DT>
 __device__ __forceinline__ float x_to_f32(uint32_t h)
@@ -102,8 +118,10 @@ __global__ __launch_bounds__(256) void dynamic_quant_rows_kernel(DynQuantParams 
     __shared__ float red[3][4];
     const int t = threadIdx.x % TPR;
     const int64_t row = (int64_t)blockIdx.x * RPW + threadIdx.x / TPR;
-    const bool live = row < p.rows;   // whole waves: TPR is a multiple of 64
+    const int64_t srow = row < p.rows ? smooth_row_of(p, row) : -1;
+    const bool live = row < p.rows && srow >= 0;   // whole waves: TPR is a multiple of 64
     const int64_t pieces = p.cols / 8;
+    const uint4* smr = (const uint4*)(p.smooth + (srow > 0 ? srow : 0) * p.cols);
     const uint4* xr = (const uint4*)(p.x + (live ? row : 0) * p.cols);
     uint4 buf[MAXP];
     float amax = 0.0f, vmax = -__builtin_inff(), vmin = __builtin_inff();
@@ -119,7 +137,7 @@ __global__ __launch_bounds__(256) void dynamic_quant_rows_kernel(DynQuantParams 
         if (live && c < pieces) {
             buf[i] = xr[c];
             uint4 sm = make_uint4(0, 0, 0, 0);
-            if (p.smooth) sm = ((const uint4*)p.smooth)[c];
+            if (p.smooth) sm = smr[c];
 #pragma unroll
             for (int e = 0; e < 8; e++) {
                 const float v = element(buf[i], sm, e);
@@ -149,7 +167,7 @@ __global__ __launch_bounds__(256) void dynamic_quant_rows_kernel(DynQuantParams 
         const int64_t c = (int64_t)i * TPR + t;
         if (c < pieces) {
             uint4 sm = make_uint4(0, 0, 0, 0);
-            if (p.smooth) sm = ((const uint4*)p.smooth)[c];
+            if (p.smooth) sm = smr[c];
             uint32_t lo = 0, hi = 0;
 #pragma unroll
             for (int e = 0; e < 8; e++) {
@@ -171,10 +189,13 @@ __global__ __launch_bounds__(256) void dynamic_quant_two_pass_kernel(DynQuantPar
     __shared__ float red[3][4];
     const int64_t row = blockIdx.x;
     const uint16_t* xr = p.x + row * p.cols;
+    const int64_t srow = smooth_row_of(p, row);
+    if (srow < 0) return;   // the whole workgroup: past the last expert's rows
+    const uint16_t* smr = p.smooth + srow * p.cols;
     float amax = 0.0f, vmax = -__builtin_inff(), vmin = __builtin_inff();
     auto element = [&](int64_t c) {
         float v = x_to_f32<X_DT>(xr[c]);
-        if (p.smooth) v = __fmul_rn(v, x_to_f32<X_DT>(p.smooth[c]));
+        if (p.smooth) v = __fmul_rn(v, x_to_f32<X_DT>(smr[c]));
         return v;
     };
     for (int64_t c = threadIdx.x; c < p.cols; c += 256) {
@@ -255,6 +276,10 @@ extern "C" int opsnnDynamicQuant(const OpsnnDynQuantArgs* a, void* stream)
     if (a->y_dtype == DT_I4 && (a->cols & 1)) return -2;
     p.x = (const uint16_t*)a->x; p.smooth = (const uint16_t*)a->smooth; p.y = a->y; p.scale = a->scale; p.offset = a->offset;
     p.rows = a->rows; p.cols = a->cols; p.y_dt = a->y_dtype;
+    if (a->group_index) {
+        if (!a->smooth || a->groups <= 0 || (a->group_index_dtype != DT_I32 && a->group_index_dtype != 9 /* INT64 */)) return -2;
+        p.gi = a->group_index; p.gi_i64 = a->group_index_dtype != DT_I32; p.groups = a->groups;
+    }
     if (a->x_dtype == DT_BF16) return launch_dynamic_quant_x<DT_BF16>(p, a->force_variant, (hipStream_t)stream);
     return launch_dynamic_quant_x<DT_F16>(p, a->force_variant, (hipStream_t)stream);
 }

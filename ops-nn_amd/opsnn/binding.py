@@ -68,6 +68,8 @@ class OpsnnDynQuantArgs(C.Structure):
         ("scale", C.c_void_p), ("offset", C.c_void_p),
         ("rows", C.c_int64), ("cols", C.c_int64),
         ("force_variant", C.c_int),
+        ("group_index", C.c_void_p), ("group_index_dtype", C.c_int),
+        ("groups", C.c_int64),
     ]
 
 

@@ -45,7 +45,8 @@
  *                       maximum instead of multiplication by its reciprocal, round-half-away, or a 16-bit smooth
  *                       product each fail; numpy float32 recomputation; dequantisation error <= scale / 2); a row of
  *                       zeros (symmetric) or a constant row (asymmetric) divides by zero in the golden: parity unpinned,
- *                       this file writes zeros there
+ *                       this file writes zeros there; with per-expert smooth rows, the rows past the last expert's end (dropped
+ *                       by the golden) are left untouched: parity unpinned
  *   orc_dynamic_block_quant pinned (numpy float32 recomputation with torch's fp8 casts; a block with max 448 has scale 1
  *                       and returns x itself through the decimal rounding; min_scale cap and clipping by hand;
  *                       infinities and NaN by the golden's stated rules)
@@ -823,8 +824,18 @@ size_t orc_dtype_bits(int dt) { return dtype_bits(dt); }
  * with (tmax, tmax2) = (127, 255) int8, (7, 15) int4, (448, 896) e4m3, (57344, 114688) e5m2; 1 / tmax is an fp32 constant
  * and every operation is a separately rounded fp32 operation.  int4 results are packed two per byte, even column low.
  * A row whose scale is zero divides by zero in the golden (NaN through an integer cast): zeros are written instead. */
+int orc_dynamic_quant_grouped(const void* x, int x_dt, int64_t rows, int64_t cols, const void* smooth, const int64_t* group_end,
+                              int64_t groups, int y_dt, int symmetric, void* y, float* scale_out, float* offset_out);
 int orc_dynamic_quant(const void* x, int x_dt, int64_t rows, int64_t cols, const void* smooth, int y_dt, int symmetric,
                       void* y, float* scale_out, float* offset_out)
+{
+    return orc_dynamic_quant_grouped(x, x_dt, rows, cols, smooth, NULL, 0, y_dt, symmetric, y, scale_out, offset_out);
+}
+/* With group_end (GD:52-64): smooth is [groups, cols], expert e owns the rows from group_end[e - 1] (0 for e = 0) up to
+ * group_end[e]; an expert whose range is empty owns none.  The golden drops the rows from group_end[groups - 1] on; here they are
+ * left untouched (parity unpinned for them). */
+int orc_dynamic_quant_grouped(const void* x, int x_dt, int64_t rows, int64_t cols, const void* smooth, const int64_t* group_end,
+                              int64_t groups, int y_dt, int symmetric, void* y, float* scale_out, float* offset_out)
 {
     float tmax, tmax2;
     switch (y_dt) {
@@ -840,10 +851,15 @@ int orc_dynamic_quant(const void* x, int x_dt, int64_t rows, int64_t cols, const
     float* v = (float*)malloc((size_t)cols * sizeof(float));
     if (!v) return -2;
     for (int64_t r = 0; r < rows; r++) {
+        int64_t expert = 0;
+        if (group_end) {
+            while (expert < groups && group_end[expert] <= r) expert++;
+            if (expert == groups) continue;
+        }
         float vmax = -INFINITY, vmin = INFINITY, amax = 0.0f;
         for (int64_t c = 0; c < cols; c++) {
             float e = load_as_f32(x, x_dt, (size_t)(r * cols + c));
-            if (smooth) e = e * load_as_f32(smooth, x_dt, (size_t)c);
+            if (smooth) e = e * load_as_f32(smooth, x_dt, (size_t)(expert * cols + c));
             v[c] = e;
             if (e > vmax) vmax = e;
             if (e < vmin) vmin = e;

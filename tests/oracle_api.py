@@ -42,6 +42,8 @@ def lib():
         L.orc_convert_weight_b4.restype = None
         L.orc_dynamic_quant.argtypes = [vp, C.c_int, i64, i64, vp, C.c_int, C.c_int, vp, vp, vp]
         L.orc_dynamic_quant.restype = C.c_int
+        L.orc_dynamic_quant_grouped.argtypes = [vp, C.c_int, i64, i64, vp, vp, i64, C.c_int, C.c_int, vp, vp, vp]
+        L.orc_dynamic_quant_grouped.restype = C.c_int
         L.orc_e5m2_from_f32.argtypes = [C.c_float]
         L.orc_e5m2_from_f32.restype = C.c_uint8
         L.orc_dynamic_block_quant.argtypes = [vp, C.c_int, i64, i64, i64, i64, i64, C.c_double, C.c_int, vp, vp]
@@ -83,8 +85,9 @@ def e8m0_to_f32(a): return _conv("orc_vec_e8m0_to_f32", np.asarray(a, np.uint8),
 E2M1_VALUES = np.array([0, .5, 1, 1.5, 2, 3, 4, 6, -0.0, -.5, -1, -1.5, -2, -3, -4, -6], np.float32)
 
 
-def dynamic_quant(x, x_dt, y_dt, smooth=None, symmetric=True):
-    """x: uint16 bits [..., cols] of x_dt.  Returns (y bytes, scale[, offset]); int4 results are packed two per byte."""
+def dynamic_quant(x, x_dt, y_dt, smooth=None, symmetric=True, group_end=None, fill=0):
+    """x: uint16 bits [..., cols] of x_dt.  Returns (y bytes, scale[, offset]); int4 results are packed two per byte.
+    group_end: per-expert row ends (then smooth is [experts, cols]); rows past the last end keep the byte `fill`."""
     x = np.ascontiguousarray(x, np.uint16)
     cols = x.shape[-1]
     rows = x.size // cols
@@ -92,8 +95,14 @@ def dynamic_quant(x, x_dt, y_dt, smooth=None, symmetric=True):
     scale = np.zeros(x.shape[:-1], np.float32)
     offset = np.zeros(x.shape[:-1], np.float32)
     sm = None if smooth is None else np.ascontiguousarray(smooth, np.uint16)
-    rc = lib().orc_dynamic_quant(x.ctypes.data, x_dt, rows, cols, sm.ctypes.data if sm is not None else None, y_dt, int(symmetric),
-                                 y.ctypes.data, scale.ctypes.data, offset.ctypes.data)
+    ge = None if group_end is None else np.ascontiguousarray(group_end, np.int64)
+    if fill:
+        y[...] = fill
+        scale.view(np.uint8)[...] = fill
+        offset.view(np.uint8)[...] = fill
+    rc = lib().orc_dynamic_quant_grouped(x.ctypes.data, x_dt, rows, cols, sm.ctypes.data if sm is not None else None,
+                                         ge.ctypes.data if ge is not None else None, ge.size if ge is not None else 0, y_dt, int(symmetric),
+                                         y.ctypes.data, scale.ctypes.data, offset.ctypes.data)
     assert rc == 0, rc
     return (y, scale) if symmetric else (y, scale, offset)
 

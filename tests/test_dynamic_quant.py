@@ -105,6 +105,19 @@ def test_dequantised_rows_are_within_half_a_step():
     assert (np.abs((y.view(np.int8) - o[:, None].astype(np.float64)) * s[:, None] - xf) <= 0.51 * s[:, None]).all()
 
 
+def test_group_index_selects_the_smooth_row():
+    """Rows [0, 3) use expert 0's factors, expert 1 owns no rows (its end equals expert 0's), rows [3, 7) use expert 2's: equal to
+    quantising each slice with its own smooth vector.  Rows from 7 on are left untouched."""
+    rng = np.random.default_rng(8)
+    xb = orc.f32_to_b16(rng.normal(0, 1, size=(9, 64)).astype(np.float32), orc.F16)
+    smb = orc.f32_to_b16(rng.uniform(0.5, 2.0, size=(3, 64)).astype(np.float32), orc.F16)
+    y, s = orc.dynamic_quant(xb, orc.F16, orc.I8, smooth=smb, group_end=[3, 3, 7], fill=0xEE)
+    y0, s0 = orc.dynamic_quant(xb[:3], orc.F16, orc.I8, smooth=smb[0])
+    y2, s2 = orc.dynamic_quant(xb[3:7], orc.F16, orc.I8, smooth=smb[2])
+    assert np.array_equal(y[:3], y0) and np.array_equal(y[3:7], y2) and np.array_equal(s[:3], s0) and np.array_equal(s[3:7], s2)
+    assert (y[7:] == 0xEE).all() and (s[7:].view(np.uint8) == 0xEE).all()
+
+
 def test_rows_without_range_give_zeros():
     """Not the golden's behaviour (it divides by zero there): the convention of this build, see the oracle's header."""
     x = _f16([[0.0] * 8, [1.0] * 8])
@@ -165,7 +178,14 @@ def test_status_rules_one_by_one(opsnn):
     assert _status(m, _t(m, (0, 32), m.ACL_BF16), _t(m, (0, 32), m.ACL_INT8), _t(m, (0,), m.ACL_FLOAT)) == 0
     # accepted by the reference, no kernel here
     assert _status(m, x, _t(m, (4, 6, 32), m.ACL_HIFLOAT8), sc) == m.STATUS_BY_NAME.get("ACLNN_ERR_INNER_TILING_ERROR", 561002)
-    assert _status(m, x, y, sc, smooth=_t(m, (2, 32), m.ACL_BF16), group_index=_t(m, (2,), m.ACL_INT32)) == 561002
+    # per-expert smooth scales (V2): smoothScales [experts, cols] with groupIndex [experts]
+    assert _status(m, x, y, sc, smooth=_t(m, (2, 32), m.ACL_BF16), group_index=_t(m, (2,), m.ACL_INT32)) == 0
+    assert _status(m, x, y, sc, smooth=_t(m, (2, 32), m.ACL_BF16), group_index=_t(m, (2,), m.ACL_INT64)) == 0
+    assert _status(m, x, y, sc, smooth=_t(m, (2, 32), m.ACL_BF16), group_index=_t(m, (2,), m.ACL_FLOAT)) == bad
+    assert _status(m, x, y, sc, smooth=_t(m, (2, 32), m.ACL_BF16), group_index=_t(m, (1, 2), m.ACL_INT32)) == bad
+    assert _status(m, x, y, sc, smooth=_t(m, (3, 32), m.ACL_BF16), group_index=_t(m, (2,), m.ACL_INT32)) == bad
+    assert _status(m, x, y, sc, smooth=_t(m, (32,), m.ACL_BF16), group_index=_t(m, (2,), m.ACL_INT32)) == bad
+    assert _status(m, x, y, sc, group_index=_t(m, (2,), m.ACL_INT32)) == bad                        # groupIndex needs smoothScales
 
 
 def test_v3_v4_attribute_rules(opsnn):
@@ -296,3 +316,32 @@ def test_gpu_v3_and_v4_pertoken_equal_v1(gpu):
         m.dynamic_quant(m.Tensor((40, 512), m.ACL_FLOAT16, d_x), m.Tensor((40, 512), m.ACL_INT8, d_y), m.Tensor((40,), m.ACL_FLOAT, d_s), **kw)
         m.check(m.lib().aclrtSynchronizeDevice(), "sync")
         assert np.array_equal(d_y.to_host(np.uint8, (40, 512)), want_y) and np.array_equal(d_s.to_host(np.float32, (40,)), want_s)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("shape,ends,gi_dt,symmetric", [((40, 256), [5, 5, 17, 40], "i32", True), ((3, 11, 4096), [10, 20, 30], "i64", False),
+                                                       ((9, 1000), [2, 9], "i32", True), ((6, 20000), [1, 4], "i64", True)])
+def test_gpu_group_index(gpu, shape, ends, gi_dt, symmetric):
+    """aclnnDynamicQuantV2 with per-expert smooth scales, on the register-resident and the two-pass kernels; rows past the last
+    expert's end keep what was in the output buffers."""
+    m = gpu
+    print(f"case dynamic quant groups {shape} ends={ends} {gi_dt} symmetric={symmetric}", flush=True)
+    rng = np.random.default_rng(sum(shape))
+    cols, rows = shape[-1], int(np.prod(shape[:-1]))
+    xb = orc.f32_to_b16(rng.normal(0, 2, size=shape).astype(np.float32), orc.BF16)
+    smb = orc.f32_to_b16(rng.uniform(0.5, 2.0, size=(len(ends), cols)).astype(np.float32), orc.BF16)
+    want = orc.dynamic_quant(xb, orc.BF16, orc.I8, smooth=smb, symmetric=symmetric, group_end=ends, fill=0xEE)
+    gi = np.array(ends, np.int32 if gi_dt == "i32" else np.int64)
+    d_x, d_sm, d_gi = m.DeviceBuffer(host=xb), m.DeviceBuffer(host=smb), m.DeviceBuffer(host=gi)
+    d_y, d_s, d_o = m.DeviceBuffer(xb.size), m.DeviceBuffer(rows * 4), m.DeviceBuffer(rows * 4)
+    for b in (d_y, d_s, d_o):
+        b.fill(0xEE)
+    off = None if symmetric else m.Tensor(shape[:-1], m.ACL_FLOAT, d_o)
+    m.dynamic_quant(m.Tensor(shape, m.ACL_BF16, d_x), m.Tensor(shape, m.ACL_INT8, d_y), m.Tensor(shape[:-1], m.ACL_FLOAT, d_s),
+                    smooth=m.Tensor((len(ends), cols), m.ACL_BF16, d_sm), offset=off,
+                    group_index=m.Tensor((len(ends),), m.ACL_INT32 if gi_dt == "i32" else m.ACL_INT64, d_gi))
+    m.check(m.lib().aclrtSynchronizeDevice(), "sync")
+    assert np.array_equal(d_y.to_host(np.uint8, shape), want[0])
+    assert np.array_equal(d_s.to_host(np.uint32, shape[:-1]), want[1].view(np.uint32))
+    if not symmetric:
+        assert np.array_equal(d_o.to_host(np.uint32, shape[:-1]), want[2].view(np.uint32))
