@@ -2,9 +2,9 @@
  * aclnnDynamicQuantV3 -- aclnnDynamicQuantV2 with the symmetry flag and the quantisation mode as attributes.
  *
  * Replaces quant/dynamic_quant/op_host/op_api/aclnn_dynamic_quant_v3.h; attribute and shape rules of
- * aclnn_dynamic_quant.cpp:171-189, 191-291.  isSymmetrical must agree with offsetOut (null when true).  quantMode "pertoken" runs
- * here; "pertensor" (scaleOut [1]) and "perchannel" (scaleOut = x's shape without the second-to-last dim) are checked as in the
- * reference and then answered with ACLNN_ERR_INNER_TILING_ERROR.
+ * aclnn_dynamic_quant.cpp:171-189, 191-291.  isSymmetrical must agree with offsetOut (null when true).  quantMode "pertoken",
+ * "pertensor" (scaleOut [1]) and "perchannel" (scaleOut = x's shape without the second-to-last dim; smoothScales one factor per
+ * row of that dim) run here.
  */
 #ifndef OPSNN_AMD_ACLNN_DYNAMIC_QUANT_V3_H_
 #define OPSNN_AMD_ACLNN_DYNAMIC_QUANT_V3_H_

@@ -160,6 +160,12 @@ typedef struct {
      * is then [groups, cols]; rows from group_index[groups - 1] on are left untouched.  NULL: one smooth row for all. */
     const void* group_index; int group_index_dtype;
     int64_t groups;
+    /* quant_mode 0: one scale per row (above).  1 "pertensor": one scale (and offset) for the whole tensor, scale[1].
+     * 2 "perchannel": x is [rows / chan_rows, chan_rows, cols], one scale per batch and column (the reduction runs over the
+     * chan_rows axis), scale [rows / chan_rows, cols], and smooth holds chan_rows factors, one per row of a batch.  In modes
+     * 1 and 2 the scale / offset buffers hold intermediate values until the call's last kernel has run. */
+    int quant_mode;
+    int64_t chan_rows;
 } OpsnnDynQuantArgs;
 OPSNN_API int opsnnDynamicQuant(const OpsnnDynQuantArgs* a, void* stream);
 

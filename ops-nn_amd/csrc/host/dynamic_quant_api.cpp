@@ -100,7 +100,7 @@ aclnnStatus get_workspace(const char* api, const aclTensor* x_, const aclTensor*
         return ACLNN_SUCCESS;
     }
     // what this build does not run
-    if (pertensor || perchannel) FAIL(ACLNN_ERR_INNER_TILING_ERROR, "%s: quantMode %s has no kernel here (pertoken has)", api, quantMode);
+    if ((pertensor || perchannel) && gi.present) FAIL(ACLNN_ERR_INNER_TILING_ERROR, "%s: groupIndex with quantMode %s has no kernel here", api, quantMode);
     if (dstTypeMax != 0.0f) FAIL(ACLNN_ERR_INNER_TILING_ERROR, "%s: a dstTypeMax other than 0 has no kernel here", api);
     if (gi.present && !sm.present) INVALID("%s: groupIndex needs smoothScales", api);
     if (gi.present && (gi.empty() || !is_contiguous(gi))) INVALID("%s: groupIndex must be a non-empty contiguous tensor here", api);
@@ -118,6 +118,8 @@ aclnnStatus get_workspace(const char* api, const aclTensor* x_, const aclTensor*
     a.rows = x.numel() / cols; a.cols = cols;
     a.force_variant = 0;
     if (gi.present) { a.group_index = gi.ptr_at(0); a.group_index_dtype = gi.dtype; a.groups = gi.dim(0); }
+    a.quant_mode = pertensor ? 1 : perchannel ? 2 : 0;
+    a.chan_rows = perchannel ? x.dim(-2) : 0;
     *executor = ex.release();
     return ACLNN_SUCCESS;
 }

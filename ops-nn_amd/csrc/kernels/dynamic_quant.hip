@@ -244,6 +244,136 @@ static int launch_dynamic_quant(const DynQuantParams& p, int variant, hipStream_
     return (int)hipGetLastError();
 }
 
+// ---------------------------------------------------------------------------------------------------------------------
+// "pertensor" and "perchannel": the extremes are reduced over many rows, so the work is split in kernels.  The scale
+// buffer (and the offset buffer in the asymmetric form) first collects the extremes through integer atomics on an
+// order-preserving key of the float (max|v| in scale; or max v in scale and min v in offset), the quantising kernel reads
+// them from there and derives scale and offset per element group, and a last small kernel turns the collected extremes
+// into the scale and offset values.  Maxima and minima do not depend on the order of the atomics: the result is exact.
+__device__ __forceinline__ uint32_t float_key(float f)
+{
+    const uint32_t u = f2u(f);
+    return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+}
+__device__ __forceinline__ float key_float(uint32_t k) { return u2f((k & 0x80000000u) ? (k & 0x7fffffffu) : ~k); }
+
+// slot of element (row, col): pertensor 0; perchannel (row / chan_rows) * cols + col
+struct WideQuantParams {
+    DynQuantParams p;
+    int mode;            // 1 pertensor, 2 perchannel
+    int64_t chan_rows, nslots;
+    uint32_t* smax;      // = p.scale
+    uint32_t* smin;      // = p.offset (asymmetric) or null
+};
+
+__global__ __launch_bounds__(256) void wide_quant_init_kernel(WideQuantParams w)
+{
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= w.nslots) return;
+    w.smax[i] = w.smin ? float_key(-__builtin_inff()) : float_key(0.0f);
+    if (w.smin) w.smin[i] = float_key(__builtin_inff());
+}
+
+// one thread per (row chunk of 64 rows, column): coalesced over columns; a workgroup covers 256 columns of one chunk
+template <int X_DT>
+__global__ __launch_bounds__(256) void wide_quant_reduce_kernel(WideQuantParams w)
+{
+    const DynQuantParams& p = w.p;
+    const int64_t col = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const int64_t r0 = (int64_t)blockIdx.y * 64;
+    const bool inside = col < p.cols;   // lanes past the last column stay for the wave reduction with neutral values
+    float vmax = -__builtin_inff(), vmin = __builtin_inff();
+    int64_t slot = -1;
+    for (int64_t r = r0; inside && r < r0 + 64 && r < p.rows; r++) {
+        const int64_t s = w.mode == 1 ? 0 : (r / w.chan_rows) * p.cols + col;
+        if (s != slot && slot >= 0) {   // a new batch begins inside the chunk: hand in what was collected
+            if (w.smin) { atomicMax(w.smax + slot, float_key(vmax)); atomicMin(w.smin + slot, float_key(vmin)); }
+            else atomicMax(w.smax + slot, float_key(fmaxf(vmax, -vmin)));
+            vmax = -__builtin_inff(); vmin = __builtin_inff();
+        }
+        slot = s;
+        float v = x_to_f32<X_DT>(p.x[r * p.cols + col]);
+        if (p.smooth) v = __fmul_rn(v, x_to_f32<X_DT>(p.smooth[w.mode == 1 ? col : r % w.chan_rows]));
+        vmax = fmaxf(vmax, v);
+        vmin = fminf(vmin, v);
+    }
+    if (w.mode == 1) {   // one slot for everybody: reduce the wave first
+        vmax = wave_max(vmax);
+        vmin = -wave_max(-vmin);
+        if ((threadIdx.x & 63) != 0 || r0 >= p.rows) return;
+        slot = 0;
+    }
+    if (slot < 0) return;
+    if (w.smin) { atomicMax(w.smax + slot, float_key(vmax)); atomicMin(w.smin + slot, float_key(vmin)); }
+    else atomicMax(w.smax + slot, float_key(fmaxf(vmax, -vmin)));
+}
+
+template <int X_DT, int Y_DT, bool ASYM>
+__global__ __launch_bounds__(256) void wide_quant_apply_kernel(WideQuantParams w)
+{
+    const DynQuantParams& p = w.p;
+    const int64_t pair = (int64_t)blockIdx.x * 256 + threadIdx.x;   // two neighbouring columns per thread (an int4 byte)
+    const int64_t ppr = (p.cols + 1) / 2;
+    if (pair >= p.rows * ppr) return;
+    const int64_t row = pair / ppr, c0 = (pair % ppr) * 2;
+    uint32_t out[2] = {0, 0};
+    for (int e = 0; e < 2 && c0 + e < p.cols; e++) {
+        const int64_t col = c0 + e;
+        const int64_t slot = w.mode == 1 ? 0 : (row / w.chan_rows) * p.cols + col;
+        const float a = key_float(w.smax[slot]);
+        const RowQuant r = row_params<ASYM>(p, a, a, ASYM ? key_float(w.smin[slot]) : 0.0f);
+        float v = x_to_f32<X_DT>(p.x[row * p.cols + col]);
+        if (p.smooth) v = __fmul_rn(v, x_to_f32<X_DT>(p.smooth[w.mode == 1 ? col : row % w.chan_rows]));
+        out[e] = quant_one<Y_DT, ASYM>(v, r);
+    }
+    if (Y_DT == DT_I4) ((uint8_t*)p.y)[(row * p.cols + c0) / 2] = (uint8_t)(out[0] | (out[1] << 4));
+    else {
+        ((uint8_t*)p.y)[row * p.cols + c0] = (uint8_t)out[0];
+        if (c0 + 1 < p.cols) ((uint8_t*)p.y)[row * p.cols + c0 + 1] = (uint8_t)out[1];
+    }
+}
+
+template <bool ASYM>
+__global__ __launch_bounds__(256) void wide_quant_finish_kernel(WideQuantParams w)
+{
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= w.nslots) return;
+    const float a = key_float(w.smax[i]);
+    const RowQuant r = row_params<ASYM>(w.p, a, a, ASYM ? key_float(w.smin[i]) : 0.0f);
+    w.p.scale[i] = r.scale;
+    if (ASYM) w.p.offset[i] = r.offset;
+}
+
+template <int X_DT, int Y_DT, bool ASYM>
+static int launch_wide_quant(const DynQuantParams& p, int mode, int64_t chan_rows, hipStream_t st)
+{
+    WideQuantParams w{};
+    w.p = p; w.mode = mode; w.chan_rows = mode == 2 ? chan_rows : p.rows;
+    w.nslots = mode == 1 ? 1 : (p.rows / w.chan_rows) * p.cols;
+    w.smax = (uint32_t*)p.scale; w.smin = ASYM ? (uint32_t*)p.offset : nullptr;
+    const int64_t row_chunks = (p.rows + 63) / 64, pairs = p.rows * ((p.cols + 1) / 2);
+    if (row_chunks > 65535 || (p.cols + 255) / 256 > 0x7fffffff || (pairs + 255) / 256 > 0x7fffffff || (w.nslots + 255) / 256 > 0x7fffffff) return -1;
+    const dim3 slots((unsigned)((w.nslots + 255) / 256));
+    hipLaunchKernelGGL(wide_quant_init_kernel, slots, dim3(256), 0, st, w);
+    hipLaunchKernelGGL(wide_quant_reduce_kernel<X_DT>, dim3((unsigned)((p.cols + 255) / 256), (unsigned)row_chunks), dim3(256), 0, st, w);
+    hipLaunchKernelGGL((wide_quant_apply_kernel<X_DT, Y_DT, ASYM>), dim3((unsigned)((pairs + 255) / 256)), dim3(256), 0, st, w);
+    hipLaunchKernelGGL(wide_quant_finish_kernel<ASYM>, slots, dim3(256), 0, st, w);
+    return (int)hipGetLastError();
+}
+
+template <int X_DT>
+static int launch_wide_quant_x(const DynQuantParams& p, int mode, int64_t chan_rows, hipStream_t st)
+{
+    const bool asym = p.offset != nullptr;
+    switch (p.y_dt) {
+        case DT_I8: return asym ? launch_wide_quant<X_DT, DT_I8, true>(p, mode, chan_rows, st) : launch_wide_quant<X_DT, DT_I8, false>(p, mode, chan_rows, st);
+        case DT_I4: return asym ? launch_wide_quant<X_DT, DT_I4, true>(p, mode, chan_rows, st) : launch_wide_quant<X_DT, DT_I4, false>(p, mode, chan_rows, st);
+        case DT_E4M3: return asym ? launch_wide_quant<X_DT, DT_E4M3, true>(p, mode, chan_rows, st) : launch_wide_quant<X_DT, DT_E4M3, false>(p, mode, chan_rows, st);
+        case DT_E5M2: return asym ? launch_wide_quant<X_DT, DT_E5M2, true>(p, mode, chan_rows, st) : launch_wide_quant<X_DT, DT_E5M2, false>(p, mode, chan_rows, st);
+        default: return -2;
+    }
+}
+
 template <int X_DT>
 static int launch_dynamic_quant_x(const DynQuantParams& p, int variant, hipStream_t st)
 {
@@ -280,6 +410,12 @@ extern "C" int opsnnDynamicQuant(const OpsnnDynQuantArgs* a, void* stream)
         if (!a->smooth || a->groups <= 0 || (a->group_index_dtype != DT_I32 && a->group_index_dtype != 9 /* INT64 */)) return -2;
         p.gi = a->group_index; p.gi_i64 = a->group_index_dtype != DT_I32; p.groups = a->groups;
     }
+    if (a->quant_mode == 1 || a->quant_mode == 2) {
+        if (a->group_index || (a->quant_mode == 2 && (a->chan_rows <= 0 || a->rows % a->chan_rows != 0))) return -2;
+        if (a->x_dtype == DT_BF16) return launch_wide_quant_x<DT_BF16>(p, a->quant_mode, a->chan_rows, (hipStream_t)stream);
+        return launch_wide_quant_x<DT_F16>(p, a->quant_mode, a->chan_rows, (hipStream_t)stream);
+    }
+    if (a->quant_mode != 0) return -2;
     if (a->x_dtype == DT_BF16) return launch_dynamic_quant_x<DT_BF16>(p, a->force_variant, (hipStream_t)stream);
     return launch_dynamic_quant_x<DT_F16>(p, a->force_variant, (hipStream_t)stream);
 }

@@ -70,6 +70,7 @@ class OpsnnDynQuantArgs(C.Structure):
         ("force_variant", C.c_int),
         ("group_index", C.c_void_p), ("group_index_dtype", C.c_int),
         ("groups", C.c_int64),
+        ("quant_mode", C.c_int), ("chan_rows", C.c_int64),
     ]
 
 

@@ -47,6 +47,8 @@
  *                       zeros (symmetric) or a constant row (asymmetric) divides by zero in the golden: parity unpinned,
  *                       this file writes zeros there; with per-expert smooth rows, the rows past the last expert's end (dropped
  *                       by the golden) are left untouched: parity unpinned
+ *   orc_dynamic_quant_wide pinned (numpy float32 recomputation of the per-tensor and per-channel goldens; a tensor of one row / a
+ *                       batch of one row reduces to orc_dynamic_quant)
  *   orc_dynamic_block_quant pinned (numpy float32 recomputation with torch's fp8 casts; a block with max 448 has scale 1
  *                       and returns x itself through the decimal rounding; min_scale cap and clipping by hand;
  *                       infinities and NaN by the golden's stated rules)
@@ -1052,4 +1054,79 @@ void orc_trans_quant_param(const float* scale, int64_t scale_len, const float* o
         }
         out[i] = v;
     }
+}
+
+/* Dynamic quantisation with one scale for the whole tensor (mode 1, GD:66-94 with quant_mode "pertensor") or one per batch
+ * and column, reduced over the second-to-last axis (mode 2, GD:125-176 _dynamic_quant_perchannel): x is
+ * [rows / chan_rows, chan_rows, cols]; smooth has cols factors in mode 1 and chan_rows factors (one per row of a batch) in
+ * mode 2.  The element formulas are those of orc_dynamic_quant.  scale_out / offset_out: 1 element, or (rows / chan_rows) * cols. */
+int orc_dynamic_quant_wide(const void* x, int x_dt, int64_t rows, int64_t cols, int64_t chan_rows, int mode, const void* smooth, int y_dt,
+                           int symmetric, void* y, float* scale_out, float* offset_out)
+{
+    float tmax, tmax2;
+    switch (y_dt) {
+        case ORC_I8: tmax = 127.0f; tmax2 = 255.0f; break;
+        case ORC_I4: tmax = 7.0f; tmax2 = 15.0f; break;
+        case ORC_E4M3: tmax = 448.0f; tmax2 = 896.0f; break;
+        case ORC_E5M2: tmax = 57344.0f; tmax2 = 114688.0f; break;
+        default: return -1;
+    }
+    if ((mode != 1 && mode != 2) || rows <= 0 || cols <= 0 || (y_dt == ORC_I4 && (cols & 1))) return -1;
+    if (mode == 1) chan_rows = rows;
+    if (chan_rows <= 0 || rows % chan_rows) return -1;
+    const float rcp = 1.0f / (symmetric ? tmax : tmax2);
+    const int64_t nb = rows / chan_rows, nslots = mode == 1 ? 1 : nb * cols;
+    float* vmax = (float*)malloc((size_t)nslots * 3 * sizeof(float));
+    if (!vmax) return -2;
+    float *vmin = vmax + nslots, *amax = vmin + nslots;
+    for (int64_t s = 0; s < nslots; s++) { vmax[s] = -INFINITY; vmin[s] = INFINITY; amax[s] = 0.0f; }
+#define WIDE_VALUE(r, c) (load_as_f32(x, x_dt, (size_t)((r) * cols + (c))) * (smooth ? load_as_f32(smooth, x_dt, (size_t)(mode == 1 ? (c) : (r) % chan_rows)) : 1.0f))
+#define WIDE_SLOT(r, c) (mode == 1 ? 0 : ((r) / chan_rows) * cols + (c))
+    for (int64_t r = 0; r < rows; r++)
+        for (int64_t c = 0; c < cols; c++) {
+            const float e = smooth ? WIDE_VALUE(r, c) : load_as_f32(x, x_dt, (size_t)(r * cols + c));
+            const int64_t s = WIDE_SLOT(r, c);
+            if (e > vmax[s]) vmax[s] = e;
+            if (e < vmin[s]) vmin[s] = e;
+            if (fabsf(e) > amax[s]) amax[s] = fabsf(e);
+        }
+    for (int64_t s = 0; s < nslots; s++) {
+        float scale, offset = 0.0f;
+        if (symmetric) scale = amax[s] * rcp;
+        else { scale = (vmax[s] - vmin[s]) * rcp; offset = tmax - vmax[s] / scale; }
+        const int degenerate = !(scale > 0.0f) || !isfinite(scale);
+        scale_out[s] = scale;
+        if (!symmetric) offset_out[s] = degenerate ? 0.0f : offset;
+        amax[s] = degenerate ? 1.0f : 0.0f;   /* reused as the flag */
+    }
+    for (int64_t r = 0; r < rows; r++)
+        for (int64_t c = 0; c < cols; c++) {
+            const int64_t s = WIDE_SLOT(r, c);
+            const size_t i = (size_t)(r * cols + c);
+            float q = 0.0f;
+            if (amax[s] == 0.0f) {
+                const float e = smooth ? WIDE_VALUE(r, c) : load_as_f32(x, x_dt, i);
+                q = e / scale_out[s];
+                if (!symmetric) q = q + offset_out[s];
+            }
+            if (y_dt == ORC_E4M3) ((uint8_t*)y)[i] = orc_e4m3_from_f32(q);
+            else if (y_dt == ORC_E5M2) ((uint8_t*)y)[i] = orc_e5m2_from_f32(q);
+            else {
+                float rq = nearbyintf(q);
+                const float lo = y_dt == ORC_I8 ? -128.0f : -8.0f, hi = y_dt == ORC_I8 ? 127.0f : 7.0f;
+                if (!(rq == rq)) rq = 0.0f;
+                if (rq < lo) rq = lo;
+                if (rq > hi) rq = hi;
+                const int iv = (int)rq;
+                if (y_dt == ORC_I8) ((int8_t*)y)[i] = (int8_t)iv;
+                else {
+                    uint8_t* b = (uint8_t*)y + (i >> 1);
+                    *b = (i & 1) ? (uint8_t)((*b & 0x0fu) | ((iv & 15) << 4)) : (uint8_t)((*b & 0xf0u) | (iv & 15));
+                }
+            }
+        }
+#undef WIDE_VALUE
+#undef WIDE_SLOT
+    free(vmax);
+    return 0;
 }

@@ -67,6 +67,8 @@ int orc_dynamic_quant(const void* x, int x_dt, int64_t rows, int64_t cols, const
                       void* y, float* scale_out, float* offset_out);
 int orc_dynamic_quant_grouped(const void* x, int x_dt, int64_t rows, int64_t cols, const void* smooth, const int64_t* group_end,
                               int64_t groups, int y_dt, int symmetric, void* y, float* scale_out, float* offset_out);
+int orc_dynamic_quant_wide(const void* x, int x_dt, int64_t rows, int64_t cols, int64_t chan_rows, int mode, const void* smooth, int y_dt,
+                           int symmetric, void* y, float* scale_out, float* offset_out);
 int orc_dynamic_block_quant(const void* x, int x_dt, int64_t batch, int64_t rows, int64_t cols, int64_t rb, int64_t cb,
                             double min_scale, int y_dt, uint8_t* y, float* scale_out);
 int orc_dynamic_mx_quant(const void* x, int x_dt, int64_t rows, int64_t cols, int64_t block, int y_dt, uint8_t* y, uint8_t* scale_out);

@@ -44,6 +44,8 @@ def lib():
         L.orc_dynamic_quant.restype = C.c_int
         L.orc_dynamic_quant_grouped.argtypes = [vp, C.c_int, i64, i64, vp, vp, i64, C.c_int, C.c_int, vp, vp, vp]
         L.orc_dynamic_quant_grouped.restype = C.c_int
+        L.orc_dynamic_quant_wide.argtypes = [vp, C.c_int, i64, i64, i64, C.c_int, vp, C.c_int, C.c_int, vp, vp, vp]
+        L.orc_dynamic_quant_wide.restype = C.c_int
         L.orc_e5m2_from_f32.argtypes = [C.c_float]
         L.orc_e5m2_from_f32.restype = C.c_uint8
         L.orc_dynamic_block_quant.argtypes = [vp, C.c_int, i64, i64, i64, i64, i64, C.c_double, C.c_int, vp, vp]
@@ -140,6 +142,23 @@ def trans_quant_param(scale, offset=None, round_mode=0):
     lib().orc_trans_quant_param(scale.ctypes.data, scale.size, off.ctypes.data if off is not None else None,
                                 off.size if off is not None else 0, round_mode, out.ctypes.data)
     return out
+
+
+def dynamic_quant_wide(x, x_dt, y_dt, mode, smooth=None, symmetric=True):
+    """mode "pertensor": one scale; "perchannel": x [..., R, C], one scale per leading index and column.  Returns (y, scale[, offset])."""
+    x = np.ascontiguousarray(x, np.uint16)
+    cols = x.shape[-1]
+    rows = x.size // cols
+    per_tensor = mode == "pertensor"
+    chan_rows = rows if per_tensor else x.shape[-2]
+    sshape = (1,) if per_tensor else x.shape[:-2] + (cols,)
+    y = np.zeros(x.shape[:-1] + ((cols // 2) if y_dt == I4 else cols,), np.uint8)
+    scale, offset = np.zeros(sshape, np.float32), np.zeros(sshape, np.float32)
+    sm = None if smooth is None else np.ascontiguousarray(smooth, np.uint16)
+    rc = lib().orc_dynamic_quant_wide(x.ctypes.data, x_dt, rows, cols, chan_rows, 1 if per_tensor else 2, sm.ctypes.data if sm is not None else None,
+                                      y_dt, int(symmetric), y.ctypes.data, scale.ctypes.data, offset.ctypes.data)
+    assert rc == 0, rc
+    return (y, scale) if symmetric else (y, scale, offset)
 
 
 def convert_weight_b4(w):

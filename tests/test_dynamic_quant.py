@@ -118,6 +118,35 @@ def test_group_index_selects_the_smooth_row():
     assert (y[7:] == 0xEE).all() and (s[7:].view(np.uint8) == 0xEE).all()
 
 
+@pytest.mark.parametrize("mode", ["pertensor", "perchannel"])
+@pytest.mark.parametrize("symmetric,with_smooth", [(True, False), (False, True)])
+def test_wide_modes_against_numpy_float32(mode, symmetric, with_smooth):
+    """quant/dynamic_quant/tests/assets/golden.py:66-94 with quant_mode "pertensor" (the maxima over everything) and :125-176
+    (_dynamic_quant_perchannel: maxima over axis -2, smooth_scales[:, None]), in numpy float32 as the golden computes them."""
+    rng = np.random.default_rng(13)
+    shape = (3, 20, 48)
+    xb = orc.f32_to_b16(rng.normal(0, 2, size=shape).astype(np.float32), orc.BF16)
+    xf = orc.b16_to_f32(xb, orc.BF16)
+    n_sm = 48 if mode == "pertensor" else 20
+    smb = orc.f32_to_b16(rng.uniform(0.5, 2.0, n_sm).astype(np.float32), orc.BF16) if with_smooth else None
+    smf = orc.b16_to_f32(smb, orc.BF16) if with_smooth else None
+    v = xf if smf is None else (xf * smf if mode == "pertensor" else xf * smf[:, None])
+    red = dict(axis=None) if mode == "pertensor" else dict(axis=-2, keepdims=True)
+    if symmetric:
+        scale = np.max(np.abs(v), **red) * (np.float32(1.0) / np.float32(127.0))
+        want_y, want_o = np.round(v / scale), None
+    else:
+        vmax, vmin = np.max(v, **red), np.min(v, **red)
+        scale = (vmax - vmin) * (np.float32(1.0) / np.float32(255.0))
+        want_o = np.float32(127.0) - vmax / scale
+        want_y = np.round(v / scale + want_o)
+    out = orc.dynamic_quant_wide(xb, orc.BF16, orc.I8, mode, smooth=smb, symmetric=symmetric)
+    assert np.array_equal(out[0].view(np.int8).astype(np.int32), want_y.astype(np.int32))
+    assert np.array_equal(out[1].reshape(-1).view(np.uint32), np.asarray(scale, np.float32).reshape(-1).view(np.uint32))
+    if not symmetric:
+        assert np.array_equal(out[2].reshape(-1).view(np.uint32), np.asarray(want_o, np.float32).reshape(-1).view(np.uint32))
+
+
 def test_rows_without_range_give_zeros():
     """Not the golden's behaviour (it divides by zero there): the convention of this build, see the oracle's header."""
     x = _f16([[0.0] * 8, [1.0] * 8])
@@ -189,8 +218,7 @@ def test_status_rules_one_by_one(opsnn):
 
 
 def test_v3_v4_attribute_rules(opsnn):
-    """aclnn_dynamic_quant.cpp:171-189 and the mode-dependent scale shapes :258-284; the modes other than pertoken pass the
-    checks and are then answered with 561002 here (quant/dynamic_quant/tests/ut/op_host/op_api/test_aclnn_dynamic_quant_v3.cpp:71-90
+    """aclnn_dynamic_quant.cpp:171-189 and the mode-dependent scale shapes :258-284; (quant/dynamic_quant/tests/ut/op_host/op_api/test_aclnn_dynamic_quant_v3.cpp:71-90
     is the per-tensor shape of scale and offset)."""
     m = opsnn
     bad, not_run = m.ACLNN_ERR_PARAM_INVALID, 561002
@@ -202,11 +230,12 @@ def test_v3_v4_attribute_rules(opsnn):
     assert _status(m, x, y, sc, quant_mode=b"pertoken", is_symmetrical=False) == bad
     assert _status(m, x, y, sc, quant_mode=b"perrow") == bad
     one = _t(m, (1,), m.ACL_FLOAT)
-    assert _status(m, x, y, one, offset=_t(m, (1,), m.ACL_FLOAT), quant_mode=b"pertensor") == not_run
+    assert _status(m, x, y, one, offset=_t(m, (1,), m.ACL_FLOAT), quant_mode=b"pertensor") == 0
     assert _status(m, x, y, sc, quant_mode=b"pertensor") == bad                                            # scale must be [1]
-    assert _status(m, x, y, _t(m, (32,), m.ACL_FLOAT), quant_mode=b"perchannel") == not_run
+    assert _status(m, x, y, _t(m, (32,), m.ACL_FLOAT), quant_mode=b"perchannel") == 0
     assert _status(m, x, y, sc, quant_mode=b"perchannel") == bad                                           # scale must be [32]
-    assert _status(m, x, y, _t(m, (32,), m.ACL_FLOAT), quant_mode=b"perchannel", smooth=_t(m, (16,), m.ACL_BF16)) == not_run
+    assert _status(m, x, y, _t(m, (32,), m.ACL_FLOAT), quant_mode=b"perchannel", smooth=_t(m, (16,), m.ACL_BF16)) == 0
+    assert _status(m, x, y, one, quant_mode=b"pertensor", smooth=_t(m, (2, 32), m.ACL_BF16), group_index=_t(m, (2,), m.ACL_INT32)) == not_run
     assert _status(m, x, y, _t(m, (32,), m.ACL_FLOAT), quant_mode=b"perchannel", smooth=_t(m, (32,), m.ACL_BF16)) == bad
     assert _status(m, x, y, _t(m, (32,), m.ACL_FLOAT), quant_mode=b"perchannel", smooth=_t(m, (2, 32), m.ACL_BF16),
                    group_index=_t(m, (2,), m.ACL_INT32)) == bad
@@ -345,3 +374,37 @@ def test_gpu_group_index(gpu, shape, ends, gi_dt, symmetric):
     assert np.array_equal(d_s.to_host(np.uint32, shape[:-1]), want[1].view(np.uint32))
     if not symmetric:
         assert np.array_equal(d_o.to_host(np.uint32, shape[:-1]), want[2].view(np.uint32))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("mode,shape", [("pertensor", (16, 32)), ("pertensor", (3, 70, 500)), ("pertensor", (1000, 257)),
+                                        ("perchannel", (16, 32)), ("perchannel", (3, 70, 500)), ("perchannel", (2, 200, 1001)), ("perchannel", (130, 64))])
+@pytest.mark.parametrize("y_dt,symmetric,with_smooth", [(orc.I8, True, False), (orc.I8, False, True), (orc.I4, True, True), (orc.E4M3, True, False)])
+def test_gpu_per_tensor_and_per_channel_modes(gpu, mode, shape, y_dt, symmetric, with_smooth):
+    m = gpu
+    if y_dt == orc.I4 and shape[-1] % 2:
+        pytest.skip("INT4 needs an even last dim")
+    print(f"case dynamic quant {mode} {shape} y={y_dt} symmetric={symmetric} smooth={with_smooth}", flush=True)
+    rng = np.random.default_rng(sum(shape) + y_dt)
+    xb = orc.f32_to_b16(rng.normal(0, 2, size=shape).astype(np.float32), orc.BF16)
+    n_sm = shape[-1] if mode == "pertensor" else shape[-2]
+    smb = orc.f32_to_b16(rng.uniform(0.5, 2.0, n_sm).astype(np.float32), orc.BF16) if with_smooth else None
+    want = orc.dynamic_quant_wide(xb, orc.BF16, y_dt, mode, smooth=smb, symmetric=symmetric)
+    sshape = (1,) if mode == "pertensor" else shape[:-2] + (shape[-1],)
+    nsc = int(np.prod(sshape))
+    d_x, d_sm = m.DeviceBuffer(host=xb), (m.DeviceBuffer(host=smb) if with_smooth else None)
+    d_y, d_s, d_o = m.DeviceBuffer(want[0].nbytes), m.DeviceBuffer(nsc * 4), m.DeviceBuffer(nsc * 4)
+    yt = m.Tensor(shape, m.DTYPE_BY_NAME[ACL_OF[y_dt]], d_y)
+    m.dynamic_quant(m.Tensor(shape, m.ACL_BF16, d_x), yt, m.Tensor(sshape, m.ACL_FLOAT, d_s),
+                    smooth=m.Tensor((n_sm,), m.ACL_BF16, d_sm) if with_smooth else None,
+                    offset=None if symmetric else m.Tensor(sshape, m.ACL_FLOAT, d_o), quant_mode=mode.encode())
+    m.check(m.lib().aclrtSynchronizeDevice(), "sync")
+    assert np.array_equal(d_s.to_host(np.uint32, sshape), want[1].view(np.uint32)), "scale differs"
+    if not symmetric:
+        assert np.array_equal(d_o.to_host(np.uint32, sshape), want[2].view(np.uint32)), "offset differs"
+    gy, wy = d_y.to_host(np.uint8, want[0].shape), want[0]
+    if y_dt == orc.E4M3:
+        z = ((gy | wy) & 0x7f) == 0
+        assert np.array_equal(gy[~z], wy[~z])
+    else:
+        assert np.array_equal(gy, wy), f"{int((gy != wy).sum())} of {wy.size} outputs differ"
