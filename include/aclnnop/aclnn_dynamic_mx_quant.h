@@ -7,9 +7,9 @@
  * aclnnDynamicMxQuant.md:76-95, 99-260, 312-320; arithmetic of quant/dynamic_mx_quant/tests/assets/golden.py:140-330.
  * x: FLOAT16 / BF16, 1 to 7 dims.  yOut: x's shape, FLOAT4_E2M1 (last dim even), FLOAT8_E4M3FN or FLOAT8_E5M2, equal to
  * dstType (40 / 36 / 35).  mxscaleOut: FLOAT8_E8M0, x's shape with the axis dim replaced by ceil(ceil(n / blocksize) / 2) and
- * a trailing dim of 2.  Run here: the last axis, blocksize 32, roundMode NULL or "rint", scaleAlg 0.  What the reference
- * accepts beyond that (another axis, blocksize 64..1024, FLOAT x, FLOAT4_E1M2, "floor" / "round", scaleAlg 1) is answered
- * with ACLNN_ERR_INNER_TILING_ERROR; tensors must be contiguous.
+ * a trailing dim of 2.  Run here: the last axis, every blocksize (a multiple of 32 up to 1024; 32 has the tuned kernel),
+ * roundMode NULL or "rint", scaleAlg 0 and (FLOAT8 outputs) 1.  What the reference accepts beyond that (another axis, FLOAT x,
+ * FLOAT4_E1M2, "floor" / "round") is answered with ACLNN_ERR_INNER_TILING_ERROR; tensors must be contiguous.
  */
 #ifndef OPSNN_AMD_ACLNN_DYNAMIC_MX_QUANT_H_
 #define OPSNN_AMD_ACLNN_DYNAMIC_MX_QUANT_H_

@@ -185,17 +185,19 @@ typedef struct {
 } OpsnnBlockQuantArgs;
 OPSNN_API int opsnnDynamicBlockQuant(const OpsnnBlockQuantArgs* a, void* stream);
 
-/* Dynamic MX quantisation of x [rows, cols] (FLOAT16 / BF16, dense) along the columns in blocks of 32: y in FLOAT4_E2M1
+/* Dynamic MX quantisation of x [rows, cols] (FLOAT16 / BF16, dense) along the columns in blocks of `block` (32 by default): y in FLOAT4_E2M1
  * (two per byte, even column in the low nibble; cols even), FLOAT8_E4M3FN or FLOAT8_E5M2, and one FLOAT8_E8M0 scale per
  * block, scale [rows, 2 * ceil(ceil(cols / 32) / 2)] (rows padded to an even number of bytes with 0).  Formula:
  * quant/dynamic_mx_quant/tests/assets/golden.py:140-153, 196-218, 263-330 (round mode "rint", scale algorithm 0).
- * force_variant: 0 automatic, 1 the lane-group kernel (cols % 8 == 0), 2 the one-thread-per-block kernel. */
+ * force_variant: 0 automatic, 1 the lane-group kernel (block 32, cols % 8 == 0), 2 the one-thread-per-block kernel. */
 typedef struct {
     const void* x; int x_dtype;
     void* y; int y_dtype;
     void* scale;
     int64_t rows, cols;
     int force_variant;
+    int64_t block;    /* elements per scale block: a multiple of 32 up to 1024; 0 means 32 */
+    int scale_alg;    /* 0: scale 2^(floor(log2 max) - emax); 1 (fp8 outputs only): max / typeMax rounded up to a power of two */
 } OpsnnMxQuantArgs;
 OPSNN_API int opsnnDynamicMxQuant(const OpsnnMxQuantArgs* a, void* stream);
 

@@ -62,10 +62,9 @@ aclnnStatus aclnnDynamicMxQuantGetWorkspaceSize(const aclTensor* x_, int64_t axi
     if (sc.shape != want) INVALID("%s: mxscaleOut %s must be %s", kApi, shape_str(sc.shape).c_str(), shape_str(want).c_str());
     // what this build does not run
     if (ax != x.rank() - 1) NOT_RUN("%s: only the last axis has a kernel here", kApi);
-    if (blocksize != 32) NOT_RUN("%s: only blocksize 32 has a kernel here", kApi);
     if (x.dtype == ACL_FLOAT) NOT_RUN("%s: a FLOAT x has no kernel here", kApi);
     if (y.dtype == ACL_FLOAT4_E1M2) NOT_RUN("%s: FLOAT4_E1M2 has no kernel here", kApi);
-    if (std::strcmp(mode, "rint") != 0 || scaleAlg != 0) NOT_RUN("%s: only roundMode rint with scaleAlg 0 has a kernel here", kApi);
+    if (std::strcmp(mode, "rint") != 0) NOT_RUN("%s: only roundMode rint has a kernel here", kApi);
     if (!is_contiguous(x) || !is_contiguous(y) || !is_contiguous(sc)) INVALID("%s: tensors must be contiguous here", kApi);
 
     std::unique_ptr<aclOpExecutor> ex(new (std::nothrow) aclOpExecutor());
@@ -83,6 +82,7 @@ aclnnStatus aclnnDynamicMxQuantGetWorkspaceSize(const aclTensor* x_, int64_t axi
     a.y = const_cast<void*>(y.ptr_at(0)); a.y_dtype = y.dtype;
     a.scale = const_cast<void*>(sc.ptr_at(0));
     a.cols = x.dim(-1); a.rows = x.numel() / a.cols; a.force_variant = 0;
+    a.block = blocksize; a.scale_alg = (int)scaleAlg;
     *executor = ex.release();
     return ACLNN_SUCCESS;
 }

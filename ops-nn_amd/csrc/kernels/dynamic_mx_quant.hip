@@ -16,6 +16,8 @@ namespace opsnn {
 struct MxQuantParams {
     const uint16_t* x; uint8_t* y; uint8_t* scale;
     int64_t rows, cols, nblk, spitch;
+    int block;       // elements per scale block (32 on the lane-group kernel)
+    int scale_alg;   // 0: floor(log2 max) - emax;  1 (fp8 elements): exponent of max / tmax, rounded up when it has mantissa bits
 };
 
 template <int X_DT>
@@ -33,8 +35,16 @@ template <> struct MxFormat<DT_E5M2> { static constexpr int emax = 15; static co
 // Shared exponent of a block from the bits of its largest magnitude (a finite, non-negative fp32).  floor(log2) of a
 // normal fp32 is its exponent field; a zero or subnormal maximum lands below the floor of -127 in any case.
 template <int Y_DT>
-__device__ __forceinline__ int mx_share_exp(float amax)
+__device__ __forceinline__ int mx_share_exp(float amax, int alg = 0)
 {
+    if (alg == 1) {   // golden.py:156-176: the scale is max / tmax rounded up to a power of two
+        if (amax == 0.0f) return -127;
+        const uint32_t u = f2u(__fdiv_rn(amax, MxFormat<Y_DT>::tmax));
+        int e = (int)(u >> 23);
+        const uint32_t mant = u & 0x7fffffu;
+        if ((e > 0 && e < 254 && mant > 0) || (e == 0 && mant > 0x400000u)) e += 1;
+        return e - 127;
+    }
     const int e = (int)(f2u(amax) >> 23);
     const int s = e - 127 - MxFormat<Y_DT>::emax;
     return (e == 0 || s < -127) ? -127 : s;
@@ -125,7 +135,7 @@ __global__ __launch_bounds__(256) void mx_quant_kernel(MxQuantParams p, int64_t 
         amax = fmaxf(amax, __shfl_xor(amax, 2));
         bad |= (bool)__shfl_xor((int)bad, 1);
         bad |= (bool)__shfl_xor((int)bad, 2);
-        const int share = bad ? 0 : mx_share_exp<Y_DT>(amax);
+        const int share = bad ? 0 : mx_share_exp<Y_DT>(amax, p.scale_alg);
         if (sidx[i] >= 0 && lane == 0) {
             p.scale[sidx[i]] = bad ? 0xFFu : (uint8_t)(share + 127);
             if (pad_after[i]) p.scale[sidx[i] + 1] = 0;
@@ -142,14 +152,14 @@ __global__ __launch_bounds__(256) void mx_quant_kernel(MxQuantParams p, int64_t 
     }
 }
 
-// any row length: one thread per block of 32
+// any row length and block size: one thread per block
 template <int X_DT, int Y_DT>
 __global__ __launch_bounds__(256) void mx_quant_generic_kernel(MxQuantParams p)
 {
     const int64_t g = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (g >= p.rows * p.nblk) return;
     const int64_t row = g / p.nblk, blk = g % p.nblk;
-    const int64_t c0 = blk * 32, c1 = c0 + 32 < p.cols ? c0 + 32 : p.cols;
+    const int64_t c0 = blk * p.block, c1 = c0 + p.block < p.cols ? c0 + p.block : p.cols;
     const uint16_t* xr = p.x + row * p.cols;
     float amax = 0.0f;
     bool bad = false;
@@ -158,7 +168,7 @@ __global__ __launch_bounds__(256) void mx_quant_generic_kernel(MxQuantParams p)
         bad |= !(a < __builtin_inff());
         amax = fmaxf(amax, a);
     }
-    const int share = bad ? 0 : mx_share_exp<Y_DT>(amax);
+    const int share = bad ? 0 : mx_share_exp<Y_DT>(amax, p.scale_alg);
     p.scale[row * p.spitch + blk] = bad ? 0xFFu : (uint8_t)(share + 127);
     if (blk == p.nblk - 1 && (p.nblk & 1)) p.scale[row * p.spitch + blk + 1] = 0;
     const float inv_scale = u2f((uint32_t)(127 - share) << 23);
@@ -179,7 +189,7 @@ __global__ __launch_bounds__(256) void mx_quant_generic_kernel(MxQuantParams p)
 template <int X_DT, int Y_DT>
 static int launch_mx_quant(const MxQuantParams& p, int variant, hipStream_t st)
 {
-    const bool vec = p.cols % 8 == 0 && (uintptr_t)p.x % 16 == 0 && (uintptr_t)p.y % 8 == 0;
+    const bool vec = p.block == 32 && p.cols % 8 == 0 && (uintptr_t)p.x % 16 == 0 && (uintptr_t)p.y % 8 == 0;
     const int64_t groups = p.rows * p.nblk;
     if (variant != 2 && vec) {
         // four pairs per group once that still leaves every SIMD eight waves
@@ -220,7 +230,10 @@ extern "C" int opsnnDynamicMxQuant(const OpsnnMxQuantArgs* a, void* stream)
     if (a->y_dtype == DT_E2M1 && (a->cols & 1)) return -2;
     MxQuantParams p{};
     p.x = (const uint16_t*)a->x; p.y = (uint8_t*)a->y; p.scale = (uint8_t*)a->scale;
-    p.rows = a->rows; p.cols = a->cols; p.nblk = (a->cols + 31) / 32; p.spitch = (p.nblk + 1) / 2 * 2;
+    p.block = a->block ? (int)a->block : 32;
+    p.scale_alg = a->scale_alg;
+    if (p.block <= 0 || p.block % 32 != 0 || p.block > 1024 || (p.scale_alg != 0 && (p.scale_alg != 1 || a->y_dtype == DT_E2M1))) return -2;
+    p.rows = a->rows; p.cols = a->cols; p.nblk = (a->cols + p.block - 1) / p.block; p.spitch = (p.nblk + 1) / 2 * 2;
     if (a->x_dtype == DT_BF16) return launch_mx_quant_x<DT_BF16>(p, a->y_dtype, a->force_variant, (hipStream_t)stream);
     return launch_mx_quant_x<DT_F16>(p, a->y_dtype, a->force_variant, (hipStream_t)stream);
 }

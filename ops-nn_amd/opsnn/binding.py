@@ -93,6 +93,7 @@ class OpsnnMxQuantArgs(C.Structure):
         ("scale", C.c_void_p),
         ("rows", C.c_int64), ("cols", C.c_int64),
         ("force_variant", C.c_int),
+        ("block", C.c_int64), ("scale_alg", C.c_int),
     ]
 
 

@@ -55,7 +55,8 @@
  *   orc_dynamic_mx_quant pinned (the OCP MX definition: shared exponent = floor(log2 max) - emax and round-to-nearest-even
  *                       onto the element grid with saturation, recomputed in numpy with torch's fp8 casts and a brute-force
  *                       nearest-grid-point search for e2m1; known answers for ties, saturation and the scale bytes; dequantised
- *                       values within half a grid step)
+ *                       values within half a grid step; scale algorithm 1 by its defining property, the smallest power of two
+ *                       under which no element saturates; larger blocks by monotonicity against blocks of 32)
  *   orc_trans_quant_param pinned (the packing utility of the matmul golden and the reference's system-test formula in numpy;
  *                       its inverse orc_u64_to_deq_scale; hand-derived cases of the rounding mode: ties, carry into the
  *                       exponent, overflow to infinity, subnormal)
@@ -966,7 +967,16 @@ static uint8_t e2m1_code_of(float v)   /* v on the e2m1 grid */
     for (uint8_t i = 0; i < 8; i++) if (kE2M1[i] == a) c = i;
     return (uint8_t)(c | (signbit(v) ? 8u : 0u));
 }
+int orc_dynamic_mx_quant_alg(const void* x, int x_dt, int64_t rows, int64_t cols, int64_t block, int scale_alg, int y_dt, uint8_t* y,
+                             uint8_t* scale_out);
 int orc_dynamic_mx_quant(const void* x, int x_dt, int64_t rows, int64_t cols, int64_t block, int y_dt, uint8_t* y, uint8_t* scale_out)
+{
+    return orc_dynamic_mx_quant_alg(x, x_dt, rows, cols, block, 0, y_dt, y, scale_out);
+}
+/* scale_alg 1 (GD:156-176, fp8 elements only): share_exp is the exponent field of fp32(amax / tmax) minus 127, plus one when that
+ * quotient is not a power of two (a normal number with mantissa bits, or a subnormal above 2^-127); the elements follow as before. */
+int orc_dynamic_mx_quant_alg(const void* x, int x_dt, int64_t rows, int64_t cols, int64_t block, int scale_alg, int y_dt, uint8_t* y,
+                             uint8_t* scale_out)
 {
     int emax, emin, mbits; float tmax;
     switch (y_dt) {
@@ -976,6 +986,7 @@ int orc_dynamic_mx_quant(const void* x, int x_dt, int64_t rows, int64_t cols, in
         default: return -1;
     }
     if ((x_dt != ORC_F16 && x_dt != ORC_BF16) || rows <= 0 || cols <= 0 || block <= 0 || (y_dt == ORC_E2M1 && (cols & 1))) return -1;
+    if (scale_alg != 0 && (scale_alg != 1 || y_dt == ORC_E2M1)) return -1;
     const int64_t nblk = (cols + block - 1) / block, spitch = (nblk + 1) / 2 * 2;
     for (int64_t r = 0; r < rows; r++) {
         for (int64_t b = 0; b < spitch; b++) scale_out[r * spitch + b] = 0;
@@ -990,6 +1001,16 @@ int orc_dynamic_mx_quant(const void* x, int x_dt, int64_t rows, int64_t cols, in
             float share;   /* an integer, or NaN */
             if (has_nan) share = NAN;
             else if (amax == 0.0f) share = -127.0f;
+            else if (scale_alg == 1) {
+                if (isinf(amax)) share = NAN;
+                else {
+                    const uint32_t u = f2u(amax / tmax);
+                    int e = (int)(u >> 23);
+                    const uint32_t mant = u & 0x7fffffu;
+                    if ((e > 0 && e < 254 && mant > 0) || (e == 0 && mant > (1u << 22))) e += 1;
+                    share = (float)(e - 127);
+                }
+            }
             else {
                 share = floorf(log2f(amax)) - (float)emax;
                 if (share > 127.0f) share = NAN;

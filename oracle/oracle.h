@@ -73,6 +73,8 @@ int orc_dynamic_block_quant(const void* x, int x_dt, int64_t batch, int64_t rows
                             double min_scale, int y_dt, uint8_t* y, float* scale_out);
 int orc_dynamic_mx_quant(const void* x, int x_dt, int64_t rows, int64_t cols, int64_t block, int y_dt, uint8_t* y, uint8_t* scale_out);
 void orc_trans_quant_param(const float* scale, int64_t scale_len, const float* offset, int64_t offset_len, int round_mode, uint64_t* out);
+int orc_dynamic_mx_quant_alg(const void* x, int x_dt, int64_t rows, int64_t cols, int64_t block, int scale_alg, int y_dt, uint8_t* y,
+                             uint8_t* scale_out);
 int orc_wqbmm(const void* x, int x_dt, const void* w, int w_dt, int64_t M, int64_t K, int64_t N, int tW,
               const void* scale, int scale_dt, int64_t scale_n, const void* offset, int64_t group,
               const void* bias, int bias_dt, void* y);

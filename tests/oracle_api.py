@@ -50,6 +50,8 @@ def lib():
         L.orc_e5m2_from_f32.restype = C.c_uint8
         L.orc_dynamic_block_quant.argtypes = [vp, C.c_int, i64, i64, i64, i64, i64, C.c_double, C.c_int, vp, vp]
         L.orc_dynamic_block_quant.restype = C.c_int
+        L.orc_dynamic_mx_quant_alg.argtypes = [vp, C.c_int, i64, i64, i64, C.c_int, C.c_int, vp, vp]
+        L.orc_dynamic_mx_quant_alg.restype = C.c_int
         L.orc_dynamic_mx_quant.argtypes = [vp, C.c_int, i64, i64, i64, C.c_int, vp, vp]
         L.orc_dynamic_mx_quant.restype = C.c_int
         L.orc_trans_quant_param.argtypes = [vp, i64, vp, i64, C.c_int, vp]
@@ -121,7 +123,7 @@ def dynamic_block_quant(x, x_dt, y_dt, rb, cb, min_scale=0.0):
     return y, scale
 
 
-def dynamic_mx_quant(x, x_dt, y_dt, block=32):
+def dynamic_mx_quant(x, x_dt, y_dt, block=32, scale_alg=0):
     """x: uint16 bits [..., cols].  Returns (y bytes [..., cols] or [..., cols / 2] for e2m1, e8m0 bytes [..., ceil(nblk / 2), 2])."""
     x = np.ascontiguousarray(x, np.uint16)
     cols = x.shape[-1]
@@ -129,7 +131,7 @@ def dynamic_mx_quant(x, x_dt, y_dt, block=32):
     nblk = -(-cols // block)
     y = np.zeros(x.shape[:-1] + ((cols // 2) if y_dt == E2M1 else cols,), np.uint8)
     scale = np.zeros(x.shape[:-1] + ((nblk + 1) // 2, 2), np.uint8)
-    rc = lib().orc_dynamic_mx_quant(x.ctypes.data, x_dt, rows, cols, block, y_dt, y.ctypes.data, scale.ctypes.data)
+    rc = lib().orc_dynamic_mx_quant_alg(x.ctypes.data, x_dt, rows, cols, block, scale_alg, y_dt, y.ctypes.data, scale.ctypes.data)
     assert rc == 0, rc
     return y, scale
 

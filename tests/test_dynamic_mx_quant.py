@@ -83,6 +83,39 @@ def test_known_answers():
     assert y[1, 40] == orc.f32_to_e4m3(np.float32([3.0 * 2.0 ** 7]))[0]
 
 
+def test_larger_blocks_take_the_larger_scale():
+    """floor(log2 max) is monotone: a block of 64 has the larger of the scale bytes of its two halves, and the half that had
+    that byte keeps its element codes."""
+    rng = np.random.default_rng(4)
+    xf = (rng.normal(0, 1, size=(32, 256)) * 2.0 ** rng.integers(-6, 6, size=(32, 8)).repeat(32, axis=1)).astype(np.float32)
+    xb = orc.f32_to_bf16(xf)
+    y32, s32 = orc.dynamic_mx_quant(xb, orc.BF16, orc.E4M3, block=32)
+    y64, s64 = orc.dynamic_mx_quant(xb, orc.BF16, orc.E4M3, block=64)
+    b32 = s32.reshape(32, 8)
+    assert s64.shape == (32, 2, 2) and np.array_equal(s64.reshape(32, 4), np.maximum(b32[:, 0::2], b32[:, 1::2]))
+    same = np.repeat(b32 == np.repeat(s64.reshape(32, 4), 2, axis=1), 32, axis=1)
+    assert same.any() and np.array_equal(y32[same], y64[same])
+
+
+def test_scale_algorithm_1_is_the_smallest_power_of_two_that_avoids_saturation():
+    """max / 448 rounded up to a power of two: every scaled element fits (no code reaches beyond 448 and the block maximum is
+    above 224 unless max / 448 is itself a power of two), and half the scale would not fit."""
+    rng = np.random.default_rng(5)
+    xf = (rng.normal(0, 1, size=(64, 128)) * 2.0 ** rng.integers(-10, 10, size=(64, 4)).repeat(32, axis=1)).astype(np.float32)
+    xf[0, :32] = 0.0
+    xf[1, :32] = 448.0 * 2.0 ** -3 * np.linspace(0, 1, 32)        # max / 448 is exactly a power of two: not rounded up
+    xb = orc.f32_to_bf16(xf)
+    xf = orc.b16_to_f32(xb, orc.BF16).astype(np.float64)
+    y, s = orc.dynamic_mx_quant(xb, orc.BF16, orc.E4M3, scale_alg=1)
+    scale = 2.0 ** (s.reshape(64, 4).astype(np.float64) - 127)
+    amax = np.abs(xf).reshape(64, 4, 32).max(axis=-1)
+    assert s.reshape(64, 4)[0, 0] == 0 and s.reshape(64, 4)[1, 0] == 127 - 3
+    nz = amax > 0
+    assert (amax[nz] <= 448.0 * scale[nz]).all() and (amax[nz] > 448.0 * scale[nz] / 2).all()
+    deq = orc.e4m3_to_f32(y).astype(np.float64) * np.repeat(scale, 32, axis=1)
+    assert (np.abs(deq - xf) <= np.maximum(np.abs(xf) * 2.0 ** -4, 2.0 ** -10 * np.repeat(scale, 32, axis=1))).all()   # never saturates
+
+
 def test_dequantised_values_are_within_half_a_grid_step():
     """Relative 2^-4 (half a step of three mantissa bits), or 2^-3 where the block maximum saturates: a block maximum in
     (448, 512) * scale comes back as 448 * scale."""
@@ -129,27 +162,29 @@ def test_status_rules(opsnn):
     assert _status(m, x, y, _t(m, (4, 6, 10), e8)) == bad and _status(m, x, y, _t(m, (4, 6, 6, 2), e8)) == bad
     # accepted by the reference, no kernel here
     assert _status(m, x, y, _t(m, (4, 1, 320, 2), e8), axis=1) == not_run
-    assert _status(m, x, y, _t(m, (4, 6, 3, 2), e8), blocksize=64) == not_run
+    assert _status(m, x, y, _t(m, (4, 6, 3, 2), e8), blocksize=64) == 0
+    assert _status(m, x, y, _t(m, (4, 6, 1, 2), e8), blocksize=1024) == 0
     assert _status(m, _t(m, (4, 6, 320), m.ACL_FLOAT), y, sc) == not_run
     assert _status(m, x, _t(m, (4, 6, 320), m.ACL_FLOAT4_E1M2), sc) == not_run
     assert _status(m, x, _t(m, (4, 6, 320), f4), sc, round_mode=b"floor") == not_run
-    assert _status(m, x, y, sc, scale_alg=1) == not_run
+    assert _status(m, x, y, sc, scale_alg=1) == 0
 
 
 # --------------------------------------------------------------------------------------------------- device parity
 ACL_OF = {orc.E2M1: "ACL_FLOAT4_E2M1", orc.E4M3: "ACL_FLOAT8_E4M3FN", orc.E5M2: "ACL_FLOAT8_E5M2"}
 
 
-def _run(m, xb, x_dt, y_dt):
+def _run(m, xb, x_dt, y_dt, block=32, scale_alg=0):
     cols = xb.shape[-1]
-    nblk = -(-cols // 32)
+    nblk = -(-cols // block)
     ybytes = xb.size // 2 if y_dt == orc.E2M1 else xb.size
     sbytes = xb.size // cols * ((nblk + 1) // 2) * 2
     d_x, d_y, d_s = m.DeviceBuffer(host=xb), m.DeviceBuffer(ybytes + 16), m.DeviceBuffer(sbytes + 16)
     d_y.fill(0xEE); d_s.fill(0xEE)
     adt = m.ACL_FLOAT16 if x_dt == orc.F16 else m.ACL_BF16
     sshape = xb.shape[:-1] + ((nblk + 1) // 2, 2)
-    m.dynamic_mx_quant(m.Tensor(xb.shape, adt, d_x), m.Tensor(xb.shape, m.DTYPE_BY_NAME[ACL_OF[y_dt]], d_y), m.Tensor(sshape, m.ACL_FLOAT8_E8M0, d_s))
+    m.dynamic_mx_quant(m.Tensor(xb.shape, adt, d_x), m.Tensor(xb.shape, m.DTYPE_BY_NAME[ACL_OF[y_dt]], d_y), m.Tensor(sshape, m.ACL_FLOAT8_E8M0, d_s),
+                       blocksize=block, scale_alg=scale_alg)
     m.check(m.lib().aclrtSynchronizeDevice(), "sync")
     gy, gs = d_y.to_host(np.uint8, (ybytes + 16,)), d_s.to_host(np.uint8, (sbytes + 16,))
     assert (gy[ybytes:] == 0xEE).all() and (gs[sbytes:] == 0xEE).all(), "wrote past an output"
@@ -201,3 +236,20 @@ def test_gpu_mx_quantised_operands_feed_the_mx_matmul(gpu, fp4):
     g, w = orc.b16_to_f32(got, orc.BF16), orc.b16_to_f32(want, orc.BF16)
     mx, mean = orc.rel_err_stats(g, w)
     assert mx <= 2.0 ** -7 and mean <= 2.0 ** -10, f"max rel {mx:.3e} mean rel {mean:.3e}"
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("shape,block,alg,y_dt", [((33, 1024), 64, 0, orc.E2M1), ((7, 1000), 128, 0, orc.E4M3), ((5, 4096), 1024, 0, orc.E5M2),
+                                                  ((33, 1024), 32, 1, orc.E4M3), ((6, 1000), 32, 1, orc.E5M2), ((9, 520), 256, 1, orc.E4M3)])
+def test_gpu_block_sizes_and_scale_algorithm_1(gpu, shape, block, alg, y_dt):
+    m = gpu
+    print(f"case mx quant {shape} block={block} scale_alg={alg} y={y_dt}", flush=True)
+    rng = np.random.default_rng(sum(shape) + block + alg)
+    xf = (rng.normal(0, 1, size=shape) * 2.0 ** rng.integers(-14, 14, size=shape[:-1] + (1,))).astype(np.float32)
+    xf.reshape(-1)[:40] = 0.0
+    xf.reshape(-1)[-1] = np.inf
+    xb = orc.f32_to_b16(xf, orc.BF16)
+    want_y, want_s = orc.dynamic_mx_quant(xb, orc.BF16, y_dt, block=block, scale_alg=alg)
+    gy, gs = _run(m, xb, orc.BF16, y_dt, block=block, scale_alg=alg)
+    assert np.array_equal(gs, want_s), "scale bytes differ"
+    assert _same_but_zero_sign(_codes(gy, y_dt), _codes(want_y.reshape(-1), y_dt), y_dt)
