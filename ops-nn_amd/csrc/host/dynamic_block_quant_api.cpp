@@ -9,6 +9,7 @@
 #include <memory>
 
 #include "aclnnop/aclnn_dynamic_block_quant.h"
+#include "aclnnop/aclnn_dynamic_block_quant_v2.h"
 #include "tensor.h"
 
 using namespace opsnn;
@@ -72,6 +73,26 @@ aclnnStatus aclnnDynamicBlockQuantGetWorkspaceSize(const aclTensor* x_, double m
     *workspaceSize = 0;
     *executor = ex.release();
     return ACLNN_SUCCESS;
+}
+
+aclnnStatus aclnnDynamicBlockQuantV2GetWorkspaceSize(const aclTensor* x, double minScale, char* roundModeOptional, int64_t dstType,
+                                                     int64_t rowBlockSize, int64_t colBlockSize, double dstTypeMax, const aclTensor* yOut,
+                                                     const aclTensor* scaleOut, uint64_t* workspaceSize, aclOpExecutor** executor)
+{
+    const aclnnStatus rc = aclnnDynamicBlockQuantGetWorkspaceSize(x, minScale, roundModeOptional, dstType, rowBlockSize, colBlockSize, yOut,
+                                                                  scaleOut, workspaceSize, executor);
+    if (rc != ACLNN_SUCCESS) return rc;
+    if (dstTypeMax != 0.0) {   // a custom maximum belongs to the HIFLOAT8 output of the reference; the fp8 formulas do not use it
+        aclDestroyAclOpExecutor(*executor);
+        *executor = nullptr;
+        FAIL(ACLNN_ERR_INNER_TILING_ERROR, "aclnnDynamicBlockQuantV2: a dstTypeMax other than 0 has no kernel here");
+    }
+    return ACLNN_SUCCESS;
+}
+
+aclnnStatus aclnnDynamicBlockQuantV2(void* workspace, uint64_t workspaceSize, aclOpExecutor* executor, aclrtStream stream)
+{
+    return aclnnDynamicBlockQuant(workspace, workspaceSize, executor, stream);
 }
 
 aclnnStatus aclnnDynamicBlockQuant(void*, uint64_t, aclOpExecutor* executor, aclrtStream stream)

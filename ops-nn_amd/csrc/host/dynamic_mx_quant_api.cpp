@@ -9,6 +9,8 @@
 #include <memory>
 
 #include "aclnnop/aclnn_dynamic_mx_quant.h"
+#include "aclnnop/aclnn_dynamic_mx_quant_v2.h"
+#include "aclnnop/aclnn_dynamic_mx_quant_v3.h"
 #include "tensor.h"
 
 using namespace opsnn;
@@ -86,6 +88,41 @@ aclnnStatus aclnnDynamicMxQuantGetWorkspaceSize(const aclTensor* x_, int64_t axi
     *executor = ex.release();
     return ACLNN_SUCCESS;
 }
+
+// V2 adds dstTypeMax, V3 maxLowBound (a lower clamp of the block maximum): both belong to scale algorithms and type maxima
+// that have no kernel here; with both at 0 the call is the first version's.
+static aclnnStatus mx_quant_later_version(const char* api, const aclTensor* x, int64_t axis, char* roundModeOptional, int64_t dstType,
+                                          int64_t blocksize, int64_t scaleAlg, double dstTypeMax, double maxLowBound, const aclTensor* yOut,
+                                          const aclTensor* mxscaleOut, uint64_t* workspaceSize, aclOpExecutor** executor)
+{
+    if (scaleAlg == 2 && x && yOut && mxscaleOut && workspaceSize && executor) NOT_RUN("%s: scaleAlg 2 has no kernel here", api);
+    const aclnnStatus rc = aclnnDynamicMxQuantGetWorkspaceSize(x, axis, roundModeOptional, dstType, blocksize, scaleAlg, yOut, mxscaleOut,
+                                                               workspaceSize, executor);
+    if (rc != ACLNN_SUCCESS) return rc;
+    if (dstTypeMax != 0.0 || maxLowBound != 0.0) {
+        aclDestroyAclOpExecutor(*executor);
+        *executor = nullptr;
+        NOT_RUN("%s: dstTypeMax / maxLowBound other than 0 have no kernel here", api);
+    }
+    return ACLNN_SUCCESS;
+}
+
+aclnnStatus aclnnDynamicMxQuantV2GetWorkspaceSize(const aclTensor* x, int64_t axis, char* roundModeOptional, int64_t dstType, int64_t blocksize,
+                                                  int64_t scaleAlg, double dstTypeMax, const aclTensor* yOut, const aclTensor* mxscaleOut,
+                                                  uint64_t* workspaceSize, aclOpExecutor** executor)
+{
+    return mx_quant_later_version("aclnnDynamicMxQuantV2", x, axis, roundModeOptional, dstType, blocksize, scaleAlg, dstTypeMax, 0.0, yOut,
+                                  mxscaleOut, workspaceSize, executor);
+}
+aclnnStatus aclnnDynamicMxQuantV3GetWorkspaceSize(const aclTensor* x, int64_t axis, char* roundModeOptional, int64_t dstType, int64_t blocksize,
+                                                  int64_t scaleAlg, double dstTypeMax, double maxLowBound, const aclTensor* yOut,
+                                                  const aclTensor* mxscaleOut, uint64_t* workspaceSize, aclOpExecutor** executor)
+{
+    return mx_quant_later_version("aclnnDynamicMxQuantV3", x, axis, roundModeOptional, dstType, blocksize, scaleAlg, dstTypeMax, maxLowBound, yOut,
+                                  mxscaleOut, workspaceSize, executor);
+}
+aclnnStatus aclnnDynamicMxQuantV2(void* ws, uint64_t n, aclOpExecutor* executor, aclrtStream stream) { return aclnnDynamicMxQuant(ws, n, executor, stream); }
+aclnnStatus aclnnDynamicMxQuantV3(void* ws, uint64_t n, aclOpExecutor* executor, aclrtStream stream) { return aclnnDynamicMxQuant(ws, n, executor, stream); }
 
 aclnnStatus aclnnDynamicMxQuant(void*, uint64_t, aclOpExecutor* executor, aclrtStream stream)
 {

@@ -151,10 +151,19 @@ _SIGS = {
     "aclnnDynamicBlockQuantGetWorkspaceSize": (C.c_int32, [_T, C.c_double, C.c_char_p, C.c_int64, C.c_int64, C.c_int64, _T, _T,
                                                           C.POINTER(C.c_uint64), C.POINTER(C.c_void_p)]),
     "aclnnDynamicBlockQuant": (C.c_int32, [C.c_void_p, C.c_uint64, C.c_void_p, C.c_void_p]),
+    "aclnnDynamicBlockQuantV2GetWorkspaceSize": (C.c_int32, [_T, C.c_double, C.c_char_p, C.c_int64, C.c_int64, C.c_int64, C.c_double, _T, _T,
+                                                            C.POINTER(C.c_uint64), C.POINTER(C.c_void_p)]),
+    "aclnnDynamicBlockQuantV2": (C.c_int32, [C.c_void_p, C.c_uint64, C.c_void_p, C.c_void_p]),
     "opsnnDynamicBlockQuant": (C.c_int, [C.POINTER(OpsnnBlockQuantArgs), C.c_void_p]),
     "aclnnDynamicMxQuantGetWorkspaceSize": (C.c_int32, [_T, C.c_int64, C.c_char_p, C.c_int64, C.c_int64, C.c_int64, _T, _T,
                                                        C.POINTER(C.c_uint64), C.POINTER(C.c_void_p)]),
     "aclnnDynamicMxQuant": (C.c_int32, [C.c_void_p, C.c_uint64, C.c_void_p, C.c_void_p]),
+    "aclnnDynamicMxQuantV2GetWorkspaceSize": (C.c_int32, [_T, C.c_int64, C.c_char_p, C.c_int64, C.c_int64, C.c_int64, C.c_double, _T, _T,
+                                                         C.POINTER(C.c_uint64), C.POINTER(C.c_void_p)]),
+    "aclnnDynamicMxQuantV2": (C.c_int32, [C.c_void_p, C.c_uint64, C.c_void_p, C.c_void_p]),
+    "aclnnDynamicMxQuantV3GetWorkspaceSize": (C.c_int32, [_T, C.c_int64, C.c_char_p, C.c_int64, C.c_int64, C.c_int64, C.c_double, C.c_double, _T, _T,
+                                                         C.POINTER(C.c_uint64), C.POINTER(C.c_void_p)]),
+    "aclnnDynamicMxQuantV3": (C.c_int32, [C.c_void_p, C.c_uint64, C.c_void_p, C.c_void_p]),
     "opsnnDynamicMxQuant": (C.c_int, [C.POINTER(OpsnnMxQuantArgs), C.c_void_p]),
     "aclnnTransQuantParamV2GetWorkspaceSize": (C.c_int32, [_T, _T, _T, C.POINTER(C.c_uint64), C.POINTER(C.c_void_p)]),
     "aclnnTransQuantParamV2": (C.c_int32, [C.c_void_p, C.c_uint64, C.c_void_p, C.c_void_p]),
@@ -389,9 +398,14 @@ def dynamic_quant(x, y, scale, stream=None, **kw):
     check(run(None, ws, ex, stream.ptr if stream else None), "aclnnDynamicQuant")
 
 
-def dynamic_block_quant_get_workspace(x, y, scale, *, dst_type=None, row_block=1, col_block=128, min_scale=0.0, round_mode=b"rint"):
+def dynamic_block_quant_get_workspace(x, y, scale, *, dst_type=None, row_block=1, col_block=128, min_scale=0.0, round_mode=b"rint",
+                                      dst_type_max=None):
     ws, ex = C.c_uint64(0), C.c_void_p()
     dst = dst_type if dst_type is not None else (y.dtype if y is not None else 36)
+    if dst_type_max is not None:   # V2
+        rc = lib().aclnnDynamicBlockQuantV2GetWorkspaceSize(_h(x), min_scale, round_mode, dst, row_block, col_block, dst_type_max, _h(y),
+                                                            _h(scale), C.byref(ws), C.byref(ex))
+        return rc, ws.value, ex.value
     rc = lib().aclnnDynamicBlockQuantGetWorkspaceSize(_h(x), min_scale, round_mode, dst, row_block, col_block, _h(y), _h(scale),
                                                       C.byref(ws), C.byref(ex))
     return rc, ws.value, ex.value
@@ -400,12 +414,23 @@ def dynamic_block_quant_get_workspace(x, y, scale, *, dst_type=None, row_block=1
 def dynamic_block_quant(x, y, scale, stream=None, **kw):
     rc, ws, ex = dynamic_block_quant_get_workspace(x, y, scale, **kw)
     check(rc, "aclnnDynamicBlockQuantGetWorkspaceSize")
-    check(lib().aclnnDynamicBlockQuant(None, ws, ex, stream.ptr if stream else None), "aclnnDynamicBlockQuant")
+    run = lib().aclnnDynamicBlockQuantV2 if kw.get("dst_type_max") is not None else lib().aclnnDynamicBlockQuant
+    check(run(None, ws, ex, stream.ptr if stream else None), "aclnnDynamicBlockQuant")
 
 
-def dynamic_mx_quant_get_workspace(x, y, scale, *, axis=-1, round_mode=b"rint", dst_type=None, blocksize=32, scale_alg=0):
+def dynamic_mx_quant_get_workspace(x, y, scale, *, axis=-1, round_mode=b"rint", dst_type=None, blocksize=32, scale_alg=0, dst_type_max=None,
+                                   max_low_bound=None):
+    """aclnnDynamicMxQuant; V2 when dst_type_max is given, V3 when max_low_bound is given too."""
     ws, ex = C.c_uint64(0), C.c_void_p()
     dst = dst_type if dst_type is not None else (y.dtype if y is not None else 40)
+    if max_low_bound is not None:
+        rc = lib().aclnnDynamicMxQuantV3GetWorkspaceSize(_h(x), axis, round_mode, dst, blocksize, scale_alg, dst_type_max or 0.0, max_low_bound,
+                                                         _h(y), _h(scale), C.byref(ws), C.byref(ex))
+        return rc, ws.value, ex.value
+    if dst_type_max is not None:
+        rc = lib().aclnnDynamicMxQuantV2GetWorkspaceSize(_h(x), axis, round_mode, dst, blocksize, scale_alg, dst_type_max, _h(y), _h(scale),
+                                                         C.byref(ws), C.byref(ex))
+        return rc, ws.value, ex.value
     rc = lib().aclnnDynamicMxQuantGetWorkspaceSize(_h(x), axis, round_mode, dst, blocksize, scale_alg, _h(y), _h(scale),
                                                    C.byref(ws), C.byref(ex))
     return rc, ws.value, ex.value
@@ -414,7 +439,12 @@ def dynamic_mx_quant_get_workspace(x, y, scale, *, axis=-1, round_mode=b"rint", 
 def dynamic_mx_quant(x, y, scale, stream=None, **kw):
     rc, ws, ex = dynamic_mx_quant_get_workspace(x, y, scale, **kw)
     check(rc, "aclnnDynamicMxQuantGetWorkspaceSize")
-    check(lib().aclnnDynamicMxQuant(None, ws, ex, stream.ptr if stream else None), "aclnnDynamicMxQuant")
+    run = lib().aclnnDynamicMxQuant
+    if kw.get("max_low_bound") is not None:
+        run = lib().aclnnDynamicMxQuantV3
+    elif kw.get("dst_type_max") is not None:
+        run = lib().aclnnDynamicMxQuantV2
+    check(run(None, ws, ex, stream.ptr if stream else None), "aclnnDynamicMxQuant")
 
 
 def trans_quant_param_get_workspace(scale, offset, out, round_mode=None):

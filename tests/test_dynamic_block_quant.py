@@ -124,6 +124,9 @@ def test_status_rules(opsnn):
     assert _status(m, _t(m, (512,), m.ACL_BF16), _t(m, (512,), f8), _t(m, (4,), m.ACL_FLOAT)) == bad
     assert _status(m, x, _t(m, (256, 256), f8), sc) == bad
     assert _status(m, x, y, _t(m, (256, 5), m.ACL_FLOAT)) == bad
+    # V2: the same with a dstTypeMax, which only 0 is run for
+    assert _status(m, x, y, sc, dst_type_max=0.0) == 0 and _status(m, x, y, sc, dst_type_max=100.0) == 561002
+    assert _status(m, x, y, sc, dst_type_max=0.0, row_block=2) == bad
     # accepted by the reference, no kernel here
     assert _status(m, x, _t(m, (256, 512), m.ACL_INT8), sc) == 561002
     assert _status(m, x, _t(m, (256, 512), m.ACL_HIFLOAT8), sc, round_mode=b"round") == 561002
@@ -189,3 +192,17 @@ def test_gpu_block_quantised_operands_feed_the_block_scale_matmul(gpu):
     g, w = orc.b16_to_f32(got, orc.BF16), orc.b16_to_f32(want, orc.BF16)
     mx, mean = orc.rel_err_stats(g, w)
     assert mx <= 2.0 ** -7 and mean <= 2.0 ** -10, f"max rel {mx:.3e} mean rel {mean:.3e}"
+
+
+@pytest.mark.gpu
+def test_gpu_v2_entry_point(gpu):
+    m = gpu
+    xb = orc.f32_to_bf16(np.random.default_rng(3).normal(0, 1, size=(64, 256)).astype(np.float32))
+    want_y, want_s = orc.dynamic_block_quant(xb, orc.BF16, orc.E4M3, 1, 128)
+    d_x, d_y, d_s = m.DeviceBuffer(host=xb), m.DeviceBuffer(xb.size), m.DeviceBuffer(64 * 2 * 4)
+    m.dynamic_block_quant(m.Tensor((64, 256), m.ACL_BF16, d_x), m.Tensor((64, 256), m.ACL_FLOAT8_E4M3FN, d_y),
+                          m.Tensor((64, 2), m.ACL_FLOAT, d_s), dst_type_max=0.0)
+    m.check(m.lib().aclrtSynchronizeDevice(), "sync")
+    gy = d_y.to_host(np.uint8, (64, 256))
+    z = ((gy | want_y) & 0x7f) == 0
+    assert np.array_equal(gy[~z], want_y[~z]) and np.array_equal(d_s.to_host(np.float32, (64, 2)), want_s)

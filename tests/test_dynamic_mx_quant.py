@@ -160,6 +160,10 @@ def test_status_rules(opsnn):
     assert _status(m, x, _t(m, (4, 6, 160), f8), sc) == bad
     assert _status(m, _t(m, (4, 31), m.ACL_BF16), _t(m, (4, 31), f4), _t(m, (4, 1, 2), e8)) == bad     # fp4 needs an even last dim
     assert _status(m, x, y, _t(m, (4, 6, 10), e8)) == bad and _status(m, x, y, _t(m, (4, 6, 6, 2), e8)) == bad
+    # V2 / V3: the added arguments at 0 are the first version
+    assert _status(m, x, y, sc, dst_type_max=0.0) == 0 and _status(m, x, y, sc, dst_type_max=0.0, max_low_bound=0.0) == 0
+    assert _status(m, x, y, sc, dst_type_max=6.0) == not_run and _status(m, x, y, sc, dst_type_max=0.0, max_low_bound=1.0) == not_run
+    assert _status(m, x, y, sc, dst_type_max=0.0, scale_alg=2) == not_run and _status(m, x, y, sc, dst_type_max=0.0, blocksize=48) == bad
     # accepted by the reference, no kernel here
     assert _status(m, x, y, _t(m, (4, 1, 320, 2), e8), axis=1) == not_run
     assert _status(m, x, y, _t(m, (4, 6, 3, 2), e8), blocksize=64) == 0

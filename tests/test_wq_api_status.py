@@ -105,8 +105,10 @@ def test_library_exports_every_declared_symbol(opsnn):
             "aclnnConvertWeightToINT4PackGetWorkspaceSize", "aclnnConvertWeightToINT4Pack", "opsnnPackB4",
             "aclnnDynamicQuantGetWorkspaceSize", "aclnnDynamicQuant", "aclnnDynamicQuantV2GetWorkspaceSize", "aclnnDynamicQuantV2",
             "aclnnDynamicQuantV3GetWorkspaceSize", "aclnnDynamicQuantV3", "aclnnDynamicQuantV4GetWorkspaceSize", "aclnnDynamicQuantV4",
-            "opsnnDynamicQuant", "aclnnDynamicBlockQuantGetWorkspaceSize", "aclnnDynamicBlockQuant", "opsnnDynamicBlockQuant",
+            "opsnnDynamicQuant", "aclnnDynamicBlockQuantGetWorkspaceSize", "aclnnDynamicBlockQuant",
+            "aclnnDynamicBlockQuantV2GetWorkspaceSize", "aclnnDynamicBlockQuantV2", "opsnnDynamicBlockQuant",
             "aclnnDynamicMxQuantGetWorkspaceSize", "aclnnDynamicMxQuant", "opsnnDynamicMxQuant",
+            "aclnnDynamicMxQuantV2GetWorkspaceSize", "aclnnDynamicMxQuantV2", "aclnnDynamicMxQuantV3GetWorkspaceSize", "aclnnDynamicMxQuantV3",
             "aclnnTransQuantParamV2GetWorkspaceSize", "aclnnTransQuantParamV2", "aclnnTransQuantParamV3GetWorkspaceSize",
             "aclnnTransQuantParamV3", "opsnnTransQuantParam",
             "opsnnQmmInt8", "opsnnWqmm", "aclCreateTensor"} <= declared
