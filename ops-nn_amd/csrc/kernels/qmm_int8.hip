@@ -140,6 +140,23 @@ extern "C" int opsnn_qmm_int8_impl(const OpsnnQmmArgs* a, void* stream)
         if (int_out) {
             g.x2off = a->x2_offset; g.x2off_len = a->x2_offset_len;
             if (p.M <= 128 || p.N <= 128 || p.M * p.N < 256 * 256 * 64) return qgemm_launch_int<128, 128, 128, 2, 2, 2, 1>(g, a->batch, p.out_dt, st);
+            // the four-wave kernel under the conditions and with the tile width of the 16-bit outputs below
+            const int64_t cus = cu_count();
+            const int64_t tm = (p.M + 255) / 256, tn = (p.N + 255) / 256;
+            // (OPSNN_VARIANT_I8_256_W8_K128 keeps the call on the 8-wave kernel: the tests compare the two)
+            if (variant != OPSNN_VARIANT_I8_256_W8_K128 && p.K % 128 == 0 && p.K >= 3072 && tm * tn * a->batch * 4 >= cus * 3) {
+                int64_t best = INT64_MAX;
+                int best_fn = 0;
+                for (int fn = 8; fn <= 11; fn++) {
+                    const int64_t tiles = tm * ((p.N + 32 * fn - 1) / (32 * fn)) * a->batch;
+                    const int64_t cost = (tiles + cus - 1) / cus * (fn + 2);
+                    if (cost < best) { best = cost; best_fn = fn; }
+                }
+                if (best <= (tm * tn * a->batch + cus - 1) / cus * 10) {
+                    const int rc = launch_int8_wide(g, best_fn, a->batch, p.out_dt, st);
+                    if (rc != OPSNN_NOT_TAKEN) return rc;
+                }
+            }
             return qgemm_launch_int<256, 256, 128, 2, 4, 2, 1>(g, a->batch, p.out_dt, st);
         }
         if (variant >= OPSNN_VARIANT_I8_WIDE8 && variant <= OPSNN_VARIANT_I8_WIDE11) {

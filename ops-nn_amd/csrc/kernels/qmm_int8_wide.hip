@@ -403,6 +403,76 @@ __global__ __launch_bounds__(256, 1) void qgemm_i8_wide_kernel(QgemmParams p, in
             sS1[i] = p.x1s ? p.x1s[p.x1s_one ? 0 : m] : 1.0f;
         }
     }
+    if constexpr (OUT_DT == DT_I32 || OUT_DT == DT_I8) {
+        // Integer outputs (no per-row scale): INT32 = acc + ib[n]; INT8 = clip(s9(s9(fp32(acc + ib[n]) * s2[n]) + s9(off[n])), the
+        // offset from p.x2off or from bits 37..45 of a UINT64 scale word, s9 = round half to even and clamp to [-256, 255].
+        // They leave straight from the registers: four consecutive columns of one row per lane and fragment.
+        static_assert(!F8 && !MXS, "integer outputs belong to the int8 mode");
+        float* sOff = (float*)smem + 3 * BN + BM;
+        const bool has_off = p.x2off != nullptr || p.x2s_dt == DT_U64;
+        if (OUT_DT == DT_I8 && has_off) {
+            for (int i = tid; i < BN; i += NT) {
+                int64_t n = n0 + i;
+                if (n >= p.N) n = p.N - 1;
+                float off;
+                if (p.x2off) off = p.x2off[p.x2off_len == 1 ? 0 : n];
+                else {
+                    const int raw = (int)((((const uint64_t*)p.x2s)[p.x2s_len == 1 ? 0 : n] >> 37) & 0x1FF);
+                    off = (float)(raw & 0x100 ? raw - 0x200 : raw);
+                }
+                const float r = __builtin_rintf(off);
+                sOff[i] = r < -256.0f ? -256.0f : (r > 255.0f ? 255.0f : r);
+            }
+        }
+        __syncthreads();
+        const bool vec_ok = (p.ldc % 4) == 0 && ((uintptr_t)p.out % 16) == 0;
+#pragma unroll
+        for (int j = 0; j < FM; j++) {
+            const int64_t m = m0 + wm * TM + j * 16 + frow;
+#pragma unroll
+            for (int i = 0; i < FN; i++) {
+                const int nl = wn * TN + i * 16 + 4 * fq;
+                const int64_t n = n0 + nl;
+                const v4i ib = *(const v4i*)(sIb + nl);
+                v4i o;
+                if constexpr (OUT_DT == DT_I32) {
+#pragma unroll
+                    for (int e = 0; e < 4; e++) o[e] = acc[i][j][e] + ib[e];
+                    if (m < p.M) {
+                        int32_t* dst = (int32_t*)p.out + (bz * p.M + m) * p.ldc + n;
+                        if (vec_ok && n + 3 < p.N) *(v4i*)dst = o;
+                        else {
+#pragma unroll
+                            for (int e = 0; e < 4; e++)
+                                if (n + e < p.N) dst[e] = o[e];
+                        }
+                    }
+                } else {
+                    const v4f s2 = *(const v4f*)(sS2 + nl);
+                    uint32_t packed = 0;
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        float t = __builtin_rintf((float)(acc[i][j][e] + ib[e]) * s2[e]);
+                        t = t < -256.0f ? -256.0f : (t > 255.0f ? 255.0f : t);
+                        if (has_off) t = t + sOff[nl + e];
+                        t = t < -128.0f ? -128.0f : (t > 127.0f ? 127.0f : t);
+                        o[e] = (int)t;
+                        packed |= ((uint32_t)o[e] & 0xffu) << (8 * e);
+                    }
+                    if (m < p.M) {
+                        int8_t* dst = (int8_t*)p.out + (bz * p.M + m) * p.ldc + n;
+                        if (vec_ok && n + 3 < p.N) *(uint32_t*)dst = packed;
+                        else {
+#pragma unroll
+                            for (int e = 0; e < 4; e++)
+                                if (n + e < p.N) dst[e] = (int8_t)o[e];
+                        }
+                    }
+                }
+            }
+        }
+        return;
+    }
     __syncthreads();
     // Results leave through LDS: each wave parks one 16 x TN block in a private patch and reads it back row-wise, so
     // that a store instruction writes runs of whole rows (16 bytes per lane, TN/8 lanes per row).
@@ -484,6 +554,17 @@ static int launch_wide_one(const QgemmParams& p, int64_t batch, hipStream_t st)
 int launch_int8_wide(const QgemmParams& p, int fn, int64_t batch, int out_dt, hipStream_t st)
 {
     if (p.KB % 128 != 0 || p.KB < 128) return OPSNN_NOT_TAKEN;
+    if (out_dt == DT_I32 || out_dt == DT_I8) {   // integer epilogue: no per-row scale, no floating bias
+        if (p.x1s || (p.bias && p.bias_dt != DT_I32)) return OPSNN_NOT_TAKEN;
+        const bool i32 = out_dt == DT_I32;
+        switch (fn) {
+            case 8: return i32 ? launch_wide_one<8, DT_I32>(p, batch, st) : launch_wide_one<8, DT_I8>(p, batch, st);
+            case 9: return i32 ? launch_wide_one<9, DT_I32>(p, batch, st) : launch_wide_one<9, DT_I8>(p, batch, st);
+            case 10: return i32 ? launch_wide_one<10, DT_I32>(p, batch, st) : launch_wide_one<10, DT_I8>(p, batch, st);
+            case 11: return i32 ? launch_wide_one<11, DT_I32>(p, batch, st) : launch_wide_one<11, DT_I8>(p, batch, st);
+            default: return OPSNN_NOT_TAKEN;
+        }
+    }
     if (out_dt != DT_BF16 && out_dt != DT_F16) return OPSNN_NOT_TAKEN;
     const bool bf = out_dt == DT_BF16;
     switch (fn) {

@@ -165,3 +165,34 @@ def test_column_split_launch(gpu, s2_dt, bias_dt, out_dt):
     rows = np.unique(np.concatenate([[0, M - 1, 255, 256], np.random.default_rng(2).integers(0, M, 28)]))
     want, _ = cases.oracle_qmm_int8(m, inp, M, K, N, True, dt[out_dt], rows=rows)
     _check_equal(got[0][rows], want[0], "column split")
+
+
+@pytest.mark.parametrize("out_dt,N", [("i8", 5632), ("i32", 5632), ("i8", 5630), ("i32", 5001)])
+def test_integer_outputs_on_the_four_wave_kernel(gpu, out_dt, N):
+    """INT8 (requantised, offset in the packed scale word) and INT32 outputs: large shapes go to the four-wave kernel, whose
+    integer epilogue must give the bits of the 8-wave kernel's (forced with its variant code; that kernel is held to the oracle in
+    test_tc_family.py), and a sample of rows is checked against the oracle directly."""
+    import ctypes as C
+    m = gpu
+    M, K = 2048, 3072
+    print(f"case int8 {M}x{K}x{N} out={out_dt} on the four-wave kernel", flush=True)
+    rng = np.random.default_rng(N)
+    x1, x2 = cases.gen_int8(rng, (1, M, K)), cases.gen_int8(rng, (1, N, K))
+    sf = cases.gen_scale(rng, N, 2e-5, 2e-4)
+    s2 = orc.pack_u64_scale(sf, rng.uniform(-20, 20, N).astype(np.float32))
+    bias = rng.integers(-3000, 3000, size=N).astype(np.int32)
+    d = {k: m.DeviceBuffer(host=v) for k, v in dict(x1=x1, x2=x2, s2=s2, bias=bias).items()}
+    odt, esz, npdt = (m.ACL_INT8, 1, np.int8) if out_dt == "i8" else (m.ACL_INT32, 4, np.int32)
+    outs = []
+    for variant in (0, 7):   # 7: OPSNN_VARIANT_I8_256_W8_K128, the 8-wave 256 x 256 tile kernel
+        d_out = m.DeviceBuffer(M * N * esz)
+        d_out.fill(0x55)
+        a = cases.qmm_args_int8(m, d, M, K, N, 1, True, d_out.ptr, odt, m.ACL_UINT64, N, m.ACL_INT32, variant=variant)
+        assert m.lib().opsnnQmmTc(C.byref(a), None) == 0
+        m.check(m.lib().aclrtSynchronizeDevice(), "sync")
+        outs.append(d_out.to_host(npdt, (M, N)))
+    assert np.array_equal(outs[0], outs[1]), f"{int((outs[0] != outs[1]).sum())} outputs differ between the two kernels"
+    rows = np.unique(np.concatenate([[0, M - 1], rng.integers(0, M, 6)]))
+    want = orc.qmm_tc(np.ascontiguousarray(x1[0][rows]), x2[0], orc.I8, orc.I8, len(rows), K, N, False, True, s2, orc.U64, None, None, bias,
+                      orc.I32, orc.I8 if out_dt == "i8" else orc.I32)
+    assert np.array_equal(outs[0][rows], want)
