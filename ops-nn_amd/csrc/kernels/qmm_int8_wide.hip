@@ -474,25 +474,20 @@ __global__ __launch_bounds__(256, 1) void qgemm_i8_wide_kernel(QgemmParams p, in
         return;
     }
     __syncthreads();
-    // Results leave through LDS: each wave parks one 16 x TN block in a private patch and reads it back row-wise, so
-    // that a store instruction writes runs of whole rows (16 bytes per lane, TN/8 lanes per row).
-    typedef v4us __attribute__((may_alias)) v4us_a;
-    typedef v4i __attribute__((may_alias)) v4i_a;
-    constexpr int EP_PITCH = TN * 2 + 16;
-    constexpr int EP_BASE = (3 * BN + BM) * 4;
-    static_assert(EP_BASE + 4 * 16 * EP_PITCH <= STAGES * STAGE, "epilogue staging fits in the operand stages");
-    char* ep = smem + EP_BASE + wave * (16 * EP_PITCH);
-    constexpr int LPR = TN / 8;                     // lanes per row when every lane moves 16 bytes
-    constexpr int PASSES = (16 * LPR + 63) / 64;
+    // Results leave straight from the registers: a lane holds four consecutive columns of one row per fragment (8 bytes of
+    // 16-bit output); the four lanes that share a row cover 32 contiguous bytes.  Parking each 16 x TN block in an LDS patch
+    // to form 16-byte stores over whole rows was measured 5 us slower per launch on 2048 x 11008 (with one wave per SIMD
+    // nothing hides the patch's write-to-read round trips; the int32 output of the same kernel, stored directly, beat the
+    // 16-bit one although it writes twice the bytes).
     uint16_t* out = (uint16_t*)p.out + bz * p.M * p.ldc;
-    const bool vec_ok = (p.ldc % 8) == 0 && ((uintptr_t)p.out % 16) == 0;
+    const bool vec_ok = (p.ldc % 4) == 0 && ((uintptr_t)p.out % 8) == 0;
 #pragma unroll
     for (int j = 0; j < FM; j++) {
         const float s1 = sS1[wm * TM + j * 16 + frow];
+        const int64_t m = m0 + wm * TM + j * 16 + frow;
 #pragma unroll
         for (int i = 0; i < FN; i++) {
-            const int nw = i * 16 + 4 * fq;   // column inside the wave's sub-tile
-            const int nl = wn * TN + nw;
+            const int nl = wn * TN + i * 16 + 4 * fq;   // column inside the workgroup's tile
             const v4f fbv = *(const v4f*)(sFb + nl);
             const v4f s2 = *(const v4f*)(sS2 + nl);
             const v4i ib = *(const v4i*)(sIb + nl);
@@ -506,26 +501,14 @@ __global__ __launch_bounds__(256, 1) void qgemm_i8_wide_kernel(QgemmParams p, in
                 tv = tv * s1;
                 v[e] = tv + fbv[e];
             }
-            *(v4us_a*)(ep + frow * EP_PITCH + nw * 2) = pack4_b16<OUT_DT>(v);
-        }
-        // this wave's 16 x TN block is complete in its patch (LDS operations of one wave complete in order)
+            const v4us o4 = pack4_b16<OUT_DT>(v);
+            const int64_t n = n0 + nl;
+            if (m < p.M) {
+                if (vec_ok && n + 3 < p.N) *(v4us*)(out + m * p.ldc + n) = o4;
+                else {
 #pragma unroll
-        for (int r = 0; r < PASSES; r++) {
-            const int idx = r * 64 + lane;
-            const int row = idx / LPR, ec = idx % LPR;
-            if (idx < 16 * LPR) {
-                const v4i o = *(const v4i_a*)(ep + row * EP_PITCH + ec * 16);
-                const int64_t m = m0 + wm * TM + j * 16 + row;
-                const int64_t n = n0 + wn * TN + ec * 8;
-                if (m < p.M) {
-                    if (vec_ok && n + 7 < p.N) {
-                        *(v4i*)(out + m * p.ldc + n) = o;
-                    } else {
-                        const uint16_t* oe = (const uint16_t*)&o;
-#pragma unroll
-                        for (int e = 0; e < 8; e++)
-                            if (n + e < p.N) out[m * p.ldc + n + e] = oe[e];
-                    }
+                    for (int e = 0; e < 4; e++)
+                        if (n + e < p.N) out[m * p.ldc + n + e] = o4[e];
                 }
             }
         }
