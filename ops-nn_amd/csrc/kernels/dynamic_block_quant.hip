@@ -138,6 +138,46 @@ __global__ __launch_bounds__(256) void block_quant_tile_kernel(BlockQuantParams 
     const int da = 256 / ppr, db = 256 % ppr;
     const int r_first = (int)threadIdx.x / ppr, c_first = (int)threadIdx.x % ppr;
     float amax = 0.0f;
+    if constexpr (VEC) {
+        // A block of at most 8 pieces per thread whose rows tile the 256 threads evenly (128 x 128 is 8 steps of 16 rows)
+        // stays in registers between the two sweeps: all its loads are issued at once and nothing is read twice.
+        constexpr int HELD = 8;
+        if (db == 0 && rows_here <= HELD * da) {   // uniform over the workgroup
+            uint4 held[HELD];
+#pragma unroll
+            for (int k = 0; k < HELD; k++) {
+                const int r = r_first + k * da;
+                held[k] = r < rows_here ? *(const uint4*)(xb + (int64_t)r * p.cols + c_first * 8) : make_uint4(0, 0, 0, 0);
+            }
+#pragma unroll
+            for (int k = 0; k < HELD; k++) {
+                const uint32_t w[4] = {held[k].x, held[k].y, held[k].z, held[k].w};
+#pragma unroll
+                for (int e = 0; e < 8; e++) {
+                    const float a = fabsf(bq_x_to_f32<X_DT>((w[e >> 1] >> (16 * (e & 1))) & 0xffffu));
+                    amax = fmaxf(amax, a < __builtin_inff() ? a : 0.0f);
+                }
+            }
+#pragma unroll
+            for (int o = 32; o > 0; o >>= 1) amax = fmaxf(amax, __shfl_xor(amax, o));
+            if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = amax;
+            __syncthreads();
+            amax = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+            const BlockScale b = block_scale(p, amax);
+            if (threadIdx.x == 0) p.scale[blk] = b.scale;
+#pragma unroll
+            for (int k = 0; k < HELD; k++) {
+                const int r = r_first + k * da;
+                const uint32_t w[4] = {held[k].x, held[k].y, held[k].z, held[k].w};
+                float v[8];
+#pragma unroll
+                for (int e = 0; e < 8; e++) v[e] = bq_x_to_f32<X_DT>((w[e >> 1] >> (16 * (e & 1))) & 0xffffu);
+                const uint2 q = block_quant_eight<Y_DT>(v, b, p.tmax);
+                if (r < rows_here) *(uint2*)(yb + (int64_t)r * p.cols + c_first * 8) = q;
+            }
+            return;
+        }
+    }
     for (int r = r_first, c = c_first; r < rows_here;) {
         const int64_t o = (int64_t)r * p.cols + c * W;
         if constexpr (VEC) {
