@@ -86,6 +86,9 @@ __global__ __launch_bounds__(256) void block_quant_rows_kernel(BlockQuantParams 
     const int64_t group = ((int64_t)blockIdx.x * 256 + threadIdx.x) / G;
     const int lane = threadIdx.x % G;
     const int64_t total = p.batch * p.rows * p.ncb;
+    // rows that are a whole number of blocks: pair number x block length is the element offset, and the 64-bit divisions by
+    // the row's block count (more instructions than the quantisation of a piece) drop out
+    const bool flat = p.cols == p.ncb * p.cb;
     uint4 buf[NB];
     int64_t at[NB];      // element offset of the lane's piece, -1 when there is none
     bool live_pair[NB];
@@ -93,10 +96,14 @@ __global__ __launch_bounds__(256) void block_quant_rows_kernel(BlockQuantParams 
     for (int i = 0; i < NB; i++) {
         const int64_t pair = (int64_t)i * ngroups + group;
         live_pair[i] = group < ngroups && pair < total;
-        const int64_t row = live_pair[i] ? pair / p.ncb : 0, bc = live_pair[i] ? pair % p.ncb : 0;
-        const int64_t col = bc * p.cb + (int64_t)lane * 8;
-        // cols % 8 == 0: a piece is inside the row or outside
-        at[i] = (live_pair[i] && lane < lpb && col < p.cols) ? row * p.cols + col : -1;
+        if (flat) {
+            at[i] = (live_pair[i] && lane < lpb) ? pair * p.cb + (int64_t)lane * 8 : -1;
+        } else {
+            const int64_t row = live_pair[i] ? pair / p.ncb : 0, bc = live_pair[i] ? pair % p.ncb : 0;
+            const int64_t col = bc * p.cb + (int64_t)lane * 8;
+            // cols % 8 == 0: a piece is inside the row or outside
+            at[i] = (live_pair[i] && lane < lpb && col < p.cols) ? row * p.cols + col : -1;
+        }
         buf[i] = make_uint4(0, 0, 0, 0);
         if (at[i] >= 0) buf[i] = *(const uint4*)(p.x + at[i]);
     }

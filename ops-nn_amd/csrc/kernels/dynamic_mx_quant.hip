@@ -96,7 +96,9 @@ __device__ __forceinline__ uint2 mx_pack8(const float* q)
 
 // cols % 8 == 0: lane groups of four.  A group takes NB (row, block) pairs, the pairs g, g + ngroups, g + 2 ngroups, ...
 // so that neighbouring groups read neighbouring blocks; all NB loads are issued before the first is used.
-template <int X_DT, int Y_DT, int NB>
+// FLAT: every row is a whole, even number of blocks, so pair number, element offset / 32 and scale index coincide and the
+// 64-bit divisions by the row's block count (more instructions than the quantisation itself) drop out.
+template <int X_DT, int Y_DT, int NB, bool FLAT>
 __global__ __launch_bounds__(256) void mx_quant_kernel(MxQuantParams p, int64_t ngroups)
 {
     const int64_t group = ((int64_t)blockIdx.x * 256 + threadIdx.x) / 4;
@@ -110,11 +112,17 @@ __global__ __launch_bounds__(256) void mx_quant_kernel(MxQuantParams p, int64_t 
     for (int i = 0; i < NB; i++) {
         const int64_t pair = (int64_t)i * ngroups + group;
         const bool live_pair = group < ngroups && pair < total;
-        const int64_t row = live_pair ? pair / p.nblk : 0, blk = live_pair ? pair % p.nblk : 0;
-        const int64_t col = blk * 32 + lane * 8;
-        at[i] = (live_pair && col < p.cols) ? row * p.cols + col : -1;
-        sidx[i] = live_pair ? row * p.spitch + blk : -1;
-        pad_after[i] = blk == p.nblk - 1 && (p.nblk & 1);
+        if constexpr (FLAT) {
+            at[i] = live_pair ? pair * 32 + lane * 8 : -1;
+            sidx[i] = live_pair ? pair : -1;
+            pad_after[i] = false;
+        } else {
+            const int64_t row = live_pair ? pair / p.nblk : 0, blk = live_pair ? pair % p.nblk : 0;
+            const int64_t col = blk * 32 + lane * 8;
+            at[i] = (live_pair && col < p.cols) ? row * p.cols + col : -1;
+            sidx[i] = live_pair ? row * p.spitch + blk : -1;
+            pad_after[i] = blk == p.nblk - 1 && (p.nblk & 1);
+        }
         buf[i] = make_uint4(0, 0, 0, 0);
         if (at[i] >= 0) buf[i] = *(const uint4*)(p.x + at[i]);
     }
@@ -197,8 +205,10 @@ static int launch_mx_quant(const MxQuantParams& p, int variant, hipStream_t st)
         const int64_t ngroups = (groups + nb - 1) / nb;
         const int64_t wgs = (ngroups * 4 + 255) / 256;
         if (wgs > 0x7fffffff) return -1;
-        if (nb == 4) hipLaunchKernelGGL((mx_quant_kernel<X_DT, Y_DT, 4>), dim3((unsigned)wgs), dim3(256), 0, st, p, ngroups);
-        else hipLaunchKernelGGL((mx_quant_kernel<X_DT, Y_DT, 1>), dim3((unsigned)wgs), dim3(256), 0, st, p, ngroups);
+        const bool flat = p.cols % 32 == 0 && (p.nblk & 1) == 0;
+        auto go = [&](auto kernel) { hipLaunchKernelGGL(kernel, dim3((unsigned)wgs), dim3(256), 0, st, p, ngroups); };
+        if (nb == 4) { if (flat) go(mx_quant_kernel<X_DT, Y_DT, 4, true>); else go(mx_quant_kernel<X_DT, Y_DT, 4, false>); }
+        else { if (flat) go(mx_quant_kernel<X_DT, Y_DT, 1, true>); else go(mx_quant_kernel<X_DT, Y_DT, 1, false>); }
     } else {
         if (variant == 1) return -4;
         const int64_t wgs = (groups + 255) / 256;
