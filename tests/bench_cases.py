@@ -16,7 +16,7 @@ import oracle_api as orc
 MEASURED_TRAFFIC = {
     (2, None): 104.5e6, (4, None): 824.4e6, (5, None): 1802.2e6,
     (3, 1): 67.2e6, (3, 16): 69.2e6, (1, None): 9.2e6,
-    (6, None): 583.0e6, (7, None): 132.4e6, (8, None): 260.2e6, (9, None): 406.1e6,
+    (6, None): 583.0e6, (7, None): 132.4e6, (8, None): 260.2e6, (9, None): 405.9e6,
 }
 
 
