@@ -80,6 +80,16 @@ typedef struct {
 OPSNN_API int opsnnQmmInt8(const OpsnnQmmArgs* a, void* stream);
 /* fp8 x fp8 with fp32 block scales: out = sum_kb (x1_kb @ x2_kb) * (s1[m/gsM,kb] * s2[kb,n/gsN]). */
 OPSNN_API int opsnnQmmBlockScale(const OpsnnQmmArgs* a, void* stream);
+/* Arithmetic of the fp8 e4m3 x e4m3 block-scale and row/column-scale modes (opsnnQmmBlockScale, opsnnQmmTc, the fp8 x fp4
+ * group-scale mode of opsnnQmmGroup), process-wide:
+ *   0 (default)  the operands are widened to fp16 in registers (exact) and contracted by the fp16 matrix instruction:
+ *                products exact, sums as good as an fp32 accumulation -- the results meet the reference's acceptance
+ *                (max relative error 2^-7, mean 2^-10, 99.9 % within rtol 1e-3) like an fp32-accumulating device;
+ *   1            the 8-bit matrix instruction, about 1.5x faster; it aligns the 128 products of one instruction in a
+ *                window narrower than fp32, which leaves about 1 % of bf16 outputs one ulp off at K = 7168.
+ * The initial value is taken from the environment variable OPSNN_FP8_FAST (unset or 0: exact). */
+OPSNN_API void opsnnSetFp8Fast(int fast);
+OPSNN_API int opsnnGetFp8Fast(void);
 /* MX: fp4/fp8 operands, e8m0 scale per 32 K. out = (x1*s1) @ (x2*s2) + fp32 bias. */
 OPSNN_API int opsnnQmmMx(const OpsnnQmmArgs* a, void* stream);
 /* Per-tensor / per-channel scales (T-T, T-C): int8 or fp8 (e4m3, e5m2) operands;

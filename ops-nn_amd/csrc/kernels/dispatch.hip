@@ -31,6 +31,13 @@ extern "C" __attribute__((visibility("hidden"))) bool opsnn_force_plain()
     return e && *e && *e != '0';
 }
 
+// fp8 x fp8 arithmetic of the block-scale and row/column-scale modes: 0 (default) exact products and sums on the fp16
+// matrix instruction, 1 the 8-bit matrix instruction (about 1.5x faster, sums aligned in a narrower window).  The
+// initial value comes from OPSNN_FP8_FAST, read once.
+static int g_fp8_fast = [] { const char* e = getenv("OPSNN_FP8_FAST"); return (e && *e && *e != '0') ? 1 : 0; }();
+extern "C" void opsnnSetFp8Fast(int fast) { __atomic_store_n(&g_fp8_fast, fast ? 1 : 0, __ATOMIC_RELAXED); }
+extern "C" int opsnnGetFp8Fast(void) { return __atomic_load_n(&g_fp8_fast, __ATOMIC_RELAXED); }
+
 static bool qmm_args_ok(const OpsnnQmmArgs* a)
 {
     return a && a->x1.ptr && a->x2.ptr && a->out && a->M > 0 && a->N > 0 && a->K > 0 && a->batch > 0 && a->batch <= 65535;

@@ -1,0 +1,385 @@
+// fp8 e4m3 x fp8 e4m3 quantized matmul whose products and partial sums are exact: the operands are widened to fp16 in
+// registers (every e4m3 value, subnormals included, is an fp16 value) and contracted by v_mfma_f32_16x16x32_f16.
+//
+//   block scales:      out[m,n] = cast( sum_kb ( sum_{k in block kb} x1[m,k] * x2[k,n] ) * ( s1[m/gsM, kb] * s2[kb, n/128] ) )
+//   row/column scales: out[m,n] = cast( (sum_k x1[m,k] * x2[k,n]) * cs[n] * rs[m] + bias[n] )
+//
+// Formulas: matmul/quant_batch_matmul_v3/tests/assets/qbmmv3_kernel_golden.py:237-358 (the two block scales are
+// multiplied together first, :337-343) and :361-387; device counterpart in the reference:
+// matmul/common/cmct/epilogue/block_epilogue_pertile.h:502-642.
+//
+// Why not the 8-bit matrix instruction: on gfx950 it aligns its 128 products in a window narrower than fp32 (measured
+// on N(0,1) data rounded to e4m3: mean error 1.2e-6, max 1.6e-5 of sum|terms| per instruction), which leaves about 1 %
+// of the bf16 outputs one ulp from the fp32-accumulated result at K = 7168 and a few two ulps away where the terms
+// cancel.  The fp16 instruction's products (22 significant bits) are summed like an fp32 accumulation or better
+// (measured: bit-identical to the correctly rounded exact sum of 128 products in 99.5 % of cases, never further than
+// fp32 ascending-k summation), at half the matrix rate.
+//
+// Tiling: 256 x 128 output tile per workgroup, 4 x 2 waves of 64 x 64 (4 x 4 fragments of 16 x 16).  The operands stay
+// e4m3 bytes on the way global -> LDS (16-byte asynchronous copies, rows XOR-swizzled) and LDS -> registers, exactly as
+// in qmm_fp8_block.hip; a lane's 32 bytes of a fragment become sixteen registers of fp16 pairs by sixteen
+// v_cvt_scalef32_pk_f16_fp8 (unit scale).  The x1 fragments are widened once per K tile and stay (64 registers), the
+// x2 fragments as they stream through.  One K tile is one 128-wide scale block: a chain of four instructions from a
+// zero accumulator leaves the block's partial sums in four registers, and the vector ALU folds them into the fp32
+// running sums (one fma each) one fragment pair later, in the shadow of the next chain.
+#include "launch.h"
+#include "qgemm_core.hip.h"
+
+namespace opsnn {
+
+struct Fp8xParams {
+    const int8_t* a;
+    const int8_t* b;
+    int64_t lda, ldb, a_bs, b_bs;
+    void* out;
+    int64_t M, N, K;
+    const float* s1;   // element (m/gsM, kb) at s1[(m/gsM)*s1_rs + kb*s1_cs]
+    const float* s2;   // element (kb, nb) at s2[kb*s2_rs + nb*s2_cs]
+    int64_t s1_rs, s1_cs, s1_bs, s2_rs, s2_cs, s2_bs;
+    int gsM;           // 1 or 128
+    // row / column scale mode: out = (sum * cs[n * cs_stride]) * rs[m * rs_stride] + bias[n]; strides 0 (one scale) or 1
+    const float* rs;
+    const float* cs;
+    int rs_stride, cs_stride;
+    const float* bias;
+    int64_t bias_bs;
+};
+
+__device__ __forceinline__ const int8_t* uniform_ptr(const int8_t* p)
+{
+    const uint64_t u = (uint64_t)p;
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)u), hi = __builtin_amdgcn_readfirstlane((uint32_t)(u >> 32));
+    return (const int8_t*)(((uint64_t)hi << 32) | lo);
+}
+
+// Eight e4m3 bytes (two registers) -> eight fp16 values (four registers), exact.
+__device__ __forceinline__ v8h widen8(int d0, int d1)
+{
+    const v2h a = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8((uint32_t)d0, 1.0f, false);
+    const v2h b = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8((uint32_t)d0, 1.0f, true);
+    const v2h c = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8((uint32_t)d1, 1.0f, false);
+    const v2h d = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8((uint32_t)d1, 1.0f, true);
+    return (v8h){a[0], a[1], b[0], b[1], c[0], c[1], d[0], d[1]};
+}
+
+template <int OUT_DT, bool RC>
+__global__ __launch_bounds__(512, 1) void qmm_fp8_exact_kernel(Fp8xParams p, int tiles_m, int tiles_n)
+{
+    constexpr int BM = 256, BN = 128, BK = 128, NT = 512;
+    constexpr int CPR = BK / 16, RPW = 16 / CPR;
+    constexpr int TM = 64, TN = 64, FM = TM / 16, FN = TN / 16;
+    constexpr int A_BYTES = BM * BK, B_BYTES = BN * BK;
+    constexpr int SC_BYTES = RC ? 0 : NT * 4;        // BM s1 floats + the s2 float of the tile's n block, one 4-byte copy per lane
+    constexpr int STAGE = A_BYTES + B_BYTES + SC_BYTES;
+    constexpr int RPI = NT / CPR;                    // 64 tile rows per copy instruction of the workgroup
+    constexpr int NA = BM / RPI, NB = BN / RPI;
+    constexpr int CPT = NA + NB + (RC ? 0 : 1);
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave >> 1, wn = wave & 1;
+
+    const uint32_t t = xcd_remap(blockIdx.x, (uint32_t)(tiles_m * tiles_n));
+    const int tm = (int)(t % (uint32_t)tiles_m), tn = (int)(t / (uint32_t)tiles_m);
+    const int64_t m0 = (int64_t)tm * BM, n0 = (int64_t)tn * BN;
+    const int64_t bz = blockIdx.y;
+    const int64_t lda = p.lda, ldb = p.ldb;
+    const int8_t* A = p.a + bz * p.a_bs + m0 * lda;
+    const int8_t* B = p.b + bz * p.b_bs + n0 * ldb;
+    const int KT = (int)(p.K / BK);
+
+    // copies: instruction i of the workgroup fills tile rows i*64 .. i*64+63; this thread handles row i*64 + tid/8 and
+    // the logical 16-byte chunk that belongs at position tid%8 of the swizzled row.  Rows past the matrix edge repeat
+    // the last valid row: they only feed outputs that are never stored.
+    const int crow = tid / CPR;
+    const int cchunk = (tid % CPR) ^ ((crow / RPW) & (CPR - 1));
+    const int a_rows = (int)((p.M - m0) < BM ? (p.M - m0) : BM);
+    const int b_rows = (int)((p.N - n0) < BN ? (p.N - n0) : BN);
+    uint32_t a_off[NA], b_off[NB];
+#pragma unroll
+    for (int i = 0; i < NA; i++) {
+        int r = i * RPI + crow;
+        r = r < a_rows ? r : a_rows - 1;
+        a_off[i] = (uint32_t)(r * lda + cchunk * 16);
+    }
+#pragma unroll
+    for (int i = 0; i < NB; i++) {
+        int r = i * RPI + crow;
+        r = r < b_rows ? r : b_rows - 1;
+        b_off[i] = (uint32_t)(r * ldb + cchunk * 16);
+    }
+    // scale copy: lanes 0..255 fetch s1 of tile row `tid`, the others the s2 of this tile's n block
+    const float* sc_src = nullptr;
+    int64_t sc_step = 0;
+    if constexpr (!RC) {
+        if (tid < BM) {
+            const int r = tid < a_rows ? tid : a_rows - 1;
+            sc_src = p.s1 + bz * p.s1_bs + ((m0 + r) / p.gsM) * p.s1_rs;
+            sc_step = p.s1_cs;
+        } else {
+            sc_src = p.s2 + bz * p.s2_bs + (n0 / 128) * p.s2_cs;
+            sc_step = p.s2_rs;
+        }
+    }
+    auto issue_piece = [&](int kt, int stage, int idx) {
+        char* sA = smem + stage * STAGE + wave * 1024;
+        char* sB = sA + A_BYTES;
+        const int8_t* Ak = uniform_ptr(A + (int64_t)kt * BK);
+        const int8_t* Bk = uniform_ptr(B + (int64_t)kt * BK);
+        if (idx < NA) async_copy16(Ak + a_off[idx], sA + idx * NT * 16);
+        else if (idx < NA + NB) async_copy16(Bk + b_off[idx - NA], sB + (idx - NA) * NT * 16);
+        else async_copy4(sc_src + (int64_t)kt * sc_step, smem + stage * STAGE + A_BYTES + B_BYTES + wave * 256);
+    };
+    auto issue_tile = [&](int kt) {
+#pragma unroll
+        for (int idx = 0; idx < CPT; idx++) issue_piece(kt, kt & 1, idx);
+    };
+
+    v4f acc[FN][FM];
+#pragma unroll
+    for (int i = 0; i < FN; i++)
+#pragma unroll
+        for (int j = 0; j < FM; j++) acc[i][j] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
+
+    // Fragment of a 16-row block, lane (row = lane%16, q = lane/16): the 32 bytes [32q, 32q+32) of the row's 128 bytes
+    // of K; instruction s of the chain of four takes bytes [32q + 8s, +8) from both operands (K is the contraction
+    // index: any assignment of K to lanes and steps is right as long as both operands use the same one).
+    const int frow = lane & 15, fq = lane >> 4;
+    const int key = (frow / RPW) & (CPR - 1);
+    const int ch0 = ((2 * fq) ^ key) << 4, ch1 = ((2 * fq + 1) ^ key) << 4;
+    const int a_rowbase = (wm * TM + frow) * BK;
+    const int b_rowbase = A_BYTES + (wn * TN + frow) * BK;
+    auto load_frag = [&](const char* st, int rowbase) -> v8i {
+        const v4i lo = *(const v4i*)(st + rowbase + ch0);
+        const v4i hi = *(const v4i*)(st + rowbase + ch1);
+        return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+    };
+
+    issue_tile(0);
+    if (KT > 1) {
+        issue_tile(1);
+        wait_vmcnt<CPT>();
+    } else {
+        wait_vmcnt<0>();
+    }
+    __builtin_amdgcn_s_barrier();
+
+    v8i fa_raw[FM], fb_raw[2];
+    v8h fa[FM][4], fb[4];
+    float sc[FM], s1raw[FM], s2raw = 0.0f, sc_last = 0.0f;
+    v4f part[2];
+    (void)sc; (void)s1raw; (void)s2raw; (void)sc_last; (void)part;
+    auto read_scales = [&](const char* st) {
+        if constexpr (!RC) {
+            const float* sS = (const float*)(st + A_BYTES + B_BYTES);
+            s2raw = sS[BM];
+#pragma unroll
+            for (int j = 0; j < FM; j++) s1raw[j] = sS[wm * TM + j * 16 + frow];
+        }
+    };
+    {
+        read_scales(smem);
+#pragma unroll
+        for (int j = 0; j < FM; j++) fa_raw[j] = load_frag(smem, a_rowbase + j * 16 * BK);
+        fb_raw[0] = load_frag(smem, b_rowbase);
+#pragma unroll
+        for (int j = 0; j < FM; j++) sc[j] = 0.0f;
+        part[0] = part[1] = v4f{0.0f, 0.0f, 0.0f, 0.0f};   // folded with scale 0 into the first tile's sums
+    }
+    constexpr int CPS = (CPT + FM - 1) / FM;   // copies issued behind each chain of the tile's last x2 fragment
+
+    for (int kt = 0; kt < KT; kt++) {
+        const char* st = smem + (kt & 1) * STAGE;
+        const char* stn = smem + ((kt + 1) & 1) * STAGE;
+        const int ktc = kt + 2 < KT ? kt + 2 : KT - 1;   // past the end the copies repeat the last tile into a stage nobody reads
+#pragma unroll
+        for (int i = 0; i < FN; i++) {
+            if (i + 1 < FN) {
+                fb_raw[(i + 1) & 1] = load_frag(st, b_rowbase + (i + 1) * 16 * BK);
+                __builtin_amdgcn_sched_barrier(0);
+                __builtin_amdgcn_s_waitcnt(0xc07f | (2 << 8));   // lgkmcnt: all but the two reads just issued
+            } else {
+                wait_vmcnt<0>();
+                wait_lgkmcnt0();
+                __builtin_amdgcn_s_barrier();   // tile kt+1 is complete in LDS; every wave has read all it needs of tile kt
+                __builtin_amdgcn_sched_barrier(0);
+                read_scales(stn);
+                fb_raw[0] = load_frag(stn, b_rowbase);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            if (i == 0) {   // this tile's x1 fragments (requested behind the previous tile's barrier) and scales
+#pragma unroll
+                for (int j = 0; j < FM; j++)
+#pragma unroll
+                    for (int s = 0; s < 4; s++) fa[j][s] = widen8(fa_raw[j][2 * s], fa_raw[j][2 * s + 1]);
+                if constexpr (!RC) {
+                    sc_last = sc[FM - 1];
+#pragma unroll
+                    for (int j = 0; j < FM; j++) sc[j] = s1raw[j] * s2raw;
+                }
+            }
+#pragma unroll
+            for (int s = 0; s < 4; s++) fb[s] = widen8(fb_raw[i & 1][2 * s], fb_raw[i & 1][2 * s + 1]);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int j = 0; j < FM; j++) {
+                const int pi = (i * FM + j) & 1;
+                if constexpr (RC) {
+#pragma unroll
+                    for (int s = 0; s < 4; s++) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fb[s], fa[j][s], acc[i][j], 0, 0, 0);
+                } else {
+                    v4f c = v4f{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+                    for (int s = 0; s < 4; s++) c = __builtin_amdgcn_mfma_f32_16x16x32_f16(fb[s], fa[j][s], c, 0, 0, 0);
+                    part[pi] = c;
+                }
+                __builtin_amdgcn_sched_barrier(0);
+                if (i == FN - 1) {
+                    fa_raw[j] = load_frag(stn, a_rowbase + j * 16 * BK);
+#pragma unroll
+                    for (int c = j * CPS; c < (j + 1) * CPS && c < CPT; c++) issue_piece(ktc, kt & 1, c);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+                if constexpr (!RC) {   // fold the pair before this one
+                    if (j > 0) {
+#pragma unroll
+                        for (int r = 0; r < 4; r++) acc[i][j - 1][r] = __builtin_fmaf(part[pi ^ 1][r], sc[j - 1], acc[i][j - 1][r]);
+                    } else if (i > 0) {
+#pragma unroll
+                        for (int r = 0; r < 4; r++) acc[i - 1][FM - 1][r] = __builtin_fmaf(part[pi ^ 1][r], sc[FM - 1], acc[i - 1][FM - 1][r]);
+                    } else {   // the previous tile's last pair, with that tile's scale
+#pragma unroll
+                        for (int r = 0; r < 4; r++) acc[FN - 1][FM - 1][r] = __builtin_fmaf(part[pi ^ 1][r], sc_last, acc[FN - 1][FM - 1][r]);
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            }
+        }
+    }
+    if constexpr (!RC) {
+#pragma unroll
+        for (int r = 0; r < 4; r++) acc[FN - 1][FM - 1][r] = __builtin_fmaf(part[(FN * FM - 1) & 1][r], sc[FM - 1], acc[FN - 1][FM - 1][r]);
+    }
+    wait_lgkmcnt0();   // the reads and copies past the last tile land before LDS is reused
+    wait_vmcnt<0>();
+
+    // Epilogue: acc[i][j][r] is out[m = m_base + 16j + lane%16][n = n_base + 16i + 4*(lane/16) + r].  Each wave parks one
+    // 16 x 64 block in a private LDS patch and reads it back row-wise, so that a store instruction writes whole
+    // 128-byte lines (16 bytes per lane, 8 lanes per row).
+    __syncthreads();
+    typedef v4us __attribute__((may_alias)) v4us_a;
+    typedef v4i __attribute__((may_alias)) v4i_a;
+    constexpr int EP_PITCH = TN * 2 + 16;
+    char* ep = smem + wave * (16 * EP_PITCH);
+    static_assert(8 * 16 * EP_PITCH <= 2 * STAGE, "epilogue staging fits in the operand stages");
+    uint16_t* out = (uint16_t*)p.out + bz * p.M * p.N;
+    const bool vec_ok = (p.N % 8) == 0 && ((uintptr_t)p.out % 16) == 0;
+    const int er = lane >> 3, ec = lane & 7;
+    float rs_j[FM];
+    (void)rs_j;
+    if constexpr (RC) {
+#pragma unroll
+        for (int j = 0; j < FM; j++) {
+            const int64_t mrow = m0 + wm * TM + j * 16 + frow;
+            rs_j[j] = p.rs[(mrow < p.M ? mrow : p.M - 1) * p.rs_stride];
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < FM; j++) {
+#pragma unroll
+        for (int i = 0; i < FN; i++) {
+            v4f v = acc[i][j];
+            if constexpr (RC) {   // (sum * x2Scale[n]) * x1Scale[m] + bias[n], each operation rounded, as compute_pertoken orders them
+                const int64_t nb = n0 + wn * TN + i * 16 + 4 * fq;
+#pragma unroll
+                for (int r = 0; r < 4; r++) {
+                    const int64_t ni = nb + r < p.N ? nb + r : p.N - 1;
+                    v[r] = (v[r] * p.cs[ni * p.cs_stride]) * rs_j[j];
+                    if (p.bias) v[r] = v[r] + p.bias[bz * p.bias_bs + ni];
+                }
+            }
+            *(v4us_a*)(ep + frow * EP_PITCH + (i * 16 + 4 * fq) * 2) = pack4_b16<OUT_DT>(v);
+        }
+#pragma unroll
+        for (int r = 0; r < 2; r++) {
+            const int row = r * 8 + er;
+            const v4i o = *(const v4i_a*)(ep + row * EP_PITCH + ec * 16);
+            const int64_t m = m0 + wm * TM + j * 16 + row;
+            const int64_t n = n0 + wn * TN + ec * 8;
+            if (m < p.M) {
+                if (vec_ok && n + 7 < p.N) {
+                    *(v4i*)(out + m * p.N + n) = o;
+                } else {
+                    const uint16_t* oe = (const uint16_t*)&o;
+#pragma unroll
+                    for (int e = 0; e < 8; e++)
+                        if (n + e < p.N) out[m * p.N + n + e] = oe[e];
+                }
+            }
+        }
+    }
+}
+
+template <int OUT_DT, bool RC>
+static int launch_fp8_exact(const Fp8xParams& p, int64_t batch, hipStream_t st)
+{
+    const int tiles_m = (int)((p.M + 255) / 256), tiles_n = (int)((p.N + 127) / 128);
+    dim3 grid((unsigned)(tiles_m * tiles_n), (unsigned)batch);
+    const size_t lds = 2 * (size_t)(256 * 128 + 128 * 128 + (RC ? 0 : 512 * 4));
+    auto k = qmm_fp8_exact_kernel<OUT_DT, RC>;
+    static bool attr_set = false;
+    if (!attr_set) {
+        hipError_t e = hipFuncSetAttribute((const void*)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return (int)e;
+        attr_set = true;
+    }
+    hipLaunchKernelGGL(k, grid, dim3(512), lds, st, p, tiles_m, tiles_n);
+    return (int)hipGetLastError();
+}
+
+// fp8 e4m3 block scales (G-B, B-B), K-contiguous operands, K % 128 == 0, 16-bit output, no bias.
+int launch_blockscale_exact(const OpsnnQmmArgs& a, hipStream_t st)
+{
+    if (a.x1_dtype != DT_E4M3 || a.x2_dtype != DT_E4M3) return OPSNN_NOT_TAKEN;
+    if (a.out_dtype != DT_BF16 && a.out_dtype != DT_F16) return OPSNN_NOT_TAKEN;
+    if (a.bias) return OPSNN_NOT_TAKEN;
+    if (a.gsK != 128 || a.gsN != 128 || (a.gsM != 1 && a.gsM != 128)) return OPSNN_NOT_TAKEN;
+    if (a.K % 128 != 0 || a.M * a.N < 64 * 64 || a.x1.col_stride != 1 || a.x2.row_stride != 1) return OPSNN_NOT_TAKEN;
+    Fp8xParams p{};
+    p.a = (const int8_t*)a.x1.ptr; p.b = (const int8_t*)a.x2.ptr;
+    p.lda = a.x1.row_stride; p.ldb = a.x2.col_stride; p.a_bs = a.x1.batch_stride; p.b_bs = a.x2.batch_stride;
+    p.out = a.out; p.M = a.M; p.N = a.N; p.K = a.K;
+    p.s1 = (const float*)a.x1_scale_mat.ptr; p.s1_rs = a.x1_scale_mat.row_stride; p.s1_cs = a.x1_scale_mat.col_stride;
+    p.s1_bs = a.x1_scale_mat.batch_stride;
+    p.s2 = (const float*)a.x2_scale_mat.ptr; p.s2_rs = a.x2_scale_mat.row_stride; p.s2_cs = a.x2_scale_mat.col_stride;
+    p.s2_bs = a.x2_scale_mat.batch_stride;
+    p.gsM = (int)a.gsM;
+    if (((uintptr_t)p.a | (uintptr_t)p.b | (uint64_t)p.lda | (uint64_t)p.ldb | (uint64_t)p.a_bs | (uint64_t)p.b_bs) % 16) return OPSNN_NOT_TAKEN;
+    if (((uintptr_t)p.s1 | (uintptr_t)p.s2) % 4) return OPSNN_NOT_TAKEN;
+    if (a.out_dtype == DT_BF16) return launch_fp8_exact<DT_BF16, false>(p, a.batch, st);
+    return launch_fp8_exact<DT_F16, false>(p, a.batch, st);
+}
+
+// fp8 e4m3 with one fp32 scale per row of x1 (or one) and one per column of x2 (or one), optional fp32 bias.
+int launch_rowcol_exact(const OpsnnQmmArgs& a, hipStream_t st)
+{
+    if (a.x1_dtype != DT_E4M3 || a.x2_dtype != DT_E4M3) return OPSNN_NOT_TAKEN;
+    if (a.out_dtype != DT_BF16 && a.out_dtype != DT_F16) return OPSNN_NOT_TAKEN;
+    if (!a.x1_scale || !a.x2_scale || a.x2_scale_dtype != DT_F32) return OPSNN_NOT_TAKEN;
+    if (a.bias && a.bias_dtype != DT_F32) return OPSNN_NOT_TAKEN;
+    if (a.K % 128 != 0 || a.M * a.N < 64 * 64 || a.x1.col_stride != 1 || a.x2.row_stride != 1) return OPSNN_NOT_TAKEN;
+    Fp8xParams p{};
+    p.a = (const int8_t*)a.x1.ptr; p.b = (const int8_t*)a.x2.ptr;
+    p.lda = a.x1.row_stride; p.ldb = a.x2.col_stride; p.a_bs = a.x1.batch_stride; p.b_bs = a.x2.batch_stride;
+    p.out = a.out; p.M = a.M; p.N = a.N; p.K = a.K; p.gsM = 1;
+    p.rs = (const float*)a.x1_scale; p.rs_stride = a.x1_scale_len == 1 ? 0 : 1;
+    p.cs = (const float*)a.x2_scale; p.cs_stride = a.x2_scale_len == 1 ? 0 : 1;
+    p.bias = (const float*)a.bias; p.bias_bs = a.bias_batch_stride;
+    if (((uintptr_t)p.a | (uintptr_t)p.b | (uint64_t)p.lda | (uint64_t)p.ldb | (uint64_t)p.a_bs | (uint64_t)p.b_bs) % 16) return OPSNN_NOT_TAKEN;
+    if (a.out_dtype == DT_BF16) return launch_fp8_exact<DT_BF16, true>(p, a.batch, st);
+    return launch_fp8_exact<DT_F16, true>(p, a.batch, st);
+}
+
+}  // namespace opsnn

@@ -73,9 +73,18 @@ def test_config4_fp8_block_scale_full(gpu):
     got = cases.run_blockscale_aclnn(m, inp, M, K, N, True, m.ACL_BF16)
     rows = _rows(M, 10, 5)
     want = cases.oracle_blockscale(m, inp, M, K, N, True, m.ACL_BF16, rows=rows)
-    check_close(got[0][rows], want[0], m.ACL_BF16, "config 4", fp8_mfma=True)
+    # default path (exact fp16 products): the stated bar -- max rel 2^-7, mean rel 2^-10, 99.9 % within rtol = atol = 1e-3
+    check_close(got[0][rows], want[0], m.ACL_BF16, "config 4")
     inp2 = dict(inp, s1=inp["s1"] * np.float32(2.0))
     _double_exactly(got, cases.run_blockscale_aclnn(m, inp2, M, K, N, True, m.ACL_BF16), m.ACL_BF16)
+    # opt-in 8-bit matrix instruction: measured here 98.9 % of bf16 outputs bit-identical, mean rel 0.05 x 2^-10, no
+    # element outside rtol = atol = 1e-3, max rel 1.25 x 2^-7 (a handful of small outputs two ulps off): the looser bar
+    m.lib().opsnnSetFp8Fast(1)
+    try:
+        fast = cases.run_blockscale_aclnn(m, inp, M, K, N, True, m.ACL_BF16)
+    finally:
+        m.lib().opsnnSetFp8Fast(0)
+    check_close(fast[0][rows], want[0], m.ACL_BF16, "config 4, 8-bit matrix instruction", fp8_mfma=True)
 
 
 def test_config5_mxfp4_batched_full(gpu):

@@ -178,13 +178,16 @@ def test_gpu_tcg(gpu, M, K, N, s_dt, out_dt, ys_i64):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("fast", [False, True])
 @pytest.mark.parametrize("M,K,N,s_dt,out_dt", [(64, 128, 64, "bf16", "bf16"), (300, 384, 260, "f16", "f16"),
                                                (512, 2048, 520, "bf16", "bf16"), (1024, 1024, 2048, "bf16", "f16")])
-def test_gpu_tcg_on_the_matrix_cores(gpu, M, K, N, s_dt, out_dt):
+def test_gpu_tcg_on_the_matrix_cores(gpu, M, K, N, s_dt, out_dt, fast):
     """fp8 x fp4 with 16-bit group scales, K % 128 == 0 and enough outputs: a prologue writes the re-quantised e4m3 weight
     (the oracle's bytes) into the workspace and the fp8 matrix-core kernel does the product with the decoded output scale
-    per column (every third group scale is negative here).  Bar: the one of MXFP8 (the 8-bit instruction's alignment error against sum|terms|, mean rel <= 2^-10); the
-    same call on the plain kernel is bit-identical to the oracle."""
+    per column (every third group scale is negative here).  Default (exact fp16 products): max rel 2^-7, mean rel 2^-10,
+    99.9 % within rtol = atol = 1e-3.  fast (the 8-bit matrix instruction): the dot product's backward-error bound with
+    the instruction's alignment error against sum|terms|, mean rel <= 2^-10.  The same call on the plain kernel is
+    bit-identical to the oracle."""
     import os
     m = gpu
     print(f"case tcg mfma {M}x{K}x{N} scale={s_dt} out={out_dt}", flush=True)
@@ -192,16 +195,24 @@ def test_gpu_tcg_on_the_matrix_cores(gpu, M, K, N, s_dt, out_dt):
     inp = cases.make_tcg_inputs(m, M, K, N, M + N, dt[s_dt][0])
     inp["s2"] = inp["s2"] ^ ((np.arange(inp["s2"].size, dtype=np.uint32).reshape(inp["s2"].shape) % 3 == 0).astype(np.uint16) << 15)
     want = cases.oracle_tcg(m, inp, M, K, N, dt[out_dt][0])
-    got = cases.run_tcg_aclnn(m, inp, M, K, N, dt[out_dt][0])
-    pos = dict(inp, x1=inp["x1"] & 0x7F, x2=inp["x2"] & 0x77, s2=inp["s2"] & 0x7FFF)
+    m.lib().opsnnSetFp8Fast(1 if fast else 0)
+    try:
+        got = cases.run_tcg_aclnn(m, inp, M, K, N, dt[out_dt][0])
+    finally:
+        m.lib().opsnnSetFp8Fast(0)
     odt = dt[out_dt][1]
-    abs_sum = orc.b16_to_f32(cases.oracle_tcg(m, pos, M, K, N, dt[out_dt][0]), odt).astype(np.float64)
     g, w = orc.b16_to_f32(got, odt), orc.b16_to_f32(want, odt)
     assert np.isfinite(g).all()
-    err = np.abs(g.astype(np.float64) - w)
-    bound = 2.0 ** -7 * np.abs(w) + 2.0 ** -14 * abs_sum
     mx, mean = orc.rel_err_stats(g, w)
-    assert float((err / np.maximum(bound, 1e-30)).max()) <= 1.0 and mean <= 2.0 ** -10, f"max rel {mx:.3e} mean rel {mean:.3e}"
+    if fast:
+        pos = dict(inp, x1=inp["x1"] & 0x7F, x2=inp["x2"] & 0x77, s2=inp["s2"] & 0x7FFF)
+        abs_sum = orc.b16_to_f32(cases.oracle_tcg(m, pos, M, K, N, dt[out_dt][0]), odt).astype(np.float64)
+        err = np.abs(g.astype(np.float64) - w)
+        bound = 2.0 ** -7 * np.abs(w) + 2.0 ** -14 * abs_sum
+        assert float((err / np.maximum(bound, 1e-30)).max()) <= 1.0 and mean <= 2.0 ** -10, f"max rel {mx:.3e} mean rel {mean:.3e}"
+    else:
+        assert mx <= 2.0 ** -7 and mean <= 2.0 ** -10, f"max rel {mx:.3e} mean rel {mean:.3e}"
+        assert orc.isclose_fraction(g, w) <= 1e-3
     os.environ["OPSNN_FORCE_PLAIN"] = "1"
     try:
         exact = cases.run_tcg_aclnn(m, inp, M, K, N, dt[out_dt][0])
