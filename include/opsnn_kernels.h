@@ -78,6 +78,17 @@ typedef struct {
 /* int8 x int8 -> int32, then  out = fp32(acc + int32 bias) * x2_scale[n] * x1_scale[m] + float bias.
  * x1_scale: fp32 [M] or NULL. */
 OPSNN_API int opsnnQmmInt8(const OpsnnQmmArgs* a, void* stream);
+/* opsnnQmmInt8 for callers that cannot allocate device memory (code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc).  It has no counterpart in the reference.  Same arguments and results as
+ * opsnnQmmInt8, except that `workspace` is ignored: when x2 is stored [K, N] with N contiguous, the K-contiguous copy
+ * the matrix-core kernel reads goes into an array of OPSNN_STATIC_SCRATCH_BYTES inside the library's device image
+ * instead.  The call makes no hipMalloc / hipFree.  A call whose opsnnQmmWorkspace(a, 0) exceeds that size launches nothing and
+ * returns OPSNN_ERR_SCRATCH_TOO_SMALL (text in aclGetRecentErrMsg).  All calls on one device share the one array:
+ * calls that overlap in time on one device (different streams, different threads) race on it; calls on one stream
+ * are ordered and safe.  Each device the library is loaded on holds the array until the process ends. */
+#define OPSNN_STATIC_SCRATCH_BYTES (64ll << 20)
+#define OPSNN_ERR_SCRATCH_TOO_SMALL (-6)
+OPSNN_API int opsnnQmmInt8Static(const OpsnnQmmArgs* a, void* stream);
 /* fp8 x fp8 with fp32 block scales: out = sum_kb (x1_kb @ x2_kb) * (s1[m/gsM,kb] * s2[kb,n/gsN]). */
 OPSNN_API int opsnnQmmBlockScale(const OpsnnQmmArgs* a, void* stream);
 /* Arithmetic of the fp8 e4m3 x e4m3 block-scale and row/column-scale modes (opsnnQmmBlockScale, opsnnQmmTc, the fp8 x fp4

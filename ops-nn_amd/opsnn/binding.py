@@ -172,6 +172,7 @@ _SIGS = {
     "opsnnTransQuantParam": (C.c_int, [C.c_void_p, C.c_int64, C.c_void_p, C.c_int64, C.c_int, C.c_void_p, C.c_void_p]),
     "opsnnPackB4": (C.c_int, [C.c_void_p, C.c_int, C.c_void_p, C.c_int64, C.c_void_p]),
     "opsnnQmmInt8": (C.c_int, [C.POINTER(OpsnnQmmArgs), C.c_void_p]),
+    "opsnnQmmInt8Static": (C.c_int, [C.POINTER(OpsnnQmmArgs), C.c_void_p]),
     "opsnnQmmBlockScale": (C.c_int, [C.POINTER(OpsnnQmmArgs), C.c_void_p]),
     "opsnnQmmMx": (C.c_int, [C.POINTER(OpsnnQmmArgs), C.c_void_p]),
     "opsnnQmmTc": (C.c_int, [C.POINTER(OpsnnQmmArgs), C.c_void_p]),
