@@ -98,14 +98,13 @@ __device__ __forceinline__ float e4m3_to_f32(uint32_t b)
 __device__ __forceinline__ uint32_t f32_to_e4m3_bits(float f)
 {
     const uint32_t u = f2u(f), sign = (u >> 24) & 0x80u, a = u & 0x7fffffffu;
-    if (a > 0x7f800000u || a >= 0x43f00000u) return sign | 0x7fu;     // NaN; >= 480
+    if (a > 0x43e80000u) return sign | 0x7fu;                          // NaN, and anything above 464 (the tie below the absent 480, which alone rounds to 448)
     if (a < 0x3a800000u) return sign;                                  // < 2^-10 rounds to zero
     int exp = (int)(a >> 23) - 127;
     if (exp < -6) exp = -6;                                            // subnormal quantum 2^-9
     const float q = u2f((uint32_t)(exp - 3 + 127) << 23);
     const float qinv = u2f((uint32_t)(127 + 3 - exp) << 23);           // 1 / q: both scalings are exact
     const float v = __fmul_rn(__builtin_rintf(__fmul_rn(u2f(a), qinv)), q);
-    if (v > 448.0f) return sign | 0x7eu;                               // 464 (the tie below the absent 480) rounds to 448
     if (v < 0.015625f) return sign | (uint32_t)__fmul_rn(v, 512.0f);
     const uint32_t vb = f2u(v);
     return sign | ((((vb >> 23) - 127 + 7) << 3) | ((vb >> 20) & 7u));

@@ -148,14 +148,16 @@ float orc_e5m2_to_f32(uint8_t b)
     else v = ldexpf((float)(4 + m), (int)e - 17);
     return (b & 0x80u) ? -v : v;
 }
-/* fp32 -> e4m3fn, round to nearest even; magnitudes that round above 448 and NaN give NaN (0x7f). */
+/* fp32 -> e4m3fn, round to nearest even; NaN and magnitudes that round above 448 (anything above the tie 464) give NaN
+ * (0x7f): the format has no infinity and the cast does not saturate -- the behaviour of torch.float8_e4m3fn, against which
+ * tests/test_oracle_pins.py compares this function over the whole fp32 range. */
 uint8_t orc_e4m3_from_f32(float f)
 {
     uint32_t u = f2u(f);
     uint8_t sign = (uint8_t)((u >> 24) & 0x80u);
     float a = fabsf(f);
     if (!(a == a)) return (uint8_t)(sign | 0x7f);
-    if (a >= 480.0f) return (uint8_t)(sign | 0x7f); /* 464 is the tie between 448 and the absent 480: stays 448 */
+    if (a > 464.0f) return (uint8_t)(sign | 0x7f);  /* 464 is the tie between 448 and the absent 480: it alone stays 448 */
     if (a < 0.0009765625f) return sign;              /* < 2^-10 -> 0 (tie at 2^-10 goes to even = 0) */
     int e;
     (void)frexpf(a, &e);                             /* a = fr * 2^e, fr in [0.5,1) */
@@ -165,7 +167,6 @@ uint8_t orc_e4m3_from_f32(float f)
     float n = a / q;                                 /* exact: power-of-two division */
     float r = nearbyintf(n);                         /* default rounding mode = nearest even */
     float v = r * q;
-    if (v > 448.0f) return (uint8_t)(sign | 0x7e);   /* 464 case rounds to 448 */
     /* encode v */
     if (v < 0.015625f) return (uint8_t)(sign | (uint8_t)(v * 512.0f));
     int e2;

@@ -282,8 +282,9 @@ def run_mx_aclnn(m, inp, M, K, N, tB, out_dtype, bias=None):
 # weight-only (aclnnWeightQuantBatchMatmulV2)
 # --------------------------------------------------------------------------------------------------
 def make_wq_inputs(m, M, K, N, seed, x_dt, w_dt, group, tW, with_offset=True, bias_dt=None, scale_lo=0.005, scale_hi=0.02,
-                   per_tensor=False):
-    """x ~N(0,1) in x_dt; weight int8 [-127,127] or int4 [-8,7]; scale U(lo,hi), offset U(-1,1) in x_dt."""
+                   per_tensor=False, mx_exp=(-6, 2)):
+    """x ~N(0,1) in x_dt; weight int8 [-127,127], int4 [-8,7], e4m3 ~N(0,1) or the 16 fp4 e2m1 codes; scale U(lo,hi) and
+    offset U(-1,1) in x_dt -- or, for fp4 weights, one e8m0 byte per 32 K with the exponent uniform in mx_exp (no offset)."""
     rng = np.random.default_rng(seed)
     x = orc.f32_to_b16(rng.normal(0, 1, size=(M, K)).astype(np.float32), x_dt)
     wshape = (N, K) if tW else (K, N)
@@ -293,20 +294,27 @@ def make_wq_inputs(m, M, K, N, seed, x_dt, w_dt, group, tW, with_offset=True, bi
         w = orc.pack_nibbles((rng.integers(-8, 8, size=wshape) & 15).astype(np.uint8))
     elif w_dt == m.ACL_FLOAT8_E4M3FN:
         w = gen_fp8(rng, wshape)
+    elif w_dt == m.ACL_FLOAT4_E2M1:
+        w = orc.pack_nibbles(rng.integers(0, 16, size=wshape, dtype=np.uint8))
     else:
         raise ValueError(w_dt)
     G = -(-K // group) if group > 0 else 1
     sshape = (1,) if per_tensor else ((N, G) if tW else (G, N))
+    bias = gen_bias(rng, N, bias_dt, m)
+    if w_dt == m.ACL_FLOAT4_E2M1:   # MX: e8m0 scales, group 32, no offset
+        assert group == 32 and not with_offset
+        scale = (127 + rng.integers(mx_exp[0], mx_exp[1] + 1, size=sshape)).astype(np.uint8)
+        return dict(x=x, w=w, scale=scale, offset=None, bias=bias, bias_dt=bias_dt, x_dt=x_dt, w_dt=w_dt, group=group, tW=tW,
+                    per_tensor=False, scale_dt=m.ACL_FLOAT8_E8M0)
     scale = orc.f32_to_b16(rng.uniform(scale_lo, scale_hi, size=sshape).astype(np.float32), x_dt)
     offset = orc.f32_to_b16(rng.uniform(-1, 1, size=sshape).astype(np.float32), x_dt) if with_offset else None
-    bias = gen_bias(rng, N, bias_dt, m)
     return dict(x=x, w=w, scale=scale, offset=offset, bias=bias, bias_dt=bias_dt, x_dt=x_dt, w_dt=w_dt, group=group, tW=tW,
-                per_tensor=per_tensor)
+                per_tensor=per_tensor, scale_dt=x_dt)
 
 
 def oracle_wq(m, inp, M, K, N, rows=None):
     x = inp["x"] if rows is None else np.ascontiguousarray(inp["x"][rows])
-    return orc.wqbmm(x, inp["x_dt"], inp["w"], inp["w_dt"], x.shape[0], K, N, inp["tW"], inp["scale"], inp["x_dt"],
+    return orc.wqbmm(x, inp["x_dt"], inp["w"], inp["w_dt"], x.shape[0], K, N, inp["tW"], inp["scale"], inp.get("scale_dt", inp["x_dt"]),
                      1 if inp["per_tensor"] else N, inp["offset"], inp["group"], inp["bias"], inp["bias_dt"] or 0)
 
 
@@ -325,7 +333,7 @@ def run_wq_aclnn(m, inp, M, K, N, v3=False, scale_2d=None):
         sshape, sst = (G, N), ((1, G) if tW else None)
     else:
         sshape, sst = (N,), None
-    sc = m.Tensor(sshape, inp["x_dt"], d["scale"], strides=sst)
+    sc = m.Tensor(sshape, inp.get("scale_dt", inp["x_dt"]), d["scale"], strides=sst)
     off = m.Tensor(sshape, inp["x_dt"], d["offset"], strides=sst) if inp["offset"] is not None else None
     bias = m.Tensor((N,), inp["bias_dt"], d["bias"]) if inp["bias"] is not None else None
     y = m.Tensor((M, N), inp["x_dt"], d_y)

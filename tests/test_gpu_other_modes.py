@@ -185,6 +185,15 @@ def test_mx_batched(gpu, M, K, N, batch):
     (5, 256, 64, "f16", "i8", 32, True, False, None),
     (33, 864, 212, "f16", "i4", 96, False, True, None),         # ragged groups (864 = 9 * 96)
     (4, 256, 128, "bf16", "e4m3", 0, True, False, "bf16"),
+    (33, 384, 130, "f16", "e4m3", 0, False, False, "f16"),     # fp8 weights, N-contiguous, fp16 (weight, scale and product rounded through fp16)
+    # mxfp4 weights with e8m0 scales per 32 K (_compute_mx): the reference's own case a16mxf4_nd_weight_fp4 (2 x 64 x 128,
+    # fp16, [K, N] storage), a decode shape in both layouts and both activation types, an odd number of 32-blocks, a bias
+    (2, 64, 128, "f16", "fp4", 32, False, False, None),
+    (1, 4096, 512, "f16", "fp4", 32, True, False, None),
+    (1, 4096, 512, "bf16", "fp4", 32, False, False, None),
+    (16, 1024, 384, "bf16", "fp4", 32, True, False, "bf16"),
+    (5, 96, 66, "f16", "fp4", 32, False, False, "f16"),
+    (40, 2048, 256, "f16", "fp4", 32, True, False, None),
     # shapes the streamlined decode kernel takes: vector scale loads (group 128 int4, K/128 a multiple of 8) ...
     (1, 2048, 528, "f16", "i4", 128, True, True, None),
     (16, 3072, 272, "f16", "i4", 128, True, False, "f16"),
@@ -214,7 +223,7 @@ def test_mx_batched(gpu, M, K, N, batch):
 def test_weight_only(gpu, M, K, N, x_dt, w_dt, group, tW, off, bias, use_plain):
     m = gpu
     dt = {"bf16": m.ACL_BF16, "f16": m.ACL_FLOAT16, "f32": m.ACL_FLOAT, "i8": m.ACL_INT8, "i4": m.ACL_INT4,
-          "e4m3": m.ACL_FLOAT8_E4M3FN, None: None}
+          "e4m3": m.ACL_FLOAT8_E4M3FN, "fp4": m.ACL_FLOAT4_E2M1, None: None}
     print(f"case wq M={M} K={K} N={N} x={x_dt} w={w_dt} g={group} tW={tW} off={off} bias={bias} plain={use_plain}", flush=True)
     inp = cases.make_wq_inputs(m, M, K, N, M * 7 + N, dt[x_dt], dt[w_dt], group, tW, off, dt[bias])
     want = cases.oracle_wq(m, inp, M, K, N)

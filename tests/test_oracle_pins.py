@@ -78,6 +78,21 @@ def test_e4m3_encode_matches_torch_in_range():
     assert np.array_equal(got[nz] & 0x80, ref[nz] & 0x80)  # sign (the sign of a zero result is not pinned)
 
 
+def test_e4m3_encode_out_of_range_matches_torch():
+    """The cast does not saturate: whatever rounds above 448 -- everything above the tie 464 -- becomes NaN, as in
+    torch.float8_e4m3fn (the cast the golden delegates to its dtype package inside compute_t_cg,
+    qbmmv4_kernel_golden.py:239).  Every 4097th fp32 bit pattern of the whole range plus a dense sweep of 440..500."""
+    bits = np.arange(0, 2 ** 32, 4097, dtype=np.uint64).astype(np.uint32)
+    f = np.concatenate([bits.view(np.float32), np.linspace(440, 500, 60001).astype(np.float32),
+                        -np.linspace(440, 500, 60001).astype(np.float32),
+                        np.float32([464.0, np.nextafter(np.float32(464), np.float32(500)), 480.0, np.inf, -np.inf, np.nan])])
+    ref = torch.from_numpy(f).to(torch.float8_e4m3fn).view(torch.uint8).numpy()
+    got = orc.f32_to_e4m3(f)
+    assert np.array_equal(got & 0x7f, ref & 0x7f)
+    nz = ((got & 0x7f) != 0) & ((got & 0x7f) != 0x7f)
+    assert np.array_equal(got[nz] & 0x80, ref[nz] & 0x80)
+
+
 def test_e8m0_and_fp4_tables():
     codes = np.arange(256, dtype=np.uint8)
     got = orc.e8m0_to_f32(codes)
@@ -321,6 +336,82 @@ def test_weight_only_dequant_double_rounding_matches_numpy_float16(w_bits):
     yt = orc.wqbmm(x, orc.F16, wt, orc.I8 if w_bits == 8 else orc.I4, K, K, N, True,
                    np.ascontiguousarray(s16.T).view(np.uint16), orc.F16, N, np.ascontiguousarray(off16.T).view(np.uint16), g, None, 0)
     assert np.array_equal(yt, y)
+
+
+def _mx_weight_case(rng, K, N, exps):
+    codes = rng.integers(0, 16, (K, N)).astype(np.uint8)
+    G = -(-K // 32)
+    e = rng.choice(np.asarray(exps), size=(G, N)).astype(np.int64)
+    return codes, (e + 127).astype(np.uint8), e
+
+
+def test_weight_only_mx_fp16_matches_numpy_float16_closed_form():
+    """_compute_mx (wqbmmv2_kernel_golden.py:300-352) with fp16 x: w = f16(fp4 * f16(2^e)) per 32 K.  x = identity makes
+    y the dequantised weight itself.  Exponents reach the fp16 subnormals (2^-24 is the smallest, 2^-25 and below round the
+    SCALE to zero; 0.5 * 2^-24 ties to zero, 1.5 * 2^-24 ties to 2 * 2^-24) and the largest scale that keeps 6 * 2^e
+    finite; three blocks (an odd count) along K."""
+    rng = np.random.default_rng(21)
+    K, N = 96, 40
+    codes, sbytes, e = _mx_weight_case(rng, K, N, list(range(-27, 14)))
+    s16 = np.ldexp(np.float32(1), e).astype(np.float32).astype(np.float16)             # the scale through fp16
+    want = (orc.E2M1_VALUES[codes] * np.repeat(s16.astype(np.float32), 32, 0)).astype(np.float16)
+    assert (s16 == 0).any() and (np.abs(want.astype(np.float32)) < 2.0 ** -14).any()   # flushed scales and subnormal weights occur
+    x = orc.f32_to_f16(np.eye(K, dtype=np.float32))
+    y = orc.wqbmm(x, orc.F16, orc.pack_nibbles(codes), orc.E2M1, K, K, N, False, sbytes, orc.E8M0, N, None, 32, None, 0)
+    z = want.view(np.uint16)
+    zero = ((y | z) & 0x7fff) == 0
+    assert np.array_equal(y[~zero], z[~zero])
+    # [N, K] storage of the weight with [N, K/32] scales gives the same result
+    yt = orc.wqbmm(x, orc.F16, orc.pack_nibbles(np.ascontiguousarray(codes.T)), orc.E2M1, K, K, N, True,
+                   np.ascontiguousarray(sbytes.T), orc.E8M0, N, None, 32, None, 0)
+    assert np.array_equal(yt, y)
+
+
+def test_weight_only_mx_fp16_scale_overflow():
+    """2^16 is not an fp16 number: the scale becomes infinity, every non-zero weight +-inf and a zero weight NaN; 2^14 keeps
+    4 * 2^14 = 65536 > 65504 -> inf but 3 * 2^14 finite.  One K element, x = 1, so nothing else enters the sum."""
+    codes = np.arange(16, dtype=np.uint8).reshape(1, 16)
+    x = orc.f32_to_f16(np.ones((1, 1), np.float32))
+    for e in (14, 16):
+        s16 = np.float32(2.0 ** e).astype(np.float16)
+        with np.errstate(over="ignore", invalid="ignore"):
+            want = (orc.E2M1_VALUES[codes] * np.float32(s16)).astype(np.float16)
+        y = orc.wqbmm(x, orc.F16, orc.pack_nibbles(codes), orc.E2M1, 1, 1, 16, False, np.full((1, 16), 127 + e, np.uint8),
+                      orc.E8M0, 16, None, 32, None, 0).view(np.float16)
+        assert np.array_equal(np.isnan(y), np.isnan(want))
+        ok = ~np.isnan(want)
+        assert np.array_equal(y[ok], want[ok])
+        assert np.isinf(want[0, 7]) and (e == 16 or np.isfinite(want[0, 5]))
+
+
+def test_weight_only_mx_bf16_matches_torch_bfloat16():
+    """bf16 x: the scale is NOT rounded (2^e is a bf16 number for every e8m0 byte but 0xFF) and fp4 * 2^e is exact in bf16
+    down to its subnormals; byte 0 is 2^-127."""
+    rng = np.random.default_rng(22)
+    K, N = 64, 24
+    codes, sbytes, e = _mx_weight_case(rng, K, N, [-127, -126, -100, -3, 0, 5, 60, 120])
+    prod = orc.E2M1_VALUES[codes].astype(np.float64) * np.repeat(np.ldexp(1.0, e), 32, 0)
+    want = torch.from_numpy(prod.astype(np.float32)).to(torch.bfloat16)
+    assert np.array_equal(want.float().numpy().astype(np.float64), prod)      # exact: nothing is rounded on this path
+    x = orc.f32_to_bf16(np.eye(K, dtype=np.float32))
+    y = orc.wqbmm(x, orc.BF16, orc.pack_nibbles(codes), orc.E2M1, K, K, N, False, sbytes, orc.E8M0, N, None, 32, None, 0)
+    z = want.view(torch.int16).numpy().view(np.uint16)
+    zero = ((y | z) & 0x7fff) == 0
+    assert np.array_equal(y[~zero], z[~zero])
+
+
+def test_weight_only_mx_full_product_against_float64():
+    """With power-of-two scales in a narrow band every product and partial sum of x (small integers) times the weight is
+    exact in fp32, so the result must equal the float64 matmul rounded once to the output type, whatever the order."""
+    rng = np.random.default_rng(23)
+    M, K, N = 7, 128, 20
+    codes, sbytes, e = _mx_weight_case(rng, K, N, [-2, -1, 0, 1, 2])
+    xi = rng.integers(-4, 5, (M, K)).astype(np.float32)
+    w = orc.E2M1_VALUES[codes].astype(np.float64) * np.repeat(np.ldexp(1.0, e), 32, 0)
+    want = (xi.astype(np.float64) @ w)
+    for dt, enc in ((orc.F16, orc.f32_to_f16), (orc.BF16, orc.f32_to_bf16)):
+        y = orc.wqbmm(enc(xi), dt, orc.pack_nibbles(codes), orc.E2M1, M, K, N, False, sbytes, orc.E8M0, N, None, 32, None, 0)
+        assert np.array_equal(y, enc(want.astype(np.float32)))
 
 
 def test_weight_only_bf16_dequant_matches_torch_bfloat16():
