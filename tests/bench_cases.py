@@ -10,13 +10,15 @@ import cases
 import oracle_api as orc
 
 
-# HBM-side traffic per step in bytes (read + written), from the hardware counters FETCH_SIZE and WRITE_SIZE of the
-# very same bench command, each scaled by what the counter reads for a byte transpose of known size; the runs and the
-# figures are in profiles/<kernel>_<workload>.txt.  Keyed by (config, M of the weight-only configs).
-MEASURED_TRAFFIC = {
-    (2, None): 104.5e6, (4, None): 824.4e6, (5, None): 1802.2e6,
-    (3, 1): 67.2e6, (3, 16): 69.2e6, (1, None): 9.2e6,
-    (6, None): 583.0e6, (7, None): 132.4e6, (8, None): 260.2e6, (9, None): 405.9e6,
+# HBM-side traffic per step in bytes (read + written) as the hardware counters of an EARLIER profiling run of the same
+# bench command gave it (profiles/<file>: FETCH_SIZE and WRITE_SIZE, each scaled by what the counter reads for a byte
+# transpose of known size).  bench.py does not measure it; it copies the figure and names the file.  A figure below the
+# algorithmic bytes (the counter under-reads 16-byte-per-lane streams) is not evidence and is reported as null.
+# Keyed by (config, M of the weight-only configs, variant).
+PROFILED_TRAFFIC = {
+    (2, None): (104.5e6, "profiles/qgemm_int8_w8a8_m2048_k4096_n11008.txt"),
+    (4, "fast"): (824.4e6, "profiles/qmm_fp8_block_m4096_k7168_n18432.txt"),
+    (5, None): (1802.2e6, "profiles/qgemm_mxfp4_b8_m4096_k8192_n8192.txt"),
 }
 
 
@@ -29,6 +31,15 @@ class Workload:
     flop = 0
     bytes = 0
     config = {}
+
+    variant = None
+    instr_peak_key = None   # matrix instruction actually issued, when it is not the operand dtype's
+
+    def begin(self):
+        pass
+
+    def end(self):
+        pass
 
     def step(self, stream):
         raise NotImplementedError
@@ -106,13 +117,21 @@ class Config2(Workload):
 
 
 class Config4(Workload):
-    """aclnnQuantMatmulV5, fp8 e4m3 x e4m3, G-B block scales (1x128 on x1, 128x128 on x2), bf16 output."""
-    peak_key, dtype = "fp8", "fp8_e4m3"
-    kernel = "qmm_fp8_block_kernel"
+    """aclnnQuantMatmulV5, fp8 e4m3 x e4m3, G-B block scales (1x128 on x1, 128x128 on x2), bf16 output.
+    Default arithmetic: e4m3 widened exactly to fp16 in registers, fp16 matrix instruction (exact products); `fast`
+    selects the 8-bit matrix instruction (opsnnSetFp8Fast)."""
+    peak_key = "fp8"
 
     def __init__(self, m, args, M=4096, K=7168, N=18432):
         self.m, self.M, self.K, self.N = m, M, K, N
         self.packed = args.layout == "packed"
+        self.fast = bool(getattr(args, "fp8_fast", False))
+        if self.fast:
+            self.dtype, self.kernel, self.instr_peak_key = "fp8_e4m3", "qmm_fp8_block_kernel (v_mfma_scale_f32_16x16x128_f8f6f4)", "fp8"
+        else:
+            self.dtype = "f16 products of e4m3 operands (widened exactly in registers), fp32 sums"
+            self.kernel, self.instr_peak_key = "qmm_fp8_exact_kernel (v_mfma_f32_16x16x32_f16)", "f16"
+        self.variant = "fast" if self.fast else "exact"
         self.inp = cases.make_blockscale_inputs(m, M, K, N, 0, self.packed, 1)
         self.d = {k: m.DeviceBuffer(host=v) for k, v in self.inp.items() if isinstance(v, np.ndarray)}
         self.d_out = m.DeviceBuffer(M * N * 2)
@@ -135,7 +154,14 @@ class Config4(Workload):
         self.flop = 2 * M * N * K
         self.bytes = M * K + K * N + 4 * M * KB + 4 * KB * NB + 2 * M * N
         self.config = {"workload": "config4: aclnnQuantMatmulV5 fp8 e4m3 G-B (1x128 / 128x128 scales), bf16 out", "M": M, "K": K,
-                       "N": N, "x2_layout": "K-contiguous (pre-packed offline)" if self.packed else "N-contiguous (re-laid out per call)"}
+                       "N": N, "arithmetic": "8-bit matrix instruction (opsnnSetFp8Fast(1))" if self.fast else "exact fp16 products (default)",
+                       "x2_layout": "K-contiguous (pre-packed offline)" if self.packed else "N-contiguous (re-laid out per call)"}
+
+    def begin(self):
+        self.m.lib().opsnnSetFp8Fast(1 if self.fast else 0)
+
+    def end(self):
+        self.m.lib().opsnnSetFp8Fast(0)
 
     def step(self, stream):
         m = self.m
@@ -206,53 +232,72 @@ class Config5(Workload):
 
 
 class ConfigWQ(Workload):
-    """aclnnWeightQuantBatchMatmulV2: config 1 (W8A16 per-channel bf16, M=16) and config 3 (W4A16 per-group fp16 decode)."""
+    """aclnnWeightQuantBatchMatmulV2: config 1 (W8A16 per-channel bf16, M=16) and config 3 (W4A16 per-group fp16 decode).
+    One object serves every M of config 3 (set_m) and both cache states (set_cold): the weight copies stay on the device."""
     bound = "hbm"
 
-    def __init__(self, m, args, config):
+    def __init__(self, m, args, config, max_m=None):
         self.m = m
         self.packed = args.layout == "packed"
         if config == 1:
             M, K, N, x_dt, w_dt, group, off = 16, 4096, 4096, m.ACL_BF16, m.ACL_INT8, 0, False
             self.dtype, lo, hi = "bf16 (int8 weights)", 1e-4, 0.06
-            name = "config1: aclnnWeightQuantBatchMatmulV2 W8A16 per-channel bf16"
+            self.name = "config1: aclnnWeightQuantBatchMatmulV2 W8A16 per-channel bf16"
         else:
-            M, K, N, x_dt, w_dt, group, off = (args.m or 16), 8192, 28672, m.ACL_FLOAT16, m.ACL_INT4, 128, True
+            M, K, N, x_dt, w_dt, group, off = (max_m or args.m or 16), 8192, 28672, m.ACL_FLOAT16, m.ACL_INT4, 128, True
             self.dtype, lo, hi = "f16 (int4 weights)", 0.005, 0.02
-            name = "config3: aclnnWeightQuantBatchMatmulV2 W4A16 per-group(128) fp16 decode"
-        self.M, self.K, self.N, self.group = M, K, N, group
-        self.kernel = "wqmm_resx_kernel" if (config == 3 and M <= 3) else ("wqmm_rows_kernel" if M > 48 else "wqmm_stream_kernel")
-        self.inp = cases.make_wq_inputs(m, M, K, N, 0, x_dt, w_dt, group, self.packed, off, None, lo, hi)
-        inp = self.inp
-        self.ncopies = 1
-        wbytes = inp["w"].nbytes
-        if args.cold:   # rotate through enough weight copies to exceed the 256 MB last-level cache
-            self.ncopies = max(2, int(np.ceil(600e6 / wbytes)))
+            self.name = "config3: aclnnWeightQuantBatchMatmulV2 W4A16 per-group(128) fp16 decode"
+        self.cfg, self.K, self.N, self.group, self.x_dt, self.w_dt, self.off = config, K, N, group, x_dt, w_dt, off
+        self.inp_full = cases.make_wq_inputs(m, M, K, N, 0, x_dt, w_dt, group, self.packed, off, None, lo, hi)
+        inp = self.inp_full
         self.d = {k: m.DeviceBuffer(host=v) for k, v in inp.items() if isinstance(v, np.ndarray) and k != "w"}
-        self.d_w = [m.DeviceBuffer(host=inp["w"]) for _ in range(self.ncopies)]
+        self.d_w = [m.DeviceBuffer(host=inp["w"])]
         self.d_y = m.DeviceBuffer(M * N * 2)
-        G = -(-K // group) if group > 0 else 1
-        self.t_x = m.Tensor((M, K), x_dt, self.d["x"])
-        self.t_w = [m.Tensor((K, N), w_dt, d, strides=(1, K) if self.packed else None) for d in self.d_w]
+        self.G = -(-K // group) if group > 0 else 1
         if group > 0:
-            sshape, sst = (G, N), ((1, G) if self.packed else None)
+            sshape, sst = (self.G, N), ((1, self.G) if self.packed else None)
         else:
             sshape, sst = (N,), None
         self.t_sc = m.Tensor(sshape, x_dt, self.d["scale"], strides=sst)
         self.t_off = m.Tensor(sshape, x_dt, self.d["offset"], strides=sst) if off else None
-        self.t_y = m.Tensor((M, N), x_dt, self.d_y)
+        self.ncopies = 1
+        self.i = 0
+        self.set_cold(bool(getattr(args, "cold", False)))
+        self.set_m(M)
+
+    def set_cold(self, cold):
+        """cold: rotate through enough weight copies to exceed the 256 MB last-level cache between two uses of one copy."""
+        m = self.m
+        want = max(2, int(np.ceil(600e6 / self.inp_full["w"].nbytes))) if cold else 1
+        while len(self.d_w) < want:
+            self.d_w.append(m.DeviceBuffer(host=self.inp_full["w"]))
+        self.ncopies = want
+        self.t_w = [m.Tensor((self.K, self.N), self.w_dt, d, strides=(1, self.K) if self.packed else None) for d in self.d_w[:want]]
+        if hasattr(self, "M"):
+            self.set_m(self.M)
+
+    def set_m(self, M):
+        m, K, N = self.m, self.K, self.N
+        self.M = M
+        self.inp = dict(self.inp_full, x=np.ascontiguousarray(self.inp_full["x"][:M]))
+        self.kernel = "wqmm_resx_kernel" if (self.cfg == 3 and M <= 3) else ("wqmm_rows_kernel" if M > 48 else "wqmm_stream_kernel")
+        self.t_x = m.Tensor((M, K), self.x_dt, self.d["x"])
+        self.t_y = m.Tensor((M, N), self.x_dt, self.d_y)
         rc, ws, ex = m.weight_quant_batch_matmul_get_workspace(self.t_x, self.t_w[0], self.t_sc, self.t_y, offset=self.t_off,
-                                                               group_size=group)
+                                                               group_size=self.group)
         m.check(rc, "phase 1")
         m.lib().aclDestroyAclOpExecutor(ex)
         self.ws = m.DeviceBuffer(ws) if ws else None
         self.ws_size = ws
         self.flop = 2 * M * N * K
-        wb = K * N * (1 if w_dt == m.ACL_INT8 else 0.5)
-        self.bytes = int(wb + 2 * M * K + 2 * M * N + 2 * G * N * (2 if off else 1))
-        self.config = {"workload": name, "M": M, "K": K, "N": N, "group": group, "weight_copies_rotated": self.ncopies,
+        wb = K * N * (1 if self.w_dt == m.ACL_INT8 else 0.5)
+        self.bytes = int(wb + 2 * M * K + 2 * M * N + 2 * self.G * N * (2 if self.off else 1))
+        self.variant = "cold" if self.ncopies > 1 else "warm"
+        self.config = {"workload": self.name, "M": M, "K": K, "N": N, "group": self.group,
+                       "cache": "cold (weight copies rotated, %d x %.0f MB)" % (self.ncopies, self.inp_full["w"].nbytes / 1e6)
+                                if self.ncopies > 1 else "warm (one weight copy, resident in the 256 MB last-level cache between steps)",
+                       "weight_copies_rotated": self.ncopies,
                        "weight_layout": "K-contiguous (pre-packed offline)" if self.packed else "N-contiguous (re-laid out per call)"}
-        self.i = 0
 
     def step(self, stream):
         m = self.m
@@ -264,11 +309,16 @@ class ConfigWQ(Workload):
         m.check(m.lib().aclnnWeightQuantBatchMatmulV2(self.ws.ptr if self.ws else None, self.ws_size, ex, stream.ptr), "phase 2")
 
     def cpu_baseline(self):
+        # bounded sample: at most the first 16 rows of x against the whole weight (the weight dequantisation dominates)
+        rows = min(self.M, 16)
+        inp = dict(self.inp, x=np.ascontiguousarray(self.inp["x"][:rows]))
         t0 = time.perf_counter()
-        cases.oracle_wq(self.m, self.inp, self.M, self.K, self.N)
+        cases.oracle_wq(self.m, inp, rows, self.K, self.N)
         t = time.perf_counter() - t0
-        return {"value": self.bytes / t / 1e9, "unit": "GB/s", "cores": _cores(), "kind": "port",
-                "sample": f"the whole workload once (oracle/liboracle.so, OpenMP), {t:.2f} s"}
+        nbytes = self.bytes - (self.M - rows) * 2 * (self.K + self.N)
+        what = "the whole workload once" if rows == self.M else f"the first {rows} of {self.M} rows of x against the whole weight"
+        return {"value": nbytes / t / 1e9, "unit": "GB/s", "cores": _cores(), "kind": "port",
+                "sample": f"{what} (oracle/liboracle.so, OpenMP), {t:.2f} s"}
 
 
 class PrepOp(Workload):
