@@ -25,6 +25,12 @@
 #include "launch.h"
 #include "qgemm_core.hip.h"
 
+// -DXABL=<bits> removes parts of the loop for timing harnesses (results are then wrong): 1 the conversions, 2 the fold,
+// 4 the global -> LDS copies, 8 the LDS reads, 16 the barrier.  Never set in the library build.
+#ifndef XABL
+#define XABL 0
+#endif
+
 namespace opsnn {
 
 struct Fp8xParams {
@@ -43,6 +49,9 @@ struct Fp8xParams {
     int rs_stride, cs_stride;
     const float* bias;
     int64_t bias_bs;
+#if QG_DBG
+    unsigned long long* dbg;   // timing harness only: per wave, loop clocks / barrier-wait clocks / K tiles
+#endif
 };
 
 __device__ __forceinline__ const int8_t* uniform_ptr(const int8_t* p)
@@ -74,6 +83,11 @@ __global__ __launch_bounds__(512, 1) void qmm_fp8_exact_kernel(Fp8xParams p, int
     constexpr int RPI = NT / CPR;                    // 64 tile rows per copy instruction of the workgroup
     constexpr int NA = BM / RPI, NB = BN / RPI;
     constexpr int CPT = NA + NB + (RC ? 0 : 1);
+    // Three stages: the tile being consumed, the next one (complete at this tile's barrier) and one more in flight, so a
+    // copy has two tile times to land.  With two stages a copy had one tile time, about 1.1 us of matrix work, and the
+    // loaded latency of an L2 miss is longer: the loop ran at the pace of the memory latency (measured: copies and
+    // barriers alone 0.70 ms of config 4's 1.0).
+    constexpr int STAGES = 3;
     extern __shared__ __attribute__((aligned(16))) char smem[];
 
     const int tid = threadIdx.x;
@@ -81,8 +95,15 @@ __global__ __launch_bounds__(512, 1) void qmm_fp8_exact_kernel(Fp8xParams p, int
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave >> 1, wn = wave & 1;
 
+    // Tile order: each XCD (own L2) gets a contiguous range of ids, and ids run down groups of GM row tiles and across
+    // the columns inside a group, so the 32 tiles an XCD works on at a time form a GM x (32 / GM) block that shares
+    // GM x1 panels and 32 / GM x2 panels (for GM = 4: 2 KB-steps of 256 KB instead of 557 KB with whole columns).
+    constexpr int GM = 4;
     const uint32_t t = xcd_remap(blockIdx.x, (uint32_t)(tiles_m * tiles_n));
-    const int tm = (int)(t % (uint32_t)tiles_m), tn = (int)(t / (uint32_t)tiles_m);
+    const uint32_t gsz_full = (uint32_t)(GM * tiles_n), grp = t / gsz_full, in_grp = t % gsz_full;
+    const int first_m = (int)grp * GM;
+    const int gh = tiles_m - first_m < GM ? tiles_m - first_m : GM;
+    const int tm = first_m + (int)(in_grp % (uint32_t)gh), tn = (int)(in_grp / (uint32_t)gh);
     const int64_t m0 = (int64_t)tm * BM, n0 = (int64_t)tn * BN;
     const int64_t bz = blockIdx.y;
     const int64_t lda = p.lda, ldb = p.ldb;
@@ -124,6 +145,7 @@ __global__ __launch_bounds__(512, 1) void qmm_fp8_exact_kernel(Fp8xParams p, int
         }
     }
     auto issue_piece = [&](int kt, int stage, int idx) {
+        if (XABL & 4) return;
         char* sA = smem + stage * STAGE + wave * 1024;
         char* sB = sA + A_BYTES;
         const int8_t* Ak = uniform_ptr(A + (int64_t)kt * BK);
@@ -134,7 +156,7 @@ __global__ __launch_bounds__(512, 1) void qmm_fp8_exact_kernel(Fp8xParams p, int
     };
     auto issue_tile = [&](int kt) {
 #pragma unroll
-        for (int idx = 0; idx < CPT; idx++) issue_piece(kt, kt & 1, idx);
+        for (int idx = 0; idx < CPT; idx++) issue_piece(kt, kt % STAGES, idx);
     };
 
     v4f acc[FN][FM];
@@ -143,34 +165,36 @@ __global__ __launch_bounds__(512, 1) void qmm_fp8_exact_kernel(Fp8xParams p, int
 #pragma unroll
         for (int j = 0; j < FM; j++) acc[i][j] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
 
-    // Fragment of a 16-row block, lane (row = lane%16, q = lane/16): the 32 bytes [32q, 32q+32) of the row's 128 bytes
-    // of K; instruction s of the chain of four takes bytes [32q + 8s, +8) from both operands (K is the contraction
-    // index: any assignment of K to lanes and steps is right as long as both operands use the same one).
+    // Fragment of a 16-row block, lane (row = lane%16, q = lane/16): the bytes [16q, 16q+16) and [64+16q, 64+16q+16) of
+    // the row's 128 bytes of K; instruction s of the chain of four takes eight of them from both operands (K is the
+    // contraction index: any assignment of K to lanes and steps is right as long as both operands use the same one).
     const int frow = lane & 15, fq = lane >> 4;
     const int key = (frow / RPW) & (CPR - 1);
-    const int ch0 = ((2 * fq) ^ key) << 4, ch1 = ((2 * fq + 1) ^ key) << 4;
+    const int ch0 = (fq ^ key) << 4, ch1 = ((4 + fq) ^ key) << 4;
     const int a_rowbase = (wm * TM + frow) * BK;
     const int b_rowbase = A_BYTES + (wn * TN + frow) * BK;
     auto load_frag = [&](const char* st, int rowbase) -> v8i {
+        if (XABL & 8) return v8i{lane + rowbase, 1, 2, 3, 4, 5, 6, 7} + (int)(size_t)st;
         const v4i lo = *(const v4i*)(st + rowbase + ch0);
         const v4i hi = *(const v4i*)(st + rowbase + ch1);
         return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
     };
 
     issue_tile(0);
-    if (KT > 1) {
-        issue_tile(1);
-        wait_vmcnt<CPT>();
-    } else {
-        wait_vmcnt<0>();
-    }
+    issue_tile(KT > 1 ? 1 : 0);   // (a K of one or two tiles repeats the last tile into stages nobody reads)
+    issue_tile(KT > 2 ? 2 : KT - 1);
+    wait_vmcnt<2 * CPT>();
     __builtin_amdgcn_s_barrier();
 
-    v8i fa_raw[FM], fb_raw[2];
-    v8h fa[FM][4], fb[4];
-    float sc[FM], s1raw[FM], s2raw = 0.0f, sc_last = 0.0f;
-    v4f part[2];
-    (void)sc; (void)s1raw; (void)s2raw; (void)sc_last; (void)part;
+    // Registers: fa[j][s] the x1 fragments of the current tile as fp16 (eight values per K step s), fbc[2][s] the current
+    // and the next x2 fragment as fp16, a_half[j] sixteen raw bytes per x1 fragment on their way to fp16 (first the low
+    // halves of the next tile, then its high halves), b_raw the raw bytes of the next x2 fragment.
+    v4i a_half[FM];
+    v8i b_raw;
+    v8h fa[FM][4], fbc[2][4];
+    float sc[FM], scp[FM], s1raw[FM], s2raw = 0.0f;
+    v4f part[2][FM];
+    (void)sc; (void)scp; (void)s1raw; (void)s2raw; (void)part;
     auto read_scales = [&](const char* st) {
         if constexpr (!RC) {
             const float* sS = (const float*)(st + A_BYTES + B_BYTES);
@@ -179,88 +203,154 @@ __global__ __launch_bounds__(512, 1) void qmm_fp8_exact_kernel(Fp8xParams p, int
             for (int j = 0; j < FM; j++) s1raw[j] = sS[wm * TM + j * 16 + frow];
         }
     };
-    {
+    auto widen4 = [&](int d, v8h& h, int half) {   // four bytes -> elements 4*half .. 4*half+3
+        if (XABL & 1) { h[4 * half] = __builtin_bit_cast(v2h, d)[0]; return; }
+        const v2h lo = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8((uint32_t)d, 1.0f, false);
+        const v2h hi = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8((uint32_t)d, 1.0f, true);
+        h[4 * half] = lo[0]; h[4 * half + 1] = lo[1]; h[4 * half + 2] = hi[0]; h[4 * half + 3] = hi[1];
+    };
+    {   // first tile: everything converted up front
         read_scales(smem);
 #pragma unroll
-        for (int j = 0; j < FM; j++) fa_raw[j] = load_frag(smem, a_rowbase + j * 16 * BK);
-        fb_raw[0] = load_frag(smem, b_rowbase);
+        for (int j = 0; j < FM; j++) {
+            const v8i r = load_frag(smem, a_rowbase + j * 16 * BK);
 #pragma unroll
-        for (int j = 0; j < FM; j++) sc[j] = 0.0f;
-        part[0] = part[1] = v4f{0.0f, 0.0f, 0.0f, 0.0f};   // folded with scale 0 into the first tile's sums
+            for (int s = 0; s < 4; s++) fa[j][s] = widen8(r[2 * s], r[2 * s + 1]);
+            a_half[j] = __builtin_shufflevector(r, r, 4, 5, 6, 7);   // converted once more behind the first instructions (same values)
+        }
+        b_raw = load_frag(smem, b_rowbase);
+#pragma unroll
+        for (int s = 0; s < 4; s++) fbc[0][s] = widen8(b_raw[2 * s], b_raw[2 * s + 1]);
+#pragma unroll
+        for (int j = 0; j < FM; j++) {
+            sc[j] = 0.0f;   // multiplies the zero partial sums folded during the first tile's first fragment
+            part[1][j] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
+        }
     }
-    constexpr int CPS = (CPT + FM - 1) / FM;   // copies issued behind each chain of the tile's last x2 fragment
+    constexpr int CPS = (CPT + 3) / 4;   // copies issued behind each of the four instruction groups of the tile's last x2 fragment
 
+    // Schedule.  A tile is FN x2 fragments; a fragment is four groups (K steps s) of FM matrix instructions, one per x1
+    // fragment j, i.e. FM interleaved chains, so no instruction waits for the one issued just before it.  Everything the
+    // vector ALU has to do rides behind those instructions, a few operations each:
+    //   * the fold of the previous fragment's partial sums (one fused multiply-add per instruction);
+    //   * the conversion of the next x2 fragment, requested at the start of this one, behind groups 2 and 3;
+    //   * the conversion of the next tile's x1 fragments: K steps 0 and 1 behind groups 2 and 3 of the tile's LAST fragment
+    //     (whose groups 0 and 1 were those steps' last readers; the bytes were requested behind the barrier, two groups
+    //     earlier), steps 2 and 3 behind groups 1 and 2 of the next tile's first.
+    // The barrier sits before the last fragment: the next tile is complete in LDS and every wave is done reading this one.
+    int cur = 0;
+#if QG_DBG
+    unsigned long long dbg_bar = 0, dbg_lgkm = 0;
+    const unsigned long long dbg_c0 = clock64();
+#endif
     for (int kt = 0; kt < KT; kt++) {
-        const char* st = smem + (kt & 1) * STAGE;
-        const char* stn = smem + ((kt + 1) & 1) * STAGE;
-        const int ktc = kt + 2 < KT ? kt + 2 : KT - 1;   // past the end the copies repeat the last tile into a stage nobody reads
+        const int nxt = cur == STAGES - 1 ? 0 : cur + 1;
+        const char* st = smem + cur * STAGE;
+        const char* stn = smem + nxt * STAGE;
+        const int ktc = kt + 3 < KT ? kt + 3 : KT - 1;   // past the end the copies repeat the last tile into a stage nobody reads
 #pragma unroll
         for (int i = 0; i < FN; i++) {
             if (i + 1 < FN) {
-                fb_raw[(i + 1) & 1] = load_frag(st, b_rowbase + (i + 1) * 16 * BK);
-                __builtin_amdgcn_sched_barrier(0);
-                __builtin_amdgcn_s_waitcnt(0xc07f | (2 << 8));   // lgkmcnt: all but the two reads just issued
+                b_raw = load_frag(st, b_rowbase + (i + 1) * 16 * BK);
             } else {
-                wait_vmcnt<0>();
+#if QG_DBG
+                const unsigned long long c0 = clock64();
+#endif
+                wait_vmcnt<CPT>();   // tile kt+1 has landed (this thread's part); tile kt+2 may still be in flight
                 wait_lgkmcnt0();
-                __builtin_amdgcn_s_barrier();   // tile kt+1 is complete in LDS; every wave has read all it needs of tile kt
+#if QG_DBG
+                const unsigned long long c1 = clock64();
+#endif
+                if (!(XABL & 16)) __builtin_amdgcn_s_barrier();   // tile kt+1 is complete in LDS; every wave is done reading tile kt
+#if QG_DBG
+                dbg_lgkm += c1 - c0; dbg_bar += clock64() - c1;
+#endif
                 __builtin_amdgcn_sched_barrier(0);
-                read_scales(stn);
-                fb_raw[0] = load_frag(stn, b_rowbase);
-            }
-            __builtin_amdgcn_sched_barrier(0);
-            if (i == 0) {   // this tile's x1 fragments (requested behind the previous tile's barrier) and scales
+                b_raw = load_frag(stn, b_rowbase);
 #pragma unroll
                 for (int j = 0; j < FM; j++)
+                    if (!(XABL & 8)) a_half[j] = *(const v4i*)(stn + a_rowbase + j * 16 * BK + ch0);
+                read_scales(stn);
+            }
+            if (!RC && i == 0) {
 #pragma unroll
-                    for (int s = 0; s < 4; s++) fa[j][s] = widen8(fa_raw[j][2 * s], fa_raw[j][2 * s + 1]);
-                if constexpr (!RC) {
-                    sc_last = sc[FM - 1];
-#pragma unroll
-                    for (int j = 0; j < FM; j++) sc[j] = s1raw[j] * s2raw;
+                for (int j = 0; j < FM; j++) {
+                    scp[j] = sc[j];
+                    sc[j] = s1raw[j] * s2raw;
                 }
             }
-#pragma unroll
-            for (int s = 0; s < 4; s++) fb[s] = widen8(fb_raw[i & 1][2 * s], fb_raw[i & 1][2 * s + 1]);
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-            for (int j = 0; j < FM; j++) {
-                const int pi = (i * FM + j) & 1;
-                if constexpr (RC) {
+            for (int s = 0; s < 4; s++) {
 #pragma unroll
-                    for (int s = 0; s < 4; s++) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fb[s], fa[j][s], acc[i][j], 0, 0, 0);
-                } else {
-                    v4f c = v4f{0.0f, 0.0f, 0.0f, 0.0f};
+                for (int j = 0; j < FM; j++) {
+                    if constexpr (RC) {
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fbc[i & 1][s], fa[j][s], acc[i][j], 0, 0, 0);
+                    } else {
+                        if (XABL & 128) {   // partial sums in accumulation registers
+                            if (s == 0) asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, 0" : "=a"(part[i & 1][j]) : "v"(fbc[i & 1][s]), "v"(fa[j][s]));
+                            else asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(part[i & 1][j]) : "v"(fbc[i & 1][s]), "v"(fa[j][s]));
+                        } else
+                        part[i & 1][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fbc[i & 1][s], fa[j][s], s == 0 ? v4f{0.0f, 0.0f, 0.0f, 0.0f} : part[i & 1][j], 0, 0, 0);
+                        // fold element j of x1 fragment s of the previous x2 fragment (for i == 0: the previous tile's last, with its scales)
+                        if (XABL & 2) {
+                            if (kt == KT - 1 && i == FN - 1 && s == 3) acc[0][0][j] += part[1][j][0] + part[0][j][1];
+                        } else if (XABL & 32) {   // same count of fused multiply-adds, but none reads a matrix-instruction result
+                            acc[i][s][j] = __builtin_fmaf(s1raw[j], sc[s], acc[i][s][j]);
+                            if (kt == KT - 1 && i == FN - 1 && s == 3) acc[0][0][j] += part[1][j][0] + part[0][j][1];
+                        } else if (XABL & 64) {   // the whole fold of the previous fragment in one burst behind the first instruction of group 1
+                            if (s == 1 && j == 0) {
 #pragma unroll
-                    for (int s = 0; s < 4; s++) c = __builtin_amdgcn_mfma_f32_16x16x32_f16(fb[s], fa[j][s], c, 0, 0, 0);
-                    part[pi] = c;
-                }
-                __builtin_amdgcn_sched_barrier(0);
-                if (i == FN - 1) {
-                    fa_raw[j] = load_frag(stn, a_rowbase + j * 16 * BK);
+                                for (int jj = 0; jj < FM; jj++)
 #pragma unroll
-                    for (int c = j * CPS; c < (j + 1) * CPS && c < CPT; c++) issue_piece(ktc, kt & 1, c);
+                                    for (int r = 0; r < 4; r++) {
+                                        if (i > 0) acc[i - 1][jj][r] = __builtin_fmaf(part[(i - 1) & 1][jj][r], sc[jj], acc[i - 1][jj][r]);
+                                        else acc[FN - 1][jj][r] = __builtin_fmaf(part[1][jj][r], scp[jj], acc[FN - 1][jj][r]);
+                                    }
+                            }
+                        } else if (i > 0) acc[i - 1][s][j] = __builtin_fmaf(part[(i - 1) & 1][s][j], sc[s], acc[i - 1][s][j]);
+                        else acc[FN - 1][s][j] = __builtin_fmaf(part[1][s][j], scp[s], acc[FN - 1][s][j]);
+                    }
+                    if (s >= 2) {   // next x2 fragment: half a K step per instruction
+                        const int idx = (s - 2) * 4 + j;
+                        widen4(b_raw[idx], fbc[(i + 1) & 1][idx / 2], idx % 2);
+                    }
+                    if (XABL & 1) {
+                        if (i == FN - 1 && s >= 2) fa[j][s - 2][0] = __builtin_bit_cast(v2h, a_half[j][2 * (s - 2)])[0];
+                        if (i == 0 && (s == 1 || s == 2)) fa[j][1 + s][0] = __builtin_bit_cast(v2h, a_half[j][2 * (s - 1)])[0];
+                    } else {
+                    if (i == FN - 1 && s >= 2)                // next tile's x1 fragments, K step s - 2 (low halves)
+                        fa[j][s - 2] = widen8(a_half[j][2 * (s - 2)], a_half[j][2 * (s - 2) + 1]);
+                    if (i == 0 && (s == 1 || s == 2))         // this tile's x1 fragments, K steps 2 and 3 (high halves)
+                        fa[j][1 + s] = widen8(a_half[j][2 * (s - 1)], a_half[j][2 * (s - 1) + 1]);
+                    }
                     __builtin_amdgcn_sched_barrier(0);
                 }
-                if constexpr (!RC) {   // fold the pair before this one
-                    if (j > 0) {
+                if (i == FN - 1) {
+                    if (s == 3) {   // the low halves are converted: fetch the high halves into the same registers
 #pragma unroll
-                        for (int r = 0; r < 4; r++) acc[i][j - 1][r] = __builtin_fmaf(part[pi ^ 1][r], sc[j - 1], acc[i][j - 1][r]);
-                    } else if (i > 0) {
-#pragma unroll
-                        for (int r = 0; r < 4; r++) acc[i - 1][FM - 1][r] = __builtin_fmaf(part[pi ^ 1][r], sc[FM - 1], acc[i - 1][FM - 1][r]);
-                    } else {   // the previous tile's last pair, with that tile's scale
-#pragma unroll
-                        for (int r = 0; r < 4; r++) acc[FN - 1][FM - 1][r] = __builtin_fmaf(part[pi ^ 1][r], sc_last, acc[FN - 1][FM - 1][r]);
+                        for (int j = 0; j < FM; j++)
+                            if (!(XABL & 8)) a_half[j] = *(const v4i*)(stn + a_rowbase + j * 16 * BK + ch1);
                     }
+#pragma unroll
+                    for (int c = s * CPS; c < (s + 1) * CPS && c < CPT; c++) issue_piece(ktc, cur, c);   // tile kt+3 into the stage of tile kt
                     __builtin_amdgcn_sched_barrier(0);
                 }
             }
         }
+        cur = nxt;
     }
+#if QG_DBG
+    if (lane == 0 && p.dbg) {
+        unsigned long long* d = p.dbg + ((size_t)blockIdx.x * 8 + wave) * 4;
+        d[0] = clock64() - dbg_c0; d[1] = dbg_bar; d[2] = dbg_lgkm; d[3] = (unsigned long long)KT;
+    }
+#endif
     if constexpr (!RC) {
 #pragma unroll
-        for (int r = 0; r < 4; r++) acc[FN - 1][FM - 1][r] = __builtin_fmaf(part[(FN * FM - 1) & 1][r], sc[FM - 1], acc[FN - 1][FM - 1][r]);
+        for (int j = 0; j < FM; j++)
+#pragma unroll
+            for (int r = 0; r < 4; r++) acc[FN - 1][j][r] = __builtin_fmaf(part[(FN - 1) & 1][j][r], sc[j], acc[FN - 1][j][r]);
     }
     wait_lgkmcnt0();   // the reads and copies past the last tile land before LDS is reused
     wait_vmcnt<0>();
@@ -273,7 +363,7 @@ __global__ __launch_bounds__(512, 1) void qmm_fp8_exact_kernel(Fp8xParams p, int
     typedef v4i __attribute__((may_alias)) v4i_a;
     constexpr int EP_PITCH = TN * 2 + 16;
     char* ep = smem + wave * (16 * EP_PITCH);
-    static_assert(8 * 16 * EP_PITCH <= 2 * STAGE, "epilogue staging fits in the operand stages");
+    static_assert(8 * 16 * EP_PITCH <= STAGES * STAGE, "epilogue staging fits in the operand stages");
     uint16_t* out = (uint16_t*)p.out + bz * p.M * p.N;
     const bool vec_ok = (p.N % 8) == 0 && ((uintptr_t)p.out % 16) == 0;
     const int er = lane >> 3, ec = lane & 7;
@@ -327,7 +417,7 @@ static int launch_fp8_exact(const Fp8xParams& p, int64_t batch, hipStream_t st)
 {
     const int tiles_m = (int)((p.M + 255) / 256), tiles_n = (int)((p.N + 127) / 128);
     dim3 grid((unsigned)(tiles_m * tiles_n), (unsigned)batch);
-    const size_t lds = 2 * (size_t)(256 * 128 + 128 * 128 + (RC ? 0 : 512 * 4));
+    const size_t lds = 3 * (size_t)(256 * 128 + 128 * 128 + (RC ? 0 : 512 * 4));
     auto k = qmm_fp8_exact_kernel<OUT_DT, RC>;
     static bool attr_set = false;
     if (!attr_set) {
