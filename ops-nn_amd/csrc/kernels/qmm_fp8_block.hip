@@ -191,7 +191,6 @@ __global__ __launch_bounds__(WGM * 128, 1) void qmm_fp8_block_kernel(Fp8BlkParam
     // operands use the same one.)
     const int frow = lane & 15, fq = lane >> 4;
     const int key = (frow / RPW) & (CPR - 1);
-    const int ch0 = ((2 * fq) ^ key) << 4, ch1 = ((2 * fq + 1) ^ key) << 4;
     const int a_rowbase = (wm * TM + frow) * BK;
     const int b_rowbase = A_BYTES + (wn * TN + frow) * BKB;
     // MX mode, where the position of K matters: the instruction takes registers 0..3 of lane group q as the 16 elements
@@ -200,8 +199,11 @@ __global__ __launch_bounds__(WGM * 128, 1) void qmm_fp8_block_kernel(Fp8BlkParam
     // (measured on the device with one-hot scale patterns; the 32x32x64 form is built the same way from two lane halves).
     const int mx0 = (fq ^ key) << 4, mx1 = ((4 + fq) ^ key) << 4;
     auto load_frag = [&](const char* st, int rowbase) -> v8i {
-        const v4i lo = *(const v4i*)(st + rowbase + (MX ? mx0 : ch0));
-        const v4i hi = *(const v4i*)(st + rowbase + (MX ? mx1 : ch1));
+        // every mode reads the chunk pair (q, 4 + q): for the modes without scales inside the instruction any assignment
+        // of K to lanes is right, and this one is free of LDS bank conflicts (the pair (2q, 2q + 1) cost four conflict
+        // cycles per read: SQ_LDS_BANK_CONFLICT 68M -> 1.8M cycles on config 4 in the kernel of qmm_fp8_exact.hip)
+        const v4i lo = *(const v4i*)(st + rowbase + mx0);
+        const v4i hi = *(const v4i*)(st + rowbase + mx1);
         return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
     };
     // fp4 x2 fragment (W4): a 4-bit operand is four registers, and lane group q holds the 32 CONSECUTIVE elements
