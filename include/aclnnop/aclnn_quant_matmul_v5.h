@@ -27,8 +27,9 @@ extern "C" {
  *  x2        same family as x1, [.., k, n] (or [.., n, k] if transposeX2)
  *  x1Scale   optional; fp32 per-token [m], fp32 block scale [m, ceil(k/128)] or e8m0 [m, ceil(k/64), 2]
  *  x2Scale   required; fp32/bf16 [1] or [n], uint64/int64 packed, fp32 block scale, or e8m0
- *  yScale, x1Offset, yOffset   must be NULL on this route
- *  x2Offset  only with int8 inputs and int8 output
+ *  yScale    uint64 [1] or [n] output scale of the fp8 x fp4 group-scale mode (x2Scale bf16/fp16 [ceil(k/gsK), n]); NULL otherwise
+ *  x1Offset, yOffset   must be NULL
+ *  x2Offset  fp32 [1] or [n] with int8 inputs and int8 output; fp16 [ceil(k/256), n] in the int4 K-group mode
  *  bias      optional [n] (int32 / bf16 / fp16 / fp32 depending on the mode)
  *  groupSize gsK | gsN << 16 | gsM << 32; 0 outside block/MX modes
  */

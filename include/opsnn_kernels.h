@@ -101,6 +101,12 @@ OPSNN_API int opsnnQmmBlockScale(const OpsnnQmmArgs* a, void* stream);
  * The initial value is taken from the environment variable OPSNN_FP8_FAST (unset or 0: exact). */
 OPSNN_API void opsnnSetFp8Fast(int fast);
 OPSNN_API int opsnnGetFp8Fast(void);
+/* Routing switches for tests and tuning, process-wide; each starts from the environment variable of the same meaning,
+ * read once when the library is loaded (OPSNN_FORCE_PLAIN, OPSNN_MX8_WIDE):
+ *   opsnnSetForcePlain(1)  every call runs on the plain one-thread-per-output kernels (bit-identical to the CPU oracle);
+ *   opsnnSetMx8Wide(n)     MXFP8 on the four-wave kernel with 256 x 32n tiles (n = 8, 9), 0 never, -1 automatic. */
+OPSNN_API void opsnnSetForcePlain(int on);
+OPSNN_API void opsnnSetMx8Wide(int n);
 /* MX: fp4/fp8 operands, e8m0 scale per 32 K. out = (x1*s1) @ (x2*s2) + fp32 bias. */
 OPSNN_API int opsnnQmmMx(const OpsnnQmmArgs* a, void* stream);
 /* Per-tensor / per-channel scales (T-T, T-C): int8 or fp8 (e4m3, e5m2) operands;

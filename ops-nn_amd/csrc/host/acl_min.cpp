@@ -6,9 +6,28 @@
 #include <cstring>
 #include <mutex>
 
+#include <mutex>
+#include <unordered_set>
+
 #include "tensor.h"
 
 namespace opsnn {
+
+namespace {
+std::mutex g_exec_mutex;
+std::unordered_set<const void*> g_live_executors;
+}
+void* executor_publish(void* ex)
+{
+    std::lock_guard<std::mutex> lock(g_exec_mutex);
+    g_live_executors.insert(ex);
+    return ex;
+}
+bool executor_claim(const void* ex)
+{
+    std::lock_guard<std::mutex> lock(g_exec_mutex);
+    return g_live_executors.erase(ex) != 0;
+}
 
 static thread_local char g_err[1024] = "";
 
@@ -252,7 +271,7 @@ aclnnStatus aclGetFormat(const aclTensor* tensor, aclFormat* format)
 }
 aclnnStatus aclDestroyAclOpExecutor(aclOpExecutor* executor)
 {
-    if (executor && executor->magic == kExecutorMagic) { executor->magic = 0; delete executor; }
+    if (executor && opsnn::executor_claim(executor)) delete executor;   // unknown, already run or already destroyed: nothing to do
     return ACLNN_SUCCESS;
 }
 

@@ -71,7 +71,7 @@ aclnnStatus aclnnDynamicBlockQuantGetWorkspaceSize(const aclTensor* x_, double m
     a.batch = x.rank() == 3 ? x.dim(0) : 1; a.rows = x.dim(-2); a.cols = x.dim(-1);
     a.row_block = rowBlockSize; a.col_block = colBlockSize; a.min_scale = minScale; a.force_variant = 0;
     *workspaceSize = 0;
-    *executor = ex.release();
+    *executor = (aclOpExecutor*)executor_publish(ex.release());
     return ACLNN_SUCCESS;
 }
 
@@ -99,7 +99,7 @@ aclnnStatus aclnnDynamicBlockQuant(void*, uint64_t, aclOpExecutor* executor, acl
 {
     clear_error();
     if (!executor) FAIL(ACLNN_ERR_PARAM_NULLPTR, "%s: executor is null", kApi);
-    if (executor->magic != kExecutorMagic) INVALID("%s: executor is not valid (already run or destroyed)", kApi);
+    if (!executor_claim(executor)) INVALID("%s: executor is not valid (already run or destroyed)", kApi);
     std::unique_ptr<aclOpExecutor> ex(executor);
     ex->magic = 0;
     if (ex->kind != OpKind::BlockQuant) INVALID("%s: executor belongs to another operator", kApi);

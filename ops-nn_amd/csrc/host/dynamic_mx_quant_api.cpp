@@ -75,7 +75,7 @@ aclnnStatus aclnnDynamicMxQuantGetWorkspaceSize(const aclTensor* x_, int64_t axi
     *workspaceSize = 0;
     if (x.empty()) {
         ex->kind = OpKind::None;
-        *executor = ex.release();
+        *executor = (aclOpExecutor*)executor_publish(ex.release());
         return ACLNN_SUCCESS;
     }
     ex->kind = OpKind::MxQuant;
@@ -85,7 +85,7 @@ aclnnStatus aclnnDynamicMxQuantGetWorkspaceSize(const aclTensor* x_, int64_t axi
     a.scale = const_cast<void*>(sc.ptr_at(0));
     a.cols = x.dim(-1); a.rows = x.numel() / a.cols; a.force_variant = 0;
     a.block = blocksize; a.scale_alg = (int)scaleAlg;
-    *executor = ex.release();
+    *executor = (aclOpExecutor*)executor_publish(ex.release());
     return ACLNN_SUCCESS;
 }
 
@@ -128,7 +128,7 @@ aclnnStatus aclnnDynamicMxQuant(void*, uint64_t, aclOpExecutor* executor, aclrtS
 {
     clear_error();
     if (!executor) FAIL(ACLNN_ERR_PARAM_NULLPTR, "%s: executor is null", kApi);
-    if (executor->magic != kExecutorMagic) INVALID("%s: executor is not valid (already run or destroyed)", kApi);
+    if (!executor_claim(executor)) INVALID("%s: executor is not valid (already run or destroyed)", kApi);
     std::unique_ptr<aclOpExecutor> ex(executor);
     ex->magic = 0;
     if (ex->kind == OpKind::None) return ACLNN_SUCCESS;

@@ -96,7 +96,7 @@ aclnnStatus get_workspace(const char* api, const aclTensor* x_, const aclTensor*
     *workspaceSize = 0;
     if (x.empty() || y.empty() || sc.empty()) {   // :366-371
         ex->kind = OpKind::None;
-        *executor = ex.release();
+        *executor = (aclOpExecutor*)executor_publish(ex.release());
         return ACLNN_SUCCESS;
     }
     // what this build does not run
@@ -120,7 +120,7 @@ aclnnStatus get_workspace(const char* api, const aclTensor* x_, const aclTensor*
     if (gi.present) { a.group_index = gi.ptr_at(0); a.group_index_dtype = gi.dtype; a.groups = gi.dim(0); }
     a.quant_mode = pertensor ? 1 : perchannel ? 2 : 0;
     a.chan_rows = perchannel ? x.dim(-2) : 0;
-    *executor = ex.release();
+    *executor = (aclOpExecutor*)executor_publish(ex.release());
     return ACLNN_SUCCESS;
 }
 
@@ -128,7 +128,7 @@ aclnnStatus run(const char* api, aclOpExecutor* executor, aclrtStream stream)
 {
     clear_error();
     if (!executor) FAIL(ACLNN_ERR_PARAM_NULLPTR, "%s: executor is null", api);
-    if (executor->magic != kExecutorMagic) INVALID("%s: executor is not valid (already run or destroyed)", api);
+    if (!executor_claim(executor)) INVALID("%s: executor is not valid (already run or destroyed)", api);
     std::unique_ptr<aclOpExecutor> ex(executor);
     ex->magic = 0;
     if (ex->kind == OpKind::None) return ACLNN_SUCCESS;

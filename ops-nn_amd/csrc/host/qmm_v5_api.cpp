@@ -521,7 +521,7 @@ extern "C" aclnnStatus aclnnQuantMatmulV5GetWorkspaceSize(const aclTensor* x1, c
         int64_t n = c.tB ? c.x2.dim(-2) : c.x2.dim(-1);
         if (m == 0 || n == 0) {
             *workspaceSize = 0;
-            *executor = ex.release();
+            *executor = (aclOpExecutor*)executor_publish(ex.release());
             return ACLNN_SUCCESS;
         }
     }
@@ -674,7 +674,7 @@ extern "C" aclnnStatus aclnnQuantMatmulV5GetWorkspaceSize(const aclTensor* x1, c
     }
     ex->workspace_size = opsnnQmmWorkspace(&a, mode);
     *workspaceSize = ex->workspace_size;
-    *executor = ex.release();
+    *executor = (aclOpExecutor*)executor_publish(ex.release());
     return ACLNN_SUCCESS;
 }
 
@@ -683,7 +683,7 @@ extern "C" aclnnStatus aclnnQuantMatmulV5(void* workspace, uint64_t workspaceSiz
 {
     clear_error();
     if (!executor) FAIL(ACLNN_ERR_PARAM_NULLPTR, "aclnnQuantMatmulV5: executor is null");
-    if (executor->magic != kExecutorMagic) INVALID("aclnnQuantMatmulV5: executor is not valid (already run or destroyed)");
+    if (!executor_claim(executor)) INVALID("aclnnQuantMatmulV5: executor is not valid (already run or destroyed)");
     std::unique_ptr<aclOpExecutor> ex(executor);  // consumed by this call
     ex->magic = 0;
     if (ex->kind == OpKind::None) return ACLNN_SUCCESS;

@@ -38,6 +38,13 @@ struct aclOpExecutorImpl {
     const char* api = "";
 };
 
+// Live executors.  Phase 1 hands an executor over with executor_publish(); phase 2 and aclDestroyAclOpExecutor take it
+// back with executor_claim(), which succeeds once per published pointer.  A handle that was already run or destroyed
+// is recognised by its absence from the set, without reading through the (freed) pointer.
+struct aclOpExecutorImpl;
+void* executor_publish(void* ex);
+bool executor_claim(const void* ex);
+
 // Thread-local last-error text (aclGetRecentErrMsg).
 void set_error(const char* fmt, ...) __attribute__((format(printf, 1, 2)));
 void clear_error();

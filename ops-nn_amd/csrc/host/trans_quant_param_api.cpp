@@ -56,7 +56,7 @@ aclnnStatus get_workspace(const char* api, const aclTensor* scale_, const aclTen
     ex->tqp.round_mode = (int)roundMode;
     ex->tqp.out = (uint64_t*)const_cast<void*>(out.ptr_at(0));
     *workspaceSize = 0;
-    *executor = ex.release();
+    *executor = (aclOpExecutor*)executor_publish(ex.release());
     return ACLNN_SUCCESS;
 }
 
@@ -64,7 +64,7 @@ aclnnStatus run(const char* api, aclOpExecutor* executor, aclrtStream stream)
 {
     clear_error();
     if (!executor) FAIL(ACLNN_ERR_PARAM_NULLPTR, "%s: executor is null", api);
-    if (executor->magic != kExecutorMagic) INVALID("%s: executor is not valid (already run or destroyed)", api);
+    if (!executor_claim(executor)) INVALID("%s: executor is not valid (already run or destroyed)", api);
     std::unique_ptr<aclOpExecutor> ex(executor);
     ex->magic = 0;
     if (ex->kind != OpKind::TransQuantParam) INVALID("%s: executor belongs to another operator", api);

@@ -180,7 +180,7 @@ aclnnStatus get_workspace(const char* api, const aclTensor* x_, const aclTensor*
     a.y = const_cast<void*>(y.ptr_at(0));
     ex->workspace_size = opsnnWqmmWorkspace(&a);
     *workspaceSize = ex->workspace_size;
-    *executor = ex.release();
+    *executor = (aclOpExecutor*)executor_publish(ex.release());
     return ACLNN_SUCCESS;
 }
 
@@ -188,7 +188,7 @@ aclnnStatus run(const char* api, void* workspace, uint64_t workspaceSize, aclOpE
 {
     clear_error();
     if (!executor) FAIL(ACLNN_ERR_PARAM_NULLPTR, "%s: executor is null", api);
-    if (executor->magic != kExecutorMagic) INVALID("%s: executor is not valid (already run or destroyed)", api);
+    if (!executor_claim(executor)) INVALID("%s: executor is not valid (already run or destroyed)", api);
     std::unique_ptr<aclOpExecutor> ex(executor);
     ex->magic = 0;
     if (ex->kind == OpKind::None) return ACLNN_SUCCESS;

@@ -24,12 +24,18 @@ uint64_t mx_workspace_bytes(const OpsnnQmmArgs& a);
 
 using namespace opsnn;
 
-// OPSNN_FORCE_PLAIN=1 routes every call to the plain kernels (used by the parity tests).
-extern "C" __attribute__((visibility("hidden"))) bool opsnn_force_plain()
-{
-    const char* e = getenv("OPSNN_FORCE_PLAIN");
-    return e && *e && *e != '0';
-}
+// Routing switches for tests and tuning, process-wide.  Each starts from an environment variable read ONCE when the
+// library is loaded (no getenv on the call path) and can be changed at run time through its setter.
+//   OPSNN_FORCE_PLAIN=1 / opsnnSetForcePlain(1): every call runs on the plain one-thread-per-output kernels (the parity
+//   tests compare them bit for bit with the oracle);
+//   OPSNN_MX8_WIDE=n / opsnnSetMx8Wide(n): MXFP8 on the four-wave kernel with 256 x 32n tiles, n = 8 or 9; 0 never; -1 the
+//   selector decides (default).
+static int g_force_plain = [] { const char* e = getenv("OPSNN_FORCE_PLAIN"); return (e && *e && *e != '0') ? 1 : 0; }();
+static int g_mx8_wide = [] { const char* e = getenv("OPSNN_MX8_WIDE"); return e ? atoi(e) : -1; }();
+extern "C" void opsnnSetForcePlain(int on) { __atomic_store_n(&g_force_plain, on ? 1 : 0, __ATOMIC_RELAXED); }
+extern "C" void opsnnSetMx8Wide(int n) { __atomic_store_n(&g_mx8_wide, n, __ATOMIC_RELAXED); }
+extern "C" __attribute__((visibility("hidden"))) bool opsnn_force_plain() { return __atomic_load_n(&g_force_plain, __ATOMIC_RELAXED) != 0; }
+extern "C" __attribute__((visibility("hidden"))) int opsnn_mx8_wide() { return __atomic_load_n(&g_mx8_wide, __ATOMIC_RELAXED); }
 
 // fp8 x fp8 arithmetic of the block-scale and row/column-scale modes: 0 (default) exact products and sums on the fp16
 // matrix instruction, 1 the 8-bit matrix instruction (about 1.5x faster, sums aligned in a narrower window).  The

@@ -470,6 +470,7 @@ static int launch_fp8_block(const Fp8BlkParams& p, int64_t batch, hipStream_t st
 }
 
 int launch_mxfp8_wide(const QgemmParams& p, int fn, int64_t batch, int out_dt, hipStream_t st);   // qmm_int8_wide.hip
+extern "C" int opsnn_mx8_wide();   // dispatch.hip
 
 // MXFP8 (e4m3 x e4m3, e8m0 scale per 32 K) on the same kernel in MX mode.  Operands and scales must be K-contiguous with
 // K % 128 == 0 (four scale bytes per row per K tile); out[m,n] = sum_k (x1 s1)(x2 s2) + fp32 bias.
@@ -489,13 +490,12 @@ int launch_mxfp8_mfma(const OpsnnQmmArgs& a, hipStream_t st)
     if (((uintptr_t)p.sa | (uintptr_t)p.sb | (uint64_t)p.sa_rs | (uint64_t)p.sb_rs | (uint64_t)p.sa_bs | (uint64_t)p.sb_bs) % 4) return OPSNN_NOT_TAKEN;
     if (a.bias && a.bias_dtype != DT_F32) return OPSNN_NOT_TAKEN;
     // Large problems: the four-wave kernel with the tile width that fills its rounds of CUs best, as for the row/column
-    // scale modes below (K % 512 == 0 and 16-byte aligned scale rows, else it declines).  OPSNN_MX8_WIDE = 8 or 9 forces that
+    // scale modes below (K % 512 == 0 and 16-byte aligned scale rows, else it declines).  opsnnSetMx8Wide(8 or 9) forces that
     // kernel with that width (tests, tuning), 0 forbids it.
     {
         int dev = 0, cus = 0;
         if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0) cus = 256;
-        const char* e = getenv("OPSNN_MX8_WIDE");
-        const int forced = e ? atoi(e) : -1;
+        const int forced = opsnn_mx8_wide();
         const int64_t tm = (a.M + 255) / 256, tn = (a.N + 255) / 256;
         int wide_fn = 0;
         if (forced >= 8 && forced <= 9) {

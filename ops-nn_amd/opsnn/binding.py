@@ -183,6 +183,8 @@ _SIGS = {
     "opsnnTranspose8": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int64, C.c_int64, C.c_int64, C.c_void_p]),
     "opsnnTranspose4": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int64, C.c_int64, C.c_int64, C.c_void_p]),
     "opsnnSetFp8Fast": (None, [C.c_int]),
+    "opsnnSetForcePlain": (None, [C.c_int]),
+    "opsnnSetMx8Wide": (None, [C.c_int]),
     "opsnnGetFp8Fast": (C.c_int, []),
     "opsnnDeviceInfo": (C.c_int, [C.POINTER(C.c_int), C.POINTER(C.c_int), C.POINTER(C.c_int64), C.c_char_p, C.c_int]),
 }

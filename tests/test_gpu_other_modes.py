@@ -57,16 +57,15 @@ def check_close(got_bits, want_bits, dt, what, exact=False, fp8_mfma=False, abs_
 
 def plain(flag):
     """Route through the plain kernels (set) or let the selector choose (unset)."""
-    if flag:
-        os.environ["OPSNN_FORCE_PLAIN"] = "1"
-    else:
-        os.environ.pop("OPSNN_FORCE_PLAIN", None)
+    import opsnn
+    opsnn.lib().opsnnSetForcePlain(1 if flag else 0)
 
 
 @pytest.fixture(autouse=True)
 def _reset_env(opsnn):
     yield
-    os.environ.pop("OPSNN_FORCE_PLAIN", None)
+    opsnn.lib().opsnnSetForcePlain(0)
+    opsnn.lib().opsnnSetMx8Wide(-1)
     opsnn.lib().opsnnSetFp8Fast(0)
 
 
@@ -156,11 +155,11 @@ def test_mxfp8_on_the_four_wave_kernel(gpu, fn, M, K, N, tB, batch, bias):
     want = cases.oracle_mx(m, inp, M, K, N, tB, m.ACL_BF16, b)
     pos = dict(inp, x1=inp["x1"] & 0x7F, x2=inp["x2"] & 0x7F)
     abs_sum = orc.b16_to_f32(cases.oracle_mx(m, pos, M, K, N, tB, m.ACL_BF16), orc.BF16).astype(np.float64)
-    os.environ["OPSNN_MX8_WIDE"] = str(fn)
+    m.lib().opsnnSetMx8Wide(fn)
     try:
         got = cases.run_mx_aclnn(m, inp, M, K, N, tB, m.ACL_BF16, b)
     finally:
-        os.environ.pop("OPSNN_MX8_WIDE", None)
+        m.lib().opsnnSetMx8Wide(-1)
     check_close(got, want, orc.BF16, "mxfp8 four-wave", fp8_mfma=True, abs_sum=abs_sum)
 
 

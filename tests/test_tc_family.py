@@ -258,9 +258,9 @@ def test_gpu_fp8_row_and_column_scales_on_the_matrix_cores(gpu, M, K, N, s_len, 
     assert mean <= 2.0 ** -10 and mx <= (10 if fast else 1) * 2.0 ** -7, f"max rel {mx:.3e} mean rel {mean:.3e}"
     assert orc.isclose_fraction(g, w) <= (3e-2 if fast else 1e-3)
     assert not np.array_equal(got, np.full_like(got, 0x7F7F))
-    os.environ["OPSNN_FORCE_PLAIN"] = "1"
+    m.lib().opsnnSetForcePlain(1)
     try:
         exact = cases.run_tc_aclnn(m, inp, M, K, N, dt[out_dt])
     finally:
-        os.environ.pop("OPSNN_FORCE_PLAIN", None)
+        m.lib().opsnnSetForcePlain(0)
     assert np.array_equal(exact, want)

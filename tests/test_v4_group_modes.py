@@ -156,11 +156,11 @@ def test_gpu_a8w4_mx_on_the_matrix_cores(gpu, M, K, N):
     bound = 2.0 ** -7 * np.abs(w) + 2.0 ** -14 * abs_sum
     mx, mean = orc.rel_err_stats(g, w)
     assert float((err / np.maximum(bound, 1e-30)).max()) <= 1.0 and mean <= 2.0 ** -10, f"max rel {mx:.3e} mean rel {mean:.3e}"
-    os.environ["OPSNN_FORCE_PLAIN"] = "1"
+    m.lib().opsnnSetForcePlain(1)
     try:
         exact = cases.run_a8w4_mx_aclnn(m, inp, M, K, N, True, m.ACL_FLOAT16)
     finally:
-        os.environ.pop("OPSNN_FORCE_PLAIN", None)
+        m.lib().opsnnSetForcePlain(0)
     assert np.array_equal(exact, want)
 
 
@@ -213,11 +213,11 @@ def test_gpu_tcg_on_the_matrix_cores(gpu, M, K, N, s_dt, out_dt, fast):
     else:
         assert mx <= 2.0 ** -7 and mean <= 2.0 ** -10, f"max rel {mx:.3e} mean rel {mean:.3e}"
         assert orc.isclose_fraction(g, w) <= 1e-3
-    os.environ["OPSNN_FORCE_PLAIN"] = "1"
+    m.lib().opsnnSetForcePlain(1)
     try:
         exact = cases.run_tcg_aclnn(m, inp, M, K, N, dt[out_dt][0])
     finally:
-        os.environ.pop("OPSNN_FORCE_PLAIN", None)
+        m.lib().opsnnSetForcePlain(0)
     assert np.array_equal(exact, want)
 
 
@@ -249,11 +249,11 @@ def test_gpu_pertile_i8_on_the_matrix_cores(gpu, M, K, N, tB):
     mx, mean = orc.rel_err_stats(g, w)
     assert mx <= 2.0 ** -7 and mean <= 2.0 ** -10, f"max rel {mx:.3e} mean rel {mean:.3e}"
     assert orc.isclose_fraction(g, w) <= 1e-3
-    os.environ["OPSNN_FORCE_PLAIN"] = "1"
+    m.lib().opsnnSetForcePlain(1)
     try:
         exact = cases.run_pertile_i8_aclnn(m, inp, M, K, N, tB, m.ACL_BF16)
     finally:
-        os.environ.pop("OPSNN_FORCE_PLAIN", None)
+        m.lib().opsnnSetForcePlain(0)
     assert np.array_equal(exact, want)
 
 

@@ -90,3 +90,26 @@ def test_phase1_is_thread_safe(opsnn):
     [t.start() for t in ts]
     [t.join() for t in ts]
     assert not errors, errors[:5]
+
+
+def test_executor_is_single_use_and_destroy_after_run_is_harmless(opsnn):
+    """An empty output (M == 0) validates and yields an executor with nothing to launch, so both phases run without a
+    GPU.  Phase 2 consumes the executor (two_phase_api.md:17-24): a second phase 2 with the same handle is refused with
+    161002, and aclDestroyAclOpExecutor on a consumed or already destroyed handle does nothing -- the library recognises
+    such handles by address, without reading the freed object."""
+    m = opsnn
+    K, N = 64, 32
+    x1 = m.Tensor((0, K), m.ACL_INT8, None)
+    x2 = m.Tensor((K, N), m.ACL_INT8, None)
+    s2 = m.Tensor((N,), m.ACL_FLOAT, None)
+    out = m.Tensor((0, N), m.ACL_BF16, None)
+    rc, ws, ex = m.quant_matmul_v5_get_workspace(x1, x2, None, s2, out)
+    assert rc == 0 and ex, m.err_msg()
+    assert m.lib().aclnnQuantMatmulV5(None, 0, ex, None) == 0
+    # garbage churn on the heap between the calls: the freed block is likely to be handed out again
+    junk = [m.quant_matmul_v5_get_workspace(x1, x2, None, s2, out) for _ in range(8)]
+    assert m.lib().aclnnQuantMatmulV5(None, 0, ex, None) == m.STATUS_BY_NAME["ACLNN_ERR_PARAM_INVALID"] or any(j[2] == ex for j in junk)
+    for rc_j, _, ex_j in junk:
+        assert rc_j == 0
+        assert m.lib().aclDestroyAclOpExecutor(ex_j) == 0
+        assert m.lib().aclDestroyAclOpExecutor(ex_j) == 0   # twice: the second call finds nothing to do
