@@ -156,6 +156,13 @@ OPSNN_API int opsnnTranspose8(const void* src, void* dst, int64_t rows, int64_t 
  * rows and cols must be even. */
 OPSNN_API int opsnnTranspose4(const void* src, void* dst, int64_t rows, int64_t cols, int64_t batch, void* stream);
 
+/* FRACTAL_NZ <-> ND re-layout of a dense [rows, row_bytes] byte matrix (batched): nz[b / c0][r / 16][r % 16][b % c0] =
+ * nd[r][b], the NZ array being [ceil(row_bytes / c0), ceil(rows / 16), 16, c0] with zero padding; c0_bytes is 32 for 8-bit
+ * elements, 8 or 16 for 4-bit elements (16 or 32 elements per fractal row).  Layout definition:
+ * matmul/common/tests/st/arch35/matmul_golden_util.py:76-114, 284-313. */
+OPSNN_API int opsnnNzToNd(const void* nz, void* nd, int64_t rows, int64_t row_bytes, int c0_bytes, int64_t batch, void* stream);
+OPSNN_API int opsnnNdToNz(const void* nd, void* nz, int64_t rows, int64_t row_bytes, int c0_bytes, int64_t batch, void* stream);
+
 /* Weight pre-pack: `count` 4-bit values, one per 32-bit carrier element (int32: value & 0xF; fp32: the fp4 e2m1 code of
  * the value, 0 for a value that is not one of the 16), into count / 2 bytes, low nibble = even index.  count even, src
  * 16-byte and dst 8-byte aligned.  Device form of the host loop in

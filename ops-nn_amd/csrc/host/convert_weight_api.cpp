@@ -48,8 +48,8 @@ aclnnStatus aclnnConvertWeightToINT4PackGetWorkspaceSize(const aclTensor* weight
                 dtype_name(p.dtype));
     // formats :184-189
     if (w.format != ACL_FORMAT_ND) INVALID("%s: weight must be in ND format", kApi);
-    if (p.format != ACL_FORMAT_ND)
-        INVALID("%s: weightInt4Pack must be in ND format (FRACTAL_NZ output is not supported here: the matmul entry points take ND weights)", kApi);
+    const bool nz_out = p.format == ACL_FORMAT_FRACTAL_NZ || p.format == ACL_FORMAT_FRACTAL_NZ_C0_16 || p.format == ACL_FORMAT_FRACTAL_NZ_C0_32;
+    if (p.format != ACL_FORMAT_ND && !nz_out) INVALID("%s: weightInt4Pack must be in ND or FRACTAL_NZ format", kApi);
     // dims :191-197
     if (w.rank() < 2 || w.rank() > 3) INVALID("%s: weight must have 2 or 3 dims, got %ld", kApi, (long)w.rank());
     if (p.rank() < 2 || p.rank() > 3) INVALID("%s: weightInt4Pack must have 2 or 3 dims, got %ld", kApi, (long)p.rank());
@@ -68,6 +68,9 @@ aclnnStatus aclnnConvertWeightToINT4PackGetWorkspaceSize(const aclTensor* weight
     // The reference sizes its buffers from weight alone (:380-390); a leading dim that differs would overrun the output here.
     if (w.rank() != p.rank() || (w.rank() == 3 && w.dim(0) != p.dim(0)))
         INVALID("%s: weight %s and weightInt4Pack %s differ in their leading dim", kApi, shape_str(w.shape).c_str(), shape_str(p.shape).c_str());
+    // FRACTAL_NZ output: storage [ceil(n / c0), ceil(k / 16), 16, c0] of the packed [k, n] matrix (:205-250, 318-366)
+    aclOpExecutorImpl::NzStep nz;
+    if (nz_out && !describe_nz_operand(kApi, "weightInt4Pack", pack_, &nz)) return ACLNN_ERR_PARAM_INVALID;
     if (workspaceSize) *workspaceSize = 0;
     if (executor) *executor = nullptr;
     const int64_t count = w.numel();
@@ -76,6 +79,20 @@ aclnnStatus aclnnConvertWeightToINT4PackGetWorkspaceSize(const aclTensor* weight
     const void* src = w.ptr_at(0);
     void* dst = const_cast<void*>(p.ptr_at(0));
     if ((uintptr_t)src % 16 != 0 || (uintptr_t)dst % 8 != 0) INVALID("%s: weight must be 16-byte and weightInt4Pack 8-byte aligned", kApi);
+    if (nz_out) {
+        // pack into a temporary ND buffer, then write the fractals (zero padding included).  This operator is the offline
+        // weight preparation (the reference does it on the host inside this very call), so it may allocate.
+        void* tmp = nullptr;
+        hipError_t e = hipMalloc(&tmp, (size_t)count / 2);
+        if (e != hipSuccess) FAIL(ACLNN_ERR_RUNTIME_ERROR, "%s: cannot allocate %ld bytes for the ND intermediate: %s", kApi, (long)(count / 2), hipGetErrorString(e));
+        int rc = opsnnPackB4(src, fp ? 1 : 0, tmp, count, nullptr);
+        if (rc == 0) rc = opsnnNdToNz(tmp, dst, nz.rows, nz.row_bytes, nz.c0, nz.batch, nullptr);
+        e = hipStreamSynchronize(nullptr);
+        (void)hipFree(tmp);
+        if (rc != 0) FAIL(ACLNN_ERR_RUNTIME_ERROR, "%s: kernel launch failed (%d)", kApi, rc);
+        if (e != hipSuccess) FAIL(ACLNN_ERR_RUNTIME_ERROR, "%s: %s", kApi, hipGetErrorString(e));
+        return ACLNN_SUCCESS;
+    }
     const int rc = opsnnPackB4(src, fp ? 1 : 0, dst, count, nullptr);
     if (rc != 0) FAIL(ACLNN_ERR_RUNTIME_ERROR, "%s: kernel launch failed (%d)", kApi, rc);
     const hipError_t e = hipStreamSynchronize(nullptr);

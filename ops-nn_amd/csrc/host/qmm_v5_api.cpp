@@ -692,6 +692,14 @@ extern "C" aclnnStatus aclnnQuantMatmulV5(void* workspace, uint64_t workspaceSiz
     ex->qmm.workspace = ex->workspace_size ? workspace : nullptr;
     if (!ex->qmm.x1.ptr || !ex->qmm.x2.ptr || !ex->qmm.out) INVALID("aclnnQuantMatmulV5: a tensor has no device address");
     int rc = 0;
+    if (ex->nz.active) {   // x2 arrived in FRACTAL_NZ (aclnnQuantMatmulWeightNz): lay it out as ND in the front of the workspace
+        const void* nd = nullptr;
+        void* rest = nullptr;
+        rc = run_nz_step(*ex, workspace, stream, &nd, &rest);
+        if (rc != 0) FAIL(ACLNN_ERR_RUNTIME_ERROR, "%s: FRACTAL_NZ re-layout failed with code %d", ex->api, rc);
+        ex->qmm.x2.ptr = nd;
+        ex->qmm.workspace = ex->workspace_size > nz_front_bytes(*ex) ? rest : nullptr;
+    }
     switch (ex->kind) {
         case OpKind::QmmInt8: rc = opsnnQmmInt8(&ex->qmm, stream); break;
         case OpKind::QmmBlockScale: rc = opsnnQmmBlockScale(&ex->qmm, stream); break;

@@ -36,6 +36,10 @@ struct aclOpExecutorImpl {
     struct { const float* scale; int64_t scale_len; const float* offset; int64_t offset_len; int round_mode; uint64_t* out; } tqp{};
     uint64_t workspace_size = 0;
     const char* api = "";
+    // Right operand handed over in FRACTAL_NZ (the ...WeightNz / ...Nz entry points): phase 2 first re-lays it out as the
+    // dense ND matrix into the front of the workspace (nd_bytes, rounded up to 256), points the operand there, and gives
+    // the rest of the workspace to the launcher.
+    struct NzStep { bool active = false; const void* src = nullptr; int64_t rows = 0, row_bytes = 0, batch = 1; int c0 = 0; uint64_t nd_bytes = 0; } nz;
 };
 
 // Live executors.  Phase 1 hands an executor over with executor_publish(); phase 2 and aclDestroyAclOpExecutor take it
@@ -92,6 +96,14 @@ bool is_contiguous(const TView& v);
 // Last two dims transposed: stride[-2]==1, stride[-1]==shape[-2], dense batch strides, not both extents 1.
 bool is_transposed_last2(const TView& v);
 void swap_last2(TView& v);
+
+// Phase 1 helper: checks the FRACTAL_NZ storage shape [.., ceil(cols / c0), ceil(rows / 16), 16, c0] of a right operand whose
+// stored matrix is [.., rows, cols] (the view, or its last two dims swapped for a transposed view) and fills the step.
+// Returns false with the error text set.
+bool describe_nz_operand(const char* api, const char* name, const aclTensor* t, aclOpExecutorImpl::NzStep* step);
+// Phase 2 helper for executors with an NZ pre-step: runs it, returns the ND operand's address and the rest of the workspace.
+int run_nz_step(const aclOpExecutorImpl& ex, void* workspace, void* stream, const void** nd_ptr, void** rest);
+inline uint64_t nz_front_bytes(const aclOpExecutorImpl& ex) { return ex.nz.active ? (ex.nz.nd_bytes + 255) / 256 * 256 : 0; }
 
 }  // namespace opsnn
 

@@ -10,6 +10,7 @@
 
 #include "aclnnop/aclnn_weight_quant_batch_matmul_v2.h"
 #include "aclnnop/aclnn_weight_quant_batch_matmul_v3.h"
+#include "aclnnop/aclnn_weight_quant_batch_matmul_nz.h"
 #include "tensor.h"
 
 using namespace opsnn;
@@ -197,6 +198,14 @@ aclnnStatus run(const char* api, void* workspace, uint64_t workspaceSize, aclOpE
         INVALID("%s: workspace of %lu bytes required", api, (unsigned long)ex->workspace_size);
     ex->wqmm.workspace = ex->workspace_size ? workspace : nullptr;
     if (!ex->wqmm.x || !ex->wqmm.w.ptr || !ex->wqmm.y || !ex->wqmm.scale.ptr) INVALID("%s: a tensor has no device address", api);
+    if (ex->nz.active) {   // weight arrived in FRACTAL_NZ (aclnnWeightQuantBatchMatmulNz): lay it out as ND in the front of the workspace
+        const void* nd = nullptr;
+        void* rest = nullptr;
+        const int nrc = run_nz_step(*ex, workspace, stream, &nd, &rest);
+        if (nrc != 0) FAIL(ACLNN_ERR_RUNTIME_ERROR, "%s: FRACTAL_NZ re-layout failed with code %d", api, nrc);
+        ex->wqmm.w.ptr = nd;
+        ex->wqmm.workspace = ex->workspace_size > nz_front_bytes(*ex) ? rest : nullptr;
+    }
     int rc = opsnnWqmm(&ex->wqmm, stream);
     if (rc != 0) FAIL(rc < 0 ? ACLNN_ERR_INNER_TILING_ERROR : ACLNN_ERR_RUNTIME_ERROR, "%s: launch failed with code %d", api, rc);
     return ACLNN_SUCCESS;
@@ -244,6 +253,49 @@ aclnnStatus aclnnWeightQuantBatchMatmulV3(void* workspace, uint64_t workspaceSiz
                                           aclrtStream stream)
 {
     return run("aclnnWeightQuantBatchMatmulV3", workspace, workspaceSize, executor, stream);
+}
+
+// aclnnWeightQuantBatchMatmulNz (aclnn_weight_quant_batch_matmul_nz.h:38-54): the V2 operator with the weight handed over
+// in FRACTAL_NZ, as aclnnConvertWeightToINT4Pack produces it for 4-bit weights ([ceil(n/16), ceil(k/16), 16, 16] elements,
+// or 32 in the last dimension; INT32 / FLOAT carriers: 2 or 4) and the format cast produces it for INT8
+// ([ceil(n/32), ceil(k/16), 16, 32]).  Everything else -- argument rules, quantisation modes, results -- is V2's.  The
+// weight is laid out as the dense ND matrix once per call, into the front of the workspace.
+aclnnStatus aclnnWeightQuantBatchMatmulNzGetWorkspaceSize(const aclTensor* x, const aclTensor* weight,
+                                                          const aclTensor* antiquantScale,
+                                                          const aclTensor* antiquantOffsetOptional,
+                                                          const aclTensor* quantScaleOptional,
+                                                          const aclTensor* quantOffsetOptional,
+                                                          const aclTensor* biasOptional, int antiquantGroupSize,
+                                                          const aclTensor* y, uint64_t* workspaceSize,
+                                                          aclOpExecutor** executor)
+{
+    const char* api = "aclnnWeightQuantBatchMatmulNzGetWorkspaceSize";
+    clear_error();
+    if (!weight) FAIL(ACLNN_ERR_PARAM_NULLPTR, "%s: weight is null", api);
+    if (!workspaceSize || !executor) FAIL(ACLNN_ERR_PARAM_NULLPTR, "%s: workspaceSize/executor is null", api);
+    if (!is_nz(weight->format)) INVALID("%s: weight must be in FRACTAL_NZ format (aclnn_weight_quant_batch_matmul_v2.cpp:1836-1839)", api);
+    aclOpExecutorImpl::NzStep step;
+    if (!describe_nz_operand(api, "weight", weight, &step)) return ACLNN_ERR_PARAM_INVALID;
+    aclTensor nd = *weight;   // the same view over the dense ND matrix the pre-step will write
+    nd.format = ACL_FORMAT_ND;
+    nd.storage = nd.view;
+    uint64_t inner = 0;
+    aclOpExecutor* ex = nullptr;
+    const aclnnStatus rc = get_workspace(api, x, &nd, antiquantScale, antiquantOffsetOptional, quantScaleOptional, quantOffsetOptional,
+                                         biasOptional, antiquantGroupSize, 0, y, &inner, &ex);
+    if (rc != ACLNN_SUCCESS) return rc;
+    if (ex->kind != OpKind::None) {
+        ex->nz = step;
+        ex->workspace_size = nz_front_bytes(*ex) + inner;
+    }
+    *workspaceSize = ex->workspace_size;
+    *executor = ex;
+    return ACLNN_SUCCESS;
+}
+
+aclnnStatus aclnnWeightQuantBatchMatmulNz(void* workspace, uint64_t workspaceSize, aclOpExecutor* executor, aclrtStream stream)
+{
+    return run("aclnnWeightQuantBatchMatmulNz", workspace, workspaceSize, executor, stream);
 }
 
 }  // extern "C"

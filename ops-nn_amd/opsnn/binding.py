@@ -131,6 +131,14 @@ _SIGS = {
     "aclnnQuantMatmulV5GetWorkspaceSize": (C.c_int32, [_T] * 9 + [C.c_bool, C.c_bool, C.c_int64, _T,
                                                               C.POINTER(C.c_uint64), C.POINTER(C.c_void_p)]),
     "aclnnQuantMatmulV5": (C.c_int32, [C.c_void_p, C.c_uint64, C.c_void_p, C.c_void_p]),
+    "aclnnQuantMatmulWeightNzGetWorkspaceSize": (C.c_int32, [_T] * 9 + [C.c_bool, C.c_bool, C.c_int64, _T,
+                                                                    C.POINTER(C.c_uint64), C.POINTER(C.c_void_p)]),
+    "aclnnQuantMatmulWeightNz": (C.c_int32, [C.c_void_p, C.c_uint64, C.c_void_p, C.c_void_p]),
+    "aclnnWeightQuantBatchMatmulNzGetWorkspaceSize": (C.c_int32, [_T] * 7 + [C.c_int, _T, C.POINTER(C.c_uint64),
+                                                                         C.POINTER(C.c_void_p)]),
+    "aclnnWeightQuantBatchMatmulNz": (C.c_int32, [C.c_void_p, C.c_uint64, C.c_void_p, C.c_void_p]),
+    "opsnnNzToNd": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int64, C.c_int64, C.c_int, C.c_int64, C.c_void_p]),
+    "opsnnNdToNz": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int64, C.c_int64, C.c_int, C.c_int64, C.c_void_p]),
     "aclnnWeightQuantBatchMatmulV2GetWorkspaceSize": (C.c_int32, [_T] * 7 + [C.c_int, _T, C.POINTER(C.c_uint64),
                                                                          C.POINTER(C.c_void_p)]),
     "aclnnWeightQuantBatchMatmulV2": (C.c_int32, [C.c_void_p, C.c_uint64, C.c_void_p, C.c_void_p]),
@@ -329,10 +337,11 @@ class Event:
 
 def quant_matmul_v5_get_workspace(x1, x2, x1_scale, x2_scale, out, *, y_scale=None, x1_offset=None, x2_offset=None,
                                   y_offset=None, bias=None, transpose_x1=False, transpose_x2=False, group_size=0,
-                                  ws_ptr=True, ex_ptr=True):
-    """Phase 1.  Returns (status, workspace_size, executor)."""
+                                  ws_ptr=True, ex_ptr=True, weight_nz=False):
+    """Phase 1 (of aclnnQuantMatmulWeightNz when weight_nz).  Returns (status, workspace_size, executor)."""
     ws, ex = C.c_uint64(0), C.c_void_p()
-    rc = lib().aclnnQuantMatmulV5GetWorkspaceSize(
+    fn = lib().aclnnQuantMatmulWeightNzGetWorkspaceSize if weight_nz else lib().aclnnQuantMatmulV5GetWorkspaceSize
+    rc = fn(
         _h(x1), _h(x2), _h(x1_scale), _h(x2_scale), _h(y_scale), _h(x1_offset), _h(x2_offset), _h(y_offset), _h(bias),
         transpose_x1, transpose_x2, group_size, _h(out), C.byref(ws) if ws_ptr else None, C.byref(ex) if ex_ptr else None)
     return rc, ws.value, ex.value
@@ -343,14 +352,19 @@ def quant_matmul_v5(x1, x2, x1_scale, x2_scale, out, stream=None, **kw):
     rc, ws, ex = quant_matmul_v5_get_workspace(x1, x2, x1_scale, x2_scale, out, **kw)
     check(rc, "aclnnQuantMatmulV5GetWorkspaceSize")
     wbuf = DeviceBuffer(ws) if ws else None
-    check(lib().aclnnQuantMatmulV5(wbuf.ptr if wbuf else None, ws, ex, stream.ptr if stream else None), "aclnnQuantMatmulV5")
+    run = lib().aclnnQuantMatmulWeightNz if kw.get("weight_nz") else lib().aclnnQuantMatmulV5
+    check(run(wbuf.ptr if wbuf else None, ws, ex, stream.ptr if stream else None), "aclnnQuantMatmulV5")
     return wbuf  # keep alive until the stream has been synchronised
 
 
 def weight_quant_batch_matmul_get_workspace(x, weight, scale, y, *, offset=None, quant_scale=None, quant_offset=None,
-                                            bias=None, group_size=0, inner_precise=None):
+                                            bias=None, group_size=0, inner_precise=None, weight_nz=False):
     ws, ex = C.c_uint64(0), C.c_void_p()
-    if inner_precise is None:
+    if weight_nz:
+        rc = lib().aclnnWeightQuantBatchMatmulNzGetWorkspaceSize(_h(x), _h(weight), _h(scale), _h(offset), _h(quant_scale),
+                                                                 _h(quant_offset), _h(bias), group_size, _h(y),
+                                                                 C.byref(ws), C.byref(ex))
+    elif inner_precise is None:
         rc = lib().aclnnWeightQuantBatchMatmulV2GetWorkspaceSize(_h(x), _h(weight), _h(scale), _h(offset), _h(quant_scale),
                                                                  _h(quant_offset), _h(bias), group_size, _h(y),
                                                                  C.byref(ws), C.byref(ex))
@@ -367,6 +381,8 @@ def weight_quant_batch_matmul(x, weight, scale, y, stream=None, **kw):
     check(rc, "aclnnWeightQuantBatchMatmulGetWorkspaceSize")
     wbuf = DeviceBuffer(ws) if ws else None
     run = lib().aclnnWeightQuantBatchMatmulV3 if v3 else lib().aclnnWeightQuantBatchMatmulV2
+    if kw.get("weight_nz"):
+        run = lib().aclnnWeightQuantBatchMatmulNz
     check(run(wbuf.ptr if wbuf else None, ws, ex, stream.ptr if stream else None), "aclnnWeightQuantBatchMatmul")
     return wbuf
 

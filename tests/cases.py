@@ -69,7 +69,7 @@ def oracle_qmm_int8(m, inp, M, K, N, transpose_x2, out_dtype, rows=None):
     return np.stack(outs), np.stack(accs)
 
 
-def run_qmm_int8_aclnn(m, inp, M, K, N, transpose_x2, out_dtype, x2_as_view=False):
+def run_qmm_int8_aclnn(m, inp, M, K, N, transpose_x2, out_dtype, x2_as_view=False, nz_storage=None):
     """aclnnQuantMatmulV5 on the device.  x2_as_view: pass x2 [N,K] storage as a transposed view of logical [K,N]
     with transposeX2 = false (the reference treats both spellings alike)."""
     batch = inp["x1"].shape[0]
@@ -84,13 +84,15 @@ def run_qmm_int8_aclnn(m, inp, M, K, N, transpose_x2, out_dtype, x2_as_view=Fals
         x2 = m.Tensor((K, N), m.ACL_INT8, d["x2"], strides=(1, K))
         tflag = False
     else:
-        x2 = m.Tensor(bshape + ((N, K) if transpose_x2 else (K, N)), m.ACL_INT8, d["x2"])
+        # nz_storage: inp["x2"] holds the FRACTAL_NZ bytes of the stored matrix and the call goes to aclnnQuantMatmulWeightNz
+        x2 = m.Tensor(bshape + ((N, K) if transpose_x2 else (K, N)), m.ACL_INT8, d["x2"], fmt=29 if nz_storage else m.ACL_FORMAT_ND,
+                      storage_shape=nz_storage)
         tflag = transpose_x2
     s1 = m.Tensor((M,), m.ACL_FLOAT, d["s1"]) if inp["s1"] is not None else None
     s2 = m.Tensor((inp["s2"].size,), inp["s2_dtype"], d["s2"])
     bias = m.Tensor((N,), inp["bias_dtype"], d["bias"]) if inp["bias"] is not None else None
     out = m.Tensor(bshape + (M, N), out_dtype, d_out)
-    ws = m.quant_matmul_v5(x1, x2, s1, s2, out, bias=bias, transpose_x2=tflag)
+    ws = m.quant_matmul_v5(x1, x2, s1, s2, out, bias=bias, transpose_x2=tflag, weight_nz=bool(nz_storage))
     m.check(m.lib().aclrtSynchronizeDevice(), "sync")
     del ws
     return d_out.to_host(out_np.dtype, out_np.shape)
@@ -257,7 +259,7 @@ def oracle_mx(m, inp, M, K, N, tB, out_dtype, bias=None, rows=None):
     return np.stack(outs)
 
 
-def run_mx_aclnn(m, inp, M, K, N, tB, out_dtype, bias=None):
+def run_mx_aclnn(m, inp, M, K, N, tB, out_dtype, bias=None, nz_storage=None):
     batch = inp["x1"].shape[0]
     bshape = (batch,) if batch > 1 else ()
     adt = m.ACL_FLOAT4_E2M1 if inp["fp4"] else m.ACL_FLOAT8_E4M3FN
@@ -266,13 +268,14 @@ def run_mx_aclnn(m, inp, M, K, N, tB, out_dtype, bias=None):
     d_out = m.DeviceBuffer(out_np.nbytes)
     d_out.fill(0xFF)
     x1 = m.Tensor(bshape + (M, K), adt, d["x1"])
-    x2 = m.Tensor(bshape + ((N, K) if tB else (K, N)), adt, d["x2"])
+    x2 = m.Tensor(bshape + ((N, K) if tB else (K, N)), adt, d["x2"], fmt=29 if nz_storage else m.ACL_FORMAT_ND, storage_shape=nz_storage)
     s1 = m.Tensor(bshape + inp["s1"].shape[1:], m.ACL_FLOAT8_E8M0, d["s1"])
     s2 = m.Tensor(bshape + inp["s2"].shape[1:], m.ACL_FLOAT8_E8M0, d["s2"])
     out = m.Tensor(bshape + (M, N), out_dtype, d_out)
     d_bias = m.DeviceBuffer(host=bias) if bias is not None else None
     t_bias = m.Tensor((N,), m.ACL_FLOAT, d_bias) if bias is not None else None
-    ws = m.quant_matmul_v5(x1, x2, s1, s2, out, bias=t_bias, transpose_x2=tB, group_size=(1 << 32) | (1 << 16) | 32)
+    ws = m.quant_matmul_v5(x1, x2, s1, s2, out, bias=t_bias, transpose_x2=tB, group_size=(1 << 32) | (1 << 16) | 32,
+                           weight_nz=bool(nz_storage))
     m.check(m.lib().aclrtSynchronizeDevice(), "sync")
     del ws
     return d_out.to_host(out_np.dtype, out_np.shape)
@@ -318,7 +321,7 @@ def oracle_wq(m, inp, M, K, N, rows=None):
                      1 if inp["per_tensor"] else N, inp["offset"], inp["group"], inp["bias"], inp["bias_dt"] or 0)
 
 
-def run_wq_aclnn(m, inp, M, K, N, v3=False, scale_2d=None):
+def run_wq_aclnn(m, inp, M, K, N, v3=False, scale_2d=None, nz_storage=None):
     d = {k: m.DeviceBuffer(host=v) for k, v in inp.items() if isinstance(v, np.ndarray)}
     d_y = m.DeviceBuffer(M * N * 2)
     d_y.fill(0xFF)
@@ -326,7 +329,9 @@ def run_wq_aclnn(m, inp, M, K, N, v3=False, scale_2d=None):
     G = -(-K // group) if group > 0 else 1
     x = m.Tensor((M, K), inp["x_dt"], d["x"])
     # the weight view is always the logical [K, N]; [N, K] storage is expressed through strides (1, K)
-    w = m.Tensor((K, N), inp["w_dt"], d["w"], strides=(1, K) if tW else None)
+    # nz_storage: inp["w"] holds the FRACTAL_NZ bytes of the stored matrix and the call goes to aclnnWeightQuantBatchMatmulNz
+    w = m.Tensor((K, N), inp["w_dt"], d["w"], strides=(1, K) if tW else None, fmt=29 if nz_storage else m.ACL_FORMAT_ND,
+                 storage_shape=nz_storage)
     if inp["per_tensor"]:
         sshape, sst = (1,), None
     elif group > 0 or scale_2d:
@@ -337,7 +342,8 @@ def run_wq_aclnn(m, inp, M, K, N, v3=False, scale_2d=None):
     off = m.Tensor(sshape, inp["x_dt"], d["offset"], strides=sst) if inp["offset"] is not None else None
     bias = m.Tensor((N,), inp["bias_dt"], d["bias"]) if inp["bias"] is not None else None
     y = m.Tensor((M, N), inp["x_dt"], d_y)
-    ws = m.weight_quant_batch_matmul(x, w, sc, y, offset=off, bias=bias, group_size=group, inner_precise=0 if v3 else None)
+    ws = m.weight_quant_batch_matmul(x, w, sc, y, offset=off, bias=bias, group_size=group, inner_precise=0 if v3 else None,
+                                     weight_nz=bool(nz_storage))
     m.check(m.lib().aclrtSynchronizeDevice(), "sync")
     del ws
     return d_y.to_host(np.uint16, (M, N))
