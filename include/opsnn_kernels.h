@@ -156,6 +156,9 @@ OPSNN_API int opsnnTranspose8(const void* src, void* dst, int64_t rows, int64_t 
  * rows and cols must be even. */
 OPSNN_API int opsnnTranspose4(const void* src, void* dst, int64_t rows, int64_t cols, int64_t batch, void* stream);
 
+/* The same for 16-bit elements (pairs of e8m0 MX scales, 16-bit group scales). */
+OPSNN_API int opsnnTranspose16(const void* src, void* dst, int64_t rows, int64_t cols, int64_t batch, void* stream);
+
 /* FRACTAL_NZ <-> ND re-layout of a dense [rows, row_bytes] byte matrix (batched): nz[b / c0][r / 16][r % 16][b % c0] =
  * nd[r][b], the NZ array being [ceil(row_bytes / c0), ceil(rows / 16), 16, c0] with zero padding; c0_bytes is 32 for 8-bit
  * elements, 8 or 16 for 4-bit elements (16 or 32 elements per fractal row).  Layout definition:

@@ -22,7 +22,7 @@ namespace opsnn {
 
 constexpr uint32_t kExecutorMagic = 0x51454D4Du;
 
-enum class OpKind { None, QmmInt8, QmmBlockScale, QmmMx, QmmTc, QmmGroup, Wqmm, DynQuant, BlockQuant, MxQuant, TransQuantParam };
+enum class OpKind { None, QmmInt8, QmmBlockScale, QmmMx, QmmTc, QmmGroup, Wqmm, DynQuant, BlockQuant, MxQuant, TransQuantParam, Prepack };
 
 // What phase 1 decided; phase 2 only fills in workspace/stream and launches.
 struct aclOpExecutorImpl {
@@ -34,6 +34,9 @@ struct aclOpExecutorImpl {
     OpsnnBlockQuantArgs blkq{};
     OpsnnMxQuantArgs mxq{};
     struct { const float* scale; int64_t scale_len; const float* offset; int64_t offset_len; int round_mode; uint64_t* out; } tqp{};
+    // aclnnPrepackMatmulWeight: [batch, k, n] -> [batch, n, k] of `bits`-wide elements (src in ND, or in FRACTAL_NZ via `nz`),
+    // and optionally a 16-bit scale matrix [batch, srows, scols] -> [batch, scols, srows]
+    struct { const void* src; void* dst; int64_t k, n, batch; int bits; const void* ssrc; void* sdst; int64_t srows, scols, sbatch; } prepack{};
     uint64_t workspace_size = 0;
     const char* api = "";
     // Right operand handed over in FRACTAL_NZ (the ...WeightNz / ...Nz entry points): phase 2 first re-lays it out as the

@@ -38,6 +38,17 @@ __global__ __launch_bounds__(256) void transpose16_kernel(const uint16_t* __rest
     }
 }
 
+}  // namespace opsnn
+extern "C" int opsnnTranspose16(const void* src, void* dst, int64_t rows, int64_t cols, int64_t batch, void* stream)
+{
+    if (!src || !dst || rows <= 0 || cols <= 0 || batch <= 0 || batch > 65535) return -1;
+    dim3 grid((unsigned)((cols + 31) / 32), (unsigned)((rows + 31) / 32), (unsigned)batch);
+    if (grid.y > 65535u) return -2;
+    hipLaunchKernelGGL(opsnn::transpose16_kernel, grid, dim3(256), 0, (hipStream_t)stream, (const uint16_t*)src, (uint16_t*)dst, rows, cols);
+    return (int)hipGetLastError();
+}
+namespace opsnn {
+
 static inline uint64_t align_up(uint64_t v, uint64_t a) { return (v + a - 1) / a * a; }
 
 uint64_t mx_workspace_bytes(const OpsnnQmmArgs& a)

@@ -137,6 +137,9 @@ _SIGS = {
     "aclnnWeightQuantBatchMatmulNzGetWorkspaceSize": (C.c_int32, [_T] * 7 + [C.c_int, _T, C.POINTER(C.c_uint64),
                                                                          C.POINTER(C.c_void_p)]),
     "aclnnWeightQuantBatchMatmulNz": (C.c_int32, [C.c_void_p, C.c_uint64, C.c_void_p, C.c_void_p]),
+    "aclnnPrepackMatmulWeightGetWorkspaceSize": (C.c_int32, [_T, _T, _T, _T, C.POINTER(C.c_uint64), C.POINTER(C.c_void_p)]),
+    "aclnnPrepackMatmulWeight": (C.c_int32, [C.c_void_p, C.c_uint64, C.c_void_p, C.c_void_p]),
+    "opsnnTranspose16": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int64, C.c_int64, C.c_int64, C.c_void_p]),
     "opsnnNzToNd": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int64, C.c_int64, C.c_int, C.c_int64, C.c_void_p]),
     "opsnnNdToNz": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int64, C.c_int64, C.c_int, C.c_int64, C.c_void_p]),
     "aclnnWeightQuantBatchMatmulV2GetWorkspaceSize": (C.c_int32, [_T] * 7 + [C.c_int, _T, C.POINTER(C.c_uint64),
@@ -355,6 +358,17 @@ def quant_matmul_v5(x1, x2, x1_scale, x2_scale, out, stream=None, **kw):
     run = lib().aclnnQuantMatmulWeightNz if kw.get("weight_nz") else lib().aclnnQuantMatmulV5
     check(run(wbuf.ptr if wbuf else None, ws, ex, stream.ptr if stream else None), "aclnnQuantMatmulV5")
     return wbuf  # keep alive until the stream has been synchronised
+
+
+def prepack_matmul_weight(weight, packed, scale=None, scale_packed=None, stream=None):
+    """Both phases of aclnnPrepackMatmulWeight; returns (status of phase 1, workspace buffer kept alive)."""
+    ws, ex = C.c_uint64(0), C.c_void_p()
+    rc = lib().aclnnPrepackMatmulWeightGetWorkspaceSize(_h(weight), _h(scale), _h(packed), _h(scale_packed), C.byref(ws), C.byref(ex))
+    if rc != 0:
+        return rc, None
+    wbuf = DeviceBuffer(ws.value) if ws.value else None
+    check(lib().aclnnPrepackMatmulWeight(wbuf.ptr if wbuf else None, ws.value, ex, stream.ptr if stream else None), "aclnnPrepackMatmulWeight")
+    return 0, wbuf
 
 
 def weight_quant_batch_matmul_get_workspace(x, weight, scale, y, *, offset=None, quant_scale=None, quant_offset=None,
