@@ -102,11 +102,14 @@ OPSNN_API int opsnnQmmBlockScale(const OpsnnQmmArgs* a, void* stream);
 OPSNN_API void opsnnSetFp8Fast(int fast);
 OPSNN_API int opsnnGetFp8Fast(void);
 /* Routing switches for tests and tuning, process-wide; each starts from the environment variable of the same meaning,
- * read once when the library is loaded (OPSNN_FORCE_PLAIN, OPSNN_MX8_WIDE):
+ * read once when the library is loaded (OPSNN_FORCE_PLAIN, OPSNN_MX8_WIDE, OPSNN_WQ_TILE_MIN):
  *   opsnnSetForcePlain(1)  every call runs on the plain one-thread-per-output kernels (bit-identical to the CPU oracle);
- *   opsnnSetMx8Wide(n)     MXFP8 on the four-wave kernel with 256 x 32n tiles (n = 8, 9), 0 never, -1 automatic. */
+ *   opsnnSetMx8Wide(n)     MXFP8 on the four-wave kernel with 256 x 32n tiles (n = 8, 9), 0 never, -1 automatic;
+ *   opsnnSetWqTileMin(m)   weight-only int4/int8 calls with m .. 256 rows of x run on the dequantise-once tile kernel
+ *                          (default 129; 1 sends every eligible call there, 257 none). */
 OPSNN_API void opsnnSetForcePlain(int on);
 OPSNN_API void opsnnSetMx8Wide(int n);
+OPSNN_API void opsnnSetWqTileMin(int m);
 /* MX: fp4/fp8 operands, e8m0 scale per 32 K. out = (x1*s1) @ (x2*s2) + fp32 bias. */
 OPSNN_API int opsnnQmmMx(const OpsnnQmmArgs* a, void* stream);
 /* Per-tensor / per-channel scales (T-T, T-C): int8 or fp8 (e4m3, e5m2) operands;

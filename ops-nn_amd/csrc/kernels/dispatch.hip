@@ -29,7 +29,12 @@ using namespace opsnn;
 //   OPSNN_FORCE_PLAIN=1 / opsnnSetForcePlain(1): every call runs on the plain one-thread-per-output kernels (the parity
 //   tests compare them bit for bit with the oracle);
 //   OPSNN_MX8_WIDE=n / opsnnSetMx8Wide(n): MXFP8 on the four-wave kernel with 256 x 32n tiles, n = 8 or 9; 0 never; -1 the
-//   selector decides (default).
+//   selector decides (default);
+//   OPSNN_WQ_TILE_MIN=m / opsnnSetWqTileMin(m): weight-only int4/int8 calls with m .. 256 rows of x run on the
+//   dequantise-once tile kernel (default 129: below that the streaming kernels are faster).
+static int g_wq_tile_min = [] { const char* e = getenv("OPSNN_WQ_TILE_MIN"); return e ? atoi(e) : 129; }();
+extern "C" void opsnnSetWqTileMin(int m) { __atomic_store_n(&g_wq_tile_min, m, __ATOMIC_RELAXED); }
+extern "C" __attribute__((visibility("hidden"))) int opsnn_wq_tile_min() { return __atomic_load_n(&g_wq_tile_min, __ATOMIC_RELAXED); }
 static int g_force_plain = [] { const char* e = getenv("OPSNN_FORCE_PLAIN"); return (e && *e && *e != '0') ? 1 : 0; }();
 static int g_mx8_wide = [] { const char* e = getenv("OPSNN_MX8_WIDE"); return e ? atoi(e) : -1; }();
 extern "C" void opsnnSetForcePlain(int on) { __atomic_store_n(&g_force_plain, on ? 1 : 0, __ATOMIC_RELAXED); }

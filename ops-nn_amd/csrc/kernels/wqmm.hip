@@ -317,8 +317,21 @@ static bool stream_eligible(WqParams& p, WqStreamOpts& o)
 }
 
 template <int XDT, int WBITS>
+int launch_wq_tile(const WqParams& p, hipStream_t st);   // wqmm_tile.hip
+}  // namespace opsnn
+extern "C" int opsnn_wq_tile_min();   // dispatch.hip
+namespace opsnn {
+
+template <int XDT, int WBITS>
 static int launch_slabs(WqParams p, hipStream_t st)
 {
+    // many rows: the dequantise-once tile kernel, one pass over the weight for up to 256 rows.  (Measured on 8192 x 28672
+    // int4, group 128: 256 rows 165 us against 207 in two passes of the streaming kernel below; 128 rows 116 against 105,
+    // 64 rows 94 against 69 -- hence the default switch at 129 rows; opsnnSetWqTileMin moves it.)
+    if (p.M >= opsnn_wq_tile_min() && p.M <= 256) {
+        const int rc = launch_wq_tile<XDT, WBITS>(p, st);
+        if (rc != OPSNN_NOT_TAKEN) return rc;
+    }
     WqStreamOpts o{};
     const bool stream = stream_eligible<WBITS>(p, o);
     // rows per launch: as many as one pass over the weights can serve, in equal slabs

@@ -196,6 +196,7 @@ _SIGS = {
     "opsnnSetFp8Fast": (None, [C.c_int]),
     "opsnnSetForcePlain": (None, [C.c_int]),
     "opsnnSetMx8Wide": (None, [C.c_int]),
+    "opsnnSetWqTileMin": (None, [C.c_int]),
     "opsnnGetFp8Fast": (C.c_int, []),
     "opsnnDeviceInfo": (C.c_int, [C.POINTER(C.c_int), C.POINTER(C.c_int), C.POINTER(C.c_int64), C.c_char_p, C.c_int]),
 }

@@ -231,6 +231,44 @@ def test_weight_only(gpu, M, K, N, x_dt, w_dt, group, tW, off, bias, use_plain):
     check_close(got, want, dt[x_dt], "weight-only", exact=use_plain)
 
 
+@pytest.mark.parametrize("M,K,N,x_dt,w_dt,group,tW,off,bias", [
+    # 64-, 128- and 256-row instances; int4 (two K steps per weight copy) and int8 (one); groups of 64, 128, 256 and
+    # per channel; ragged rows and columns; a single K step; N-contiguous weight (re-laid out first); bias
+    (64, 512, 384, "f16", "i4", 128, True, True, None),
+    (50, 2048, 288, "bf16", "i4", 128, True, False, "bf16"),
+    (64, 1024, 256, "f16", "i8", 64, True, True, None),
+    (60, 256, 100, "bf16", "i4", 64, True, True, None),
+    (64, 128, 128, "f16", "i4", 0, True, False, None),
+    (64, 64, 128, "f16", "i8", 0, True, True, None),
+    (1, 1024, 256, "f16", "i4", 128, True, True, None),
+    (100, 2048, 512, "f16", "i4", 128, True, True, None),
+    (128, 1024, 256, "f16", "i8", 64, True, True, "f16"),
+    (77, 192, 130, "f16", "i8", 64, True, True, None),
+    (130, 1024, 256, "bf16", "i8", 0, False, False, "bf16"),
+    (200, 2048, 320, "bf16", "i4", 256, True, True, None),
+    (256, 1024, 256, "f16", "i4", 128, True, False, "f16"),
+    (256, 512, 256, "f16", "i4", 128, False, True, None),
+    (129, 1152, 200, "bf16", "i4", 384, True, True, None),      # three groups of 384 = 6 steps each
+    (256, 320, 136, "f16", "i8", 0, True, False, None),         # five steps (odd count)
+])
+def test_weight_only_tile_kernel(gpu, M, K, N, x_dt, w_dt, group, tW, off, bias):
+    """The dequantise-once tile kernel, which by itself takes 129 .. 256 rows of x, forced onto every row count it has an
+    instance for (opsnnSetWqTileMin(1)); the bar of the other matrix-instruction kernels."""
+    m = gpu
+    dt = {"bf16": m.ACL_BF16, "f16": m.ACL_FLOAT16, "i8": m.ACL_INT8, "i4": m.ACL_INT4, None: None}
+    print(f"case wq tile kernel M={M} K={K} N={N} x={x_dt} w={w_dt} g={group} tW={tW} off={off} bias={bias}", flush=True)
+    inp = cases.make_wq_inputs(m, M, K, N, M * 5 + N, dt[x_dt], dt[w_dt], group, tW, off, dt[bias])
+    want = cases.oracle_wq(m, inp, M, K, N)
+    plain(False)
+    m.lib().opsnnSetWqTileMin(1)
+    try:
+        got = cases.run_wq_aclnn(m, inp, M, K, N)
+    finally:
+        m.lib().opsnnSetWqTileMin(129)
+    check_close(got, want, dt[x_dt], "weight-only tile kernel")
+
+
+
 def test_weight_only_v3_and_per_tensor(gpu):
     m = gpu
     inp = cases.make_wq_inputs(m, 8, 256, 128, 2, m.ACL_FLOAT16, m.ACL_INT8, 0, False, True, None, per_tensor=True)
