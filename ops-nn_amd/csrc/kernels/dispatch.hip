@@ -54,10 +54,105 @@ static bool qmm_args_ok(const OpsnnQmmArgs* a)
     return a && a->x1.ptr && a->x2.ptr && a->out && a->M > 0 && a->N > 0 && a->K > 0 && a->batch > 0 && a->batch <= 65535;
 }
 
+// ---- K tail ----
+// The matrix-core kernels walk K in tiles of 128 bytes fetched by 16-byte copies: they take K % 128 == 0 (int8: K % 16 == 0)
+// and 16-byte aligned rows.  Any other K of an 8-bit operand pair is first copied, both operands, into K-contiguous rows
+// padded with zeros to the next multiple of 128 (zero products change no sum, integer or floating point; the scale
+// tables of the block-scale modes already have ceil(K / 128) entries).  The copies live in the workspace: two passes
+// over the operands instead of the one-thread-per-output kernel.
+namespace {
+__global__ __launch_bounds__(256) void pad_k8_kernel(const uint8_t* __restrict__ src, int64_t o_stride, int64_t k_stride, int64_t b_stride,
+                                                     uint8_t* __restrict__ dst, int64_t rows, int64_t K, int64_t Kp, int k_fast)
+{
+    // one thread per 16-byte piece of the output; threadIdx.x runs along the dimension that is contiguous in the source
+    const int64_t chunks = Kp / 16;
+    const int64_t ix = (int64_t)blockIdx.x * 64 + (threadIdx.x & 63), iy = (int64_t)blockIdx.y * 4 + (threadIdx.x >> 6);
+    const int64_t c = k_fast ? ix : iy, o = k_fast ? iy : ix;
+    if (c >= chunks || o >= rows) return;
+    const uint8_t* s = src + (int64_t)blockIdx.z * b_stride + o * o_stride;
+    uint32_t v[4] = {0, 0, 0, 0};
+#pragma unroll
+    for (int j = 0; j < 16; j++) {
+        const int64_t k = c * 16 + j;
+        const uint32_t b = k < K ? s[k * k_stride] : 0u;
+        v[j >> 2] |= b << (8 * (j & 3));
+    }
+    *(uint4*)(dst + ((int64_t)blockIdx.z * rows + o) * Kp + c * 16) = make_uint4(v[0], v[1], v[2], v[3]);
+}
+
+int launch_pad_k8(const OpsnnMat& m, bool k_is_col, int64_t rows, int64_t K, int64_t Kp, int64_t nb, void* dst, hipStream_t st)
+{
+    const int64_t o_stride = k_is_col ? m.row_stride : m.col_stride, k_stride = k_is_col ? m.col_stride : m.row_stride;
+    const int k_fast = k_stride == 1 || o_stride != 1;
+    const int64_t chunks = Kp / 16;
+    const int64_t nx = k_fast ? chunks : rows, ny = k_fast ? rows : chunks;
+    if ((ny + 3) / 4 > 65535 || nb > 65535) return OPSNN_NOT_TAKEN;
+    const dim3 grid((unsigned)((nx + 63) / 64), (unsigned)((ny + 3) / 4), (unsigned)nb);
+    hipLaunchKernelGGL(pad_k8_kernel, grid, dim3(256), 0, st, (const uint8_t*)m.ptr, o_stride, k_stride, m.batch_stride, (uint8_t*)dst, rows, K, Kp, k_fast);
+    return (int)hipGetLastError();
+}
+
+inline int64_t round_up(int64_t v, int64_t a) { return (v + a - 1) / a * a; }
+
+// Padded K (a multiple of 128) if the call is one that the padding pre-step serves, else 0.
+// mode as in opsnnQmmWorkspace.
+int64_t k_pad_for(const OpsnnQmmArgs& a, int mode)
+{
+    if (a.force_variant == OPSNN_VARIANT_PLAIN || opsnn_force_plain()) return 0;
+    if (a.M * a.N < 64 * 64) return 0;   // below the matrix-core kernels' own minimum
+    const bool i8 = a.x1_dtype == DT_I8 && a.x2_dtype == DT_I8, f8 = a.x1_dtype == DT_E4M3 && a.x2_dtype == DT_E4M3;
+    bool tail = false;
+    if (mode == 0) tail = i8 && a.K % 16 != 0;
+    else if (mode == 1) tail = (f8 || i8) && a.K % 128 != 0 && a.gsK == 128;
+    else if (mode == 3) tail = (i8 && !a.x1_scale && a.K % 16 != 0) || (f8 && a.x1_scale && a.K % 128 != 0);
+    if (!tail || a.K < 16) return 0;
+    if (a.x1.batch_stride < 0 || a.x2.batch_stride < 0) return 0;
+    return round_up(a.K, 128);
+}
+uint64_t k_pad_bytes(const OpsnnQmmArgs& a, int64_t Kp)
+{
+    const uint64_t nb2 = a.x2.batch_stride == 0 ? 1 : (uint64_t)a.batch, nb1 = a.x1.batch_stride == 0 && a.batch > 1 ? 1 : (uint64_t)a.batch;
+    return round_up((int64_t)(nb1 * (uint64_t)a.M * (uint64_t)Kp), 256) + nb2 * (uint64_t)a.N * (uint64_t)Kp;
+}
+// Launches the two copies and returns, in b, the same call on the padded operands (K = Kp, no workspace needed any more).
+int k_pad_prestep(const OpsnnQmmArgs& a, int64_t Kp, hipStream_t st, OpsnnQmmArgs& b)
+{
+    if (!a.workspace) return OPSNN_NOT_TAKEN;
+    const int64_t nb2 = a.x2.batch_stride == 0 ? 1 : a.batch, nb1 = a.x1.batch_stride == 0 && a.batch > 1 ? 1 : a.batch;
+    uint8_t* w1 = (uint8_t*)a.workspace;
+    uint8_t* w2 = w1 + round_up(nb1 * a.M * Kp, 256);
+    int rc = launch_pad_k8(a.x1, true, a.M, a.K, Kp, nb1, w1, st);
+    if (rc != 0) return rc;
+    rc = launch_pad_k8(a.x2, false, a.N, a.K, Kp, nb2, w2, st);
+    if (rc != 0) return rc;
+    b = a;
+    b.K = Kp;
+    b.x1 = OpsnnMat{w1, Kp, 1, nb1 == 1 && a.batch > 1 ? 0 : a.M * Kp};
+    b.x2 = OpsnnMat{w2, 1, Kp, nb2 == 1 && a.batch > 1 ? 0 : a.N * Kp};
+    b.workspace = nullptr;
+    return 0;
+}
+}  // namespace
+
+// OPSNN_NOT_TAKEN if the call needs no padding (or has no workspace); 0 with *b filled after launching the copies
+extern "C" __attribute__((visibility("hidden"))) int opsnn_qmm_k_pad(const OpsnnQmmArgs* a, int mode, void* stream, OpsnnQmmArgs* b)
+{
+    const int64_t Kp = k_pad_for(*a, mode);
+    if (!Kp) return OPSNN_NOT_TAKEN;
+    return k_pad_prestep(*a, Kp, (hipStream_t)stream, *b);
+}
+
 extern "C" int opsnnQmmBlockScale(const OpsnnQmmArgs* a, void* stream)
 {
     if (!qmm_args_ok(a) || !a->x1_scale_mat.ptr || !a->x2_scale_mat.ptr) return -1;
     if (a->force_variant != OPSNN_VARIANT_PLAIN && !opsnn_force_plain()) {
+        OpsnnQmmArgs b;
+        const int64_t Kp = k_pad_for(*a, 1);
+        if (Kp) {
+            int rc = k_pad_prestep(*a, Kp, (hipStream_t)stream, b);
+            if (rc == 0) rc = launch_blockscale_mfma(b, (hipStream_t)stream);
+            if (rc != OPSNN_NOT_TAKEN) return rc;
+        }
         int rc = launch_blockscale_mfma(*a, (hipStream_t)stream);
         if (rc != OPSNN_NOT_TAKEN) return rc;
         if (a->force_variant != 0) return -4;
@@ -90,6 +185,12 @@ extern "C" int opsnnQmmTc(const OpsnnQmmArgs* a, void* stream)
     if (a->x2_scale_len != 1 && a->x2_scale_len != a->N) return -2;
     if (a->x1_scale && ((a->x1_scale_len != 1 && a->x1_scale_len != a->M) || !f8)) return -2;
     if (a->out_dtype == DT_I8 || a->out_dtype == DT_I32) { if (!i8) return -2; }
+    OpsnnQmmArgs padded;
+    if (const int64_t Kp = k_pad_for(*a, 3)) {   // K tail: continue on zero-padded K-contiguous copies
+        const int rc = k_pad_prestep(*a, Kp, (hipStream_t)stream, padded);
+        if (rc == 0) a = &padded;
+        else if (rc != OPSNN_NOT_TAKEN) return rc;
+    }
     // int8 operands, 16-bit output, no per-token scale: out = fp32(acc + int32 bias) * scale' + float bias, where scale'
     // is the scale with only its upper 19 bits kept for 64-bit words and for a one-element scale without a bf16 / fp32
     // bias (qbmmv3_kernel_golden.py:403-475).  That is the per-token x per-channel formula with x1_scale = 1: the MFMA
@@ -159,6 +260,7 @@ extern "C" int opsnnWqmm(const OpsnnWqmmArgs* a, void* stream)
 extern "C" uint64_t opsnnQmmWorkspace(const OpsnnQmmArgs* a, int mode)
 {
     if (!a) return 0;
+    if (const int64_t Kp = k_pad_for(*a, mode)) return k_pad_bytes(*a, Kp);
     if (mode == 2) return mx_workspace_bytes(*a);
     // per-tensor / per-channel family: int8 operands share the int8 kernels and their re-layout; fp8 needs none
     if (mode == 3 && !(a->x1_dtype == DT_I8 && a->x2_dtype == DT_I8 && !a->x1_scale)) return 0;

@@ -90,8 +90,15 @@ static int64_t cu_count()
 
 // OPSNN_NOT_TAKEN: an INT8 output was asked for and the shape does not fit the MFMA kernels (the caller falls back).
 extern "C" __attribute__((visibility("hidden"))) int opsnn_qmm_int8_impl(const OpsnnQmmArgs* a, void* stream);
+extern "C" __attribute__((visibility("hidden"))) int opsnn_qmm_k_pad(const OpsnnQmmArgs* a, int mode, void* stream, OpsnnQmmArgs* b);   // dispatch.hip
 extern "C" int opsnnQmmInt8(const OpsnnQmmArgs* a, void* stream)
 {
+    OpsnnQmmArgs padded;
+    if (a && a->x1.ptr && a->x2.ptr && a->M > 0 && a->N > 0 && a->K > 0 && a->batch > 0) {
+        const int prc = opsnn_qmm_k_pad(a, 0, stream, &padded);   // K % 16 != 0: zero-padded K-contiguous copies
+        if (prc == 0) a = &padded;
+        else if (prc != OPSNN_NOT_TAKEN) return prc;
+    }
     const int rc = opsnn_qmm_int8_impl(a, stream);
     return rc == OPSNN_NOT_TAKEN ? -2 : rc;
 }
