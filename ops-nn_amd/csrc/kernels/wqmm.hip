@@ -33,7 +33,10 @@ int launch_wqmm_plain(const OpsnnWqmmArgs& a, hipStream_t st);
 // WK: waves of the workgroup that split K between them (1, 2 or 4); the other 4/WK waves take different column
 // blocks.  WK > 1 is for narrow N, where column blocks alone cannot fill the chip; partial sums meet in LDS and
 // are added in a fixed order.
-template <int XDT, int WBITS, int MB, int WK>
+// WFLT: the weights are floating-point codes (e2m1 in 4 bits, e4m3 in 8), possibly with e8m0 scales per 32 k (MX:
+// wqbmmv2_kernel_golden.py:300-352 -- the weight is exact in x's dtype, the scale goes through x's dtype, one rounding of
+// the product); they take the element-wise dequantisation below.
+template <int XDT, int WBITS, int MB, int WK, bool WFLT>
 __global__ __launch_bounds__(256, 2) void wqmm_decode_kernel(WqParams p)
 {
     constexpr int WN = 4 / WK;
@@ -117,7 +120,8 @@ __global__ __launch_bounds__(256, 2) void wqmm_decode_kernel(WqParams p)
             const int kk = k < Ki ? k : Ki - KPL;
             wq[i] = n_ok ? *(const v4i*)(wrow + (int64_t)kk * WBITS / 8) : (v4i){0, 0, 0, 0};
             const int gi = p.group_shift >= 0 ? (kk >> p.group_shift) : (kk / groupi);
-            sq[i] = srow[(int64_t)gi * p.s_rs];
+            if (WFLT && p.scale_e8m0) sq[i] = bits_x<XDT>(e8m0_to_f32(((const uint8_t*)p.scale)[n * p.s_cs + (int64_t)gi * p.s_rs]));
+            else sq[i] = srow[(int64_t)gi * p.s_rs];
             oq[i] = has_off ? orow[(int64_t)gi * p.s_rs] : (uint16_t)0;
         }
     };
@@ -155,7 +159,7 @@ __global__ __launch_bounds__(256, 2) void wqmm_decode_kernel(WqParams p)
             for (int s = 0; s < STEPS; s++) {
                 // operand A: this lane's 8 dequantised weights for MFMA step s
                 v4i aop;
-                if constexpr (XDT == DT_F16 && WBITS == 4) {
+                if constexpr (XDT == DT_F16 && WBITS == 4 && !WFLT) {
                     const _Float16 sh = __builtin_bit_cast(_Float16, sb), oh = __builtin_bit_cast(_Float16, ob);
                     h2 o4[4];
                     dequant_i4_f16(live ? (uint32_t)cur[i][s] : 0x88888888u, (h2){oh, oh}, (h2){sh, sh}, has_off, o4);
@@ -171,17 +175,23 @@ __global__ __launch_bounds__(256, 2) void wqmm_decode_kernel(WqParams p)
                         const int ord[8] = {0, 4, 1, 5, 2, 6, 3, 7};   // element order of the staged x
 #pragma unroll
                         for (int j = 0; j < 8; j++) {
-                            int v = (int)((q >> (4 * ord[j])) & 15u);
-                            v = v >= 8 ? v - 16 : v;
-                            e[j] = live ? bits_x<XDT>(dequant_one<XDT>((float)v, off, scf, has_off)) : (uint16_t)0;
+                            float wv;
+                            if constexpr (WFLT) {
+                                wv = e2m1_to_f32((q >> (4 * ord[j])) & 15u);
+                            } else {
+                                int v = (int)((q >> (4 * ord[j])) & 15u);
+                                wv = (float)(v >= 8 ? v - 16 : v);
+                            }
+                            e[j] = live ? bits_x<XDT>(dequant_one<XDT>(wv, off, scf, has_off)) : (uint16_t)0;
                         }
                     } else {
                         // int8: 16 bytes per piece, step s uses bytes 8s..8s+7 in natural order
 #pragma unroll
                         for (int j = 0; j < 8; j++) {
                             const uint32_t q = (uint32_t)cur[i][2 * s + (j >> 2)];
-                            const int v = (int)(int8_t)((q >> (8 * (j & 3))) & 0xffu);
-                            e[j] = live ? bits_x<XDT>(dequant_one<XDT>((float)v, off, scf, has_off)) : (uint16_t)0;
+                            const uint32_t byte = (q >> (8 * (j & 3))) & 0xffu;
+                            const float wv = WFLT ? e4m3_to_f32(byte) : (float)(int)(int8_t)byte;
+                            e[j] = live ? bits_x<XDT>(dequant_one<XDT>(wv, off, scf, has_off)) : (uint16_t)0;
                         }
                     }
                     aop = (v4i){(int)(e[0] | ((uint32_t)e[1] << 16)), (int)(e[2] | ((uint32_t)e[3] << 16)),
@@ -249,13 +259,13 @@ __global__ __launch_bounds__(256, 2) void wqmm_decode_kernel(WqParams p)
     }
 }
 
-template <int XDT, int WBITS, int MB, int WK>
+template <int XDT, int WBITS, int MB, int WK, bool WFLT = false>
 static int launch_decode(const WqParams& p, hipStream_t st)
 {
     constexpr int KC = 4 * (128 / WBITS), KX = 8 * KC / MB, WN = 4 / WK;
     const size_t lds = 2 * (size_t)(16 * MB) * (KX * 2 + 16);
     const unsigned grid = (unsigned)((p.N + 16 * WN - 1) / (16 * WN));
-    auto k = wqmm_decode_kernel<XDT, WBITS, MB, WK>;
+    auto k = wqmm_decode_kernel<XDT, WBITS, MB, WK, WFLT>;
     static bool attr_set = false;
     if (!attr_set) {
         hipError_t e = hipFuncSetAttribute((const void*)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
@@ -266,13 +276,13 @@ static int launch_decode(const WqParams& p, hipStream_t st)
     return (int)hipGetLastError();
 }
 
-template <int XDT, int WBITS, int MB>
+template <int XDT, int WBITS, int MB, bool WFLT = false>
 static int launch_wk(const WqParams& p, hipStream_t st)
 {
     // split K between the waves of a workgroup when column blocks alone would leave most of the chip idle
     const int64_t nblocks = (p.N + 15) / 16;
-    if (nblocks < 1024 && p.K >= 2048) return launch_decode<XDT, WBITS, MB, 4>(p, st);
-    return launch_decode<XDT, WBITS, MB, 1>(p, st);
+    if (nblocks < 1024 && p.K >= 2048) return launch_decode<XDT, WBITS, MB, 4, WFLT>(p, st);
+    return launch_decode<XDT, WBITS, MB, 1, WFLT>(p, st);
 }
 
 template <> int launch_wq_stream<DT_F16, 4>(const WqParams&, const WqStreamOpts&, hipStream_t);
@@ -322,6 +332,22 @@ int launch_wq_tile(const WqParams& p, hipStream_t st);   // wqmm_tile.hip
 extern "C" int opsnn_wq_tile_min();   // dispatch.hip
 namespace opsnn {
 
+// floating-point weight codes: the general kernel, in row slabs of 64
+template <int XDT, int WBITS>
+static int launch_slabs_float(WqParams p, hipStream_t st)
+{
+    for (int64_t m0 = 0; m0 < p.M; m0 += 64) {
+        p.m_base = m0;
+        p.m_rows = (p.M - m0) < 64 ? (p.M - m0) : 64;
+        int rc;
+        if (p.m_rows <= 16) rc = launch_wk<XDT, WBITS, 1, true>(p, st);
+        else if (p.m_rows <= 32) rc = launch_wk<XDT, WBITS, 2, true>(p, st);
+        else rc = launch_wk<XDT, WBITS, 4, true>(p, st);
+        if (rc != 0) return rc;
+    }
+    return 0;
+}
+
 template <int XDT, int WBITS>
 static int launch_slabs(WqParams p, hipStream_t st)
 {
@@ -357,9 +383,12 @@ int launch_wqmm_mfma(const OpsnnWqmmArgs& a0, hipStream_t st)
 {
     OpsnnWqmmArgs a = a0;
     if (a.x_dtype != DT_F16 && a.x_dtype != DT_BF16) return OPSNN_NOT_TAKEN;
-    if (a.w_dtype != DT_I4 && a.w_dtype != DT_I8) return OPSNN_NOT_TAKEN;
-    if (a.scale_dtype != a.x_dtype) return OPSNN_NOT_TAKEN;
-    const int wbits = a.w_dtype == DT_I4 ? 4 : 8;
+    const bool wflt = a.w_dtype == DT_E2M1 || a.w_dtype == DT_E4M3;
+    if (a.w_dtype != DT_I4 && a.w_dtype != DT_I8 && !wflt) return OPSNN_NOT_TAKEN;
+    const bool mx = wflt && a.scale_dtype == DT_E8M0;
+    if (a.scale_dtype != a.x_dtype && !mx) return OPSNN_NOT_TAKEN;
+    if (mx && (a.offset || a.group <= 0 || a.scale_n == 1)) return OPSNN_NOT_TAKEN;
+    const int wbits = (a.w_dtype == DT_I4 || a.w_dtype == DT_E2M1) ? 4 : 8;
     const int64_t kpl = 128 / wbits;
     if (a.K % kpl != 0 || a.K < kpl) return OPSNN_NOT_TAKEN;
     const int64_t group = a.group > 0 ? a.group : a.K;
@@ -382,6 +411,12 @@ int launch_wqmm_mfma(const OpsnnWqmmArgs& a0, hipStream_t st)
     p.group_shift = (group & (group - 1)) == 0 ? __builtin_ctzll((unsigned long long)group) : -1;
     if (a.K >= (1ll << 31) || a.N >= (1ll << 31)) return OPSNN_NOT_TAKEN;
     if (((uintptr_t)p.w | (uint64_t)p.ldw) % 16 || ((uintptr_t)p.x % 16) || (a.K % 8)) return OPSNN_NOT_TAKEN;
+    if (wflt) {
+        p.w_float = 1;
+        p.scale_e8m0 = mx ? 1 : 0;
+        if (a.x_dtype == DT_F16) return wbits == 4 ? launch_slabs_float<DT_F16, 4>(p, st) : launch_slabs_float<DT_F16, 8>(p, st);
+        return wbits == 4 ? launch_slabs_float<DT_BF16, 4>(p, st) : launch_slabs_float<DT_BF16, 8>(p, st);
+    }
     if (a.x_dtype == DT_F16) return wbits == 4 ? launch_slabs<DT_F16, 4>(p, st) : launch_slabs<DT_F16, 8>(p, st);
     return wbits == 4 ? launch_slabs<DT_BF16, 4>(p, st) : launch_slabs<DT_BF16, 8>(p, st);
 }

@@ -21,6 +21,8 @@ struct WqParams {
     int group_shift;         // log2(group) if it is a power of two, else -1
     int cpg_shift;           // streamlined kernel: log2(group / chunk), 31 for a per-channel scale
     int64_t m_base, m_rows;  // row slab handled by this launch
+    int w_float;             // weights are floating-point codes (4 bits: e2m1, 8 bits: e4m3), not two's-complement integers
+    int scale_e8m0;          // scale is one e8m0 byte per element (MX), not a 16-bit value of x's dtype
 };
 
 typedef _Float16 h2 __attribute__((ext_vector_type(2)));

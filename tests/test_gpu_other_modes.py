@@ -193,6 +193,12 @@ def test_mx_batched(gpu, M, K, N, batch):
     (16, 1024, 384, "bf16", "fp4", 32, True, False, "bf16"),
     (5, 96, 66, "f16", "fp4", 32, False, False, "f16"),
     (40, 2048, 256, "f16", "fp4", 32, True, False, None),
+    # ... on the matrix cores these take the general decode kernel: a K split between waves (narrow N, K >= 2048), several
+    # row slabs, e4m3 weights (per channel: the only form the API admits)
+    (16, 4096, 1024, "bf16", "fp4", 32, True, False, None),
+    (130, 2048, 512, "f16", "fp4", 32, True, False, "f16"),
+    (100, 2048, 512, "bf16", "e4m3", 0, True, False, None),
+    (16, 4096, 320, "f16", "e4m3", 0, True, False, None),
     # shapes the streamlined decode kernel takes: vector scale loads (group 128 int4, K/128 a multiple of 8) ...
     (1, 2048, 528, "f16", "i4", 128, True, True, None),
     (16, 3072, 272, "f16", "i4", 128, True, False, "f16"),
