@@ -66,7 +66,7 @@ def run_workload(m, bench_cases, wl, stream, steps, warmup, with_cpu):
         roof["frac_of_instruction_peak"] = roof["achieved"] / PEAK[wl.instr_peak_key]
     if wl.bound == "hbm" and wl.flop:
         roof["tflops"] = wl.flop / (dev_ms * 1e-3) / 1e12
-    key = (wl.key[0], wl.key[1]) if wl.variant is None else (wl.key[0], wl.variant)
+    key = (wl.key[0], wl.key[1], wl.variant)
     traffic = bench_cases.PROFILED_TRAFFIC.get(key)
     if traffic and traffic[0] >= wl.bytes:
         roof["traffic"] = traffic[0]

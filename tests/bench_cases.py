@@ -10,15 +10,26 @@ import cases
 import oracle_api as orc
 
 
-# HBM-side traffic per step in bytes (read + written) as the hardware counters of an EARLIER profiling run of the same
-# bench command gave it (profiles/<file>: FETCH_SIZE and WRITE_SIZE, each scaled by what the counter reads for a byte
-# transpose of known size).  bench.py does not measure it; it copies the figure and names the file.  A figure below the
-# algorithmic bytes (the counter under-reads 16-byte-per-lane streams) is not evidence and is reported as null.
-# Keyed by (config, M of the weight-only configs, variant).
+# HBM-side traffic per step in bytes (read + written) as the memory-side request counters of an EARLIER profiling run of
+# the same bench command gave it (profiles/<file>: TCC_EA0_RDREQ / _32B and TCC_EA0_WRREQ / _64B, with the bytes per
+# request taken from two kernels of known size in the same run: a 16-byte-per-lane streaming read and a byte transpose).
+# bench.py does not measure it; it copies the figure and names the file.  A figure below the algorithmic bytes would not
+# be evidence and is reported as null.  Keyed by (config, M of the weight-only configs, variant).
 PROFILED_TRAFFIC = {
-    (2, None): (104.5e6, "profiles/qgemm_int8_w8a8_m2048_k4096_n11008.txt"),
-    (4, "fast"): (824.4e6, "profiles/qmm_fp8_block_m4096_k7168_n18432.txt"),
-    (5, None): (1802.2e6, "profiles/qgemm_mxfp4_b8_m4096_k8192_n8192.txt"),
+    (1, None, "warm"): (18.3e6, "profiles/wqmm_decode_w8a16_m16_k4096_n4096.txt"),
+    (1, None, "cold"): (18.3e6, "profiles/wqmm_decode_w8a16_m16_k4096_n4096_cold.txt"),
+    (2, None, None): (162.2e6, "profiles/qgemm_int8_w8a8_m2048_k4096_n11008.txt"),
+    (3, 1, "warm"): (144.0e6, "profiles/wqmm_decode_w4a16_m1_k8192_n28672.txt"),
+    (3, 1, "cold"): (140.9e6, "profiles/wqmm_decode_w4a16_m1_k8192_n28672_cold.txt"),
+    (3, 16, "warm"): (137.6e6, "profiles/wqmm_decode_w4a16_m16_k8192_n28672.txt"),
+    (3, 16, "cold"): (137.5e6, "profiles/wqmm_decode_w4a16_m16_k8192_n28672_cold.txt"),
+    (3, 64, "warm"): (151.3e6, "profiles/wqmm_decode_w4a16_m64_k8192_n28672.txt"),
+    (3, 64, "cold"): (151.2e6, "profiles/wqmm_decode_w4a16_m64_k8192_n28672_cold.txt"),
+    (3, 256, "warm"): (257.7e6, "profiles/wqmm_decode_w4a16_m256_k8192_n28672.txt"),
+    (3, 256, "cold"): (255.9e6, "profiles/wqmm_decode_w4a16_m256_k8192_n28672_cold.txt"),
+    (4, None, "exact"): (1220.2e6, "profiles/qmm_fp8_exact_m4096_k7168_n18432.txt"),
+    (4, None, "fast"): (1502.4e6, "profiles/qmm_fp8_block_m4096_k7168_n18432.txt"),
+    (5, None, None): (3084.6e6, "profiles/qgemm_mxfp4_b8_m4096_k8192_n8192.txt"),
 }
 
 
@@ -280,7 +291,7 @@ class ConfigWQ(Workload):
         m, K, N = self.m, self.K, self.N
         self.M = M
         self.inp = dict(self.inp_full, x=np.ascontiguousarray(self.inp_full["x"][:M]))
-        self.kernel = "wqmm_resx_kernel" if (self.cfg == 3 and M <= 3) else ("wqmm_rows_kernel" if M > 48 else "wqmm_stream_kernel")
+        self.kernel = "wqmm_resx_kernel" if (self.cfg == 3 and M <= 3) else ("wqmm_tile_kernel" if M > 128 else "wqmm_rows_kernel" if M > 48 else "wqmm_stream_kernel")
         self.t_x = m.Tensor((M, K), self.x_dt, self.d["x"])
         self.t_y = m.Tensor((M, N), self.x_dt, self.d_y)
         rc, ws, ex = m.weight_quant_batch_matmul_get_workspace(self.t_x, self.t_w[0], self.t_sc, self.t_y, offset=self.t_off,
