@@ -15,6 +15,7 @@ int launch_wqmm_plain(const OpsnnWqmmArgs& a, hipStream_t st);
 // Return OPSNN_NOT_TAKEN when the arguments are outside what the fast kernels handle.
 int launch_blockscale_mfma(const OpsnnQmmArgs& a, hipStream_t st);
 int launch_fp8_rowcol_mfma(const OpsnnQmmArgs& a, hipStream_t st, bool merged_scales_ok);
+int launch_rowcol_exact(const OpsnnQmmArgs& a, hipStream_t st, int ep_mode);   // qmm_fp8_exact.hip
 int launch_tcg_mfma(const OpsnnQmmArgs& a, hipStream_t st);
 uint64_t tcg_workspace_bytes(const OpsnnQmmArgs& a);
 int launch_mx_mfma(const OpsnnQmmArgs& a, hipStream_t st);
@@ -101,10 +102,18 @@ int64_t k_pad_for(const OpsnnQmmArgs& a, int mode)
     if (a.force_variant == OPSNN_VARIANT_PLAIN || opsnn_force_plain()) return 0;
     if (a.M * a.N < 64 * 64) return 0;   // below the matrix-core kernels' own minimum
     const bool i8 = a.x1_dtype == DT_I8 && a.x2_dtype == DT_I8, f8 = a.x1_dtype == DT_E4M3 && a.x2_dtype == DT_E4M3;
+    const bool f8any = (a.x1_dtype == DT_E4M3 || a.x1_dtype == DT_E5M2) && (a.x2_dtype == DT_E4M3 || a.x2_dtype == DT_E5M2);
     bool tail = false;
     if (mode == 0) tail = i8 && a.K % 16 != 0;
     else if (mode == 1) tail = (f8 || i8) && a.K % 128 != 0 && a.gsK == 128;
-    else if (mode == 3) tail = (i8 && !a.x1_scale && a.K % 16 != 0) || (f8 && a.x1_scale && a.K % 128 != 0);
+    else if (mode == 3) {
+        // the fp8 members of this family have no transposition step of their own: an operand that is not K-contiguous
+        // (or not 16-byte aligned) is gathered by the same copy
+        const bool f8_16 = f8any && (a.out_dtype == DT_BF16 || a.out_dtype == DT_F16) && (!a.bias || a.bias_dtype == DT_F32);
+        const bool loose = a.x1.col_stride != 1 || a.x2.row_stride != 1 || ((uint64_t)a.x1.row_stride | (uint64_t)a.x2.col_stride) % 16 ||
+                           ((uintptr_t)a.x1.ptr | (uintptr_t)a.x2.ptr) % 16;
+        tail = (i8 && !a.x1_scale && a.K % 16 != 0) || (f8_16 && (a.K % 128 != 0 || loose));
+    }
     if (!tail || a.K < 16) return 0;
     if (a.x1.batch_stride < 0 || a.x2.batch_stride < 0) return 0;
     return round_up(a.K, 128);
@@ -210,6 +219,19 @@ extern "C" int opsnnQmmTc(const OpsnnQmmArgs* a, void* stream)
         b.x2_scale_trunc = 0;   // UINT64 words are always truncated; a float scale is used as it is
         const int rc = opsnn_qmm_int8_impl(&b, stream);
         if (rc != OPSNN_NOT_TAKEN) return rc;
+    }
+    // fp8 operands, 16-bit output: the forms of compute_tc (qbmmv3_kernel_golden.py:390-475) on the exact matrix-core kernel --
+    // no per-token scale: (sum + float bias) * scale; both scales one element and no bias: sum * trunc19(scale * pertoken);
+    // otherwise (sum * scale) * pertoken + bias.  The last form with e4m3 operands and an fp32 scale goes on to the
+    // launcher below, which also knows the 8-bit-instruction variant; e5m2 operands, bf16 and 64-bit scale words, and
+    // the other two forms run here.
+    if (f8 && a->force_variant != OPSNN_VARIANT_PLAIN && !opsnn_force_plain()) {
+        const int ep = !a->x1_scale ? 1 : (a->x1_scale_len == 1 && a->x2_scale_len == 1 && !a->bias) ? 2 : 0;
+        const bool e4 = a->x1_dtype == DT_E4M3 && a->x2_dtype == DT_E4M3;
+        if (ep != 0 || !e4 || a->x2_scale_dtype != DT_F32) {
+            const int rc = launch_rowcol_exact(*a, (hipStream_t)stream, ep);
+            if (rc != OPSNN_NOT_TAKEN) return rc;
+        }
     }
     // fp8 e4m3 operands with a row scale and a column scale that are multiplied in separately (K-C, K-T, T-C with the
     // one-element x1Scale): matrix-core kernel when the layout allows, else the plain kernel

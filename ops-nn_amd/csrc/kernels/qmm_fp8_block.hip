@@ -527,7 +527,7 @@ int launch_mxfp8_mfma(const OpsnnQmmArgs& a, hipStream_t st)
 
 int launch_f8_wide(const QgemmParams& p, int fn, int64_t batch, int out_dt, hipStream_t st);   // qmm_int8_wide.hip
 int launch_blockscale_exact(const OpsnnQmmArgs& a, hipStream_t st);   // qmm_fp8_exact.hip
-int launch_rowcol_exact(const OpsnnQmmArgs& a, hipStream_t st);
+int launch_rowcol_exact(const OpsnnQmmArgs& a, hipStream_t st, int ep_mode);
 
 // fp8 e4m3 x fp4 e2m1 with e8m0 scales per 32 K on both operands (compute_mx of quant_batch_matmul_v4,
 // qbmmv4_kernel_golden.py:119-186): the MX mode with a 4-bit x2.  x2 [N, K] K-contiguous (two elements per byte),
@@ -572,7 +572,7 @@ int launch_fp8_rowcol_mfma(const OpsnnQmmArgs& a, hipStream_t st, bool merged_sc
     if (a.bias && a.bias_dtype != DT_F32) return OPSNN_NOT_TAKEN;
     if (a.K % 128 != 0 || a.M * a.N < 64 * 64 || a.x1.col_stride != 1 || a.x2.row_stride != 1) return OPSNN_NOT_TAKEN;
     if (!opsnnGetFp8Fast()) {   // exact products and sums unless the caller asked for the 8-bit matrix instruction
-        const int rc = launch_rowcol_exact(a, st);
+        const int rc = launch_rowcol_exact(a, st, 0);
         if (rc != OPSNN_NOT_TAKEN) return rc;
     }
     Fp8BlkParams p{};

@@ -44,9 +44,14 @@ struct Fp8xParams {
     int64_t s1_rs, s1_cs, s1_bs, s2_rs, s2_cs, s2_bs;
     int gsM;           // 1 or 128
     // row / column scale mode: out = (sum * cs[n * cs_stride]) * rs[m * rs_stride] + bias[n]; strides 0 (one scale) or 1
+    // ep_mode 1 (no row scale; a float bias is added BEFORE the scaling):   out = (sum + bias[n]) * cs[n]
+    // ep_mode 2 (one row scale, one column scale, merged and truncated):    out = sum * trunc19(cs[0] * rs[0])
+    // (compute_tc, qbmmv3_kernel_golden.py:390-475).  cs may be fp32, bf16 or 64-bit words (fp32 in the low word, upper
+    // 19 bits kept); rs may be null (= 1).
     const float* rs;
-    const float* cs;
+    const void* cs;
     int rs_stride, cs_stride;
+    int cs_dt, ep_mode;
     const float* bias;
     int64_t bias_bs;
 #if QG_DBG
@@ -62,18 +67,28 @@ __device__ __forceinline__ const int8_t* uniform_ptr(const int8_t* p)
 }
 
 // Eight e4m3 bytes (two registers) -> eight fp16 values (four registers), exact.
-__device__ __forceinline__ v8h widen8(int d0, int d1)
+// two of a dword's four fp8 codes -> fp16, exact: every e4m3 and every e5m2 value is an fp16 value (E5: the code is e5m2)
+template <bool E5> __device__ __forceinline__ v2h cvt_lo(uint32_t d)
 {
-    const v2h a = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8((uint32_t)d0, 1.0f, false);
-    const v2h b = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8((uint32_t)d0, 1.0f, true);
-    const v2h c = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8((uint32_t)d1, 1.0f, false);
-    const v2h d = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8((uint32_t)d1, 1.0f, true);
+    if constexpr (E5) return __builtin_amdgcn_cvt_scalef32_pk_f16_bf8(d, 1.0f, false);
+    else return __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(d, 1.0f, false);
+}
+template <bool E5> __device__ __forceinline__ v2h cvt_hi(uint32_t d)
+{
+    if constexpr (E5) return __builtin_amdgcn_cvt_scalef32_pk_f16_bf8(d, 1.0f, true);
+    else return __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(d, 1.0f, true);
+}
+template <bool E5> __device__ __forceinline__ v8h widen8(int d0, int d1)
+{
+    const v2h a = cvt_lo<E5>((uint32_t)d0), b = cvt_hi<E5>((uint32_t)d0), c = cvt_lo<E5>((uint32_t)d1), d = cvt_hi<E5>((uint32_t)d1);
     return (v8h){a[0], a[1], b[0], b[1], c[0], c[1], d[0], d[1]};
 }
 
-template <int OUT_DT, bool RC>
+// FMT: bit 0 set = x1 holds e5m2 codes, bit 1 set = x2 does (else e4m3)
+template <int OUT_DT, bool RC, int FMT = 0>
 __global__ __launch_bounds__(512, 1) void qmm_fp8_exact_kernel(Fp8xParams p, int tiles_m, int tiles_n)
 {
+    constexpr bool AE5 = (FMT & 1) != 0, BE5 = (FMT & 2) != 0;
     constexpr int BM = 256, BN = 128, BK = 128, NT = 512;
     constexpr int CPR = BK / 16, RPW = 16 / CPR;
     constexpr int TM = 64, TN = 64, FM = TM / 16, FN = TN / 16;
@@ -205,8 +220,7 @@ __global__ __launch_bounds__(512, 1) void qmm_fp8_exact_kernel(Fp8xParams p, int
     };
     auto widen4 = [&](int d, v8h& h, int half) {   // four bytes -> elements 4*half .. 4*half+3
         if (XABL & 1) { h[4 * half] = __builtin_bit_cast(v2h, d)[0]; return; }
-        const v2h lo = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8((uint32_t)d, 1.0f, false);
-        const v2h hi = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8((uint32_t)d, 1.0f, true);
+        const v2h lo = cvt_lo<BE5>((uint32_t)d), hi = cvt_hi<BE5>((uint32_t)d);
         h[4 * half] = lo[0]; h[4 * half + 1] = lo[1]; h[4 * half + 2] = hi[0]; h[4 * half + 3] = hi[1];
     };
     {   // first tile: everything converted up front
@@ -215,12 +229,12 @@ __global__ __launch_bounds__(512, 1) void qmm_fp8_exact_kernel(Fp8xParams p, int
         for (int j = 0; j < FM; j++) {
             const v8i r = load_frag(smem, a_rowbase + j * 16 * BK);
 #pragma unroll
-            for (int s = 0; s < 4; s++) fa[j][s] = widen8(r[2 * s], r[2 * s + 1]);
+            for (int s = 0; s < 4; s++) fa[j][s] = widen8<AE5>(r[2 * s], r[2 * s + 1]);
             a_half[j] = __builtin_shufflevector(r, r, 4, 5, 6, 7);   // converted once more behind the first instructions (same values)
         }
         b_raw = load_frag(smem, b_rowbase);
 #pragma unroll
-        for (int s = 0; s < 4; s++) fbc[0][s] = widen8(b_raw[2 * s], b_raw[2 * s + 1]);
+        for (int s = 0; s < 4; s++) fbc[0][s] = widen8<BE5>(b_raw[2 * s], b_raw[2 * s + 1]);
 #pragma unroll
         for (int j = 0; j < FM; j++) {
             sc[j] = 0.0f;   // multiplies the zero partial sums folded during the first tile's first fragment
@@ -320,9 +334,9 @@ __global__ __launch_bounds__(512, 1) void qmm_fp8_exact_kernel(Fp8xParams p, int
                         if (i == 0 && (s == 1 || s == 2)) fa[j][1 + s][0] = __builtin_bit_cast(v2h, a_half[j][2 * (s - 1)])[0];
                     } else {
                     if (i == FN - 1 && s >= 2)                // next tile's x1 fragments, K step s - 2 (low halves)
-                        fa[j][s - 2] = widen8(a_half[j][2 * (s - 2)], a_half[j][2 * (s - 2) + 1]);
+                        fa[j][s - 2] = widen8<AE5>(a_half[j][2 * (s - 2)], a_half[j][2 * (s - 2) + 1]);
                     if (i == 0 && (s == 1 || s == 2))         // this tile's x1 fragments, K steps 2 and 3 (high halves)
-                        fa[j][1 + s] = widen8(a_half[j][2 * (s - 1)], a_half[j][2 * (s - 1) + 1]);
+                        fa[j][1 + s] = widen8<AE5>(a_half[j][2 * (s - 1)], a_half[j][2 * (s - 1) + 1]);
                     }
                     __builtin_amdgcn_sched_barrier(0);
                 }
@@ -373,7 +387,7 @@ __global__ __launch_bounds__(512, 1) void qmm_fp8_exact_kernel(Fp8xParams p, int
 #pragma unroll
         for (int j = 0; j < FM; j++) {
             const int64_t mrow = m0 + wm * TM + j * 16 + frow;
-            rs_j[j] = p.rs[(mrow < p.M ? mrow : p.M - 1) * p.rs_stride];
+            rs_j[j] = p.rs ? p.rs[(mrow < p.M ? mrow : p.M - 1) * p.rs_stride] : 1.0f;
         }
     }
 #pragma unroll
@@ -386,8 +400,20 @@ __global__ __launch_bounds__(512, 1) void qmm_fp8_exact_kernel(Fp8xParams p, int
 #pragma unroll
                 for (int r = 0; r < 4; r++) {
                     const int64_t ni = nb + r < p.N ? nb + r : p.N - 1;
-                    v[r] = (v[r] * p.cs[ni * p.cs_stride]) * rs_j[j];
-                    if (p.bias) v[r] = v[r] + p.bias[bz * p.bias_bs + ni];
+                    const int64_t ci = ni * p.cs_stride;
+                    float csv;
+                    if (p.cs_dt == DT_U64) csv = u2f((uint32_t)((const uint64_t*)p.cs)[ci] & 0xFFFFE000u);
+                    else if (p.cs_dt == DT_BF16) csv = bf16_to_f32(((const uint16_t*)p.cs)[ci]);
+                    else csv = ((const float*)p.cs)[ci];
+                    if (p.ep_mode == 1) {
+                        if (p.bias) v[r] = v[r] + p.bias[bz * p.bias_bs + ni];
+                        v[r] = v[r] * csv;
+                    } else if (p.ep_mode == 2) {
+                        v[r] = v[r] * u2f(f2u(csv * rs_j[j]) & 0xFFFFE000u);
+                    } else {
+                        v[r] = (v[r] * csv) * rs_j[j];
+                        if (p.bias) v[r] = v[r] + p.bias[bz * p.bias_bs + ni];
+                    }
                 }
             }
             *(v4us_a*)(ep + frow * EP_PITCH + (i * 16 + 4 * fq) * 2) = pack4_b16<OUT_DT>(v);
@@ -412,13 +438,13 @@ __global__ __launch_bounds__(512, 1) void qmm_fp8_exact_kernel(Fp8xParams p, int
     }
 }
 
-template <int OUT_DT, bool RC>
+template <int OUT_DT, bool RC, int FMT = 0>
 static int launch_fp8_exact(const Fp8xParams& p, int64_t batch, hipStream_t st)
 {
     const int tiles_m = (int)((p.M + 255) / 256), tiles_n = (int)((p.N + 127) / 128);
     dim3 grid((unsigned)(tiles_m * tiles_n), (unsigned)batch);
     const size_t lds = 3 * (size_t)(256 * 128 + 128 * 128 + (RC ? 0 : 512 * 4));
-    auto k = qmm_fp8_exact_kernel<OUT_DT, RC>;
+    auto k = qmm_fp8_exact_kernel<OUT_DT, RC, FMT>;
     static bool attr_set = false;
     if (!attr_set) {
         hipError_t e = hipFuncSetAttribute((const void*)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
@@ -452,24 +478,35 @@ int launch_blockscale_exact(const OpsnnQmmArgs& a, hipStream_t st)
     return launch_fp8_exact<DT_F16, false>(p, a.batch, st);
 }
 
-// fp8 e4m3 with one fp32 scale per row of x1 (or one) and one per column of x2 (or one), optional fp32 bias.
-int launch_rowcol_exact(const OpsnnQmmArgs& a, hipStream_t st)
+// fp8 (e4m3 or e5m2, each operand by itself) with scales applied to the finished sums: one fp32 scale per row of x1 (or
+// one, or none) and one per column of x2 (or one; fp32, bf16 or 64-bit words), optional fp32 bias.  ep_mode as in
+// Fp8xParams: 0 = (sum * cs) * rs + bias (compute_pertoken; compute_tc with a per-token scale), 1 = (sum + bias) * cs,
+// 2 = sum * trunc19(cs * rs).
+int launch_rowcol_exact(const OpsnnQmmArgs& a, hipStream_t st, int ep_mode)
 {
-    if (a.x1_dtype != DT_E4M3 || a.x2_dtype != DT_E4M3) return OPSNN_NOT_TAKEN;
+    const bool e1 = a.x1_dtype == DT_E5M2, e2 = a.x2_dtype == DT_E5M2;
+    if ((a.x1_dtype != DT_E4M3 && !e1) || (a.x2_dtype != DT_E4M3 && !e2)) return OPSNN_NOT_TAKEN;
     if (a.out_dtype != DT_BF16 && a.out_dtype != DT_F16) return OPSNN_NOT_TAKEN;
-    if (!a.x1_scale || !a.x2_scale || a.x2_scale_dtype != DT_F32) return OPSNN_NOT_TAKEN;
+    if (!a.x2_scale || (a.x2_scale_dtype != DT_F32 && a.x2_scale_dtype != DT_BF16 && a.x2_scale_dtype != DT_U64)) return OPSNN_NOT_TAKEN;
+    if (ep_mode != 1 && !a.x1_scale) return OPSNN_NOT_TAKEN;
     if (a.bias && a.bias_dtype != DT_F32) return OPSNN_NOT_TAKEN;
     if (a.K % 128 != 0 || a.M * a.N < 64 * 64 || a.x1.col_stride != 1 || a.x2.row_stride != 1) return OPSNN_NOT_TAKEN;
     Fp8xParams p{};
     p.a = (const int8_t*)a.x1.ptr; p.b = (const int8_t*)a.x2.ptr;
     p.lda = a.x1.row_stride; p.ldb = a.x2.col_stride; p.a_bs = a.x1.batch_stride; p.b_bs = a.x2.batch_stride;
     p.out = a.out; p.M = a.M; p.N = a.N; p.K = a.K; p.gsM = 1;
-    p.rs = (const float*)a.x1_scale; p.rs_stride = a.x1_scale_len == 1 ? 0 : 1;
-    p.cs = (const float*)a.x2_scale; p.cs_stride = a.x2_scale_len == 1 ? 0 : 1;
+    p.rs = ep_mode == 1 ? nullptr : (const float*)a.x1_scale; p.rs_stride = a.x1_scale_len == 1 ? 0 : 1;
+    p.cs = a.x2_scale; p.cs_stride = a.x2_scale_len == 1 ? 0 : 1; p.cs_dt = a.x2_scale_dtype;
+    p.ep_mode = ep_mode;
     p.bias = (const float*)a.bias; p.bias_bs = a.bias_batch_stride;
     if (((uintptr_t)p.a | (uintptr_t)p.b | (uint64_t)p.lda | (uint64_t)p.ldb | (uint64_t)p.a_bs | (uint64_t)p.b_bs) % 16) return OPSNN_NOT_TAKEN;
-    if (a.out_dtype == DT_BF16) return launch_fp8_exact<DT_BF16, true>(p, a.batch, st);
-    return launch_fp8_exact<DT_F16, true>(p, a.batch, st);
+    const bool bf = a.out_dtype == DT_BF16;
+    switch ((e1 ? 1 : 0) | (e2 ? 2 : 0)) {
+        case 0: return bf ? launch_fp8_exact<DT_BF16, true, 0>(p, a.batch, st) : launch_fp8_exact<DT_F16, true, 0>(p, a.batch, st);
+        case 1: return bf ? launch_fp8_exact<DT_BF16, true, 1>(p, a.batch, st) : launch_fp8_exact<DT_F16, true, 1>(p, a.batch, st);
+        case 2: return bf ? launch_fp8_exact<DT_BF16, true, 2>(p, a.batch, st) : launch_fp8_exact<DT_F16, true, 2>(p, a.batch, st);
+        default: return bf ? launch_fp8_exact<DT_BF16, true, 3>(p, a.batch, st) : launch_fp8_exact<DT_F16, true, 3>(p, a.batch, st);
+    }
 }
 
 }  // namespace opsnn

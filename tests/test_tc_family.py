@@ -264,3 +264,44 @@ def test_gpu_fp8_row_and_column_scales_on_the_matrix_cores(gpu, M, K, N, s_len, 
     finally:
         m.lib().opsnnSetForcePlain(0)
     assert np.array_equal(exact, want)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("M,K,N,in_dt,s_dt,s_len,bias,out_dt,tB,pt", [
+    # no per-token scale (the scale is then a packed 64-bit word, 19 bits kept): (sum + float bias) * scale
+    (256, 2048, 384, "e4m3", "u64", "N", True, "bf16", True, False),
+    (300, 384, 260, "e4m3", "u64", 1, False, "f16", True, False),
+    # both scales one element, no bias: merged and truncated
+    (256, 1024, 256, "e4m3", "f32", 1, False, "bf16", True, True),
+    # one-element per-token scale with a bias: multiplied separately, bias after
+    (200, 384, 136, "e4m3", "f32", 1, True, "f16", True, True),
+    # e5m2 operands: per-token x per-channel with bias, packed scale without a per-token scale, one scale per row
+    (256, 2048, 256, "e5m2", "f32", "N", True, "bf16", True, True),
+    (130, 384, 200, "e5m2", "u64", "N", False, "f16", True, False),
+    (128, 256, 192, "e5m2", "f32", "N", True, "bf16", True, "M"),
+    # K tails and an N-contiguous x2: gathered into zero-padded K-contiguous copies first
+    (256, 1000, 264, "e4m3", "u64", "N", True, "bf16", True, False),
+    (128, 512, 256, "e4m3", "f32", 1, False, "f16", False, True),
+    (160, 200, 136, "e5m2", "f32", "N", True, "bf16", False, True),
+])
+def test_gpu_fp8_tc_forms_on_the_matrix_cores(gpu, M, K, N, in_dt, s_dt, s_len, bias, out_dt, tB, pt):
+    """The fp8 members of the per-tensor / per-channel family with a 16-bit output on the exact matrix-core kernel (fp16
+    products of the widened operands, fp32 sums): bar of any fp32-accumulating device; the same call on the plain kernel is
+    bit-identical to the oracle (test_gpu_matches_oracle covers the small shapes that stay there)."""
+    m = gpu
+    dt = {"e4m3": m.ACL_FLOAT8_E4M3FN, "e5m2": m.ACL_FLOAT8_E5M2, "u64": m.ACL_UINT64, "f32": m.ACL_FLOAT, "bf16": m.ACL_BF16,
+          "f16": m.ACL_FLOAT16}
+    print(f"case fp8 tc form {M}x{K}x{N} in={in_dt} scale={s_dt}/{s_len} bias={bias} out={out_dt} tB={tB} pt={pt}", flush=True)
+    inp = cases.make_tc_inputs(m, M, K, N, M + K, dt[in_dt], dt[s_dt], 1 if s_len == 1 else N, m.ACL_FLOAT if bias else None, tB,
+                               pertoken=pt, e5m2=in_dt == "e5m2")
+    want = cases.oracle_tc(m, inp, M, K, N, dt[out_dt])
+    got = cases.run_tc_aclnn(m, inp, M, K, N, dt[out_dt])
+    code = orc.BF16 if out_dt == "bf16" else orc.F16
+    g, w = orc.b16_to_f32(got, code), orc.b16_to_f32(want, code)
+    assert np.isfinite(g).all()
+    mx, mean = orc.rel_err_stats(g, w)
+    assert mean <= 2.0 ** -10 and mx <= 2.0 ** -7, f"max rel {mx:.3e} mean rel {mean:.3e}"
+    assert orc.isclose_fraction(g, w) <= 1e-3
+    differ = float(np.mean(got != want))
+    print(f"   {differ:.2e} of outputs differ from the ascending-k oracle", flush=True)
+    assert differ < 2e-2   # summation order only: a wrong scale decoding or epilogue order would change most outputs
