@@ -96,6 +96,11 @@ extern "C" aclnnStatus aclnnQuantMatmulWeightNzGetWorkspaceSize(const aclTensor*
     const aclnnStatus rc = aclnnQuantMatmulV5GetWorkspaceSize(x1, &nd, x1Scale, x2Scale, yScale, x1Offset, x2Offset, yOffset, bias, transposeX1,
                                                               transposeX2, groupSize, out, &inner, &ex);
     if (rc != ACLNN_SUCCESS) return rc;
+    if (!ex->batch_runs.empty()) {   // several launches with their own operand addresses: not combined with the NZ pre-step
+        aclDestroyAclOpExecutor(ex);
+        set_error("%s: batch dims that broadcast partially are not supported with a FRACTAL_NZ x2", api);
+        return ACLNN_ERR_PARAM_INVALID;
+    }
     if (ex->kind != OpKind::None) {
         ex->nz = step;
         ex->workspace_size = nz_front_bytes(*ex) + inner;

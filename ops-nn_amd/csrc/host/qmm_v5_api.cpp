@@ -70,10 +70,23 @@ struct Ctx {
     }
 };
 
+// A matrix operand whose view is neither dense nor a dense transpose, but regular: 8-bit elements, positive strides on
+// the last two dims, and batch dims that collapse into one stride.  The reference makes such a view contiguous by a copy
+// (quant_matmul_common_check.cpp:106-123); here the kernels take the strides as they are (the matrix-core route gathers
+// the operand into the workspace, the plain kernels index it directly).
+bool regular_strided_matrix(const TView& t)
+{
+    if (t.rank() < 2 || dtype_bits(t.dtype) != 8) return false;
+    if (t.stride(-1) < 1 || t.stride(-2) < 1) return false;
+    for (int64_t i = t.rank() - 4; i >= 0; i--)
+        if (t.strides[(size_t)i] != t.strides[(size_t)i + 1] * t.shape[(size_t)i + 1]) return false;
+    return t.rank() < 3 || t.stride(-3) >= 0;
+}
+
 // quant_matmul_common_check.cpp:106-123.  A last-two-dims-transposed view becomes a dense view of the
-// swapped shape and flips the flag.  Other non-contiguous views would need a gather copy, which this
-// implementation does not provide: they are rejected.
-aclnnStatus contiguous_process(TView& t, bool& transpose, const char* name)
+// swapped shape and flips the flag.  Other non-contiguous views are accepted for the two matrix operands when they are
+// regular (see above) and rejected otherwise.
+aclnnStatus contiguous_process(TView& t, bool& transpose, const char* name, bool matrix_operand = false)
 {
     if (!t.present) return ACLNN_SUCCESS;
     if (t.rank() >= 2 && is_transposed_last2(t)) {
@@ -81,8 +94,9 @@ aclnnStatus contiguous_process(TView& t, bool& transpose, const char* name)
         transpose = !transpose;
         return ACLNN_SUCCESS;
     }
-    if (!is_contiguous(t)) INVALID("%s: %s has strides that are neither dense nor a last-two-dims transpose", kApi, name);
-    return ACLNN_SUCCESS;
+    if (is_contiguous(t)) return ACLNN_SUCCESS;
+    if (matrix_operand && regular_strided_matrix(t)) return ACLNN_SUCCESS;
+    INVALID("%s: %s has strides that are neither dense nor a last-two-dims transpose", kApi, name);
 }
 
 // aclnn_quant_matmul_v5.cpp:908-945: an MX scale [.., a, b, 2] whose strides describe [.., b, a, 2].
@@ -465,6 +479,12 @@ OpsnnMat mat_of(const TView& t, bool transposed)
     // logical [R, C] over a dense view of [.., R, C] (or [.., C, R] when transposed)
     OpsnnMat m{};
     m.ptr = t.ptr_at(0);
+    if (!is_contiguous(t)) {   // a regular strided view (contiguous_process admitted it): its own strides
+        m.row_stride = transposed ? t.stride(-1) : t.stride(-2);
+        m.col_stride = transposed ? t.stride(-2) : t.stride(-1);
+        m.batch_stride = t.rank() > 2 ? t.stride(-3) : 0;
+        return m;
+    }
     int64_t d1 = t.dim(-1);
     if (transposed) { m.row_stride = 1; m.col_stride = d1; }
     else { m.row_stride = d1; m.col_stride = 1; }
@@ -529,7 +549,7 @@ extern "C" aclnnStatus aclnnQuantMatmulV5GetWorkspaceSize(const aclTensor* x1, c
     // view normalisation (PreMatmulCalcProcess, aclnn_quant_matmul_v5.cpp:967-1016)
     aclnnStatus rc;
     bool tmp = false;
-    if ((rc = contiguous_process(c.x1, c.tA, "x1")) != ACLNN_SUCCESS) return rc;
+    if ((rc = contiguous_process(c.x1, c.tA, "x1", true)) != ACLNN_SUCCESS) return rc;
     const bool mx_like = c.mx() && (c.fp4_in() || c.fp8_in() || isA8W4F);
     if (c.x1s.present) {
         rc = mx_like ? mx_scale_process(c.x1s, "x1Scale") : contiguous_process(c.x1s, tmp, "x1Scale");
@@ -540,7 +560,7 @@ extern "C" aclnnStatus aclnnQuantMatmulV5GetWorkspaceSize(const aclTensor* x1, c
     if ((rc = contiguous_process(c.bias, tmp, "bias")) != ACLNN_SUCCESS) return rc;
     if ((rc = contiguous_process(c.x2o, tmp, "x2Offset")) != ACLNN_SUCCESS) return rc;
     if ((rc = contiguous_process(c.ys, tmp, "yScale")) != ACLNN_SUCCESS) return rc;
-    if ((rc = contiguous_process(c.x2, c.tB, "x2")) != ACLNN_SUCCESS) return rc;
+    if ((rc = contiguous_process(c.x2, c.tB, "x2", true)) != ACLNN_SUCCESS) return rc;
 
     if (isA8W4) {
         if (c.a8w4i_raw()) FAIL(ACLNN_ERR_RUNTIME_ERROR, "%s: int8 x int4 (A8W4 int) is not supported on this device generation", kApi);
@@ -595,9 +615,9 @@ extern "C" aclnnStatus aclnnQuantMatmulV5GetWorkspaceSize(const aclTensor* x1, c
     for (int64_t i = 0; i < c.out.rank() - 2; i++) ob *= c.out.dim(i);
     if (c.x1.rank() == 2 && c.x2.rank() == 2) ob = 1;
     a.batch = ob;
-    // batch broadcasting is supported when an operand has no batch dims (or all ones) or the full batch
-    if (b1 != 1 && b1 != ob) INVALID("%s: partial batch broadcast of x1 is not supported", kApi);
-    if (b2 != 1 && b2 != ob) INVALID("%s: partial batch broadcast of x2 is not supported", kApi);
+    // one launch covers an operand with no batch dims (or all ones) or with the full out batch; any other broadcast
+    // pattern (qbmmv3_kernel_golden.py:288-330 broadcasts any pair) is split into launches over the innermost batch dim below
+    const bool general_broadcast = (b1 != 1 && b1 != ob) || (b2 != 1 && b2 != ob);
     if (b1 == 1) a.x1.batch_stride = 0;
     if (b2 == 1) a.x2.batch_stride = 0;
     if (c.bias.present) {
@@ -672,6 +692,55 @@ extern "C" aclnnStatus aclnnQuantMatmulV5GetWorkspaceSize(const aclTensor* x1, c
         FAIL(ACLNN_ERR_INNER_TILING_ERROR, "%s: no kernel for x1 %s, x2 %s, x2Scale %s, out %s on this device yet", kApi,
              dtype_name(c.x1.dtype), dtype_name(c.x2.dtype), dtype_name(c.x2s.dtype), dtype_name(c.out.dtype));
     }
+    if (general_broadcast) {
+        if (!is_contiguous(c.x1) || !is_contiguous(c.x2)) INVALID("%s: batch dims that broadcast partially need dense x1 and x2", kApi);
+        if (c.bias.present && c.bias.rank() == 3) INVALID("%s: a 3-D bias cannot go with partially broadcast batch dims", kApi);
+        const int64_t nb = c.out.rank() - 2, r1 = c.x1.rank() - 2, r2 = c.x2.rank() - 2;
+        std::vector<int64_t> od((size_t)nb), d1((size_t)nb, 1), d2((size_t)nb, 1);
+        for (int64_t i = 0; i < nb; i++) od[(size_t)i] = c.out.dim(i);
+        for (int64_t i = 0; i < r1; i++) d1[(size_t)(nb - r1 + i)] = c.x1.dim(i);
+        for (int64_t i = 0; i < r2; i++) d2[(size_t)(nb - r2 + i)] = c.x2.dim(i);
+        const int64_t L = nb - 1, inner = od[(size_t)L];
+        int64_t outer = 1;
+        for (int64_t i = 0; i < L; i++) outer *= od[(size_t)i];
+        auto bytes_of = [](int64_t elems, int dt) { return elems * dtype_bits((aclDataType)dt) / 8; };
+        const int64_t x1_slice = a.x1.batch_stride, x2_slice = a.x2.batch_stride;   // elements per batch slice (dense operands)
+        const int64_t s1_slice = a.x1_scale_mat.batch_stride, s2_slice = a.x2_scale_mat.batch_stride;
+        // element size of the scale tables: fp32 in the block-scale modes, e8m0 bytes in the MX modes; no other mode gives
+        // its scales batch dims
+        const int64_t s_esize = mode == 2 ? 1 : 4;
+        const int64_t out_slice_bytes = bytes_of(c.M * c.N, c.out.dtype);
+        for (int64_t o = 0; o < outer; o++) {
+            int64_t rem = o, f1 = 0, f2 = 0, st1 = d1[(size_t)L], st2 = d2[(size_t)L];   // flat slice index of the run's first slice
+            for (int64_t i = L - 1; i >= 0; i--) {
+                const int64_t idx = rem % od[(size_t)i];
+                rem /= od[(size_t)i];
+                if (d1[(size_t)i] > 1) f1 += idx * st1;
+                if (d2[(size_t)i] > 1) f2 += idx * st2;
+                st1 *= d1[(size_t)i];
+                st2 *= d2[(size_t)i];
+            }
+            OpsnnQmmArgs q = a;
+            q.batch = inner;
+            q.x1.ptr = (const char*)a.x1.ptr + bytes_of(f1 * x1_slice, a.x1_dtype);
+            q.x2.ptr = (const char*)a.x2.ptr + bytes_of(f2 * x2_slice, a.x2_dtype);
+            q.x1.batch_stride = d1[(size_t)L] > 1 ? x1_slice : 0;
+            q.x2.batch_stride = d2[(size_t)L] > 1 ? x2_slice : 0;
+            if (a.x1_scale_mat.ptr) {
+                q.x1_scale_mat.ptr = (const char*)a.x1_scale_mat.ptr + f1 * s1_slice * s_esize;
+                q.x1_scale_mat.batch_stride = d1[(size_t)L] > 1 ? s1_slice : 0;
+            }
+            if (a.x2_scale_mat.ptr) {
+                q.x2_scale_mat.ptr = (const char*)a.x2_scale_mat.ptr + f2 * s2_slice * s_esize;
+                q.x2_scale_mat.batch_stride = d2[(size_t)L] > 1 ? s2_slice : 0;
+            }
+            q.out = (char*)a.out + o * inner * out_slice_bytes;
+            ex->batch_runs.push_back(q);
+        }
+        a.batch = inner;   // the workspace one launch needs; the launches run one after the other on the stream and share it
+        a.x1.batch_stride = ex->batch_runs[0].x1.batch_stride;
+        a.x2.batch_stride = ex->batch_runs[0].x2.batch_stride;
+    }
     ex->workspace_size = opsnnQmmWorkspace(&a, mode);
     *workspaceSize = ex->workspace_size;
     *executor = (aclOpExecutor*)executor_publish(ex.release());
@@ -700,13 +769,23 @@ extern "C" aclnnStatus aclnnQuantMatmulV5(void* workspace, uint64_t workspaceSiz
         ex->qmm.x2.ptr = nd;
         ex->qmm.workspace = ex->workspace_size > nz_front_bytes(*ex) ? rest : nullptr;
     }
-    switch (ex->kind) {
-        case OpKind::QmmInt8: rc = opsnnQmmInt8(&ex->qmm, stream); break;
-        case OpKind::QmmBlockScale: rc = opsnnQmmBlockScale(&ex->qmm, stream); break;
-        case OpKind::QmmMx: rc = opsnnQmmMx(&ex->qmm, stream); break;
-        case OpKind::QmmTc: rc = opsnnQmmTc(&ex->qmm, stream); break;
-        case OpKind::QmmGroup: rc = opsnnQmmGroup(&ex->qmm, stream); break;
-        default: rc = -100; break;
+    auto launch = [&](const OpsnnQmmArgs& q) -> int {
+        switch (ex->kind) {
+            case OpKind::QmmInt8: return opsnnQmmInt8(&q, stream);
+            case OpKind::QmmBlockScale: return opsnnQmmBlockScale(&q, stream);
+            case OpKind::QmmMx: return opsnnQmmMx(&q, stream);
+            case OpKind::QmmTc: return opsnnQmmTc(&q, stream);
+            case OpKind::QmmGroup: return opsnnQmmGroup(&q, stream);
+            default: return -100;
+        }
+    };
+    if (ex->batch_runs.empty()) {
+        rc = launch(ex->qmm);
+    } else {
+        for (OpsnnQmmArgs& q : ex->batch_runs) {   // partially broadcast batch dims: one launch per outer combination
+            q.workspace = ex->qmm.workspace;
+            if ((rc = launch(q)) != 0) break;
+        }
     }
     if (rc != 0) FAIL(rc < 0 ? ACLNN_ERR_INNER_TILING_ERROR : ACLNN_ERR_RUNTIME_ERROR, "aclnnQuantMatmulV5: launch failed with code %d", rc);
     return ACLNN_SUCCESS;

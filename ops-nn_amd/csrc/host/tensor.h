@@ -42,6 +42,9 @@ struct aclOpExecutorImpl {
     // Right operand handed over in FRACTAL_NZ (the ...WeightNz / ...Nz entry points): phase 2 first re-lays it out as the
     // dense ND matrix into the front of the workspace (nd_bytes, rounded up to 256), points the operand there, and gives
     // the rest of the workspace to the launcher.
+    // General batch broadcast of aclnnQuantMatmulV5 (x1 [2, 1, M, K] with x2 [1, 3, K, N] and the like): one launch per
+    // combination of the outer batch dims, each over the innermost batch dim; empty for the usual cases, which are one launch.
+    std::vector<OpsnnQmmArgs> batch_runs;
     struct NzStep { bool active = false; const void* src = nullptr; int64_t rows = 0, row_bytes = 0, batch = 1; int c0 = 0; uint64_t nd_bytes = 0; } nz;
 };
 

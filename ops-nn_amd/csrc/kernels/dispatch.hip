@@ -103,16 +103,18 @@ int64_t k_pad_for(const OpsnnQmmArgs& a, int mode)
     if (a.M * a.N < 64 * 64) return 0;   // below the matrix-core kernels' own minimum
     const bool i8 = a.x1_dtype == DT_I8 && a.x2_dtype == DT_I8, f8 = a.x1_dtype == DT_E4M3 && a.x2_dtype == DT_E4M3;
     const bool f8any = (a.x1_dtype == DT_E4M3 || a.x1_dtype == DT_E5M2) && (a.x2_dtype == DT_E4M3 || a.x2_dtype == DT_E5M2);
+    // an operand the matrix-core kernels cannot fetch as it lies (not K-contiguous, or rows not 16-byte aligned) is gathered
+    // by the same copy; a dense N-contiguous x2 is not: the int8 and block-scale launchers transpose it themselves, faster
+    const bool x1_ok = a.x1.col_stride == 1 && (((uint64_t)a.x1.row_stride | (uint64_t)a.x1.batch_stride | (uintptr_t)a.x1.ptr) % 16) == 0;
+    const bool x2_k = a.x2.row_stride == 1 && (((uint64_t)a.x2.col_stride | (uint64_t)a.x2.batch_stride | (uintptr_t)a.x2.ptr) % 16) == 0;
+    const bool x2_n = a.x2.col_stride == 1 && a.x2.row_stride == a.N && (a.x2.batch_stride == 0 || a.x2.batch_stride == a.K * a.N);
     bool tail = false;
-    if (mode == 0) tail = i8 && a.K % 16 != 0;
-    else if (mode == 1) tail = (f8 || i8) && a.K % 128 != 0 && a.gsK == 128;
+    if (mode == 0) tail = i8 && (a.K % 16 != 0 || !x1_ok || !(x2_k || x2_n));
+    else if (mode == 1) tail = (f8 || i8) && a.gsK == 128 && (a.K % 128 != 0 || !x1_ok || !(x2_k || x2_n));
     else if (mode == 3) {
-        // the fp8 members of this family have no transposition step of their own: an operand that is not K-contiguous
-        // (or not 16-byte aligned) is gathered by the same copy
+        // (the fp8 members of this family have no transposition step of their own)
         const bool f8_16 = f8any && (a.out_dtype == DT_BF16 || a.out_dtype == DT_F16) && (!a.bias || a.bias_dtype == DT_F32);
-        const bool loose = a.x1.col_stride != 1 || a.x2.row_stride != 1 || ((uint64_t)a.x1.row_stride | (uint64_t)a.x2.col_stride) % 16 ||
-                           ((uintptr_t)a.x1.ptr | (uintptr_t)a.x2.ptr) % 16;
-        tail = (i8 && !a.x1_scale && a.K % 16 != 0) || (f8_16 && (a.K % 128 != 0 || loose));
+        tail = (i8 && !a.x1_scale && (a.K % 16 != 0 || !x1_ok || !(x2_k || x2_n))) || (f8_16 && (a.K % 128 != 0 || !x1_ok || !x2_k));
     }
     if (!tail || a.K < 16) return 0;
     if (a.x1.batch_stride < 0 || a.x2.batch_stride < 0) return 0;

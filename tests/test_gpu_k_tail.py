@@ -82,3 +82,70 @@ def test_fp8_row_and_column_scales_k_tail(gpu, M, K, N, s_len, pt):
     want = cases.oracle_tc(m, inp, M, K, N, m.ACL_BF16)
     got = cases.run_tc_aclnn(m, inp, M, K, N, m.ACL_BF16)
     check_close(got, want, orc.BF16, "fp8 row and column scales with a K tail")
+
+
+def _strided_case(m, M, K, N, x1_pad, x2_step, batch=1):
+    """int8 operands as regular strided views: x1 rows of K inside storage rows of K + x1_pad, x2 [K, N] as every
+    x2_step-th column of a [K, N * x2_step] storage.  Returns (logical inputs, device tensors, storages kept alive)."""
+    inp = cases.make_qmm_int8_inputs(m, M, K, N, M + K, m.ACL_BF16, False, batch=batch)
+    rng = np.random.default_rng(5)
+    s1 = rng.integers(-128, 128, size=(batch, M, K + x1_pad), dtype=np.int8)
+    s1[:, :, :K] = inp["x1"]
+    s2 = rng.integers(-128, 128, size=(batch, K, N * x2_step), dtype=np.int8)
+    s2[:, :, ::x2_step] = inp["x2"]
+    d1, d2 = m.DeviceBuffer(host=s1), m.DeviceBuffer(host=s2)
+    bshape = (batch,) if batch > 1 else ()
+    bs1 = (M * (K + x1_pad),) if batch > 1 else ()
+    bs2 = (K * N * x2_step,) if batch > 1 else ()
+    x1 = m.Tensor(bshape + (M, K), m.ACL_INT8, d1, strides=bs1 + (K + x1_pad, 1), storage_shape=bshape + (M, K + x1_pad))
+    x2 = m.Tensor(bshape + (K, N), m.ACL_INT8, d2, strides=bs2 + (N * x2_step, x2_step), storage_shape=bshape + (K, N * x2_step))
+    return inp, x1, x2, (d1, d2)
+
+
+@pytest.mark.parametrize("M,K,N,x1_pad,x2_step,batch", [
+    (256, 512, 384, 48, 2, 1),     # x1 rows 16-byte aligned but not dense (taken as it lies), x2 every other column (gathered)
+    (130, 1000, 264, 7, 3, 1),     # nothing aligned, a K tail on top
+    (128, 256, 192, 16, 2, 3),     # batched
+])
+def test_int8_regular_strided_views(gpu, M, K, N, x1_pad, x2_step, batch):
+    """Views that are neither dense nor a dense transpose (the reference copies them contiguous; here they are gathered
+    into the workspace on the way to the matrix cores): same bits as the dense call."""
+    m = gpu
+    print(f"case int8 strided views M={M} K={K} N={N} x1_pad={x1_pad} x2_step={x2_step} batch={batch}", flush=True)
+    inp, x1, x2, keep = _strided_case(m, M, K, N, x1_pad, x2_step, batch)
+    want, _ = cases.oracle_qmm_int8(m, inp, M, K, N, False, m.ACL_BF16)
+    d = {k: m.DeviceBuffer(host=v) for k, v in inp.items() if isinstance(v, np.ndarray) and k not in ("x1", "x2")}
+    bshape = (batch,) if batch > 1 else ()
+    d_out = m.DeviceBuffer(batch * M * N * 2)
+    d_out.fill(0xFF)
+    s1 = m.Tensor((M,), m.ACL_FLOAT, d["s1"])
+    s2 = m.Tensor((inp["s2"].size,), inp["s2_dtype"], d["s2"])
+    b = m.Tensor((N,), inp["bias_dtype"], d["bias"])
+    out = m.Tensor(bshape + (M, N), m.ACL_BF16, d_out)
+    rc, ws, ex = m.quant_matmul_v5_get_workspace(x1, x2, s1, s2, out, bias=b)
+    assert rc == 0 and ws == _pad_bytes(M, K, N, batch), (rc, ws)
+    m.lib().aclDestroyAclOpExecutor(ex)
+    wbuf = m.quant_matmul_v5(x1, x2, s1, s2, out, bias=b)
+    m.check(m.lib().aclrtSynchronizeDevice(), "sync")
+    got = d_out.to_host(np.uint16, (batch, M, N))
+    assert np.array_equal(got, want)
+    # and on the plain kernels, which index the views directly
+    m.lib().opsnnSetForcePlain(1)
+    try:
+        d_out.fill(0xFF)
+        wbuf = m.quant_matmul_v5(x1, x2, s1, s2, out, bias=b)
+        m.check(m.lib().aclrtSynchronizeDevice(), "sync")
+    finally:
+        m.lib().opsnnSetForcePlain(0)
+    assert np.array_equal(d_out.to_host(np.uint16, (batch, M, N)), want)
+
+
+def test_irregular_views_are_still_rejected(gpu):
+    m = gpu
+    d = m.DeviceBuffer(4096 * 16)
+    x1 = m.Tensor((2, 2, 16, 32), m.ACL_INT8, d, strides=(4096, 1000, 64, 1), storage_shape=(16, 4096))   # batch dims do not collapse
+    x2 = m.Tensor((32, 16), m.ACL_INT8, d)
+    s2 = m.Tensor((16,), m.ACL_FLOAT, d)
+    out = m.Tensor((2, 2, 16, 16), m.ACL_BF16, d)
+    rc, ws, ex = m.quant_matmul_v5_get_workspace(x1, x2, None, s2, out)
+    assert rc == 161002
