@@ -165,6 +165,13 @@ __global__ __launch_bounds__(256, 2) void wqmm_decode_kernel(WqParams p)
                     dequant_i4_f16(live ? (uint32_t)cur[i][s] : 0x88888888u, (h2){oh, oh}, (h2){sh, sh}, has_off, o4);
                     if (!live) { o4[0] = o4[1] = o4[2] = o4[3] = (h2){(_Float16)0.0f, (_Float16)0.0f}; }
                     aop = (v4i){(int)u32(o4[0]), (int)u32(o4[1]), (int)u32(o4[2]), (int)u32(o4[3])};
+                } else if constexpr (XDT == DT_F16 && WBITS == 4 && WFLT) {
+                    // e2m1 codes (no offset in the formats that carry them): packed-fp16 form
+                    const _Float16 sh = __builtin_bit_cast(_Float16, sb);
+                    h2 o4[4];
+                    dequant_fp4_f16(live ? (uint32_t)cur[i][s] : 0u, (h2){sh, sh}, o4);
+                    if (!live) { o4[0] = o4[1] = o4[2] = o4[3] = (h2){(_Float16)0.0f, (_Float16)0.0f}; }
+                    aop = (v4i){(int)u32(o4[0]), (int)u32(o4[1]), (int)u32(o4[2]), (int)u32(o4[3])};
                 } else {
                     float scf, off;
                     if constexpr (XDT == DT_F16) { scf = f16_to_f32(sb); off = f16_to_f32(ob); }
@@ -388,6 +395,7 @@ int launch_wqmm_mfma(const OpsnnWqmmArgs& a0, hipStream_t st)
     const bool mx = wflt && a.scale_dtype == DT_E8M0;
     if (a.scale_dtype != a.x_dtype && !mx) return OPSNN_NOT_TAKEN;
     if (mx && (a.offset || a.group <= 0 || a.scale_n == 1)) return OPSNN_NOT_TAKEN;
+    if (a.w_dtype == DT_E2M1 && a.offset) return OPSNN_NOT_TAKEN;   // the packed e2m1 dequantisation has no offset step
     const int wbits = (a.w_dtype == DT_I4 || a.w_dtype == DT_E2M1) ? 4 : 8;
     const int64_t kpl = 128 / wbits;
     if (a.K % kpl != 0 || a.K < kpl) return OPSNN_NOT_TAKEN;

@@ -50,6 +50,22 @@ __device__ __forceinline__ void dequant_i4_f16(uint32_t q, h2 off, h2 sc, bool h
     out[0] = t0 * sc; out[1] = t1 * sc; out[2] = t2 * sc; out[3] = t3 * sc;         // second rounding
 }
 
+// ---- fp16 dequantisation of 8 e2m1 codes of one dword -> 4 packed pairs in element order [0,4], [1,5], [2,6], [3,7] ----
+// A code's three magnitude bits, placed at bits 11..9 of a half, read as the half 2^-14 times the code's value -- for the
+// normal codes (exponent field 1..3 against a bias of 15 instead of 1) and for the two subnormal ones alike (0 and 2^-15 =
+// 2^-14 * 0.5): one exact multiplication by 2^14 gives the weight, and the multiplication by the scale then rounds once,
+// as the formula does (the weight is exact in fp16, T(w * s)).
+__device__ __forceinline__ void dequant_fp4_f16(uint32_t q, h2 sc, h2 (&out)[4])
+{
+    const h2 k14 = {(_Float16)16384.0f, (_Float16)16384.0f};
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const uint32_t t = q >> (4 * i);
+        const uint32_t bits = ((t & 0x00070007u) << 9) | ((t & 0x00080008u) << 12);
+        out[i] = (__builtin_bit_cast(h2, bits) * k14) * sc;
+    }
+}
+
 // ---- generic dequantisation of one weight to fp32 holding a value of x's dtype ----
 template <int XDT>
 __device__ __forceinline__ float round_x(float v)
