@@ -25,12 +25,6 @@
 #include "launch.h"
 #include "qgemm_core.hip.h"
 
-// -DXABL=<bits> removes parts of the loop for timing harnesses (results are then wrong): 1 the conversions, 2 the fold,
-// 4 the global -> LDS copies, 8 the LDS reads, 16 the barrier.  Never set in the library build.
-#ifndef XABL
-#define XABL 0
-#endif
-
 namespace opsnn {
 
 struct Fp8xParams {
@@ -160,7 +154,6 @@ __global__ __launch_bounds__(512, 1) void qmm_fp8_exact_kernel(Fp8xParams p, int
         }
     }
     auto issue_piece = [&](int kt, int stage, int idx) {
-        if (XABL & 4) return;
         char* sA = smem + stage * STAGE + wave * 1024;
         char* sB = sA + A_BYTES;
         const int8_t* Ak = uniform_ptr(A + (int64_t)kt * BK);
@@ -189,7 +182,6 @@ __global__ __launch_bounds__(512, 1) void qmm_fp8_exact_kernel(Fp8xParams p, int
     const int a_rowbase = (wm * TM + frow) * BK;
     const int b_rowbase = A_BYTES + (wn * TN + frow) * BK;
     auto load_frag = [&](const char* st, int rowbase) -> v8i {
-        if (XABL & 8) return v8i{lane + rowbase, 1, 2, 3, 4, 5, 6, 7} + (int)(size_t)st;
         const v4i lo = *(const v4i*)(st + rowbase + ch0);
         const v4i hi = *(const v4i*)(st + rowbase + ch1);
         return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
@@ -219,7 +211,6 @@ __global__ __launch_bounds__(512, 1) void qmm_fp8_exact_kernel(Fp8xParams p, int
         }
     };
     auto widen4 = [&](int d, v8h& h, int half) {   // four bytes -> elements 4*half .. 4*half+3
-        if (XABL & 1) { h[4 * half] = __builtin_bit_cast(v2h, d)[0]; return; }
         const v2h lo = cvt_lo<BE5>((uint32_t)d), hi = cvt_hi<BE5>((uint32_t)d);
         h[4 * half] = lo[0]; h[4 * half + 1] = lo[1]; h[4 * half + 2] = hi[0]; h[4 * half + 3] = hi[1];
     };
@@ -275,7 +266,7 @@ __global__ __launch_bounds__(512, 1) void qmm_fp8_exact_kernel(Fp8xParams p, int
 #if QG_DBG
                 const unsigned long long c1 = clock64();
 #endif
-                if (!(XABL & 16)) __builtin_amdgcn_s_barrier();   // tile kt+1 is complete in LDS; every wave is done reading tile kt
+                __builtin_amdgcn_s_barrier();   // tile kt+1 is complete in LDS; every wave is done reading tile kt
 #if QG_DBG
                 dbg_lgkm += c1 - c0; dbg_bar += clock64() - c1;
 #endif
@@ -283,7 +274,7 @@ __global__ __launch_bounds__(512, 1) void qmm_fp8_exact_kernel(Fp8xParams p, int
                 b_raw = load_frag(stn, b_rowbase);
 #pragma unroll
                 for (int j = 0; j < FM; j++)
-                    if (!(XABL & 8)) a_half[j] = *(const v4i*)(stn + a_rowbase + j * 16 * BK + ch0);
+                    a_half[j] = *(const v4i*)(stn + a_rowbase + j * 16 * BK + ch0);
                 read_scales(stn);
             }
             if (!RC && i == 0) {
@@ -301,50 +292,26 @@ __global__ __launch_bounds__(512, 1) void qmm_fp8_exact_kernel(Fp8xParams p, int
                     if constexpr (RC) {
                         acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fbc[i & 1][s], fa[j][s], acc[i][j], 0, 0, 0);
                     } else {
-                        if (XABL & 128) {   // partial sums in accumulation registers
-                            if (s == 0) asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, 0" : "=a"(part[i & 1][j]) : "v"(fbc[i & 1][s]), "v"(fa[j][s]));
-                            else asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(part[i & 1][j]) : "v"(fbc[i & 1][s]), "v"(fa[j][s]));
-                        } else
                         part[i & 1][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fbc[i & 1][s], fa[j][s], s == 0 ? v4f{0.0f, 0.0f, 0.0f, 0.0f} : part[i & 1][j], 0, 0, 0);
                         // fold element j of x1 fragment s of the previous x2 fragment (for i == 0: the previous tile's last, with its scales)
-                        if (XABL & 2) {
-                            if (kt == KT - 1 && i == FN - 1 && s == 3) acc[0][0][j] += part[1][j][0] + part[0][j][1];
-                        } else if (XABL & 32) {   // same count of fused multiply-adds, but none reads a matrix-instruction result
-                            acc[i][s][j] = __builtin_fmaf(s1raw[j], sc[s], acc[i][s][j]);
-                            if (kt == KT - 1 && i == FN - 1 && s == 3) acc[0][0][j] += part[1][j][0] + part[0][j][1];
-                        } else if (XABL & 64) {   // the whole fold of the previous fragment in one burst behind the first instruction of group 1
-                            if (s == 1 && j == 0) {
-#pragma unroll
-                                for (int jj = 0; jj < FM; jj++)
-#pragma unroll
-                                    for (int r = 0; r < 4; r++) {
-                                        if (i > 0) acc[i - 1][jj][r] = __builtin_fmaf(part[(i - 1) & 1][jj][r], sc[jj], acc[i - 1][jj][r]);
-                                        else acc[FN - 1][jj][r] = __builtin_fmaf(part[1][jj][r], scp[jj], acc[FN - 1][jj][r]);
-                                    }
-                            }
-                        } else if (i > 0) acc[i - 1][s][j] = __builtin_fmaf(part[(i - 1) & 1][s][j], sc[s], acc[i - 1][s][j]);
+                        if (i > 0) acc[i - 1][s][j] = __builtin_fmaf(part[(i - 1) & 1][s][j], sc[s], acc[i - 1][s][j]);
                         else acc[FN - 1][s][j] = __builtin_fmaf(part[1][s][j], scp[s], acc[FN - 1][s][j]);
                     }
                     if (s >= 2) {   // next x2 fragment: half a K step per instruction
                         const int idx = (s - 2) * 4 + j;
                         widen4(b_raw[idx], fbc[(i + 1) & 1][idx / 2], idx % 2);
                     }
-                    if (XABL & 1) {
-                        if (i == FN - 1 && s >= 2) fa[j][s - 2][0] = __builtin_bit_cast(v2h, a_half[j][2 * (s - 2)])[0];
-                        if (i == 0 && (s == 1 || s == 2)) fa[j][1 + s][0] = __builtin_bit_cast(v2h, a_half[j][2 * (s - 1)])[0];
-                    } else {
                     if (i == FN - 1 && s >= 2)                // next tile's x1 fragments, K step s - 2 (low halves)
                         fa[j][s - 2] = widen8<AE5>(a_half[j][2 * (s - 2)], a_half[j][2 * (s - 2) + 1]);
                     if (i == 0 && (s == 1 || s == 2))         // this tile's x1 fragments, K steps 2 and 3 (high halves)
                         fa[j][1 + s] = widen8<AE5>(a_half[j][2 * (s - 1)], a_half[j][2 * (s - 1) + 1]);
-                    }
                     __builtin_amdgcn_sched_barrier(0);
                 }
                 if (i == FN - 1) {
                     if (s == 3) {   // the low halves are converted: fetch the high halves into the same registers
 #pragma unroll
                         for (int j = 0; j < FM; j++)
-                            if (!(XABL & 8)) a_half[j] = *(const v4i*)(stn + a_rowbase + j * 16 * BK + ch1);
+                            a_half[j] = *(const v4i*)(stn + a_rowbase + j * 16 * BK + ch1);
                     }
 #pragma unroll
                     for (int c = s * CPS; c < (s + 1) * CPS && c < CPT; c++) issue_piece(ktc, cur, c);   // tile kt+3 into the stage of tile kt
