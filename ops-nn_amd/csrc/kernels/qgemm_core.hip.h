@@ -237,7 +237,7 @@ __global__ __launch_bounds__(WGM* WGN * 64, MINWG) void qgemm_kernel(QgemmParams
 
     typedef int frag_t __attribute__((ext_vector_type(FREG)));
     frag_t fa[2][FM], fb[2][FN];
-    uint32_t sca[FM][SCW], scb[FN][SCW];  // MX: this lane's scale bytes of the current tile, shifted down by its K half
+    uint32_t sca[FM], scb[FN];  // MX: this lane's scale bytes of the current tile, moved into place (see place_scales)
     (void)swz; (void)swz0; (void)swz1; (void)sca; (void)scb;
 
     auto load_frags = [&](int kt, int s, int buf) {
@@ -264,37 +264,51 @@ __global__ __launch_bounds__(WGM* WGN * 64, MINWG) void qgemm_kernel(QgemmParams
         }
     };
     // MX: byte b of a row's scale bytes of a tile covers the tile's K block b (32 elements).  MFMA step s of a lane
-    // in K half h multiplies block 2s + h, i.e. byte 2(s % 2) of scale dword s / 2 once that dword is shifted right
-    // by 8h.  read_scales_raw fetches dword w of tile kt's scales for this lane's rows; shift_scales moves them into
-    // place.
-    auto read_scales_raw = [&](int kt, int w, uint32_t (&ra)[FM], uint32_t (&rb)[FN]) {
+    // in K half h multiplies block 2s + h.
+    // Four bytes per row and tile (SCW == 1): the dword is shifted right by 8h and the instruction's byte select
+    // picks byte 2s.
+    // Eight bytes per row and tile (SC16): one 8-byte LDS read brings both dwords (d0, d1) of the tile -- 4-byte reads
+    // at the ring's 16-byte row pitch take three times as long as conflict-free ones (measured: 3.75 against 1.31
+    // clocks per wave read), so fewer and wider reads -- and one byte permute packs this lane's four scales into one
+    // register, [d0.b(h), d1.b(h), d0.b(h+2), d1.b(h+2)]: step s selects byte 2 (s % 2) + s / 2.
+    typedef uint32_t raw_t __attribute__((ext_vector_type(SC16 ? 2 : 1)));
+    const uint32_t sc_sel = fkc ? 0x07030501u : 0x06020400u;
+    (void)sc_sel;
+    auto read_scales_raw = [&](int kt, raw_t (&ra)[FM], raw_t (&rb)[FN]) {
         if constexpr (MX) {
             const char* sS;
             int pitch, off;
             if constexpr (SC16) {
                 sS = smem + SC_RING + ((kt >> 1) & 1) * ((BM + BN) * 16);
-                pitch = 16; off = (kt & 1) * 8 + 4 * w;
+                pitch = 16; off = (kt & 1) * 8;
             } else {
                 sS = smem + (kt % STAGES) * STAGE + A_BYTES + B_BYTES;
-                pitch = SCB; off = 4 * w;
+                pitch = SCB; off = 0;
             }
 #pragma unroll
-            for (int j = 0; j < FM; j++) ra[j] = *(const uint32_t*)(sS + (wm * TM + j * 32 + frow) * pitch + off);
+            for (int j = 0; j < FM; j++) ra[j] = *(const raw_t*)(sS + (wm * TM + j * 32 + frow) * pitch + off);
 #pragma unroll
-            for (int i = 0; i < FN; i++) rb[i] = *(const uint32_t*)(sS + (BM + wn * TN + i * 32 + frow) * pitch + off);
+            for (int i = 0; i < FN; i++) rb[i] = *(const raw_t*)(sS + (BM + wn * TN + i * 32 + frow) * pitch + off);
         }
     };
-    auto shift_scales = [&](int w, const uint32_t (&ra)[FM], const uint32_t (&rb)[FN]) {
+    auto place_scales = [&](const raw_t (&ra)[FM], const raw_t (&rb)[FN]) {
+        if constexpr (SC16) {
 #pragma unroll
-        for (int j = 0; j < FM; j++) sca[j][w] = ra[j] >> (8 * fkc);
+            for (int j = 0; j < FM; j++) sca[j] = __builtin_amdgcn_perm(ra[j][1], ra[j][0], sc_sel);
 #pragma unroll
-        for (int i = 0; i < FN; i++) scb[i][w] = rb[i] >> (8 * fkc);
+            for (int i = 0; i < FN; i++) scb[i] = __builtin_amdgcn_perm(rb[i][1], rb[i][0], sc_sel);
+        } else {
+#pragma unroll
+            for (int j = 0; j < FM; j++) sca[j] = ra[j][0] >> (8 * fkc);
+#pragma unroll
+            for (int i = 0; i < FN; i++) scb[i] = rb[i][0] >> (8 * fkc);
+        }
     };
-    auto load_scales = [&](int kt) {   // dword 0 of tile kt, ready to use
+    auto load_scales = [&](int kt) {   // the scales of tile kt, ready to use
         if constexpr (MX) {
-            uint32_t ra[FM], rb[FN];
-            read_scales_raw(kt, 0, ra, rb);
-            shift_scales(0, ra, rb);
+            raw_t ra[FM], rb[FN];
+            read_scales_raw(kt, ra, rb);
+            place_scales(ra, rb);
         }
     };
     auto mma = [&](int buf, auto sidx) {
@@ -310,9 +324,10 @@ __global__ __launch_bounds__(WGM* WGN * 64, MINWG) void qgemm_kernel(QgemmParams
                     const v4i z = {0, 0, 0, 0};  // fp4 operands occupy the first four of the eight operand dwords
                     const v8i bb = __builtin_shufflevector(fb[buf][i], z, 0, 1, 2, 3, 4, 5, 6, 7);
                     const v8i aa = __builtin_shufflevector(fa[buf][j], z, 0, 1, 2, 3, 4, 5, 6, 7);
-                    acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(bb, aa, acc[i][j], 4, 4, 2 * (S % 2), (int)scb[i][S / 2], 2 * (S % 2), (int)sca[j][S / 2]);
+                    constexpr int SEL = SC16 ? 2 * (S % 2) + S / 2 : 2 * S;
+                    acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(bb, aa, acc[i][j], 4, 4, SEL, (int)scb[i], SEL, (int)sca[j]);
                 } else {
-                    acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb[buf][i], fa[buf][j], acc[i][j], 0, 0, 2 * S, (int)scb[i][0], 2 * S, (int)sca[j][0]);
+                    acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb[buf][i], fa[buf][j], acc[i][j], 0, 0, 2 * S, (int)scb[i], 2 * S, (int)sca[j]);
                 }
             }
     };
@@ -352,26 +367,15 @@ __global__ __launch_bounds__(WGM* WGN * 64, MINWG) void qgemm_kernel(QgemmParams
 
     auto k_tile = [&](int kt, auto issue, auto next, auto even) {
         constexpr bool ISSUE = decltype(issue)::value, NEXT = decltype(next)::value;
-        uint32_t ra[FM], rb[FN];   // raw scale dwords on their way in
+        raw_t ra[FM], rb[FN];   // raw scale bytes of the next tile on their way in
         (void)ra; (void)rb;
         if constexpr (KS >= 4) {
-            // SC16: scale dword 1 of this tile (K steps 2, 3) is fetched now, dword 0 of the next tile after the
-            // barrier below, each into the registers its predecessor has just stopped using
-            if constexpr (SC16) {
-                read_scales_raw(kt, 1, ra, rb);
-                __builtin_amdgcn_sched_barrier(0);
-            }
             load_frags(kt, 1, 1);
             mma(0, std::integral_constant<int, 0>{});
             interleave(false);
             load_frags(kt, 2, 0);
             mma(1, std::integral_constant<int, 1>{});
             interleave(false);
-            if constexpr (SC16) {
-                __builtin_amdgcn_sched_barrier(0);
-                shift_scales(1, ra, rb);
-                __builtin_amdgcn_sched_barrier(0);
-            }
             load_frags(kt, 3, 1);
             mma(0, std::integral_constant<int, 2>{});
             interleave(false);
@@ -398,9 +402,9 @@ __global__ __launch_bounds__(WGM* WGN * 64, MINWG) void qgemm_kernel(QgemmParams
         dbg_vm += c1 - c0; dbg_bar += c2 - c1; dbg_n++;
 #endif
         if constexpr (NEXT && MX) {
-            // the next tile's first scale dword is requested ahead of its operands (LDS returns in order) and moved
+            // the next tile's scale bytes are requested ahead of its operands (LDS returns in order) and moved
             // into place only after this tile's last MFMAs, which still use the current ones, have been issued
-            read_scales_raw(kt + 1, 0, ra, rb);
+            read_scales_raw(kt + 1, ra, rb);
             __builtin_amdgcn_sched_barrier(0);
         }
         if constexpr (ISSUE) issue_tile(kt + STAGES, even);
@@ -409,7 +413,7 @@ __global__ __launch_bounds__(WGM* WGN * 64, MINWG) void qgemm_kernel(QgemmParams
         if constexpr (NEXT) interleave(ISSUE);
         if constexpr (NEXT && MX) {
             __builtin_amdgcn_sched_barrier(0);
-            shift_scales(0, ra, rb);
+            place_scales(ra, rb);
         }
     };
     using T = std::true_type;

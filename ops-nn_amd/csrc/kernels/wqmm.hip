@@ -323,6 +323,14 @@ static bool stream_eligible(WqParams& p, WqStreamOpts& o)
     o.resx = !no_resx && p.M <= 16 && nch % 4 == 0 && (p.M + 1) * (p.K * 2 + 16) <= 65536;
     o.resx_vscale = o.resx && p.group == KC && p.s_rs == 1 && p.s_cs % 8 == 0 && (nch / 4) % 8 == 0 &&
                     (uintptr_t)p.scale % 16 == 0 && (!p.offset || (uintptr_t)p.offset % 16 == 0);
+    // 4 to 16 rows (fewer stay on the kernel above): x in registers, K in 8 or 16 contiguous ranges per workgroup
+    static const int xreg_min = [] { const char* e = getenv("OPSNN_WQ_XREG_MIN"); return e ? atoi(e) : 4; }();
+    static const int xreg_nw = [] { const char* e = getenv("OPSNN_WQ_XREG_NW"); return e ? atoi(e) : 0; }();
+    int xnw = 0, xnch = 0;
+    o.xreg_nw = xreg_nw;
+    o.xreg = p.M >= xreg_min && p.M <= 16 && xreg_shape(WBITS, p.K, xreg_nw, xnw, xnch);
+    o.xreg_vscale = o.xreg && p.group == KC && p.s_rs == 1 && p.s_cs % 8 == 0 &&
+                    (uintptr_t)p.scale % 16 == 0 && (!p.offset || (uintptr_t)p.offset % 16 == 0);
     // more than 48 rows: two weight blocks per wave share every x fragment, up to 128 rows per pass over the weights
     // (needs whole groups of chunks in flight and whole wave tiles of columns)
     static const bool no_rows = [] { const char* e = getenv("OPSNN_WQ_NO_ROWS"); return e && e[0] == '1'; }();

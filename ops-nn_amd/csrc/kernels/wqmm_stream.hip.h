@@ -713,6 +713,204 @@ __global__ __launch_bounds__(256, 2) void wqmm_resx_kernel(WqParams p)
     }
 }
 
+// ---- up to 16 rows of x, moderate K: x lives in REGISTERS ----
+// A workgroup is NW = 8 or 16 waves; wave w owns the K range [w * K/NW, (w+1) * K/NW) of every block of 16 weight rows
+// the workgroup walks (blockIdx.x, + gridDim.x, ...).  The x operands of that range -- NCH chunks x STEPS fragments of
+// 16 bytes per lane -- are loaded once, before the weight stream starts, and stay in registers for the whole kernel:
+// the loop has no LDS read, no x staging and no slab barrier, only the dequantisation and the MFMA.  The NW partial
+// sums of a row block meet in LDS in a fixed order (one barrier per row block, buffer alternating); the wave whose turn
+// it is (row block count % NW) adds them and stores.  As in the kernel above the weight stream runs across row blocks:
+// the slot a chunk was consumed from is refilled with the chunk PF further on, in this row block or the next.
+// Sixteen waves (four per SIMD, 128 registers each, 16 fragments of x) hide the dequantisation's vector work best.
+template <int XDT, int WBITS, int NW, int NCH, bool HAS_OFF, bool VSCALE>
+__global__ __launch_bounds__(NW * 64) void wqmm_xreg_kernel(WqParams p)
+{
+    constexpr int KPL = 128 / WBITS, KC = 4 * KPL, STEPS = KC / 32;
+    constexpr int PF = NW == 16 ? 4 : (NCH < 8 ? NCH : 8);   // weight pieces in flight per lane
+    constexpr int NX = NCH * STEPS;                          // x fragments per lane
+    static_assert(NW == 8 || NW == 16, "one or two workgroup halves per SIMD pair");
+    static_assert(NX <= (NW == 16 ? 16 : 32), "x fragments must fit the register file beside the weight stream");
+    static_assert(NCH % 4 == 0 && NCH >= PF, "whole groups of four chunks");
+    constexpr int NU = NX / 4, HU = NU / 2;   // 256-byte units of x per wave, and per staging half
+    static_assert(NU % 2 == 0 && HU * 4096 >= 2048, "two staging halves that also hold the partial sums");
+    extern __shared__ __attribute__((aligned(16))) char dyn[];
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int nrow = lane & 15, g = lane >> 4;
+    const int rows = (int)p.m_rows;
+    const int cbase = wave * NCH;           // first chunk of this wave's K range
+    const int nblocks = (int)((p.N + 15) / 16);
+
+    auto row_of = [&](int rb) { const int64_t n = (int64_t)rb * 16 + nrow; return n < p.N ? n : p.N - 1; };
+    auto wptr_of = [&](int rb) { return p.w + row_of(rb) * p.ldw + g * 16 + (int64_t)cbase * 64; };
+    int rb = blockIdx.x;
+    const uint8_t* wptr = wptr_of(rb);
+    const uint16_t* srow = p.scale + row_of(rb) * p.s_cs;
+    const uint16_t* orow = HAS_OFF ? p.offset + row_of(rb) * p.s_cs : nullptr;
+
+    // VSCALE (one scale per chunk, a row's scales contiguous): the NCH scales of this wave's K range as NCH/2 dwords,
+    // fetched with 8- or 16-byte loads one row block ahead
+    constexpr int SW = NCH / 2;
+    uint32_t sv[SW], ov[SW], svn[SW], ovn[SW];
+    auto load_scales = [&](const uint16_t* sr, const uint16_t* orw, uint32_t (&sd)[SW], uint32_t (&od)[SW]) {
+        if constexpr (NCH % 8 == 0) {
+#pragma unroll
+            for (int h = 0; h < NCH / 8; h++) {
+                const v4i t = *(const v4i*)(sr + cbase + 8 * h);
+#pragma unroll
+                for (int e = 0; e < 4; e++) sd[4 * h + e] = (uint32_t)t[e];
+                if constexpr (HAS_OFF) {
+                    const v4i u = *(const v4i*)(orw + cbase + 8 * h);
+#pragma unroll
+                    for (int e = 0; e < 4; e++) od[4 * h + e] = (uint32_t)u[e];
+                }
+            }
+        } else {
+            const v2i t = *(const v2i*)(sr + cbase);
+            sd[0] = (uint32_t)t[0]; sd[1] = (uint32_t)t[1];
+            if constexpr (HAS_OFF) {
+                const v2i u = *(const v2i*)(orw + cbase);
+                od[0] = (uint32_t)u[0]; od[1] = (uint32_t)u[1];
+            }
+        }
+    };
+#pragma unroll
+    for (int h = 0; h < SW; h++) sv[h] = ov[h] = svn[h] = ovn[h] = 0;
+    if constexpr (VSCALE) load_scales(srow, orow, svn, ovn);
+    v4i wq[PF];
+    uint16_t sq[PF], oq[PF];
+    auto fetch = [&](int j, const uint8_t* wp, const uint16_t* sr, const uint16_t* orw, int cw) {
+        wq[j] = *(const v4i*)(wp + (int64_t)cw * 64);
+        if constexpr (!VSCALE) {
+            const int64_t so = (int64_t)((cbase + cw) >> p.cpg_shift) * p.s_rs;
+            sq[j] = sr[so];
+            if constexpr (HAS_OFF) oq[j] = orw[so];
+        }
+    };
+#pragma unroll
+    for (int j = 0; j < PF; j++) fetch(j, wptr, srow, orow, j);
+    const DqConst dqc = make_dq_const();
+
+    // x: the fragment (c, s) of lane (nrow, g) is row nrow, k = cbase*KC + c*KC + g*KPL + 8s .. +8.  Read straight from
+    // global memory that is 64 lanes x 16 bytes out of 32 different cache lines per instruction; instead the wave's K
+    // range travels through LDS once, in units of 16 rows x 256 bytes: four 16-byte asynchronous copies per unit, each
+    // fetching four rows x 256 contiguous bytes, land the 16-byte segment `seg` of row m at position seg ^ m of the
+    // row (conflict free for the 16-byte reads below), half of the range at a time (the whole of x would not fit).
+    // Rows that x does not have repeat its last row: they only feed output rows that are never stored.
+    v4i xr[NX];
+    {
+        char* stage = dyn + wave * (HU * 4096);
+        const int cm = lane >> 4, cp = lane & 15;
+        const uint16_t* xw = p.x + p.m_base * p.K + (int64_t)wave * (NU * 128);
+#pragma unroll
+        for (int r = 0; r < 2; r++) {
+#pragma unroll
+            for (int ul = 0; ul < HU; ul++) {
+#pragma unroll
+                for (int q = 0; q < 4; q++) {
+                    if (4 * q < rows) {
+                        const int m = 4 * q + cm;
+                        const int mm = m < rows ? m : rows - 1;
+                        async_copy16(xw + (int64_t)mm * p.K + (r * HU + ul) * 128 + ((cp ^ m) << 3), stage + ul * 4096 + q * 1024);
+                    }
+                }
+            }
+            wait_vmcnt<0>();
+            asm volatile("" ::: "memory");
+#pragma unroll
+            for (int i = 0; i < NX; i++) {
+                const int u = ((i / STEPS) * KC) / 128;   // the unit does not depend on the lane
+                if (u / HU != r) continue;
+                const int seg = (((i / STEPS) * KC) % 128 + g * KPL + 8 * (i % STEPS)) >> 3;
+                v4i v = *(const v4i*)(stage + (u % HU) * 4096 + nrow * 256 + ((seg ^ nrow) << 4));
+                if constexpr (WBITS == 4) {
+                    // halves [0..7] -> [0,4,1,5,2,6,3,7]: the order in which the nibble splicing yields pairs
+                    const uint32_t a0 = (uint32_t)v[0], a1 = (uint32_t)v[1], a2 = (uint32_t)v[2], a3 = (uint32_t)v[3];
+                    v = (v4i){(int)__builtin_amdgcn_perm(a2, a0, 0x05040100u), (int)__builtin_amdgcn_perm(a2, a0, 0x07060302u),
+                              (int)__builtin_amdgcn_perm(a3, a1, 0x05040100u), (int)__builtin_amdgcn_perm(a3, a1, 0x07060302u)};
+                }
+                xr[i] = v;
+            }
+            wait_lgkmcnt0();   // this wave's reads have retired before the next copies overwrite the units
+            asm volatile("" ::: "memory");
+        }
+    }
+    __syncthreads();   // the staging area now becomes the partial-sum buffers
+    float* const red = (float*)dyn;   // [2][NW][256]
+
+    for (int it = 0; rb < nblocks; it++) {
+        const int rb_next = rb + (int)gridDim.x;
+        const bool has_next = rb_next < nblocks;
+        const uint8_t* wptr_n = has_next ? wptr_of(rb_next) : wptr;   // past the end: harmless reloads of this block
+        const uint16_t* srow_n = has_next ? p.scale + row_of(rb_next) * p.s_cs : srow;
+        const uint16_t* orow_n = HAS_OFF ? (has_next ? p.offset + row_of(rb_next) * p.s_cs : orow) : nullptr;
+        if constexpr (VSCALE) {
+            // the next row block's scales are requested before the refills below fetch its weights (loads return in
+            // issue order: waiting for a scale issued after them would drain the weight stream)
+#pragma unroll
+            for (int h = 0; h < SW; h++) { sv[h] = svn[h]; ov[h] = ovn[h]; }
+            load_scales(srow_n, orow_n, svn, ovn);
+        }
+        v4f acc = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+        for (int c = 0; c < NCH; c++) {
+            const int j = c % PF;
+            uint16_t sb, ob = 0;
+            if constexpr (VSCALE) {
+                sb = (uint16_t)(sv[c / 2] >> (16 * (c % 2)));
+                if constexpr (HAS_OFF) ob = (uint16_t)(ov[c / 2] >> (16 * (c % 2)));
+            } else {
+                sb = sq[j];
+                if constexpr (HAS_OFF) ob = oq[j];
+            }
+#pragma unroll
+            for (int s = 0; s < STEPS; s++) {
+                const v4i aop = dequant8<XDT, WBITS, HAS_OFF>(wq[j], s, sb, ob, dqc);
+                if constexpr (XDT == DT_F16) {
+                    acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(v8h, aop), __builtin_bit_cast(v8h, xr[c * STEPS + s]), acc, 0, 0, 0);
+                } else {
+                    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf, aop), __builtin_bit_cast(v8bf, xr[c * STEPS + s]), acc, 0, 0, 0);
+                }
+            }
+            if (c + PF < NCH) fetch(j, wptr, srow, orow, c + PF);
+            else fetch(j, wptr_n, srow_n, orow_n, c + PF - NCH);
+        }
+
+        // fixed-order reduction of the NW K ranges
+        float* rd = red + (it & 1) * (NW * 256);
+        *(v4f*)(rd + wave * 256 + lane * 4) = acc;
+        __syncthreads();
+        if (wave == (it & (NW - 1))) {
+            v4f sum = *(const v4f*)(rd + lane * 4);
+#pragma unroll 4
+            for (int j = 1; j < NW; j++) sum = sum + *(const v4f*)(rd + j * 256 + lane * 4);
+            if (nrow < rows) {
+                const int64_t n0 = (int64_t)rb * 16;
+                const int64_t m = p.m_base + nrow;
+                float v[4];
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    const int64_t nn = n0 + 4 * g + i;
+                    v[i] = sum[i];
+                    if (p.bias && nn < p.N) v[i] = v[i] + load_scalar_as_f32(p.bias, p.bias_dt, nn);
+                    if constexpr (XDT == DT_BF16) v[i] = bf16_to_f32(bf16_bits(v[i]));
+                }
+                const int64_t nn0 = n0 + 4 * g;
+                if (nn0 + 3 < p.N && (p.N % 4) == 0) {
+                    const v4us o = {bits_x<XDT>(v[0]), bits_x<XDT>(v[1]), bits_x<XDT>(v[2]), bits_x<XDT>(v[3])};
+                    *(v4us*)(p.y + m * p.N + nn0) = o;
+                } else {
+#pragma unroll
+                    for (int i = 0; i < 4; i++)
+                        if (nn0 + i < p.N) p.y[m * p.N + nn0 + i] = bits_x<XDT>(v[i]);
+                }
+            }
+        }
+        rb = rb_next; wptr = wptr_n; srow = srow_n; orow = orow_n;
+    }
+}
+
 // Workgroups of the persistent kernel: two per CU (row blocks are dealt round-robin, so the workgroups i and
 // i + CUs, which share a CU, together get an even share), or one per row block when there are fewer than that.
 static inline unsigned resx_grid(int64_t nblocks)
@@ -739,6 +937,57 @@ static int launch_resx_one(const WqParams& p, hipStream_t st)
     }
     hipLaunchKernelGGL(k, dim3(resx_grid((p.N + 15) / 16)), dim3(256), lds, st, p);
     return (int)hipGetLastError();
+}
+
+// One workgroup per CU (its waves fill the register file), or one per row block when there are fewer.
+template <int XDT, int WBITS, int NW, int NCH, bool HAS_OFF, bool VSCALE>
+static int launch_xreg_one(const WqParams& p, hipStream_t st)
+{
+    const int64_t nblocks = (p.N + 15) / 16;
+    const int64_t g = (int64_t)resx_grid(1ll << 40) / 2;
+    constexpr int STEPS = (4 * (128 / WBITS)) / 32;
+    constexpr int lds = NW * (NCH * STEPS / 8) * 4096;   // half of the K range of every wave: 16 rows x 256 bytes per unit
+    auto k = wqmm_xreg_kernel<XDT, WBITS, NW, NCH, HAS_OFF, VSCALE>;
+    static bool attr_set = false;
+    if (!attr_set) {
+        hipError_t e = hipFuncSetAttribute((const void*)k, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+        if (e != hipSuccess) return (int)e;
+        attr_set = true;
+    }
+    hipLaunchKernelGGL(k, dim3((unsigned)(nblocks < g ? nblocks : g)), dim3(NW * 64), lds, st, p);
+    return (int)hipGetLastError();
+}
+
+template <int XDT, int WBITS, int NW, int NCH>
+static int launch_xreg_nch(const WqParams& p, bool has_off, bool vscale, hipStream_t st)
+{
+    if (vscale) return has_off ? launch_xreg_one<XDT, WBITS, NW, NCH, true, true>(p, st) : launch_xreg_one<XDT, WBITS, NW, NCH, false, true>(p, st);
+    return has_off ? launch_xreg_one<XDT, WBITS, NW, NCH, true, false>(p, st) : launch_xreg_one<XDT, WBITS, NW, NCH, false, false>(p, st);
+}
+
+// K = waves x chunks per wave x chunk.  Sixteen waves with 4 chunks each (8-bit weights: or 8), else eight waves with 4 or 8.
+static inline bool xreg_shape(int wbits, int64_t K, int force_nw, int& nw, int& nch)
+{
+    const int64_t kc = 4 * (128 / wbits);
+    if (K % (32 * kc) != 0) return false;
+    const int64_t c16 = K / (16 * kc), c8 = K / (8 * kc);
+    if (force_nw != 8 && K % (64 * kc) == 0 && (c16 == 4 || (wbits == 8 && c16 == 8))) { nw = 16; nch = (int)c16; return true; }
+    if (c8 == 4 || c8 == 8) { nw = 8; nch = (int)c8; return true; }
+    return false;
+}
+
+template <int XDT, int WBITS>
+static int launch_xreg(const WqParams& p, bool has_off, bool vscale, int force_nw, hipStream_t st)
+{
+    int nw = 0, nch = 0;
+    if (!xreg_shape(WBITS, p.K, force_nw, nw, nch)) return OPSNN_NOT_TAKEN;
+    if (nw == 16 && nch == 4) return launch_xreg_nch<XDT, WBITS, 16, 4>(p, has_off, vscale, st);
+    if constexpr (WBITS == 8) {
+        if (nw == 16 && nch == 8) return launch_xreg_nch<XDT, WBITS, 16, 8>(p, has_off, vscale, st);
+    }
+    if (nw == 8 && nch == 4) return launch_xreg_nch<XDT, WBITS, 8, 4>(p, has_off, vscale, st);
+    if (nw == 8 && nch == 8) return launch_xreg_nch<XDT, WBITS, 8, 8>(p, has_off, vscale, st);
+    return OPSNN_NOT_TAKEN;
 }
 
 template <int XDT, int WBITS, int MB, int NW, int WK, bool HAS_OFF, bool VSCALE>
@@ -784,6 +1033,8 @@ struct WqStreamOpts {
     bool has_off, vscale, ksplit;
     bool rows;                // many-rows kernel eligible (row slabs of up to 128)
     bool resx, resx_vscale;   // whole-x-in-LDS kernel eligible, and with vector scale loads
+    bool xreg, xreg_vscale;   // x-in-registers kernel eligible (up to 16 rows), and with vector scale loads
+    int xreg_nw;              // 8: keep it to eight waves (tuning)
 };
 
 // One row slab (p.m_rows <= 128 with o.rows, else <= 64) of one dtype pair; defined once per pair in its own translation unit.
@@ -805,6 +1056,10 @@ int launch_wq_stream(const WqParams& p, const WqStreamOpts& o, hipStream_t st);
     template <>                                                                                                     \
     int launch_wq_stream<XDT, WBITS>(const WqParams& p, const WqStreamOpts& o, hipStream_t st)                      \
     {                                                                                                               \
+        if (o.xreg && p.m_rows <= 16) {                                                                             \
+            const int rc = launch_xreg<XDT, WBITS>(p, o.has_off, o.xreg_vscale, o.xreg_nw, st);                     \
+            if (rc != OPSNN_NOT_TAKEN) return rc;                                                                   \
+        }                                                                                                           \
         if (o.resx) {                                                                                               \
             if (o.resx_vscale) return o.has_off ? launch_resx_one<XDT, WBITS, true, true>(p, st)                    \
                                                 : launch_resx_one<XDT, WBITS, false, true>(p, st);                  \

@@ -291,7 +291,8 @@ class ConfigWQ(Workload):
         m, K, N = self.m, self.K, self.N
         self.M = M
         self.inp = dict(self.inp_full, x=np.ascontiguousarray(self.inp_full["x"][:M]))
-        self.kernel = "wqmm_resx_kernel" if (self.cfg == 3 and M <= 3) else ("wqmm_tile_kernel" if M > 128 else "wqmm_rows_kernel" if M > 48 else "wqmm_stream_kernel")
+        self.kernel = ("wqmm_resx_kernel" if (self.cfg == 3 and M <= 3) else "wqmm_xreg_kernel" if M <= 16 else
+                       "wqmm_tile_kernel" if M > 128 else "wqmm_rows_kernel" if M > 48 else "wqmm_stream_kernel")
         self.t_x = m.Tensor((M, K), self.x_dt, self.d["x"])
         self.t_y = m.Tensor((M, N), self.x_dt, self.d_y)
         rc, ws, ex = m.weight_quant_batch_matmul_get_workspace(self.t_x, self.t_w[0], self.t_sc, self.t_y, offset=self.t_off,

@@ -275,6 +275,34 @@ def test_weight_only_tile_kernel(gpu, M, K, N, x_dt, w_dt, group, tW, off, bias)
 
 
 
+@pytest.mark.parametrize("M,K,N,x_dt,w_dt,group,tW,off,bias", [
+    # 4 .. 16 rows with K a multiple of 8 waves x 4, 8 or 16 chunks (int4: 4096, 8192; int8: 2048, 4096, 8192): groups of one
+    # chunk (vector scale loads), of several chunks and per channel; with and without offset; ragged columns; fewer row
+    # blocks than workgroups and more (a workgroup walks several); N-contiguous weight; bias
+    (16, 8192, 256, "f16", "i4", 128, True, True, None),
+    (16, 8192, 4400, "f16", "i4", 128, True, False, "f16"),    # 275 row blocks: some workgroups take two
+    (5, 8192, 100, "bf16", "i4", 128, True, True, None),
+    (4, 4096, 1000, "f16", "i4", 256, True, True, None),
+    (9, 4096, 64, "bf16", "i4", 0, True, False, "bf16"),
+    (16, 8192, 128, "f16", "i4", 1024, True, True, None),
+    (16, 4096, 4096, "bf16", "i8", 0, True, False, None),
+    (12, 2048, 72, "f16", "i8", 64, True, True, None),
+    (16, 8192, 200, "f16", "i8", 64, True, True, "f16"),
+    (7, 4096, 320, "bf16", "i8", 128, True, True, None),
+    (16, 8192, 96, "bf16", "i4", 128, False, True, None),
+])
+def test_weight_only_x_in_registers_kernel(gpu, M, K, N, x_dt, w_dt, group, tW, off, bias):
+    """4 .. 16 rows of x with K in eight equal ranges of whole chunks: the kernel that keeps x in registers."""
+    m = gpu
+    dt = {"bf16": m.ACL_BF16, "f16": m.ACL_FLOAT16, "i8": m.ACL_INT8, "i4": m.ACL_INT4, None: None}
+    print(f"case wq x-in-registers M={M} K={K} N={N} x={x_dt} w={w_dt} g={group} tW={tW} off={off} bias={bias}", flush=True)
+    inp = cases.make_wq_inputs(m, M, K, N, M * 3 + N, dt[x_dt], dt[w_dt], group, tW, off, dt[bias])
+    want = cases.oracle_wq(m, inp, M, K, N)
+    plain(False)
+    got = cases.run_wq_aclnn(m, inp, M, K, N)
+    check_close(got, want, dt[x_dt], "weight-only, x in registers")
+
+
 def test_weight_only_v3_and_per_tensor(gpu):
     m = gpu
     inp = cases.make_wq_inputs(m, 8, 256, 128, 2, m.ACL_FLOAT16, m.ACL_INT8, 0, False, True, None, per_tensor=True)
