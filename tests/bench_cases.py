@@ -16,20 +16,20 @@ import oracle_api as orc
 # bench.py does not measure it; it copies the figure and names the file.  A figure below the algorithmic bytes would not
 # be evidence and is reported as null.  Keyed by (config, M of the weight-only configs, variant).
 PROFILED_TRAFFIC = {
-    (1, None, "warm"): (18.3e6, "profiles/wqmm_decode_w8a16_m16_k4096_n4096.txt"),
-    (1, None, "cold"): (18.3e6, "profiles/wqmm_decode_w8a16_m16_k4096_n4096_cold.txt"),
+    (1, None, "warm"): (20.9e6, "profiles/wqmm_decode_w8a16_m16_k4096_n4096.txt"),
+    (1, None, "cold"): (20.8e6, "profiles/wqmm_decode_w8a16_m16_k4096_n4096_cold.txt"),
     (2, None, None): (162.2e6, "profiles/qgemm_int8_w8a8_m2048_k4096_n11008.txt"),
     (3, 1, "warm"): (144.0e6, "profiles/wqmm_decode_w4a16_m1_k8192_n28672.txt"),
     (3, 1, "cold"): (140.9e6, "profiles/wqmm_decode_w4a16_m1_k8192_n28672_cold.txt"),
-    (3, 16, "warm"): (137.6e6, "profiles/wqmm_decode_w4a16_m16_k8192_n28672.txt"),
-    (3, 16, "cold"): (137.5e6, "profiles/wqmm_decode_w4a16_m16_k8192_n28672_cold.txt"),
+    (3, 16, "warm"): (131.4e6, "profiles/wqmm_decode_w4a16_m16_k8192_n28672.txt"),
+    (3, 16, "cold"): (132.1e6, "profiles/wqmm_decode_w4a16_m16_k8192_n28672_cold.txt"),
     (3, 64, "warm"): (151.3e6, "profiles/wqmm_decode_w4a16_m64_k8192_n28672.txt"),
     (3, 64, "cold"): (151.2e6, "profiles/wqmm_decode_w4a16_m64_k8192_n28672_cold.txt"),
     (3, 256, "warm"): (257.7e6, "profiles/wqmm_decode_w4a16_m256_k8192_n28672.txt"),
     (3, 256, "cold"): (255.9e6, "profiles/wqmm_decode_w4a16_m256_k8192_n28672_cold.txt"),
     (4, None, "exact"): (1220.2e6, "profiles/qmm_fp8_exact_m4096_k7168_n18432.txt"),
     (4, None, "fast"): (1502.4e6, "profiles/qmm_fp8_block_m4096_k7168_n18432.txt"),
-    (5, None, None): (3084.6e6, "profiles/qgemm_mxfp4_b8_m4096_k8192_n8192.txt"),
+    (5, None, None): (3083.5e6, "profiles/qgemm_mxfp4_b8_m4096_k8192_n8192.txt"),
 }
 
 
