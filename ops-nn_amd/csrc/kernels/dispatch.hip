@@ -18,6 +18,8 @@ int launch_fp8_rowcol_mfma(const OpsnnQmmArgs& a, hipStream_t st, bool merged_sc
 int launch_rowcol_exact(const OpsnnQmmArgs& a, hipStream_t st, int ep_mode);   // qmm_fp8_exact.hip
 int launch_tcg_mfma(const OpsnnQmmArgs& a, hipStream_t st);
 uint64_t tcg_workspace_bytes(const OpsnnQmmArgs& a);
+int launch_kg_mfma(const OpsnnQmmArgs& a, hipStream_t st);   // qmm_i4_kg.hip
+uint64_t kg_workspace_bytes(const OpsnnQmmArgs& a);
 int launch_mx_mfma(const OpsnnQmmArgs& a, hipStream_t st);
 int launch_wqmm_mfma(const OpsnnWqmmArgs& a, hipStream_t st);
 uint64_t mx_workspace_bytes(const OpsnnQmmArgs& a);
@@ -263,6 +265,10 @@ extern "C" int opsnnQmmGroup(const OpsnnQmmArgs* a, void* stream)
         const int rc = launch_tcg_mfma(*a, (hipStream_t)stream);
         if (rc != OPSNN_NOT_TAKEN) return rc;
     }
+    if (i4 && a->force_variant != OPSNN_VARIANT_PLAIN && !opsnn_force_plain()) {
+        const int rc = launch_kg_mfma(*a, (hipStream_t)stream);
+        if (rc != OPSNN_NOT_TAKEN) return rc;
+    }
     return launch_group_plain(*a, tcg, (hipStream_t)stream);
 }
 
@@ -288,7 +294,9 @@ extern "C" uint64_t opsnnQmmWorkspace(const OpsnnQmmArgs* a, int mode)
     if (mode == 2) return mx_workspace_bytes(*a);
     // per-tensor / per-channel family: int8 operands share the int8 kernels and their re-layout; fp8 needs none
     if (mode == 3 && !(a->x1_dtype == DT_I8 && a->x2_dtype == DT_I8 && !a->x1_scale)) return 0;
-    if (mode == 4) return tcg_workspace_bytes(*a);   // K-group modes: the re-quantised weight of the fp8 x fp4 group-scale mode
+    // K-group modes: the re-quantised weight of the fp8 x fp4 group-scale mode; the widened operands, row sums and fp32
+    // scale / offset copies of the int4 mode with offsets
+    if (mode == 4) return a->x1_dtype == DT_I4 ? kg_workspace_bytes(*a) : tcg_workspace_bytes(*a);
     if (a->x2.row_stride == 1 || a->K == 1) return 0;           // already K-contiguous
     if (a->x2.col_stride != 1 || a->x2.row_stride != a->N) return 0;  // not a dense [K, N]: plain kernel
     uint64_t bits = (a->x2_dtype == DT_I4 || a->x2_dtype == DT_E2M1) ? 4 : 8;

@@ -258,12 +258,52 @@ def test_gpu_pertile_i8_on_the_matrix_cores(gpu, M, K, N, tB):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("M,K,N,out_dt", [(9, 1024, 256, "bf16"), (9, 1024, 256, "f16"), (33, 2048, 512, "bf16")])
+@pytest.mark.parametrize("M,K,N,out_dt", [(9, 1024, 256, "bf16"), (9, 1024, 256, "f16"), (33, 2048, 512, "bf16"),
+                                          # several row and column tiles, ragged in both; one group; a last group of 128; the
+                                          # one-thread-per-output kernel (fewer than 32 x 32 outputs)
+                                          (130, 1024, 512, "bf16"), (257, 4096, 768, "f16"), (1, 1024, 1280, "bf16"),
+                                          (3, 1024, 256, "f16")])
 def test_gpu_i4_asym(gpu, M, K, N, out_dt):
+    """int4 x int4 with group scales and offsets: the matrix-core kernel (operands widened to int8 in the workspace) is
+    bit-identical to the oracle, as the integer group sums are exact and the fp32 fold follows the golden's order."""
     m = gpu
     print(f"case int4 K-G {M}x{K}x{N} out={out_dt}", flush=True)
     dt = {"bf16": m.ACL_BF16, "f16": m.ACL_FLOAT16}
     inp = cases.make_i4_asym_inputs(m, M, K, N, M + N)
     want = cases.oracle_i4_asym(m, inp, M, K, N, dt[out_dt])
     got = cases.run_i4_asym_aclnn(m, inp, M, K, N, dt[out_dt])
+    assert np.array_equal(got, want), f"{int((got != want).sum())} of {got.size} outputs differ"
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("M,K,N,variant", [(130, 768, 200, 0), (70, 400, 1030, 0), (33, 250, 36, 0), (130, 768, 200, "plain")])
+def test_gpu_i4_asym_kernel_level_ragged_shapes(gpu, M, K, N, variant):
+    """opsnnQmmGroup called directly with shapes the aclnn layer does not let through (it wants K % 1024 == 0 and
+    N % 256 == 0): ragged row and column tiles and a partial last group, against the oracle bit for bit."""
+    m = gpu
+    print(f"case int4 K-G kernel level {M}x{K}x{N} variant={variant}", flush=True)
+    inp = cases.make_i4_asym_inputs(m, M, K, N, M + N + K)
+    want = cases.oracle_i4_asym(m, inp, M, K, N, m.ACL_BF16)
+    d = {k: m.DeviceBuffer(host=v) for k, v in inp.items()}
+    d_out = m.DeviceBuffer(M * N * 2); d_out.fill(0xFF)
+    G = -(-K // 256)
+    a = m.OpsnnQmmArgs()
+    a.M, a.N, a.K, a.batch = M, N, K, 1
+    a.x1 = m.OpsnnMat(d["x1"].ptr, K, 1, 0)
+    a.x2 = m.OpsnnMat(d["x2"].ptr, 1, K, 0)
+    a.x1_dtype = a.x2_dtype = m.ACL_INT4
+    a.out, a.out_dtype = d_out.ptr, m.ACL_BF16
+    a.x1_scale = d["s1"].ptr
+    a.gsM, a.gsN, a.gsK = 1, 1, 256
+    a.x2_scale_mat = m.OpsnnMat(d["s2"].ptr, N, 1, 0)
+    a.x2_offset_mat = m.OpsnnMat(d["off"].ptr, N, 1, 0)
+    a.x2_scale_dtype = m.ACL_FLOAT
+    a.force_variant = m.VARIANT_PLAIN if variant == "plain" else m.VARIANT_AUTO
+    need = m.lib().opsnnQmmWorkspace(a, 4)
+    assert (need > 0) == (M * N >= 1024)
+    ws = m.DeviceBuffer(need) if need else None
+    a.workspace = ws.ptr if ws else None
+    assert m.lib().opsnnQmmGroup(a, None) == 0
+    m.check(m.lib().aclrtSynchronizeDevice(), "sync")
+    got = d_out.to_host(np.uint16, (M, N))
     assert np.array_equal(got, want), f"{int((got != want).sum())} of {got.size} outputs differ"
