@@ -296,6 +296,10 @@ template <> int launch_wq_stream<DT_F16, 4>(const WqParams&, const WqStreamOpts&
 template <> int launch_wq_stream<DT_F16, 8>(const WqParams&, const WqStreamOpts&, hipStream_t);
 template <> int launch_wq_stream<DT_BF16, 4>(const WqParams&, const WqStreamOpts&, hipStream_t);
 template <> int launch_wq_stream<DT_BF16, 8>(const WqParams&, const WqStreamOpts&, hipStream_t);
+template <> int launch_wq_xreg_float<DT_F16, 4>(const WqParams&, hipStream_t);
+template <> int launch_wq_xreg_float<DT_F16, 8>(const WqParams&, hipStream_t);
+template <> int launch_wq_xreg_float<DT_BF16, 4>(const WqParams&, hipStream_t);
+template <> int launch_wq_xreg_float<DT_BF16, 8>(const WqParams&, hipStream_t);
 
 // Can the streamlined kernel take this problem, and in which form?
 template <int WBITS>
@@ -351,6 +355,18 @@ namespace opsnn {
 template <int XDT, int WBITS>
 static int launch_slabs_float(WqParams p, hipStream_t st)
 {
+    // up to 16 rows: x in registers (mxfp4: e2m1 codes with a row's e8m0 bytes contiguous; e4m3 codes with per-channel scales)
+    static const bool no_xreg = [] { const char* e = getenv("OPSNN_WQ_XREG_MIN"); return e && atoi(e) > 16; }();
+    if (!no_xreg && p.M <= 16 && !p.offset) {
+        bool ok;
+        if (WBITS == 4) ok = p.scale_e8m0 && p.group == 32 && p.s_rs == 1 && p.s_cs % 16 == 0 && (uintptr_t)p.scale % 16 == 0;
+        else ok = !p.scale_e8m0 && p.group >= p.K;
+        if (ok) {
+            p.m_base = 0; p.m_rows = p.M; p.cpg_shift = 31;
+            const int rc = launch_wq_xreg_float<XDT, WBITS>(p, st);
+            if (rc != OPSNN_NOT_TAKEN) return rc;
+        }
+    }
     for (int64_t m0 = 0; m0 < p.M; m0 += 64) {
         p.m_base = m0;
         p.m_rows = (p.M - m0) < 64 ? (p.M - m0) : 64;

@@ -106,6 +106,46 @@ __device__ __forceinline__ v4i dequant8(const v4i& piece, int s, uint16_t sb, ui
     }
 }
 
+// ---- 8 floating-point weight codes of one lane -> MFMA row operand ----
+// WBITS 4: the e2m1 codes of dword s, delivered in element order [0,4,1,5,2,6,3,7] like dequant8's int4 form; WBITS 8:
+// the e4m3 codes of dwords 2s, 2s+1 in natural order.  Every code is exact in fp16 and in bf16, so T(w * scale) rounds
+// once, in the multiplication: packed fp16 for fp16; for bf16 the exact fp16 value is widened to fp32, multiplied and
+// rounded to bf16 by the hardware conversion.
+template <int XDT, int WBITS>
+__device__ __forceinline__ v4i dequant8_float(const v4i& piece, int s, uint16_t sb)
+{
+    h2 w[4];   // the eight weights, exact, as fp16 pairs
+    if constexpr (WBITS == 4) {
+        const uint32_t q = (uint32_t)piece[s];
+        const h2 k14 = {(_Float16)16384.0f, (_Float16)16384.0f};
+#pragma unroll
+        for (int i = 0; i < 4; i++) {   // see dequant_fp4_f16: magnitude bits at bits 11..9 of a half read as 2^-14 times the value
+            const uint32_t t = q >> (4 * i);
+            w[i] = __builtin_bit_cast(h2, ((t & 0x00070007u) << 9) | ((t & 0x00080008u) << 12)) * k14;
+        }
+    } else {
+        const uint32_t d0 = (uint32_t)piece[2 * s], d1 = (uint32_t)piece[2 * s + 1];
+        w[0] = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(d0, 1.0f, false);
+        w[1] = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(d0, 1.0f, true);
+        w[2] = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(d1, 1.0f, false);
+        w[3] = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(d1, 1.0f, true);
+    }
+    if constexpr (XDT == DT_F16) {
+        const _Float16 sh = __builtin_bit_cast(_Float16, sb);
+        const h2 sc = {sh, sh};
+        return (v4i){(int)u32(w[0] * sc), (int)u32(w[1] * sc), (int)u32(w[2] * sc), (int)u32(w[3] * sc)};
+    } else {
+        const float scf = bf16_to_f32(sb);
+        v4i r;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const v2f t = {(float)w[i][0] * scf, (float)w[i][1] * scf};
+            r[i] = (int)pack2_bf16(t);
+        }
+        return r;
+    }
+}
+
 // NW waves per workgroup (4 or 8) = WN row blocks x WK waves that split K chunk by chunk.
 template <int XDT, int WBITS, int MB, int NW, int WK, bool HAS_OFF, bool VSCALE>
 __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(NW == 8 ? 4 : 2))) void wqmm_stream_kernel(WqParams p)
@@ -722,9 +762,16 @@ __global__ __launch_bounds__(256, 2) void wqmm_resx_kernel(WqParams p)
 // it is (row block count % NW) adds them and stores.  As in the kernel above the weight stream runs across row blocks:
 // the slot a chunk was consumed from is refilled with the chunk PF further on, in this row block or the next.
 // Sixteen waves (four per SIMD, 128 registers each, 16 fragments of x) hide the dequantisation's vector work best.
-template <int XDT, int WBITS, int NW, int NCH, bool HAS_OFF, bool VSCALE>
+// SCM, where a chunk's scale comes from: 0 one 16-bit load per chunk (any group that is a power-of-two multiple of the
+// chunk, or per channel); 1 one scale per chunk, a row's scales contiguous: 8- or 16-byte loads one row block ahead;
+// 2 (4-bit weights) one e8m0 byte per 32 weights, i.e. per lane piece, a row's bytes contiguous: 16-byte loads one row
+// block ahead.  WFLT: the weights are floating-point codes (e2m1 / e4m3), no offset.
+template <int XDT, int WBITS, int NW, int NCH, bool HAS_OFF, int SCM, bool WFLT = false>
 __global__ __launch_bounds__(NW * 64) void wqmm_xreg_kernel(WqParams p)
 {
+    constexpr bool VSCALE = SCM == 1, MXS = SCM == 2;
+    static_assert(!MXS || WBITS == 4, "one e8m0 byte per lane piece of 32 weights");
+    static_assert(!WFLT || !HAS_OFF, "floating-point weight codes carry no offset");
     constexpr int KPL = 128 / WBITS, KC = 4 * KPL, STEPS = KC / 32;
     constexpr int PF = NW == 16 ? 4 : (NCH < 8 ? NCH : 8);   // weight pieces in flight per lane
     constexpr int NX = NCH * STEPS;                          // x fragments per lane
@@ -744,17 +791,26 @@ __global__ __launch_bounds__(NW * 64) void wqmm_xreg_kernel(WqParams p)
 
     auto row_of = [&](int rb) { const int64_t n = (int64_t)rb * 16 + nrow; return n < p.N ? n : p.N - 1; };
     auto wptr_of = [&](int rb) { return p.w + row_of(rb) * p.ldw + g * 16 + (int64_t)cbase * 64; };
+    // a row's scales: 16-bit elements, or (MXS) e8m0 bytes
+    auto srow_of = [&](int rb) { return (const uint16_t*)((const char*)p.scale + row_of(rb) * p.s_cs * (MXS ? 1 : 2)); };
     int rb = blockIdx.x;
     const uint8_t* wptr = wptr_of(rb);
-    const uint16_t* srow = p.scale + row_of(rb) * p.s_cs;
+    const uint16_t* srow = srow_of(rb);
     const uint16_t* orow = HAS_OFF ? p.offset + row_of(rb) * p.s_cs : nullptr;
 
-    // VSCALE (one scale per chunk, a row's scales contiguous): the NCH scales of this wave's K range as NCH/2 dwords,
-    // fetched with 8- or 16-byte loads one row block ahead
-    constexpr int SW = NCH / 2;
+    // VSCALE: the NCH scales of this wave's K range as NCH/2 dwords; MXS: its 4 NCH scale bytes as NCH dwords (byte g of
+    // dword c belongs to lane group g); fetched one row block ahead
+    constexpr int SW = MXS ? NCH : NCH / 2;
     uint32_t sv[SW], ov[SW], svn[SW], ovn[SW];
     auto load_scales = [&](const uint16_t* sr, const uint16_t* orw, uint32_t (&sd)[SW], uint32_t (&od)[SW]) {
-        if constexpr (NCH % 8 == 0) {
+        if constexpr (MXS) {
+#pragma unroll
+            for (int h = 0; h < NCH / 4; h++) {
+                const v4i t = *(const v4i*)((const uint8_t*)sr + cbase * 4 + 16 * h);
+#pragma unroll
+                for (int e = 0; e < 4; e++) sd[4 * h + e] = (uint32_t)t[e];
+            }
+        } else if constexpr (NCH % 8 == 0) {
 #pragma unroll
             for (int h = 0; h < NCH / 8; h++) {
                 const v4i t = *(const v4i*)(sr + cbase + 8 * h);
@@ -777,12 +833,12 @@ __global__ __launch_bounds__(NW * 64) void wqmm_xreg_kernel(WqParams p)
     };
 #pragma unroll
     for (int h = 0; h < SW; h++) sv[h] = ov[h] = svn[h] = ovn[h] = 0;
-    if constexpr (VSCALE) load_scales(srow, orow, svn, ovn);
+    if constexpr (VSCALE || MXS) load_scales(srow, orow, svn, ovn);
     v4i wq[PF];
     uint16_t sq[PF], oq[PF];
     auto fetch = [&](int j, const uint8_t* wp, const uint16_t* sr, const uint16_t* orw, int cw) {
         wq[j] = *(const v4i*)(wp + (int64_t)cw * 64);
-        if constexpr (!VSCALE) {
+        if constexpr (SCM == 0) {
             const int64_t so = (int64_t)((cbase + cw) >> p.cpg_shift) * p.s_rs;
             sq[j] = sr[so];
             if constexpr (HAS_OFF) oq[j] = orw[so];
@@ -843,9 +899,9 @@ __global__ __launch_bounds__(NW * 64) void wqmm_xreg_kernel(WqParams p)
         const int rb_next = rb + (int)gridDim.x;
         const bool has_next = rb_next < nblocks;
         const uint8_t* wptr_n = has_next ? wptr_of(rb_next) : wptr;   // past the end: harmless reloads of this block
-        const uint16_t* srow_n = has_next ? p.scale + row_of(rb_next) * p.s_cs : srow;
+        const uint16_t* srow_n = has_next ? srow_of(rb_next) : srow;
         const uint16_t* orow_n = HAS_OFF ? (has_next ? p.offset + row_of(rb_next) * p.s_cs : orow) : nullptr;
-        if constexpr (VSCALE) {
+        if constexpr (VSCALE || MXS) {
             // the next row block's scales are requested before the refills below fetch its weights (loads return in
             // issue order: waiting for a scale issued after them would drain the weight stream)
 #pragma unroll
@@ -857,7 +913,10 @@ __global__ __launch_bounds__(NW * 64) void wqmm_xreg_kernel(WqParams p)
         for (int c = 0; c < NCH; c++) {
             const int j = c % PF;
             uint16_t sb, ob = 0;
-            if constexpr (VSCALE) {
+            if constexpr (MXS) {
+                // the scale goes through x's dtype (2^e: exact in bf16; fp16 flushes, denormalises or overflows it as the cast does)
+                sb = bits_x<XDT>(e8m0_to_f32((sv[c] >> (8 * g)) & 0xffu));
+            } else if constexpr (VSCALE) {
                 sb = (uint16_t)(sv[c / 2] >> (16 * (c % 2)));
                 if constexpr (HAS_OFF) ob = (uint16_t)(ov[c / 2] >> (16 * (c % 2)));
             } else {
@@ -866,7 +925,9 @@ __global__ __launch_bounds__(NW * 64) void wqmm_xreg_kernel(WqParams p)
             }
 #pragma unroll
             for (int s = 0; s < STEPS; s++) {
-                const v4i aop = dequant8<XDT, WBITS, HAS_OFF>(wq[j], s, sb, ob, dqc);
+                v4i aop;
+                if constexpr (WFLT) aop = dequant8_float<XDT, WBITS>(wq[j], s, sb);
+                else aop = dequant8<XDT, WBITS, HAS_OFF>(wq[j], s, sb, ob, dqc);
                 if constexpr (XDT == DT_F16) {
                     acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(v8h, aop), __builtin_bit_cast(v8h, xr[c * STEPS + s]), acc, 0, 0, 0);
                 } else {
@@ -940,14 +1001,14 @@ static int launch_resx_one(const WqParams& p, hipStream_t st)
 }
 
 // One workgroup per CU (its waves fill the register file), or one per row block when there are fewer.
-template <int XDT, int WBITS, int NW, int NCH, bool HAS_OFF, bool VSCALE>
+template <int XDT, int WBITS, int NW, int NCH, bool HAS_OFF, int SCM, bool WFLT = false>
 static int launch_xreg_one(const WqParams& p, hipStream_t st)
 {
     const int64_t nblocks = (p.N + 15) / 16;
     const int64_t g = (int64_t)resx_grid(1ll << 40) / 2;
     constexpr int STEPS = (4 * (128 / WBITS)) / 32;
     constexpr int lds = NW * (NCH * STEPS / 8) * 4096;   // half of the K range of every wave: 16 rows x 256 bytes per unit
-    auto k = wqmm_xreg_kernel<XDT, WBITS, NW, NCH, HAS_OFF, VSCALE>;
+    auto k = wqmm_xreg_kernel<XDT, WBITS, NW, NCH, HAS_OFF, SCM, WFLT>;
     static bool attr_set = false;
     if (!attr_set) {
         hipError_t e = hipFuncSetAttribute((const void*)k, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
@@ -961,8 +1022,8 @@ static int launch_xreg_one(const WqParams& p, hipStream_t st)
 template <int XDT, int WBITS, int NW, int NCH>
 static int launch_xreg_nch(const WqParams& p, bool has_off, bool vscale, hipStream_t st)
 {
-    if (vscale) return has_off ? launch_xreg_one<XDT, WBITS, NW, NCH, true, true>(p, st) : launch_xreg_one<XDT, WBITS, NW, NCH, false, true>(p, st);
-    return has_off ? launch_xreg_one<XDT, WBITS, NW, NCH, true, false>(p, st) : launch_xreg_one<XDT, WBITS, NW, NCH, false, false>(p, st);
+    if (vscale) return has_off ? launch_xreg_one<XDT, WBITS, NW, NCH, true, 1>(p, st) : launch_xreg_one<XDT, WBITS, NW, NCH, false, 1>(p, st);
+    return has_off ? launch_xreg_one<XDT, WBITS, NW, NCH, true, 0>(p, st) : launch_xreg_one<XDT, WBITS, NW, NCH, false, 0>(p, st);
 }
 
 // K = waves x chunks per wave x chunk.  Sixteen waves with 4 chunks each (8-bit weights: or 8), else eight waves with 4 or 8.
@@ -987,6 +1048,23 @@ static int launch_xreg(const WqParams& p, bool has_off, bool vscale, int force_n
     }
     if (nw == 8 && nch == 4) return launch_xreg_nch<XDT, WBITS, 8, 4>(p, has_off, vscale, st);
     if (nw == 8 && nch == 8) return launch_xreg_nch<XDT, WBITS, 8, 8>(p, has_off, vscale, st);
+    return OPSNN_NOT_TAKEN;
+}
+
+// Floating-point weight codes without offset: e2m1 with e8m0 scales per 32 weights (mxfp4; a row's scale bytes contiguous and
+// 16-byte aligned), e4m3 with one scale per channel.  p.cpg_shift must be set for the latter.
+template <int XDT, int WBITS>
+static int launch_xreg_float(const WqParams& p, hipStream_t st)
+{
+    int nw = 0, nch = 0;
+    if (!xreg_shape(WBITS, p.K, 0, nw, nch)) return OPSNN_NOT_TAKEN;
+    constexpr int SCM = WBITS == 4 ? 2 : 0;
+    if (nw == 16 && nch == 4) return launch_xreg_one<XDT, WBITS, 16, 4, false, SCM, true>(p, st);
+    if constexpr (WBITS == 8) {
+        if (nw == 16 && nch == 8) return launch_xreg_one<XDT, WBITS, 16, 8, false, SCM, true>(p, st);
+    }
+    if (nw == 8 && nch == 4) return launch_xreg_one<XDT, WBITS, 8, 4, false, SCM, true>(p, st);
+    if (nw == 8 && nch == 8) return launch_xreg_one<XDT, WBITS, 8, 8, false, SCM, true>(p, st);
     return OPSNN_NOT_TAKEN;
 }
 
@@ -1040,8 +1118,13 @@ struct WqStreamOpts {
 // One row slab (p.m_rows <= 128 with o.rows, else <= 64) of one dtype pair; defined once per pair in its own translation unit.
 template <int XDT, int WBITS>
 int launch_wq_stream(const WqParams& p, const WqStreamOpts& o, hipStream_t st);
+// Up to 16 rows, floating-point weight codes (see launch_xreg_float); OPSNN_NOT_TAKEN if K does not split.
+template <int XDT, int WBITS>
+int launch_wq_xreg_float(const WqParams& p, hipStream_t st);
 
 #define OPSNN_WQ_STREAM_DEFINE(XDT, WBITS)                                                                          \
+    template <>                                                                                                     \
+    int launch_wq_xreg_float<XDT, WBITS>(const WqParams& p, hipStream_t st) { return launch_xreg_float<XDT, WBITS>(p, st); } \
     template <int MB, int NW, int WK, bool VS>                                                                      \
     static int wq_stream_off(const WqParams& p, bool has_off, hipStream_t st)                                       \
     {                                                                                                               \

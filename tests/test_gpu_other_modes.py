@@ -290,11 +290,22 @@ def test_weight_only_tile_kernel(gpu, M, K, N, x_dt, w_dt, group, tW, off, bias)
     (16, 8192, 200, "f16", "i8", 64, True, True, "f16"),
     (7, 4096, 320, "bf16", "i8", 128, True, True, None),
     (16, 8192, 96, "bf16", "i4", 128, False, True, None),
+    # floating-point weight codes (1 .. 16 rows): mxfp4 (e2m1 with one e8m0 byte per 32 K, a row's bytes contiguous) on 16 and
+    # on 8 waves, both activation types; e4m3 with per-channel scales on 16 waves x 8 chunks, 16 x 4 and 8 x 4
+    (16, 8192, 256, "f16", "fp4", 32, True, False, None),
+    (5, 8192, 1000, "bf16", "fp4", 32, True, False, "bf16"),
+    (1, 4096, 130, "bf16", "fp4", 32, True, False, None),
+    (16, 4096, 4400, "f16", "fp4", 32, True, False, "f16"),
+    (16, 8192, 96, "bf16", "e4m3", 0, True, False, None),
+    (12, 4096, 200, "bf16", "e4m3", 0, True, False, "bf16"),
+    (7, 2048, 72, "f16", "e4m3", 0, True, False, None),
 ])
 def test_weight_only_x_in_registers_kernel(gpu, M, K, N, x_dt, w_dt, group, tW, off, bias):
-    """4 .. 16 rows of x with K in eight equal ranges of whole chunks: the kernel that keeps x in registers."""
+    """4 .. 16 rows of x (floating-point weight codes: 1 .. 16) with K in 8 or 16 equal ranges of whole chunks: the kernel
+    that keeps x in registers."""
     m = gpu
-    dt = {"bf16": m.ACL_BF16, "f16": m.ACL_FLOAT16, "i8": m.ACL_INT8, "i4": m.ACL_INT4, None: None}
+    dt = {"bf16": m.ACL_BF16, "f16": m.ACL_FLOAT16, "i8": m.ACL_INT8, "i4": m.ACL_INT4, "e4m3": m.ACL_FLOAT8_E4M3FN,
+          "fp4": m.ACL_FLOAT4_E2M1, None: None}
     print(f"case wq x-in-registers M={M} K={K} N={N} x={x_dt} w={w_dt} g={group} tW={tW} off={off} bias={bias}", flush=True)
     inp = cases.make_wq_inputs(m, M, K, N, M * 3 + N, dt[x_dt], dt[w_dt], group, tW, off, dt[bias])
     want = cases.oracle_wq(m, inp, M, K, N)
