@@ -239,6 +239,12 @@ typedef struct {
     int force_variant;
     int64_t block;    /* elements per scale block: a multiple of 32 up to 1024; 0 means 32 */
     int scale_alg;    /* 0: scale 2^(floor(log2 max) - emax); 1 (fp8 outputs only): max / typeMax rounded up to a power of two */
+    /* General form, used when axis_len > 0 (rows and cols are then ignored): x is [outer, axis_len, inner] and the blocks run
+     * along axis_len; x may also be FLOAT, y also FLOAT4_E1M2; round_mode 0 rint, 1 round (ties away from zero), 2 floor,
+     * 3 ceil, 4 trunc.  scale is [outer, ceil(nblocks / 2), inner, 2].  4-bit outputs need an even inner (or, with
+     * inner == 1, an even axis_len). */
+    int64_t outer, axis_len, inner;
+    int round_mode;
 } OpsnnMxQuantArgs;
 OPSNN_API int opsnnDynamicMxQuant(const OpsnnMxQuantArgs* a, void* stream);
 

@@ -62,12 +62,10 @@ aclnnStatus aclnnDynamicMxQuantGetWorkspaceSize(const aclTensor* x_, int64_t axi
     want[(size_t)ax] = ((x.dim(ax) + blocksize - 1) / blocksize + 1) / 2;
     want.push_back(2);
     if (sc.shape != want) INVALID("%s: mxscaleOut %s must be %s", kApi, shape_str(sc.shape).c_str(), shape_str(want).c_str());
-    // what this build does not run
-    if (ax != x.rank() - 1) NOT_RUN("%s: only the last axis has a kernel here", kApi);
-    if (x.dtype == ACL_FLOAT) NOT_RUN("%s: a FLOAT x has no kernel here", kApi);
-    if (y.dtype == ACL_FLOAT4_E1M2) NOT_RUN("%s: FLOAT4_E1M2 has no kernel here", kApi);
-    if (std::strcmp(mode, "rint") != 0) NOT_RUN("%s: only roundMode rint has a kernel here", kApi);
     if (!is_contiguous(x) || !is_contiguous(y) || !is_contiguous(sc)) INVALID("%s: tensors must be contiguous here", kApi);
+    // the last axis of a 16-bit x, rounded to nearest even onto e2m1 / fp8: the tuned kernels; anything else the general one
+    const int round_mode = !std::strcmp(mode, "rint") ? 0 : !std::strcmp(mode, "round") ? 1 : 2;
+    const bool general = ax != x.rank() - 1 || x.dtype == ACL_FLOAT || y.dtype == ACL_FLOAT4_E1M2 || round_mode != 0;
 
     std::unique_ptr<aclOpExecutor> ex(new (std::nothrow) aclOpExecutor());
     if (!ex) FAIL(ACLNN_ERR_INNER_CREATE_EXECUTOR, "%s: cannot allocate executor", kApi);
@@ -85,6 +83,12 @@ aclnnStatus aclnnDynamicMxQuantGetWorkspaceSize(const aclTensor* x_, int64_t axi
     a.scale = const_cast<void*>(sc.ptr_at(0));
     a.cols = x.dim(-1); a.rows = x.numel() / a.cols; a.force_variant = 0;
     a.block = blocksize; a.scale_alg = (int)scaleAlg;
+    a.outer = a.axis_len = a.inner = 0; a.round_mode = 0;
+    if (general) {
+        a.axis_len = x.dim(ax); a.outer = 1; a.inner = 1; a.round_mode = round_mode;
+        for (int64_t i = 0; i < ax; i++) a.outer *= x.dim(i);
+        for (int64_t i = ax + 1; i < x.rank(); i++) a.inner *= x.dim(i);
+    }
     *executor = (aclOpExecutor*)executor_publish(ex.release());
     return ACLNN_SUCCESS;
 }

@@ -19,7 +19,7 @@ typedef unsigned short v4us __attribute__((ext_vector_type(4)));
 // Element type codes: the aclDataType values.
 enum : int {
     DT_F32 = 0, DT_F16 = 1, DT_I8 = 2, DT_I32 = 3, DT_BF16 = 27, DT_I4 = 29,
-    DT_E5M2 = 35, DT_E4M3 = 36, DT_E8M0 = 37, DT_E2M1 = 40, DT_U64 = 10
+    DT_E5M2 = 35, DT_E4M3 = 36, DT_E8M0 = 37, DT_E2M1 = 40, DT_E1M2 = 41, DT_U64 = 10
 };
 
 __device__ __forceinline__ uint32_t f2u(float f) { return __builtin_bit_cast(uint32_t, f); }

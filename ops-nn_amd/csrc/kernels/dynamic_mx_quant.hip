@@ -194,6 +194,139 @@ __global__ __launch_bounds__(256) void mx_quant_generic_kernel(MxQuantParams p)
     }
 }
 
+// ---- general form: blocks along any axis of [outer, A, inner], fp32 input, e1m2 elements, every rounding mode ----
+// (golden.py:181-218, 263-330).  One thread per block and inner column -- two neighbouring columns for the 4-bit types,
+// whose bytes hold two elements of the last axis -- so that neighbouring threads read neighbouring addresses when
+// inner > 1; not tuned beyond that.  floor(log2) of the block maximum and of every scaled element is the exponent field of
+// the fp32 (the element's clamped from below at the format's smallest normal exponent), all scalings are by powers of two
+// and exact, and the mantissa is rounded as an integer by the mode.
+struct MxGeneralParams {
+    const void* x; uint8_t* y; uint8_t* scale;
+    int64_t outer, A, inner, nblk, np;
+    int block, scale_alg, round_mode, x_dt, y_dt;
+};
+
+__device__ __forceinline__ float mxg_load(const void* x, int dt, int64_t i)
+{
+    if (dt == DT_F32) return ((const float*)x)[i];
+    const uint32_t h = ((const uint16_t*)x)[i];
+    return dt == DT_BF16 ? u2f(h << 16) : f16_to_f32((uint16_t)h);
+}
+
+// one scaled element -> its code (8-bit formats: the byte; 4-bit: the nibble)
+__device__ __forceinline__ uint32_t mxg_element(float v, float inv_scale, bool bad, int emin, int mbits, float tmax, int mode, int y_dt)
+{
+    float q = 0.0f;
+    if (!bad) {
+        q = __fmul_rn(v, inv_scale);
+        int e = (int)((f2u(q) >> 23) & 0xffu) - 127;
+        e = e < emin ? emin : e;
+        // q / 2^e * 2^mbits and back: exact scalings (|q| < 2 tmax, e >= emin >= -14)
+        const float up = u2f((uint32_t)(127 + mbits - e) << 23), down = u2f((uint32_t)(127 - mbits + e) << 23);
+        float r = __fmul_rn(q, up);
+        switch (mode) {
+            case 0: r = __builtin_rintf(r); break;
+            case 1: { const float t = __builtin_floorf(__fadd_rn(fabsf(r), 0.5f)); r = (f2u(r) >> 31) ? -t : t; break; }
+            case 2: r = __builtin_floorf(r); break;
+            case 3: r = __builtin_ceilf(r); break;
+            default: r = __builtin_truncf(r); break;
+        }
+        q = __fmul_rn(r, down);
+        q = fminf(fmaxf(q, -tmax), tmax);
+    }
+    if (y_dt == DT_E4M3) return f32_to_e4m3_bits(q) & 0xffu;
+    if (y_dt == DT_E5M2) return f32_to_e5m2_bits(q) & 0xffu;
+    if (y_dt == DT_E2M1) return mx_e2m1_code(q);                     // q is on the grid: the code of q itself
+    return (uint32_t)__fmul_rn(fabsf(q), 4.0f) | ((f2u(q) >> 28) & 8u);   // e1m2: the magnitudes are k / 4
+}
+
+__global__ __launch_bounds__(256) void mx_quant_general_kernel(MxGeneralParams p)
+{
+    const bool fp4 = p.y_dt == DT_E2M1 || p.y_dt == DT_E1M2;
+    const bool pair_inner = fp4 && p.inner > 1;            // a thread takes the inner columns 2 iw, 2 iw + 1
+    const int64_t iw = pair_inner ? p.inner / 2 : p.inner;
+    const int64_t g = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (g >= p.outer * p.nblk * iw) return;
+    const int64_t o = g / (p.nblk * iw), rem = g - o * (p.nblk * iw), b = rem / iw, ic = rem - b * iw;
+    int emax, emin, mbits; float tmax;
+    switch (p.y_dt) {
+        case DT_E2M1: emax = 2; emin = 0; mbits = 1; tmax = 6.0f; break;
+        case DT_E1M2: emax = 0; emin = 0; mbits = 2; tmax = 1.75f; break;
+        case DT_E4M3: emax = 8; emin = -6; mbits = 3; tmax = 448.0f; break;
+        default: emax = 15; emin = -14; mbits = 2; tmax = 57344.0f; break;
+    }
+    const int64_t a0 = b * p.block, a1 = a0 + p.block < p.A ? a0 + p.block : p.A;
+    const int ncol = pair_inner ? 2 : 1;
+    float inv_scale[2]; bool bad[2];
+    for (int c = 0; c < ncol; c++) {
+        const int64_t in = pair_inner ? 2 * ic + c : ic;
+        float amax = 0.0f; bool bd = false;
+        for (int64_t a = a0; a < a1; a++) {
+            const float v = fabsf(mxg_load(p.x, p.x_dt, (o * p.A + a) * p.inner + in));
+            bd |= !(v < __builtin_inff());
+            amax = fmaxf(amax, v);
+        }
+        int share = -127;
+        if (!bd && amax != 0.0f) {
+            if (p.scale_alg == 1) {
+                const uint32_t u = f2u(__fdiv_rn(amax, tmax));
+                int e = (int)(u >> 23);
+                const uint32_t mant = u & 0x7fffffu;
+                if ((e > 0 && e < 254 && mant > 0) || (e == 0 && mant > 0x400000u)) e += 1;
+                share = e - 127;
+            } else {
+                const int e = (int)(f2u(amax) >> 23);
+                share = (e == 0 || e - 127 - emax < -127) ? -127 : e - 127 - emax;
+            }
+        }
+        p.scale[((o * p.np + b / 2) * p.inner + in) * 2 + (b & 1)] = bd ? 0xFFu : (uint8_t)(share + 127);
+        if (b == p.nblk - 1 && (p.nblk & 1)) p.scale[((o * p.np + b / 2) * p.inner + in) * 2 + 1] = 0;
+        inv_scale[c] = u2f((uint32_t)(127 - share) << 23);
+        bad[c] = bd;
+    }
+    if (pair_inner) {
+        for (int64_t a = a0; a < a1; a++) {
+            const int64_t i = (o * p.A + a) * p.inner + 2 * ic;
+            const uint32_t lo = mxg_element(mxg_load(p.x, p.x_dt, i), inv_scale[0], bad[0], emin, mbits, tmax, p.round_mode, p.y_dt);
+            const uint32_t hi = mxg_element(mxg_load(p.x, p.x_dt, i + 1), inv_scale[1], bad[1], emin, mbits, tmax, p.round_mode, p.y_dt);
+            p.y[i >> 1] = (uint8_t)(lo | (hi << 4));
+        }
+    } else if (fp4) {   // inner == 1: the block's own elements pair up (A is even, blocks are multiples of 32)
+        for (int64_t a = a0; a < a1; a += 2) {
+            const int64_t i = o * p.A + a;
+            const uint32_t lo = mxg_element(mxg_load(p.x, p.x_dt, i), inv_scale[0], bad[0], emin, mbits, tmax, p.round_mode, p.y_dt);
+            const uint32_t hi = a + 1 < a1 ? mxg_element(mxg_load(p.x, p.x_dt, i + 1), inv_scale[0], bad[0], emin, mbits, tmax, p.round_mode, p.y_dt) : 0u;
+            p.y[i >> 1] = (uint8_t)(lo | (hi << 4));
+        }
+    } else {
+        for (int64_t a = a0; a < a1; a++) {
+            const int64_t i = (o * p.A + a) * p.inner + ic;
+            p.y[i] = (uint8_t)mxg_element(mxg_load(p.x, p.x_dt, i), inv_scale[0], bad[0], emin, mbits, tmax, p.round_mode, p.y_dt);
+        }
+    }
+}
+
+static int launch_mx_quant_general(const OpsnnMxQuantArgs& a, hipStream_t st)
+{
+    MxGeneralParams p{};
+    p.x = a.x; p.y = (uint8_t*)a.y; p.scale = (uint8_t*)a.scale;
+    p.outer = a.outer; p.A = a.axis_len; p.inner = a.inner;
+    p.block = a.block ? (int)a.block : 32; p.scale_alg = a.scale_alg; p.round_mode = a.round_mode;
+    p.x_dt = a.x_dtype; p.y_dt = a.y_dtype;
+    if (p.outer <= 0 || p.A <= 0 || p.inner <= 0 || p.block <= 0 || p.block % 32 != 0 || p.block > 1024) return -2;
+    if (p.x_dt != DT_F16 && p.x_dt != DT_BF16 && p.x_dt != DT_F32) return -2;
+    const bool fp4 = p.y_dt == DT_E2M1 || p.y_dt == DT_E1M2;
+    if (!fp4 && p.y_dt != DT_E4M3 && p.y_dt != DT_E5M2) return -2;
+    if (p.round_mode < 0 || p.round_mode > 4 || (p.scale_alg != 0 && (p.scale_alg != 1 || fp4))) return -2;
+    if (fp4 && ((p.inner > 1 ? p.inner : p.A) & 1)) return -2;
+    p.nblk = (p.A + p.block - 1) / p.block; p.np = (p.nblk + 1) / 2;
+    const int64_t iw = fp4 && p.inner > 1 ? p.inner / 2 : p.inner;
+    const int64_t wgs = (p.outer * p.nblk * iw + 255) / 256;
+    if (wgs > 0x7fffffff) return -1;
+    hipLaunchKernelGGL(mx_quant_general_kernel, dim3((unsigned)wgs), dim3(256), 0, st, p);
+    return (int)hipGetLastError();
+}
+
 template <int X_DT, int Y_DT>
 static int launch_mx_quant(const MxQuantParams& p, int variant, hipStream_t st)
 {
@@ -235,7 +368,9 @@ using namespace opsnn;
 
 extern "C" int opsnnDynamicMxQuant(const OpsnnMxQuantArgs* a, void* stream)
 {
-    if (!a || !a->x || !a->y || !a->scale || a->rows <= 0 || a->cols <= 0) return -1;
+    if (!a || !a->x || !a->y || !a->scale) return -1;
+    if (a->axis_len > 0) return launch_mx_quant_general(*a, (hipStream_t)stream);
+    if (a->rows <= 0 || a->cols <= 0) return -1;
     if (a->x_dtype != DT_F16 && a->x_dtype != DT_BF16) return -2;
     if (a->y_dtype == DT_E2M1 && (a->cols & 1)) return -2;
     MxQuantParams p{};

@@ -94,6 +94,7 @@ class OpsnnMxQuantArgs(C.Structure):
         ("rows", C.c_int64), ("cols", C.c_int64),
         ("force_variant", C.c_int),
         ("block", C.c_int64), ("scale_alg", C.c_int),
+        ("outer", C.c_int64), ("axis_len", C.c_int64), ("inner", C.c_int64), ("round_mode", C.c_int),
     ]
 
 

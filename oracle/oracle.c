@@ -56,7 +56,11 @@
  *                       onto the element grid with saturation, recomputed in numpy with torch's fp8 casts and a brute-force
  *                       nearest-grid-point search for e2m1; known answers for ties, saturation and the scale bytes; dequantised
  *                       values within half a grid step; scale algorithm 1 by its defining property, the smallest power of two
- *                       under which no element saturates; larger blocks by monotonicity against blocks of 32)
+ *                       under which no element saturates; larger blocks by monotonicity against blocks of 32);
+ *                       its general form (another axis, fp32 input, e1m2 elements, round / floor / ceil / trunc) by the modes'
+ *                       definitions on the explicit e2m1 and e1m2 grids with every tie, by transposition against the
+ *                       last-axis form, and by fp32 inputs that are 16-bit values; parity unpinned for fp32 inputs within an
+ *                       ulp or two below a power of two, where the golden's float32 log2 rounds up
  *   orc_trans_quant_param pinned (the packing utility of the matmul golden and the reference's system-test formula in numpy;
  *                       its inverse orc_u64_to_deq_scale; hand-derived cases of the rounding mode: ties, carry into the
  *                       exponent, overflow to infinity, subnormal)
@@ -968,79 +972,105 @@ static uint8_t e2m1_code_of(float v)   /* v on the e2m1 grid */
     for (uint8_t i = 0; i < 8; i++) if (kE2M1[i] == a) c = i;
     return (uint8_t)(c | (signbit(v) ? 8u : 0u));
 }
+int orc_dynamic_mx_quant_general(const void* x, int x_dt, int64_t outer, int64_t A, int64_t inner, int64_t block, int scale_alg,
+                                 int round_mode, int y_dt, uint8_t* y, uint8_t* scale_out);
 int orc_dynamic_mx_quant_alg(const void* x, int x_dt, int64_t rows, int64_t cols, int64_t block, int scale_alg, int y_dt, uint8_t* y,
-                             uint8_t* scale_out);
+                             uint8_t* scale_out)
+{
+    if (x_dt != ORC_F16 && x_dt != ORC_BF16) return -1;
+    return orc_dynamic_mx_quant_general(x, x_dt, rows, cols, 1, block, scale_alg, 0, y_dt, y, scale_out);
+}
 int orc_dynamic_mx_quant(const void* x, int x_dt, int64_t rows, int64_t cols, int64_t block, int y_dt, uint8_t* y, uint8_t* scale_out)
 {
     return orc_dynamic_mx_quant_alg(x, x_dt, rows, cols, block, 0, y_dt, y, scale_out);
 }
-/* scale_alg 1 (GD:156-176, fp8 elements only): share_exp is the exponent field of fp32(amax / tmax) minus 127, plus one when that
- * quotient is not a power of two (a normal number with mantissa bits, or a subnormal above 2^-127); the elements follow as before. */
-int orc_dynamic_mx_quant_alg(const void* x, int x_dt, int64_t rows, int64_t cols, int64_t block, int scale_alg, int y_dt, uint8_t* y,
-                             uint8_t* scale_out)
+/* The general form (GD:263-330 with its helpers): x is [outer, A, inner] and the blocks run along A; x in fp16, bf16 or fp32;
+ * elements e2m1, e1m2 (emax 0, emin 0, two mantissa bits, maximum 1.75: the eight magnitudes k/4), e4m3, e5m2;
+ * round_mode (_mx_round_mantissa, GD:181-197, applied to the element's mantissa scaled to an integer): 0 rint (ties to even),
+ * 1 round (ties away from zero: floor(|v| + 0.5) with the sign), 2 floor, 3 ceil, 4 trunc.
+ * scale_alg 1 (GD:156-176, fp8 elements only): share_exp is the exponent field of fp32(amax / tmax) minus 127, plus one when that
+ * quotient is not a power of two (a normal number with mantissa bits, or a subnormal above 2^-127).
+ * y has x's shape, 4-bit codes packed two per byte along the last axis (even flat index in the low nibble);
+ * scale_out is [outer, ceil(nblocks / 2), inner, 2]: the two blocks of a pair side by side (_interleave, GD:235-262), a missing
+ * second block padded with byte 0 (_pad_to_even pads with 2^-127). */
+int orc_dynamic_mx_quant_general(const void* x, int x_dt, int64_t outer, int64_t A, int64_t inner, int64_t block, int scale_alg,
+                                 int round_mode, int y_dt, uint8_t* y, uint8_t* scale_out)
 {
     int emax, emin, mbits; float tmax;
     switch (y_dt) {
         case ORC_E2M1: emax = 2; emin = 0; mbits = 1; tmax = 6.0f; break;
+        case ORC_E1M2: emax = 0; emin = 0; mbits = 2; tmax = 1.75f; break;
         case ORC_E4M3: emax = 8; emin = -6; mbits = 3; tmax = 448.0f; break;
         case ORC_E5M2: emax = 15; emin = -14; mbits = 2; tmax = 57344.0f; break;
         default: return -1;
     }
-    if ((x_dt != ORC_F16 && x_dt != ORC_BF16) || rows <= 0 || cols <= 0 || block <= 0 || (y_dt == ORC_E2M1 && (cols & 1))) return -1;
-    if (scale_alg != 0 && (scale_alg != 1 || y_dt == ORC_E2M1)) return -1;
-    const int64_t nblk = (cols + block - 1) / block, spitch = (nblk + 1) / 2 * 2;
-    for (int64_t r = 0; r < rows; r++) {
-        for (int64_t b = 0; b < spitch; b++) scale_out[r * spitch + b] = 0;
-        for (int64_t b = 0; b < nblk; b++) {
-            const int64_t c1 = (b + 1) * block < cols ? (b + 1) * block : cols;
-            float amax = 0.0f; int has_nan = 0;
-            for (int64_t c = b * block; c < c1; c++) {
-                const float a = fabsf(load_as_f32(x, x_dt, (size_t)(r * cols + c)));
-                if (a != a) has_nan = 1;
-                if (a > amax) amax = a;
-            }
-            float share;   /* an integer, or NaN */
-            if (has_nan) share = NAN;
-            else if (amax == 0.0f) share = -127.0f;
-            else if (scale_alg == 1) {
-                if (isinf(amax)) share = NAN;
+    const int fp4 = y_dt == ORC_E2M1 || y_dt == ORC_E1M2;
+    if ((x_dt != ORC_F16 && x_dt != ORC_BF16 && x_dt != ORC_F32) || outer <= 0 || A <= 0 || inner <= 0 || block <= 0) return -1;
+    if (fp4 && ((outer * A * inner) & 1)) return -1;
+    if (scale_alg != 0 && (scale_alg != 1 || fp4)) return -1;
+    if (round_mode < 0 || round_mode > 4) return -1;
+    const int64_t nblk = (A + block - 1) / block, np = (nblk + 1) / 2;
+    memset(scale_out, 0, (size_t)(outer * np * inner * 2));
+    for (int64_t o = 0; o < outer; o++)
+        for (int64_t in = 0; in < inner; in++)
+            for (int64_t b = 0; b < nblk; b++) {
+                const int64_t a1 = (b + 1) * block < A ? (b + 1) * block : A;
+                float amax = 0.0f; int has_nan = 0;
+                for (int64_t a = b * block; a < a1; a++) {
+                    const float v = fabsf(load_as_f32(x, x_dt, (size_t)((o * A + a) * inner + in)));
+                    if (v != v) has_nan = 1;
+                    if (v > amax) amax = v;
+                }
+                float share;   /* an integer, or NaN */
+                if (has_nan) share = NAN;
+                else if (amax == 0.0f) share = -127.0f;
+                else if (scale_alg == 1) {
+                    if (isinf(amax)) share = NAN;
+                    else {
+                        const uint32_t u = f2u(amax / tmax);
+                        int e = (int)(u >> 23);
+                        const uint32_t mant = u & 0x7fffffu;
+                        if ((e > 0 && e < 254 && mant > 0) || (e == 0 && mant > (1u << 22))) e += 1;
+                        share = (float)(e - 127);
+                    }
+                }
                 else {
-                    const uint32_t u = f2u(amax / tmax);
-                    int e = (int)(u >> 23);
-                    const uint32_t mant = u & 0x7fffffu;
-                    if ((e > 0 && e < 254 && mant > 0) || (e == 0 && mant > (1u << 22))) e += 1;
-                    share = (float)(e - 127);
+                    share = floorf(log2f(amax)) - (float)emax;
+                    if (share > 127.0f) share = NAN;
+                    else if (share < -127.0f) share = -127.0f;
+                }
+                scale_out[((o * np + b / 2) * inner + in) * 2 + (b & 1)] = (share == share) ? (uint8_t)((int)share + 127) : 0xFFu;
+                for (int64_t a = b * block; a < a1; a++) {
+                    const size_t i = (size_t)((o * A + a) * inner + in);
+                    float q = 0.0f;
+                    if (share == share) {
+                        q = load_as_f32(x, x_dt, i) / ldexpf(1.0f, (int)share);
+                        float e = floorf(log2f(fabsf(q) + (q == 0.0f ? 1.0f : 0.0f)));
+                        if (e < (float)emin) e = (float)emin;
+                        const float pe = ldexpf(1.0f, (int)e), pm = ldexpf(1.0f, mbits);
+                        float r = q / pe * pm;
+                        switch (round_mode) {
+                            case 0: r = nearbyintf(r); break;
+                            case 1: { const float t = floorf(fabsf(r) + 0.5f); r = signbit(r) ? -t : t; break; }
+                            case 2: r = floorf(r); break;
+                            case 3: r = ceilf(r); break;
+                            default: r = truncf(r); break;
+                        }
+                        q = r / pm * pe;
+                        if (q > tmax) q = tmax;
+                        if (q < -tmax) q = -tmax;
+                        if (!(q == q)) q = 0.0f;
+                    }
+                    if (y_dt == ORC_E4M3) y[i] = orc_e4m3_from_f32(q);
+                    else if (y_dt == ORC_E5M2) y[i] = orc_e5m2_from_f32(q);
+                    else {
+                        const uint8_t code = y_dt == ORC_E2M1 ? e2m1_code_of(q)
+                                                              : (uint8_t)((uint8_t)(fabsf(q) * 4.0f) | (signbit(q) ? 8u : 0u));
+                        uint8_t* pb = y + (i >> 1);
+                        *pb = (i & 1) ? (uint8_t)((*pb & 0x0fu) | (code << 4)) : (uint8_t)((*pb & 0xf0u) | code);
+                    }
                 }
             }
-            else {
-                share = floorf(log2f(amax)) - (float)emax;
-                if (share > 127.0f) share = NAN;
-                else if (share < -127.0f) share = -127.0f;
-            }
-            scale_out[r * spitch + b] = (share == share) ? (uint8_t)((int)share + 127) : 0xFFu;
-            for (int64_t c = b * block; c < c1; c++) {
-                const size_t i = (size_t)(r * cols + c);
-                float q = 0.0f;
-                if (share == share) {
-                    q = load_as_f32(x, x_dt, i) / ldexpf(1.0f, (int)share);
-                    float e = floorf(log2f(fabsf(q) + (q == 0.0f ? 1.0f : 0.0f)));
-                    if (e < (float)emin) e = (float)emin;
-                    const float pe = ldexpf(1.0f, (int)e), pm = ldexpf(1.0f, mbits);
-                    q = nearbyintf(q / pe * pm) / pm * pe;
-                    if (q > tmax) q = tmax;
-                    if (q < -tmax) q = -tmax;
-                    if (!(q == q)) q = 0.0f;
-                }
-                if (y_dt == ORC_E4M3) y[i] = orc_e4m3_from_f32(q);
-                else if (y_dt == ORC_E5M2) y[i] = orc_e5m2_from_f32(q);
-                else {
-                    const uint8_t code = e2m1_code_of(q);
-                    uint8_t* p = y + (i >> 1);
-                    *p = (i & 1) ? (uint8_t)((*p & 0x0fu) | (code << 4)) : (uint8_t)((*p & 0xf0u) | code);
-                }
-            }
-        }
-    }
     return 0;
 }
 

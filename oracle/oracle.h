@@ -13,7 +13,7 @@ extern "C" {
 
 enum {
     ORC_F32 = 0, ORC_F16 = 1, ORC_I8 = 2, ORC_I32 = 3, ORC_BF16 = 27, ORC_I4 = 29,
-    ORC_E5M2 = 35, ORC_E4M3 = 36, ORC_E8M0 = 37, ORC_E2M1 = 40, ORC_U64 = 10
+    ORC_E5M2 = 35, ORC_E4M3 = 36, ORC_E8M0 = 37, ORC_E2M1 = 40, ORC_E1M2 = 41, ORC_U64 = 10
 };
 
 uint16_t orc_bf16_from_f32(float f);
@@ -75,6 +75,8 @@ int orc_dynamic_mx_quant(const void* x, int x_dt, int64_t rows, int64_t cols, in
 void orc_trans_quant_param(const float* scale, int64_t scale_len, const float* offset, int64_t offset_len, int round_mode, uint64_t* out);
 int orc_dynamic_mx_quant_alg(const void* x, int x_dt, int64_t rows, int64_t cols, int64_t block, int scale_alg, int y_dt, uint8_t* y,
                              uint8_t* scale_out);
+int orc_dynamic_mx_quant_general(const void* x, int x_dt, int64_t outer, int64_t A, int64_t inner, int64_t block, int scale_alg,
+                                 int round_mode, int y_dt, uint8_t* y, uint8_t* scale_out);
 int orc_wqbmm(const void* x, int x_dt, const void* w, int w_dt, int64_t M, int64_t K, int64_t N, int tW,
               const void* scale, int scale_dt, int64_t scale_n, const void* offset, int64_t group,
               const void* bias, int bias_dt, void* y);

@@ -9,7 +9,7 @@ import numpy as np
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 LIB = os.path.join(ROOT, "oracle", "liboracle.so")
 
-F32, F16, I8, I32, BF16, I4, E5M2, E4M3, E8M0, E2M1 = 0, 1, 2, 3, 27, 29, 35, 36, 37, 40
+F32, F16, I8, I32, BF16, I4, E5M2, E4M3, E8M0, E2M1, E1M2 = 0, 1, 2, 3, 27, 29, 35, 36, 37, 40, 41
 U64 = 10
 _lib = None
 
@@ -54,6 +54,8 @@ def lib():
         L.orc_dynamic_mx_quant_alg.restype = C.c_int
         L.orc_dynamic_mx_quant.argtypes = [vp, C.c_int, i64, i64, i64, C.c_int, vp, vp]
         L.orc_dynamic_mx_quant.restype = C.c_int
+        L.orc_dynamic_mx_quant_general.argtypes = [vp, C.c_int, i64, i64, i64, i64, C.c_int, C.c_int, C.c_int, vp, vp]
+        L.orc_dynamic_mx_quant_general.restype = C.c_int
         L.orc_trans_quant_param.argtypes = [vp, i64, vp, i64, C.c_int, vp]
         L.orc_trans_quant_param.restype = None
         L.orc_scale_generate.argtypes = [C.c_float]
@@ -132,6 +134,27 @@ def dynamic_mx_quant(x, x_dt, y_dt, block=32, scale_alg=0):
     y = np.zeros(x.shape[:-1] + ((cols // 2) if y_dt == E2M1 else cols,), np.uint8)
     scale = np.zeros(x.shape[:-1] + ((nblk + 1) // 2, 2), np.uint8)
     rc = lib().orc_dynamic_mx_quant_alg(x.ctypes.data, x_dt, rows, cols, block, scale_alg, y_dt, y.ctypes.data, scale.ctypes.data)
+    assert rc == 0, rc
+    return y, scale
+
+
+ROUND_MODES = {"rint": 0, "round": 1, "floor": 2, "ceil": 3, "trunc": 4}
+
+
+def dynamic_mx_quant_general(x, x_dt, y_dt, axis=-1, block=32, scale_alg=0, round_mode="rint"):
+    """x: uint16 bits (fp16 / bf16) or float32, any shape; blocks along `axis`.  Returns (y bytes with x's shape, the last dim
+    halved for the 4-bit types, e8m0 bytes with x's shape where the axis holds ceil(nblk / 2) and a trailing 2)."""
+    x = np.ascontiguousarray(x, np.float32 if x_dt == F32 else np.uint16)
+    ax = axis % x.ndim
+    A = x.shape[ax]
+    outer = int(np.prod(x.shape[:ax], dtype=np.int64))
+    inner = int(np.prod(x.shape[ax + 1:], dtype=np.int64))
+    nblk = -(-A // block)
+    fp4 = y_dt in (E2M1, E1M2)
+    y = np.zeros(x.shape[:-1] + ((x.shape[-1] // 2) if fp4 else x.shape[-1],), np.uint8)
+    scale = np.zeros(x.shape[:ax] + ((nblk + 1) // 2,) + x.shape[ax + 1:] + (2,), np.uint8)
+    rc = lib().orc_dynamic_mx_quant_general(x.ctypes.data, x_dt, outer, A, inner, block, scale_alg, ROUND_MODES[round_mode], y_dt,
+                                            y.ctypes.data, scale.ctypes.data)
     assert rc == 0, rc
     return y, scale
 

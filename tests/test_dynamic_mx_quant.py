@@ -139,6 +139,92 @@ def _status(m, x, y, sc, **kw):
     return rc
 
 
+# ---- the general form: another axis, fp32 input, e1m2 elements, the other rounding modes
+GRID_E1M2 = np.arange(8) / 4.0
+
+
+def _nearest_on_grid(q, grid, mode):
+    """q float64 inside the grid's range -> index of the grid point that `mode` selects, from the definition of the mode on
+    the explicit list of magnitudes (floor / ceil / trunc: the neighbouring grid point in that direction; rint: nearest, ties to
+    the even mantissa, i.e. the even index; round: nearest, ties away from zero).  Returns signed values."""
+    full = np.concatenate([-grid[:0:-1], grid])   # ascending signed grid
+    out = np.empty_like(q)
+    for i, v in enumerate(q.reshape(-1)):
+        lo = full[full <= v].max(); hi = full[full >= v].min()
+        if mode == "floor": r = lo
+        elif mode == "ceil": r = hi
+        elif mode == "trunc": r = lo if v >= 0 else hi
+        elif lo == hi: r = lo
+        elif v - lo < hi - v: r = lo
+        elif v - lo > hi - v: r = hi
+        elif mode == "round": r = hi if v > 0 else lo
+        else:   # rint: the candidate with an even index in the magnitude grid
+            r = lo if int(np.where(grid == abs(lo))[0][0]) % 2 == 0 else hi
+        out.reshape(-1)[i] = r
+    return out
+
+
+@pytest.mark.parametrize("y_dt,grid", [(orc.E2M1, GRID4), (orc.E1M2, GRID_E1M2)])
+@pytest.mark.parametrize("mode", ["rint", "round", "floor", "ceil", "trunc"])
+def test_round_modes_select_the_grid_point_their_definition_names(y_dt, grid, mode):
+    """One block whose maximum is the format's largest power-of-two binade (share_exp 0, scale byte 127), so q = x: every
+    element must land on the grid point that the mode's definition selects, ties included (multiples of 1/8 hit every tie)."""
+    top = 6.0 if y_dt == orc.E2M1 else 1.75
+    vals = np.concatenate([np.arange(-48, 49) / 8.0 * (top / 6.0), [top, -top, 0.3, -0.3, 0.26, -0.26, 0.74]]).astype(np.float32)
+    vals = vals[np.abs(vals) <= top]
+    for start in range(0, len(vals), 31):
+        blk = np.zeros(32, np.float32)
+        part = vals[start:start + 31]
+        blk[:len(part)] = part
+        blk[31] = top
+        y, sc = orc.dynamic_mx_quant_general(blk, orc.F32, y_dt, round_mode=mode)
+        assert sc.reshape(-1)[0] == 127
+        codes = orc.unpack_nibbles(y)
+        got = np.where(codes & 8, -1.0, 1.0) * grid[codes & 7]
+        want = _nearest_on_grid(blk.astype(np.float64), grid, mode)
+        assert np.array_equal(np.abs(got), np.abs(want)) and np.array_equal(got[want != 0], want[want != 0]), (mode, blk, got, want)
+
+
+def test_e1m2_share_exponent_and_saturation():
+    """e1m2: emax 0, so a block maximum in [2^k, 2^(k+1)) gives scale byte 127 + k; 1.9 * 2^k saturates at code 7 (1.75)."""
+    for k in (-3, 0, 5):
+        blk = np.zeros(32, np.float32); blk[0] = 1.9 * 2.0 ** k; blk[1] = -1.0 * 2.0 ** k; blk[2] = 0.13 * 2.0 ** k
+        y, sc = orc.dynamic_mx_quant_general(blk, orc.F32, orc.E1M2)
+        codes = orc.unpack_nibbles(y)
+        assert sc.reshape(-1)[0] == 127 + k and codes[0] == 7 and codes[1] == (8 | 4) and codes[2] == 1   # 0.13 -> 0.25 (nearest)
+
+
+@pytest.mark.parametrize("y_dt", [orc.E2M1, orc.E4M3])
+def test_another_axis_is_the_last_axis_of_the_transposed_tensor(y_dt):
+    rng = np.random.default_rng(5)
+    x = (rng.normal(0, 1, size=(3, 70, 6)) * 2.0 ** rng.integers(-6, 6, size=(3, 1, 6))).astype(np.float32)
+    xb = orc.f32_to_b16(x, orc.BF16)
+    y, sc = orc.dynamic_mx_quant_general(xb, orc.BF16, y_dt, axis=1)
+    xt = np.ascontiguousarray(xb.transpose(0, 2, 1))                         # [3, 6, 70]
+    yt, sct = orc.dynamic_mx_quant(xt, orc.BF16, y_dt)                       # the pinned last-axis form
+    ct = _codes(yt.reshape(-1), y_dt).reshape(3, 6, 70)
+    assert np.array_equal(_codes(y.reshape(-1), y_dt).reshape(3, 70, 6), ct.transpose(0, 2, 1))
+    assert sc.shape == (3, 2, 6, 2)                                          # 3 blocks of 32 -> 2 pairs; the pair's two bytes last
+    assert np.array_equal(sc.transpose(0, 2, 1, 3).reshape(3, 6, 4), sct.reshape(3, 6, 4))
+    # axis 0 as well, with a block of 64
+    y0, sc0 = orc.dynamic_mx_quant_general(xb, orc.BF16, y_dt, axis=0, block=64)
+    x0 = np.ascontiguousarray(xb.transpose(1, 2, 0))                         # [70, 6, 3]
+    y0t, sc0t = orc.dynamic_mx_quant(np.concatenate([x0, np.zeros((70, 6, 1), np.uint16)], axis=-1) if y_dt == orc.E2M1 else x0, orc.BF16, y_dt, block=64)
+    c0t = _codes(y0t.reshape(-1), y_dt).reshape(70, 6, -1)[..., :3]
+    assert np.array_equal(_codes(y0.reshape(-1), y_dt).reshape(3, 70, 6), c0t.transpose(2, 0, 1))
+    assert np.array_equal(sc0.reshape(70, 6, 2), sc0t.reshape(70, 6, 2))
+
+
+@pytest.mark.parametrize("y_dt", [orc.E2M1, orc.E4M3, orc.E5M2])
+def test_fp32_input_equals_the_16_bit_input_it_came_from(y_dt):
+    rng = np.random.default_rng(8)
+    xf = (rng.normal(0, 1, size=(9, 96)) * 2.0 ** rng.integers(-10, 10, size=(9, 1))).astype(np.float32)
+    xh = orc.f32_to_b16(xf, orc.F16)
+    y16, s16 = orc.dynamic_mx_quant(xh, orc.F16, y_dt)
+    y32, s32 = orc.dynamic_mx_quant_general(orc.b16_to_f32(xh, orc.F16), orc.F32, y_dt)
+    assert np.array_equal(y16, y32) and np.array_equal(s16, s32)
+
+
 def test_status_rules(opsnn):
     """The documented rules (docs/aclnnDynamicMxQuant.md:99-260, 312-320) and its example call (:428-454: axis -1, rint,
     dstType 36, blocksize 32)."""
@@ -164,13 +250,16 @@ def test_status_rules(opsnn):
     assert _status(m, x, y, sc, dst_type_max=0.0) == 0 and _status(m, x, y, sc, dst_type_max=0.0, max_low_bound=0.0) == 0
     assert _status(m, x, y, sc, dst_type_max=6.0) == not_run and _status(m, x, y, sc, dst_type_max=0.0, max_low_bound=1.0) == not_run
     assert _status(m, x, y, sc, dst_type_max=0.0, scale_alg=2) == not_run and _status(m, x, y, sc, dst_type_max=0.0, blocksize=48) == bad
-    # accepted by the reference, no kernel here
-    assert _status(m, x, y, _t(m, (4, 1, 320, 2), e8), axis=1) == not_run
+    # another axis, a FLOAT x, e1m2 elements and the fp4 rounding modes run on the general kernel
+    assert _status(m, x, y, _t(m, (4, 1, 320, 2), e8), axis=1) == 0
     assert _status(m, x, y, _t(m, (4, 6, 3, 2), e8), blocksize=64) == 0
     assert _status(m, x, y, _t(m, (4, 6, 1, 2), e8), blocksize=1024) == 0
-    assert _status(m, _t(m, (4, 6, 320), m.ACL_FLOAT), y, sc) == not_run
-    assert _status(m, x, _t(m, (4, 6, 320), m.ACL_FLOAT4_E1M2), sc) == not_run
-    assert _status(m, x, _t(m, (4, 6, 320), f4), sc, round_mode=b"floor") == not_run
+    assert _status(m, _t(m, (4, 6, 320), m.ACL_FLOAT), y, sc) == 0
+    assert _status(m, _t(m, (4, 6, 320), m.ACL_FLOAT), y, _t(m, (4, 6, 3, 2), e8), blocksize=64) == bad     # FLOAT x: blocks of 32 only
+    assert _status(m, x, _t(m, (4, 6, 320), m.ACL_FLOAT4_E1M2), sc) == 0
+    assert _status(m, x, _t(m, (4, 6, 320), f4), sc, round_mode=b"floor") == 0
+    assert _status(m, x, _t(m, (4, 6, 320), f4), sc, round_mode=b"round") == 0
+    assert _status(m, x, _t(m, (4, 6, 320), f4), sc, round_mode=b"ceil") == bad
     assert _status(m, x, y, sc, scale_alg=1) == 0
 
 
@@ -257,3 +346,65 @@ def test_gpu_block_sizes_and_scale_algorithm_1(gpu, shape, block, alg, y_dt):
     gy, gs = _run(m, xb, orc.BF16, y_dt, block=block, scale_alg=alg)
     assert np.array_equal(gs, want_s), "scale bytes differ"
     assert _same_but_zero_sign(_codes(gy, y_dt), _codes(want_y.reshape(-1), y_dt), y_dt)
+
+
+def _run_general(m, x, x_dt, y_dt, axis, block=32, scale_alg=0, round_mode="rint"):
+    """x: uint16 bits or float32, any shape -> (y bytes flat, scale bytes in the API's shape) from the device."""
+    ax = axis % x.ndim
+    nblk = -(-x.shape[ax] // block)
+    fp4 = y_dt in (orc.E2M1, orc.E1M2)
+    ybytes = x.size // 2 if fp4 else x.size
+    sshape = x.shape[:ax] + ((nblk + 1) // 2,) + x.shape[ax + 1:] + (2,)
+    sbytes = int(np.prod(sshape))
+    d_x, d_y, d_s = m.DeviceBuffer(host=x), m.DeviceBuffer(ybytes + 16), m.DeviceBuffer(sbytes + 16)
+    d_y.fill(0xEE); d_s.fill(0xEE)
+    adt = {orc.F16: m.ACL_FLOAT16, orc.BF16: m.ACL_BF16, orc.F32: m.ACL_FLOAT}[x_dt]
+    ydt = {orc.E2M1: m.ACL_FLOAT4_E2M1, orc.E1M2: m.ACL_FLOAT4_E1M2, orc.E4M3: m.ACL_FLOAT8_E4M3FN, orc.E5M2: m.ACL_FLOAT8_E5M2}[y_dt]
+    m.dynamic_mx_quant(m.Tensor(x.shape, adt, d_x), m.Tensor(x.shape, ydt, d_y), m.Tensor(sshape, m.ACL_FLOAT8_E8M0, d_s),
+                       axis=axis, blocksize=block, scale_alg=scale_alg, round_mode=round_mode.encode())
+    m.check(m.lib().aclrtSynchronizeDevice(), "sync")
+    gy, gs = d_y.to_host(np.uint8, (ybytes + 16,)), d_s.to_host(np.uint8, (sbytes + 16,))
+    assert (gy[ybytes:] == 0xEE).all() and (gs[sbytes:] == 0xEE).all(), "wrote past an output"
+    return gy[:ybytes], gs[:sbytes].reshape(sshape)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("shape,axis,x_dt,y_dt,block,alg,mode", [
+    ((3, 70, 6), 1, orc.BF16, orc.E2M1, 32, 0, "rint"),        # a middle axis, three blocks (one pair and a half), fp4 pairs along the last axis
+    ((100, 40), 0, orc.F16, orc.E4M3, 32, 0, "rint"),          # the first axis
+    ((100, 40), 0, orc.BF16, orc.E5M2, 64, 1, "rint"),         # larger blocks and the second scale algorithm on another axis
+    ((2, 96, 4, 10), -3, orc.BF16, orc.E2M1, 32, 0, "floor"),
+    ((5, 320), -1, orc.F32, orc.E4M3, 32, 0, "rint"),          # FLOAT x
+    ((5, 320), -1, orc.F32, orc.E2M1, 32, 0, "round"),
+    ((7, 40), -1, orc.BF16, orc.E1M2, 32, 0, "rint"),          # e1m2 elements, a ragged last block
+    ((7, 40), -1, orc.F16, orc.E1M2, 32, 0, "floor"),
+    ((6, 1000), -1, orc.BF16, orc.E2M1, 32, 0, "floor"),       # the rounding modes of the 4-bit types on the last axis
+    ((6, 1000), -1, orc.F16, orc.E2M1, 128, 0, "round"),
+    ((64, 33, 2), 0, orc.F32, orc.E1M2, 32, 0, "round"),
+])
+def test_gpu_general_form_is_bit_identical(gpu, shape, axis, x_dt, y_dt, block, alg, mode):
+    """Blocks along another axis, fp32 input, e1m2 elements and the floor / round modes (the one-thread-per-block kernel)
+    against the oracle, scale bytes and element codes (the sign of a zero aside).  fp32 inputs keep 12 mantissa bits, away
+    from the values just below a power of two where numpy's float32 log2 rounds up to the next integer."""
+    m = gpu
+    print(f"case mx quant general {shape} axis={axis} x={x_dt} y={y_dt} block={block} alg={alg} mode={mode}", flush=True)
+    rng = np.random.default_rng(sum(shape) + y_dt + block)
+    ax = axis % len(shape)
+    sc_shape = tuple(1 if i == ax else d for i, d in enumerate(shape))
+    xf = (rng.normal(0, 1, size=shape) * 2.0 ** rng.integers(-14, 14, size=sc_shape)).astype(np.float32)
+    flat = xf.reshape(-1)
+    flat[:min(40, flat.size // 4)] = 0.0
+    flat[-1] = np.inf
+    flat[flat.size // 2] = np.nan
+    if x_dt == orc.F32:
+        x = (xf.view(np.uint32) & np.uint32(0xFFFFF800)).view(np.float32)
+    else:
+        x = orc.f32_to_b16(xf, x_dt)
+    want_y, want_s = orc.dynamic_mx_quant_general(x, x_dt, y_dt, axis=axis, block=block, scale_alg=alg, round_mode=mode)
+    gy, gs = _run_general(m, x, x_dt, y_dt, axis, block, alg, mode)
+    assert np.array_equal(gs, want_s), "scale bytes differ"
+    fp4 = y_dt in (orc.E2M1, orc.E1M2)
+    a, b = (orc.unpack_nibbles(gy), orc.unpack_nibbles(want_y.reshape(-1))) if fp4 else (gy, want_y.reshape(-1))
+    mag = 0x7 if fp4 else 0x7f
+    z = ((a | b) & mag) == 0
+    assert np.array_equal(a[~z], b[~z]), f"{int((a[~z] != b[~z]).sum())} element codes differ"
