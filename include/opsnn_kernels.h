@@ -110,6 +110,22 @@ OPSNN_API int opsnnGetFp8Fast(void);
 OPSNN_API void opsnnSetForcePlain(int on);
 OPSNN_API void opsnnSetMx8Wide(int n);
 OPSNN_API void opsnnSetWqTileMin(int m);
+/* Opt-in cache of re-laid-out right operands.  The matrix-core kernels stream a K-contiguous right operand; x2 / weight
+ * stored [K, N] with N contiguous is re-laid out inside every call (into the caller's workspace) unless this cache is on:
+ * then opsnnQmmInt8, opsnnQmmBlockScale and opsnnWqmm keep the K-contiguous copy in device memory of the library's own, keyed
+ * by the operand's address, shape, element width and batch count, and later calls with the same operand skip the pass
+ * (the workspace is then not touched).  It has no counterpart among the reference's entry points: the reference folds the
+ * re-layout into its graphs offline (weight_quant_batch_matmul_v2_transpose_fusion_pass.cpp,
+ * quant_batch_matmul_v4_transpose_fusion_pass.cpp).
+ *   opsnnSetWeightCache(max_bytes)  0 switches the cache off and frees it (the default; OPSNN_WEIGHT_CACHE_MB sets the
+ *                                   initial limit); entries are evicted least recently used first;
+ *   opsnnWeightCacheClear()         frees every entry.  The cache cannot see a weight change: call this before
+ *                                   overwriting, freeing or re-using the memory of an operand that may be cached;
+ *   opsnnWeightCacheStats(...)      entries, bytes held, hits and misses so far (any pointer may be NULL).
+ * Calls made while their stream is being captured into a graph bypass the cache. */
+OPSNN_API void opsnnSetWeightCache(int64_t max_bytes);
+OPSNN_API void opsnnWeightCacheClear(void);
+OPSNN_API void opsnnWeightCacheStats(int64_t* entries, int64_t* bytes, int64_t* hits, int64_t* misses);
 /* MX: fp4/fp8 operands, e8m0 scale per 32 K. out = (x1*s1) @ (x2*s2) + fp32 bias. */
 OPSNN_API int opsnnQmmMx(const OpsnnQmmArgs* a, void* stream);
 /* Per-tensor / per-channel scales (T-T, T-C): int8 or fp8 (e4m3, e5m2) operands;

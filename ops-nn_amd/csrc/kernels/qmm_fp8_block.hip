@@ -26,6 +26,7 @@
 #include "qgemm_core.hip.h"
 
 namespace opsnn {
+const void* weight_cache_get(const void* src, int64_t K, int64_t N, int bits, int64_t nb, hipStream_t st);   // weight_cache.hip
 
 struct Fp8BlkParams {
     const int8_t* a;
@@ -631,12 +632,17 @@ int launch_blockscale_mfma(const OpsnnQmmArgs& a0, hipStream_t st)
     if (a.K % 128 != 0 || a.M * a.N < 64 * 64 || a.x1.col_stride != 1) return OPSNN_NOT_TAKEN;
     if (a.x2.row_stride != 1) {
         // x2 is [K, N] with N contiguous: re-lay it out K-contiguous in the workspace (scales keep their layout)
-        if (!a.workspace || a.x2.col_stride != 1 || a.x2.row_stride != a.N) return OPSNN_NOT_TAKEN;
+        if (a.x2.col_stride != 1 || a.x2.row_stride != a.N) return OPSNN_NOT_TAKEN;
         if (a.x2.batch_stride != 0 && a.x2.batch_stride != a.K * a.N) return OPSNN_NOT_TAKEN;
         const int64_t nb = a.x2.batch_stride == 0 ? 1 : a.batch;
-        int rc = opsnnTranspose8(a.x2.ptr, a.workspace, a.K, a.N, nb, st);
-        if (rc != 0) return rc;
-        a.x2.ptr = a.workspace; a.x2.row_stride = 1; a.x2.col_stride = a.K;
+        if (const void* cached = weight_cache_get(a.x2.ptr, a.K, a.N, 8, nb, st)) a.x2.ptr = cached;   // the weight cache, when on
+        else {
+            if (!a.workspace) return OPSNN_NOT_TAKEN;
+            int rc = opsnnTranspose8(a.x2.ptr, a.workspace, a.K, a.N, nb, st);
+            if (rc != 0) return rc;
+            a.x2.ptr = a.workspace;
+        }
+        a.x2.row_stride = 1; a.x2.col_stride = a.K;
     }
     if (!i8 && !opsnnGetFp8Fast()) {   // exact products and sums unless the caller asked for the 8-bit matrix instruction
         const int rc = launch_blockscale_exact(a, st);

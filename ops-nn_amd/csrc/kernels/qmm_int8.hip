@@ -17,6 +17,7 @@
 #include "qgemm_core.hip.h"
 
 namespace opsnn {
+const void* weight_cache_get(const void* src, int64_t K, int64_t N, int bits, int64_t nb, hipStream_t st);   // weight_cache.hip
 
 struct QmmI8Params {
     const int8_t* a;  // x1
@@ -130,12 +131,18 @@ extern "C" int opsnn_qmm_int8_impl(const OpsnnQmmArgs* a, void* stream)
     }
     bool want_fast = b16 && a_kmajor && variant != OPSNN_VARIANT_PLAIN && p.M * p.N >= 64 * 64 && (p.K % 16) == 0 &&
                      (p.a_rs % 16) == 0 && ((uintptr_t)p.a % 16) == 0 && (p.a_bs % 16) == 0;
-    if (want_fast && !b_kmajor && p.b_cs == 1 && a->workspace && p.b_rs == p.N && (p.b_bs == 0 || p.b_bs == p.K * p.N)) {
+    if (want_fast && !b_kmajor && p.b_cs == 1 && p.b_rs == p.N && (p.b_bs == 0 || p.b_bs == p.K * p.N)) {
         int64_t nb = p.b_bs == 0 ? 1 : a->batch;
-        int rc = opsnnTranspose8(p.b, a->workspace, p.K, p.N, nb, stream);
-        if (rc != 0) return rc;
-        p.b = (const int8_t*)a->workspace; p.b_rs = 1; p.b_cs = p.K; p.b_bs = p.b_bs == 0 ? 0 : p.K * p.N;
-        b_kmajor = true;
+        const void* copy = weight_cache_get(p.b, p.K, p.N, 8, nb, st);   // the weight cache, when it is switched on
+        if (!copy && a->workspace) {
+            int rc = opsnnTranspose8(p.b, a->workspace, p.K, p.N, nb, stream);
+            if (rc != 0) return rc;
+            copy = a->workspace;
+        }
+        if (copy) {
+            p.b = (const int8_t*)copy; p.b_rs = 1; p.b_cs = p.K; p.b_bs = p.b_bs == 0 ? 0 : p.K * p.N;
+            b_kmajor = true;
+        }
     }
     bool fast = want_fast && b_kmajor && (p.b_cs % 16) == 0 && ((uintptr_t)p.b % 16) == 0 && (p.b_bs % 16) == 0;
     if (fast) {

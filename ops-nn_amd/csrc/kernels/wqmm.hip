@@ -345,6 +345,7 @@ static bool stream_eligible(WqParams& p, WqStreamOpts& o)
     return true;
 }
 
+const void* weight_cache_get(const void* src, int64_t K, int64_t N, int bits, int64_t nb, hipStream_t st);   // weight_cache.hip
 template <int XDT, int WBITS>
 int launch_wq_tile(const WqParams& p, hipStream_t st);   // wqmm_tile.hip
 }  // namespace opsnn
@@ -426,11 +427,17 @@ int launch_wqmm_mfma(const OpsnnWqmmArgs& a0, hipStream_t st)
     const int64_t group = a.group > 0 ? a.group : a.K;
     if (group % kpl != 0) return OPSNN_NOT_TAKEN;   // a lane's piece must lie inside one group
     if (a.w.row_stride != 1) {
-        // weight is [K, N] with N contiguous: re-lay it out K-contiguous in the workspace
-        if (!a.workspace || a.w.col_stride != 1 || a.w.row_stride != a.N || a.K == 1) return OPSNN_NOT_TAKEN;
-        int rc = wbits == 4 ? opsnnTranspose4(a.w.ptr, a.workspace, a.K, a.N, 1, st) : opsnnTranspose8(a.w.ptr, a.workspace, a.K, a.N, 1, st);
-        if (rc != 0) return rc;
-        a.w.ptr = a.workspace; a.w.row_stride = 1; a.w.col_stride = a.K;
+        // weight is [K, N] with N contiguous: the K-contiguous copy comes from the weight cache when that is switched on,
+        // else it is re-laid out into the workspace
+        if (a.w.col_stride != 1 || a.w.row_stride != a.N || a.K == 1) return OPSNN_NOT_TAKEN;
+        if (const void* cached = weight_cache_get(a.w.ptr, a.K, a.N, wbits, 1, st)) a.w.ptr = cached;
+        else {
+            if (!a.workspace) return OPSNN_NOT_TAKEN;
+            int rc = wbits == 4 ? opsnnTranspose4(a.w.ptr, a.workspace, a.K, a.N, 1, st) : opsnnTranspose8(a.w.ptr, a.workspace, a.K, a.N, 1, st);
+            if (rc != 0) return rc;
+            a.w.ptr = a.workspace;
+        }
+        a.w.row_stride = 1; a.w.col_stride = a.K;
     }
     WqParams p{};
     p.x = (const uint16_t*)a.x;

@@ -183,6 +183,9 @@ _SIGS = {
     "aclnnTransQuantParamV3": (C.c_int32, [C.c_void_p, C.c_uint64, C.c_void_p, C.c_void_p]),
     "opsnnTransQuantParam": (C.c_int, [C.c_void_p, C.c_int64, C.c_void_p, C.c_int64, C.c_int, C.c_void_p, C.c_void_p]),
     "opsnnPackB4": (C.c_int, [C.c_void_p, C.c_int, C.c_void_p, C.c_int64, C.c_void_p]),
+    "opsnnSetWeightCache": (None, [C.c_int64]),
+    "opsnnWeightCacheClear": (None, []),
+    "opsnnWeightCacheStats": (None, [C.POINTER(C.c_int64), C.POINTER(C.c_int64), C.POINTER(C.c_int64), C.POINTER(C.c_int64)]),
     "opsnnQmmInt8": (C.c_int, [C.POINTER(OpsnnQmmArgs), C.c_void_p]),
     "opsnnQmmInt8Static": (C.c_int, [C.POINTER(OpsnnQmmArgs), C.c_void_p]),
     "opsnnQmmBlockScale": (C.c_int, [C.POINTER(OpsnnQmmArgs), C.c_void_p]),
@@ -260,6 +263,13 @@ class DeviceBuffer:
 
     def fill(self, byte):
         check(lib().aclrtMemset(self.ptr, self.nbytes, byte, self.nbytes), "aclrtMemset")
+
+    def upload(self, host):
+        """Overwrite the allocation's first bytes with a numpy array's."""
+        host = np.ascontiguousarray(host)
+        assert host.nbytes <= self.nbytes, (host.nbytes, self.nbytes)
+        if host.nbytes:
+            check(lib().aclrtMemcpy(self.ptr, host.nbytes, host.ctypes.data, host.nbytes, H2D), "aclrtMemcpy H2D")
 
     def free(self):
         if self.ptr:

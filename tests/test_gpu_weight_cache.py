@@ -1,0 +1,100 @@
+"""The opt-in cache of re-laid-out right operands (opsnnSetWeightCache): an N-contiguous weight / x2 is re-laid out once, later
+calls with the same operand find the K-contiguous copy; results are those of the uncached path."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+import cases
+import oracle_api as orc
+
+pytestmark = pytest.mark.gpu
+
+
+def _stats(m):
+    v = [C.c_int64(0) for _ in range(4)]
+    m.lib().opsnnWeightCacheStats(*[C.byref(x) for x in v])
+    return tuple(x.value for x in v)   # entries, bytes, hits, misses
+
+
+@pytest.fixture
+def cache(gpu):
+    m = gpu
+    m.lib().opsnnSetWeightCache(256 << 20)
+    try:
+        yield m
+    finally:
+        m.lib().opsnnSetWeightCache(0)
+
+
+def _wq_call(m, inp, d, d_y, M, K, N):
+    group = inp["group"]
+    G = K // group
+    x = m.Tensor((M, K), inp["x_dt"], d["x"])
+    w = m.Tensor((K, N), inp["w_dt"], d["w"])                       # [K, N] storage, N contiguous
+    sc = m.Tensor((G, N), inp["x_dt"], d["scale"])
+    off = m.Tensor((G, N), inp["x_dt"], d["offset"])
+    y = m.Tensor((M, N), inp["x_dt"], d_y)
+    ws = m.weight_quant_batch_matmul(x, w, sc, y, offset=off, group_size=group)
+    m.check(m.lib().aclrtSynchronizeDevice(), "sync")
+    del ws
+    return d_y.to_host(np.uint16, (M, N))
+
+
+def test_weight_only_weight_is_re_laid_out_once(cache):
+    m = cache
+    M, K, N = 16, 1024, 512
+    print(f"case weight cache, weight-only int4 {M}x{K}x{N}", flush=True)
+    inp = cases.make_wq_inputs(m, M, K, N, 3, m.ACL_FLOAT16, m.ACL_INT4, 128, False, True, None)
+    want = cases.oracle_wq(m, inp, M, K, N)
+    d = {k: m.DeviceBuffer(host=v) for k, v in inp.items() if isinstance(v, np.ndarray)}
+    d_y = m.DeviceBuffer(M * N * 2)
+    e0, _, h0, m0 = _stats(m)
+    first = _wq_call(m, inp, d, d_y, M, K, N)
+    second = _wq_call(m, inp, d, d_y, M, K, N)
+    third = _wq_call(m, inp, d, d_y, M, K, N)
+    e1, b1, h1, m1 = _stats(m)
+    assert (e1 - e0, m1 - m0, h1 - h0) == (1, 1, 2) and b1 >= K * N // 2
+    assert np.array_equal(first, second) and np.array_equal(first, third)
+    g, w = orc.b16_to_f32(first, orc.F16), orc.b16_to_f32(want, orc.F16)
+    mx, mean = orc.rel_err_stats(g, w)
+    assert mx <= 2.0 ** -7 and mean <= 2.0 ** -10
+    # a new weight in the same memory: the caller clears the cache, and the next call re-lays the new bytes out
+    inp2 = cases.make_wq_inputs(m, M, K, N, 4, m.ACL_FLOAT16, m.ACL_INT4, 128, False, True, None)
+    m.lib().opsnnWeightCacheClear()
+    assert _stats(m)[0] == 0
+    d["w"].upload(inp2["w"])
+    inp2 = dict(inp2, x=inp["x"], scale=inp["scale"], offset=inp["offset"])
+    got2 = _wq_call(m, inp2, d, d_y, M, K, N)
+    want2 = cases.oracle_wq(m, inp2, M, K, N)
+    mx, mean = orc.rel_err_stats(orc.b16_to_f32(got2, orc.F16), orc.b16_to_f32(want2, orc.F16))
+    assert mx <= 2.0 ** -7 and mean <= 2.0 ** -10
+    assert not np.array_equal(got2, first)
+
+
+def test_int8_x2_is_re_laid_out_once_and_the_limit_evicts(cache):
+    m = cache
+    M, K, N = 128, 512, 384
+    print(f"case weight cache, int8 {M}x{K}x{N}", flush=True)
+    inp = cases.make_qmm_int8_inputs(m, M, K, N, 5, m.ACL_BF16, False)
+    want, _ = cases.oracle_qmm_int8(m, inp, M, K, N, False, m.ACL_BF16)
+    d = {k: m.DeviceBuffer(host=v) for k, v in inp.items() if isinstance(v, np.ndarray)}
+    d_out = m.DeviceBuffer(M * N * 2)
+    a = cases.qmm_args_int8(m, d, M, K, N, 1, False, d_out.ptr, m.ACL_BF16, inp["s2_dtype"], N, inp["bias_dtype"])
+    e0, _, h0, m0 = _stats(m)
+    outs = []
+    for _ in range(3):                      # no workspace at all: only the cache can serve the matrix-core kernel
+        d_out.fill(0xFF)
+        assert m.lib().opsnnQmmInt8(a, None) == 0
+        m.check(m.lib().aclrtSynchronizeDevice(), "sync")
+        outs.append(d_out.to_host(np.uint16, (1, M, N)))
+    e1, _, h1, m1 = _stats(m)
+    assert (e1 - e0, m1 - m0, h1 - h0) == (1, 1, 2)
+    assert all(np.array_equal(o, want) for o in outs)
+    # a limit below the entry's size evicts it; with the cache off the same call (still no workspace) takes the plain kernel
+    m.lib().opsnnSetWeightCache(1024)
+    assert _stats(m)[0] == 0
+    d_out.fill(0xFF)
+    assert m.lib().opsnnQmmInt8(a, None) == 0
+    m.check(m.lib().aclrtSynchronizeDevice(), "sync")
+    assert np.array_equal(d_out.to_host(np.uint16, (1, M, N)), want) and _stats(m)[0] == 0
