@@ -314,6 +314,23 @@ def test_weight_only_x_in_registers_kernel(gpu, M, K, N, x_dt, w_dt, group, tW, 
     check_close(got, want, dt[x_dt], "weight-only, x in registers")
 
 
+@pytest.mark.parametrize("M,K,N,x_dt,w_dt,tW,off,bias", [
+    (16, 4096, 256, "f16", "i8", True, True, None),        # one scale and offset for the whole tensor, 16 waves x 4 chunks
+    (9, 8192, 100, "f16", "i4", True, True, "f16"),        # ragged columns, per tensor, a bias
+    (6, 2048, 72, "bf16", "i8", True, True, "f32"),        # fp32 bias (bf16 activations only), 8 waves x 4 chunks
+    (4, 4096, 48, "bf16", "i8", False, False, "bf16"),     # N-contiguous weight (re-laid out first), three row blocks
+])
+def test_weight_only_x_in_registers_per_tensor_scale_and_fp32_bias(gpu, M, K, N, x_dt, w_dt, tW, off, bias):
+    m = gpu
+    dt = {"bf16": m.ACL_BF16, "f16": m.ACL_FLOAT16, "f32": m.ACL_FLOAT, "i8": m.ACL_INT8, "i4": m.ACL_INT4, None: None}
+    print(f"case wq x-in-registers per-tensor M={M} K={K} N={N} x={x_dt} w={w_dt} tW={tW} off={off} bias={bias}", flush=True)
+    inp = cases.make_wq_inputs(m, M, K, N, M + N, dt[x_dt], dt[w_dt], 0, tW, off, dt[bias], per_tensor=True)
+    want = cases.oracle_wq(m, inp, M, K, N)
+    plain(False)
+    got = cases.run_wq_aclnn(m, inp, M, K, N)
+    check_close(got, want, dt[x_dt], "weight-only, x in registers, per tensor")
+
+
 def test_weight_only_v3_and_per_tensor(gpu):
     m = gpu
     inp = cases.make_wq_inputs(m, 8, 256, 128, 2, m.ACL_FLOAT16, m.ACL_INT8, 0, False, True, None, per_tensor=True)
