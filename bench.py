@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the quantized-matmul hot path on one MI355X.
 
-  python bench.py [--gpus 1] [--steps K] [--warmup W] [--config 1..9] [--m M] [--cold] [--fp8-fast] [--no-cpu] [--calib-copy]
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--config 1..9] [--m M] [--cold] [--fp8-fast] [--no-cpu] [--calib-copy] [--layout packed|nd] [--weight-cache MB]
 
 A step is one pass of the operator (both aclnn phases) over one batch of synthetic, seeded input that is already
 resident in HBM.  One JSON line is printed.
@@ -9,7 +9,8 @@ resident in HBM.  One JSON line is printed.
 Without --config the headline record is BASELINE config 2 (aclnnQuantMatmulV5, int8 per-token x per-channel, M=2048
 K=4096 N=11008, bf16 bias and output), timed with exactly --steps steps after --warmup, and "configs" holds one record
 for every BASELINE config -- 1 (warm and cold), 2, 3 with M = 1, 16, 64, 256 (each warm and cold), 4 (the default exact
-arithmetic and the opt-in 8-bit matrix instruction), 5 -- each with its own roofline record (algorithmic work / HIP-event
+arithmetic and the opt-in 8-bit matrix instruction), 5, and configs 2 and 3 (16 rows) once more with the right operand in
+the literal [K, N] storage and the library's weight cache on -- each with its own roofline record (algorithmic work / HIP-event
 time measured here on the launch stream) and CPU baseline (the C oracle on a bounded sample of the same workload, on this
 host's cores).  "cold" rotates through weight copies larger than the 256 MB last-level cache, so the weight really comes
 from HBM; "warm" re-reads one copy.  With --config N only that workload runs (what the rocprofv3 commands in profiles/ use).
@@ -101,6 +102,9 @@ def main():
                     help="also run, three times each before the timed loop, a byte transpose of an 8192x8192 matrix (64 MiB read, "
                          "64 MiB written) and the 4-bit pack of 16 Mi carriers (64 MiB read in 16-byte pieces per lane, 8 MiB "
                          "written): the known-size kernels that hardware traffic counters are scaled by")
+    ap.add_argument("--weight-cache", type=int, default=0, metavar="MB",
+                    help="switch on the library's cache of re-laid-out right operands with this limit (only matters with --layout nd: "
+                         "the first call re-lays the operand out, the timed ones find the copy)")
     ap.add_argument("--layout", default="packed", choices=["packed", "nd"],
                     help="packed: right operand K-contiguous (offline pre-pack, [N,K] storage); nd: [K,N] storage, "
                          "re-laid out inside every call")
@@ -119,10 +123,14 @@ def main():
     m.check(m.lib().aclrtSetDevice(0), "aclrtSetDevice")
     stream = m.Stream()
     with_cpu = not args.no_cpu
+    if args.weight_cache:
+        m.lib().opsnnSetWeightCache(args.weight_cache << 20)
 
     def top(rec):
         rec.update({"n_gpus": 1, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "data": "synthetic",
                     "device": m.device_info()})
+        if args.weight_cache:
+            rec["config"]["weight_cache_MB"] = args.weight_cache
         return rec
 
     if args.config:
@@ -176,6 +184,24 @@ def main():
     wl = bench_cases.make_workload(m, 5, args)
     sub(wl, (5, None), 6, 2)
     del wl
+    # the literal [K, N] storage of the reference's callers with the library's weight cache on: the re-layout is paid by the
+    # first (warm-up) call, the timed calls find the K-contiguous copy (configs 2 and 3; cold rotation would only measure
+    # the cache's eviction, so warm only)
+    if args.layout == "packed":
+        args.layout = "nd"
+        m.lib().opsnnSetWeightCache(1024 << 20)
+        wl = bench_cases.make_workload(m, 2, args)
+        sub(wl, (2, None), 30, 6)
+        records[-1]["config"].update({"weight_cache_MB": 1024, "x2_layout": "N-contiguous, the literal [K, N] storage (re-laid out once: weight cache)"})
+        del wl
+        wq = bench_cases.ConfigWQ(m, args, 3, max_m=16)
+        wq.set_cold(False)
+        wq.set_m(16)
+        sub(wq, (3, 16), 30, 6)
+        records[-1]["config"].update({"weight_cache_MB": 1024, "weight_layout": "N-contiguous, the literal [K, N] storage (re-laid out once: weight cache)"})
+        del wq
+        m.lib().opsnnSetWeightCache(0)
+        args.layout = "packed"
     head["configs"] = records
     print(json.dumps(top(head)))
 
