@@ -778,8 +778,9 @@ __global__ __launch_bounds__(NW * 64) void wqmm_xreg_kernel(WqParams p)
     static_assert(NW == 8 || NW == 16, "one or two workgroup halves per SIMD pair");
     static_assert(NX <= (NW == 16 ? 16 : 32), "x fragments must fit the register file beside the weight stream");
     static_assert(NCH % 4 == 0 && NCH >= PF, "whole groups of four chunks");
-    constexpr int NU = NX / 4, HU = NU / 2;   // 256-byte units of x per wave, and per staging half
-    static_assert(NU % 2 == 0 && HU * 4096 >= 2048, "two staging halves that also hold the partial sums");
+    // 256-byte units of x per wave; the staging takes them in one round when all waves' units fit 128 KB of LDS, else in two
+    constexpr int NU = NX / 4, NR = NW * NU * 4096 <= 128 * 1024 ? 1 : 2, HU = NU / NR;
+    static_assert(NU % NR == 0 && HU * 4096 >= 2048, "whole staging rounds that also hold the partial sums");
     extern __shared__ __attribute__((aligned(16))) char dyn[];
 
     const int tid = threadIdx.x, lane = tid & 63;
@@ -852,7 +853,7 @@ __global__ __launch_bounds__(NW * 64) void wqmm_xreg_kernel(WqParams p)
     // global memory that is 64 lanes x 16 bytes out of 32 different cache lines per instruction; instead the wave's K
     // range travels through LDS once, in units of 16 rows x 256 bytes: four 16-byte asynchronous copies per unit, each
     // fetching four rows x 256 contiguous bytes, land the 16-byte segment `seg` of row m at position seg ^ m of the
-    // row (conflict free for the 16-byte reads below), half of the range at a time (the whole of x would not fit).
+    // row (conflict free for the 16-byte reads below), half of the range at a time where the whole of x would not fit.
     // Rows that x does not have repeat its last row: they only feed output rows that are never stored.
     v4i xr[NX];
     {
@@ -860,7 +861,7 @@ __global__ __launch_bounds__(NW * 64) void wqmm_xreg_kernel(WqParams p)
         const int cm = lane >> 4, cp = lane & 15;
         const uint16_t* xw = p.x + p.m_base * p.K + (int64_t)wave * (NU * 128);
 #pragma unroll
-        for (int r = 0; r < 2; r++) {
+        for (int r = 0; r < NR; r++) {
 #pragma unroll
             for (int ul = 0; ul < HU; ul++) {
 #pragma unroll
@@ -1007,7 +1008,8 @@ static int launch_xreg_one(const WqParams& p, hipStream_t st)
     const int64_t nblocks = (p.N + 15) / 16;
     const int64_t g = (int64_t)resx_grid(1ll << 40) / 2;
     constexpr int STEPS = (4 * (128 / WBITS)) / 32;
-    constexpr int lds = NW * (NCH * STEPS / 8) * 4096;   // half of the K range of every wave: 16 rows x 256 bytes per unit
+    constexpr int NU = NCH * STEPS / 4;                  // units of 16 rows x 256 bytes per wave
+    constexpr int lds = NW * NU * 4096 <= 128 * 1024 ? NW * NU * 4096 : NW * (NU / 2) * 4096;   // all of x, or half of it at a time
     auto k = wqmm_xreg_kernel<XDT, WBITS, NW, NCH, HAS_OFF, SCM, WFLT>;
     static bool attr_set = false;
     if (!attr_set) {

@@ -16,8 +16,8 @@ import oracle_api as orc
 # bench.py does not measure it; it copies the figure and names the file.  A figure below the algorithmic bytes would not
 # be evidence and is reported as null.  Keyed by (config, M of the weight-only configs, variant).
 PROFILED_TRAFFIC = {
-    (1, None, "warm"): (20.9e6, "profiles/wqmm_decode_w8a16_m16_k4096_n4096.txt"),
-    (1, None, "cold"): (20.8e6, "profiles/wqmm_decode_w8a16_m16_k4096_n4096_cold.txt"),
+    (1, None, "warm"): (20.7e6, "profiles/wqmm_decode_w8a16_m16_k4096_n4096.txt"),
+    (1, None, "cold"): (20.7e6, "profiles/wqmm_decode_w8a16_m16_k4096_n4096_cold.txt"),
     (2, None, None): (162.2e6, "profiles/qgemm_int8_w8a8_m2048_k4096_n11008.txt"),
     (3, 1, "warm"): (144.0e6, "profiles/wqmm_decode_w4a16_m1_k8192_n28672.txt"),
     (3, 1, "cold"): (140.9e6, "profiles/wqmm_decode_w4a16_m1_k8192_n28672_cold.txt"),
