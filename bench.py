@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the quantized-matmul hot path on one MI355X.
 
-  python bench.py [--gpus 1] [--steps K] [--warmup W] [--config 1..9] [--m M] [--cold] [--fp8-fast] [--no-cpu] [--calib-copy] [--layout packed|nd] [--weight-cache MB]
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--config 1..11] [--m M] [--cold] [--fp8-fast] [--no-cpu] [--calib-copy] [--layout packed|nd] [--weight-cache MB]
 
 A step is one pass of the operator (both aclnn phases) over one batch of synthetic, seeded input that is already
 resident in HBM.  One JSON line is printed.
@@ -91,7 +91,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--config", type=int, default=0,
                     help="0 (default): every BASELINE config, headline config 2; 1-5: that BASELINE config only; 6-9: the "
-                         "pre-pack / quantizer operators that prepare their tensors")
+                         "pre-pack / quantizer operators that prepare their tensors; 10: the int4 x int4 K-G mode at 4096^3; "
+                         "11: config 3's shape with mxfp4 weights")
     ap.add_argument("--m", type=int, default=None, help="M for config 3 (1, 16, 64 or 256)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--int8-range", type=int, default=None,
@@ -135,7 +136,7 @@ def main():
 
     if args.config:
         wl = bench_cases.make_workload(m, args.config, args)
-        wl.key = (args.config, (args.m or 16) if args.config == 3 else None)
+        wl.key = (args.config, (args.m or 16) if args.config in (3, 11) else None)
         if args.calib_copy:
             src, dst = m.DeviceBuffer(8192 * 8192), m.DeviceBuffer(8192 * 8192)
             src.fill(1)

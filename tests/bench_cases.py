@@ -30,6 +30,8 @@ PROFILED_TRAFFIC = {
     (4, None, "exact"): (1220.2e6, "profiles/qmm_fp8_exact_m4096_k7168_n18432.txt"),
     (4, None, "fast"): (1502.4e6, "profiles/qmm_fp8_block_m4096_k7168_n18432.txt"),
     (5, None, None): (3083.5e6, "profiles/qgemm_mxfp4_b8_m4096_k8192_n8192.txt"),
+    (10, None, None): (280.7e6, "profiles/qmm_i4_kg_m4096_k4096_n4096.txt"),
+    (11, 16, "warm"): (133.6e6, "profiles/wqmm_decode_mxfp4_m16_k8192_n28672.txt"),
 }
 
 
@@ -254,6 +256,10 @@ class ConfigWQ(Workload):
             M, K, N, x_dt, w_dt, group, off = 16, 4096, 4096, m.ACL_BF16, m.ACL_INT8, 0, False
             self.dtype, lo, hi = "bf16 (int8 weights)", 1e-4, 0.06
             self.name = "config1: aclnnWeightQuantBatchMatmulV2 W8A16 per-channel bf16"
+        elif config == 11:   # not a BASELINE config: config 3's shape with mxfp4 weights (e2m1, one e8m0 scale per 32 K, no offset)
+            M, K, N, x_dt, w_dt, group, off = (max_m or args.m or 16), 8192, 28672, m.ACL_FLOAT16, m.ACL_FLOAT4_E2M1, 32, False
+            self.dtype, lo, hi = "f16 (mxfp4 weights)", 0.005, 0.02
+            self.name = "aclnnWeightQuantBatchMatmulV2 mxfp4 weights (e2m1, e8m0 per 32 K), fp16 decode, config 3's shape"
         else:
             M, K, N, x_dt, w_dt, group, off = (max_m or args.m or 16), 8192, 28672, m.ACL_FLOAT16, m.ACL_INT4, 128, True
             self.dtype, lo, hi = "f16 (int4 weights)", 0.005, 0.02
@@ -269,7 +275,8 @@ class ConfigWQ(Workload):
             sshape, sst = (self.G, N), ((1, self.G) if self.packed else None)
         else:
             sshape, sst = (N,), None
-        self.t_sc = m.Tensor(sshape, x_dt, self.d["scale"], strides=sst)
+        self.scale_dt = inp.get("scale_dt", x_dt)
+        self.t_sc = m.Tensor(sshape, self.scale_dt, self.d["scale"], strides=sst)
         self.t_off = m.Tensor(sshape, x_dt, self.d["offset"], strides=sst) if off else None
         self.ncopies = 1
         self.i = 0
@@ -292,6 +299,7 @@ class ConfigWQ(Workload):
         self.M = M
         self.inp = dict(self.inp_full, x=np.ascontiguousarray(self.inp_full["x"][:M]))
         self.kernel = ("wqmm_resx_kernel" if (self.cfg == 3 and M <= 3) else "wqmm_xreg_kernel" if M <= 16 else
+                       "wqmm_decode_kernel" if self.cfg == 11 else
                        "wqmm_tile_kernel" if M > 128 else "wqmm_rows_kernel" if M > 48 else "wqmm_stream_kernel")
         self.t_x = m.Tensor((M, K), self.x_dt, self.d["x"])
         self.t_y = m.Tensor((M, N), self.x_dt, self.d_y)
@@ -303,7 +311,8 @@ class ConfigWQ(Workload):
         self.ws_size = ws
         self.flop = 2 * M * N * K
         wb = K * N * (1 if self.w_dt == m.ACL_INT8 else 0.5)
-        self.bytes = int(wb + 2 * M * K + 2 * M * N + 2 * self.G * N * (2 if self.off else 1))
+        sb = 1 if self.scale_dt == m.ACL_FLOAT8_E8M0 else 2
+        self.bytes = int(wb + 2 * M * K + 2 * M * N + sb * self.G * N * (2 if self.off else 1))
         self.variant = "cold" if self.ncopies > 1 else "warm"
         self.config = {"workload": self.name, "M": M, "K": K, "N": N, "group": self.group,
                        "cache": "cold (weight copies rotated, %d x %.0f MB)" % (self.ncopies, self.inp_full["w"].nbytes / 1e6)
@@ -331,6 +340,54 @@ class ConfigWQ(Workload):
         what = "the whole workload once" if rows == self.M else f"the first {rows} of {self.M} rows of x against the whole weight"
         return {"value": nbytes / t / 1e9, "unit": "GB/s", "cores": _cores(), "kind": "port",
                 "sample": f"{what} (oracle/liboracle.so, OpenMP), {t:.2f} s"}
+
+
+class ConfigKG(Workload):
+    """Not a BASELINE config: aclnnQuantMatmulV5 in the int4 x int4 mode with per-group (256 K) scales and offsets of x2
+    ("K-G" of quant_batch_matmul_v4), 4096 x 4096 x 4096, bf16 output.  The operands are widened to int8 in the workspace
+    by every call (four small kernels before the matrix kernel): they are inside the timed step."""
+    peak_key, dtype = "int8", "int8 (int4 operands widened)"
+    kernel = "kg_gemm_kernel (+ kg_widen / kg_rowsum / kg_scales pre-steps)"
+
+    def __init__(self, m, args, M=4096, K=4096, N=4096):
+        self.m, self.M, self.K, self.N = m, M, K, N
+        self.inp = cases.make_i4_asym_inputs(m, M, K, N, 0)
+        self.d = {k: m.DeviceBuffer(host=v) for k, v in self.inp.items()}
+        self.d_out = m.DeviceBuffer(M * N * 2)
+        G = K // 256
+        self.t = dict(x1=m.Tensor((M, K), m.ACL_INT4, self.d["x1"]), x2=m.Tensor((N, K), m.ACL_INT4, self.d["x2"]),
+                      s1=m.Tensor((M, 1), m.ACL_FLOAT, self.d["s1"]), s2=m.Tensor((G, N), m.ACL_FLOAT, self.d["s2"]),
+                      off=m.Tensor((G, N), m.ACL_FLOAT16, self.d["off"]), out=m.Tensor((M, N), m.ACL_BF16, self.d_out))
+        rc, ws, ex = self._phase1()
+        m.lib().aclDestroyAclOpExecutor(ex)
+        self.ws = m.DeviceBuffer(ws) if ws else None
+        self.ws_size = ws
+        self.flop = 2 * M * N * K
+        self.bytes = M * K // 2 + K * N // 2 + 4 * M + 6 * G * N + 2 * M * N
+        self.config = {"workload": "aclnnQuantMatmulV5 int4 x int4 K-G (groups of 256, fp32 scale + fp16 offset per group and column), bf16 out",
+                       "M": M, "K": K, "N": N, "x2_layout": "K-contiguous (transposeX2, as the mode requires)"}
+
+    def _phase1(self):
+        m, t = self.m, self.t
+        rc, ws, ex = m.quant_matmul_v5_get_workspace(t["x1"], t["x2"], t["s1"], t["s2"], t["out"], x2_offset=t["off"], transpose_x2=True,
+                                                     group_size=256)
+        m.check(rc, "phase 1")
+        return rc, ws, ex
+
+    def step(self, stream):
+        m = self.m
+        rc, ws, ex = self._phase1()
+        m.check(m.lib().aclnnQuantMatmulV5(self.ws.ptr if self.ws else None, self.ws_size, ex, stream.ptr), "phase 2")
+
+    def cpu_baseline(self):
+        rows = 64
+        inp = self.inp
+        x1 = np.ascontiguousarray(inp["x1"][:rows]); s1 = np.ascontiguousarray(inp["s1"][:rows])
+        t0 = time.perf_counter()
+        orc.qmm_i4_asym(x1, inp["x2"], rows, self.K, self.N, True, s1, inp["s2"], inp["off"], self.m.ACL_BF16)
+        t = time.perf_counter() - t0
+        return {"value": 2.0 * rows * self.K * self.N / t / 1e12, "unit": "TFLOP/s", "cores": _cores(), "kind": "port",
+                "sample": f"first {rows} of {self.M} rows of x1 against the full x2 (oracle/liboracle.so, OpenMP), {t:.2f} s"}
 
 
 class PrepOp(Workload):
@@ -405,8 +462,10 @@ class PrepOp(Workload):
 def make_workload(m, config, args):
     if config in (6, 7, 8, 9):
         return PrepOp(m, args, config)
-    if config in (1, 3):
+    if config in (1, 3, 11):
         return ConfigWQ(m, args, config)
+    if config == 10:
+        return ConfigKG(m, args)
     if config == 2:
         return Config2(m, args)
     if config == 4:
