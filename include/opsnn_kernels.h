@@ -112,7 +112,7 @@ OPSNN_API void opsnnSetMx8Wide(int n);
 OPSNN_API void opsnnSetWqTileMin(int m);
 /* Opt-in cache of re-laid-out right operands.  The matrix-core kernels stream a K-contiguous right operand; x2 / weight
  * stored [K, N] with N contiguous is re-laid out inside every call (into the caller's workspace) unless this cache is on:
- * then opsnnQmmInt8, opsnnQmmBlockScale and opsnnWqmm keep the K-contiguous copy in device memory of the library's own, keyed
+ * then opsnnQmmInt8, opsnnQmmBlockScale, opsnnQmmMx (data and scales) and opsnnWqmm keep the K-contiguous copy in device memory of the library's own, keyed
  * by the operand's address, shape, element width and batch count, and later calls with the same operand skip the pass
  * (the workspace is then not touched).  It has no counterpart among the reference's entry points: the reference folds the
  * re-layout into its graphs offline (weight_quant_batch_matmul_v2_transpose_fusion_pass.cpp,

@@ -63,6 +63,9 @@ uint64_t mx_workspace_bytes(const OpsnnQmmArgs& a)
     return data + align_up((uint64_t)a.N * ks * 2, 256) * snb;
 }
 
+void* weight_cache_blob(const void* src, const void* src2, int64_t K, int64_t N, int bits, int64_t nb, uint64_t bytes, hipStream_t st, bool* fresh);
+void weight_cache_commit(void* buffer, hipStream_t st);   // weight_cache.hip
+void weight_cache_abandon(void* buffer);
 int launch_mxfp8_mfma(const OpsnnQmmArgs& a, hipStream_t st);   // qmm_fp8_block.hip
 int launch_mx_a8w4_mfma(const OpsnnQmmArgs& a, hipStream_t st);   // qmm_fp8_block.hip
 
@@ -86,28 +89,40 @@ int launch_mx_mfma(const OpsnnQmmArgs& a0, hipStream_t st)
     const int64_t epb = fp4 ? 2 : 1;  // elements per byte
 
     if (a.x2.row_stride != 1) {
-        // x2 is [K, N] with N contiguous: re-lay data and scales out K-contiguous in the workspace
-        if (!a.workspace || a.x2.col_stride != 1 || a.x2.row_stride != a.N) return OPSNN_NOT_TAKEN;
+        // x2 is [K, N] with N contiguous: re-lay data and scales out K-contiguous, into the weight cache's buffer for this
+        // operand when the cache is on (a hit skips the passes), else into the workspace
+        if (a.x2.col_stride != 1 || a.x2.row_stride != a.N) return OPSNN_NOT_TAKEN;
         if (a.x2_scale_mat.row_stride != 2 || a.x2_scale_mat.col_stride != a.N * 2) return OPSNN_NOT_TAKEN;
         if (a.x2.batch_stride != 0 && a.x2.batch_stride != a.K * a.N) return OPSNN_NOT_TAKEN;
         const int64_t nb = a.x2.batch_stride == 0 ? 1 : a.batch;
         const int64_t snb = a.x2_scale_mat.batch_stride == 0 ? 1 : a.batch;
         if (snb != 1 && a.x2_scale_mat.batch_stride != ks * a.N * 2) return OPSNN_NOT_TAKEN;
         const uint64_t data_one = align_up((uint64_t)a.N * a.K / epb, 256);
-        char* wdata = (char*)a.workspace;
-        char* wscale = wdata + data_one * nb;
         const uint64_t scale_one = align_up((uint64_t)a.N * ks * 2, 256);
-        for (int64_t b = 0; b < nb; b++) {  // per-batch because of the aligned pitch
+        bool fresh = false;
+        char* wdata = (char*)weight_cache_blob(a.x2.ptr, a.x2_scale_mat.ptr, a.K, a.N, fp4 ? 4 : 8, nb * 16 + snb,
+                                               data_one * (uint64_t)nb + scale_one * (uint64_t)snb, st, &fresh);
+        const bool cached = wdata != nullptr;
+        if (!cached) {
+            if (!a.workspace) return OPSNN_NOT_TAKEN;
+            wdata = (char*)a.workspace;
+        }
+        char* wscale = wdata + data_one * nb;
+        for (int64_t b = 0; b < nb && (!cached || fresh); b++) {  // per-batch because of the aligned pitch
             const char* src = (const char*)a.x2.ptr + b * (a.K * a.N / epb);
             int rc = fp4 ? opsnnTranspose4(src, wdata + b * data_one, a.K, a.N, 1, st) : opsnnTranspose8(src, wdata + b * data_one, a.K, a.N, 1, st);
-            if (rc != 0) return rc;
+            if (rc != 0) {
+                if (cached) weight_cache_abandon(wdata);
+                return rc;
+            }
         }
-        for (int64_t b = 0; b < snb; b++) {
+        for (int64_t b = 0; b < snb && (!cached || fresh); b++) {
             dim3 grid((unsigned)((a.N + 31) / 32), (unsigned)((ks + 31) / 32), 1);
             hipLaunchKernelGGL(transpose16_kernel, grid, dim3(256), 0, st,
                                (const uint16_t*)((const char*)a.x2_scale_mat.ptr + b * (ks * a.N * 2)),
                                (uint16_t*)(wscale + b * scale_one), ks, a.N);
         }
+        if (cached && fresh) weight_cache_commit(wdata, st);
         a.x2.ptr = wdata; a.x2.row_stride = 1; a.x2.col_stride = a.K; a.x2.batch_stride = nb == 1 ? 0 : (int64_t)(data_one * epb);
         a.x2_scale_mat.ptr = wscale; a.x2_scale_mat.row_stride = ks * 2; a.x2_scale_mat.col_stride = 2;
         a.x2_scale_mat.batch_stride = snb == 1 ? 0 : (int64_t)scale_one;

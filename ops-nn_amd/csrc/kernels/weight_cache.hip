@@ -25,8 +25,9 @@ namespace opsnn {
 namespace {
 
 struct Entry {
-    const void* src; int64_t K, N, nb; int bits;
+    const void* src; const void* src2; int64_t K, N, nb; int bits;
     void* copy; uint64_t bytes; hipEvent_t ready; int device;
+    bool committed;   // filled and its event recorded; until then other callers do not use it
 };
 
 std::mutex g_mu;
@@ -44,19 +45,23 @@ void drop(std::list<Entry>::iterator it)
 
 }  // namespace
 
-// The K-contiguous copy of the [K, N] matrix (N contiguous, nb dense batches) of `bits`-wide elements at src, ready for
-// use on `st`; nullptr when the cache does not serve this call (the caller then re-lays the operand out itself).
-const void* weight_cache_get(const void* src, int64_t K, int64_t N, int bits, int64_t nb, hipStream_t st)
+// A buffer of `bytes` that belongs to the operand (src, src2 -- e.g. data and scales --, shape, element width, batch count):
+// on a hit (*fresh = false) it holds what an earlier call put there and is ordered behind that call's writes on `st`; on a
+// miss (*fresh = true) it is new: the caller fills it with launches on `st` and then calls weight_cache_commit(buffer, st).
+// nullptr when the cache does not serve this call (off, under graph capture, larger than the limit, allocation failure).
+void* weight_cache_blob(const void* src, const void* src2, int64_t K, int64_t N, int bits, int64_t nb, uint64_t bytes, hipStream_t st, bool* fresh)
 {
-    if (!g_limit || !src || K <= 0 || N <= 0 || nb <= 0) return nullptr;
+    *fresh = false;
+    if (!g_limit || !src || K <= 0 || N <= 0 || nb <= 0 || !bytes) return nullptr;
     hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
     if (hipStreamIsCapturing(st, &cap) != hipSuccess || cap != hipStreamCaptureStatusNone) return nullptr;
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess) return nullptr;
-    const uint64_t bytes = (uint64_t)K * (uint64_t)N * (uint64_t)bits / 8 * (uint64_t)nb;
     std::lock_guard<std::mutex> lock(g_mu);
     for (auto it = g_entries.begin(); it != g_entries.end(); ++it) {
-        if (it->src == src && it->K == K && it->N == N && it->bits == bits && it->nb == nb && it->device == dev) {
+        if (it->src == src && it->src2 == src2 && it->K == K && it->N == N && it->bits == bits && it->nb == nb && it->bytes == bytes &&
+            it->device == dev) {
+            if (!it->committed) return nullptr;   // another call is still filling it: this one goes its own way
             if (hipStreamWaitEvent(st, it->ready, 0) != hipSuccess) return nullptr;
             g_entries.splice(g_entries.begin(), g_entries, it);
             g_hits++;
@@ -65,19 +70,49 @@ const void* weight_cache_get(const void* src, int64_t K, int64_t N, int bits, in
     }
     if (bytes > g_limit) return nullptr;
     while (g_used + bytes > g_limit && !g_entries.empty()) drop(std::prev(g_entries.end()));
-    Entry e{src, K, N, nb, bits, nullptr, bytes, nullptr, dev};
+    Entry e{src, src2, K, N, nb, bits, nullptr, bytes, nullptr, dev, false};
     if (hipMalloc(&e.copy, bytes) != hipSuccess) { (void)hipGetLastError(); return nullptr; }
     if (hipEventCreateWithFlags(&e.ready, hipEventDisableTiming) != hipSuccess) { (void)hipFree(e.copy); return nullptr; }
-    const int rc = bits == 4 ? opsnnTranspose4(src, e.copy, K, N, nb, st) : opsnnTranspose8(src, e.copy, K, N, nb, st);
-    if (rc != 0 || hipEventRecord(e.ready, st) != hipSuccess) {
-        (void)hipEventDestroy(e.ready);
-        (void)hipFree(e.copy);
-        return nullptr;
-    }
+    // until the commit nobody else uses the entry; one whose filling call fails is removed by weight_cache_abandon
     g_used += bytes;
     g_misses++;
     g_entries.push_front(e);
+    *fresh = true;
     return e.copy;
+}
+
+// The fresh buffer has been filled by the launches already enqueued on st.
+void weight_cache_commit(void* buffer, hipStream_t st)
+{
+    std::lock_guard<std::mutex> lock(g_mu);
+    for (auto it = g_entries.begin(); it != g_entries.end(); ++it)
+        if (it->copy == buffer) {
+            if (hipEventRecord(it->ready, st) == hipSuccess) it->committed = true;
+            else drop(it);
+            return;
+        }
+}
+
+// The fresh buffer could not be filled: forget it.
+void weight_cache_abandon(void* buffer)
+{
+    std::lock_guard<std::mutex> lock(g_mu);
+    for (auto it = g_entries.begin(); it != g_entries.end(); ++it)
+        if (it->copy == buffer) { drop(it); return; }
+}
+
+// The K-contiguous copy of the [K, N] matrix (N contiguous, nb dense batches) of `bits`-wide elements at src, ready for
+// use on `st`; nullptr when the cache does not serve this call (the caller then re-lays the operand out itself).
+const void* weight_cache_get(const void* src, int64_t K, int64_t N, int bits, int64_t nb, hipStream_t st)
+{
+    const uint64_t bytes = (uint64_t)K * (uint64_t)N * (uint64_t)bits / 8 * (uint64_t)nb;
+    bool fresh = false;
+    void* copy = weight_cache_blob(src, nullptr, K, N, bits, nb, bytes, st, &fresh);
+    if (!copy || !fresh) return copy;
+    const int rc = bits == 4 ? opsnnTranspose4(src, copy, K, N, nb, st) : opsnnTranspose8(src, copy, K, N, nb, st);
+    if (rc != 0) { weight_cache_abandon(copy); return nullptr; }
+    weight_cache_commit(copy, st);
+    return copy;
 }
 
 }  // namespace opsnn

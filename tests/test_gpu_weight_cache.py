@@ -98,3 +98,17 @@ def test_int8_x2_is_re_laid_out_once_and_the_limit_evicts(cache):
     assert m.lib().opsnnQmmInt8(a, None) == 0
     m.check(m.lib().aclrtSynchronizeDevice(), "sync")
     assert np.array_equal(d_out.to_host(np.uint16, (1, M, N)), want) and _stats(m)[0] == 0
+
+
+def test_mx_operand_and_its_scales_are_re_laid_out_once(cache):
+    """MXFP4 with x2 stored [K, N]: data and the [K/64, N, 2] scales go into one cached buffer; the product stays the oracle's."""
+    m = cache
+    M, K, N = 128, 512, 256
+    print(f"case weight cache, mxfp4 {M}x{K}x{N}", flush=True)
+    inp = cases.make_mx_inputs(m, M, K, N, 7, False, True)
+    want = cases.oracle_mx(m, inp, M, K, N, False, m.ACL_BF16)
+    e0, _, h0, m0 = _stats(m)
+    first = cases.run_mx_aclnn(m, inp, M, K, N, False, m.ACL_BF16)       # fresh device buffers: a miss
+    assert np.array_equal(first, want)
+    e1, _, h1, m1 = _stats(m)
+    assert (m1 - m0, h1 - h0) == (1, 0) and e1 - e0 == 1
