@@ -7,28 +7,39 @@
 // sums of a group are exact (at most 256 products of magnitude 64), so the result is the golden's bit for bit whatever
 // the order inside a group; the groups are folded in ascending order with separately rounded fp32 operations.
 //
-// This chip has no 4-bit integer matrix instruction, so a pre-step widens both operands to int8 in the workspace --
-// zero-padded to whole tiles (rows to 128, K to 256), so that the matrix kernel reads only memory laid out by this
-// file -- together with the row sums of x1 per group and zero-padded fp32 copies of the scales and offsets.
+// This chip has no 4-bit integer matrix instruction.  Every int4 value is an fp8 e4m3 value, the products (magnitude at
+// most 64) and a group's sum (at most 16384) are small integers, and v_mfma_f32_16x16x128_f8f6f4 adds them without
+// loss, so the group sum leaves the matrix pipe as the fp32 the fold needs and no conversion is spent on it.
+//
+// A pre-step writes both operands as e4m3 bytes into the workspace, zero-padded to whole tiles (rows to 128, K to 256)
+// and stored block by block: the 128 rows x 256 bytes of one tile and group, followed by 1 KiB of that group's fp32
+// side values (x1: the negated row sums; x2: scales, then offsets), are one contiguous block that already is the LDS
+// image (16-byte chunks of a row xor-swizzled by the row, so that fragment reads are free of bank conflicts).  The
+// matrix kernel fetches a block with linear 16-byte asynchronous copies: consecutive addresses spread over all memory
+// channels (rows 4096 bytes apart would all fall into one), and the side values arrive in LDS with the tile instead of
+// costing every wave eight vector loads per group.
+//
 // The matrix kernel: 128 x 128 output tile per workgroup, eight waves of 64 x 32 (4 x 2 fragments of 16 x 16), one K
-// tile = one group (256 bytes per row), v_mfma_i32_16x16x64_i8 chained over the group's four 64-byte steps from a
-// zero accumulator, then the fold on the vector ALU (five operations per output and group).  The next group's
-// operands are fetched into registers while the current one is multiplied, and written to the one LDS buffer between
-// two barriers; rows are stored with their 16-byte chunks xor-swizzled by row so that the fragment reads are free of
-// bank conflicts.
+// tile = one group, two matrix instructions per fragment pair from a zero accumulator, then the fold on the vector
+// ALU, three operations per output and group:  sum += fma(-rowsum, off, t) * s2.  The product rowsum * off is exact in
+// fp32 (an integer of magnitude at most 2048 times an fp16 value has at most 22 significant bits), so the fused form
+// rounds exactly where the golden's separate subtraction does.  A wave issues in order, so the three kinds of work
+// are interleaved in the source: the copies of group g + 1 (into the other of two LDS buffers) go out between the
+// matrix instructions of group g, and the fold of group g - 1 fills the vector ALU meanwhile; one barrier per group.
 #include "launch.h"
-#include "common.hip.h"
+#include "qgemm_core.hip.h"
 
 namespace opsnn {
 namespace {
 
 constexpr int64_t KG_GROUP = 256, KG_TILE = 128;
+constexpr int64_t KG_ROWS = KG_TILE * KG_GROUP, KG_BLOCK = KG_ROWS + 1024;   // operand bytes of one tile and group; with its side values
 inline int64_t kg_rup(int64_t v, int64_t m) { return (v + m - 1) / m * m; }
 inline uint64_t kg_a256(uint64_t v) { return (v + 255) / 256 * 256; }
 
 struct KgLayout {
     int64_t Mp, Np, Kp, G;
-    uint64_t o_b, o_rs, o_s2, o_of, total;   // byte offsets in the workspace (the widened x1 sits at 0)
+    uint64_t o_b, total;   // byte offset of the x2 blocks in the workspace (the x1 blocks sit at 0)
 };
 
 bool kg_layout(const OpsnnQmmArgs& a, KgLayout& L)
@@ -41,61 +52,55 @@ bool kg_layout(const OpsnnQmmArgs& a, KgLayout& L)
     if (a.x2.row_stride != 1 || a.x2.col_stride % 2 != 0 || a.x2.col_stride < a.K) return false;
     if (a.K % 2 != 0 || a.M * a.N < 32 * 32) return false;
     L.Mp = kg_rup(a.M, KG_TILE); L.Np = kg_rup(a.N, KG_TILE); L.Kp = kg_rup(a.K, KG_GROUP); L.G = L.Kp / KG_GROUP;
-    if (L.Mp * L.Kp >= (1ll << 31) || L.Np * L.Kp >= (1ll << 31)) return false;   // 32-bit offsets inside the kernels
-    L.o_b = kg_a256((uint64_t)L.Mp * L.Kp);
-    L.o_rs = L.o_b + kg_a256((uint64_t)L.Np * L.Kp);
-    L.o_s2 = L.o_rs + kg_a256((uint64_t)L.Mp * L.G * 4);
-    L.o_of = L.o_s2 + kg_a256((uint64_t)L.G * L.Np * 4);
-    L.total = L.o_of + kg_a256((uint64_t)L.G * L.Np * 4);
+    L.o_b = (uint64_t)(L.Mp / KG_TILE * L.G * KG_BLOCK);
+    L.total = L.o_b + (uint64_t)(L.Np / KG_TILE * L.G * KG_BLOCK);
     return true;
 }
 
-// 16 int4 (8 bytes) of row r -> 16 int8; rows past `rows` and columns past K become zero.  ld: elements between rows.
+// 16 int4 (8 bytes) of row r -> 16 e4m3 bytes in the block layout; rows past `rows` and columns past K become zero.
+// ld: elements between rows.  WITH_RS: the block's first side value array gets -fp32(sum of the row over the group)
+// (exact: at most 256 values of magnitude 8); the 16 threads of one row and group are neighbours in one wave.
+template <bool WITH_RS>
 __global__ __launch_bounds__(256) void kg_widen_kernel(const uint8_t* __restrict__ src, int64_t rows, int64_t K, int64_t ld,
-                                                       int8_t* __restrict__ dst, int64_t rows_p, int64_t Kp)
+                                                       int8_t* __restrict__ dst, int64_t rows_p, int64_t Kp, int64_t G)
 {
-    const int64_t per_row = Kp / 16;
+    const int64_t per_row = Kp / 16;   // a multiple of 16; rows_p * per_row is a multiple of the block size
     const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (idx >= rows_p * per_row) return;
-    const int64_t r = idx / per_row, k0 = (idx - r * per_row) * 16;
-    uint32_t o[4] = {0, 0, 0, 0};
-    if (r < rows) {
+    const int64_t r = idx / per_row, kc = idx - r * per_row, k0 = kc * 16;
+    uint64_t nib = 0;   // 16 nibbles, element k0 + e in bits [4 e, 4 e + 4)
+    if (r < rows && k0 < K) {
+        const uint8_t* p = src + ((r * ld + k0) >> 1);   // ld and k0 are even: the row piece starts on a byte
+        if (k0 + 16 <= K && ((uintptr_t)p & 7) == 0) nib = *(const uint64_t*)p;
+        else {
 #pragma unroll
-        for (int b = 0; b < 8; b++) {
-            const int64_t k = k0 + 2 * b;
-            if (k < K) {   // K is even: both nibbles of the byte are inside the row
-                const uint32_t byte = src[(r * ld + k) >> 1];
-                const uint32_t lo = (uint32_t)(((int32_t)(int8_t)(byte << 4)) >> 4) & 0xffu;   // sign-extended low nibble
-                const uint32_t hi = (uint32_t)(((int32_t)(int8_t)byte) >> 4) & 0xffu;
-                o[b / 2] |= (lo | (hi << 8)) << (16 * (b % 2));
-            }
+            for (int b = 0; b < 8; b++)
+                if (k0 + 2 * b < K) nib |= (uint64_t)p[b] << (8 * b);   // K is even: both nibbles of the byte are inside the row
         }
     }
-    *(uint4*)(dst + r * Kp + k0) = make_uint4(o[0], o[1], o[2], o[3]);
-}
-
-// rs[m * G + g] = fp32 of the sum of the widened x1 over group g (exact: at most 256 values of magnitude 8)
-__global__ __launch_bounds__(256) void kg_rowsum_kernel(const int8_t* __restrict__ a8, int64_t Mp, int64_t Kp, int64_t G, float* __restrict__ rs)
-{
-    const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    if (idx >= Mp * G) return;
-    const int64_t m = idx / G, g = idx - m * G;
-    const uint4* p = (const uint4*)(a8 + m * Kp + g * KG_GROUP);
+    // e4m3 of the two's-complement nibble n: 0..7 -> 0, 1, 2, ... 7; 8..15 -> -8, -7, ... -1
+    constexpr uint64_t POS = 0x4E4C4A4844403800ull, NEG = 0xB8C0C4C8CACCCED0ull;
+    uint32_t o[4] = {0, 0, 0, 0};
     int32_t s = 0;
-#pragma unroll 4
-    for (int i = 0; i < 16; i++) {
-        const uint4 v = p[i];
-        const uint32_t w[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
-        for (int e = 0; e < 4; e++)
-            s += (int32_t)(int8_t)w[e] + (int32_t)(int8_t)(w[e] >> 8) + (int32_t)(int8_t)(w[e] >> 16) + (int32_t)(int8_t)(w[e] >> 24);
+    for (int e = 0; e < 16; e++) {
+        const uint32_t n = (uint32_t)(nib >> (4 * e)) & 15u;
+        const uint32_t f = (uint32_t)(((n & 8u) ? NEG : POS) >> (8 * (n & 7u))) & 0xffu;
+        o[e / 4] |= f << (8 * (e % 4));
+        s += (int32_t)(n ^ 8u) - 8;
     }
-    rs[idx] = (float)s;
+    const int64_t g = kc >> 4, c = kc & 15;
+    int8_t* block = dst + ((r >> 7) * G + g) * KG_BLOCK;
+    *(uint4*)(block + ((r & 127) << 8) + ((c ^ (r & 15)) << 4)) = make_uint4(o[0], o[1], o[2], o[3]);
+    if (WITH_RS) {
+#pragma unroll
+        for (int d = 8; d >= 1; d >>= 1) s += __shfl_xor(s, d, 16);
+        if (c == 0) ((float*)(block + KG_ROWS))[r & 127] = -(float)s;
+    }
 }
 
-// fp32 copies of scale[g, n] and offset[g, n] with the columns padded to Np (zeros)
-__global__ __launch_bounds__(256) void kg_scales_kernel(OpsnnMat sc, OpsnnMat of, int64_t N, int64_t Np, int64_t G, int64_t Greal,
-                                                        float* __restrict__ s2p, float* __restrict__ ofp)
+// fp32 scale[g, n] and offset[g, n] into the side values of the x2 blocks (zeros for padded columns and groups)
+__global__ __launch_bounds__(256) void kg_scales_kernel(OpsnnMat sc, OpsnnMat of, int64_t N, int64_t Np, int64_t G, int64_t Greal, int8_t* __restrict__ dst)
 {
     const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (idx >= G * Np) return;
@@ -105,97 +110,123 @@ __global__ __launch_bounds__(256) void kg_scales_kernel(OpsnnMat sc, OpsnnMat of
         s = ((const float*)sc.ptr)[g * sc.row_stride + n * sc.col_stride];
         o = load_scalar_as_f32(of.ptr, DT_F16, g * of.row_stride + n * of.col_stride);
     }
-    s2p[idx] = s;
-    ofp[idx] = o;
+    float* side = (float*)(dst + ((n >> 7) * G + g) * KG_BLOCK + KG_ROWS);
+    side[n & 127] = s;
+    side[128 + (n & 127)] = o;
 }
 
 template <int OUT_DT>
-__global__ __launch_bounds__(512) void kg_gemm_kernel(const int8_t* __restrict__ A, const int8_t* __restrict__ B, const float* __restrict__ rs,
-                                                      const float* __restrict__ s2p, const float* __restrict__ ofp,
-                                                      const float* __restrict__ x1s, uint16_t* __restrict__ out,
-                                                      int64_t M, int64_t N, int Kp, int Np, int G)
+__global__ __launch_bounds__(512) void kg_gemm_kernel(const int8_t* __restrict__ A, const int8_t* __restrict__ B, const float* __restrict__ x1s,
+                                                      uint16_t* __restrict__ out, int64_t M, int64_t N, int G)
 {
     constexpr int FM = 4, FN = 2;
-    __shared__ __attribute__((aligned(16))) char lds[2 * 128 * 256];
+    constexpr int ROWS = (int)KG_ROWS, BLOCK = (int)KG_BLOCK, BUF = 2 * BLOCK;   // LDS: two buffers of an x1 block and an x2 block
+    extern __shared__ __attribute__((aligned(16))) char lds[];
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave >> 2, wn = wave & 3;
     const int frow = lane & 15, fq = lane >> 4;
-    const int m0 = blockIdx.y * 128, n0 = blockIdx.x * 128;   // inside the padded operands by construction of the grid
+    const int m0 = blockIdx.y * 128, n0 = blockIdx.x * 128;
 
-    // staging: chunk idx = tid + 512 i of an operand tile is row idx / 16, 16-byte chunk idx % 16
-    v4i ra[4], rb[4];
-    auto gload = [&](int g) {
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-            const int idx = tid + 512 * i, r = idx >> 4, c = idx & 15;
-            ra[i] = *(const v4i*)(A + (int64_t)(m0 + r) * Kp + g * 256 + c * 16);
-            rb[i] = *(const v4i*)(B + (int64_t)(n0 + r) * Kp + g * 256 + c * 16);
-        }
+    // Copies of one group: eight per wave for the operand rows (copy c of the workgroup's 2 x 4 moves 8 KiB, this
+    // wave's share is 1 KiB of it), and waves 0 and 1 move the side values of the x1 and the x2 block.
+    const int8_t* ga = A + (int64_t)blockIdx.y * G * BLOCK;
+    const int8_t* gb = B + (int64_t)blockIdx.x * G * BLOCK;
+    auto copy_rows = [&](int g, int buf, int c) {   // c = 0..7, compile-time after unrolling
+        const int8_t* src = (c < 4 ? ga : gb) + (int64_t)g * BLOCK + (c & 3) * 8192 + tid * 16;
+        async_copy16_uncounted(src, lds + buf * BUF + (c < 4 ? 0 : BLOCK) + (c & 3) * 8192 + wave * 1024);
     };
-    auto lstore = [&]() {
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-            const int idx = tid + 512 * i, r = idx >> 4, c = idx & 15;
-            *(v4i*)(lds + r * 256 + ((c ^ (r & 15)) << 4)) = ra[i];
-            *(v4i*)(lds + 32768 + r * 256 + ((c ^ (r & 15)) << 4)) = rb[i];
+    auto copy_side = [&](int g, int buf) {
+        if (wave < 2) {
+            const int8_t* src = (wave == 0 ? ga : gb) + (int64_t)g * BLOCK + ROWS + lane * 16;
+            async_copy16_uncounted(src, lds + buf * BUF + wave * BLOCK + ROWS);
         }
     };
 
-    v4f sum[FN][FM];
+    v4f sum[FN][FM], tp[FN][FM];   // running sums; the previous group's integer sums, folded while this group is multiplied
+    float rsp[FM];
+    v4f s2q[FN], ofq[FN];
 #pragma unroll
-    for (int i = 0; i < FN; i++)
+    for (int i = 0; i < FN; i++) {
+        s2q[i] = ofq[i] = (v4f){0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
-        for (int j = 0; j < FM; j++) sum[i][j] = (v4f){0.0f, 0.0f, 0.0f, 0.0f};
+        for (int j = 0; j < FM; j++) sum[i][j] = tp[i][j] = (v4f){0.0f, 0.0f, 0.0f, 0.0f};
+    }
+#pragma unroll
+    for (int j = 0; j < FM; j++) rsp[j] = 0.0f;
+    auto fold = [&](int i, int j) {
+#pragma unroll
+        for (int r = 0; r < 4; r++) sum[i][j][r] = sum[i][j][r] + __builtin_fmaf(rsp[j], ofq[i][r], tp[i][j][r]) * s2q[i][r];
+    };
 
-    const char* la = lds + (wm * 64 + frow) * 256;
-    const char* lb = lds + 32768 + (wn * 32 + frow) * 256;
-    gload(0);
+#pragma unroll
+    for (int c = 0; c < 8; c++) copy_rows(0, 0, c);
+    copy_side(0, 0);
     for (int g = 0; g < G; g++) {
-        __syncthreads();   // every wave has read the previous group
-        lstore();
+        // this wave's copies of group g have landed; behind the barrier everybody's have, and every wave has finished
+        // its reads of the other buffer (group g - 1)
+        wait_vmcnt<0>();
         __syncthreads();
-        if (g + 1 < G) gload(g + 1);
+        const int buf = g & 1;
+        const bool more = g + 1 < G;
+        const char* la = lds + buf * BUF + (wm * 64 + frow) * 256;
+        const char* lb = lds + buf * BUF + BLOCK + (wn * 32 + frow) * 256;
+        // this group's side values, for its fold during the next group (by then the buffer is being refilled)
         float rsv[FM];
         v4f s2v[FN], ofv[FN];
 #pragma unroll
-        for (int j = 0; j < FM; j++) rsv[j] = rs[(int64_t)(m0 + wm * 64 + 16 * j + frow) * G + g];
+        for (int j = 0; j < FM; j++) rsv[j] = *(const float*)(lds + buf * BUF + ROWS + (wm * 64 + 16 * j + frow) * 4);
 #pragma unroll
         for (int i = 0; i < FN; i++) {
-            const int64_t o = (int64_t)g * Np + n0 + wn * 32 + 16 * i + 4 * fq;
-            s2v[i] = *(const v4f*)(s2p + o);
-            ofv[i] = *(const v4f*)(ofp + o);
+            const char* sv = lds + buf * BUF + BLOCK + ROWS + (wn * 32 + 16 * i + 4 * fq) * 4;
+            s2v[i] = *(const v4f*)sv;
+            ofv[i] = *(const v4f*)(sv + 512);
         }
-        v4i t[FN][FM];
+        if (more) copy_side(g + 1, buf ^ 1);
+        v4f t[FN][FM];
 #pragma unroll
-        for (int i = 0; i < FN; i++)
+        for (int s = 0; s < 2; s++) {
+            // lane (row, q) holds bytes [128 s + 32 q, + 32) of its row: the same K for both operands
+            const int p0 = ((8 * s + 2 * fq) ^ frow) << 4, p1 = ((8 * s + 2 * fq + 1) ^ frow) << 4;
+            v8i fa[FM], fb[FN];
 #pragma unroll
-            for (int j = 0; j < FM; j++) t[i][j] = (v4i){0, 0, 0, 0};
+            for (int j = 0; j < FM; j++) {
+                const v4i lo = *(const v4i*)(la + j * 16 * 256 + p0), hi = *(const v4i*)(la + j * 16 * 256 + p1);
+                fa[j] = (v8i){lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+            }
 #pragma unroll
-        for (int s = 0; s < 4; s++) {
-            // lane (row, q) holds bytes [64 s + 16 q, + 16) of its row: the same K for both operands
-            const int pos = ((4 * s + fq) ^ frow) << 4;
-            v4i fa[FM], fb[FN];
+            for (int i = 0; i < FN; i++) {
+                const v4i lo = *(const v4i*)(lb + i * 16 * 256 + p0), hi = *(const v4i*)(lb + i * 16 * 256 + p1);
+                fb[i] = (v8i){lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+            }
+            if (more) {
 #pragma unroll
-            for (int j = 0; j < FM; j++) fa[j] = *(const v4i*)(la + j * 16 * 256 + pos);
-#pragma unroll
-            for (int i = 0; i < FN; i++) fb[i] = *(const v4i*)(lb + i * 16 * 256 + pos);
+                for (int c = 0; c < 4; c++) copy_rows(g + 1, buf ^ 1, 4 * s + c);
+            }
 #pragma unroll
             for (int i = 0; i < FN; i++)
 #pragma unroll
-                for (int j = 0; j < FM; j++) t[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fb[i], fa[j], t[i][j], 0, 0, 0);
+                for (int j = 0; j < FM; j++) {
+                    t[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(fb[i], fa[j], s == 0 ? (v4f){0.0f, 0.0f, 0.0f, 0.0f} : t[i][j], 0, 0, 0,
+                                                                               0x7f7f7f7f, 0, 0x7f7f7f7f);
+                    if (i == s) fold(i, j);   // half of the previous group's fold in the shadow of each step
+                }
         }
         // t[i][j][r] is the group's integer sum for m = 16 j + lane % 16, n = 16 i + 4 (lane / 16) + r of the wave tile
 #pragma unroll
-        for (int i = 0; i < FN; i++)
+        for (int i = 0; i < FN; i++) {
+            s2q[i] = s2v[i];
+            ofq[i] = ofv[i];
 #pragma unroll
-            for (int j = 0; j < FM; j++)
+            for (int j = 0; j < FM; j++) tp[i][j] = t[i][j];
+        }
 #pragma unroll
-                for (int r = 0; r < 4; r++) {
-                    const float off = rsv[j] * ofv[i][r];
-                    sum[i][j][r] = sum[i][j][r] + ((float)t[i][j][r] - off) * s2v[i][r];
-                }
+        for (int j = 0; j < FM; j++) rsp[j] = rsv[j];
     }
+#pragma unroll
+    for (int i = 0; i < FN; i++)
+#pragma unroll
+        for (int j = 0; j < FM; j++) fold(i, j);
 
     const bool vec_ok = (N % 4) == 0 && ((uintptr_t)out % 8) == 0;
 #pragma unroll
@@ -232,25 +263,28 @@ int launch_kg_mfma(const OpsnnQmmArgs& a, hipStream_t st)
 {
     KgLayout L;
     if (!kg_layout(a, L) || !a.workspace || (uintptr_t)a.workspace % 16 != 0) return OPSNN_NOT_TAKEN;
-    char* ws = (char*)a.workspace;
-    int8_t* a8 = (int8_t*)ws;
-    int8_t* b8 = (int8_t*)(ws + L.o_b);
-    float* rs = (float*)(ws + L.o_rs);
-    float* s2p = (float*)(ws + L.o_s2);
-    float* ofp = (float*)(ws + L.o_of);
+    int8_t* a8 = (int8_t*)a.workspace;
+    int8_t* b8 = a8 + L.o_b;
     const int64_t Greal = (a.K + KG_GROUP - 1) / KG_GROUP;
     auto blocks = [](int64_t n) { return dim3((unsigned)((n + 255) / 256)); };
-    hipLaunchKernelGGL(kg_widen_kernel, blocks(L.Mp * (L.Kp / 16)), dim3(256), 0, st, (const uint8_t*)a.x1.ptr, a.M, a.K, a.x1.row_stride, a8, L.Mp, L.Kp);
-    hipLaunchKernelGGL(kg_widen_kernel, blocks(L.Np * (L.Kp / 16)), dim3(256), 0, st, (const uint8_t*)a.x2.ptr, a.N, a.K, a.x2.col_stride, b8, L.Np, L.Kp);
-    hipLaunchKernelGGL(kg_rowsum_kernel, blocks(L.Mp * L.G), dim3(256), 0, st, a8, L.Mp, L.Kp, L.G, rs);
-    hipLaunchKernelGGL(kg_scales_kernel, blocks(L.G * L.Np), dim3(256), 0, st, a.x2_scale_mat, a.x2_offset_mat, a.N, L.Np, L.G, Greal, s2p, ofp);
+    hipLaunchKernelGGL(kg_widen_kernel<true>, blocks(L.Mp * (L.Kp / 16)), dim3(256), 0, st, (const uint8_t*)a.x1.ptr, a.M, a.K, a.x1.row_stride, a8, L.Mp,
+                       L.Kp, L.G);
+    hipLaunchKernelGGL(kg_widen_kernel<false>, blocks(L.Np * (L.Kp / 16)), dim3(256), 0, st, (const uint8_t*)a.x2.ptr, a.N, a.K, a.x2.col_stride, b8, L.Np,
+                       L.Kp, L.G);
+    hipLaunchKernelGGL(kg_scales_kernel, blocks(L.G * L.Np), dim3(256), 0, st, a.x2_scale_mat, a.x2_offset_mat, a.N, L.Np, L.G, Greal, b8);
     const dim3 grid((unsigned)(L.Np / KG_TILE), (unsigned)(L.Mp / KG_TILE));
+    constexpr int KG_LDS = 2 * 2 * (int)KG_BLOCK;
+    static bool attr_set = false;
+    if (!attr_set) {
+        hipError_t e = hipFuncSetAttribute((const void*)kg_gemm_kernel<DT_BF16>, hipFuncAttributeMaxDynamicSharedMemorySize, KG_LDS);
+        if (e == hipSuccess) e = hipFuncSetAttribute((const void*)kg_gemm_kernel<DT_F16>, hipFuncAttributeMaxDynamicSharedMemorySize, KG_LDS);
+        if (e != hipSuccess) return (int)e;
+        attr_set = true;
+    }
     if (a.out_dtype == DT_BF16)
-        hipLaunchKernelGGL(kg_gemm_kernel<DT_BF16>, grid, dim3(512), 0, st, a8, b8, rs, s2p, ofp, (const float*)a.x1_scale, (uint16_t*)a.out, a.M, a.N,
-                           (int)L.Kp, (int)L.Np, (int)L.G);
+        hipLaunchKernelGGL(kg_gemm_kernel<DT_BF16>, grid, dim3(512), KG_LDS, st, a8, b8, (const float*)a.x1_scale, (uint16_t*)a.out, a.M, a.N, (int)L.G);
     else
-        hipLaunchKernelGGL(kg_gemm_kernel<DT_F16>, grid, dim3(512), 0, st, a8, b8, rs, s2p, ofp, (const float*)a.x1_scale, (uint16_t*)a.out, a.M, a.N,
-                           (int)L.Kp, (int)L.Np, (int)L.G);
+        hipLaunchKernelGGL(kg_gemm_kernel<DT_F16>, grid, dim3(512), KG_LDS, st, a8, b8, (const float*)a.x1_scale, (uint16_t*)a.out, a.M, a.N, (int)L.G);
     return (int)hipGetLastError();
 }
 

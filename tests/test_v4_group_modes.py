@@ -307,3 +307,49 @@ def test_gpu_i4_asym_kernel_level_ragged_shapes(gpu, M, K, N, variant):
     m.check(m.lib().aclrtSynchronizeDevice(), "sync")
     got = d_out.to_host(np.uint16, (M, N))
     assert np.array_equal(got, want), f"{int((got != want).sum())} of {got.size} outputs differ"
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("pattern", ["all_min", "min_with_units", "alternating", "sparse_units"])
+def test_gpu_i4_asym_extreme_group_sums(gpu, pattern):
+    """The matrix-core kernel multiplies the int4 operands as e4m3 bytes and takes the group sum from the matrix
+    pipe as fp32.  That is exact only if the pipe adds 256 products of magnitude up to 64 onto a running sum of up
+    to 16384 without dropping low bits: checked here on operands built to need every bit (largest products
+    throughout with a few products of magnitude 1 among them, sums that cancel, lone units), bit for bit against
+    the oracle's integer sums."""
+    m = gpu
+    M, K, N = 64, 1024, 256
+    print(f"case int4 K-G extreme sums pattern={pattern}", flush=True)
+    rng = np.random.default_rng(7)
+    inp = cases.make_i4_asym_inputs(m, M, K, N, 11)
+    a = np.full((M, K), 8, dtype=np.uint8)   # nibble 8 = -8
+    b = np.full((N, K), 8, dtype=np.uint8)
+    if pattern == "min_with_units":
+        # most products 64, a handful of +-1 and +-7 at random places of each row
+        for mat in (a, b):
+            idx = rng.integers(0, K, size=(mat.shape[0], 24))
+            vals = rng.choice(np.array([1, 15, 7, 9], dtype=np.uint8), size=idx.shape)
+            np.put_along_axis(mat, idx, vals, axis=1)
+    elif pattern == "alternating":
+        a[:, 1::2] = 7          # -8, 7, -8, 7 ... against -8 everywhere: +64 and -56 alternate
+        b[1::2, :] = 7          # and against 7 everywhere in every other column
+    elif pattern == "sparse_units":
+        a[:] = 0
+        b[:] = 0
+        for mat in (a, b):
+            idx = rng.integers(0, K, size=(mat.shape[0], 40))
+            np.put_along_axis(mat, idx, rng.choice(np.array([1, 15], dtype=np.uint8), size=idx.shape), axis=1)
+        a[:, ::256] = 8
+        b[:, ::256] = 8         # one product of 64 per group next to the units
+    inp["x1"], inp["x2"] = orc.pack_nibbles(a), orc.pack_nibbles(b)
+    if pattern in ("all_min", "min_with_units"):
+        # offset -8 takes the bulk (x2 = -8) out of every group: what is left of a group is the small integer
+        # sum x1 * (x2 + 8), so one lost unit of the group sum changes the output beyond any rounding
+        inp["off"] = orc.f32_to_f16(np.full(inp["off"].shape, -8.0, dtype=np.float32))
+    want = cases.oracle_i4_asym(m, inp, M, K, N, m.ACL_BF16)
+    got = cases.run_i4_asym_aclnn(m, inp, M, K, N, m.ACL_BF16)
+    assert np.array_equal(got, want), f"{int((got != want).sum())} of {got.size} outputs differ"
+    # the output rounds to bf16: compare the fp16 output too (three more bits of the fold's result)
+    want = cases.oracle_i4_asym(m, inp, M, K, N, m.ACL_FLOAT16)
+    got = cases.run_i4_asym_aclnn(m, inp, M, K, N, m.ACL_FLOAT16)
+    assert np.array_equal(got, want), f"{int((got != want).sum())} of {got.size} fp16 outputs differ"
