@@ -30,6 +30,12 @@
 #include "qgemm_core.hip.h"
 
 namespace opsnn {
+
+void* weight_cache_blob3(const void* src, const void* src2, const void* src3, int64_t K, int64_t N, int bits, int64_t nb, uint64_t bytes, hipStream_t st,
+                         bool* fresh);   // weight_cache.hip
+void weight_cache_commit(void* buffer, hipStream_t st);
+void weight_cache_abandon(void* buffer);
+
 namespace {
 
 constexpr int64_t KG_GROUP = 256, KG_TILE = 128;
@@ -52,30 +58,59 @@ bool kg_layout(const OpsnnQmmArgs& a, KgLayout& L)
     if (a.x2.row_stride != 1 || a.x2.col_stride % 2 != 0 || a.x2.col_stride < a.K) return false;
     if (a.K % 2 != 0 || a.M * a.N < 32 * 32) return false;
     L.Mp = kg_rup(a.M, KG_TILE); L.Np = kg_rup(a.N, KG_TILE); L.Kp = kg_rup(a.K, KG_GROUP); L.G = L.Kp / KG_GROUP;
+    if (L.G * ((L.Mp + L.Np) / 16 + (L.Np + 255) / 256) >= (1ll << 31)) return false;   // workgroups of the pre-step
     L.o_b = (uint64_t)(L.Mp / KG_TILE * L.G * KG_BLOCK);
     L.total = L.o_b + (uint64_t)(L.Np / KG_TILE * L.G * KG_BLOCK);
     return true;
 }
 
-// 16 int4 (8 bytes) of row r -> 16 e4m3 bytes in the block layout; rows past `rows` and columns past K become zero.
-// ld: elements between rows.  WITH_RS: the block's first side value array gets -fp32(sum of the row over the group)
-// (exact: at most 256 values of magnitude 8); the 16 threads of one row and group are neighbours in one wave.
-template <bool WITH_RS>
-__global__ __launch_bounds__(256) void kg_widen_kernel(const uint8_t* __restrict__ src, int64_t rows, int64_t K, int64_t ld,
-                                                       int8_t* __restrict__ dst, int64_t rows_p, int64_t Kp, int64_t G)
+struct KgPrepare {
+    const uint8_t* x[2];   // x1 [M, K] and x2 [N, K], K contiguous, two elements per byte
+    int64_t rows[2], ld[2], K;
+    int8_t* blocks[2];
+    int rows_p[2], G, Greal;
+    OpsnnMat sc, of;
+    int64_t N;
+    uint32_t first[3];   // first workgroup of the x2 blocks, of their side values, and the grid size
+};
+
+// The pre-step, one launch: the first workgroups write the x1 blocks, the next the x2 blocks, the last the side values
+// of the x2 blocks; within a role the group is the fastest index.  Operand roles: a workgroup takes 16 rows of one group, a thread 16 int4 (8 bytes) -> 16 e4m3
+// bytes in the block layout; rows past the operand's and columns past K become zero.  For x1 the 16 threads of a row
+// (neighbours in one wave) also add up its elements, and the block's first side value array gets -fp32(sum) (exact: at
+// most 256 values of magnitude 8).  Side value role: a thread takes one column: fp32 scale[g, n] and offset[g, n],
+// zeros for padded columns and groups.
+__global__ __launch_bounds__(256) void kg_prepare_kernel(KgPrepare p)
 {
-    const int64_t per_row = Kp / 16;   // a multiple of 16; rows_p * per_row is a multiple of the block size
-    const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    if (idx >= rows_p * per_row) return;
-    const int64_t r = idx / per_row, kc = idx - r * per_row, k0 = kc * 16;
+    const uint32_t bid = blockIdx.x;
+    const int role = bid >= p.first[1] ? 2 : bid >= p.first[0] ? 1 : 0, tid = threadIdx.x;
+    const uint32_t local = bid - (role == 2 ? p.first[1] : role == 1 ? p.first[0] : 0u);
+    const uint32_t bx = local / (uint32_t)p.G;
+    const int g = (int)(local - bx * (uint32_t)p.G);
+    if (role == 2) {
+        const int64_t n = (int64_t)bx * 256 + tid;
+        if (n >= p.rows_p[1]) return;
+        float s = 0.0f, o = 0.0f;
+        if (n < p.N && g < p.Greal) {
+            s = ((const float*)p.sc.ptr)[g * p.sc.row_stride + n * p.sc.col_stride];
+            o = load_scalar_as_f32(p.of.ptr, DT_F16, g * p.of.row_stride + n * p.of.col_stride);
+        }
+        float* side = (float*)(p.blocks[1] + ((n >> 7) * p.G + g) * KG_BLOCK + KG_ROWS);
+        side[n & 127] = s;
+        side[128 + (n & 127)] = o;
+        return;
+    }
+    const int64_t r = (int64_t)bx * 16 + (tid >> 4), K = p.K;
+    const int c = tid & 15;
+    const int64_t k0 = (int64_t)g * KG_GROUP + c * 16;
     uint64_t nib = 0;   // 16 nibbles, element k0 + e in bits [4 e, 4 e + 4)
-    if (r < rows && k0 < K) {
-        const uint8_t* p = src + ((r * ld + k0) >> 1);   // ld and k0 are even: the row piece starts on a byte
-        if (k0 + 16 <= K && ((uintptr_t)p & 7) == 0) nib = *(const uint64_t*)p;
+    if (r < p.rows[role] && k0 < K) {
+        const uint8_t* src = p.x[role] + ((r * p.ld[role] + k0) >> 1);   // ld and k0 are even: the row piece starts on a byte
+        if (k0 + 16 <= K && ((uintptr_t)src & 7) == 0) nib = *(const uint64_t*)src;
         else {
 #pragma unroll
             for (int b = 0; b < 8; b++)
-                if (k0 + 2 * b < K) nib |= (uint64_t)p[b] << (8 * b);   // K is even: both nibbles of the byte are inside the row
+                if (k0 + 2 * b < K) nib |= (uint64_t)src[b] << (8 * b);   // K is even: both nibbles of the byte are inside the row
         }
     }
     // e4m3 of the two's-complement nibble n: 0..7 -> 0, 1, 2, ... 7; 8..15 -> -8, -7, ... -1
@@ -89,30 +124,13 @@ __global__ __launch_bounds__(256) void kg_widen_kernel(const uint8_t* __restrict
         o[e / 4] |= f << (8 * (e % 4));
         s += (int32_t)(n ^ 8u) - 8;
     }
-    const int64_t g = kc >> 4, c = kc & 15;
-    int8_t* block = dst + ((r >> 7) * G + g) * KG_BLOCK;
+    int8_t* block = p.blocks[role] + ((r >> 7) * p.G + g) * KG_BLOCK;
     *(uint4*)(block + ((r & 127) << 8) + ((c ^ (r & 15)) << 4)) = make_uint4(o[0], o[1], o[2], o[3]);
-    if (WITH_RS) {
+    if (role == 0) {
 #pragma unroll
         for (int d = 8; d >= 1; d >>= 1) s += __shfl_xor(s, d, 16);
         if (c == 0) ((float*)(block + KG_ROWS))[r & 127] = -(float)s;
     }
-}
-
-// fp32 scale[g, n] and offset[g, n] into the side values of the x2 blocks (zeros for padded columns and groups)
-__global__ __launch_bounds__(256) void kg_scales_kernel(OpsnnMat sc, OpsnnMat of, int64_t N, int64_t Np, int64_t G, int64_t Greal, int8_t* __restrict__ dst)
-{
-    const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    if (idx >= G * Np) return;
-    const int64_t g = idx / Np, n = idx - g * Np;
-    float s = 0.0f, o = 0.0f;
-    if (n < N && g < Greal) {
-        s = ((const float*)sc.ptr)[g * sc.row_stride + n * sc.col_stride];
-        o = load_scalar_as_f32(of.ptr, DT_F16, g * of.row_stride + n * of.col_stride);
-    }
-    float* side = (float*)(dst + ((n >> 7) * G + g) * KG_BLOCK + KG_ROWS);
-    side[n & 127] = s;
-    side[128 + (n & 127)] = o;
 }
 
 template <int OUT_DT>
@@ -143,21 +161,11 @@ __global__ __launch_bounds__(512) void kg_gemm_kernel(const int8_t* __restrict__
         }
     };
 
-    v4f sum[FN][FM], tp[FN][FM];   // running sums; the previous group's integer sums, folded while this group is multiplied
-    float rsp[FM];
-    v4f s2q[FN], ofq[FN];
+    v4f sum[FN][FM];
 #pragma unroll
-    for (int i = 0; i < FN; i++) {
-        s2q[i] = ofq[i] = (v4f){0.0f, 0.0f, 0.0f, 0.0f};
+    for (int i = 0; i < FN; i++)
 #pragma unroll
-        for (int j = 0; j < FM; j++) sum[i][j] = tp[i][j] = (v4f){0.0f, 0.0f, 0.0f, 0.0f};
-    }
-#pragma unroll
-    for (int j = 0; j < FM; j++) rsp[j] = 0.0f;
-    auto fold = [&](int i, int j) {
-#pragma unroll
-        for (int r = 0; r < 4; r++) sum[i][j][r] = sum[i][j][r] + __builtin_fmaf(rsp[j], ofq[i][r], tp[i][j][r]) * s2q[i][r];
-    };
+        for (int j = 0; j < FM; j++) sum[i][j] = (v4f){0.0f, 0.0f, 0.0f, 0.0f};
 
 #pragma unroll
     for (int c = 0; c < 8; c++) copy_rows(0, 0, c);
@@ -171,7 +179,6 @@ __global__ __launch_bounds__(512) void kg_gemm_kernel(const int8_t* __restrict__
         const bool more = g + 1 < G;
         const char* la = lds + buf * BUF + (wm * 64 + frow) * 256;
         const char* lb = lds + buf * BUF + BLOCK + (wn * 32 + frow) * 256;
-        // this group's side values, for its fold during the next group (by then the buffer is being refilled)
         float rsv[FM];
         v4f s2v[FN], ofv[FN];
 #pragma unroll
@@ -203,30 +210,21 @@ __global__ __launch_bounds__(512) void kg_gemm_kernel(const int8_t* __restrict__
 #pragma unroll
                 for (int c = 0; c < 4; c++) copy_rows(g + 1, buf ^ 1, 4 * s + c);
             }
+            // t[i][j][r] becomes the group's integer sum for m = 16 j + lane % 16, n = 16 i + 4 (lane / 16) + r of the wave tile;
+            // a fragment pair is folded as soon as its second instruction is out, in the shadow of the following ones
 #pragma unroll
             for (int i = 0; i < FN; i++)
 #pragma unroll
                 for (int j = 0; j < FM; j++) {
                     t[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(fb[i], fa[j], s == 0 ? (v4f){0.0f, 0.0f, 0.0f, 0.0f} : t[i][j], 0, 0, 0,
                                                                                0x7f7f7f7f, 0, 0x7f7f7f7f);
-                    if (i == s) fold(i, j);   // half of the previous group's fold in the shadow of each step
+                    if (s == 1) {
+#pragma unroll
+                        for (int r = 0; r < 4; r++) sum[i][j][r] = sum[i][j][r] + __builtin_fmaf(rsv[j], ofv[i][r], t[i][j][r]) * s2v[i][r];
+                    }
                 }
         }
-        // t[i][j][r] is the group's integer sum for m = 16 j + lane % 16, n = 16 i + 4 (lane / 16) + r of the wave tile
-#pragma unroll
-        for (int i = 0; i < FN; i++) {
-            s2q[i] = s2v[i];
-            ofq[i] = ofv[i];
-#pragma unroll
-            for (int j = 0; j < FM; j++) tp[i][j] = t[i][j];
-        }
-#pragma unroll
-        for (int j = 0; j < FM; j++) rsp[j] = rsv[j];
     }
-#pragma unroll
-    for (int i = 0; i < FN; i++)
-#pragma unroll
-        for (int j = 0; j < FM; j++) fold(i, j);
 
     const bool vec_ok = (N % 4) == 0 && ((uintptr_t)out % 8) == 0;
 #pragma unroll
@@ -263,15 +261,33 @@ int launch_kg_mfma(const OpsnnQmmArgs& a, hipStream_t st)
 {
     KgLayout L;
     if (!kg_layout(a, L) || !a.workspace || (uintptr_t)a.workspace % 16 != 0) return OPSNN_NOT_TAKEN;
+    // The x2 blocks depend on the weights, their scales and their offsets only: with the weight cache on they are
+    // written by the first call and found by the later ones.
     int8_t* a8 = (int8_t*)a.workspace;
     int8_t* b8 = a8 + L.o_b;
-    const int64_t Greal = (a.K + KG_GROUP - 1) / KG_GROUP;
-    auto blocks = [](int64_t n) { return dim3((unsigned)((n + 255) / 256)); };
-    hipLaunchKernelGGL(kg_widen_kernel<true>, blocks(L.Mp * (L.Kp / 16)), dim3(256), 0, st, (const uint8_t*)a.x1.ptr, a.M, a.K, a.x1.row_stride, a8, L.Mp,
-                       L.Kp, L.G);
-    hipLaunchKernelGGL(kg_widen_kernel<false>, blocks(L.Np * (L.Kp / 16)), dim3(256), 0, st, (const uint8_t*)a.x2.ptr, a.N, a.K, a.x2.col_stride, b8, L.Np,
-                       L.Kp, L.G);
-    hipLaunchKernelGGL(kg_scales_kernel, blocks(L.G * L.Np), dim3(256), 0, st, a.x2_scale_mat, a.x2_offset_mat, a.N, L.Np, L.G, Greal, b8);
+    bool fresh = false;
+    const bool dense = a.x2.col_stride == a.K && a.x2_scale_mat.row_stride == a.N && a.x2_scale_mat.col_stride == 1 &&
+                       a.x2_offset_mat.row_stride == a.N && a.x2_offset_mat.col_stride == 1;   // what the cache key does not tell apart
+    void* cached = dense ? weight_cache_blob3(a.x2.ptr, a.x2_scale_mat.ptr, a.x2_offset_mat.ptr, a.K, a.N, 4, 1, L.total - L.o_b, st, &fresh) : nullptr;
+    if (cached) b8 = (int8_t*)cached;
+    KgPrepare p;
+    p.x[0] = (const uint8_t*)a.x1.ptr; p.x[1] = (const uint8_t*)a.x2.ptr;
+    p.rows[0] = a.M; p.rows[1] = a.N;
+    p.ld[0] = a.x1.row_stride; p.ld[1] = a.x2.col_stride;
+    p.K = a.K;
+    p.blocks[0] = a8; p.blocks[1] = b8;
+    p.rows_p[0] = (int)L.Mp; p.rows_p[1] = (int)L.Np;
+    p.G = (int)L.G; p.Greal = (int)((a.K + KG_GROUP - 1) / KG_GROUP);
+    p.sc = a.x2_scale_mat; p.of = a.x2_offset_mat;
+    p.N = a.N;
+    const bool x1_only = cached && !fresh;
+    const int64_t wg0 = L.G * (L.Mp / 16), wg1 = x1_only ? 0 : L.G * (L.Np / 16), wg2 = x1_only ? 0 : L.G * ((L.Np + 255) / 256);
+    p.first[0] = (uint32_t)wg0; p.first[1] = (uint32_t)(wg0 + wg1); p.first[2] = (uint32_t)(wg0 + wg1 + wg2);
+    hipLaunchKernelGGL(kg_prepare_kernel, dim3(p.first[2]), dim3(256), 0, st, p);
+    if (cached && fresh) {
+        if (hipGetLastError() != hipSuccess) { weight_cache_abandon(cached); return (int)hipErrorLaunchFailure; }
+        weight_cache_commit(cached, st);
+    }
     const dim3 grid((unsigned)(L.Np / KG_TILE), (unsigned)(L.Mp / KG_TILE));
     constexpr int KG_LDS = 2 * 2 * (int)KG_BLOCK;
     static bool attr_set = false;

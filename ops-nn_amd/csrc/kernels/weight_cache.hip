@@ -25,7 +25,7 @@ namespace opsnn {
 namespace {
 
 struct Entry {
-    const void* src; const void* src2; int64_t K, N, nb; int bits;
+    const void* src; const void* src2; const void* src3; int64_t K, N, nb; int bits;
     void* copy; uint64_t bytes; hipEvent_t ready; int device;
     bool committed;   // filled and its event recorded; until then other callers do not use it
 };
@@ -45,11 +45,13 @@ void drop(std::list<Entry>::iterator it)
 
 }  // namespace
 
-// A buffer of `bytes` that belongs to the operand (src, src2 -- e.g. data and scales --, shape, element width, batch count):
+// A buffer of `bytes` that belongs to the operand (src, src2, src3 -- e.g. data, scales and offsets --, shape, element width,
+// batch count):
 // on a hit (*fresh = false) it holds what an earlier call put there and is ordered behind that call's writes on `st`; on a
 // miss (*fresh = true) it is new: the caller fills it with launches on `st` and then calls weight_cache_commit(buffer, st).
 // nullptr when the cache does not serve this call (off, under graph capture, larger than the limit, allocation failure).
-void* weight_cache_blob(const void* src, const void* src2, int64_t K, int64_t N, int bits, int64_t nb, uint64_t bytes, hipStream_t st, bool* fresh)
+void* weight_cache_blob3(const void* src, const void* src2, const void* src3, int64_t K, int64_t N, int bits, int64_t nb, uint64_t bytes, hipStream_t st,
+                         bool* fresh)
 {
     *fresh = false;
     if (!g_limit || !src || K <= 0 || N <= 0 || nb <= 0 || !bytes) return nullptr;
@@ -59,7 +61,7 @@ void* weight_cache_blob(const void* src, const void* src2, int64_t K, int64_t N,
     if (hipGetDevice(&dev) != hipSuccess) return nullptr;
     std::lock_guard<std::mutex> lock(g_mu);
     for (auto it = g_entries.begin(); it != g_entries.end(); ++it) {
-        if (it->src == src && it->src2 == src2 && it->K == K && it->N == N && it->bits == bits && it->nb == nb && it->bytes == bytes &&
+        if (it->src == src && it->src2 == src2 && it->src3 == src3 && it->K == K && it->N == N && it->bits == bits && it->nb == nb && it->bytes == bytes &&
             it->device == dev) {
             if (!it->committed) return nullptr;   // another call is still filling it: this one goes its own way
             if (hipStreamWaitEvent(st, it->ready, 0) != hipSuccess) return nullptr;
@@ -70,7 +72,7 @@ void* weight_cache_blob(const void* src, const void* src2, int64_t K, int64_t N,
     }
     if (bytes > g_limit) return nullptr;
     while (g_used + bytes > g_limit && !g_entries.empty()) drop(std::prev(g_entries.end()));
-    Entry e{src, src2, K, N, nb, bits, nullptr, bytes, nullptr, dev, false};
+    Entry e{src, src2, src3, K, N, nb, bits, nullptr, bytes, nullptr, dev, false};
     if (hipMalloc(&e.copy, bytes) != hipSuccess) { (void)hipGetLastError(); return nullptr; }
     if (hipEventCreateWithFlags(&e.ready, hipEventDisableTiming) != hipSuccess) { (void)hipFree(e.copy); return nullptr; }
     // until the commit nobody else uses the entry; one whose filling call fails is removed by weight_cache_abandon
@@ -79,6 +81,11 @@ void* weight_cache_blob(const void* src, const void* src2, int64_t K, int64_t N,
     g_entries.push_front(e);
     *fresh = true;
     return e.copy;
+}
+
+void* weight_cache_blob(const void* src, const void* src2, int64_t K, int64_t N, int bits, int64_t nb, uint64_t bytes, hipStream_t st, bool* fresh)
+{
+    return weight_cache_blob3(src, src2, nullptr, K, N, bits, nb, bytes, st, fresh);
 }
 
 // The fresh buffer has been filled by the launches already enqueued on st.

@@ -344,10 +344,11 @@ class ConfigWQ(Workload):
 
 class ConfigKG(Workload):
     """Not a BASELINE config: aclnnQuantMatmulV5 in the int4 x int4 mode with per-group (256 K) scales and offsets of x2
-    ("K-G" of quant_batch_matmul_v4), 4096 x 4096 x 4096, bf16 output.  The operands are widened to int8 in the workspace
-    by every call (four small kernels before the matrix kernel): they are inside the timed step."""
-    peak_key, dtype = "int8", "int8 (int4 operands widened)"
-    kernel = "kg_gemm_kernel (+ kg_widen / kg_rowsum / kg_scales pre-steps)"
+    ("K-G" of quant_batch_matmul_v4), 4096 x 4096 x 4096, bf16 output.  Every call rewrites the operands as e4m3 bytes
+    in the workspace (one kernel before the matrix kernel; with --weight-cache the x2 half of it only on the first call):
+    that is inside the timed step."""
+    peak_key, dtype = "fp8", "fp8 e4m3 (int4 operands, exact)"
+    kernel = "kg_gemm_kernel (+ kg_prepare_kernel)"
 
     def __init__(self, m, args, M=4096, K=4096, N=4096):
         self.m, self.M, self.K, self.N = m, M, K, N

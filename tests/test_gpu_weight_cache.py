@@ -112,3 +112,38 @@ def test_mx_operand_and_its_scales_are_re_laid_out_once(cache):
     assert np.array_equal(first, want)
     e1, _, h1, m1 = _stats(m)
     assert (m1 - m0, h1 - h0) == (1, 0) and e1 - e0 == 1
+
+
+def test_int4_group_mode_x2_blocks_are_written_once(cache):
+    """int4 x int4 with group scales and offsets: the x2 half of the pre-step (e4m3 blocks with their scales and offsets)
+    is kept; x1 is rewritten by every call, so a second call with other activations is still right."""
+    m = cache
+    M, K, N = 130, 1024, 512
+    print(f"case weight cache, int4 K-G {M}x{K}x{N}", flush=True)
+    inp = cases.make_i4_asym_inputs(m, M, K, N, 5)
+    want = cases.oracle_i4_asym(m, inp, M, K, N, m.ACL_BF16)
+    d = {k: m.DeviceBuffer(host=v) for k, v in inp.items()}
+    d_out = m.DeviceBuffer(M * N * 2)
+    t = dict(x1=m.Tensor((M, K), m.ACL_INT4, d["x1"]), x2=m.Tensor((N, K), m.ACL_INT4, d["x2"]),
+             s1=m.Tensor(inp["s1"].shape, m.ACL_FLOAT, d["s1"]), s2=m.Tensor(inp["s2"].shape, m.ACL_FLOAT, d["s2"]),
+             off=m.Tensor(inp["off"].shape, m.ACL_FLOAT16, d["off"]), out=m.Tensor((M, N), m.ACL_BF16, d_out))
+
+    def call():
+        ws = m.quant_matmul_v5(t["x1"], t["x2"], t["s1"], t["s2"], t["out"], x2_offset=t["off"], transpose_x2=True, group_size=256)
+        m.check(m.lib().aclrtSynchronizeDevice(), "sync")
+        del ws
+        return d_out.to_host(np.uint16, (M, N))
+
+    e0, _, h0, m0 = _stats(m)
+    first = call()
+    second = call()
+    e1, _, h1, m1 = _stats(m)
+    assert (e1 - e0, m1 - m0, h1 - h0) == (1, 1, 1)
+    assert np.array_equal(first, want) and np.array_equal(second, want)
+    # other activations against the kept x2 blocks
+    inp2 = cases.make_i4_asym_inputs(m, M, K, N, 6)
+    d["x1"].upload(inp2["x1"])
+    inp2.update(x2=inp["x2"], s2=inp["s2"], off=inp["off"], s1=inp["s1"])
+    third = call()
+    assert np.array_equal(third, cases.oracle_i4_asym(m, inp2, M, K, N, m.ACL_BF16))
+    assert _stats(m)[2] - h0 == 2
