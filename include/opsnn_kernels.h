@@ -144,8 +144,9 @@ OPSNN_API int opsnnQmmTc(const OpsnnQmmArgs* a, void* stream);
 OPSNN_API int opsnnQmmGroup(const OpsnnQmmArgs* a, void* stream);
 /* Device workspace bytes a launcher needs for these arguments (0 if none).  mode names the entry point the arguments
  * are for: 0 opsnnQmmInt8, 1 opsnnQmmBlockScale, 2 opsnnQmmMx, 3 opsnnQmmTc, 4 opsnnQmmGroup (the fp8 x fp4 mode's
- * re-quantised weight, N * K bytes plus the decoded output scale, or the int4 mode's operands widened to int8 and padded
- * to whole tiles with their row sums and fp32 scale / offset copies, when the mode's matrix-core path applies). */
+ * re-quantised weight, N * K bytes plus the decoded output scale, or the int4 mode's operands rewritten as e4m3 bytes in
+ * tile blocks padded to whole tiles, each with its row sums or fp32 scales and offsets, when the mode's matrix-core path
+ * applies). */
 OPSNN_API uint64_t opsnnQmmWorkspace(const OpsnnQmmArgs* a, int mode);
 
 typedef struct {

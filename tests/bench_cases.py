@@ -30,7 +30,7 @@ PROFILED_TRAFFIC = {
     (4, None, "exact"): (1220.2e6, "profiles/qmm_fp8_exact_m4096_k7168_n18432.txt"),
     (4, None, "fast"): (1502.4e6, "profiles/qmm_fp8_block_m4096_k7168_n18432.txt"),
     (5, None, None): (3083.5e6, "profiles/qgemm_mxfp4_b8_m4096_k8192_n8192.txt"),
-    (10, None, None): (280.7e6, "profiles/qmm_i4_kg_m4096_k4096_n4096.txt"),
+    (10, None, None): (290.3e6, "profiles/qmm_i4_kg_m4096_k4096_n4096.txt"),
     (11, 16, "warm"): (133.6e6, "profiles/wqmm_decode_mxfp4_m16_k8192_n28672.txt"),
 }
 
