@@ -368,6 +368,26 @@ static int launch_slabs_float(WqParams p, hipStream_t st)
             if (rc != OPSNN_NOT_TAKEN) return rc;
         }
     }
+    // more rows: the many-rows streaming kernel, up to 128 rows per pass over the weights, in equal slabs
+    {
+        constexpr int64_t KC = 4 * (128 / WBITS);
+        static const int rows_min = [] { const char* e = getenv("OPSNN_WQ_ROWS_MIN"); return e ? atoi(e) : 17; }();
+        bool ok = !p.offset && p.M >= rows_min && p.K % KC == 0 && (p.K / KC) % 8 == 0 && p.N % 32 == 0 && p.N >= 256;
+        if (WBITS == 4) ok = ok && p.scale_e8m0 && p.group == 32 && p.s_rs == 1;
+        else ok = ok && !p.scale_e8m0 && p.group >= p.K;
+        if (ok) {
+            const int64_t passes = (p.M + 127) / 128;
+            const int64_t slab = ((p.M + passes - 1) / passes + 15) / 16 * 16;
+            p.cpg_shift = 31;
+            for (int64_t m0 = 0; m0 < p.M; m0 += slab) {
+                p.m_base = m0;
+                p.m_rows = (p.M - m0) < slab ? (p.M - m0) : slab;
+                const int rc = launch_wq_rows_float<XDT, WBITS>(p, st);
+                if (rc != 0) return rc;
+            }
+            return 0;
+        }
+    }
     for (int64_t m0 = 0; m0 < p.M; m0 += 64) {
         p.m_base = m0;
         p.m_rows = (p.M - m0) < 64 ? (p.M - m0) : 64;

@@ -107,13 +107,19 @@ __device__ __forceinline__ v4i dequant8(const v4i& piece, int s, uint16_t sb, ui
 }
 
 // ---- 8 floating-point weight codes of one lane -> MFMA row operand ----
-// WBITS 4: the e2m1 codes of dword s, delivered in element order [0,4,1,5,2,6,3,7] like dequant8's int4 form; WBITS 8:
-// the e4m3 codes of dwords 2s, 2s+1 in natural order.  Every code is exact in fp16 and in bf16, so T(w * scale) rounds
-// once, in the multiplication: packed fp16 for fp16; for bf16 the exact fp16 value is widened to fp32, multiplied and
-// rounded to bf16 by the hardware conversion.
-template <int XDT, int WBITS>
+// WBITS 4: the e2m1 codes of dword s, delivered in element order [0,4,1,5,2,6,3,7] like dequant8's int4 form (NATURAL:
+// in element order, four byte permutes more); WBITS 8: the e4m3 codes of dwords 2s, 2s+1 in natural order.  Every code
+// is exact in fp16 and in bf16, so T(w * scale) rounds once, in the multiplication: packed fp16 for fp16; for bf16 the
+// exact fp16 value is widened to fp32, multiplied and rounded to bf16 by the hardware conversion.
+template <int XDT, int WBITS, bool NATURAL = false>
 __device__ __forceinline__ v4i dequant8_float(const v4i& piece, int s, uint16_t sb)
 {
+    if constexpr (NATURAL && WBITS == 4) {
+        const v4i r = dequant8_float<XDT, WBITS, false>(piece, s, sb);   // halves (0,4) (1,5) (2,6) (3,7)
+        const uint32_t a = (uint32_t)r[0], b = (uint32_t)r[1], c = (uint32_t)r[2], d = (uint32_t)r[3];
+        return (v4i){(int)__builtin_amdgcn_perm(b, a, 0x05040100u), (int)__builtin_amdgcn_perm(d, c, 0x05040100u),
+                     (int)__builtin_amdgcn_perm(b, a, 0x07060302u), (int)__builtin_amdgcn_perm(d, c, 0x07060302u)};
+    }
     h2 w[4];   // the eight weights, exact, as fp16 pairs
     if constexpr (WBITS == 4) {
         const uint32_t q = (uint32_t)piece[s];
@@ -402,10 +408,15 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(NW == 8
 // Scale and offset of a chunk travel with its weights (one 16-bit load each per row block).
 // The launcher guarantees: N % (16 * NB) == 0, (K / KC) % (WK * PF) == 0, group a power-of-two multiple of KC or
 // per channel, x rows 16-byte aligned.
-template <int XDT, int WBITS, int MB, int NB, int WN, int WK, bool HAS_OFF>
+// WF: 0 integer codes; 1 floating-point codes (e4m3) with one scale of x's type per channel; 2 e2m1 codes with e8m0
+// scales per 32 k, a row's scale bytes contiguous: a lane's 32 weights of a chunk are exactly one group, so its scale
+// is one byte per chunk, fetched with the weights like the 16-bit scales of the other forms.
+template <int XDT, int WBITS, int MB, int NB, int WN, int WK, bool HAS_OFF, int WF = 0>
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void wqmm_rows_kernel(WqParams p)
 {
     static_assert(WN * WK == 8, "eight waves");
+    static_assert(WF == 0 || !HAS_OFF, "floating-point weight codes have no offset");
+    static_assert(WF != 2 || WBITS == 4, "e8m0 group scales go with e2m1 codes");
     constexpr int NT = 512;
     constexpr int KPL = 128 / WBITS, KC = 4 * KPL, STEPS = KC / 32;
     constexpr int PF = 8 / NB;           // of this wave's chunks in flight per row block (a chunk is 500 to 1000 clocks of MFMA work here)
@@ -434,6 +445,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void w
     const uint16_t* srow = p.scale + (n0 + nrow) * p.s_cs;
     const uint16_t* orow = HAS_OFF ? p.offset + (n0 + nrow) * p.s_cs : nullptr;
     const int64_t sblk = 16 * p.s_cs;
+    const uint8_t* srow8 = (const uint8_t*)p.scale + (n0 + nrow) * p.s_cs + g;   // WF 2: the byte of this lane's group in chunk 0
 
     // x copies: instruction `it` of this thread fills LDS piece it*NT + tid of the buffer, i.e. position
     // (it*NT + tid) % XPR of row (it*NT + tid) / XPR, with the row's piece position ^ (row % 16)
@@ -474,7 +486,8 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void w
 #pragma unroll
         for (int q = 0; q < NB; q++) {
             wq[j][q] = *(const v4i*)(wptr + q * wblk + (int64_t)cw * (WK * 64));
-            sq[j][q] = srow[q * sblk + so];
+            if constexpr (WF == 2) sq[j][q] = srow8[q * sblk + (cw * WK + wk) * 4];
+            else sq[j][q] = srow[q * sblk + so];
             if constexpr (HAS_OFF) oq[j][q] = orow[q * sblk + so];
             else oq[j][q] = 0;
         }
@@ -497,7 +510,11 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void w
             for (int s = 0; s < STEPS; s++) {
                 v4i aop[NB];
 #pragma unroll
-                for (int q = 0; q < NB; q++) aop[q] = dequant8<XDT, WBITS, HAS_OFF, true>(wq[j][q], s, sq[j][q], oq[j][q], dqc);
+                for (int q = 0; q < NB; q++) {
+                    if constexpr (WF == 0) aop[q] = dequant8<XDT, WBITS, HAS_OFF, true>(wq[j][q], s, sq[j][q], oq[j][q], dqc);
+                    else if constexpr (WF == 1) aop[q] = dequant8_float<XDT, WBITS, true>(wq[j][q], s, sq[j][q]);
+                    else aop[q] = dequant8_float<XDT, WBITS, true>(wq[j][q], s, bits_x<XDT>(e8m0_to_f32(sq[j][q])));
+                }
 #pragma unroll
                 for (int b = 0; b < MB; b++) {
                     const v4i bop = *(const v4i*)(xs + (xoff[b] ^ (16 * s)));
@@ -1090,7 +1107,7 @@ static int launch_stream_one(const WqParams& p, hipStream_t st)
     return (int)hipGetLastError();
 }
 
-template <int XDT, int WBITS, int MB, int NB, int WN, int WK, bool HAS_OFF>
+template <int XDT, int WBITS, int MB, int NB, int WN, int WK, bool HAS_OFF, int WF = 0>
 static int launch_rows_one(const WqParams& p, hipStream_t st)
 {
     constexpr int KC = 4 * (128 / WBITS);
@@ -1098,7 +1115,7 @@ static int launch_rows_one(const WqParams& p, hipStream_t st)
     constexpr size_t lds_red = (size_t)WN * (WK - 1) * NB * MB * 4 * 64 * 4;
     constexpr size_t lds = lds_x > lds_red ? lds_x : lds_red;
     const unsigned grid = (unsigned)((p.N + 16 * NB * WN - 1) / (16 * NB * WN));
-    auto k = wqmm_rows_kernel<XDT, WBITS, MB, NB, WN, WK, HAS_OFF>;
+    auto k = wqmm_rows_kernel<XDT, WBITS, MB, NB, WN, WK, HAS_OFF, WF>;
     static bool attr_set = false;
     if (!attr_set) {
         hipError_t e = hipFuncSetAttribute((const void*)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
@@ -1123,10 +1140,21 @@ int launch_wq_stream(const WqParams& p, const WqStreamOpts& o, hipStream_t st);
 // Up to 16 rows, floating-point weight codes (see launch_xreg_float); OPSNN_NOT_TAKEN if K does not split.
 template <int XDT, int WBITS>
 int launch_wq_xreg_float(const WqParams& p, hipStream_t st);
+// One row slab of up to 128 rows, floating-point weight codes, on the many-rows kernel (WBITS 4: mxfp4 with a row's
+// e8m0 bytes contiguous; 8: e4m3 with per-channel scales).  The caller has checked the kernel's shape conditions.
+template <int XDT, int WBITS>
+int launch_wq_rows_float(const WqParams& p, hipStream_t st);
 
 #define OPSNN_WQ_STREAM_DEFINE(XDT, WBITS)                                                                          \
     template <>                                                                                                     \
     int launch_wq_xreg_float<XDT, WBITS>(const WqParams& p, hipStream_t st) { return launch_xreg_float<XDT, WBITS>(p, st); } \
+    template <>                                                                                                     \
+    int launch_wq_rows_float<XDT, WBITS>(const WqParams& p, hipStream_t st)                                         \
+    {                                                                                                               \
+        constexpr int WF = WBITS == 4 ? 2 : 1;                                                                      \
+        return p.m_rows > 64 ? launch_rows_one<XDT, WBITS, 8, 2, 4, 2, false, WF>(p, st)                            \
+                             : launch_rows_one<XDT, WBITS, 4, 2, 4, 2, false, WF>(p, st);                           \
+    }                                                                                                               \
     template <int MB, int NW, int WK, bool VS>                                                                      \
     static int wq_stream_off(const WqParams& p, bool has_off, hipStream_t st)                                       \
     {                                                                                                               \

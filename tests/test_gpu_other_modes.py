@@ -314,6 +314,33 @@ def test_weight_only_x_in_registers_kernel(gpu, M, K, N, x_dt, w_dt, group, tW, 
     check_close(got, want, dt[x_dt], "weight-only, x in registers")
 
 
+@pytest.mark.parametrize("M,K,N,x_dt,w_dt,group,bias", [
+    # mxfp4 (K % 1024 == 0, N % 32 == 0, N >= 256; 17 rows and more): up to 64 rows, up to 128 rows (the 8-block form), two passes of equal
+    # slabs, ragged last row block of x, both activation types, a bias
+    (17, 1024, 256, "bf16", "fp4", 32, None),
+    (40, 2048, 256, "f16", "fp4", 32, None),
+    (64, 8192, 512, "bf16", "fp4", 32, "bf16"),
+    (100, 4096, 288, "f16", "fp4", 32, "f16"),
+    (128, 1024, 1024, "bf16", "fp4", 32, None),
+    (200, 2048, 320, "f16", "fp4", 32, None),
+    # e4m3 with per-channel scales (K % 512 == 0)
+    (48, 512, 256, "bf16", "e4m3", 0, None),
+    (96, 4096, 544, "f16", "e4m3", 0, "f16"),
+    (130, 1536, 256, "bf16", "e4m3", 0, "bf16"),
+])
+def test_weight_only_float_codes_on_the_many_rows_kernel(gpu, M, K, N, x_dt, w_dt, group, bias):
+    """17 rows of x and more against mxfp4 / e4m3 weights: the many-rows streaming kernel (two weight blocks per wave
+    share every x fragment; a lane's 32 e2m1 codes of a chunk are one MX group, so its e8m0 byte travels with them)."""
+    m = gpu
+    dt = {"bf16": m.ACL_BF16, "f16": m.ACL_FLOAT16, "e4m3": m.ACL_FLOAT8_E4M3FN, "fp4": m.ACL_FLOAT4_E2M1, None: None}
+    print(f"case wq float codes, many rows M={M} K={K} N={N} x={x_dt} w={w_dt} g={group} bias={bias}", flush=True)
+    inp = cases.make_wq_inputs(m, M, K, N, M * 3 + N, dt[x_dt], dt[w_dt], group, True, False, dt[bias])
+    want = cases.oracle_wq(m, inp, M, K, N)
+    plain(False)
+    got = cases.run_wq_aclnn(m, inp, M, K, N)
+    check_close(got, want, dt[x_dt], "weight-only float codes, many rows")
+
+
 @pytest.mark.parametrize("M,K,N,x_dt,w_dt,tW,off,bias", [
     (16, 4096, 256, "f16", "i8", True, True, None),        # one scale and offset for the whole tensor, 16 waves x 4 chunks
     (9, 8192, 100, "f16", "i4", True, True, "f16"),        # ragged columns, per tensor, a bias
