@@ -11,7 +11,9 @@
 // Fast paths: operands and scales K-contiguous, K % 128 == 0, 16-bit output.  fp4: qgemm_core.hip.h, MODE_MXFP4
 // (K % 512 == 0 takes 256-element K tiles, otherwise 128-element ones); fp8: the MX mode of the kernel in
 // qmm_fp8_block.hip.  An N-contiguous x2 (data [K, N], scales [K/64, N, 2]) is first re-laid out into the
-// workspace; everything else runs the plain kernel.
+// workspace.  K % 128 == 64 with K-contiguous operands: both operands and both scale tables are first copied into
+// the workspace with one more scale pair per row, the new elements zero and their scales 2^0 (zero products change
+// no sum).  Everything else runs the plain kernel.
 #include "launch.h"
 #include "qgemm_core.hip.h"
 
@@ -50,9 +52,88 @@ extern "C" int opsnnTranspose16(const void* src, void* dst, int64_t rows, int64_
 namespace opsnn {
 
 static inline uint64_t align_up(uint64_t v, uint64_t a) { return (v + a - 1) / a * a; }
+extern "C" bool opsnn_force_plain();   // dispatch.hip
+
+// ---- K % 128 == 64 ----
+// rows of kb bytes (pitch ld) -> rows of kbp bytes, the tail filled with the byte `fill`; E = bytes per thread
+template <int E>
+__global__ __launch_bounds__(256) void mx_pad_rows_kernel(const uint8_t* __restrict__ src, int64_t ld, int64_t bs, uint8_t* __restrict__ dst,
+                                                          int64_t rows, int64_t kb, int64_t kbp, uint32_t fill)
+{
+    const int64_t c = (int64_t)blockIdx.x * 64 + (threadIdx.x & 63), r = (int64_t)blockIdx.y * 4 + (threadIdx.x >> 6);
+    if (c * E >= kbp || r >= rows) return;
+    const uint8_t* s = src + (int64_t)blockIdx.z * bs + r * ld + c * E;
+    uint8_t* d = dst + ((int64_t)blockIdx.z * rows + r) * kbp + c * E;
+    if constexpr (E == 16) *(uint4*)d = c * E < kb ? *(const uint4*)s : make_uint4(fill, fill, fill, fill);
+    else *(uint16_t*)d = c * E < kb ? *(const uint16_t*)s : (uint16_t)fill;
+}
+
+struct MxPad {
+    int64_t Kp, nb1, nb2, snb1, snb2;
+    uint64_t o_x2, o_s1, o_s2, total;
+};
+
+// Whether the padding pre-step serves this call, and its workspace layout.
+static bool mx_pad_layout(const OpsnnQmmArgs& a, MxPad& L)
+{
+    const bool fp4 = a.x1_dtype == DT_E2M1 && a.x2_dtype == DT_E2M1, fp8 = a.x1_dtype == DT_E4M3 && a.x2_dtype == DT_E4M3;
+    if ((!fp4 && !fp8) || a.K % 128 != 64 || a.M * a.N < 64 * 64) return false;
+    if (a.out_dtype != DT_BF16 && a.out_dtype != DT_F16) return false;
+    if (a.bias && a.bias_dtype != DT_F32) return false;
+    const int64_t epb = fp4 ? 2 : 1, ks = a.K / 64;
+    if (a.x1.col_stride != 1 || a.x2.row_stride != 1) return false;
+    if (a.x1_scale_mat.col_stride != 2 || a.x1_scale_mat.row_stride != ks * 2) return false;
+    if (a.x2_scale_mat.col_stride != 2 || a.x2_scale_mat.row_stride != ks * 2) return false;
+    if (a.x1.batch_stride < 0 || a.x2.batch_stride < 0 || a.x1_scale_mat.batch_stride < 0 || a.x2_scale_mat.batch_stride < 0) return false;
+    // 16-byte pieces of the data rows, 2-byte pieces of the scale rows
+    if (((uintptr_t)a.x1.ptr | (uintptr_t)a.x2.ptr | (uint64_t)(a.x1.row_stride / epb) | (uint64_t)(a.x2.col_stride / epb) |
+         (uint64_t)(a.x1.batch_stride / epb) | (uint64_t)(a.x2.batch_stride / epb)) % 16) return false;
+    if (((uintptr_t)a.x1_scale_mat.ptr | (uintptr_t)a.x2_scale_mat.ptr | (uint64_t)a.x1_scale_mat.batch_stride | (uint64_t)a.x2_scale_mat.batch_stride) % 2) return false;
+    if ((a.M + 3) / 4 > 65535 || (a.N + 3) / 4 > 65535) return false;
+    L.Kp = a.K + 64;
+    L.nb1 = a.x1.batch_stride == 0 && a.batch > 1 ? 1 : a.batch;
+    L.nb2 = a.x2.batch_stride == 0 ? 1 : a.batch;
+    L.snb1 = a.x1_scale_mat.batch_stride == 0 && a.batch > 1 ? 1 : a.batch;
+    L.snb2 = a.x2_scale_mat.batch_stride == 0 ? 1 : a.batch;
+    const uint64_t ksp = (uint64_t)L.Kp / 64;
+    L.o_x2 = align_up((uint64_t)L.nb1 * a.M * (L.Kp / epb), 256);
+    L.o_s1 = L.o_x2 + align_up((uint64_t)L.nb2 * a.N * (L.Kp / epb), 256);
+    L.o_s2 = L.o_s1 + align_up((uint64_t)L.snb1 * a.M * ksp * 2, 256);
+    L.total = L.o_s2 + align_up((uint64_t)L.snb2 * a.N * ksp * 2, 256);
+    return true;
+}
+
+// Launches the four copies and rewrites `a` as the same call on the padded operands.
+static int mx_pad_prestep(OpsnnQmmArgs& a, const MxPad& L, hipStream_t st)
+{
+    if (!a.workspace || (uintptr_t)a.workspace % 16) return OPSNN_NOT_TAKEN;
+    const bool fp4 = a.x1_dtype == DT_E2M1;
+    const int64_t epb = fp4 ? 2 : 1, kb = a.K / epb, kbp = L.Kp / epb, ks2 = a.K / 64 * 2, ksp2 = L.Kp / 64 * 2;
+    uint8_t* w = (uint8_t*)a.workspace;
+    auto grid = [](int64_t pieces, int64_t rows, int64_t nb) { return dim3((unsigned)((pieces + 63) / 64), (unsigned)((rows + 3) / 4), (unsigned)nb); };
+    hipLaunchKernelGGL(mx_pad_rows_kernel<16>, grid(kbp / 16, a.M, L.nb1), dim3(256), 0, st, (const uint8_t*)a.x1.ptr, a.x1.row_stride / epb,
+                       a.x1.batch_stride / epb, w, a.M, kb, kbp, 0u);
+    hipLaunchKernelGGL(mx_pad_rows_kernel<16>, grid(kbp / 16, a.N, L.nb2), dim3(256), 0, st, (const uint8_t*)a.x2.ptr, a.x2.col_stride / epb,
+                       a.x2.batch_stride / epb, w + L.o_x2, a.N, kb, kbp, 0u);
+    hipLaunchKernelGGL(mx_pad_rows_kernel<2>, grid(ksp2 / 2, a.M, L.snb1), dim3(256), 0, st, (const uint8_t*)a.x1_scale_mat.ptr, ks2,
+                       a.x1_scale_mat.batch_stride, w + L.o_s1, a.M, ks2, ksp2, 0x7f7fu);
+    hipLaunchKernelGGL(mx_pad_rows_kernel<2>, grid(ksp2 / 2, a.N, L.snb2), dim3(256), 0, st, (const uint8_t*)a.x2_scale_mat.ptr, ks2,
+                       a.x2_scale_mat.batch_stride, w + L.o_s2, a.N, ks2, ksp2, 0x7f7fu);
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return (int)e;
+    a.x1 = OpsnnMat{w, L.Kp, 1, L.nb1 == 1 && a.batch > 1 ? 0 : a.M * L.Kp};
+    a.x2 = OpsnnMat{w + L.o_x2, 1, L.Kp, L.nb2 == 1 && a.batch > 1 ? 0 : a.N * L.Kp};
+    a.x1_scale_mat = OpsnnMat{w + L.o_s1, ksp2, 2, L.snb1 == 1 && a.batch > 1 ? 0 : a.M * ksp2};
+    a.x2_scale_mat = OpsnnMat{w + L.o_s2, ksp2, 2, L.snb2 == 1 && a.batch > 1 ? 0 : a.N * ksp2};
+    a.K = L.Kp;
+    a.workspace = nullptr;
+    return 0;
+}
 
 uint64_t mx_workspace_bytes(const OpsnnQmmArgs& a)
 {
+    MxPad L;
+    if (a.force_variant != OPSNN_VARIANT_PLAIN && !opsnn_force_plain() && mx_pad_layout(a, L)) return L.total;
     if (a.x2.row_stride == 1 || a.K == 1) return 0;
     if (a.x2.col_stride != 1 || a.x2.row_stride != a.N) return 0;
     const uint64_t bits = a.x2_dtype == DT_E2M1 ? 4 : 8;
@@ -83,6 +164,13 @@ int launch_mx_mfma(const OpsnnQmmArgs& a0, hipStream_t st)
     // datapath.
     if (a.out_dtype != DT_BF16 && a.out_dtype != DT_F16) return OPSNN_NOT_TAKEN;
     if (a.bias && a.bias_dtype != DT_F32) return OPSNN_NOT_TAKEN;
+    {
+        MxPad L;
+        if (mx_pad_layout(a, L)) {
+            const int rc = mx_pad_prestep(a, L, st);
+            if (rc != 0) return rc;
+        }
+    }
     if (a.K % 128 != 0 || a.M * a.N < 64 * 64) return OPSNN_NOT_TAKEN;
     const int64_t ks = a.K / 64;  // scale pairs per row
     if (a.x1.col_stride != 1 || a.x1_scale_mat.col_stride != 2 || a.x1_scale_mat.row_stride != ks * 2) return OPSNN_NOT_TAKEN;

@@ -74,6 +74,44 @@ def test_fp8_blockscale_k_tail(gpu, M, K, N, tB, gsM, fast):
     m.lib().aclDestroyAclOpExecutor(ex)
 
 
+def _mx_pad_bytes(M, K, N, fp4, batch=1):
+    Kp, epb = K + 64, 2 if fp4 else 1
+    up = lambda v: -(-v // 256) * 256
+    return up(batch * M * Kp // epb) + up(batch * N * Kp // epb) + up(batch * M * (Kp // 64) * 2) + up(batch * N * (Kp // 64) * 2)
+
+
+@pytest.mark.parametrize("M,K,N,fp4,batch,bias", [
+    (197, 960, 854, True, 1, True),      # MXFP4, 7.5 K tiles, ragged rows and columns
+    (256, 1472, 384, False, 1, False),   # MXFP8, 11.5 K tiles
+    (128, 192, 256, True, 2, True),      # batched, 1.5 K tiles
+    (64, 64, 64, False, 1, False),       # half a K tile
+])
+def test_mx_k_tail(gpu, M, K, N, fp4, batch, bias):
+    """MX operands with K % 128 == 64 (a whole number of scale pairs, half a K tile left over): both operands and both
+    scale tables are copied with one more pair per row (zero elements, scales 2^0), then the matrix-core kernels run."""
+    m = gpu
+    print(f"case mx K tail M={M} K={K} N={N} fp4={fp4} batch={batch} bias={bias}", flush=True)
+    inp = cases.make_mx_inputs(m, M, K, N, K + N, True, fp4, batch=batch)
+    b = np.random.default_rng(3).normal(0, 1, N).astype(np.float32) if bias else None
+    want = cases.oracle_mx(m, inp, M, K, N, True, m.ACL_BF16, b)
+    got = cases.run_mx_aclnn(m, inp, M, K, N, True, m.ACL_BF16, b)
+    abs_sum = None
+    if not fp4:
+        pos = dict(inp, x1=inp["x1"] & 0x7F, x2=inp["x2"] & 0x7F)
+        abs_sum = orc.b16_to_f32(cases.oracle_mx(m, pos, M, K, N, True, m.ACL_BF16), orc.BF16).astype(np.float64)
+    check_close(got, want, orc.BF16, "mx with a K tail", fp8_mfma=not fp4, abs_sum=abs_sum)
+    # phase 1 plans the four padded copies
+    adt = m.ACL_FLOAT4_E2M1 if fp4 else m.ACL_FLOAT8_E4M3FN
+    bs = (batch,) if batch > 1 else ()
+    d = {k: m.DeviceBuffer(host=v) for k, v in inp.items() if isinstance(v, np.ndarray)}
+    x1 = m.Tensor(bs + (M, K), adt, d["x1"]); x2 = m.Tensor(bs + (N, K), adt, d["x2"])
+    s1 = m.Tensor(bs + inp["s1"].shape[1:], m.ACL_FLOAT8_E8M0, d["s1"]); s2 = m.Tensor(bs + inp["s2"].shape[1:], m.ACL_FLOAT8_E8M0, d["s2"])
+    o = m.Tensor(bs + (M, N), m.ACL_BF16, m.DeviceBuffer(batch * M * N * 2))
+    rc, ws, ex = m.quant_matmul_v5_get_workspace(x1, x2, s1, s2, o, transpose_x2=True, group_size=(1 << 32) | (1 << 16) | 32)
+    assert rc == 0 and ws == _mx_pad_bytes(M, K, N, fp4, batch), (rc, ws, _mx_pad_bytes(M, K, N, fp4, batch))
+    m.lib().aclDestroyAclOpExecutor(ex)
+
+
 @pytest.mark.parametrize("M,K,N,s_len,pt", [(256, 1000, 264, "N", "M"), (128, 72, 512, "N", True)])
 def test_fp8_row_and_column_scales_k_tail(gpu, M, K, N, s_len, pt):
     m = gpu
