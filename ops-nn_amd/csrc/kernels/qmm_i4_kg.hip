@@ -15,9 +15,9 @@
 // and stored block by block: the 128 rows x 256 bytes of one tile and group, followed by 1 KiB of that group's fp32
 // side values (x1: the negated row sums; x2: scales, then offsets), are one contiguous block that already is the LDS
 // image (16-byte chunks of a row xor-swizzled by the row, so that fragment reads are free of bank conflicts).  The
-// matrix kernel fetches a block with linear 16-byte asynchronous copies: consecutive addresses spread over all memory
-// channels (rows 4096 bytes apart would all fall into one), and the side values arrive in LDS with the tile instead of
-// costing every wave eight vector loads per group.
+// matrix kernel fetches a block with linear 16-byte asynchronous copies (one base address per group, no swizzle or row
+// arithmetic per lane), and the side values arrive in LDS with the tile instead of costing every wave eight vector
+// loads per group.
 //
 // The matrix kernel: 128 x 128 output tile per workgroup, eight waves of 64 x 32 (4 x 2 fragments of 16 x 16), one K
 // tile = one group, two matrix instructions per fragment pair from a zero accumulator, then the fold on the vector
