@@ -333,6 +333,132 @@ __global__ __launch_bounds__(256) void wide_quant_apply_kernel(WideQuantParams w
     }
 }
 
+// ---- the same two passes for rows of whole 16-byte pieces (cols % 8 == 0, x 16-byte aligned) ----
+// A workgroup is 64 pieces of 8 columns x 4 row lanes and walks `rpb` rows of one batch (rows that share their slots);
+// a thread keeps its 8 columns' extremes (reduce) or their quantisation parameters (apply) in registers over its rows.
+// blockIdx.x = block of 64 pieces, blockIdx.y = batch * chunks + chunk of rpb rows.
+struct WideTile { int64_t col0, r_begin, r_end, batch; bool inside; };
+__device__ __forceinline__ WideTile wide_tile(const WideQuantParams& w, int rpb, int chunks)
+{
+    WideTile t;
+    const int64_t b = blockIdx.y / chunks, c = blockIdx.y - b * chunks;
+    t.batch = b;
+    t.col0 = ((int64_t)blockIdx.x * 64 + (threadIdx.x & 63)) * 8;
+    t.inside = t.col0 < w.p.cols;
+    t.r_begin = b * w.chan_rows + c * rpb;
+    const int64_t batch_end = (b + 1) * w.chan_rows;
+    t.r_end = t.r_begin + rpb < batch_end ? t.r_begin + rpb : batch_end;
+    return t;
+}
+// the 8 values of a piece, smoothed: pertensor by the column's factor, perchannel by the row's
+template <int X_DT>
+__device__ __forceinline__ void wide_piece(const WideQuantParams& w, const WideTile& t, int64_t r, const float (&smc)[8], float (&v)[8])
+{
+    const uint4 xv = *(const uint4*)(w.p.x + r * w.p.cols + t.col0);
+    const uint32_t xw[4] = {xv.x, xv.y, xv.z, xv.w};
+    float smr = 1.0f;
+    if (w.p.smooth && w.mode == 2) smr = x_to_f32<X_DT>(w.p.smooth[r - t.batch * w.chan_rows]);
+#pragma unroll
+    for (int e = 0; e < 8; e++) {
+        v[e] = x_to_f32<X_DT>((xw[e >> 1] >> (16 * (e & 1))) & 0xffffu);
+        if (w.p.smooth) v[e] = __fmul_rn(v[e], w.mode == 1 ? smc[e] : smr);
+    }
+}
+template <int X_DT>
+__device__ __forceinline__ void wide_column_smooth(const WideQuantParams& w, const WideTile& t, float (&smc)[8])
+{
+#pragma unroll
+    for (int e = 0; e < 8; e++) smc[e] = 1.0f;
+    if (w.p.smooth && w.mode == 1 && t.inside) {
+        const uint4 sv = *(const uint4*)(w.p.smooth + t.col0);
+        const uint32_t sw[4] = {sv.x, sv.y, sv.z, sv.w};
+#pragma unroll
+        for (int e = 0; e < 8; e++) smc[e] = x_to_f32<X_DT>((sw[e >> 1] >> (16 * (e & 1))) & 0xffffu);
+    }
+}
+
+template <int X_DT>
+__global__ __launch_bounds__(256) void wide_quant_reduce8_kernel(WideQuantParams w, int rpb, int chunks)
+{
+    __shared__ float red[2][3][64][8];
+    const WideTile t = wide_tile(w, rpb, chunks);
+    const int rl = threadIdx.x >> 6, lv = threadIdx.x & 63;
+    float smc[8], vmax[8], vmin[8];
+    wide_column_smooth<X_DT>(w, t, smc);
+#pragma unroll
+    for (int e = 0; e < 8; e++) { vmax[e] = -__builtin_inff(); vmin[e] = __builtin_inff(); }
+    if (t.inside) {
+        for (int64_t r = t.r_begin + rl; r < t.r_end; r += 4) {
+            float v[8];
+            wide_piece<X_DT>(w, t, r, smc, v);
+#pragma unroll
+            for (int e = 0; e < 8; e++) { vmax[e] = fmaxf(vmax[e], v[e]); vmin[e] = fminf(vmin[e], v[e]); }
+        }
+    }
+    if (rl > 0) {
+#pragma unroll
+        for (int e = 0; e < 8; e++) { red[0][rl - 1][lv][e] = vmax[e]; red[1][rl - 1][lv][e] = vmin[e]; }
+    }
+    __syncthreads();
+    if (rl > 0) return;
+#pragma unroll
+    for (int j = 0; j < 3; j++)
+#pragma unroll
+        for (int e = 0; e < 8; e++) { vmax[e] = fmaxf(vmax[e], red[0][j][lv][e]); vmin[e] = fminf(vmin[e], red[1][j][lv][e]); }
+    if (w.mode == 1) {   // one slot for everybody: the wave's extremes, one lane hands them in
+        float a = vmax[0], b = vmin[0];
+#pragma unroll
+        for (int e = 1; e < 8; e++) { a = fmaxf(a, vmax[e]); b = fminf(b, vmin[e]); }
+        a = wave_max(a);
+        b = -wave_max(-b);
+        if (lv != 0) return;
+        if (w.smin) { atomicMax(w.smax, float_key(a)); atomicMin(w.smin, float_key(b)); }
+        else atomicMax(w.smax, float_key(fmaxf(a, -b)));
+        return;
+    }
+    if (!t.inside || t.r_begin >= t.r_end) return;
+    const int64_t slot0 = t.batch * w.p.cols + t.col0;
+#pragma unroll
+    for (int e = 0; e < 8; e++) {
+        if (w.smin) { atomicMax(w.smax + slot0 + e, float_key(vmax[e])); atomicMin(w.smin + slot0 + e, float_key(vmin[e])); }
+        else atomicMax(w.smax + slot0 + e, float_key(fmaxf(vmax[e], -vmin[e])));
+    }
+}
+
+template <int X_DT, int Y_DT, bool ASYM>
+__global__ __launch_bounds__(256) void wide_quant_apply8_kernel(WideQuantParams w, int rpb, int chunks)
+{
+    const WideTile t = wide_tile(w, rpb, chunks);
+    if (!t.inside) return;
+    const int rl = threadIdx.x >> 6;
+    float smc[8];
+    wide_column_smooth<X_DT>(w, t, smc);
+    RowQuant rq[8];
+#pragma unroll
+    for (int e = 0; e < 8; e++) {
+        if (w.mode == 1 && e > 0) { rq[e] = rq[0]; continue; }
+        const int64_t slot = w.mode == 1 ? 0 : t.batch * w.p.cols + t.col0 + e;
+        const float a = key_float(w.smax[slot]);
+        rq[e] = row_params<ASYM>(w.p, a, a, ASYM ? key_float(w.smin[slot]) : 0.0f);
+    }
+    for (int64_t r = t.r_begin + rl; r < t.r_end; r += 4) {
+        float v[8];
+        wide_piece<X_DT>(w, t, r, smc, v);
+        uint32_t q[8];
+#pragma unroll
+        for (int e = 0; e < 8; e++) q[e] = quant_one<Y_DT, ASYM>(v[e], rq[e]);
+        if constexpr (Y_DT == DT_I4) {
+            uint32_t o = 0;
+#pragma unroll
+            for (int e = 0; e < 8; e++) o |= q[e] << (4 * e);
+            *(uint32_t*)((uint8_t*)w.p.y + (r * w.p.cols + t.col0) / 2) = o;
+        } else {
+            const uint32_t lo = q[0] | (q[1] << 8) | (q[2] << 16) | (q[3] << 24), hi = q[4] | (q[5] << 8) | (q[6] << 16) | (q[7] << 24);
+            *(uint2*)((uint8_t*)w.p.y + r * w.p.cols + t.col0) = make_uint2(lo, hi);
+        }
+    }
+}
+
 template <bool ASYM>
 __global__ __launch_bounds__(256) void wide_quant_finish_kernel(WideQuantParams w)
 {
@@ -355,8 +481,21 @@ static int launch_wide_quant(const DynQuantParams& p, int mode, int64_t chan_row
     if (row_chunks > 65535 || (p.cols + 255) / 256 > 0x7fffffff || (pairs + 255) / 256 > 0x7fffffff || (w.nslots + 255) / 256 > 0x7fffffff) return -1;
     const dim3 slots((unsigned)((w.nslots + 255) / 256));
     hipLaunchKernelGGL(wide_quant_init_kernel, slots, dim3(256), 0, st, w);
-    hipLaunchKernelGGL(wide_quant_reduce_kernel<X_DT>, dim3((unsigned)((p.cols + 255) / 256), (unsigned)row_chunks), dim3(256), 0, st, w);
-    hipLaunchKernelGGL((wide_quant_apply_kernel<X_DT, Y_DT, ASYM>), dim3((unsigned)((pairs + 255) / 256)), dim3(256), 0, st, w);
+    // rows of whole 16-byte pieces: the vector kernels, chunks of 64 rows (more when there would be too many workgroups)
+    const int64_t batches = p.rows / w.chan_rows;
+    int64_t rpb = 64;
+    while (batches * ((w.chan_rows + rpb - 1) / rpb) > 65535) rpb *= 2;
+    const int64_t chunks = (w.chan_rows + rpb - 1) / rpb;
+    const bool vec = p.cols % 8 == 0 && (uintptr_t)p.x % 16 == 0 && (uintptr_t)p.y % 8 == 0 && (!p.smooth || (uintptr_t)p.smooth % 16 == 0) &&
+                     rpb < (1 << 30) && chunks < (1 << 30);
+    if (vec) {
+        const dim3 grid((unsigned)((p.cols / 8 + 63) / 64), (unsigned)(batches * chunks));
+        hipLaunchKernelGGL(wide_quant_reduce8_kernel<X_DT>, grid, dim3(256), 0, st, w, (int)rpb, (int)chunks);
+        hipLaunchKernelGGL((wide_quant_apply8_kernel<X_DT, Y_DT, ASYM>), grid, dim3(256), 0, st, w, (int)rpb, (int)chunks);
+    } else {
+        hipLaunchKernelGGL(wide_quant_reduce_kernel<X_DT>, dim3((unsigned)((p.cols + 255) / 256), (unsigned)row_chunks), dim3(256), 0, st, w);
+        hipLaunchKernelGGL((wide_quant_apply_kernel<X_DT, Y_DT, ASYM>), dim3((unsigned)((pairs + 255) / 256)), dim3(256), 0, st, w);
+    }
     hipLaunchKernelGGL(wide_quant_finish_kernel<ASYM>, slots, dim3(256), 0, st, w);
     return (int)hipGetLastError();
 }

@@ -378,7 +378,11 @@ def test_gpu_group_index(gpu, shape, ends, gi_dt, symmetric):
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("mode,shape", [("pertensor", (16, 32)), ("pertensor", (3, 70, 500)), ("pertensor", (1000, 257)),
-                                        ("perchannel", (16, 32)), ("perchannel", (3, 70, 500)), ("perchannel", (2, 200, 1001)), ("perchannel", (130, 64))])
+                                        ("perchannel", (16, 32)), ("perchannel", (3, 70, 500)), ("perchannel", (2, 200, 1001)), ("perchannel", (130, 64)),
+                                        # rows of whole 16-byte pieces (the vector kernels): several row chunks per batch, a ragged
+                                        # last chunk, more than one block of 64 pieces, fewer pieces than a block
+                                        ("pertensor", (1000, 256)), ("pertensor", (2, 70, 1032)), ("perchannel", (3, 200, 512)),
+                                        ("perchannel", (5, 64, 1032)), ("perchannel", (300, 8))])
 @pytest.mark.parametrize("y_dt,symmetric,with_smooth", [(orc.I8, True, False), (orc.I8, False, True), (orc.I4, True, True), (orc.E4M3, True, False)])
 def test_gpu_per_tensor_and_per_channel_modes(gpu, mode, shape, y_dt, symmetric, with_smooth):
     m = gpu
