@@ -306,6 +306,122 @@ __global__ __launch_bounds__(256) void mx_quant_general_kernel(MxGeneralParams p
     }
 }
 
+// The same arithmetic for blocks along an axis that is not the last, 16-bit x and inner % 8 == 0: a thread takes 8
+// neighbouring inner columns (16-byte loads, 8- or 4-byte stores) and one PAIR of blocks, so that it also owns the 16
+// contiguous scale bytes of its columns ([.., pair, inner, 2]).  x is read twice (the second time from cache).
+// YT: the element type when the rounding is to nearest even (the hardware conversions of the last-axis kernels), or 0:
+// any type and rounding mode through mxg_element.
+template <int YT>
+__global__ __launch_bounds__(256) void mx_quant_inner8_kernel(MxGeneralParams p)
+{
+    const int64_t iw = p.inner / 8;
+    const int64_t g = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (g >= p.outer * p.np * iw) return;
+    const int64_t o = g / (p.np * iw), rem = g - o * (p.np * iw), pb = rem / iw, ic = rem - pb * iw;
+    int emax, emin, mbits; float tmax;
+    switch (p.y_dt) {
+        case DT_E2M1: emax = 2; emin = 0; mbits = 1; tmax = 6.0f; break;
+        case DT_E1M2: emax = 0; emin = 0; mbits = 2; tmax = 1.75f; break;
+        case DT_E4M3: emax = 8; emin = -6; mbits = 3; tmax = 448.0f; break;
+        default: emax = 15; emin = -14; mbits = 2; tmax = 57344.0f; break;
+    }
+    const bool fp4 = p.y_dt == DT_E2M1 || p.y_dt == DT_E1M2;
+    const uint16_t* xs = (const uint16_t*)p.x;
+    // rows travel eight at a time (eight independent 16-byte loads in flight per thread); rows past the block repeat its last
+    auto fetch8 = [&](int64_t a, int64_t a1, uint4 (&buf)[8]) {
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            const int64_t aj = a + j < a1 ? a + j : a1 - 1;
+            buf[j] = *(const uint4*)(xs + (o * p.A + aj) * p.inner + ic * 8);
+        }
+    };
+    auto widen = [&](const uint4& xv, float (&v)[8]) {
+        const uint32_t w[4] = {xv.x, xv.y, xv.z, xv.w};
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+            const uint32_t h = (w[e >> 1] >> (16 * (e & 1))) & 0xffffu;
+            v[e] = p.x_dt == DT_BF16 ? u2f(h << 16) : f16_to_f32((uint16_t)h);
+        }
+    };
+    uint32_t sb[8] = {0, 0, 0, 0, 0, 0, 0, 0};   // per column: the pair's two scale bytes (an absent second block: 0)
+    for (int h = 0; h < 2; h++) {
+        const int64_t b = 2 * pb + h;
+        if (b >= p.nblk) break;
+        const int64_t a0 = b * p.block, a1 = a0 + p.block < p.A ? a0 + p.block : p.A;
+        float amax[8], inv_scale[8];
+        uint32_t badm = 0;
+#pragma unroll
+        for (int e = 0; e < 8; e++) amax[e] = 0.0f;
+        for (int64_t a = a0; a < a1; a += 8) {
+            uint4 buf[8];
+            fetch8(a, a1, buf);
+#pragma unroll
+            for (int j = 0; j < 8; j++) {   // (a repeated last row changes neither the maximum nor the flags)
+                float v[8];
+                widen(buf[j], v);
+#pragma unroll
+                for (int e = 0; e < 8; e++) {
+                    const float t = fabsf(v[e]);
+                    badm |= (t < __builtin_inff() ? 0u : 1u) << e;
+                    amax[e] = fmaxf(amax[e], t);
+                }
+            }
+        }
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+            const bool bd = (badm >> e) & 1u;
+            int share = -127;
+            if (!bd && amax[e] != 0.0f) {
+                if (p.scale_alg == 1) {
+                    const uint32_t u = f2u(__fdiv_rn(amax[e], tmax));
+                    int ex = (int)(u >> 23);
+                    const uint32_t mant = u & 0x7fffffu;
+                    if ((ex > 0 && ex < 254 && mant > 0) || (ex == 0 && mant > 0x400000u)) ex += 1;
+                    share = ex - 127;
+                } else {
+                    const int ex = (int)(f2u(amax[e]) >> 23);
+                    share = (ex == 0 || ex - 127 - emax < -127) ? -127 : ex - 127 - emax;
+                }
+            }
+            sb[e] |= (bd ? 0xFFu : (uint32_t)(share + 127)) << (8 * h);
+            inv_scale[e] = u2f((uint32_t)(127 - share) << 23);
+        }
+        for (int64_t a = a0; a < a1; a += 8) {
+            uint4 buf[8];
+            fetch8(a, a1, buf);
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                if (a + j >= a1) break;
+                float v[8];
+                widen(buf[j], v);
+                const int64_t i = (o * p.A + a + j) * p.inner + ic * 8;
+                if constexpr (YT != 0) {
+                    float qf[8];
+#pragma unroll
+                    for (int e = 0; e < 8; e++) qf[e] = mx_scaled<YT>(v[e], inv_scale[e], (badm >> e) & 1u);
+                    const uint2 pk = mx_pack8<YT>(qf);
+                    if constexpr (YT == DT_E2M1) *(uint32_t*)(p.y + (i >> 1)) = pk.x;
+                    else *(uint2*)(p.y + i) = pk;
+                    continue;
+                }
+                uint32_t q[8];
+#pragma unroll
+                for (int e = 0; e < 8; e++) q[e] = mxg_element(v[e], inv_scale[e], (badm >> e) & 1u, emin, mbits, tmax, p.round_mode, p.y_dt);
+                if (fp4) {
+                    uint32_t w = 0;
+#pragma unroll
+                    for (int e = 0; e < 8; e++) w |= q[e] << (4 * e);
+                    *(uint32_t*)(p.y + (i >> 1)) = w;
+                } else {
+                    *(uint2*)(p.y + i) = make_uint2(q[0] | (q[1] << 8) | (q[2] << 16) | (q[3] << 24), q[4] | (q[5] << 8) | (q[6] << 16) | (q[7] << 24));
+                }
+            }
+        }
+    }
+    *(uint4*)(p.scale + ((o * p.np + pb) * p.inner + ic * 8) * 2) =
+        make_uint4(sb[0] | (sb[1] << 16), sb[2] | (sb[3] << 16), sb[4] | (sb[5] << 16), sb[6] | (sb[7] << 16));
+}
+
 static int launch_mx_quant_general(const OpsnnMxQuantArgs& a, hipStream_t st)
 {
     MxGeneralParams p{};
@@ -320,6 +436,16 @@ static int launch_mx_quant_general(const OpsnnMxQuantArgs& a, hipStream_t st)
     if (p.round_mode < 0 || p.round_mode > 4 || (p.scale_alg != 0 && (p.scale_alg != 1 || fp4))) return -2;
     if (fp4 && ((p.inner > 1 ? p.inner : p.A) & 1)) return -2;
     p.nblk = (p.A + p.block - 1) / p.block; p.np = (p.nblk + 1) / 2;
+    if (p.x_dt != DT_F32 && p.inner % 8 == 0 && (uintptr_t)p.x % 16 == 0 && (uintptr_t)p.y % 8 == 0 && (uintptr_t)p.scale % 16 == 0) {
+        const int64_t wgs8 = (p.outer * p.np * (p.inner / 8) + 255) / 256;
+        if (wgs8 > 0x7fffffff) return -1;
+        const dim3 grid((unsigned)wgs8);
+        if (p.round_mode == 0 && p.y_dt == DT_E2M1) hipLaunchKernelGGL(mx_quant_inner8_kernel<DT_E2M1>, grid, dim3(256), 0, st, p);
+        else if (p.round_mode == 0 && p.y_dt == DT_E4M3) hipLaunchKernelGGL(mx_quant_inner8_kernel<DT_E4M3>, grid, dim3(256), 0, st, p);
+        else if (p.round_mode == 0 && p.y_dt == DT_E5M2) hipLaunchKernelGGL(mx_quant_inner8_kernel<DT_E5M2>, grid, dim3(256), 0, st, p);
+        else hipLaunchKernelGGL(mx_quant_inner8_kernel<0>, grid, dim3(256), 0, st, p);
+        return (int)hipGetLastError();
+    }
     const int64_t iw = fp4 && p.inner > 1 ? p.inner / 2 : p.inner;
     const int64_t wgs = (p.outer * p.nblk * iw + 255) / 256;
     if (wgs > 0x7fffffff) return -1;

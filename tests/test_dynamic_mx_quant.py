@@ -381,6 +381,11 @@ def _run_general(m, x, x_dt, y_dt, axis, block=32, scale_alg=0, round_mode="rint
     ((6, 1000), -1, orc.BF16, orc.E2M1, 32, 0, "floor"),       # the rounding modes of the 4-bit types on the last axis
     ((6, 1000), -1, orc.F16, orc.E2M1, 128, 0, "round"),
     ((64, 33, 2), 0, orc.F32, orc.E1M2, 32, 0, "round"),
+    # inner extents of whole 16-byte pieces of a 16-bit x (the vector kernel: 8 columns and a pair of blocks per thread):
+    # an odd number of blocks with a ragged last one, two outer slices, 4-bit and 8-bit elements
+    ((130, 64), 0, orc.BF16, orc.E2M1, 32, 0, "rint"),
+    ((2, 70, 16), 1, orc.F16, orc.E1M2, 32, 0, "round"),
+    ((3, 200, 8), -2, orc.BF16, orc.E4M3, 64, 1, "rint"),
 ])
 def test_gpu_general_form_is_bit_identical(gpu, shape, axis, x_dt, y_dt, block, alg, mode):
     """Blocks along another axis, fp32 input, e1m2 elements and the floor / round modes (the one-thread-per-block kernel)
