@@ -160,6 +160,63 @@ __global__ __launch_bounds__(256) void mx_quant_kernel(MxQuantParams p, int64_t 
     }
 }
 
+// Blocks of 64, 128, 256, 512 or 1024 elements, cols % 8 == 0: a wave takes 512 * PPL consecutive elements of a row (a whole
+// number of blocks), every lane PPL 16-byte pieces (1024: two, 512 elements apart; otherwise one), and the block maximum is
+// an exchange over the 2^lg neighbouring lanes that share a block.  One pass, every access of a wave contiguous.
+template <int X_DT, int Y_DT, int PPL>
+__global__ __launch_bounds__(256) void mx_quant_wideblock_kernel(MxQuantParams p, int lg, int chunks_per_row)
+{
+    const int lane = threadIdx.x & 63;
+    const int64_t wave = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int64_t row = wave / chunks_per_row;
+    if (row >= p.rows) return;
+    const int64_t col_base = (wave - row * chunks_per_row) * (512 * PPL);
+    float v[PPL][8];
+    bool live[PPL];
+    float amax = 0.0f;
+    bool bad = false;
+#pragma unroll
+    for (int k = 0; k < PPL; k++) {
+        const int64_t col = col_base + (k * 64 + lane) * 8;
+        live[k] = col < p.cols;
+        uint4 b = make_uint4(0, 0, 0, 0);
+        if (live[k]) b = *(const uint4*)(p.x + row * p.cols + col);
+        const uint32_t w[4] = {b.x, b.y, b.z, b.w};
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+            v[k][e] = mx_x_to_f32<X_DT>((w[e >> 1] >> (16 * (e & 1))) & 0xffffu);
+            const float a = fabsf(v[k][e]);
+            bad |= !(a < __builtin_inff());
+            amax = fmaxf(amax, a);
+        }
+    }
+    int badi = bad;
+    for (int d = 1; d < (1 << lg); d <<= 1) {
+        amax = fmaxf(amax, __shfl_xor(amax, d));
+        badi |= __shfl_xor(badi, d);
+    }
+    bad = badi != 0;
+    const int share = bad ? 0 : mx_share_exp<Y_DT>(amax, p.scale_alg);
+    const int64_t col0 = col_base + lane * 8;
+    if ((lane & ((1 << lg) - 1)) == 0 && live[0]) {
+        const int64_t blk = col0 / p.block;
+        p.scale[row * p.spitch + blk] = bad ? 0xFFu : (uint8_t)(share + 127);
+        if (blk == p.nblk - 1 && (p.nblk & 1)) p.scale[row * p.spitch + blk + 1] = 0;
+    }
+    const float inv_scale = u2f((uint32_t)(127 - share) << 23);
+#pragma unroll
+    for (int k = 0; k < PPL; k++) {
+        if (!live[k]) continue;
+        float q[8];
+#pragma unroll
+        for (int e = 0; e < 8; e++) q[e] = mx_scaled<Y_DT>(v[k][e], inv_scale, bad);
+        const uint2 out = mx_pack8<Y_DT>(q);
+        const int64_t at = row * p.cols + col_base + (k * 64 + lane) * 8;
+        if constexpr (Y_DT == DT_E2M1) *(uint32_t*)(p.y + at / 2) = out.x;
+        else *(uint2*)(p.y + at) = out;
+    }
+}
+
 // any row length and block size: one thread per block
 template <int X_DT, int Y_DT>
 __global__ __launch_bounds__(256) void mx_quant_generic_kernel(MxQuantParams p)
@@ -458,6 +515,18 @@ static int launch_mx_quant(const MxQuantParams& p, int variant, hipStream_t st)
 {
     const bool vec = p.block == 32 && p.cols % 8 == 0 && (uintptr_t)p.x % 16 == 0 && (uintptr_t)p.y % 8 == 0;
     const int64_t groups = p.rows * p.nblk;
+    const bool wide = variant != 2 && p.block >= 64 && p.block <= 1024 && (p.block & (p.block - 1)) == 0 && p.cols % 8 == 0 &&
+                      (uintptr_t)p.x % 16 == 0 && (uintptr_t)p.y % 8 == 0;
+    if (wide) {
+        const int ppl = p.block == 1024 ? 2 : 1;
+        const int lg = __builtin_ctzll((unsigned long long)(p.block / 8 / ppl));
+        const int64_t cpr = (p.cols + 512 * ppl - 1) / (512 * ppl);
+        const int64_t wgs = (p.rows * cpr + 3) / 4;
+        if (wgs > 0x7fffffff || cpr > 0x7fffffff) return -1;
+        if (ppl == 2) hipLaunchKernelGGL((mx_quant_wideblock_kernel<X_DT, Y_DT, 2>), dim3((unsigned)wgs), dim3(256), 0, st, p, lg, (int)cpr);
+        else hipLaunchKernelGGL((mx_quant_wideblock_kernel<X_DT, Y_DT, 1>), dim3((unsigned)wgs), dim3(256), 0, st, p, lg, (int)cpr);
+        return (int)hipGetLastError();
+    }
     if (variant != 2 && vec) {
         // four pairs per group once that still leaves every SIMD eight waves
         const int nb = groups * 4 / 64 >= (int64_t)4 * 8 * 1024 ? 4 : 1;

@@ -333,7 +333,12 @@ def test_gpu_mx_quantised_operands_feed_the_mx_matmul(gpu, fp4):
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("shape,block,alg,y_dt", [((33, 1024), 64, 0, orc.E2M1), ((7, 1000), 128, 0, orc.E4M3), ((5, 4096), 1024, 0, orc.E5M2),
-                                                  ((33, 1024), 32, 1, orc.E4M3), ((6, 1000), 32, 1, orc.E5M2), ((9, 520), 256, 1, orc.E4M3)])
+                                                  ((33, 1024), 32, 1, orc.E4M3), ((6, 1000), 32, 1, orc.E5M2), ((9, 520), 256, 1, orc.E4M3),
+                                                  # the wave-per-512-elements kernel: several waves per row, a ragged last wave and
+                                                  # block, an odd number of blocks, two pieces per lane (1024); a block that is not a
+                                                  # power of two stays on the one-thread-per-block kernel
+                                                  ((3, 2048), 512, 0, orc.E2M1), ((4, 1544), 64, 0, orc.E4M3), ((2, 3072), 1024, 0, orc.E2M1),
+                                                  ((5, 2200), 1024, 1, orc.E4M3), ((6, 960), 96, 0, orc.E4M3)])
 def test_gpu_block_sizes_and_scale_algorithm_1(gpu, shape, block, alg, y_dt):
     m = gpu
     print(f"case mx quant {shape} block={block} scale_alg={alg} y={y_dt}", flush=True)
