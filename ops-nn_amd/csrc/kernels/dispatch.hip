@@ -115,7 +115,7 @@ int64_t k_pad_for(const OpsnnQmmArgs& a, int mode)
     else if (mode == 1) tail = (f8 || i8) && a.gsK == 128 && (a.K % 128 != 0 || !x1_ok || !(x2_k || x2_n));
     else if (mode == 3) {
         // (the fp8 members of this family have no transposition step of their own)
-        const bool f8_16 = f8any && (a.out_dtype == DT_BF16 || a.out_dtype == DT_F16) && (!a.bias || a.bias_dtype == DT_F32);
+        const bool f8_16 = f8any && (a.out_dtype == DT_BF16 || a.out_dtype == DT_F16 || a.out_dtype == DT_F32) && (!a.bias || a.bias_dtype == DT_F32);
         tail = (i8 && !a.x1_scale && (a.K % 16 != 0 || !x1_ok || !(x2_k || x2_n))) || (f8_16 && (a.K % 128 != 0 || !x1_ok || !x2_k));
     }
     if (!tail || a.K < 16) return 0;
@@ -232,7 +232,7 @@ extern "C" int opsnnQmmTc(const OpsnnQmmArgs* a, void* stream)
     if (f8 && a->force_variant != OPSNN_VARIANT_PLAIN && !opsnn_force_plain()) {
         const int ep = !a->x1_scale ? 1 : (a->x1_scale_len == 1 && a->x2_scale_len == 1 && !a->bias) ? 2 : 0;
         const bool e4 = a->x1_dtype == DT_E4M3 && a->x2_dtype == DT_E4M3;
-        if (ep != 0 || !e4 || a->x2_scale_dtype != DT_F32) {
+        if (ep != 0 || !e4 || a->x2_scale_dtype != DT_F32 || a->out_dtype == DT_F32) {
             const int rc = launch_rowcol_exact(*a, (hipStream_t)stream, ep);
             if (rc != OPSNN_NOT_TAKEN) return rc;
         }

@@ -537,6 +537,38 @@ __global__ __launch_bounds__(WGM* WGN * 64, MINWG) void qgemm_kernel(QgemmParams
         }
         return;
     }
+    if constexpr (OUT_DT == DT_F32) {
+        // FLOAT output (the MX modes): like the integer outputs, straight from the registers, 16 bytes per lane
+        static_assert(MODE != MODE_I8, "the int8 mode has no FLOAT output here");
+        __syncthreads();
+        const bool vec_ok = (p.ldc % 4) == 0 && ((uintptr_t)p.out % 16) == 0;
+#pragma unroll
+        for (int j = 0; j < FM; j++) {
+            const int64_t m = m0 + wm * TM + j * 32 + frow;
+#pragma unroll
+            for (int i = 0; i < FN; i++) {
+#pragma unroll
+                for (int q = 0; q < 4; q++) {
+                    const int nl = wn * TN + i * 32 + 8 * q + 4 * fkc;
+                    const int64_t n = n0 + nl;
+                    const v4f fbv = *(const v4f*)(sFb + nl);
+                    v4f v;
+#pragma unroll
+                    for (int e = 0; e < 4; e++) v[e] = acc[i][j][q * 4 + e] + fbv[e];
+                    if (m < p.M) {
+                        float* dst = (float*)p.out + (bz * p.M + m) * p.ldc + n;
+                        if (vec_ok && n + 3 < p.N) *(v4f*)dst = v;
+                        else {
+#pragma unroll
+                            for (int e = 0; e < 4; e++)
+                                if (n + e < p.N) dst[e] = v[e];
+                        }
+                    }
+                }
+            }
+        }
+        return;
+    }
     __syncthreads();
     uint16_t* out = (uint16_t*)p.out + bz * p.M * p.ldc;
     // Results leave through LDS: a lane holds 4 consecutive columns of one row per register quad, which would make
@@ -647,6 +679,9 @@ static int qgemm_launch(const QgemmParams& p, int64_t batch, int out_dt, hipStre
             return bf ? qgemm_launch_one<MODE, BM, BN, BK, WGM, WGN, STAGES, MINWG, true, DT_BF16>(p, batch, st)
                       : qgemm_launch_one<MODE, BM, BN, BK, WGM, WGN, STAGES, MINWG, true, DT_F16>(p, batch, st);
         }
+    }
+    if constexpr (MODE != MODE_I8) {
+        if (out_dt == DT_F32) return qgemm_launch_one<MODE, BM, BN, BK, WGM, WGN, STAGES, MINWG, false, DT_F32>(p, batch, st);
     }
     return bf ? qgemm_launch_one<MODE, BM, BN, BK, WGM, WGN, STAGES, MINWG, false, DT_BF16>(p, batch, st)
               : qgemm_launch_one<MODE, BM, BN, BK, WGM, WGN, STAGES, MINWG, false, DT_F16>(p, batch, st);

@@ -626,7 +626,8 @@ int launch_blockscale_mfma(const OpsnnQmmArgs& a0, hipStream_t st)
     OpsnnQmmArgs a = a0;
     const bool i8 = a.x1_dtype == DT_I8 && a.x2_dtype == DT_I8;   // the per-tile mode of quant_batch_matmul_v4 (qbmmv4_kernel_golden.py:258-325)
     if (!i8 && (a.x1_dtype != DT_E4M3 || a.x2_dtype != DT_E4M3)) return OPSNN_NOT_TAKEN;
-    if (a.out_dtype != DT_BF16 && a.out_dtype != DT_F16) return OPSNN_NOT_TAKEN;
+    const bool out32 = a.out_dtype == DT_F32 && !i8;   // fp32 output: the exact kernel only
+    if (a.out_dtype != DT_BF16 && a.out_dtype != DT_F16 && !out32) return OPSNN_NOT_TAKEN;
     if (a.bias && !(i8 && a.bias_dtype == DT_F32)) return OPSNN_NOT_TAKEN;
     if (a.gsK != 128 || a.gsN != 128 || (a.gsM != 1 && a.gsM != 128)) return OPSNN_NOT_TAKEN;
     if (a.K % 128 != 0 || a.M * a.N < 64 * 64 || a.x1.col_stride != 1) return OPSNN_NOT_TAKEN;
@@ -644,9 +645,9 @@ int launch_blockscale_mfma(const OpsnnQmmArgs& a0, hipStream_t st)
         }
         a.x2.row_stride = 1; a.x2.col_stride = a.K;
     }
-    if (!i8 && !opsnnGetFp8Fast()) {   // exact products and sums unless the caller asked for the 8-bit matrix instruction
+    if (!i8 && (!opsnnGetFp8Fast() || out32)) {   // exact products and sums unless the caller asked for the 8-bit matrix instruction
         const int rc = launch_blockscale_exact(a, st);
-        if (rc != OPSNN_NOT_TAKEN) return rc;
+        if (rc != OPSNN_NOT_TAKEN || out32) return rc;
     }
     Fp8BlkParams p{};
     p.a = (const int8_t*)a.x1.ptr; p.b = (const int8_t*)a.x2.ptr;

@@ -383,8 +383,23 @@ __global__ __launch_bounds__(512, 1) void qmm_fp8_exact_kernel(Fp8xParams p, int
                     }
                 }
             }
-            *(v4us_a*)(ep + frow * EP_PITCH + (i * 16 + 4 * fq) * 2) = pack4_b16<OUT_DT>(v);
+            if constexpr (OUT_DT == DT_F32) {
+                // fp32 output: the lane's four neighbouring columns are 16 bytes, four lanes a 64-byte piece of a row: stored as they are
+                float* outf = (float*)p.out + bz * p.M * p.N;
+                const int64_t m = m0 + wm * TM + j * 16 + frow, n = n0 + wn * TN + i * 16 + 4 * fq;
+                if (m < p.M) {
+                    if ((p.N % 4) == 0 && ((uintptr_t)p.out % 16) == 0 && n + 3 < p.N) *(v4f*)(outf + m * p.N + n) = v;
+                    else {
+#pragma unroll
+                        for (int r = 0; r < 4; r++)
+                            if (n + r < p.N) outf[m * p.N + n + r] = v[r];
+                    }
+                }
+            } else {
+                *(v4us_a*)(ep + frow * EP_PITCH + (i * 16 + 4 * fq) * 2) = pack4_b16<OUT_DT>(v);
+            }
         }
+        if constexpr (OUT_DT == DT_F32) continue;
 #pragma unroll
         for (int r = 0; r < 2; r++) {
             const int row = r * 8 + er;
@@ -422,11 +437,11 @@ static int launch_fp8_exact(const Fp8xParams& p, int64_t batch, hipStream_t st)
     return (int)hipGetLastError();
 }
 
-// fp8 e4m3 block scales (G-B, B-B), K-contiguous operands, K % 128 == 0, 16-bit output, no bias.
+// fp8 e4m3 block scales (G-B, B-B), K-contiguous operands, K % 128 == 0, 16-bit or fp32 output, no bias.
 int launch_blockscale_exact(const OpsnnQmmArgs& a, hipStream_t st)
 {
     if (a.x1_dtype != DT_E4M3 || a.x2_dtype != DT_E4M3) return OPSNN_NOT_TAKEN;
-    if (a.out_dtype != DT_BF16 && a.out_dtype != DT_F16) return OPSNN_NOT_TAKEN;
+    if (a.out_dtype != DT_BF16 && a.out_dtype != DT_F16 && a.out_dtype != DT_F32) return OPSNN_NOT_TAKEN;
     if (a.bias) return OPSNN_NOT_TAKEN;
     if (a.gsK != 128 || a.gsN != 128 || (a.gsM != 1 && a.gsM != 128)) return OPSNN_NOT_TAKEN;
     if (a.K % 128 != 0 || a.M * a.N < 64 * 64 || a.x1.col_stride != 1 || a.x2.row_stride != 1) return OPSNN_NOT_TAKEN;
@@ -442,6 +457,7 @@ int launch_blockscale_exact(const OpsnnQmmArgs& a, hipStream_t st)
     if (((uintptr_t)p.a | (uintptr_t)p.b | (uint64_t)p.lda | (uint64_t)p.ldb | (uint64_t)p.a_bs | (uint64_t)p.b_bs) % 16) return OPSNN_NOT_TAKEN;
     if (((uintptr_t)p.s1 | (uintptr_t)p.s2) % 4) return OPSNN_NOT_TAKEN;
     if (a.out_dtype == DT_BF16) return launch_fp8_exact<DT_BF16, false>(p, a.batch, st);
+    if (a.out_dtype == DT_F32) return launch_fp8_exact<DT_F32, false>(p, a.batch, st);
     return launch_fp8_exact<DT_F16, false>(p, a.batch, st);
 }
 
@@ -453,7 +469,7 @@ int launch_rowcol_exact(const OpsnnQmmArgs& a, hipStream_t st, int ep_mode)
 {
     const bool e1 = a.x1_dtype == DT_E5M2, e2 = a.x2_dtype == DT_E5M2;
     if ((a.x1_dtype != DT_E4M3 && !e1) || (a.x2_dtype != DT_E4M3 && !e2)) return OPSNN_NOT_TAKEN;
-    if (a.out_dtype != DT_BF16 && a.out_dtype != DT_F16) return OPSNN_NOT_TAKEN;
+    if (a.out_dtype != DT_BF16 && a.out_dtype != DT_F16 && a.out_dtype != DT_F32) return OPSNN_NOT_TAKEN;
     if (!a.x2_scale || (a.x2_scale_dtype != DT_F32 && a.x2_scale_dtype != DT_BF16 && a.x2_scale_dtype != DT_U64)) return OPSNN_NOT_TAKEN;
     if (ep_mode != 1 && !a.x1_scale) return OPSNN_NOT_TAKEN;
     if (a.bias && a.bias_dtype != DT_F32) return OPSNN_NOT_TAKEN;
@@ -467,12 +483,12 @@ int launch_rowcol_exact(const OpsnnQmmArgs& a, hipStream_t st, int ep_mode)
     p.ep_mode = ep_mode;
     p.bias = (const float*)a.bias; p.bias_bs = a.bias_batch_stride;
     if (((uintptr_t)p.a | (uintptr_t)p.b | (uint64_t)p.lda | (uint64_t)p.ldb | (uint64_t)p.a_bs | (uint64_t)p.b_bs) % 16) return OPSNN_NOT_TAKEN;
-    const bool bf = a.out_dtype == DT_BF16;
+    const bool bf = a.out_dtype == DT_BF16, f32 = a.out_dtype == DT_F32;
     switch ((e1 ? 1 : 0) | (e2 ? 2 : 0)) {
-        case 0: return bf ? launch_fp8_exact<DT_BF16, true, 0>(p, a.batch, st) : launch_fp8_exact<DT_F16, true, 0>(p, a.batch, st);
-        case 1: return bf ? launch_fp8_exact<DT_BF16, true, 1>(p, a.batch, st) : launch_fp8_exact<DT_F16, true, 1>(p, a.batch, st);
-        case 2: return bf ? launch_fp8_exact<DT_BF16, true, 2>(p, a.batch, st) : launch_fp8_exact<DT_F16, true, 2>(p, a.batch, st);
-        default: return bf ? launch_fp8_exact<DT_BF16, true, 3>(p, a.batch, st) : launch_fp8_exact<DT_F16, true, 3>(p, a.batch, st);
+        case 0: return f32 ? launch_fp8_exact<DT_F32, true, 0>(p, a.batch, st) : bf ? launch_fp8_exact<DT_BF16, true, 0>(p, a.batch, st) : launch_fp8_exact<DT_F16, true, 0>(p, a.batch, st);
+        case 1: return f32 ? launch_fp8_exact<DT_F32, true, 1>(p, a.batch, st) : bf ? launch_fp8_exact<DT_BF16, true, 1>(p, a.batch, st) : launch_fp8_exact<DT_F16, true, 1>(p, a.batch, st);
+        case 2: return f32 ? launch_fp8_exact<DT_F32, true, 2>(p, a.batch, st) : bf ? launch_fp8_exact<DT_BF16, true, 2>(p, a.batch, st) : launch_fp8_exact<DT_F16, true, 2>(p, a.batch, st);
+        default: return f32 ? launch_fp8_exact<DT_F32, true, 3>(p, a.batch, st) : bf ? launch_fp8_exact<DT_BF16, true, 3>(p, a.batch, st) : launch_fp8_exact<DT_F16, true, 3>(p, a.batch, st);
     }
 }
 

@@ -89,6 +89,26 @@ def test_fp8_blockscale(gpu, M, K, N, tB, gsM, path):
     check_close(got, want, orc.BF16, "fp8 block scale", exact=path == "plain", fp8_mfma=path == "fast")
 
 
+@pytest.mark.parametrize("M,K,N,tB,gsM,fast", [(256, 1024, 384, True, 1, False), (300, 512, 262, False, 128, False), (128, 200, 256, True, 1, False),
+                                               (256, 1024, 384, True, 1, True)])
+def test_fp8_blockscale_fp32_output(gpu, M, K, N, tB, gsM, fast):
+    """FLOAT output of the block-scale modes: the exact matrix-core kernel stores its fp32 sums as they are (ragged
+    columns, an N-contiguous x2, a K tail; with the 8-bit instruction requested the exact kernel still serves it)."""
+    m = gpu
+    print(f"case fp8 block fp32 out M={M} K={K} N={N} tB={tB} gsM={gsM} fast={fast}", flush=True)
+    inp = cases.make_blockscale_inputs(m, M, K, N, M + N, tB, gsM)
+    want = cases.oracle_blockscale(m, inp, M, K, N, tB, m.ACL_FLOAT)
+    m.lib().opsnnSetFp8Fast(1 if fast else 0)
+    got = cases.run_blockscale_aclnn(m, inp, M, K, N, tB, m.ACL_FLOAT)
+    assert got.dtype == np.float32 and np.isfinite(got).all()
+    mx, mean = orc.rel_err_stats(got, want)
+    print(f"   max rel {mx:.3e} mean rel {mean:.3e}, {float(np.mean(got != want)):.3f} of fp32 outputs differ in some bit", flush=True)
+    assert mean <= 2.0 ** -16 and orc.isclose_fraction(got, want) == 0.0
+    assert not np.array_equal(got, want) or K <= 256   # the matrix-core route: its sums run in another order than the oracle's
+    plain(True)
+    assert np.array_equal(cases.run_blockscale_aclnn(m, inp, M, K, N, tB, m.ACL_FLOAT), want)
+
+
 def test_fp8_blockscale_exact_path_is_nearly_bit_identical(gpu):
     """The exact path differs from the ascending-k fp32 oracle only by summation order: at K = 2048 far fewer than
     0.5 % of bf16 outputs may differ at all (the 8-bit instruction leaves about 1 % one ulp off)."""
@@ -136,6 +156,29 @@ def test_mx(gpu, M, K, N, tB, fp4, use_plain):
         pos = dict(inp, x1=inp["x1"] & 0x7F, x2=inp["x2"] & 0x7F)
         abs_sum = orc.b16_to_f32(cases.oracle_mx(m, pos, M, K, N, tB, m.ACL_BF16), orc.BF16).astype(np.float64)
     check_close(got, want, orc.BF16, "mx", exact=use_plain, fp8_mfma=not fp4, abs_sum=abs_sum)
+
+
+@pytest.mark.parametrize("M,K,N,tB,fp4,bias", [(256, 1024, 384, True, True, True), (300, 512, 262, True, True, False), (128, 512, 256, False, True, True),
+                                               (200, 960, 264, True, True, False), (256, 1024, 384, True, False, True), (130, 256, 200, True, False, False)])
+def test_mx_fp32_output(gpu, M, K, N, tB, fp4, bias):
+    """FLOAT output of the MX modes on the tile kernels (fp32 sums plus bias stored straight from the registers): small
+    and large tiles, ragged columns, an N-contiguous x2, a K tail of half a tile; the plain kernel is bit-identical."""
+    m = gpu
+    print(f"case mx fp32 out M={M} K={K} N={N} tB={tB} fp4={fp4} bias={bias}", flush=True)
+    inp = cases.make_mx_inputs(m, M, K, N, K + N, tB, fp4)
+    b = np.random.default_rng(1).normal(0, 1, N).astype(np.float32) if bias else None
+    want = cases.oracle_mx(m, inp, M, K, N, tB, m.ACL_FLOAT, b)
+    got = cases.run_mx_aclnn(m, inp, M, K, N, tB, m.ACL_FLOAT, b)
+    assert got.dtype == np.float32 and np.isfinite(got).all()
+    pos = dict(inp, x1=inp["x1"] & (0x77 if fp4 else 0x7F), x2=inp["x2"] & (0x77 if fp4 else 0x7F))
+    abs_sum = cases.oracle_mx(m, pos, M, K, N, tB, m.ACL_FLOAT).astype(np.float64)
+    err = np.abs(got.astype(np.float64) - want.astype(np.float64))
+    # fp4 products are exact and the sums run in fp32: a few ulps of the sum of magnitudes; the 8-bit instruction aligns
+    # its 128 products in a narrower window (see check_close)
+    bound = (2.0 ** -20 if fp4 else 2.0 ** -14) * abs_sum + 1e-30
+    assert (err <= bound).all(), f"worst error / sum of magnitudes: {float((err / (abs_sum + 1e-30)).max()):.3e}"
+    plain(True)
+    assert np.array_equal(cases.run_mx_aclnn(m, inp, M, K, N, tB, m.ACL_FLOAT, b), want)
 
 
 @pytest.mark.parametrize("fn", [8, 9])

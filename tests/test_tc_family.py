@@ -283,6 +283,11 @@ def test_gpu_fp8_row_and_column_scales_on_the_matrix_cores(gpu, M, K, N, s_len, 
     (256, 1000, 264, "e4m3", "u64", "N", True, "bf16", True, False),
     (128, 512, 256, "e4m3", "f32", 1, False, "f16", False, True),
     (160, 200, 136, "e5m2", "f32", "N", True, "bf16", False, True),
+    # fp32 output (stored straight from the sums' registers): the three forms, ragged columns, a K tail
+    (256, 1024, 384, "e4m3", "f32", "N", True, "f32", True, "M"),
+    (200, 512, 130, "e4m3", "u64", "N", True, "f32", True, False),
+    (128, 256, 256, "e5m2", "f32", 1, False, "f32", True, True),
+    (130, 1000, 264, "e4m3", "f32", "N", False, "f32", True, "M"),
 ])
 def test_gpu_fp8_tc_forms_on_the_matrix_cores(gpu, M, K, N, in_dt, s_dt, s_len, bias, out_dt, tB, pt):
     """The fp8 members of the per-tensor / per-channel family with a 16-bit output on the exact matrix-core kernel (fp16
@@ -292,6 +297,17 @@ def test_gpu_fp8_tc_forms_on_the_matrix_cores(gpu, M, K, N, in_dt, s_dt, s_len, 
     dt = {"e4m3": m.ACL_FLOAT8_E4M3FN, "e5m2": m.ACL_FLOAT8_E5M2, "u64": m.ACL_UINT64, "f32": m.ACL_FLOAT, "bf16": m.ACL_BF16,
           "f16": m.ACL_FLOAT16}
     print(f"case fp8 tc form {M}x{K}x{N} in={in_dt} scale={s_dt}/{s_len} bias={bias} out={out_dt} tB={tB} pt={pt}", flush=True)
+    if out_dt == "f32":
+        # the matrix-core route is the one taken: the plain kernel would be bit-identical to the oracle, this one differs in
+        # the order of the sums only
+        inp = cases.make_tc_inputs(m, M, K, N, M + K, dt[in_dt], dt[s_dt], 1 if s_len == 1 else N, m.ACL_FLOAT if bias else None, tB,
+                                   pertoken=pt, e5m2=in_dt == "e5m2")
+        want = cases.oracle_tc(m, inp, M, K, N, m.ACL_FLOAT)
+        got = cases.run_tc_aclnn(m, inp, M, K, N, m.ACL_FLOAT)
+        assert got.dtype == np.float32 and np.isfinite(got).all()
+        mx, mean = orc.rel_err_stats(got, want)
+        assert mean <= 2.0 ** -16 and orc.isclose_fraction(got, want) == 0.0, f"max rel {mx:.3e} mean rel {mean:.3e}"
+        return
     inp = cases.make_tc_inputs(m, M, K, N, M + K, dt[in_dt], dt[s_dt], 1 if s_len == 1 else N, m.ACL_FLOAT if bias else None, tB,
                                pertoken=pt, e5m2=in_dt == "e5m2")
     want = cases.oracle_tc(m, inp, M, K, N, dt[out_dt])
