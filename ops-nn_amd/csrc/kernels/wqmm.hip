@@ -410,6 +410,23 @@ static int launch_slabs(WqParams p, hipStream_t st)
         const int rc = launch_wq_tile<XDT, WBITS>(p, st);
         if (rc != OPSNN_NOT_TAKEN) return rc;
     }
+    // more rows still: the same kernel in passes of up to 256 rows, in equal slabs (2048 rows: 8 passes over the weight
+    // instead of 16 of the streaming kernel)
+    if (p.M > 256 && opsnn_wq_tile_min() <= 256) {
+        const int64_t passes = (p.M + 255) / 256;
+        const int64_t slab = ((p.M + passes - 1) / passes + 15) / 16 * 16;
+        bool taken = true;
+        for (int64_t m0 = 0; m0 < p.M && taken; m0 += slab) {
+            WqParams q = p;
+            q.x = p.x + m0 * p.K;
+            q.y = p.y + m0 * p.N;
+            q.M = (p.M - m0) < slab ? (p.M - m0) : slab;
+            const int rc = launch_wq_tile<XDT, WBITS>(q, st);
+            if (rc == OPSNN_NOT_TAKEN && m0 == 0) taken = false;   // the shape conditions are the same for every slab
+            else if (rc != 0) return rc;
+        }
+        if (taken) return 0;
+    }
     WqStreamOpts o{};
     const bool stream = stream_eligible<WBITS>(p, o);
     // rows per launch: as many as one pass over the weights can serve, in equal slabs

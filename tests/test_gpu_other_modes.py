@@ -267,6 +267,11 @@ def test_mx_batched(gpu, M, K, N, batch):
     (200, 2048, 320, "bf16", "i4", 256, True, True, None),
     (256, 1024, 256, "f16", "i4", 128, True, False, "f16"),
     (130, 1024, 256, "bf16", "i8", 0, False, False, "bf16"),
+    # ... more than 256 rows: the dequantise-once tile kernel in passes of equal slabs (three of 208 rows, the last ragged;
+    # two of 144), and the streaming kernel's slabs where the tile kernel does not apply (a group of 32)
+    (600, 1024, 384, "f16", "i4", 128, True, True, "f16"),
+    (280, 512, 256, "bf16", "i8", 0, True, False, None),
+    (300, 1024, 256, "f16", "i4", 32, True, True, None),
 ])
 def test_weight_only(gpu, M, K, N, x_dt, w_dt, group, tW, off, bias, use_plain):
     m = gpu
