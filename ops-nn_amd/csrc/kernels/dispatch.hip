@@ -16,6 +16,7 @@ int launch_wqmm_plain(const OpsnnWqmmArgs& a, hipStream_t st);
 int launch_blockscale_mfma(const OpsnnQmmArgs& a, hipStream_t st);
 int launch_fp8_rowcol_mfma(const OpsnnQmmArgs& a, hipStream_t st, bool merged_scales_ok);
 int launch_rowcol_exact(const OpsnnQmmArgs& a, hipStream_t st, int ep_mode);   // qmm_fp8_exact.hip
+int launch_rowcol_decode(const OpsnnQmmArgs& a, hipStream_t st);   // qmm_fp8_decode.hip
 int launch_tcg_mfma(const OpsnnQmmArgs& a, hipStream_t st);
 uint64_t tcg_workspace_bytes(const OpsnnQmmArgs& a);
 int launch_kg_mfma(const OpsnnQmmArgs& a, hipStream_t st);   // qmm_i4_kg.hip
@@ -231,6 +232,10 @@ extern "C" int opsnnQmmTc(const OpsnnQmmArgs* a, void* stream)
     // the other two forms run here.
     if (f8 && a->force_variant != OPSNN_VARIANT_PLAIN && !opsnn_force_plain()) {
         const int ep = !a->x1_scale ? 1 : (a->x1_scale_len == 1 && a->x2_scale_len == 1 && !a->bias) ? 2 : 0;
+        if (ep == 0) {   // up to 32 rows: the stream over x2 with x1 in registers
+            const int rc = launch_rowcol_decode(*a, (hipStream_t)stream);
+            if (rc != OPSNN_NOT_TAKEN) return rc;
+        }
         const bool e4 = a->x1_dtype == DT_E4M3 && a->x2_dtype == DT_E4M3;
         if (ep != 0 || !e4 || a->x2_scale_dtype != DT_F32 || a->out_dtype == DT_F32) {
             const int rc = launch_rowcol_exact(*a, (hipStream_t)stream, ep);

@@ -621,6 +621,8 @@ int launch_fp8_rowcol_mfma(const OpsnnQmmArgs& a, hipStream_t st, bool merged_sc
     return launch_fp8_block<2, 2, DT_F16, FP8_ROWCOL>(p, a.batch, st);
 }
 
+int launch_blockscale_decode(const OpsnnQmmArgs& a, hipStream_t st);   // qmm_fp8_decode.hip
+
 int launch_blockscale_mfma(const OpsnnQmmArgs& a0, hipStream_t st)
 {
     OpsnnQmmArgs a = a0;
@@ -644,6 +646,10 @@ int launch_blockscale_mfma(const OpsnnQmmArgs& a0, hipStream_t st)
             a.x2.ptr = a.workspace;
         }
         a.x2.row_stride = 1; a.x2.col_stride = a.K;
+    }
+    if (!i8) {   // up to 32 rows: the stream over x2 with x1 in registers (exact products and sums)
+        const int rc = launch_blockscale_decode(a, st);
+        if (rc != OPSNN_NOT_TAKEN) return rc;
     }
     if (!i8 && (!opsnnGetFp8Fast() || out32)) {   // exact products and sums unless the caller asked for the 8-bit matrix instruction
         const int rc = launch_blockscale_exact(a, st);

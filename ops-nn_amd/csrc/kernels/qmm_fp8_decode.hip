@@ -1,0 +1,270 @@
+// fp8 e4m3 x fp8 e4m3 with block scales (G-B, B-B) for up to 16 rows of x1 per pass: the decode shape of an fp8 model.
+//
+//   out[m,n] = cast( sum_kb ( sum_{k in block kb} x1[m,k] * x2[k,n] ) * ( s1[m/gsM, kb] * s2[kb, n/128] ) )
+//
+// Formula: matmul/quant_batch_matmul_v3/tests/assets/qbmmv3_kernel_golden.py:237-358 (the two block scales are multiplied
+// together first, :337-343).  Arithmetic as in qmm_fp8_exact.hip: the operands are widened to fp16 (exact), the products
+// are exact, a block's sum is an fp32 accumulation inside v_mfma_f32_16x16x32_f16 chained over the block's four steps from
+// a zero accumulator, and one fused multiply-add per output folds it into the running sum.
+//
+// With so few rows the work is a stream over x2 (N * K bytes), not a GEMM: a 256-row tile kernel spends 16 times the
+// matrix work and conversions on rows that do not exist.  Here, as in the x-in-registers kernel of wqmm_stream.hip.h:
+//   * the workgroup's NW waves split K into NW equal ranges of NBLK scale blocks; a wave keeps the fp16 fragments of
+//     x1 for its range in registers for the whole launch (16 registers per block),
+//   * all waves work on the same 16 columns of the output (16 rows of the K-contiguous x2) at a time and the workgroup
+//     walks column blocks blockIdx.x, + gridDim.x, ...; the stream of x2 pieces (16 bytes per lane) never stops: the
+//     refills issued while one column block is multiplied already fetch the next one's pieces,
+//   * a lane's 16-byte piece of an x2 row feeds two matrix instructions (bytes 0..7 and 8..15); which k a lane holds
+//     inside an instruction does not matter as long as both operands agree, and x1's fragments are cut the same way,
+//   * the NW partial sums of a column block meet in LDS (double-buffered, one barrier per column block) and one wave,
+//     taking turns, adds them in wave order and stores 16 x 16 outputs.
+// The order of the fp32 additions differs from the golden's ascending blocks (NW ranges are added at the end): the bar
+// of the exact tile kernel.
+#include <cstdlib>
+
+#include "launch.h"
+#include "common.hip.h"
+
+namespace opsnn {
+namespace {
+
+struct Fp8DecParams {
+    const uint8_t* a;   // x1 [M, K], K contiguous
+    const uint8_t* b;   // x2 as [N, K], K contiguous
+    int64_t lda, ldb;
+    void* out; int out_dt;
+    int64_t M, N, K;
+    const float* s1; int64_t s1_rs, s1_cs;
+    const float* s2; int64_t s2_rs, s2_cs;
+    int gsM;
+    // row / column scale form (RC): out = (sum * cs[n * cs_stride]) * rs[m * rs_stride] + bias[n]; strides 0 (one scale) or 1
+    const float* rs; const float* cs; const float* bias;
+    int rs_stride, cs_stride;
+};
+
+// 8 e4m3 bytes (two dwords) -> 8 fp16 in byte order
+__device__ __forceinline__ v4i widen8_e4m3(uint32_t d0, uint32_t d1)
+{
+    typedef _Float16 h2v __attribute__((ext_vector_type(2)));
+    const h2v w0 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(d0, 1.0f, false), w1 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(d0, 1.0f, true);
+    const h2v w2 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(d1, 1.0f, false), w3 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(d1, 1.0f, true);
+    return (v4i){(int)__builtin_bit_cast(uint32_t, w0), (int)__builtin_bit_cast(uint32_t, w1), (int)__builtin_bit_cast(uint32_t, w2),
+                 (int)__builtin_bit_cast(uint32_t, w3)};
+}
+
+template <int NW, int NBLK, bool RC>
+__global__ __launch_bounds__(NW * 64) void fp8_block_decode_kernel(Fp8DecParams p)
+{
+    constexpr int NCH = 2 * NBLK;                    // 64-byte chunks of an x2 row in a wave's K range
+    constexpr int PF = NW == 16 ? (NCH < 4 ? NCH : 4) : NCH;   // pieces in flight per lane; divides NCH
+    static_assert(NCH % PF == 0, "a piece's slot must not depend on the column block");
+    extern __shared__ __attribute__((aligned(16))) float red[];   // [2][NW][256]
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int nrow = lane & 15, q = lane >> 4;
+    const int64_t kbase = (int64_t)wave * (NBLK * 128);
+    const int kb0 = wave * NBLK;
+    const int nblocks = (int)((p.N + 15) / 16);
+    const int M = (int)p.M;
+
+    // x1: lane (m = lane % 16, q) holds, for chunk c and half h, the 8 elements k = kbase + 64 c + 16 q + 8 h .. + 7
+    v4i xf[NCH][2];
+#pragma unroll
+    for (int c = 0; c < NCH; c++) {
+        uint4 raw = make_uint4(0, 0, 0, 0);
+        if (nrow < M) raw = *(const uint4*)(p.a + (int64_t)nrow * p.lda + kbase + 64 * c + 16 * q);
+        xf[c][0] = widen8_e4m3(raw.x, raw.y);
+        xf[c][1] = widen8_e4m3(raw.z, raw.w);
+    }
+    // the scales of this lane's row of x1 for the wave's blocks (rows past M: the last row's, their outputs are not stored)
+    float s1v[NBLK];
+    if constexpr (!RC) {
+        const int64_t mr = (nrow < M ? nrow : M - 1) / p.gsM;
+#pragma unroll
+        for (int j = 0; j < NBLK; j++) s1v[j] = p.s1[mr * p.s1_rs + (kb0 + j) * p.s1_cs];
+    }
+
+    auto wload = [&](int rb, int c) {
+        const int64_t n = (int64_t)rb * 16 + nrow;
+        return *(const uint4*)(p.b + (n < p.N ? n : p.N - 1) * p.ldb + kbase + 64 * c + 16 * q);   // columns past the edge repeat the last one
+    };
+    int rb = blockIdx.x;
+    uint4 wq[PF];
+#pragma unroll
+    for (int i = 0; i < PF; i++) wq[i] = wload(rb < nblocks ? rb : nblocks - 1, i);
+
+    for (int it = 0; rb < nblocks; it++, rb += (int)gridDim.x) {
+        const int rbn = rb + (int)gridDim.x < nblocks ? rb + (int)gridDim.x : rb;   // past the end: a harmless reload
+        const int64_t n0 = (int64_t)rb * 16;
+        float s2v[NBLK];
+        if constexpr (!RC) {
+#pragma unroll
+            for (int j = 0; j < NBLK; j++) s2v[j] = p.s2[(kb0 + j) * p.s2_rs + (n0 / 128) * p.s2_cs];
+        }
+        v4f acc = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+        for (int j = 0; j < NBLK; j++) {
+            v4f t = RC ? acc : (v4f){0.0f, 0.0f, 0.0f, 0.0f};   // RC: one chain over the whole range
+#pragma unroll
+            for (int cc = 0; cc < 2; cc++) {
+                const int c = 2 * j + cc;
+                const uint4 cur = wq[c % PF];
+                wq[c % PF] = c + PF < NCH ? wload(rb, c + PF) : wload(rbn, c + PF - NCH);
+                const v4i w0 = widen8_e4m3(cur.x, cur.y), w1 = widen8_e4m3(cur.z, cur.w);
+                t = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(v8h, w0), __builtin_bit_cast(v8h, xf[c][0]), t, 0, 0, 0);
+                t = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(v8h, w1), __builtin_bit_cast(v8h, xf[c][1]), t, 0, 0, 0);
+            }
+            if constexpr (RC) acc = t;
+            else {
+                const float sc = s1v[j] * s2v[j];
+#pragma unroll
+                for (int r = 0; r < 4; r++) acc[r] = __builtin_fmaf(t[r], sc, acc[r]);
+            }
+        }
+        // acc[r]: m = lane % 16, n = n0 + 4 (lane / 16) + r, over this wave's K range
+        float* mine = red + ((it & 1) * NW + wave) * 256;
+        *(v4f*)(mine + lane * 4) = acc;
+        __syncthreads();
+        if (wave != (it & (NW - 1))) continue;
+        const float* all = red + (it & 1) * NW * 256 + lane * 4;
+        v4f sum = *(const v4f*)all;
+#pragma unroll 4
+        for (int w = 1; w < NW; w++) {
+            const v4f o = *(const v4f*)(all + w * 256);
+#pragma unroll
+            for (int r = 0; r < 4; r++) sum[r] = sum[r] + o[r];
+        }
+        if (nrow >= M) continue;
+        const int64_t n = n0 + 4 * q;
+        if constexpr (RC) {   // (sum * x2Scale[n]) * x1Scale[m] + bias[n], each operation rounded
+            const float rsv = p.rs[(int64_t)nrow * p.rs_stride];
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                const int64_t ni = n + r < p.N ? n + r : p.N - 1;
+                sum[r] = (sum[r] * p.cs[ni * p.cs_stride]) * rsv;
+                if (p.bias) sum[r] = sum[r] + p.bias[ni];
+            }
+        }
+        if (p.out_dt == DT_F32) {
+            float* dst = (float*)p.out + (int64_t)nrow * p.N + n;
+#pragma unroll
+            for (int r = 0; r < 4; r++)
+                if (n + r < p.N) dst[r] = sum[r];
+        } else {
+            const v4us o = p.out_dt == DT_BF16 ? pack4_b16<DT_BF16>(sum) : pack4_b16<DT_F16>(sum);
+            uint16_t* dst = (uint16_t*)p.out + (int64_t)nrow * p.N + n;
+            if ((p.N % 4) == 0 && ((uintptr_t)p.out % 8) == 0 && n + 3 < p.N) *(v4us*)dst = o;
+            else {
+#pragma unroll
+                for (int r = 0; r < 4; r++)
+                    if (n + r < p.N) dst[r] = o[r];
+            }
+        }
+    }
+}
+
+template <int NW, int NBLK, bool RC>
+int launch_decode_one(const Fp8DecParams& p, hipStream_t st)
+{
+    const int nblocks = (int)((p.N + 15) / 16);
+    const int cus = 256;
+    const int grid = nblocks < cus ? nblocks : cus;
+    const size_t lds = (size_t)2 * NW * 256 * sizeof(float);
+    hipLaunchKernelGGL((fp8_block_decode_kernel<NW, NBLK, RC>), dim3((unsigned)grid), dim3(NW * 64), lds, st, p);
+    return (int)hipGetLastError();
+}
+
+// K as a whole number of 128-element blocks that 16 or 8 waves share equally (the registers hold up to 7 blocks of x1)
+bool decode_split(int64_t K, int& nw, int& nblk)
+{
+    if (K % 128 != 0) return false;
+    const int64_t nb = K / 128;
+    if (nb % 16 == 0 && nb / 16 <= 4 && nb / 16 != 3) { nw = 16; nblk = (int)(nb / 16); return true; }
+    if (nb % 8 == 0 && nb / 8 <= 7) { nw = 8; nblk = (int)(nb / 8); return true; }
+    return false;
+}
+
+template <bool RC>
+int launch_decode_split(const Fp8DecParams& p, int nw, int nblk, hipStream_t st)
+{
+    if (nw == 16) {
+        if (nblk == 1) return launch_decode_one<16, 1, RC>(p, st);
+        if (nblk == 2) return launch_decode_one<16, 2, RC>(p, st);
+        return launch_decode_one<16, 4, RC>(p, st);
+    }
+    switch (nblk) {
+        case 1: return launch_decode_one<8, 1, RC>(p, st);
+        case 2: return launch_decode_one<8, 2, RC>(p, st);
+        case 3: return launch_decode_one<8, 3, RC>(p, st);
+        case 4: return launch_decode_one<8, 4, RC>(p, st);
+        case 5: return launch_decode_one<8, 5, RC>(p, st);
+        case 6: return launch_decode_one<8, 6, RC>(p, st);
+        default: return launch_decode_one<8, 7, RC>(p, st);
+    }
+}
+
+}  // namespace
+
+// fp8 e4m3 block scales with up to 32 rows of x1 (two passes beyond 16), K-contiguous operands, K a whole number of
+// blocks that 16 or 8 waves share equally; OPSNN_NOT_TAKEN otherwise.
+int launch_blockscale_decode(const OpsnnQmmArgs& a, hipStream_t st)
+{
+    static const bool off = [] { const char* e = getenv("OPSNN_FP8_NO_DECODE"); return e && e[0] == '1'; }();
+    if (off || a.x1_dtype != DT_E4M3 || a.x2_dtype != DT_E4M3 || a.batch != 1) return OPSNN_NOT_TAKEN;
+    if (a.out_dtype != DT_BF16 && a.out_dtype != DT_F16 && a.out_dtype != DT_F32) return OPSNN_NOT_TAKEN;
+    if (a.bias || a.M > 32 || a.N < 256) return OPSNN_NOT_TAKEN;
+    if (a.gsK != 128 || a.gsN != 128 || (a.gsM != 1 && a.gsM != 128)) return OPSNN_NOT_TAKEN;
+    if (a.K % 128 != 0 || a.x1.col_stride != 1 || a.x2.row_stride != 1) return OPSNN_NOT_TAKEN;
+    if (((uintptr_t)a.x1.ptr | (uintptr_t)a.x2.ptr | (uint64_t)a.x1.row_stride | (uint64_t)a.x2.col_stride) % 16) return OPSNN_NOT_TAKEN;
+    if (((uintptr_t)a.x1_scale_mat.ptr | (uintptr_t)a.x2_scale_mat.ptr) % 4) return OPSNN_NOT_TAKEN;
+    if (a.x1.row_stride < a.K || a.x2.col_stride < a.K) return OPSNN_NOT_TAKEN;
+    int nw = 0, nblk = 0;
+    if (!decode_split(a.K, nw, nblk)) return OPSNN_NOT_TAKEN;
+    for (int64_t m0 = 0; m0 < a.M; m0 += 16) {
+        Fp8DecParams p{};
+        p.M = a.M - m0 < 16 ? a.M - m0 : 16; p.N = a.N; p.K = a.K;
+        p.a = (const uint8_t*)a.x1.ptr + m0 * a.x1.row_stride; p.b = (const uint8_t*)a.x2.ptr;
+        p.lda = a.x1.row_stride; p.ldb = a.x2.col_stride;
+        p.out_dt = a.out_dtype;
+        p.out = (char*)a.out + m0 * a.N * (a.out_dtype == DT_F32 ? 4 : 2);
+        p.gsM = (int)a.gsM;
+        // gsM 1: the pass's own rows of the scale table; gsM 128: up to 32 rows share row 0
+        p.s1 = (const float*)a.x1_scale_mat.ptr + (a.gsM == 1 ? m0 * a.x1_scale_mat.row_stride : 0);
+        p.s1_rs = a.x1_scale_mat.row_stride; p.s1_cs = a.x1_scale_mat.col_stride;
+        p.s2 = (const float*)a.x2_scale_mat.ptr; p.s2_rs = a.x2_scale_mat.row_stride; p.s2_cs = a.x2_scale_mat.col_stride;
+        const int rc = launch_decode_split<false>(p, nw, nblk, st);
+        if (rc != 0) return rc;
+    }
+    return 0;
+}
+
+// fp8 e4m3 with one fp32 scale per row of x1 (or one) and one per column of x2 (or one), optional fp32 bias -- the form
+// (sum * x2Scale) * x1Scale + bias of compute_pertoken (qbmmv3_kernel_golden.py:361-387) -- for up to 32 rows.
+int launch_rowcol_decode(const OpsnnQmmArgs& a, hipStream_t st)
+{
+    static const bool off = [] { const char* e = getenv("OPSNN_FP8_NO_DECODE"); return e && e[0] == '1'; }();
+    if (off || a.x1_dtype != DT_E4M3 || a.x2_dtype != DT_E4M3 || a.batch != 1) return OPSNN_NOT_TAKEN;
+    if (a.out_dtype != DT_BF16 && a.out_dtype != DT_F16 && a.out_dtype != DT_F32) return OPSNN_NOT_TAKEN;
+    if (!a.x1_scale || !a.x2_scale || a.x2_scale_dtype != DT_F32 || (a.bias && a.bias_dtype != DT_F32)) return OPSNN_NOT_TAKEN;
+    if (a.M > 32 || a.N < 256 || a.x1.col_stride != 1 || a.x2.row_stride != 1) return OPSNN_NOT_TAKEN;
+    if (((uintptr_t)a.x1.ptr | (uintptr_t)a.x2.ptr | (uint64_t)a.x1.row_stride | (uint64_t)a.x2.col_stride) % 16) return OPSNN_NOT_TAKEN;
+    if (a.x1.row_stride < a.K || a.x2.col_stride < a.K) return OPSNN_NOT_TAKEN;
+    int nw = 0, nblk = 0;
+    if (!decode_split(a.K, nw, nblk)) return OPSNN_NOT_TAKEN;
+    for (int64_t m0 = 0; m0 < a.M; m0 += 16) {
+        Fp8DecParams p{};
+        p.M = a.M - m0 < 16 ? a.M - m0 : 16; p.N = a.N; p.K = a.K;
+        p.a = (const uint8_t*)a.x1.ptr + m0 * a.x1.row_stride; p.b = (const uint8_t*)a.x2.ptr;
+        p.lda = a.x1.row_stride; p.ldb = a.x2.col_stride;
+        p.out_dt = a.out_dtype;
+        p.out = (char*)a.out + m0 * a.N * (a.out_dtype == DT_F32 ? 4 : 2);
+        p.rs_stride = a.x1_scale_len == 1 ? 0 : 1; p.cs_stride = a.x2_scale_len == 1 ? 0 : 1;
+        p.rs = (const float*)a.x1_scale + (p.rs_stride ? m0 : 0);
+        p.cs = (const float*)a.x2_scale; p.bias = (const float*)a.bias;
+        const int rc = launch_decode_split<true>(p, nw, nblk, st);
+        if (rc != 0) return rc;
+    }
+    return 0;
+}
+
+}  // namespace opsnn

@@ -109,6 +109,37 @@ def test_fp8_blockscale_fp32_output(gpu, M, K, N, tB, gsM, fast):
     assert np.array_equal(cases.run_blockscale_aclnn(m, inp, M, K, N, tB, m.ACL_FLOAT), want)
 
 
+@pytest.mark.parametrize("M,K,N,gsM,out", [
+    # up to 16 rows (one pass): K shared by 16 waves (2048, 4096, 8192) or by 8 (1024, 3072, 5120, 6144, 7168); ragged columns;
+    # more column blocks than workgroups (N = 8192: 512 blocks on 256 workgroups) and fewer
+    (1, 2048, 256, 1, "bf16"), (16, 4096, 512, 1, "f16"), (7, 8192, 8192, 1, "bf16"), (16, 1024, 264, 1, "bf16"),
+    (5, 3072, 1000, 1, "f16"), (16, 5120, 384, 1, "f32"), (9, 6144, 256, 128, "bf16"), (16, 7168, 2304, 1, "bf16"),
+    # 17 .. 32 rows: two passes; one scale row for all of x1 (B-B)
+    (17, 2048, 512, 1, "bf16"), (32, 7168, 520, 128, "f16"), (24, 4096, 256, 1, "f32"),
+])
+def test_fp8_blockscale_decode_rows(gpu, M, K, N, gsM, out):
+    """The block-scale modes with up to 32 rows of x1 (x2 K-contiguous): x1 stays in registers as exact fp16 and x2 is
+    streamed once per 16 rows; exact products, fp32 sums per block, one fused multiply-add per block (the exact tile
+    kernel's arithmetic, its bar)."""
+    m = gpu
+    dt = {"bf16": m.ACL_BF16, "f16": m.ACL_FLOAT16, "f32": m.ACL_FLOAT}[out]
+    print(f"case fp8 block decode M={M} K={K} N={N} gsM={gsM} out={out}", flush=True)
+    inp = cases.make_blockscale_inputs(m, M, K, N, M + N + K, True, gsM)
+    want = cases.oracle_blockscale(m, inp, M, K, N, True, dt)
+    got = cases.run_blockscale_aclnn(m, inp, M, K, N, True, dt)
+    if out == "f32":
+        assert np.isfinite(got).all()
+        mx, mean = orc.rel_err_stats(got, want)
+        assert mean <= 2.0 ** -16 and orc.isclose_fraction(got, want) == 0.0, f"max rel {mx:.3e} mean rel {mean:.3e}"
+    else:
+        check_close(got, want, orc.BF16 if out == "bf16" else orc.F16, "fp8 block scale, decode rows")
+        differ = float(np.mean(got != want))
+        print(f"   {differ:.2e} of outputs differ from the ascending-block oracle", flush=True)
+        assert differ < 2e-2
+    plain(True)
+    assert np.array_equal(cases.run_blockscale_aclnn(m, inp, M, K, N, True, dt), want)
+
+
 def test_fp8_blockscale_exact_path_is_nearly_bit_identical(gpu):
     """The exact path differs from the ascending-k fp32 oracle only by summation order: at K = 2048 far fewer than
     0.5 % of bf16 outputs may differ at all (the 8-bit instruction leaves about 1 % one ulp off)."""

@@ -232,6 +232,12 @@ def test_gpu_matches_oracle(gpu, M, K, N, in_dt, s_dt, s_len, bias_dt, out_dt, t
     # 4 x 60 tiles of 256 x 288 one (ragged last column tile; one-element x1Scale in the second case)
     (1000, 1024, 16600, "N", True, "bf16", "M"),
     (1024, 1024, 16640, "N", False, "f16", True),
+    # up to 32 rows (x1 in registers, x2 streamed once per 16 rows): K shared by 16 waves and by 8, ragged columns, one pass
+    # and two, one-element scales
+    (1, 4096, 512, "N", True, "bf16", "M"),
+    (16, 7168, 1000, "N", False, "f16", "M"),
+    (20, 2048, 264, "N", True, "bf16", "M"),
+    (32, 1024, 256, 1, True, "f16", True),
 ])
 def test_gpu_fp8_row_and_column_scales_on_the_matrix_cores(gpu, M, K, N, s_len, bias, out_dt, pt, fast):
     """fp8 e4m3 K-C / K-T / T-C-double-scale on the matrix cores (K-contiguous x2, K % 128 == 0, 16-bit output).  Default:
