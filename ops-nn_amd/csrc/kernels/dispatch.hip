@@ -17,6 +17,7 @@ int launch_blockscale_mfma(const OpsnnQmmArgs& a, hipStream_t st);
 int launch_fp8_rowcol_mfma(const OpsnnQmmArgs& a, hipStream_t st, bool merged_scales_ok);
 int launch_rowcol_exact(const OpsnnQmmArgs& a, hipStream_t st, int ep_mode);   // qmm_fp8_exact.hip
 int launch_rowcol_decode(const OpsnnQmmArgs& a, hipStream_t st);   // qmm_fp8_decode.hip
+uint64_t blockscale_rows_workspace(const OpsnnQmmArgs& a);         // qmm_fp8_rows.hip
 int launch_tcg_mfma(const OpsnnQmmArgs& a, hipStream_t st);
 uint64_t tcg_workspace_bytes(const OpsnnQmmArgs& a);
 int launch_kg_mfma(const OpsnnQmmArgs& a, hipStream_t st);   // qmm_i4_kg.hip
@@ -297,6 +298,9 @@ extern "C" uint64_t opsnnQmmWorkspace(const OpsnnQmmArgs* a, int mode)
     if (!a) return 0;
     if (const int64_t Kp = k_pad_for(*a, mode)) return k_pad_bytes(*a, Kp);
     if (mode == 2) return mx_workspace_bytes(*a);
+    if (mode == 1 && a->x2.row_stride == 1 && a->force_variant != OPSNN_VARIANT_PLAIN && !opsnn_force_plain()) {
+        if (const uint64_t b = blockscale_rows_workspace(*a)) return b;   // fp8 block scales with 33 .. 64 rows: x1 widened to fp16
+    }
     // per-tensor / per-channel family: int8 operands share the int8 kernels and their re-layout; fp8 needs none
     if (mode == 3 && !(a->x1_dtype == DT_I8 && a->x2_dtype == DT_I8 && !a->x1_scale)) return 0;
     // K-group modes: the re-quantised weight of the fp8 x fp4 group-scale mode; the widened operands, row sums and fp32

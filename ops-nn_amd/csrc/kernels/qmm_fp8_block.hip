@@ -622,6 +622,7 @@ int launch_fp8_rowcol_mfma(const OpsnnQmmArgs& a, hipStream_t st, bool merged_sc
 }
 
 int launch_blockscale_decode(const OpsnnQmmArgs& a, hipStream_t st);   // qmm_fp8_decode.hip
+int launch_blockscale_rows(const OpsnnQmmArgs& a, hipStream_t st);     // qmm_fp8_rows.hip
 
 int launch_blockscale_mfma(const OpsnnQmmArgs& a0, hipStream_t st)
 {
@@ -649,6 +650,10 @@ int launch_blockscale_mfma(const OpsnnQmmArgs& a0, hipStream_t st)
     }
     if (!i8) {   // up to 32 rows: the stream over x2 with x1 in registers (exact products and sums)
         const int rc = launch_blockscale_decode(a, st);
+        if (rc != OPSNN_NOT_TAKEN) return rc;
+    }
+    if (!i8 && a0.x2.row_stride == 1) {   // 33 .. 64 rows: x1 widened into the workspace, then the many-rows streaming kernel
+        const int rc = launch_blockscale_rows(a, st);
         if (rc != OPSNN_NOT_TAKEN) return rc;
     }
     if (!i8 && (!opsnnGetFp8Fast() || out32)) {   // exact products and sums unless the caller asked for the 8-bit matrix instruction

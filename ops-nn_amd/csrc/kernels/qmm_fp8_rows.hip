@@ -1,0 +1,74 @@
+// fp8 e4m3 block-scale matmul (G-B, B-B) with 33 .. 64 rows of x1: the many-rows streaming kernel of wqmm_stream.hip.h
+// in its block-scale form (WF = 3).  A pre-step widens x1 to fp16 in the workspace (exact; M * K * 2 bytes), so that x
+// travels global -> LDS by asynchronous copies like the activations of the weight-only path; x2 is streamed once and
+// widened in registers.  Formula and arithmetic: see qmm_fp8_decode.hip (exact products, fp32 sums per half block, one
+// fused multiply-add per half block and output).
+#include <cstdlib>
+
+#include "wqmm_stream.hip.h"
+
+namespace opsnn {
+namespace {
+
+// 16 e4m3 bytes -> 16 fp16
+__global__ __launch_bounds__(256) void widen_e4m3_f16_kernel(const uint8_t* __restrict__ src, int64_t ld, uint16_t* __restrict__ dst, int64_t rows, int64_t K)
+{
+    const int64_t pieces = K / 16;
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= rows * pieces) return;
+    const int64_t r = i / pieces, c = i - r * pieces;
+    const uint4 v = *(const uint4*)(src + r * ld + c * 16);
+    const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+    uint32_t o[8];
+#pragma unroll
+    for (int d = 0; d < 4; d++) {
+        typedef _Float16 h2v __attribute__((ext_vector_type(2)));
+        o[2 * d] = __builtin_bit_cast(uint32_t, (h2v)__builtin_amdgcn_cvt_scalef32_pk_f16_fp8(w[d], 1.0f, false));
+        o[2 * d + 1] = __builtin_bit_cast(uint32_t, (h2v)__builtin_amdgcn_cvt_scalef32_pk_f16_fp8(w[d], 1.0f, true));
+    }
+    uint4* out = (uint4*)(dst + r * K + c * 16);
+    out[0] = make_uint4(o[0], o[1], o[2], o[3]);
+    out[1] = make_uint4(o[4], o[5], o[6], o[7]);
+}
+
+bool rows_eligible(const OpsnnQmmArgs& a)
+{
+    static const bool off = [] { const char* e = getenv("OPSNN_FP8_NO_DECODE"); return e && e[0] == '1'; }();
+    if (off || a.x1_dtype != DT_E4M3 || a.x2_dtype != DT_E4M3 || a.batch != 1 || a.bias) return false;
+    if (a.out_dtype != DT_BF16 && a.out_dtype != DT_F16 && a.out_dtype != DT_F32) return false;
+    if (a.M <= 32 || a.M > 64) return false;   // (the 128-row instance of the kernel does not fit the register file in this form)
+    if (a.gsK != 128 || a.gsN != 128 || (a.gsM != 1 && a.gsM != 128)) return false;
+    // the kernel's shape conditions: whole workgroups of 128 columns inside one scale block, K in slabs of 128 with the
+    // weight stream four chunks deep, 16-byte pieces
+    if (a.N % 128 != 0 || a.N < 256 || a.K % 512 != 0 || a.K / 128 * 16 * 4 * 4 > 65536) return false;
+    if (a.x1.col_stride != 1 || a.x2.row_stride != 1 || a.x1.row_stride < a.K || a.x2.col_stride < a.K) return false;
+    if (((uintptr_t)a.x1.ptr | (uintptr_t)a.x2.ptr | (uint64_t)a.x1.row_stride | (uint64_t)a.x2.col_stride) % 16) return false;
+    if (((uintptr_t)a.x1_scale_mat.ptr | (uintptr_t)a.x2_scale_mat.ptr) % 4 || (uintptr_t)a.out % 16) return false;
+    if (a.K >= (1ll << 31) || a.N >= (1ll << 31)) return false;
+    return true;
+}
+
+}  // namespace
+
+uint64_t blockscale_rows_workspace(const OpsnnQmmArgs& a) { return rows_eligible(a) ? (uint64_t)a.M * (uint64_t)a.K * 2 : 0; }
+
+int launch_blockscale_rows(const OpsnnQmmArgs& a, hipStream_t st)
+{
+    if (!rows_eligible(a) || !a.workspace || (uintptr_t)a.workspace % 16) return OPSNN_NOT_TAKEN;
+    uint16_t* x16 = (uint16_t*)a.workspace;
+    const int64_t pieces = a.M * (a.K / 16);
+    hipLaunchKernelGGL(widen_e4m3_f16_kernel, dim3((unsigned)((pieces + 255) / 256)), dim3(256), 0, st, (const uint8_t*)a.x1.ptr, a.x1.row_stride, x16,
+                       a.M, a.K);
+    WqParams p{};
+    p.x = x16; p.w = (const uint8_t*)a.x2.ptr; p.ldw = a.x2.col_stride;
+    p.y = (uint16_t*)a.out; p.M = a.M; p.N = a.N; p.K = a.K;
+    p.group = a.K; p.group_shift = -1; p.cpg_shift = 31;
+    p.m_base = 0; p.m_rows = a.M;
+    p.w_float = 1;
+    p.bs1 = (const float*)a.x1_scale_mat.ptr; p.bs1_rs = a.x1_scale_mat.row_stride; p.bs1_cs = a.x1_scale_mat.col_stride;
+    p.bs2 = (const float*)a.x2_scale_mat.ptr; p.bs2_rs = a.x2_scale_mat.row_stride; p.bs2_cs = a.x2_scale_mat.col_stride;
+    p.bs_gsm = (int)a.gsM; p.bs_out_dt = a.out_dtype;
+    return launch_rows_one<DT_F16, 8, 4, 2, 4, 2, false, 3>(p, st);
+}
+
+}  // namespace opsnn

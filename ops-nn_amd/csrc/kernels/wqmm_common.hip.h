@@ -23,6 +23,11 @@ struct WqParams {
     int64_t m_base, m_rows;  // row slab handled by this launch
     int w_float;             // weights are floating-point codes (4 bits: e2m1, 8 bits: e4m3), not two's-complement integers
     int scale_e8m0;          // scale is one e8m0 byte per element (MX), not a 16-bit value of x's dtype
+    // fp8 block-scale form of the many-rows kernel (x is x1 widened to fp16, w is x2 in e4m3): fp32 scales per 128 x 128
+    // block of w (bs2) and per row group and 128-block of x (bs1), output type of the call
+    const float* bs1; const float* bs2;
+    int64_t bs1_rs, bs1_cs, bs2_rs, bs2_cs;
+    int bs_gsm, bs_out_dt;
 };
 
 typedef _Float16 h2 __attribute__((ext_vector_type(2)));

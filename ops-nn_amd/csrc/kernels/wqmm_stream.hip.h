@@ -411,12 +411,19 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(NW == 8
 // WF: 0 integer codes; 1 floating-point codes (e4m3) with one scale of x's type per channel; 2 e2m1 codes with e8m0
 // scales per 32 k, a row's scale bytes contiguous: a lane's 32 weights of a chunk are exactly one group, so its scale
 // is one byte per chunk, fetched with the weights like the 16-bit scales of the other forms.
+// WF 3: the fp8 block-scale matmul (quant_batch_matmul_v3, G-B / B-B) with 33 .. 64 rows (MB = 4): x is x1 widened to fp16 by a
+// pre-step, w is x2 in e4m3, widened in registers without a scale (exact products); a slab of x is exactly one
+// 128-element scale block (WK = 2 chunks of 64), each wave chains its chunk's two instructions from a zero accumulator
+// and folds the partial block sum in with one fused multiply-add by s1[m, kb] * s2[kb, n / 128] -- the products of the
+// two scales for all blocks and the slab's rows are laid down in LDS once per workgroup (its 128 columns lie in one
+// scale block of w).  The output type is the call's (bf16, fp16 or fp32).
 template <int XDT, int WBITS, int MB, int NB, int WN, int WK, bool HAS_OFF, int WF = 0>
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void wqmm_rows_kernel(WqParams p)
 {
     static_assert(WN * WK == 8, "eight waves");
     static_assert(WF == 0 || !HAS_OFF, "floating-point weight codes have no offset");
     static_assert(WF != 2 || WBITS == 4, "e8m0 group scales go with e2m1 codes");
+    static_assert(WF != 3 || (WBITS == 8 && XDT == DT_F16 && WK == 2 && NB == 2), "the block-scale form: fp16 x, e4m3 w, a slab per 128-block");
     constexpr int NT = 512;
     constexpr int KPL = 128 / WBITS, KC = 4 * KPL, STEPS = KC / 32;
     constexpr int PF = 8 / NB;           // of this wave's chunks in flight per row block (a chunk is 500 to 1000 clocks of MFMA work here)
@@ -425,7 +432,8 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void w
     constexpr int XPR = KX / 8;          // 16-byte pieces per x row per slab
     constexpr int XBUF = 16 * MB * XROW; // one slab buffer
     constexpr int XITEMS = 16 * MB * XPR / NT;
-    constexpr int NBL = NB * (HAS_OFF ? 3 : 2);   // loads of one weight fetch
+    constexpr int NBL = WF == 3 ? NB : NB * (HAS_OFF ? 3 : 2);   // loads of one weight fetch
+    constexpr int LDS_MAIN = (2 * XBUF > WN * (WK - 1) * NB * MB * 4 * 64 * 4) ? 2 * XBUF : WN * (WK - 1) * NB * MB * 4 * 64 * 4;
     static_assert((16 * MB * XPR) % NT == 0 && XPR >= 16 && PF >= 2, "staging and prefetch shape");
     extern __shared__ __attribute__((aligned(16))) char sx[];
 
@@ -479,6 +487,18 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void w
         for (int b = 0; b < MB; b++) acc[q][b] = (v4f){0.0f, 0.0f, 0.0f, 0.0f};
     const DqConst dqc = make_dq_const();
 
+    // WF 3: sct[kb][r] = s1[row r of the slab, kb] * s2[kb, this workgroup's column block], behind the x buffers (and the
+    // partial sums that take their place at the end); complete behind the loop's first barrier
+    float* sct = (float*)(sx + LDS_MAIN);
+    if constexpr (WF == 3) {
+        const int64_t nbw = ((int64_t)blockIdx.x * (16 * NB * WN)) / 128;
+        for (int i = tid; i < NSLAB * 16 * MB; i += NT) {
+            const int kb = i / (16 * MB), r = i - kb * (16 * MB);
+            const int64_t m = p.m_base + (r < rows ? r : rows - 1);
+            sct[i] = p.bs1[(m / p.bs_gsm) * p.bs1_rs + kb * p.bs1_cs] * p.bs2[kb * p.bs2_rs + nbw * p.bs2_cs];
+        }
+    }
+
     v4i wq[PF][NB];
     uint16_t sq[PF][NB], oq[PF][NB];
     auto fetch = [&](int j, int cw) {   // chunk cw of this wave (chunk cw * WK + wk of the row) into slot j
@@ -486,7 +506,8 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void w
 #pragma unroll
         for (int q = 0; q < NB; q++) {
             wq[j][q] = *(const v4i*)(wptr + q * wblk + (int64_t)cw * (WK * 64));
-            if constexpr (WF == 2) sq[j][q] = srow8[q * sblk + (cw * WK + wk) * 4];
+            if constexpr (WF == 3) sq[j][q] = 0;
+            else if constexpr (WF == 2) sq[j][q] = srow8[q * sblk + (cw * WK + wk) * 4];
             else sq[j][q] = srow[q * sblk + so];
             if constexpr (HAS_OFF) oq[j][q] = orow[q * sblk + so];
             else oq[j][q] = 0;
@@ -506,8 +527,42 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void w
             __syncthreads();   // slab cw is complete and visible; every wave has finished slab cw-1
             if (cw + 1 < NSLAB) issue_x(cw + 1);
             const char* xs = sx + (cw & 1) * XBUF;
+            if constexpr (WF == 3) {
+                // this wave's half of block cw: two instructions per fragment pair from zero, then the fold
+                v4i aw[NB][2];
 #pragma unroll
-            for (int s = 0; s < STEPS; s++) {
+                for (int q = 0; q < NB; q++) {
+                    const v4i pc = wq[j][q];
+#pragma unroll
+                    for (int s = 0; s < 2; s++) {
+                        typedef _Float16 h2v __attribute__((ext_vector_type(2)));
+                        const uint32_t d0 = (uint32_t)pc[2 * s], d1 = (uint32_t)pc[2 * s + 1];
+                        const h2v w0 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(d0, 1.0f, false), w1 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(d0, 1.0f, true);
+                        const h2v w2 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(d1, 1.0f, false), w3 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(d1, 1.0f, true);
+                        aw[q][s] = (v4i){(int)__builtin_bit_cast(uint32_t, w0), (int)__builtin_bit_cast(uint32_t, w1),
+                                         (int)__builtin_bit_cast(uint32_t, w2), (int)__builtin_bit_cast(uint32_t, w3)};
+                    }
+                }
+                const float* scr = sct + cw * (16 * MB) + nrow;
+#pragma unroll
+                for (int b = 0; b < MB; b++) {
+                    const v4i b0 = *(const v4i*)(xs + xoff[b]), b1 = *(const v4i*)(xs + (xoff[b] ^ 16));
+                    const float sc = scr[16 * b];
+                    v4f t[NB];
+#pragma unroll
+                    for (int q = 0; q < NB; q++)
+                        t[q] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(v8h, aw[q][0]), __builtin_bit_cast(v8h, b0), (v4f){0.0f, 0.0f, 0.0f, 0.0f}, 0, 0, 0);
+#pragma unroll
+                    for (int q = 0; q < NB; q++)
+                        t[q] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(v8h, aw[q][1]), __builtin_bit_cast(v8h, b1), t[q], 0, 0, 0);
+#pragma unroll
+                    for (int q = 0; q < NB; q++)
+#pragma unroll
+                        for (int i = 0; i < 4; i++) acc[q][b][i] = __builtin_fmaf(t[q][i], sc, acc[q][b][i]);
+                }
+            }
+#pragma unroll
+            for (int s = 0; s < (WF == 3 ? 0 : STEPS); s++) {
                 v4i aop[NB];
 #pragma unroll
                 for (int q = 0; q < NB; q++) {
@@ -572,6 +627,12 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void w
                 v[i] = acc[q][b][i];
                 if (p.bias) v[i] = v[i] + load_scalar_as_f32(p.bias, p.bias_dt, nn0 + i);
                 if constexpr (XDT == DT_BF16) v[i] = bf16_to_f32(bf16_bits(v[i]));   // the golden rounds bf16 results twice (a no-op)
+            }
+            if constexpr (WF == 3) {
+                const v4f vv = {v[0], v[1], v[2], v[3]};
+                if (p.bs_out_dt == DT_F32) *(v4f*)((float*)p.y + m * p.N + nn0) = vv;
+                else *(v4us*)(p.y + m * p.N + nn0) = p.bs_out_dt == DT_BF16 ? pack4_b16<DT_BF16>(vv) : pack4_b16<DT_F16>(vv);
+                continue;
             }
             const v4us o = {bits_x<XDT>(v[0]), bits_x<XDT>(v[1]), bits_x<XDT>(v[2]), bits_x<XDT>(v[3])};
             *(v4us*)(p.y + m * p.N + nn0) = o;   // N % 16 == 0 here: 8-byte aligned
@@ -1113,12 +1174,15 @@ static int launch_rows_one(const WqParams& p, hipStream_t st)
     constexpr int KC = 4 * (128 / WBITS);
     constexpr size_t lds_x = 2 * (size_t)(16 * MB) * (WK * KC * 2);
     constexpr size_t lds_red = (size_t)WN * (WK - 1) * NB * MB * 4 * 64 * 4;
-    constexpr size_t lds = lds_x > lds_red ? lds_x : lds_red;
+    constexpr size_t lds_main = lds_x > lds_red ? lds_x : lds_red;
+    constexpr size_t lds_table = WF == 3 ? 65536 : 0;   // products of the block scales: (K / 128) * 16 MB floats, at most this
+    const size_t lds = lds_main + (WF == 3 ? (size_t)(p.K / 128) * 16 * MB * 4 : 0);
+    if (lds > lds_main + lds_table) return OPSNN_NOT_TAKEN;
     const unsigned grid = (unsigned)((p.N + 16 * NB * WN - 1) / (16 * NB * WN));
     auto k = wqmm_rows_kernel<XDT, WBITS, MB, NB, WN, WK, HAS_OFF, WF>;
     static bool attr_set = false;
     if (!attr_set) {
-        hipError_t e = hipFuncSetAttribute((const void*)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        hipError_t e = hipFuncSetAttribute((const void*)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)(lds_main + lds_table));
         if (e != hipSuccess) return (int)e;
         attr_set = true;
     }
