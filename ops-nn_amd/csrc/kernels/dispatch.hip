@@ -18,6 +18,8 @@ int launch_fp8_rowcol_mfma(const OpsnnQmmArgs& a, hipStream_t st, bool merged_sc
 int launch_rowcol_exact(const OpsnnQmmArgs& a, hipStream_t st, int ep_mode);   // qmm_fp8_exact.hip
 int launch_rowcol_decode(const OpsnnQmmArgs& a, hipStream_t st);   // qmm_fp8_decode.hip
 uint64_t blockscale_rows_workspace(const OpsnnQmmArgs& a);         // qmm_fp8_rows.hip
+uint64_t rowcol_rows_workspace(const OpsnnQmmArgs& a);
+int launch_rowcol_rows(const OpsnnQmmArgs& a, hipStream_t st);
 int launch_tcg_mfma(const OpsnnQmmArgs& a, hipStream_t st);
 uint64_t tcg_workspace_bytes(const OpsnnQmmArgs& a);
 int launch_kg_mfma(const OpsnnQmmArgs& a, hipStream_t st);   // qmm_i4_kg.hip
@@ -233,8 +235,10 @@ extern "C" int opsnnQmmTc(const OpsnnQmmArgs* a, void* stream)
     // the other two forms run here.
     if (f8 && a->force_variant != OPSNN_VARIANT_PLAIN && !opsnn_force_plain()) {
         const int ep = !a->x1_scale ? 1 : (a->x1_scale_len == 1 && a->x2_scale_len == 1 && !a->bias) ? 2 : 0;
-        if (ep == 0) {   // up to 32 rows: the stream over x2 with x1 in registers
-            const int rc = launch_rowcol_decode(*a, (hipStream_t)stream);
+        if (ep == 0) {   // 17 .. 64 rows: the many-rows streaming kernel; up to 16 (32 in two passes where that does not apply): x1 in registers
+            int rc = launch_rowcol_rows(*a, (hipStream_t)stream);
+            if (rc != OPSNN_NOT_TAKEN) return rc;
+            rc = launch_rowcol_decode(*a, (hipStream_t)stream);
             if (rc != OPSNN_NOT_TAKEN) return rc;
         }
         const bool e4 = a->x1_dtype == DT_E4M3 && a->x2_dtype == DT_E4M3;
@@ -299,9 +303,12 @@ extern "C" uint64_t opsnnQmmWorkspace(const OpsnnQmmArgs* a, int mode)
     if (const int64_t Kp = k_pad_for(*a, mode)) return k_pad_bytes(*a, Kp);
     if (mode == 2) return mx_workspace_bytes(*a);
     if (mode == 1 && a->x2.row_stride == 1 && a->force_variant != OPSNN_VARIANT_PLAIN && !opsnn_force_plain()) {
-        if (const uint64_t b = blockscale_rows_workspace(*a)) return b;   // fp8 block scales with 33 .. 64 rows: x1 widened to fp16
+        if (const uint64_t b = blockscale_rows_workspace(*a)) return b;   // fp8 block scales with 17 .. 64 rows: x1 widened to fp16
     }
     // per-tensor / per-channel family: int8 operands share the int8 kernels and their re-layout; fp8 needs none
+    if (mode == 3 && a->x2.row_stride == 1 && a->force_variant != OPSNN_VARIANT_PLAIN && !opsnn_force_plain()) {
+        if (const uint64_t b = rowcol_rows_workspace(*a)) return b;   // fp8 row / column scales with 17 .. 64 rows: x1 widened to fp16
+    }
     if (mode == 3 && !(a->x1_dtype == DT_I8 && a->x2_dtype == DT_I8 && !a->x1_scale)) return 0;
     // K-group modes: the re-quantised weight of the fp8 x fp4 group-scale mode; the widened operands, row sums and fp32
     // scale / offset copies of the int4 mode with offsets

@@ -648,12 +648,12 @@ int launch_blockscale_mfma(const OpsnnQmmArgs& a0, hipStream_t st)
         }
         a.x2.row_stride = 1; a.x2.col_stride = a.K;
     }
-    if (!i8) {   // up to 32 rows: the stream over x2 with x1 in registers (exact products and sums)
-        const int rc = launch_blockscale_decode(a, st);
+    if (!i8 && a0.x2.row_stride == 1) {   // 17 .. 64 rows: x1 widened into the workspace, then the many-rows streaming kernel
+        const int rc = launch_blockscale_rows(a, st);
         if (rc != OPSNN_NOT_TAKEN) return rc;
     }
-    if (!i8 && a0.x2.row_stride == 1) {   // 33 .. 64 rows: x1 widened into the workspace, then the many-rows streaming kernel
-        const int rc = launch_blockscale_rows(a, st);
+    if (!i8) {   // up to 16 rows (32 in two passes where the kernel above does not apply): the stream over x2 with x1 in registers
+        const int rc = launch_blockscale_decode(a, st);
         if (rc != OPSNN_NOT_TAKEN) return rc;
     }
     if (!i8 && (!opsnnGetFp8Fast() || out32)) {   // exact products and sums unless the caller asked for the 8-bit matrix instruction

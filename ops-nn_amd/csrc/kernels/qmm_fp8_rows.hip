@@ -1,4 +1,4 @@
-// fp8 e4m3 block-scale matmul (G-B, B-B) with 33 .. 64 rows of x1: the many-rows streaming kernel of wqmm_stream.hip.h
+// fp8 e4m3 block-scale matmul (G-B, B-B) with 17 .. 64 rows of x1: the many-rows streaming kernel of wqmm_stream.hip.h
 // in its block-scale form (WF = 3).  A pre-step widens x1 to fp16 in the workspace (exact; M * K * 2 bytes), so that x
 // travels global -> LDS by asynchronous copies like the activations of the weight-only path; x2 is streamed once and
 // widened in registers.  Formula and arithmetic: see qmm_fp8_decode.hip (exact products, fp32 sums per half block, one
@@ -36,7 +36,7 @@ bool rows_eligible(const OpsnnQmmArgs& a)
     static const bool off = [] { const char* e = getenv("OPSNN_FP8_NO_DECODE"); return e && e[0] == '1'; }();
     if (off || a.x1_dtype != DT_E4M3 || a.x2_dtype != DT_E4M3 || a.batch != 1 || a.bias) return false;
     if (a.out_dtype != DT_BF16 && a.out_dtype != DT_F16 && a.out_dtype != DT_F32) return false;
-    if (a.M <= 32 || a.M > 64) return false;   // (the 128-row instance of the kernel does not fit the register file in this form)
+    if (a.M <= 16 || a.M > 64) return false;   // (the 128-row instance of the kernel does not fit the register file in this form)
     if (a.gsK != 128 || a.gsN != 128 || (a.gsM != 1 && a.gsM != 128)) return false;
     // the kernel's shape conditions: whole workgroups of 128 columns inside one scale block, K in slabs of 128 with the
     // weight stream four chunks deep, 16-byte pieces
@@ -69,6 +69,43 @@ int launch_blockscale_rows(const OpsnnQmmArgs& a, hipStream_t st)
     p.bs2 = (const float*)a.x2_scale_mat.ptr; p.bs2_rs = a.x2_scale_mat.row_stride; p.bs2_cs = a.x2_scale_mat.col_stride;
     p.bs_gsm = (int)a.gsM; p.bs_out_dt = a.out_dtype;
     return launch_rows_one<DT_F16, 8, 4, 2, 4, 2, false, 3>(p, st);
+}
+
+// The row / column scale form, (sum * x2Scale[n]) * x1Scale[m] + bias[n] with fp32 scales (K-C, K-T), 17 .. 64 rows.
+static bool rowcol_rows_eligible(const OpsnnQmmArgs& a)
+{
+    static const bool off = [] { const char* e = getenv("OPSNN_FP8_NO_DECODE"); return e && e[0] == '1'; }();
+    if (off || a.x1_dtype != DT_E4M3 || a.x2_dtype != DT_E4M3 || a.batch != 1) return false;
+    if (a.out_dtype != DT_BF16 && a.out_dtype != DT_F16 && a.out_dtype != DT_F32) return false;
+    if (!a.x1_scale || !a.x2_scale || a.x2_scale_dtype != DT_F32 || (a.bias && a.bias_dtype != DT_F32)) return false;
+    if (a.x1_scale_len == 1 && a.x2_scale_len == 1 && !a.bias) return false;   // that case merges and truncates the scales
+    if (a.M <= 16 || a.M > 64 || a.N % 32 != 0 || a.N < 256 || a.K % 512 != 0) return false;
+    if (a.x1.col_stride != 1 || a.x2.row_stride != 1 || a.x1.row_stride < a.K || a.x2.col_stride < a.K) return false;
+    if (((uintptr_t)a.x1.ptr | (uintptr_t)a.x2.ptr | (uint64_t)a.x1.row_stride | (uint64_t)a.x2.col_stride) % 16 || (uintptr_t)a.out % 16) return false;
+    if (a.K >= (1ll << 31) || a.N >= (1ll << 31)) return false;
+    return true;
+}
+
+uint64_t rowcol_rows_workspace(const OpsnnQmmArgs& a) { return rowcol_rows_eligible(a) ? (uint64_t)a.M * (uint64_t)a.K * 2 : 0; }
+
+int launch_rowcol_rows(const OpsnnQmmArgs& a, hipStream_t st)
+{
+    if (!rowcol_rows_eligible(a) || !a.workspace || (uintptr_t)a.workspace % 16) return OPSNN_NOT_TAKEN;
+    uint16_t* x16 = (uint16_t*)a.workspace;
+    const int64_t pieces = a.M * (a.K / 16);
+    hipLaunchKernelGGL(widen_e4m3_f16_kernel, dim3((unsigned)((pieces + 255) / 256)), dim3(256), 0, st, (const uint8_t*)a.x1.ptr, a.x1.row_stride, x16,
+                       a.M, a.K);
+    WqParams p{};
+    p.x = x16; p.w = (const uint8_t*)a.x2.ptr; p.ldw = a.x2.col_stride;
+    p.y = (uint16_t*)a.out; p.M = a.M; p.N = a.N; p.K = a.K;
+    p.group = a.K; p.group_shift = -1; p.cpg_shift = 31;
+    p.m_base = 0; p.m_rows = a.M;
+    p.w_float = 1;
+    p.bias = a.bias; p.bias_dt = a.bias_dtype;
+    p.bs1 = (const float*)a.x1_scale; p.bs1_rs = a.x1_scale_len == 1 ? 0 : 1;
+    p.bs2 = (const float*)a.x2_scale; p.bs2_cs = a.x2_scale_len == 1 ? 0 : 1;
+    p.bs_out_dt = a.out_dtype;
+    return launch_rows_one<DT_F16, 8, 4, 2, 4, 2, false, 4>(p, st);
 }
 
 }  // namespace opsnn

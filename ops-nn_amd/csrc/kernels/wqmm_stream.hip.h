@@ -411,12 +411,14 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(NW == 8
 // WF: 0 integer codes; 1 floating-point codes (e4m3) with one scale of x's type per channel; 2 e2m1 codes with e8m0
 // scales per 32 k, a row's scale bytes contiguous: a lane's 32 weights of a chunk are exactly one group, so its scale
 // is one byte per chunk, fetched with the weights like the 16-bit scales of the other forms.
-// WF 3: the fp8 block-scale matmul (quant_batch_matmul_v3, G-B / B-B) with 33 .. 64 rows (MB = 4): x is x1 widened to fp16 by a
+// WF 3: the fp8 block-scale matmul (quant_batch_matmul_v3, G-B / B-B) with 17 .. 64 rows (MB = 4): x is x1 widened to fp16 by a
 // pre-step, w is x2 in e4m3, widened in registers without a scale (exact products); a slab of x is exactly one
 // 128-element scale block (WK = 2 chunks of 64), each wave chains its chunk's two instructions from a zero accumulator
 // and folds the partial block sum in with one fused multiply-add by s1[m, kb] * s2[kb, n / 128] -- the products of the
 // two scales for all blocks and the slab's rows are laid down in LDS once per workgroup (its 128 columns lie in one
 // scale block of w).  The output type is the call's (bf16, fp16 or fp32).
+// WF 4: the fp8 row / column scale form (K-C, K-T) of the same operands: one chain over all of K, and the epilogue
+// computes (sum * x2Scale[n]) * x1Scale[m] + bias[n] (bs2 / bs1 with element strides bs2_cs / bs1_rs of 0 or 1).
 template <int XDT, int WBITS, int MB, int NB, int WN, int WK, bool HAS_OFF, int WF = 0>
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void wqmm_rows_kernel(WqParams p)
 {
@@ -424,6 +426,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void w
     static_assert(WF == 0 || !HAS_OFF, "floating-point weight codes have no offset");
     static_assert(WF != 2 || WBITS == 4, "e8m0 group scales go with e2m1 codes");
     static_assert(WF != 3 || (WBITS == 8 && XDT == DT_F16 && WK == 2 && NB == 2), "the block-scale form: fp16 x, e4m3 w, a slab per 128-block");
+    static_assert(WF != 4 || (WBITS == 8 && XDT == DT_F16 && !HAS_OFF), "the row / column scale form: fp16 x, e4m3 w");
     constexpr int NT = 512;
     constexpr int KPL = 128 / WBITS, KC = 4 * KPL, STEPS = KC / 32;
     constexpr int PF = 8 / NB;           // of this wave's chunks in flight per row block (a chunk is 500 to 1000 clocks of MFMA work here)
@@ -432,7 +435,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void w
     constexpr int XPR = KX / 8;          // 16-byte pieces per x row per slab
     constexpr int XBUF = 16 * MB * XROW; // one slab buffer
     constexpr int XITEMS = 16 * MB * XPR / NT;
-    constexpr int NBL = WF == 3 ? NB : NB * (HAS_OFF ? 3 : 2);   // loads of one weight fetch
+    constexpr int NBL = WF >= 3 ? NB : NB * (HAS_OFF ? 3 : 2);   // loads of one weight fetch
     constexpr int LDS_MAIN = (2 * XBUF > WN * (WK - 1) * NB * MB * 4 * 64 * 4) ? 2 * XBUF : WN * (WK - 1) * NB * MB * 4 * 64 * 4;
     static_assert((16 * MB * XPR) % NT == 0 && XPR >= 16 && PF >= 2, "staging and prefetch shape");
     extern __shared__ __attribute__((aligned(16))) char sx[];
@@ -506,7 +509,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void w
 #pragma unroll
         for (int q = 0; q < NB; q++) {
             wq[j][q] = *(const v4i*)(wptr + q * wblk + (int64_t)cw * (WK * 64));
-            if constexpr (WF == 3) sq[j][q] = 0;
+            if constexpr (WF >= 3) sq[j][q] = 0;
             else if constexpr (WF == 2) sq[j][q] = srow8[q * sblk + (cw * WK + wk) * 4];
             else sq[j][q] = srow[q * sblk + so];
             if constexpr (HAS_OFF) oq[j][q] = orow[q * sblk + so];
@@ -568,6 +571,14 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void w
                 for (int q = 0; q < NB; q++) {
                     if constexpr (WF == 0) aop[q] = dequant8<XDT, WBITS, HAS_OFF, true>(wq[j][q], s, sq[j][q], oq[j][q], dqc);
                     else if constexpr (WF == 1) aop[q] = dequant8_float<XDT, WBITS, true>(wq[j][q], s, sq[j][q]);
+                    else if constexpr (WF == 4) {
+                        typedef _Float16 h2v __attribute__((ext_vector_type(2)));
+                        const uint32_t d0 = (uint32_t)wq[j][q][2 * s], d1 = (uint32_t)wq[j][q][2 * s + 1];
+                        const h2v w0 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(d0, 1.0f, false), w1 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(d0, 1.0f, true);
+                        const h2v w2 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(d1, 1.0f, false), w3 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(d1, 1.0f, true);
+                        aop[q] = (v4i){(int)__builtin_bit_cast(uint32_t, w0), (int)__builtin_bit_cast(uint32_t, w1),
+                                       (int)__builtin_bit_cast(uint32_t, w2), (int)__builtin_bit_cast(uint32_t, w3)};
+                    }
                     else aop[q] = dequant8_float<XDT, WBITS, true>(wq[j][q], s, bits_x<XDT>(e8m0_to_f32(sq[j][q])));
                 }
 #pragma unroll
@@ -625,10 +636,11 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void w
 #pragma unroll
             for (int i = 0; i < 4; i++) {
                 v[i] = acc[q][b][i];
+                if constexpr (WF == 4) v[i] = (v[i] * p.bs2[(nn0 + i) * p.bs2_cs]) * p.bs1[m * p.bs1_rs];
                 if (p.bias) v[i] = v[i] + load_scalar_as_f32(p.bias, p.bias_dt, nn0 + i);
                 if constexpr (XDT == DT_BF16) v[i] = bf16_to_f32(bf16_bits(v[i]));   // the golden rounds bf16 results twice (a no-op)
             }
-            if constexpr (WF == 3) {
+            if constexpr (WF >= 3) {
                 const v4f vv = {v[0], v[1], v[2], v[3]};
                 if (p.bs_out_dt == DT_F32) *(v4f*)((float*)p.y + m * p.N + nn0) = vv;
                 else *(v4us*)(p.y + m * p.N + nn0) = p.bs_out_dt == DT_BF16 ? pack4_b16<DT_BF16>(vv) : pack4_b16<DT_F16>(vv);

@@ -238,6 +238,10 @@ def test_gpu_matches_oracle(gpu, M, K, N, in_dt, s_dt, s_len, bias_dt, out_dt, t
     (16, 7168, 1000, "N", False, "f16", "M"),
     (20, 2048, 264, "N", True, "bf16", "M"),
     (32, 1024, 256, 1, True, "f16", True),
+    # 33 .. 64 rows (N % 32 == 0, K % 512 == 0): x1 widened into the workspace, the many-rows streaming kernel
+    (40, 2048, 512, "N", True, "bf16", "M"),
+    (64, 7168, 288, "N", False, "f16", "M"),
+    (33, 512, 256, 1, True, "f16", True),
 ])
 def test_gpu_fp8_row_and_column_scales_on_the_matrix_cores(gpu, M, K, N, s_len, bias, out_dt, pt, fast):
     """fp8 e4m3 K-C / K-T / T-C-double-scale on the matrix cores (K-contiguous x2, K % 128 == 0, 16-bit output).  Default:
