@@ -31,6 +31,8 @@ PROFILED_TRAFFIC = {
     (4, None, "fast"): (1502.4e6, "profiles/qmm_fp8_block_m4096_k7168_n18432.txt"),
     (5, None, None): (3083.5e6, "profiles/qgemm_mxfp4_b8_m4096_k8192_n8192.txt"),
     (10, None, None): (290.3e6, "profiles/qmm_i4_kg_m4096_k4096_n4096.txt"),
+    (12, 16, "exact"): (136.9e6, "profiles/qmm_fp8_block_decode_m16_k7168_n18432.txt"),
+    (12, 64, "exact"): (143.5e6, "profiles/qmm_fp8_block_rows_m64_k7168_n18432.txt"),
     (11, 16, "warm"): (133.6e6, "profiles/wqmm_decode_mxfp4_m16_k8192_n28672.txt"),
 }
 
@@ -192,6 +194,20 @@ class Config4(Workload):
         t = time.perf_counter() - t0
         return {"value": 2.0 * rows * self.K * self.N / t / 1e12, "unit": "TFLOP/s", "cores": _cores(), "kind": "port",
                 "sample": f"first {rows} of {self.M} rows of x1 against the full x2 (oracle/liboracle.so, OpenMP), {t:.2f} s"}
+
+
+class Config4Rows(Config4):
+    """Not a BASELINE config: config 4's operator, K and N with the few rows of x1 of a decode step (--m, default 16).  The
+    call is a stream over x2: reported against the HBM roofline (bytes of both operands, scales and the output per step)."""
+    metric = "quant_gemm_stream_bandwidth"
+    bound = "hbm"
+
+    def __init__(self, m, args):
+        M = args.m or 16
+        super().__init__(m, args, M=M)
+        self.instr_peak_key = None
+        self.kernel = "fp8_block_decode_kernel" if M <= 16 else "wqmm_rows_kernel<f16, e4m3, block scales> (+ widen_e4m3_f16_kernel)" if M <= 64 else self.kernel
+        self.config = dict(self.config, workload="aclnnQuantMatmulV5 fp8 e4m3 G-B (1x128 / 128x128 scales), bf16 out, decode rows")
 
 
 class Config5(Workload):
@@ -471,6 +487,8 @@ def make_workload(m, config, args):
         return Config2(m, args)
     if config == 4:
         return Config4(m, args)
+    if config == 12:
+        return Config4Rows(m, args)
     if config == 5:
         return Config5(m, args)
     raise SystemExit(f"bench.py: config {config} is not wired up yet")
