@@ -243,6 +243,9 @@ int launch_mx_mfma(const OpsnnQmmArgs& a0, hipStream_t st)
         if (small || a.force_variant == OPSNN_VARIANT_MX_128) return qgemm_launch<MODE_MXFP8, 128, 128, 128, 2, 2, 2, 1>(g, a.batch, a.out_dtype, st);
         return qgemm_launch<MODE_MXFP8, 256, 256, 128, 2, 2, 2, 1>(g, a.batch, a.out_dtype, st);
     }
+    // few rows: the 128 x 128 tiles of the tile kernel (the block kernel's 128 x 256 tiles leave most CUs' matrix work on
+    // rows that do not exist and half as many workgroups to stream x2)
+    if (a.M <= 256) return qgemm_launch<MODE_MXFP8, 128, 128, 128, 2, 2, 2, 1>(g, a.batch, a.out_dtype, st);
     return launch_mxfp8_mfma(a, st);
 }
 
