@@ -235,7 +235,7 @@ extern "C" int opsnnQmmTc(const OpsnnQmmArgs* a, void* stream)
     // the other two forms run here.
     if (f8 && a->force_variant != OPSNN_VARIANT_PLAIN && !opsnn_force_plain()) {
         const int ep = !a->x1_scale ? 1 : (a->x1_scale_len == 1 && a->x2_scale_len == 1 && !a->bias) ? 2 : 0;
-        if (ep == 0) {   // 17 .. 64 rows: the many-rows streaming kernel; up to 16 (32 in two passes where that does not apply): x1 in registers
+        if (ep == 0) {   // 17 .. 128 rows: the many-rows streaming kernel; up to 16 (32 in two passes where that does not apply): x1 in registers
             int rc = launch_rowcol_rows(*a, (hipStream_t)stream);
             if (rc != OPSNN_NOT_TAKEN) return rc;
             rc = launch_rowcol_decode(*a, (hipStream_t)stream);
@@ -303,11 +303,11 @@ extern "C" uint64_t opsnnQmmWorkspace(const OpsnnQmmArgs* a, int mode)
     if (const int64_t Kp = k_pad_for(*a, mode)) return k_pad_bytes(*a, Kp);
     if (mode == 2) return mx_workspace_bytes(*a);
     if (mode == 1 && a->x2.row_stride == 1 && a->force_variant != OPSNN_VARIANT_PLAIN && !opsnn_force_plain()) {
-        if (const uint64_t b = blockscale_rows_workspace(*a)) return b;   // fp8 block scales with 17 .. 64 rows: x1 widened to fp16
+        if (const uint64_t b = blockscale_rows_workspace(*a)) return b;   // fp8 block scales with 17 .. 128 rows: x1 widened to fp16
     }
     // per-tensor / per-channel family: int8 operands share the int8 kernels and their re-layout; fp8 needs none
     if (mode == 3 && a->x2.row_stride == 1 && a->force_variant != OPSNN_VARIANT_PLAIN && !opsnn_force_plain()) {
-        if (const uint64_t b = rowcol_rows_workspace(*a)) return b;   // fp8 row / column scales with 17 .. 64 rows: x1 widened to fp16
+        if (const uint64_t b = rowcol_rows_workspace(*a)) return b;   // fp8 row / column scales with 17 .. 128 rows: x1 widened to fp16
     }
     if (mode == 3 && !(a->x1_dtype == DT_I8 && a->x2_dtype == DT_I8 && !a->x1_scale)) return 0;
     // K-group modes: the re-quantised weight of the fp8 x fp4 group-scale mode; the widened operands, row sums and fp32

@@ -648,7 +648,7 @@ int launch_blockscale_mfma(const OpsnnQmmArgs& a0, hipStream_t st)
         }
         a.x2.row_stride = 1; a.x2.col_stride = a.K;
     }
-    if (!i8 && a0.x2.row_stride == 1) {   // 17 .. 64 rows: x1 widened into the workspace, then the many-rows streaming kernel
+    if (!i8 && a0.x2.row_stride == 1) {   // 17 .. 128 rows: x1 widened into the workspace, then the many-rows streaming kernel
         const int rc = launch_blockscale_rows(a, st);
         if (rc != OPSNN_NOT_TAKEN) return rc;
     }

@@ -1,4 +1,4 @@
-// fp8 e4m3 block-scale matmul (G-B, B-B) with 17 .. 64 rows of x1: the many-rows streaming kernel of wqmm_stream.hip.h
+// fp8 e4m3 block-scale matmul (G-B, B-B) with 17 .. 128 rows of x1: the many-rows streaming kernel of wqmm_stream.hip.h
 // in its block-scale form (WF = 3).  A pre-step widens x1 to fp16 in the workspace (exact; M * K * 2 bytes), so that x
 // travels global -> LDS by asynchronous copies like the activations of the weight-only path; x2 is streamed once and
 // widened in registers.  Formula and arithmetic: see qmm_fp8_decode.hip (exact products, fp32 sums per half block, one
@@ -36,11 +36,11 @@ bool rows_eligible(const OpsnnQmmArgs& a)
     static const bool off = [] { const char* e = getenv("OPSNN_FP8_NO_DECODE"); return e && e[0] == '1'; }();
     if (off || a.x1_dtype != DT_E4M3 || a.x2_dtype != DT_E4M3 || a.batch != 1 || a.bias) return false;
     if (a.out_dtype != DT_BF16 && a.out_dtype != DT_F16 && a.out_dtype != DT_F32) return false;
-    if (a.M <= 16 || a.M > 64) return false;   // (the 128-row instance of the kernel does not fit the register file in this form)
+    if (a.M <= 16 || a.M > 128) return false;
     if (a.gsK != 128 || a.gsN != 128 || (a.gsM != 1 && a.gsM != 128)) return false;
     // the kernel's shape conditions: whole workgroups of 128 columns inside one scale block, K in slabs of 128 with the
     // weight stream four chunks deep, 16-byte pieces
-    if (a.N % 128 != 0 || a.N < 256 || a.K % 512 != 0 || a.K / 128 * 16 * 4 * 4 > 65536) return false;
+    if (a.N % 128 != 0 || a.N < 256 || a.K % 512 != 0 || a.K / 128 * 16 * (a.M > 64 ? 8 : 4) * 4 > 65536) return false;
     if (a.x1.col_stride != 1 || a.x2.row_stride != 1 || a.x1.row_stride < a.K || a.x2.col_stride < a.K) return false;
     if (((uintptr_t)a.x1.ptr | (uintptr_t)a.x2.ptr | (uint64_t)a.x1.row_stride | (uint64_t)a.x2.col_stride) % 16) return false;
     if (((uintptr_t)a.x1_scale_mat.ptr | (uintptr_t)a.x2_scale_mat.ptr) % 4 || (uintptr_t)a.out % 16) return false;
@@ -68,10 +68,10 @@ int launch_blockscale_rows(const OpsnnQmmArgs& a, hipStream_t st)
     p.bs1 = (const float*)a.x1_scale_mat.ptr; p.bs1_rs = a.x1_scale_mat.row_stride; p.bs1_cs = a.x1_scale_mat.col_stride;
     p.bs2 = (const float*)a.x2_scale_mat.ptr; p.bs2_rs = a.x2_scale_mat.row_stride; p.bs2_cs = a.x2_scale_mat.col_stride;
     p.bs_gsm = (int)a.gsM; p.bs_out_dt = a.out_dtype;
-    return launch_rows_one<DT_F16, 8, 4, 2, 4, 2, false, 3>(p, st);
+    return a.M > 64 ? launch_rows_one<DT_F16, 8, 8, 2, 4, 2, false, 3>(p, st) : launch_rows_one<DT_F16, 8, 4, 2, 4, 2, false, 3>(p, st);
 }
 
-// The row / column scale form, (sum * x2Scale[n]) * x1Scale[m] + bias[n] with fp32 scales (K-C, K-T), 17 .. 64 rows.
+// The row / column scale form, (sum * x2Scale[n]) * x1Scale[m] + bias[n] with fp32 scales (K-C, K-T), 17 .. 128 rows.
 static bool rowcol_rows_eligible(const OpsnnQmmArgs& a)
 {
     static const bool off = [] { const char* e = getenv("OPSNN_FP8_NO_DECODE"); return e && e[0] == '1'; }();
@@ -79,7 +79,7 @@ static bool rowcol_rows_eligible(const OpsnnQmmArgs& a)
     if (a.out_dtype != DT_BF16 && a.out_dtype != DT_F16 && a.out_dtype != DT_F32) return false;
     if (!a.x1_scale || !a.x2_scale || a.x2_scale_dtype != DT_F32 || (a.bias && a.bias_dtype != DT_F32)) return false;
     if (a.x1_scale_len == 1 && a.x2_scale_len == 1 && !a.bias) return false;   // that case merges and truncates the scales
-    if (a.M <= 16 || a.M > 64 || a.N % 32 != 0 || a.N < 256 || a.K % 512 != 0) return false;
+    if (a.M <= 16 || a.M > 128 || a.N % 32 != 0 || a.N < 256 || a.K % 512 != 0) return false;
     if (a.x1.col_stride != 1 || a.x2.row_stride != 1 || a.x1.row_stride < a.K || a.x2.col_stride < a.K) return false;
     if (((uintptr_t)a.x1.ptr | (uintptr_t)a.x2.ptr | (uint64_t)a.x1.row_stride | (uint64_t)a.x2.col_stride) % 16 || (uintptr_t)a.out % 16) return false;
     if (a.K >= (1ll << 31) || a.N >= (1ll << 31)) return false;
@@ -105,7 +105,7 @@ int launch_rowcol_rows(const OpsnnQmmArgs& a, hipStream_t st)
     p.bs1 = (const float*)a.x1_scale; p.bs1_rs = a.x1_scale_len == 1 ? 0 : 1;
     p.bs2 = (const float*)a.x2_scale; p.bs2_cs = a.x2_scale_len == 1 ? 0 : 1;
     p.bs_out_dt = a.out_dtype;
-    return launch_rows_one<DT_F16, 8, 4, 2, 4, 2, false, 4>(p, st);
+    return a.M > 64 ? launch_rows_one<DT_F16, 8, 8, 2, 4, 2, false, 4>(p, st) : launch_rows_one<DT_F16, 8, 4, 2, 4, 2, false, 4>(p, st);
 }
 
 }  // namespace opsnn

@@ -411,7 +411,7 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(NW == 8
 // WF: 0 integer codes; 1 floating-point codes (e4m3) with one scale of x's type per channel; 2 e2m1 codes with e8m0
 // scales per 32 k, a row's scale bytes contiguous: a lane's 32 weights of a chunk are exactly one group, so its scale
 // is one byte per chunk, fetched with the weights like the 16-bit scales of the other forms.
-// WF 3: the fp8 block-scale matmul (quant_batch_matmul_v3, G-B / B-B) with 17 .. 64 rows (MB = 4): x is x1 widened to fp16 by a
+// WF 3: the fp8 block-scale matmul (quant_batch_matmul_v3, G-B / B-B) with 17 .. 128 rows (MB = 4 up to 64 rows, else 8): x is x1 widened to fp16 by a
 // pre-step, w is x2 in e4m3, widened in registers without a scale (exact products); a slab of x is exactly one
 // 128-element scale block (WK = 2 chunks of 64), each wave chains its chunk's two instructions from a zero accumulator
 // and folds the partial block sum in with one fused multiply-add by s1[m, kb] * s2[kb, n / 128] -- the products of the
@@ -547,6 +547,50 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void w
                     }
                 }
                 const float* scr = sct + cw * (16 * MB) + nrow;
+                if constexpr (MB > 4) {
+                    // 128 rows: two row blocks at a time, and the fold of a pair rides behind the next pair's matrix
+                    // instructions.  The empty asm statements pin each fold where it is written: left alone the compiler
+                    // postpones the folds, keeps all eight blocks' partial sums alive and spills the weight prefetch.
+                    v4f tp[2][NB];
+                    float scp[2] = {0.0f, 0.0f};
+#pragma unroll
+                    for (int bp = 0; bp <= MB / 2; bp++) {
+                        v4f tc[2][NB];
+                        float scc[2] = {0.0f, 0.0f};
+                        if (bp < MB / 2) {
+#pragma unroll
+                            for (int h = 0; h < 2; h++) {
+                                const int b = 2 * bp + h;
+                                const v4i b0 = *(const v4i*)(xs + xoff[b]), b1 = *(const v4i*)(xs + (xoff[b] ^ 16));
+                                scc[h] = scr[16 * b];
+#pragma unroll
+                                for (int q = 0; q < NB; q++)
+                                    tc[h][q] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(v8h, aw[q][0]), __builtin_bit_cast(v8h, b0), (v4f){0.0f, 0.0f, 0.0f, 0.0f}, 0, 0, 0);
+#pragma unroll
+                                for (int q = 0; q < NB; q++)
+                                    tc[h][q] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(v8h, aw[q][1]), __builtin_bit_cast(v8h, b1), tc[h][q], 0, 0, 0);
+                            }
+                        }
+                        if (bp > 0) {
+#pragma unroll
+                            for (int h = 0; h < 2; h++)
+#pragma unroll
+                                for (int q = 0; q < NB; q++) {
+                                    v4f& a = acc[q][2 * (bp - 1) + h];
+#pragma unroll
+                                    for (int i = 0; i < 4; i++) a[i] = __builtin_fmaf(tp[h][q][i], scp[h], a[i]);
+                                    asm volatile("" : "+v"(a));
+                                }
+                        }
+#pragma unroll
+                        for (int h = 0; h < 2; h++) {
+                            scp[h] = scc[h];
+#pragma unroll
+                            for (int q = 0; q < NB; q++) tp[h][q] = tc[h][q];
+                        }
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
+                } else {
 #pragma unroll
                 for (int b = 0; b < MB; b++) {
                     const v4i b0 = *(const v4i*)(xs + xoff[b]), b1 = *(const v4i*)(xs + (xoff[b] ^ 16));
@@ -562,6 +606,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void w
                     for (int q = 0; q < NB; q++)
 #pragma unroll
                         for (int i = 0; i < 4; i++) acc[q][b][i] = __builtin_fmaf(t[q][i], sc, acc[q][b][i]);
+                }
                 }
             }
 #pragma unroll

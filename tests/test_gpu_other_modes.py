@@ -119,6 +119,8 @@ def test_fp8_blockscale_fp32_output(gpu, M, K, N, tB, gsM, fast):
     # 17 .. 64 rows (N % 128 == 0, K % 512 == 0): x1 widened into the workspace, the many-rows streaming kernel
     (33, 2048, 512, 1, "bf16"), (64, 8192, 1024, 1, "f16"), (50, 7168, 256, 128, "bf16"), (64, 512, 384, 1, "f32"),
     (40, 1536, 2304, 1, "bf16"),
+    # 65 .. 128 rows: the same kernel's 128-row instance
+    (65, 2048, 512, 1, "bf16"), (128, 7168, 1024, 1, "f16"), (100, 1024, 256, 128, "f32"), (96, 16384, 256, 1, "bf16"),
 ])
 def test_fp8_blockscale_decode_rows(gpu, M, K, N, gsM, out):
     """The block-scale modes with up to 32 rows of x1 (x2 K-contiguous): x1 stays in registers as exact fp16 and x2 is

@@ -242,6 +242,10 @@ def test_gpu_matches_oracle(gpu, M, K, N, in_dt, s_dt, s_len, bias_dt, out_dt, t
     (40, 2048, 512, "N", True, "bf16", "M"),
     (64, 7168, 288, "N", False, "f16", "M"),
     (33, 512, 256, 1, True, "f16", True),
+    # 65 .. 128 rows: the same kernel's 128-row instance
+    (65, 1024, 288, "N", True, "bf16", "M"),
+    (128, 3584, 512, "N", False, "f16", "M"),
+    (100, 512, 256, 1, True, "bf16", True),
 ])
 def test_gpu_fp8_row_and_column_scales_on_the_matrix_cores(gpu, M, K, N, s_len, bias, out_dt, pt, fast):
     """fp8 e4m3 K-C / K-T / T-C-double-scale on the matrix cores (K-contiguous x2, K % 128 == 0, 16-bit output).  Default:
