@@ -287,7 +287,17 @@ __global__ void qmm_i4_asym_plain(OpsnnQmmArgs a)
 }
 int launch_fp8_rowcol_mfma(const OpsnnQmmArgs& a, hipStream_t st, bool merged_scales_ok);   // qmm_fp8_block.hip
 
+int launch_rowcol_rows(const OpsnnQmmArgs& a, hipStream_t st);      // qmm_fp8_rows.hip
+int launch_rowcol_decode(const OpsnnQmmArgs& a, hipStream_t st);    // qmm_fp8_decode.hip
+void* weight_cache_blob3(const void* src, const void* src2, const void* src3, int64_t K, int64_t N, int bits, int64_t nb, uint64_t bytes, hipStream_t st,
+                         bool* fresh);   // weight_cache.hip
+void weight_cache_commit(void* buffer, hipStream_t st);
+
 static inline uint64_t align256(uint64_t v) { return (v + 255) / 256 * 256; }
+// The re-quantised weight with its side values: e4m3 bytes [N, K], the decoded output scale per column, a 1.0.
+static inline uint64_t tcg_blob_bytes(const OpsnnQmmArgs& a) { return align256((uint64_t)a.N * a.K) + align256((uint64_t)a.N * 4) + 256; }
+// 17 .. 128 rows go to the many-rows streaming kernel, which wants x1 widened to fp16 (M * K * 2 bytes behind the blob)
+static inline uint64_t tcg_rows_bytes(const OpsnnQmmArgs& a) { return a.M > 16 && a.M <= 128 ? (uint64_t)a.M * a.K * 2 : 0; }
 // Workspace of the matrix-core path of the fp8 x fp4 group-scale mode (0: the shape stays on the plain kernel).
 uint64_t tcg_workspace_bytes(const OpsnnQmmArgs& a)
 {
@@ -296,22 +306,45 @@ uint64_t tcg_workspace_bytes(const OpsnnQmmArgs& a)
     if (a.x1.col_stride != 1 || a.x2.row_stride != 1 || a.x2.col_stride != a.K) return 0;
     if (a.out_dtype != DT_BF16 && a.out_dtype != DT_F16) return 0;
     if (a.bias && a.bias_dtype != DT_F32) return 0;
-    return align256((uint64_t)a.N * a.K) + align256((uint64_t)a.N * 4) + 256;
+    return tcg_blob_bytes(a) + tcg_rows_bytes(a);
 }
-// Re-quantise x2 into the workspace, then the fp8 kernel with a column scale (the decoded output scale) and a unit row scale.
+// Re-quantise x2 into the workspace -- or, with the weight cache on and dense scales, once into a cached buffer that
+// later calls with the same x2, scales and output scale find again -- then an fp8 kernel with a column scale (the
+// decoded output scale) and a unit row scale: the streaming kernels with up to 128 rows of x1, else the tile kernel.
 int launch_tcg_mfma(const OpsnnQmmArgs& a, hipStream_t st)
 {
     const uint64_t need = tcg_workspace_bytes(a);
     if (!need || !a.workspace || (uintptr_t)a.workspace % 16 != 0) return OPSNN_NOT_TAKEN;
+    const uint64_t blob = tcg_blob_bytes(a);
     uint8_t* w8 = (uint8_t*)a.workspace;
+    // what the cache key has to tell apart beside the three pointers, K, N and the size: group size, scale type, which
+    // way the dense scale matrix lies, one output scale or N
+    const int64_t kg = a.K / a.gsK;
+    const bool s_nk = a.x2_scale_mat.row_stride == 1 && a.x2_scale_mat.col_stride == kg;
+    const bool s_kn = a.x2_scale_mat.row_stride == a.N && a.x2_scale_mat.col_stride == 1;
+    const bool dense = (s_nk || s_kn) && a.K % a.gsK == 0;
+    const int64_t key = (a.gsK << 8) | ((int64_t)(a.x2_scale_dtype & 31) << 3) | (s_nk ? 4 : 0) | (a.y_scale_len == 1 ? 2 : 0) | 1;
+    bool fresh = false;
+    void* cached = dense ? weight_cache_blob3(a.x2.ptr, a.x2_scale_mat.ptr, a.y_scale, a.K, a.N, 4, key, blob, st, &fresh) : nullptr;
+    if (cached) w8 = (uint8_t*)cached;
     float* cs = (float*)(w8 + align256((uint64_t)a.N * a.K));
     float* one = (float*)((char*)cs + align256((uint64_t)a.N * 4));
-    const int64_t threads = a.N * (a.K / 32);   // >= N since K >= 128
-    hipLaunchKernelGGL(tcg_requant_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, st, a, w8, cs, one);
+    if (!cached || fresh) {
+        const int64_t threads = a.N * (a.K / 32);   // >= N since K >= 128
+        hipLaunchKernelGGL(tcg_requant_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, st, a, w8, cs, one);
+        if (cached) weight_cache_commit(cached, st);
+    }
     OpsnnQmmArgs b = a;
     b.x2.ptr = w8; b.x2_dtype = DT_E4M3; b.x2.row_stride = 1; b.x2.col_stride = a.K; b.x2.batch_stride = 0;
     b.x1_scale = one; b.x1_scale_len = 1;
     b.x2_scale = cs; b.x2_scale_dtype = DT_F32; b.x2_scale_len = a.N;
+    b.workspace = tcg_rows_bytes(a) ? (char*)a.workspace + blob : nullptr;
+    if (a.force_variant == 0) {
+        int rc = launch_rowcol_rows(b, st);
+        if (rc != OPSNN_NOT_TAKEN) return rc;
+        rc = launch_rowcol_decode(b, st);
+        if (rc != OPSNN_NOT_TAKEN) return rc;
+    }
     return launch_fp8_rowcol_mfma(b, st, true);
 }
 int launch_group_plain(const OpsnnQmmArgs& a, bool tcg, hipStream_t st)

@@ -147,3 +147,43 @@ def test_int4_group_mode_x2_blocks_are_written_once(cache):
     third = call()
     assert np.array_equal(third, cases.oracle_i4_asym(m, inp2, M, K, N, m.ACL_BF16))
     assert _stats(m)[2] - h0 == 2
+
+
+def test_fp8_fp4_group_mode_requantised_weight_is_written_once(cache):
+    """fp8 x fp4 with 16-bit group scales: the re-quantised e4m3 weight with the decoded output scales is kept, keyed
+    by x2, its scales and the output scale; a second call with other activations is still right (few rows: the
+    streaming kernel reads the kept bytes)."""
+    m = cache
+    M, K, N = 40, 2048, 512
+    print(f"case weight cache, fp8 x fp4 T-CG {M}x{K}x{N}", flush=True)
+    inp = cases.make_tcg_inputs(m, M, K, N, 5, m.ACL_BF16)
+    want = cases.oracle_tcg(m, inp, M, K, N, m.ACL_BF16)
+    d = {k: m.DeviceBuffer(host=v) for k, v in inp.items() if isinstance(v, np.ndarray)}
+    d_out = m.DeviceBuffer(M * N * 2)
+    t = dict(x1=m.Tensor((M, K), m.ACL_FLOAT8_E4M3FN, d["x1"]), x2=m.Tensor((N, K), m.ACL_FLOAT4_E2M1, d["x2"]),
+             s2=m.Tensor((N, K // 32), m.ACL_BF16, d["s2"]), ys=m.Tensor((1, N), m.ACL_UINT64, d["ys"]),
+             out=m.Tensor((M, N), m.ACL_BF16, d_out))
+
+    def call():
+        ws = m.quant_matmul_v5(t["x1"], t["x2"], None, t["s2"], t["out"], y_scale=t["ys"], transpose_x2=True, group_size=32)
+        m.check(m.lib().aclrtSynchronizeDevice(), "sync")
+        del ws
+        return d_out.to_host(np.uint16, (M, N))
+
+    def close(got, want):
+        g, w = orc.b16_to_f32(got, orc.BF16), orc.b16_to_f32(want, orc.BF16)
+        mx, mean = orc.rel_err_stats(g, w)
+        return mx <= 2.0 ** -7 and mean <= 2.0 ** -10 and orc.isclose_fraction(g, w) <= 1e-3
+
+    e0, _, h0, m0 = _stats(m)
+    first = call()
+    second = call()
+    e1, _, h1, m1 = _stats(m)
+    assert (e1 - e0, m1 - m0, h1 - h0) == (1, 1, 1)
+    assert close(first, want) and np.array_equal(first, second)
+    inp2 = cases.make_tcg_inputs(m, M, K, N, 6, m.ACL_BF16)
+    d["x1"].upload(inp2["x1"])
+    inp2.update(x2=inp["x2"], s2=inp["s2"], ys=inp["ys"])
+    third = call()
+    assert close(third, cases.oracle_tcg(m, inp2, M, K, N, m.ACL_BF16))
+    assert _stats(m)[2] - h0 == 2

@@ -180,7 +180,12 @@ def test_gpu_tcg(gpu, M, K, N, s_dt, out_dt, ys_i64):
 @pytest.mark.gpu
 @pytest.mark.parametrize("fast", [False, True])
 @pytest.mark.parametrize("M,K,N,s_dt,out_dt", [(64, 128, 64, "bf16", "bf16"), (300, 384, 260, "f16", "f16"),
-                                               (512, 2048, 520, "bf16", "bf16"), (1024, 1024, 2048, "bf16", "f16")])
+                                               (512, 2048, 520, "bf16", "bf16"), (1024, 1024, 2048, "bf16", "f16"),
+                                               # few rows: the streaming kernels behind the same prologue (x1 in registers up
+                                               # to 16 rows, two passes up to 32, the many-rows kernel from 17 to 128)
+                                               (16, 4096, 512, "bf16", "bf16"), (9, 2048, 264, "f16", "f16"),
+                                               (24, 1024, 520, "bf16", "f16"), (40, 2048, 512, "bf16", "bf16"),
+                                               (100, 1024, 256, "f16", "bf16")])
 def test_gpu_tcg_on_the_matrix_cores(gpu, M, K, N, s_dt, out_dt, fast):
     """fp8 x fp4 with 16-bit group scales, K % 128 == 0 and enough outputs: a prologue writes the re-quantised e4m3 weight
     (the oracle's bytes) into the workspace and the fp8 matrix-core kernel does the product with the decoded output scale
