@@ -652,7 +652,7 @@ int launch_blockscale_mfma(const OpsnnQmmArgs& a0, hipStream_t st)
         const int rc = launch_blockscale_rows(a, st);
         if (rc != OPSNN_NOT_TAKEN) return rc;
     }
-    if (!i8) {   // up to 16 rows (32 in two passes where the kernel above does not apply): the stream over x2 with x1 in registers
+    {   // up to 16 rows (32 in two passes where the kernel above does not apply): the stream over x2 with x1 in registers
         const int rc = launch_blockscale_decode(a, st);
         if (rc != OPSNN_NOT_TAKEN) return rc;
     }

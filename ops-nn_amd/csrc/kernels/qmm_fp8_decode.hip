@@ -52,9 +52,13 @@ __device__ __forceinline__ v4i widen8_e4m3(uint32_t d0, uint32_t d1)
                  (int)__builtin_bit_cast(uint32_t, w3)};
 }
 
-template <int NW, int NBLK, bool RC>
+// I8: int8 operands with the same block scales and an fp32 bias (the per-tile mode of quant_batch_matmul_v4,
+// qbmmv4_kernel_golden.py:258-325): a lane's 16-byte piece is one operand of v_mfma_i32_16x16x64_i8 as it is, a block's
+// sum is two of them from a zero accumulator (an exact integer below 2^21), converted to fp32 for the fold.
+template <int NW, int NBLK, bool RC, bool I8 = false>
 __global__ __launch_bounds__(NW * 64) void fp8_block_decode_kernel(Fp8DecParams p)
 {
+    static_assert(!(RC && I8), "int8: the block-scale form only");
     constexpr int NCH = 2 * NBLK;                    // 64-byte chunks of an x2 row in a wave's K range
     constexpr int PF = NW == 16 ? (NCH < 4 ? NCH : 4) : NCH;   // pieces in flight per lane; divides NCH
     static_assert(NCH % PF == 0, "a piece's slot must not depend on the column block");
@@ -73,8 +77,12 @@ __global__ __launch_bounds__(NW * 64) void fp8_block_decode_kernel(Fp8DecParams 
     for (int c = 0; c < NCH; c++) {
         uint4 raw = make_uint4(0, 0, 0, 0);
         if (nrow < M) raw = *(const uint4*)(p.a + (int64_t)nrow * p.lda + kbase + 64 * c + 16 * q);
-        xf[c][0] = widen8_e4m3(raw.x, raw.y);
-        xf[c][1] = widen8_e4m3(raw.z, raw.w);
+        if constexpr (I8) {
+            xf[c][0] = (v4i){(int)raw.x, (int)raw.y, (int)raw.z, (int)raw.w};
+        } else {
+            xf[c][0] = widen8_e4m3(raw.x, raw.y);
+            xf[c][1] = widen8_e4m3(raw.z, raw.w);
+        }
     }
     // the scales of this lane's row of x1 for the wave's blocks (rows past M: the last row's, their outputs are not stored)
     float s1v[NBLK];
@@ -105,15 +113,21 @@ __global__ __launch_bounds__(NW * 64) void fp8_block_decode_kernel(Fp8DecParams 
 #pragma unroll
         for (int j = 0; j < NBLK; j++) {
             v4f t = RC ? acc : (v4f){0.0f, 0.0f, 0.0f, 0.0f};   // RC: one chain over the whole range
+            v4i ti = {0, 0, 0, 0};
 #pragma unroll
             for (int cc = 0; cc < 2; cc++) {
                 const int c = 2 * j + cc;
                 const uint4 cur = wq[c % PF];
                 wq[c % PF] = c + PF < NCH ? wload(rb, c + PF) : wload(rbn, c + PF - NCH);
-                const v4i w0 = widen8_e4m3(cur.x, cur.y), w1 = widen8_e4m3(cur.z, cur.w);
-                t = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(v8h, w0), __builtin_bit_cast(v8h, xf[c][0]), t, 0, 0, 0);
-                t = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(v8h, w1), __builtin_bit_cast(v8h, xf[c][1]), t, 0, 0, 0);
+                if constexpr (I8) {
+                    ti = __builtin_amdgcn_mfma_i32_16x16x64_i8((v4i){(int)cur.x, (int)cur.y, (int)cur.z, (int)cur.w}, xf[c][0], ti, 0, 0, 0);
+                } else {
+                    const v4i w0 = widen8_e4m3(cur.x, cur.y), w1 = widen8_e4m3(cur.z, cur.w);
+                    t = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(v8h, w0), __builtin_bit_cast(v8h, xf[c][0]), t, 0, 0, 0);
+                    t = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(v8h, w1), __builtin_bit_cast(v8h, xf[c][1]), t, 0, 0, 0);
+                }
             }
+            if constexpr (I8) t = (v4f){(float)ti[0], (float)ti[1], (float)ti[2], (float)ti[3]};
             if constexpr (RC) acc = t;
             else {
                 const float sc = s1v[j] * s2v[j];
@@ -144,6 +158,9 @@ __global__ __launch_bounds__(NW * 64) void fp8_block_decode_kernel(Fp8DecParams 
                 sum[r] = (sum[r] * p.cs[ni * p.cs_stride]) * rsv;
                 if (p.bias) sum[r] = sum[r] + p.bias[ni];
             }
+        } else if (p.bias) {
+#pragma unroll
+            for (int r = 0; r < 4; r++) sum[r] = sum[r] + p.bias[n + r < p.N ? n + r : p.N - 1];
         }
         if (p.out_dt == DT_F32) {
             float* dst = (float*)p.out + (int64_t)nrow * p.N + n;
@@ -163,14 +180,14 @@ __global__ __launch_bounds__(NW * 64) void fp8_block_decode_kernel(Fp8DecParams 
     }
 }
 
-template <int NW, int NBLK, bool RC>
+template <int NW, int NBLK, bool RC, bool I8 = false>
 int launch_decode_one(const Fp8DecParams& p, hipStream_t st)
 {
     const int nblocks = (int)((p.N + 15) / 16);
     const int cus = 256;
     const int grid = nblocks < cus ? nblocks : cus;
     const size_t lds = (size_t)2 * NW * 256 * sizeof(float);
-    hipLaunchKernelGGL((fp8_block_decode_kernel<NW, NBLK, RC>), dim3((unsigned)grid), dim3(NW * 64), lds, st, p);
+    hipLaunchKernelGGL((fp8_block_decode_kernel<NW, NBLK, RC, I8>), dim3((unsigned)grid), dim3(NW * 64), lds, st, p);
     return (int)hipGetLastError();
 }
 
@@ -184,35 +201,38 @@ bool decode_split(int64_t K, int& nw, int& nblk)
     return false;
 }
 
-template <bool RC>
+template <bool RC, bool I8 = false>
 int launch_decode_split(const Fp8DecParams& p, int nw, int nblk, hipStream_t st)
 {
     if (nw == 16) {
-        if (nblk == 1) return launch_decode_one<16, 1, RC>(p, st);
-        if (nblk == 2) return launch_decode_one<16, 2, RC>(p, st);
-        return launch_decode_one<16, 4, RC>(p, st);
+        if (nblk == 1) return launch_decode_one<16, 1, RC, I8>(p, st);
+        if (nblk == 2) return launch_decode_one<16, 2, RC, I8>(p, st);
+        return launch_decode_one<16, 4, RC, I8>(p, st);
     }
     switch (nblk) {
-        case 1: return launch_decode_one<8, 1, RC>(p, st);
-        case 2: return launch_decode_one<8, 2, RC>(p, st);
-        case 3: return launch_decode_one<8, 3, RC>(p, st);
-        case 4: return launch_decode_one<8, 4, RC>(p, st);
-        case 5: return launch_decode_one<8, 5, RC>(p, st);
-        case 6: return launch_decode_one<8, 6, RC>(p, st);
-        default: return launch_decode_one<8, 7, RC>(p, st);
+        case 1: return launch_decode_one<8, 1, RC, I8>(p, st);
+        case 2: return launch_decode_one<8, 2, RC, I8>(p, st);
+        case 3: return launch_decode_one<8, 3, RC, I8>(p, st);
+        case 4: return launch_decode_one<8, 4, RC, I8>(p, st);
+        case 5: return launch_decode_one<8, 5, RC, I8>(p, st);
+        case 6: return launch_decode_one<8, 6, RC, I8>(p, st);
+        default: return launch_decode_one<8, 7, RC, I8>(p, st);
     }
 }
 
 }  // namespace
 
-// fp8 e4m3 block scales with up to 32 rows of x1 (two passes beyond 16), K-contiguous operands, K a whole number of
-// blocks that 16 or 8 waves share equally; OPSNN_NOT_TAKEN otherwise.
+// fp8 e4m3 block scales (or int8 per-tile: the same scales, an fp32 bias, 16-bit output) with up to 32 rows of x1 (two
+// passes beyond 16), K-contiguous operands, K a whole number of blocks that 16 or 8 waves share equally; OPSNN_NOT_TAKEN
+// otherwise.
 int launch_blockscale_decode(const OpsnnQmmArgs& a, hipStream_t st)
 {
     static const bool off = [] { const char* e = getenv("OPSNN_FP8_NO_DECODE"); return e && e[0] == '1'; }();
-    if (off || a.x1_dtype != DT_E4M3 || a.x2_dtype != DT_E4M3 || a.batch != 1) return OPSNN_NOT_TAKEN;
-    if (a.out_dtype != DT_BF16 && a.out_dtype != DT_F16 && a.out_dtype != DT_F32) return OPSNN_NOT_TAKEN;
-    if (a.bias || a.M > 32 || a.N < 256) return OPSNN_NOT_TAKEN;
+    const bool i8 = a.x1_dtype == DT_I8 && a.x2_dtype == DT_I8;
+    if (off || (!i8 && (a.x1_dtype != DT_E4M3 || a.x2_dtype != DT_E4M3)) || a.batch != 1) return OPSNN_NOT_TAKEN;
+    if (a.out_dtype != DT_BF16 && a.out_dtype != DT_F16 && !(a.out_dtype == DT_F32 && !i8)) return OPSNN_NOT_TAKEN;
+    if (a.bias && !(i8 && a.bias_dtype == DT_F32)) return OPSNN_NOT_TAKEN;
+    if (a.M > 32 || a.N < 256) return OPSNN_NOT_TAKEN;
     if (a.gsK != 128 || a.gsN != 128 || (a.gsM != 1 && a.gsM != 128)) return OPSNN_NOT_TAKEN;
     if (a.K % 128 != 0 || a.x1.col_stride != 1 || a.x2.row_stride != 1) return OPSNN_NOT_TAKEN;
     if (((uintptr_t)a.x1.ptr | (uintptr_t)a.x2.ptr | (uint64_t)a.x1.row_stride | (uint64_t)a.x2.col_stride) % 16) return OPSNN_NOT_TAKEN;
@@ -232,7 +252,8 @@ int launch_blockscale_decode(const OpsnnQmmArgs& a, hipStream_t st)
         p.s1 = (const float*)a.x1_scale_mat.ptr + (a.gsM == 1 ? m0 * a.x1_scale_mat.row_stride : 0);
         p.s1_rs = a.x1_scale_mat.row_stride; p.s1_cs = a.x1_scale_mat.col_stride;
         p.s2 = (const float*)a.x2_scale_mat.ptr; p.s2_rs = a.x2_scale_mat.row_stride; p.s2_cs = a.x2_scale_mat.col_stride;
-        const int rc = launch_decode_split<false>(p, nw, nblk, st);
+        p.bias = (const float*)a.bias;
+        const int rc = i8 ? launch_decode_split<false, true>(p, nw, nblk, st) : launch_decode_split<false>(p, nw, nblk, st);
         if (rc != 0) return rc;
     }
     return 0;

@@ -238,7 +238,10 @@ def test_gpu_pertile_i8(gpu, M, K, N, tB):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("M,K,N,tB", [(128, 256, 256, True), (300, 384, 260, True), (640, 1024, 520, False)])
+@pytest.mark.parametrize("M,K,N,tB", [(128, 256, 256, True), (300, 384, 260, True), (640, 1024, 520, False),
+                                      # up to 32 rows: x1 in registers, x2 streamed once per 16 rows (int8 instructions)
+                                      (16, 4096, 512, True), (9, 2048, 264, True), (24, 1024, 520, True), (16, 1024, 256, False),
+                                      (1, 7168, 384, True)])
 def test_gpu_pertile_i8_on_the_matrix_cores(gpu, M, K, N, tB):
     """int8 per-tile with K % 128 == 0 and enough outputs runs on the block-scale kernel with int8 instructions: the
     block sums are exact integers, the fold into the running sum is a fused multiply-add (one rounding where the oracle
