@@ -220,6 +220,124 @@ int launch_decode_split(const Fp8DecParams& p, int nw, int nblk, hipStream_t st)
     }
 }
 
+
+// ---- fp8 e4m3 x fp4 e2m1 with e8m0 scales per 32 elements of K (the MX mode of quant_batch_matmul_v4,
+// qbmmv4_kernel_golden.py:119-186), up to 16 rows of x1 per pass ----
+// The same stream over x2, here N * K / 2 bytes: a lane's 16-byte piece is the 32 consecutive elements of one scale
+// block, four lanes cover the 128 elements of one v_mfma_scale_f32_16x16x128_f8f6f4, and the instruction applies both
+// operands' scales (one byte per lane: lane group q supplies block q) and accumulates in place -- the arithmetic of the
+// tile kernel's FP8_MX_W4 form.  The 8-bit operand's lane group q holds elements [16q, 16q + 16) and [64 + 16q, + 16) of
+// the 128, the 4-bit operand's [32q, 32q + 32): the instruction pairs K indices, not lane groups.
+struct MxW4DecParams {
+    const uint8_t* a;    // x1 [M, K] e4m3, K contiguous
+    const uint8_t* b;    // x2 as [N, K / 2] bytes, K contiguous, two e2m1 per byte
+    int64_t lda, ldb;    // bytes per row
+    const uint8_t* sa;   // e8m0 [M, K / 32], K contiguous
+    const uint8_t* sb;   // e8m0 [N, K / 32]
+    int64_t sa_rs, sb_rs;
+    void* out; int out_dt;
+    int64_t M, N, K;
+    const void* bias; int bias_dt;
+};
+
+template <int NW, int NCH>
+__global__ __launch_bounds__(NW * 64) void mx_a8w4_decode_kernel(MxW4DecParams p)
+{
+    extern __shared__ __attribute__((aligned(16))) float red[];   // [2][NW][256]
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int nrow = lane & 15, q = lane >> 4;
+    const int64_t kbase = (int64_t)wave * (NCH * 128);   // this wave's K range, in elements
+    const int nblocks = (int)((p.N + 15) / 16);
+    const int M = (int)p.M;
+
+    // x1: chunk c of this lane's row, bytes [16q, +16) and [64 + 16q, +16) of the chunk's 128; the scale of block q
+    v8i xf[NCH];
+    int xs[NCH];
+#pragma unroll
+    for (int c = 0; c < NCH; c++) {
+        uint4 lo = make_uint4(0, 0, 0, 0), hi = make_uint4(0, 0, 0, 0);
+        uint32_t sw = 0x7f7f7f7fu;
+        if (nrow < M) {
+            const uint8_t* src = p.a + (int64_t)nrow * p.lda + kbase + 128 * c + 16 * q;
+            lo = *(const uint4*)src;
+            hi = *(const uint4*)(src + 64);
+            sw = *(const uint32_t*)(p.sa + (int64_t)nrow * p.sa_rs + kbase / 32 + 4 * c);
+        }
+        xf[c] = (v8i){(int)lo.x, (int)lo.y, (int)lo.z, (int)lo.w, (int)hi.x, (int)hi.y, (int)hi.z, (int)hi.w};
+        xs[c] = (int)(sw >> (8 * q));
+    }
+
+    auto wload = [&](int rb, int c) {
+        const int64_t n = (int64_t)rb * 16 + nrow;
+        return *(const uint4*)(p.b + (n < p.N ? n : p.N - 1) * p.ldb + (kbase + 128 * c) / 2 + 16 * q);   // columns past the edge repeat the last one
+    };
+    auto sload = [&](int rb, int c) {
+        const int64_t n = (int64_t)rb * 16 + nrow;
+        return *(const uint32_t*)(p.sb + (n < p.N ? n : p.N - 1) * p.sb_rs + kbase / 32 + 4 * c);
+    };
+    int rb = blockIdx.x;
+    uint4 wq[NCH];
+    uint32_t sq[NCH];
+#pragma unroll
+    for (int c = 0; c < NCH; c++) {
+        wq[c] = wload(rb < nblocks ? rb : nblocks - 1, c);
+        sq[c] = sload(rb < nblocks ? rb : nblocks - 1, c);
+    }
+
+    for (int it = 0; rb < nblocks; it++, rb += (int)gridDim.x) {
+        const int rbn = rb + (int)gridDim.x < nblocks ? rb + (int)gridDim.x : rb;   // past the end: a harmless reload
+        const int64_t n0 = (int64_t)rb * 16;
+        v4f acc = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+        for (int c = 0; c < NCH; c++) {
+            const uint4 cur = wq[c];
+            const uint32_t sw = sq[c];
+            wq[c] = wload(rbn, c);   // the next column block's piece takes the register this one leaves
+            sq[c] = sload(rbn, c);
+            const v8i wf = {(int)cur.x, (int)cur.y, (int)cur.z, (int)cur.w, 0, 0, 0, 0};
+            acc = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf, xf[c], acc, 4, 0, 0, (int)(sw >> (8 * q)), 0, xs[c]);
+        }
+        // acc[r]: m = lane % 16, n = n0 + 4 (lane / 16) + r, over this wave's K range
+        float* mine = red + ((it & 1) * NW + wave) * 256;
+        *(v4f*)(mine + lane * 4) = acc;
+        __syncthreads();
+        if (wave != (it & (NW - 1))) continue;
+        const float* all = red + (it & 1) * NW * 256 + lane * 4;
+        v4f sum = *(const v4f*)all;
+#pragma unroll 4
+        for (int w = 1; w < NW; w++) {
+            const v4f o = *(const v4f*)(all + w * 256);
+#pragma unroll
+            for (int r = 0; r < 4; r++) sum[r] = sum[r] + o[r];
+        }
+        if (nrow >= M) continue;
+        const int64_t n = n0 + 4 * q;
+        if (p.bias) {
+#pragma unroll
+            for (int r = 0; r < 4; r++) sum[r] = sum[r] + load_scalar_as_f32(p.bias, p.bias_dt, n + r < p.N ? n + r : p.N - 1);
+        }
+        const v4us o = p.out_dt == DT_BF16 ? pack4_b16<DT_BF16>(sum) : pack4_b16<DT_F16>(sum);
+        uint16_t* dst = (uint16_t*)p.out + (int64_t)nrow * p.N + n;
+        if ((p.N % 4) == 0 && ((uintptr_t)p.out % 8) == 0 && n + 3 < p.N) *(v4us*)dst = o;
+        else {
+#pragma unroll
+            for (int r = 0; r < 4; r++)
+                if (n + r < p.N) dst[r] = o[r];
+        }
+    }
+}
+
+template <int NW, int NCH>
+int launch_mxw4_one(const MxW4DecParams& p, hipStream_t st)
+{
+    const int nblocks = (int)((p.N + 15) / 16);
+    const int grid = nblocks < 256 ? nblocks : 256;
+    const size_t lds = (size_t)2 * NW * 256 * sizeof(float);
+    hipLaunchKernelGGL((mx_a8w4_decode_kernel<NW, NCH>), dim3((unsigned)grid), dim3(NW * 64), lds, st, p);
+    return (int)hipGetLastError();
+}
+
 }  // namespace
 
 // fp8 e4m3 block scales (or int8 per-tile: the same scales, an fp32 bias, 16-bit output) with up to 32 rows of x1 (two
@@ -283,6 +401,52 @@ int launch_rowcol_decode(const OpsnnQmmArgs& a, hipStream_t st)
         p.rs = (const float*)a.x1_scale + (p.rs_stride ? m0 : 0);
         p.cs = (const float*)a.x2_scale; p.bias = (const float*)a.bias;
         const int rc = launch_decode_split<true>(p, nw, nblk, st);
+        if (rc != 0) return rc;
+    }
+    return 0;
+}
+
+// fp8 x fp4 MX with up to 32 rows of x1 (two passes beyond 16): K a whole number of 128-element chunks that 16 waves
+// share 2 or 4 each, or 8 waves 1 .. 7 each; K-contiguous operands and scales; OPSNN_NOT_TAKEN otherwise.
+int launch_mx_a8w4_decode(const OpsnnQmmArgs& a, hipStream_t st)
+{
+    static const bool off = [] { const char* e = getenv("OPSNN_FP8_NO_DECODE"); return e && e[0] == '1'; }();
+    if (off || a.x1_dtype != DT_E4M3 || a.x2_dtype != DT_E2M1 || a.batch != 1) return OPSNN_NOT_TAKEN;
+    if (a.out_dtype != DT_BF16 && a.out_dtype != DT_F16) return OPSNN_NOT_TAKEN;
+    if (a.M > 32 || a.N < 256 || a.K % 128 != 0 || a.x1.col_stride != 1 || a.x2.row_stride != 1 || a.x2.col_stride % 2) return OPSNN_NOT_TAKEN;
+    if (a.x1_scale_mat.col_stride != 2 || a.x2_scale_mat.col_stride != 2) return OPSNN_NOT_TAKEN;   // [rows, K / 64, 2]: a row's bytes contiguous
+    if (a.bias && a.bias_dtype != DT_F32 && a.bias_dtype != DT_BF16 && a.bias_dtype != DT_F16) return OPSNN_NOT_TAKEN;
+    const int64_t ldb = a.x2.col_stride / 2;
+    if (a.x1.row_stride < a.K || ldb < a.K / 2) return OPSNN_NOT_TAKEN;
+    if (((uintptr_t)a.x1.ptr | (uintptr_t)a.x2.ptr | (uint64_t)a.x1.row_stride | (uint64_t)ldb) % 16) return OPSNN_NOT_TAKEN;
+    if (((uintptr_t)a.x1_scale_mat.ptr | (uintptr_t)a.x2_scale_mat.ptr | (uint64_t)a.x1_scale_mat.row_stride | (uint64_t)a.x2_scale_mat.row_stride) % 4)
+        return OPSNN_NOT_TAKEN;
+    if (a.x1_scale_mat.row_stride < a.K / 32 || a.x2_scale_mat.row_stride < a.K / 32) return OPSNN_NOT_TAKEN;
+    const int64_t nb = a.K / 128;
+    int nw = 0, nch = 0;
+    if (nb % 16 == 0 && (nb / 16 == 2 || nb / 16 == 4)) { nw = 16; nch = (int)(nb / 16); }
+    else if (nb % 8 == 0 && nb / 8 <= 7) { nw = 8; nch = (int)(nb / 8); }
+    else return OPSNN_NOT_TAKEN;
+    for (int64_t m0 = 0; m0 < a.M; m0 += 16) {
+        MxW4DecParams p{};
+        p.M = a.M - m0 < 16 ? a.M - m0 : 16; p.N = a.N; p.K = a.K;
+        p.a = (const uint8_t*)a.x1.ptr + m0 * a.x1.row_stride; p.b = (const uint8_t*)a.x2.ptr;
+        p.lda = a.x1.row_stride; p.ldb = ldb;
+        p.sa = (const uint8_t*)a.x1_scale_mat.ptr + m0 * a.x1_scale_mat.row_stride; p.sb = (const uint8_t*)a.x2_scale_mat.ptr;
+        p.sa_rs = a.x1_scale_mat.row_stride; p.sb_rs = a.x2_scale_mat.row_stride;
+        p.out_dt = a.out_dtype; p.out = (char*)a.out + m0 * a.N * 2;
+        p.bias = a.bias; p.bias_dt = a.bias_dtype;
+        int rc;
+        if (nw == 16) rc = nch == 2 ? launch_mxw4_one<16, 2>(p, st) : launch_mxw4_one<16, 4>(p, st);
+        else switch (nch) {
+            case 1: rc = launch_mxw4_one<8, 1>(p, st); break;
+            case 2: rc = launch_mxw4_one<8, 2>(p, st); break;
+            case 3: rc = launch_mxw4_one<8, 3>(p, st); break;
+            case 4: rc = launch_mxw4_one<8, 4>(p, st); break;
+            case 5: rc = launch_mxw4_one<8, 5>(p, st); break;
+            case 6: rc = launch_mxw4_one<8, 6>(p, st); break;
+            default: rc = launch_mxw4_one<8, 7>(p, st); break;
+        }
         if (rc != 0) return rc;
     }
     return 0;

@@ -137,7 +137,11 @@ def test_gpu_a8w4_mx(gpu, M, K, N, tB):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("M,K,N", [(64, 128, 64), (300, 384, 260), (512, 2048, 520), (100, 1024, 1000)])
+@pytest.mark.parametrize("M,K,N", [(64, 128, 64), (300, 384, 260), (512, 2048, 520), (100, 1024, 1000),
+                                   # up to 32 rows: x1 in registers, x2 streamed once per 16 rows; K shared by 16 waves
+                                   # (2 or 4 chunks of 128 each) or by 8 (1 .. 7), ragged columns, two passes
+                                   (16, 4096, 512), (9, 8192, 264), (24, 1024, 520), (1, 7168, 384), (32, 3072, 256),
+                                   (16, 2048, 256)])
 def test_gpu_a8w4_mx_on_the_matrix_cores(gpu, M, K, N):
     """fp8 x fp4 MX with K % 128 == 0 and enough outputs runs on the scaled matrix instruction with a 4-bit x2 operand.
     Bar: the one of MXFP8 (the instruction's alignment error against sum|terms|, mean rel <= 2^-10); the same call on
