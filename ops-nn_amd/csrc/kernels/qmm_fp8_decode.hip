@@ -272,29 +272,36 @@ __global__ __launch_bounds__(NW * 64) void mx_a8w4_decode_kernel(MxW4DecParams p
         const int64_t n = (int64_t)rb * 16 + nrow;
         return *(const uint4*)(p.b + (n < p.N ? n : p.N - 1) * p.ldb + (kbase + 128 * c) / 2 + 16 * q);   // columns past the edge repeat the last one
     };
-    auto sload = [&](int rb, int c) {
+    // x2's scale bytes: the wave's range is NCH words of four per row; lane (row, q) fetches word 4 i + q (one load
+    // instruction per four chunks, 16 rows x one 16-byte run each) and chunk c's word comes over from lane (row, c % 4)
+    constexpr int NSW = (NCH + 3) / 4;
+    auto sload = [&](int rb, int i) {
         const int64_t n = (int64_t)rb * 16 + nrow;
-        return *(const uint32_t*)(p.sb + (n < p.N ? n : p.N - 1) * p.sb_rs + kbase / 32 + 4 * c);
+        const int w = 4 * i + q < NCH ? 4 * i + q : NCH - 1;
+        return *(const uint32_t*)(p.sb + (n < p.N ? n : p.N - 1) * p.sb_rs + kbase / 32 + 4 * w);
     };
     int rb = blockIdx.x;
     uint4 wq[NCH];
-    uint32_t sq[NCH];
+    uint32_t sq[NSW];
 #pragma unroll
-    for (int c = 0; c < NCH; c++) {
-        wq[c] = wload(rb < nblocks ? rb : nblocks - 1, c);
-        sq[c] = sload(rb < nblocks ? rb : nblocks - 1, c);
-    }
+    for (int c = 0; c < NCH; c++) wq[c] = wload(rb, c);
+#pragma unroll
+    for (int i = 0; i < NSW; i++) sq[i] = sload(rb, i);
 
     for (int it = 0; rb < nblocks; it++, rb += (int)gridDim.x) {
         const int rbn = rb + (int)gridDim.x < nblocks ? rb + (int)gridDim.x : rb;   // past the end: a harmless reload
         const int64_t n0 = (int64_t)rb * 16;
         v4f acc = {0.0f, 0.0f, 0.0f, 0.0f};
+        uint32_t sws[NCH];
+#pragma unroll
+        for (int c = 0; c < NCH; c++) sws[c] = (uint32_t)__shfl((int)sq[c / 4], nrow + 16 * (c % 4));
+#pragma unroll
+        for (int i = 0; i < NSW; i++) sq[i] = sload(rbn, i);
 #pragma unroll
         for (int c = 0; c < NCH; c++) {
             const uint4 cur = wq[c];
-            const uint32_t sw = sq[c];
+            const uint32_t sw = sws[c];
             wq[c] = wload(rbn, c);   // the next column block's piece takes the register this one leaves
-            sq[c] = sload(rbn, c);
             const v8i wf = {(int)cur.x, (int)cur.y, (int)cur.z, (int)cur.w, 0, 0, 0, 0};
             acc = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf, xf[c], acc, 4, 0, 0, (int)(sw >> (8 * q)), 0, xs[c]);
         }
