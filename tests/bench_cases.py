@@ -33,6 +33,7 @@ PROFILED_TRAFFIC = {
     (10, None, None): (290.3e6, "profiles/qmm_i4_kg_m4096_k4096_n4096.txt"),
     (12, 16, "exact"): (136.9e6, "profiles/qmm_fp8_block_decode_m16_k7168_n18432.txt"),
     (12, 64, "exact"): (143.5e6, "profiles/qmm_fp8_block_rows_m64_k7168_n18432.txt"),
+    (12, 128, "exact"): (154.8e6, "profiles/qmm_fp8_block_rows_m128_k7168_n18432.txt"),
     (11, 16, "warm"): (133.6e6, "profiles/wqmm_decode_mxfp4_m16_k8192_n28672.txt"),
 }
 
@@ -206,7 +207,7 @@ class Config4Rows(Config4):
         M = args.m or 16
         super().__init__(m, args, M=M)
         self.instr_peak_key = None
-        self.kernel = "fp8_block_decode_kernel" if M <= 16 else "wqmm_rows_kernel<f16, e4m3, block scales> (+ widen_e4m3_f16_kernel)" if M <= 64 else self.kernel
+        self.kernel = "fp8_block_decode_kernel" if M <= 16 else "wqmm_rows_kernel<f16, e4m3, block scales> (+ widen_e4m3_f16_kernel)" if M <= 128 else self.kernel
         self.config = dict(self.config, workload="aclnnQuantMatmulV5 fp8 e4m3 G-B (1x128 / 128x128 scales), bf16 out, decode rows")
 
 
