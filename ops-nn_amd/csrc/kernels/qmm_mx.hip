@@ -77,17 +77,18 @@ struct MxPad {
 static bool mx_pad_layout(const OpsnnQmmArgs& a, MxPad& L)
 {
     const bool fp4 = a.x1_dtype == DT_E2M1 && a.x2_dtype == DT_E2M1, fp8 = a.x1_dtype == DT_E4M3 && a.x2_dtype == DT_E4M3;
-    if ((!fp4 && !fp8) || a.K % 128 != 64 || a.M * a.N < 64 * 64) return false;
-    if (a.out_dtype != DT_BF16 && a.out_dtype != DT_F16 && a.out_dtype != DT_F32) return false;
-    if (a.bias && a.bias_dtype != DT_F32) return false;
-    const int64_t epb = fp4 ? 2 : 1, ks = a.K / 64;
+    const bool a8w4 = a.x1_dtype == DT_E4M3 && a.x2_dtype == DT_E2M1;   // the matrix-core kernel of that mode: 16-bit output, fp32 or 16-bit bias
+    if ((!fp4 && !fp8 && !a8w4) || a.K % 128 != 64 || a.M * a.N < 64 * 64) return false;
+    if (a.out_dtype != DT_BF16 && a.out_dtype != DT_F16 && !(a.out_dtype == DT_F32 && !a8w4)) return false;
+    if (a.bias && a.bias_dtype != DT_F32 && !(a8w4 && (a.bias_dtype == DT_BF16 || a.bias_dtype == DT_F16))) return false;
+    const int64_t epb1 = a.x1_dtype == DT_E2M1 ? 2 : 1, epb2 = a.x2_dtype == DT_E2M1 ? 2 : 1, ks = a.K / 64;   // elements per byte
     if (a.x1.col_stride != 1 || a.x2.row_stride != 1) return false;
     if (a.x1_scale_mat.col_stride != 2 || a.x1_scale_mat.row_stride != ks * 2) return false;
     if (a.x2_scale_mat.col_stride != 2 || a.x2_scale_mat.row_stride != ks * 2) return false;
     if (a.x1.batch_stride < 0 || a.x2.batch_stride < 0 || a.x1_scale_mat.batch_stride < 0 || a.x2_scale_mat.batch_stride < 0) return false;
     // 16-byte pieces of the data rows, 2-byte pieces of the scale rows
-    if (((uintptr_t)a.x1.ptr | (uintptr_t)a.x2.ptr | (uint64_t)(a.x1.row_stride / epb) | (uint64_t)(a.x2.col_stride / epb) |
-         (uint64_t)(a.x1.batch_stride / epb) | (uint64_t)(a.x2.batch_stride / epb)) % 16) return false;
+    if (((uintptr_t)a.x1.ptr | (uintptr_t)a.x2.ptr | (uint64_t)(a.x1.row_stride / epb1) | (uint64_t)(a.x2.col_stride / epb2) |
+         (uint64_t)(a.x1.batch_stride / epb1) | (uint64_t)(a.x2.batch_stride / epb2)) % 16) return false;
     if (((uintptr_t)a.x1_scale_mat.ptr | (uintptr_t)a.x2_scale_mat.ptr | (uint64_t)a.x1_scale_mat.batch_stride | (uint64_t)a.x2_scale_mat.batch_stride) % 2) return false;
     if ((a.M + 3) / 4 > 65535 || (a.N + 3) / 4 > 65535) return false;
     L.Kp = a.K + 64;
@@ -96,8 +97,8 @@ static bool mx_pad_layout(const OpsnnQmmArgs& a, MxPad& L)
     L.snb1 = a.x1_scale_mat.batch_stride == 0 && a.batch > 1 ? 1 : a.batch;
     L.snb2 = a.x2_scale_mat.batch_stride == 0 ? 1 : a.batch;
     const uint64_t ksp = (uint64_t)L.Kp / 64;
-    L.o_x2 = align_up((uint64_t)L.nb1 * a.M * (L.Kp / epb), 256);
-    L.o_s1 = L.o_x2 + align_up((uint64_t)L.nb2 * a.N * (L.Kp / epb), 256);
+    L.o_x2 = align_up((uint64_t)L.nb1 * a.M * (L.Kp / epb1), 256);
+    L.o_s1 = L.o_x2 + align_up((uint64_t)L.nb2 * a.N * (L.Kp / epb2), 256);
     L.o_s2 = L.o_s1 + align_up((uint64_t)L.snb1 * a.M * ksp * 2, 256);
     L.total = L.o_s2 + align_up((uint64_t)L.snb2 * a.N * ksp * 2, 256);
     return true;
@@ -107,14 +108,14 @@ static bool mx_pad_layout(const OpsnnQmmArgs& a, MxPad& L)
 static int mx_pad_prestep(OpsnnQmmArgs& a, const MxPad& L, hipStream_t st)
 {
     if (!a.workspace || (uintptr_t)a.workspace % 16) return OPSNN_NOT_TAKEN;
-    const bool fp4 = a.x1_dtype == DT_E2M1;
-    const int64_t epb = fp4 ? 2 : 1, kb = a.K / epb, kbp = L.Kp / epb, ks2 = a.K / 64 * 2, ksp2 = L.Kp / 64 * 2;
+    const int64_t epb1 = a.x1_dtype == DT_E2M1 ? 2 : 1, epb2 = a.x2_dtype == DT_E2M1 ? 2 : 1;
+    const int64_t kb1 = a.K / epb1, kbp1 = L.Kp / epb1, kb2 = a.K / epb2, kbp2 = L.Kp / epb2, ks2 = a.K / 64 * 2, ksp2 = L.Kp / 64 * 2;
     uint8_t* w = (uint8_t*)a.workspace;
     auto grid = [](int64_t pieces, int64_t rows, int64_t nb) { return dim3((unsigned)((pieces + 63) / 64), (unsigned)((rows + 3) / 4), (unsigned)nb); };
-    hipLaunchKernelGGL(mx_pad_rows_kernel<16>, grid(kbp / 16, a.M, L.nb1), dim3(256), 0, st, (const uint8_t*)a.x1.ptr, a.x1.row_stride / epb,
-                       a.x1.batch_stride / epb, w, a.M, kb, kbp, 0u);
-    hipLaunchKernelGGL(mx_pad_rows_kernel<16>, grid(kbp / 16, a.N, L.nb2), dim3(256), 0, st, (const uint8_t*)a.x2.ptr, a.x2.col_stride / epb,
-                       a.x2.batch_stride / epb, w + L.o_x2, a.N, kb, kbp, 0u);
+    hipLaunchKernelGGL(mx_pad_rows_kernel<16>, grid(kbp1 / 16, a.M, L.nb1), dim3(256), 0, st, (const uint8_t*)a.x1.ptr, a.x1.row_stride / epb1,
+                       a.x1.batch_stride / epb1, w, a.M, kb1, kbp1, 0u);
+    hipLaunchKernelGGL(mx_pad_rows_kernel<16>, grid(kbp2 / 16, a.N, L.nb2), dim3(256), 0, st, (const uint8_t*)a.x2.ptr, a.x2.col_stride / epb2,
+                       a.x2.batch_stride / epb2, w + L.o_x2, a.N, kb2, kbp2, 0u);
     hipLaunchKernelGGL(mx_pad_rows_kernel<2>, grid(ksp2 / 2, a.M, L.snb1), dim3(256), 0, st, (const uint8_t*)a.x1_scale_mat.ptr, ks2,
                        a.x1_scale_mat.batch_stride, w + L.o_s1, a.M, ks2, ksp2, 0x7f7fu);
     hipLaunchKernelGGL(mx_pad_rows_kernel<2>, grid(ksp2 / 2, a.N, L.snb2), dim3(256), 0, st, (const uint8_t*)a.x2_scale_mat.ptr, ks2,
@@ -155,7 +156,14 @@ int launch_mx_mfma(const OpsnnQmmArgs& a0, hipStream_t st)
     OpsnnQmmArgs a = a0;
     const bool fp4 = a.x1_dtype == DT_E2M1 && a.x2_dtype == DT_E2M1;
     const bool fp8 = a.x1_dtype == DT_E4M3 && a.x2_dtype == DT_E4M3;
-    if (a.x1_dtype == DT_E4M3 && a.x2_dtype == DT_E2M1) return launch_mx_a8w4_mfma(a, st);   // fp8 x fp4: qmm_fp8_block.hip
+    if (a.x1_dtype == DT_E4M3 && a.x2_dtype == DT_E2M1) {   // fp8 x fp4: qmm_fp8_block.hip, behind the same padding of a K tail
+        MxPad L;
+        if (mx_pad_layout(a, L)) {
+            const int rc = mx_pad_prestep(a, L, st);
+            if (rc != 0) return rc;
+        }
+        return launch_mx_a8w4_mfma(a, st);
+    }
     if (!fp4 && !fp8) return OPSNN_NOT_TAKEN;
     // MXFP8 runs on the block kernel of qmm_fp8_block.hip in MX mode (16x16x128 instructions, 64 x 128 per wave, the
     // pipeline tuned for the fp8 block-scale path); the 32x32x64 tile kernel stays available on request

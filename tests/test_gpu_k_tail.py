@@ -112,6 +112,42 @@ def test_mx_k_tail(gpu, M, K, N, fp4, batch, bias):
     m.lib().aclDestroyAclOpExecutor(ex)
 
 
+@pytest.mark.parametrize("M,K,N", [(300, 960, 260), (128, 192, 256), (16, 1984, 512)])
+def test_mx_fp8_fp4_k_tail(gpu, M, K, N):
+    """fp8 x fp4 MX with K % 128 == 64: the same padded copies (x1 rows of K + 64 bytes, x2 rows of half that), then the
+    matrix-core kernel of the mode (the stream kernel with 16 rows); its bar, the plain kernel bit-identical."""
+    m = gpu
+    print(f"case fp8 x fp4 mx K tail M={M} K={K} N={N}", flush=True)
+    inp = cases.make_a8w4_mx_inputs(m, M, K, N, K + N, True)
+    want = cases.oracle_a8w4_mx(m, inp, M, K, N, True, m.ACL_FLOAT16)
+    got = cases.run_a8w4_mx_aclnn(m, inp, M, K, N, True, m.ACL_FLOAT16)
+    pos = dict(inp, x1=inp["x1"] & 0x7F, x2=inp["x2"] & 0x77, bias=np.zeros_like(inp["bias"]))
+    abs_sum = orc.b16_to_f32(cases.oracle_a8w4_mx(m, pos, M, K, N, True, m.ACL_FLOAT16), orc.F16).astype(np.float64)
+    g, w = orc.b16_to_f32(got, orc.F16), orc.b16_to_f32(want, orc.F16)
+    assert np.isfinite(g).all()
+    err = np.abs(g.astype(np.float64) - w)
+    bound = 2.0 ** -7 * np.abs(w) + 2.0 ** -14 * abs_sum
+    mx, mean = orc.rel_err_stats(g, w)
+    assert float((err / np.maximum(bound, 1e-30)).max()) <= 1.0 and mean <= 2.0 ** -10, f"max rel {mx:.3e} mean rel {mean:.3e}"
+    # phase 1 plans the four padded copies
+    up = lambda v: -(-v // 256) * 256
+    Kp = K + 64
+    d = {k: m.DeviceBuffer(host=v) for k, v in inp.items()}
+    x1 = m.Tensor((M, K), m.ACL_FLOAT8_E4M3FN, d["x1"]); x2 = m.Tensor((N, K), m.ACL_FLOAT4_E2M1, d["x2"])
+    s1 = m.Tensor(inp["s1"].shape, m.ACL_FLOAT8_E8M0, d["s1"]); s2 = m.Tensor(inp["s2"].shape, m.ACL_FLOAT8_E8M0, d["s2"])
+    bias = m.Tensor((1, N), m.ACL_FLOAT16, d["bias"])
+    o = m.Tensor((M, N), m.ACL_FLOAT16, m.DeviceBuffer(M * N * 2))
+    rc, ws, ex = m.quant_matmul_v5_get_workspace(x1, x2, s1, s2, o, bias=bias, transpose_x2=True, group_size=32)
+    assert rc == 0 and ws == up(M * Kp) + up(N * Kp // 2) + up(M * (Kp // 64) * 2) + up(N * (Kp // 64) * 2), (rc, ws)
+    m.lib().aclDestroyAclOpExecutor(ex)
+    m.lib().opsnnSetForcePlain(1)
+    try:
+        exact = cases.run_a8w4_mx_aclnn(m, inp, M, K, N, True, m.ACL_FLOAT16)
+    finally:
+        m.lib().opsnnSetForcePlain(0)
+    assert np.array_equal(exact, want)
+
+
 @pytest.mark.parametrize("M,K,N,s_len,pt", [(256, 1000, 264, "N", "M"), (128, 72, 512, "N", True)])
 def test_fp8_row_and_column_scales_k_tail(gpu, M, K, N, s_len, pt):
     m = gpu
