@@ -34,6 +34,7 @@ PROFILED_TRAFFIC = {
     (12, 16, "exact"): (136.9e6, "profiles/qmm_fp8_block_decode_m16_k7168_n18432.txt"),
     (12, 64, "exact"): (143.5e6, "profiles/qmm_fp8_block_rows_m64_k7168_n18432.txt"),
     (12, 128, "exact"): (154.8e6, "profiles/qmm_fp8_block_rows_m128_k7168_n18432.txt"),
+    (13, 16, None): (131.0e6, "profiles/qmm_mx_a8w4_decode_m16_k8192_n28672.txt"),
     (11, 16, "warm"): (133.6e6, "profiles/wqmm_decode_mxfp4_m16_k8192_n28672.txt"),
 }
 
@@ -209,6 +210,56 @@ class Config4Rows(Config4):
         self.instr_peak_key = None
         self.kernel = "fp8_block_decode_kernel" if M <= 16 else "wqmm_rows_kernel<f16, e4m3, block scales> (+ widen_e4m3_f16_kernel)" if M <= 128 else self.kernel
         self.config = dict(self.config, workload="aclnnQuantMatmulV5 fp8 e4m3 G-B (1x128 / 128x128 scales), bf16 out, decode rows")
+
+
+class ConfigA8W4Rows(Workload):
+    """Not a BASELINE config: the fp8 x fp4 MX mode of aclnnQuantMatmulV5 (e8m0 scales per 32 elements of K) at config 3's
+    K and N with the few rows of x1 of a decode step (--m, default 16): a stream over the 4-bit x2, reported against the
+    HBM roofline (both operands, both scale tables, bias and output per step)."""
+    metric = "quant_gemm_stream_bandwidth"
+    bound = "hbm"
+    peak_key = "fp8"
+    dtype = "fp8_e4m3 x fp4_e2m1, e8m0 scales inside the matrix instruction, fp32 sums"
+    kernel = "mx_a8w4_decode_kernel (v_mfma_scale_f32_16x16x128_f8f6f4)"
+
+    def __init__(self, m, args, K=8192, N=28672):
+        M = args.m or 16
+        self.m, self.M, self.K, self.N = m, M, K, N
+        self.inp = cases.make_a8w4_mx_inputs(m, M, K, N, 0, True)
+        self.d = {k: m.DeviceBuffer(host=v) for k, v in self.inp.items()}
+        self.d_out = m.DeviceBuffer(M * N * 2)
+        self.t_x1 = m.Tensor((M, K), m.ACL_FLOAT8_E4M3FN, self.d["x1"])
+        self.t_x2 = m.Tensor((N, K), m.ACL_FLOAT4_E2M1, self.d["x2"])
+        self.t_s1 = m.Tensor(self.inp["s1"].shape, m.ACL_FLOAT8_E8M0, self.d["s1"])
+        self.t_s2 = m.Tensor(self.inp["s2"].shape, m.ACL_FLOAT8_E8M0, self.d["s2"])
+        self.t_bias = m.Tensor((1, N), m.ACL_FLOAT16, self.d["bias"])
+        self.t_out = m.Tensor((M, N), m.ACL_FLOAT16, self.d_out)
+        rc, ws, ex = m.quant_matmul_v5_get_workspace(self.t_x1, self.t_x2, self.t_s1, self.t_s2, self.t_out, bias=self.t_bias,
+                                                     transpose_x2=True, group_size=32)
+        m.check(rc, "phase 1")
+        m.lib().aclDestroyAclOpExecutor(ex)
+        self.ws = m.DeviceBuffer(ws) if ws else None
+        self.ws_size = ws
+        self.flop = 2 * M * N * K
+        self.bytes = M * K + N * K // 2 + M * K // 32 + N * K // 32 + 2 * N + 2 * M * N
+        self.config = {"workload": "aclnnQuantMatmulV5 fp8 e4m3 x fp4 e2m1 MX, fp16 bias and out, decode rows", "M": M, "K": K, "N": N,
+                       "x2_layout": "K-contiguous (transposeX2)"}
+
+    def step(self, stream):
+        m = self.m
+        rc, ws, ex = m.quant_matmul_v5_get_workspace(self.t_x1, self.t_x2, self.t_s1, self.t_s2, self.t_out, bias=self.t_bias,
+                                                     transpose_x2=True, group_size=32)
+        m.check(rc, "phase 1")
+        m.check(m.lib().aclnnQuantMatmulV5(self.ws.ptr if self.ws else None, self.ws_size, ex, stream.ptr), "phase 2")
+
+    def cpu_baseline(self):
+        rows = min(self.M, 16)
+        t0 = time.perf_counter()
+        orc.qmm_mx(np.ascontiguousarray(self.inp["x1"][:rows]), self.inp["x2"], orc.E4M3, orc.E2M1, rows, self.K, self.N, False, True,
+                   np.ascontiguousarray(self.inp["s1"][:rows]), self.inp["s2"], orc.f16_to_f32(self.inp["bias"]), orc.F16)
+        t = time.perf_counter() - t0
+        return {"value": self.bytes * rows / self.M / t / 1e9, "unit": "GB/s", "cores": _cores(), "kind": "port",
+                "sample": f"first {rows} of {self.M} rows of x1 against the full x2 (oracle/liboracle.so, OpenMP), {t:.2f} s"}
 
 
 class Config5(Workload):
@@ -490,6 +541,8 @@ def make_workload(m, config, args):
         return Config4(m, args)
     if config == 12:
         return Config4Rows(m, args)
+    if config == 13:
+        return ConfigA8W4Rows(m, args)
     if config == 5:
         return Config5(m, args)
     raise SystemExit(f"bench.py: config {config} is not wired up yet")
