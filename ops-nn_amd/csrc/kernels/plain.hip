@@ -224,14 +224,20 @@ __global__ void qmm_tcg_plain(OpsnnQmmArgs a)
 // the 32 elements k0 .. k0+31 of row n (16 bytes in, 32 bytes out), t = n * K/32 + k0/32.  They share one scale
 // (gsK % 32 == 0), and every step of the operation is odd in the weight, so the thread converts the 8 magnitudes once
 // into a table of 8 bytes and each element is a table byte with the nibble's sign bit.
-__global__ __launch_bounds__(256) void tcg_requant_kernel(OpsnnQmmArgs a, uint8_t* w8, float* cs, float* one)
+// Rows of w8 are Kp >= K bytes long (K rounded up to the matrix-core kernels' 128): the tail is written as zeros.
+__global__ __launch_bounds__(256) void tcg_requant_kernel(OpsnnQmmArgs a, uint8_t* w8, float* cs, float* one, int64_t Kp)
 {
     const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    const int64_t kq = a.K / 32;
+    const int64_t kq = Kp / 32;
     if (t == 0) one[0] = 1.0f;
     if (t < a.N) cs[t] = a.y_scale ? trunc19(u2f((uint32_t)((const uint64_t*)a.y_scale)[a.y_scale_len == 1 ? 0 : t])) : 1.0f;
     if (t >= a.N * kq) return;
     const int64_t n = t / kq, k0 = (t % kq) * 32;
+    if (k0 >= a.K) {
+        uint4* z = (uint4*)(w8 + n * Kp + k0);
+        z[0] = z[1] = make_uint4(0, 0, 0, 0);
+        return;
+    }
     const int sdt = a.x2_scale_dtype;
     const float sc = load_scalar_as_f32(a.x2_scale_mat.ptr, sdt, (k0 / a.gsK) * a.x2_scale_mat.row_stride + n * a.x2_scale_mat.col_stride);
     uint64_t table = 0;
@@ -256,9 +262,17 @@ __global__ __launch_bounds__(256) void tcg_requant_kernel(OpsnnQmmArgs a, uint8_
         }
         o[w] = r;
     }
-    uint4* dst = (uint4*)(w8 + n * a.K + k0);
+    uint4* dst = (uint4*)(w8 + n * Kp + k0);
     dst[0] = make_uint4(o[0], o[1], o[2], o[3]);
     dst[1] = make_uint4(o[4], o[5], o[6], o[7]);
+}
+// x1 [M, K] (rows of 16-byte pieces) into rows of Kp bytes, the tail zero
+__global__ __launch_bounds__(256) void tcg_pad_x1_kernel(const uint8_t* __restrict__ src, int64_t ld, uint8_t* __restrict__ dst, int64_t M, int64_t K, int64_t Kp)
+{
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x, pieces = Kp / 16;
+    if (i >= M * pieces) return;
+    const int64_t r = i / pieces, c = i - r * pieces;
+    *(uint4*)(dst + r * Kp + c * 16) = c * 16 < K ? *(const uint4*)(src + r * ld + c * 16) : make_uint4(0, 0, 0, 0);
 }
 __global__ void qmm_i4_asym_plain(OpsnnQmmArgs a)
 {
@@ -295,18 +309,22 @@ void weight_cache_commit(void* buffer, hipStream_t st);
 
 static inline uint64_t align256(uint64_t v) { return (v + 255) / 256 * 256; }
 // The re-quantised weight with its side values: e4m3 bytes [N, K], the decoded output scale per column, a 1.0.
-static inline uint64_t tcg_blob_bytes(const OpsnnQmmArgs& a) { return align256((uint64_t)a.N * a.K) + align256((uint64_t)a.N * 4) + 256; }
-// 17 .. 128 rows go to the many-rows streaming kernel, which wants x1 widened to fp16 (M * K * 2 bytes behind the blob)
-static inline uint64_t tcg_rows_bytes(const OpsnnQmmArgs& a) { return a.M > 16 && a.M <= 128 ? (uint64_t)a.M * a.K * 2 : 0; }
+static inline int64_t tcg_kp(const OpsnnQmmArgs& a) { return (a.K + 127) / 128 * 128; }   // K as the matrix-core kernels walk it
+static inline uint64_t tcg_blob_bytes(const OpsnnQmmArgs& a) { return align256((uint64_t)a.N * tcg_kp(a)) + align256((uint64_t)a.N * 4) + 256; }
+// a K tail: x1 copied into rows of Kp bytes behind the blob
+static inline uint64_t tcg_x1pad_bytes(const OpsnnQmmArgs& a) { return tcg_kp(a) != a.K ? align256((uint64_t)a.M * tcg_kp(a)) : 0; }
+// 17 .. 128 rows go to the many-rows streaming kernel, which wants x1 widened to fp16 (M * Kp * 2 bytes behind those)
+static inline uint64_t tcg_rows_bytes(const OpsnnQmmArgs& a) { return a.M > 16 && a.M <= 128 ? (uint64_t)a.M * tcg_kp(a) * 2 : 0; }
 // Workspace of the matrix-core path of the fp8 x fp4 group-scale mode (0: the shape stays on the plain kernel).
 uint64_t tcg_workspace_bytes(const OpsnnQmmArgs& a)
 {
     if (a.x1_dtype != DT_E4M3 || a.x2_dtype != DT_E2M1 || a.batch != 1) return 0;
-    if (a.K % 128 != 0 || a.gsK <= 0 || a.gsK % 32 != 0 || (uintptr_t)a.x2.ptr % 16 != 0 || a.M * a.N < 64 * 64) return 0;
+    if (a.K % 32 != 0 || a.K < 128 || a.gsK <= 0 || a.gsK % 32 != 0 || (uintptr_t)a.x2.ptr % 16 != 0 || a.M * a.N < 64 * 64) return 0;
     if (a.x1.col_stride != 1 || a.x2.row_stride != 1 || a.x2.col_stride != a.K) return 0;
+    if (a.K % 128 != 0 && (((uintptr_t)a.x1.ptr | (uint64_t)a.x1.row_stride) % 16 != 0 || a.x1.row_stride < a.K)) return 0;   // the padded copy of x1 moves 16-byte pieces
     if (a.out_dtype != DT_BF16 && a.out_dtype != DT_F16) return 0;
     if (a.bias && a.bias_dtype != DT_F32) return 0;
-    return tcg_blob_bytes(a) + tcg_rows_bytes(a);
+    return tcg_blob_bytes(a) + tcg_x1pad_bytes(a) + tcg_rows_bytes(a);
 }
 // Re-quantise x2 into the workspace -- or, with the weight cache on and dense scales, once into a cached buffer that
 // later calls with the same x2, scales and output scale find again -- then an fp8 kernel with a column scale (the
@@ -319,26 +337,34 @@ int launch_tcg_mfma(const OpsnnQmmArgs& a, hipStream_t st)
     uint8_t* w8 = (uint8_t*)a.workspace;
     // what the cache key has to tell apart beside the three pointers, K, N and the size: group size, scale type, which
     // way the dense scale matrix lies, one output scale or N
-    const int64_t kg = a.K / a.gsK;
+    const int64_t Kp = tcg_kp(a);
+    const int64_t kg = (a.K + a.gsK - 1) / a.gsK;
     const bool s_nk = a.x2_scale_mat.row_stride == 1 && a.x2_scale_mat.col_stride == kg;
     const bool s_kn = a.x2_scale_mat.row_stride == a.N && a.x2_scale_mat.col_stride == 1;
-    const bool dense = (s_nk || s_kn) && a.K % a.gsK == 0;
+    const bool dense = s_nk || s_kn;
     const int64_t key = (a.gsK << 8) | ((int64_t)(a.x2_scale_dtype & 31) << 3) | (s_nk ? 4 : 0) | (a.y_scale_len == 1 ? 2 : 0) | 1;
     bool fresh = false;
     void* cached = dense ? weight_cache_blob3(a.x2.ptr, a.x2_scale_mat.ptr, a.y_scale, a.K, a.N, 4, key, blob, st, &fresh) : nullptr;
     if (cached) w8 = (uint8_t*)cached;
-    float* cs = (float*)(w8 + align256((uint64_t)a.N * a.K));
+    float* cs = (float*)(w8 + align256((uint64_t)a.N * Kp));
     float* one = (float*)((char*)cs + align256((uint64_t)a.N * 4));
     if (!cached || fresh) {
-        const int64_t threads = a.N * (a.K / 32);   // >= N since K >= 128
-        hipLaunchKernelGGL(tcg_requant_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, st, a, w8, cs, one);
+        const int64_t threads = a.N * (Kp / 32);   // >= N since Kp >= 128
+        hipLaunchKernelGGL(tcg_requant_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, st, a, w8, cs, one, Kp);
         if (cached) weight_cache_commit(cached, st);
     }
     OpsnnQmmArgs b = a;
-    b.x2.ptr = w8; b.x2_dtype = DT_E4M3; b.x2.row_stride = 1; b.x2.col_stride = a.K; b.x2.batch_stride = 0;
+    if (Kp != a.K) {   // a K tail: x1 into rows of Kp bytes behind the blob's place in the workspace; zero products change no sum
+        uint8_t* x1p = (uint8_t*)a.workspace + blob;
+        const int64_t pieces = a.M * (Kp / 16);
+        hipLaunchKernelGGL(tcg_pad_x1_kernel, dim3((unsigned)((pieces + 255) / 256)), dim3(256), 0, st, (const uint8_t*)a.x1.ptr, a.x1.row_stride, x1p,
+                           a.M, a.K, Kp);
+        b.x1.ptr = x1p; b.x1.row_stride = Kp; b.K = Kp;
+    }
+    b.x2.ptr = w8; b.x2_dtype = DT_E4M3; b.x2.row_stride = 1; b.x2.col_stride = Kp; b.x2.batch_stride = 0;
     b.x1_scale = one; b.x1_scale_len = 1;
     b.x2_scale = cs; b.x2_scale_dtype = DT_F32; b.x2_scale_len = a.N;
-    b.workspace = tcg_rows_bytes(a) ? (char*)a.workspace + blob : nullptr;
+    b.workspace = tcg_rows_bytes(a) ? (char*)a.workspace + blob + tcg_x1pad_bytes(a) : nullptr;
     if (a.force_variant == 0) {
         int rc = launch_rowcol_rows(b, st);
         if (rc != OPSNN_NOT_TAKEN) return rc;

@@ -189,7 +189,11 @@ def test_gpu_tcg(gpu, M, K, N, s_dt, out_dt, ys_i64):
                                                # to 16 rows, two passes up to 32, the many-rows kernel from 17 to 128)
                                                (16, 4096, 512, "bf16", "bf16"), (9, 2048, 264, "f16", "f16"),
                                                (24, 1024, 520, "bf16", "f16"), (40, 2048, 512, "bf16", "bf16"),
-                                               (100, 1024, 256, "f16", "bf16")])
+                                               (100, 1024, 256, "f16", "bf16"),
+                                               # K tails (K % 128 = 32, 64, 96): the re-quantised weight and a copy of x1 in
+                                               # rows padded with zeros to the next multiple of 128
+                                               (300, 416, 260, "bf16", "bf16"), (16, 1984, 512, "f16", "f16"),
+                                               (64, 1120, 256, "bf16", "f16")])
 def test_gpu_tcg_on_the_matrix_cores(gpu, M, K, N, s_dt, out_dt, fast):
     """fp8 x fp4 with 16-bit group scales, K % 128 == 0 and enough outputs: a prologue writes the re-quantised e4m3 weight
     (the oracle's bytes) into the workspace and the fp8 matrix-core kernel does the product with the decoded output scale
