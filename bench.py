@@ -93,8 +93,8 @@ def main():
                     help="0 (default): every BASELINE config, headline config 2; 1-5: that BASELINE config only; 6-9: the "
                          "pre-pack / quantizer operators that prepare their tensors; 10: the int4 x int4 K-G mode at 4096^3; "
                          "11: config 3's shape with mxfp4 weights; 12: config 4's operator with the --m rows of a decode step; "
-                         "13: the fp8 x fp4 MX mode at config 3's K and N with the --m rows of a decode step")
-    ap.add_argument("--m", type=int, default=None, help="M for config 3 (1, 16, 64 or 256) and configs 11, 12, 13 (default 16)")
+                         "13 / 14: the fp8 x fp4 MX mode / the int8 per-tile mode at config 3's K and N with the --m rows of a decode step")
+    ap.add_argument("--m", type=int, default=None, help="M for config 3 (1, 16, 64 or 256) and configs 11 to 14 (default 16)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--int8-range", type=int, default=None,
                     help="config 2: operands uniform in [-R, R] (default: the full int8 range, the most power-hungry data)")
@@ -137,7 +137,7 @@ def main():
 
     if args.config:
         wl = bench_cases.make_workload(m, args.config, args)
-        wl.key = (args.config, (args.m or 16) if args.config in (3, 11, 12, 13) else None)
+        wl.key = (args.config, (args.m or 16) if args.config in (3, 11, 12, 13, 14) else None)
         if args.calib_copy:
             src, dst = m.DeviceBuffer(8192 * 8192), m.DeviceBuffer(8192 * 8192)
             src.fill(1)

@@ -35,6 +35,7 @@ PROFILED_TRAFFIC = {
     (12, 64, "exact"): (143.5e6, "profiles/qmm_fp8_block_rows_m64_k7168_n18432.txt"),
     (12, 128, "exact"): (154.8e6, "profiles/qmm_fp8_block_rows_m128_k7168_n18432.txt"),
     (13, 16, None): (131.0e6, "profiles/qmm_mx_a8w4_decode_m16_k8192_n28672.txt"),
+    (14, 16, None): (244.0e6, "profiles/qmm_i8_pertile_decode_m16_k8192_n28672.txt"),
     (11, 16, "warm"): (133.6e6, "profiles/wqmm_decode_mxfp4_m16_k8192_n28672.txt"),
 }
 
@@ -257,6 +258,59 @@ class ConfigA8W4Rows(Workload):
         t0 = time.perf_counter()
         orc.qmm_mx(np.ascontiguousarray(self.inp["x1"][:rows]), self.inp["x2"], orc.E4M3, orc.E2M1, rows, self.K, self.N, False, True,
                    np.ascontiguousarray(self.inp["s1"][:rows]), self.inp["s2"], orc.f16_to_f32(self.inp["bias"]), orc.F16)
+        t = time.perf_counter() - t0
+        return {"value": self.bytes * rows / self.M / t / 1e9, "unit": "GB/s", "cores": _cores(), "kind": "port",
+                "sample": f"first {rows} of {self.M} rows of x1 against the full x2 (oracle/liboracle.so, OpenMP), {t:.2f} s"}
+
+
+class ConfigPerTileRows(Workload):
+    """Not a BASELINE config: the int8 per-tile mode of aclnnQuantMatmulV5 (1x128 scales on x1, 128x128 on x2, fp32 bias) at
+    config 3's K and N with the few rows of x1 of a decode step (--m, default 16): a stream over x2 against the HBM roofline."""
+    metric = "quant_gemm_stream_bandwidth"
+    bound = "hbm"
+    peak_key = "int8"
+    dtype = "int8 x int8, exact int32 sums per 128-block, fp32 fold"
+    kernel = "fp8_block_decode_kernel<int8> (v_mfma_i32_16x16x64_i8)"
+
+    def __init__(self, m, args, K=8192, N=28672):
+        M = args.m or 16
+        self.m, self.M, self.K, self.N = m, M, K, N
+        self.inp = cases.make_pertile_i8_inputs(m, M, K, N, 0, True)
+        self.d = {k: m.DeviceBuffer(host=v) for k, v in self.inp.items()}
+        self.d_out = m.DeviceBuffer(M * N * 2)
+        self.t_x1 = m.Tensor((M, K), m.ACL_INT8, self.d["x1"])
+        self.t_x2 = m.Tensor((N, K), m.ACL_INT8, self.d["x2"])
+        self.t_s1 = m.Tensor(self.inp["s1"].shape, m.ACL_FLOAT, self.d["s1"])
+        self.t_s2 = m.Tensor(self.inp["s2"].shape, m.ACL_FLOAT, self.d["s2"])
+        self.t_bias = m.Tensor((N,), m.ACL_FLOAT, self.d["bias"])
+        self.t_out = m.Tensor((M, N), m.ACL_BF16, self.d_out)
+        self.gs = (1 << 32) | (128 << 16) | 128
+        rc, ws, ex = self._phase1()
+        m.lib().aclDestroyAclOpExecutor(ex)
+        self.ws = m.DeviceBuffer(ws) if ws else None
+        self.ws_size = ws
+        self.flop = 2 * M * N * K
+        self.bytes = M * K + N * K + 4 * M * (K // 128) + 4 * (N // 128) * (K // 128) + 4 * N + 2 * M * N
+        self.config = {"workload": "aclnnQuantMatmulV5 int8 per-tile (1x128 / 128x128 scales), fp32 bias, bf16 out, decode rows", "M": M, "K": K,
+                       "N": N, "x2_layout": "K-contiguous (transposeX2)"}
+
+    def _phase1(self):
+        m = self.m
+        rc, ws, ex = m.quant_matmul_v5_get_workspace(self.t_x1, self.t_x2, self.t_s1, self.t_s2, self.t_out, bias=self.t_bias,
+                                                     transpose_x2=True, group_size=self.gs)
+        m.check(rc, "phase 1")
+        return rc, ws, ex
+
+    def step(self, stream):
+        m = self.m
+        rc, ws, ex = self._phase1()
+        m.check(m.lib().aclnnQuantMatmulV5(self.ws.ptr if self.ws else None, self.ws_size, ex, stream.ptr), "phase 2")
+
+    def cpu_baseline(self):
+        rows = min(self.M, 16)
+        t0 = time.perf_counter()
+        orc.qmm_perblock(np.ascontiguousarray(self.inp["x1"][:rows]), self.inp["x2"], orc.I8, orc.I8, rows, self.K, self.N, False, True,
+                         np.ascontiguousarray(self.inp["s1"][:rows]), self.inp["s2"], 1, 128, 128, self.inp["bias"], orc.BF16)
         t = time.perf_counter() - t0
         return {"value": self.bytes * rows / self.M / t / 1e9, "unit": "GB/s", "cores": _cores(), "kind": "port",
                 "sample": f"first {rows} of {self.M} rows of x1 against the full x2 (oracle/liboracle.so, OpenMP), {t:.2f} s"}
@@ -543,6 +597,8 @@ def make_workload(m, config, args):
         return Config4Rows(m, args)
     if config == 13:
         return ConfigA8W4Rows(m, args)
+    if config == 14:
+        return ConfigPerTileRows(m, args)
     if config == 5:
         return Config5(m, args)
     raise SystemExit(f"bench.py: config {config} is not wired up yet")
