@@ -12,6 +12,7 @@
 #include <memory>
 
 #include "aclnnop/aclnn_quant_matmul_v5.h"
+#include "launch.h"
 #include "tensor.h"
 
 using namespace opsnn;
@@ -761,6 +762,8 @@ extern "C" aclnnStatus aclnnQuantMatmulV5(void* workspace, uint64_t workspaceSiz
     ex->qmm.workspace = ex->workspace_size ? workspace : nullptr;
     if (!ex->qmm.x1.ptr || !ex->qmm.x2.ptr || !ex->qmm.out) INVALID("aclnnQuantMatmulV5: a tensor has no device address");
     int rc = 0;
+    // a FRACTAL_NZ x2 is re-written into the workspace on every call: an address the weight cache must not key on
+    WeightCacheScope cache_scope(ex->nz.active);
     if (ex->nz.active) {   // x2 arrived in FRACTAL_NZ (aclnnQuantMatmulWeightNz): lay it out as ND in the front of the workspace
         const void* nd = nullptr;
         void* rest = nullptr;

@@ -11,6 +11,7 @@
 #include "aclnnop/aclnn_weight_quant_batch_matmul_v2.h"
 #include "aclnnop/aclnn_weight_quant_batch_matmul_v3.h"
 #include "aclnnop/aclnn_weight_quant_batch_matmul_nz.h"
+#include "launch.h"
 #include "tensor.h"
 
 using namespace opsnn;
@@ -198,6 +199,8 @@ aclnnStatus run(const char* api, void* workspace, uint64_t workspaceSize, aclOpE
         INVALID("%s: workspace of %lu bytes required", api, (unsigned long)ex->workspace_size);
     ex->wqmm.workspace = ex->workspace_size ? workspace : nullptr;
     if (!ex->wqmm.x || !ex->wqmm.w.ptr || !ex->wqmm.y || !ex->wqmm.scale.ptr) INVALID("%s: a tensor has no device address", api);
+    // a FRACTAL_NZ weight is re-written into the workspace on every call: an address the weight cache must not key on
+    WeightCacheScope cache_scope(ex->nz.active);
     if (ex->nz.active) {   // weight arrived in FRACTAL_NZ (aclnnWeightQuantBatchMatmulNz): lay it out as ND in the front of the workspace
         const void* nd = nullptr;
         void* rest = nullptr;

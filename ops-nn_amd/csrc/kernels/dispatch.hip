@@ -161,6 +161,7 @@ extern "C" __attribute__((visibility("hidden"))) int opsnn_qmm_k_pad(const Opsnn
 
 extern "C" int opsnnQmmBlockScale(const OpsnnQmmArgs* a, void* stream)
 {
+    WeightCacheScope cache_scope;
     if (!qmm_args_ok(a) || !a->x1_scale_mat.ptr || !a->x2_scale_mat.ptr) return -1;
     if (a->force_variant != OPSNN_VARIANT_PLAIN && !opsnn_force_plain()) {
         OpsnnQmmArgs b;
@@ -179,6 +180,7 @@ extern "C" int opsnnQmmBlockScale(const OpsnnQmmArgs* a, void* stream)
 
 extern "C" int opsnnQmmMx(const OpsnnQmmArgs* a, void* stream)
 {
+    WeightCacheScope cache_scope;
     if (!qmm_args_ok(a) || !a->x1_scale_mat.ptr || !a->x2_scale_mat.ptr) return -1;
     if (a->force_variant != OPSNN_VARIANT_PLAIN && !opsnn_force_plain()) {
         int rc = launch_mx_mfma(*a, (hipStream_t)stream);
@@ -195,6 +197,7 @@ extern "C" int opsnnQmmMx(const OpsnnQmmArgs* a, void* stream)
 extern "C" __attribute__((visibility("hidden"))) int opsnn_qmm_int8_impl(const OpsnnQmmArgs* a, void* stream);   // qmm_int8.hip
 extern "C" int opsnnQmmTc(const OpsnnQmmArgs* a, void* stream)
 {
+    WeightCacheScope cache_scope;
     if (!qmm_args_ok(a) || !a->x2_scale) return -1;
     const bool i8 = a->x1_dtype == DT_I8 && a->x2_dtype == DT_I8;
     const bool f8 = (a->x1_dtype == DT_E4M3 || a->x1_dtype == DT_E5M2) && (a->x2_dtype == DT_E4M3 || a->x2_dtype == DT_E5M2);
@@ -258,6 +261,7 @@ extern "C" int opsnnQmmTc(const OpsnnQmmArgs* a, void* stream)
 
 extern "C" int opsnnQmmGroup(const OpsnnQmmArgs* a, void* stream)
 {
+    WeightCacheScope cache_scope;
     if (!qmm_args_ok(a) || a->batch != 1 || a->gsK <= 0 || !a->x2_scale_mat.ptr) return -1;
     const bool tcg = a->x1_dtype == DT_E4M3 && a->x2_dtype == DT_E2M1;
     const bool i4 = a->x1_dtype == DT_I4 && a->x2_dtype == DT_I4;
@@ -284,6 +288,7 @@ extern "C" int opsnnQmmGroup(const OpsnnQmmArgs* a, void* stream)
 
 extern "C" int opsnnWqmm(const OpsnnWqmmArgs* a, void* stream)
 {
+    WeightCacheScope cache_scope;
     if (!a || !a->x || !a->w.ptr || !a->scale.ptr || !a->y || a->M <= 0 || a->N <= 0 || a->K <= 0) return -1;
     if (a->force_variant != OPSNN_VARIANT_PLAIN && !opsnn_force_plain()) {
         int rc = launch_wqmm_mfma(*a, (hipStream_t)stream);

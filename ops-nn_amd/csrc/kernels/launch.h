@@ -18,3 +18,20 @@ enum {
     OPSNN_VARIANT_MX_128 = 16,    // MX MFMA, 128x128 tile
     OPSNN_VARIANT_MX_FP8_MFMA = 17,  // MXFP8 on the MFMA path (reduced accumulation precision, see qmm_mx.hip)
 };
+
+#ifdef __cplusplus
+namespace opsnn {
+// Opened by every exported matmul entry point for the time it enqueues its launches (weight_cache.hip): copies that the
+// weight cache hands out inside the scope cannot be evicted before it closes; bypass = true switches the cache off for
+// this thread while the scope is open.  Scopes nest; the pins drop when the outermost one closes.
+class WeightCacheScope {
+public:
+    explicit WeightCacheScope(bool bypass = false);
+    ~WeightCacheScope();
+    WeightCacheScope(const WeightCacheScope&) = delete;
+    WeightCacheScope& operator=(const WeightCacheScope&) = delete;
+private:
+    bool saved_bypass_;
+};
+}  // namespace opsnn
+#endif

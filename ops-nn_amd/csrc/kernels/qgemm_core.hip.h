@@ -56,6 +56,10 @@ struct QgemmParams {
     const uint8_t* sa;
     const uint8_t* sb;
     int64_t sa_rs, sb_rs, sa_bs, sb_bs;
+    // When set: the launch computes only if one of gate[0 .. gate_n) is non-zero (the flags of the pass that prepares the
+    // exact MX route, whose kernel then left the call to this one); otherwise every workgroup returns at once.
+    const int* gate;
+    int gate_n;
 #if QG_DBG
     unsigned long long* dbg;
 #endif
@@ -123,6 +127,13 @@ __global__ __launch_bounds__(WGM* WGN * 64, MINWG) void qgemm_kernel(QgemmParams
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave / WGN, wn = wave % WGN;
+    if constexpr (MX) {
+        if (p.gate) {
+            int f = 0;
+            for (int i = tid; i < p.gate_n; i += NT) f |= p.gate[i];
+            if (!__syncthreads_or(f)) return;
+        }
+    }
 
     // tile id: XCD-contiguous, m fastest so that one XCD works on few x2 panels at a time
     const uint32_t t = xcd_remap(blockIdx.x, (uint32_t)(tiles_m * tiles_n));

@@ -576,12 +576,12 @@ int launch_fp8_rowcol_mfma(const OpsnnQmmArgs& a, hipStream_t st, bool merged_sc
     // both scales one element and no bias is the double-scale mode whose scales are merged and truncated: plain kernel
     // (callers whose scales are not that mode's say so)
     if (!merged_scales_ok && a.x1_scale_len == 1 && a.x2_scale_len == 1 && !a.bias) return OPSNN_NOT_TAKEN;
-    if (a.bias && a.bias_dtype != DT_F32) return OPSNN_NOT_TAKEN;
     if (a.K % 128 != 0 || a.M * a.N < 64 * 64 || a.x1.col_stride != 1 || a.x2.row_stride != 1) return OPSNN_NOT_TAKEN;
-    if (!opsnnGetFp8Fast()) {   // exact products and sums unless the caller asked for the 8-bit matrix instruction
+    if (!opsnnGetFp8Fast() || (a.bias && a.bias_dtype != DT_F32)) {   // exact products and sums unless the caller asked for the 8-bit matrix instruction (whose epilogue takes an fp32 bias only)
         const int rc = launch_rowcol_exact(a, st, 0);
         if (rc != OPSNN_NOT_TAKEN) return rc;
     }
+    if (a.bias && a.bias_dtype != DT_F32) return OPSNN_NOT_TAKEN;
     Fp8BlkParams p{};
     p.a = (const int8_t*)a.x1.ptr; p.b = (const int8_t*)a.x2.ptr;
     p.lda = a.x1.row_stride; p.ldb = a.x2.col_stride; p.a_bs = a.x1.batch_stride; p.b_bs = a.x2.batch_stride;

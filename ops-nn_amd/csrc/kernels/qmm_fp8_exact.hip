@@ -46,8 +46,22 @@ struct Fp8xParams {
     const void* cs;
     int rs_stride, cs_stride;
     int cs_dt, ep_mode;
-    const float* bias;
+    const void* bias;   // fp32, or 16-bit floats widened on the way in (bias_dt)
+    int bias_dt;
     int64_t bias_bs;
+    int64_t rs_bs, cs_bs;   // batch strides of rs / cs in elements (0: shared by all batches)
+    // MX mode (template flag MXS): one e8m0 byte per 32 K and row, four per K tile (sa, sb: K-contiguous, 4-byte aligned
+    // rows).  Every row has a base exponent; the widening conversion multiplies a block by 2^(byte - base), exactly (the
+    // result is an fp16 value as long as byte - base is in [-15, 7]), and 2^(base - 127) comes back in through rs / cs.
+    // a_c / b_c hold 127 - base per row; gate[0 .. gate_n) are flags of the pass that chose the bases: any flag set means
+    // some row's bytes do not fit that window, and the kernel leaves the whole call to the launch that follows it.
+    const uint8_t* sa;
+    const uint8_t* sb;
+    int64_t sa_rs, sb_rs, sa_bs, sb_bs;
+    const int* a_c;
+    const int* b_c;
+    const int* gate;
+    int gate_n;
 #if QG_DBG
     unsigned long long* dbg;   // timing harness only: per wave, loop clocks / barrier-wait clocks / K tiles
 #endif
@@ -78,20 +92,31 @@ template <bool E5> __device__ __forceinline__ v8h widen8(int d0, int d1)
     return (v8h){a[0], a[1], b[0], b[1], c[0], c[1], d[0], d[1]};
 }
 
+// the same with the power of two `sc` multiplied in (e4m3 only): exact while the scaled value is an fp16 value
+__device__ __forceinline__ v8h widen8_scaled(int d0, int d1, float sc)
+{
+    const v2h a = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8((uint32_t)d0, sc, false), b = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8((uint32_t)d0, sc, true);
+    const v2h c = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8((uint32_t)d1, sc, false), d = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8((uint32_t)d1, sc, true);
+    return (v8h){a[0], a[1], b[0], b[1], c[0], c[1], d[0], d[1]};
+}
+
 // FMT: bit 0 set = x1 holds e5m2 codes, bit 1 set = x2 does (else e4m3)
-template <int OUT_DT, bool RC, int FMT = 0>
+// MXS: MX block scales (e8m0 per 32 K) folded into the widening conversion; row / column epilogue (RC) with the bases
+template <int OUT_DT, bool RC, int FMT = 0, bool MXS = false>
 __global__ __launch_bounds__(512, 1) void qmm_fp8_exact_kernel(Fp8xParams p, int tiles_m, int tiles_n)
 {
+    static_assert(!MXS || (RC && FMT == 0), "the MX mode is e4m3 x e4m3 with the row / column epilogue");
     constexpr bool AE5 = (FMT & 1) != 0, BE5 = (FMT & 2) != 0;
     constexpr int BM = 256, BN = 128, BK = 128, NT = 512;
     constexpr int CPR = BK / 16, RPW = 16 / CPR;
     constexpr int TM = 64, TN = 64, FM = TM / 16, FN = TN / 16;
     constexpr int A_BYTES = BM * BK, B_BYTES = BN * BK;
-    constexpr int SC_BYTES = RC ? 0 : NT * 4;        // BM s1 floats + the s2 float of the tile's n block, one 4-byte copy per lane
+    constexpr bool SCC = !RC || MXS;                 // a 4-byte copy per lane rides with every K tile
+    constexpr int SC_BYTES = SCC ? NT * 4 : 0;       // block scales: BM s1 floats + the s2 float of the tile's n block; MX: four e8m0 bytes per tile row
     constexpr int STAGE = A_BYTES + B_BYTES + SC_BYTES;
     constexpr int RPI = NT / CPR;                    // 64 tile rows per copy instruction of the workgroup
     constexpr int NA = BM / RPI, NB = BN / RPI;
-    constexpr int CPT = NA + NB + (RC ? 0 : 1);
+    constexpr int CPT = NA + NB + (SCC ? 1 : 0);
     // Three stages: the tile being consumed, the next one (complete at this tile's barrier) and one more in flight, so a
     // copy has two tile times to land.  With two stages a copy had one tile time, about 1.1 us of matrix work, and the
     // loaded latency of an L2 miss is longer: the loop ran at the pace of the memory latency (measured: copies and
@@ -103,6 +128,11 @@ __global__ __launch_bounds__(512, 1) void qmm_fp8_exact_kernel(Fp8xParams p, int
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave >> 1, wn = wave & 1;
+    if constexpr (MXS) {
+        int f = 0;
+        for (int i = tid; i < p.gate_n; i += NT) f |= p.gate[i];
+        if (__syncthreads_or(f)) return;   // some row's scale bytes do not fit the exact window: the next launch computes the call
+    }
 
     // Tile order: each XCD (own L2) gets a contiguous range of ids, and ids run down groups of GM row tiles and across
     // the columns inside a group, so the 32 tiles an XCD works on at a time form a GM x (32 / GM) block that shares
@@ -141,16 +171,25 @@ __global__ __launch_bounds__(512, 1) void qmm_fp8_exact_kernel(Fp8xParams p, int
         b_off[i] = (uint32_t)(r * ldb + cchunk * 16);
     }
     // scale copy: lanes 0..255 fetch s1 of tile row `tid`, the others the s2 of this tile's n block
-    const float* sc_src = nullptr;
-    int64_t sc_step = 0;
-    if constexpr (!RC) {
+    const char* sc_src = nullptr;
+    int64_t sc_step = 0;   // bytes per K tile
+    if constexpr (MXS) {   // lanes 0..255: the four bytes of x1 row `tid`; the others: of x2 row tid - 256 (the last 128 lanes repeat the last row)
         if (tid < BM) {
             const int r = tid < a_rows ? tid : a_rows - 1;
-            sc_src = p.s1 + bz * p.s1_bs + ((m0 + r) / p.gsM) * p.s1_rs;
-            sc_step = p.s1_cs;
+            sc_src = (const char*)(p.sa + bz * p.sa_bs + (m0 + r) * p.sa_rs);
         } else {
-            sc_src = p.s2 + bz * p.s2_bs + (n0 / 128) * p.s2_cs;
-            sc_step = p.s2_rs;
+            const int r = tid - BM < b_rows ? tid - BM : b_rows - 1;
+            sc_src = (const char*)(p.sb + bz * p.sb_bs + (n0 + r) * p.sb_rs);
+        }
+        sc_step = 4;
+    } else if constexpr (!RC) {
+        if (tid < BM) {
+            const int r = tid < a_rows ? tid : a_rows - 1;
+            sc_src = (const char*)(p.s1 + bz * p.s1_bs + ((m0 + r) / p.gsM) * p.s1_rs);
+            sc_step = p.s1_cs * 4;
+        } else {
+            sc_src = (const char*)(p.s2 + bz * p.s2_bs + (n0 / 128) * p.s2_cs);
+            sc_step = p.s2_rs * 4;
         }
     }
     auto issue_piece = [&](int kt, int stage, int idx) {
@@ -202,30 +241,79 @@ __global__ __launch_bounds__(512, 1) void qmm_fp8_exact_kernel(Fp8xParams p, int
     float sc[FM], scp[FM], s1raw[FM], s2raw = 0.0f;
     v4f part[2][FM];
     (void)sc; (void)scp; (void)s1raw; (void)s2raw; (void)part;
+    // MX: raw scale dwords of the tile being converted (one per fragment row of this lane), 127 - base of those rows, and
+    // the powers of two for the lane's two K blocks of a tile: bytes [16q, 16q+16) lie in block q/2, [64+16q, ..) in 2 + q/2
+    uint32_t a_sraw[FM], b_sraw[FN];
+    int a_c[FM], b_c[FN];
+    float a_lo[FM], a_hi[FM], b_lo[FN], b_hi[FN];
+    (void)a_sraw; (void)b_sraw; (void)a_c; (void)b_c; (void)a_lo; (void)a_hi; (void)b_lo; (void)b_hi;
+    const int sblk = 8 * (fq >> 1);
+    if constexpr (MXS) {
+#pragma unroll
+        for (int j = 0; j < FM; j++) {
+            const int r = wm * TM + j * 16 + frow;
+            a_c[j] = p.a_c[bz * p.rs_bs + m0 + (r < a_rows ? r : a_rows - 1)];
+        }
+#pragma unroll
+        for (int i = 0; i < FN; i++) {
+            const int r = wn * TN + i * 16 + frow;
+            b_c[i] = p.b_c[bz * p.cs_bs + n0 + (r < b_rows ? r : b_rows - 1)];
+        }
+    }
+    auto mx_pow = [&](uint32_t raw, int c, float& lo, float& hi) {
+        lo = u2f((((raw >> sblk) & 0xFFu) + (uint32_t)c) << 23);
+        hi = u2f((((raw >> (16 + sblk)) & 0xFFu) + (uint32_t)c) << 23);
+    };
     auto read_scales = [&](const char* st) {
-        if constexpr (!RC) {
+        if constexpr (MXS) {
+            const uint32_t* sS = (const uint32_t*)(st + A_BYTES + B_BYTES);
+#pragma unroll
+            for (int j = 0; j < FM; j++) a_sraw[j] = sS[wm * TM + j * 16 + frow];
+#pragma unroll
+            for (int i = 0; i < FN; i++) b_sraw[i] = sS[BM + wn * TN + i * 16 + frow];
+        } else if constexpr (!RC) {
             const float* sS = (const float*)(st + A_BYTES + B_BYTES);
             s2raw = sS[BM];
 #pragma unroll
             for (int j = 0; j < FM; j++) s1raw[j] = sS[wm * TM + j * 16 + frow];
         }
     };
-    auto widen4 = [&](int d, v8h& h, int half) {   // four bytes -> elements 4*half .. 4*half+3
-        const v2h lo = cvt_lo<BE5>((uint32_t)d), hi = cvt_hi<BE5>((uint32_t)d);
+    auto widen4 = [&](int d, v8h& h, int half, float scl) {   // four bytes -> elements 4*half .. 4*half+3
+        v2h lo, hi;
+        if constexpr (MXS) {
+            lo = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8((uint32_t)d, scl, false);
+            hi = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8((uint32_t)d, scl, true);
+        } else {
+            lo = cvt_lo<BE5>((uint32_t)d); hi = cvt_hi<BE5>((uint32_t)d);
+        }
         h[4 * half] = lo[0]; h[4 * half + 1] = lo[1]; h[4 * half + 2] = hi[0]; h[4 * half + 3] = hi[1];
+    };
+    auto widen_a = [&](int d0, int d1, int j, int s) -> v8h {   // K step s of x1 fragment j
+        if constexpr (MXS) return widen8_scaled(d0, d1, s < 2 ? a_lo[j] : a_hi[j]);
+        else return widen8<AE5>(d0, d1);
     };
     {   // first tile: everything converted up front
         read_scales(smem);
+        if constexpr (MXS) {
+#pragma unroll
+            for (int j = 0; j < FM; j++) {
+                mx_pow(a_sraw[j], a_c[j], a_lo[j], a_hi[j]);
+                mx_pow(b_sraw[j], b_c[j], b_lo[j], b_hi[j]);
+            }
+        }
 #pragma unroll
         for (int j = 0; j < FM; j++) {
             const v8i r = load_frag(smem, a_rowbase + j * 16 * BK);
 #pragma unroll
-            for (int s = 0; s < 4; s++) fa[j][s] = widen8<AE5>(r[2 * s], r[2 * s + 1]);
+            for (int s = 0; s < 4; s++) fa[j][s] = widen_a(r[2 * s], r[2 * s + 1], j, s);
             a_half[j] = __builtin_shufflevector(r, r, 4, 5, 6, 7);   // converted once more behind the first instructions (same values)
         }
         b_raw = load_frag(smem, b_rowbase);
 #pragma unroll
-        for (int s = 0; s < 4; s++) fbc[0][s] = widen8<BE5>(b_raw[2 * s], b_raw[2 * s + 1]);
+        for (int s = 0; s < 4; s++) {
+            if constexpr (MXS) fbc[0][s] = widen8_scaled(b_raw[2 * s], b_raw[2 * s + 1], s < 2 ? b_lo[0] : b_hi[0]);
+            else fbc[0][s] = widen8<BE5>(b_raw[2 * s], b_raw[2 * s + 1]);
+        }
 #pragma unroll
         for (int j = 0; j < FM; j++) {
             sc[j] = 0.0f;   // multiplies the zero partial sums folded during the first tile's first fragment
@@ -297,14 +385,24 @@ __global__ __launch_bounds__(512, 1) void qmm_fp8_exact_kernel(Fp8xParams p, int
                         if (i > 0) acc[i - 1][s][j] = __builtin_fmaf(part[(i - 1) & 1][s][j], sc[s], acc[i - 1][s][j]);
                         else acc[FN - 1][s][j] = __builtin_fmaf(part[1][s][j], scp[s], acc[FN - 1][s][j]);
                     }
+                    if constexpr (MXS) {
+                        // the next tile's scale bytes were requested behind the barrier; every conversion that used the
+                        // current tile's has been issued (x2 fragments 1 .. FN-1 during the earlier fragments, the x1 high
+                        // halves during the first)
+                        if (i == FN - 1 && s == 1) {
+                            mx_pow(a_sraw[j], a_c[j], a_lo[j], a_hi[j]);
+                            mx_pow(b_sraw[j], b_c[j], b_lo[j], b_hi[j]);
+                        }
+                    }
                     if (s >= 2) {   // next x2 fragment: half a K step per instruction
                         const int idx = (s - 2) * 4 + j;
-                        widen4(b_raw[idx], fbc[(i + 1) & 1][idx / 2], idx % 2);
+                        const int nf = (i + 1) % FN;
+                        widen4(b_raw[idx], fbc[(i + 1) & 1][idx / 2], idx % 2, idx / 2 < 2 ? b_lo[nf] : b_hi[nf]);
                     }
                     if (i == FN - 1 && s >= 2)                // next tile's x1 fragments, K step s - 2 (low halves)
-                        fa[j][s - 2] = widen8<AE5>(a_half[j][2 * (s - 2)], a_half[j][2 * (s - 2) + 1]);
+                        fa[j][s - 2] = widen_a(a_half[j][2 * (s - 2)], a_half[j][2 * (s - 2) + 1], j, s - 2);
                     if (i == 0 && (s == 1 || s == 2))         // this tile's x1 fragments, K steps 2 and 3 (high halves)
-                        fa[j][1 + s] = widen8<AE5>(a_half[j][2 * (s - 1)], a_half[j][2 * (s - 1) + 1]);
+                        fa[j][1 + s] = widen_a(a_half[j][2 * (s - 1)], a_half[j][2 * (s - 1) + 1], j, 1 + s);
                     __builtin_amdgcn_sched_barrier(0);
                 }
                 if (i == FN - 1) {
@@ -354,7 +452,7 @@ __global__ __launch_bounds__(512, 1) void qmm_fp8_exact_kernel(Fp8xParams p, int
 #pragma unroll
         for (int j = 0; j < FM; j++) {
             const int64_t mrow = m0 + wm * TM + j * 16 + frow;
-            rs_j[j] = p.rs ? p.rs[(mrow < p.M ? mrow : p.M - 1) * p.rs_stride] : 1.0f;
+            rs_j[j] = p.rs ? p.rs[bz * p.rs_bs + (mrow < p.M ? mrow : p.M - 1) * p.rs_stride] : 1.0f;
         }
     }
 #pragma unroll
@@ -367,19 +465,19 @@ __global__ __launch_bounds__(512, 1) void qmm_fp8_exact_kernel(Fp8xParams p, int
 #pragma unroll
                 for (int r = 0; r < 4; r++) {
                     const int64_t ni = nb + r < p.N ? nb + r : p.N - 1;
-                    const int64_t ci = ni * p.cs_stride;
+                    const int64_t ci = bz * p.cs_bs + ni * p.cs_stride;
                     float csv;
                     if (p.cs_dt == DT_U64) csv = u2f((uint32_t)((const uint64_t*)p.cs)[ci] & 0xFFFFE000u);
                     else if (p.cs_dt == DT_BF16) csv = bf16_to_f32(((const uint16_t*)p.cs)[ci]);
                     else csv = ((const float*)p.cs)[ci];
                     if (p.ep_mode == 1) {
-                        if (p.bias) v[r] = v[r] + p.bias[bz * p.bias_bs + ni];
+                        if (p.bias) v[r] = v[r] + load_scalar_as_f32(p.bias, p.bias_dt, bz * p.bias_bs + ni);
                         v[r] = v[r] * csv;
                     } else if (p.ep_mode == 2) {
                         v[r] = v[r] * u2f(f2u(csv * rs_j[j]) & 0xFFFFE000u);
                     } else {
                         v[r] = (v[r] * csv) * rs_j[j];
-                        if (p.bias) v[r] = v[r] + p.bias[bz * p.bias_bs + ni];
+                        if (p.bias) v[r] = v[r] + load_scalar_as_f32(p.bias, p.bias_dt, bz * p.bias_bs + ni);
                     }
                 }
             }
@@ -420,13 +518,13 @@ __global__ __launch_bounds__(512, 1) void qmm_fp8_exact_kernel(Fp8xParams p, int
     }
 }
 
-template <int OUT_DT, bool RC, int FMT = 0>
+template <int OUT_DT, bool RC, int FMT = 0, bool MXS = false>
 static int launch_fp8_exact(const Fp8xParams& p, int64_t batch, hipStream_t st)
 {
     const int tiles_m = (int)((p.M + 255) / 256), tiles_n = (int)((p.N + 127) / 128);
     dim3 grid((unsigned)(tiles_m * tiles_n), (unsigned)batch);
-    const size_t lds = 3 * (size_t)(256 * 128 + 128 * 128 + (RC ? 0 : 512 * 4));
-    auto k = qmm_fp8_exact_kernel<OUT_DT, RC, FMT>;
+    const size_t lds = 3 * (size_t)(256 * 128 + 128 * 128 + ((RC && !MXS) ? 0 : 512 * 4));
+    auto k = qmm_fp8_exact_kernel<OUT_DT, RC, FMT, MXS>;
     static bool attr_set = false;
     if (!attr_set) {
         hipError_t e = hipFuncSetAttribute((const void*)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
@@ -472,7 +570,7 @@ int launch_rowcol_exact(const OpsnnQmmArgs& a, hipStream_t st, int ep_mode)
     if (a.out_dtype != DT_BF16 && a.out_dtype != DT_F16 && a.out_dtype != DT_F32) return OPSNN_NOT_TAKEN;
     if (!a.x2_scale || (a.x2_scale_dtype != DT_F32 && a.x2_scale_dtype != DT_BF16 && a.x2_scale_dtype != DT_U64)) return OPSNN_NOT_TAKEN;
     if (ep_mode != 1 && !a.x1_scale) return OPSNN_NOT_TAKEN;
-    if (a.bias && a.bias_dtype != DT_F32) return OPSNN_NOT_TAKEN;
+    if (a.bias && a.bias_dtype != DT_F32 && a.bias_dtype != DT_BF16 && a.bias_dtype != DT_F16) return OPSNN_NOT_TAKEN;
     if (a.K % 128 != 0 || a.M * a.N < 64 * 64 || a.x1.col_stride != 1 || a.x2.row_stride != 1) return OPSNN_NOT_TAKEN;
     Fp8xParams p{};
     p.a = (const int8_t*)a.x1.ptr; p.b = (const int8_t*)a.x2.ptr;
@@ -481,7 +579,7 @@ int launch_rowcol_exact(const OpsnnQmmArgs& a, hipStream_t st, int ep_mode)
     p.rs = ep_mode == 1 ? nullptr : (const float*)a.x1_scale; p.rs_stride = a.x1_scale_len == 1 ? 0 : 1;
     p.cs = a.x2_scale; p.cs_stride = a.x2_scale_len == 1 ? 0 : 1; p.cs_dt = a.x2_scale_dtype;
     p.ep_mode = ep_mode;
-    p.bias = (const float*)a.bias; p.bias_bs = a.bias_batch_stride;
+    p.bias = a.bias; p.bias_dt = a.bias_dtype; p.bias_bs = a.bias_batch_stride;
     if (((uintptr_t)p.a | (uintptr_t)p.b | (uint64_t)p.lda | (uint64_t)p.ldb | (uint64_t)p.a_bs | (uint64_t)p.b_bs) % 16) return OPSNN_NOT_TAKEN;
     const bool bf = a.out_dtype == DT_BF16, f32 = a.out_dtype == DT_F32;
     switch ((e1 ? 1 : 0) | (e2 ? 2 : 0)) {
@@ -490,6 +588,110 @@ int launch_rowcol_exact(const OpsnnQmmArgs& a, hipStream_t st, int ep_mode)
         case 2: return f32 ? launch_fp8_exact<DT_F32, true, 2>(p, a.batch, st) : bf ? launch_fp8_exact<DT_BF16, true, 2>(p, a.batch, st) : launch_fp8_exact<DT_F16, true, 2>(p, a.batch, st);
         default: return f32 ? launch_fp8_exact<DT_F32, true, 3>(p, a.batch, st) : bf ? launch_fp8_exact<DT_BF16, true, 3>(p, a.batch, st) : launch_fp8_exact<DT_F16, true, 3>(p, a.batch, st);
     }
+}
+
+// ---- MX (e8m0 scale per 32 K) on exact products ----
+// Per row of a scale table [rows, K/32] (K-contiguous, nd = K/128 dwords per row): base = max byte - 7, c = 127 - base and
+// 2^(base - 127).  With byte - base in [-15, 7] an e4m3 value times 2^(byte - base) is an fp16 value (largest 448 * 2^7,
+// smallest 2^-9 * 2^-15 = 2^-24).  flags[block] = 1 when one of the block's rows holds a byte below max - 22 or the NaN
+// code 255.  One wave per row at a time, 64 rows per workgroup.
+__global__ __launch_bounds__(256) void mx_row_base_kernel(const uint8_t* __restrict__ s, int64_t rs, int64_t bs, int64_t rows, int64_t total, int nd,
+                                                          int* __restrict__ c_out, float* __restrict__ pow_out, int* __restrict__ flags)
+{
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    int bad = 0;
+    for (int i = 0; i < 16; i++) {
+        const int64_t r = (int64_t)blockIdx.x * 64 + wave * 16 + i;
+        if (r >= total) break;
+        const uint32_t* row = (const uint32_t*)(s + (r / rows) * bs + (r % rows) * rs);
+        uint32_t mn = 255, mx = 0;
+        for (int d = lane; d < nd; d += 64) {
+            const uint32_t w = row[d];
+#pragma unroll
+            for (int b = 0; b < 4; b++) {
+                const uint32_t v = (w >> (8 * b)) & 0xFFu;
+                mn = v < mn ? v : mn;
+                mx = v > mx ? v : mx;
+            }
+        }
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) {
+            const uint32_t a = (uint32_t)__shfl_xor((int)mn, o), b = (uint32_t)__shfl_xor((int)mx, o);
+            mn = a < mn ? a : mn;
+            mx = b > mx ? b : mx;
+        }
+        const int base = (int)mx - 7;
+        if (lane == 0) {
+            c_out[r] = 127 - base;
+            pow_out[r] = ldexpf(1.0f, base - 127);
+        }
+        bad |= (mx == 255u || mx - mn > 22u) ? 1 : 0;
+    }
+    const int any = __syncthreads_or(bad);
+    if (threadIdx.x == 0) flags[blockIdx.x] = any ? 1 : 0;
+}
+
+static inline uint64_t up256(uint64_t v) { return (v + 255) / 256 * 256; }
+
+// Bytes of workspace the exact MXFP8 route wants in front of everything else: 127 - base and 2^(base - 127) per row of
+// both operands, and the flags.
+uint64_t mx_exact_bytes(const OpsnnQmmArgs& a)
+{
+    if (a.x1_dtype != DT_E4M3 || a.x2_dtype != DT_E4M3) return 0;
+    if (a.M <= 0 || a.N <= 0 || a.K < 64 || a.batch <= 0) return 0;
+    const uint64_t rows = (uint64_t)a.batch * (uint64_t)(a.M + a.N);
+    return up256(rows * 8) + up256(((rows + 63) / 64 + 2) * 4);
+}
+
+// MXFP8 with exact products: the bases pass, this kernel, and -- computing
+// only when a flag is set -- the tile kernel on the scaled 8-bit instruction.  `a`: both operands e4m3, K-contiguous,
+// K % 128 == 0, scale rows K-contiguous; `region`: mx_exact_bytes(a) bytes.  OPSNN_NOT_TAKEN before anything is launched.
+int launch_mx_exact(const OpsnnQmmArgs& a, void* region, hipStream_t st)
+{
+    if (!region || (uintptr_t)region % 16) return OPSNN_NOT_TAKEN;
+    if (a.x1_dtype != DT_E4M3 || a.x2_dtype != DT_E4M3) return OPSNN_NOT_TAKEN;
+    if (a.out_dtype != DT_BF16 && a.out_dtype != DT_F16 && a.out_dtype != DT_F32) return OPSNN_NOT_TAKEN;
+    if (a.bias && a.bias_dtype != DT_F32 && a.bias_dtype != DT_BF16 && a.bias_dtype != DT_F16) return OPSNN_NOT_TAKEN;
+    if (a.K % 128 != 0 || a.M * a.N < 64 * 64 || a.x1.col_stride != 1 || a.x2.row_stride != 1) return OPSNN_NOT_TAKEN;
+    if (a.x1_scale_mat.col_stride != 2 || a.x2_scale_mat.col_stride != 2) return OPSNN_NOT_TAKEN;
+    const int64_t nb1 = a.x1_scale_mat.batch_stride == 0 ? 1 : a.batch, nb2 = a.x2_scale_mat.batch_stride == 0 ? 1 : a.batch;
+    Fp8xParams p{};
+    p.a = (const int8_t*)a.x1.ptr; p.b = (const int8_t*)a.x2.ptr;
+    p.lda = a.x1.row_stride; p.ldb = a.x2.col_stride; p.a_bs = a.x1.batch_stride; p.b_bs = a.x2.batch_stride;
+    p.out = a.out; p.M = a.M; p.N = a.N; p.K = a.K; p.gsM = 1;
+    p.sa = (const uint8_t*)a.x1_scale_mat.ptr; p.sb = (const uint8_t*)a.x2_scale_mat.ptr;
+    p.sa_rs = a.x1_scale_mat.row_stride; p.sb_rs = a.x2_scale_mat.row_stride;
+    p.sa_bs = a.x1_scale_mat.batch_stride; p.sb_bs = a.x2_scale_mat.batch_stride;
+    if (((uintptr_t)p.a | (uintptr_t)p.b | (uint64_t)p.lda | (uint64_t)p.ldb | (uint64_t)p.a_bs | (uint64_t)p.b_bs) % 16) return OPSNN_NOT_TAKEN;
+    if (((uintptr_t)p.sa | (uintptr_t)p.sb | (uint64_t)p.sa_rs | (uint64_t)p.sb_rs | (uint64_t)p.sa_bs | (uint64_t)p.sb_bs) % 4) return OPSNN_NOT_TAKEN;
+    const int64_t rows1 = nb1 * a.M, rows2 = nb2 * a.N;
+    const uint64_t all_rows = (uint64_t)a.batch * (uint64_t)(a.M + a.N);
+    int* c1 = (int*)region;
+    int* c2 = c1 + rows1;
+    float* pw1 = (float*)((char*)region + all_rows * 4);
+    float* pw2 = pw1 + rows1;
+    int* flags = (int*)((char*)region + up256(all_rows * 8));
+    const int g1 = (int)((rows1 + 63) / 64), g2 = (int)((rows2 + 63) / 64), nd = (int)(a.K / 128);
+    hipLaunchKernelGGL(mx_row_base_kernel, dim3((unsigned)g1), dim3(256), 0, st, p.sa, p.sa_rs, p.sa_bs, a.M, rows1, nd, c1, pw1, flags);
+    hipLaunchKernelGGL(mx_row_base_kernel, dim3((unsigned)g2), dim3(256), 0, st, p.sb, p.sb_rs, p.sb_bs, a.N, rows2, nd, c2, pw2, flags + g1);
+    p.a_c = c1; p.b_c = c2;
+    p.rs = pw1; p.rs_stride = 1; p.rs_bs = nb1 == 1 ? 0 : a.M;
+    p.cs = pw2; p.cs_stride = 1; p.cs_bs = nb2 == 1 ? 0 : a.N; p.cs_dt = DT_F32;
+    p.ep_mode = 0;
+    p.bias = a.bias; p.bias_dt = a.bias_dtype; p.bias_bs = a.bias_batch_stride;
+    p.gate = flags; p.gate_n = g1 + g2;
+    const int rc = a.out_dtype == DT_F32    ? launch_fp8_exact<DT_F32, true, 0, true>(p, a.batch, st)
+                   : a.out_dtype == DT_BF16 ? launch_fp8_exact<DT_BF16, true, 0, true>(p, a.batch, st)
+                                            : launch_fp8_exact<DT_F16, true, 0, true>(p, a.batch, st);
+    if (rc != 0) return rc;
+    QgemmParams g{};
+    g.a = p.a; g.b = p.b; g.lda = p.lda; g.ldb = p.ldb; g.a_bs = p.a_bs; g.b_bs = p.b_bs;
+    g.out = a.out; g.M = a.M; g.N = a.N; g.ldc = a.N; g.KB = a.K;
+    g.bias = a.bias; g.bias_dt = a.bias_dtype; g.bias_bs = a.bias_batch_stride;
+    g.sa = p.sa; g.sb = p.sb; g.sa_rs = p.sa_rs; g.sb_rs = p.sb_rs; g.sa_bs = p.sa_bs; g.sb_bs = p.sb_bs;
+    g.gate = flags; g.gate_n = g1 + g2;
+    if (a.M <= 128 || a.N <= 128) return qgemm_launch<MODE_MXFP8, 128, 128, 128, 2, 2, 2, 1>(g, a.batch, a.out_dtype, st);
+    return qgemm_launch<MODE_MXFP8, 256, 256, 128, 2, 2, 2, 1>(g, a.batch, a.out_dtype, st);
 }
 
 }  // namespace opsnn

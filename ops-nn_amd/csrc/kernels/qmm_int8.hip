@@ -94,6 +94,7 @@ extern "C" __attribute__((visibility("hidden"))) int opsnn_qmm_int8_impl(const O
 extern "C" __attribute__((visibility("hidden"))) int opsnn_qmm_k_pad(const OpsnnQmmArgs* a, int mode, void* stream, OpsnnQmmArgs* b);   // dispatch.hip
 extern "C" int opsnnQmmInt8(const OpsnnQmmArgs* a, void* stream)
 {
+    WeightCacheScope cache_scope;
     OpsnnQmmArgs padded;
     if (a && a->x1.ptr && a->x2.ptr && a->M > 0 && a->N > 0 && a->K > 0 && a->batch > 0) {
         const int prc = opsnn_qmm_k_pad(a, 0, stream, &padded);   // K % 16 != 0: zero-padded K-contiguous copies

@@ -50,6 +50,7 @@ extern "C" int opsnnQmmInt8Static(const OpsnnQmmArgs* a, void* stream)
                          (unsigned long long)need, (unsigned long long)OPSNN_STATIC_SCRATCH_BYTES);
         return OPSNN_ERR_SCRATCH_TOO_SMALL;
     }
+    opsnn::WeightCacheScope no_cache(true);   // a miss in the weight cache allocates, an eviction frees: not from this entry point
     OpsnnQmmArgs b = *a;
     b.workspace = nullptr;
     if (need) {

@@ -12,7 +12,14 @@
 // A copy is written on the stream of the call that misses; an event recorded behind it orders every later use on
 // any stream.  Nothing is cached (and the caller's workspace path runs) while the stream is being captured into a
 // graph, when the copy does not fit the limit, or when the allocation fails.  Entries are evicted least recently
-// used first; hipFree waits for the device, so no kernel can still be reading an evicted copy.
+// used first; hipFree waits for the device, so no kernel that is already enqueued can still be reading an evicted copy.
+// A call that has been handed a copy but has not enqueued its kernels yet is protected by a pin: every exported matmul
+// entry point opens a WeightCacheScope, each copy handed out inside it is pinned, and the pins drop when the scope
+// closes (all launches enqueued).  Pinned entries are never evicted; clearing the cache or lowering the limit takes a
+// pinned entry out of the table at once and frees it when its last pin drops.
+// A scope can also switch the cache off for its thread (WeightCacheScope(true)): the FRACTAL_NZ entry points, which
+// re-write the keyed memory -- the front of the caller's workspace -- on every call, and the entry point that promises to
+// allocate nothing.
 #include <cstdlib>
 #include <list>
 #include <mutex>
@@ -28,22 +35,87 @@ struct Entry {
     const void* src; const void* src2; const void* src3; int64_t K, N, nb; int bits;
     void* copy; uint64_t bytes; hipEvent_t ready; int device;
     bool committed;   // filled and its event recorded; until then other callers do not use it
+    int pins;         // calls that hold `copy` and may not have enqueued their kernels yet
 };
 
 std::mutex g_mu;
 std::list<Entry> g_entries;   // most recently used first
+std::list<Entry> g_zombies;   // taken out of the table while pinned: freed when the last pin drops
 uint64_t g_limit = [] { const char* e = getenv("OPSNN_WEIGHT_CACHE_MB"); return e ? (uint64_t)atoll(e) << 20 : (uint64_t)0; }();
 uint64_t g_used = 0, g_hits = 0, g_misses = 0;
 
-void drop(std::list<Entry>::iterator it)
+struct ThreadScope {
+    int depth = 0;
+    bool bypass = false;
+    void* pinned[8];
+    int n = 0;
+};
+thread_local ThreadScope t_scope;
+
+void release(const Entry& e)
 {
-    (void)hipEventDestroy(it->ready);
-    (void)hipFree(it->copy);
+    (void)hipEventDestroy(e.ready);
+    (void)hipFree(e.copy);
+}
+
+// Takes the entry out of the table (g_mu held); its memory goes at once unless a call still holds it.  Returns the
+// entry that followed it.
+std::list<Entry>::iterator drop(std::list<Entry>::iterator it)
+{
     g_used -= it->bytes;
-    g_entries.erase(it);
+    const auto next = std::next(it);
+    if (it->pins > 0) g_zombies.splice(g_zombies.begin(), g_entries, it);
+    else {
+        release(*it);
+        g_entries.erase(it);
+    }
+    return next;
+}
+
+// Pins the entry for the open scope of this thread (g_mu held).  False when no scope is open or it is full: the entry
+// is then not handed out.
+bool pin(Entry& e)
+{
+    ThreadScope& t = t_scope;
+    if (t.depth <= 0 || t.n >= (int)(sizeof(t.pinned) / sizeof(t.pinned[0]))) return false;
+    t.pinned[t.n++] = e.copy;
+    e.pins++;
+    return true;
+}
+
+void unpin_all()
+{
+    ThreadScope& t = t_scope;
+    if (!t.n) return;
+    std::lock_guard<std::mutex> lock(g_mu);
+    for (int i = 0; i < t.n; i++) {
+        bool found = false;
+        for (auto it = g_entries.begin(); it != g_entries.end() && !found; ++it)
+            if (it->copy == t.pinned[i]) { it->pins--; found = true; }
+        for (auto it = g_zombies.begin(); it != g_zombies.end() && !found; ++it)
+            if (it->copy == t.pinned[i]) {
+                found = true;
+                if (--it->pins <= 0) {
+                    release(*it);
+                    g_zombies.erase(it);
+                }
+            }
+    }
+    t.n = 0;
 }
 
 }  // namespace
+
+WeightCacheScope::WeightCacheScope(bool bypass) : saved_bypass_(t_scope.bypass)
+{
+    t_scope.depth++;
+    if (bypass) t_scope.bypass = true;
+}
+WeightCacheScope::~WeightCacheScope()
+{
+    t_scope.bypass = saved_bypass_;
+    if (--t_scope.depth == 0) unpin_all();
+}
 
 // A buffer of `bytes` that belongs to the operand (src, src2, src3 -- e.g. data, scales and offsets --, shape, element width,
 // batch count):
@@ -54,7 +126,7 @@ void* weight_cache_blob3(const void* src, const void* src2, const void* src3, in
                          bool* fresh)
 {
     *fresh = false;
-    if (!g_limit || !src || K <= 0 || N <= 0 || nb <= 0 || !bytes) return nullptr;
+    if (!g_limit || t_scope.bypass || t_scope.depth <= 0 || !src || K <= 0 || N <= 0 || nb <= 0 || !bytes) return nullptr;
     hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
     if (hipStreamIsCapturing(st, &cap) != hipSuccess || cap != hipStreamCaptureStatusNone) return nullptr;
     int dev = 0;
@@ -65,16 +137,24 @@ void* weight_cache_blob3(const void* src, const void* src2, const void* src3, in
             it->device == dev) {
             if (!it->committed) return nullptr;   // another call is still filling it: this one goes its own way
             if (hipStreamWaitEvent(st, it->ready, 0) != hipSuccess) return nullptr;
+            if (!pin(*it)) return nullptr;
             g_entries.splice(g_entries.begin(), g_entries, it);
             g_hits++;
             return it->copy;
         }
     }
     if (bytes > g_limit) return nullptr;
-    while (g_used + bytes > g_limit && !g_entries.empty()) drop(std::prev(g_entries.end()));
-    Entry e{src, src2, src3, K, N, nb, bits, nullptr, bytes, nullptr, dev, false};
+    // make room: least recently used first, skipping what a call still holds or is still filling
+    for (auto it = g_entries.end(); g_used + bytes > g_limit && it != g_entries.begin();) {
+        --it;
+        if (it->pins > 0 || !it->committed) continue;
+        it = drop(it);
+    }
+    if (g_used + bytes > g_limit) return nullptr;   // everything else is in use
+    Entry e{src, src2, src3, K, N, nb, bits, nullptr, bytes, nullptr, dev, false, 0};
     if (hipMalloc(&e.copy, bytes) != hipSuccess) { (void)hipGetLastError(); return nullptr; }
     if (hipEventCreateWithFlags(&e.ready, hipEventDisableTiming) != hipSuccess) { (void)hipFree(e.copy); return nullptr; }
+    if (!pin(e)) { release(e); return nullptr; }
     // until the commit nobody else uses the entry; one whose filling call fails is removed by weight_cache_abandon
     g_used += bytes;
     g_misses++;
@@ -130,7 +210,7 @@ extern "C" void opsnnSetWeightCache(int64_t max_bytes)
 {
     std::lock_guard<std::mutex> lock(g_mu);
     g_limit = max_bytes > 0 ? (uint64_t)max_bytes : 0;
-    while (g_used > g_limit && !g_entries.empty()) drop(std::prev(g_entries.end()));
+    while (g_used > g_limit && !g_entries.empty()) drop(std::prev(g_entries.end()));   // (pinned ones leave the table now and are freed by their holders)
 }
 
 extern "C" void opsnnWeightCacheClear(void)

@@ -367,11 +367,13 @@ def make_a8w4_mx_inputs(m, M, K, N, seed, tB):
     return dict(x1=x1, x2=x2, s1=s1, s2=s2, bias=bias)
 
 
-def oracle_a8w4_mx(m, inp, M, K, N, tB, out_dt):
-    return orc.qmm_mx(inp["x1"], inp["x2"], orc.E4M3, orc.E2M1, M, K, N, False, tB, inp["s1"], inp["s2"], orc.f16_to_f32(inp["bias"]), out_dt)
+def oracle_a8w4_mx(m, inp, M, K, N, tB, out_dt, bias_dt=None):
+    """inp["bias"] holds 16-bit patterns: fp16 unless bias_dt says bf16 (the mode wants the bias in the output's type)."""
+    bias = orc.bf16_to_f32(inp["bias"]) if bias_dt == orc.BF16 else orc.f16_to_f32(inp["bias"])
+    return orc.qmm_mx(inp["x1"], inp["x2"], orc.E4M3, orc.E2M1, M, K, N, False, tB, inp["s1"], inp["s2"], bias, out_dt)
 
 
-def run_a8w4_mx_aclnn(m, inp, M, K, N, tB, out_dt):
+def run_a8w4_mx_aclnn(m, inp, M, K, N, tB, out_dt, bias_dt=None):
     d = {k: m.DeviceBuffer(host=v) for k, v in inp.items()}
     out_np = orc.out_array((M, N), out_dt)
     d_out = m.DeviceBuffer(out_np.nbytes); d_out.fill(0xFF)
@@ -379,7 +381,7 @@ def run_a8w4_mx_aclnn(m, inp, M, K, N, tB, out_dt):
     x2 = m.Tensor((N, K) if tB else (K, N), m.ACL_FLOAT4_E2M1, d["x2"])
     s1 = m.Tensor(inp["s1"].shape, m.ACL_FLOAT8_E8M0, d["s1"])
     s2 = m.Tensor(inp["s2"].shape, m.ACL_FLOAT8_E8M0, d["s2"])
-    bias = m.Tensor((1, N), m.ACL_FLOAT16, d["bias"])
+    bias = m.Tensor((1, N), bias_dt if bias_dt is not None else m.ACL_FLOAT16, d["bias"])
     out = m.Tensor((M, N), out_dt, d_out)
     ws = m.quant_matmul_v5(x1, x2, s1, s2, out, bias=bias, transpose_x2=tB, group_size=32)
     m.check(m.lib().aclrtSynchronizeDevice(), "sync")

@@ -104,6 +104,36 @@ def test_config5_mxfp4_batched_full(gpu):
     _double_exactly(got, cases.run_mx_aclnn(m, inp2, M, K, N, True, m.ACL_BF16), m.ACL_BF16)
 
 
+# ---- the MX modes with fp8 operands, at sizes of the configs' class, BASELINE's distributions (e4m3 from N(0,1), scale
+# exponents uniform in [-4, 4]): the default route (exact fp16 products) at the stated bar ----
+@pytest.mark.parametrize("M,K,N", [(4096, 8192, 8192), (16, 8192, 28672)])
+def test_mxfp8_large(gpu, M, K, N):
+    m = gpu
+    print(f"case mxfp8 large M={M} K={K} N={N}", flush=True)
+    inp = cases.make_mx_inputs(m, M, K, N, 7, True, False)
+    got = cases.run_mx_aclnn(m, inp, M, K, N, True, m.ACL_BF16)
+    rows = _rows(M, 6, 8)
+    want = cases.oracle_mx(m, inp, M, K, N, True, m.ACL_BF16, rows=rows)
+    check_close(got[0][rows], want[0], m.ACL_BF16, "mxfp8 large")
+    inp2 = dict(inp, s1=(inp["s1"] + 1).astype(np.uint8))
+    _double_exactly(got, cases.run_mx_aclnn(m, inp2, M, K, N, True, m.ACL_BF16), m.ACL_BF16)
+
+
+@pytest.mark.parametrize("M,K,N", [(4096, 8192, 8192), (16, 8192, 28672)])
+def test_fp8_fp4_mx_large(gpu, M, K, N):
+    m = gpu
+    print(f"case fp8 x fp4 mx large M={M} K={K} N={N}", flush=True)
+    inp = cases.make_a8w4_mx_inputs(m, M, K, N, 9, True)
+    rng = np.random.default_rng(5)
+    inp["s1"] = (127 + rng.integers(-4, 5, size=inp["s1"].shape)).astype(np.uint8)
+    inp["s2"] = (127 + rng.integers(-4, 5, size=inp["s2"].shape)).astype(np.uint8)
+    got = cases.run_a8w4_mx_aclnn(m, inp, M, K, N, True, m.ACL_BF16, bias_dt=m.ACL_BF16)
+    rows = _rows(M, 6, 9)
+    sub = dict(inp, x1=np.ascontiguousarray(inp["x1"][rows]), s1=np.ascontiguousarray(inp["s1"][rows]))
+    want = cases.oracle_a8w4_mx(m, sub, len(rows), K, N, True, m.ACL_BF16, bias_dt=m.ACL_BF16)
+    check_close(got[rows], want, m.ACL_BF16, "fp8 x fp4 mx large")
+
+
 # ---- the operators that prepare the configs' tensors, at the configs' sizes (bit-identical to the oracle) ----
 def test_prepack_of_config3_weight_full(gpu):
     """8192 x 28672 int32 carriers -> packed int4: every byte against the oracle, and unpacking returns the carriers' nibbles."""

@@ -5,8 +5,8 @@ the oracle does, so they must match it bit for bit.  (2) The MFMA kernels accumu
 reference hardware and BLAS do); for them the bar is: max relative error <= 2^-7 and mean relative error <= 2^-10
 against the fp32-accumulated oracle (denominator floored at 1 % of the mean magnitude), plus the reference's own
 acceptance rule (>= 99.9 % of elements within rtol = atol = 1e-3).  The fp8 block-scale and row/column-scale modes
-run by default on exact fp16 products (that bar); their opt-in 8-bit matrix-instruction form (opsnnSetFp8Fast) and
-MXFP8 are held to the looser bars written out in check_close.
+and the MX modes with fp8 operands run by default on exact fp16 products (that bar); their opt-in 8-bit
+matrix-instruction form (opsnnSetFp8Fast) is held to the looser bars written out in check_close.
 """
 import os
 
@@ -175,7 +175,7 @@ def test_fp8_blockscale_group_size_inferred(gpu):
     assert np.array_equal(a, b)
 
 
-@pytest.mark.parametrize("use_plain", [True, False])
+@pytest.mark.parametrize("use_plain", [True, False, "fast"])
 @pytest.mark.parametrize("M,K,N,tB,fp4", [
     (128, 256, 256, True, True), (128, 256, 256, False, True), (197, 960, 854, True, True), (64, 128, 64, True, False),
     (64, 320, 96, False, False), (33, 192, 50, True, True),
@@ -187,19 +187,45 @@ def test_fp8_blockscale_group_size_inferred(gpu):
     (300, 128, 260, True, False), (512, 4096, 256, True, False), (100, 1024, 520, False, False),
 ])
 def test_mx(gpu, M, K, N, tB, fp4, use_plain):
+    """plain: bit-identical.  Default: MXFP4 on the scaled 4-bit instruction (its products and sums are exact), MXFP8 on
+    exact fp16 products with the block scales folded into the widening -- both at the stated bar.  fast: MXFP8 on the scaled
+    8-bit matrix instruction (four 32-element blocks per instruction), held to the backward-error bound of check_close."""
     m = gpu
+    fast = use_plain == "fast"
+    if fast and fp4:
+        pytest.skip("MXFP4 has one matrix-core form")
     print(f"case mx M={M} K={K} N={N} tB={tB} fp4={fp4} plain={use_plain}", flush=True)
     inp = cases.make_mx_inputs(m, M, K, N, K + N, tB, fp4)
     bias = np.random.default_rng(1).normal(0, 1, N).astype(np.float32)
     want = cases.oracle_mx(m, inp, M, K, N, tB, m.ACL_BF16, bias)
-    plain(use_plain)
+    plain(use_plain is True)
+    m.lib().opsnnSetFp8Fast(1 if fast else 0)
     got = cases.run_mx_aclnn(m, inp, M, K, N, tB, m.ACL_BF16, bias)
-    # MXFP8 runs on the scaled 8-bit matrix instruction, four 32-element blocks per instruction
     abs_sum = None
-    if not fp4 and not use_plain:   # sum |x1 s1 x2 s2| per element: the oracle on the inputs with their sign bits cleared
+    if fast:   # sum |x1 s1 x2 s2| per element: the oracle on the inputs with their sign bits cleared
         pos = dict(inp, x1=inp["x1"] & 0x7F, x2=inp["x2"] & 0x7F)
         abs_sum = orc.b16_to_f32(cases.oracle_mx(m, pos, M, K, N, tB, m.ACL_BF16), orc.BF16).astype(np.float64)
-    check_close(got, want, orc.BF16, "mx", exact=use_plain, fp8_mfma=not fp4, abs_sum=abs_sum)
+    check_close(got, want, orc.BF16, "mx", exact=use_plain is True, fp8_mfma=fast, abs_sum=abs_sum)
+
+
+@pytest.mark.parametrize("exp_range,batch", [(10, 1), (11, 2), (14, 1), (4, 3)])
+def test_mxfp8_exact_window(gpu, exp_range, batch):
+    """The exact MXFP8 route folds a block's scale into the widening conversion as 2^(byte - base) with one base per row,
+    exact while byte - base stays in [-15, 7].  Exponent ranges +-10 and +-11 (a spread of up to 22 binades inside a row)
+    reach the fp16 subnormals and must still meet the stated bar; +-14 exceeds the window in some row, the bases pass flags
+    it and the call runs on the scaled 8-bit instruction instead (its looser bar)."""
+    m = gpu
+    M, K, N = 300, 1024, 260
+    print(f"case mxfp8 window exp_range={exp_range} batch={batch}", flush=True)
+    inp = cases.make_mx_inputs(m, M, K, N, 3 + exp_range, True, False, batch=batch, exp_range=exp_range)
+    want = cases.oracle_mx(m, inp, M, K, N, True, m.ACL_BF16)
+    got = cases.run_mx_aclnn(m, inp, M, K, N, True, m.ACL_BF16)
+    if exp_range <= 11:
+        check_close(got, want, orc.BF16, "mxfp8 exact window")
+    else:
+        pos = dict(inp, x1=inp["x1"] & 0x7F, x2=inp["x2"] & 0x7F)
+        abs_sum = orc.b16_to_f32(cases.oracle_mx(m, pos, M, K, N, True, m.ACL_BF16), orc.BF16).astype(np.float64)
+        check_close(got, want, orc.BF16, "mxfp8 beyond the window", fp8_mfma=True, abs_sum=abs_sum)
 
 
 @pytest.mark.parametrize("M,K,N,tB,fp4,bias", [(256, 1024, 384, True, True, True), (300, 512, 262, True, True, False), (128, 512, 256, False, True, True),
@@ -243,10 +269,12 @@ def test_mxfp8_on_the_four_wave_kernel(gpu, fn, M, K, N, tB, batch, bias):
     pos = dict(inp, x1=inp["x1"] & 0x7F, x2=inp["x2"] & 0x7F)
     abs_sum = orc.b16_to_f32(cases.oracle_mx(m, pos, M, K, N, tB, m.ACL_BF16), orc.BF16).astype(np.float64)
     m.lib().opsnnSetMx8Wide(fn)
+    m.lib().opsnnSetFp8Fast(1)   # the scaled 8-bit instruction is the opt-in form of MXFP8
     try:
         got = cases.run_mx_aclnn(m, inp, M, K, N, tB, m.ACL_BF16, b)
     finally:
         m.lib().opsnnSetMx8Wide(-1)
+        m.lib().opsnnSetFp8Fast(0)
     check_close(got, want, orc.BF16, "mxfp8 four-wave", fp8_mfma=True, abs_sum=abs_sum)
 
 

@@ -187,3 +187,58 @@ def test_fp8_fp4_group_mode_requantised_weight_is_written_once(cache):
     third = call()
     assert close(third, cases.oracle_tcg(m, inp2, M, K, N, m.ACL_BF16))
     assert _stats(m)[2] - h0 == 2
+
+
+def test_nz_entry_points_do_not_key_the_cache_on_the_workspace(cache):
+    """A FRACTAL_NZ weight is first written as the ND matrix into the front of the caller's workspace.  Two weights of one
+    shape that share one workspace (as the layers of a model do) would meet under one cache key; the NZ entry points
+    therefore leave the cache alone: both results equal the ND entry point's, and the cache holds nothing afterwards."""
+    from test_nz_entry_points import nd_to_nz
+    m = cache
+    M, K, N = 16, 512, 256
+    print(f"case weight cache with FRACTAL_NZ weights sharing a workspace, int8 {M}x{K}x{N}", flush=True)
+    e0 = _stats(m)[0]
+    inps = [cases.make_qmm_int8_inputs(m, M, K, N, seed, m.ACL_BF16, False) for seed in (21, 22)]
+    wants = [cases.oracle_qmm_int8(m, inp, M, K, N, False, m.ACL_BF16)[0][0] for inp in inps]
+    m.lib().opsnnSetWeightCache(0)
+    nd = [cases.run_qmm_int8_aclnn(m, inp, M, K, N, False, m.ACL_BF16)[0] for inp in inps]
+    m.lib().opsnnSetWeightCache(256 << 20)
+    assert all(np.array_equal(a, b) for a, b in zip(nd, wants))
+    shared_ws = None
+    got = []
+    for inp in inps:
+        nz = nd_to_nz(inp["x2"][0].view(np.uint8), 32)
+        d = {k: m.DeviceBuffer(host=v) for k, v in dict(inp, x2=nz[None]).items() if isinstance(v, np.ndarray)}
+        d_out = m.DeviceBuffer(M * N * 2)
+        d_out.fill(0xFF)
+        x1 = m.Tensor((M, K), m.ACL_INT8, d["x1"])
+        x2 = m.Tensor((K, N), m.ACL_INT8, d["x2"], fmt=29, storage_shape=(nz.shape[0], nz.shape[1], 16, 32))
+        s1, s2 = m.Tensor((M,), m.ACL_FLOAT, d["s1"]), m.Tensor((N,), m.ACL_FLOAT, d["s2"])
+        bias = m.Tensor((N,), m.ACL_BF16, d["bias"])
+        out = m.Tensor((M, N), m.ACL_BF16, d_out)
+        rc, ws, ex = m.quant_matmul_v5_get_workspace(x1, x2, s1, s2, out, bias=bias, weight_nz=True)
+        assert rc == 0 and ws > 0, m.err_msg()
+        if shared_ws is None:
+            shared_ws = m.DeviceBuffer(ws)
+        m.check(m.lib().aclnnQuantMatmulWeightNz(shared_ws.ptr, ws, ex, None), "aclnnQuantMatmulWeightNz")
+        m.check(m.lib().aclrtSynchronizeDevice(), "sync")
+        got.append(d_out.to_host(np.uint16, (M, N)))
+    assert np.array_equal(got[0], wants[0]), "first NZ weight"
+    assert np.array_equal(got[1], wants[1]), "second NZ weight through the same workspace: a stale cached copy was used"
+    assert _stats(m)[0] == e0, "the NZ entry point put its workspace address into the cache"
+
+
+def test_static_entry_point_leaves_the_cache_alone(cache):
+    """opsnnQmmInt8Static promises no allocation: with the cache on it must not look the operand up (a miss allocates)."""
+    m = cache
+    M, K, N = 128, 256, 192
+    inp = cases.make_qmm_int8_inputs(m, M, K, N, 5, m.ACL_BF16, False)
+    d = {k: m.DeviceBuffer(host=v) for k, v in inp.items() if isinstance(v, np.ndarray)}
+    out = m.DeviceBuffer(M * N * 2)
+    before = _stats(m)
+    a = cases.qmm_args_int8(m, d, M, K, N, 1, False, out.ptr, m.ACL_BF16, m.ACL_FLOAT, N, m.ACL_BF16)
+    assert m.lib().opsnnQmmInt8Static(C.byref(a), None) == 0, m.err_msg()
+    m.check(m.lib().aclrtSynchronizeDevice(), "sync")
+    assert _stats(m) == before, (before, _stats(m))
+    want, _ = cases.oracle_qmm_int8(m, inp, M, K, N, False, m.ACL_BF16)
+    assert np.array_equal(out.to_host(np.uint16, (M, N)), want[0])

@@ -137,29 +137,27 @@ def test_gpu_a8w4_mx(gpu, M, K, N, tB):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("M,K,N", [(64, 128, 64), (300, 384, 260), (512, 2048, 520), (100, 1024, 1000),
-                                   # up to 32 rows: x1 in registers, x2 streamed once per 16 rows; K shared by 16 waves
-                                   # (2 or 4 chunks of 128 each) or by 8 (1 .. 7), ragged columns, two passes
+@pytest.mark.parametrize("M,K,N", [(64, 128, 64), (300, 384, 260), (512, 2048, 520), (100, 1024, 1000), (1024, 4096, 1024),
+                                   # up to 32 rows: x1 in registers, x2 streamed once per 16 rows; K shared by 16 waves (2 or 4
+                                   # chunks of 128 each) or by 8 (1 .. 7), ragged columns, two passes
                                    (16, 4096, 512), (9, 8192, 264), (24, 1024, 520), (1, 7168, 384), (32, 3072, 256),
                                    (16, 2048, 256)])
 def test_gpu_a8w4_mx_on_the_matrix_cores(gpu, M, K, N):
     """fp8 x fp4 MX with K % 128 == 0 and enough outputs runs on the scaled matrix instruction with a 4-bit x2 operand.
-    Bar: the one of MXFP8 (the instruction's alignment error against sum|terms|, mean rel <= 2^-10); the same call on
-    the plain kernel is bit-identical to the oracle."""
-    import os
+    With a 4-bit operand the instruction's sums are as close to the fp32-accumulated ones as exact fp16 products are
+    (measured at these shapes and at 4096 x 8192 x 8192 / 16 x 8192 x 28672: the same share of bit-identical outputs), so
+    the bar is the stated one: max rel 2^-7, mean rel 2^-10, 99.9 % within rtol = atol = 1e-3.  The same call on the plain
+    kernel is bit-identical to the oracle."""
     m = gpu
     print(f"case a8w4 mx mfma {M}x{K}x{N}", flush=True)
     inp = cases.make_a8w4_mx_inputs(m, M, K, N, M + N, True)
     want = cases.oracle_a8w4_mx(m, inp, M, K, N, True, m.ACL_FLOAT16)
     got = cases.run_a8w4_mx_aclnn(m, inp, M, K, N, True, m.ACL_FLOAT16)
-    pos = dict(inp, x1=inp["x1"] & 0x7F, x2=inp["x2"] & 0x77, bias=np.zeros_like(inp["bias"]))
-    abs_sum = orc.b16_to_f32(cases.oracle_a8w4_mx(m, pos, M, K, N, True, m.ACL_FLOAT16), orc.F16).astype(np.float64)
     g, w = orc.b16_to_f32(got, orc.F16), orc.b16_to_f32(want, orc.F16)
     assert np.isfinite(g).all()
-    err = np.abs(g.astype(np.float64) - w)
-    bound = 2.0 ** -7 * np.abs(w) + 2.0 ** -14 * abs_sum
     mx, mean = orc.rel_err_stats(g, w)
-    assert float((err / np.maximum(bound, 1e-30)).max()) <= 1.0 and mean <= 2.0 ** -10, f"max rel {mx:.3e} mean rel {mean:.3e}"
+    assert mx <= 2.0 ** -7 and mean <= 2.0 ** -10, f"max rel {mx:.3e} mean rel {mean:.3e}"
+    assert orc.isclose_fraction(g, w) <= 1e-3
     m.lib().opsnnSetForcePlain(1)
     try:
         exact = cases.run_a8w4_mx_aclnn(m, inp, M, K, N, True, m.ACL_FLOAT16)
