@@ -419,10 +419,18 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(NW == 8
 // scale block of w).  The output type is the call's (bf16, fp16 or fp32).
 // WF 4: the fp8 row / column scale form (K-C, K-T) of the same operands: one chain over all of K, and the epilogue
 // computes (sum * x2Scale[n]) * x1Scale[m] + bias[n] (bs2 / bs1 with element strides bs2_cs / bs1_rs of 0 or 1).
-template <int XDT, int WBITS, int MB, int NB, int WN, int WK, bool HAS_OFF, int WF = 0>
+// SLDS (integer codes, a row's scales contiguous, power-of-two group count): the workgroup lays all scales and offsets of
+// its columns down in LDS once, one 32-bit word (scale | offset << 16) per column and group, instead of fetching two
+// 16-bit values per row block and chunk from global memory.  Such a load is one instruction per 16-bit value and touches
+// 16 cache lines (one per weight row): at 8192 x 28672 with groups of 128 they were half of all the cache-line requests
+// of the loop (512 of 1024 per slab and CU, against about 0.45 requests per clock that a CU's texture path takes) --
+// more than weights and x together; per-wave timestamps showed the waves stalled in the issue of their memory
+// instructions (1180 of 4120 clocks per slab) and at the barrier behind them.
+template <int XDT, int WBITS, int MB, int NB, int WN, int WK, bool HAS_OFF, int WF = 0, bool SLDS = false>
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void wqmm_rows_kernel(WqParams p)
 {
     static_assert(WN * WK == 8, "eight waves");
+    static_assert(!SLDS || WF == 0, "the scale table serves the integer forms");
     static_assert(WF == 0 || !HAS_OFF, "floating-point weight codes have no offset");
     static_assert(WF != 2 || WBITS == 4, "e8m0 group scales go with e2m1 codes");
     static_assert(WF != 3 || (WBITS == 8 && XDT == DT_F16 && WK == 2 && NB == 2), "the block-scale form: fp16 x, e4m3 w, a slab per 128-block");
@@ -435,7 +443,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void w
     constexpr int XPR = KX / 8;          // 16-byte pieces per x row per slab
     constexpr int XBUF = 16 * MB * XROW; // one slab buffer
     constexpr int XITEMS = 16 * MB * XPR / NT;
-    constexpr int NBL = WF >= 3 ? NB : NB * (HAS_OFF ? 3 : 2);   // loads of one weight fetch
+    constexpr int NBL = (WF >= 3 || SLDS) ? NB : NB * (HAS_OFF ? 3 : 2);   // loads of one weight fetch
     constexpr int LDS_MAIN = (2 * XBUF > WN * (WK - 1) * NB * MB * 4 * 64 * 4) ? 2 * XBUF : WN * (WK - 1) * NB * MB * 4 * 64 * 4;
     static_assert((16 * MB * XPR) % NT == 0 && XPR >= 16 && PF >= 2, "staging and prefetch shape");
     extern __shared__ __attribute__((aligned(16))) char sx[];
@@ -460,13 +468,23 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void w
 
     // x copies: instruction `it` of this thread fills LDS piece it*NT + tid of the buffer, i.e. position
     // (it*NT + tid) % XPR of row (it*NT + tid) / XPR, with the row's piece position ^ (row % 16)
+    // Which 16-byte piece of a slab row sits where.  A 16-byte-per-lane LDS read is served 16 lanes at a time, two passes
+    // per half-wave; measured with address patterns on this chip, the pass of lane l inside its half-wave is
+    // bit 4 of l xor bit 2 of l (lanes 0-3, 8-11, 20-23, 28-31 go together), and a read runs at the full 256 bytes per
+    // clock only if the 16 lanes of every pass hit 16 different 16-byte columns of the 256-byte bank row.  Here lane
+    // l = 16 g + row reads piece (16 wk + 4 g + s) ^ row of a 512-byte row: lanes (g, row) and (g ^ 1, row ^ 4) share a pass
+    // and, since bit 2 of the piece number is bit 0 of g, a column -- half the LDS rate.  So rows of 32 pieces store piece P
+    // at position swap24(P) ^ (row % 16), bits 2 and 4 of the piece number exchanged: bit 2 of the position is then
+    // wk ^ bit 2 of the row, the same for both lane groups of a half-wave, and the two passes split the columns evenly.
+    constexpr bool SWAP24 = XPR == 32 && KPL == 32;
+    auto piece_of_pos = [](int q) { return SWAP24 ? ((q & ~0x14) | ((q & 4) << 2) | ((q & 16) >> 2)) : q; };   // (its own inverse)
     const uint16_t* xsrc[XITEMS];
 #pragma unroll
     for (int it = 0; it < XITEMS; it++) {
         const int L = it * NT + tid;
         const int r = L / XPR, pos = L % XPR;
         const int rr = r < rows ? r : rows - 1;
-        xsrc[it] = p.x + (p.m_base + rr) * p.K + (pos ^ (r & 15)) * 8;
+        xsrc[it] = p.x + (p.m_base + rr) * p.K + piece_of_pos(pos ^ (r & 15)) * 8;
     }
     auto issue_x = [&](int slab) {
         char* dst = sx + (slab & 1) * XBUF + wave * 1024;
@@ -480,7 +498,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void w
 #pragma unroll
     for (int b = 0; b < MB; b++) {
         const int r = 16 * b + nrow;
-        xoff[b] = r * XROW + ((wk * (KC / 8) + g * (KPL / 8)) ^ (r & 15)) * 16;
+        xoff[b] = r * XROW + (piece_of_pos(wk * (KC / 8) + g * (KPL / 8)) ^ (r & 15)) * 16;
     }
 
     v4f acc[NB][MB];
@@ -502,6 +520,32 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void w
         }
     }
 
+    // SLDS: word (row rw of the workgroup's 16 NB WN columns, group gi) at stab[rw * G + (gi ^ swizzle(rw))], G = groups per
+    // row; the swizzle (4 * (rw % 16), kept below G) spreads the 16 rows that one read touches over the banks.  The table is
+    // complete behind the loop's first barrier.
+    uint32_t* stab = (uint32_t*)(sx + LDS_MAIN);
+    const int sG = p.cpg_shift >= 31 ? 1 : (int)((p.K / KC) >> p.cpg_shift);
+    int stab_row[NB], stab_sw[NB];
+    (void)stab; (void)sG; (void)stab_row; (void)stab_sw;
+    if constexpr (SLDS) {
+        constexpr int RW = 16 * NB * WN;
+        for (int i = tid; i < RW * sG; i += NT) {
+            const int rw = i / sG, gi = i - rw * sG;
+            int64_t nb0 = ((int64_t)blockIdx.x * WN + rw / (16 * NB)) * (16 * NB);
+            if (nb0 >= p.N) nb0 = p.N - 16 * NB;
+            const int64_t n = nb0 + rw % (16 * NB);
+            uint32_t w = p.scale[n * p.s_cs + gi];
+            if constexpr (HAS_OFF) w |= (uint32_t)p.offset[n * p.s_cs + gi] << 16;
+            stab[rw * sG + (gi ^ (((rw & 15) << 2) & (sG - 1)))] = w;
+        }
+#pragma unroll
+        for (int q = 0; q < NB; q++) {
+            const int rw = wn * (16 * NB) + 16 * q + nrow;
+            stab_row[q] = rw * sG;
+            stab_sw[q] = ((rw & 15) << 2) & (sG - 1);
+        }
+    }
+
     v4i wq[PF][NB];
     uint16_t sq[PF][NB], oq[PF][NB];
     auto fetch = [&](int j, int cw) {   // chunk cw of this wave (chunk cw * WK + wk of the row) into slot j
@@ -509,6 +553,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void w
 #pragma unroll
         for (int q = 0; q < NB; q++) {
             wq[j][q] = *(const v4i*)(wptr + q * wblk + (int64_t)cw * (WK * 64));
+            if constexpr (SLDS) { sq[j][q] = 0; oq[j][q] = 0; continue; }
             if constexpr (WF >= 3) sq[j][q] = 0;
             else if constexpr (WF == 2) sq[j][q] = srow8[q * sblk + (cw * WK + wk) * 4];
             else sq[j][q] = srow[q * sblk + so];
@@ -609,12 +654,20 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void w
                 }
                 }
             }
+            uint32_t sow[NB];
+            (void)sow;
+            if constexpr (SLDS) {
+                const int gi = (cw * WK + wk) >> p.cpg_shift;
+#pragma unroll
+                for (int q = 0; q < NB; q++) sow[q] = stab[stab_row[q] + (gi ^ stab_sw[q])];
+            }
 #pragma unroll
             for (int s = 0; s < (WF == 3 ? 0 : STEPS); s++) {
                 v4i aop[NB];
 #pragma unroll
                 for (int q = 0; q < NB; q++) {
-                    if constexpr (WF == 0) aop[q] = dequant8<XDT, WBITS, HAS_OFF, true>(wq[j][q], s, sq[j][q], oq[j][q], dqc);
+                    if constexpr (WF == 0 && SLDS) aop[q] = dequant8<XDT, WBITS, HAS_OFF, true>(wq[j][q], s, (uint16_t)sow[q], (uint16_t)(sow[q] >> 16), dqc);
+                    else if constexpr (WF == 0) aop[q] = dequant8<XDT, WBITS, HAS_OFF, true>(wq[j][q], s, sq[j][q], oq[j][q], dqc);
                     else if constexpr (WF == 1) aop[q] = dequant8_float<XDT, WBITS, true>(wq[j][q], s, sq[j][q]);
                     else if constexpr (WF == 4) {
                         typedef _Float16 h2v __attribute__((ext_vector_type(2)));
@@ -1225,21 +1278,31 @@ static int launch_stream_one(const WqParams& p, hipStream_t st)
     return (int)hipGetLastError();
 }
 
-template <int XDT, int WBITS, int MB, int NB, int WN, int WK, bool HAS_OFF, int WF = 0>
+template <int XDT, int WBITS, int MB, int NB, int WN, int WK, bool HAS_OFF, int WF = 0, bool SLDS = false>
 static int launch_rows_one(const WqParams& p, hipStream_t st)
 {
     constexpr int KC = 4 * (128 / WBITS);
     constexpr size_t lds_x = 2 * (size_t)(16 * MB) * (WK * KC * 2);
+    size_t lds_stab = 0;
+    if constexpr (WF == 0 && !SLDS) {
+        // the scales and offsets of the workgroup's columns in LDS when a row's scales are contiguous, their count per row
+        // is a power of two and the table fits beside the x buffers
+        const int64_t G = p.cpg_shift >= 31 ? 1 : ((p.K / KC) >> p.cpg_shift);
+        const size_t red = (size_t)WN * (WK - 1) * NB * MB * 4 * 64 * 4;
+        if ((p.s_rs == 1 || G == 1) && (G & (G - 1)) == 0 && (lds_x > red ? lds_x : red) + (size_t)(16 * NB * WN) * G * 4 <= 160 * 1024)
+            return launch_rows_one<XDT, WBITS, MB, NB, WN, WK, HAS_OFF, WF, true>(p, st);
+    }
+    if constexpr (SLDS) lds_stab = (size_t)(16 * NB * WN) * (p.cpg_shift >= 31 ? 1 : ((p.K / KC) >> p.cpg_shift)) * 4;
     constexpr size_t lds_red = (size_t)WN * (WK - 1) * NB * MB * 4 * 64 * 4;
     constexpr size_t lds_main = lds_x > lds_red ? lds_x : lds_red;
     constexpr size_t lds_table = WF == 3 ? 65536 : 0;   // products of the block scales: (K / 128) * 16 MB floats, at most this
-    const size_t lds = lds_main + (WF == 3 ? (size_t)(p.K / 128) * 16 * MB * 4 : 0);
-    if (lds > lds_main + lds_table) return OPSNN_NOT_TAKEN;
+    const size_t lds = lds_main + (WF == 3 ? (size_t)(p.K / 128) * 16 * MB * 4 : 0) + lds_stab;
+    if (lds > lds_main + lds_table + lds_stab) return OPSNN_NOT_TAKEN;
     const unsigned grid = (unsigned)((p.N + 16 * NB * WN - 1) / (16 * NB * WN));
-    auto k = wqmm_rows_kernel<XDT, WBITS, MB, NB, WN, WK, HAS_OFF, WF>;
+    auto k = wqmm_rows_kernel<XDT, WBITS, MB, NB, WN, WK, HAS_OFF, WF, SLDS>;
     static bool attr_set = false;
     if (!attr_set) {
-        hipError_t e = hipFuncSetAttribute((const void*)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)(lds_main + lds_table));
+        hipError_t e = hipFuncSetAttribute((const void*)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)(SLDS ? 160 * 1024 : lds_main + lds_table));
         if (e != hipSuccess) return (int)e;
         attr_set = true;
     }
