@@ -135,9 +135,16 @@ __global__ __launch_bounds__(WGM* WGN * 64, MINWG) void qgemm_kernel(QgemmParams
         }
     }
 
-    // tile id: XCD-contiguous, m fastest so that one XCD works on few x2 panels at a time
+    // Tile order: each XCD (own L2) gets a contiguous range of ids, and ids run down groups of GM row tiles and across the
+    // columns inside a group, so that the 32 tiles an XCD works on at a time form a GM x (32 / GM) block sharing GM x1
+    // panels and 32 / GM x2 panels (with whole columns of 16 row tiles it was 16 + 2 panels per K step, and every x1 panel
+    // was fetched once per pair of columns).
+    constexpr int GM = 4;
     const uint32_t t = xcd_remap(blockIdx.x, (uint32_t)(tiles_m * tiles_n));
-    const int tm = (int)(t % (uint32_t)tiles_m), tn = (int)(t / (uint32_t)tiles_m);
+    const uint32_t gsz_full = (uint32_t)(GM * tiles_n), grp = t / gsz_full, in_grp = t % gsz_full;
+    const int first_m = (int)grp * GM;
+    const int gh = tiles_m - first_m < GM ? tiles_m - first_m : GM;
+    const int tm = first_m + (int)(in_grp % (uint32_t)gh), tn = (int)(in_grp / (uint32_t)gh);
     const int64_t m0 = (int64_t)tm * BM, n0 = (int64_t)tn * BN;
     const int64_t bz = blockIdx.y;
 
