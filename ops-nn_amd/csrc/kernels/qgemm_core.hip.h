@@ -130,8 +130,8 @@ __global__ __launch_bounds__(WGM* WGN * 64, MINWG) void qgemm_kernel(QgemmParams
     if constexpr (MX) {
         if (p.gate) {
             int f = 0;
-            for (int i = tid; i < p.gate_n; i += NT) f |= p.gate[i];
-            if (!__syncthreads_or(f)) return;
+            for (int i = 0; i < p.gate_n; i++) f |= p.gate[i];   // every thread reads every flag: uniform loads, no LDS for a vote
+            if (!f) return;
         }
     }
 

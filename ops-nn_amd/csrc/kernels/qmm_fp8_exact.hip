@@ -130,8 +130,8 @@ __global__ __launch_bounds__(512, 1) void qmm_fp8_exact_kernel(Fp8xParams p, int
     const int wm = wave >> 1, wn = wave & 1;
     if constexpr (MXS) {
         int f = 0;
-        for (int i = tid; i < p.gate_n; i += NT) f |= p.gate[i];
-        if (__syncthreads_or(f)) return;   // some row's scale bytes do not fit the exact window: the next launch computes the call
+        for (int i = 0; i < p.gate_n; i++) f |= p.gate[i];   // (every thread reads every flag: uniform loads)
+        if (f) return;   // some row's scale bytes do not fit the exact window: the next launch computes the call
     }
 
     // Tile order: each XCD (own L2) gets a contiguous range of ids, and ids run down groups of GM row tiles and across

@@ -278,6 +278,31 @@ def test_mxfp8_on_the_four_wave_kernel(gpu, fn, M, K, N, tB, batch, bias):
     check_close(got, want, orc.BF16, "mxfp8 four-wave", fp8_mfma=True, abs_sum=abs_sum)
 
 
+@pytest.mark.parametrize("M,K,N,batch,bias", [
+    (512, 2048, 1024, 2, True),     # 16 whole tiles in two batches
+    (768, 1024, 768, 3, False),     # 27 tiles: the grouped tile order with a ragged last group of row tiles
+    (256, 4096, 2048, 1, True),     # one row of tiles, a long K loop
+    (1024, 1024, 512, 5, True),     # five batches of 8 tiles
+])
+def test_mxfp4_batched_whole_tiles(gpu, M, K, N, batch, bias):
+    """Batched MXFP4 on whole 256 x 256 tiles (config 5's form at small sizes): the stated bar against the oracle, and the
+    same columns bit for bit when one more column tile makes the launch ragged (another tile count and tile order)."""
+    m = gpu
+    print(f"case mxfp4 whole tiles M={M} K={K} N={N} batch={batch} bias={bias}", flush=True)
+    inp = cases.make_mx_inputs(m, M, K, N, M + batch, True, True, batch=batch)
+    b = np.random.default_rng(4).normal(0, 1, N).astype(np.float32) if bias else None
+    want = cases.oracle_mx(m, inp, M, K, N, True, m.ACL_BF16, b)
+    got = cases.run_mx_aclnn(m, inp, M, K, N, True, m.ACL_BF16, b)
+    check_close(got, want, orc.BF16, "mxfp4 whole tiles")
+    # eight more columns: a ragged last column tile; the shared columns must agree bit for bit
+    inp2 = cases.make_mx_inputs(m, M, K, N + 8, M + batch, True, True, batch=batch)
+    inp2["x1"], inp2["s1"] = inp["x1"], inp["s1"]
+    inp2["x2"][:, :N], inp2["s2"][:, :N] = inp["x2"], inp["s2"]
+    b2 = np.concatenate([b, np.zeros(8, np.float32)]) if bias else None
+    got2 = cases.run_mx_aclnn(m, inp2, M, K, N + 8, True, m.ACL_BF16, b2)
+    assert np.array_equal(got2[:, :, :N], got), "whole-tile and ragged launches differ on shared columns"
+
+
 @pytest.mark.parametrize("M,K,N,batch", [(96, 256, 128, 3), (256, 1024, 264, 2)])
 def test_mx_batched(gpu, M, K, N, batch):
     m = gpu
