@@ -56,6 +56,20 @@ static int g_fp8_fast = [] { const char* e = getenv("OPSNN_FP8_FAST"); return (e
 extern "C" void opsnnSetFp8Fast(int fast) { __atomic_store_n(&g_fp8_fast, fast ? 1 : 0, __ATOMIC_RELAXED); }
 extern "C" int opsnnGetFp8Fast(void) { return __atomic_load_n(&g_fp8_fast, __ATOMIC_RELAXED); }
 
+// OPSNN_LOG=1 (read once, like the switches above): one line on stderr whenever a call of more than 10^7 multiply-adds
+// lands on a plain one-thread-per-output kernel without having been sent there -- those kernels are the parity
+// reference and the route of last resort, three to four orders of magnitude slower than the matrix-core kernels.
+static const bool g_log = [] { const char* e = getenv("OPSNN_LOG"); return e && *e && *e != '0'; }();
+extern "C" __attribute__((visibility("hidden"))) void opsnn_note_plain(const char* mode, int forced, int64_t batch, int64_t M, int64_t N, int64_t K)
+{
+    if (!g_log || forced || opsnn_force_plain()) return;
+    const double macs = (double)batch * (double)M * (double)N * (double)K;
+    if (macs <= 1e7) return;
+    fprintf(stderr, "[opsnn] %s: batch %lld, %lld x %lld x %lld (%.3g multiply-adds) runs on the plain kernel: no matrix-core route takes "
+                    "this combination of layout, strides, dtypes and shape\n", mode, (long long)batch, (long long)M, (long long)K, (long long)N, macs);
+}
+#define NOTE_PLAIN(mode, a) opsnn_note_plain(mode, (a)->force_variant == OPSNN_VARIANT_PLAIN, (a)->batch, (a)->M, (a)->N, (a)->K)
+
 static bool qmm_args_ok(const OpsnnQmmArgs* a)
 {
     return a && a->x1.ptr && a->x2.ptr && a->out && a->M > 0 && a->N > 0 && a->K > 0 && a->batch > 0 && a->batch <= 65535;
@@ -175,6 +189,7 @@ extern "C" int opsnnQmmBlockScale(const OpsnnQmmArgs* a, void* stream)
         if (rc != OPSNN_NOT_TAKEN) return rc;
         if (a->force_variant != 0) return -4;
     }
+    NOTE_PLAIN("block-scale quant matmul", a);
     return launch_blockscale_plain(*a, (hipStream_t)stream);
 }
 
@@ -187,6 +202,7 @@ extern "C" int opsnnQmmMx(const OpsnnQmmArgs* a, void* stream)
         if (rc != OPSNN_NOT_TAKEN) return rc;
         if (a->force_variant != 0) return -4;
     }
+    NOTE_PLAIN("MX quant matmul", a);
     return launch_mx_plain(*a, (hipStream_t)stream);
 }
 
@@ -256,6 +272,7 @@ extern "C" int opsnnQmmTc(const OpsnnQmmArgs* a, void* stream)
         const int rc = launch_fp8_rowcol_mfma(*a, (hipStream_t)stream, false);
         if (rc != OPSNN_NOT_TAKEN) return rc;
     }
+    NOTE_PLAIN("per-tensor / per-channel quant matmul", a);
     return launch_tc_plain(*a, (hipStream_t)stream);
 }
 
@@ -283,6 +300,7 @@ extern "C" int opsnnQmmGroup(const OpsnnQmmArgs* a, void* stream)
         const int rc = launch_kg_mfma(*a, (hipStream_t)stream);
         if (rc != OPSNN_NOT_TAKEN) return rc;
     }
+    NOTE_PLAIN(tcg ? "fp8 x fp4 group quant matmul" : "int4 K-G quant matmul", a);
     return launch_group_plain(*a, tcg, (hipStream_t)stream);
 }
 
@@ -295,6 +313,7 @@ extern "C" int opsnnWqmm(const OpsnnWqmmArgs* a, void* stream)
         if (rc != OPSNN_NOT_TAKEN) return rc;
         if (a->force_variant != 0) return -4;
     }
+    opsnn_note_plain("weight-only matmul", a->force_variant == OPSNN_VARIANT_PLAIN, 1, a->M, a->N, a->K);
     return launch_wqmm_plain(*a, (hipStream_t)stream);
 }
 

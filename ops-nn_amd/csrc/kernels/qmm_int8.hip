@@ -75,6 +75,7 @@ __global__ void qmm_i8_plain(QmmI8Params p)
 using namespace opsnn;
 
 extern "C" bool opsnn_force_plain();
+extern "C" void opsnn_note_plain(const char* mode, int forced, int64_t batch, int64_t M, int64_t N, int64_t K);   // dispatch.hip
 namespace opsnn {
 int launch_int8_wide(const QgemmParams& p, int fn, int64_t batch, int out_dt, hipStream_t st);   // qmm_int8_wide.hip
 }
@@ -238,6 +239,7 @@ extern "C" int opsnn_qmm_int8_impl(const OpsnnQmmArgs* a, void* stream)
         return qgemm_launch<MODE_I8, 256, 128, 64, 2, 2, 3, 2>(g, a->batch, p.out_dt, st);
     }
     if (p.out_dt == DT_I8) return OPSNN_NOT_TAKEN;   // the strided kernel below has no requantising epilogue
+    opsnn_note_plain("int8 per-token x per-channel quant matmul", variant == OPSNN_VARIANT_PLAIN, a->batch, p.M, p.N, p.K);
     dim3 block(256), grid((unsigned)(((p.N + 255) / 256) * p.M), (unsigned)a->batch);
     hipLaunchKernelGGL(qmm_i8_plain, grid, block, 0, st, p);
     return (int)hipGetLastError();

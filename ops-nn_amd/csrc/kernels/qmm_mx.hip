@@ -11,9 +11,9 @@
 // Fast paths: operands and scales K-contiguous, K % 128 == 0, 16-bit output.  fp4: qgemm_core.hip.h, MODE_MXFP4
 // (K % 512 == 0 takes 256-element K tiles, otherwise 128-element ones); fp8: the MX mode of the kernel in
 // qmm_fp8_block.hip.  An N-contiguous x2 (data [K, N], scales [K/64, N, 2]) is first re-laid out into the
-// workspace.  K % 128 == 64 with K-contiguous operands: both operands and both scale tables are first copied into
-// the workspace with one more scale pair per row, the new elements zero and their scales 2^0 (zero products change
-// no sum).  Everything else runs the plain kernel.
+// workspace.  K % 128 == 64: both operands and both scale tables (x2's after that re-layout, if it was needed) are first
+// copied into the workspace with one more scale pair per row, the new elements zero and their scales 2^0 (zero products
+// change no sum).  All of this is planned before the first pre-step is launched.  Everything else runs the plain kernel.
 #include "launch.h"
 #include "qgemm_core.hip.h"
 
@@ -134,28 +134,105 @@ static int mx_pad_prestep(OpsnnQmmArgs& a, const MxPad& L, hipStream_t st)
 uint64_t mx_exact_bytes(const OpsnnQmmArgs& a);           // qmm_fp8_exact.hip
 int launch_mx_exact(const OpsnnQmmArgs& a, void* region, hipStream_t st);
 
-static uint64_t mx_rest_bytes(const OpsnnQmmArgs& a);
+// ---- x2 stored [K, N] with N contiguous (data dense, scales [K/64, N, 2]) ----
+// The kernels stream K-contiguous operands: data and scales are first re-laid out, per batch, at 256-byte aligned pitches.
+struct MxRelayout {
+    int64_t nb, snb;                 // batches of the data / of the scales (1 when every batch shares them)
+    uint64_t data_one, scale_one, bytes;
+};
+
+static bool mx_relayout_layout(const OpsnnQmmArgs& a, MxRelayout& R)
+{
+    if (a.x2.row_stride == 1 || a.K == 1 || a.K % 64 != 0) return false;
+    const int64_t ks = a.K / 64, epb = a.x2_dtype == DT_E2M1 ? 2 : 1;
+    if (a.x2.col_stride != 1 || a.x2.row_stride != a.N) return false;
+    if (epb == 2 && (a.N & 1)) return false;   // the 4-bit transposition works on byte pairs
+    if (a.x2_scale_mat.row_stride != 2 || a.x2_scale_mat.col_stride != a.N * 2) return false;
+    if (a.x2.batch_stride != 0 && a.x2.batch_stride != a.K * a.N) return false;
+    R.nb = a.x2.batch_stride == 0 ? 1 : a.batch;
+    R.snb = a.x2_scale_mat.batch_stride == 0 ? 1 : a.batch;
+    if (R.snb != 1 && a.x2_scale_mat.batch_stride != ks * a.N * 2) return false;
+    if (R.nb > 65535 || R.snb > 65535) return false;
+    R.data_one = align_up((uint64_t)a.N * a.K / epb, 256);
+    R.scale_one = align_up((uint64_t)a.N * ks * 2, 256);
+    R.bytes = R.data_one * (uint64_t)R.nb + R.scale_one * (uint64_t)R.snb;
+    return true;
+}
+
+// `a` as the same call on the copies at `w` (which the passes of mx_relayout_run fill)
+static void mx_relayout_view(OpsnnQmmArgs& a, const MxRelayout& R, char* w)
+{
+    const int64_t ks = a.K / 64, epb = a.x2_dtype == DT_E2M1 ? 2 : 1;
+    char* wscale = w + R.data_one * R.nb;
+    a.x2.ptr = w; a.x2.row_stride = 1; a.x2.col_stride = a.K; a.x2.batch_stride = R.nb == 1 ? 0 : (int64_t)(R.data_one * epb);
+    a.x2_scale_mat.ptr = wscale; a.x2_scale_mat.row_stride = ks * 2; a.x2_scale_mat.col_stride = 2;
+    a.x2_scale_mat.batch_stride = R.snb == 1 ? 0 : (int64_t)R.scale_one;
+}
+
+static int mx_relayout_run(const OpsnnQmmArgs& a, const MxRelayout& R, char* w, hipStream_t st)
+{
+    const int64_t ks = a.K / 64, epb = a.x2_dtype == DT_E2M1 ? 2 : 1;
+    char* wscale = w + R.data_one * R.nb;
+    for (int64_t b = 0; b < R.nb; b++) {  // per batch because of the aligned pitch
+        const char* src = (const char*)a.x2.ptr + b * (a.K * a.N / epb);
+        const int rc = epb == 2 ? opsnnTranspose4(src, w + b * R.data_one, a.K, a.N, 1, st) : opsnnTranspose8(src, w + b * R.data_one, a.K, a.N, 1, st);
+        if (rc != 0) return rc;
+    }
+    for (int64_t b = 0; b < R.snb; b++) {
+        dim3 grid((unsigned)((a.N + 31) / 32), (unsigned)((ks + 31) / 32), 1);
+        hipLaunchKernelGGL(transpose16_kernel, grid, dim3(256), 0, st, (const uint16_t*)((const char*)a.x2_scale_mat.ptr + b * (ks * a.N * 2)),
+                           (uint16_t*)(wscale + b * R.scale_one), ks, a.N);
+    }
+    return (int)hipGetLastError();
+}
+
+// What every matrix-core route of this file needs of the call, whatever x2's layout and K's tail: checked before any
+// pre-step is launched or a cache entry made.
+static bool mx_call_ok(const OpsnnQmmArgs& a)
+{
+    const bool fp4 = a.x1_dtype == DT_E2M1 && a.x2_dtype == DT_E2M1, fp8 = a.x1_dtype == DT_E4M3 && a.x2_dtype == DT_E4M3;
+    const bool a8w4 = a.x1_dtype == DT_E4M3 && a.x2_dtype == DT_E2M1;
+    if (!fp4 && !fp8 && !a8w4) return false;
+    if (a8w4) {   // launch_mx_a8w4_mfma (qmm_fp8_block.hip): a tile kernel, and a streaming kernel for up to 32 rows
+        if (a.out_dtype != DT_BF16 && a.out_dtype != DT_F16) return false;
+        if (a.bias && a.bias_dtype != DT_F32 && a.bias_dtype != DT_BF16 && a.bias_dtype != DT_F16) return false;
+        if (a.K % 64 != 0 || a.x1.col_stride != 1 || a.x1_scale_mat.col_stride != 2) return false;
+        const bool few_rows = a.M <= 32 && a.N >= 256 && a.batch == 1;
+        if (!few_rows && a.M * a.N < 64 * 64) return false;
+        return (((uintptr_t)a.x1.ptr | (uint64_t)a.x1.row_stride | (uint64_t)a.x1.batch_stride) % 16) == 0;
+    }
+    if (a.out_dtype != DT_BF16 && a.out_dtype != DT_F16 && a.out_dtype != DT_F32) return false;
+    if (a.bias && a.bias_dtype != DT_F32) return false;
+    if (a.K % 64 != 0 || a.M * a.N < 64 * 64) return false;
+    const int64_t ks = a.K / 64, epb = fp4 ? 2 : 1;
+    if (a.x1.col_stride != 1 || a.x1_scale_mat.col_stride != 2 || a.x1_scale_mat.row_stride != ks * 2) return false;
+    if (((uintptr_t)a.x1.ptr | (uint64_t)(a.x1.row_stride / epb) | (uint64_t)(a.x1.batch_stride / epb)) % 16) return false;
+    if (a.K % 128 == 0 && ((uintptr_t)a.x1_scale_mat.ptr | (uint64_t)a.x1_scale_mat.row_stride | (uint64_t)a.x1_scale_mat.batch_stride) % 4) return false;
+    return true;
+}
+
+// Bytes behind the exact route's tables: the K-contiguous copies of an N-contiguous x2, then the padded copies of a K tail.
+static uint64_t mx_rest_bytes(const OpsnnQmmArgs& a0)
+{
+    if (a0.force_variant == OPSNN_VARIANT_PLAIN || opsnn_force_plain() || !mx_call_ok(a0)) return 0;
+    OpsnnQmmArgs a = a0;
+    uint64_t total = 0;
+    MxRelayout R;
+    if (mx_relayout_layout(a, R)) {
+        total = align_up(R.bytes, 256);
+        mx_relayout_view(a, R, (char*)(uintptr_t)256);   // any aligned address: only the layout matters below
+    }
+    MxPad L;
+    if (mx_pad_layout(a, L)) total += L.total;
+    return total;
+}
 
 // Workspace of an MX call: in front, what the exact route of MXFP8 needs (nothing for the other operand pairs), then the
-// padded or re-laid-out operand copies.
+// re-laid-out and padded operand copies.
 uint64_t mx_workspace_bytes(const OpsnnQmmArgs& a)
 {
     const bool matrix_cores = a.force_variant != OPSNN_VARIANT_PLAIN && !opsnn_force_plain();
     return (matrix_cores ? mx_exact_bytes(a) : 0) + mx_rest_bytes(a);
-}
-
-static uint64_t mx_rest_bytes(const OpsnnQmmArgs& a)
-{
-    MxPad L;
-    if (a.force_variant != OPSNN_VARIANT_PLAIN && !opsnn_force_plain() && mx_pad_layout(a, L)) return L.total;
-    if (a.x2.row_stride == 1 || a.K == 1) return 0;
-    if (a.x2.col_stride != 1 || a.x2.row_stride != a.N) return 0;
-    const uint64_t bits = a.x2_dtype == DT_E2M1 ? 4 : 8;
-    const uint64_t nb = a.x2.batch_stride == 0 ? 1 : (uint64_t)a.batch;
-    const uint64_t data = align_up((uint64_t)a.N * (uint64_t)a.K * bits / 8, 256) * nb;
-    const uint64_t ks = ((uint64_t)a.K + 63) / 64;
-    const uint64_t snb = a.x2_scale_mat.batch_stride == 0 ? 1 : (uint64_t)a.batch;
-    return data + align_up((uint64_t)a.N * ks * 2, 256) * snb;
 }
 
 void* weight_cache_blob(const void* src, const void* src2, int64_t K, int64_t N, int bits, int64_t nb, uint64_t bytes, hipStream_t st, bool* fresh);
@@ -166,6 +243,7 @@ int launch_mx_a8w4_mfma(const OpsnnQmmArgs& a, hipStream_t st);   // qmm_fp8_blo
 
 int launch_mx_mfma(const OpsnnQmmArgs& a0, hipStream_t st)
 {
+    if (!mx_call_ok(a0)) return OPSNN_NOT_TAKEN;
     OpsnnQmmArgs a = a0;
     const bool fp4 = a.x1_dtype == DT_E2M1 && a.x2_dtype == DT_E2M1;
     const bool fp8 = a.x1_dtype == DT_E4M3 && a.x2_dtype == DT_E4M3;
@@ -180,74 +258,52 @@ int launch_mx_mfma(const OpsnnQmmArgs& a0, hipStream_t st)
         a.workspace = mxx + front;
     }
     const bool exact = mxx && !opsnnGetFp8Fast();
-    if (a.x1_dtype == DT_E4M3 && a.x2_dtype == DT_E2M1) {   // fp8 x fp4: qmm_fp8_block.hip, behind the same padding of a K tail
-        MxPad L;
-        if (mx_pad_layout(a, L)) {
-            const int rc = mx_pad_prestep(a, L, st);
-            if (rc != 0) return rc;
+
+    // Pre-steps, planned in full before the first of them is launched: an N-contiguous x2 is re-laid out K-contiguous (into
+    // the weight cache's buffer for this operand when the cache is on -- a hit skips the passes -- else into the workspace);
+    // a K tail (K % 128 == 64) then continues on zero-padded copies of all four operands.
+    MxRelayout R;
+    const bool relayout = mx_relayout_layout(a, R);
+    if (!relayout && a.x2.row_stride != 1) return OPSNN_NOT_TAKEN;
+    OpsnnQmmArgs planned = a;
+    if (relayout) mx_relayout_view(planned, R, (char*)(uintptr_t)256);
+    MxPad L;
+    const bool pad = mx_pad_layout(planned, L);
+    if (!pad && planned.K % 128 != 0) return OPSNN_NOT_TAKEN;
+    if (planned.x2_scale_mat.col_stride != 2 || (fp4 || fp8 ? planned.x2_scale_mat.row_stride != planned.K / 64 * 2 : planned.x2_scale_mat.row_stride % 4 != 0)) return OPSNN_NOT_TAKEN;
+    if (pad && (!a.workspace || (uintptr_t)a.workspace % 16)) return OPSNN_NOT_TAKEN;
+    if (relayout) {
+        bool fresh = false;
+        char* w = (char*)weight_cache_blob(a.x2.ptr, a.x2_scale_mat.ptr, a.K, a.N, a.x2_dtype == DT_E2M1 ? 4 : 8, R.nb * 16 + R.snb, R.bytes, st, &fresh);
+        const bool cached = w != nullptr;
+        if (!cached) {
+            if (!a.workspace || (uintptr_t)a.workspace % 16) return OPSNN_NOT_TAKEN;
+            w = (char*)a.workspace;
+            a.workspace = w + align_up(R.bytes, 256);
         }
-        return launch_mx_a8w4_mfma(a, st);
+        if (!cached || fresh) {
+            const int rc = mx_relayout_run(a, R, w, st);
+            if (rc != 0) {
+                if (cached) weight_cache_abandon(w);
+                return rc;
+            }
+        }
+        if (cached && fresh) weight_cache_commit(w, st);
+        mx_relayout_view(a, R, w);
     }
-    if (!fp4 && !fp8) return OPSNN_NOT_TAKEN;
+    if (pad) {
+        if (!mx_pad_layout(a, L)) return OPSNN_NOT_TAKEN;   // (the same answer as for the planned view: its conditions do not look at x2's address beyond its alignment)
+        const int rc = mx_pad_prestep(a, L, st);
+        if (rc != 0) return rc;
+    }
+    if (a.x1_dtype == DT_E4M3 && a.x2_dtype == DT_E2M1) return launch_mx_a8w4_mfma(a, st);   // fp8 x fp4: qmm_fp8_block.hip
     // MXFP8 runs on the block kernel of qmm_fp8_block.hip in MX mode (16x16x128 instructions, 64 x 128 per wave, the
     // pipeline tuned for the fp8 block-scale path); the 32x32x64 tile kernel stays available on request
     // (OPSNN_VARIANT_MX_FP8_MFMA) for comparison.  The 8-bit forms of the matrix instruction sum their products with a
     // reduced-width aligner (measured: mean error 1e-5 of sum|terms| per instruction); fp4 products are exact in that
     // datapath.
-    if (a.out_dtype != DT_BF16 && a.out_dtype != DT_F16 && a.out_dtype != DT_F32) return OPSNN_NOT_TAKEN;
-    if (a.bias && a.bias_dtype != DT_F32) return OPSNN_NOT_TAKEN;
-    {
-        MxPad L;
-        if (mx_pad_layout(a, L)) {
-            const int rc = mx_pad_prestep(a, L, st);
-            if (rc != 0) return rc;
-        }
-    }
-    if (a.K % 128 != 0 || a.M * a.N < 64 * 64) return OPSNN_NOT_TAKEN;
     const int64_t ks = a.K / 64;  // scale pairs per row
-    if (a.x1.col_stride != 1 || a.x1_scale_mat.col_stride != 2 || a.x1_scale_mat.row_stride != ks * 2) return OPSNN_NOT_TAKEN;
     const int64_t epb = fp4 ? 2 : 1;  // elements per byte
-
-    if (a.x2.row_stride != 1) {
-        // x2 is [K, N] with N contiguous: re-lay data and scales out K-contiguous, into the weight cache's buffer for this
-        // operand when the cache is on (a hit skips the passes), else into the workspace
-        if (a.x2.col_stride != 1 || a.x2.row_stride != a.N) return OPSNN_NOT_TAKEN;
-        if (a.x2_scale_mat.row_stride != 2 || a.x2_scale_mat.col_stride != a.N * 2) return OPSNN_NOT_TAKEN;
-        if (a.x2.batch_stride != 0 && a.x2.batch_stride != a.K * a.N) return OPSNN_NOT_TAKEN;
-        const int64_t nb = a.x2.batch_stride == 0 ? 1 : a.batch;
-        const int64_t snb = a.x2_scale_mat.batch_stride == 0 ? 1 : a.batch;
-        if (snb != 1 && a.x2_scale_mat.batch_stride != ks * a.N * 2) return OPSNN_NOT_TAKEN;
-        const uint64_t data_one = align_up((uint64_t)a.N * a.K / epb, 256);
-        const uint64_t scale_one = align_up((uint64_t)a.N * ks * 2, 256);
-        bool fresh = false;
-        char* wdata = (char*)weight_cache_blob(a.x2.ptr, a.x2_scale_mat.ptr, a.K, a.N, fp4 ? 4 : 8, nb * 16 + snb,
-                                               data_one * (uint64_t)nb + scale_one * (uint64_t)snb, st, &fresh);
-        const bool cached = wdata != nullptr;
-        if (!cached) {
-            if (!a.workspace) return OPSNN_NOT_TAKEN;
-            wdata = (char*)a.workspace;
-        }
-        char* wscale = wdata + data_one * nb;
-        for (int64_t b = 0; b < nb && (!cached || fresh); b++) {  // per-batch because of the aligned pitch
-            const char* src = (const char*)a.x2.ptr + b * (a.K * a.N / epb);
-            int rc = fp4 ? opsnnTranspose4(src, wdata + b * data_one, a.K, a.N, 1, st) : opsnnTranspose8(src, wdata + b * data_one, a.K, a.N, 1, st);
-            if (rc != 0) {
-                if (cached) weight_cache_abandon(wdata);
-                return rc;
-            }
-        }
-        for (int64_t b = 0; b < snb && (!cached || fresh); b++) {
-            dim3 grid((unsigned)((a.N + 31) / 32), (unsigned)((ks + 31) / 32), 1);
-            hipLaunchKernelGGL(transpose16_kernel, grid, dim3(256), 0, st,
-                               (const uint16_t*)((const char*)a.x2_scale_mat.ptr + b * (ks * a.N * 2)),
-                               (uint16_t*)(wscale + b * scale_one), ks, a.N);
-        }
-        if (cached && fresh) weight_cache_commit(wdata, st);
-        a.x2.ptr = wdata; a.x2.row_stride = 1; a.x2.col_stride = a.K; a.x2.batch_stride = nb == 1 ? 0 : (int64_t)(data_one * epb);
-        a.x2_scale_mat.ptr = wscale; a.x2_scale_mat.row_stride = ks * 2; a.x2_scale_mat.col_stride = 2;
-        a.x2_scale_mat.batch_stride = snb == 1 ? 0 : (int64_t)scale_one;
-    }
-    if (a.x2_scale_mat.col_stride != 2 || a.x2_scale_mat.row_stride != ks * 2) return OPSNN_NOT_TAKEN;
 
     QgemmParams g{};
     g.a = (const int8_t*)a.x1.ptr; g.b = (const int8_t*)a.x2.ptr;

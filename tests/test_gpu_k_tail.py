@@ -117,6 +117,37 @@ def test_mx_k_tail(gpu, M, K, N, fp4, batch, bias):
     m.lib().aclDestroyAclOpExecutor(ex)
 
 
+@pytest.mark.parametrize("M,K,N,fp4,batch", [
+    (197, 960, 854, True, 1),      # MXFP4, ragged rows and columns
+    (256, 1472, 384, False, 1),    # MXFP8
+    (128, 192, 256, True, 2),      # batched
+    (64, 64, 128, False, 3),       # half a K tile, batched
+])
+def test_mx_k_tail_n_contiguous_x2(gpu, M, K, N, fp4, batch):
+    """K % 128 == 64 with x2 stored [K, N] (N contiguous, scales [K/64, N, 2]): x2 and its scales are first re-laid out
+    K-contiguous, then all four operands are padded as for K-contiguous callers; the matrix-core kernels run (the log line
+    of a plain-kernel landing must not appear: checked through the workspace plan, which is zero for the plain route)."""
+    m = gpu
+    print(f"case mx K tail, N-contiguous x2 M={M} K={K} N={N} fp4={fp4} batch={batch}", flush=True)
+    inp = cases.make_mx_inputs(m, M, K, N, K + N + 1, False, fp4, batch=batch)
+    b = np.random.default_rng(5).normal(0, 1, N).astype(np.float32)
+    want = cases.oracle_mx(m, inp, M, K, N, False, m.ACL_BF16, b)
+    got = cases.run_mx_aclnn(m, inp, M, K, N, False, m.ACL_BF16, b)
+    check_close(got, want, orc.BF16, "mx with a K tail, N-contiguous x2")
+    adt = m.ACL_FLOAT4_E2M1 if fp4 else m.ACL_FLOAT8_E4M3FN
+    bs = (batch,) if batch > 1 else ()
+    d = {k: m.DeviceBuffer(host=v) for k, v in inp.items() if isinstance(v, np.ndarray)}
+    x1 = m.Tensor(bs + (M, K), adt, d["x1"]); x2 = m.Tensor(bs + (K, N), adt, d["x2"])
+    s1 = m.Tensor(bs + inp["s1"].shape[1:], m.ACL_FLOAT8_E8M0, d["s1"]); s2 = m.Tensor(bs + inp["s2"].shape[1:], m.ACL_FLOAT8_E8M0, d["s2"])
+    o = m.Tensor(bs + (M, N), m.ACL_BF16, m.DeviceBuffer(batch * M * N * 2))
+    rc, ws, ex = m.quant_matmul_v5_get_workspace(x1, x2, s1, s2, o, transpose_x2=False, group_size=(1 << 32) | (1 << 16) | 32)
+    up = lambda v: -(-v // 256) * 256
+    relaid = up(batch * up(N * K // (2 if fp4 else 1)) + batch * up(N * (K // 64) * 2))
+    plan = relaid + _mx_pad_bytes(M, K, N, fp4, batch) + (0 if fp4 else _mx_exact_bytes(M, K, N, batch))
+    assert rc == 0 and ws == plan, (rc, ws, plan)
+    m.lib().aclDestroyAclOpExecutor(ex)
+
+
 @pytest.mark.parametrize("M,K,N", [(300, 960, 260), (128, 192, 256), (16, 1984, 512)])
 def test_mx_fp8_fp4_k_tail(gpu, M, K, N):
     """fp8 x fp4 MX with K % 128 == 64: the same padded copies (x1 rows of K + 64 bytes, x2 rows of half that), then the
