@@ -11,8 +11,8 @@
 // Fast paths: operands and scales K-contiguous, K % 128 == 0, 16-bit output.  fp4: qgemm_core.hip.h, MODE_MXFP4
 // (K % 512 == 0 takes 256-element K tiles, otherwise 128-element ones); fp8: the MX mode of the kernel in
 // qmm_fp8_block.hip.  An N-contiguous x2 (data [K, N], scales [K/64, N, 2]) is first re-laid out into the
-// workspace.  K % 128 == 64: both operands and both scale tables (x2's after that re-layout, if it was needed) are first
-// copied into the workspace with one more scale pair per row, the new elements zero and their scales 2^0 (zero products
+// workspace.  K % 128 != 0 (K a whole number of 32-element blocks): both operands and both scale tables (x2's after that re-layout, if it was needed) are first
+// copied into the workspace with K rounded up to 128, the new elements zero and their scales a repeat of the row's last one (zero products
 // change no sum).  All of this is planned before the first pre-step is launched.  Everything else runs the plain kernel.
 #include "launch.h"
 #include "qgemm_core.hip.h"
@@ -54,8 +54,11 @@ namespace opsnn {
 static inline uint64_t align_up(uint64_t v, uint64_t a) { return (v + a - 1) / a * a; }
 extern "C" bool opsnn_force_plain();   // dispatch.hip
 
-// ---- K % 128 == 64 ----
-// rows of kb bytes (pitch ld) -> rows of kbp bytes, the tail filled with the byte `fill`; E = bytes per thread
+// ---- K % 128 != 0 (whole MX blocks: K % 32 == 0) ----
+// rows of kb bytes (pitch ld) -> rows of kbp bytes, the tail filled with the byte `fill`; E = bytes per thread.  E == 16:
+// kb is a multiple of 16.  E == 2 (scale rows): kb counts the bytes that scale existing elements; the second byte of a
+// source pair may lie past it (K % 64 == 32) and is replaced like the rest of the tail, whatever the caller left there.
+// Scale tails repeat the row's last valid byte; data tails are zero.
 template <int E>
 __global__ __launch_bounds__(256) void mx_pad_rows_kernel(const uint8_t* __restrict__ src, int64_t ld, int64_t bs, uint8_t* __restrict__ dst,
                                                           int64_t rows, int64_t kb, int64_t kbp, uint32_t fill)
@@ -64,8 +67,18 @@ __global__ __launch_bounds__(256) void mx_pad_rows_kernel(const uint8_t* __restr
     if (c * E >= kbp || r >= rows) return;
     const uint8_t* s = src + (int64_t)blockIdx.z * bs + r * ld + c * E;
     uint8_t* d = dst + ((int64_t)blockIdx.z * rows + r) * kbp + c * E;
-    if constexpr (E == 16) *(uint4*)d = c * E < kb ? *(const uint4*)s : make_uint4(fill, fill, fill, fill);
-    else *(uint16_t*)d = c * E < kb ? *(const uint16_t*)s : (uint16_t)fill;
+    if constexpr (E == 16) {
+        *(uint4*)d = c * E < kb ? *(const uint4*)s : make_uint4(fill, fill, fill, fill);
+    } else {
+        // the tail repeats the row's last valid scale byte (its elements are zero, so any finite scale will do, and this
+        // one leaves the spread of the row's scales as it was: the exact MXFP8 route looks at that spread)
+        (void)fill;
+        const uint32_t last = (src + (int64_t)blockIdx.z * bs + r * ld)[kb - 1];
+        uint16_t v = (uint16_t)(last | (last << 8));
+        if (c * 2 + 1 < kb) v = *(const uint16_t*)s;
+        else if (c * 2 < kb) v = (uint16_t)((v & 0xFF00u) | s[0]);
+        *(uint16_t*)d = v;
+    }
 }
 
 struct MxPad {
@@ -78,10 +91,10 @@ static bool mx_pad_layout(const OpsnnQmmArgs& a, MxPad& L)
 {
     const bool fp4 = a.x1_dtype == DT_E2M1 && a.x2_dtype == DT_E2M1, fp8 = a.x1_dtype == DT_E4M3 && a.x2_dtype == DT_E4M3;
     const bool a8w4 = a.x1_dtype == DT_E4M3 && a.x2_dtype == DT_E2M1;   // the matrix-core kernel of that mode: 16-bit output, fp32 or 16-bit bias
-    if ((!fp4 && !fp8 && !a8w4) || a.K % 128 != 64 || a.M * a.N < 64 * 64) return false;
+    if ((!fp4 && !fp8 && !a8w4) || a.K % 128 == 0 || a.K % 32 != 0 || a.M * a.N < 64 * 64) return false;
     if (a.out_dtype != DT_BF16 && a.out_dtype != DT_F16 && !(a.out_dtype == DT_F32 && !a8w4)) return false;
     if (a.bias && a.bias_dtype != DT_F32 && !(a8w4 && (a.bias_dtype == DT_BF16 || a.bias_dtype == DT_F16))) return false;
-    const int64_t epb1 = a.x1_dtype == DT_E2M1 ? 2 : 1, epb2 = a.x2_dtype == DT_E2M1 ? 2 : 1, ks = a.K / 64;   // elements per byte
+    const int64_t epb1 = a.x1_dtype == DT_E2M1 ? 2 : 1, epb2 = a.x2_dtype == DT_E2M1 ? 2 : 1, ks = (a.K + 63) / 64;   // elements per byte; scale pairs per row
     if (a.x1.col_stride != 1 || a.x2.row_stride != 1) return false;
     if (a.x1_scale_mat.col_stride != 2 || a.x1_scale_mat.row_stride != ks * 2) return false;
     if (a.x2_scale_mat.col_stride != 2 || a.x2_scale_mat.row_stride != ks * 2) return false;
@@ -91,7 +104,7 @@ static bool mx_pad_layout(const OpsnnQmmArgs& a, MxPad& L)
          (uint64_t)(a.x1.batch_stride / epb1) | (uint64_t)(a.x2.batch_stride / epb2)) % 16) return false;
     if (((uintptr_t)a.x1_scale_mat.ptr | (uintptr_t)a.x2_scale_mat.ptr | (uint64_t)a.x1_scale_mat.batch_stride | (uint64_t)a.x2_scale_mat.batch_stride) % 2) return false;
     if ((a.M + 3) / 4 > 65535 || (a.N + 3) / 4 > 65535) return false;
-    L.Kp = a.K + 64;
+    L.Kp = (a.K + 127) / 128 * 128;
     L.nb1 = a.x1.batch_stride == 0 && a.batch > 1 ? 1 : a.batch;
     L.nb2 = a.x2.batch_stride == 0 ? 1 : a.batch;
     L.snb1 = a.x1_scale_mat.batch_stride == 0 && a.batch > 1 ? 1 : a.batch;
@@ -109,7 +122,8 @@ static int mx_pad_prestep(OpsnnQmmArgs& a, const MxPad& L, hipStream_t st)
 {
     if (!a.workspace || (uintptr_t)a.workspace % 16) return OPSNN_NOT_TAKEN;
     const int64_t epb1 = a.x1_dtype == DT_E2M1 ? 2 : 1, epb2 = a.x2_dtype == DT_E2M1 ? 2 : 1;
-    const int64_t kb1 = a.K / epb1, kbp1 = L.Kp / epb1, kb2 = a.K / epb2, kbp2 = L.Kp / epb2, ks2 = a.K / 64 * 2, ksp2 = L.Kp / 64 * 2;
+    const int64_t kb1 = a.K / epb1, kbp1 = L.Kp / epb1, kb2 = a.K / epb2, kbp2 = L.Kp / epb2, ks2 = (a.K + 63) / 64 * 2, ksp2 = L.Kp / 64 * 2;
+    const int64_t sv = a.K / 32;   // scale bytes per row that scale existing elements
     uint8_t* w = (uint8_t*)a.workspace;
     auto grid = [](int64_t pieces, int64_t rows, int64_t nb) { return dim3((unsigned)((pieces + 63) / 64), (unsigned)((rows + 3) / 4), (unsigned)nb); };
     hipLaunchKernelGGL(mx_pad_rows_kernel<16>, grid(kbp1 / 16, a.M, L.nb1), dim3(256), 0, st, (const uint8_t*)a.x1.ptr, a.x1.row_stride / epb1,
@@ -117,9 +131,9 @@ static int mx_pad_prestep(OpsnnQmmArgs& a, const MxPad& L, hipStream_t st)
     hipLaunchKernelGGL(mx_pad_rows_kernel<16>, grid(kbp2 / 16, a.N, L.nb2), dim3(256), 0, st, (const uint8_t*)a.x2.ptr, a.x2.col_stride / epb2,
                        a.x2.batch_stride / epb2, w + L.o_x2, a.N, kb2, kbp2, 0u);
     hipLaunchKernelGGL(mx_pad_rows_kernel<2>, grid(ksp2 / 2, a.M, L.snb1), dim3(256), 0, st, (const uint8_t*)a.x1_scale_mat.ptr, ks2,
-                       a.x1_scale_mat.batch_stride, w + L.o_s1, a.M, ks2, ksp2, 0x7f7fu);
+                       a.x1_scale_mat.batch_stride, w + L.o_s1, a.M, sv, ksp2, 0x7f7fu);
     hipLaunchKernelGGL(mx_pad_rows_kernel<2>, grid(ksp2 / 2, a.N, L.snb2), dim3(256), 0, st, (const uint8_t*)a.x2_scale_mat.ptr, ks2,
-                       a.x2_scale_mat.batch_stride, w + L.o_s2, a.N, ks2, ksp2, 0x7f7fu);
+                       a.x2_scale_mat.batch_stride, w + L.o_s2, a.N, sv, ksp2, 0x7f7fu);
     const hipError_t e = hipGetLastError();
     if (e != hipSuccess) return (int)e;
     a.x1 = OpsnnMat{w, L.Kp, 1, L.nb1 == 1 && a.batch > 1 ? 0 : a.M * L.Kp};
@@ -143,8 +157,8 @@ struct MxRelayout {
 
 static bool mx_relayout_layout(const OpsnnQmmArgs& a, MxRelayout& R)
 {
-    if (a.x2.row_stride == 1 || a.K == 1 || a.K % 64 != 0) return false;
-    const int64_t ks = a.K / 64, epb = a.x2_dtype == DT_E2M1 ? 2 : 1;
+    if (a.x2.row_stride == 1 || a.K == 1 || a.K % 32 != 0) return false;
+    const int64_t ks = (a.K + 63) / 64, epb = a.x2_dtype == DT_E2M1 ? 2 : 1;
     if (a.x2.col_stride != 1 || a.x2.row_stride != a.N) return false;
     if (epb == 2 && (a.N & 1)) return false;   // the 4-bit transposition works on byte pairs
     if (a.x2_scale_mat.row_stride != 2 || a.x2_scale_mat.col_stride != a.N * 2) return false;
@@ -162,7 +176,7 @@ static bool mx_relayout_layout(const OpsnnQmmArgs& a, MxRelayout& R)
 // `a` as the same call on the copies at `w` (which the passes of mx_relayout_run fill)
 static void mx_relayout_view(OpsnnQmmArgs& a, const MxRelayout& R, char* w)
 {
-    const int64_t ks = a.K / 64, epb = a.x2_dtype == DT_E2M1 ? 2 : 1;
+    const int64_t ks = (a.K + 63) / 64, epb = a.x2_dtype == DT_E2M1 ? 2 : 1;
     char* wscale = w + R.data_one * R.nb;
     a.x2.ptr = w; a.x2.row_stride = 1; a.x2.col_stride = a.K; a.x2.batch_stride = R.nb == 1 ? 0 : (int64_t)(R.data_one * epb);
     a.x2_scale_mat.ptr = wscale; a.x2_scale_mat.row_stride = ks * 2; a.x2_scale_mat.col_stride = 2;
@@ -171,7 +185,7 @@ static void mx_relayout_view(OpsnnQmmArgs& a, const MxRelayout& R, char* w)
 
 static int mx_relayout_run(const OpsnnQmmArgs& a, const MxRelayout& R, char* w, hipStream_t st)
 {
-    const int64_t ks = a.K / 64, epb = a.x2_dtype == DT_E2M1 ? 2 : 1;
+    const int64_t ks = (a.K + 63) / 64, epb = a.x2_dtype == DT_E2M1 ? 2 : 1;
     char* wscale = w + R.data_one * R.nb;
     for (int64_t b = 0; b < R.nb; b++) {  // per batch because of the aligned pitch
         const char* src = (const char*)a.x2.ptr + b * (a.K * a.N / epb);
@@ -196,15 +210,15 @@ static bool mx_call_ok(const OpsnnQmmArgs& a)
     if (a8w4) {   // launch_mx_a8w4_mfma (qmm_fp8_block.hip): a tile kernel, and a streaming kernel for up to 32 rows
         if (a.out_dtype != DT_BF16 && a.out_dtype != DT_F16) return false;
         if (a.bias && a.bias_dtype != DT_F32 && a.bias_dtype != DT_BF16 && a.bias_dtype != DT_F16) return false;
-        if (a.K % 64 != 0 || a.x1.col_stride != 1 || a.x1_scale_mat.col_stride != 2) return false;
+        if (a.K % 32 != 0 || a.x1.col_stride != 1 || a.x1_scale_mat.col_stride != 2) return false;
         const bool few_rows = a.M <= 32 && a.N >= 256 && a.batch == 1;
         if (!few_rows && a.M * a.N < 64 * 64) return false;
         return (((uintptr_t)a.x1.ptr | (uint64_t)a.x1.row_stride | (uint64_t)a.x1.batch_stride) % 16) == 0;
     }
     if (a.out_dtype != DT_BF16 && a.out_dtype != DT_F16 && a.out_dtype != DT_F32) return false;
     if (a.bias && a.bias_dtype != DT_F32) return false;
-    if (a.K % 64 != 0 || a.M * a.N < 64 * 64) return false;
-    const int64_t ks = a.K / 64, epb = fp4 ? 2 : 1;
+    if (a.K % 32 != 0 || a.M * a.N < 64 * 64) return false;
+    const int64_t ks = (a.K + 63) / 64, epb = fp4 ? 2 : 1;
     if (a.x1.col_stride != 1 || a.x1_scale_mat.col_stride != 2 || a.x1_scale_mat.row_stride != ks * 2) return false;
     if (((uintptr_t)a.x1.ptr | (uint64_t)(a.x1.row_stride / epb) | (uint64_t)(a.x1.batch_stride / epb)) % 16) return false;
     if (a.K % 128 == 0 && ((uintptr_t)a.x1_scale_mat.ptr | (uint64_t)a.x1_scale_mat.row_stride | (uint64_t)a.x1_scale_mat.batch_stride) % 4) return false;
@@ -270,7 +284,7 @@ int launch_mx_mfma(const OpsnnQmmArgs& a0, hipStream_t st)
     MxPad L;
     const bool pad = mx_pad_layout(planned, L);
     if (!pad && planned.K % 128 != 0) return OPSNN_NOT_TAKEN;
-    if (planned.x2_scale_mat.col_stride != 2 || (fp4 || fp8 ? planned.x2_scale_mat.row_stride != planned.K / 64 * 2 : planned.x2_scale_mat.row_stride % 4 != 0)) return OPSNN_NOT_TAKEN;
+    if (planned.x2_scale_mat.col_stride != 2 || (fp4 || fp8 ? planned.x2_scale_mat.row_stride != (planned.K + 63) / 64 * 2 : planned.x2_scale_mat.row_stride % 4 != 0)) return OPSNN_NOT_TAKEN;
     if (pad && (!a.workspace || (uintptr_t)a.workspace % 16)) return OPSNN_NOT_TAKEN;
     if (relayout) {
         bool fresh = false;

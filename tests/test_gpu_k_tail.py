@@ -75,7 +75,7 @@ def test_fp8_blockscale_k_tail(gpu, M, K, N, tB, gsM, fast):
 
 
 def _mx_pad_bytes(M, K, N, fp4, batch=1):
-    Kp, epb = K + 64, 2 if fp4 else 1
+    Kp, epb = -(-K // 128) * 128, 2 if fp4 else 1
     up = lambda v: -(-v // 256) * 256
     return up(batch * M * Kp // epb) + up(batch * N * Kp // epb) + up(batch * M * (Kp // 64) * 2) + up(batch * N * (Kp // 64) * 2)
 
@@ -93,13 +93,20 @@ def _mx_exact_bytes(M, K, N, batch=1):
     (256, 1472, 384, False, 1, False),   # MXFP8, 11.5 K tiles
     (128, 192, 256, True, 2, True),      # batched, 1.5 K tiles
     (64, 64, 64, False, 1, False),       # half a K tile
+    (384, 544, 512, True, 1, True),      # K % 64 == 32: the last scale pair is half used
+    (200, 96, 320, False, 2, True),      # the same for MXFP8, batched, three quarters of a K tile
+    (130, 32, 70, True, 1, False),       # one MX block
 ])
 def test_mx_k_tail(gpu, M, K, N, fp4, batch, bias):
-    """MX operands with K % 128 == 64 (a whole number of scale pairs, half a K tile left over): both operands and both
-    scale tables are copied with one more pair per row (zero elements, scales 2^0), then the matrix-core kernels run."""
+    """MX operands with K % 128 != 0 (whole 32-element blocks): both operands and both scale tables are copied with K
+    rounded up to 128 (zero elements; their scales repeat the row's last one, also in the unused half of a half-used
+    pair, which the caller may have left at any value), then the matrix-core kernels run."""
     m = gpu
     print(f"case mx K tail M={M} K={K} N={N} fp4={fp4} batch={batch} bias={bias}", flush=True)
     inp = cases.make_mx_inputs(m, M, K, N, K + N, True, fp4, batch=batch)
+    if K % 64:   # the byte behind the last block scales nothing: a NaN code there must not reach any sum
+        inp["s1"][..., -1, 1] = 0xFF
+        inp["s2"][..., -1, 1] = 0xFF
     b = np.random.default_rng(3).normal(0, 1, N).astype(np.float32) if bias else None
     want = cases.oracle_mx(m, inp, M, K, N, True, m.ACL_BF16, b)
     got = cases.run_mx_aclnn(m, inp, M, K, N, True, m.ACL_BF16, b)
@@ -122,9 +129,11 @@ def test_mx_k_tail(gpu, M, K, N, fp4, batch, bias):
     (256, 1472, 384, False, 1),    # MXFP8
     (128, 192, 256, True, 2),      # batched
     (64, 64, 128, False, 3),       # half a K tile, batched
+    (384, 544, 512, True, 1),      # K % 64 == 32
+    (96, 96, 192, False, 2),       # the same for MXFP8, batched
 ])
 def test_mx_k_tail_n_contiguous_x2(gpu, M, K, N, fp4, batch):
-    """K % 128 == 64 with x2 stored [K, N] (N contiguous, scales [K/64, N, 2]): x2 and its scales are first re-laid out
+    """K % 128 != 0 with x2 stored [K, N] (N contiguous, scales [K/64, N, 2]): x2 and its scales are first re-laid out
     K-contiguous, then all four operands are padded as for K-contiguous callers; the matrix-core kernels run (the log line
     of a plain-kernel landing must not appear: checked through the workspace plan, which is zero for the plain route)."""
     m = gpu
@@ -142,15 +151,15 @@ def test_mx_k_tail_n_contiguous_x2(gpu, M, K, N, fp4, batch):
     o = m.Tensor(bs + (M, N), m.ACL_BF16, m.DeviceBuffer(batch * M * N * 2))
     rc, ws, ex = m.quant_matmul_v5_get_workspace(x1, x2, s1, s2, o, transpose_x2=False, group_size=(1 << 32) | (1 << 16) | 32)
     up = lambda v: -(-v // 256) * 256
-    relaid = up(batch * up(N * K // (2 if fp4 else 1)) + batch * up(N * (K // 64) * 2))
+    relaid = up(batch * up(N * K // (2 if fp4 else 1)) + batch * up(N * -(-K // 64) * 2))
     plan = relaid + _mx_pad_bytes(M, K, N, fp4, batch) + (0 if fp4 else _mx_exact_bytes(M, K, N, batch))
     assert rc == 0 and ws == plan, (rc, ws, plan)
     m.lib().aclDestroyAclOpExecutor(ex)
 
 
-@pytest.mark.parametrize("M,K,N", [(300, 960, 260), (128, 192, 256), (16, 1984, 512)])
+@pytest.mark.parametrize("M,K,N", [(300, 960, 260), (128, 192, 256), (16, 1984, 512), (96, 544, 320)])
 def test_mx_fp8_fp4_k_tail(gpu, M, K, N):
-    """fp8 x fp4 MX with K % 128 == 64: the same padded copies (x1 rows of K + 64 bytes, x2 rows of half that), then the
+    """fp8 x fp4 MX with K % 128 != 0: the same padded copies (x1 rows of K + 64 bytes, x2 rows of half that), then the
     matrix-core kernel of the mode (the stream kernel with 16 rows): the stated bar."""
     m = gpu
     print(f"case fp8 x fp4 mx K tail M={M} K={K} N={N}", flush=True)
@@ -160,7 +169,7 @@ def test_mx_fp8_fp4_k_tail(gpu, M, K, N):
     check_close(got, want, orc.F16, "fp8 x fp4 mx with a K tail")
     # phase 1 plans the four padded copies
     up = lambda v: -(-v // 256) * 256
-    Kp = K + 64
+    Kp = -(-K // 128) * 128
     d = {k: m.DeviceBuffer(host=v) for k, v in inp.items()}
     x1 = m.Tensor((M, K), m.ACL_FLOAT8_E4M3FN, d["x1"]); x2 = m.Tensor((N, K), m.ACL_FLOAT4_E2M1, d["x2"])
     s1 = m.Tensor(inp["s1"].shape, m.ACL_FLOAT8_E8M0, d["s1"]); s2 = m.Tensor(inp["s2"].shape, m.ACL_FLOAT8_E8M0, d["s2"])
