@@ -176,6 +176,12 @@ OPSNN_API int opsnnTranspose8(const void* src, void* dst, int64_t rows, int64_t 
 /* Same for 4-bit elements packed two per byte along the last axis (low nibble = even index);
  * rows and cols must be even. */
 OPSNN_API int opsnnTranspose4(const void* src, void* dst, int64_t rows, int64_t cols, int64_t batch, void* stream);
+/* The dense copy of a strided view of packed 4-bit elements: dst[b, r, c] (two per byte, cols even) = element
+ * offset + b * batch_stride + r * row_stride + c * col_stride of the storage at base (offset and strides in elements, none
+ * negative).  What aclnnQuantMatmulV5 does to a non-contiguous 4-bit operand before anything else, in place of the
+ * reference's l0op::Contiguous (matmul/quant_batch_matmul_v4/op_host/op_api/quant_matmul_common_check.cpp:106-123). */
+OPSNN_API int opsnnGather4(const void* base, int64_t offset, int64_t batch, int64_t rows, int64_t cols, int64_t batch_stride,
+                           int64_t row_stride, int64_t col_stride, void* dst, void* stream);
 
 /* The same for 16-bit elements (pairs of e8m0 MX scales, 16-bit group scales). */
 OPSNN_API int opsnnTranspose16(const void* src, void* dst, int64_t rows, int64_t cols, int64_t batch, void* stream);

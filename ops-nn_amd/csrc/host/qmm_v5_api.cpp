@@ -73,11 +73,17 @@ struct Ctx {
 
 // A matrix operand whose view is neither dense nor a dense transpose, but regular: 8-bit elements, positive strides on
 // the last two dims, and batch dims that collapse into one stride.  The reference makes such a view contiguous by a copy
-// (quant_matmul_common_check.cpp:106-123); here the kernels take the strides as they are (the matrix-core route gathers
-// the operand into the workspace, the plain kernels index it directly).
+// (quant_matmul_common_check.cpp:106-123); here the kernels take the strides of an 8-bit operand as they are (the
+// matrix-core route gathers the operand into the workspace, the plain kernels index it directly), and a 4-bit operand is
+// copied densely into the front of the workspace before anything else.
 bool regular_strided_matrix(const TView& t)
 {
-    if (t.rank() < 2 || dtype_bits(t.dtype) != 8) return false;
+    // 8-bit operands: the kernels take the strides; 4-bit operands (also in their INT32 carriers, whose eight elements per
+    // word must stay together): gathered into a dense copy in front of the workspace by phase 2
+    const int bits = dtype_bits(t.dtype);
+    if (t.rank() < 2 || (bits != 8 && bits != 4 && t.dtype != ACL_INT32)) return false;
+    if (t.dtype == ACL_INT32 && t.stride(-1) != 1) return false;
+    if (bits == 4 && (t.dim(-1) % 2) != 0) return false;
     if (t.stride(-1) < 1 || t.stride(-2) < 1) return false;
     for (int64_t i = t.rank() - 4; i >= 0; i--)
         if (t.strides[(size_t)i] != t.strides[(size_t)i + 1] * t.shape[(size_t)i + 1]) return false;
@@ -605,6 +611,23 @@ extern "C" aclnnStatus aclnnQuantMatmulV5GetWorkspaceSize(const aclTensor* x1, c
     // ---- route (aclnn_quant_matmul_v5.cpp:1163-1174) and build the launch plan ----
     OpsnnQmmArgs& a = ex->qmm;
     a.M = c.M; a.N = c.N; a.K = c.K1;
+    // a strided 4-bit operand: phase 2 gathers it; from here on the view is the dense copy (its address is filled in then)
+    auto plan_gather = [&](TView& t, int which) {
+        if (!is_4bit(t.dtype) || is_contiguous(t)) return;
+        auto& g = ex->gather[which];
+        g.active = true; g.base = t.data; g.off = t.offset;
+        g.rows = t.dim(-2); g.cols = t.dim(-1); g.rs = t.stride(-2); g.cs = t.stride(-1);
+        g.nb = 1;
+        for (int64_t i = 0; i < t.rank() - 2; i++) g.nb *= t.dim(i);
+        g.bs = t.rank() > 2 ? t.stride(-3) : 0;
+        g.bytes = (uint64_t)(g.nb * g.rows * g.cols / 2);
+        t.offset = 0;
+        int64_t st = 1;
+        for (int64_t i = t.rank() - 1; i >= 0; i--) { t.strides[(size_t)i] = st; st *= t.shape[(size_t)i]; }
+        t.data = (void*)(uintptr_t)256;   // any aligned non-null address until phase 2 knows the workspace
+    };
+    plan_gather(c.x1, 0);
+    plan_gather(c.x2, 1);
     a.x1 = mat_of(c.x1, c.tA);
     a.x2 = mat_of(c.x2, c.tB);
     a.x1_dtype = c.x1.dtype; a.x2_dtype = c.x2.dtype;
@@ -694,7 +717,8 @@ extern "C" aclnnStatus aclnnQuantMatmulV5GetWorkspaceSize(const aclTensor* x1, c
              dtype_name(c.x1.dtype), dtype_name(c.x2.dtype), dtype_name(c.x2s.dtype), dtype_name(c.out.dtype));
     }
     if (general_broadcast) {
-        if (!is_contiguous(c.x1) || !is_contiguous(c.x2)) INVALID("%s: batch dims that broadcast partially need dense x1 and x2", kApi);
+        if (!is_contiguous(c.x1) || !is_contiguous(c.x2) || ex->gather[0].active || ex->gather[1].active)
+            INVALID("%s: batch dims that broadcast partially need dense x1 and x2", kApi);
         if (c.bias.present && c.bias.rank() == 3) INVALID("%s: a 3-D bias cannot go with partially broadcast batch dims", kApi);
         const int64_t nb = c.out.rank() - 2, r1 = c.x1.rank() - 2, r2 = c.x2.rank() - 2;
         std::vector<int64_t> od((size_t)nb), d1((size_t)nb, 1), d2((size_t)nb, 1);
@@ -742,7 +766,7 @@ extern "C" aclnnStatus aclnnQuantMatmulV5GetWorkspaceSize(const aclTensor* x1, c
         a.x1.batch_stride = ex->batch_runs[0].x1.batch_stride;
         a.x2.batch_stride = ex->batch_runs[0].x2.batch_stride;
     }
-    ex->workspace_size = opsnnQmmWorkspace(&a, mode);
+    ex->workspace_size = ex->gather_front() + opsnnQmmWorkspace(&a, mode);
     *workspaceSize = ex->workspace_size;
     *executor = (aclOpExecutor*)executor_publish(ex.release());
     return ACLNN_SUCCESS;
@@ -759,18 +783,31 @@ extern "C" aclnnStatus aclnnQuantMatmulV5(void* workspace, uint64_t workspaceSiz
     if (ex->kind == OpKind::None) return ACLNN_SUCCESS;
     if (ex->workspace_size > 0 && (!workspace || workspaceSize < ex->workspace_size))
         INVALID("aclnnQuantMatmulV5: workspace of %lu bytes required", (unsigned long)ex->workspace_size);
-    ex->qmm.workspace = ex->workspace_size ? workspace : nullptr;
     if (!ex->qmm.x1.ptr || !ex->qmm.x2.ptr || !ex->qmm.out) INVALID("aclnnQuantMatmulV5: a tensor has no device address");
     int rc = 0;
-    // a FRACTAL_NZ x2 is re-written into the workspace on every call: an address the weight cache must not key on
-    WeightCacheScope cache_scope(ex->nz.active);
+    // strided 4-bit operands first become dense copies at the front of the workspace
+    char* w = (char*)workspace;
+    for (int i = 0; i < 2; i++) {
+        const auto& g = ex->gather[i];
+        if (!g.active) continue;
+        if (!g.base) INVALID("aclnnQuantMatmulV5: a tensor has no device address");
+        rc = opsnnGather4(g.base, g.off, g.nb, g.rows, g.cols, g.bs, g.rs, g.cs, w, stream);
+        if (rc != 0) FAIL(ACLNN_ERR_RUNTIME_ERROR, "%s: gathering the strided 4-bit %s failed with code %d", ex->api, i ? "x2" : "x1", rc);
+        (i ? ex->qmm.x2 : ex->qmm.x1).ptr = w;
+        w += (g.bytes + 255) / 256 * 256;
+    }
+    const uint64_t front = ex->gather_front();
+    ex->qmm.workspace = ex->workspace_size > front ? w : nullptr;
+    // a FRACTAL_NZ x2 is re-written into the workspace on every call, and so is a gathered one: addresses the weight cache
+    // must not key on
+    WeightCacheScope cache_scope(ex->nz.active || ex->gather[1].active);
     if (ex->nz.active) {   // x2 arrived in FRACTAL_NZ (aclnnQuantMatmulWeightNz): lay it out as ND in the front of the workspace
         const void* nd = nullptr;
         void* rest = nullptr;
-        rc = run_nz_step(*ex, workspace, stream, &nd, &rest);
+        rc = run_nz_step(*ex, w, stream, &nd, &rest);
         if (rc != 0) FAIL(ACLNN_ERR_RUNTIME_ERROR, "%s: FRACTAL_NZ re-layout failed with code %d", ex->api, rc);
         ex->qmm.x2.ptr = nd;
-        ex->qmm.workspace = ex->workspace_size > nz_front_bytes(*ex) ? rest : nullptr;
+        ex->qmm.workspace = ex->workspace_size > front + nz_front_bytes(*ex) ? rest : nullptr;
     }
     auto launch = [&](const OpsnnQmmArgs& q) -> int {
         switch (ex->kind) {

@@ -51,9 +51,34 @@ __global__ __launch_bounds__(256) void transpose4_kernel(const uint8_t* __restri
     }
 }
 
+// dst (dense [batch, rows, cols], two elements per byte, low nibble = even column) = the 4-bit elements at
+// off + b * bs + r * rs + c * cs (in elements) of the packed storage at base: any view whose batch dims collapse into one stride
+__global__ __launch_bounds__(256) void gather4_kernel(const uint8_t* __restrict__ base, int64_t off, int64_t rows, int64_t cols,
+                                                      int64_t bs, int64_t rs, int64_t cs, uint8_t* __restrict__ dst)
+{
+    const int64_t cb = (int64_t)blockIdx.x * 256 + threadIdx.x, b = blockIdx.z;
+    if (2 * cb >= cols) return;
+    for (int64_t r = blockIdx.y; r < rows; r += gridDim.y) {
+        const int64_t e0 = off + b * bs + r * rs + 2 * cb * cs, e1 = e0 + cs;
+        const uint32_t n0 = (base[e0 >> 1] >> ((e0 & 1) * 4)) & 15u, n1 = (base[e1 >> 1] >> ((e1 & 1) * 4)) & 15u;
+        dst[(b * rows + r) * (cols / 2) + cb] = (uint8_t)(n0 | (n1 << 4));
+    }
+}
+
 }  // namespace opsnn
 
 using namespace opsnn;
+
+extern "C" int opsnnGather4(const void* base, int64_t offset, int64_t batch, int64_t rows, int64_t cols, int64_t batch_stride, int64_t row_stride,
+                            int64_t col_stride, void* dst, void* stream)
+{
+    if (!base || !dst || rows <= 0 || cols <= 0 || batch <= 0 || batch > 65535 || (cols & 1)) return -1;
+    if (offset < 0 || batch_stride < 0 || row_stride < 0 || col_stride < 0) return -1;
+    dim3 grid((unsigned)((cols / 2 + 255) / 256), (unsigned)(rows < 65535 ? rows : 65535), (unsigned)batch);
+    hipLaunchKernelGGL(gather4_kernel, grid, dim3(256), 0, (hipStream_t)stream, (const uint8_t*)base, offset, rows, cols, batch_stride, row_stride,
+                       col_stride, (uint8_t*)dst);
+    return (int)hipGetLastError();
+}
 
 extern "C" int opsnnTranspose8(const void* src, void* dst, int64_t rows, int64_t cols, int64_t batch, void* stream)
 {

@@ -252,6 +252,53 @@ def test_int8_regular_strided_views(gpu, M, K, N, x1_pad, x2_step, batch):
     assert np.array_equal(d_out.to_host(np.uint16, (batch, M, N)), want)
 
 
+@pytest.mark.parametrize("M,K,N,x1_off,x1_pad,x2_step,batch", [
+    (256, 512, 384, 0, 64, 2, 1),    # x1 rows byte-aligned but not dense, x2 every other stored row
+    (130, 320, 264, 3, 10, 3, 1),    # x1 starts on an odd nibble, its row pitch is 5 bytes more than the row; a K tail on top
+    (128, 256, 192, 2, 32, 2, 3),    # batched
+])
+def test_fp4_strided_views(gpu, M, K, N, x1_off, x1_pad, x2_step, batch):
+    """Strided views of 4-bit operands (MXFP4): the reference copies any non-contiguous operand contiguous first
+    (quant_matmul_common_check.cpp:106-123); here phase 2 gathers them nibble by nibble into dense copies at the front of the
+    workspace, then the call goes on as the dense one: same bits as the dense call."""
+    m = gpu
+    print(f"case fp4 strided views M={M} K={K} N={N} x1_off={x1_off} x1_pad={x1_pad} x2_step={x2_step} batch={batch}", flush=True)
+    inp = cases.make_mx_inputs(m, M, K, N, M + K, True, True, batch=batch)
+    b = np.random.default_rng(8).normal(0, 1, N).astype(np.float32)
+    want = cases.run_mx_aclnn(m, inp, M, K, N, True, m.ACL_BF16, b)
+    check_close(want, cases.oracle_mx(m, inp, M, K, N, True, m.ACL_BF16, b), orc.BF16, "mxfp4 dense")
+    rng = np.random.default_rng(9)
+    # nibble images: x1 rows of K + x1_pad nibbles behind x1_off nibbles; x2 rows at every x2_step-th stored row
+    n1 = rng.integers(0, 16, size=(batch, M * (K + x1_pad) + x1_off + 1), dtype=np.uint8)
+    c1 = orc.unpack_nibbles(inp["x1"]).reshape(batch, M, K)
+    for r in range(M):
+        n1[:, x1_off + r * (K + x1_pad): x1_off + r * (K + x1_pad) + K] = c1[:, r]
+    if n1.shape[1] % 2:
+        n1 = n1[:, :-1]
+    n2 = rng.integers(0, 16, size=(batch, N * x2_step, K), dtype=np.uint8)
+    n2[:, ::x2_step] = orc.unpack_nibbles(inp["x2"]).reshape(batch, N, K)
+    d1, d2 = m.DeviceBuffer(host=orc.pack_nibbles(n1)), m.DeviceBuffer(host=orc.pack_nibbles(n2))
+    bs = (batch,) if batch > 1 else ()
+    x1 = m.Tensor(bs + (M, K), m.ACL_FLOAT4_E2M1, d1, strides=((n1.shape[1],) if batch > 1 else ()) + (K + x1_pad, 1), offset=x1_off,
+                  storage_shape=(batch * n1.shape[1],))
+    x2 = m.Tensor(bs + (N, K), m.ACL_FLOAT4_E2M1, d2, strides=((N * x2_step * K,) if batch > 1 else ()) + (K * x2_step, 1),
+                  storage_shape=bs + (N * x2_step, K))
+    d = {k: m.DeviceBuffer(host=v) for k, v in inp.items() if isinstance(v, np.ndarray) and k in ("s1", "s2")}
+    s1 = m.Tensor(bs + inp["s1"].shape[1:], m.ACL_FLOAT8_E8M0, d["s1"]); s2 = m.Tensor(bs + inp["s2"].shape[1:], m.ACL_FLOAT8_E8M0, d["s2"])
+    d_out = m.DeviceBuffer(batch * M * N * 2); d_out.fill(0xFF)
+    out = m.Tensor(bs + (M, N), m.ACL_BF16, d_out)
+    d_b = m.DeviceBuffer(host=b); t_b = m.Tensor((N,), m.ACL_FLOAT, d_b)
+    gs = (1 << 32) | (1 << 16) | 32
+    rc, ws, ex = m.quant_matmul_v5_get_workspace(x1, x2, s1, s2, out, bias=t_b, transpose_x2=True, group_size=gs)
+    up = lambda v: -(-v // 256) * 256
+    assert rc == 0 and ws >= up(batch * M * K // 2) + up(batch * N * K // 2), (rc, ws, m.err_msg())
+    m.lib().aclDestroyAclOpExecutor(ex)
+    wbuf = m.quant_matmul_v5(x1, x2, s1, s2, out, bias=t_b, transpose_x2=True, group_size=gs)
+    m.check(m.lib().aclrtSynchronizeDevice(), "sync")
+    assert np.array_equal(d_out.to_host(np.uint16, (batch, M, N)), want)
+    del wbuf
+
+
 def test_irregular_views_are_still_rejected(gpu):
     m = gpu
     d = m.DeviceBuffer(4096 * 16)
