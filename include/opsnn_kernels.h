@@ -182,6 +182,10 @@ OPSNN_API int opsnnTranspose4(const void* src, void* dst, int64_t rows, int64_t 
  * reference's l0op::Contiguous (matmul/quant_batch_matmul_v4/op_host/op_api/quant_matmul_common_check.cpp:106-123). */
 OPSNN_API int opsnnGather4(const void* base, int64_t offset, int64_t batch, int64_t rows, int64_t cols, int64_t batch_stride,
                            int64_t row_stride, int64_t col_stride, void* dst, void* stream);
+/* The same for 8-bit elements: the MX modes of aclnnQuantMatmulV5 gather a strided fp8 operand this way (the other 8-bit
+ * modes gather inside their launchers, together with the padding of a K tail). */
+OPSNN_API int opsnnGather8(const void* base, int64_t offset, int64_t batch, int64_t rows, int64_t cols, int64_t batch_stride,
+                           int64_t row_stride, int64_t col_stride, void* dst, void* stream);
 
 /* The same for 16-bit elements (pairs of e8m0 MX scales, 16-bit group scales). */
 OPSNN_API int opsnnTranspose16(const void* src, void* dst, int64_t rows, int64_t cols, int64_t batch, void* stream);

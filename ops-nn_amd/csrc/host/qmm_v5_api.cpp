@@ -611,16 +611,17 @@ extern "C" aclnnStatus aclnnQuantMatmulV5GetWorkspaceSize(const aclTensor* x1, c
     // ---- route (aclnn_quant_matmul_v5.cpp:1163-1174) and build the launch plan ----
     OpsnnQmmArgs& a = ex->qmm;
     a.M = c.M; a.N = c.N; a.K = c.K1;
-    // a strided 4-bit operand: phase 2 gathers it; from here on the view is the dense copy (its address is filled in then)
+    // a strided 4-bit operand (or 8-bit MX operand): phase 2 gathers it; from here on the view is the dense copy (its address is filled in then)
     auto plan_gather = [&](TView& t, int which) {
-        if (!is_4bit(t.dtype) || is_contiguous(t)) return;
+        const bool mx8 = dtype_bits(t.dtype) == 8 && c.mx();   // (the other 8-bit modes gather in their launchers)
+        if ((!is_4bit(t.dtype) && !mx8) || is_contiguous(t)) return;
         auto& g = ex->gather[which];
-        g.active = true; g.base = t.data; g.off = t.offset;
+        g.active = true; g.bits = mx8 ? 8 : 4; g.base = t.data; g.off = t.offset;
         g.rows = t.dim(-2); g.cols = t.dim(-1); g.rs = t.stride(-2); g.cs = t.stride(-1);
         g.nb = 1;
         for (int64_t i = 0; i < t.rank() - 2; i++) g.nb *= t.dim(i);
         g.bs = t.rank() > 2 ? t.stride(-3) : 0;
-        g.bytes = (uint64_t)(g.nb * g.rows * g.cols / 2);
+        g.bytes = (uint64_t)(g.nb * g.rows * g.cols * g.bits / 8);
         t.offset = 0;
         int64_t st = 1;
         for (int64_t i = t.rank() - 1; i >= 0; i--) { t.strides[(size_t)i] = st; st *= t.shape[(size_t)i]; }
@@ -785,14 +786,14 @@ extern "C" aclnnStatus aclnnQuantMatmulV5(void* workspace, uint64_t workspaceSiz
         INVALID("aclnnQuantMatmulV5: workspace of %lu bytes required", (unsigned long)ex->workspace_size);
     if (!ex->qmm.x1.ptr || !ex->qmm.x2.ptr || !ex->qmm.out) INVALID("aclnnQuantMatmulV5: a tensor has no device address");
     int rc = 0;
-    // strided 4-bit operands first become dense copies at the front of the workspace
+    // strided 4-bit (and 8-bit MX) operands first become dense copies at the front of the workspace
     char* w = (char*)workspace;
     for (int i = 0; i < 2; i++) {
         const auto& g = ex->gather[i];
         if (!g.active) continue;
         if (!g.base) INVALID("aclnnQuantMatmulV5: a tensor has no device address");
-        rc = opsnnGather4(g.base, g.off, g.nb, g.rows, g.cols, g.bs, g.rs, g.cs, w, stream);
-        if (rc != 0) FAIL(ACLNN_ERR_RUNTIME_ERROR, "%s: gathering the strided 4-bit %s failed with code %d", ex->api, i ? "x2" : "x1", rc);
+        rc = (g.bits == 4 ? opsnnGather4 : opsnnGather8)(g.base, g.off, g.nb, g.rows, g.cols, g.bs, g.rs, g.cs, w, stream);
+        if (rc != 0) FAIL(ACLNN_ERR_RUNTIME_ERROR, "%s: gathering the strided %s failed with code %d", ex->api, i ? "x2" : "x1", rc);
         (i ? ex->qmm.x2 : ex->qmm.x1).ptr = w;
         w += (g.bytes + 255) / 256 * 256;
     }

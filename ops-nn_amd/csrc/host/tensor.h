@@ -45,9 +45,9 @@ struct aclOpExecutorImpl {
     // General batch broadcast of aclnnQuantMatmulV5 (x1 [2, 1, M, K] with x2 [1, 3, K, N] and the like): one launch per
     // combination of the outer batch dims, each over the innermost batch dim; empty for the usual cases, which are one launch.
     std::vector<OpsnnQmmArgs> batch_runs;
-    // Strided view of a 4-bit matrix operand (index 0: x1, 1: x2): phase 2 first gathers it into a dense copy at the very front
-    // of the workspace (bytes, rounded up to 256, each) and points the operand there.
-    struct GatherStep { bool active = false; const void* base = nullptr; int64_t off = 0, nb = 1, rows = 0, cols = 0, bs = 0, rs = 0, cs = 0; uint64_t bytes = 0; } gather[2];
+    // Strided view of a 4-bit matrix operand, or of an 8-bit one in the MX modes (index 0: x1, 1: x2): phase 2 first gathers it
+    // into a dense copy at the very front of the workspace (bytes, rounded up to 256, each) and points the operand there.
+    struct GatherStep { bool active = false; int bits = 4; const void* base = nullptr; int64_t off = 0, nb = 1, rows = 0, cols = 0, bs = 0, rs = 0, cs = 0; uint64_t bytes = 0; } gather[2];
     uint64_t gather_front() const { return (gather[0].active ? (gather[0].bytes + 255) / 256 * 256 : 0) + (gather[1].active ? (gather[1].bytes + 255) / 256 * 256 : 0); }
     struct NzStep { bool active = false; const void* src = nullptr; int64_t rows = 0, row_bytes = 0, batch = 1; int c0 = 0; uint64_t nd_bytes = 0; } nz;
 };

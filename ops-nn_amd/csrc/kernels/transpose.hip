@@ -65,9 +65,29 @@ __global__ __launch_bounds__(256) void gather4_kernel(const uint8_t* __restrict_
     }
 }
 
+// the same for 8-bit elements
+__global__ __launch_bounds__(256) void gather8_kernel(const uint8_t* __restrict__ base, int64_t off, int64_t rows, int64_t cols,
+                                                      int64_t bs, int64_t rs, int64_t cs, uint8_t* __restrict__ dst)
+{
+    const int64_t c = (int64_t)blockIdx.x * 256 + threadIdx.x, b = blockIdx.z;
+    if (c >= cols) return;
+    for (int64_t r = blockIdx.y; r < rows; r += gridDim.y) dst[(b * rows + r) * cols + c] = base[off + b * bs + r * rs + c * cs];
+}
+
 }  // namespace opsnn
 
 using namespace opsnn;
+
+extern "C" int opsnnGather8(const void* base, int64_t offset, int64_t batch, int64_t rows, int64_t cols, int64_t batch_stride, int64_t row_stride,
+                            int64_t col_stride, void* dst, void* stream)
+{
+    if (!base || !dst || rows <= 0 || cols <= 0 || batch <= 0 || batch > 65535) return -1;
+    if (offset < 0 || batch_stride < 0 || row_stride < 0 || col_stride < 0) return -1;
+    dim3 grid((unsigned)((cols + 255) / 256), (unsigned)(rows < 65535 ? rows : 65535), (unsigned)batch);
+    hipLaunchKernelGGL(gather8_kernel, grid, dim3(256), 0, (hipStream_t)stream, (const uint8_t*)base, offset, rows, cols, batch_stride, row_stride,
+                       col_stride, (uint8_t*)dst);
+    return (int)hipGetLastError();
+}
 
 extern "C" int opsnnGather4(const void* base, int64_t offset, int64_t batch, int64_t rows, int64_t cols, int64_t batch_stride, int64_t row_stride,
                             int64_t col_stride, void* dst, void* stream)

@@ -299,6 +299,53 @@ def test_fp4_strided_views(gpu, M, K, N, x1_off, x1_pad, x2_step, batch):
     del wbuf
 
 
+@pytest.mark.parametrize("mode", ["mxfp8", "blockscale"])
+@pytest.mark.parametrize("M,K,N,x1_off,x1_pad,x2_step,batch,expand", [
+    (256, 512, 384, 0, 64, 2, 1, False),
+    (130, 320, 264, 3, 5, 3, 1, False),     # nothing aligned, a K tail (MX) / a ragged last K block (block scales) on top
+    (128, 256, 192, 16, 32, 2, 3, True),    # batched, x2 one matrix expanded over the batch (batch stride 0)
+])
+def test_fp8_strided_views_mx_and_blockscale(gpu, mode, M, K, N, x1_off, x1_pad, x2_step, batch, expand):
+    """Strided views of fp8 operands in the MX mode (gathered by phase 2 into the front of the workspace) and in the
+    block-scale mode (gathered by its launcher): same bits as the dense call; a batch dim of stride 0 included."""
+    m = gpu
+    print(f"case fp8 strided views {mode} M={M} K={K} N={N} x1_off={x1_off} x1_pad={x1_pad} x2_step={x2_step} batch={batch} expand={expand}", flush=True)
+    if mode == "mxfp8":
+        inp = cases.make_mx_inputs(m, M, K, N, M + K + 1, True, False, batch=batch)
+        sdt, gs = m.ACL_FLOAT8_E8M0, (1 << 32) | (1 << 16) | 32
+    else:
+        inp = cases.make_blockscale_inputs(m, M, K, N, M + K + 2, True, batch=batch)
+        sdt, gs = m.ACL_FLOAT, (1 << 32) | (128 << 16) | 128
+    if expand:
+        inp["x2"][1:] = inp["x2"][0]
+        inp["s2"][1:] = inp["s2"][0]
+    if mode == "mxfp8":
+        want = cases.run_mx_aclnn(m, inp, M, K, N, True, m.ACL_BF16)
+    else:
+        want = cases.run_blockscale_aclnn(m, inp, M, K, N, True, m.ACL_BF16)
+    rng = np.random.default_rng(10)
+    L1 = M * (K + x1_pad) + x1_off
+    b1 = rng.integers(0, 120, size=(batch, L1), dtype=np.uint8)
+    for r in range(M):
+        b1[:, x1_off + r * (K + x1_pad): x1_off + r * (K + x1_pad) + K] = inp["x1"][:, r]
+    nb2 = 1 if expand else batch
+    b2 = rng.integers(0, 120, size=(nb2, N * x2_step, K), dtype=np.uint8)
+    b2[:, ::x2_step] = inp["x2"][:nb2]
+    d1, d2 = m.DeviceBuffer(host=b1), m.DeviceBuffer(host=b2)
+    bs = (batch,) if batch > 1 else ()
+    x1 = m.Tensor(bs + (M, K), m.ACL_FLOAT8_E4M3FN, d1, strides=((L1,) if batch > 1 else ()) + (K + x1_pad, 1), offset=x1_off, storage_shape=(batch * L1,))
+    x2 = m.Tensor(bs + (N, K), m.ACL_FLOAT8_E4M3FN, d2, strides=((0 if expand else N * x2_step * K,) if batch > 1 else ()) + (K * x2_step, 1),
+                  storage_shape=(nb2, N * x2_step, K))
+    ds1, ds2 = m.DeviceBuffer(host=inp["s1"]), m.DeviceBuffer(host=inp["s2"])
+    s1 = m.Tensor(bs + inp["s1"].shape[1:], sdt, ds1); s2 = m.Tensor(bs + inp["s2"].shape[1:], sdt, ds2)
+    d_out = m.DeviceBuffer(batch * M * N * 2); d_out.fill(0xFF)
+    out = m.Tensor(bs + (M, N), m.ACL_BF16, d_out)
+    wbuf = m.quant_matmul_v5(x1, x2, s1, s2, out, transpose_x2=True, group_size=gs)
+    m.check(m.lib().aclrtSynchronizeDevice(), "sync")
+    assert np.array_equal(d_out.to_host(np.uint16, (batch, M, N)), want)
+    del wbuf
+
+
 def test_irregular_views_are_still_rejected(gpu):
     m = gpu
     d = m.DeviceBuffer(4096 * 16)
