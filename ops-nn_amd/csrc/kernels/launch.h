@@ -20,6 +20,25 @@ enum {
 };
 
 #ifdef __cplusplus
+#ifdef __HIPCC__
+#include <hip/hip_runtime.h>
+#include <atomic>
+namespace opsnn {
+// hipFuncSetAttribute belongs to a (kernel, device) pair: launchers keep one of these masks per kernel instantiation,
+// a bit per device ordinal (mod 64).  Two threads that both find the bit clear both set the attribute: harmless.
+inline bool device_flag_test(const std::atomic<uint64_t>& mask)
+{
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return false;
+    return (mask.load(std::memory_order_acquire) >> (dev & 63)) & 1u;
+}
+inline void device_flag_set(std::atomic<uint64_t>& mask)
+{
+    int dev = 0;
+    if (hipGetDevice(&dev) == hipSuccess) mask.fetch_or(1ull << (dev & 63), std::memory_order_release);
+}
+}  // namespace opsnn
+#endif
 namespace opsnn {
 // Opened by every exported matmul entry point for the time it enqueues its launches (weight_cache.hip): copies that the
 // weight cache hands out inside the scope cannot be evicted before it closes; bypass = true switches the cache off for

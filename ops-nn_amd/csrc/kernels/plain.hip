@@ -321,7 +321,9 @@ uint64_t tcg_workspace_bytes(const OpsnnQmmArgs& a)
     if (a.x1_dtype != DT_E4M3 || a.x2_dtype != DT_E2M1 || a.batch != 1) return 0;
     if (a.K % 32 != 0 || a.K < 128 || a.gsK <= 0 || a.gsK % 32 != 0 || (uintptr_t)a.x2.ptr % 16 != 0 || a.M * a.N < 64 * 64) return 0;
     if (a.x1.col_stride != 1 || a.x2.row_stride != 1 || a.x2.col_stride != a.K) return 0;
-    if (a.K % 128 != 0 && (((uintptr_t)a.x1.ptr | (uint64_t)a.x1.row_stride) % 16 != 0 || a.x1.row_stride < a.K)) return 0;   // the padded copy of x1 moves 16-byte pieces
+    // x1 in 16-byte pieces: what the matrix-core kernels (and the padded copy of a K tail) move; checked here, before the
+    // re-quantisation is launched or cached, so that no later step of launch_tcg_mfma can still decline the call
+    if (((uintptr_t)a.x1.ptr | (uint64_t)a.x1.row_stride) % 16 != 0 || a.x1.row_stride < a.K) return 0;
     if (a.out_dtype != DT_BF16 && a.out_dtype != DT_F16) return 0;
     if (a.bias && a.bias_dtype != DT_F32) return 0;
     return tcg_blob_bytes(a) + tcg_x1pad_bytes(a) + tcg_rows_bytes(a);

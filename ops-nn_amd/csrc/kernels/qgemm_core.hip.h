@@ -676,11 +676,11 @@ static int qgemm_launch_one(const QgemmParams& p, int64_t batch, hipStream_t st)
     size_t lds = SCB == 8 ? (size_t)STAGES * (BM + BN) * BK + 2 * (BM + BN) * 16   // scales in their own ring of two slots
                           : (size_t)STAGES * ((BM + BN) * BK + (BM + BN) * SCB);
     auto k = qgemm_kernel<MODE, BM, BN, BK, WGM, WGN, STAGES, MINWG, KTAIL, OUT_DT>;
-    static bool attr_set = false;  // per instantiation; benign if two threads both set it
-    if (!attr_set) {
+    static std::atomic<uint64_t> attr_set{0};   // one bit per device: the attribute belongs to the (kernel, device) pair
+    if (!device_flag_test(attr_set)) {
         hipError_t e = hipFuncSetAttribute((const void*)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (e != hipSuccess) return (int)e;
-        attr_set = true;
+        device_flag_set(attr_set);
     }
     hipLaunchKernelGGL(k, grid, dim3(WGM * WGN * 64), lds, st, p, tiles_m, tiles_n);
     return (int)hipGetLastError();

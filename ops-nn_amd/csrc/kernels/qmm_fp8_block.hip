@@ -460,11 +460,11 @@ static int launch_fp8_block(const Fp8BlkParams& p, int64_t batch, hipStream_t st
     dim3 grid((unsigned)(tiles_m * tiles_n), (unsigned)batch);
     size_t lds = (size_t)STAGES * (BM * 128 + 256 * (MODE == FP8_MX_W4 ? 64 : 128) + WGM * 128 * 4);
     auto k = qmm_fp8_block_kernel<WGM, STAGES, OUT_DT, MODE>;
-    static bool attr_set = false;
-    if (!attr_set) {
+    static std::atomic<uint64_t> attr_set{0};   // one bit per device: the attribute belongs to the (kernel, device) pair
+    if (!device_flag_test(attr_set)) {
         hipError_t e = hipFuncSetAttribute((const void*)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (e != hipSuccess) return (int)e;
-        attr_set = true;
+        device_flag_set(attr_set);
     }
     hipLaunchKernelGGL(k, grid, dim3(WGM * 128), lds, st, p, tiles_m, tiles_n);
     return (int)hipGetLastError();

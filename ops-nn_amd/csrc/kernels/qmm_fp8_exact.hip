@@ -525,11 +525,11 @@ static int launch_fp8_exact(const Fp8xParams& p, int64_t batch, hipStream_t st)
     dim3 grid((unsigned)(tiles_m * tiles_n), (unsigned)batch);
     const size_t lds = 3 * (size_t)(256 * 128 + 128 * 128 + ((RC && !MXS) ? 0 : 512 * 4));
     auto k = qmm_fp8_exact_kernel<OUT_DT, RC, FMT, MXS>;
-    static bool attr_set = false;
-    if (!attr_set) {
+    static std::atomic<uint64_t> attr_set{0};   // one bit per device: the attribute belongs to the (kernel, device) pair
+    if (!device_flag_test(attr_set)) {
         hipError_t e = hipFuncSetAttribute((const void*)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (e != hipSuccess) return (int)e;
-        attr_set = true;
+        device_flag_set(attr_set);
     }
     hipLaunchKernelGGL(k, grid, dim3(512), lds, st, p, tiles_m, tiles_n);
     return (int)hipGetLastError();

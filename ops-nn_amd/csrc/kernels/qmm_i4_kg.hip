@@ -290,12 +290,12 @@ int launch_kg_mfma(const OpsnnQmmArgs& a, hipStream_t st)
     }
     const dim3 grid((unsigned)(L.Np / KG_TILE), (unsigned)(L.Mp / KG_TILE));
     constexpr int KG_LDS = 2 * 2 * (int)KG_BLOCK;
-    static bool attr_set = false;
-    if (!attr_set) {
+    static std::atomic<uint64_t> attr_set{0};   // one bit per device: the attribute belongs to the (kernel, device) pair
+    if (!device_flag_test(attr_set)) {
         hipError_t e = hipFuncSetAttribute((const void*)kg_gemm_kernel<DT_BF16>, hipFuncAttributeMaxDynamicSharedMemorySize, KG_LDS);
         if (e == hipSuccess) e = hipFuncSetAttribute((const void*)kg_gemm_kernel<DT_F16>, hipFuncAttributeMaxDynamicSharedMemorySize, KG_LDS);
         if (e != hipSuccess) return (int)e;
-        attr_set = true;
+        device_flag_set(attr_set);
     }
     if (a.out_dtype == DT_BF16)
         hipLaunchKernelGGL(kg_gemm_kernel<DT_BF16>, grid, dim3(512), KG_LDS, st, a8, b8, (const float*)a.x1_scale, (uint16_t*)a.out, a.M, a.N, (int)L.G);

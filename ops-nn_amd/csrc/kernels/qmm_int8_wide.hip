@@ -522,11 +522,11 @@ static int launch_wide_one(const QgemmParams& p, int64_t batch, hipStream_t st)
     const int tiles_m = (int)((p.M + BM - 1) / BM), tiles_n = (int)((p.N + BN - 1) / BN);
     const size_t lds = (size_t)2 * (BM + BN) * BK + (MXS ? (size_t)2 * ((BM + BN + 255) / 256) * 4096 : 0);
     auto k = qgemm_i8_wide_kernel<FN, OUT_DT, F8, MXS>;
-    static bool attr_set = false;   // per instantiation; benign if two threads both set it
-    if (!attr_set) {
+    static std::atomic<uint64_t> attr_set{0};   // one bit per device: the attribute belongs to the (kernel, device) pair
+    if (!device_flag_test(attr_set)) {
         hipError_t e = hipFuncSetAttribute((const void*)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (e != hipSuccess) return (int)e;
-        attr_set = true;
+        device_flag_set(attr_set);
     }
     hipLaunchKernelGGL(k, dim3((unsigned)(tiles_m * tiles_n), (unsigned)batch), dim3(256), lds, st, p, tiles_m, tiles_n);
     return (int)hipGetLastError();

@@ -273,11 +273,11 @@ static int launch_decode(const WqParams& p, hipStream_t st)
     const size_t lds = 2 * (size_t)(16 * MB) * (KX * 2 + 16);
     const unsigned grid = (unsigned)((p.N + 16 * WN - 1) / (16 * WN));
     auto k = wqmm_decode_kernel<XDT, WBITS, MB, WK, WFLT>;
-    static bool attr_set = false;
-    if (!attr_set) {
+    static std::atomic<uint64_t> attr_set{0};   // one bit per device: the attribute belongs to the (kernel, device) pair
+    if (!device_flag_test(attr_set)) {
         hipError_t e = hipFuncSetAttribute((const void*)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (e != hipSuccess) return (int)e;
-        attr_set = true;
+        device_flag_set(attr_set);
     }
     hipLaunchKernelGGL(k, dim3(grid), dim3(256), lds, st, p);
     return (int)hipGetLastError();
@@ -422,7 +422,9 @@ static int launch_slabs(WqParams p, hipStream_t st)
             q.y = p.y + m0 * p.N;
             q.M = (p.M - m0) < slab ? (p.M - m0) : slab;
             const int rc = launch_wq_tile<XDT, WBITS>(q, st);
-            if (rc == OPSNN_NOT_TAKEN && m0 == 0) taken = false;   // the shape conditions are the same for every slab
+            // launch_wq_tile's conditions hold for every slab once they hold for the first (slabs are no larger, K % 64 == 0
+            // keeps their x rows 16-byte aligned), so a refusal can only come before anything has been written
+            if (rc == OPSNN_NOT_TAKEN && m0 == 0) taken = false;
             else if (rc != 0) return rc;
         }
         if (taken) return 0;

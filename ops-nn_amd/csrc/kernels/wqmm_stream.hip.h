@@ -1200,11 +1200,11 @@ static int launch_resx_one(const WqParams& p, hipStream_t st)
 {
     const size_t lds = (size_t)(p.m_rows + 1) * (p.K * 2 + 16) + 2 * 3 * 4 * 64 * 4;
     auto k = wqmm_resx_kernel<XDT, WBITS, HAS_OFF, VSCALE>;
-    static bool attr_set = false;
-    if (!attr_set) {
+    static std::atomic<uint64_t> attr_set{0};   // one bit per device: the attribute belongs to the (kernel, device) pair
+    if (!device_flag_test(attr_set)) {
         hipError_t e = hipFuncSetAttribute((const void*)k, hipFuncAttributeMaxDynamicSharedMemorySize, 65536 + 8192);
         if (e != hipSuccess) return (int)e;
-        attr_set = true;
+        device_flag_set(attr_set);
     }
     hipLaunchKernelGGL(k, dim3(resx_grid((p.N + 15) / 16)), dim3(256), lds, st, p);
     return (int)hipGetLastError();
@@ -1220,11 +1220,11 @@ static int launch_xreg_one(const WqParams& p, hipStream_t st)
     constexpr int NU = NCH * STEPS / 4;                  // units of 16 rows x 256 bytes per wave
     constexpr int lds = NW * NU * 4096 <= 128 * 1024 ? NW * NU * 4096 : NW * (NU / 2) * 4096;   // all of x, or half of it at a time
     auto k = wqmm_xreg_kernel<XDT, WBITS, NW, NCH, HAS_OFF, SCM, WFLT>;
-    static bool attr_set = false;
-    if (!attr_set) {
+    static std::atomic<uint64_t> attr_set{0};   // one bit per device: the attribute belongs to the (kernel, device) pair
+    if (!device_flag_test(attr_set)) {
         hipError_t e = hipFuncSetAttribute((const void*)k, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
         if (e != hipSuccess) return (int)e;
-        attr_set = true;
+        device_flag_set(attr_set);
     }
     hipLaunchKernelGGL(k, dim3((unsigned)(nblocks < g ? nblocks : g)), dim3(NW * 64), lds, st, p);
     return (int)hipGetLastError();
@@ -1288,12 +1288,12 @@ static int launch_stream_one(const WqParams& p, hipStream_t st)
     const size_t lds = lds_x > lds_red ? lds_x : lds_red;
     const unsigned grid = (unsigned)((p.N + 16 * WN - 1) / (16 * WN));
     auto k = wqmm_stream_kernel<XDT, WBITS, MB, NW, WK, HAS_OFF, VSCALE>;
-    static bool attr_set = false;
-    if (!attr_set) {
+    static std::atomic<uint64_t> attr_set{0};   // one bit per device: the attribute belongs to the (kernel, device) pair
+    if (!device_flag_test(attr_set)) {
         constexpr size_t lds_max = 2 * (size_t)(16 * MB + 1) * (KX * 2 + 16);
         hipError_t e = hipFuncSetAttribute((const void*)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_max);
         if (e != hipSuccess) return (int)e;
-        attr_set = true;
+        device_flag_set(attr_set);
     }
     hipLaunchKernelGGL(k, dim3(grid), dim3(NW * 64), lds, st, p);
     return (int)hipGetLastError();
@@ -1321,11 +1321,11 @@ static int launch_rows_one(const WqParams& p, hipStream_t st)
     if (lds > lds_main + lds_table + lds_stab) return OPSNN_NOT_TAKEN;
     const unsigned grid = (unsigned)((p.N + 16 * NB * WN - 1) / (16 * NB * WN));
     auto k = wqmm_rows_kernel<XDT, WBITS, MB, NB, WN, WK, HAS_OFF, WF, SLDS>;
-    static bool attr_set = false;
-    if (!attr_set) {
+    static std::atomic<uint64_t> attr_set{0};   // one bit per device: the attribute belongs to the (kernel, device) pair
+    if (!device_flag_test(attr_set)) {
         hipError_t e = hipFuncSetAttribute((const void*)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)(SLDS ? 160 * 1024 : lds_main + lds_table));
         if (e != hipSuccess) return (int)e;
-        attr_set = true;
+        device_flag_set(attr_set);
     }
     hipLaunchKernelGGL(k, dim3(grid), dim3(512), lds, st, p);
     return (int)hipGetLastError();

@@ -332,11 +332,11 @@ static int launch_tile_bm(const WqParams& p, hipStream_t st)
     const size_t lds = wq_tile_lds_bytes<BM>();
     const dim3 grid((unsigned)((p.N + 127) / 128));
     auto launch = [&](auto kern) -> int {
-        static bool attr_set = false;
-        if (!attr_set) {
+        static std::atomic<uint64_t> attr_set{0};   // one bit per device: the attribute belongs to the (kernel, device) pair
+        if (!device_flag_test(attr_set)) {
             hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
             if (e != hipSuccess) return (int)e;
-            attr_set = true;
+            device_flag_set(attr_set);
         }
 #ifdef OPSNN_WQ_AUDIT
         {
