@@ -101,8 +101,8 @@ OPSNN_API int opsnnQmmBlockScale(const OpsnnQmmArgs* a, void* stream);
  * The initial value is taken from the environment variable OPSNN_FP8_FAST (unset or 0: exact). */
 OPSNN_API void opsnnSetFp8Fast(int fast);
 OPSNN_API int opsnnGetFp8Fast(void);
-/* Routing switches for tests and tuning, process-wide; each starts from the environment variable of the same meaning,
- * read once when the library is loaded (OPSNN_FORCE_PLAIN, OPSNN_MX8_WIDE, OPSNN_WQ_TILE_MIN):
+/* Routing switches, process-wide.  The first also starts from the environment variable OPSNN_FORCE_PLAIN, read once when
+ * the library is loaded; the other two are hooks of the parity tests, which compare two kernels on the same call:
  *   opsnnSetForcePlain(1)  every call runs on the plain one-thread-per-output kernels (bit-identical to the CPU oracle);
  *   opsnnSetMx8Wide(n)     MXFP8 on the four-wave kernel with 256 x 32n tiles (n = 8, 9), 0 never, -1 automatic;
  *   opsnnSetWqTileMin(m)   weight-only int4/int8 calls with m .. 256 rows of x run on the dequantise-once tile kernel

@@ -31,19 +31,19 @@ uint64_t mx_workspace_bytes(const OpsnnQmmArgs& a);
 
 using namespace opsnn;
 
-// Routing switches for tests and tuning, process-wide.  Each starts from an environment variable read ONCE when the
-// library is loaded (no getenv on the call path) and can be changed at run time through its setter.
+// Routing switches, process-wide.  OPSNN_FORCE_PLAIN is read ONCE when the library is loaded (no getenv on the call
+// path); every switch can be changed at run time through its setter.
 //   OPSNN_FORCE_PLAIN=1 / opsnnSetForcePlain(1): every call runs on the plain one-thread-per-output kernels (the parity
 //   tests compare them bit for bit with the oracle);
-//   OPSNN_MX8_WIDE=n / opsnnSetMx8Wide(n): MXFP8 on the four-wave kernel with 256 x 32n tiles, n = 8 or 9; 0 never; -1 the
-//   selector decides (default);
-//   OPSNN_WQ_TILE_MIN=m / opsnnSetWqTileMin(m): weight-only int4/int8 calls with m .. 256 rows of x run on the
-//   dequantise-once tile kernel (default 129: below that the streaming kernels are faster).
-static int g_wq_tile_min = [] { const char* e = getenv("OPSNN_WQ_TILE_MIN"); return e ? atoi(e) : 129; }();
+//   opsnnSetMx8Wide(n) (test hook): MXFP8 on the four-wave kernel with 256 x 32n tiles, n = 8 or 9; 0 never; -1 the selector
+//   decides (default);
+//   opsnnSetWqTileMin(m) (test hook): weight-only int4/int8 calls with m .. 256 rows of x run on the dequantise-once tile
+//   kernel (default 129: below that the streaming kernels are faster).
+static int g_wq_tile_min = 129;
 extern "C" void opsnnSetWqTileMin(int m) { __atomic_store_n(&g_wq_tile_min, m, __ATOMIC_RELAXED); }
 extern "C" __attribute__((visibility("hidden"))) int opsnn_wq_tile_min() { return __atomic_load_n(&g_wq_tile_min, __ATOMIC_RELAXED); }
 static int g_force_plain = [] { const char* e = getenv("OPSNN_FORCE_PLAIN"); return (e && *e && *e != '0') ? 1 : 0; }();
-static int g_mx8_wide = [] { const char* e = getenv("OPSNN_MX8_WIDE"); return e ? atoi(e) : -1; }();
+static int g_mx8_wide = -1;
 extern "C" void opsnnSetForcePlain(int on) { __atomic_store_n(&g_force_plain, on ? 1 : 0, __ATOMIC_RELAXED); }
 extern "C" void opsnnSetMx8Wide(int n) { __atomic_store_n(&g_mx8_wide, n, __ATOMIC_RELAXED); }
 extern "C" __attribute__((visibility("hidden"))) bool opsnn_force_plain() { return __atomic_load_n(&g_force_plain, __ATOMIC_RELAXED) != 0; }

@@ -597,8 +597,7 @@ int launch_fp8_rowcol_mfma(const OpsnnQmmArgs& a, hipStream_t st, bool merged_sc
         int dev = 0, cus = 0;
         if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0) cus = 256;
         const int64_t tm = (a.M + 255) / 256, tn = (a.N + 255) / 256;
-        static const bool no_wide = [] { const char* e = getenv("OPSNN_F8_NO_WIDE"); return e && e[0] == '1'; }();   // tuning aid
-        if (!no_wide && a.K >= 1024 && tm * tn * a.batch * 4 >= cus * 3) {
+        if (a.K >= 1024 && tm * tn * a.batch * 4 >= cus * 3) {
             const int64_t block_cost = (tm * tn * a.batch + cus - 1) / cus * 10;   // tile cost = width / 32 + 2, as for int8
             int64_t wide_cost = INT64_MAX;
             int wide_fn = 0;
@@ -679,8 +678,7 @@ int launch_blockscale_mfma(const OpsnnQmmArgs& a0, hipStream_t st)
     if (((uintptr_t)p.a | (uintptr_t)p.b | (uint64_t)p.lda | (uint64_t)p.ldb | (uint64_t)p.a_bs | (uint64_t)p.b_bs) % 16) return OPSNN_NOT_TAKEN;
     if (((uintptr_t)p.s1 | (uintptr_t)p.s2) % 4) return OPSNN_NOT_TAKEN;
     // 256 x 256 tiles (8 waves) halve the operand traffic per flop; 128 x 256 (4 waves) keeps small M efficient
-    static const int ev = [] { const char* e = getenv("OPSNN_FP8_WGM"); return e ? atoi(e) : 0; }();
-    const bool big = ev ? ev == 4 : a.M >= 512;
+    const bool big = a.M >= 512;
     if (i8) {
         if (big) return a.out_dtype == DT_BF16 ? launch_fp8_block<4, 2, DT_BF16, I8_BLOCK>(p, a.batch, st) : launch_fp8_block<4, 2, DT_F16, I8_BLOCK>(p, a.batch, st);
         return a.out_dtype == DT_BF16 ? launch_fp8_block<2, 2, DT_BF16, I8_BLOCK>(p, a.batch, st) : launch_fp8_block<2, 2, DT_F16, I8_BLOCK>(p, a.batch, st);

@@ -352,9 +352,8 @@ int launch_mxw4_one(const MxW4DecParams& p, hipStream_t st)
 // otherwise.
 int launch_blockscale_decode(const OpsnnQmmArgs& a, hipStream_t st)
 {
-    static const bool off = [] { const char* e = getenv("OPSNN_FP8_NO_DECODE"); return e && e[0] == '1'; }();
     const bool i8 = a.x1_dtype == DT_I8 && a.x2_dtype == DT_I8;
-    if (off || (!i8 && (a.x1_dtype != DT_E4M3 || a.x2_dtype != DT_E4M3)) || a.batch != 1) return OPSNN_NOT_TAKEN;
+    if ((!i8 && (a.x1_dtype != DT_E4M3 || a.x2_dtype != DT_E4M3)) || a.batch != 1) return OPSNN_NOT_TAKEN;
     if (a.out_dtype != DT_BF16 && a.out_dtype != DT_F16 && !(a.out_dtype == DT_F32 && !i8)) return OPSNN_NOT_TAKEN;
     if (a.bias && !(i8 && a.bias_dtype == DT_F32)) return OPSNN_NOT_TAKEN;
     if (a.M > 32 || a.N < 256) return OPSNN_NOT_TAKEN;
@@ -388,8 +387,7 @@ int launch_blockscale_decode(const OpsnnQmmArgs& a, hipStream_t st)
 // (sum * x2Scale) * x1Scale + bias of compute_pertoken (qbmmv3_kernel_golden.py:361-387) -- for up to 32 rows.
 int launch_rowcol_decode(const OpsnnQmmArgs& a, hipStream_t st)
 {
-    static const bool off = [] { const char* e = getenv("OPSNN_FP8_NO_DECODE"); return e && e[0] == '1'; }();
-    if (off || a.x1_dtype != DT_E4M3 || a.x2_dtype != DT_E4M3 || a.batch != 1) return OPSNN_NOT_TAKEN;
+    if (a.x1_dtype != DT_E4M3 || a.x2_dtype != DT_E4M3 || a.batch != 1) return OPSNN_NOT_TAKEN;
     if (a.out_dtype != DT_BF16 && a.out_dtype != DT_F16 && a.out_dtype != DT_F32) return OPSNN_NOT_TAKEN;
     if (!a.x1_scale || !a.x2_scale || a.x2_scale_dtype != DT_F32 || (a.bias && a.bias_dtype != DT_F32)) return OPSNN_NOT_TAKEN;
     if (a.M > 32 || a.N < 256 || a.x1.col_stride != 1 || a.x2.row_stride != 1) return OPSNN_NOT_TAKEN;
@@ -417,8 +415,7 @@ int launch_rowcol_decode(const OpsnnQmmArgs& a, hipStream_t st)
 // share 2 or 4 each, or 8 waves 1 .. 7 each; K-contiguous operands and scales; OPSNN_NOT_TAKEN otherwise.
 int launch_mx_a8w4_decode(const OpsnnQmmArgs& a, hipStream_t st)
 {
-    static const bool off = [] { const char* e = getenv("OPSNN_FP8_NO_DECODE"); return e && e[0] == '1'; }();
-    if (off || a.x1_dtype != DT_E4M3 || a.x2_dtype != DT_E2M1 || a.batch != 1) return OPSNN_NOT_TAKEN;
+    if (a.x1_dtype != DT_E4M3 || a.x2_dtype != DT_E2M1 || a.batch != 1) return OPSNN_NOT_TAKEN;
     if (a.out_dtype != DT_BF16 && a.out_dtype != DT_F16) return OPSNN_NOT_TAKEN;
     if (a.M > 32 || a.N < 256 || a.K % 128 != 0 || a.x1.col_stride != 1 || a.x2.row_stride != 1 || a.x2.col_stride % 2) return OPSNN_NOT_TAKEN;
     if (a.x1_scale_mat.col_stride != 2 || a.x2_scale_mat.col_stride != 2) return OPSNN_NOT_TAKEN;   // [rows, K / 64, 2]: a row's bytes contiguous

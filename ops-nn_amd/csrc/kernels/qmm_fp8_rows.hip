@@ -33,8 +33,7 @@ __global__ __launch_bounds__(256) void widen_e4m3_f16_kernel(const uint8_t* __re
 
 bool rows_eligible(const OpsnnQmmArgs& a)
 {
-    static const bool off = [] { const char* e = getenv("OPSNN_FP8_NO_DECODE"); return e && e[0] == '1'; }();
-    if (off || a.x1_dtype != DT_E4M3 || a.x2_dtype != DT_E4M3 || a.batch != 1 || a.bias) return false;
+    if (a.x1_dtype != DT_E4M3 || a.x2_dtype != DT_E4M3 || a.batch != 1 || a.bias) return false;
     if (a.out_dtype != DT_BF16 && a.out_dtype != DT_F16 && a.out_dtype != DT_F32) return false;
     if (a.M <= 16 || a.M > 128) return false;
     if (a.gsK != 128 || a.gsN != 128 || (a.gsM != 1 && a.gsM != 128)) return false;
@@ -74,8 +73,7 @@ int launch_blockscale_rows(const OpsnnQmmArgs& a, hipStream_t st)
 // The row / column scale form, (sum * x2Scale[n]) * x1Scale[m] + bias[n] with fp32 scales (K-C, K-T), 17 .. 128 rows.
 static bool rowcol_rows_eligible(const OpsnnQmmArgs& a)
 {
-    static const bool off = [] { const char* e = getenv("OPSNN_FP8_NO_DECODE"); return e && e[0] == '1'; }();
-    if (off || a.x1_dtype != DT_E4M3 || a.x2_dtype != DT_E4M3 || a.batch != 1) return false;
+    if (a.x1_dtype != DT_E4M3 || a.x2_dtype != DT_E4M3 || a.batch != 1) return false;
     if (a.out_dtype != DT_BF16 && a.out_dtype != DT_F16 && a.out_dtype != DT_F32) return false;
     if (!a.x1_scale || !a.x2_scale || a.x2_scale_dtype != DT_F32 || (a.bias && a.bias_dtype != DT_F32)) return false;
     if (a.x1_scale_len == 1 && a.x2_scale_len == 1 && !a.bias) return false;   // that case merges and truncates the scales

@@ -127,10 +127,6 @@ extern "C" int opsnn_qmm_int8_impl(const OpsnnQmmArgs* a, void* stream)
     bool b16 = (p.out_dt == DT_BF16 || p.out_dt == DT_F16) || int_out;
     int variant = a->force_variant;
     if (opsnn_force_plain()) variant = OPSNN_VARIANT_PLAIN;
-    if (variant == 0) {  // tuning aid: OPSNN_I8_VARIANT pins a kernel variant for calls that do not ask for one
-        static const int env_variant = [] { const char* e = getenv("OPSNN_I8_VARIANT"); return e ? atoi(e) : 0; }();
-        variant = env_variant;
-    }
     bool want_fast = b16 && a_kmajor && variant != OPSNN_VARIANT_PLAIN && p.M * p.N >= 64 * 64 && (p.K % 16) == 0 &&
                      (p.a_rs % 16) == 0 && ((uintptr_t)p.a % 16) == 0 && (p.a_bs % 16) == 0;
     if (want_fast && !b_kmajor && p.b_cs == 1 && p.b_rs == p.N && (p.b_bs == 0 || p.b_bs == p.K * p.N)) {

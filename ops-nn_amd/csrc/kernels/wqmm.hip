@@ -306,8 +306,7 @@ template <int WBITS>
 static bool stream_eligible(WqParams& p, WqStreamOpts& o)
 {
     constexpr int64_t KC = 4 * (128 / WBITS);
-    static const bool off = [] { const char* e = getenv("OPSNN_WQ_GENERAL"); return e && e[0] == '1'; }();
-    if (off || p.K % KC != 0) return false;
+    if (p.K % KC != 0) return false;
     const int64_t nch = p.K / KC;
     if (p.group >= p.K) p.cpg_shift = 31;
     else {
@@ -323,13 +322,11 @@ static bool stream_eligible(WqParams& p, WqStreamOpts& o)
     o.vscale = !o.ksplit && p.group == KC && p.s_rs == 1 && p.s_cs % 8 == 0 && ngroups % 8 == 0 &&
                (uintptr_t)p.scale % 16 == 0 && (!p.offset || (uintptr_t)p.offset % 16 == 0);
     // few rows: x whole in LDS (<= 64 KB), K in four contiguous quarters per workgroup
-    static const bool no_resx = [] { const char* e = getenv("OPSNN_WQ_NO_RESX"); return e && e[0] == '1'; }();
-    o.resx = !no_resx && p.M <= 16 && nch % 4 == 0 && (p.M + 1) * (p.K * 2 + 16) <= 65536;
+    o.resx = p.M <= 16 && nch % 4 == 0 && (p.M + 1) * (p.K * 2 + 16) <= 65536;
     o.resx_vscale = o.resx && p.group == KC && p.s_rs == 1 && p.s_cs % 8 == 0 && (nch / 4) % 8 == 0 &&
                     (uintptr_t)p.scale % 16 == 0 && (!p.offset || (uintptr_t)p.offset % 16 == 0);
     // 4 to 16 rows (fewer stay on the kernel above): x in registers, K in 8 or 16 contiguous ranges per workgroup
-    static const int xreg_min = [] { const char* e = getenv("OPSNN_WQ_XREG_MIN"); return e ? atoi(e) : 4; }();
-    static const int xreg_nw = [] { const char* e = getenv("OPSNN_WQ_XREG_NW"); return e ? atoi(e) : 0; }();
+    constexpr int xreg_min = 4, xreg_nw = 0;   // (0: xreg_shape picks the wave count)
     int xnw = 0, xnch = 0;
     o.xreg_nw = xreg_nw;
     o.xreg = p.M >= xreg_min && p.M <= 16 && xreg_shape(WBITS, p.K, xreg_nw, xnw, xnch);
@@ -337,11 +334,10 @@ static bool stream_eligible(WqParams& p, WqStreamOpts& o)
                     (uintptr_t)p.scale % 16 == 0 && (!p.offset || (uintptr_t)p.offset % 16 == 0);
     // more than 48 rows: two weight blocks per wave share every x fragment, up to 128 rows per pass over the weights
     // (needs whole groups of chunks in flight and whole wave tiles of columns)
-    static const bool no_rows = [] { const char* e = getenv("OPSNN_WQ_NO_ROWS"); return e && e[0] == '1'; }();
     // (measured on 8192 x 28672 int4: 16 rows 43 us on the streaming kernel against 55 on this one, 32 rows 53 / 68,
-    // 48 rows 69 / 70, 64 rows 82 / 70, 128 rows 105; OPSNN_WQ_ROWS_MIN moves the switch for tuning)
-    static const int rows_min = [] { const char* e = getenv("OPSNN_WQ_ROWS_MIN"); return e ? atoi(e) : 49; }();
-    o.rows = !no_rows && p.M >= rows_min && nch % 8 == 0 && p.N % 32 == 0 && p.N >= 256;
+    // 48 rows 69 / 70, 64 rows 82 / 70, 128 rows 105: hence the switch at 49 rows)
+    constexpr int rows_min = 49;
+    o.rows = p.M >= rows_min && nch % 8 == 0 && p.N % 32 == 0 && p.N >= 256;
     return true;
 }
 
@@ -357,8 +353,7 @@ template <int XDT, int WBITS>
 static int launch_slabs_float(WqParams p, hipStream_t st)
 {
     // up to 16 rows: x in registers (mxfp4: e2m1 codes with a row's e8m0 bytes contiguous; e4m3 codes with per-channel scales)
-    static const bool no_xreg = [] { const char* e = getenv("OPSNN_WQ_XREG_MIN"); return e && atoi(e) > 16; }();
-    if (!no_xreg && p.M <= 16 && !p.offset) {
+    if (p.M <= 16 && !p.offset) {
         bool ok;
         if (WBITS == 4) ok = p.scale_e8m0 && p.group == 32 && p.s_rs == 1 && p.s_cs % 16 == 0 && (uintptr_t)p.scale % 16 == 0;
         else ok = !p.scale_e8m0 && p.group >= p.K;
@@ -371,7 +366,7 @@ static int launch_slabs_float(WqParams p, hipStream_t st)
     // more rows: the many-rows streaming kernel, up to 128 rows per pass over the weights, in equal slabs
     {
         constexpr int64_t KC = 4 * (128 / WBITS);
-        static const int rows_min = [] { const char* e = getenv("OPSNN_WQ_ROWS_MIN"); return e ? atoi(e) : 17; }();
+        constexpr int rows_min = 17;
         bool ok = !p.offset && p.M >= rows_min && p.K % KC == 0 && (p.K / KC) % 8 == 0 && p.N % 32 == 0 && p.N >= 256;
         if (WBITS == 4) ok = ok && p.scale_e8m0 && p.group == 32 && p.s_rs == 1;
         else ok = ok && !p.scale_e8m0 && p.group >= p.K;
