@@ -67,6 +67,18 @@ struct Fp8xParams {
 #endif
 };
 
+// Asynchronous copies global -> LDS with the address as a wave-uniform 64-bit base in scalar registers plus a 32-bit byte
+// offset per lane: the loop spends no vector instruction on addresses.  (Written out: hidden from the compiler's wait-count
+// pass, like async_copy16_uncounted; the kernel waits for its copies by count.)  lds: wave-uniform LDS byte address.
+__device__ __forceinline__ void copy16_sbase(const void* base, uint32_t voff, uint32_t lds)
+{
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(lds), "v"(voff), "s"(base) : "memory", "m0");
+}
+__device__ __forceinline__ void copy4_sbase(const void* base, uint32_t voff, uint32_t lds)
+{
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2" : : "s"(lds), "v"(voff), "s"(base) : "memory", "m0");
+}
+
 __device__ __forceinline__ const int8_t* uniform_ptr(const int8_t* p)
 {
     const uint64_t u = (uint64_t)p;
@@ -170,36 +182,40 @@ __global__ __launch_bounds__(512, 1) void qmm_fp8_exact_kernel(Fp8xParams p, int
         r = r < b_rows ? r : b_rows - 1;
         b_off[i] = (uint32_t)(r * ldb + cchunk * 16);
     }
-    // scale copy: lanes 0..255 fetch s1 of tile row `tid`, the others the s2 of this tile's n block
-    const char* sc_src = nullptr;
+    // scale copy: lanes 0..255 (waves 0..3) fetch s1 of tile row `tid`, the others the s2 of this tile's n block: a
+    // wave-uniform table base, a 32-bit byte offset per lane (the launcher checks that the tables stay below 4 GB)
+    const char* sc_base = nullptr;
+    uint32_t sc_off = 0;
     int64_t sc_step = 0;   // bytes per K tile
     if constexpr (MXS) {   // lanes 0..255: the four bytes of x1 row `tid`; the others: of x2 row tid - 256 (the last 128 lanes repeat the last row)
-        if (tid < BM) {
+        if (wave < BM / 64) {
             const int r = tid < a_rows ? tid : a_rows - 1;
-            sc_src = (const char*)(p.sa + bz * p.sa_bs + (m0 + r) * p.sa_rs);
+            sc_base = (const char*)(p.sa + bz * p.sa_bs + m0 * p.sa_rs);
+            sc_off = (uint32_t)(r * p.sa_rs);
         } else {
             const int r = tid - BM < b_rows ? tid - BM : b_rows - 1;
-            sc_src = (const char*)(p.sb + bz * p.sb_bs + (n0 + r) * p.sb_rs);
+            sc_base = (const char*)(p.sb + bz * p.sb_bs + n0 * p.sb_rs);
+            sc_off = (uint32_t)(r * p.sb_rs);
         }
         sc_step = 4;
     } else if constexpr (!RC) {
-        if (tid < BM) {
+        if (wave < BM / 64) {
             const int r = tid < a_rows ? tid : a_rows - 1;
-            sc_src = (const char*)(p.s1 + bz * p.s1_bs + ((m0 + r) / p.gsM) * p.s1_rs);
+            sc_base = (const char*)(p.s1 + bz * p.s1_bs);
+            sc_off = (uint32_t)(((m0 + r) / p.gsM) * p.s1_rs * 4);
             sc_step = p.s1_cs * 4;
         } else {
-            sc_src = (const char*)(p.s2 + bz * p.s2_bs + (n0 / 128) * p.s2_cs);
+            sc_base = (const char*)(p.s2 + bz * p.s2_bs + (n0 / 128) * p.s2_cs);
             sc_step = p.s2_rs * 4;
         }
     }
+    const uint32_t lds0 = (uint32_t)(uintptr_t)(const __attribute__((address_space(3))) void*)smem + (uint32_t)wave * 1024u;
+    const uint32_t lds_sc0 = (uint32_t)(uintptr_t)(const __attribute__((address_space(3))) void*)smem + A_BYTES + B_BYTES + (uint32_t)wave * 256u;
     auto issue_piece = [&](int kt, int stage, int idx) {
-        char* sA = smem + stage * STAGE + wave * 1024;
-        char* sB = sA + A_BYTES;
-        const int8_t* Ak = uniform_ptr(A + (int64_t)kt * BK);
-        const int8_t* Bk = uniform_ptr(B + (int64_t)kt * BK);
-        if (idx < NA) async_copy16(Ak + a_off[idx], sA + idx * NT * 16);
-        else if (idx < NA + NB) async_copy16(Bk + b_off[idx - NA], sB + (idx - NA) * NT * 16);
-        else async_copy4(sc_src + (int64_t)kt * sc_step, smem + stage * STAGE + A_BYTES + B_BYTES + wave * 256);
+        const uint32_t sA = lds0 + stage * STAGE, sB = sA + A_BYTES;
+        if (idx < NA) copy16_sbase(uniform_ptr(A + (int64_t)kt * BK), a_off[idx], sA + idx * NT * 16);
+        else if (idx < NA + NB) copy16_sbase(uniform_ptr(B + (int64_t)kt * BK), b_off[idx - NA], sB + (idx - NA) * NT * 16);
+        else copy4_sbase(uniform_ptr((const int8_t*)sc_base + (int64_t)kt * sc_step), sc_off, lds_sc0 + stage * STAGE);
     };
     auto issue_tile = [&](int kt) {
 #pragma unroll
@@ -331,13 +347,14 @@ __global__ __launch_bounds__(512, 1) void qmm_fp8_exact_kernel(Fp8xParams p, int
     //     (whose groups 0 and 1 were those steps' last readers; the bytes were requested behind the barrier, two groups
     //     earlier), steps 2 and 3 behind groups 1 and 2 of the next tile's first.
     // The barrier sits before the last fragment: the next tile is complete in LDS and every wave is done reading this one.
-    int cur = 0;
 #if QG_DBG
     unsigned long long dbg_bar = 0, dbg_lgkm = 0;
     const unsigned long long dbg_c0 = clock64();
 #endif
-    for (int kt = 0; kt < KT; kt++) {
-        const int nxt = cur == STAGES - 1 ? 0 : cur + 1;
+    // (the stage index is a compile-time constant of each of the three copies of the loop body: LDS offsets are immediates)
+    auto k_step = [&](int kt, auto curc) {
+        constexpr int cur = decltype(curc)::value;
+        constexpr int nxt = cur == STAGES - 1 ? 0 : cur + 1;
         const char* st = smem + cur * STAGE;
         const char* stn = smem + nxt * STAGE;
         const int ktc = kt + 3 < KT ? kt + 3 : KT - 1;   // past the end the copies repeat the last tile into a stage nobody reads
@@ -417,7 +434,16 @@ __global__ __launch_bounds__(512, 1) void qmm_fp8_exact_kernel(Fp8xParams p, int
                 }
             }
         }
-        cur = nxt;
+    };
+    {
+        int kt = 0;
+        for (; kt + 3 <= KT; kt += 3) {
+            k_step(kt, std::integral_constant<int, 0>{});
+            k_step(kt + 1, std::integral_constant<int, 1>{});
+            k_step(kt + 2, std::integral_constant<int, 2>{});
+        }
+        if (kt < KT) k_step(kt, std::integral_constant<int, 0>{});
+        if (kt + 1 < KT) k_step(kt + 1, std::integral_constant<int, 1>{});
     }
 #if QG_DBG
     if (lane == 0 && p.dbg) {
@@ -554,6 +580,10 @@ int launch_blockscale_exact(const OpsnnQmmArgs& a, hipStream_t st)
     p.gsM = (int)a.gsM;
     if (((uintptr_t)p.a | (uintptr_t)p.b | (uint64_t)p.lda | (uint64_t)p.ldb | (uint64_t)p.a_bs | (uint64_t)p.b_bs) % 16) return OPSNN_NOT_TAKEN;
     if (((uintptr_t)p.s1 | (uintptr_t)p.s2) % 4) return OPSNN_NOT_TAKEN;
+    // the kernel addresses a row's s1 entries by a 32-bit byte offset from the batch's table, and operand rows of a tile
+    // by 32-bit offsets from the tile's first row
+    if (p.s1_rs < 0 || p.s1_cs < 0 || ((a.M + p.gsM - 1) / p.gsM) * p.s1_rs * 4 >= (1ll << 32)) return OPSNN_NOT_TAKEN;
+    if (p.lda < 0 || p.ldb < 0 || 256 * p.lda >= (1ll << 32) || 128 * p.ldb >= (1ll << 32)) return OPSNN_NOT_TAKEN;
     if (a.out_dtype == DT_BF16) return launch_fp8_exact<DT_BF16, false>(p, a.batch, st);
     if (a.out_dtype == DT_F32) return launch_fp8_exact<DT_F32, false>(p, a.batch, st);
     return launch_fp8_exact<DT_F16, false>(p, a.batch, st);
