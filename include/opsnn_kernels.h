@@ -121,10 +121,14 @@ OPSNN_API void opsnnSetWqTileMin(int m);
  *                                   initial limit); entries are evicted least recently used first;
  *   opsnnWeightCacheClear()         frees every entry.  The cache cannot see a weight change: call this before
  *                                   overwriting, freeing or re-using the memory of an operand that may be cached;
+ *   opsnnWeightCacheInvalidate(ptr, bytes)  frees the entries made from operands (data, scales or offsets) whose address
+ *                                   lies in [ptr, ptr + bytes) (bytes = 0: equals ptr) and returns their number: the
+ *                                   per-weight form of the call above, for a caller that updates one weight in place;
  *   opsnnWeightCacheStats(...)      entries, bytes held, hits and misses so far (any pointer may be NULL).
  * Calls made while their stream is being captured into a graph bypass the cache. */
 OPSNN_API void opsnnSetWeightCache(int64_t max_bytes);
 OPSNN_API void opsnnWeightCacheClear(void);
+OPSNN_API int opsnnWeightCacheInvalidate(const void* ptr, uint64_t bytes);
 OPSNN_API void opsnnWeightCacheStats(int64_t* entries, int64_t* bytes, int64_t* hits, int64_t* misses);
 /* MX: fp4/fp8 operands, e8m0 scale per 32 K. out = (x1*s1) @ (x2*s2) + fp32 bias. */
 OPSNN_API int opsnnQmmMx(const OpsnnQmmArgs* a, void* stream);

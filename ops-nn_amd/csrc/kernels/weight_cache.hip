@@ -8,7 +8,8 @@
 // matmul/quant_batch_matmul_v4/op_graph/fusion_pass/quant_batch_matmul_v4_transpose_fusion_pass.cpp).
 //
 // Contract: the cache cannot see a weight change.  A caller that overwrites, frees or re-uses the memory of a cached
-// operand must call opsnnWeightCacheClear() first.  Off by default.
+// operand must call opsnnWeightCacheInvalidate(ptr, bytes) for that operand (or opsnnWeightCacheClear()) first.  Off by
+// default.
 // A copy is written on the stream of the call that misses; an event recorded behind it orders every later use on
 // any stream.  Nothing is cached (and the caller's workspace path runs) while the stream is being captured into a
 // graph, when the copy does not fit the limit, or when the allocation fails.  Entries are evicted least recently
@@ -217,6 +218,22 @@ extern "C" void opsnnWeightCacheClear(void)
 {
     std::lock_guard<std::mutex> lock(g_mu);
     while (!g_entries.empty()) drop(g_entries.begin());
+}
+
+// Drops the entries made from one operand: every entry whose data, scale or offset address lies inside
+// [ptr, ptr + bytes) (bytes = 0: equals ptr).  Returns how many.
+extern "C" int opsnnWeightCacheInvalidate(const void* ptr, uint64_t bytes)
+{
+    if (!ptr) return 0;
+    const uintptr_t lo = (uintptr_t)ptr, hi = lo + (bytes ? bytes : 1);
+    auto inside = [&](const void* q) { return q && (uintptr_t)q >= lo && (uintptr_t)q < hi; };
+    std::lock_guard<std::mutex> lock(g_mu);
+    int n = 0;
+    for (auto it = g_entries.begin(); it != g_entries.end();) {
+        if (inside(it->src) || inside(it->src2) || inside(it->src3)) { it = drop(it); n++; }
+        else ++it;
+    }
+    return n;
 }
 
 extern "C" void opsnnWeightCacheStats(int64_t* entries, int64_t* bytes, int64_t* hits, int64_t* misses)

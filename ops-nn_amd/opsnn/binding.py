@@ -185,6 +185,7 @@ _SIGS = {
     "opsnnPackB4": (C.c_int, [C.c_void_p, C.c_int, C.c_void_p, C.c_int64, C.c_void_p]),
     "opsnnSetWeightCache": (None, [C.c_int64]),
     "opsnnWeightCacheClear": (None, []),
+    "opsnnWeightCacheInvalidate": (C.c_int, [C.c_void_p, C.c_uint64]),
     "opsnnWeightCacheStats": (None, [C.POINTER(C.c_int64), C.POINTER(C.c_int64), C.POINTER(C.c_int64), C.POINTER(C.c_int64)]),
     "opsnnQmmInt8": (C.c_int, [C.POINTER(OpsnnQmmArgs), C.c_void_p]),
     "opsnnQmmInt8Static": (C.c_int, [C.POINTER(OpsnnQmmArgs), C.c_void_p]),

@@ -72,6 +72,36 @@ def test_weight_only_weight_is_re_laid_out_once(cache):
     assert not np.array_equal(got2, first)
 
 
+def test_weight_overwritten_in_place_is_stale_until_invalidated(cache):
+    """The documented limit of the cache and its per-weight remedy: a weight overwritten in place keeps giving the old
+    weight's results (the cache keys on the address), opsnnWeightCacheInvalidate(ptr, bytes) drops exactly that operand's
+    entry -- another cached weight stays -- and the next call re-lays the new bytes out."""
+    m = cache
+    M, K, N = 16, 1024, 512
+    print(f"case weight cache, in-place overwrite {M}x{K}x{N}", flush=True)
+    inp = cases.make_wq_inputs(m, M, K, N, 5, m.ACL_FLOAT16, m.ACL_INT4, 128, False, True, None)
+    other = cases.make_wq_inputs(m, M, K, N, 6, m.ACL_FLOAT16, m.ACL_INT4, 128, False, True, None)
+    d = {k: m.DeviceBuffer(host=v) for k, v in inp.items() if isinstance(v, np.ndarray)}
+    d_other = {k: m.DeviceBuffer(host=v) for k, v in other.items() if isinstance(v, np.ndarray)}
+    d_y = m.DeviceBuffer(M * N * 2)
+    e0 = _stats(m)[0]
+    first = _wq_call(m, inp, d, d_y, M, K, N)
+    _wq_call(m, other, d_other, d_y, M, K, N)
+    assert _stats(m)[0] - e0 == 2
+    inp2 = cases.make_wq_inputs(m, M, K, N, 7, m.ACL_FLOAT16, m.ACL_INT4, 128, False, True, None)
+    inp2 = dict(inp2, x=inp["x"], scale=inp["scale"], offset=inp["offset"])
+    d["w"].upload(inp2["w"])
+    stale = _wq_call(m, inp2, d, d_y, M, K, N)
+    assert np.array_equal(stale, first), "the cache is expected to serve the old copy until it is told"
+    assert m.lib().opsnnWeightCacheInvalidate(d["w"].ptr, K * N // 2) == 1
+    assert _stats(m)[0] - e0 == 1   # the other weight's entry is still there
+    fresh = _wq_call(m, inp2, d, d_y, M, K, N)
+    want2 = cases.oracle_wq(m, inp2, M, K, N)
+    mx, mean = orc.rel_err_stats(orc.b16_to_f32(fresh, orc.F16), orc.b16_to_f32(want2, orc.F16))
+    assert mx <= 2.0 ** -7 and mean <= 2.0 ** -10 and not np.array_equal(fresh, first)
+    assert m.lib().opsnnWeightCacheInvalidate(d["w"].ptr, 0) == 1 and m.lib().opsnnWeightCacheInvalidate(d["w"].ptr, 0) == 0
+
+
 def test_int8_x2_is_re_laid_out_once_and_the_limit_evicts(cache):
     m = cache
     M, K, N = 128, 512, 384
