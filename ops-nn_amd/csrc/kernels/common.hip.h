@@ -202,6 +202,18 @@ __device__ __forceinline__ void async_copy16_uncounted(const void* g, void* lds)
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" : : "s"(l), "v"(g) : "memory", "m0");
 }
 
+// Asynchronous copies global -> LDS with the address as a wave-uniform 64-bit base in scalar registers plus a 32-bit byte
+// offset per lane: the loop spends no vector instruction on addresses.  (Written out: hidden from the compiler's wait-count
+// pass, like async_copy16_uncounted; the kernel waits for its copies by count.)  lds: wave-uniform LDS byte address.
+__device__ __forceinline__ void copy16_sbase(const void* base, uint32_t voff, uint32_t lds)
+{
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(lds), "v"(voff), "s"(base) : "memory", "m0");
+}
+__device__ __forceinline__ void copy4_sbase(const void* base, uint32_t voff, uint32_t lds)
+{
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2" : : "s"(lds), "v"(voff), "s"(base) : "memory", "m0");
+}
+
 // Workgroup ids are dealt round-robin over the 8 XCDs; give each XCD (own L2) a contiguous
 // range of logical tile ids so that neighbouring tiles share operand panels in one L2.
 __device__ __forceinline__ uint32_t xcd_remap(uint32_t wg, uint32_t total)

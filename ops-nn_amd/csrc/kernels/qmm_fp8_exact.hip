@@ -67,18 +67,6 @@ struct Fp8xParams {
 #endif
 };
 
-// Asynchronous copies global -> LDS with the address as a wave-uniform 64-bit base in scalar registers plus a 32-bit byte
-// offset per lane: the loop spends no vector instruction on addresses.  (Written out: hidden from the compiler's wait-count
-// pass, like async_copy16_uncounted; the kernel waits for its copies by count.)  lds: wave-uniform LDS byte address.
-__device__ __forceinline__ void copy16_sbase(const void* base, uint32_t voff, uint32_t lds)
-{
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(lds), "v"(voff), "s"(base) : "memory", "m0");
-}
-__device__ __forceinline__ void copy4_sbase(const void* base, uint32_t voff, uint32_t lds)
-{
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2" : : "s"(lds), "v"(voff), "s"(base) : "memory", "m0");
-}
-
 __device__ __forceinline__ const int8_t* uniform_ptr(const int8_t* p)
 {
     const uint64_t u = (uint64_t)p;

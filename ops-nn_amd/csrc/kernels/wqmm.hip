@@ -401,6 +401,31 @@ static int launch_slabs(WqParams p, hipStream_t st)
     // many rows: the dequantise-once tile kernel, one pass over the weight for up to 256 rows.  (Measured on 8192 x 28672
     // int4, group 128: 256 rows 165 us against 207 in two passes of the streaming kernel below; 128 rows 116 against 105,
     // 64 rows 94 against 69 -- hence the default switch at 129 rows; opsnnSetWqTileMin moves it.)
+    // From 129 rows: first the 256-row instance of the many-rows kernel (one pass over the weights per 256 rows, every weight
+    // dequantised once per wave and multiplied with all sixteen row blocks of x; needs the scale table in LDS), in equal
+    // slabs of up to 256 rows; then the tile kernel.  (Measured on 8192 x 28672 int4, fp16: 256 rows 151-155 us against 170 on
+    // the tile kernel, 192 rows 142-149 against 168.  Test hook: opsnnSetWqTileMin(m <= 128) sends such calls to the tile
+    // kernel first.)
+    if (p.M > 128 && opsnn_wq_tile_min() > 128) {
+        WqParams q = p;
+        WqStreamOpts o{};
+        if (stream_eligible<WBITS>(q, o) && o.rows) {
+            // whole passes of 256 rows, then the rest in one pass (up to 128 rows: the smaller instances, whose time grows
+            // with the rows they serve; measured at 300 rows: 256 + 44 rows 20 % ahead of two passes of 150)
+            const int64_t slab = 256;
+            bool taken = true;
+            for (int64_t m0 = 0; m0 < q.M && taken; m0 += slab) {
+                q.m_base = m0;
+                q.m_rows = (q.M - m0) < slab ? (q.M - m0) : slab;
+                const int rc = launch_wq_stream<XDT, WBITS>(q, o, st);
+                // (the kernel's conditions look at K, N, the group size and the scale layout, not at the slab: a refusal
+                // can only come before anything has been written)
+                if (rc == OPSNN_NOT_TAKEN && m0 == 0) taken = false;
+                else if (rc != 0) return rc;
+            }
+            if (taken) return 0;
+        }
+    }
     if (p.M >= opsnn_wq_tile_min() && p.M <= 256) {
         const int rc = launch_wq_tile<XDT, WBITS>(p, st);
         if (rc != OPSNN_NOT_TAKEN) return rc;

@@ -436,16 +436,27 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void w
     static_assert(WF != 3 || (WBITS == 8 && XDT == DT_F16 && WK == 2 && NB == 2), "the block-scale form: fp16 x, e4m3 w, a slab per 128-block");
     static_assert(WF != 4 || (WBITS == 8 && XDT == DT_F16 && !HAS_OFF), "the row / column scale form: fp16 x, e4m3 w");
     constexpr int NT = 512;
-    constexpr int KPL = 128 / WBITS, KC = 4 * KPL, STEPS = KC / 32;
-    constexpr int PF = 8 / NB;           // of this wave's chunks in flight per row block (a chunk is 500 to 1000 clocks of MFMA work here)
-    constexpr int KX = WK * KC;          // k per slab
-    constexpr int XROW = KX * 2;         // LDS row pitch (bytes)
-    constexpr int XPR = KX / 8;          // 16-byte pieces per x row per slab
+    // 256 rows of x (MB = 16) with 4-bit weights: a lane's weight piece is 8 bytes instead of 16 (HP), so that a chunk is
+    // 64 k per wave like an 8-bit one and two slab buffers of 256 rows fit the LDS (2 x 64 KB).  (Half-chunk slabs under
+    // 16-byte pieces were built first: the wait for a chunk's second slab is a wait for everything older, the weight
+    // fetch just issued included -- loads return in order --, and the 256-row instance ran at 224 us against the tile
+    // kernel's 167.)
+    constexpr bool HP = MB == 16 && WBITS == 4;
+    constexpr int PB = HP ? 8 : 16;                // bytes of a lane's weight piece
+    constexpr int KCH = 4 * (128 / WBITS);         // the chunk the launcher counts groups in (cpg_shift)
+    constexpr int KPL = PB * 8 / WBITS, KC = 4 * KPL, STEPS = KC / 32;
+    constexpr int PF = MB > 8 ? 4 : 8 / NB;   // of this wave's chunks in flight per row block (a chunk is 500 to 1000 clocks of MFMA work here)
+    constexpr int XH = 1;
+    constexpr int PPH = KPL / 8 / XH;    // 16-byte pieces of x per lane group and slab (= K steps per slab)
+    constexpr int KX = WK * KC;          // k per chunk of the workgroup (all WK waves)
+    constexpr int XROW = KX * 2 / XH;    // LDS row pitch (bytes)
+    constexpr int XPR = KX / 8 / XH;     // 16-byte pieces per x row per slab
     constexpr int XBUF = 16 * MB * XROW; // one slab buffer
     constexpr int XITEMS = 16 * MB * XPR / NT;
     constexpr int NBL = (WF >= 3 || SLDS) ? NB : NB * (HAS_OFF ? 3 : 2);   // loads of one weight fetch
     constexpr int LDS_MAIN = (2 * XBUF > WN * (WK - 1) * NB * MB * 4 * 64 * 4) ? 2 * XBUF : WN * (WK - 1) * NB * MB * 4 * 64 * 4;
-    static_assert((16 * MB * XPR) % NT == 0 && XPR >= 16 && PF >= 2, "staging and prefetch shape");
+    static_assert((16 * MB * XPR) % NT == 0 && XPR >= 16 && PF >= 2 && PPH >= 1 && STEPS == PPH * XH, "staging and prefetch shape");
+    static_assert(MB <= 8 || (WF == 0 && SLDS), "the 256-row instance is built for integer codes with the scale table in LDS");
     extern __shared__ __attribute__((aligned(16))) char sx[];
 
     const int tid = threadIdx.x, lane = tid & 63;
@@ -459,7 +470,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void w
     const int NSLAB = Ki / KX;           // = chunks per wave
     const int rows = (int)p.m_rows;
 
-    const uint8_t* wptr = p.w + (n0 + nrow) * p.ldw + g * 16 + wk * 64;
+    const uint8_t* wptr = p.w + (n0 + nrow) * p.ldw + g * PB + wk * (4 * PB);
     const int64_t wblk = 16 * p.ldw;     // bytes between the row blocks of a wave
     const uint16_t* srow = p.scale + (n0 + nrow) * p.s_cs;
     const uint16_t* orow = HAS_OFF ? p.offset + (n0 + nrow) * p.s_cs : nullptr;
@@ -478,28 +489,54 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void w
     // wk ^ bit 2 of the row, the same for both lane groups of a half-wave, and the two passes split the columns evenly.
     constexpr bool SWAP24 = XPR == 32 && KPL == 32;
     auto piece_of_pos = [](int q) { return SWAP24 ? ((q & ~0x14) | ((q & 4) << 2) | ((q & 16) >> 2)) : q; };   // (its own inverse)
-    const uint16_t* xsrc[XITEMS];
+    // Byte offsets from the slab's first row at K position 0 (the launcher keeps rows * K * 2 below 4 GB).  Rows past the
+    // last one repeat it.  With 16 pieces per slab row an instruction covers 32 whole rows and a thread keeps its piece
+    // position, so offset(it) = min(offset(0) + it * 32 rows, offset of the same piece in the last row): two registers
+    // instead of XITEMS (the 256-row instance has none to spare).
+    constexpr bool XLIN = XPR == 16;
+    uint32_t xsrc[XLIN ? 1 : XITEMS];
+    uint32_t xsrc_max = 0;
+    const uint16_t* xbase = p.x + p.m_base * p.K;
+    (void)xsrc_max;
 #pragma unroll
-    for (int it = 0; it < XITEMS; it++) {
+    for (int it = 0; it < (XLIN ? 1 : XITEMS); it++) {
         const int L = it * NT + tid;
         const int r = L / XPR, pos = L % XPR;
         const int rr = r < rows ? r : rows - 1;
-        xsrc[it] = p.x + (p.m_base + rr) * p.K + piece_of_pos(pos ^ (r & 15)) * 8;
+        // piece q of a slab row: wave column q / (XPR / WK), lane group (q % (XPR / WK)) / PPH, K step q % PPH of the slab; in x
+        // that is piece wk * (KC / 8) + g * (KPL / 8) + step of the chunk (the identity when a slab holds whole chunks)
+        const int q = piece_of_pos(pos ^ (r & 15));
+        const int src_piece = (q / (XPR / WK)) * (KC / 8) + ((q % (XPR / WK)) / PPH) * (KPL / 8) + q % PPH;
+        xsrc[it] = (uint32_t)(rr * Ki + src_piece * 8) * 2u;
+        if constexpr (XLIN) {
+            xsrc[0] = (uint32_t)(r * Ki + src_piece * 8) * 2u;   // (r may lie past the last row: the minimum below puts it back)
+            xsrc_max = (uint32_t)((rows - 1) * Ki + src_piece * 8) * 2u;
+        }
     }
-    auto issue_x = [&](int slab) {
-        char* dst = sx + (slab & 1) * XBUF + wave * 1024;
+    auto xsrc_at = [&](int it) -> uint32_t {
+        if constexpr (XLIN) {
+            const uint32_t o = xsrc[0] + (uint32_t)it * (uint32_t)(NT / XPR) * (uint32_t)Ki * 2u;
+            return o < xsrc_max ? o : xsrc_max;
+        } else {
+            return xsrc[it];
+        }
+    };
+    auto issue_x = [&](int slab) {   // slab = chunk * XH + half
+        const uint32_t dst = (uint32_t)(uintptr_t)(const __attribute__((address_space(3))) void*)sx + (slab & 1) * XBUF + wave * 1024;
+        const uint16_t* src = xbase + (int64_t)(slab / XH) * KX + (slab % XH) * (PPH * 8);
+        // (readfirstlane returns a signed int: each half goes through uint32_t before the halves are joined)
+        const uint32_t sb_lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(uintptr_t)src);
+        const uint32_t sb_hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)((uintptr_t)src >> 32));
+        const uint64_t sb = ((uint64_t)sb_hi << 32) | (uint64_t)sb_lo;
 #pragma unroll
-        for (int it = 0; it < XITEMS; it++) async_copy16_uncounted(xsrc[it] + (int64_t)slab * KX, dst + it * NT * 16);
+        for (int it = 0; it < XITEMS; it++) copy16_sbase((const void*)sb, xsrc_at(it), dst + it * NT * 16);
     };
     // LDS byte offset of this lane's column operand inside a buffer, per 16-row block of x, at K step 0 (the lane's
     // weights cover k = g*KPL .. +KPL of the chunk, step s the 8 at 8s); step s is s pieces further on, which the
     // swizzle turns into an exclusive-or with 16s
-    int xoff[MB];
-#pragma unroll
-    for (int b = 0; b < MB; b++) {
-        const int r = 16 * b + nrow;
-        xoff[b] = r * XROW + (piece_of_pos(wk * (KC / 8) + g * (KPL / 8)) ^ (r & 15)) * 16;
-    }
+    // (row block b of x lies b * 16 * XROW further on: an immediate offset of the read, since the swizzle only looks at the row's low four bits)
+    const int xoff0 = nrow * XROW + (piece_of_pos(wk * (XPR / WK) + g * PPH) ^ nrow) * 16;
+    auto xoff_at = [&](int b, int s) { return (xoff0 ^ (16 * s)) + b * (16 * XROW); };
 
     v4f acc[NB][MB];
 #pragma unroll
@@ -524,7 +561,8 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void w
     // row; the swizzle (4 * (rw % 16), kept below G) spreads the 16 rows that one read touches over the banks.  The table is
     // complete behind the loop's first barrier.
     uint32_t* stab = (uint32_t*)(sx + LDS_MAIN);
-    const int sG = p.cpg_shift >= 31 ? 1 : (int)((p.K / KC) >> p.cpg_shift);
+    const int sG = p.cpg_shift >= 31 ? 1 : (int)((p.K / KCH) >> p.cpg_shift);
+    const int cpg_shift = p.cpg_shift >= 31 ? 31 : p.cpg_shift + (HP ? 1 : 0);   // chunks of this kernel per group
     int stab_row[NB], stab_sw[NB];
     (void)stab; (void)sG; (void)stab_row; (void)stab_sw;
     if constexpr (SLDS) {
@@ -549,10 +587,15 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void w
     v4i wq[PF][NB];
     uint16_t sq[PF][NB], oq[PF][NB];
     auto fetch = [&](int j, int cw) {   // chunk cw of this wave (chunk cw * WK + wk of the row) into slot j
-        const int64_t so = (int64_t)((cw * WK + wk) >> p.cpg_shift) * p.s_rs;
+        const int64_t so = (int64_t)((cw * WK + wk) >> cpg_shift) * p.s_rs;
 #pragma unroll
         for (int q = 0; q < NB; q++) {
-            wq[j][q] = *(const v4i*)(wptr + q * wblk + (int64_t)cw * (WK * 64));
+            if constexpr (HP) {
+                const v2i t = *(const v2i*)(wptr + q * wblk + (int64_t)cw * (WK * 4 * PB));
+                wq[j][q] = (v4i){t[0], t[1], 0, 0};
+            } else {
+                wq[j][q] = *(const v4i*)(wptr + q * wblk + (int64_t)cw * (WK * 64));
+            }
             if constexpr (SLDS) { sq[j][q] = 0; oq[j][q] = 0; continue; }
             if constexpr (WF >= 3) sq[j][q] = 0;
             else if constexpr (WF == 2) sq[j][q] = srow8[q * sblk + (cw * WK + wk) * 4];
@@ -565,7 +608,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void w
     v4i aop[NB];                   // the dequantised weights of the K step about to be multiplied
     auto load_sow = [&](int cw, uint32_t (&sow)[NB]) {
         if constexpr (SLDS) {
-            const int gi = (cw * WK + wk) >> p.cpg_shift;
+            const int gi = (cw * WK + wk) >> cpg_shift;
 #pragma unroll
             for (int q = 0; q < NB; q++) sow[q] = stab[stab_row[q] + (gi ^ stab_sw[q])];
         } else {
@@ -592,7 +635,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void w
     };
     auto read_frags = [&](const char* xs, int s, v4i (&bops)[MB]) {
 #pragma unroll
-        for (int b = 0; b < MB; b++) bops[b] = *(const v4i*)(xs + (xoff[b] ^ (16 * s)));
+        for (int b = 0; b < MB; b++) bops[b] = *(const v4i*)(xs + xoff_at(b, s));
     };
     auto mma_step = [&](const v4i (&a)[NB], const v4i (&bops)[MB]) {
 #pragma unroll
@@ -601,6 +644,21 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void w
             for (int q = 0; q < NB; q++) {
                 if constexpr (XDT == DT_F16) acc[q][b] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(v8h, a[q]), __builtin_bit_cast(v8h, bops[b]), acc[q][b], 0, 0, 0);
                 else acc[q][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf, a[q]), __builtin_bit_cast(v8bf, bops[b]), acc[q][b], 0, 0, 0);
+            }
+    };
+    auto read_frags_part = [&](auto b0c, const char* xs, int s, v4i (&bops)[MB / 4]) {
+        constexpr int B0 = decltype(b0c)::value;
+#pragma unroll
+        for (int b = 0; b < MB / 4; b++) bops[b] = *(const v4i*)(xs + xoff_at(B0 + b, s));
+    };
+    auto mma_part = [&](auto b0c, const v4i (&a)[NB], const v4i (&bops)[MB / 4]) {
+        constexpr int B0 = decltype(b0c)::value;
+#pragma unroll
+        for (int b = 0; b < MB / 4; b++)
+#pragma unroll
+            for (int q = 0; q < NB; q++) {
+                if constexpr (XDT == DT_F16) acc[q][B0 + b] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(v8h, a[q]), __builtin_bit_cast(v8h, bops[b]), acc[q][B0 + b], 0, 0, 0);
+                else acc[q][B0 + b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf, a[q]), __builtin_bit_cast(v8bf, bops[b]), acc[q][B0 + b], 0, 0, 0);
             }
     };
 #pragma unroll
@@ -612,11 +670,18 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void w
 #pragma unroll
         for (int j = 0; j < PF; j++) {
             const int cw = c0 + j;
-            // this thread's copies of slab cw have landed (only the weight fetch issued after them may be in flight)
-            if (cw > 0) wait_vmcnt<NBL>();
-            __syncthreads();   // slab cw is complete and visible; every wave has finished slab cw-1
-            if (cw + 1 < NSLAB) issue_x(cw + 1);
-            const char* xs = sx + (cw & 1) * XBUF;
+            uint32_t sow[NB];
+#pragma unroll
+            for (int h = 0; h < XH; h++) {
+            // this thread's copies of the slab have landed (behind a chunk's first slab only the weight fetch issued after
+            // them may be in flight; behind its second one nothing was issued)
+            if (h > 0) wait_vmcnt<0>();
+            else if (cw > 0) wait_vmcnt<NBL>();
+            __syncthreads();   // the slab is complete and visible; every wave has finished the one before
+            const int sl = cw * XH + h;
+            if (sl + 1 < NSLAB * XH) issue_x(sl + 1);
+            const char* xs = sx + (sl & 1) * XBUF;
+            if constexpr (WF != 3) { if (h == 0) load_sow(cw, sow); }   // (behind the barrier: the first one also completes the scale table)
             if constexpr (WF == 3) {
                 // this wave's half of block cw: two instructions per fragment pair from zero, then the fold
                 v4i aw[NB][2];
@@ -648,7 +713,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void w
 #pragma unroll
                             for (int h = 0; h < 2; h++) {
                                 const int b = 2 * bp + h;
-                                const v4i b0 = *(const v4i*)(xs + xoff[b]), b1 = *(const v4i*)(xs + (xoff[b] ^ 16));
+                                const v4i b0 = *(const v4i*)(xs + xoff_at(b, 0)), b1 = *(const v4i*)(xs + xoff_at(b, 1));
                                 scc[h] = scr[16 * b];
 #pragma unroll
                                 for (int q = 0; q < NB; q++)
@@ -680,7 +745,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void w
                 } else {
 #pragma unroll
                 for (int b = 0; b < MB; b++) {
-                    const v4i b0 = *(const v4i*)(xs + xoff[b]), b1 = *(const v4i*)(xs + (xoff[b] ^ 16));
+                    const v4i b0 = *(const v4i*)(xs + xoff_at(b, 0)), b1 = *(const v4i*)(xs + xoff_at(b, 1));
                     const float sc = scr[16 * b];
                     v4f t[NB];
 #pragma unroll
@@ -697,21 +762,38 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void w
                 }
             }
             if constexpr (WF != 3) {
-                // A chunk's work: per K step the x fragments are requested first, so that they arrive in the shadow of the
+                // A slab's work: per K step the x fragments are requested first, so that they arrive in the shadow of the
                 // step's dequantisation (vector ALU) instead of each pair of matrix instructions waiting for a read issued
-                // just in front of it.  (Measured and not kept: the second wave of each SIMD running half a step ahead of
-                // the first; the matrix instructions of a step interleaved one by one with the next step's dequantisation;
-                // sixteen waves, four per SIMD -- all within 3 % of this order at 64 rows, none better at 128.)
-                uint32_t sow[NB];
-                load_sow(cw, sow);
+                // just in front of it.
 #pragma unroll
-                for (int s = 0; s < STEPS; s++) {
-                    v4i bops[MB];
-                    read_frags(xs, s, bops);
-                    __builtin_amdgcn_sched_barrier(0);
-                    dequant_step(j, s, sow, aop);
-                    mma_step(aop, bops);
+                for (int s = 0; s < PPH; s++) {
+                    if constexpr (MB <= 8) {
+                        v4i bops[MB];
+                        read_frags(xs, s, bops);
+                        __builtin_amdgcn_sched_barrier(0);
+                        dequant_step(j, h * PPH + s, sow, aop);
+                        mma_step(aop, bops);
+                    } else {
+                        // 256 rows: the fragments in four groups of four, two groups requested ahead of the matrix
+                        // instructions that use them (all sixteen at once would need 64 registers beside 128 sums)
+                        constexpr int Q = MB / 4;
+                        v4i b0[Q], b1[Q], b2[Q], b3[Q];
+                        read_frags_part(std::integral_constant<int, 0>{}, xs, s, b0);
+                        read_frags_part(std::integral_constant<int, Q>{}, xs, s, b1);
+                        __builtin_amdgcn_sched_barrier(0);
+                        dequant_step(j, h * PPH + s, sow, aop);
+                        __builtin_amdgcn_sched_barrier(0);
+                        mma_part(std::integral_constant<int, 0>{}, aop, b0);
+                        read_frags_part(std::integral_constant<int, 2 * Q>{}, xs, s, b2);
+                        __builtin_amdgcn_sched_barrier(0);
+                        mma_part(std::integral_constant<int, Q>{}, aop, b1);
+                        read_frags_part(std::integral_constant<int, 3 * Q>{}, xs, s, b3);
+                        __builtin_amdgcn_sched_barrier(0);
+                        mma_part(std::integral_constant<int, 2 * Q>{}, aop, b2);
+                        mma_part(std::integral_constant<int, 3 * Q>{}, aop, b3);
+                    }
                 }
+            }
             }
             const int nx = cw + PF;
             fetch(j, nx < NSLAB ? nx : NSLAB - 1);   // past the end: a harmless reload of the last chunk
@@ -1303,7 +1385,8 @@ template <int XDT, int WBITS, int MB, int NB, int WN, int WK, bool HAS_OFF, int 
 static int launch_rows_one(const WqParams& p, hipStream_t st)
 {
     constexpr int KC = 4 * (128 / WBITS);
-    constexpr size_t lds_x = 2 * (size_t)(16 * MB) * (WK * KC * 2);
+    constexpr int XH = (MB == 16 && WBITS == 4) ? 2 : 1;   // as in the kernel: half-chunk slabs for 256 rows of x with 4-bit weights
+    constexpr size_t lds_x = 2 * (size_t)(16 * MB) * (WK * KC * 2 / XH);
     size_t lds_stab = 0;
     if constexpr (WF == 0 && !SLDS) {
         // the scales and offsets of the workgroup's columns in LDS when a row's scales are contiguous, their count per row
@@ -1313,6 +1396,8 @@ static int launch_rows_one(const WqParams& p, hipStream_t st)
         if ((p.s_rs == 1 || G == 1) && (G & (G - 1)) == 0 && (lds_x > red ? lds_x : red) + (size_t)(16 * NB * WN) * G * 4 <= 160 * 1024)
             return launch_rows_one<XDT, WBITS, MB, NB, WN, WK, HAS_OFF, WF, true>(p, st);
     }
+    if constexpr (MB > 8 && !SLDS) return OPSNN_NOT_TAKEN;   // the 256-row instance exists with the scale table only
+    else {
     if constexpr (SLDS) lds_stab = (size_t)(16 * NB * WN) * (p.cpg_shift >= 31 ? 1 : ((p.K / KC) >> p.cpg_shift)) * 4;
     constexpr size_t lds_red = (size_t)WN * (WK - 1) * NB * MB * 4 * 64 * 4;
     constexpr size_t lds_main = lds_x > lds_red ? lds_x : lds_red;
@@ -1329,6 +1414,7 @@ static int launch_rows_one(const WqParams& p, hipStream_t st)
     }
     hipLaunchKernelGGL(k, dim3(grid), dim3(512), lds, st, p);
     return (int)hipGetLastError();
+    }
 }
 
 struct WqStreamOpts {
@@ -1384,6 +1470,8 @@ int launch_wq_rows_float(const WqParams& p, hipStream_t st);
             return o.has_off ? launch_resx_one<XDT, WBITS, true, false>(p, st)                                      \
                              : launch_resx_one<XDT, WBITS, false, false>(p, st);                                    \
         }                                                                                                           \
+        if (o.rows && p.m_rows > 128) return o.has_off ? launch_rows_one<XDT, WBITS, 16, 2, 4, 2, true>(p, st)            \
+                                                       : launch_rows_one<XDT, WBITS, 16, 2, 4, 2, false>(p, st);          \
         if (o.rows && p.m_rows > 64) return o.has_off ? launch_rows_one<XDT, WBITS, 8, 2, 4, 2, true>(p, st)              \
                                                       : launch_rows_one<XDT, WBITS, 8, 2, 4, 2, false>(p, st);            \
         if (o.rows) return o.has_off ? launch_rows_one<XDT, WBITS, 4, 2, 4, 2, true>(p, st)                               \

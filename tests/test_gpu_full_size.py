@@ -49,6 +49,9 @@ def test_config3_w4a16_per_group_full(gpu, M):
     rows = _rows(M, 6, 3)
     want = cases.oracle_wq(m, inp, M, K, N, rows=rows)
     check_close(got[rows], want, m.ACL_FLOAT16, f"config 3 M={M}")
+    # the same call again: the same bits (a workgroup-wide table read before the barrier that completes it once showed as
+    # one or two wrong columns in some runs only, and only at this size)
+    assert np.array_equal(cases.run_wq_aclnn(m, inp, M, K, N), got), "two runs of the same call differ"
     # doubling x (exact in fp16, subnormals included) doubles every product, every partial sum and every output
     # exactly, except outputs so small that fp16 rounds them on the subnormal grid
     inp2 = dict(inp, x=orc.f32_to_b16(orc.b16_to_f32(inp["x"], m.ACL_FLOAT16) * np.float32(2.0), m.ACL_FLOAT16))
@@ -63,6 +66,7 @@ def test_config3_m256_sampled(gpu):
     got = cases.run_wq_aclnn(m, inp, M, K, N)
     rows = _rows(M, 6, 4)
     check_close(got[rows], cases.oracle_wq(m, inp, M, K, N, rows=rows), m.ACL_FLOAT16, "config 3 M=256")
+    assert np.array_equal(cases.run_wq_aclnn(m, inp, M, K, N), got), "two runs of the same call differ"
 
 
 def test_config4_fp8_block_scale_full(gpu):

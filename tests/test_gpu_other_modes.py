@@ -421,6 +421,41 @@ def test_weight_only_tile_kernel(gpu, M, K, N, x_dt, w_dt, group, tW, off, bias)
 
 
 @pytest.mark.parametrize("M,K,N,x_dt,w_dt,group,tW,off,bias", [
+    # 129 .. 256 rows on the 256-row instance of the many-rows kernel (a weight row's scales contiguous, a power-of-two
+    # group count, K a multiple of two chunk pairs, N % 32 == 0): int4 with half-chunk x slabs, int8 with whole ones;
+    # ragged row counts (the slab's missing rows repeat the last one), ragged last column block, per-channel scales, bias
+    (256, 2048, 512, "f16", "i4", 128, True, True, None),
+    (200, 4096, 288, "f16", "i4", 128, True, False, "f16"),
+    (129, 1024, 256, "bf16", "i4", 256, True, True, None),
+    (256, 1024, 320, "bf16", "i4", 0, True, False, "bf16"),
+    (256, 1024, 512, "f16", "i8", 128, True, True, None),
+    (177, 2048, 256, "bf16", "i8", 0, True, False, None),
+    # more than 256 rows: whole passes of 256, then the rest on the instance that fits it (44, 8 and 200 rows here)
+    (300, 1024, 256, "f16", "i4", 128, True, True, None),
+    (520, 1024, 288, "bf16", "i4", 128, True, False, "bf16"),
+    (712, 1024, 256, "f16", "i8", 128, True, True, None),
+])
+def test_weight_only_256_row_instance(gpu, M, K, N, x_dt, w_dt, group, tW, off, bias):
+    """From 129 rows of x: passes of up to 256 rows on the many-rows kernel's 256-row instance (the default route for these
+    row counts; the tile kernel takes what it declines): the bar of the other matrix-instruction kernels, and the same call
+    on the tile kernel (opsnnSetWqTileMin(1)) within the same bar of the oracle."""
+    m = gpu
+    dt = {"bf16": m.ACL_BF16, "f16": m.ACL_FLOAT16, "i8": m.ACL_INT8, "i4": m.ACL_INT4, None: None}
+    print(f"case wq 256-row instance M={M} K={K} N={N} x={x_dt} w={w_dt} g={group} tW={tW} off={off} bias={bias}", flush=True)
+    inp = cases.make_wq_inputs(m, M, K, N, M * 7 + N, dt[x_dt], dt[w_dt], group, tW, off, dt[bias])
+    want = cases.oracle_wq(m, inp, M, K, N)
+    plain(False)
+    got = cases.run_wq_aclnn(m, inp, M, K, N)
+    check_close(got, want, dt[x_dt], "weight-only 256-row instance")
+    m.lib().opsnnSetWqTileMin(1)
+    try:
+        tile = cases.run_wq_aclnn(m, inp, M, K, N)
+    finally:
+        m.lib().opsnnSetWqTileMin(129)
+    check_close(tile, want, dt[x_dt], "weight-only tile kernel")
+
+
+@pytest.mark.parametrize("M,K,N,x_dt,w_dt,group,tW,off,bias", [
     # 4 .. 16 rows with K a multiple of 8 waves x 4, 8 or 16 chunks (int4: 4096, 8192; int8: 2048, 4096, 8192): groups of one
     # chunk (vector scale loads), of several chunks and per channel; with and without offset; ragged columns; fewer row
     # blocks than workgroups and more (a workgroup walks several); N-contiguous weight; bias
