@@ -436,12 +436,12 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void w
     static_assert(WF != 3 || (WBITS == 8 && XDT == DT_F16 && WK == 2 && NB == 2), "the block-scale form: fp16 x, e4m3 w, a slab per 128-block");
     static_assert(WF != 4 || (WBITS == 8 && XDT == DT_F16 && !HAS_OFF), "the row / column scale form: fp16 x, e4m3 w");
     constexpr int NT = 512;
-    // 256 rows of x (MB = 16) with 4-bit weights: a lane's weight piece is 8 bytes instead of 16 (HP), so that a chunk is
+    // More than 128 rows of x (MB = 12: up to 192, MB = 16: up to 256) with 4-bit weights: a lane's weight piece is 8 bytes instead of 16 (HP), so that a chunk is
     // 64 k per wave like an 8-bit one and two slab buffers of 256 rows fit the LDS (2 x 64 KB).  (Half-chunk slabs under
     // 16-byte pieces were built first: the wait for a chunk's second slab is a wait for everything older, the weight
     // fetch just issued included -- loads return in order --, and the 256-row instance ran at 224 us against the tile
     // kernel's 167.)
-    constexpr bool HP = MB == 16 && WBITS == 4;
+    constexpr bool HP = MB > 8 && WBITS == 4;
     constexpr int PB = HP ? 8 : 16;                // bytes of a lane's weight piece
     constexpr int KCH = 4 * (128 / WBITS);         // the chunk the launcher counts groups in (cpg_shift)
     constexpr int KPL = PB * 8 / WBITS, KC = 4 * KPL, STEPS = KC / 32;
@@ -530,6 +530,17 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void w
         const uint64_t sb = ((uint64_t)sb_hi << 32) | (uint64_t)sb_lo;
 #pragma unroll
         for (int it = 0; it < XITEMS; it++) copy16_sbase((const void*)sb, xsrc_at(it), dst + it * NT * 16);
+    };
+    // the same in parts: copies it0 .. it0 + n - 1
+    auto issue_x_part = [&](int slab, int it0, int n) {
+        const uint32_t dst = (uint32_t)(uintptr_t)(const __attribute__((address_space(3))) void*)sx + (slab & 1) * XBUF + wave * 1024;
+        const uint16_t* src = xbase + (int64_t)(slab / XH) * KX + (slab % XH) * (PPH * 8);
+        const uint32_t sb_lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(uintptr_t)src);
+        const uint32_t sb_hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)((uintptr_t)src >> 32));
+        const uint64_t sb = ((uint64_t)sb_hi << 32) | (uint64_t)sb_lo;
+#pragma unroll
+        for (int it = it0; it < it0 + n; it++)
+            if (it < XITEMS) copy16_sbase((const void*)sb, xsrc_at(it), dst + it * NT * 16);
     };
     // LDS byte offset of this lane's column operand inside a buffer, per 16-row block of x, at K step 0 (the lane's
     // weights cover k = g*KPL .. +KPL of the chunk, step s the 8 at 8s); step s is s pieces further on, which the
@@ -679,7 +690,12 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void w
             else if (cw > 0) wait_vmcnt<NBL>();
             __syncthreads();   // the slab is complete and visible; every wave has finished the one before
             const int sl = cw * XH + h;
-            if (sl + 1 < NSLAB * XH) issue_x(sl + 1);
+            // 256 rows: the slab's copies go out in pairs between the first groups of matrix instructions instead of in one
+            // burst behind the barrier (eight waves x eight copies of 1 KB fill the memory pipeline's queue, and every wave
+            // stood in front of its first matrix instruction until its last copy was accepted: a quarter of the slab's time)
+            constexpr bool SPREAD = MB > 8;
+            const bool more_x = sl + 1 < NSLAB * XH;
+            if (!SPREAD && more_x) issue_x(sl + 1);
             const char* xs = sx + (sl & 1) * XBUF;
             if constexpr (WF != 3) { if (h == 0) load_sow(cw, sow); }   // (behind the barrier: the first one also completes the scale table)
             if constexpr (WF == 3) {
@@ -783,13 +799,19 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void w
                         __builtin_amdgcn_sched_barrier(0);
                         dequant_step(j, h * PPH + s, sow, aop);
                         __builtin_amdgcn_sched_barrier(0);
+                        constexpr int CPG = (XITEMS + 3) / 4;   // copies behind each of the first step's four groups
+                        if (s == 0 && more_x) issue_x_part(sl + 1, 0, CPG);
                         mma_part(std::integral_constant<int, 0>{}, aop, b0);
                         read_frags_part(std::integral_constant<int, 2 * Q>{}, xs, s, b2);
+                        if (s == 0 && more_x) issue_x_part(sl + 1, CPG, CPG);
                         __builtin_amdgcn_sched_barrier(0);
                         mma_part(std::integral_constant<int, Q>{}, aop, b1);
                         read_frags_part(std::integral_constant<int, 3 * Q>{}, xs, s, b3);
+                        if (s == 0 && more_x) issue_x_part(sl + 1, 2 * CPG, CPG);
                         __builtin_amdgcn_sched_barrier(0);
                         mma_part(std::integral_constant<int, 2 * Q>{}, aop, b2);
+                        if (s == 0 && more_x) issue_x_part(sl + 1, 3 * CPG, CPG);
+                        __builtin_amdgcn_sched_barrier(0);
                         mma_part(std::integral_constant<int, 3 * Q>{}, aop, b3);
                     }
                 }
@@ -1385,7 +1407,7 @@ template <int XDT, int WBITS, int MB, int NB, int WN, int WK, bool HAS_OFF, int 
 static int launch_rows_one(const WqParams& p, hipStream_t st)
 {
     constexpr int KC = 4 * (128 / WBITS);
-    constexpr int XH = (MB == 16 && WBITS == 4) ? 2 : 1;   // as in the kernel: half-chunk slabs for 256 rows of x with 4-bit weights
+    constexpr int XH = (MB > 8 && WBITS == 4) ? 2 : 1;   // as in the kernel: 8-byte weight pieces, i.e. slabs of half the K, for more than 128 rows of x with 4-bit weights
     constexpr size_t lds_x = 2 * (size_t)(16 * MB) * (WK * KC * 2 / XH);
     size_t lds_stab = 0;
     if constexpr (WF == 0 && !SLDS) {
@@ -1470,8 +1492,10 @@ int launch_wq_rows_float(const WqParams& p, hipStream_t st);
             return o.has_off ? launch_resx_one<XDT, WBITS, true, false>(p, st)                                      \
                              : launch_resx_one<XDT, WBITS, false, false>(p, st);                                    \
         }                                                                                                           \
-        if (o.rows && p.m_rows > 128) return o.has_off ? launch_rows_one<XDT, WBITS, 16, 2, 4, 2, true>(p, st)            \
+        if (o.rows && p.m_rows > 192) return o.has_off ? launch_rows_one<XDT, WBITS, 16, 2, 4, 2, true>(p, st)            \
                                                        : launch_rows_one<XDT, WBITS, 16, 2, 4, 2, false>(p, st);          \
+        if (o.rows && p.m_rows > 128) return o.has_off ? launch_rows_one<XDT, WBITS, 12, 2, 4, 2, true>(p, st)            \
+                                                       : launch_rows_one<XDT, WBITS, 12, 2, 4, 2, false>(p, st);          \
         if (o.rows && p.m_rows > 64) return o.has_off ? launch_rows_one<XDT, WBITS, 8, 2, 4, 2, true>(p, st)              \
                                                       : launch_rows_one<XDT, WBITS, 8, 2, 4, 2, false>(p, st);            \
         if (o.rows) return o.has_off ? launch_rows_one<XDT, WBITS, 4, 2, 4, 2, true>(p, st)                               \

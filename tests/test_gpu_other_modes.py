@@ -430,6 +430,8 @@ def test_weight_only_tile_kernel(gpu, M, K, N, x_dt, w_dt, group, tW, off, bias)
     (256, 1024, 320, "bf16", "i4", 0, True, False, "bf16"),
     (256, 1024, 512, "f16", "i8", 128, True, True, None),
     (177, 2048, 256, "bf16", "i8", 0, True, False, None),
+    (193, 2048, 256, "f16", "i4", 128, True, True, "f16"),     # one row more than the 192-row instance takes
+    (192, 1024, 288, "f16", "i8", 128, True, True, None),
     # more than 256 rows: whole passes of 256, then the rest on the instance that fits it (44, 8 and 200 rows here)
     (300, 1024, 256, "f16", "i4", 128, True, True, None),
     (520, 1024, 288, "bf16", "i4", 128, True, False, "bf16"),
