@@ -693,7 +693,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void w
             // 256 rows: the slab's copies go out in pairs between the first groups of matrix instructions instead of in one
             // burst behind the barrier (eight waves x eight copies of 1 KB fill the memory pipeline's queue, and every wave
             // stood in front of its first matrix instruction until its last copy was accepted: a quarter of the slab's time)
-            constexpr bool SPREAD = MB > 8;
+            constexpr bool SPREAD = MB > 8 || (WF == 0 && PPH >= 2);
             const bool more_x = sl + 1 < NSLAB * XH;
             if (!SPREAD && more_x) issue_x(sl + 1);
             const char* xs = sx + (sl & 1) * XBUF;
@@ -787,6 +787,10 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void w
                         v4i bops[MB];
                         read_frags(xs, s, bops);
                         __builtin_amdgcn_sched_barrier(0);
+                        if constexpr (SPREAD) {   // the next slab's copies in two halves, behind the fragment requests of the first two steps
+                            constexpr int CPH = (XITEMS + 1) / 2;
+                            if (s < 2 && more_x) issue_x_part(sl + 1, s * CPH, CPH);
+                        }
                         dequant_step(j, h * PPH + s, sow, aop);
                         mma_step(aop, bops);
                     } else {
