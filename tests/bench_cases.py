@@ -25,8 +25,8 @@ PROFILED_TRAFFIC = {
     (3, 16, "cold"): (132.1e6, "profiles/wqmm_decode_w4a16_m16_k8192_n28672_cold.txt"),
     (3, 64, "warm"): (137.8e6, "profiles/wqmm_decode_w4a16_m64_k8192_n28672.txt"),
     (3, 64, "cold"): (137.9e6, "profiles/wqmm_decode_w4a16_m64_k8192_n28672_cold.txt"),
-    (3, 256, "warm"): (257.7e6, "profiles/wqmm_decode_w4a16_m256_k8192_n28672.txt"),
-    (3, 256, "cold"): (255.9e6, "profiles/wqmm_decode_w4a16_m256_k8192_n28672_cold.txt"),
+    (3, 256, "warm"): (196.9e6, "profiles/wqmm_decode_w4a16_m256_k8192_n28672.txt"),
+    (3, 256, "cold"): (193.0e6, "profiles/wqmm_decode_w4a16_m256_k8192_n28672_cold.txt"),
     (4, None, "exact"): (1220.4e6, "profiles/qmm_fp8_exact_m4096_k7168_n18432.txt"),
     (4, None, "fast"): (1502.4e6, "profiles/qmm_fp8_block_m4096_k7168_n18432.txt"),
     (5, None, None): (2229.0e6, "profiles/qgemm_mxfp4_b8_m4096_k8192_n8192.txt"),
@@ -426,7 +426,7 @@ class ConfigWQ(Workload):
         self.inp = dict(self.inp_full, x=np.ascontiguousarray(self.inp_full["x"][:M]))
         self.kernel = ("wqmm_resx_kernel" if (self.cfg == 3 and M <= 3) else "wqmm_xreg_kernel" if M <= 16 else
                        "wqmm_decode_kernel" if self.cfg == 11 else
-                       "wqmm_tile_kernel" if M > 128 else "wqmm_rows_kernel" if M > 48 else "wqmm_stream_kernel")
+                       "wqmm_rows_kernel<256 or 192 rows>" if M > 128 else "wqmm_rows_kernel" if M > 48 else "wqmm_stream_kernel")
         self.t_x = m.Tensor((M, K), self.x_dt, self.d["x"])
         self.t_y = m.Tensor((M, N), self.x_dt, self.d_y)
         rc, ws, ex = m.weight_quant_batch_matmul_get_workspace(self.t_x, self.t_w[0], self.t_sc, self.t_y, offset=self.t_off,
