@@ -205,13 +205,16 @@ __device__ __forceinline__ void async_copy16_uncounted(const void* g, void* lds)
 // Asynchronous copies global -> LDS with the address as a wave-uniform 64-bit base in scalar registers plus a 32-bit byte
 // offset per lane: the loop spends no vector instruction on addresses.  (Written out: hidden from the compiler's wait-count
 // pass, like async_copy16_uncounted; the kernel waits for its copies by count.)  lds: wave-uniform LDS byte address.
+// Five wait states stand between whatever precedes the statement and the load: the compiler inserts none for hazards it
+// cannot see inside the statement, and a base that a vector instruction (v_readfirstlane) has just written into scalar
+// registers needs that many before a memory instruction may read it.
 __device__ __forceinline__ void copy16_sbase(const void* base, uint32_t voff, uint32_t lds)
 {
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(lds), "v"(voff), "s"(base) : "memory", "m0");
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 4\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(lds), "v"(voff), "s"(base) : "memory", "m0");
 }
 __device__ __forceinline__ void copy4_sbase(const void* base, uint32_t voff, uint32_t lds)
 {
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2" : : "s"(lds), "v"(voff), "s"(base) : "memory", "m0");
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 4\n\tglobal_load_lds_dword %1, %2" : : "s"(lds), "v"(voff), "s"(base) : "memory", "m0");
 }
 
 // Workgroup ids are dealt round-robin over the 8 XCDs; give each XCD (own L2) a contiguous
