@@ -337,7 +337,8 @@ static bool stream_eligible(WqParams& p, WqStreamOpts& o)
     // (measured on 8192 x 28672 int4: 16 rows 43 us on the streaming kernel against 55 on this one, 32 rows 53 / 68,
     // 48 rows 69 / 70, 64 rows 82 / 70, 128 rows 105: hence the switch at 49 rows)
     constexpr int rows_min = 49;
-    o.rows = p.M >= rows_min && nch % 8 == 0 && p.N % 32 == 0 && p.N >= 256;
+    // (the kernel addresses the x rows of a slab, up to 256, with 32-bit byte offsets)
+    o.rows = p.M >= rows_min && nch % 8 == 0 && p.N % 32 == 0 && p.N >= 256 && p.K < (1ll << 23);
     return true;
 }
 
@@ -363,17 +364,17 @@ static int launch_slabs_float(WqParams p, hipStream_t st)
             if (rc != OPSNN_NOT_TAKEN) return rc;
         }
     }
-    // more rows: the many-rows streaming kernel, up to 128 rows per pass over the weights, in equal slabs
+    // more rows: the many-rows streaming kernel, up to 256 rows per pass over the weights
     {
         constexpr int64_t KC = 4 * (128 / WBITS);
         constexpr int rows_min = 17;
-        bool ok = !p.offset && p.M >= rows_min && p.K % KC == 0 && (p.K / KC) % 8 == 0 && p.N % 32 == 0 && p.N >= 256;
+        bool ok = !p.offset && p.M >= rows_min && p.K % KC == 0 && (p.K / KC) % 8 == 0 && p.N % 32 == 0 && p.N >= 256 && p.K < (1ll << 23);
         if (WBITS == 4) ok = ok && p.scale_e8m0 && p.group == 32 && p.s_rs == 1;
         else ok = ok && !p.scale_e8m0 && p.group >= p.K;
         if (ok) {
-            const int64_t passes = (p.M + 127) / 128;
-            const int64_t slab = ((p.M + passes - 1) / passes + 15) / 16 * 16;
-            p.cpg_shift = 31;
+            // up to 128 rows one pass; more: whole passes of 256 rows and the rest in one (as for integer codes below)
+            const int64_t slab = p.M <= 128 ? 128 : 256;
+            p.cpg_shift = WBITS == 4 ? 0 : 31;   // (e2m1: the kernel's scale table counts in words of four e8m0 bytes, one per 128 k chunk)
             for (int64_t m0 = 0; m0 < p.M; m0 += slab) {
                 p.m_base = m0;
                 p.m_rows = (p.M - m0) < slab ? (p.M - m0) : slab;

@@ -430,7 +430,7 @@ template <int XDT, int WBITS, int MB, int NB, int WN, int WK, bool HAS_OFF, int 
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void wqmm_rows_kernel(WqParams p)
 {
     static_assert(WN * WK == 8, "eight waves");
-    static_assert(!SLDS || WF == 0, "the scale table serves the integer forms");
+    static_assert(!SLDS || WF == 0 || WF == 2, "the scale table serves the integer forms and the e8m0 bytes of e2m1 codes");
     static_assert(WF == 0 || !HAS_OFF, "floating-point weight codes have no offset");
     static_assert(WF != 2 || WBITS == 4, "e8m0 group scales go with e2m1 codes");
     static_assert(WF != 3 || (WBITS == 8 && XDT == DT_F16 && WK == 2 && NB == 2), "the block-scale form: fp16 x, e4m3 w, a slab per 128-block");
@@ -453,10 +453,11 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void w
     constexpr int XPR = KX / 8 / XH;     // 16-byte pieces per x row per slab
     constexpr int XBUF = 16 * MB * XROW; // one slab buffer
     constexpr int XITEMS = 16 * MB * XPR / NT;
-    constexpr int NBL = (WF >= 3 || SLDS) ? NB : NB * (HAS_OFF ? 3 : 2);   // loads of one weight fetch
+    constexpr int NBL = (WF >= 3 || WF == 1 || SLDS) ? NB : NB * (HAS_OFF ? 3 : 2);   // loads of one weight fetch
     constexpr int LDS_MAIN = (2 * XBUF > WN * (WK - 1) * NB * MB * 4 * 64 * 4) ? 2 * XBUF : WN * (WK - 1) * NB * MB * 4 * 64 * 4;
     static_assert((16 * MB * XPR) % NT == 0 && XPR >= 16 && PF >= 2 && PPH >= 1 && STEPS == PPH * XH, "staging and prefetch shape");
-    static_assert(MB <= 8 || (WF == 0 && SLDS), "the 256-row instance is built for integer codes with the scale table in LDS");
+    static_assert(MB <= 8 || (WF == 0 && SLDS) || WF == 1 || WF == 2, "the 192- / 256-row instances: integer codes with the scale table in LDS, or floating-point codes");
+    static_assert(!(SLDS && WF == 2) || WK == 2, "byte position of a lane's e8m0 scale inside the table word");
     extern __shared__ __attribute__((aligned(16))) char sx[];
 
     const int tid = threadIdx.x, lane = tid & 63;
@@ -475,7 +476,8 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void w
     const uint16_t* srow = p.scale + (n0 + nrow) * p.s_cs;
     const uint16_t* orow = HAS_OFF ? p.offset + (n0 + nrow) * p.s_cs : nullptr;
     const int64_t sblk = 16 * p.s_cs;
-    const uint8_t* srow8 = (const uint8_t*)p.scale + (n0 + nrow) * p.s_cs + g;   // WF 2: the byte of this lane's group in chunk 0
+    // WF 2: the byte of this lane's group in chunk 0 (8-byte pieces: a lane's 16 weights are half a group, two lanes share a byte)
+    const uint8_t* srow8 = (const uint8_t*)p.scale + (n0 + nrow) * p.s_cs + (HP ? g >> 1 : g);
 
     // x copies: instruction `it` of this thread fills LDS piece it*NT + tid of the buffer, i.e. position
     // (it*NT + tid) % XPR of row (it*NT + tid) / XPR, with the row's piece position ^ (row % 16)
@@ -583,7 +585,9 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void w
             int64_t nb0 = ((int64_t)blockIdx.x * WN + rw / (16 * NB)) * (16 * NB);
             if (nb0 >= p.N) nb0 = p.N - 16 * NB;
             const int64_t n = nb0 + rw % (16 * NB);
-            uint32_t w = p.scale[n * p.s_cs + gi];
+            uint32_t w;
+            if constexpr (WF == 2) w = *(const uint32_t*)((const uint8_t*)p.scale + n * p.s_cs + 4 * gi);   // four e8m0 bytes: 128 k
+            else w = p.scale[n * p.s_cs + gi];
             if constexpr (HAS_OFF) w |= (uint32_t)p.offset[n * p.s_cs + gi] << 16;
             stab[rw * sG + (gi ^ (((rw & 15) << 2) & (sG - 1)))] = w;
         }
@@ -595,6 +599,15 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void w
         }
     }
 
+    // WF 1: one scale per channel, read once.  WF 2 with the table: a table word holds the e8m0 bytes of 128 k; this lane's
+    // 32 (8-byte pieces: 16) codes of a chunk belong to byte g of the chunk's word (g / 2 of the half that the chunk is)
+    uint16_t sch[NB];
+    const int e8sh = 8 * (HP ? 2 * wk + (g >> 1) : g);
+    (void)sch; (void)e8sh;
+    if constexpr (WF == 1) {
+#pragma unroll
+        for (int q = 0; q < NB; q++) sch[q] = srow[q * sblk];
+    }
     v4i wq[PF][NB];
     uint16_t sq[PF][NB], oq[PF][NB];
     auto fetch = [&](int j, int cw) {   // chunk cw of this wave (chunk cw * WK + wk of the row) into slot j
@@ -608,8 +621,8 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void w
                 wq[j][q] = *(const v4i*)(wptr + q * wblk + (int64_t)cw * (WK * 64));
             }
             if constexpr (SLDS) { sq[j][q] = 0; oq[j][q] = 0; continue; }
-            if constexpr (WF >= 3) sq[j][q] = 0;
-            else if constexpr (WF == 2) sq[j][q] = srow8[q * sblk + (cw * WK + wk) * 4];
+            if constexpr (WF >= 3 || WF == 1) sq[j][q] = 0;
+            else if constexpr (WF == 2) sq[j][q] = srow8[q * sblk + (cw * WK + wk) * (KC / 32)];
             else sq[j][q] = srow[q * sblk + so];
             if constexpr (HAS_OFF) oq[j][q] = orow[q * sblk + so];
             else oq[j][q] = 0;
@@ -621,7 +634,13 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void w
         if constexpr (SLDS) {
             const int gi = (cw * WK + wk) >> cpg_shift;
 #pragma unroll
-            for (int q = 0; q < NB; q++) sow[q] = stab[stab_row[q] + (gi ^ stab_sw[q])];
+            for (int q = 0; q < NB; q++) {
+                sow[q] = stab[stab_row[q] + (gi ^ stab_sw[q])];
+                if constexpr (WF == 2) sow[q] = bits_x<XDT>(e8m0_to_f32((sow[q] >> e8sh) & 0xFFu));
+            }
+        } else if constexpr (WF == 1) {
+#pragma unroll
+            for (int q = 0; q < NB; q++) sow[q] = sch[q];
         } else {
 #pragma unroll
             for (int q = 0; q < NB; q++) sow[q] = 0;
@@ -632,7 +651,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void w
         for (int q = 0; q < NB; q++) {
             if constexpr (WF == 0 && SLDS) out[q] = dequant8<XDT, WBITS, HAS_OFF, true>(wq[j][q], s, (uint16_t)sow[q], (uint16_t)(sow[q] >> 16), dqc);
             else if constexpr (WF == 0) out[q] = dequant8<XDT, WBITS, HAS_OFF, true>(wq[j][q], s, sq[j][q], oq[j][q], dqc);
-            else if constexpr (WF == 1) out[q] = dequant8_float<XDT, WBITS, true>(wq[j][q], s, sq[j][q]);
+            else if constexpr (WF == 1 || (WF == 2 && SLDS)) out[q] = dequant8_float<XDT, WBITS, true>(wq[j][q], s, (uint16_t)sow[q]);
             else if constexpr (WF == 4) {
                 typedef _Float16 h2v __attribute__((ext_vector_type(2)));
                 const uint32_t d0 = (uint32_t)wq[j][q][2 * s], d1 = (uint32_t)wq[j][q][2 * s + 1];
@@ -1414,15 +1433,17 @@ static int launch_rows_one(const WqParams& p, hipStream_t st)
     constexpr int XH = (MB > 8 && WBITS == 4) ? 2 : 1;   // as in the kernel: 8-byte weight pieces, i.e. slabs of half the K, for more than 128 rows of x with 4-bit weights
     constexpr size_t lds_x = 2 * (size_t)(16 * MB) * (WK * KC * 2 / XH);
     size_t lds_stab = 0;
-    if constexpr (WF == 0 && !SLDS) {
+    if constexpr ((WF == 0 || WF == 2) && !SLDS) {
         // the scales and offsets of the workgroup's columns in LDS when a row's scales are contiguous, their count per row
-        // is a power of two and the table fits beside the x buffers
+        // is a power of two and the table fits beside the x buffers (e2m1 codes: one word per 128 k, the four e8m0 bytes of
+        // a row read as a word; the caller passes cpg_shift 0)
         const int64_t G = p.cpg_shift >= 31 ? 1 : ((p.K / KC) >> p.cpg_shift);
         const size_t red = (size_t)WN * (WK - 1) * NB * MB * 4 * 64 * 4;
-        if ((p.s_rs == 1 || G == 1) && (G & (G - 1)) == 0 && (lds_x > red ? lds_x : red) + (size_t)(16 * NB * WN) * G * 4 <= 160 * 1024)
+        const bool rows_ok = WF == 2 ? (p.s_cs % 4 == 0 && (uintptr_t)p.scale % 4 == 0 && p.cpg_shift == 0) : (p.s_rs == 1 || G == 1);
+        if (rows_ok && (G & (G - 1)) == 0 && (lds_x > red ? lds_x : red) + (size_t)(16 * NB * WN) * G * 4 <= 160 * 1024)
             return launch_rows_one<XDT, WBITS, MB, NB, WN, WK, HAS_OFF, WF, true>(p, st);
     }
-    if constexpr (MB > 8 && !SLDS) return OPSNN_NOT_TAKEN;   // the 256-row instance exists with the scale table only
+    if constexpr (MB > 8 && WF == 0 && !SLDS) return OPSNN_NOT_TAKEN;   // integer codes: the 192- / 256-row instances exist with the scale table only
     else {
     if constexpr (SLDS) lds_stab = (size_t)(16 * NB * WN) * (p.cpg_shift >= 31 ? 1 : ((p.K / KC) >> p.cpg_shift)) * 4;
     constexpr size_t lds_red = (size_t)WN * (WK - 1) * NB * MB * 4 * 64 * 4;
@@ -1457,7 +1478,7 @@ int launch_wq_stream(const WqParams& p, const WqStreamOpts& o, hipStream_t st);
 // Up to 16 rows, floating-point weight codes (see launch_xreg_float); OPSNN_NOT_TAKEN if K does not split.
 template <int XDT, int WBITS>
 int launch_wq_xreg_float(const WqParams& p, hipStream_t st);
-// One row slab of up to 128 rows, floating-point weight codes, on the many-rows kernel (WBITS 4: mxfp4 with a row's
+// One row slab of up to 256 rows, floating-point weight codes, on the many-rows kernel (WBITS 4: mxfp4 with a row's
 // e8m0 bytes contiguous; 8: e4m3 with per-channel scales).  The caller has checked the kernel's shape conditions.
 template <int XDT, int WBITS>
 int launch_wq_rows_float(const WqParams& p, hipStream_t st);
@@ -1469,6 +1490,8 @@ int launch_wq_rows_float(const WqParams& p, hipStream_t st);
     int launch_wq_rows_float<XDT, WBITS>(const WqParams& p, hipStream_t st)                                         \
     {                                                                                                               \
         constexpr int WF = WBITS == 4 ? 2 : 1;                                                                      \
+        if (p.m_rows > 192) return launch_rows_one<XDT, WBITS, 16, 2, 4, 2, false, WF>(p, st);                      \
+        if (p.m_rows > 128) return launch_rows_one<XDT, WBITS, 12, 2, 4, 2, false, WF>(p, st);                      \
         return p.m_rows > 64 ? launch_rows_one<XDT, WBITS, 8, 2, 4, 2, false, WF>(p, st)                            \
                              : launch_rows_one<XDT, WBITS, 4, 2, 4, 2, false, WF>(p, st);                           \
     }                                                                                                               \

@@ -509,6 +509,18 @@ def test_weight_only_x_in_registers_kernel(gpu, M, K, N, x_dt, w_dt, group, tW, 
     (48, 512, 256, "bf16", "e4m3", 0, None),
     (96, 4096, 544, "f16", "e4m3", 0, "f16"),
     (130, 1536, 256, "bf16", "e4m3", 0, "bf16"),
+    # 129 rows and more: the 192- and 256-row instances (8-byte pieces of e2m1 codes: two lanes share an e8m0 byte), whole
+    # passes of 256 rows and the rest on the instance that fits it (44, 8 and 200 rows)
+    (129, 2048, 256, "bf16", "fp4", 32, None),
+    (192, 1024, 288, "f16", "fp4", 32, "f16"),
+    (193, 4096, 256, "f16", "fp4", 32, None),
+    (256, 8192, 512, "bf16", "fp4", 32, "bf16"),
+    (300, 1024, 256, "f16", "fp4", 32, None),
+    (712, 2048, 320, "bf16", "fp4", 32, None),
+    (160, 512, 256, "f16", "e4m3", 0, None),
+    (250, 4096, 544, "bf16", "e4m3", 0, "bf16"),
+    (256, 1024, 256, "f16", "e4m3", 0, "f16"),
+    (520, 1536, 288, "bf16", "e4m3", 0, None),
 ])
 def test_weight_only_float_codes_on_the_many_rows_kernel(gpu, M, K, N, x_dt, w_dt, group, bias):
     """17 rows of x and more against mxfp4 / e4m3 weights: the many-rows streaming kernel (two weight blocks per wave
