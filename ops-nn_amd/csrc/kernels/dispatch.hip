@@ -13,7 +13,7 @@ int launch_tc_plain(const OpsnnQmmArgs& a, hipStream_t st);
 int launch_group_plain(const OpsnnQmmArgs& a, bool tcg, hipStream_t st);
 int launch_wqmm_plain(const OpsnnWqmmArgs& a, hipStream_t st);
 // Return OPSNN_NOT_TAKEN when the arguments are outside what the fast kernels handle.
-int launch_blockscale_mfma(const OpsnnQmmArgs& a, hipStream_t st);
+int launch_blockscale_mfma(const OpsnnQmmArgs& a, hipStream_t st, SplitK sk = {});
 int launch_fp8_rowcol_mfma(const OpsnnQmmArgs& a, hipStream_t st, bool merged_scales_ok);
 int launch_rowcol_exact(const OpsnnQmmArgs& a, hipStream_t st, int ep_mode);   // qmm_fp8_exact.hip
 int launch_rowcol_decode(const OpsnnQmmArgs& a, hipStream_t st);   // qmm_fp8_decode.hip
@@ -24,7 +24,7 @@ int launch_tcg_mfma(const OpsnnQmmArgs& a, hipStream_t st);
 uint64_t tcg_workspace_bytes(const OpsnnQmmArgs& a);
 int launch_kg_mfma(const OpsnnQmmArgs& a, hipStream_t st);   // qmm_i4_kg.hip
 uint64_t kg_workspace_bytes(const OpsnnQmmArgs& a);
-int launch_mx_mfma(const OpsnnQmmArgs& a, hipStream_t st);
+int launch_mx_mfma(const OpsnnQmmArgs& a, hipStream_t st, SplitK sk = {});
 int launch_wqmm_mfma(const OpsnnWqmmArgs& a, hipStream_t st);
 uint64_t mx_workspace_bytes(const OpsnnQmmArgs& a);
 }  // namespace opsnn
@@ -173,24 +173,61 @@ extern "C" __attribute__((visibility("hidden"))) int opsnn_qmm_k_pad(const Opsnn
     return k_pad_prestep(*a, Kp, (hipStream_t)stream, *b);
 }
 
-extern "C" int opsnnQmmBlockScale(const OpsnnQmmArgs* a, void* stream)
+// The K split of a call that will run on the tile kernel of qmm_fp8_block.hip with few tiles (fp8 x fp4 MX from 33 rows,
+// int8 per-tile from 33 rows): 1 = none.  Looks only at what the caller passed (shapes, types), so that the workspace
+// query and the launch agree.
+static int splitk_for(const OpsnnQmmArgs& a, int mode)
+{
+    if (a.force_variant == OPSNN_VARIANT_PLAIN || opsnn_force_plain()) return 1;
+    if (a.out_dtype != DT_BF16 && a.out_dtype != DT_F16) return 1;
+    if (a.M <= 32 || a.M * a.N < 64 * 64 || a.K < 1024) return 1;   // (up to 32 rows the streaming kernels take these modes)
+    int64_t bm;
+    if (mode == 2 && a.x1_dtype == DT_E4M3 && a.x2_dtype == DT_E2M1) bm = 256;
+    else if (mode == 1 && a.x1_dtype == DT_I8 && a.x2_dtype == DT_I8 && a.gsK == 128 && a.gsN == 128) bm = a.M >= 512 ? 256 : 128;
+    else return 1;
+    const int64_t tiles = ((a.M + bm - 1) / bm) * ((a.N + 255) / 256) * a.batch;
+    return splitk_factor(tiles, (a.K + 127) / 128);
+}
+static uint64_t splitk_bytes(const OpsnnQmmArgs& a, int splits)
+{
+    return splits > 1 ? (uint64_t)round_up((int64_t)splits * a.batch * a.M * a.N * 4, 256) : 0;
+}
+static uint64_t qmm_workspace_base(const OpsnnQmmArgs* a, int mode);
+// Takes the partial sums' share off the front of the workspace: `c` is the call as the launchers below see it.
+static SplitK splitk_carve(const OpsnnQmmArgs& a, int mode, OpsnnQmmArgs& c)
+{
+    SplitK sk;
+    c = a;
+    const int s = splitk_for(a, mode);
+    if (s > 1 && a.workspace) {
+        sk.splits = s;
+        sk.part = (float*)a.workspace;
+        c.workspace = qmm_workspace_base(&a, mode) ? (char*)a.workspace + splitk_bytes(a, s) : nullptr;
+    }
+    return sk;
+}
+
+extern "C" int opsnnQmmBlockScale(const OpsnnQmmArgs* a0, void* stream)
 {
     WeightCacheScope cache_scope;
-    if (!qmm_args_ok(a) || !a->x1_scale_mat.ptr || !a->x2_scale_mat.ptr) return -1;
+    if (!qmm_args_ok(a0) || !a0->x1_scale_mat.ptr || !a0->x2_scale_mat.ptr) return -1;
+    const OpsnnQmmArgs* a = a0;
     if (a->force_variant != OPSNN_VARIANT_PLAIN && !opsnn_force_plain()) {
-        OpsnnQmmArgs b;
+        OpsnnQmmArgs b, c;
+        const SplitK sk = splitk_carve(*a0, 1, c);
+        a = &c;
         const int64_t Kp = k_pad_for(*a, 1);
         if (Kp) {
             int rc = k_pad_prestep(*a, Kp, (hipStream_t)stream, b);
-            if (rc == 0) rc = launch_blockscale_mfma(b, (hipStream_t)stream);
+            if (rc == 0) rc = launch_blockscale_mfma(b, (hipStream_t)stream, sk);
             if (rc != OPSNN_NOT_TAKEN) return rc;
         }
-        int rc = launch_blockscale_mfma(*a, (hipStream_t)stream);
+        int rc = launch_blockscale_mfma(*a, (hipStream_t)stream, sk);
         if (rc != OPSNN_NOT_TAKEN) return rc;
         if (a->force_variant != 0) return -4;
     }
-    NOTE_PLAIN("block-scale quant matmul", a);
-    return launch_blockscale_plain(*a, (hipStream_t)stream);
+    NOTE_PLAIN("block-scale quant matmul", a0);
+    return launch_blockscale_plain(*a0, (hipStream_t)stream);
 }
 
 extern "C" int opsnnQmmMx(const OpsnnQmmArgs* a, void* stream)
@@ -198,7 +235,9 @@ extern "C" int opsnnQmmMx(const OpsnnQmmArgs* a, void* stream)
     WeightCacheScope cache_scope;
     if (!qmm_args_ok(a) || !a->x1_scale_mat.ptr || !a->x2_scale_mat.ptr) return -1;
     if (a->force_variant != OPSNN_VARIANT_PLAIN && !opsnn_force_plain()) {
-        int rc = launch_mx_mfma(*a, (hipStream_t)stream);
+        OpsnnQmmArgs c;
+        const SplitK sk = splitk_carve(*a, 2, c);
+        int rc = launch_mx_mfma(c, (hipStream_t)stream, sk);
         if (rc != OPSNN_NOT_TAKEN) return rc;
         if (a->force_variant != 0) return -4;
     }
@@ -324,6 +363,11 @@ extern "C" int opsnnWqmm(const OpsnnWqmmArgs* a, void* stream)
 extern "C" uint64_t opsnnQmmWorkspace(const OpsnnQmmArgs* a, int mode)
 {
     if (!a) return 0;
+    return splitk_bytes(*a, splitk_for(*a, mode)) + qmm_workspace_base(a, mode);   // partial sums of a K split in front
+}
+
+static uint64_t qmm_workspace_base(const OpsnnQmmArgs* a, int mode)
+{
     if (const int64_t Kp = k_pad_for(*a, mode)) return k_pad_bytes(*a, Kp);
     if (mode == 2) return mx_workspace_bytes(*a);
     if (mode == 1 && a->x2.row_stride == 1 && a->force_variant != OPSNN_VARIANT_PLAIN && !opsnn_force_plain()) {

@@ -40,6 +40,24 @@ inline void device_flag_set(std::atomic<uint64_t>& mask)
 }  // namespace opsnn
 #endif
 namespace opsnn {
+// K split over workgroups for tile-kernel calls whose tiles would leave most of the chip idle (few rows against a narrow N):
+// `splits` workgroups per tile each take a contiguous range of K tiles and leave fp32 partial sums in `part`
+// ([splits][batch][M][N], at the front of the call's workspace); a second kernel adds them in split order, adds the bias
+// and rounds.  splits <= 1: one workgroup per tile, no partial sums.
+struct SplitK {
+    int splits = 1;
+    float* part = nullptr;
+};
+// How many ways a call with `tiles` output tiles and `ktiles` K tiles is split: enough to give every CU a workgroup,
+// at least four K tiles per workgroup, at most sixteen ways.
+inline int splitk_factor(int64_t tiles, int64_t ktiles)
+{
+    if (tiles <= 0 || tiles * 2 > 256) return 1;
+    int64_t s = 256 / tiles;
+    if (s > ktiles / 4) s = ktiles / 4;
+    if (s > 16) s = 16;
+    return s >= 2 ? (int)s : 1;
+}
 // Opened by every exported matmul entry point for the time it enqueues its launches (weight_cache.hip): copies that the
 // weight cache hands out inside the scope cannot be evicted before it closes; bypass = true switches the cache off for
 // this thread while the scope is open.  Scopes nest; the pins drop when the outermost one closes.

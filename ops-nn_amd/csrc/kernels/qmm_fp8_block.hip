@@ -50,6 +50,9 @@ struct Fp8BlkParams {
     const float* rs;
     const float* cs;
     int rs_stride, cs_stride;
+    // K split over `splits` workgroups per tile (SPLIT instantiations, grid.z): fp32 partial sums [splits][batch][M][N]
+    int splits;
+    float* part;
 #if QG_DBG
     unsigned long long* dbg;   // timing harness only (see qgemm_core.hip.h)
 #endif
@@ -72,9 +75,10 @@ __device__ __forceinline__ const int8_t* scalar_ptr(const int8_t* p)
 
 enum : int { FP8_BLOCK = 0, FP8_MX = 1, FP8_ROWCOL = 2, FP8_MX_W4 = 3, I8_BLOCK = 4 };
 
-template <int WGM, int STAGES, int OUT_DT, int MODE = FP8_BLOCK>
+template <int WGM, int STAGES, int OUT_DT, int MODE = FP8_BLOCK, bool SPLIT = false>
 __global__ __launch_bounds__(WGM * 128, 1) void qmm_fp8_block_kernel(Fp8BlkParams p, int tiles_m, int tiles_n)
 {
+    static_assert(!SPLIT || MODE != FP8_ROWCOL, "partial sums leave before the epilogue's scales: the modes whose sums carry their scales");
     constexpr bool W4 = MODE == FP8_MX_W4;     // MX with fp4 e2m1 x2 (fp8 x fp4): x2 rows are 64 bytes per K tile
     constexpr bool MX = MODE == FP8_MX || W4;  // e8m0 scales inside the instruction
     constexpr bool RC = MODE == FP8_ROWCOL;    // plain fp8 products, one scale per row and per column in the epilogue
@@ -111,7 +115,15 @@ __global__ __launch_bounds__(WGM * 128, 1) void qmm_fp8_block_kernel(Fp8BlkParam
     const int64_t lda = p.lda, ldb = p.ldb;
     const int8_t* A = p.a + bz * p.a_bs + m0 * lda;
     const int8_t* B = p.b + bz * p.b_bs + n0 * ldb;
-    const int KT = (int)(p.K / BK);
+    int KT = (int)(p.K / BK);
+    int kt_first = 0;   // SPLIT: this workgroup's K tiles are kt_first .. kt_first + KT - 1 (at least one: the launcher splits at most KT / 4 ways)
+    if constexpr (SPLIT) {
+        const int z = (int)blockIdx.z;
+        kt_first = (int)((int64_t)z * KT / p.splits);
+        KT = (int)((int64_t)(z + 1) * KT / p.splits) - kt_first;
+        A += (int64_t)kt_first * BK;
+        B += (int64_t)kt_first * BKB;
+    }
 
     const int crow = tid / CPR;
     const int cchunk = (tid % CPR) ^ ((crow / RPW) & (CPR - 1));
@@ -162,6 +174,8 @@ __global__ __launch_bounds__(WGM * 128, 1) void qmm_fp8_block_kernel(Fp8BlkParam
             sc_step = p.s2_rs;
         }
     }
+
+    if constexpr (SPLIT && !RC) sc_src += (int64_t)kt_first * sc_step;
 
     // copy instruction `idx` (0 .. CPT-1) of K tile kt: x1 rows, then x2 rows, then the scales
     // The tile's base addresses are pinned in scalar registers (which also hides them from loop-invariant code
@@ -379,6 +393,28 @@ __global__ __launch_bounds__(WGM * 128, 1) void qmm_fp8_block_kernel(Fp8BlkParam
     const unsigned long long dbg_t2 = wall_clock64();
     const unsigned long long dbg_c2 = clock64();
 #endif
+    if constexpr (SPLIT) {
+        // partial sums straight from the registers: a lane holds four consecutive columns of one row per fragment
+        float* part = p.part + (((int64_t)blockIdx.z * gridDim.y + bz) * p.M) * p.N;
+        const bool vec_ok4 = (p.N % 4) == 0 && ((uintptr_t)p.part % 16) == 0;
+#pragma unroll
+        for (int j = 0; j < FM; j++) {
+            const int64_t m = m0 + wm * TM + j * 16 + frow;
+#pragma unroll
+            for (int i = 0; i < FN; i++) {
+                const int64_t n = n0 + wn * TN + i * 16 + 4 * fq;
+                if (m >= p.M) continue;
+                if (vec_ok4 && n + 3 < p.N) {
+                    *(v4f*)(part + m * p.N + n) = acc[i][j];
+                } else {
+#pragma unroll
+                    for (int r = 0; r < 4; r++)
+                        if (n + r < p.N) part[m * p.N + n + r] = acc[i][j][r];
+                }
+            }
+        }
+        return;
+    }
     typedef v4us __attribute__((may_alias)) v4us_a;
     typedef v4i __attribute__((may_alias)) v4i_a;
     constexpr int EP_PITCH = TN * 2 + 16;
@@ -452,6 +488,20 @@ __global__ __launch_bounds__(WGM * 128, 1) void qmm_fp8_block_kernel(Fp8BlkParam
 #endif
 }
 
+// out[b, m, n] = rounded(sum over the splits, in split order, of part[s, b, m, n] + bias[b, n])
+template <int OUT_DT>
+__global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* part, int splits, int64_t total, int64_t MN, int64_t N,
+                                                            const void* bias, int bias_dt, int64_t bias_bs, uint16_t* out)
+{
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
+        float v = part[i];
+        for (int s = 1; s < splits; s++) v = v + part[(int64_t)s * total + i];
+        if (bias) v = v + load_scalar_as_f32(bias, bias_dt, (i / MN) * bias_bs + i % N);
+        out[i] = OUT_DT == DT_BF16 ? bf16_bits(v) : f16_bits(v);
+    }
+}
+
 template <int WGM, int STAGES, int OUT_DT, int MODE = FP8_BLOCK>
 static int launch_fp8_block(const Fp8BlkParams& p, int64_t batch, hipStream_t st)
 {
@@ -459,6 +509,27 @@ static int launch_fp8_block(const Fp8BlkParams& p, int64_t batch, hipStream_t st
     int tiles_m = (int)((p.M + BM - 1) / BM), tiles_n = (int)((p.N + 255) / 256);
     dim3 grid((unsigned)(tiles_m * tiles_n), (unsigned)batch);
     size_t lds = (size_t)STAGES * (BM * 128 + 256 * (MODE == FP8_MX_W4 ? 64 : 128) + WGM * 128 * 4);
+    if constexpr (MODE == FP8_MX_W4 || MODE == I8_BLOCK) {
+        if (p.splits > 1) {   // K split over workgroups, then the sum of the partial sums, the bias and the rounding
+            if (!p.part || p.splits > p.K / 128) return -1;
+            auto ks = qmm_fp8_block_kernel<WGM, STAGES, DT_F32, MODE, true>;
+            static std::atomic<uint64_t> attr_set_s{0};
+            if (!device_flag_test(attr_set_s)) {
+                hipError_t e = hipFuncSetAttribute((const void*)ks, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+                if (e != hipSuccess) return (int)e;
+                device_flag_set(attr_set_s);
+            }
+            grid.z = (unsigned)p.splits;
+            hipLaunchKernelGGL(ks, grid, dim3(WGM * 128), lds, st, p, tiles_m, tiles_n);
+            hipError_t e = hipGetLastError();
+            if (e != hipSuccess) return (int)e;
+            const int64_t total = batch * p.M * p.N;
+            const unsigned rgrid = (unsigned)((total + 256 * 4 - 1) / (256 * 4) < 2048 ? (total + 256 * 4 - 1) / (256 * 4) : 2048);
+            hipLaunchKernelGGL(splitk_reduce_kernel<OUT_DT>, dim3(rgrid ? rgrid : 1), dim3(256), 0, st, (const float*)p.part, p.splits, total,
+                               p.M * p.N, p.N, (const void*)p.bias, MODE == FP8_MX_W4 ? p.bias_dt : DT_F32, p.bias_bs, (uint16_t*)p.out);
+            return (int)hipGetLastError();
+        }
+    }
     auto k = qmm_fp8_block_kernel<WGM, STAGES, OUT_DT, MODE>;
     static std::atomic<uint64_t> attr_set{0};   // one bit per device: the attribute belongs to the (kernel, device) pair
     if (!device_flag_test(attr_set)) {
@@ -535,7 +606,7 @@ int launch_rowcol_exact(const OpsnnQmmArgs& a, hipStream_t st, int ep_mode);
 // K % 128 == 0, bias fp32 or 16-bit.
 int launch_mx_a8w4_decode(const OpsnnQmmArgs& a, hipStream_t st);   // qmm_fp8_decode.hip
 
-int launch_mx_a8w4_mfma(const OpsnnQmmArgs& a, hipStream_t st)
+int launch_mx_a8w4_mfma(const OpsnnQmmArgs& a, hipStream_t st, SplitK sk)
 {
     if (a.x1_dtype != DT_E4M3 || a.x2_dtype != DT_E2M1) return OPSNN_NOT_TAKEN;
     {   // up to 32 rows: the stream over x2 with x1 in registers
@@ -558,6 +629,7 @@ int launch_mx_a8w4_mfma(const OpsnnQmmArgs& a, hipStream_t st)
     if (a.x2.col_stride % 2) return OPSNN_NOT_TAKEN;
     if (((uintptr_t)p.a | (uintptr_t)p.b | (uint64_t)p.lda | (uint64_t)p.ldb | (uint64_t)p.a_bs | (uint64_t)p.b_bs) % 16) return OPSNN_NOT_TAKEN;
     if (((uintptr_t)p.sa | (uintptr_t)p.sb | (uint64_t)p.sa_rs | (uint64_t)p.sb_rs | (uint64_t)p.sa_bs | (uint64_t)p.sb_bs) % 4) return OPSNN_NOT_TAKEN;
+    p.splits = sk.splits; p.part = sk.part;
     if (a.out_dtype == DT_BF16) return launch_fp8_block<4, 2, DT_BF16, FP8_MX_W4>(p, a.batch, st);
     return launch_fp8_block<4, 2, DT_F16, FP8_MX_W4>(p, a.batch, st);
 }
@@ -629,7 +701,7 @@ int launch_fp8_rowcol_mfma(const OpsnnQmmArgs& a, hipStream_t st, bool merged_sc
 int launch_blockscale_decode(const OpsnnQmmArgs& a, hipStream_t st);   // qmm_fp8_decode.hip
 int launch_blockscale_rows(const OpsnnQmmArgs& a, hipStream_t st);     // qmm_fp8_rows.hip
 
-int launch_blockscale_mfma(const OpsnnQmmArgs& a0, hipStream_t st)
+int launch_blockscale_mfma(const OpsnnQmmArgs& a0, hipStream_t st, SplitK sk)
 {
     OpsnnQmmArgs a = a0;
     const bool i8 = a.x1_dtype == DT_I8 && a.x2_dtype == DT_I8;   // the per-tile mode of quant_batch_matmul_v4 (qbmmv4_kernel_golden.py:258-325)
@@ -680,6 +752,7 @@ int launch_blockscale_mfma(const OpsnnQmmArgs& a0, hipStream_t st)
     // 256 x 256 tiles (8 waves) halve the operand traffic per flop; 128 x 256 (4 waves) keeps small M efficient
     const bool big = a.M >= 512;
     if (i8) {
+        p.splits = sk.splits; p.part = sk.part;
         if (big) return a.out_dtype == DT_BF16 ? launch_fp8_block<4, 2, DT_BF16, I8_BLOCK>(p, a.batch, st) : launch_fp8_block<4, 2, DT_F16, I8_BLOCK>(p, a.batch, st);
         return a.out_dtype == DT_BF16 ? launch_fp8_block<2, 2, DT_BF16, I8_BLOCK>(p, a.batch, st) : launch_fp8_block<2, 2, DT_F16, I8_BLOCK>(p, a.batch, st);
     }

@@ -253,9 +253,9 @@ void* weight_cache_blob(const void* src, const void* src2, int64_t K, int64_t N,
 void weight_cache_commit(void* buffer, hipStream_t st);   // weight_cache.hip
 void weight_cache_abandon(void* buffer);
 int launch_mxfp8_mfma(const OpsnnQmmArgs& a, hipStream_t st);   // qmm_fp8_block.hip
-int launch_mx_a8w4_mfma(const OpsnnQmmArgs& a, hipStream_t st);   // qmm_fp8_block.hip
+int launch_mx_a8w4_mfma(const OpsnnQmmArgs& a, hipStream_t st, SplitK sk);   // qmm_fp8_block.hip
 
-int launch_mx_mfma(const OpsnnQmmArgs& a0, hipStream_t st)
+int launch_mx_mfma(const OpsnnQmmArgs& a0, hipStream_t st, SplitK sk)
 {
     if (!mx_call_ok(a0)) return OPSNN_NOT_TAKEN;
     OpsnnQmmArgs a = a0;
@@ -310,7 +310,7 @@ int launch_mx_mfma(const OpsnnQmmArgs& a0, hipStream_t st)
         const int rc = mx_pad_prestep(a, L, st);
         if (rc != 0) return rc;
     }
-    if (a.x1_dtype == DT_E4M3 && a.x2_dtype == DT_E2M1) return launch_mx_a8w4_mfma(a, st);   // fp8 x fp4: qmm_fp8_block.hip
+    if (a.x1_dtype == DT_E4M3 && a.x2_dtype == DT_E2M1) return launch_mx_a8w4_mfma(a, st, sk);   // fp8 x fp4: qmm_fp8_block.hip
     // MXFP8 runs on the block kernel of qmm_fp8_block.hip in MX mode (16x16x128 instructions, 64 x 128 per wave, the
     // pipeline tuned for the fp8 block-scale path); the 32x32x64 tile kernel stays available on request
     // (OPSNN_VARIANT_MX_FP8_MFMA) for comparison.  The 8-bit forms of the matrix instruction sum their products with a

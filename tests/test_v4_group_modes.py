@@ -141,7 +141,11 @@ def test_gpu_a8w4_mx(gpu, M, K, N, tB):
                                    # up to 32 rows: x1 in registers, x2 streamed once per 16 rows; K shared by 16 waves (2 or 4
                                    # chunks of 128 each) or by 8 (1 .. 7), ragged columns, two passes
                                    (16, 4096, 512), (9, 8192, 264), (24, 1024, 520), (1, 7168, 384), (32, 3072, 256),
-                                   (16, 2048, 256)])
+                                   (16, 2048, 256),
+                                   # few tiles against a long K: K split over 2 .. 16 workgroups per tile, fp32 partial sums in the
+                                   # workspace, summed in split order (also (512, 2048, 520), (100, 1024, 1000) and
+                                   # (1024, 4096, 1024) above); a column count that is no multiple of 4
+                                   (128, 4096, 4096), (40, 8192, 256), (77, 1024, 258), (200, 2048, 1000)])
 def test_gpu_a8w4_mx_on_the_matrix_cores(gpu, M, K, N):
     """fp8 x fp4 MX with K % 128 == 0 and enough outputs runs on the scaled matrix instruction with a 4-bit x2 operand.
     With a 4-bit operand the instruction's sums are as close to the fp32-accumulated ones as exact fp16 products are
@@ -247,7 +251,10 @@ def test_gpu_pertile_i8(gpu, M, K, N, tB):
 @pytest.mark.parametrize("M,K,N,tB", [(128, 256, 256, True), (300, 384, 260, True), (640, 1024, 520, False),
                                       # up to 32 rows: x1 in registers, x2 streamed once per 16 rows (int8 instructions)
                                       (16, 4096, 512, True), (9, 2048, 264, True), (24, 1024, 520, True), (16, 1024, 256, False),
-                                      (1, 7168, 384, True)])
+                                      (1, 7168, 384, True),
+                                      # few tiles against a long K: the K split ((640, 1024, 520) above: with the re-layout of
+                                      # an N-contiguous x2 behind the partial sums in the workspace)
+                                      (128, 4096, 4096, True), (40, 8192, 256, True), (96, 1024, 258, True), (200, 2048, 1000, False)])
 def test_gpu_pertile_i8_on_the_matrix_cores(gpu, M, K, N, tB):
     """int8 per-tile with K % 128 == 0 and enough outputs runs on the block-scale kernel with int8 instructions: the
     block sums are exact integers, the fold into the running sum is a fused multiply-add (one rounding where the oracle
