@@ -14,8 +14,8 @@ int launch_group_plain(const OpsnnQmmArgs& a, bool tcg, hipStream_t st);
 int launch_wqmm_plain(const OpsnnWqmmArgs& a, hipStream_t st);
 // Return OPSNN_NOT_TAKEN when the arguments are outside what the fast kernels handle.
 int launch_blockscale_mfma(const OpsnnQmmArgs& a, hipStream_t st, SplitK sk = {});
-int launch_fp8_rowcol_mfma(const OpsnnQmmArgs& a, hipStream_t st, bool merged_scales_ok);
-int launch_rowcol_exact(const OpsnnQmmArgs& a, hipStream_t st, int ep_mode);   // qmm_fp8_exact.hip
+int launch_fp8_rowcol_mfma(const OpsnnQmmArgs& a, hipStream_t st, bool merged_scales_ok, SplitK sk = {});
+int launch_rowcol_exact(const OpsnnQmmArgs& a, hipStream_t st, int ep_mode, SplitK sk = {});   // qmm_fp8_exact.hip
 int launch_rowcol_decode(const OpsnnQmmArgs& a, hipStream_t st);   // qmm_fp8_decode.hip
 uint64_t blockscale_rows_workspace(const OpsnnQmmArgs& a);         // qmm_fp8_rows.hip
 uint64_t rowcol_rows_workspace(const OpsnnQmmArgs& a);
@@ -173,19 +173,25 @@ extern "C" __attribute__((visibility("hidden"))) int opsnn_qmm_k_pad(const Opsnn
     return k_pad_prestep(*a, Kp, (hipStream_t)stream, *b);
 }
 
-// The K split of a call that will run on the tile kernel of qmm_fp8_block.hip with few tiles (fp8 x fp4 MX from 33 rows,
-// int8 per-tile from 33 rows): 1 = none.  Looks only at what the caller passed (shapes, types), so that the workspace
-// query and the launch agree.
+// The K split of a call that will run with few tiles on the tile kernel of qmm_fp8_block.hip (fp8 x fp4 MX and int8
+// per-tile from 33 rows) or on the exact fp8 kernel of qmm_fp8_exact.hip (fp8 block scales from 129 rows, MXFP8 from 33):
+// 1 = none.  Looks only at what the caller passed (shapes, types), so that the workspace query and the launch agree; a
+// route that ends on another kernel leaves the partial sums' share of the workspace unused.
 static int splitk_for(const OpsnnQmmArgs& a, int mode)
 {
     if (a.force_variant == OPSNN_VARIANT_PLAIN || opsnn_force_plain()) return 1;
-    if (a.out_dtype != DT_BF16 && a.out_dtype != DT_F16) return 1;
     if (a.M <= 32 || a.M * a.N < 64 * 64 || a.K < 1024) return 1;   // (up to 32 rows the streaming kernels take these modes)
-    int64_t bm;
-    if (mode == 2 && a.x1_dtype == DT_E4M3 && a.x2_dtype == DT_E2M1) bm = 256;
-    else if (mode == 1 && a.x1_dtype == DT_I8 && a.x2_dtype == DT_I8 && a.gsK == 128 && a.gsN == 128) bm = a.M >= 512 ? 256 : 128;
+    const bool out16 = a.out_dtype == DT_BF16 || a.out_dtype == DT_F16;
+    const bool f8 = a.x1_dtype == DT_E4M3 && a.x2_dtype == DT_E4M3;
+    int64_t bm, bn = 256;
+    if (mode == 2 && a.x1_dtype == DT_E4M3 && a.x2_dtype == DT_E2M1 && out16) bm = 256;
+    else if (mode == 1 && a.x1_dtype == DT_I8 && a.x2_dtype == DT_I8 && a.gsK == 128 && a.gsN == 128 && out16) bm = a.M >= 512 ? 256 : 128;
+    else if (mode == 1 && f8 && a.gsK == 128 && a.gsN == 128 && !a.bias && a.M > 128 && (out16 || a.out_dtype == DT_F32)) { bm = 256; bn = 128; }
+    else if (mode == 2 && f8 && (out16 || a.out_dtype == DT_F32)) { bm = 256; bn = 128; }
+    else if (mode == 3 && (a.x1_dtype == DT_E4M3 || a.x1_dtype == DT_E5M2) && (a.x2_dtype == DT_E4M3 || a.x2_dtype == DT_E5M2) && a.M > 128 &&
+             (out16 || a.out_dtype == DT_F32)) { bm = 256; bn = 128; }
     else return 1;
-    const int64_t tiles = ((a.M + bm - 1) / bm) * ((a.N + 255) / 256) * a.batch;
+    const int64_t tiles = ((a.M + bm - 1) / bm) * ((a.N + bn - 1) / bn) * a.batch;
     return splitk_factor(tiles, (a.K + 127) / 128);
 }
 static uint64_t splitk_bytes(const OpsnnQmmArgs& a, int splits)
@@ -260,6 +266,13 @@ extern "C" int opsnnQmmTc(const OpsnnQmmArgs* a, void* stream)
     if (a->x2_scale_len != 1 && a->x2_scale_len != a->N) return -2;
     if (a->x1_scale && ((a->x1_scale_len != 1 && a->x1_scale_len != a->M) || !f8)) return -2;
     if (a->out_dtype == DT_I8 || a->out_dtype == DT_I32) { if (!i8) return -2; }
+    // fp8 with few output tiles against a long K: the partial sums of a K split sit at the front of the workspace
+    OpsnnQmmArgs carved;
+    SplitK sk;
+    if (f8 && a->force_variant != OPSNN_VARIANT_PLAIN && !opsnn_force_plain()) {
+        sk = splitk_carve(*a, 3, carved);
+        a = &carved;
+    }
     OpsnnQmmArgs padded;
     if (const int64_t Kp = k_pad_for(*a, 3)) {   // K tail: continue on zero-padded K-contiguous copies
         const int rc = k_pad_prestep(*a, Kp, (hipStream_t)stream, padded);
@@ -301,14 +314,14 @@ extern "C" int opsnnQmmTc(const OpsnnQmmArgs* a, void* stream)
         }
         const bool e4 = a->x1_dtype == DT_E4M3 && a->x2_dtype == DT_E4M3;
         if (ep != 0 || !e4 || a->x2_scale_dtype != DT_F32 || a->out_dtype == DT_F32) {
-            const int rc = launch_rowcol_exact(*a, (hipStream_t)stream, ep);
+            const int rc = launch_rowcol_exact(*a, (hipStream_t)stream, ep, sk);
             if (rc != OPSNN_NOT_TAKEN) return rc;
         }
     }
     // fp8 e4m3 operands with a row scale and a column scale that are multiplied in separately (K-C, K-T, T-C with the
     // one-element x1Scale): matrix-core kernel when the layout allows, else the plain kernel
     if (f8 && a->x1_scale && a->force_variant != OPSNN_VARIANT_PLAIN && !opsnn_force_plain()) {
-        const int rc = launch_fp8_rowcol_mfma(*a, (hipStream_t)stream, false);
+        const int rc = launch_fp8_rowcol_mfma(*a, (hipStream_t)stream, false, sk);
         if (rc != OPSNN_NOT_TAKEN) return rc;
     }
     NOTE_PLAIN("per-tensor / per-channel quant matmul", a);

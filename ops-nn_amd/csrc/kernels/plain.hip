@@ -299,7 +299,7 @@ __global__ void qmm_i4_asym_plain(OpsnnQmmArgs a)
     out = __fmul_rn(out, ((const float*)a.x1_scale)[m]);
     store_f32_as(a.out, a.out_dtype, m * a.N + n, out);
 }
-int launch_fp8_rowcol_mfma(const OpsnnQmmArgs& a, hipStream_t st, bool merged_scales_ok);   // qmm_fp8_block.hip
+int launch_fp8_rowcol_mfma(const OpsnnQmmArgs& a, hipStream_t st, bool merged_scales_ok, SplitK sk = {});   // qmm_fp8_block.hip
 
 int launch_rowcol_rows(const OpsnnQmmArgs& a, hipStream_t st);      // qmm_fp8_rows.hip
 int launch_rowcol_decode(const OpsnnQmmArgs& a, hipStream_t st);    // qmm_fp8_decode.hip

@@ -598,8 +598,8 @@ int launch_mxfp8_mfma(const OpsnnQmmArgs& a, hipStream_t st)
 }
 
 int launch_f8_wide(const QgemmParams& p, int fn, int64_t batch, int out_dt, hipStream_t st);   // qmm_int8_wide.hip
-int launch_blockscale_exact(const OpsnnQmmArgs& a, hipStream_t st);   // qmm_fp8_exact.hip
-int launch_rowcol_exact(const OpsnnQmmArgs& a, hipStream_t st, int ep_mode);
+int launch_blockscale_exact(const OpsnnQmmArgs& a, hipStream_t st, SplitK sk = {});   // qmm_fp8_exact.hip
+int launch_rowcol_exact(const OpsnnQmmArgs& a, hipStream_t st, int ep_mode, SplitK sk = {});
 
 // fp8 e4m3 x fp4 e2m1 with e8m0 scales per 32 K on both operands (compute_mx of quant_batch_matmul_v4,
 // qbmmv4_kernel_golden.py:119-186): the MX mode with a 4-bit x2.  x2 [N, K] K-contiguous (two elements per byte),
@@ -638,7 +638,7 @@ int launch_mx_a8w4_mfma(const OpsnnQmmArgs& a, hipStream_t st, SplitK sk)
 // K-C, K-T and the double-scale modes whose two scales are multiplied in separately
 // (qbmmv3_kernel_golden.py:361-387 and :432-441).  out = (sum * x2Scale[n]) * x1Scale[m] + fp32 bias.
 // Needs K-contiguous operands with K % 128 == 0 and a 16-bit output; anything else stays on the plain kernel.
-int launch_fp8_rowcol_mfma(const OpsnnQmmArgs& a, hipStream_t st, bool merged_scales_ok)
+int launch_fp8_rowcol_mfma(const OpsnnQmmArgs& a, hipStream_t st, bool merged_scales_ok, SplitK sk)
 {
     if (a.x1_dtype != DT_E4M3 || a.x2_dtype != DT_E4M3) return OPSNN_NOT_TAKEN;
     if (a.out_dtype != DT_BF16 && a.out_dtype != DT_F16) return OPSNN_NOT_TAKEN;
@@ -650,7 +650,7 @@ int launch_fp8_rowcol_mfma(const OpsnnQmmArgs& a, hipStream_t st, bool merged_sc
     if (!merged_scales_ok && a.x1_scale_len == 1 && a.x2_scale_len == 1 && !a.bias) return OPSNN_NOT_TAKEN;
     if (a.K % 128 != 0 || a.M * a.N < 64 * 64 || a.x1.col_stride != 1 || a.x2.row_stride != 1) return OPSNN_NOT_TAKEN;
     if (!opsnnGetFp8Fast() || (a.bias && a.bias_dtype != DT_F32)) {   // exact products and sums unless the caller asked for the 8-bit matrix instruction (whose epilogue takes an fp32 bias only)
-        const int rc = launch_rowcol_exact(a, st, 0);
+        const int rc = launch_rowcol_exact(a, st, 0, sk);
         if (rc != OPSNN_NOT_TAKEN) return rc;
     }
     if (a.bias && a.bias_dtype != DT_F32) return OPSNN_NOT_TAKEN;
@@ -734,7 +734,7 @@ int launch_blockscale_mfma(const OpsnnQmmArgs& a0, hipStream_t st, SplitK sk)
         if (rc != OPSNN_NOT_TAKEN) return rc;
     }
     if (!i8 && (!opsnnGetFp8Fast() || out32)) {   // exact products and sums unless the caller asked for the 8-bit matrix instruction
-        const int rc = launch_blockscale_exact(a, st);
+        const int rc = launch_blockscale_exact(a, st, sk);
         if (rc != OPSNN_NOT_TAKEN || out32) return rc;
     }
     Fp8BlkParams p{};

@@ -62,6 +62,10 @@ struct Fp8xParams {
     const int* b_c;
     const int* gate;
     int gate_n;
+    // K split over `splits` workgroups per tile (SPLIT instantiations, grid.z): fp32 partial sums [splits][batch][M][N] --
+    // block scales already applied, row / column scales and bias not yet (fp8x_splitk_reduce_kernel applies them)
+    int splits;
+    float* part;
 #if QG_DBG
     unsigned long long* dbg;   // timing harness only: per wave, loop clocks / barrier-wait clocks / K tiles
 #endif
@@ -102,7 +106,27 @@ __device__ __forceinline__ v8h widen8_scaled(int d0, int d1, float sc)
 
 // FMT: bit 0 set = x1 holds e5m2 codes, bit 1 set = x2 does (else e4m3)
 // MXS: MX block scales (e8m0 per 32 K) folded into the widening conversion; row / column epilogue (RC) with the bases
-template <int OUT_DT, bool RC, int FMT = 0, bool MXS = false>
+// The epilogue of the row / column scale forms for one output (Fp8xParams::ep_mode); rs = the row's scale (1 if none)
+__device__ __forceinline__ float fp8x_rowcol_epilogue(const Fp8xParams& p, float v, float rs, int64_t bz, int64_t ni)
+{
+    const int64_t ci = bz * p.cs_bs + ni * p.cs_stride;
+    float csv;
+    if (p.cs_dt == DT_U64) csv = u2f((uint32_t)((const uint64_t*)p.cs)[ci] & 0xFFFFE000u);
+    else if (p.cs_dt == DT_BF16) csv = bf16_to_f32(((const uint16_t*)p.cs)[ci]);
+    else csv = ((const float*)p.cs)[ci];
+    if (p.ep_mode == 1) {
+        if (p.bias) v = v + load_scalar_as_f32(p.bias, p.bias_dt, bz * p.bias_bs + ni);
+        v = v * csv;
+    } else if (p.ep_mode == 2) {
+        v = v * u2f(f2u(csv * rs) & 0xFFFFE000u);
+    } else {
+        v = (v * csv) * rs;
+        if (p.bias) v = v + load_scalar_as_f32(p.bias, p.bias_dt, bz * p.bias_bs + ni);
+    }
+    return v;
+}
+
+template <int OUT_DT, bool RC, int FMT = 0, bool MXS = false, bool SPLIT = false>
 __global__ __launch_bounds__(512, 1) void qmm_fp8_exact_kernel(Fp8xParams p, int tiles_m, int tiles_n)
 {
     static_assert(!MXS || (RC && FMT == 0), "the MX mode is e4m3 x e4m3 with the row / column epilogue");
@@ -148,7 +172,15 @@ __global__ __launch_bounds__(512, 1) void qmm_fp8_exact_kernel(Fp8xParams p, int
     const int64_t lda = p.lda, ldb = p.ldb;
     const int8_t* A = p.a + bz * p.a_bs + m0 * lda;
     const int8_t* B = p.b + bz * p.b_bs + n0 * ldb;
-    const int KT = (int)(p.K / BK);
+    int KT = (int)(p.K / BK);
+    int kt_first = 0;   // SPLIT: this workgroup's K tiles are kt_first .. kt_first + KT - 1 (at least one)
+    if constexpr (SPLIT) {
+        const int z = (int)blockIdx.z;
+        kt_first = (int)((int64_t)z * KT / p.splits);
+        KT = (int)((int64_t)(z + 1) * KT / p.splits) - kt_first;
+        A += (int64_t)kt_first * BK;
+        B += (int64_t)kt_first * BK;
+    }
 
     // copies: instruction i of the workgroup fills tile rows i*64 .. i*64+63; this thread handles row i*64 + tid/8 and
     // the logical 16-byte chunk that belongs at position tid%8 of the swizzled row.  Rows past the matrix edge repeat
@@ -197,6 +229,7 @@ __global__ __launch_bounds__(512, 1) void qmm_fp8_exact_kernel(Fp8xParams p, int
             sc_step = p.s2_rs * 4;
         }
     }
+    if constexpr (SPLIT) sc_base += (int64_t)kt_first * sc_step;
     const uint32_t lds0 = (uint32_t)(uintptr_t)(const __attribute__((address_space(3))) void*)smem + (uint32_t)wave * 1024u;
     const uint32_t lds_sc0 = (uint32_t)(uintptr_t)(const __attribute__((address_space(3))) void*)smem + A_BYTES + B_BYTES + (uint32_t)wave * 256u;
     auto issue_piece = [&](int kt, int stage, int idx) {
@@ -448,6 +481,28 @@ __global__ __launch_bounds__(512, 1) void qmm_fp8_exact_kernel(Fp8xParams p, int
     wait_lgkmcnt0();   // the reads and copies past the last tile land before LDS is reused
     wait_vmcnt<0>();
 
+    if constexpr (SPLIT) {
+        // partial sums straight from the registers: a lane holds four consecutive columns of one row per fragment
+        float* part = p.part + (((int64_t)blockIdx.z * gridDim.y + bz) * p.M) * p.N;
+        const bool vec_ok4 = (p.N % 4) == 0 && ((uintptr_t)p.part % 16) == 0;
+#pragma unroll
+        for (int j = 0; j < FM; j++) {
+            const int64_t m = m0 + wm * TM + j * 16 + frow;
+#pragma unroll
+            for (int i = 0; i < FN; i++) {
+                const int64_t n = n0 + wn * TN + i * 16 + 4 * fq;
+                if (m >= p.M) continue;
+                if (vec_ok4 && n + 3 < p.N) {
+                    *(v4f*)(part + m * p.N + n) = acc[i][j];
+                } else {
+#pragma unroll
+                    for (int r = 0; r < 4; r++)
+                        if (n + r < p.N) part[m * p.N + n + r] = acc[i][j][r];
+                }
+            }
+        }
+        return;
+    }
     // Epilogue: acc[i][j][r] is out[m = m_base + 16j + lane%16][n = n_base + 16i + 4*(lane/16) + r].  Each wave parks one
     // 16 x 64 block in a private LDS patch and reads it back row-wise, so that a store instruction writes whole
     // 128-byte lines (16 bytes per lane, 8 lanes per row).
@@ -477,23 +532,7 @@ __global__ __launch_bounds__(512, 1) void qmm_fp8_exact_kernel(Fp8xParams p, int
             if constexpr (RC) {   // (sum * x2Scale[n]) * x1Scale[m] + bias[n], each operation rounded, as compute_pertoken orders them
                 const int64_t nb = n0 + wn * TN + i * 16 + 4 * fq;
 #pragma unroll
-                for (int r = 0; r < 4; r++) {
-                    const int64_t ni = nb + r < p.N ? nb + r : p.N - 1;
-                    const int64_t ci = bz * p.cs_bs + ni * p.cs_stride;
-                    float csv;
-                    if (p.cs_dt == DT_U64) csv = u2f((uint32_t)((const uint64_t*)p.cs)[ci] & 0xFFFFE000u);
-                    else if (p.cs_dt == DT_BF16) csv = bf16_to_f32(((const uint16_t*)p.cs)[ci]);
-                    else csv = ((const float*)p.cs)[ci];
-                    if (p.ep_mode == 1) {
-                        if (p.bias) v[r] = v[r] + load_scalar_as_f32(p.bias, p.bias_dt, bz * p.bias_bs + ni);
-                        v[r] = v[r] * csv;
-                    } else if (p.ep_mode == 2) {
-                        v[r] = v[r] * u2f(f2u(csv * rs_j[j]) & 0xFFFFE000u);
-                    } else {
-                        v[r] = (v[r] * csv) * rs_j[j];
-                        if (p.bias) v[r] = v[r] + load_scalar_as_f32(p.bias, p.bias_dt, bz * p.bias_bs + ni);
-                    }
-                }
+                for (int r = 0; r < 4; r++) v[r] = fp8x_rowcol_epilogue(p, v[r], rs_j[j], bz, nb + r < p.N ? nb + r : p.N - 1);
             }
             if constexpr (OUT_DT == DT_F32) {
                 // fp32 output: the lane's four neighbouring columns are 16 bytes, four lanes a 64-byte piece of a row: stored as they are
@@ -532,12 +571,54 @@ __global__ __launch_bounds__(512, 1) void qmm_fp8_exact_kernel(Fp8xParams p, int
     }
 }
 
+// out[b, m, n] = the sum over the splits, in split order, of part[s, b, m, n], then the row / column epilogue (RC) and
+// the rounding.  With gate flags (the MX mode) nothing is written when one is set: the launch that follows computes the call.
+template <int OUT_DT, bool RC>
+__global__ __launch_bounds__(256) void fp8x_splitk_reduce_kernel(Fp8xParams p, int64_t total)
+{
+    if (p.gate) {
+        int f = 0;
+        for (int i = 0; i < p.gate_n; i++) f |= p.gate[i];
+        if (f) return;
+    }
+    const int64_t MN = p.M * p.N, stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
+        float v = p.part[i];
+        for (int s = 1; s < p.splits; s++) v = v + p.part[(int64_t)s * total + i];
+        if constexpr (RC) {
+            const int64_t bz = i / MN, m = (i % MN) / p.N, n = i % p.N;
+            v = fp8x_rowcol_epilogue(p, v, p.rs ? p.rs[bz * p.rs_bs + m * p.rs_stride] : 1.0f, bz, n);
+        }
+        if constexpr (OUT_DT == DT_F32) ((float*)p.out)[i] = v;
+        else ((uint16_t*)p.out)[i] = OUT_DT == DT_BF16 ? bf16_bits(v) : f16_bits(v);
+    }
+}
+
 template <int OUT_DT, bool RC, int FMT = 0, bool MXS = false>
 static int launch_fp8_exact(const Fp8xParams& p, int64_t batch, hipStream_t st)
 {
     const int tiles_m = (int)((p.M + 255) / 256), tiles_n = (int)((p.N + 127) / 128);
     dim3 grid((unsigned)(tiles_m * tiles_n), (unsigned)batch);
     const size_t lds = 3 * (size_t)(256 * 128 + 128 * 128 + ((RC && !MXS) ? 0 : 512 * 4));
+    if (p.splits > 1) {   // K split over workgroups, then the sum of the partial sums, the epilogue and the rounding
+        if (!p.part || p.splits > p.K / 128) return -1;
+        auto ks = qmm_fp8_exact_kernel<DT_F32, RC, FMT, MXS, true>;
+        static std::atomic<uint64_t> attr_set_s{0};
+        if (!device_flag_test(attr_set_s)) {
+            hipError_t e = hipFuncSetAttribute((const void*)ks, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+            if (e != hipSuccess) return (int)e;
+            device_flag_set(attr_set_s);
+        }
+        grid.z = (unsigned)p.splits;
+        hipLaunchKernelGGL(ks, grid, dim3(512), lds, st, p, tiles_m, tiles_n);
+        hipError_t e = hipGetLastError();
+        if (e != hipSuccess) return (int)e;
+        const int64_t total = batch * p.M * p.N;
+        const int64_t want = (total + 256 * 4 - 1) / (256 * 4);
+        const unsigned rgrid = (unsigned)(want < 1 ? 1 : want > 2048 ? 2048 : want);
+        hipLaunchKernelGGL((fp8x_splitk_reduce_kernel<OUT_DT, RC>), dim3(rgrid), dim3(256), 0, st, p, total);
+        return (int)hipGetLastError();
+    }
     auto k = qmm_fp8_exact_kernel<OUT_DT, RC, FMT, MXS>;
     static std::atomic<uint64_t> attr_set{0};   // one bit per device: the attribute belongs to the (kernel, device) pair
     if (!device_flag_test(attr_set)) {
@@ -550,7 +631,7 @@ static int launch_fp8_exact(const Fp8xParams& p, int64_t batch, hipStream_t st)
 }
 
 // fp8 e4m3 block scales (G-B, B-B), K-contiguous operands, K % 128 == 0, 16-bit or fp32 output, no bias.
-int launch_blockscale_exact(const OpsnnQmmArgs& a, hipStream_t st)
+int launch_blockscale_exact(const OpsnnQmmArgs& a, hipStream_t st, SplitK sk)
 {
     if (a.x1_dtype != DT_E4M3 || a.x2_dtype != DT_E4M3) return OPSNN_NOT_TAKEN;
     if (a.out_dtype != DT_BF16 && a.out_dtype != DT_F16 && a.out_dtype != DT_F32) return OPSNN_NOT_TAKEN;
@@ -572,6 +653,7 @@ int launch_blockscale_exact(const OpsnnQmmArgs& a, hipStream_t st)
     // by 32-bit offsets from the tile's first row
     if (p.s1_rs < 0 || p.s1_cs < 0 || ((a.M + p.gsM - 1) / p.gsM) * p.s1_rs * 4 >= (1ll << 32)) return OPSNN_NOT_TAKEN;
     if (p.lda < 0 || p.ldb < 0 || 256 * p.lda >= (1ll << 32) || 128 * p.ldb >= (1ll << 32)) return OPSNN_NOT_TAKEN;
+    p.splits = sk.splits; p.part = sk.part;
     if (a.out_dtype == DT_BF16) return launch_fp8_exact<DT_BF16, false>(p, a.batch, st);
     if (a.out_dtype == DT_F32) return launch_fp8_exact<DT_F32, false>(p, a.batch, st);
     return launch_fp8_exact<DT_F16, false>(p, a.batch, st);
@@ -581,7 +663,7 @@ int launch_blockscale_exact(const OpsnnQmmArgs& a, hipStream_t st)
 // one, or none) and one per column of x2 (or one; fp32, bf16 or 64-bit words), optional fp32 bias.  ep_mode as in
 // Fp8xParams: 0 = (sum * cs) * rs + bias (compute_pertoken; compute_tc with a per-token scale), 1 = (sum + bias) * cs,
 // 2 = sum * trunc19(cs * rs).
-int launch_rowcol_exact(const OpsnnQmmArgs& a, hipStream_t st, int ep_mode)
+int launch_rowcol_exact(const OpsnnQmmArgs& a, hipStream_t st, int ep_mode, SplitK sk)
 {
     const bool e1 = a.x1_dtype == DT_E5M2, e2 = a.x2_dtype == DT_E5M2;
     if ((a.x1_dtype != DT_E4M3 && !e1) || (a.x2_dtype != DT_E4M3 && !e2)) return OPSNN_NOT_TAKEN;
@@ -599,6 +681,7 @@ int launch_rowcol_exact(const OpsnnQmmArgs& a, hipStream_t st, int ep_mode)
     p.ep_mode = ep_mode;
     p.bias = a.bias; p.bias_dt = a.bias_dtype; p.bias_bs = a.bias_batch_stride;
     if (((uintptr_t)p.a | (uintptr_t)p.b | (uint64_t)p.lda | (uint64_t)p.ldb | (uint64_t)p.a_bs | (uint64_t)p.b_bs) % 16) return OPSNN_NOT_TAKEN;
+    p.splits = sk.splits; p.part = sk.part;
     const bool bf = a.out_dtype == DT_BF16, f32 = a.out_dtype == DT_F32;
     switch ((e1 ? 1 : 0) | (e2 ? 2 : 0)) {
         case 0: return f32 ? launch_fp8_exact<DT_F32, true, 0>(p, a.batch, st) : bf ? launch_fp8_exact<DT_BF16, true, 0>(p, a.batch, st) : launch_fp8_exact<DT_F16, true, 0>(p, a.batch, st);
@@ -664,7 +747,7 @@ uint64_t mx_exact_bytes(const OpsnnQmmArgs& a)
 // MXFP8 with exact products: the bases pass, this kernel, and -- computing
 // only when a flag is set -- the tile kernel on the scaled 8-bit instruction.  `a`: both operands e4m3, K-contiguous,
 // K % 128 == 0, scale rows K-contiguous; `region`: mx_exact_bytes(a) bytes.  OPSNN_NOT_TAKEN before anything is launched.
-int launch_mx_exact(const OpsnnQmmArgs& a, void* region, hipStream_t st)
+int launch_mx_exact(const OpsnnQmmArgs& a, void* region, hipStream_t st, SplitK sk)
 {
     if (!region || (uintptr_t)region % 16) return OPSNN_NOT_TAKEN;
     if (a.x1_dtype != DT_E4M3 || a.x2_dtype != DT_E4M3) return OPSNN_NOT_TAKEN;
@@ -698,6 +781,7 @@ int launch_mx_exact(const OpsnnQmmArgs& a, void* region, hipStream_t st)
     p.ep_mode = 0;
     p.bias = a.bias; p.bias_dt = a.bias_dtype; p.bias_bs = a.bias_batch_stride;
     p.gate = flags; p.gate_n = g1 + g2;
+    p.splits = sk.splits; p.part = sk.part;
     const int rc = a.out_dtype == DT_F32    ? launch_fp8_exact<DT_F32, true, 0, true>(p, a.batch, st)
                    : a.out_dtype == DT_BF16 ? launch_fp8_exact<DT_BF16, true, 0, true>(p, a.batch, st)
                                             : launch_fp8_exact<DT_F16, true, 0, true>(p, a.batch, st);

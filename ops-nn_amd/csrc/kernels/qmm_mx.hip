@@ -146,7 +146,7 @@ static int mx_pad_prestep(OpsnnQmmArgs& a, const MxPad& L, hipStream_t st)
 }
 
 uint64_t mx_exact_bytes(const OpsnnQmmArgs& a);           // qmm_fp8_exact.hip
-int launch_mx_exact(const OpsnnQmmArgs& a, void* region, hipStream_t st);
+int launch_mx_exact(const OpsnnQmmArgs& a, void* region, hipStream_t st, SplitK sk);
 
 // ---- x2 stored [K, N] with N contiguous (data dense, scales [K/64, N, 2]) ----
 // The kernels stream K-contiguous operands: data and scales are first re-laid out, per batch, at 256-byte aligned pitches.
@@ -331,7 +331,7 @@ int launch_mx_mfma(const OpsnnQmmArgs& a0, hipStream_t st, SplitK sk)
     if (((uintptr_t)g.a | (uintptr_t)g.b | (uint64_t)g.lda | (uint64_t)g.ldb | (uint64_t)g.a_bs | (uint64_t)g.b_bs) % 16) return OPSNN_NOT_TAKEN;
     if (((uintptr_t)g.sa | (uintptr_t)g.sb | (uint64_t)g.sa_rs | (uint64_t)g.sb_rs | (uint64_t)g.sa_bs | (uint64_t)g.sb_bs) % 4) return OPSNN_NOT_TAKEN;
     if (fp8 && exact) {
-        const int rc = launch_mx_exact(a, mxx, st);
+        const int rc = launch_mx_exact(a, mxx, st, sk);
         if (rc != OPSNN_NOT_TAKEN) return rc;
     }
     const bool small = a.M <= 128 || a.N <= 128;

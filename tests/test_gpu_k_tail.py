@@ -74,6 +74,19 @@ def test_fp8_blockscale_k_tail(gpu, M, K, N, tB, gsM, fast):
     m.lib().aclDestroyAclOpExecutor(ex)
 
 
+def _splitk_bytes(M, K, N, bm, bn, batch=1):
+    """The fp32 partial sums that phase 1 puts in front of the workspace when a call of a mode that can split K (fp8 block
+    scales from 129 rows, MXFP8, fp8 x fp4 MX and int8 per-tile from 33 rows; K >= 1024) has tiles for at most half of the
+    256 CUs: 2 .. 16 splits, at least four K tiles each."""
+    if M <= 32 or M * N < 64 * 64 or K < 1024:
+        return 0
+    tiles = -(-M // bm) * -(-N // bn) * batch
+    if tiles * 2 > 256:
+        return 0
+    s = min(256 // tiles, -(-K // 128) // 4, 16)
+    return -(-(s * batch * M * N * 4) // 256) * 256 if s >= 2 else 0
+
+
 def _mx_pad_bytes(M, K, N, fp4, batch=1):
     Kp, epb = -(-K // 128) * 128, 2 if fp4 else 1
     up = lambda v: -(-v // 256) * 256
@@ -119,7 +132,7 @@ def test_mx_k_tail(gpu, M, K, N, fp4, batch, bias):
     s1 = m.Tensor(bs + inp["s1"].shape[1:], m.ACL_FLOAT8_E8M0, d["s1"]); s2 = m.Tensor(bs + inp["s2"].shape[1:], m.ACL_FLOAT8_E8M0, d["s2"])
     o = m.Tensor(bs + (M, N), m.ACL_BF16, m.DeviceBuffer(batch * M * N * 2))
     rc, ws, ex = m.quant_matmul_v5_get_workspace(x1, x2, s1, s2, o, transpose_x2=True, group_size=(1 << 32) | (1 << 16) | 32)
-    plan = _mx_pad_bytes(M, K, N, fp4, batch) + (0 if fp4 else _mx_exact_bytes(M, K, N, batch))
+    plan = _mx_pad_bytes(M, K, N, fp4, batch) + (0 if fp4 else _mx_exact_bytes(M, K, N, batch) + _splitk_bytes(M, K, N, 256, 128, batch))
     assert rc == 0 and ws == plan, (rc, ws, plan)
     m.lib().aclDestroyAclOpExecutor(ex)
 
@@ -152,7 +165,7 @@ def test_mx_k_tail_n_contiguous_x2(gpu, M, K, N, fp4, batch):
     rc, ws, ex = m.quant_matmul_v5_get_workspace(x1, x2, s1, s2, o, transpose_x2=False, group_size=(1 << 32) | (1 << 16) | 32)
     up = lambda v: -(-v // 256) * 256
     relaid = up(batch * up(N * K // (2 if fp4 else 1)) + batch * up(N * -(-K // 64) * 2))
-    plan = relaid + _mx_pad_bytes(M, K, N, fp4, batch) + (0 if fp4 else _mx_exact_bytes(M, K, N, batch))
+    plan = relaid + _mx_pad_bytes(M, K, N, fp4, batch) + (0 if fp4 else _mx_exact_bytes(M, K, N, batch) + _splitk_bytes(M, K, N, 256, 128, batch))
     assert rc == 0 and ws == plan, (rc, ws, plan)
     m.lib().aclDestroyAclOpExecutor(ex)
 
@@ -176,7 +189,7 @@ def test_mx_fp8_fp4_k_tail(gpu, M, K, N):
     bias = m.Tensor((1, N), m.ACL_FLOAT16, d["bias"])
     o = m.Tensor((M, N), m.ACL_FLOAT16, m.DeviceBuffer(M * N * 2))
     rc, ws, ex = m.quant_matmul_v5_get_workspace(x1, x2, s1, s2, o, bias=bias, transpose_x2=True, group_size=32)
-    assert rc == 0 and ws == up(M * Kp) + up(N * Kp // 2) + up(M * (Kp // 64) * 2) + up(N * (Kp // 64) * 2), (rc, ws)
+    assert rc == 0 and ws == up(M * Kp) + up(N * Kp // 2) + up(M * (Kp // 64) * 2) + up(N * (Kp // 64) * 2) + _splitk_bytes(M, K, N, 256, 256), (rc, ws)
     m.lib().aclDestroyAclOpExecutor(ex)
     m.lib().opsnnSetForcePlain(1)
     try:

@@ -75,6 +75,9 @@ def _reset_env(opsnn):
     (130, 256, 130, False, 128), (1, 1024, 256, True, 1),
     (512, 1024, 768, True, 1), (300, 512, 520, True, 1), (384, 2048, 512, False, 1), (256, 1024, 256, True, 128),
     (700, 384, 520, True, 1), (640, 256, 264, False, 128),     # ragged edges in both directions, several row tiles
+    # few tiles against a long K (also (512, 1024, 768), (384, 2048, 512) and (256, 1024, 256) above): K split over 2 .. 16
+    # workgroups per tile on the exact path, partial sums in the workspace
+    (300, 4096, 1000, True, 1), (256, 7168, 2048, True, 128), (200, 8192, 130, False, 1),
 ])
 def test_fp8_blockscale(gpu, M, K, N, tB, gsM, path):
     """plain: one thread per output, bit-identical.  exact (the default): e4m3 widened to fp16, exact products, the bar
