@@ -33,6 +33,27 @@ __device__ __forceinline__ uint16_t bf16_bits(float f)
     u += 0x7fffu + ((u >> 16) & 1u);
     return (uint16_t)(u >> 16);
 }
+// Element i of the sum, in split order, of `splits` partial arrays of `total` elements each (the K split of the tile
+// kernels); four loads in flight at a time.
+template <typename T>
+__device__ __forceinline__ T splitk_sum(const T* part, int splits, int64_t total, int64_t i)
+{
+    T v = part[i];
+    int s = 1;
+    for (; s + 3 < splits; s += 4) {
+        const T a = part[(int64_t)s * total + i], b = part[(int64_t)(s + 1) * total + i];
+        const T c = part[(int64_t)(s + 2) * total + i], d = part[(int64_t)(s + 3) * total + i];
+        v = v + a; v = v + b; v = v + c; v = v + d;
+    }
+    for (; s < splits; s++) v = v + part[(int64_t)s * total + i];
+    return v;
+}
+// Blocks of 256 threads for a grid-stride loop with one element per thread and pass.
+inline unsigned splitk_reduce_grid(int64_t total)
+{
+    const int64_t want = (total + 255) / 256;
+    return (unsigned)(want < 1 ? 1 : want > (1 << 20) ? (1 << 20) : want);
+}
 __device__ __forceinline__ float bf16_to_f32(uint16_t h) { return u2f((uint32_t)h << 16); }
 __device__ __forceinline__ uint16_t f16_bits(float f)
 {

@@ -179,12 +179,21 @@ extern "C" __attribute__((visibility("hidden"))) int opsnn_qmm_k_pad(const Opsnn
 // route that ends on another kernel leaves the partial sums' share of the workspace unused.
 static int splitk_for(const OpsnnQmmArgs& a, int mode)
 {
-    if (a.force_variant == OPSNN_VARIANT_PLAIN || opsnn_force_plain()) return 1;
-    if (a.M <= 32 || a.M * a.N < 64 * 64 || a.K < 1024) return 1;   // (up to 32 rows the streaming kernels take these modes)
+    if (a.force_variant != 0 || opsnn_force_plain()) return 1;   // (a pinned kernel variant runs as it is)
+    if (a.M * a.N < 64 * 64 || a.K < 1024) return 1;
     const bool out16 = a.out_dtype == DT_BF16 || a.out_dtype == DT_F16;
     const bool f8 = a.x1_dtype == DT_E4M3 && a.x2_dtype == DT_E4M3;
-    int64_t bm, bn = 256;
-    if (mode == 2 && a.x1_dtype == DT_E4M3 && a.x2_dtype == DT_E2M1 && out16) bm = 256;
+    int64_t bm, bn = 256, max_tiles = 128;
+    // int8 with per-token / per-channel scales on 128 x 128 tiles (the selector's choice below 256 x 256 x 64 outputs; whole K
+    // tiles): integer partial sums, so the result stays bit-identical
+    if ((mode == 0 || (mode == 3 && !a.x1_scale)) && a.x1_dtype == DT_I8 && a.x2_dtype == DT_I8 && out16 && a.K % 128 == 0 &&
+        (a.M <= 128 || a.N <= 128 || a.M * a.N < 256 * 256 * 64) && a.M * a.N * a.batch <= 256 * 1024) {
+        // (a 128 x 128 int8 tile is quick, and the partial sums cost their own traffic: measured at 4096 x 4096, 64 rows,
+        // 32 tiles, 20 -> 15 us; 128 rows, 32 tiles, 19.5 -> 22; 256 rows, 64 tiles, 21 -> 24)
+        bm = 128; bn = 128; max_tiles = 32;
+    }
+    else if (a.M <= 32) return 1;   // (up to 32 rows the streaming kernels take the modes below)
+    else if (mode == 2 && a.x1_dtype == DT_E4M3 && a.x2_dtype == DT_E2M1 && out16) bm = 256;
     else if (mode == 1 && a.x1_dtype == DT_I8 && a.x2_dtype == DT_I8 && a.gsK == 128 && a.gsN == 128 && out16) bm = a.M >= 512 ? 256 : 128;
     else if (mode == 1 && f8 && a.gsK == 128 && a.gsN == 128 && !a.bias && a.M > 128 && (out16 || a.out_dtype == DT_F32)) { bm = 256; bn = 128; }
     else if (mode == 2 && f8 && (out16 || a.out_dtype == DT_F32)) { bm = 256; bn = 128; }
@@ -192,7 +201,7 @@ static int splitk_for(const OpsnnQmmArgs& a, int mode)
              (out16 || a.out_dtype == DT_F32)) { bm = 256; bn = 128; }
     else return 1;
     const int64_t tiles = ((a.M + bm - 1) / bm) * ((a.N + bn - 1) / bn) * a.batch;
-    return splitk_factor(tiles, (a.K + 127) / 128);
+    return splitk_factor(tiles, (a.K + 127) / 128, max_tiles);
 }
 static uint64_t splitk_bytes(const OpsnnQmmArgs& a, int splits)
 {
@@ -211,6 +220,12 @@ static SplitK splitk_carve(const OpsnnQmmArgs& a, int mode, OpsnnQmmArgs& c)
         c.workspace = qmm_workspace_base(&a, mode) ? (char*)a.workspace + splitk_bytes(a, s) : nullptr;
     }
     return sk;
+}
+
+// For the launchers of other files: the call with the partial sums' share taken off the front of its workspace.
+extern "C" __attribute__((visibility("hidden"))) void opsnn_qmm_splitk_carve(const OpsnnQmmArgs* a, int mode, OpsnnQmmArgs* c, SplitK* sk)
+{
+    *sk = splitk_carve(*a, mode, *c);
 }
 
 extern "C" int opsnnQmmBlockScale(const OpsnnQmmArgs* a0, void* stream)
@@ -377,6 +392,11 @@ extern "C" uint64_t opsnnQmmWorkspace(const OpsnnQmmArgs* a, int mode)
 {
     if (!a) return 0;
     return splitk_bytes(*a, splitk_for(*a, mode)) + qmm_workspace_base(a, mode);   // partial sums of a K split in front
+}
+
+extern "C" __attribute__((visibility("hidden"))) uint64_t opsnn_qmm_workspace_base(const OpsnnQmmArgs* a, int mode)
+{
+    return a ? qmm_workspace_base(a, mode) : 0;
 }
 
 static uint64_t qmm_workspace_base(const OpsnnQmmArgs* a, int mode)

@@ -48,11 +48,11 @@ struct SplitK {
     int splits = 1;
     float* part = nullptr;
 };
-// How many ways a call with `tiles` output tiles and `ktiles` K tiles is split: enough to give every CU a workgroup,
-// at least four K tiles per workgroup, at most sixteen ways.
-inline int splitk_factor(int64_t tiles, int64_t ktiles)
+// How many ways a call with `tiles` output tiles (at most max_tiles, else it is not split) and `ktiles` K tiles is split:
+// enough to give every CU a workgroup, at least four K tiles per workgroup, at most sixteen ways.
+inline int splitk_factor(int64_t tiles, int64_t ktiles, int64_t max_tiles = 128)
 {
-    if (tiles <= 0 || tiles * 2 > 256) return 1;
+    if (tiles <= 0 || tiles > max_tiles) return 1;
     int64_t s = 256 / tiles;
     if (s > ktiles / 4) s = ktiles / 4;
     if (s > 16) s = 16;

@@ -60,6 +60,10 @@ struct QgemmParams {
     // exact MX route, whose kernel then left the call to this one); otherwise every workgroup returns at once.
     const int* gate;
     int gate_n;
+    // MODE_I8, K split over `splits` workgroups per tile (SPLIT instantiations, grid.z): int32 partial sums
+    // [splits][batch][M][N]; qg_i8_splitk_reduce_kernel adds them (exactly: integers) and applies the epilogue
+    int splits;
+    int32_t* part;
 #if QG_DBG
     unsigned long long* dbg;
 #endif
@@ -83,9 +87,10 @@ __device__ __forceinline__ void async_copy4(const void* g, void* lds)
                                      (__attribute__((address_space(3))) void*)lds, 4, 0, 0);
 }
 
-template <int MODE, int BM, int BN, int BK, int WGM, int WGN, int STAGES, int MINWG, bool KTAIL, int OUT_DT>
+template <int MODE, int BM, int BN, int BK, int WGM, int WGN, int STAGES, int MINWG, bool KTAIL, int OUT_DT, bool SPLIT = false>
 __global__ __launch_bounds__(WGM* WGN * 64, MINWG) void qgemm_kernel(QgemmParams p, int tiles_m, int tiles_n)
 {
+    static_assert(!SPLIT || (MODE == MODE_I8 && !KTAIL), "the K split: int8 operands, whole K tiles");
     constexpr bool MX = MODE != MODE_I8;
     constexpr int NT = WGM * WGN * 64;
     constexpr int CPR = BK / 16;                 // 16-byte chunks per LDS row
@@ -152,7 +157,14 @@ __global__ __launch_bounds__(WGM* WGN * 64, MINWG) void qgemm_kernel(QgemmParams
     const int8_t* A = p.a + bz * p.a_bs + m0 * lda;
     const int8_t* B = p.b + bz * p.b_bs + n0 * ldb;
     const int64_t K = p.KB;
-    const int KT = (int)((K + BK - 1) / BK);
+    int KT = (int)((K + BK - 1) / BK);
+    if constexpr (SPLIT) {   // this workgroup's K tiles: kt_first .. kt_first + KT - 1 (at least STAGES: the launcher splits at most KT / 4 ways)
+        const int z = (int)blockIdx.z;
+        const int kt_first = (int)((int64_t)z * KT / p.splits);
+        KT = (int)((int64_t)(z + 1) * KT / p.splits) - kt_first;
+        A += (int64_t)kt_first * BK;
+        B += (int64_t)kt_first * BK;
+    }
 
     // LDS layout of one operand tile: row r holds CPR chunks of 16 bytes; logical chunk c is stored at position
     // c ^ key(r), key(r) = (r / RPW) % CPR, so that 16 consecutive rows at one logical chunk hit 16 different
@@ -447,6 +459,32 @@ __global__ __launch_bounds__(WGM* WGN * 64, MINWG) void qgemm_kernel(QgemmParams
     }
     for (; kt + 1 < KT; kt++) k_tile(kt, F{}, T{}, F{});
     k_tile(kt, F{}, F{}, F{});
+    if constexpr (SPLIT) {
+        // partial sums straight from the registers (acc[i][j][r]: n = n_base + 8*(r/4) + 4*(lane/32) + r%4, m = m_base + lane%32)
+        int32_t* part = p.part + (((int64_t)blockIdx.z * gridDim.y + bz) * p.M) * p.N;
+        const bool vec_ok4 = (p.N % 4) == 0 && ((uintptr_t)p.part % 16) == 0;
+#pragma unroll
+        for (int j = 0; j < FM; j++) {
+            const int64_t m = m0 + wm * TM + j * 32 + (lane & 31);
+#pragma unroll
+            for (int i = 0; i < FN; i++) {
+#pragma unroll
+                for (int q = 0; q < 4; q++) {
+                    const int64_t n = n0 + wn * TN + i * 32 + 8 * q + 4 * (lane >> 5);
+                    if (m >= p.M) continue;
+                    const v4i o = {acc[i][j][q * 4], acc[i][j][q * 4 + 1], acc[i][j][q * 4 + 2], acc[i][j][q * 4 + 3]};
+                    if (vec_ok4 && n + 3 < p.N) {
+                        *(v4i*)(part + m * p.N + n) = o;
+                    } else {
+#pragma unroll
+                        for (int e = 0; e < 4; e++)
+                            if (n + e < p.N) part[m * p.N + n + e] = o[e];
+                    }
+                }
+            }
+        }
+        return;
+    }
     __syncthreads();  // all operand reads done before LDS is reused below
 #if QG_DBG
     const unsigned long long dbg_t2 = wall_clock64();
@@ -664,6 +702,56 @@ __global__ __launch_bounds__(WGM* WGN * 64, MINWG) void qgemm_kernel(QgemmParams
         }
     }
 #endif
+}
+
+// MODE_I8 after a K split: out[b, m, n] = rounded(fp32(sum of the partial sums + ib[n]) * x2s[n] * x1s[m] + fb[n]), the
+// terms as the tile kernel's epilogue stages them
+template <int OUT_DT>
+__global__ __launch_bounds__(256) void qg_i8_splitk_reduce_kernel(QgemmParams p, int64_t total)
+{
+    const int64_t MN = p.M * p.N, stride = (int64_t)gridDim.x * blockDim.x;
+    const bool has_ib = p.bias && p.bias_dt == DT_I32, has_fb = p.bias && p.bias_dt != DT_I32;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
+        const int32_t a = splitk_sum(p.part, p.splits, total, i);
+        const int64_t bz = i / MN, m = (i % MN) / p.N, n = i % p.N;
+        const int64_t si = p.x2s_len == 1 ? 0 : n;
+        float sv = p.x2s_dt == DT_U64 ? u2f((uint32_t)((const uint64_t*)p.x2s)[si]) : load_scalar_as_f32(p.x2s, p.x2s_dt, si);
+        if (p.x2s_trunc || p.x2s_dt == DT_U64) sv = u2f(f2u(sv) & 0xFFFFE000u);
+        const int32_t ib = has_ib ? ((const int32_t*)p.bias)[bz * p.bias_bs + n] : 0;
+        const float fb = has_fb ? load_scalar_as_f32(p.bias, p.bias_dt, bz * p.bias_bs + n) : -0.0f;
+        const float s1 = p.x1s ? p.x1s[m] : 1.0f;
+        float tv = (float)(a + ib);
+        tv = tv * sv;
+        tv = tv * s1;
+        const float v = tv + fb;
+        ((uint16_t*)p.out)[(bz * p.M + m) * p.ldc + n] = OUT_DT == DT_BF16 ? bf16_bits(v) : f16_bits(v);
+    }
+}
+
+// The K split of MODE_I8 (p.splits > 1, K a multiple of BK): the tile kernel per split, then the reduction.
+template <int BM, int BN, int BK, int WGM, int WGN, int STAGES, int MINWG>
+static int qgemm_launch_split_i8(const QgemmParams& p, int64_t batch, int out_dt, hipStream_t st)
+{
+    if (!p.part || p.splits < 2 || (p.KB % BK) != 0 || p.splits > p.KB / BK / 2) return -1;
+    if (out_dt != DT_BF16 && out_dt != DT_F16) return -2;
+    int tiles_m = (int)((p.M + BM - 1) / BM), tiles_n = (int)((p.N + BN - 1) / BN);
+    dim3 grid((unsigned)(tiles_m * tiles_n), (unsigned)batch, (unsigned)p.splits);
+    const size_t lds = (size_t)STAGES * (BM + BN) * BK;
+    auto k = qgemm_kernel<MODE_I8, BM, BN, BK, WGM, WGN, STAGES, MINWG, false, DT_I32, true>;
+    static std::atomic<uint64_t> attr_set{0};
+    if (!device_flag_test(attr_set)) {
+        hipError_t e = hipFuncSetAttribute((const void*)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return (int)e;
+        device_flag_set(attr_set);
+    }
+    hipLaunchKernelGGL(k, grid, dim3(WGM * WGN * 64), lds, st, p, tiles_m, tiles_n);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return (int)e;
+    const int64_t total = batch * p.M * p.N;
+    const unsigned rgrid = splitk_reduce_grid(total);
+    if (out_dt == DT_BF16) hipLaunchKernelGGL(qg_i8_splitk_reduce_kernel<DT_BF16>, dim3(rgrid), dim3(256), 0, st, p, total);
+    else hipLaunchKernelGGL(qg_i8_splitk_reduce_kernel<DT_F16>, dim3(rgrid), dim3(256), 0, st, p, total);
+    return (int)hipGetLastError();
 }
 
 template <int MODE, int BM, int BN, int BK, int WGM, int WGN, int STAGES, int MINWG, bool KTAIL, int OUT_DT>

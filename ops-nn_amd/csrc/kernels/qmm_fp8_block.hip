@@ -495,8 +495,7 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* part, i
 {
     const int64_t stride = (int64_t)gridDim.x * blockDim.x;
     for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
-        float v = part[i];
-        for (int s = 1; s < splits; s++) v = v + part[(int64_t)s * total + i];
+        float v = splitk_sum(part, splits, total, i);
         if (bias) v = v + load_scalar_as_f32(bias, bias_dt, (i / MN) * bias_bs + i % N);
         out[i] = OUT_DT == DT_BF16 ? bf16_bits(v) : f16_bits(v);
     }
@@ -524,8 +523,8 @@ static int launch_fp8_block(const Fp8BlkParams& p, int64_t batch, hipStream_t st
             hipError_t e = hipGetLastError();
             if (e != hipSuccess) return (int)e;
             const int64_t total = batch * p.M * p.N;
-            const unsigned rgrid = (unsigned)((total + 256 * 4 - 1) / (256 * 4) < 2048 ? (total + 256 * 4 - 1) / (256 * 4) : 2048);
-            hipLaunchKernelGGL(splitk_reduce_kernel<OUT_DT>, dim3(rgrid ? rgrid : 1), dim3(256), 0, st, (const float*)p.part, p.splits, total,
+            const unsigned rgrid = splitk_reduce_grid(total);
+            hipLaunchKernelGGL(splitk_reduce_kernel<OUT_DT>, dim3(rgrid), dim3(256), 0, st, (const float*)p.part, p.splits, total,
                                p.M * p.N, p.N, (const void*)p.bias, MODE == FP8_MX_W4 ? p.bias_dt : DT_F32, p.bias_bs, (uint16_t*)p.out);
             return (int)hipGetLastError();
         }

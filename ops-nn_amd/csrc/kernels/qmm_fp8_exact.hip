@@ -583,8 +583,7 @@ __global__ __launch_bounds__(256) void fp8x_splitk_reduce_kernel(Fp8xParams p, i
     }
     const int64_t MN = p.M * p.N, stride = (int64_t)gridDim.x * blockDim.x;
     for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
-        float v = p.part[i];
-        for (int s = 1; s < p.splits; s++) v = v + p.part[(int64_t)s * total + i];
+        float v = splitk_sum(p.part, p.splits, total, i);
         if constexpr (RC) {
             const int64_t bz = i / MN, m = (i % MN) / p.N, n = i % p.N;
             v = fp8x_rowcol_epilogue(p, v, p.rs ? p.rs[bz * p.rs_bs + m * p.rs_stride] : 1.0f, bz, n);
@@ -614,8 +613,7 @@ static int launch_fp8_exact(const Fp8xParams& p, int64_t batch, hipStream_t st)
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) return (int)e;
         const int64_t total = batch * p.M * p.N;
-        const int64_t want = (total + 256 * 4 - 1) / (256 * 4);
-        const unsigned rgrid = (unsigned)(want < 1 ? 1 : want > 2048 ? 2048 : want);
+        const unsigned rgrid = splitk_reduce_grid(total);
         hipLaunchKernelGGL((fp8x_splitk_reduce_kernel<OUT_DT, RC>), dim3(rgrid), dim3(256), 0, st, p, total);
         return (int)hipGetLastError();
     }

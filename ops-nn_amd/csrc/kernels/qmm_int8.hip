@@ -93,19 +93,39 @@ static int64_t cu_count()
 // OPSNN_NOT_TAKEN: an INT8 output was asked for and the shape does not fit the MFMA kernels (the caller falls back).
 extern "C" __attribute__((visibility("hidden"))) int opsnn_qmm_int8_impl(const OpsnnQmmArgs* a, void* stream);
 extern "C" __attribute__((visibility("hidden"))) int opsnn_qmm_k_pad(const OpsnnQmmArgs* a, int mode, void* stream, OpsnnQmmArgs* b);   // dispatch.hip
+extern "C" __attribute__((visibility("hidden"))) void opsnn_qmm_splitk_carve(const OpsnnQmmArgs* a, int mode, OpsnnQmmArgs* c, SplitK* sk);   // dispatch.hip
+static int qmm_int8_impl(const OpsnnQmmArgs* a, void* stream, SplitK sk);
 extern "C" int opsnnQmmInt8(const OpsnnQmmArgs* a, void* stream)
 {
     WeightCacheScope cache_scope;
-    OpsnnQmmArgs padded;
+    OpsnnQmmArgs padded, carved;
+    SplitK sk;
     if (a && a->x1.ptr && a->x2.ptr && a->M > 0 && a->N > 0 && a->K > 0 && a->batch > 0) {
+        opsnn_qmm_splitk_carve(a, 0, &carved, &sk);   // few tiles against a long K: the partial sums of a K split come first in the workspace
+        a = &carved;
         const int prc = opsnn_qmm_k_pad(a, 0, stream, &padded);   // K % 16 != 0: zero-padded K-contiguous copies
         if (prc == 0) a = &padded;
         else if (prc != OPSNN_NOT_TAKEN) return prc;
     }
-    const int rc = opsnn_qmm_int8_impl(a, stream);
+    const int rc = qmm_int8_impl(a, stream, sk);
     return rc == OPSNN_NOT_TAKEN ? -2 : rc;
 }
-extern "C" int opsnn_qmm_int8_impl(const OpsnnQmmArgs* a, void* stream)
+extern "C" int opsnn_qmm_int8_impl(const OpsnnQmmArgs* a, void* stream) { return qmm_int8_impl(a, stream, SplitK{}); }
+// opsnnQmmInt8 without the K split: the workspace is opsnn_qmm_workspace_base(a, 0) bytes (for the entry point whose
+// workspace is a fixed array)
+extern "C" __attribute__((visibility("hidden"))) int opsnn_qmm_int8_nosplit(const OpsnnQmmArgs* a, void* stream)
+{
+    WeightCacheScope cache_scope;
+    OpsnnQmmArgs padded;
+    if (a && a->x1.ptr && a->x2.ptr && a->M > 0 && a->N > 0 && a->K > 0 && a->batch > 0) {
+        const int prc = opsnn_qmm_k_pad(a, 0, stream, &padded);
+        if (prc == 0) a = &padded;
+        else if (prc != OPSNN_NOT_TAKEN) return prc;
+    }
+    const int rc = qmm_int8_impl(a, stream, SplitK{});
+    return rc == OPSNN_NOT_TAKEN ? -2 : rc;
+}
+static int qmm_int8_impl(const OpsnnQmmArgs* a, void* stream, SplitK sk)
 {
     if (!a || !a->x1.ptr || !a->x2.ptr || !a->out || !a->x2_scale) return -1;
     if (a->x1_dtype != DT_I8 || a->x2_dtype != DT_I8) return -2;
@@ -184,7 +204,13 @@ extern "C" int opsnn_qmm_int8_impl(const OpsnnQmmArgs* a, void* stream)
             case OPSNN_VARIANT_I8_256_W8_K128: return qgemm_launch<MODE_I8, 256, 256, 128, 2, 4, 2, 1>(g, a->batch, p.out_dt, st);
             default: break;
         }
-        if (p.M <= 128 || p.N <= 128 || p.M * p.N < 256 * 256 * 64) return qgemm_launch<MODE_I8, 128, 128, 128, 2, 2, 2, 1>(g, a->batch, p.out_dt, st);
+        if (p.M <= 128 || p.N <= 128 || p.M * p.N < 256 * 256 * 64) {
+            if (sk.splits > 1 && p.K % 128 == 0) {   // few tiles against a long K: K split over workgroups, integer partial sums
+                g.splits = sk.splits; g.part = (int32_t*)sk.part;
+                return qgemm_launch_split_i8<128, 128, 128, 2, 2, 2, 1>(g, a->batch, p.out_dt, st);
+            }
+            return qgemm_launch<MODE_I8, 128, 128, 128, 2, 2, 2, 1>(g, a->batch, p.out_dt, st);
+        }
         // Large shapes: 256x256 tiles, one per CU at a time, are the most economical in operand traffic, but only
         // whole rounds of them keep every CU busy.  Columns that fill whole rounds go to that kernel; the remaining
         // columns (less than one round) go to 128x128 tiles, two workgroups per CU, in a second launch.

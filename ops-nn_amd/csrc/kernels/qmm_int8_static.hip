@@ -40,10 +40,14 @@ int scratch_address(void** out)
 }
 }  // namespace
 
+extern "C" __attribute__((visibility("hidden"))) uint64_t opsnn_qmm_workspace_base(const OpsnnQmmArgs* a, int mode);   // dispatch.hip
+extern "C" __attribute__((visibility("hidden"))) int opsnn_qmm_int8_nosplit(const OpsnnQmmArgs* a, void* stream);       // qmm_int8.hip
+
 extern "C" int opsnnQmmInt8Static(const OpsnnQmmArgs* a, void* stream)
 {
     if (!a) return -1;
-    const uint64_t need = opsnnQmmWorkspace(a, 0);
+    // (the workspace of opsnnQmmInt8 without the partial sums of a K split: this entry point runs every call unsplit)
+    const uint64_t need = opsnn_qmm_workspace_base(a, 0);
     if (need > (uint64_t)OPSNN_STATIC_SCRATCH_BYTES) {
         opsnn::set_error("opsnnQmmInt8Static: the re-laid-out x2 needs %llu bytes, the built-in scratch array holds %llu; "
                          "pass x2 K-contiguous or use opsnnQmmInt8 with a workspace",
@@ -62,5 +66,5 @@ extern "C" int opsnnQmmInt8Static(const OpsnnQmmArgs* a, void* stream)
         }
         b.workspace = ptr;   // written in full by the re-layout before the matmul reads it: nothing to clear
     }
-    return opsnnQmmInt8(&b, stream);
+    return opsnn_qmm_int8_nosplit(&b, stream);
 }

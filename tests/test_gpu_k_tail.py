@@ -76,12 +76,14 @@ def test_fp8_blockscale_k_tail(gpu, M, K, N, tB, gsM, fast):
 
 def _splitk_bytes(M, K, N, bm, bn, batch=1):
     """The fp32 partial sums that phase 1 puts in front of the workspace when a call of a mode that can split K (fp8 block
-    scales from 129 rows, MXFP8, fp8 x fp4 MX and int8 per-tile from 33 rows; K >= 1024) has tiles for at most half of the
-    256 CUs: 2 .. 16 splits, at least four K tiles each."""
-    if M <= 32 or M * N < 64 * 64 or K < 1024:
+    scales from 129 rows, MXFP8, fp8 x fp4 MX and int8 per-tile from 33 rows, int8 per-token / per-channel on 128 x 128
+    tiles; K >= 1024) has at most 128 tiles (int8 per-token / per-channel: 32): 2 .. 16 splits, at least four K tiles each."""
+    if (M <= 32 and bm != 128) or M * N < 64 * 64 or K < 1024:
         return 0
     tiles = -(-M // bm) * -(-N // bn) * batch
-    if tiles * 2 > 256:
+    if bm == bn == 128 and (tiles > 32 or M * N * batch > 256 * 1024):   # the int8 per-token / per-channel kernel's tiles
+        return 0
+    if tiles > 128:
         return 0
     s = min(256 // tiles, -(-K // 128) // 4, 16)
     return -(-(s * batch * M * N * 4) // 256) * 256 if s >= 2 else 0

@@ -11,6 +11,7 @@ import numpy as np
 import pytest
 
 import cases
+from test_gpu_k_tail import _splitk_bytes
 
 pytestmark = pytest.mark.gpu
 
@@ -23,7 +24,9 @@ def _run_pair(m, M, K, N, seed):
     out_st.fill(0xEE)
     a = cases.qmm_args_int8(m, d, M, K, N, 1, False, out_ws.ptr, m.ACL_BF16, m.ACL_FLOAT, N, m.ACL_BF16)
     need = m.lib().opsnnQmmWorkspace(C.byref(a), 0)
-    assert need == N * K, need   # the fast path applies: the re-laid-out operand is the scratch buffer in question
+    # the fast path applies: the re-laid-out operand is the scratch buffer in question; opsnnQmmInt8 also gets room for the
+    # integer partial sums of a K split when the call has few tiles (the no-alloc entry point runs unsplit: same bits)
+    assert need == N * K + _splitk_bytes(M, K, N, 128, 128), need
     ws = m.DeviceBuffer(need)
     a.workspace = ws.ptr
     assert m.lib().opsnnQmmInt8(C.byref(a), None) == 0
