@@ -183,25 +183,34 @@ static int splitk_for(const OpsnnQmmArgs& a, int mode)
     if (a.M * a.N < 64 * 64 || a.K < 1024) return 1;
     const bool out16 = a.out_dtype == DT_BF16 || a.out_dtype == DT_F16;
     const bool f8 = a.x1_dtype == DT_E4M3 && a.x2_dtype == DT_E4M3;
-    int64_t bm, bn = 256, max_tiles = 128;
+    int64_t bm, bn = 256, kunit = 128;
+    double tile_us;   // one K tile (kunit elements) of the kernel in question, measured on calls with few tiles
+    double bytes_per_us = 5.0e6;   // what its partial sums' traffic was measured to cost (splitk_factor)
     // int8 with per-token / per-channel scales on 128 x 128 tiles (the selector's choice below 256 x 256 x 64 outputs; whole K
     // tiles): integer partial sums, so the result stays bit-identical
     if ((mode == 0 || (mode == 3 && !a.x1_scale)) && a.x1_dtype == DT_I8 && a.x2_dtype == DT_I8 && out16 && a.K % 128 == 0 &&
-        (a.M <= 128 || a.N <= 128 || a.M * a.N < 256 * 256 * 64) && a.M * a.N * a.batch <= 256 * 1024) {
-        // (a 128 x 128 int8 tile is quick, and the partial sums cost their own traffic: measured at 4096 x 4096, 64 rows,
-        // 32 tiles, 20 -> 15 us; 128 rows, 32 tiles, 19.5 -> 22; 256 rows, 64 tiles, 21 -> 24)
-        bm = 128; bn = 128; max_tiles = 32;
+        (a.M <= 128 || a.N <= 128 || a.M * a.N < 256 * 256 * 64)) {
+        // (a 128 x 128 int8 tile is quick, and the partial sums cost their own traffic: measured at 4096 x 4096 in eight
+        // splits, 64 rows 20 -> 15 us, 128 rows 19.5 -> 22, 256 rows in four 21 -> 24)
+        bm = 128; bn = 128; tile_us = 0.55; bytes_per_us = 2.4e6;
+    }
+    // MXFP4: 128 x 128 tiles when 256 x 256 ones would be few (the launcher's rule), K tiles counted in 256 elements
+    else if (mode == 2 && a.x1_dtype == DT_E2M1 && a.x2_dtype == DT_E2M1 && (out16 || a.out_dtype == DT_F32)) {
+        const int64_t t256 = ((a.M + 255) / 256) * ((a.N + 255) / 256) * a.batch;
+        bm = bn = (a.M <= 128 || a.N <= 128 || t256 <= 32) ? 128 : 256;
+        kunit = 256;
+        tile_us = bm == 128 ? 0.6 : 1.3; bytes_per_us = 2.4e6;
     }
     else if (a.M <= 32) return 1;   // (up to 32 rows the streaming kernels take the modes below)
-    else if (mode == 2 && a.x1_dtype == DT_E4M3 && a.x2_dtype == DT_E2M1 && out16) bm = 256;
-    else if (mode == 1 && a.x1_dtype == DT_I8 && a.x2_dtype == DT_I8 && a.gsK == 128 && a.gsN == 128 && out16) bm = a.M >= 512 ? 256 : 128;
-    else if (mode == 1 && f8 && a.gsK == 128 && a.gsN == 128 && !a.bias && a.M > 128 && (out16 || a.out_dtype == DT_F32)) { bm = 256; bn = 128; }
-    else if (mode == 2 && f8 && (out16 || a.out_dtype == DT_F32)) { bm = 256; bn = 128; }
+    else if (mode == 2 && a.x1_dtype == DT_E4M3 && a.x2_dtype == DT_E2M1 && out16) { bm = 256; tile_us = 1.8; }
+    else if (mode == 1 && a.x1_dtype == DT_I8 && a.x2_dtype == DT_I8 && a.gsK == 128 && a.gsN == 128 && out16) { bm = a.M >= 512 ? 256 : 128; tile_us = 1.8; }
+    else if (mode == 1 && f8 && a.gsK == 128 && a.gsN == 128 && !a.bias && a.M > 128 && (out16 || a.out_dtype == DT_F32)) { bm = 256; bn = 128; tile_us = 1.4; }
+    else if (mode == 2 && f8 && (out16 || a.out_dtype == DT_F32)) { bm = 256; bn = 128; tile_us = 1.4; }
     else if (mode == 3 && (a.x1_dtype == DT_E4M3 || a.x1_dtype == DT_E5M2) && (a.x2_dtype == DT_E4M3 || a.x2_dtype == DT_E5M2) && a.M > 128 &&
-             (out16 || a.out_dtype == DT_F32)) { bm = 256; bn = 128; }
+             (out16 || a.out_dtype == DT_F32)) { bm = 256; bn = 128; tile_us = 1.4; }
     else return 1;
     const int64_t tiles = ((a.M + bm - 1) / bm) * ((a.N + bn - 1) / bn) * a.batch;
-    return splitk_factor(tiles, (a.K + 127) / 128, max_tiles);
+    return splitk_factor(tiles, (a.K + kunit - 1) / kunit, tile_us, a.M * a.N * a.batch, bytes_per_us);
 }
 static uint64_t splitk_bytes(const OpsnnQmmArgs& a, int splits)
 {

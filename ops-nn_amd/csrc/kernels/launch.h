@@ -48,15 +48,25 @@ struct SplitK {
     int splits = 1;
     float* part = nullptr;
 };
-// How many ways a call with `tiles` output tiles (at most max_tiles, else it is not split) and `ktiles` K tiles is split:
-// enough to give every CU a workgroup, at least four K tiles per workgroup, at most sixteen ways.
-inline int splitk_factor(int64_t tiles, int64_t ktiles, int64_t max_tiles = 128)
+// How many ways a call with `tiles` output tiles, `ktiles` K tiles of `tile_us` microseconds each and `out_elems` outputs
+// is split: at most one workgroup per CU, at least four K tiles per workgroup, at most sixteen ways -- and among those the
+// count with the largest estimated gain, if that is at least 3 us: the loop time saved, ktiles * tile_us * (1 - 1/s), less
+// a second launch (4 us) and the partial sums written and read back (2 s out_elems 4 bytes at `bytes_per_us`: fitted to
+// measurements, 5e6 for the kernels that store 64-byte row pieces from 16 x 16 fragments, 2.4e6 for the 32 x 32-fragment
+// kernel's 32-byte pieces).  (Measured without the traffic term: MXFP4 1024 x 4096 x 4096 in four splits 28 -> 65 us.)
+inline int splitk_factor(int64_t tiles, int64_t ktiles, double tile_us, int64_t out_elems, double bytes_per_us)
 {
-    if (tiles <= 0 || tiles > max_tiles) return 1;
-    int64_t s = 256 / tiles;
-    if (s > ktiles / 4) s = ktiles / 4;
-    if (s > 16) s = 16;
-    return s >= 2 ? (int)s : 1;
+    if (tiles <= 0 || tiles > 128) return 1;
+    int64_t smax = 256 / tiles;
+    if (smax > ktiles / 4) smax = ktiles / 4;
+    if (smax > 16) smax = 16;
+    int best = 1;
+    double best_gain = 3.0;
+    for (int64_t s = 2; s <= smax; s++) {
+        const double gain = (double)ktiles * tile_us * (1.0 - 1.0 / (double)s) - 4.0 - 2.0 * (double)s * (double)out_elems * 4.0 / bytes_per_us;
+        if (gain > best_gain) { best = (int)s; best_gain = gain; }
+    }
+    return best;
 }
 // Opened by every exported matmul entry point for the time it enqueues its launches (weight_cache.hip): copies that the
 // weight cache hands out inside the scope cannot be evicted before it closes; bypass = true switches the cache off for

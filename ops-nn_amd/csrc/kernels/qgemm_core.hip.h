@@ -60,8 +60,9 @@ struct QgemmParams {
     // exact MX route, whose kernel then left the call to this one); otherwise every workgroup returns at once.
     const int* gate;
     int gate_n;
-    // MODE_I8, K split over `splits` workgroups per tile (SPLIT instantiations, grid.z): int32 partial sums
-    // [splits][batch][M][N]; qg_i8_splitk_reduce_kernel adds them (exactly: integers) and applies the epilogue
+    // K split over `splits` workgroups per tile (SPLIT instantiations, grid.z): partial sums [splits][batch][M][N] -- int32
+    // for MODE_I8 (qg_i8_splitk_reduce_kernel adds them exactly and applies the epilogue), fp32 with the MX scales applied
+    // for the MX modes (qg_mx_splitk_reduce_kernel adds them in split order, then the bias)
     int splits;
     int32_t* part;
 #if QG_DBG
@@ -90,7 +91,7 @@ __device__ __forceinline__ void async_copy4(const void* g, void* lds)
 template <int MODE, int BM, int BN, int BK, int WGM, int WGN, int STAGES, int MINWG, bool KTAIL, int OUT_DT, bool SPLIT = false>
 __global__ __launch_bounds__(WGM* WGN * 64, MINWG) void qgemm_kernel(QgemmParams p, int tiles_m, int tiles_n)
 {
-    static_assert(!SPLIT || (MODE == MODE_I8 && !KTAIL), "the K split: int8 operands, whole K tiles");
+    static_assert(!SPLIT || !KTAIL, "the K split: whole K tiles");
     constexpr bool MX = MODE != MODE_I8;
     constexpr int NT = WGM * WGN * 64;
     constexpr int CPR = BK / 16;                 // 16-byte chunks per LDS row
@@ -158,10 +159,13 @@ __global__ __launch_bounds__(WGM* WGN * 64, MINWG) void qgemm_kernel(QgemmParams
     const int8_t* B = p.b + bz * p.b_bs + n0 * ldb;
     const int64_t K = p.KB;
     int KT = (int)((K + BK - 1) / BK);
+    int kt_first = 0;
     if constexpr (SPLIT) {   // this workgroup's K tiles: kt_first .. kt_first + KT - 1 (at least STAGES: the launcher splits at most KT / 4 ways)
-        const int z = (int)blockIdx.z;
-        const int kt_first = (int)((int64_t)z * KT / p.splits);
-        KT = (int)((int64_t)(z + 1) * KT / p.splits) - kt_first;
+        // (tiles whose scales travel in pairs are dealt in pairs)
+        constexpr int U = (MX && BK / (MODE == MODE_MXFP8 ? 32 : 16) == 8) ? 2 : 1;
+        const int z = (int)blockIdx.z, units = KT / U;
+        kt_first = (int)((int64_t)z * units / p.splits) * U;
+        KT = (int)((int64_t)(z + 1) * units / p.splits) * U - kt_first;
         A += (int64_t)kt_first * BK;
         B += (int64_t)kt_first * BK;
     }
@@ -206,6 +210,7 @@ __global__ __launch_bounds__(WGM* WGN * 64, MINWG) void qgemm_kernel(QgemmParams
                 rr = rr < b_rows ? rr : b_rows - 1;
                 sc_src[i] = p.sb + bz * p.sb_bs + (n0 + rr) * p.sb_rs + part * 4;
             }
+            if constexpr (SPLIT) sc_src[i] += SC16 ? (int64_t)(kt_first >> 1) * 16 : (int64_t)kt_first * SCB;
         }
     }
 
@@ -461,7 +466,9 @@ __global__ __launch_bounds__(WGM* WGN * 64, MINWG) void qgemm_kernel(QgemmParams
     k_tile(kt, F{}, F{}, F{});
     if constexpr (SPLIT) {
         // partial sums straight from the registers (acc[i][j][r]: n = n_base + 8*(r/4) + 4*(lane/32) + r%4, m = m_base + lane%32)
-        int32_t* part = p.part + (((int64_t)blockIdx.z * gridDim.y + bz) * p.M) * p.N;
+        typedef std::conditional_t<MODE == MODE_I8, v4i, v4f> quad_t;
+        typedef std::conditional_t<MODE == MODE_I8, int32_t, float> elem_t;
+        elem_t* part = (elem_t*)p.part + (((int64_t)blockIdx.z * gridDim.y + bz) * p.M) * p.N;
         const bool vec_ok4 = (p.N % 4) == 0 && ((uintptr_t)p.part % 16) == 0;
 #pragma unroll
         for (int j = 0; j < FM; j++) {
@@ -472,9 +479,9 @@ __global__ __launch_bounds__(WGM* WGN * 64, MINWG) void qgemm_kernel(QgemmParams
                 for (int q = 0; q < 4; q++) {
                     const int64_t n = n0 + wn * TN + i * 32 + 8 * q + 4 * (lane >> 5);
                     if (m >= p.M) continue;
-                    const v4i o = {acc[i][j][q * 4], acc[i][j][q * 4 + 1], acc[i][j][q * 4 + 2], acc[i][j][q * 4 + 3]};
+                    const quad_t o = {acc[i][j][q * 4], acc[i][j][q * 4 + 1], acc[i][j][q * 4 + 2], acc[i][j][q * 4 + 3]};
                     if (vec_ok4 && n + 3 < p.N) {
-                        *(v4i*)(part + m * p.N + n) = o;
+                        *(quad_t*)(part + m * p.N + n) = o;
                     } else {
 #pragma unroll
                         for (int e = 0; e < 4; e++)
@@ -726,6 +733,51 @@ __global__ __launch_bounds__(256) void qg_i8_splitk_reduce_kernel(QgemmParams p,
         const float v = tv + fb;
         ((uint16_t*)p.out)[(bz * p.M + m) * p.ldc + n] = OUT_DT == DT_BF16 ? bf16_bits(v) : f16_bits(v);
     }
+}
+
+// The MX modes after a K split: out[b, m, n] = rounded(sum of the fp32 partial sums, in split order, + bias[n])
+template <int OUT_DT>
+__global__ __launch_bounds__(256) void qg_mx_splitk_reduce_kernel(QgemmParams p, int64_t total)
+{
+    const int64_t MN = p.M * p.N, stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
+        float v = splitk_sum((const float*)p.part, p.splits, total, i);
+        const int64_t bz = i / MN, m = (i % MN) / p.N, n = i % p.N;
+        if (p.bias) v = v + load_scalar_as_f32(p.bias, p.bias_dt, bz * p.bias_bs + n);
+        const int64_t o = (bz * p.M + m) * p.ldc + n;
+        if constexpr (OUT_DT == DT_F32) ((float*)p.out)[o] = v;
+        else ((uint16_t*)p.out)[o] = OUT_DT == DT_BF16 ? bf16_bits(v) : f16_bits(v);
+    }
+}
+
+// The K split of an MX mode (p.splits > 1, whole K tiles, no gate): the tile kernel per split, then the reduction.
+template <int MODE, int BM, int BN, int BK, int WGM, int WGN, int STAGES, int MINWG>
+static int qgemm_launch_split_mx(const QgemmParams& p, int64_t batch, int out_dt, hipStream_t st)
+{
+    static_assert(MODE != MODE_I8, "the MX modes");
+    constexpr int SCB = BK / (MODE == MODE_MXFP8 ? 32 : 16);
+    constexpr int U = SCB == 8 ? 2 : 1;
+    if (!p.part || p.splits < 2 || p.gate || (p.KB % (BK * U)) != 0 || p.splits > p.KB / BK / U / 2) return -1;
+    int tiles_m = (int)((p.M + BM - 1) / BM), tiles_n = (int)((p.N + BN - 1) / BN);
+    dim3 grid((unsigned)(tiles_m * tiles_n), (unsigned)batch, (unsigned)p.splits);
+    const size_t lds = SCB == 8 ? (size_t)STAGES * (BM + BN) * BK + 2 * (BM + BN) * 16 : (size_t)STAGES * ((BM + BN) * BK + (BM + BN) * SCB);
+    auto k = qgemm_kernel<MODE, BM, BN, BK, WGM, WGN, STAGES, MINWG, false, DT_F32, true>;
+    static std::atomic<uint64_t> attr_set{0};
+    if (!device_flag_test(attr_set)) {
+        hipError_t e = hipFuncSetAttribute((const void*)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return (int)e;
+        device_flag_set(attr_set);
+    }
+    hipLaunchKernelGGL(k, grid, dim3(WGM * WGN * 64), lds, st, p, tiles_m, tiles_n);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return (int)e;
+    const int64_t total = batch * p.M * p.N;
+    const unsigned rgrid = splitk_reduce_grid(total);
+    if (out_dt == DT_BF16) hipLaunchKernelGGL(qg_mx_splitk_reduce_kernel<DT_BF16>, dim3(rgrid), dim3(256), 0, st, p, total);
+    else if (out_dt == DT_F16) hipLaunchKernelGGL(qg_mx_splitk_reduce_kernel<DT_F16>, dim3(rgrid), dim3(256), 0, st, p, total);
+    else if (out_dt == DT_F32) hipLaunchKernelGGL(qg_mx_splitk_reduce_kernel<DT_F32>, dim3(rgrid), dim3(256), 0, st, p, total);
+    else return -2;
+    return (int)hipGetLastError();
 }
 
 // The K split of MODE_I8 (p.splits > 1, K a multiple of BK): the tile kernel per split, then the reduction.

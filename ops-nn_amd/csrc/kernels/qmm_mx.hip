@@ -336,12 +336,25 @@ int launch_mx_mfma(const OpsnnQmmArgs& a0, hipStream_t st, SplitK sk)
     }
     const bool small = a.M <= 128 || a.N <= 128;
     if (fp4) {
-        if (small || a.force_variant == OPSNN_VARIANT_MX_128) return qgemm_launch<MODE_MXFP4, 128, 128, 64, 2, 2, 4, 1>(g, a.batch, a.out_dtype, st);
+        // few tiles against a long K: K split over workgroups (fp32 partial sums in front of the workspace), on the tiles
+        // chosen below
+        const bool split = sk.splits > 1 && sk.part && a.force_variant == 0 && a.K % 256 == 0;
+        if (split) { g.splits = sk.splits; g.part = (int32_t*)sk.part; }
+        // 128 x 128 tiles also when 256 x 256 ones would be at most 32 (an eighth of the CUs)
+        const int64_t t256 = ((a.M + 255) / 256) * ((a.N + 255) / 256) * a.batch;
+        if (small || t256 <= 32 || a.force_variant == OPSNN_VARIANT_MX_128) {
+            if (split) return qgemm_launch_split_mx<MODE_MXFP4, 128, 128, 64, 2, 2, 4, 1>(g, a.batch, a.out_dtype, st);
+            return qgemm_launch<MODE_MXFP4, 128, 128, 64, 2, 2, 4, 1>(g, a.batch, a.out_dtype, st);
+        }
         // K tiles of 128 bytes (256 elements) with the scales of two tiles per 16-byte copy: needs an even number of
         // such tiles and 16-byte aligned scale rows
         const bool sc16 = a.K % 512 == 0 &&
                           (((uintptr_t)g.sa | (uintptr_t)g.sb | (uint64_t)g.sa_rs | (uint64_t)g.sb_rs | (uint64_t)g.sa_bs | (uint64_t)g.sb_bs) % 16) == 0;
-        if (sc16) return qgemm_launch<MODE_MXFP4, 256, 256, 128, 2, 4, 2, 1>(g, a.batch, a.out_dtype, st);
+        if (sc16) {
+            if (split) return qgemm_launch_split_mx<MODE_MXFP4, 256, 256, 128, 2, 4, 2, 1>(g, a.batch, a.out_dtype, st);
+            return qgemm_launch<MODE_MXFP4, 256, 256, 128, 2, 4, 2, 1>(g, a.batch, a.out_dtype, st);
+        }
+        if (split) return qgemm_launch_split_mx<MODE_MXFP4, 256, 256, 64, 2, 2, 4, 1>(g, a.batch, a.out_dtype, st);
         return qgemm_launch<MODE_MXFP4, 256, 256, 64, 2, 2, 4, 1>(g, a.batch, a.out_dtype, st);
     }
     // FLOAT output: the tile kernel, whose epilogue stores fp32 straight from the registers

@@ -74,19 +74,24 @@ def test_fp8_blockscale_k_tail(gpu, M, K, N, tB, gsM, fast):
     m.lib().aclDestroyAclOpExecutor(ex)
 
 
-def _splitk_bytes(M, K, N, bm, bn, batch=1):
-    """The fp32 partial sums that phase 1 puts in front of the workspace when a call of a mode that can split K (fp8 block
-    scales from 129 rows, MXFP8, fp8 x fp4 MX and int8 per-tile from 33 rows, int8 per-token / per-channel on 128 x 128
-    tiles; K >= 1024) has at most 128 tiles (int8 per-token / per-channel: 32): 2 .. 16 splits, at least four K tiles each."""
+def _splitk_bytes(M, K, N, bm, bn, batch=1, tile_us=1.4, kunit=128, bytes_per_us=5.0e6):
+    """The partial sums that phase 1 puts in front of the workspace when a call of a mode that can split K has few tiles
+    against a long K (splitk_factor in launch.h): at most 128 tiles, K >= 1024, 2 .. 16 splits of at least four K tiles, the
+    count with the largest estimated gain (loop time saved less a launch and the partial sums' traffic), if at least 3 us.
+    bm x bn: the mode's tile; tile_us: one K tile of its kernel (1.4 the exact fp8 kernel, 1.8 fp8 x fp4 MX and int8
+    per-tile, 0.55 int8 per-token / per-channel on 128 x 128 tiles -- that one with bytes_per_us = 2.4e6)."""
     if (M <= 32 and bm != 128) or M * N < 64 * 64 or K < 1024:
         return 0
     tiles = -(-M // bm) * -(-N // bn) * batch
-    if bm == bn == 128 and (tiles > 32 or M * N * batch > 256 * 1024):   # the int8 per-token / per-channel kernel's tiles
-        return 0
     if tiles > 128:
         return 0
-    s = min(256 // tiles, -(-K // 128) // 4, 16)
-    return -(-(s * batch * M * N * 4) // 256) * 256 if s >= 2 else 0
+    kt = -(-K // kunit)
+    best, best_gain = 1, 3.0
+    for s in range(2, min(256 // tiles, kt // 4, 16) + 1):
+        gain = kt * tile_us * (1.0 - 1.0 / s) - 4.0 - 2.0 * s * (M * N * batch) * 4.0 / bytes_per_us
+        if gain > best_gain:
+            best, best_gain = s, gain
+    return -(-(best * batch * M * N * 4) // 256) * 256 if best >= 2 else 0
 
 
 def _mx_pad_bytes(M, K, N, fp4, batch=1):
@@ -191,7 +196,7 @@ def test_mx_fp8_fp4_k_tail(gpu, M, K, N):
     bias = m.Tensor((1, N), m.ACL_FLOAT16, d["bias"])
     o = m.Tensor((M, N), m.ACL_FLOAT16, m.DeviceBuffer(M * N * 2))
     rc, ws, ex = m.quant_matmul_v5_get_workspace(x1, x2, s1, s2, o, bias=bias, transpose_x2=True, group_size=32)
-    assert rc == 0 and ws == up(M * Kp) + up(N * Kp // 2) + up(M * (Kp // 64) * 2) + up(N * (Kp // 64) * 2) + _splitk_bytes(M, K, N, 256, 256), (rc, ws)
+    assert rc == 0 and ws == up(M * Kp) + up(N * Kp // 2) + up(M * (Kp // 64) * 2) + up(N * (Kp // 64) * 2) + _splitk_bytes(M, K, N, 256, 256, tile_us=1.8), (rc, ws)
     m.lib().aclDestroyAclOpExecutor(ex)
     m.lib().opsnnSetForcePlain(1)
     try:

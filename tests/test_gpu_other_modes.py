@@ -188,6 +188,10 @@ def test_fp8_blockscale_group_size_inferred(gpu):
     (260, 1536, 300, True, True), (512, 2048, 264, False, True), (384, 768, 256, True, True),
     # MXFP8 on the block kernel: ragged tiles, one K tile, many K tiles, N-contiguous x2
     (300, 128, 260, True, False), (512, 4096, 256, True, False), (100, 1024, 520, False, False),
+    # MXFP4 with few tiles against a long K: the K split on 128 x 128 tiles (which also replace 256 x 256 ones when those
+    # would be at most 32), on 256 x 256 tiles with paired scale copies (K % 512 == 0) and without
+    (64, 8192, 512, True, True), (256, 8192, 1024, True, True), (257, 8192, 4200, True, True), (257, 7936, 4200, True, True),
+    (40, 8192, 300, False, True),
 ])
 def test_mx(gpu, M, K, N, tB, fp4, use_plain):
     """plain: bit-identical.  Default: MXFP4 on the scaled 4-bit instruction (its products and sums are exact), MXFP8 on

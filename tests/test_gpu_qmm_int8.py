@@ -33,9 +33,9 @@ def _check_equal(got, want, what):
     # few 128 x 128 tiles against a long K: K split over 2 .. 16 workgroups per tile, int32 partial sums in the workspace
     # (behind them the re-laid-out x2 of the N-contiguous case), summed exactly: still bit-identical
     (64, 4096, 512, True),
-    (200, 2048, 1000, False),
+    (200, 8192, 1000, False),
     (16, 8192, 264, True),
-    (130, 1024, 130, True),    # a column count that is no multiple of 4
+    (130, 4096, 130, True),    # a column count that is no multiple of 4
 ])
 @pytest.mark.parametrize("out_dt,bias_dt", [("bf16", "bf16"), ("bf16", None), ("f16", "f32"), ("bf16", "i32"), ("f16", "f16")])
 def test_kc_matches_oracle(gpu, M, K, N, tB, out_dt, bias_dt):
@@ -76,7 +76,7 @@ def test_batched(gpu):
                                            transpose_x2=True, batch=3)
     _check_equal(got, want, "batched K-C")
     print("case int8 batched, K split", flush=True)
-    got, want, _ = cases.run_qmm_int8_case(m, orc, 130, 2048, 140, seed=10, out_dtype=m.ACL_F16 if hasattr(m, "ACL_F16") else m.ACL_FLOAT16,
+    got, want, _ = cases.run_qmm_int8_case(m, orc, 130, 4096, 140, seed=10, out_dtype=m.ACL_F16 if hasattr(m, "ACL_F16") else m.ACL_FLOAT16,
                                            bias_dtype=m.ACL_INT32, transpose_x2=True, batch=3)
     _check_equal(got, want, "batched K-C with a K split")
 

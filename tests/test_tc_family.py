@@ -189,7 +189,7 @@ GPU_CASES = [
     # few tiles against a long K: the int8 kernel's K split (integer partial sums: bit-identical), packed scale words with
     # the 19-bit truncation, K-contiguous and N-contiguous x2
     (64, 4096, 256, "i8", "u64", "N", "i32", "f16", True, False, 0),
-    (200, 2048, 520, "i8", "f32", 1, "i32", "bf16", False, False, 0),
+    (200, 8192, 520, "i8", "f32", 1, "i32", "bf16", False, False, 0),
     # INT8 (requantised) and INT32 outputs on the MFMA kernel's integer epilogue: 128 x 128 and 256 x 256 tiles, K tails,
     # ragged and odd N, N-contiguous x2 (re-laid out into the workspace), offsets from the tensor and from the packed word
     (128, 256, 192, "i8", "u64", "N", "i32", "i8", True, False, "N"),

@@ -26,7 +26,7 @@ def _run_pair(m, M, K, N, seed):
     need = m.lib().opsnnQmmWorkspace(C.byref(a), 0)
     # the fast path applies: the re-laid-out operand is the scratch buffer in question; opsnnQmmInt8 also gets room for the
     # integer partial sums of a K split when the call has few tiles (the no-alloc entry point runs unsplit: same bits)
-    assert need == N * K + _splitk_bytes(M, K, N, 128, 128), need
+    assert need == N * K + _splitk_bytes(M, K, N, 128, 128, tile_us=0.55, bytes_per_us=2.4e6), need
     ws = m.DeviceBuffer(need)
     a.workspace = ws.ptr
     assert m.lib().opsnnQmmInt8(C.byref(a), None) == 0
