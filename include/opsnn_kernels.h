@@ -102,14 +102,17 @@ OPSNN_API int opsnnQmmBlockScale(const OpsnnQmmArgs* a, void* stream);
 OPSNN_API void opsnnSetFp8Fast(int fast);
 OPSNN_API int opsnnGetFp8Fast(void);
 /* Routing switches, process-wide.  The first also starts from the environment variable OPSNN_FORCE_PLAIN, read once when
- * the library is loaded; the other two are hooks of the parity tests, which compare two kernels on the same call:
+ * the library is loaded; the others are hooks of the parity tests, which compare two kernels on the same call:
  *   opsnnSetForcePlain(1)  every call runs on the plain one-thread-per-output kernels (bit-identical to the CPU oracle);
  *   opsnnSetMx8Wide(n)     MXFP8 on the four-wave kernel with 256 x 32n tiles (n = 8, 9), 0 never, -1 automatic;
  *   opsnnSetWqTileMin(m)   weight-only int4/int8 calls with m .. 256 rows of x run on the dequantise-once tile kernel
- *                          (default 129; 1 sends every eligible call there, 257 none). */
+ *                          (default 129; 1 sends every eligible call there, 257 none);
+ *   opsnnSetWqNarrowSlabs(0) weight-only calls against a narrow weight (N <= 16384) run one pass of up to 256 rows per
+ *                          launch, as wide ones do (default 1: equal row slabs of 64 .. 256 rows, all in one launch). */
 OPSNN_API void opsnnSetForcePlain(int on);
 OPSNN_API void opsnnSetMx8Wide(int n);
 OPSNN_API void opsnnSetWqTileMin(int m);
+OPSNN_API void opsnnSetWqNarrowSlabs(int on);
 /* Opt-in cache of re-laid-out right operands.  The matrix-core kernels stream a K-contiguous right operand; x2 / weight
  * stored [K, N] with N contiguous is re-laid out inside every call (into the caller's workspace) unless this cache is on:
  * then opsnnQmmInt8, opsnnQmmBlockScale, opsnnQmmMx (data and scales) and opsnnWqmm keep the K-contiguous copy in device memory of the library's own, keyed

@@ -38,8 +38,14 @@ using namespace opsnn;
 //   opsnnSetMx8Wide(n) (test hook): MXFP8 on the four-wave kernel with 256 x 32n tiles, n = 8 or 9; 0 never; -1 the selector
 //   decides (default);
 //   opsnnSetWqTileMin(m) (test hook): weight-only int4/int8 calls with m .. 256 rows of x run on the dequantise-once tile
-//   kernel (default 129: below that the streaming kernels are faster).
+//   kernel (default 129: below that the streaming kernels are faster);
+//   opsnnSetWqNarrowSlabs(on) (test hook): 0 keeps weight-only calls against a narrow weight (at most 128 workgroups of 128
+//   columns) on one pass per launch, as wide ones run, so that small test shapes reach every instance of the many-rows kernel
+//   (default 1: their rows go out as equal slabs in one launch).
 static int g_wq_tile_min = 129;
+static int g_wq_narrow_slabs = 1;
+extern "C" void opsnnSetWqNarrowSlabs(int on) { __atomic_store_n(&g_wq_narrow_slabs, on ? 1 : 0, __ATOMIC_RELAXED); }
+extern "C" __attribute__((visibility("hidden"))) int opsnn_wq_narrow_slabs() { return __atomic_load_n(&g_wq_narrow_slabs, __ATOMIC_RELAXED); }
 extern "C" void opsnnSetWqTileMin(int m) { __atomic_store_n(&g_wq_tile_min, m, __ATOMIC_RELAXED); }
 extern "C" __attribute__((visibility("hidden"))) int opsnn_wq_tile_min() { return __atomic_load_n(&g_wq_tile_min, __ATOMIC_RELAXED); }
 static int g_force_plain = [] { const char* e = getenv("OPSNN_FORCE_PLAIN"); return (e && *e && *e != '0') ? 1 : 0; }();

@@ -347,7 +347,24 @@ template <int XDT, int WBITS>
 int launch_wq_tile(const WqParams& p, hipStream_t st);   // wqmm_tile.hip
 }  // namespace opsnn
 extern "C" int opsnn_wq_tile_min();   // dispatch.hip
+extern "C" int opsnn_wq_narrow_slabs();
 namespace opsnn {
+
+// The many-rows kernel's workgroups take 128 columns each, so one pass over a narrow weight leaves most CUs idle, and
+// passes launched one after the other do not overlap (4096 x 4096 int4: 32 workgroups, 256 rows 56 us, 1024 rows in four
+// passes 219 us).  With at most 128 workgroups per pass and more than 64 rows the rows are cut into equal slabs of 64 ..
+// 256 rows, as many as give every CU a workgroup in one round, and all slabs go out in one launch (grid.y).  Returns the
+// slab's rows, or 0 where the one-pass-at-a-time order stays.
+static int64_t narrow_n_slab(int64_t M, int64_t N)
+{
+    const int64_t wgs = (N + 127) / 128;
+    if (M <= 64 || wgs > 128 || !opsnn_wq_narrow_slabs()) return 0;
+    int64_t n = 256 / wgs;
+    if (n > (M + 63) / 64) n = (M + 63) / 64;
+    if (n < (M + 255) / 256) n = (M + 255) / 256;
+    if (n < 2) return 0;
+    return ((M + n - 1) / n + 15) / 16 * 16;
+}
 
 // floating-point weight codes: the general kernel, in row slabs of 64
 template <int XDT, int WBITS>
@@ -372,6 +389,11 @@ static int launch_slabs_float(WqParams p, hipStream_t st)
         if (WBITS == 4) ok = ok && p.scale_e8m0 && p.group == 32 && p.s_rs == 1;
         else ok = ok && !p.scale_e8m0 && p.group >= p.K;
         if (ok) {
+            if (const int64_t slab = narrow_n_slab(p.M, p.N)) {   // narrow N: all row slabs in one launch
+                p.cpg_shift = WBITS == 4 ? 0 : 31;
+                p.m_base = 0; p.m_rows = slab; p.m_slab = slab; p.m_end = p.M;
+                return launch_wq_rows_float<XDT, WBITS>(p, st);
+            }
             // up to 128 rows one pass; more: whole passes of 256 rows and the rest in one (as for integer codes below)
             const int64_t slab = p.M <= 128 ? 128 : 256;
             p.cpg_shift = WBITS == 4 ? 0 : 31;   // (e2m1: the kernel's scale table counts in words of four e8m0 bytes, one per 128 k chunk)
@@ -407,6 +429,17 @@ static int launch_slabs(WqParams p, hipStream_t st)
     // slabs of up to 256 rows; then the tile kernel.  (Measured on 8192 x 28672 int4, fp16: 256 rows 151-155 us against 170 on
     // the tile kernel, 192 rows 142-149 against 168.  Test hook: opsnnSetWqTileMin(m <= 128) sends such calls to the tile
     // kernel first.)
+    if (opsnn_wq_tile_min() > 128) {
+        if (const int64_t slab = narrow_n_slab(p.M, p.N)) {   // narrow N: all row slabs in one launch
+            WqParams q = p;
+            WqStreamOpts o{};
+            if (stream_eligible<WBITS>(q, o) && o.rows) {
+                q.m_base = 0; q.m_rows = slab; q.m_slab = slab; q.m_end = q.M;
+                const int rc = launch_wq_stream<XDT, WBITS>(q, o, st);
+                if (rc != OPSNN_NOT_TAKEN) return rc;
+            }
+        }
+    }
     if (p.M > 128 && opsnn_wq_tile_min() > 128) {
         WqParams q = p;
         WqStreamOpts o{};

@@ -436,6 +436,11 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void w
     static_assert(WF != 3 || (WBITS == 8 && XDT == DT_F16 && WK == 2 && NB == 2), "the block-scale form: fp16 x, e4m3 w, a slab per 128-block");
     static_assert(WF != 4 || (WBITS == 8 && XDT == DT_F16 && !HAS_OFF), "the row / column scale form: fp16 x, e4m3 w");
     constexpr int NT = 512;
+    if (p.m_slab > 0) {   // several row slabs in one launch: this workgroup's is number blockIdx.y
+        p.m_base += (int64_t)blockIdx.y * p.m_slab;
+        const int64_t left = p.m_end - p.m_base;
+        p.m_rows = left < p.m_slab ? left : p.m_slab;
+    }
     // More than 128 rows of x (MB = 12: up to 192, MB = 16: up to 256) with 4-bit weights: a lane's weight piece is 8 bytes instead of 16 (HP), so that a chunk is
     // 64 k per wave like an 8-bit one and two slab buffers of 256 rows fit the LDS (2 x 64 KB).  (Half-chunk slabs under
     // 16-byte pieces were built first: the wait for a chunk's second slab is a wait for everything older, the weight
@@ -1452,6 +1457,8 @@ static int launch_rows_one(const WqParams& p, hipStream_t st)
     const size_t lds = lds_main + (WF == 3 ? (size_t)(p.K / 128) * 16 * MB * 4 : 0) + lds_stab;
     if (lds > lds_main + lds_table + lds_stab) return OPSNN_NOT_TAKEN;
     const unsigned grid = (unsigned)((p.N + 16 * NB * WN - 1) / (16 * NB * WN));
+    const int64_t slabs = p.m_slab > 0 ? (p.m_end - p.m_base + p.m_slab - 1) / p.m_slab : 1;
+    if (slabs < 1 || slabs > 65535 || p.m_rows > 16 * MB || (p.m_slab > 0 && p.m_slab != p.m_rows)) return -1;
     auto k = wqmm_rows_kernel<XDT, WBITS, MB, NB, WN, WK, HAS_OFF, WF, SLDS>;
     static std::atomic<uint64_t> attr_set{0};   // one bit per device: the attribute belongs to the (kernel, device) pair
     if (!device_flag_test(attr_set)) {
@@ -1459,7 +1466,7 @@ static int launch_rows_one(const WqParams& p, hipStream_t st)
         if (e != hipSuccess) return (int)e;
         device_flag_set(attr_set);
     }
-    hipLaunchKernelGGL(k, dim3(grid), dim3(512), lds, st, p);
+    hipLaunchKernelGGL(k, dim3(grid, (unsigned)slabs), dim3(512), lds, st, p);
     return (int)hipGetLastError();
     }
 }

@@ -454,7 +454,15 @@ def test_weight_only_256_row_instance(gpu, M, K, N, x_dt, w_dt, group, tW, off, 
     inp = cases.make_wq_inputs(m, M, K, N, M * 7 + N, dt[x_dt], dt[w_dt], group, tW, off, dt[bias])
     want = cases.oracle_wq(m, inp, M, K, N)
     plain(False)
-    got = cases.run_wq_aclnn(m, inp, M, K, N)
+    # these weights are narrow: by default the rows go out as equal slabs of 64 .. 256 rows in one launch; with the hook the
+    # call runs one pass of up to 256 rows per launch, as against a wide weight -- the instance this test is about
+    narrow = cases.run_wq_aclnn(m, inp, M, K, N)
+    check_close(narrow, want, dt[x_dt], "weight-only, row slabs in one launch")
+    m.lib().opsnnSetWqNarrowSlabs(0)
+    try:
+        got = cases.run_wq_aclnn(m, inp, M, K, N)
+    finally:
+        m.lib().opsnnSetWqNarrowSlabs(1)
     check_close(got, want, dt[x_dt], "weight-only 256-row instance")
     m.lib().opsnnSetWqTileMin(1)
     try:
@@ -543,7 +551,13 @@ def test_weight_only_float_codes_on_the_many_rows_kernel(gpu, M, K, N, x_dt, w_d
     inp = cases.make_wq_inputs(m, M, K, N, M * 3 + N, dt[x_dt], dt[w_dt], group, True, False, dt[bias])
     want = cases.oracle_wq(m, inp, M, K, N)
     plain(False)
-    got = cases.run_wq_aclnn(m, inp, M, K, N)
+    narrow = cases.run_wq_aclnn(m, inp, M, K, N)   # (narrow weights: from 65 rows equal row slabs in one launch)
+    check_close(narrow, want, dt[x_dt], "weight-only float codes, row slabs in one launch")
+    m.lib().opsnnSetWqNarrowSlabs(0)
+    try:
+        got = cases.run_wq_aclnn(m, inp, M, K, N)      # one pass of up to 256 rows per launch: the 64- .. 256-row instances
+    finally:
+        m.lib().opsnnSetWqNarrowSlabs(1)
     check_close(got, want, dt[x_dt], "weight-only float codes, many rows")
 
 
