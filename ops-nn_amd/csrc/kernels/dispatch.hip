@@ -192,10 +192,10 @@ static int splitk_for(const OpsnnQmmArgs& a, int mode)
     int64_t bm, bn = 256, kunit = 128;
     double tile_us;   // one K tile (kunit elements) of the kernel in question, measured on calls with few tiles
     double bytes_per_us = 5.0e6;   // what its partial sums' traffic was measured to cost (splitk_factor)
-    // int8 with per-token / per-channel scales on 128 x 128 tiles (the selector's choice below 256 x 256 x 64 outputs; whole K
+    // int8 with per-token / per-channel scales on 128 x 128 tiles (the selector's choice up to 256 x 256 x 64 outputs; whole K
     // tiles): integer partial sums, so the result stays bit-identical
     if ((mode == 0 || (mode == 3 && !a.x1_scale)) && a.x1_dtype == DT_I8 && a.x2_dtype == DT_I8 && out16 && a.K % 128 == 0 &&
-        (a.M <= 128 || a.N <= 128 || a.M * a.N < 256 * 256 * 64)) {
+        (a.M <= 128 || a.N <= 128 || a.M * a.N <= 256 * 256 * 64)) {
         // (a 128 x 128 int8 tile is quick, and the partial sums cost their own traffic: measured at 4096 x 4096 in eight
         // splits, 64 rows 20 -> 15 us, 128 rows 19.5 -> 22, 256 rows in four 21 -> 24)
         bm = 128; bn = 128; tile_us = 0.55; bytes_per_us = 2.4e6;

@@ -171,7 +171,7 @@ static int qmm_int8_impl(const OpsnnQmmArgs* a, void* stream, SplitK sk)
         g.bias = p.bias; g.bias_dt = p.bias_dt; g.bias_bs = p.bias_bs;
         if (int_out) {
             g.x2off = a->x2_offset; g.x2off_len = a->x2_offset_len;
-            if (p.M <= 128 || p.N <= 128 || p.M * p.N < 256 * 256 * 64) return qgemm_launch_int<128, 128, 128, 2, 2, 2, 1>(g, a->batch, p.out_dt, st);
+            if (p.M <= 128 || p.N <= 128 || p.M * p.N <= 256 * 256 * 64) return qgemm_launch_int<128, 128, 128, 2, 2, 2, 1>(g, a->batch, p.out_dt, st);
             // the four-wave kernel under the conditions and with the tile width of the 16-bit outputs below
             const int64_t cus = cu_count();
             const int64_t tm = (p.M + 255) / 256, tn = (p.N + 255) / 256;
@@ -204,7 +204,7 @@ static int qmm_int8_impl(const OpsnnQmmArgs* a, void* stream, SplitK sk)
             case OPSNN_VARIANT_I8_256_W8_K128: return qgemm_launch<MODE_I8, 256, 256, 128, 2, 4, 2, 1>(g, a->batch, p.out_dt, st);
             default: break;
         }
-        if (p.M <= 128 || p.N <= 128 || p.M * p.N < 256 * 256 * 64) {
+        if (p.M <= 128 || p.N <= 128 || p.M * p.N <= 256 * 256 * 64) {
             if (sk.splits > 1 && p.K % 128 == 0) {   // few tiles against a long K: K split over workgroups, integer partial sums
                 g.splits = sk.splits; g.part = (int32_t*)sk.part;
                 return qgemm_launch_split_i8<128, 128, 128, 2, 2, 2, 1>(g, a->batch, p.out_dt, st);
