@@ -203,7 +203,7 @@ static int splitk_for(const OpsnnQmmArgs& a, int mode)
     // MXFP4: 128 x 128 tiles when 256 x 256 ones would be few (the launcher's rule), K tiles counted in 256 elements
     else if (mode == 2 && a.x1_dtype == DT_E2M1 && a.x2_dtype == DT_E2M1 && (out16 || a.out_dtype == DT_F32)) {
         const int64_t t256 = ((a.M + 255) / 256) * ((a.N + 255) / 256) * a.batch;
-        bm = bn = (a.M <= 128 || a.N <= 128 || t256 <= 32) ? 128 : 256;
+        bm = bn = (a.M <= 128 || a.N <= 128 || t256 <= 64) ? 128 : 256;
         kunit = 256;
         tile_us = bm == 128 ? 0.6 : 1.3; bytes_per_us = 2.4e6;
     }
