@@ -67,6 +67,10 @@ int launch_blockscale_rows(const OpsnnQmmArgs& a, hipStream_t st)
     p.bs1 = (const float*)a.x1_scale_mat.ptr; p.bs1_rs = a.x1_scale_mat.row_stride; p.bs1_cs = a.x1_scale_mat.col_stride;
     p.bs2 = (const float*)a.x2_scale_mat.ptr; p.bs2_rs = a.x2_scale_mat.row_stride; p.bs2_cs = a.x2_scale_mat.col_stride;
     p.bs_gsm = (int)a.gsM; p.bs_out_dt = a.out_dtype;
+    if (a.M > 64 && (a.N + 127) / 128 <= 128) {   // narrow x2 (at most 128 workgroups): two slabs of 64 rows in one launch, twice the workgroups
+        p.m_rows = 64; p.m_slab = 64; p.m_end = a.M;
+        return launch_rows_one<DT_F16, 8, 4, 2, 4, 2, false, 3>(p, st);
+    }
     return a.M > 64 ? launch_rows_one<DT_F16, 8, 8, 2, 4, 2, false, 3>(p, st) : launch_rows_one<DT_F16, 8, 4, 2, 4, 2, false, 3>(p, st);
 }
 
@@ -103,6 +107,10 @@ int launch_rowcol_rows(const OpsnnQmmArgs& a, hipStream_t st)
     p.bs1 = (const float*)a.x1_scale; p.bs1_rs = a.x1_scale_len == 1 ? 0 : 1;
     p.bs2 = (const float*)a.x2_scale; p.bs2_cs = a.x2_scale_len == 1 ? 0 : 1;
     p.bs_out_dt = a.out_dtype;
+    if (a.M > 64 && (a.N + 127) / 128 <= 128) {   // narrow x2 (at most 128 workgroups): two slabs of 64 rows in one launch, twice the workgroups
+        p.m_rows = 64; p.m_slab = 64; p.m_end = a.M;
+        return launch_rows_one<DT_F16, 8, 4, 2, 4, 2, false, 4>(p, st);
+    }
     return a.M > 64 ? launch_rows_one<DT_F16, 8, 8, 2, 4, 2, false, 4>(p, st) : launch_rows_one<DT_F16, 8, 4, 2, 4, 2, false, 4>(p, st);
 }
 
