@@ -355,6 +355,15 @@ namespace opsnn {
 // passes 219 us).  With at most 128 workgroups per pass and more than 64 rows the rows are cut into equal slabs of 64 ..
 // 256 rows, as many as give every CU a workgroup in one round, and all slabs go out in one launch (grid.y).  Returns the
 // slab's rows, or 0 where the one-pass-at-a-time order stays.
+// Up to 64 rows per slab, `slabs` slabs, and still at most 128 workgroups of 128 columns: the instance whose workgroups
+// take 64 columns (K split over four waves instead of two; needs K in whole groups of 16 chunks) doubles their number.
+template <int WBITS>
+static int use_cols64(int64_t rows, int64_t slabs, int64_t N, int64_t K)
+{
+    constexpr int64_t KC = 4 * (128 / WBITS);
+    return (rows <= 64 && slabs * ((N + 127) / 128) <= 128 && K % (16 * KC) == 0 && N % 32 == 0 && opsnn_wq_narrow_slabs()) ? 1 : 0;
+}
+
 static int64_t narrow_n_slab(int64_t M, int64_t N)
 {
     const int64_t wgs = (N + 127) / 128;
@@ -392,8 +401,10 @@ static int launch_slabs_float(WqParams p, hipStream_t st)
             if (const int64_t slab = narrow_n_slab(p.M, p.N)) {   // narrow N: all row slabs in one launch
                 p.cpg_shift = WBITS == 4 ? 0 : 31;
                 p.m_base = 0; p.m_rows = slab; p.m_slab = slab; p.m_end = p.M;
+                p.cols64 = use_cols64<WBITS>(slab, (p.M + slab - 1) / slab, p.N, p.K);
                 return launch_wq_rows_float<XDT, WBITS>(p, st);
             }
+            p.cols64 = use_cols64<WBITS>(p.M, 1, p.N, p.K);
             // up to 128 rows one pass; more: whole passes of 256 rows and the rest in one (as for integer codes below)
             const int64_t slab = p.M <= 128 ? 128 : 256;
             p.cpg_shift = WBITS == 4 ? 0 : 31;   // (e2m1: the kernel's scale table counts in words of four e8m0 bytes, one per 128 k chunk)
@@ -435,6 +446,7 @@ static int launch_slabs(WqParams p, hipStream_t st)
             WqStreamOpts o{};
             if (stream_eligible<WBITS>(q, o) && o.rows) {
                 q.m_base = 0; q.m_rows = slab; q.m_slab = slab; q.m_end = q.M;
+                q.cols64 = use_cols64<WBITS>(slab, (q.M + slab - 1) / slab, q.N, q.K);
                 const int rc = launch_wq_stream<XDT, WBITS>(q, o, st);
                 if (rc != OPSNN_NOT_TAKEN) return rc;
             }
@@ -490,6 +502,7 @@ static int launch_slabs(WqParams p, hipStream_t st)
     if (stream && o.rows) {
         const int64_t passes = (p.M + 127) / 128;
         slab = ((p.M + passes - 1) / passes + 15) / 16 * 16;
+        p.cols64 = use_cols64<WBITS>(p.M, 1, p.N, p.K);
     }
     for (int64_t m0 = 0; m0 < p.M; m0 += slab) {
         p.m_base = m0;

@@ -462,7 +462,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void w
     constexpr int LDS_MAIN = (2 * XBUF > WN * (WK - 1) * NB * MB * 4 * 64 * 4) ? 2 * XBUF : WN * (WK - 1) * NB * MB * 4 * 64 * 4;
     static_assert((16 * MB * XPR) % NT == 0 && XPR >= 16 && PF >= 2 && PPH >= 1 && STEPS == PPH * XH, "staging and prefetch shape");
     static_assert(MB <= 8 || (WF == 0 && SLDS) || WF == 1 || WF == 2, "the 192- / 256-row instances: integer codes with the scale table in LDS, or floating-point codes");
-    static_assert(!(SLDS && WF == 2) || WK == 2, "byte position of a lane's e8m0 scale inside the table word");
+    static_assert(!(SLDS && WF == 2 && MB > 8) || WK == 2, "8-byte pieces: byte position of a lane's e8m0 scale inside the table word");
     extern __shared__ __attribute__((aligned(16))) char sx[];
 
     const int tid = threadIdx.x, lane = tid & 63;
@@ -1499,6 +1499,7 @@ int launch_wq_rows_float(const WqParams& p, hipStream_t st);
         constexpr int WF = WBITS == 4 ? 2 : 1;                                                                      \
         if (p.m_rows > 192) return launch_rows_one<XDT, WBITS, 16, 2, 4, 2, false, WF>(p, st);                      \
         if (p.m_rows > 128) return launch_rows_one<XDT, WBITS, 12, 2, 4, 2, false, WF>(p, st);                      \
+        if (p.cols64 && p.m_rows <= 64) return launch_rows_one<XDT, WBITS, 4, 2, 2, 4, false, WF>(p, st);           \
         return p.m_rows > 64 ? launch_rows_one<XDT, WBITS, 8, 2, 4, 2, false, WF>(p, st)                            \
                              : launch_rows_one<XDT, WBITS, 4, 2, 4, 2, false, WF>(p, st);                           \
     }                                                                                                               \
@@ -1532,6 +1533,8 @@ int launch_wq_rows_float(const WqParams& p, hipStream_t st);
                                                        : launch_rows_one<XDT, WBITS, 12, 2, 4, 2, false>(p, st);          \
         if (o.rows && p.m_rows > 64) return o.has_off ? launch_rows_one<XDT, WBITS, 8, 2, 4, 2, true>(p, st)              \
                                                       : launch_rows_one<XDT, WBITS, 8, 2, 4, 2, false>(p, st);            \
+        if (o.rows && p.cols64) return o.has_off ? launch_rows_one<XDT, WBITS, 4, 2, 2, 4, true>(p, st)                   \
+                                                 : launch_rows_one<XDT, WBITS, 4, 2, 2, 4, false>(p, st);                 \
         if (o.rows) return o.has_off ? launch_rows_one<XDT, WBITS, 4, 2, 4, 2, true>(p, st)                               \
                                      : launch_rows_one<XDT, WBITS, 4, 2, 4, 2, false>(p, st);                             \
         if (o.ksplit && p.m_rows <= 16) return wq_stream_off<1, 4, 4, false>(p, o.has_off, st);                     \

@@ -472,6 +472,40 @@ def test_weight_only_256_row_instance(gpu, M, K, N, x_dt, w_dt, group, tW, off, 
     check_close(tile, want, dt[x_dt], "weight-only tile kernel")
 
 
+@pytest.mark.parametrize("M,K,N,x_dt,w_dt,group,off,bias", [
+    # up to 64 rows per slab against a narrow weight, K in whole groups of 16 chunks (int4 / mxfp4: K % 2048 == 0, int8 / e4m3:
+    # K % 1024 == 0): workgroups of 64 columns with K split over four waves; ragged last workgroup, scale table in LDS and
+    # per-lane scales, per-channel scales, four slabs of 64 rows in one launch
+    (64, 2048, 288, "f16", "i4", 128, True, None),
+    (49, 4096, 256, "bf16", "i4", 0, False, "bf16"),
+    (50, 1024, 320, "f16", "i8", 128, True, None),
+    (64, 3072, 256, "bf16", "i8", 64, True, None),          # 48 groups per row: no scale table
+    (64, 2048, 256, "bf16", "fp4", 32, False, None),
+    (33, 6144, 288, "f16", "fp4", 32, False, "f16"),        # K / 128 = 48: the e8m0 byte travels with the weight piece
+    (33, 1024, 288, "f16", "e4m3", 0, False, None),
+    (200, 2048, 512, "f16", "i4", 128, True, "f16"),
+    (130, 1024, 256, "bf16", "e4m3", 0, False, None),
+])
+def test_weight_only_64_column_workgroups(gpu, M, K, N, x_dt, w_dt, group, off, bias):
+    """The many-rows kernel's instance whose workgroups take 64 columns (chosen when 128-column ones would number at most 128)
+    against the oracle, and the same call on the 128-column instances (opsnnSetWqNarrowSlabs(0))."""
+    m = gpu
+    dt = {"bf16": m.ACL_BF16, "f16": m.ACL_FLOAT16, "i8": m.ACL_INT8, "i4": m.ACL_INT4, "e4m3": m.ACL_FLOAT8_E4M3FN,
+          "fp4": m.ACL_FLOAT4_E2M1, None: None}
+    print(f"case wq 64-column workgroups M={M} K={K} N={N} x={x_dt} w={w_dt} g={group} off={off} bias={bias}", flush=True)
+    inp = cases.make_wq_inputs(m, M, K, N, M * 5 + N, dt[x_dt], dt[w_dt], group, True, off, dt[bias])
+    want = cases.oracle_wq(m, inp, M, K, N)
+    plain(False)
+    got = cases.run_wq_aclnn(m, inp, M, K, N)
+    check_close(got, want, dt[x_dt], "weight-only, 64-column workgroups")
+    m.lib().opsnnSetWqNarrowSlabs(0)
+    try:
+        wide = cases.run_wq_aclnn(m, inp, M, K, N)
+    finally:
+        m.lib().opsnnSetWqNarrowSlabs(1)
+    check_close(wide, want, dt[x_dt], "weight-only, 128-column workgroups")
+
+
 @pytest.mark.parametrize("M,K,N,x_dt,w_dt,group,tW,off,bias", [
     # 4 .. 16 rows with K a multiple of 8 waves x 4, 8 or 16 chunks (int4: 4096, 8192; int8: 2048, 4096, 8192): groups of one
     # chunk (vector scale loads), of several chunks and per channel; with and without offset; ragged columns; fewer row
