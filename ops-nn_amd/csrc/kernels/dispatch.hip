@@ -438,9 +438,13 @@ static uint64_t qmm_workspace_base(const OpsnnQmmArgs* a, int mode)
 
 extern "C" uint64_t opsnnWqmmWorkspace(const OpsnnWqmmArgs* a)
 {
-    if (!a) return 0;
-    if (a->w.row_stride == 1 || a->K == 1) return 0;
-    if (a->w.col_stride != 1 || a->w.row_stride != a->N) return 0;
-    uint64_t bits = (a->w_dtype == DT_I4 || a->w_dtype == DT_E2M1) ? 4 : 8;
-    return (uint64_t)a->N * (uint64_t)a->K * bits / 8;
+    if (!a || a->M <= 0 || a->N <= 0 || a->K <= 0) return 0;
+    const uint64_t bits = (a->w_dtype == DT_I4 || a->w_dtype == DT_E2M1) ? 4 : 8;
+    // up to 16 rows against a long K: fp32 partial sums of the x-in-registers kernel's K split, in front of everything else
+    uint64_t part = 0;
+    if (const int xs = wq_xreg_splits((int)bits, a->M, a->K); xs > 1 && a->force_variant != OPSNN_VARIANT_PLAIN && !opsnn_force_plain())
+        part = ((uint64_t)xs * (uint64_t)a->M * (uint64_t)a->N * 4 + 255) / 256 * 256;
+    if (a->w.row_stride == 1 || a->K == 1) return part;
+    if (a->w.col_stride != 1 || a->w.row_stride != a->N) return part;
+    return part + (uint64_t)a->N * (uint64_t)a->K * bits / 8;
 }

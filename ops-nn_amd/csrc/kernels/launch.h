@@ -68,6 +68,19 @@ inline int splitk_factor(int64_t tiles, int64_t ktiles, double tile_us, int64_t 
     }
     return best;
 }
+// Weight-only calls with up to 16 rows of x and a K longer than one workgroup of the x-in-registers kernel holds (16 waves x
+// 4 chunks, i.e. 64 chunks of 64 weight bytes; 8-bit weights also 128; or 8 waves x 4 or 8 chunks): K in 2 .. 16 equal
+// segments of 64 chunks (else of 32), one workgroup column per segment, fp32 partial sums [segments][M][N] at the front of
+// the workspace.  1: no split (K fits one workgroup, or is not a whole number of segments).
+inline int wq_xreg_splits(int wbits, int64_t M, int64_t K)
+{
+    const int64_t kc = 4 * (128 / wbits);
+    if (M < 1 || M > 16 || K % (32 * kc) != 0) return 1;
+    const int64_t c32 = K / (32 * kc);
+    if (c32 == 1 || c32 == 2 || (wbits == 8 && c32 == 4)) return 1;   // one workgroup
+    if (c32 % 2 == 0 && c32 / 2 <= 16) return (int)(c32 / 2);
+    return c32 <= 16 ? (int)c32 : 1;
+}
 // Opened by every exported matmul entry point for the time it enqueues its launches (weight_cache.hip): copies that the
 // weight cache hands out inside the scope cannot be evicted before it closes; bypass = true switches the cache off for
 // this thread while the scope is open.  Scopes nest; the pins drop when the outermost one closes.

@@ -329,7 +329,9 @@ static bool stream_eligible(WqParams& p, WqStreamOpts& o)
     constexpr int xreg_min = 4, xreg_nw = 0;   // (0: xreg_shape picks the wave count)
     int xnw = 0, xnch = 0;
     o.xreg_nw = xreg_nw;
-    o.xreg = p.M >= xreg_min && p.M <= 16 && xreg_shape(WBITS, p.K, xreg_nw, xnw, xnch);
+    // (with room for partial sums also a K of several workgroup segments, and then fewer than 4 rows too where x does not fit the LDS)
+    int xsplits = 1;
+    o.xreg = p.M <= 16 && xreg_shape(WBITS, p.K, xreg_nw, xnw, xnch, p.M, p.part != nullptr, &xsplits) && (p.M >= xreg_min || (xsplits > 1 && !o.resx));
     o.xreg_vscale = o.xreg && p.group == KC && p.s_rs == 1 && p.s_cs % 8 == 0 &&
                     (uintptr_t)p.scale % 16 == 0 && (!p.offset || (uintptr_t)p.offset % 16 == 0);
     // more than 48 rows: two weight blocks per wave share every x fragment, up to 128 rows per pass over the weights
@@ -528,6 +530,14 @@ int launch_wqmm_mfma(const OpsnnWqmmArgs& a0, hipStream_t st)
     if (mx && (a.offset || a.group <= 0 || a.scale_n == 1)) return OPSNN_NOT_TAKEN;
     if (a.w_dtype == DT_E2M1 && a.offset) return OPSNN_NOT_TAKEN;   // the packed e2m1 dequantisation has no offset step
     const int wbits = (a.w_dtype == DT_I4 || a.w_dtype == DT_E2M1) ? 4 : 8;
+    // up to 16 rows against a long K: the partial sums of the x-in-registers kernel's K split sit at the front of the workspace
+    float* part = nullptr;
+    if (const int xs = wq_xreg_splits(wbits, a.M, a.K); xs > 1 && a.workspace) {
+        part = (float*)a.workspace;
+        const uint64_t pb = ((uint64_t)xs * (uint64_t)a.M * (uint64_t)a.N * 4 + 255) / 256 * 256;
+        const bool relayout = a.w.row_stride != 1 && a.K != 1;
+        a.workspace = relayout ? (char*)a.workspace + pb : nullptr;
+    }
     const int64_t kpl = 128 / wbits;
     if (a.K % kpl != 0 || a.K < kpl) return OPSNN_NOT_TAKEN;
     const int64_t group = a.group > 0 ? a.group : a.K;
@@ -553,6 +563,7 @@ int launch_wqmm_mfma(const OpsnnWqmmArgs& a0, hipStream_t st)
     p.s_rs = a.scale.row_stride; p.s_cs = a.scale_n == 1 ? 0 : a.scale.col_stride;
     p.bias = a.bias; p.bias_dt = a.bias_dtype;
     p.y = (uint16_t*)a.y; p.M = a.M; p.N = a.N; p.K = a.K; p.group = group;
+    p.part = part;
     p.group_shift = (group & (group - 1)) == 0 ? __builtin_ctzll((unsigned long long)group) : -1;
     if (a.K >= (1ll << 31) || a.N >= (1ll << 31)) return OPSNN_NOT_TAKEN;
     if (((uintptr_t)p.w | (uint64_t)p.ldw) % 16 || ((uintptr_t)p.x % 16) || (a.K % 8)) return OPSNN_NOT_TAKEN;

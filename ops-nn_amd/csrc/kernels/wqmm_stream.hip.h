@@ -1107,9 +1107,12 @@ __global__ __launch_bounds__(256, 2) void wqmm_resx_kernel(WqParams p)
 // chunk, or per channel); 1 one scale per chunk, a row's scales contiguous: 8- or 16-byte loads one row block ahead;
 // 2 (4-bit weights) one e8m0 byte per 32 weights, i.e. per lane piece, a row's bytes contiguous: 16-byte loads one row
 // block ahead.  WFLT: the weights are floating-point codes (e2m1 / e4m3), no offset.
-template <int XDT, int WBITS, int NW, int NCH, bool HAS_OFF, int SCM, bool WFLT = false>
+// TWO (eight waves x four chunks, the K split's smaller segment): x staged in two rounds through 64 KB of LDS, so that two
+// such workgroups (at most 128 registers per lane) share a CU.
+template <int XDT, int WBITS, int NW, int NCH, bool HAS_OFF, int SCM, bool WFLT = false, bool TWO = false>
 __global__ __launch_bounds__(NW * 64) void wqmm_xreg_kernel(WqParams p)
 {
+    static_assert(!TWO || (NW == 8 && NCH == 4), "two workgroups per CU: the eight-wave, four-chunk shape");
     constexpr bool VSCALE = SCM == 1, MXS = SCM == 2;
     static_assert(!MXS || WBITS == 4, "one e8m0 byte per lane piece of 32 weights");
     static_assert(!WFLT || !HAS_OFF, "floating-point weight codes carry no offset");
@@ -1119,8 +1122,8 @@ __global__ __launch_bounds__(NW * 64) void wqmm_xreg_kernel(WqParams p)
     static_assert(NW == 8 || NW == 16, "one or two workgroup halves per SIMD pair");
     static_assert(NX <= (NW == 16 ? 16 : 32), "x fragments must fit the register file beside the weight stream");
     static_assert(NCH % 4 == 0 && NCH >= PF, "whole groups of four chunks");
-    // 256-byte units of x per wave; the staging takes them in one round when all waves' units fit 128 KB of LDS, else in two
-    constexpr int NU = NX / 4, NR = NW * NU * 4096 <= 128 * 1024 ? 1 : 2, HU = NU / NR;
+    // 256-byte units of x per wave; the staging takes them in one round when all waves' units fit 128 KB of LDS (TWO: 64 KB), else in two
+    constexpr int NU = NX / 4, NR = NW * NU * 4096 <= (TWO ? 64 : 128) * 1024 ? 1 : 2, HU = NU / NR;
     static_assert(NU % NR == 0 && HU * 4096 >= 2048, "whole staging rounds that also hold the partial sums");
     extern __shared__ __attribute__((aligned(16))) char dyn[];
 
@@ -1128,7 +1131,9 @@ __global__ __launch_bounds__(NW * 64) void wqmm_xreg_kernel(WqParams p)
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int nrow = lane & 15, g = lane >> 4;
     const int rows = (int)p.m_rows;
-    const int cbase = wave * NCH;           // first chunk of this wave's K range
+    // first chunk of this wave's K range; with K split over gridDim.y workgroup columns this workgroup's segment is the
+    // blockIdx.y-th run of NW * NCH chunks
+    const int cbase = ((int)blockIdx.y * NW + wave) * NCH;
     const int nblocks = (int)((p.N + 15) / 16);
 
     auto row_of = [&](int rb) { const int64_t n = (int64_t)rb * 16 + nrow; return n < p.N ? n : p.N - 1; };
@@ -1200,7 +1205,7 @@ __global__ __launch_bounds__(NW * 64) void wqmm_xreg_kernel(WqParams p)
     {
         char* stage = dyn + wave * (HU * 4096);
         const int cm = lane >> 4, cp = lane & 15;
-        const uint16_t* xw = p.x + p.m_base * p.K + (int64_t)wave * (NU * 128);
+        const uint16_t* xw = p.x + p.m_base * p.K + (int64_t)cbase * KC;   // (NU * 128 = NCH * KC elements per wave)
 #pragma unroll
         for (int r = 0; r < NR; r++) {
 #pragma unroll
@@ -1288,7 +1293,17 @@ __global__ __launch_bounds__(NW * 64) void wqmm_xreg_kernel(WqParams p)
             v4f sum = *(const v4f*)(rd + lane * 4);
 #pragma unroll 4
             for (int j = 1; j < NW; j++) sum = sum + *(const v4f*)(rd + j * 256 + lane * 4);
-            if (nrow < rows) {
+            if (nrow < rows && gridDim.y > 1) {   // K split: this segment's sums, as they are, for wq_splitk_reduce_kernel
+                const int64_t m = p.m_base + nrow, nn0 = (int64_t)rb * 16 + 4 * g;
+                float* dst = p.part + ((int64_t)blockIdx.y * p.M + m) * p.N + nn0;
+                if (nn0 + 3 < p.N && (p.N % 4) == 0 && ((uintptr_t)p.part % 16) == 0) {
+                    *(v4f*)dst = sum;
+                } else {
+#pragma unroll
+                    for (int i = 0; i < 4; i++)
+                        if (nn0 + i < p.N) dst[i] = sum[i];
+                }
+            } else if (nrow < rows) {
                 const int64_t n0 = (int64_t)rb * 16;
                 const int64_t m = p.m_base + nrow;
                 float v[4];
@@ -1342,54 +1357,88 @@ static int launch_resx_one(const WqParams& p, hipStream_t st)
     return (int)hipGetLastError();
 }
 
-// One workgroup per CU (its waves fill the register file), or one per row block when there are fewer.
-template <int XDT, int WBITS, int NW, int NCH, bool HAS_OFF, int SCM, bool WFLT = false>
-static int launch_xreg_one(const WqParams& p, hipStream_t st)
+// y[m, n] = rounded(sum over the K segments, in order, of part[s, m, n] + bias[n])
+template <int XDT>
+__global__ __launch_bounds__(256) void wq_splitk_reduce_kernel(const float* part, int splits, int64_t total, int64_t N, const void* bias, int bias_dt,
+                                                               uint16_t* y)
 {
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
+        float v = splitk_sum(part, splits, total, i);
+        if (bias) v = v + load_scalar_as_f32(bias, bias_dt, i % N);
+        y[i] = bits_x<XDT>(v);
+    }
+}
+
+// One workgroup per CU (its waves fill the register file), or one per row block when there are fewer; with K split into
+// `splits` segments one workgroup column per segment, the CUs shared between the columns.
+template <int XDT, int WBITS, int NW, int NCH, bool HAS_OFF, int SCM, bool WFLT = false, bool TWO = false>
+static int launch_xreg_one(const WqParams& p, hipStream_t st, int splits = 1)
+{
+    if constexpr (NW == 8 && NCH == 4 && !TWO) {
+        if (splits > 1) return launch_xreg_one<XDT, WBITS, NW, NCH, HAS_OFF, SCM, WFLT, true>(p, st, splits);   // (measured at 16 x 28672 x 8192: 54 -> 42 us)
+    }
     const int64_t nblocks = (p.N + 15) / 16;
-    const int64_t g = (int64_t)resx_grid(1ll << 40) / 2;
+    if (splits < 1 || splits > 16 || (splits > 1 && (!p.part || p.m_base != 0 || p.m_rows != p.M))) return -1;
+    if ((int64_t)splits * NW * NCH * (4 * (128 / WBITS)) != p.K) return -1;
+    const int64_t g = ((int64_t)resx_grid(1ll << 40) / (TWO ? 1 : 2) + splits - 1) / splits;   // (resx_grid: two per CU)
     constexpr int STEPS = (4 * (128 / WBITS)) / 32;
     constexpr int NU = NCH * STEPS / 4;                  // units of 16 rows x 256 bytes per wave
-    constexpr int lds = NW * NU * 4096 <= 128 * 1024 ? NW * NU * 4096 : NW * (NU / 2) * 4096;   // all of x, or half of it at a time
-    auto k = wqmm_xreg_kernel<XDT, WBITS, NW, NCH, HAS_OFF, SCM, WFLT>;
+    constexpr int lds = NW * NU * 4096 <= (TWO ? 64 : 128) * 1024 ? NW * NU * 4096 : NW * (NU / 2) * 4096;   // all of x, or half of it at a time
+    auto k = wqmm_xreg_kernel<XDT, WBITS, NW, NCH, HAS_OFF, SCM, WFLT, TWO>;
     static std::atomic<uint64_t> attr_set{0};   // one bit per device: the attribute belongs to the (kernel, device) pair
     if (!device_flag_test(attr_set)) {
         hipError_t e = hipFuncSetAttribute((const void*)k, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
         if (e != hipSuccess) return (int)e;
         device_flag_set(attr_set);
     }
-    hipLaunchKernelGGL(k, dim3((unsigned)(nblocks < g ? nblocks : g)), dim3(NW * 64), lds, st, p);
+    hipLaunchKernelGGL(k, dim3((unsigned)(nblocks < g ? nblocks : g), (unsigned)splits), dim3(NW * 64), lds, st, p);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess || splits == 1) return (int)e;
+    const int64_t total = p.M * p.N;
+    hipLaunchKernelGGL(wq_splitk_reduce_kernel<XDT>, dim3(splitk_reduce_grid(total)), dim3(256), 0, st, (const float*)p.part, splits, total, p.N, p.bias,
+                       p.bias_dt, p.y);
     return (int)hipGetLastError();
 }
 
 template <int XDT, int WBITS, int NW, int NCH>
-static int launch_xreg_nch(const WqParams& p, bool has_off, bool vscale, hipStream_t st)
+static int launch_xreg_nch(const WqParams& p, bool has_off, bool vscale, hipStream_t st, int splits = 1)
 {
-    if (vscale) return has_off ? launch_xreg_one<XDT, WBITS, NW, NCH, true, 1>(p, st) : launch_xreg_one<XDT, WBITS, NW, NCH, false, 1>(p, st);
-    return has_off ? launch_xreg_one<XDT, WBITS, NW, NCH, true, 0>(p, st) : launch_xreg_one<XDT, WBITS, NW, NCH, false, 0>(p, st);
+    if (vscale) return has_off ? launch_xreg_one<XDT, WBITS, NW, NCH, true, 1>(p, st, splits) : launch_xreg_one<XDT, WBITS, NW, NCH, false, 1>(p, st, splits);
+    return has_off ? launch_xreg_one<XDT, WBITS, NW, NCH, true, 0>(p, st, splits) : launch_xreg_one<XDT, WBITS, NW, NCH, false, 0>(p, st, splits);
 }
 
 // K = waves x chunks per wave x chunk.  Sixteen waves with 4 chunks each (8-bit weights: or 8), else eight waves with 4 or 8.
-static inline bool xreg_shape(int wbits, int64_t K, int force_nw, int& nw, int& nch)
+// With room for partial sums (`may_split`) a longer K goes in `splits` segments of 16 x 4 chunks, else of 8 x 4
+// (wq_xreg_splits in launch.h names the count: the workspace query uses the same function).
+static inline bool xreg_shape(int wbits, int64_t K, int force_nw, int& nw, int& nch, int64_t M = 1, bool may_split = false, int* splits = nullptr)
 {
     const int64_t kc = 4 * (128 / wbits);
+    if (splits) *splits = 1;
     if (K % (32 * kc) != 0) return false;
     const int64_t c16 = K / (16 * kc), c8 = K / (8 * kc);
     if (force_nw != 8 && K % (64 * kc) == 0 && (c16 == 4 || (wbits == 8 && c16 == 8))) { nw = 16; nch = (int)c16; return true; }
     if (c8 == 4 || c8 == 8) { nw = 8; nch = (int)c8; return true; }
+    const int s = (may_split && splits) ? wq_xreg_splits(wbits, M, K) : 1;
+    if (s > 1) {
+        *splits = s;
+        nch = 4;
+        nw = (K / s == 64 * kc) ? 16 : 8;
+        return true;
+    }
     return false;
 }
 
 template <int XDT, int WBITS>
 static int launch_xreg(const WqParams& p, bool has_off, bool vscale, int force_nw, hipStream_t st)
 {
-    int nw = 0, nch = 0;
-    if (!xreg_shape(WBITS, p.K, force_nw, nw, nch)) return OPSNN_NOT_TAKEN;
-    if (nw == 16 && nch == 4) return launch_xreg_nch<XDT, WBITS, 16, 4>(p, has_off, vscale, st);
+    int nw = 0, nch = 0, splits = 1;
+    if (!xreg_shape(WBITS, p.K, force_nw, nw, nch, p.M, p.part != nullptr, &splits)) return OPSNN_NOT_TAKEN;
+    if (nw == 16 && nch == 4) return launch_xreg_nch<XDT, WBITS, 16, 4>(p, has_off, vscale, st, splits);
     if constexpr (WBITS == 8) {
         if (nw == 16 && nch == 8) return launch_xreg_nch<XDT, WBITS, 16, 8>(p, has_off, vscale, st);
     }
-    if (nw == 8 && nch == 4) return launch_xreg_nch<XDT, WBITS, 8, 4>(p, has_off, vscale, st);
+    if (nw == 8 && nch == 4) return launch_xreg_nch<XDT, WBITS, 8, 4>(p, has_off, vscale, st, splits);
     if (nw == 8 && nch == 8) return launch_xreg_nch<XDT, WBITS, 8, 8>(p, has_off, vscale, st);
     return OPSNN_NOT_TAKEN;
 }
@@ -1399,14 +1448,14 @@ static int launch_xreg(const WqParams& p, bool has_off, bool vscale, int force_n
 template <int XDT, int WBITS>
 static int launch_xreg_float(const WqParams& p, hipStream_t st)
 {
-    int nw = 0, nch = 0;
-    if (!xreg_shape(WBITS, p.K, 0, nw, nch)) return OPSNN_NOT_TAKEN;
+    int nw = 0, nch = 0, splits = 1;
+    if (!xreg_shape(WBITS, p.K, 0, nw, nch, p.M, p.part != nullptr, &splits)) return OPSNN_NOT_TAKEN;
     constexpr int SCM = WBITS == 4 ? 2 : 0;
-    if (nw == 16 && nch == 4) return launch_xreg_one<XDT, WBITS, 16, 4, false, SCM, true>(p, st);
+    if (nw == 16 && nch == 4) return launch_xreg_one<XDT, WBITS, 16, 4, false, SCM, true>(p, st, splits);
     if constexpr (WBITS == 8) {
         if (nw == 16 && nch == 8) return launch_xreg_one<XDT, WBITS, 16, 8, false, SCM, true>(p, st);
     }
-    if (nw == 8 && nch == 4) return launch_xreg_one<XDT, WBITS, 8, 4, false, SCM, true>(p, st);
+    if (nw == 8 && nch == 4) return launch_xreg_one<XDT, WBITS, 8, 4, false, SCM, true>(p, st, splits);
     if (nw == 8 && nch == 8) return launch_xreg_one<XDT, WBITS, 8, 8, false, SCM, true>(p, st);
     return OPSNN_NOT_TAKEN;
 }

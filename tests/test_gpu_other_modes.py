@@ -530,6 +530,17 @@ def test_weight_only_64_column_workgroups(gpu, M, K, N, x_dt, w_dt, group, off, 
     (16, 8192, 96, "bf16", "e4m3", 0, True, False, None),
     (12, 4096, 200, "bf16", "e4m3", 0, True, False, "bf16"),
     (7, 2048, 72, "f16", "e4m3", 0, True, False, None),
+    # a K of several workgroup segments (2 .. 16 of 16 x 4 chunks, else of 8 x 4): one workgroup column per segment, fp32
+    # partial sums in front of the workspace (behind them the re-laid-out weight of the N-contiguous case), a reduce kernel;
+    # one row (x does not fit the LDS of the few-rows kernel at this K)
+    (16, 16384, 256, "f16", "i4", 128, True, True, None),
+    (5, 12288, 100, "bf16", "i4", 128, True, True, "bf16"),
+    (1, 28672, 264, "f16", "i4", 128, True, True, None),
+    (8, 12288, 64, "f16", "i4", 128, False, True, None),
+    (16, 6144, 200, "f16", "i8", 64, True, True, "f16"),
+    (9, 16384, 64, "bf16", "i8", 0, True, False, None),
+    (16, 16384, 256, "f16", "fp4", 32, True, False, None),
+    (12, 6144, 200, "bf16", "e4m3", 0, True, False, "bf16"),
 ])
 def test_weight_only_x_in_registers_kernel(gpu, M, K, N, x_dt, w_dt, group, tW, off, bias):
     """4 .. 16 rows of x (floating-point weight codes: 1 .. 16) with K in 8 or 16 equal ranges of whole chunks: the kernel
