@@ -68,18 +68,35 @@ inline int splitk_factor(int64_t tiles, int64_t ktiles, double tile_us, int64_t 
     }
     return best;
 }
-// Weight-only calls with up to 16 rows of x and a K longer than one workgroup of the x-in-registers kernel holds (16 waves x
-// 4 chunks, i.e. 64 chunks of 64 weight bytes; 8-bit weights also 128; or 8 waves x 4 or 8 chunks): K in 2 .. 16 equal
-// segments of 64 chunks (else of 32), one workgroup column per segment, fp32 partial sums [segments][M][N] at the front of
-// the workspace.  1: no split (K fits one workgroup, or is not a whole number of segments).
-inline int wq_xreg_splits(int wbits, int64_t M, int64_t K)
+// How the x-in-registers kernel (weight-only, up to 16 rows of x) covers K.  A workgroup holds `nw` waves x `nch` chunks
+// (of 64 weight bytes): 16 x 4, 8-bit weights also 16 x 8, or 8 x 4 / 8 x 8.  A K that is exactly one such shape runs on
+// one workgroup per row block range; any other K of whole 128-element units goes in `splits` segments of 16 x 4 chunks
+// (else of 8 x 4), one workgroup column per segment, the last one with idle chunks past the end of K (`exact` false) when
+// that wastes at most a sixth of K's chunks; with more than one segment the columns leave fp32 partial sums
+// [splits][M][N] at the front of the workspace.  False: the kernel does not take this K.
+struct WqXregPlan {
+    int nw, nch, splits;
+    bool exact;
+};
+inline bool wq_xreg_plan(int wbits, int64_t M, int64_t K, WqXregPlan& pl)
 {
     const int64_t kc = 4 * (128 / wbits);
-    if (M < 1 || M > 16 || K % (32 * kc) != 0) return 1;
-    const int64_t c32 = K / (32 * kc);
-    if (c32 == 1 || c32 == 2 || (wbits == 8 && c32 == 4)) return 1;   // one workgroup
-    if (c32 % 2 == 0 && c32 / 2 <= 16) return (int)(c32 / 2);
-    return c32 <= 16 ? (int)c32 : 1;
+    if (M < 1 || M > 16 || K < 128 || K % 128 != 0) return false;
+    const int64_t nch = K / kc;
+    if (nch == 64) { pl = {16, 4, 1, true}; return true; }
+    if (wbits == 8 && nch == 128) { pl = {16, 8, 1, true}; return true; }
+    if (nch == 32) { pl = {8, 4, 1, true}; return true; }
+    const int64_t s64 = (nch + 63) / 64, w64 = s64 * 64 - nch, s32 = (nch + 31) / 32, w32 = s32 * 32 - nch;
+    if (s64 == 1 && w64 * 6 <= nch) { pl = {16, 4, 1, false}; return true; }   // one workgroup, its last waves idle
+    if (s32 <= 16 && w32 * 6 <= nch) { pl = {8, 4, (int)s32, w32 == 0}; return true; }
+    if (s64 <= 16 && w64 * 6 <= nch) { pl = {16, 4, (int)s64, w64 == 0}; return true; }
+    return false;
+}
+// the count of partial-sum slices that plan needs (0: none)
+inline int wq_xreg_splits(int wbits, int64_t M, int64_t K)
+{
+    WqXregPlan pl;
+    return (wq_xreg_plan(wbits, M, K, pl) && pl.splits > 1) ? pl.splits : 1;
 }
 // Opened by every exported matmul entry point for the time it enqueues its launches (weight_cache.hip): copies that the
 // weight cache hands out inside the scope cannot be evicted before it closes; bypass = true switches the cache off for

@@ -331,8 +331,9 @@ static bool stream_eligible(WqParams& p, WqStreamOpts& o)
     o.xreg_nw = xreg_nw;
     // (with room for partial sums also a K of several workgroup segments, and then fewer than 4 rows too where x does not fit the LDS)
     int xsplits = 1;
-    o.xreg = p.M <= 16 && xreg_shape(WBITS, p.K, xreg_nw, xnw, xnch, p.M, p.part != nullptr, &xsplits) && (p.M >= xreg_min || (xsplits > 1 && !o.resx));
-    o.xreg_vscale = o.xreg && p.group == KC && p.s_rs == 1 && p.s_cs % 8 == 0 &&
+    bool xexact = true;
+    o.xreg = p.M <= 16 && xreg_shape(WBITS, p.K, xreg_nw, xnw, xnch, p.M, p.part != nullptr, &xsplits, &xexact) && (p.M >= xreg_min || (xsplits > 1 && !o.resx));
+    o.xreg_vscale = o.xreg && xexact && p.group == KC && p.s_rs == 1 && p.s_cs % 8 == 0 &&
                     (uintptr_t)p.scale % 16 == 0 && (!p.offset || (uintptr_t)p.offset % 16 == 0);
     // more than 48 rows: two weight blocks per wave share every x fragment, up to 128 rows per pass over the weights
     // (needs whole groups of chunks in flight and whole wave tiles of columns)

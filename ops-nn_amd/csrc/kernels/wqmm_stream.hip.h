@@ -1135,6 +1135,10 @@ __global__ __launch_bounds__(NW * 64) void wqmm_xreg_kernel(WqParams p)
     // blockIdx.y-th run of NW * NCH chunks
     const int cbase = ((int)blockIdx.y * NW + wave) * NCH;
     const int nblocks = (int)((p.N + 15) / 16);
+    // chunks of this wave that lie inside K (the last segment of a K that is no whole number of segments has idle chunks:
+    // their weights are fetched from the row's last chunk instead and nothing is multiplied)
+    const int nlive = (int)(p.K / KC) - cbase;
+    auto chunk_at = [&](int c) { return c < nlive ? c : (nlive > 0 ? nlive - 1 : -cbase); };   // (a wave with no live chunk reloads the row's first one)
 
     auto row_of = [&](int rb) { const int64_t n = (int64_t)rb * 16 + nrow; return n < p.N ? n : p.N - 1; };
     auto wptr_of = [&](int rb) { return p.w + row_of(rb) * p.ldw + g * 16 + (int64_t)cbase * 64; };
@@ -1183,7 +1187,8 @@ __global__ __launch_bounds__(NW * 64) void wqmm_xreg_kernel(WqParams p)
     if constexpr (VSCALE || MXS) load_scales(srow, orow, svn, ovn);
     v4i wq[PF];
     uint16_t sq[PF], oq[PF];
-    auto fetch = [&](int j, const uint8_t* wp, const uint16_t* sr, const uint16_t* orw, int cw) {
+    auto fetch = [&](int j, const uint8_t* wp, const uint16_t* sr, const uint16_t* orw, int cw0) {
+        const int cw = chunk_at(cw0);
         wq[j] = *(const v4i*)(wp + (int64_t)cw * 64);
         if constexpr (SCM == 0) {
             const int64_t so = (int64_t)((cbase + cw) >> p.cpg_shift) * p.s_rs;
@@ -1212,7 +1217,7 @@ __global__ __launch_bounds__(NW * 64) void wqmm_xreg_kernel(WqParams p)
             for (int ul = 0; ul < HU; ul++) {
 #pragma unroll
                 for (int q = 0; q < 4; q++) {
-                    if (4 * q < rows) {
+                    if (4 * q < rows && (int64_t)cbase * KC + (r * HU + ul) * 128 < p.K) {   // (units past the end of K stay unread and unused)
                         const int m = 4 * q + cm;
                         const int mm = m < rows ? m : rows - 1;
                         async_copy16(xw + (int64_t)mm * p.K + (r * HU + ul) * 128 + ((cp ^ m) << 3), stage + ul * 4096 + q * 1024);
@@ -1270,6 +1275,7 @@ __global__ __launch_bounds__(NW * 64) void wqmm_xreg_kernel(WqParams p)
                 sb = sq[j];
                 if constexpr (HAS_OFF) ob = oq[j];
             }
+            if (c < nlive) {
 #pragma unroll
             for (int s = 0; s < STEPS; s++) {
                 v4i aop;
@@ -1280,6 +1286,7 @@ __global__ __launch_bounds__(NW * 64) void wqmm_xreg_kernel(WqParams p)
                 } else {
                     acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf, aop), __builtin_bit_cast(v8bf, xr[c * STEPS + s]), acc, 0, 0, 0);
                 }
+            }
             }
             if (c + PF < NCH) fetch(j, wptr, srow, orow, c + PF);
             else fetch(j, wptr_n, srow_n, orow_n, c + PF - NCH);
@@ -1380,7 +1387,11 @@ static int launch_xreg_one(const WqParams& p, hipStream_t st, int splits = 1)
     }
     const int64_t nblocks = (p.N + 15) / 16;
     if (splits < 1 || splits > 16 || (splits > 1 && (!p.part || p.m_base != 0 || p.m_rows != p.M))) return -1;
-    if ((int64_t)splits * NW * NCH * (4 * (128 / WBITS)) != p.K) return -1;
+    {   // the segments cover K, the last one with idle chunks worth at most a sixth of K; vector scale loads only for whole segments
+        const int64_t kc = 4 * (128 / WBITS), nch = p.K / kc, cover = (int64_t)splits * NW * NCH;
+        if (p.K % 128 != 0 || cover < nch || (cover - nch) * 6 > nch || cover - nch >= (int64_t)NW * NCH) return -1;
+        if (cover != nch && SCM != 0) return -1;
+    }
     const int64_t g = ((int64_t)resx_grid(1ll << 40) / (TWO ? 1 : 2) + splits - 1) / splits;   // (resx_grid: two per CU)
     constexpr int STEPS = (4 * (128 / WBITS)) / 32;
     constexpr int NU = NCH * STEPS / 4;                  // units of 16 rows x 256 bytes per wave
@@ -1409,31 +1420,29 @@ static int launch_xreg_nch(const WqParams& p, bool has_off, bool vscale, hipStre
 }
 
 // K = waves x chunks per wave x chunk.  Sixteen waves with 4 chunks each (8-bit weights: or 8), else eight waves with 4 or 8.
-// With room for partial sums (`may_split`) a longer K goes in `splits` segments of 16 x 4 chunks, else of 8 x 4
-// (wq_xreg_splits in launch.h names the count: the workspace query uses the same function).
-static inline bool xreg_shape(int wbits, int64_t K, int force_nw, int& nw, int& nch, int64_t M = 1, bool may_split = false, int* splits = nullptr)
+// The plan of wq_xreg_plan (launch.h; the workspace query uses the same function); force_nw == 8 keeps a K of 64 chunks
+// on eight waves x eight chunks.  With more than one segment the call needs room for partial sums (`may_split`).
+static inline bool xreg_shape(int wbits, int64_t K, int force_nw, int& nw, int& nch, int64_t M = 1, bool may_split = false, int* splits = nullptr,
+                              bool* exact = nullptr)
 {
-    const int64_t kc = 4 * (128 / wbits);
-    if (splits) *splits = 1;
-    if (K % (32 * kc) != 0) return false;
-    const int64_t c16 = K / (16 * kc), c8 = K / (8 * kc);
-    if (force_nw != 8 && K % (64 * kc) == 0 && (c16 == 4 || (wbits == 8 && c16 == 8))) { nw = 16; nch = (int)c16; return true; }
-    if (c8 == 4 || c8 == 8) { nw = 8; nch = (int)c8; return true; }
-    const int s = (may_split && splits) ? wq_xreg_splits(wbits, M, K) : 1;
-    if (s > 1) {
-        *splits = s;
-        nch = 4;
-        nw = (K / s == 64 * kc) ? 16 : 8;
-        return true;
-    }
-    return false;
+    WqXregPlan pl;
+    if (!wq_xreg_plan(wbits, M, K, pl)) return false;
+    if (pl.splits > 1 && !(may_split && splits)) return false;
+    if (!pl.exact && !exact) return false;
+    if (force_nw == 8 && pl.splits == 1 && pl.exact && pl.nw == 16 && pl.nch == 4) pl = {8, 8, 1, true};
+    nw = pl.nw; nch = pl.nch;
+    if (splits) *splits = pl.splits;
+    if (exact) *exact = pl.exact;
+    return true;
 }
 
 template <int XDT, int WBITS>
 static int launch_xreg(const WqParams& p, bool has_off, bool vscale, int force_nw, hipStream_t st)
 {
     int nw = 0, nch = 0, splits = 1;
-    if (!xreg_shape(WBITS, p.K, force_nw, nw, nch, p.M, p.part != nullptr, &splits)) return OPSNN_NOT_TAKEN;
+    bool exact = true;
+    if (!xreg_shape(WBITS, p.K, force_nw, nw, nch, p.M, p.part != nullptr, &splits, &exact)) return OPSNN_NOT_TAKEN;
+    if (!exact) vscale = false;   // (vector scale loads would read past the row's last scale)
     if (nw == 16 && nch == 4) return launch_xreg_nch<XDT, WBITS, 16, 4>(p, has_off, vscale, st, splits);
     if constexpr (WBITS == 8) {
         if (nw == 16 && nch == 8) return launch_xreg_nch<XDT, WBITS, 16, 8>(p, has_off, vscale, st);

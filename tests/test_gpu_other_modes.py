@@ -541,6 +541,16 @@ def test_weight_only_64_column_workgroups(gpu, M, K, N, x_dt, w_dt, group, off, 
     (9, 16384, 64, "bf16", "i8", 0, True, False, None),
     (16, 16384, 256, "f16", "fp4", 32, True, False, None),
     (12, 6144, 200, "bf16", "e4m3", 0, True, False, "bf16"),
+    # a K that is no whole number of segments (integer codes): the last segment's waves past the end of K stay idle --
+    # 14336 = 2 x 8192 - 2048, 11008 = 3 x 4096 - 1280, 28672 = 4 x 8192 - 4096, 7168 = 8192 - 1024 in one workgroup;
+    # int8: 7168 = 2 x 4096 - 1024; the last weight row's reads stay inside the row (N = 16: one row block)
+    (16, 14336, 256, "f16", "i4", 128, True, True, None),
+    (7, 11008, 100, "bf16", "i4", 128, True, False, "bf16"),
+    (16, 28672, 64, "f16", "i4", 128, True, True, None),
+    (16, 7168, 16, "f16", "i4", 128, True, True, "f16"),
+    (16, 7168, 200, "bf16", "i8", 128, True, True, None),
+    (4, 14336, 48, "f16", "i4", 0, True, False, None),
+    (2, 14336, 72, "f16", "i4", 256, False, True, None),
 ])
 def test_weight_only_x_in_registers_kernel(gpu, M, K, N, x_dt, w_dt, group, tW, off, bias):
     """4 .. 16 rows of x (floating-point weight codes: 1 .. 16) with K in 8 or 16 equal ranges of whole chunks: the kernel
