@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the quantized-matmul hot path on one MI355X.
 
-  python bench.py [--gpus 1] [--steps K] [--warmup W] [--config 1..11] [--m M] [--cold] [--fp8-fast] [--no-cpu] [--calib-copy] [--layout packed|nd] [--weight-cache MB]
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--config 1..14] [--shape M,K,N] [--m M] [--cold] [--fp8-fast] [--no-cpu] [--calib-copy] [--layout packed|nd] [--weight-cache MB]
 
 A step is one pass of the operator (both aclnn phases) over one batch of synthetic, seeded input that is already
 resident in HBM.  One JSON line is printed.
@@ -96,6 +96,9 @@ def main():
                          "11: config 3's shape with mxfp4 weights; 12: config 4's operator with the --m rows of a decode step; "
                          "13 / 14: the fp8 x fp4 MX mode / the int8 per-tile mode at config 3's K and N with the --m rows of a decode step")
     ap.add_argument("--m", type=int, default=None, help="M for config 3 (1, 16, 64 or 256) and configs 11 to 14 (default 16)")
+    ap.add_argument("--shape", default=None, metavar="M,K,N",
+                    help="configs 2, 4 and 5 (one batch) at another shape, e.g. --config 4 --shape 512,7168,2048: the mid-size "
+                         "calls whose few tiles split K (not a BASELINE workload; the record says so)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--int8-range", type=int, default=None,
                     help="config 2: operands uniform in [-R, R] (default: the full int8 range, the most power-hungry data)")

@@ -593,6 +593,13 @@ def make_workload(m, config, args):
         return ConfigWQ(m, args, config)
     if config == 10:
         return ConfigKG(m, args)
+    shape = getattr(args, "shape", None)
+    if shape and config in (2, 4, 5):   # the same operator at another shape (not the BASELINE workload)
+        M, K, N = (int(v) for v in shape.split(","))
+        wl = Config2(m, args, M, K, N) if config == 2 else Config4(m, args, M, K, N) if config == 4 else Config5(m, args, 1, M, K, N)
+        wl.kernel = "the selector's choice for this shape (tile kernel, with a K split where the tiles are few)"
+        wl.config = dict(wl.config, workload=wl.config["workload"].split(":")[-1].strip() + f" at {M} x {K} x {N} (not a BASELINE shape)")
+        return wl
     if config == 2:
         return Config2(m, args)
     if config == 4:
