@@ -14,6 +14,8 @@ pytestmark = pytest.mark.gpu
     ((2, 1), (1, 3), 128, 256, 192),      # both operands broadcast, on different dims
     ((2, 3), (3,), 64, 128, 64),          # x2 has fewer batch dims and is reused for every outer index
     ((1, 2), (4, 1), 96, 512, 136),
+    ((2,), (2,), 64, 4096, 256),          # equal batches, few tiles against a long K: the K split inside a batched launch
+    ((2, 1), (1, 2), 48, 8192, 136),      # and inside the launches of a broadcast pattern (they share the partial sums' buffer, in stream order)
 ])
 def test_int8_partial_batch_broadcast(gpu, b1, b2, M, K, N):
     m = gpu
@@ -42,10 +44,11 @@ def test_int8_partial_batch_broadcast(gpu, b1, b2, M, K, N):
     assert np.array_equal(got, want)
 
 
-def test_fp8_blockscale_partial_batch_broadcast(gpu):
+@pytest.mark.parametrize("M,K,N", [(128, 256, 256), (256, 2048, 256)])   # (the second: the exact kernel's K split in every launch)
+def test_fp8_blockscale_partial_batch_broadcast(gpu, M, K, N):
     """The scale tables carry their operand's batch dims: they are offset with it."""
     m = gpu
-    b1, b2, M, K, N = (2, 1), (3,), 128, 256, 256
+    b1, b2 = (2, 1), (3,)
     n1, n2 = 2, 3
     inp1 = cases.make_blockscale_inputs(m, M, K, N, 3, True, 1, batch=n1)
     inp2 = cases.make_blockscale_inputs(m, M, K, N, 4, True, 1, batch=n2)
