@@ -17,19 +17,19 @@ import oracle_api as orc
 # be evidence and is reported as null.  Keyed by (config, M of the weight-only configs, variant).
 PROFILED_TRAFFIC = {
     (1, None, "warm"): (20.7e6, "profiles/wqmm_decode_w8a16_m16_k4096_n4096.txt"),
-    (1, None, "cold"): (20.7e6, "profiles/wqmm_decode_w8a16_m16_k4096_n4096_cold.txt"),
+    (1, None, "cold"): (20.5e6, "profiles/wqmm_decode_w8a16_m16_k4096_n4096_cold.txt"),
     (2, None, None): (162.5e6, "profiles/qgemm_int8_w8a8_m2048_k4096_n11008.txt"),
     (3, 1, "warm"): (144.0e6, "profiles/wqmm_decode_w4a16_m1_k8192_n28672.txt"),
     (3, 1, "cold"): (140.9e6, "profiles/wqmm_decode_w4a16_m1_k8192_n28672_cold.txt"),
-    (3, 16, "warm"): (131.4e6, "profiles/wqmm_decode_w4a16_m16_k8192_n28672.txt"),
-    (3, 16, "cold"): (132.1e6, "profiles/wqmm_decode_w4a16_m16_k8192_n28672_cold.txt"),
+    (3, 16, "warm"): (132.5e6, "profiles/wqmm_decode_w4a16_m16_k8192_n28672.txt"),
+    (3, 16, "cold"): (132.7e6, "profiles/wqmm_decode_w4a16_m16_k8192_n28672_cold.txt"),
     (3, 64, "warm"): (137.8e6, "profiles/wqmm_decode_w4a16_m64_k8192_n28672.txt"),
     (3, 64, "cold"): (137.9e6, "profiles/wqmm_decode_w4a16_m64_k8192_n28672_cold.txt"),
     (3, 256, "warm"): (196.9e6, "profiles/wqmm_decode_w4a16_m256_k8192_n28672.txt"),
     (3, 256, "cold"): (193.0e6, "profiles/wqmm_decode_w4a16_m256_k8192_n28672_cold.txt"),
-    (4, None, "exact"): (1220.4e6, "profiles/qmm_fp8_exact_m4096_k7168_n18432.txt"),
-    (4, None, "fast"): (1502.4e6, "profiles/qmm_fp8_block_m4096_k7168_n18432.txt"),
-    (5, None, None): (2229.0e6, "profiles/qgemm_mxfp4_b8_m4096_k8192_n8192.txt"),
+    (4, None, "exact"): (1220.1e6, "profiles/qmm_fp8_exact_m4096_k7168_n18432.txt"),
+    (4, None, "fast"): (1502.5e6, "profiles/qmm_fp8_block_m4096_k7168_n18432.txt"),
+    (5, None, None): (2229.7e6, "profiles/qgemm_mxfp4_b8_m4096_k8192_n8192.txt"),
     (6, None, None): (1052.7e6, "profiles/pack_b4_k8192_n28672.txt"),
     (7, None, None): (199.4e6, "profiles/dynamic_quant_int8_16384x4096.txt"),
     (8, None, None): (392.1e6, "profiles/block_quant_e4m3_128x128_18432x7168.txt"),
@@ -40,7 +40,7 @@ PROFILED_TRAFFIC = {
     (12, 128, "exact"): (154.8e6, "profiles/qmm_fp8_block_rows_m128_k7168_n18432.txt"),
     (13, 16, None): (131.0e6, "profiles/qmm_mx_a8w4_decode_m16_k8192_n28672.txt"),
     (14, 16, None): (244.0e6, "profiles/qmm_i8_pertile_decode_m16_k8192_n28672.txt"),
-    (11, 16, "warm"): (133.6e6, "profiles/wqmm_decode_mxfp4_m16_k8192_n28672.txt"),
+    (11, 16, "warm"): (133.5e6, "profiles/wqmm_decode_mxfp4_m16_k8192_n28672.txt"),
 }
 
 
