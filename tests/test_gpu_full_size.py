@@ -139,6 +139,51 @@ def test_fp8_fp4_mx_large(gpu, M, K, N):
 
 
 # ---- the operators that prepare the configs' tensors, at the configs' sizes (bit-identical to the oracle) ----
+# ---- model-size shapes off the BASELINE list, whose routes differ from the configs': few tiles against a long K (the K
+# split), narrow weights (row slabs in one launch, 64-column workgroups), down-projection shapes of the weight-only
+# operator (K segments of the x-in-registers kernel, a K that is no whole number of them) ----
+@pytest.mark.parametrize("M,K,N", [(512, 7168, 2048), (256, 8192, 1024)])
+def test_fp8_block_scale_k_split_at_model_sizes(gpu, M, K, N):
+    m = gpu
+    print(f"case fp8 block scale, K split, {M}x{K}x{N}", flush=True)
+    inp = cases.make_blockscale_inputs(m, M, K, N, 1, True, 1)
+    got = cases.run_blockscale_aclnn(m, inp, M, K, N, True, m.ACL_BF16)
+    rows = _rows(M, 12, 7)
+    want = cases.oracle_blockscale(m, inp, M, K, N, True, m.ACL_BF16, rows=rows)
+    check_close(got[0][rows], want[0], m.ACL_BF16, "fp8 block scale with a K split")
+    assert np.array_equal(cases.run_blockscale_aclnn(m, inp, M, K, N, True, m.ACL_BF16), got), "two runs of the same call differ"
+    inp2 = dict(inp, s1=inp["s1"] * np.float32(2.0))
+    _double_exactly(got, cases.run_blockscale_aclnn(m, inp2, M, K, N, True, m.ACL_BF16), m.ACL_BF16)
+
+
+@pytest.mark.parametrize("M,K,N", [(64, 8192, 4096), (16, 14336, 4096)])
+def test_int8_k_split_at_model_sizes_is_bit_identical(gpu, M, K, N):
+    m = gpu
+    print(f"case int8 K-C, K split, {M}x{K}x{N}", flush=True)
+    got, want, _ = cases.run_qmm_int8_case(m, orc, M, K, N, seed=11, out_dtype=m.ACL_BF16, bias_dtype=m.ACL_BF16, transpose_x2=True)
+    assert np.array_equal(got, want), f"{int((got != want).sum())} of {got.size} outputs differ"
+
+
+@pytest.mark.parametrize("M,K,N,w_dt,group,off", [
+    (16, 28672, 8192, "i4", 128, True),      # seven K segments of the x-in-registers kernel
+    (16, 14336, 4096, "i4", 128, True),      # four, the last one a quarter idle
+    (1, 11008, 4096, "i4", 128, False),      # three, one row
+    (16, 7168, 18432, "i8", 0, False),       # 8-bit weights: two segments, the last one a quarter idle
+    (512, 4096, 4096, "i4", 128, True),      # narrow weight: eight row slabs of 64 rows in one launch
+    (64, 8192, 8192, "i4", 128, True),       # 64-column workgroups
+    (200, 4096, 14336, "fp4", 32, False),    # mxfp4: row slabs, the e8m0 table in LDS
+])
+def test_weight_only_at_model_sizes_off_the_configs(gpu, M, K, N, w_dt, group, off):
+    m = gpu
+    dt = {"i4": m.ACL_INT4, "i8": m.ACL_INT8, "fp4": m.ACL_FLOAT4_E2M1}
+    print(f"case weight-only {M}x{K}x{N} w={w_dt} g={group} off={off}", flush=True)
+    inp = cases.make_wq_inputs(m, M, K, N, 2, m.ACL_FLOAT16, dt[w_dt], group, True, off, m.ACL_FLOAT16)
+    got = cases.run_wq_aclnn(m, inp, M, K, N)
+    rows = _rows(M, 6, 8)
+    check_close(got[rows], cases.oracle_wq(m, inp, M, K, N, rows=rows), m.ACL_FLOAT16, "weight-only off the configs")
+    assert np.array_equal(cases.run_wq_aclnn(m, inp, M, K, N), got), "two runs of the same call differ"
+
+
 def test_prepack_of_config3_weight_full(gpu):
     """8192 x 28672 int32 carriers -> packed int4: every byte against the oracle, and unpacking returns the carriers' nibbles."""
     m = gpu
