@@ -98,6 +98,48 @@ inline int wq_xreg_splits(int wbits, int64_t M, int64_t K)
     WqXregPlan pl;
     return (wq_xreg_plan(wbits, M, K, pl) && pl.splits > 1) ? pl.splits : 1;
 }
+// Row slabs of the many-rows weight-only kernel for a narrow N.  Its workgroups take 128 columns each, so one pass over a
+// narrow weight leaves most CUs idle, and passes launched one after the other do not overlap (4096 x 4096 int4: 32
+// workgroups, 256 rows 56 us, 1024 rows in four passes 219 us).  With at most 128 workgroups per pass and more than 64
+// rows the rows are cut into equal slabs of 64 .. 256 rows, as many as give every CU a workgroup in one round, and all
+// slabs go out in one launch (grid.y).  Returns the slab's rows, or 0 where the one-pass-at-a-time order stays.
+inline int64_t wq_narrow_slab_rows(int64_t M, int64_t N, bool on)
+{
+    const int64_t wgs = (N + 127) / 128;
+    if (M <= 64 || wgs > 128 || !on) return 0;
+    int64_t n = 256 / wgs;
+    if (n > (M + 63) / 64) n = (M + 63) / 64;
+    if (n < (M + 255) / 256) n = (M + 255) / 256;
+    if (n < 2) return 0;
+    return ((M + n - 1) / n + 15) / 16 * 16;
+}
+// The same kernel, integer codes, from 49 rows: a narrow N leaves CUs without a workgroup even with all row slabs in one
+// launch (64 rows against 28672 x 8192: 64 workgroups of 128 columns), and a long K makes each of them slow.  Then K is
+// cut into segments, one per blockIdx.z, whose fp32 partial sums a second kernel adds in segment order.  Segments are
+// whole rounds of the kernel's chunk pipeline (eight chunks of 128 bytes of a weight row), as equal as that allows, at
+// least 2048 k each, and hold whole groups.  Returns the segment count (1: no split).
+// (Measured, int4 with groups of 128, 64 rows: 14336 x 4096 64 -> 22 us, 28672 x 8192 124 -> 66, 8192 x 8192 30 -> 24; a K
+// of 4096 lost 2 to 6 us to the second kernel, and so did two segments of 128 workgroups at K = 8192.)
+inline int wq_rows_ksplit(int wbits, int64_t M, int64_t N, int64_t K, int64_t group, bool on)
+{
+    if (!on || M < 49 || N % 32 != 0 || N < 256 || K < 8192 || K >= (1ll << 23)) return 1;
+    const int64_t slab = wq_narrow_slab_rows(M, N, on);
+    if (M > 64 && slab == 0) return 1;
+    const int64_t slabs = slab ? (M + slab - 1) / slab : 1;
+    const int64_t wgs = slabs * ((N + 127) / 128), round = 8 * 4 * (128 / wbits);
+    if (wgs > 128 || K % round != 0 || (group < K && round % group != 0)) return 1;
+    int64_t s = 256 / wgs;
+    if (s > 8) s = 8;
+    if (s > K / 2048) s = K / 2048;
+    if (s == 2 && K < 12288) return 1;
+    return s < 2 ? 1 : (int)s;
+}
+// fp32 partial-sum slices [slices][M][N] at the front of a weight-only call's workspace (1: none)
+inline int wq_part_slices(int wbits, bool wint, int64_t M, int64_t N, int64_t K, int64_t group, bool narrow_on)
+{
+    if (M <= 16) return wq_xreg_splits(wbits, M, K);
+    return wint ? wq_rows_ksplit(wbits, M, N, K, group, narrow_on) : 1;
+}
 // Opened by every exported matmul entry point for the time it enqueues its launches (weight_cache.hip): copies that the
 // weight cache hands out inside the scope cannot be evicted before it closes; bypass = true switches the cache off for
 // this thread while the scope is open.  Scopes nest; the pins drop when the outermost one closes.

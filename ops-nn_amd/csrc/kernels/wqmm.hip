@@ -353,11 +353,6 @@ extern "C" int opsnn_wq_tile_min();   // dispatch.hip
 extern "C" int opsnn_wq_narrow_slabs();
 namespace opsnn {
 
-// The many-rows kernel's workgroups take 128 columns each, so one pass over a narrow weight leaves most CUs idle, and
-// passes launched one after the other do not overlap (4096 x 4096 int4: 32 workgroups, 256 rows 56 us, 1024 rows in four
-// passes 219 us).  With at most 128 workgroups per pass and more than 64 rows the rows are cut into equal slabs of 64 ..
-// 256 rows, as many as give every CU a workgroup in one round, and all slabs go out in one launch (grid.y).  Returns the
-// slab's rows, or 0 where the one-pass-at-a-time order stays.
 // Up to 64 rows per slab, `slabs` slabs, and still at most 128 workgroups of 128 columns: the instance whose workgroups
 // take 64 columns (K split over four waves instead of two; needs K in whole groups of 16 chunks) doubles their number.
 template <int WBITS>
@@ -367,16 +362,8 @@ static int use_cols64(int64_t rows, int64_t slabs, int64_t N, int64_t K)
     return (rows <= 64 && slabs * ((N + 127) / 128) <= 128 && K % (16 * KC) == 0 && N % 32 == 0 && opsnn_wq_narrow_slabs()) ? 1 : 0;
 }
 
-static int64_t narrow_n_slab(int64_t M, int64_t N)
-{
-    const int64_t wgs = (N + 127) / 128;
-    if (M <= 64 || wgs > 128 || !opsnn_wq_narrow_slabs()) return 0;
-    int64_t n = 256 / wgs;
-    if (n > (M + 63) / 64) n = (M + 63) / 64;
-    if (n < (M + 255) / 256) n = (M + 255) / 256;
-    if (n < 2) return 0;
-    return ((M + n - 1) / n + 15) / 16 * 16;
-}
+// rows per slab of a narrow weight's one-launch form (0: one pass at a time)
+static int64_t narrow_n_slab(int64_t M, int64_t N) { return wq_narrow_slab_rows(M, N, opsnn_wq_narrow_slabs() != 0); }
 
 // floating-point weight codes: the general kernel, in row slabs of 64
 template <int XDT, int WBITS>
@@ -443,6 +430,20 @@ static int launch_slabs(WqParams p, hipStream_t st)
     // slabs of up to 256 rows; then the tile kernel.  (Measured on 8192 x 28672 int4, fp16: 256 rows 151-155 us against 170 on
     // the tile kernel, 192 rows 142-149 against 168.  Test hook: opsnnSetWqTileMin(m <= 128) sends such calls to the tile
     // kernel first.)
+    // narrow N against a long K, integer codes, from 49 rows: the row slabs in one launch and K in segments on top
+    if (p.part && opsnn_wq_tile_min() > 128) {
+        const int64_t slab = p.M <= 64 ? 0 : narrow_n_slab(p.M, p.N);
+        const int ks = wq_rows_ksplit(WBITS, p.M, p.N, p.K, p.group, opsnn_wq_narrow_slabs() != 0);
+        WqParams q = p;
+        WqStreamOpts o{};
+        if (ks > 1 && (p.M <= 64 || slab > 0) && stream_eligible<WBITS>(q, o) && o.rows) {
+            q.m_base = 0; q.m_rows = q.M;
+            if (slab > 0) { q.m_rows = slab; q.m_slab = slab; q.m_end = q.M; }
+            q.ksplit = ks;
+            const int rc = launch_wq_stream<XDT, WBITS>(q, o, st);
+            if (rc != OPSNN_NOT_TAKEN) return rc;
+        }
+    }
     if (opsnn_wq_tile_min() > 128) {
         if (const int64_t slab = narrow_n_slab(p.M, p.N)) {   // narrow N: all row slabs in one launch
             WqParams q = p;
@@ -532,8 +533,9 @@ int launch_wqmm_mfma(const OpsnnWqmmArgs& a0, hipStream_t st)
     if (a.w_dtype == DT_E2M1 && a.offset) return OPSNN_NOT_TAKEN;   // the packed e2m1 dequantisation has no offset step
     const int wbits = (a.w_dtype == DT_I4 || a.w_dtype == DT_E2M1) ? 4 : 8;
     // up to 16 rows against a long K: the partial sums of the x-in-registers kernel's K split sit at the front of the workspace
+    // (and those of the many-rows kernel's K split, from 49 rows of integer codes against a narrow N)
     float* part = nullptr;
-    if (const int xs = wq_xreg_splits(wbits, a.M, a.K); xs > 1 && a.workspace) {
+    if (const int xs = wq_part_slices(wbits, !wflt, a.M, a.N, a.K, a.group > 0 ? a.group : a.K, opsnn_wq_narrow_slabs() != 0); xs > 1 && a.workspace) {
         part = (float*)a.workspace;
         const uint64_t pb = ((uint64_t)xs * (uint64_t)a.M * (uint64_t)a.N * 4 + 255) / 256 * 256;
         const bool relayout = a.w.row_stride != 1 && a.K != 1;

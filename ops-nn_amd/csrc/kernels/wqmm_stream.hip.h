@@ -463,6 +463,27 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void w
     static_assert((16 * MB * XPR) % NT == 0 && XPR >= 16 && PF >= 2 && PPH >= 1 && STEPS == PPH * XH, "staging and prefetch shape");
     static_assert(MB <= 8 || (WF == 0 && SLDS) || WF == 1 || WF == 2, "the 192- / 256-row instances: integer codes with the scale table in LDS, or floating-point codes");
     static_assert(!(SLDS && WF == 2 && MB > 8) || WK == 2, "8-byte pieces: byte position of a lane's e8m0 scale inside the table word");
+    // K in segments: this workgroup's is number blockIdx.z.  Segments are whole rounds of the chunk pipeline (ROUND k), as
+    // equal as that allows, the longer ones first.  From here on p.K is the segment's length and x, w, the scales and
+    // offsets start at the segment; a row of x keeps its pitch ldx.
+    const int64_t ldx = p.K;
+    const bool ksplit = p.ksplit > 1;
+    if constexpr (WF <= 2) {
+        if (ksplit) {
+            constexpr int ROUND = KX * PF;
+            const int z = (int)blockIdx.z, rounds = (int)(p.K / ROUND), base = rounds / p.ksplit, rem = rounds % p.ksplit;
+            const int64_t k0 = (int64_t)(z * base + (z < rem ? z : rem)) * ROUND;
+            p.x += k0;
+            p.w += k0 * WBITS / 8;
+            if constexpr (WF == 2) p.scale = (const uint16_t*)((const uint8_t*)p.scale + k0 / 32);   // one e8m0 byte per 32 k
+            else if (p.group < p.K) {
+                const int64_t g0 = (k0 / p.group) * p.s_rs;
+                p.scale += g0;
+                if constexpr (HAS_OFF) p.offset += g0;
+            }
+            p.K = (int64_t)(base + (z < rem ? 1 : 0)) * ROUND;
+        }
+    }
     extern __shared__ __attribute__((aligned(16))) char sx[];
 
     const int tid = threadIdx.x, lane = tid & 63;
@@ -503,7 +524,8 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void w
     constexpr bool XLIN = XPR == 16;
     uint32_t xsrc[XLIN ? 1 : XITEMS];
     uint32_t xsrc_max = 0;
-    const uint16_t* xbase = p.x + p.m_base * p.K;
+    const uint16_t* xbase = p.x + p.m_base * ldx;
+    const uint32_t xpitch = (uint32_t)ldx;
     (void)xsrc_max;
 #pragma unroll
     for (int it = 0; it < (XLIN ? 1 : XITEMS); it++) {
@@ -514,15 +536,15 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void w
         // that is piece wk * (KC / 8) + g * (KPL / 8) + step of the chunk (the identity when a slab holds whole chunks)
         const int q = piece_of_pos(pos ^ (r & 15));
         const int src_piece = (q / (XPR / WK)) * (KC / 8) + ((q % (XPR / WK)) / PPH) * (KPL / 8) + q % PPH;
-        xsrc[it] = (uint32_t)(rr * Ki + src_piece * 8) * 2u;
+        xsrc[it] = ((uint32_t)rr * xpitch + (uint32_t)(src_piece * 8)) * 2u;
         if constexpr (XLIN) {
-            xsrc[0] = (uint32_t)(r * Ki + src_piece * 8) * 2u;   // (r may lie past the last row: the minimum below puts it back)
-            xsrc_max = (uint32_t)((rows - 1) * Ki + src_piece * 8) * 2u;
+            xsrc[0] = ((uint32_t)r * xpitch + (uint32_t)(src_piece * 8)) * 2u;   // (r may lie past the last row: the minimum below puts it back)
+            xsrc_max = ((uint32_t)(rows - 1) * xpitch + (uint32_t)(src_piece * 8)) * 2u;
         }
     }
     auto xsrc_at = [&](int it) -> uint32_t {
         if constexpr (XLIN) {
-            const uint32_t o = xsrc[0] + (uint32_t)it * (uint32_t)(NT / XPR) * (uint32_t)Ki * 2u;
+            const uint32_t o = xsrc[0] + (uint32_t)it * (uint32_t)(NT / XPR) * xpitch * 2u;
             return o < xsrc_max ? o : xsrc_max;
         } else {
             return xsrc[it];
@@ -575,14 +597,15 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void w
         }
     }
 
-    // SLDS: word (row rw of the workgroup's 16 NB WN columns, group gi) at stab[rw * G + (gi ^ swizzle(rw))], G = groups per
-    // row; the swizzle (4 * (rw % 16), kept below G) spreads the 16 rows that one read touches over the banks.  The table is
-    // complete behind the loop's first barrier.
+    // SLDS: word (row rw of the workgroup's 16 NB WN columns, group gi) at stab[rw * P + (gi ^ swizzle(rw))], P = the power of
+    // two at or above the groups per row; the swizzle (4 * (rw % 16), kept below P) spreads the 16 rows that one read touches
+    // over the banks.  The table is complete behind the loop's first barrier.
     uint32_t* stab = (uint32_t*)(sx + LDS_MAIN);
-    const int sG = p.cpg_shift >= 31 ? 1 : (int)((p.K / KCH) >> p.cpg_shift);
+    const int sG = p.cpg_shift >= 31 ? 1 : (int)((p.K / KCH) >> p.cpg_shift);   // groups of this workgroup's K
+    const int sP = sG <= 1 ? 1 : 1 << (32 - __builtin_clz((unsigned)(sG - 1)));    // a table row's pitch: the power of two at or above
     const int cpg_shift = p.cpg_shift >= 31 ? 31 : p.cpg_shift + (HP ? 1 : 0);   // chunks of this kernel per group
     int stab_row[NB], stab_sw[NB];
-    (void)stab; (void)sG; (void)stab_row; (void)stab_sw;
+    (void)stab; (void)sG; (void)sP; (void)stab_row; (void)stab_sw;
     if constexpr (SLDS) {
         constexpr int RW = 16 * NB * WN;
         for (int i = tid; i < RW * sG; i += NT) {
@@ -594,13 +617,13 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void w
             if constexpr (WF == 2) w = *(const uint32_t*)((const uint8_t*)p.scale + n * p.s_cs + 4 * gi);   // four e8m0 bytes: 128 k
             else w = p.scale[n * p.s_cs + gi];
             if constexpr (HAS_OFF) w |= (uint32_t)p.offset[n * p.s_cs + gi] << 16;
-            stab[rw * sG + (gi ^ (((rw & 15) << 2) & (sG - 1)))] = w;
+            stab[rw * sP + (gi ^ (((rw & 15) << 2) & (sP - 1)))] = w;
         }
 #pragma unroll
         for (int q = 0; q < NB; q++) {
             const int rw = wn * (16 * NB) + 16 * q + nrow;
-            stab_row[q] = rw * sG;
-            stab_sw[q] = ((rw & 15) << 2) & (sG - 1);
+            stab_row[q] = rw * sP;
+            stab_sw[q] = ((rw & 15) << 2) & (sP - 1);
         }
     }
 
@@ -883,6 +906,12 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void w
             if (r >= rows) continue;
             const int64_t m = p.m_base + r;
             const int64_t nn0 = n0 + 16 * q + 4 * g;
+            if constexpr (WF <= 2) {
+                if (ksplit) {   // this segment's partial sums; bias and rounding follow in the kernel that adds the segments
+                    *(v4f*)(p.part + ((int64_t)blockIdx.z * p.M + m) * p.N + nn0) = acc[q][b];
+                    continue;
+                }
+            }
             float v[4];
 #pragma unroll
             for (int i = 0; i < 4; i++) {
@@ -1496,19 +1525,33 @@ static int launch_rows_one(const WqParams& p, hipStream_t st)
     constexpr int XH = (MB > 8 && WBITS == 4) ? 2 : 1;   // as in the kernel: 8-byte weight pieces, i.e. slabs of half the K, for more than 128 rows of x with 4-bit weights
     constexpr size_t lds_x = 2 * (size_t)(16 * MB) * (WK * KC * 2 / XH);
     size_t lds_stab = 0;
+    const bool split = p.ksplit > 1;
+    // (a split launch covers all rows: the kernel that adds the segments walks the whole output)
+    if (split && (WF > 2 || !p.part || p.ksplit > 64 || p.m_base != 0 || (p.m_slab > 0 ? p.m_end : p.m_rows) != p.M)) return -1;
+    // the longest K one workgroup walks: segments are whole rounds of the kernel's chunk pipeline, as equal as that allows
+    constexpr int64_t ROUND = (int64_t)WK * 4 * (((MB > 8 && WBITS == 4) ? 8 : 16) * 8 / WBITS) * (MB > 8 ? 4 : 8 / NB);
+    int64_t kseg = p.K;
+    if (split) {
+        const int64_t rounds = p.K / ROUND;
+        if (p.K % ROUND != 0 || rounds < p.ksplit || (p.group < p.K && ROUND % p.group != 0)) return -1;   // (a segment holds whole groups)
+        kseg = (rounds + p.ksplit - 1) / p.ksplit * ROUND;
+    }
+    // groups of that K, and the pitch of a scale table row: the power of two at or above
+    const int64_t G = p.cpg_shift >= 31 ? 1 : ((kseg / KC) >> p.cpg_shift);
+    int64_t GP = 1;
+    while (GP < G) GP *= 2;
     if constexpr ((WF == 0 || WF == 2) && !SLDS) {
-        // the scales and offsets of the workgroup's columns in LDS when a row's scales are contiguous, their count per row
-        // is a power of two and the table fits beside the x buffers (e2m1 codes: one word per 128 k, the four e8m0 bytes of
-        // a row read as a word; the caller passes cpg_shift 0)
-        const int64_t G = p.cpg_shift >= 31 ? 1 : ((p.K / KC) >> p.cpg_shift);
+        // the scales and offsets of the workgroup's columns in LDS when a row's scales are contiguous and the table fits
+        // beside the x buffers (e2m1 codes: one word per 128 k, the four e8m0 bytes of a row read as a word; the caller
+        // passes cpg_shift 0)
         const size_t red = (size_t)WN * (WK - 1) * NB * MB * 4 * 64 * 4;
         const bool rows_ok = WF == 2 ? (p.s_cs % 4 == 0 && (uintptr_t)p.scale % 4 == 0 && p.cpg_shift == 0) : (p.s_rs == 1 || G == 1);
-        if (rows_ok && (G & (G - 1)) == 0 && (lds_x > red ? lds_x : red) + (size_t)(16 * NB * WN) * G * 4 <= 160 * 1024)
+        if (rows_ok && (lds_x > red ? lds_x : red) + (size_t)(16 * NB * WN) * GP * 4 <= 160 * 1024)
             return launch_rows_one<XDT, WBITS, MB, NB, WN, WK, HAS_OFF, WF, true>(p, st);
     }
     if constexpr (MB > 8 && WF == 0 && !SLDS) return OPSNN_NOT_TAKEN;   // integer codes: the 192- / 256-row instances exist with the scale table only
     else {
-    if constexpr (SLDS) lds_stab = (size_t)(16 * NB * WN) * (p.cpg_shift >= 31 ? 1 : ((p.K / KC) >> p.cpg_shift)) * 4;
+    if constexpr (SLDS) lds_stab = (size_t)(16 * NB * WN) * GP * 4;
     constexpr size_t lds_red = (size_t)WN * (WK - 1) * NB * MB * 4 * 64 * 4;
     constexpr size_t lds_main = lds_x > lds_red ? lds_x : lds_red;
     constexpr size_t lds_table = WF == 3 ? 65536 : 0;   // products of the block scales: (K / 128) * 16 MB floats, at most this
@@ -1524,8 +1567,15 @@ static int launch_rows_one(const WqParams& p, hipStream_t st)
         if (e != hipSuccess) return (int)e;
         device_flag_set(attr_set);
     }
-    hipLaunchKernelGGL(k, dim3(grid, (unsigned)slabs), dim3(512), lds, st, p);
-    return (int)hipGetLastError();
+    hipLaunchKernelGGL(k, dim3(grid, (unsigned)slabs, split ? (unsigned)p.ksplit : 1u), dim3(512), lds, st, p);
+    if (hipError_t e = hipGetLastError(); e != hipSuccess) return (int)e;
+    if (split) {
+        const int64_t total = p.M * p.N;
+        hipLaunchKernelGGL(wq_splitk_reduce_kernel<XDT>, dim3(splitk_reduce_grid(total)), dim3(256), 0, st, (const float*)p.part, p.ksplit, total, p.N,
+                           p.bias, p.bias_dt, p.y);
+        return (int)hipGetLastError();
+    }
+    return 0;
     }
 }
 

@@ -479,9 +479,9 @@ def test_weight_only_256_row_instance(gpu, M, K, N, x_dt, w_dt, group, tW, off, 
     (64, 2048, 288, "f16", "i4", 128, True, None),
     (49, 4096, 256, "bf16", "i4", 0, False, "bf16"),
     (50, 1024, 320, "f16", "i8", 128, True, None),
-    (64, 3072, 256, "bf16", "i8", 64, True, None),          # 48 groups per row: no scale table
+    (64, 3072, 256, "bf16", "i8", 64, True, None),          # 48 groups per row: table rows of 64 words
     (64, 2048, 256, "bf16", "fp4", 32, False, None),
-    (33, 6144, 288, "f16", "fp4", 32, False, "f16"),        # K / 128 = 48: the e8m0 byte travels with the weight piece
+    (33, 6144, 288, "f16", "fp4", 32, False, "f16"),        # K / 128 = 48: table rows of 64 words
     (33, 1024, 288, "f16", "e4m3", 0, False, None),
     (200, 2048, 512, "f16", "i4", 128, True, "f16"),
     (130, 1024, 256, "bf16", "e4m3", 0, False, None),
@@ -504,6 +504,42 @@ def test_weight_only_64_column_workgroups(gpu, M, K, N, x_dt, w_dt, group, off, 
     finally:
         m.lib().opsnnSetWqNarrowSlabs(1)
     check_close(wide, want, dt[x_dt], "weight-only, 128-column workgroups")
+
+
+@pytest.mark.parametrize("M,K,N,x_dt,w_dt,group,off,bias", [
+    # from 49 rows of integer codes against a narrow N and a K of 8192 or more: K in 2 .. 8 segments over blockIdx.z (whole
+    # rounds of eight chunks -- 1024 k of int4, 512 of int8 --, as equal as that allows, at least 2048 k), partial sums added
+    # by a second kernel; one row slab and several, ragged last workgroup, ragged last slab, unequal segments, group counts
+    # per segment that are no power of two, per-channel scales
+    (64, 8192, 256, "f16", "i4", 128, True, None),            # four segments
+    (49, 8192, 288, "bf16", "i4", 0, False, "bf16"),          # per-channel scale, a last workgroup of 32 columns
+    (100, 8192, 256, "f16", "i8", 128, True, None),           # two slabs of 64 rows (the second with 36)
+    (64, 10240, 256, "bf16", "i8", 64, True, None),           # five segments of four rounds
+    (64, 14336, 256, "f16", "i4", 128, False, "f16"),         # seven segments
+    (64, 11264, 256, "f16", "i4", 512, True, None),           # eleven rounds in five segments (3, 2, 2, 2, 2): six groups or four
+    (200, 8192, 512, "f16", "i4", 128, True, "f16"),          # four slabs
+    (300, 12288, 256, "bf16", "i4", 256, True, None),         # five slabs, six segments
+    (64, 16384, 1024, "f16", "i4", 128, True, None),          # eight workgroups: eight segments
+    (64, 32768, 256, "f16", "i4", 128, True, None),           # (in one piece: 256 groups per row, too many for the scale table)
+])
+def test_weight_only_rows_k_segments(gpu, M, K, N, x_dt, w_dt, group, off, bias):
+    """The many-rows kernel with K split over workgroups against the oracle, the same call without the split
+    (opsnnSetWqNarrowSlabs(0)), and two runs of the split call bit for bit (the segments are added in a fixed order)."""
+    m = gpu
+    dt = {"bf16": m.ACL_BF16, "f16": m.ACL_FLOAT16, "i8": m.ACL_INT8, "i4": m.ACL_INT4, None: None}
+    print(f"case wq rows K segments M={M} K={K} N={N} x={x_dt} w={w_dt} g={group} off={off} bias={bias}", flush=True)
+    inp = cases.make_wq_inputs(m, M, K, N, M * 3 + N, dt[x_dt], dt[w_dt], group, True, off, dt[bias])
+    want = cases.oracle_wq(m, inp, M, K, N)
+    plain(False)
+    got = cases.run_wq_aclnn(m, inp, M, K, N)
+    check_close(got, want, dt[x_dt], "weight-only, K segments")
+    assert np.array_equal(cases.run_wq_aclnn(m, inp, M, K, N), got), "two runs of the same call differ"
+    m.lib().opsnnSetWqNarrowSlabs(0)
+    try:
+        whole = cases.run_wq_aclnn(m, inp, M, K, N)
+    finally:
+        m.lib().opsnnSetWqNarrowSlabs(1)
+    check_close(whole, want, dt[x_dt], "weight-only, K in one piece")
 
 
 @pytest.mark.parametrize("M,K,N,x_dt,w_dt,group,tW,off,bias", [
@@ -587,11 +623,14 @@ def test_weight_only_x_in_registers_kernel(gpu, M, K, N, x_dt, w_dt, group, tW, 
     (256, 8192, 512, "bf16", "fp4", 32, "bf16"),
     (300, 1024, 256, "f16", "fp4", 32, None),
     (712, 2048, 320, "bf16", "fp4", 32, None),
-    # K / 128 not a power of two: no scale table in LDS, a lane's e8m0 byte travels with its weight piece (8-byte pieces at
-    # 129+ rows: two lanes share a byte)
+    # K / 128 not a power of two: the scale table's rows are padded to one
     (100, 3072, 256, "bf16", "fp4", 32, None),
     (256, 3072, 288, "f16", "fp4", 32, "f16"),
     (180, 5120, 256, "bf16", "fp4", 32, None),
+    # a K whose scale table does not fit beside the x buffers: a lane's e8m0 byte travels with its weight piece (8-byte
+    # pieces at 129+ rows: two lanes share a byte)
+    (100, 32768, 256, "bf16", "fp4", 32, None),
+    (256, 12288, 288, "f16", "fp4", 32, "f16"),
     (160, 512, 256, "f16", "e4m3", 0, None),
     (250, 4096, 544, "bf16", "e4m3", 0, "bf16"),
     (256, 1024, 256, "f16", "e4m3", 0, "f16"),
