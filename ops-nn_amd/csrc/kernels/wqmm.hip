@@ -388,13 +388,16 @@ static int launch_slabs_float(WqParams p, hipStream_t st)
         if (WBITS == 4) ok = ok && p.scale_e8m0 && p.group == 32 && p.s_rs == 1;
         else ok = ok && !p.scale_e8m0 && p.group >= p.K;
         if (ok) {
+            // (a long K against few workgroups: K in segments as well, then on 128-column workgroups)
+            const int ks = p.part ? wq_rows_ksplit(WBITS, false, p.M, p.N, p.K, p.group, opsnn_wq_narrow_slabs() != 0) : 1;
+            p.ksplit = ks > 1 ? ks : 0;
             if (const int64_t slab = narrow_n_slab(p.M, p.N)) {   // narrow N: all row slabs in one launch
                 p.cpg_shift = WBITS == 4 ? 0 : 31;
                 p.m_base = 0; p.m_rows = slab; p.m_slab = slab; p.m_end = p.M;
-                p.cols64 = use_cols64<WBITS>(slab, (p.M + slab - 1) / slab, p.N, p.K);
+                p.cols64 = ks > 1 ? 0 : use_cols64<WBITS>(slab, (p.M + slab - 1) / slab, p.N, p.K);
                 return launch_wq_rows_float<XDT, WBITS>(p, st);
             }
-            p.cols64 = use_cols64<WBITS>(p.M, 1, p.N, p.K);
+            p.cols64 = ks > 1 ? 0 : use_cols64<WBITS>(p.M, 1, p.N, p.K);
             // up to 128 rows one pass; more: whole passes of 256 rows and the rest in one (as for integer codes below)
             const int64_t slab = p.M <= 128 ? 128 : 256;
             p.cpg_shift = WBITS == 4 ? 0 : 31;   // (e2m1: the kernel's scale table counts in words of four e8m0 bytes, one per 128 k chunk)
@@ -433,7 +436,7 @@ static int launch_slabs(WqParams p, hipStream_t st)
     // narrow N against a long K, integer codes, from 49 rows: the row slabs in one launch and K in segments on top
     if (p.part && opsnn_wq_tile_min() > 128) {
         const int64_t slab = p.M <= 64 ? 0 : narrow_n_slab(p.M, p.N);
-        const int ks = wq_rows_ksplit(WBITS, p.M, p.N, p.K, p.group, opsnn_wq_narrow_slabs() != 0);
+        const int ks = wq_rows_ksplit(WBITS, true, p.M, p.N, p.K, p.group, opsnn_wq_narrow_slabs() != 0);
         WqParams q = p;
         WqStreamOpts o{};
         if (ks > 1 && (p.M <= 64 || slab > 0) && stream_eligible<WBITS>(q, o) && o.rows) {
@@ -533,7 +536,7 @@ int launch_wqmm_mfma(const OpsnnWqmmArgs& a0, hipStream_t st)
     if (a.w_dtype == DT_E2M1 && a.offset) return OPSNN_NOT_TAKEN;   // the packed e2m1 dequantisation has no offset step
     const int wbits = (a.w_dtype == DT_I4 || a.w_dtype == DT_E2M1) ? 4 : 8;
     // up to 16 rows against a long K: the partial sums of the x-in-registers kernel's K split sit at the front of the workspace
-    // (and those of the many-rows kernel's K split, from 49 rows of integer codes against a narrow N)
+    // (and those of the many-rows kernel's K split against a narrow N)
     float* part = nullptr;
     if (const int xs = wq_part_slices(wbits, !wflt, a.M, a.N, a.K, a.group > 0 ? a.group : a.K, opsnn_wq_narrow_slabs() != 0); xs > 1 && a.workspace) {
         part = (float*)a.workspace;

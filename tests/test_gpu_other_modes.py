@@ -507,7 +507,7 @@ def test_weight_only_64_column_workgroups(gpu, M, K, N, x_dt, w_dt, group, off, 
 
 
 @pytest.mark.parametrize("M,K,N,x_dt,w_dt,group,off,bias", [
-    # from 49 rows of integer codes against a narrow N and a K of 8192 or more: K in 2 .. 8 segments over blockIdx.z (whole
+    # from 49 rows of integer codes (17 of floating-point ones) against a narrow N and a K of 8192 or more: K in 2 .. 8 segments over blockIdx.z (whole
     # rounds of eight chunks -- 1024 k of int4, 512 of int8 --, as equal as that allows, at least 2048 k), partial sums added
     # by a second kernel; one row slab and several, ragged last workgroup, ragged last slab, unequal segments, group counts
     # per segment that are no power of two, per-channel scales
@@ -521,12 +521,19 @@ def test_weight_only_64_column_workgroups(gpu, M, K, N, x_dt, w_dt, group, off, 
     (300, 12288, 256, "bf16", "i4", 256, True, None),         # five slabs, six segments
     (64, 16384, 1024, "f16", "i4", 128, True, None),          # eight workgroups: eight segments
     (64, 32768, 256, "f16", "i4", 128, True, None),           # (in one piece: 256 groups per row, too many for the scale table)
+    # floating-point codes, from 17 rows
+    (17, 8192, 256, "f16", "fp4", 32, False, None),
+    (64, 14336, 288, "bf16", "fp4", 32, False, "bf16"),       # seven segments, a last workgroup of 32 columns
+    (40, 11264, 256, "f16", "e4m3", 0, False, None),          # 22 rounds of 512 in five segments (5, 5, 4, 4, 4)
+    (150, 8192, 256, "bf16", "fp4", 32, False, None),         # three row slabs
+    (100, 9216, 512, "f16", "e4m3", 0, False, "f16"),         # two row slabs, 18 rounds in four segments
 ])
 def test_weight_only_rows_k_segments(gpu, M, K, N, x_dt, w_dt, group, off, bias):
     """The many-rows kernel with K split over workgroups against the oracle, the same call without the split
     (opsnnSetWqNarrowSlabs(0)), and two runs of the split call bit for bit (the segments are added in a fixed order)."""
     m = gpu
-    dt = {"bf16": m.ACL_BF16, "f16": m.ACL_FLOAT16, "i8": m.ACL_INT8, "i4": m.ACL_INT4, None: None}
+    dt = {"bf16": m.ACL_BF16, "f16": m.ACL_FLOAT16, "i8": m.ACL_INT8, "i4": m.ACL_INT4, "e4m3": m.ACL_FLOAT8_E4M3FN,
+          "fp4": m.ACL_FLOAT4_E2M1, None: None}
     print(f"case wq rows K segments M={M} K={K} N={N} x={x_dt} w={w_dt} g={group} off={off} bias={bias}", flush=True)
     inp = cases.make_wq_inputs(m, M, K, N, M * 3 + N, dt[x_dt], dt[w_dt], group, True, off, dt[bias])
     want = cases.oracle_wq(m, inp, M, K, N)
