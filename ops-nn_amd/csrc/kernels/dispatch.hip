@@ -441,10 +441,9 @@ extern "C" uint64_t opsnnWqmmWorkspace(const OpsnnWqmmArgs* a)
     if (!a || a->M <= 0 || a->N <= 0 || a->K <= 0) return 0;
     const uint64_t bits = (a->w_dtype == DT_I4 || a->w_dtype == DT_E2M1) ? 4 : 8;
     // up to 16 rows against a long K: fp32 partial sums of the x-in-registers kernel's K split, in front of everything else
-    // (from 49 rows of integer codes, 17 of floating-point ones, against a narrow N and a long K: those of the many-rows kernel's K split)
+    // (from 17 rows against a narrow N and a long K: those of the many-rows kernel's K split)
     uint64_t part = 0;
-    const bool wint = a->w_dtype == DT_I4 || a->w_dtype == DT_I8;
-    if (const int xs = wq_part_slices((int)bits, wint, a->M, a->N, a->K, a->group > 0 ? a->group : a->K, opsnn_wq_narrow_slabs() != 0); xs > 1 && a->force_variant != OPSNN_VARIANT_PLAIN && !opsnn_force_plain())
+    if (const int xs = wq_part_slices((int)bits, a->M, a->N, a->K, a->group > 0 ? a->group : a->K, opsnn_wq_narrow_slabs() != 0); xs > 1 && a->force_variant != OPSNN_VARIANT_PLAIN && !opsnn_force_plain())
         part = ((uint64_t)xs * (uint64_t)a->M * (uint64_t)a->N * 4 + 255) / 256 * 256;
     if (a->w.row_stride == 1 || a->K == 1) return part;
     if (a->w.col_stride != 1 || a->w.row_stride != a->N) return part;

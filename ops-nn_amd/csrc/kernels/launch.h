@@ -113,16 +113,16 @@ inline int64_t wq_narrow_slab_rows(int64_t M, int64_t N, bool on)
     if (n < 2) return 0;
     return ((M + n - 1) / n + 15) / 16 * 16;
 }
-// The same kernel, from 49 rows of integer codes or 17 of floating-point ones (where it takes over): a narrow N leaves CUs without a workgroup even with all row slabs in one
+// The same kernel, from 17 rows: a narrow N leaves CUs without a workgroup even with all row slabs in one
 // launch (64 rows against 28672 x 8192: 64 workgroups of 128 columns), and a long K makes each of them slow.  Then K is
 // cut into segments, one per blockIdx.z, whose fp32 partial sums a second kernel adds in segment order.  Segments are
 // whole rounds of the kernel's chunk pipeline (eight chunks of 128 bytes of a weight row), as equal as that allows, at
 // least 2048 k each, and hold whole groups.  Returns the segment count (1: no split).
 // (Measured, int4 with groups of 128, 64 rows: 14336 x 4096 64 -> 22 us, 28672 x 8192 124 -> 66, 8192 x 8192 30 -> 24; a K
 // of 4096 lost 2 to 6 us to the second kernel, and so did two segments of 128 workgroups at K = 8192.)
-inline int wq_rows_ksplit(int wbits, bool wint, int64_t M, int64_t N, int64_t K, int64_t group, bool on)
+inline int wq_rows_ksplit(int wbits, int64_t M, int64_t N, int64_t K, int64_t group, bool on)
 {
-    if (!on || M < (wint ? 49 : 17) || N % 32 != 0 || N < 256 || K < 8192 || K >= (1ll << 23)) return 1;
+    if (!on || M < 17 || N % 32 != 0 || N < 256 || K < 8192 || K >= (1ll << 23)) return 1;
     const int64_t slab = wq_narrow_slab_rows(M, N, on);
     if (M > 64 && slab == 0) return 1;
     const int64_t slabs = slab ? (M + slab - 1) / slab : 1;
@@ -135,10 +135,10 @@ inline int wq_rows_ksplit(int wbits, bool wint, int64_t M, int64_t N, int64_t K,
     return s < 2 ? 1 : (int)s;
 }
 // fp32 partial-sum slices [slices][M][N] at the front of a weight-only call's workspace (1: none)
-inline int wq_part_slices(int wbits, bool wint, int64_t M, int64_t N, int64_t K, int64_t group, bool narrow_on)
+inline int wq_part_slices(int wbits, int64_t M, int64_t N, int64_t K, int64_t group, bool narrow_on)
 {
     if (M <= 16) return wq_xreg_splits(wbits, M, K);
-    return wq_rows_ksplit(wbits, wint, M, N, K, group, narrow_on);
+    return wq_rows_ksplit(wbits, M, N, K, group, narrow_on);
 }
 // Opened by every exported matmul entry point for the time it enqueues its launches (weight_cache.hip): copies that the
 // weight cache hands out inside the scope cannot be evicted before it closes; bypass = true switches the cache off for

@@ -341,7 +341,8 @@ static bool stream_eligible(WqParams& p, WqStreamOpts& o)
     // 48 rows 69 / 70, 64 rows 82 / 70, 128 rows 105: hence the switch at 49 rows)
     constexpr int rows_min = 49;
     // (the kernel addresses the x rows of a slab, up to 256, with 32-bit byte offsets)
-    o.rows = p.M >= rows_min && nch % 8 == 0 && p.N % 32 == 0 && p.N >= 256 && p.K < (1ll << 23);
+    o.rows_shape = nch % 8 == 0 && p.N % 32 == 0 && p.N >= 256 && p.K < (1ll << 23);
+    o.rows = p.M >= rows_min && o.rows_shape;
     return true;
 }
 
@@ -389,7 +390,7 @@ static int launch_slabs_float(WqParams p, hipStream_t st)
         else ok = ok && !p.scale_e8m0 && p.group >= p.K;
         if (ok) {
             // (a long K against few workgroups: K in segments as well, then on 128-column workgroups)
-            const int ks = p.part ? wq_rows_ksplit(WBITS, false, p.M, p.N, p.K, p.group, opsnn_wq_narrow_slabs() != 0) : 1;
+            const int ks = p.part ? wq_rows_ksplit(WBITS, p.M, p.N, p.K, p.group, opsnn_wq_narrow_slabs() != 0) : 1;
             p.ksplit = ks > 1 ? ks : 0;
             if (const int64_t slab = narrow_n_slab(p.M, p.N)) {   // narrow N: all row slabs in one launch
                 p.cpg_shift = WBITS == 4 ? 0 : 31;
@@ -433,13 +434,14 @@ static int launch_slabs(WqParams p, hipStream_t st)
     // slabs of up to 256 rows; then the tile kernel.  (Measured on 8192 x 28672 int4, fp16: 256 rows 151-155 us against 170 on
     // the tile kernel, 192 rows 142-149 against 168.  Test hook: opsnnSetWqTileMin(m <= 128) sends such calls to the tile
     // kernel first.)
-    // narrow N against a long K, integer codes, from 49 rows: the row slabs in one launch and K in segments on top
+    // narrow N against a long K, from 17 rows: the row slabs in one launch and K in segments on top
     if (p.part && opsnn_wq_tile_min() > 128) {
         const int64_t slab = p.M <= 64 ? 0 : narrow_n_slab(p.M, p.N);
-        const int ks = wq_rows_ksplit(WBITS, true, p.M, p.N, p.K, p.group, opsnn_wq_narrow_slabs() != 0);
+        const int ks = wq_rows_ksplit(WBITS, p.M, p.N, p.K, p.group, opsnn_wq_narrow_slabs() != 0);
         WqParams q = p;
         WqStreamOpts o{};
-        if (ks > 1 && (p.M <= 64 || slab > 0) && stream_eligible<WBITS>(q, o) && o.rows) {
+        if (ks > 1 && (p.M <= 64 || slab > 0) && stream_eligible<WBITS>(q, o) && o.rows_shape) {
+            o.rows = true;   // (with K in segments the many-rows kernel is ahead from 17 rows: 48 x 28672 x 8192 int4 153 -> 53 us)
             q.m_base = 0; q.m_rows = q.M;
             if (slab > 0) { q.m_rows = slab; q.m_slab = slab; q.m_end = q.M; }
             q.ksplit = ks;
@@ -538,7 +540,7 @@ int launch_wqmm_mfma(const OpsnnWqmmArgs& a0, hipStream_t st)
     // up to 16 rows against a long K: the partial sums of the x-in-registers kernel's K split sit at the front of the workspace
     // (and those of the many-rows kernel's K split against a narrow N)
     float* part = nullptr;
-    if (const int xs = wq_part_slices(wbits, !wflt, a.M, a.N, a.K, a.group > 0 ? a.group : a.K, opsnn_wq_narrow_slabs() != 0); xs > 1 && a.workspace) {
+    if (const int xs = wq_part_slices(wbits, a.M, a.N, a.K, a.group > 0 ? a.group : a.K, opsnn_wq_narrow_slabs() != 0); xs > 1 && a.workspace) {
         part = (float*)a.workspace;
         const uint64_t pb = ((uint64_t)xs * (uint64_t)a.M * (uint64_t)a.N * 4 + 255) / 256 * 256;
         const bool relayout = a.w.row_stride != 1 && a.K != 1;

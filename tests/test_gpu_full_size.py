@@ -175,6 +175,8 @@ def test_int8_k_split_at_model_sizes_is_bit_identical(gpu, M, K, N):
     (64, 28672, 8192, "i4", 128, True),      # many-rows kernel, K in four segments of seven rounds
     (128, 14336, 4096, "i4", 128, True),     # two row slabs, K in four segments of 4, 4, 3 and 3 rounds
     (64, 14336, 4096, "i8", 0, False),       # 8-bit weights: seven segments
+    (32, 28672, 8192, "i4", 128, True),      # 17 .. 48 rows: the many-rows kernel because of the K split
+    (20, 14336, 4096, "fp4", 32, False),     # mxfp4, seven segments
     (512, 14336, 4096, "i4", 128, True),     # 112 groups per row: scale table rows of 128 words
 ])
 def test_weight_only_at_model_sizes_off_the_configs(gpu, M, K, N, w_dt, group, off):

@@ -507,7 +507,7 @@ def test_weight_only_64_column_workgroups(gpu, M, K, N, x_dt, w_dt, group, off, 
 
 
 @pytest.mark.parametrize("M,K,N,x_dt,w_dt,group,off,bias", [
-    # from 49 rows of integer codes (17 of floating-point ones) against a narrow N and a K of 8192 or more: K in 2 .. 8 segments over blockIdx.z (whole
+    # from 17 rows against a narrow N and a K of 8192 or more: K in 2 .. 8 segments over blockIdx.z (whole
     # rounds of eight chunks -- 1024 k of int4, 512 of int8 --, as equal as that allows, at least 2048 k), partial sums added
     # by a second kernel; one row slab and several, ragged last workgroup, ragged last slab, unequal segments, group counts
     # per segment that are no power of two, per-channel scales
@@ -521,7 +521,11 @@ def test_weight_only_64_column_workgroups(gpu, M, K, N, x_dt, w_dt, group, off, 
     (300, 12288, 256, "bf16", "i4", 256, True, None),         # five slabs, six segments
     (64, 16384, 1024, "f16", "i4", 128, True, None),          # eight workgroups: eight segments
     (64, 32768, 256, "f16", "i4", 128, True, None),           # (in one piece: 256 groups per row, too many for the scale table)
-    # floating-point codes, from 17 rows
+    # 17 .. 48 rows of integer codes (in one piece they run on the streaming kernel)
+    (17, 8192, 256, "bf16", "i4", 128, True, None),
+    (33, 10240, 288, "f16", "i8", 0, False, "f16"),
+    (48, 8192, 1024, "f16", "i4", 64, True, None),
+    # floating-point codes
     (17, 8192, 256, "f16", "fp4", 32, False, None),
     (64, 14336, 288, "bf16", "fp4", 32, False, "bf16"),       # seven segments, a last workgroup of 32 columns
     (40, 11264, 256, "f16", "e4m3", 0, False, None),          # 22 rounds of 512 in five segments (5, 5, 4, 4, 4)
