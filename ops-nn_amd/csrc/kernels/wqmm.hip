@@ -335,11 +335,12 @@ static bool stream_eligible(WqParams& p, WqStreamOpts& o)
     o.xreg = p.M <= 16 && xreg_shape(WBITS, p.K, xreg_nw, xnw, xnch, p.M, p.part != nullptr, &xsplits, &xexact) && (p.M >= xreg_min || (xsplits > 1 && !o.resx));
     o.xreg_vscale = o.xreg && xexact && p.group == KC && p.s_rs == 1 && p.s_cs % 8 == 0 &&
                     (uintptr_t)p.scale % 16 == 0 && (!p.offset || (uintptr_t)p.offset % 16 == 0);
-    // more than 48 rows: two weight blocks per wave share every x fragment, up to 128 rows per pass over the weights
+    // more than 32 rows: two weight blocks per wave share every x fragment, up to 128 rows per pass over the weights
     // (needs whole groups of chunks in flight and whole wave tiles of columns)
-    // (measured on 8192 x 28672 int4: 16 rows 43 us on the streaming kernel against 55 on this one, 32 rows 53 / 68,
-    // 48 rows 69 / 70, 64 rows 82 / 70, 128 rows 105: hence the switch at 49 rows)
-    constexpr int rows_min = 49;
+    // (measured on 8192 x 28672 int4, streaming kernel / this one: 17 rows 45 / 53 us, 32 rows 51 / 53, 40 rows 64 / 53,
+    // 48 rows 68 / 53, 64 rows 54; on 4096 x 4096: 32 rows 17.5 / 15.7, 40 rows 23.5 / 16.0; int8 8192 x 28672: 32 rows
+    // 55 / 68, 40 rows 75 / 68: hence the switch at 33 rows)
+    constexpr int rows_min = 33;
     // (the kernel addresses the x rows of a slab, up to 256, with 32-bit byte offsets)
     o.rows_shape = nch % 8 == 0 && p.N % 32 == 0 && p.N >= 256 && p.K < (1ll << 23);
     o.rows = p.M >= rows_min && o.rows_shape;

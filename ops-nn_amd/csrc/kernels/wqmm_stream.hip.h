@@ -1582,7 +1582,7 @@ static int launch_rows_one(const WqParams& p, hipStream_t st)
 struct WqStreamOpts {
     bool has_off, vscale, ksplit;
     bool rows;                // many-rows kernel eligible (row slabs of up to 128)
-    bool rows_shape;          // ... as far as K, N and the scale layout go (rows also asks for 49 rows or more)
+    bool rows_shape;          // ... as far as K, N and the scale layout go (rows also asks for 33 rows or more)
     bool resx, resx_vscale;   // whole-x-in-LDS kernel eligible, and with vector scale loads
     bool xreg, xreg_vscale;   // x-in-registers kernel eligible (up to 16 rows), and with vector scale loads
     int xreg_nw;              // 8: keep it to eight waves (tuning)

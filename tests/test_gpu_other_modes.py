@@ -521,7 +521,7 @@ def test_weight_only_64_column_workgroups(gpu, M, K, N, x_dt, w_dt, group, off, 
     (300, 12288, 256, "bf16", "i4", 256, True, None),         # five slabs, six segments
     (64, 16384, 1024, "f16", "i4", 128, True, None),          # eight workgroups: eight segments
     (64, 32768, 256, "f16", "i4", 128, True, None),           # (in one piece: 256 groups per row, too many for the scale table)
-    # 17 .. 48 rows of integer codes (in one piece they run on the streaming kernel)
+    # 17 .. 48 rows of integer codes (in one piece the first of them runs on the streaming kernel)
     (17, 8192, 256, "bf16", "i4", 128, True, None),
     (33, 10240, 288, "f16", "i8", 0, False, "f16"),
     (48, 8192, 1024, "f16", "i4", 64, True, None),
