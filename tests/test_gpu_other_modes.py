@@ -521,6 +521,10 @@ def test_weight_only_64_column_workgroups(gpu, M, K, N, x_dt, w_dt, group, off, 
     (300, 12288, 256, "bf16", "i4", 256, True, None),         # five slabs, six segments
     (64, 16384, 1024, "f16", "i4", 128, True, None),          # eight workgroups: eight segments
     (64, 32768, 256, "f16", "i4", 128, True, None),           # (in one piece: 256 groups per row, too many for the scale table)
+    # K below 8192 where the 64-column workgroups cannot run (K no multiple of 16 chunks), from 33 rows
+    (64, 5120, 256, "f16", "i4", 128, True, None),            # five rounds in two segments (3, 2)
+    (40, 7168, 288, "bf16", "i4", 256, False, "bf16"),        # seven rounds in three
+    (128, 5120, 1024, "f16", "i4", 128, True, None),          # two row slabs
     # 17 .. 48 rows of integer codes (in one piece the first of them runs on the streaming kernel)
     (17, 8192, 256, "bf16", "i4", 128, True, None),
     (33, 10240, 288, "f16", "i8", 0, False, "f16"),
