@@ -426,9 +426,10 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(NW == 8
 // of the loop (512 of 1024 per slab and CU, against about 0.45 requests per clock that a CU's texture path takes) --
 // more than weights and x together; per-wave timestamps showed the waves stalled in the issue of their memory
 // instructions (1180 of 4120 clocks per slab) and at the barrier behind them.
-template <int XDT, int WBITS, int MB, int NB, int WN, int WK, bool HAS_OFF, int WF = 0, bool SLDS = false>
+template <int XDT, int WBITS, int MB, int NB, int WN, int WK, bool HAS_OFF, int WF = 0, bool SLDS = false, bool KSP = false>
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void wqmm_rows_kernel(WqParams p)
 {
+    static_assert(!KSP || WF <= 2, "K in segments: the weight-only forms");
     static_assert(WN * WK == 8, "eight waves");
     static_assert(!SLDS || WF == 0 || WF == 2, "the scale table serves the integer forms and the e8m0 bytes of e2m1 codes");
     static_assert(WF == 0 || !HAS_OFF, "floating-point weight codes have no offset");
@@ -466,10 +467,11 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void w
     // K in segments: this workgroup's is number blockIdx.z.  Segments are whole rounds of the chunk pipeline (ROUND k), as
     // equal as that allows, the longer ones first.  From here on p.K is the segment's length and x, w, the scales and
     // offsets start at the segment; a row of x keeps its pitch ldx.
+    // (KSP instantiations; the others keep p as it came)
     const int64_t ldx = p.K;
-    const bool ksplit = p.ksplit > 1;
-    if constexpr (WF <= 2) {
-        if (ksplit) {
+    constexpr bool ksplit = KSP;
+    if constexpr (KSP) {
+        {
             constexpr int ROUND = KX * PF;
             const int z = (int)blockIdx.z, rounds = (int)(p.K / ROUND), base = rounds / p.ksplit, rem = rounds % p.ksplit;
             const int64_t k0 = (int64_t)(z * base + (z < rem ? z : rem)) * ROUND;
@@ -906,11 +908,9 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void w
             if (r >= rows) continue;
             const int64_t m = p.m_base + r;
             const int64_t nn0 = n0 + 16 * q + 4 * g;
-            if constexpr (WF <= 2) {
-                if (ksplit) {   // this segment's partial sums; bias and rounding follow in the kernel that adds the segments
-                    *(v4f*)(p.part + ((int64_t)blockIdx.z * p.M + m) * p.N + nn0) = acc[q][b];
-                    continue;
-                }
+            if constexpr (ksplit) {   // this segment's partial sums; bias and rounding follow in the kernel that adds the segments
+                *(v4f*)(p.part + ((int64_t)blockIdx.z * p.M + m) * p.N + nn0) = acc[q][b];
+                continue;
             }
             float v[4];
 #pragma unroll
@@ -1518,16 +1518,22 @@ static int launch_stream_one(const WqParams& p, hipStream_t st)
     return (int)hipGetLastError();
 }
 
-template <int XDT, int WBITS, int MB, int NB, int WN, int WK, bool HAS_OFF, int WF = 0, bool SLDS = false>
+template <int XDT, int WBITS, int MB, int NB, int WN, int WK, bool HAS_OFF, int WF = 0, bool SLDS = false, bool KSP = false>
 static int launch_rows_one(const WqParams& p, hipStream_t st)
 {
+    if constexpr (!KSP) {   // K in segments: the instantiations of the 64-row instance with 128-column workgroups that know them
+        if (p.ksplit > 1) {
+            if constexpr (MB == 4 && NB == 2 && WN == 4 && WK == 2 && WF <= 2 && !SLDS) return launch_rows_one<XDT, WBITS, MB, NB, WN, WK, HAS_OFF, WF, false, true>(p, st);
+            else return -1;
+        }
+    }
     constexpr int KC = 4 * (128 / WBITS);
     constexpr int XH = (MB > 8 && WBITS == 4) ? 2 : 1;   // as in the kernel: 8-byte weight pieces, i.e. slabs of half the K, for more than 128 rows of x with 4-bit weights
     constexpr size_t lds_x = 2 * (size_t)(16 * MB) * (WK * KC * 2 / XH);
     size_t lds_stab = 0;
-    const bool split = p.ksplit > 1;
+    const bool split = KSP;
     // (a split launch covers all rows: the kernel that adds the segments walks the whole output)
-    if (split && (WF > 2 || !p.part || p.ksplit > 64 || p.m_base != 0 || (p.m_slab > 0 ? p.m_end : p.m_rows) != p.M)) return -1;
+    if (split && (!p.part || p.ksplit < 2 || p.ksplit > 64 || p.m_base != 0 || (p.m_slab > 0 ? p.m_end : p.m_rows) != p.M)) return -1;
     // the longest K one workgroup walks: segments are whole rounds of the kernel's chunk pipeline, as equal as that allows
     constexpr int64_t ROUND = (int64_t)WK * 4 * (((MB > 8 && WBITS == 4) ? 8 : 16) * 8 / WBITS) * (MB > 8 ? 4 : 8 / NB);
     int64_t kseg = p.K;
@@ -1547,7 +1553,7 @@ static int launch_rows_one(const WqParams& p, hipStream_t st)
         const size_t red = (size_t)WN * (WK - 1) * NB * MB * 4 * 64 * 4;
         const bool rows_ok = WF == 2 ? (p.s_cs % 4 == 0 && (uintptr_t)p.scale % 4 == 0 && p.cpg_shift == 0) : (p.s_rs == 1 || G == 1);
         if (rows_ok && (lds_x > red ? lds_x : red) + (size_t)(16 * NB * WN) * GP * 4 <= 160 * 1024)
-            return launch_rows_one<XDT, WBITS, MB, NB, WN, WK, HAS_OFF, WF, true>(p, st);
+            return launch_rows_one<XDT, WBITS, MB, NB, WN, WK, HAS_OFF, WF, true, KSP>(p, st);
     }
     if constexpr (MB > 8 && WF == 0 && !SLDS) return OPSNN_NOT_TAKEN;   // integer codes: the 192- / 256-row instances exist with the scale table only
     else {
@@ -1560,7 +1566,7 @@ static int launch_rows_one(const WqParams& p, hipStream_t st)
     const unsigned grid = (unsigned)((p.N + 16 * NB * WN - 1) / (16 * NB * WN));
     const int64_t slabs = p.m_slab > 0 ? (p.m_end - p.m_base + p.m_slab - 1) / p.m_slab : 1;
     if (slabs < 1 || slabs > 65535 || p.m_rows > 16 * MB || (p.m_slab > 0 && p.m_slab != p.m_rows)) return -1;
-    auto k = wqmm_rows_kernel<XDT, WBITS, MB, NB, WN, WK, HAS_OFF, WF, SLDS>;
+    auto k = wqmm_rows_kernel<XDT, WBITS, MB, NB, WN, WK, HAS_OFF, WF, SLDS, KSP>;
     static std::atomic<uint64_t> attr_set{0};   // one bit per device: the attribute belongs to the (kernel, device) pair
     if (!device_flag_test(attr_set)) {
         hipError_t e = hipFuncSetAttribute((const void*)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)(SLDS ? 160 * 1024 : lds_main + lds_table));
