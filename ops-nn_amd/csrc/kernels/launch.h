@@ -116,26 +116,33 @@ inline int64_t wq_narrow_slab_rows(int64_t M, int64_t N, bool on)
 // The same kernel, from 17 rows: a narrow N leaves CUs without a workgroup even with all row slabs in one
 // launch (64 rows against 28672 x 8192: 64 workgroups of 128 columns), and a long K makes each of them slow.  Then K is
 // cut into segments, one per blockIdx.z, whose fp32 partial sums a second kernel adds in segment order.  Segments are
-// whole rounds of the kernel's chunk pipeline (eight chunks of 128 bytes of a weight row), as equal as that allows, at
-// least 2048 k each, and hold whole groups.  Returns the segment count (1: no split).
+// whole units (a slab of x of the 64-row instance -- two chunks of 128 bytes of a weight row -- or a group where that is
+// longer), as equal as that allows, at least 2048 k each.  Returns the segment count (1: no split) and the unit.
 // (Measured, int4 with groups of 128, 64 rows: 14336 x 4096 64 -> 22 us, 28672 x 8192 124 -> 66, 8192 x 8192 30 -> 24; a K
 // of 4096 lost 2 to 6 us to the second kernel, and so did two segments of 128 workgroups at K = 8192; 64 x 7168 x 7168, where
 // the 64-column workgroups cannot run, 42 -> 26.)
-inline int wq_rows_ksplit(int wbits, int64_t M, int64_t N, int64_t K, int64_t group, bool on)
+inline int wq_rows_ksplit(int wbits, int64_t M, int64_t N, int64_t K, int64_t group, bool on, int64_t* kunit = nullptr)
 {
     if (!on || M < 17 || N % 32 != 0 || N < 256 || K < 4096 || K >= (1ll << 23)) return 1;
     const int64_t slab = wq_narrow_slab_rows(M, N, on);
     if (M > 64 && slab == 0) return 1;
     const int64_t slabs = slab ? (M + slab - 1) / slab : 1;
-    const int64_t wgs = slabs * ((N + 127) / 128), round = 8 * 4 * (128 / wbits);
-    if (wgs > 128 || K % round != 0 || (group < K && round % group != 0)) return 1;
+    const int64_t wgs = slabs * ((N + 127) / 128), kx = 2 * 4 * (128 / wbits);
+    int64_t unit = kx;
+    if (group < K) {
+        if (group > kx) unit = group;
+        if (unit % group != 0 || unit % kx != 0) return 1;
+    }
+    if (wgs > 128 || K % unit != 0) return 1;
     // (below 8192 only where the 64-column workgroups, which double the workgroups without a second kernel, cannot run: they
-    // want K in whole groups of 16 chunks; and from 33 rows: 17 x 5120 x 5120 int4 took 19 us on the streaming kernel, 22 here)
-    if (K < 8192 && (K % (2 * round) == 0 || wgs > 64 || M < 33)) return 1;
+    // want K in whole slabs of four chunks; and from 33 rows: 17 x 5120 x 5120 int4 took 19 us on the streaming kernel, 22 here)
+    if (K < 8192 && (K % (2 * kx) == 0 || wgs > 64 || M < 33)) return 1;
     int64_t s = 256 / wgs;
     if (s > 8) s = 8;
     if (s > K / 2048) s = K / 2048;
+    if (s > K / unit) s = K / unit;
     if (s == 2 && wgs > 64 && K < 12288) return 1;
+    if (kunit) *kunit = unit;
     return s < 2 ? 1 : (int)s;
 }
 // fp32 partial-sum slices [slices][M][N] at the front of a weight-only call's workspace (1: none)

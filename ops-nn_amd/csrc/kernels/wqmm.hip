@@ -342,7 +342,7 @@ static bool stream_eligible(WqParams& p, WqStreamOpts& o)
     // 55 / 68, 40 rows 75 / 68: hence the switch at 33 rows)
     constexpr int rows_min = 33;
     // (the kernel addresses the x rows of a slab, up to 256, with 32-bit byte offsets)
-    o.rows_shape = nch % 8 == 0 && p.N % 32 == 0 && p.N >= 256 && p.K < (1ll << 23);
+    o.rows_shape = nch % 2 == 0 && p.N % 32 == 0 && p.N >= 256 && p.K < (1ll << 23);
     o.rows = p.M >= rows_min && o.rows_shape;
     return true;
 }
@@ -356,12 +356,12 @@ extern "C" int opsnn_wq_narrow_slabs();
 namespace opsnn {
 
 // Up to 64 rows per slab, `slabs` slabs, and still at most 128 workgroups of 128 columns: the instance whose workgroups
-// take 64 columns (K split over four waves instead of two; needs K in whole groups of 16 chunks) doubles their number.
+// take 64 columns (K split over four waves instead of two; needs K in whole x slabs of four chunks) doubles their number.
 template <int WBITS>
 static int use_cols64(int64_t rows, int64_t slabs, int64_t N, int64_t K)
 {
     constexpr int64_t KC = 4 * (128 / WBITS);
-    return (rows <= 64 && slabs * ((N + 127) / 128) <= 128 && K % (16 * KC) == 0 && N % 32 == 0 && opsnn_wq_narrow_slabs()) ? 1 : 0;
+    return (rows <= 64 && slabs * ((N + 127) / 128) <= 128 && K % (4 * KC) == 0 && N % 32 == 0 && opsnn_wq_narrow_slabs()) ? 1 : 0;
 }
 
 // rows per slab of a narrow weight's one-launch form (0: one pass at a time)
@@ -386,13 +386,18 @@ static int launch_slabs_float(WqParams p, hipStream_t st)
     {
         constexpr int64_t KC = 4 * (128 / WBITS);
         constexpr int rows_min = 17;
-        bool ok = !p.offset && p.M >= rows_min && p.K % KC == 0 && (p.K / KC) % 8 == 0 && p.N % 32 == 0 && p.N >= 256 && p.K < (1ll << 23);
+        bool ok = !p.offset && p.M >= rows_min && p.K % KC == 0 && (p.K / KC) % 2 == 0 && p.N % 32 == 0 && p.N >= 256 && p.K < (1ll << 23);
         if (WBITS == 4) ok = ok && p.scale_e8m0 && p.group == 32 && p.s_rs == 1;
         else ok = ok && !p.scale_e8m0 && p.group >= p.K;
+        // (the 192- / 256-row instances want K in whole rounds of four x slabs)
+        const int64_t nslab = narrow_n_slab(p.M, p.N);
+        if (ok && (p.K / KC) % 8 != 0 && (nslab ? nslab : p.M) > 128) ok = false;
         if (ok) {
             // (a long K against few workgroups: K in segments as well, then on 128-column workgroups)
-            const int ks = p.part ? wq_rows_ksplit(WBITS, p.M, p.N, p.K, p.group, opsnn_wq_narrow_slabs() != 0) : 1;
+            int64_t kunit = 0;
+            const int ks = p.part ? wq_rows_ksplit(WBITS, p.M, p.N, p.K, p.group, opsnn_wq_narrow_slabs() != 0, &kunit) : 1;
             p.ksplit = ks > 1 ? ks : 0;
+            p.kunit = kunit;
             if (const int64_t slab = narrow_n_slab(p.M, p.N)) {   // narrow N: all row slabs in one launch
                 p.cpg_shift = WBITS == 4 ? 0 : 31;
                 p.m_base = 0; p.m_rows = slab; p.m_slab = slab; p.m_end = p.M;
@@ -438,7 +443,8 @@ static int launch_slabs(WqParams p, hipStream_t st)
     // narrow N against a long K, from 17 rows: the row slabs in one launch and K in segments on top
     if (p.part && opsnn_wq_tile_min() > 128) {
         const int64_t slab = p.M <= 64 ? 0 : narrow_n_slab(p.M, p.N);
-        const int ks = wq_rows_ksplit(WBITS, p.M, p.N, p.K, p.group, opsnn_wq_narrow_slabs() != 0);
+        int64_t kunit = 0;
+        const int ks = wq_rows_ksplit(WBITS, p.M, p.N, p.K, p.group, opsnn_wq_narrow_slabs() != 0, &kunit);
         WqParams q = p;
         WqStreamOpts o{};
         if (ks > 1 && (p.M <= 64 || slab > 0) && stream_eligible<WBITS>(q, o) && o.rows_shape) {
@@ -446,6 +452,7 @@ static int launch_slabs(WqParams p, hipStream_t st)
             q.m_base = 0; q.m_rows = q.M;
             if (slab > 0) { q.m_rows = slab; q.m_slab = slab; q.m_end = q.M; }
             q.ksplit = ks;
+            q.kunit = kunit;
             const int rc = launch_wq_stream<XDT, WBITS>(q, o, st);
             if (rc != OPSNN_NOT_TAKEN) return rc;
         }

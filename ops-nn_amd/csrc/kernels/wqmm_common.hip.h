@@ -26,8 +26,10 @@ struct WqParams {
     int64_t m_slab, m_end;
     // x-in-registers kernel with K split over workgroup columns (grid.y segments): fp32 partial sums [segments][M][N]
     float* part;
-    // many-rows kernel with K split over blockIdx.z: ksplit equal segments (K stays the whole K), partial sums in part
+    // many-rows kernel with K split over blockIdx.z: ksplit segments of whole units of kunit k, as equal as that allows (K
+    // stays the whole K), partial sums in part
     int ksplit;
+    int64_t kunit;
     int cols64;              // launcher hint: up to 64 rows on the instance whose workgroups take 64 columns (K split over four waves)
     int w_float;             // weights are floating-point codes (4 bits: e2m1, 8 bits: e4m3), not two's-complement integers
     int scale_e8m0;          // scale is one e8m0 byte per element (MX), not a 16-bit value of x's dtype

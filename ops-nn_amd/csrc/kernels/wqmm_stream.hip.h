@@ -464,17 +464,16 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void w
     static_assert((16 * MB * XPR) % NT == 0 && XPR >= 16 && PF >= 2 && PPH >= 1 && STEPS == PPH * XH, "staging and prefetch shape");
     static_assert(MB <= 8 || (WF == 0 && SLDS) || WF == 1 || WF == 2, "the 192- / 256-row instances: integer codes with the scale table in LDS, or floating-point codes");
     static_assert(!(SLDS && WF == 2 && MB > 8) || WK == 2, "8-byte pieces: byte position of a lane's e8m0 scale inside the table word");
-    // K in segments: this workgroup's is number blockIdx.z.  Segments are whole rounds of the chunk pipeline (ROUND k), as
-    // equal as that allows, the longer ones first.  From here on p.K is the segment's length and x, w, the scales and
+    // K in segments: this workgroup's is number blockIdx.z.  Segments are whole units of p.kunit k (whole slabs of x and
+    // whole groups), as equal as that allows, the longer ones first.  From here on p.K is the segment's length and x, w, the scales and
     // offsets start at the segment; a row of x keeps its pitch ldx.
     // (KSP instantiations; the others keep p as it came)
     const int64_t ldx = p.K;
     constexpr bool ksplit = KSP;
     if constexpr (KSP) {
         {
-            constexpr int ROUND = KX * PF;
-            const int z = (int)blockIdx.z, rounds = (int)(p.K / ROUND), base = rounds / p.ksplit, rem = rounds % p.ksplit;
-            const int64_t k0 = (int64_t)(z * base + (z < rem ? z : rem)) * ROUND;
+            const int z = (int)blockIdx.z, units = (int)(p.K / p.kunit), base = units / p.ksplit, rem = units % p.ksplit;
+            const int64_t k0 = (int64_t)(z * base + (z < rem ? z : rem)) * p.kunit;
             p.x += k0;
             p.w += k0 * WBITS / 8;
             if constexpr (WF == 2) p.scale = (const uint16_t*)((const uint8_t*)p.scale + k0 / 32);   // one e8m0 byte per 32 k
@@ -483,7 +482,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void w
                 p.scale += g0;
                 if constexpr (HAS_OFF) p.offset += g0;
             }
-            p.K = (int64_t)(base + (z < rem ? 1 : 0)) * ROUND;
+            p.K = (int64_t)(base + (z < rem ? 1 : 0)) * p.kunit;
         }
     }
     extern __shared__ __attribute__((aligned(16))) char sx[];
@@ -722,20 +721,22 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void w
             }
     };
 #pragma unroll
-    for (int j = 0; j < PF; j++) fetch(j, j);
+    for (int j = 0; j < PF; j++) fetch(j, (MB > 8 || j < NSLAB) ? j : NSLAB - 1);   // (the 192- / 256-row instances: whole rounds)
     issue_x(0);
     wait_vmcnt<0>();
 
-    for (int c0 = 0; c0 < NSLAB; c0 += PF) {
-#pragma unroll
-        for (int j = 0; j < PF; j++) {
-            const int cw = c0 + j;
+    // chunk cw of this wave, held in prefetch slot j
+    auto chunk_step = [&](auto jc, auto lastc, const int cw) {
+            constexpr int j = decltype(jc)::value;
+            constexpr bool LAST_ROUND = decltype(lastc)::value;   // a step of the shorter round behind the loop
             uint32_t sow[NB];
 #pragma unroll
             for (int h = 0; h < XH; h++) {
             // this thread's copies of the slab have landed (behind a chunk's first slab only the weight fetch issued after
             // them may be in flight; behind its second one nothing was issued)
-            if (h > 0) wait_vmcnt<0>();
+            // (behind the loop everything: no refill follows a step there -- nothing would read it --, so the count of
+            // loads behind the copies is not NBL)
+            if (h > 0 || LAST_ROUND) wait_vmcnt<0>();
             else if (cw > 0) wait_vmcnt<NBL>();
             __syncthreads();   // the slab is complete and visible; every wave has finished the one before
             const int sl = cw * XH + h;
@@ -870,8 +871,29 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void w
                 }
             }
             }
-            const int nx = cw + PF;
-            fetch(j, nx < NSLAB ? nx : NSLAB - 1);   // past the end: a harmless reload of the last chunk
+            if constexpr (!LAST_ROUND) {
+                const int nx = cw + PF;
+                fetch(j, nx < NSLAB ? nx : NSLAB - 1);   // past the end: a harmless reload of the last chunk
+            }
+    };
+    // whole rounds of PF chunks, then the chunks of a last, shorter round (the same count for all waves).  The shorter round
+    // stands behind the loop, not as an exit inside it: with the exit inside, the 256-row instance spilled 700 bytes per lane
+    // and ran eight times as long.  The 192- / 256-row instances have whole rounds only (their launcher sees to it).
+    int c0 = 0;
+    for (; MB > 8 ? c0 < NSLAB : c0 + PF <= NSLAB; c0 += PF) {
+        chunk_step(std::integral_constant<int, 0>{}, std::false_type{}, c0);
+        chunk_step(std::integral_constant<int, 1>{}, std::false_type{}, c0 + 1);
+        if constexpr (PF > 2) {
+            chunk_step(std::integral_constant<int, 2>{}, std::false_type{}, c0 + 2);
+            chunk_step(std::integral_constant<int, 3>{}, std::false_type{}, c0 + 3);
+        }
+        static_assert(PF == 2 || PF == 4, "prefetch slots");
+    }
+    if constexpr (MB <= 8) {
+        if (c0 < NSLAB) chunk_step(std::integral_constant<int, 0>{}, std::true_type{}, c0);
+        if constexpr (PF > 2) {
+            if (c0 + 1 < NSLAB) chunk_step(std::integral_constant<int, 1>{}, std::true_type{}, c0 + 1);
+            if (c0 + 2 < NSLAB) chunk_step(std::integral_constant<int, 2>{}, std::true_type{}, c0 + 2);
         }
     }
 
@@ -1534,13 +1556,15 @@ static int launch_rows_one(const WqParams& p, hipStream_t st)
     const bool split = KSP;
     // (a split launch covers all rows: the kernel that adds the segments walks the whole output)
     if (split && (!p.part || p.ksplit < 2 || p.ksplit > 64 || p.m_base != 0 || (p.m_slab > 0 ? p.m_end : p.m_rows) != p.M)) return -1;
-    // the longest K one workgroup walks: segments are whole rounds of the kernel's chunk pipeline, as equal as that allows
-    constexpr int64_t ROUND = (int64_t)WK * 4 * (((MB > 8 && WBITS == 4) ? 8 : 16) * 8 / WBITS) * (MB > 8 ? 4 : 8 / NB);
+    // the longest K one workgroup walks: segments are whole units of p.kunit k (whole slabs of x, whole groups), as equal as
+    // that allows
+    constexpr int64_t KXS = (int64_t)WK * 4 * (((MB > 8 && WBITS == 4) ? 8 : 16) * 8 / WBITS);   // k per slab of x
+    if (p.K % KXS != 0) return -1;
+    if (MB > 8 && p.K % (4 * KXS) != 0) return OPSNN_NOT_TAKEN;   // the 192- / 256-row instances: whole rounds of four slabs
     int64_t kseg = p.K;
     if (split) {
-        const int64_t rounds = p.K / ROUND;
-        if (p.K % ROUND != 0 || rounds < p.ksplit || (p.group < p.K && ROUND % p.group != 0)) return -1;   // (a segment holds whole groups)
-        kseg = (rounds + p.ksplit - 1) / p.ksplit * ROUND;
+        if (p.kunit <= 0 || p.kunit % KXS != 0 || p.K % p.kunit != 0 || p.K / p.kunit < p.ksplit || (p.group < p.K && p.kunit % p.group != 0)) return -1;
+        kseg = (p.K / p.kunit + p.ksplit - 1) / p.ksplit * p.kunit;
     }
     // groups of that K, and the pitch of a scale table row: the power of two at or above
     const int64_t G = p.cpg_shift >= 31 ? 1 : ((kseg / KC) >> p.cpg_shift);

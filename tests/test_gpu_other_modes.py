@@ -485,6 +485,17 @@ def test_weight_only_256_row_instance(gpu, M, K, N, x_dt, w_dt, group, tW, off, 
     (33, 1024, 288, "f16", "e4m3", 0, False, None),
     (200, 2048, 512, "f16", "i4", 128, True, "f16"),
     (130, 1024, 256, "bf16", "e4m3", 0, False, None),
+    # K in whole x slabs (two chunks on 128-column workgroups, four on 64-column ones) but no whole rounds of the chunk
+    # pipeline: a shorter last round behind the loop, on the 64- and 128-row instances; the 192- / 256-row ones decline
+    (64, 1280, 256, "f16", "i4", 128, True, None),            # five slabs on 128-column workgroups
+    (64, 1536, 288, "bf16", "i4", 128, False, "bf16"),        # three slabs on 64-column workgroups, six on 128-column ones
+    (128, 3584, 256, "f16", "i4", 128, True, None),           # seven / fourteen slabs; one pass: the 128-row instance
+    (100, 640, 320, "bf16", "i8", 64, True, None),
+    (40, 768, 256, "f16", "i8", 0, False, "f16"),
+    (33, 2560, 288, "f16", "fp4", 32, False, None),
+    (120, 896, 256, "bf16", "e4m3", 0, False, None),
+    (256, 1536, 256, "f16", "i4", 128, True, None),           # one pass: whole rounds of the 256-row instance (512 k)
+    (256, 1280, 256, "f16", "i4", 128, True, None),           # one pass: no whole rounds there, the tile kernel
 ])
 def test_weight_only_64_column_workgroups(gpu, M, K, N, x_dt, w_dt, group, off, bias):
     """The many-rows kernel's instance whose workgroups take 64 columns (chosen when 128-column ones would number at most 128)
@@ -521,10 +532,14 @@ def test_weight_only_64_column_workgroups(gpu, M, K, N, x_dt, w_dt, group, off, 
     (300, 12288, 256, "bf16", "i4", 256, True, None),         # five slabs, six segments
     (64, 16384, 1024, "f16", "i4", 128, True, None),          # eight workgroups: eight segments
     (64, 32768, 256, "f16", "i4", 128, True, None),           # (in one piece: 256 groups per row, too many for the scale table)
-    # K below 8192 where the 64-column workgroups cannot run (K no multiple of 16 chunks), from 33 rows
-    (64, 5120, 256, "f16", "i4", 128, True, None),            # five rounds in two segments (3, 2)
-    (40, 7168, 288, "bf16", "i4", 256, False, "bf16"),        # seven rounds in three
-    (128, 5120, 1024, "f16", "i4", 128, True, None),          # two row slabs
+    # K below 8192 where the 64-column workgroups cannot run (K no multiple of four chunks), from 33 rows
+    (64, 4864, 256, "f16", "i4", 128, True, None),            # 19 x slabs in two segments (10, 9)
+    (40, 6400, 288, "bf16", "i4", 256, False, "bf16"),        # 25 in three
+    (128, 7424, 1024, "f16", "i4", 128, True, None),          # two row slabs, 29 in three
+    # segments that are no whole rounds of the chunk pipeline
+    (64, 11008, 256, "f16", "i4", 128, True, None),           # 43 x slabs in five segments (9, 9, 9, 8, 8)
+    (64, 9472, 256, "bf16", "i8", 0, False, None),            # 74 in four (19, 19, 18, 18)
+    (48, 8448, 256, "f16", "fp4", 32, False, None),           # 33 in four
     # 17 .. 48 rows of integer codes (in one piece the first of them runs on the streaming kernel)
     (17, 8192, 256, "bf16", "i4", 128, True, None),
     (33, 10240, 288, "f16", "i8", 0, False, "f16"),
