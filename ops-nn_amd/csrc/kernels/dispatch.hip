@@ -16,8 +16,9 @@ int launch_wqmm_plain(const OpsnnWqmmArgs& a, hipStream_t st);
 int launch_blockscale_mfma(const OpsnnQmmArgs& a, hipStream_t st, SplitK sk = {});
 int launch_fp8_rowcol_mfma(const OpsnnQmmArgs& a, hipStream_t st, bool merged_scales_ok, SplitK sk = {});
 int launch_rowcol_exact(const OpsnnQmmArgs& a, hipStream_t st, int ep_mode, SplitK sk = {});   // qmm_fp8_exact.hip
-int launch_rowcol_decode(const OpsnnQmmArgs& a, hipStream_t st);   // qmm_fp8_decode.hip
+int launch_rowcol_decode(const OpsnnQmmArgs& a, hipStream_t st, SplitK sk);   // qmm_fp8_decode.hip
 uint64_t blockscale_rows_workspace(const OpsnnQmmArgs& a);         // qmm_fp8_rows.hip
+int blockscale_rows_ksplit(const OpsnnQmmArgs& a);
 uint64_t rowcol_rows_workspace(const OpsnnQmmArgs& a);
 int launch_rowcol_rows(const OpsnnQmmArgs& a, hipStream_t st);
 int launch_tcg_mfma(const OpsnnQmmArgs& a, hipStream_t st);
@@ -186,9 +187,23 @@ extern "C" __attribute__((visibility("hidden"))) int opsnn_qmm_k_pad(const Opsnn
 static int splitk_for(const OpsnnQmmArgs& a, int mode)
 {
     if (a.force_variant != 0 || opsnn_force_plain()) return 1;   // (a pinned kernel variant runs as it is)
-    if (a.M * a.N < 64 * 64 || a.K < 1024) return 1;
     const bool out16 = a.out_dtype == DT_BF16 || a.out_dtype == DT_F16;
     const bool f8 = a.x1_dtype == DT_E4M3 && a.x2_dtype == DT_E4M3;
+    // up to 32 rows of fp8 with block scales or row / column scales, or of int8 per-tile: the decode kernel's K segments
+    if (a.M <= 32 && a.batch == 1 && a.N >= 256 &&
+        ((mode == 1 && (f8 || (a.x1_dtype == DT_I8 && a.x2_dtype == DT_I8)) && a.gsK == 128 && a.gsN == 128) ||
+         (mode == 3 && f8 && a.x1_scale && a.x2_scale))) {
+        QmmDecodePlan pl;
+        const int sd = qmm_decode_plan(a.K, true, pl) ? pl.splits : 1;
+        // (17 .. 32 rows of fp8 with block scales may also run on the many-rows kernel, with its own segments: room for either)
+        const int sr = mode == 1 && f8 ? blockscale_rows_ksplit(a) : 1;
+        return sd > sr ? sd : sr;
+    }
+    // 33 .. 128 rows of fp8 with block scales on the many-rows kernel
+    if (mode == 1 && f8 && a.M <= 128) {
+        if (const int sr = blockscale_rows_ksplit(a); sr > 1) return sr;
+    }
+    if (a.M * a.N < 64 * 64 || a.K < 1024) return 1;
     int64_t bm, bn = 256, kunit = 128;
     double tile_us;   // one K tile (kunit elements) of the kernel in question, measured on calls with few tiles
     double bytes_per_us = 5.0e6;   // what its partial sums' traffic was measured to cost (splitk_factor)
@@ -339,19 +354,21 @@ extern "C" int opsnnQmmTc(const OpsnnQmmArgs* a, void* stream)
         if (ep == 0) {   // 17 .. 128 rows: the many-rows streaming kernel; up to 16 (32 in two passes where that does not apply): x1 in registers
             int rc = launch_rowcol_rows(*a, (hipStream_t)stream);
             if (rc != OPSNN_NOT_TAKEN) return rc;
-            rc = launch_rowcol_decode(*a, (hipStream_t)stream);
+            rc = launch_rowcol_decode(*a, (hipStream_t)stream, sk);
             if (rc != OPSNN_NOT_TAKEN) return rc;
         }
+        // (up to 32 rows the partial sums were laid out for the kernel above; the tile kernels run unsplit)
+        const SplitK sk_tiles = a->M <= 32 ? SplitK{} : sk;
         const bool e4 = a->x1_dtype == DT_E4M3 && a->x2_dtype == DT_E4M3;
         if (ep != 0 || !e4 || a->x2_scale_dtype != DT_F32 || a->out_dtype == DT_F32) {
-            const int rc = launch_rowcol_exact(*a, (hipStream_t)stream, ep, sk);
+            const int rc = launch_rowcol_exact(*a, (hipStream_t)stream, ep, sk_tiles);
             if (rc != OPSNN_NOT_TAKEN) return rc;
         }
     }
     // fp8 e4m3 operands with a row scale and a column scale that are multiplied in separately (K-C, K-T, T-C with the
     // one-element x1Scale): matrix-core kernel when the layout allows, else the plain kernel
     if (f8 && a->x1_scale && a->force_variant != OPSNN_VARIANT_PLAIN && !opsnn_force_plain()) {
-        const int rc = launch_fp8_rowcol_mfma(*a, (hipStream_t)stream, false, sk);
+        const int rc = launch_fp8_rowcol_mfma(*a, (hipStream_t)stream, false, a->M <= 32 ? SplitK{} : sk);
         if (rc != OPSNN_NOT_TAKEN) return rc;
     }
     NOTE_PLAIN("per-tensor / per-channel quant matmul", a);

@@ -151,6 +151,33 @@ inline int wq_part_slices(int wbits, int64_t M, int64_t N, int64_t K, int64_t gr
     if (M <= 16) return wq_xreg_splits(wbits, M, K);
     return wq_rows_ksplit(wbits, M, N, K, group, narrow_on);
 }
+// The fp8 / int8 decode kernel (qmm_fp8_decode.hip, up to 32 rows of x1): K in blocks of 128 that the NW = 16 or 8 waves
+// of a workgroup share, NBLK each (a wave keeps its blocks of x1 in registers: 16 waves up to 4, not 3; 8 waves up to 7).
+// A K that the waves of one workgroup share exactly runs as one segment; any other whole number of blocks in 1 .. 16
+// segments of NW * NBLK blocks, the last one with idle waves (K a whole number of NBLK blocks): the layout with the fewest
+// wave slots, then the fewest segments.  More than one segment needs room for fp32 partial sums (may_split).
+struct QmmDecodePlan { int nw = 0, nblk = 0, splits = 1; };
+inline bool qmm_decode_plan(int64_t K, bool may_split, QmmDecodePlan& pl)
+{
+    if (K <= 0 || K % 128 != 0) return false;
+    const int64_t nb = K / 128;
+    if (nb % 16 == 0 && nb / 16 <= 4 && nb / 16 != 3) { pl.nw = 16; pl.nblk = (int)(nb / 16); pl.splits = 1; return true; }
+    if (nb % 8 == 0 && nb / 8 <= 7) { pl.nw = 8; pl.nblk = (int)(nb / 8); pl.splits = 1; return true; }
+    static const int shapes[10][2] = {{16, 4}, {16, 2}, {16, 1}, {8, 7}, {8, 6}, {8, 5}, {8, 4}, {8, 3}, {8, 2}, {8, 1}};
+    int64_t best_slots = 0;
+    bool found = false;
+    for (const auto& sh : shapes) {
+        const int nw = sh[0], nblk = sh[1];
+        if (nb % nblk != 0) continue;
+        const int64_t waves = nb / nblk, s = (waves + nw - 1) / nw;
+        if (s > 16 || (s > 1 && !may_split)) continue;
+        const int64_t slots = s * nw * nblk;
+        if (!found || slots < best_slots || (slots == best_slots && s < pl.splits)) {
+            found = true; best_slots = slots; pl.nw = nw; pl.nblk = nblk; pl.splits = (int)s;
+        }
+    }
+    return found;
+}
 // Opened by every exported matmul entry point for the time it enqueues its launches (weight_cache.hip): copies that the
 // weight cache hands out inside the scope cannot be evicted before it closes; bypass = true switches the cache off for
 // this thread while the scope is open.  Scopes nest; the pins drop when the outermost one closes.

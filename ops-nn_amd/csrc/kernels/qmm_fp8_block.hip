@@ -697,8 +697,8 @@ int launch_fp8_rowcol_mfma(const OpsnnQmmArgs& a, hipStream_t st, bool merged_sc
     return launch_fp8_block<2, 2, DT_F16, FP8_ROWCOL>(p, a.batch, st);
 }
 
-int launch_blockscale_decode(const OpsnnQmmArgs& a, hipStream_t st);   // qmm_fp8_decode.hip
-int launch_blockscale_rows(const OpsnnQmmArgs& a, hipStream_t st);     // qmm_fp8_rows.hip
+int launch_blockscale_decode(const OpsnnQmmArgs& a, hipStream_t st, SplitK sk);   // qmm_fp8_decode.hip
+int launch_blockscale_rows(const OpsnnQmmArgs& a, hipStream_t st, SplitK sk);     // qmm_fp8_rows.hip
 
 int launch_blockscale_mfma(const OpsnnQmmArgs& a0, hipStream_t st, SplitK sk)
 {
@@ -709,7 +709,10 @@ int launch_blockscale_mfma(const OpsnnQmmArgs& a0, hipStream_t st, SplitK sk)
     if (a.out_dtype != DT_BF16 && a.out_dtype != DT_F16 && !out32) return OPSNN_NOT_TAKEN;
     if (a.bias && !(i8 && a.bias_dtype == DT_F32)) return OPSNN_NOT_TAKEN;
     if (a.gsK != 128 || a.gsN != 128 || (a.gsM != 1 && a.gsM != 128)) return OPSNN_NOT_TAKEN;
-    if (a.K % 128 != 0 || a.M * a.N < 64 * 64 || a.x1.col_stride != 1) return OPSNN_NOT_TAKEN;
+    // (fewer than 64 x 64 outputs: only the few-rows stream over x2 below, which wants 256 columns -- one row against a long K
+    // is no work for one thread per output)
+    const bool tiny = a.M * a.N < 64 * 64;
+    if (a.K % 128 != 0 || a.x1.col_stride != 1 || (tiny && !(a.M <= 32 && a.N >= 256))) return OPSNN_NOT_TAKEN;
     if (a.x2.row_stride != 1) {
         // x2 is [K, N] with N contiguous: re-lay it out K-contiguous in the workspace (scales keep their layout)
         if (a.x2.col_stride != 1 || a.x2.row_stride != a.N) return OPSNN_NOT_TAKEN;
@@ -725,13 +728,15 @@ int launch_blockscale_mfma(const OpsnnQmmArgs& a0, hipStream_t st, SplitK sk)
         a.x2.row_stride = 1; a.x2.col_stride = a.K;
     }
     if (!i8 && a0.x2.row_stride == 1) {   // 17 .. 128 rows: x1 widened into the workspace, then the many-rows streaming kernel
-        const int rc = launch_blockscale_rows(a, st);
+        const int rc = launch_blockscale_rows(a, st, sk);
         if (rc != OPSNN_NOT_TAKEN) return rc;
     }
     {   // up to 16 rows (32 in two passes where the kernel above does not apply): the stream over x2 with x1 in registers
-        const int rc = launch_blockscale_decode(a, st);
+        const int rc = launch_blockscale_decode(a, st, sk);
         if (rc != OPSNN_NOT_TAKEN) return rc;
     }
+    if (tiny) return OPSNN_NOT_TAKEN;
+    if (a.M <= 32) sk = SplitK{};   // (with so few rows the partial sums were laid out for the kernel above; the tile kernels run unsplit)
     if (!i8 && (!opsnnGetFp8Fast() || out32)) {   // exact products and sums unless the caller asked for the 8-bit matrix instruction
         const int rc = launch_blockscale_exact(a, st, sk);
         if (rc != OPSNN_NOT_TAKEN || out32) return rc;

@@ -40,6 +40,8 @@ struct Fp8DecParams {
     // row / column scale form (RC): out = (sum * cs[n * cs_stride]) * rs[m * rs_stride] + bias[n]; strides 0 (one scale) or 1
     const float* rs; const float* cs; const float* bias;
     int rs_stride, cs_stride;
+    // K in segments (SEG instantiations, gridDim.y of them): fp32 sums of this pass's rows, slice s at part + s * part_slice
+    float* part; int64_t part_slice;
 };
 
 // 8 e4m3 bytes (two dwords) -> 8 fp16 in byte order
@@ -55,7 +57,11 @@ __device__ __forceinline__ v4i widen8_e4m3(uint32_t d0, uint32_t d1)
 // I8: int8 operands with the same block scales and an fp32 bias (the per-tile mode of quant_batch_matmul_v4,
 // qbmmv4_kernel_golden.py:258-325): a lane's 16-byte piece is one operand of v_mfma_i32_16x16x64_i8 as it is, a block's
 // sum is two of them from a zero accumulator (an exact integer below 2^21), converted to fp32 for the fold.
-template <int NW, int NBLK, bool RC, bool I8 = false>
+// SEG: K is cut into gridDim.y segments of NW * NBLK blocks, one workgroup column each; wave w of segment s takes the
+// NBLK blocks from (s NW + w) NBLK on, and a wave whose blocks lie past the end of K (in the last segment; K is a whole
+// number of NBLK blocks) runs along on the last blocks and contributes zeros.  With more than one segment the
+// workgroup stores its fp32 sums for fp8dec_reduce_kernel, which adds the segments in order and applies the epilogue.
+template <int NW, int NBLK, bool RC, bool I8 = false, bool SEG = false>
 __global__ __launch_bounds__(NW * 64) void fp8_block_decode_kernel(Fp8DecParams p)
 {
     static_assert(!(RC && I8), "int8: the block-scale form only");
@@ -66,8 +72,15 @@ __global__ __launch_bounds__(NW * 64) void fp8_block_decode_kernel(Fp8DecParams 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int nrow = lane & 15, q = lane >> 4;
-    const int64_t kbase = (int64_t)wave * (NBLK * 128);
-    const int kb0 = wave * NBLK;
+    int kb0 = wave * NBLK;
+    bool live = true;
+    if constexpr (SEG) {
+        const int nbk = (int)(p.K / 128);
+        kb0 = ((int)blockIdx.y * NW + wave) * NBLK;
+        live = kb0 < nbk;
+        if (!live) kb0 = nbk - NBLK;
+    }
+    const int64_t kbase = (int64_t)kb0 * 128;
     const int nblocks = (int)((p.N + 15) / 16);
     const int M = (int)p.M;
 
@@ -136,6 +149,9 @@ __global__ __launch_bounds__(NW * 64) void fp8_block_decode_kernel(Fp8DecParams 
             }
         }
         // acc[r]: m = lane % 16, n = n0 + 4 (lane / 16) + r, over this wave's K range
+        if constexpr (SEG) {
+            if (!live) acc = (v4f){0.0f, 0.0f, 0.0f, 0.0f};
+        }
         float* mine = red + ((it & 1) * NW + wave) * 256;
         *(v4f*)(mine + lane * 4) = acc;
         __syncthreads();
@@ -150,6 +166,15 @@ __global__ __launch_bounds__(NW * 64) void fp8_block_decode_kernel(Fp8DecParams 
         }
         if (nrow >= M) continue;
         const int64_t n = n0 + 4 * q;
+        if constexpr (SEG) {
+            if (gridDim.y > 1) {
+                float* dst = p.part + (int64_t)blockIdx.y * p.part_slice + (int64_t)nrow * p.N + n;
+#pragma unroll
+                for (int r = 0; r < 4; r++)
+                    if (n + r < p.N) dst[r] = sum[r];
+                continue;
+            }
+        }
         if constexpr (RC) {   // (sum * x2Scale[n]) * x1Scale[m] + bias[n], each operation rounded
             const float rsv = p.rs[(int64_t)nrow * p.rs_stride];
 #pragma unroll
@@ -180,43 +205,59 @@ __global__ __launch_bounds__(NW * 64) void fp8_block_decode_kernel(Fp8DecParams 
     }
 }
 
-template <int NW, int NBLK, bool RC, bool I8 = false>
-int launch_decode_one(const Fp8DecParams& p, hipStream_t st)
+// out = epilogue(sum over the K segments, in order, of part[s]) for one pass of up to 16 rows: the block-scale form adds the
+// bias, the row / column scale form (RC) computes (sum * x2Scale[n]) * x1Scale[m] + bias[n]
+template <bool RC>
+__global__ __launch_bounds__(256) void fp8dec_reduce_kernel(Fp8DecParams p, int splits)
 {
+    const int64_t total = p.M * p.N, stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
+        float v = p.part[i];
+        for (int s = 1; s < splits; s++) v = v + p.part[(int64_t)s * p.part_slice + i];
+        const int64_t m = i / p.N, n = i - m * p.N;
+        if constexpr (RC) v = (v * p.cs[n * p.cs_stride]) * p.rs[m * p.rs_stride];
+        if (p.bias) v = v + p.bias[n];
+        if (p.out_dt == DT_F32) ((float*)p.out)[i] = v;
+        else ((uint16_t*)p.out)[i] = p.out_dt == DT_BF16 ? bf16_bits(v) : f16_bits(v);
+    }
+}
+
+template <int NW, int NBLK, bool RC, bool I8 = false, bool SEG = false>
+int launch_decode_one(const Fp8DecParams& p, hipStream_t st, int splits = 1)
+{
+    if constexpr (!SEG) {
+        if (splits > 1 || p.K != (int64_t)NW * NBLK * 128) return launch_decode_one<NW, NBLK, RC, I8, true>(p, st, splits);
+    }
+    const int64_t nbk = p.K / 128;
+    if (splits < 1 || splits > 16 || nbk % NBLK != 0 || nbk < NBLK || (int64_t)splits * NW * NBLK < nbk || (splits > 1 && !p.part)) return -1;
     const int nblocks = (int)((p.N + 15) / 16);
-    const int cus = 256;
+    const int cus = 256 / splits;   // the CUs shared between the segments' workgroup columns
     const int grid = nblocks < cus ? nblocks : cus;
     const size_t lds = (size_t)2 * NW * 256 * sizeof(float);
-    hipLaunchKernelGGL((fp8_block_decode_kernel<NW, NBLK, RC, I8>), dim3((unsigned)grid), dim3(NW * 64), lds, st, p);
+    hipLaunchKernelGGL((fp8_block_decode_kernel<NW, NBLK, RC, I8, SEG>), dim3((unsigned)grid, (unsigned)splits), dim3(NW * 64), lds, st, p);
+    if (hipError_t e = hipGetLastError(); e != hipSuccess || splits == 1) return (int)e;
+    hipLaunchKernelGGL(fp8dec_reduce_kernel<RC>, dim3(splitk_reduce_grid(p.M * p.N)), dim3(256), 0, st, p, splits);
     return (int)hipGetLastError();
 }
 
-// K as a whole number of 128-element blocks that 16 or 8 waves share equally (the registers hold up to 7 blocks of x1)
-bool decode_split(int64_t K, int& nw, int& nblk)
-{
-    if (K % 128 != 0) return false;
-    const int64_t nb = K / 128;
-    if (nb % 16 == 0 && nb / 16 <= 4 && nb / 16 != 3) { nw = 16; nblk = (int)(nb / 16); return true; }
-    if (nb % 8 == 0 && nb / 8 <= 7) { nw = 8; nblk = (int)(nb / 8); return true; }
-    return false;
-}
-
 template <bool RC, bool I8 = false>
-int launch_decode_split(const Fp8DecParams& p, int nw, int nblk, hipStream_t st)
+int launch_decode_split(const Fp8DecParams& p, int nw, int nblk, hipStream_t st, int splits = 1)
 {
     if (nw == 16) {
-        if (nblk == 1) return launch_decode_one<16, 1, RC, I8>(p, st);
-        if (nblk == 2) return launch_decode_one<16, 2, RC, I8>(p, st);
-        return launch_decode_one<16, 4, RC, I8>(p, st);
+        if (nblk == 1) return launch_decode_one<16, 1, RC, I8>(p, st, splits);
+        if (nblk == 2) return launch_decode_one<16, 2, RC, I8>(p, st, splits);
+        if (nblk == 4) return launch_decode_one<16, 4, RC, I8>(p, st, splits);
+        return -1;
     }
     switch (nblk) {
-        case 1: return launch_decode_one<8, 1, RC, I8>(p, st);
-        case 2: return launch_decode_one<8, 2, RC, I8>(p, st);
-        case 3: return launch_decode_one<8, 3, RC, I8>(p, st);
-        case 4: return launch_decode_one<8, 4, RC, I8>(p, st);
-        case 5: return launch_decode_one<8, 5, RC, I8>(p, st);
-        case 6: return launch_decode_one<8, 6, RC, I8>(p, st);
-        default: return launch_decode_one<8, 7, RC, I8>(p, st);
+        case 1: return launch_decode_one<8, 1, RC, I8>(p, st, splits);
+        case 2: return launch_decode_one<8, 2, RC, I8>(p, st, splits);
+        case 3: return launch_decode_one<8, 3, RC, I8>(p, st, splits);
+        case 4: return launch_decode_one<8, 4, RC, I8>(p, st, splits);
+        case 5: return launch_decode_one<8, 5, RC, I8>(p, st, splits);
+        case 6: return launch_decode_one<8, 6, RC, I8>(p, st, splits);
+        case 7: return launch_decode_one<8, 7, RC, I8>(p, st, splits);
+        default: return -1;
     }
 }
 
@@ -348,9 +389,9 @@ int launch_mxw4_one(const MxW4DecParams& p, hipStream_t st)
 }  // namespace
 
 // fp8 e4m3 block scales (or int8 per-tile: the same scales, an fp32 bias, 16-bit output) with up to 32 rows of x1 (two
-// passes beyond 16), K-contiguous operands, K a whole number of blocks that 16 or 8 waves share equally; OPSNN_NOT_TAKEN
-// otherwise.
-int launch_blockscale_decode(const OpsnnQmmArgs& a, hipStream_t st)
+// passes beyond 16), K-contiguous operands, K a whole number of 128-element blocks as qmm_decode_plan lays them out (more
+// than one segment only with room for the partial sums in sk); OPSNN_NOT_TAKEN otherwise.
+int launch_blockscale_decode(const OpsnnQmmArgs& a, hipStream_t st, SplitK sk)
 {
     const bool i8 = a.x1_dtype == DT_I8 && a.x2_dtype == DT_I8;
     if ((!i8 && (a.x1_dtype != DT_E4M3 || a.x2_dtype != DT_E4M3)) || a.batch != 1) return OPSNN_NOT_TAKEN;
@@ -362,8 +403,8 @@ int launch_blockscale_decode(const OpsnnQmmArgs& a, hipStream_t st)
     if (((uintptr_t)a.x1.ptr | (uintptr_t)a.x2.ptr | (uint64_t)a.x1.row_stride | (uint64_t)a.x2.col_stride) % 16) return OPSNN_NOT_TAKEN;
     if (((uintptr_t)a.x1_scale_mat.ptr | (uintptr_t)a.x2_scale_mat.ptr) % 4) return OPSNN_NOT_TAKEN;
     if (a.x1.row_stride < a.K || a.x2.col_stride < a.K) return OPSNN_NOT_TAKEN;
-    int nw = 0, nblk = 0;
-    if (!decode_split(a.K, nw, nblk)) return OPSNN_NOT_TAKEN;
+    QmmDecodePlan pl;
+    if (!qmm_decode_plan(a.K, sk.part != nullptr, pl) || pl.splits > (sk.part ? sk.splits : 1)) return OPSNN_NOT_TAKEN;
     for (int64_t m0 = 0; m0 < a.M; m0 += 16) {
         Fp8DecParams p{};
         p.M = a.M - m0 < 16 ? a.M - m0 : 16; p.N = a.N; p.K = a.K;
@@ -371,13 +412,14 @@ int launch_blockscale_decode(const OpsnnQmmArgs& a, hipStream_t st)
         p.lda = a.x1.row_stride; p.ldb = a.x2.col_stride;
         p.out_dt = a.out_dtype;
         p.out = (char*)a.out + m0 * a.N * (a.out_dtype == DT_F32 ? 4 : 2);
+        p.part = sk.part ? sk.part + m0 * a.N : nullptr; p.part_slice = a.M * a.N;
         p.gsM = (int)a.gsM;
         // gsM 1: the pass's own rows of the scale table; gsM 128: up to 32 rows share row 0
         p.s1 = (const float*)a.x1_scale_mat.ptr + (a.gsM == 1 ? m0 * a.x1_scale_mat.row_stride : 0);
         p.s1_rs = a.x1_scale_mat.row_stride; p.s1_cs = a.x1_scale_mat.col_stride;
         p.s2 = (const float*)a.x2_scale_mat.ptr; p.s2_rs = a.x2_scale_mat.row_stride; p.s2_cs = a.x2_scale_mat.col_stride;
         p.bias = (const float*)a.bias;
-        const int rc = i8 ? launch_decode_split<false, true>(p, nw, nblk, st) : launch_decode_split<false>(p, nw, nblk, st);
+        const int rc = i8 ? launch_decode_split<false, true>(p, pl.nw, pl.nblk, st, pl.splits) : launch_decode_split<false>(p, pl.nw, pl.nblk, st, pl.splits);
         if (rc != 0) return rc;
     }
     return 0;
@@ -385,7 +427,7 @@ int launch_blockscale_decode(const OpsnnQmmArgs& a, hipStream_t st)
 
 // fp8 e4m3 with one fp32 scale per row of x1 (or one) and one per column of x2 (or one), optional fp32 bias -- the form
 // (sum * x2Scale) * x1Scale + bias of compute_pertoken (qbmmv3_kernel_golden.py:361-387) -- for up to 32 rows.
-int launch_rowcol_decode(const OpsnnQmmArgs& a, hipStream_t st)
+int launch_rowcol_decode(const OpsnnQmmArgs& a, hipStream_t st, SplitK sk)
 {
     if (a.x1_dtype != DT_E4M3 || a.x2_dtype != DT_E4M3 || a.batch != 1) return OPSNN_NOT_TAKEN;
     if (a.out_dtype != DT_BF16 && a.out_dtype != DT_F16 && a.out_dtype != DT_F32) return OPSNN_NOT_TAKEN;
@@ -393,8 +435,8 @@ int launch_rowcol_decode(const OpsnnQmmArgs& a, hipStream_t st)
     if (a.M > 32 || a.N < 256 || a.x1.col_stride != 1 || a.x2.row_stride != 1) return OPSNN_NOT_TAKEN;
     if (((uintptr_t)a.x1.ptr | (uintptr_t)a.x2.ptr | (uint64_t)a.x1.row_stride | (uint64_t)a.x2.col_stride) % 16) return OPSNN_NOT_TAKEN;
     if (a.x1.row_stride < a.K || a.x2.col_stride < a.K) return OPSNN_NOT_TAKEN;
-    int nw = 0, nblk = 0;
-    if (!decode_split(a.K, nw, nblk)) return OPSNN_NOT_TAKEN;
+    QmmDecodePlan pl;
+    if (!qmm_decode_plan(a.K, sk.part != nullptr, pl) || pl.splits > (sk.part ? sk.splits : 1)) return OPSNN_NOT_TAKEN;
     for (int64_t m0 = 0; m0 < a.M; m0 += 16) {
         Fp8DecParams p{};
         p.M = a.M - m0 < 16 ? a.M - m0 : 16; p.N = a.N; p.K = a.K;
@@ -405,7 +447,8 @@ int launch_rowcol_decode(const OpsnnQmmArgs& a, hipStream_t st)
         p.rs_stride = a.x1_scale_len == 1 ? 0 : 1; p.cs_stride = a.x2_scale_len == 1 ? 0 : 1;
         p.rs = (const float*)a.x1_scale + (p.rs_stride ? m0 : 0);
         p.cs = (const float*)a.x2_scale; p.bias = (const float*)a.bias;
-        const int rc = launch_decode_split<true>(p, nw, nblk, st);
+        p.part = sk.part ? sk.part + m0 * a.N : nullptr; p.part_slice = a.M * a.N;
+        const int rc = launch_decode_split<true>(p, pl.nw, pl.nblk, st, pl.splits);
         if (rc != 0) return rc;
     }
     return 0;

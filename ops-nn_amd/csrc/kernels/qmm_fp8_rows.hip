@@ -31,15 +31,34 @@ __global__ __launch_bounds__(256) void widen_e4m3_f16_kernel(const uint8_t* __re
     out[1] = make_uint4(o[4], o[5], o[6], o[7]);
 }
 
+// rows of x1 per workgroup: all of them, or, against a narrow x2 (at most 128 workgroups of 128 columns), equal slabs of up
+// to 64 rows that go out in one launch
+int64_t rows_per_slab(const OpsnnQmmArgs& a)
+{
+    const int64_t slab = wq_narrow_slab_rows(a.M, a.N, true);
+    return slab ? slab : a.M;
+}
+// K segments for a long K against few workgroups (wq_rows_ksplit; the unit is one scale block)
+int rows_ksplit(const OpsnnQmmArgs& a, int64_t* kunit = nullptr)
+{
+    if (a.force_variant != 0 || rows_per_slab(a) > 64) return 1;
+    return wq_rows_ksplit(8, a.M, a.N, a.K, a.K, true, kunit);
+}
+
 bool rows_eligible(const OpsnnQmmArgs& a)
 {
     if (a.x1_dtype != DT_E4M3 || a.x2_dtype != DT_E4M3 || a.batch != 1 || a.bias) return false;
     if (a.out_dtype != DT_BF16 && a.out_dtype != DT_F16 && a.out_dtype != DT_F32) return false;
     if (a.M <= 16 || a.M > 128) return false;
     if (a.gsK != 128 || a.gsN != 128 || (a.gsM != 1 && a.gsM != 128)) return false;
-    // the kernel's shape conditions: whole workgroups of 128 columns inside one scale block, K in slabs of 128 with the
-    // weight stream four chunks deep, 16-byte pieces
-    if (a.N % 128 != 0 || a.N < 256 || a.K % 512 != 0 || a.K / 128 * 16 * (a.M > 64 ? 8 : 4) * 4 > 65536) return false;
+    // the kernel's shape conditions: whole workgroups of 128 columns inside one scale block, K in slabs of 128, 16-byte
+    // pieces, the products of the block scales of one workgroup's K (all of K, or its longest segment) in 64 KB of LDS
+    if (a.N % 128 != 0 || a.N < 256 || a.K % 128 != 0) return false;
+    {
+        const int ks = rows_ksplit(a);
+        const int64_t blocks = (a.K / 128 + ks - 1) / ks;
+        if (blocks * 16 * (rows_per_slab(a) > 64 ? 8 : 4) * 4 > 65536) return false;
+    }
     if (a.x1.col_stride != 1 || a.x2.row_stride != 1 || a.x1.row_stride < a.K || a.x2.col_stride < a.K) return false;
     if (((uintptr_t)a.x1.ptr | (uintptr_t)a.x2.ptr | (uint64_t)a.x1.row_stride | (uint64_t)a.x2.col_stride) % 16) return false;
     if (((uintptr_t)a.x1_scale_mat.ptr | (uintptr_t)a.x2_scale_mat.ptr) % 4 || (uintptr_t)a.out % 16) return false;
@@ -50,10 +69,15 @@ bool rows_eligible(const OpsnnQmmArgs& a)
 }  // namespace
 
 uint64_t blockscale_rows_workspace(const OpsnnQmmArgs& a) { return rows_eligible(a) ? (uint64_t)a.M * (uint64_t)a.K * 2 : 0; }
+// the K segments that kernel would run in (1: K in one piece, or another kernel's call): fp32 partial sums [segments][M][N]
+int blockscale_rows_ksplit(const OpsnnQmmArgs& a) { return rows_eligible(a) ? rows_ksplit(a) : 1; }
 
-int launch_blockscale_rows(const OpsnnQmmArgs& a, hipStream_t st)
+int launch_blockscale_rows(const OpsnnQmmArgs& a, hipStream_t st, SplitK sk)
 {
     if (!rows_eligible(a) || !a.workspace || (uintptr_t)a.workspace % 16) return OPSNN_NOT_TAKEN;
+    int64_t kunit = 0;
+    const int ks = rows_ksplit(a, &kunit);
+    if (ks > 1 && (!sk.part || sk.splits < ks)) return OPSNN_NOT_TAKEN;   // (eligibility counted on the segments' scale tables)
     uint16_t* x16 = (uint16_t*)a.workspace;
     const int64_t pieces = a.M * (a.K / 16);
     hipLaunchKernelGGL(widen_e4m3_f16_kernel, dim3((unsigned)((pieces + 255) / 256)), dim3(256), 0, st, (const uint8_t*)a.x1.ptr, a.x1.row_stride, x16,
@@ -67,8 +91,9 @@ int launch_blockscale_rows(const OpsnnQmmArgs& a, hipStream_t st)
     p.bs1 = (const float*)a.x1_scale_mat.ptr; p.bs1_rs = a.x1_scale_mat.row_stride; p.bs1_cs = a.x1_scale_mat.col_stride;
     p.bs2 = (const float*)a.x2_scale_mat.ptr; p.bs2_rs = a.x2_scale_mat.row_stride; p.bs2_cs = a.x2_scale_mat.col_stride;
     p.bs_gsm = (int)a.gsM; p.bs_out_dt = a.out_dtype;
-    if (a.M > 64 && (a.N + 127) / 128 <= 128) {   // narrow x2 (at most 128 workgroups): two slabs of 64 rows in one launch, twice the workgroups
-        p.m_rows = 64; p.m_slab = 64; p.m_end = a.M;
+    if (ks > 1) { p.ksplit = ks; p.kunit = kunit; p.part = sk.part; }
+    if (const int64_t slab = wq_narrow_slab_rows(a.M, a.N, true)) {   // narrow x2 (at most 128 workgroups): two slabs in one launch, twice the workgroups
+        p.m_rows = slab; p.m_slab = slab; p.m_end = a.M;
         return launch_rows_one<DT_F16, 8, 4, 2, 4, 2, false, 3>(p, st);
     }
     return a.M > 64 ? launch_rows_one<DT_F16, 8, 8, 2, 4, 2, false, 3>(p, st) : launch_rows_one<DT_F16, 8, 4, 2, 4, 2, false, 3>(p, st);

@@ -429,7 +429,7 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(NW == 8
 template <int XDT, int WBITS, int MB, int NB, int WN, int WK, bool HAS_OFF, int WF = 0, bool SLDS = false, bool KSP = false>
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void wqmm_rows_kernel(WqParams p)
 {
-    static_assert(!KSP || WF <= 2, "K in segments: the weight-only forms");
+    static_assert(!KSP || WF <= 3, "K in segments: the weight-only forms and the fp8 block-scale form");
     static_assert(WN * WK == 8, "eight waves");
     static_assert(!SLDS || WF == 0 || WF == 2, "the scale table serves the integer forms and the e8m0 bytes of e2m1 codes");
     static_assert(WF == 0 || !HAS_OFF, "floating-point weight codes have no offset");
@@ -477,6 +477,10 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void w
             p.x += k0;
             p.w += k0 * WBITS / 8;
             if constexpr (WF == 2) p.scale = (const uint16_t*)((const uint8_t*)p.scale + k0 / 32);   // one e8m0 byte per 32 k
+            else if constexpr (WF == 3) {   // the block scales of the segment's first 128-block
+                p.bs1 += (k0 / 128) * p.bs1_cs;
+                p.bs2 += (k0 / 128) * p.bs2_rs;
+            }
             else if (p.group < p.K) {
                 const int64_t g0 = (k0 / p.group) * p.s_rs;
                 p.scale += g0;
@@ -1428,6 +1432,19 @@ __global__ __launch_bounds__(256) void wq_splitk_reduce_kernel(const float* part
     }
 }
 
+// the fp8 block-scale form of the many-rows kernel: out[i] = cast(sum over the K segments, in order, of part[s, i])
+// (a template only so that every translation unit that includes this header may hold a copy)
+template <typename = void>
+__global__ __launch_bounds__(256) void rows_bs_splitk_reduce_kernel(const float* part, int splits, int64_t total, void* out, int out_dt)
+{
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
+        const float v = splitk_sum(part, splits, total, i);
+        if (out_dt == DT_F32) ((float*)out)[i] = v;
+        else ((uint16_t*)out)[i] = out_dt == DT_BF16 ? bf16_bits(v) : f16_bits(v);
+    }
+}
+
 // One workgroup per CU (its waves fill the register file), or one per row block when there are fewer; with K split into
 // `splits` segments one workgroup column per segment, the CUs shared between the columns.
 template <int XDT, int WBITS, int NW, int NCH, bool HAS_OFF, int SCM, bool WFLT = false, bool TWO = false>
@@ -1545,7 +1562,7 @@ static int launch_rows_one(const WqParams& p, hipStream_t st)
 {
     if constexpr (!KSP) {   // K in segments: the instantiations of the 64-row instance with 128-column workgroups that know them
         if (p.ksplit > 1) {
-            if constexpr (MB == 4 && NB == 2 && WN == 4 && WK == 2 && WF <= 2 && !SLDS) return launch_rows_one<XDT, WBITS, MB, NB, WN, WK, HAS_OFF, WF, false, true>(p, st);
+            if constexpr (MB == 4 && NB == 2 && WN == 4 && WK == 2 && WF <= 3 && !SLDS) return launch_rows_one<XDT, WBITS, MB, NB, WN, WK, HAS_OFF, WF, false, true>(p, st);
             else return -1;
         }
     }
@@ -1585,7 +1602,7 @@ static int launch_rows_one(const WqParams& p, hipStream_t st)
     constexpr size_t lds_red = (size_t)WN * (WK - 1) * NB * MB * 4 * 64 * 4;
     constexpr size_t lds_main = lds_x > lds_red ? lds_x : lds_red;
     constexpr size_t lds_table = WF == 3 ? 65536 : 0;   // products of the block scales: (K / 128) * 16 MB floats, at most this
-    const size_t lds = lds_main + (WF == 3 ? (size_t)(p.K / 128) * 16 * MB * 4 : 0) + lds_stab;
+    const size_t lds = lds_main + (WF == 3 ? (size_t)(kseg / 128) * 16 * MB * 4 : 0) + lds_stab;
     if (lds > lds_main + lds_table + lds_stab) return OPSNN_NOT_TAKEN;
     const unsigned grid = (unsigned)((p.N + 16 * NB * WN - 1) / (16 * NB * WN));
     const int64_t slabs = p.m_slab > 0 ? (p.m_end - p.m_base + p.m_slab - 1) / p.m_slab : 1;
@@ -1601,6 +1618,11 @@ static int launch_rows_one(const WqParams& p, hipStream_t st)
     if (hipError_t e = hipGetLastError(); e != hipSuccess) return (int)e;
     if (split) {
         const int64_t total = p.M * p.N;
+        if constexpr (WF == 3) {
+            hipLaunchKernelGGL(rows_bs_splitk_reduce_kernel<void>, dim3(splitk_reduce_grid(total)), dim3(256), 0, st, (const float*)p.part, p.ksplit, total,
+                               (void*)p.y, p.bs_out_dt);
+            return (int)hipGetLastError();
+        }
         hipLaunchKernelGGL(wq_splitk_reduce_kernel<XDT>, dim3(splitk_reduce_grid(total)), dim3(256), 0, st, (const float*)p.part, p.ksplit, total, p.N,
                            p.bias, p.bias_dt, p.y);
         return (int)hipGetLastError();

@@ -112,11 +112,46 @@ def test_fp8_blockscale_fp32_output(gpu, M, K, N, tB, gsM, fast):
     assert np.array_equal(cases.run_blockscale_aclnn(m, inp, M, K, N, tB, m.ACL_FLOAT), want)
 
 
+def _rows_ksplit(wbits, M, N, K, group):
+    """The many-rows kernel's K segments (the library's rule, restated): 1 = K in one piece."""
+    if M < 17 or N % 32 or N < 256 or K < 4096:
+        return 1
+    wg = -(-N // 128)
+    slabs = 1
+    if M > 64:
+        if wg > 128:
+            return 1
+        n = max(min(256 // wg, -(-M // 64)), -(-M // 256))
+        if n < 2:
+            return 1
+        slab = -(-(-(-M // n)) // 16) * 16
+        slabs = -(-M // slab)
+    wgs, kx = slabs * wg, 2 * 4 * (128 // wbits)
+    unit = kx
+    if group < K:
+        unit = max(kx, group)
+        if unit % group or unit % kx:
+            return 1
+    if wgs > 128 or K % unit:
+        return 1
+    if K < 8192 and (K % (2 * kx) == 0 or wgs > 64 or M < 33):
+        return 1
+    s = min(256 // wgs, 8, K // 2048, K // unit)
+    if s == 2 and wgs > 64 and K < 12288:
+        return 1
+    return s if s >= 2 else 1
+
+
 @pytest.mark.parametrize("M,K,N,gsM,out", [
     # up to 16 rows (one pass): K shared by 16 waves (2048, 4096, 8192) or by 8 (1024, 3072, 5120, 6144, 7168); ragged columns;
     # more column blocks than workgroups (N = 8192: 512 blocks on 256 workgroups) and fewer
     (1, 2048, 256, 1, "bf16"), (16, 4096, 512, 1, "f16"), (7, 8192, 8192, 1, "bf16"), (16, 1024, 264, 1, "bf16"),
     (5, 3072, 1000, 1, "f16"), (16, 5120, 384, 1, "f32"), (9, 6144, 256, 128, "bf16"), (16, 7168, 2304, 1, "bf16"),
+    # K that the waves of one workgroup do not share exactly: one segment with idle waves (28 blocks on 16 waves of two), or K
+    # segments over workgroup columns with fp32 partial sums and a second kernel (86 blocks: three segments of 16 x 2; 144:
+    # three of 8 x 6; 108: seven of 16 x 1; 19: three of 8 x 1; 148 in two passes: five of 16 x 2)
+    (5, 3584, 264, 1, "f16"), (16, 11008, 512, 1, "bf16"), (16, 18432, 256, 1, "bf16"), (12, 13824, 384, 128, "f32"),
+    (16, 2432, 256, 1, "f16"), (32, 18944, 264, 1, "bf16"),
     # 17 .. 32 rows where the many-rows kernel does not apply (N % 128, K % 512): two passes; one scale row for all of x1 (B-B)
     (17, 2048, 520, 1, "bf16"), (32, 7168, 520, 128, "f16"), (24, 1024, 256, 1, "f32"), (20, 4096, 256, 1, "f32"),
     # 17 .. 64 rows (N % 128 == 0, K % 512 == 0): x1 widened into the workspace, the many-rows streaming kernel
@@ -124,6 +159,10 @@ def test_fp8_blockscale_fp32_output(gpu, M, K, N, tB, gsM, fast):
     (40, 1536, 2304, 1, "bf16"),
     # 65 .. 128 rows: the same kernel's 128-row instance
     (65, 2048, 512, 1, "bf16"), (128, 7168, 1024, 1, "f16"), (100, 1024, 256, 128, "f32"), (96, 16384, 256, 1, "bf16"),
+    # ... K in whole scale blocks but no whole rounds of the chunk pipeline; K segments against a narrow x2 (86 blocks in five,
+    # 148 in eight, 144 in four with two row slabs; 17 .. 32 rows as well)
+    (40, 1664, 256, 1, "bf16"), (64, 11008, 512, 1, "f16"), (50, 18944, 256, 128, "bf16"), (128, 18432, 1024, 1, "f32"),
+    (24, 13824, 384, 1, "bf16"),
 ])
 def test_fp8_blockscale_decode_rows(gpu, M, K, N, gsM, out):
     """The block-scale modes with up to 32 rows of x1 (x2 K-contiguous): x1 stays in registers as exact fp16 and x2 is
@@ -144,13 +183,15 @@ def test_fp8_blockscale_decode_rows(gpu, M, K, N, gsM, out):
         differ = float(np.mean(got != want))
         print(f"   {differ:.2e} of outputs differ from the ascending-block oracle", flush=True)
         assert differ < 2e-2
-    if M > 16 and N % 128 == 0 and K % 512 == 0:   # phase 1 plans the fp16 copy of x1: the many-rows route is the one taken
+    if M > 32 and N % 128 == 0:   # phase 1 plans the fp16 copy of x1 (and the partial sums of a K split): the many-rows route is the one taken
         d = {k: m.DeviceBuffer(host=v) for k, v in inp.items() if isinstance(v, np.ndarray)}
         x1 = m.Tensor((M, K), m.ACL_FLOAT8_E4M3FN, d["x1"]); x2 = m.Tensor((N, K), m.ACL_FLOAT8_E4M3FN, d["x2"])
         s1 = m.Tensor(inp["s1"].shape[1:], m.ACL_FLOAT, d["s1"]); s2 = m.Tensor(inp["s2"].shape[1:], m.ACL_FLOAT, d["s2"])
         o = m.Tensor((M, N), dt, m.DeviceBuffer(M * N * 4))
         rc, ws, ex = m.quant_matmul_v5_get_workspace(x1, x2, s1, s2, o, transpose_x2=True, group_size=(gsM << 32) | (128 << 16) | 128)
-        assert rc == 0 and ws == M * K * 2, (rc, ws)
+        ks = _rows_ksplit(8, M, N, K, K)
+        part = -(-ks * M * N * 4 // 256) * 256 if ks > 1 else 0
+        assert rc == 0 and ws == part + M * K * 2, (rc, ws, ks)
         m.lib().aclDestroyAclOpExecutor(ex)
     plain(True)
     assert np.array_equal(cases.run_blockscale_aclnn(m, inp, M, K, N, True, dt), want)

@@ -242,6 +242,11 @@ def test_gpu_matches_oracle(gpu, M, K, N, in_dt, s_dt, s_len, bias_dt, out_dt, t
     (16, 7168, 1000, "N", False, "f16", "M"),
     (20, 2048, 264, "N", True, "bf16", "M"),
     (32, 1024, 256, 1, True, "f16", True),
+    # ... a K that one workgroup's waves do not share exactly: one segment with idle waves, K segments with partial sums
+    (16, 3584, 264, "N", True, "bf16", "M"),
+    (16, 11008, 256, "N", True, "f16", "M"),
+    (9, 18432, 520, "N", False, "bf16", "M"),
+    (16, 13824, 256, 1, True, "f16", True),
     # 33 .. 64 rows (N % 32 == 0, K % 512 == 0): x1 widened into the workspace, the many-rows streaming kernel
     (40, 2048, 512, "N", True, "bf16", "M"),
     (64, 7168, 288, "N", False, "f16", "M"),

@@ -252,6 +252,8 @@ def test_gpu_pertile_i8(gpu, M, K, N, tB):
                                       # up to 32 rows: x1 in registers, x2 streamed once per 16 rows (int8 instructions)
                                       (16, 4096, 512, True), (9, 2048, 264, True), (24, 1024, 520, True), (16, 1024, 256, False),
                                       (1, 7168, 384, True),
+                                      # ... a K that one workgroup's waves do not share exactly: idle waves, K segments
+                                      (16, 3584, 256, True), (16, 11008, 264, True), (20, 18432, 256, True),
                                       # few tiles against a long K: the K split ((640, 1024, 520) above: with the re-layout of
                                       # an N-contiguous x2 behind the partial sums in the workspace)
                                       (128, 4096, 4096, True), (40, 8192, 256, True), (96, 1024, 258, True), (200, 2048, 1000, False)])
