@@ -156,19 +156,20 @@ inline int wq_part_slices(int wbits, int64_t M, int64_t N, int64_t K, int64_t gr
 // A K that the waves of one workgroup share exactly runs as one segment; any other whole number of blocks in 1 .. 16
 // segments of NW * NBLK blocks, the last one with idle waves (K a whole number of NBLK blocks): the layout with the fewest
 // wave slots, then the fewest segments.  More than one segment needs room for fp32 partial sums (may_split).
+// (w4: the fp8 x fp4 MX form of the kernel, which has no instance of 16 waves with one block each.)
 struct QmmDecodePlan { int nw = 0, nblk = 0, splits = 1; };
-inline bool qmm_decode_plan(int64_t K, bool may_split, QmmDecodePlan& pl)
+inline bool qmm_decode_plan(int64_t K, bool may_split, QmmDecodePlan& pl, bool w4 = false)
 {
     if (K <= 0 || K % 128 != 0) return false;
     const int64_t nb = K / 128;
-    if (nb % 16 == 0 && nb / 16 <= 4 && nb / 16 != 3) { pl.nw = 16; pl.nblk = (int)(nb / 16); pl.splits = 1; return true; }
+    if (nb % 16 == 0 && nb / 16 <= 4 && nb / 16 != 3 && !(w4 && nb == 16)) { pl.nw = 16; pl.nblk = (int)(nb / 16); pl.splits = 1; return true; }
     if (nb % 8 == 0 && nb / 8 <= 7) { pl.nw = 8; pl.nblk = (int)(nb / 8); pl.splits = 1; return true; }
     static const int shapes[10][2] = {{16, 4}, {16, 2}, {16, 1}, {8, 7}, {8, 6}, {8, 5}, {8, 4}, {8, 3}, {8, 2}, {8, 1}};
     int64_t best_slots = 0;
     bool found = false;
     for (const auto& sh : shapes) {
         const int nw = sh[0], nblk = sh[1];
-        if (nb % nblk != 0) continue;
+        if (nb % nblk != 0 || (w4 && nw == 16 && nblk == 1)) continue;
         const int64_t waves = nb / nblk, s = (waves + nw - 1) / nw;
         if (s > 16 || (s > 1 && !may_split)) continue;
         const int64_t slots = s * nw * nblk;

@@ -603,14 +603,15 @@ int launch_rowcol_exact(const OpsnnQmmArgs& a, hipStream_t st, int ep_mode, Spli
 // fp8 e4m3 x fp4 e2m1 with e8m0 scales per 32 K on both operands (compute_mx of quant_batch_matmul_v4,
 // qbmmv4_kernel_golden.py:119-186): the MX mode with a 4-bit x2.  x2 [N, K] K-contiguous (two elements per byte),
 // K % 128 == 0, bias fp32 or 16-bit.
-int launch_mx_a8w4_decode(const OpsnnQmmArgs& a, hipStream_t st);   // qmm_fp8_decode.hip
+int launch_mx_a8w4_decode(const OpsnnQmmArgs& a, hipStream_t st, SplitK sk);   // qmm_fp8_decode.hip
 
 int launch_mx_a8w4_mfma(const OpsnnQmmArgs& a, hipStream_t st, SplitK sk)
 {
     if (a.x1_dtype != DT_E4M3 || a.x2_dtype != DT_E2M1) return OPSNN_NOT_TAKEN;
     {   // up to 32 rows: the stream over x2 with x1 in registers
-        const int rc = launch_mx_a8w4_decode(a, st);
+        const int rc = launch_mx_a8w4_decode(a, st, sk);
         if (rc != OPSNN_NOT_TAKEN) return rc;
+        if (a.M <= 32) sk = SplitK{};   // (the partial sums were laid out for the kernel above; the tile kernel runs unsplit)
     }
     if (a.out_dtype != DT_BF16 && a.out_dtype != DT_F16) return OPSNN_NOT_TAKEN;
     if (a.K % 128 != 0 || a.M * a.N < 64 * 64 || a.x1.col_stride != 1 || a.x2.row_stride != 1) return OPSNN_NOT_TAKEN;

@@ -279,16 +279,26 @@ struct MxW4DecParams {
     void* out; int out_dt;
     int64_t M, N, K;
     const void* bias; int bias_dt;
+    // K in segments (SEG instantiations, gridDim.y of them): fp32 sums of this pass's rows, slice s at part + s * part_slice
+    float* part; int64_t part_slice;
 };
 
-template <int NW, int NCH>
+// SEG: as in fp8_block_decode_kernel -- gridDim.y segments of NW * NCH chunks, idle waves past the end of K, fp32 sums
+// for mxw4dec_reduce_kernel when there is more than one segment.
+template <int NW, int NCH, bool SEG = false>
 __global__ __launch_bounds__(NW * 64) void mx_a8w4_decode_kernel(MxW4DecParams p)
 {
     extern __shared__ __attribute__((aligned(16))) float red[];   // [2][NW][256]
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int nrow = lane & 15, q = lane >> 4;
-    const int64_t kbase = (int64_t)wave * (NCH * 128);   // this wave's K range, in elements
+    int64_t kbase = (int64_t)wave * (NCH * 128);   // this wave's K range, in elements
+    bool live = true;
+    if constexpr (SEG) {
+        kbase = ((int64_t)blockIdx.y * NW + wave) * (NCH * 128);
+        live = kbase < p.K;
+        if (!live) kbase = p.K - NCH * 128;
+    }
     const int nblocks = (int)((p.N + 15) / 16);
     const int M = (int)p.M;
 
@@ -347,6 +357,9 @@ __global__ __launch_bounds__(NW * 64) void mx_a8w4_decode_kernel(MxW4DecParams p
             acc = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf, xf[c], acc, 4, 0, 0, (int)(sw >> (8 * q)), 0, xs[c]);
         }
         // acc[r]: m = lane % 16, n = n0 + 4 (lane / 16) + r, over this wave's K range
+        if constexpr (SEG) {
+            if (!live) acc = (v4f){0.0f, 0.0f, 0.0f, 0.0f};
+        }
         float* mine = red + ((it & 1) * NW + wave) * 256;
         *(v4f*)(mine + lane * 4) = acc;
         __syncthreads();
@@ -361,6 +374,15 @@ __global__ __launch_bounds__(NW * 64) void mx_a8w4_decode_kernel(MxW4DecParams p
         }
         if (nrow >= M) continue;
         const int64_t n = n0 + 4 * q;
+        if constexpr (SEG) {
+            if (gridDim.y > 1) {
+                float* dst = p.part + (int64_t)blockIdx.y * p.part_slice + (int64_t)nrow * p.N + n;
+#pragma unroll
+                for (int r = 0; r < 4; r++)
+                    if (n + r < p.N) dst[r] = sum[r];
+                continue;
+            }
+        }
         if (p.bias) {
 #pragma unroll
             for (int r = 0; r < 4; r++) sum[r] = sum[r] + load_scalar_as_f32(p.bias, p.bias_dt, n + r < p.N ? n + r : p.N - 1);
@@ -376,13 +398,33 @@ __global__ __launch_bounds__(NW * 64) void mx_a8w4_decode_kernel(MxW4DecParams p
     }
 }
 
-template <int NW, int NCH>
-int launch_mxw4_one(const MxW4DecParams& p, hipStream_t st)
+// out = cast(sum over the K segments, in order, of part[s] + bias) for one pass of up to 16 rows
+__global__ __launch_bounds__(256) void mxw4dec_reduce_kernel(MxW4DecParams p, int splits)
 {
+    const int64_t total = p.M * p.N, stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
+        float v = p.part[i];
+        for (int s = 1; s < splits; s++) v = v + p.part[(int64_t)s * p.part_slice + i];
+        if (p.bias) v = v + load_scalar_as_f32(p.bias, p.bias_dt, i % p.N);
+        ((uint16_t*)p.out)[i] = p.out_dt == DT_BF16 ? bf16_bits(v) : f16_bits(v);
+    }
+}
+
+template <int NW, int NCH, bool SEG = false>
+int launch_mxw4_one(const MxW4DecParams& p, hipStream_t st, int splits = 1)
+{
+    if constexpr (!SEG) {
+        if (splits > 1 || p.K != (int64_t)NW * NCH * 128) return launch_mxw4_one<NW, NCH, true>(p, st, splits);
+    }
+    const int64_t nbk = p.K / 128;
+    if (splits < 1 || splits > 16 || nbk % NCH != 0 || nbk < NCH || (int64_t)splits * NW * NCH < nbk || (splits > 1 && !p.part)) return -1;
     const int nblocks = (int)((p.N + 15) / 16);
-    const int grid = nblocks < 256 ? nblocks : 256;
+    const int cus = 256 / splits;   // the CUs shared between the segments' workgroup columns
+    const int grid = nblocks < cus ? nblocks : cus;
     const size_t lds = (size_t)2 * NW * 256 * sizeof(float);
-    hipLaunchKernelGGL((mx_a8w4_decode_kernel<NW, NCH>), dim3((unsigned)grid), dim3(NW * 64), lds, st, p);
+    hipLaunchKernelGGL((mx_a8w4_decode_kernel<NW, NCH, SEG>), dim3((unsigned)grid, (unsigned)splits), dim3(NW * 64), lds, st, p);
+    if (hipError_t e = hipGetLastError(); e != hipSuccess || splits == 1) return (int)e;
+    hipLaunchKernelGGL(mxw4dec_reduce_kernel, dim3(splitk_reduce_grid(p.M * p.N)), dim3(256), 0, st, p, splits);
     return (int)hipGetLastError();
 }
 
@@ -456,7 +498,7 @@ int launch_rowcol_decode(const OpsnnQmmArgs& a, hipStream_t st, SplitK sk)
 
 // fp8 x fp4 MX with up to 32 rows of x1 (two passes beyond 16): K a whole number of 128-element chunks that 16 waves
 // share 2 or 4 each, or 8 waves 1 .. 7 each; K-contiguous operands and scales; OPSNN_NOT_TAKEN otherwise.
-int launch_mx_a8w4_decode(const OpsnnQmmArgs& a, hipStream_t st)
+int launch_mx_a8w4_decode(const OpsnnQmmArgs& a, hipStream_t st, SplitK sk)
 {
     if (a.x1_dtype != DT_E4M3 || a.x2_dtype != DT_E2M1 || a.batch != 1) return OPSNN_NOT_TAKEN;
     if (a.out_dtype != DT_BF16 && a.out_dtype != DT_F16) return OPSNN_NOT_TAKEN;
@@ -469,11 +511,9 @@ int launch_mx_a8w4_decode(const OpsnnQmmArgs& a, hipStream_t st)
     if (((uintptr_t)a.x1_scale_mat.ptr | (uintptr_t)a.x2_scale_mat.ptr | (uint64_t)a.x1_scale_mat.row_stride | (uint64_t)a.x2_scale_mat.row_stride) % 4)
         return OPSNN_NOT_TAKEN;
     if (a.x1_scale_mat.row_stride < a.K / 32 || a.x2_scale_mat.row_stride < a.K / 32) return OPSNN_NOT_TAKEN;
-    const int64_t nb = a.K / 128;
-    int nw = 0, nch = 0;
-    if (nb % 16 == 0 && (nb / 16 == 2 || nb / 16 == 4)) { nw = 16; nch = (int)(nb / 16); }
-    else if (nb % 8 == 0 && nb / 8 <= 7) { nw = 8; nch = (int)(nb / 8); }
-    else return OPSNN_NOT_TAKEN;
+    QmmDecodePlan pl;
+    if (!qmm_decode_plan(a.K, sk.part != nullptr, pl, true) || pl.splits > (sk.part ? sk.splits : 1)) return OPSNN_NOT_TAKEN;
+    const int nw = pl.nw, nch = pl.nblk, splits = pl.splits;
     for (int64_t m0 = 0; m0 < a.M; m0 += 16) {
         MxW4DecParams p{};
         p.M = a.M - m0 < 16 ? a.M - m0 : 16; p.N = a.N; p.K = a.K;
@@ -483,16 +523,18 @@ int launch_mx_a8w4_decode(const OpsnnQmmArgs& a, hipStream_t st)
         p.sa_rs = a.x1_scale_mat.row_stride; p.sb_rs = a.x2_scale_mat.row_stride;
         p.out_dt = a.out_dtype; p.out = (char*)a.out + m0 * a.N * 2;
         p.bias = a.bias; p.bias_dt = a.bias_dtype;
-        int rc;
-        if (nw == 16) rc = nch == 2 ? launch_mxw4_one<16, 2>(p, st) : launch_mxw4_one<16, 4>(p, st);
+        p.part = sk.part ? sk.part + m0 * a.N : nullptr; p.part_slice = a.M * a.N;
+        int rc = -1;
+        if (nw == 16) rc = nch == 2 ? launch_mxw4_one<16, 2>(p, st, splits) : nch == 4 ? launch_mxw4_one<16, 4>(p, st, splits) : -1;
         else switch (nch) {
-            case 1: rc = launch_mxw4_one<8, 1>(p, st); break;
-            case 2: rc = launch_mxw4_one<8, 2>(p, st); break;
-            case 3: rc = launch_mxw4_one<8, 3>(p, st); break;
-            case 4: rc = launch_mxw4_one<8, 4>(p, st); break;
-            case 5: rc = launch_mxw4_one<8, 5>(p, st); break;
-            case 6: rc = launch_mxw4_one<8, 6>(p, st); break;
-            default: rc = launch_mxw4_one<8, 7>(p, st); break;
+            case 1: rc = launch_mxw4_one<8, 1>(p, st, splits); break;
+            case 2: rc = launch_mxw4_one<8, 2>(p, st, splits); break;
+            case 3: rc = launch_mxw4_one<8, 3>(p, st, splits); break;
+            case 4: rc = launch_mxw4_one<8, 4>(p, st, splits); break;
+            case 5: rc = launch_mxw4_one<8, 5>(p, st, splits); break;
+            case 6: rc = launch_mxw4_one<8, 6>(p, st, splits); break;
+            case 7: rc = launch_mxw4_one<8, 7>(p, st, splits); break;
+            default: break;
         }
         if (rc != 0) return rc;
     }

@@ -142,6 +142,9 @@ def test_gpu_a8w4_mx(gpu, M, K, N, tB):
                                    # chunks of 128 each) or by 8 (1 .. 7), ragged columns, two passes
                                    (16, 4096, 512), (9, 8192, 264), (24, 1024, 520), (1, 7168, 384), (32, 3072, 256),
                                    (16, 2048, 256),
+                                   # ... a K that one workgroup's waves do not share exactly: one segment with idle waves (28
+                                   # chunks), K segments with fp32 partial sums (86, 144, 19 chunks; two passes; one row)
+                                   (16, 3584, 256), (16, 11008, 264), (32, 18432, 256), (7, 2432, 512), (1, 18944, 384),
                                    # few tiles against a long K: K split over 2 .. 16 workgroups per tile, fp32 partial sums in the
                                    # workspace, summed in split order (also (512, 2048, 520), (100, 1024, 1000) and
                                    # (1024, 4096, 1024) above); a column count that is no multiple of 4
