@@ -20,7 +20,8 @@ int launch_rowcol_decode(const OpsnnQmmArgs& a, hipStream_t st, SplitK sk);   //
 uint64_t blockscale_rows_workspace(const OpsnnQmmArgs& a);         // qmm_fp8_rows.hip
 int blockscale_rows_ksplit(const OpsnnQmmArgs& a);
 uint64_t rowcol_rows_workspace(const OpsnnQmmArgs& a);
-int launch_rowcol_rows(const OpsnnQmmArgs& a, hipStream_t st);
+int launch_rowcol_rows(const OpsnnQmmArgs& a, hipStream_t st, SplitK sk);
+int rowcol_rows_ksplit(const OpsnnQmmArgs& a);
 int launch_tcg_mfma(const OpsnnQmmArgs& a, hipStream_t st);
 uint64_t tcg_workspace_bytes(const OpsnnQmmArgs& a);
 int launch_kg_mfma(const OpsnnQmmArgs& a, hipStream_t st);   // qmm_i4_kg.hip
@@ -197,14 +198,16 @@ static int splitk_for(const OpsnnQmmArgs& a, int mode)
         QmmDecodePlan pl;
         const int sd = qmm_decode_plan(a.K, true, pl, a8w4) ? pl.splits : 1;
         // (17 .. 32 rows of fp8 with block scales may also run on the many-rows kernel, with its own segments: room for either)
-        const int sr = mode == 1 && f8 ? blockscale_rows_ksplit(a) : 1;
+        const int sr = mode == 1 && f8 ? blockscale_rows_ksplit(a) : mode == 3 && f8 ? rowcol_rows_ksplit(a) : 1;
         return sd > sr ? sd : sr;
     }
-    // 33 .. 128 rows of fp8 with block scales on the many-rows kernel
-    if (mode == 1 && f8 && a.M <= 128) {
-        if (const int sr = blockscale_rows_ksplit(a); sr > 1) return sr;
+    // 33 .. 128 rows of fp8 with block scales or row / column scales on the many-rows kernel
+    if ((mode == 1 || mode == 3) && f8 && a.M <= 128) {
+        if (const int sr = mode == 1 ? blockscale_rows_ksplit(a) : rowcol_rows_ksplit(a); sr > 1) return sr;
     }
-    if (a.M * a.N < 64 * 64 || a.K < 1024) return 1;
+    // (fewer than 64 x 64 outputs are the plain kernels' -- except int8 with few outputs against a long K, qmm_int8.hip)
+    const bool tiny = a.M * a.N < 64 * 64;
+    if ((tiny && !(a.N >= 256 && a.M * a.N * a.K >= (1ll << 22))) || a.K < 1024) return 1;
     int64_t bm, bn = 256, kunit = 128;
     double tile_us;   // one K tile (kunit elements) of the kernel in question, measured on calls with few tiles
     double bytes_per_us = 5.0e6;   // what its partial sums' traffic was measured to cost (splitk_factor)
@@ -216,6 +219,7 @@ static int splitk_for(const OpsnnQmmArgs& a, int mode)
         // splits, 64 rows 20 -> 15 us, 128 rows 19.5 -> 22, 256 rows in four 21 -> 24)
         bm = 128; bn = 128; tile_us = 0.55; bytes_per_us = 2.4e6;
     }
+    else if (tiny) return 1;
     // MXFP4: 128 x 128 tiles when 256 x 256 ones would be few (the launcher's rule), K tiles counted in 256 elements
     else if (mode == 2 && a.x1_dtype == DT_E2M1 && a.x2_dtype == DT_E2M1 && (out16 || a.out_dtype == DT_F32)) {
         const int64_t t256 = ((a.M + 255) / 256) * ((a.N + 255) / 256) * a.batch;
@@ -353,7 +357,7 @@ extern "C" int opsnnQmmTc(const OpsnnQmmArgs* a, void* stream)
     if (f8 && a->force_variant != OPSNN_VARIANT_PLAIN && !opsnn_force_plain()) {
         const int ep = !a->x1_scale ? 1 : (a->x1_scale_len == 1 && a->x2_scale_len == 1 && !a->bias) ? 2 : 0;
         if (ep == 0) {   // 17 .. 128 rows: the many-rows streaming kernel; up to 16 (32 in two passes where that does not apply): x1 in registers
-            int rc = launch_rowcol_rows(*a, (hipStream_t)stream);
+            int rc = launch_rowcol_rows(*a, (hipStream_t)stream, sk);
             if (rc != OPSNN_NOT_TAKEN) return rc;
             rc = launch_rowcol_decode(*a, (hipStream_t)stream, sk);
             if (rc != OPSNN_NOT_TAKEN) return rc;

@@ -301,7 +301,7 @@ __global__ void qmm_i4_asym_plain(OpsnnQmmArgs a)
 }
 int launch_fp8_rowcol_mfma(const OpsnnQmmArgs& a, hipStream_t st, bool merged_scales_ok, SplitK sk = {});   // qmm_fp8_block.hip
 
-int launch_rowcol_rows(const OpsnnQmmArgs& a, hipStream_t st);      // qmm_fp8_rows.hip
+int launch_rowcol_rows(const OpsnnQmmArgs& a, hipStream_t st, SplitK sk);      // qmm_fp8_rows.hip
 int launch_rowcol_decode(const OpsnnQmmArgs& a, hipStream_t st, SplitK sk);    // qmm_fp8_decode.hip
 void* weight_cache_blob3(const void* src, const void* src2, const void* src3, int64_t K, int64_t N, int bits, int64_t nb, uint64_t bytes, hipStream_t st,
                          bool* fresh);   // weight_cache.hip
@@ -368,7 +368,7 @@ int launch_tcg_mfma(const OpsnnQmmArgs& a, hipStream_t st)
     b.x2_scale = cs; b.x2_scale_dtype = DT_F32; b.x2_scale_len = a.N;
     b.workspace = tcg_rows_bytes(a) ? (char*)a.workspace + blob + tcg_x1pad_bytes(a) : nullptr;
     if (a.force_variant == 0) {
-        int rc = launch_rowcol_rows(b, st);
+        int rc = launch_rowcol_rows(b, st, SplitK{});
         if (rc != OPSNN_NOT_TAKEN) return rc;
         rc = launch_rowcol_decode(b, st, SplitK{});
         if (rc != OPSNN_NOT_TAKEN) return rc;

@@ -106,7 +106,7 @@ static bool rowcol_rows_eligible(const OpsnnQmmArgs& a)
     if (a.out_dtype != DT_BF16 && a.out_dtype != DT_F16 && a.out_dtype != DT_F32) return false;
     if (!a.x1_scale || !a.x2_scale || a.x2_scale_dtype != DT_F32 || (a.bias && a.bias_dtype != DT_F32)) return false;
     if (a.x1_scale_len == 1 && a.x2_scale_len == 1 && !a.bias) return false;   // that case merges and truncates the scales
-    if (a.M <= 16 || a.M > 128 || a.N % 32 != 0 || a.N < 256 || a.K % 512 != 0) return false;
+    if (a.M <= 16 || a.M > 128 || a.N % 32 != 0 || a.N < 256 || a.K % 128 != 0) return false;
     if (a.x1.col_stride != 1 || a.x2.row_stride != 1 || a.x1.row_stride < a.K || a.x2.col_stride < a.K) return false;
     if (((uintptr_t)a.x1.ptr | (uintptr_t)a.x2.ptr | (uint64_t)a.x1.row_stride | (uint64_t)a.x2.col_stride) % 16 || (uintptr_t)a.out % 16) return false;
     if (a.K >= (1ll << 31) || a.N >= (1ll << 31)) return false;
@@ -114,10 +114,14 @@ static bool rowcol_rows_eligible(const OpsnnQmmArgs& a)
 }
 
 uint64_t rowcol_rows_workspace(const OpsnnQmmArgs& a) { return rowcol_rows_eligible(a) ? (uint64_t)a.M * (uint64_t)a.K * 2 : 0; }
+int rowcol_rows_ksplit(const OpsnnQmmArgs& a) { return rowcol_rows_eligible(a) ? rows_ksplit(a) : 1; }
 
-int launch_rowcol_rows(const OpsnnQmmArgs& a, hipStream_t st)
+int launch_rowcol_rows(const OpsnnQmmArgs& a, hipStream_t st, SplitK sk)
 {
     if (!rowcol_rows_eligible(a) || !a.workspace || (uintptr_t)a.workspace % 16) return OPSNN_NOT_TAKEN;
+    int64_t kunit = 0;
+    int ks = rows_ksplit(a, &kunit);
+    if (ks > 1 && (!sk.part || sk.splits < ks)) ks = 1;   // (no room for partial sums: K in one piece)
     uint16_t* x16 = (uint16_t*)a.workspace;
     const int64_t pieces = a.M * (a.K / 16);
     hipLaunchKernelGGL(widen_e4m3_f16_kernel, dim3((unsigned)((pieces + 255) / 256)), dim3(256), 0, st, (const uint8_t*)a.x1.ptr, a.x1.row_stride, x16,
@@ -132,8 +136,9 @@ int launch_rowcol_rows(const OpsnnQmmArgs& a, hipStream_t st)
     p.bs1 = (const float*)a.x1_scale; p.bs1_rs = a.x1_scale_len == 1 ? 0 : 1;
     p.bs2 = (const float*)a.x2_scale; p.bs2_cs = a.x2_scale_len == 1 ? 0 : 1;
     p.bs_out_dt = a.out_dtype;
-    if (a.M > 64 && (a.N + 127) / 128 <= 128) {   // narrow x2 (at most 128 workgroups): two slabs of 64 rows in one launch, twice the workgroups
-        p.m_rows = 64; p.m_slab = 64; p.m_end = a.M;
+    if (ks > 1) { p.ksplit = ks; p.kunit = kunit; p.part = sk.part; }
+    if (const int64_t slab = wq_narrow_slab_rows(a.M, a.N, true)) {   // narrow x2 (at most 128 workgroups): two slabs in one launch, twice the workgroups
+        p.m_rows = slab; p.m_slab = slab; p.m_end = a.M;
         return launch_rows_one<DT_F16, 8, 4, 2, 4, 2, false, 4>(p, st);
     }
     return a.M > 64 ? launch_rows_one<DT_F16, 8, 8, 2, 4, 2, false, 4>(p, st) : launch_rows_one<DT_F16, 8, 4, 2, 4, 2, false, 4>(p, st);

@@ -147,7 +147,10 @@ static int qmm_int8_impl(const OpsnnQmmArgs* a, void* stream, SplitK sk)
     bool b16 = (p.out_dt == DT_BF16 || p.out_dt == DT_F16) || int_out;
     int variant = a->force_variant;
     if (opsnn_force_plain()) variant = OPSNN_VARIANT_PLAIN;
-    bool want_fast = b16 && a_kmajor && variant != OPSNN_VARIANT_PLAIN && p.M * p.N >= 64 * 64 && (p.K % 16) == 0 &&
+    // (fewer than 64 x 64 outputs stay on the plain kernel unless K is long: one row against 3584 x 18944 is no work for one
+    // thread per output -- 2.4 ms there, 20 us on a 128 x 128 tile with K split)
+    const bool enough = p.M * p.N >= 64 * 64 || (p.N >= 256 && p.M * p.N * p.K >= (1ll << 22));
+    bool want_fast = b16 && a_kmajor && variant != OPSNN_VARIANT_PLAIN && enough && (p.K % 16) == 0 &&
                      (p.a_rs % 16) == 0 && ((uintptr_t)p.a % 16) == 0 && (p.a_bs % 16) == 0;
     if (want_fast && !b_kmajor && p.b_cs == 1 && p.b_rs == p.N && (p.b_bs == 0 || p.b_bs == p.K * p.N)) {
         int64_t nb = p.b_bs == 0 ? 1 : a->batch;

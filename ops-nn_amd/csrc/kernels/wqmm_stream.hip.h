@@ -429,7 +429,7 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(NW == 8
 template <int XDT, int WBITS, int MB, int NB, int WN, int WK, bool HAS_OFF, int WF = 0, bool SLDS = false, bool KSP = false>
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void wqmm_rows_kernel(WqParams p)
 {
-    static_assert(!KSP || WF <= 3, "K in segments: the weight-only forms and the fp8 block-scale form");
+    static_assert(!KSP || WF <= 4, "K in segments: the weight-only forms and the fp8 forms");
     static_assert(WN * WK == 8, "eight waves");
     static_assert(!SLDS || WF == 0 || WF == 2, "the scale table serves the integer forms and the e8m0 bytes of e2m1 codes");
     static_assert(WF == 0 || !HAS_OFF, "floating-point weight codes have no offset");
@@ -1432,14 +1432,21 @@ __global__ __launch_bounds__(256) void wq_splitk_reduce_kernel(const float* part
     }
 }
 
-// the fp8 block-scale form of the many-rows kernel: out[i] = cast(sum over the K segments, in order, of part[s, i])
-// (a template only so that every translation unit that includes this header may hold a copy)
-template <typename = void>
-__global__ __launch_bounds__(256) void rows_bs_splitk_reduce_kernel(const float* part, int splits, int64_t total, void* out, int out_dt)
+// the fp8 forms of the many-rows kernel: out[m, n] = cast(epilogue(sum over the K segments, in order, of part[s, m, n])); the
+// block-scale form has folded its scales in already, the row / column scale form (RC) computes
+// (sum * x2Scale[n]) * x1Scale[m] + bias[n] here as the kernel's own epilogue does
+template <bool RC>
+__global__ __launch_bounds__(256) void rows_bs_splitk_reduce_kernel(const float* part, int splits, int64_t total, int64_t N, const float* rs, int64_t rs_stride,
+                                                                    const float* cs, int64_t cs_stride, const float* bias, void* out, int out_dt)
 {
     const int64_t stride = (int64_t)gridDim.x * blockDim.x;
     for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
-        const float v = splitk_sum(part, splits, total, i);
+        float v = splitk_sum(part, splits, total, i);
+        if constexpr (RC) {
+            const int64_t m = i / N, n = i - m * N;
+            v = (v * cs[n * cs_stride]) * rs[m * rs_stride];
+            if (bias) v = v + bias[n];
+        }
         if (out_dt == DT_F32) ((float*)out)[i] = v;
         else ((uint16_t*)out)[i] = out_dt == DT_BF16 ? bf16_bits(v) : f16_bits(v);
     }
@@ -1562,7 +1569,7 @@ static int launch_rows_one(const WqParams& p, hipStream_t st)
 {
     if constexpr (!KSP) {   // K in segments: the instantiations of the 64-row instance with 128-column workgroups that know them
         if (p.ksplit > 1) {
-            if constexpr (MB == 4 && NB == 2 && WN == 4 && WK == 2 && WF <= 3 && !SLDS) return launch_rows_one<XDT, WBITS, MB, NB, WN, WK, HAS_OFF, WF, false, true>(p, st);
+            if constexpr (MB == 4 && NB == 2 && WN == 4 && WK == 2 && WF <= 4 && !SLDS) return launch_rows_one<XDT, WBITS, MB, NB, WN, WK, HAS_OFF, WF, false, true>(p, st);
             else return -1;
         }
     }
@@ -1619,8 +1626,13 @@ static int launch_rows_one(const WqParams& p, hipStream_t st)
     if (split) {
         const int64_t total = p.M * p.N;
         if constexpr (WF == 3) {
-            hipLaunchKernelGGL(rows_bs_splitk_reduce_kernel<void>, dim3(splitk_reduce_grid(total)), dim3(256), 0, st, (const float*)p.part, p.ksplit, total,
-                               (void*)p.y, p.bs_out_dt);
+            hipLaunchKernelGGL(rows_bs_splitk_reduce_kernel<false>, dim3(splitk_reduce_grid(total)), dim3(256), 0, st, (const float*)p.part, p.ksplit, total,
+                               p.N, (const float*)nullptr, (int64_t)0, (const float*)nullptr, (int64_t)0, (const float*)nullptr, (void*)p.y, p.bs_out_dt);
+            return (int)hipGetLastError();
+        }
+        if constexpr (WF == 4) {
+            hipLaunchKernelGGL(rows_bs_splitk_reduce_kernel<true>, dim3(splitk_reduce_grid(total)), dim3(256), 0, st, (const float*)p.part, p.ksplit, total,
+                               p.N, p.bs1, p.bs1_rs, p.bs2, p.bs2_cs, (const float*)p.bias, (void*)p.y, p.bs_out_dt);
             return (int)hipGetLastError();
         }
         hipLaunchKernelGGL(wq_splitk_reduce_kernel<XDT>, dim3(splitk_reduce_grid(total)), dim3(256), 0, st, (const float*)p.part, p.ksplit, total, p.N,

@@ -36,6 +36,9 @@ def _check_equal(got, want, what):
     (200, 8192, 1000, False),
     (16, 8192, 264, True),
     (130, 4096, 130, True),    # a column count that is no multiple of 4
+    # fewer than 64 x 64 outputs against a long K (one decode row against a narrow weight): the tile kernel with K split
+    (1, 18944, 3584, True),
+    (3, 3584, 1000, True),
 ])
 @pytest.mark.parametrize("out_dt,bias_dt", [("bf16", "bf16"), ("bf16", None), ("f16", "f32"), ("bf16", "i32"), ("f16", "f16")])
 def test_kc_matches_oracle(gpu, M, K, N, tB, out_dt, bias_dt):

@@ -255,6 +255,13 @@ def test_gpu_matches_oracle(gpu, M, K, N, in_dt, s_dt, s_len, bias_dt, out_dt, t
     (65, 1024, 288, "N", True, "bf16", "M"),
     (128, 3584, 512, "N", False, "f16", "M"),
     (100, 512, 256, 1, True, "bf16", True),
+    # ... K in whole 128-element blocks but no whole rounds of the chunk pipeline; K segments against a narrow x2 (86 blocks in
+    # five, 148 in eight, 144 in four with two row slabs, 108 at 17 .. 32 rows)
+    (40, 1664, 256, "N", True, "bf16", "M"),
+    (64, 11008, 512, "N", True, "f16", "M"),
+    (50, 18944, 256, "N", False, "bf16", "M"),
+    (128, 18432, 1024, 1, True, "f16", True),
+    (24, 13824, 384, "N", True, "bf16", "M"),
 ])
 def test_gpu_fp8_row_and_column_scales_on_the_matrix_cores(gpu, M, K, N, s_len, bias, out_dt, pt, fast):
     """fp8 e4m3 K-C / K-T / T-C-double-scale on the matrix cores (K-contiguous x2, K % 128 == 0, 16-bit output).  Default:
