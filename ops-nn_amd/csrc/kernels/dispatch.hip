@@ -194,7 +194,7 @@ static int splitk_for(const OpsnnQmmArgs& a, int mode)
     const bool a8w4 = mode == 2 && a.x1_dtype == DT_E4M3 && a.x2_dtype == DT_E2M1;
     if (a.M <= 32 && a.batch == 1 && a.N >= 256 &&
         ((mode == 1 && (f8 || (a.x1_dtype == DT_I8 && a.x2_dtype == DT_I8)) && a.gsK == 128 && a.gsN == 128) ||
-         (mode == 3 && f8 && a.x1_scale && a.x2_scale) || (a8w4 && out16))) {
+         (mode == 3 && f8 && a.x1_scale && a.x2_scale) || (a8w4 && out16) || (mode == 2 && f8))) {
         QmmDecodePlan pl;
         const int sd = qmm_decode_plan(a.K, true, pl, a8w4) ? pl.splits : 1;
         // (17 .. 32 rows of fp8 with block scales may also run on the many-rows kernel, with its own segments: room for either)

@@ -428,6 +428,180 @@ int launch_mxw4_one(const MxW4DecParams& p, hipStream_t st, int splits = 1)
     return (int)hipGetLastError();
 }
 
+
+// ---- MXFP8: fp8 e4m3 x fp8 e4m3 with e8m0 scales per 32 elements of K on both operands (the MX mode of
+// quant_batch_matmul_v4, qbmmv4_kernel_golden.py:119-186), up to 16 rows of x1 per pass ----
+// The stream of fp8_block_decode_kernel with the scales folded into the widening conversion: an e4m3 value times a power of
+// two is a bf16 value (v_cvt_scalef32_pk_bf16_fp8 with the scale 2^(byte - 127): exact wherever fp32 itself would hold the
+// scaled value), the product of two bf16 values is an fp32 value, and v_mfma_f32_16x16x32_bf16 sums such products in fp32
+// -- one chain over the wave's whole K range, no fold per block.  A lane's 16-byte piece lies inside one 32-element block,
+// so one scale byte serves it; x2's scale bytes arrive as words of four (128 elements) per row: lane (row, q) fetches word
+// 4 i + q of the wave's range and the word of chunk c comes over from lane (row, (c / 2) % 4).  K segments and idle
+// waves as in fp8_block_decode_kernel<..., SEG>.
+struct Mx8DecParams {
+    const uint8_t* a;    // x1 [M, K] e4m3, K contiguous
+    const uint8_t* b;    // x2 as [N, K], K contiguous
+    int64_t lda, ldb;
+    const uint8_t* sa;   // e8m0 [M, K / 32], K contiguous
+    const uint8_t* sb;   // e8m0 [N, K / 32]
+    int64_t sa_rs, sb_rs;
+    void* out; int out_dt;
+    int64_t M, N, K;
+    const float* bias;
+    float* part; int64_t part_slice;
+};
+
+// 8 e4m3 bytes (two dwords) times the scale -> 8 bf16 in byte order
+__device__ __forceinline__ v4i widen8_e4m3_bf16(uint32_t d0, uint32_t d1, float sc)
+{
+    typedef __bf16 b2v __attribute__((ext_vector_type(2)));
+    const b2v w0 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(d0, sc, false), w1 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(d0, sc, true);
+    const b2v w2 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(d1, sc, false), w3 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(d1, sc, true);
+    return (v4i){(int)__builtin_bit_cast(uint32_t, w0), (int)__builtin_bit_cast(uint32_t, w1), (int)__builtin_bit_cast(uint32_t, w2),
+                 (int)__builtin_bit_cast(uint32_t, w3)};
+}
+
+template <int NW, int NBLK>
+__global__ __launch_bounds__(NW * 64) void mx8_decode_kernel(Mx8DecParams p)
+{
+    constexpr int NCH = 2 * NBLK;                    // 64-byte chunks of an x2 row in a wave's K range
+    constexpr int PF = NW == 16 ? (NCH < 4 ? NCH : 4) : NCH;   // pieces in flight per lane; divides NCH
+    constexpr int NSW = (NBLK + 3) / 4;              // scale-word fetches per column block
+    static_assert(NCH % PF == 0, "a piece's slot must not depend on the column block");
+    extern __shared__ __attribute__((aligned(16))) float red[];   // [2][NW][256]
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int nrow = lane & 15, q = lane >> 4;
+    const int nbk = (int)(p.K / 128);
+    int kb0 = ((int)blockIdx.y * NW + wave) * NBLK;
+    const bool live = kb0 < nbk;
+    if (!live) kb0 = nbk - NBLK;
+    const int64_t kbase = (int64_t)kb0 * 128;
+    const int nblocks = (int)((p.N + 15) / 16);
+    const int M = (int)p.M;
+
+    // x1: lane (m = lane % 16, q) holds, for chunk c and half h, the 8 elements k = kbase + 64 c + 16 q + 8 h .. + 7, scaled
+    v4i xf[NCH][2];
+#pragma unroll
+    for (int c = 0; c < NCH; c++) {
+        uint4 raw = make_uint4(0, 0, 0, 0);
+        float sc = 1.0f;
+        if (nrow < M) {
+            raw = *(const uint4*)(p.a + (int64_t)nrow * p.lda + kbase + 64 * c + 16 * q);
+            sc = e8m0_to_f32(p.sa[(int64_t)nrow * p.sa_rs + (kbase + 64 * c + 16 * q) / 32]);
+        }
+        xf[c][0] = widen8_e4m3_bf16(raw.x, raw.y, sc);
+        xf[c][1] = widen8_e4m3_bf16(raw.z, raw.w, sc);
+    }
+
+    auto wload = [&](int rb, int c) {
+        const int64_t n = (int64_t)rb * 16 + nrow;
+        return *(const uint4*)(p.b + (n < p.N ? n : p.N - 1) * p.ldb + kbase + 64 * c + 16 * q);   // columns past the edge repeat the last one
+    };
+    auto sload = [&](int rb, int i) {
+        const int64_t n = (int64_t)rb * 16 + nrow;
+        const int w = 4 * i + q < NBLK ? 4 * i + q : NBLK - 1;
+        return *(const uint32_t*)(p.sb + (n < p.N ? n : p.N - 1) * p.sb_rs + kbase / 32 + 4 * w);
+    };
+    int rb = blockIdx.x;
+    uint4 wq[PF];
+    uint32_t sq[NSW];
+#pragma unroll
+    for (int i = 0; i < PF; i++) wq[i] = wload(rb < nblocks ? rb : nblocks - 1, i);
+#pragma unroll
+    for (int i = 0; i < NSW; i++) sq[i] = sload(rb < nblocks ? rb : nblocks - 1, i);
+
+    for (int it = 0; rb < nblocks; it++, rb += (int)gridDim.x) {
+        const int rbn = rb + (int)gridDim.x < nblocks ? rb + (int)gridDim.x : rb;   // past the end: a harmless reload
+        const int64_t n0 = (int64_t)rb * 16;
+        uint32_t sws[NBLK];
+#pragma unroll
+        for (int j = 0; j < NBLK; j++) sws[j] = (uint32_t)__shfl((int)sq[j / 4], nrow + 16 * (j % 4));
+#pragma unroll
+        for (int i = 0; i < NSW; i++) sq[i] = sload(rbn, i);
+        v4f acc = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+        for (int c = 0; c < NCH; c++) {
+            const uint4 cur = wq[c % PF];
+            wq[c % PF] = c + PF < NCH ? wload(rb, c + PF) : wload(rbn, c + PF - NCH);
+            const float sc = e8m0_to_f32((sws[c / 2] >> (8 * (2 * (c % 2) + (q >> 1)))) & 0xffu);
+            const v4i w0 = widen8_e4m3_bf16(cur.x, cur.y, sc), w1 = widen8_e4m3_bf16(cur.z, cur.w, sc);
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf, w0), __builtin_bit_cast(v8bf, xf[c][0]), acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf, w1), __builtin_bit_cast(v8bf, xf[c][1]), acc, 0, 0, 0);
+        }
+        // acc[r]: m = lane % 16, n = n0 + 4 (lane / 16) + r, over this wave's K range
+        if (!live) acc = (v4f){0.0f, 0.0f, 0.0f, 0.0f};
+        float* mine = red + ((it & 1) * NW + wave) * 256;
+        *(v4f*)(mine + lane * 4) = acc;
+        __syncthreads();
+        if (wave != (it & (NW - 1))) continue;
+        const float* all = red + (it & 1) * NW * 256 + lane * 4;
+        v4f sum = *(const v4f*)all;
+#pragma unroll 4
+        for (int w = 1; w < NW; w++) {
+            const v4f o = *(const v4f*)(all + w * 256);
+#pragma unroll
+            for (int r = 0; r < 4; r++) sum[r] = sum[r] + o[r];
+        }
+        if (nrow >= M) continue;
+        const int64_t n = n0 + 4 * q;
+        if (gridDim.y > 1) {
+            float* dst = p.part + (int64_t)blockIdx.y * p.part_slice + (int64_t)nrow * p.N + n;
+#pragma unroll
+            for (int r = 0; r < 4; r++)
+                if (n + r < p.N) dst[r] = sum[r];
+            continue;
+        }
+        if (p.bias) {
+#pragma unroll
+            for (int r = 0; r < 4; r++) sum[r] = sum[r] + p.bias[n + r < p.N ? n + r : p.N - 1];
+        }
+        if (p.out_dt == DT_F32) {
+            float* dst = (float*)p.out + (int64_t)nrow * p.N + n;
+#pragma unroll
+            for (int r = 0; r < 4; r++)
+                if (n + r < p.N) dst[r] = sum[r];
+        } else {
+            const v4us o = p.out_dt == DT_BF16 ? pack4_b16<DT_BF16>(sum) : pack4_b16<DT_F16>(sum);
+            uint16_t* dst = (uint16_t*)p.out + (int64_t)nrow * p.N + n;
+            if ((p.N % 4) == 0 && ((uintptr_t)p.out % 8) == 0 && n + 3 < p.N) *(v4us*)dst = o;
+            else {
+#pragma unroll
+                for (int r = 0; r < 4; r++)
+                    if (n + r < p.N) dst[r] = o[r];
+            }
+        }
+    }
+}
+
+// out = cast(sum over the K segments, in order, of part[s] + bias) for one pass of up to 16 rows
+__global__ __launch_bounds__(256) void mx8dec_reduce_kernel(Mx8DecParams p, int splits)
+{
+    const int64_t total = p.M * p.N, stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
+        float v = p.part[i];
+        for (int s = 1; s < splits; s++) v = v + p.part[(int64_t)s * p.part_slice + i];
+        if (p.bias) v = v + p.bias[i % p.N];
+        if (p.out_dt == DT_F32) ((float*)p.out)[i] = v;
+        else ((uint16_t*)p.out)[i] = p.out_dt == DT_BF16 ? bf16_bits(v) : f16_bits(v);
+    }
+}
+
+template <int NW, int NBLK>
+int launch_mx8_one(const Mx8DecParams& p, hipStream_t st, int splits)
+{
+    const int64_t nbk = p.K / 128;
+    if (splits < 1 || splits > 16 || nbk % NBLK != 0 || nbk < NBLK || (int64_t)splits * NW * NBLK < nbk || (splits > 1 && !p.part)) return -1;
+    const int nblocks = (int)((p.N + 15) / 16);
+    const int cus = 256 / splits;   // the CUs shared between the segments' workgroup columns
+    const int grid = nblocks < cus ? nblocks : cus;
+    const size_t lds = (size_t)2 * NW * 256 * sizeof(float);
+    hipLaunchKernelGGL((mx8_decode_kernel<NW, NBLK>), dim3((unsigned)grid, (unsigned)splits), dim3(NW * 64), lds, st, p);
+    if (hipError_t e = hipGetLastError(); e != hipSuccess || splits == 1) return (int)e;
+    hipLaunchKernelGGL(mx8dec_reduce_kernel, dim3(splitk_reduce_grid(p.M * p.N)), dim3(256), 0, st, p, splits);
+    return (int)hipGetLastError();
+}
+
 }  // namespace
 
 // fp8 e4m3 block scales (or int8 per-tile: the same scales, an fp32 bias, 16-bit output) with up to 32 rows of x1 (two
@@ -534,6 +708,49 @@ int launch_mx_a8w4_decode(const OpsnnQmmArgs& a, hipStream_t st, SplitK sk)
             case 5: rc = launch_mxw4_one<8, 5>(p, st, splits); break;
             case 6: rc = launch_mxw4_one<8, 6>(p, st, splits); break;
             case 7: rc = launch_mxw4_one<8, 7>(p, st, splits); break;
+            default: break;
+        }
+        if (rc != 0) return rc;
+    }
+    return 0;
+}
+
+// MXFP8 with up to 32 rows of x1 (two passes beyond 16): K-contiguous operands and scale rows ([rows, K / 64, 2] bytes), K a
+// whole number of 128-element blocks as qmm_decode_plan lays them out; OPSNN_NOT_TAKEN otherwise.
+int launch_mxfp8_decode(const OpsnnQmmArgs& a, hipStream_t st, SplitK sk)
+{
+    if (a.x1_dtype != DT_E4M3 || a.x2_dtype != DT_E4M3 || a.batch != 1) return OPSNN_NOT_TAKEN;
+    if (a.out_dtype != DT_BF16 && a.out_dtype != DT_F16 && a.out_dtype != DT_F32) return OPSNN_NOT_TAKEN;
+    if (a.M > 32 || a.N < 256 || a.K % 128 != 0 || a.x1.col_stride != 1 || a.x2.row_stride != 1) return OPSNN_NOT_TAKEN;
+    if (a.x1_scale_mat.col_stride != 2 || a.x2_scale_mat.col_stride != 2) return OPSNN_NOT_TAKEN;   // [rows, K / 64, 2]: a row's bytes contiguous
+    if (a.bias && a.bias_dtype != DT_F32) return OPSNN_NOT_TAKEN;
+    if (a.x1.row_stride < a.K || a.x2.col_stride < a.K) return OPSNN_NOT_TAKEN;
+    if (((uintptr_t)a.x1.ptr | (uintptr_t)a.x2.ptr | (uint64_t)a.x1.row_stride | (uint64_t)a.x2.col_stride) % 16) return OPSNN_NOT_TAKEN;
+    if (((uintptr_t)a.x2_scale_mat.ptr | (uint64_t)a.x2_scale_mat.row_stride) % 4) return OPSNN_NOT_TAKEN;
+    if (a.x1_scale_mat.row_stride < a.K / 32 || a.x2_scale_mat.row_stride < a.K / 32) return OPSNN_NOT_TAKEN;
+    QmmDecodePlan pl;
+    if (!qmm_decode_plan(a.K, sk.part != nullptr, pl) || pl.splits > (sk.part ? sk.splits : 1)) return OPSNN_NOT_TAKEN;
+    for (int64_t m0 = 0; m0 < a.M; m0 += 16) {
+        Mx8DecParams p{};
+        p.M = a.M - m0 < 16 ? a.M - m0 : 16; p.N = a.N; p.K = a.K;
+        p.a = (const uint8_t*)a.x1.ptr + m0 * a.x1.row_stride; p.b = (const uint8_t*)a.x2.ptr;
+        p.lda = a.x1.row_stride; p.ldb = a.x2.col_stride;
+        p.sa = (const uint8_t*)a.x1_scale_mat.ptr + m0 * a.x1_scale_mat.row_stride; p.sb = (const uint8_t*)a.x2_scale_mat.ptr;
+        p.sa_rs = a.x1_scale_mat.row_stride; p.sb_rs = a.x2_scale_mat.row_stride;
+        p.out_dt = a.out_dtype; p.out = (char*)a.out + m0 * a.N * (a.out_dtype == DT_F32 ? 4 : 2);
+        p.bias = (const float*)a.bias;
+        p.part = sk.part ? sk.part + m0 * a.N : nullptr; p.part_slice = a.M * a.N;
+        int rc = -1;
+        if (pl.nw == 16) rc = pl.nblk == 1 ? launch_mx8_one<16, 1>(p, st, pl.splits) : pl.nblk == 2 ? launch_mx8_one<16, 2>(p, st, pl.splits)
+                              : pl.nblk == 4 ? launch_mx8_one<16, 4>(p, st, pl.splits) : -1;
+        else switch (pl.nblk) {
+            case 1: rc = launch_mx8_one<8, 1>(p, st, pl.splits); break;
+            case 2: rc = launch_mx8_one<8, 2>(p, st, pl.splits); break;
+            case 3: rc = launch_mx8_one<8, 3>(p, st, pl.splits); break;
+            case 4: rc = launch_mx8_one<8, 4>(p, st, pl.splits); break;
+            case 5: rc = launch_mx8_one<8, 5>(p, st, pl.splits); break;
+            case 6: rc = launch_mx8_one<8, 6>(p, st, pl.splits); break;
+            case 7: rc = launch_mx8_one<8, 7>(p, st, pl.splits); break;
             default: break;
         }
         if (rc != 0) return rc;

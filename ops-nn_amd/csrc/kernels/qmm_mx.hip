@@ -217,7 +217,8 @@ static bool mx_call_ok(const OpsnnQmmArgs& a)
     }
     if (a.out_dtype != DT_BF16 && a.out_dtype != DT_F16 && a.out_dtype != DT_F32) return false;
     if (a.bias && a.bias_dtype != DT_F32) return false;
-    if (a.K % 32 != 0 || a.M * a.N < 64 * 64) return false;
+    // (fewer than 64 x 64 outputs: only MXFP8's few-rows stream over x2, which wants 256 columns)
+    if (a.K % 32 != 0 || (a.M * a.N < 64 * 64 && !(fp8 && a.M <= 32 && a.N >= 256 && a.batch == 1 && a.K % 128 == 0))) return false;
     const int64_t ks = (a.K + 63) / 64, epb = fp4 ? 2 : 1;
     if (a.x1.col_stride != 1 || a.x1_scale_mat.col_stride != 2 || a.x1_scale_mat.row_stride != ks * 2) return false;
     if (((uintptr_t)a.x1.ptr | (uint64_t)(a.x1.row_stride / epb) | (uint64_t)(a.x1.batch_stride / epb)) % 16) return false;
@@ -254,6 +255,7 @@ void weight_cache_commit(void* buffer, hipStream_t st);   // weight_cache.hip
 void weight_cache_abandon(void* buffer);
 int launch_mxfp8_mfma(const OpsnnQmmArgs& a, hipStream_t st);   // qmm_fp8_block.hip
 int launch_mx_a8w4_mfma(const OpsnnQmmArgs& a, hipStream_t st, SplitK sk);   // qmm_fp8_block.hip
+int launch_mxfp8_decode(const OpsnnQmmArgs& a, hipStream_t st, SplitK sk);   // qmm_fp8_decode.hip
 
 int launch_mx_mfma(const OpsnnQmmArgs& a0, hipStream_t st, SplitK sk)
 {
@@ -311,6 +313,12 @@ int launch_mx_mfma(const OpsnnQmmArgs& a0, hipStream_t st, SplitK sk)
         if (rc != 0) return rc;
     }
     if (a.x1_dtype == DT_E4M3 && a.x2_dtype == DT_E2M1) return launch_mx_a8w4_mfma(a, st, sk);   // fp8 x fp4: qmm_fp8_block.hip
+    if (fp8 && a.M <= 32) {   // MXFP8 with up to 32 rows: the stream over x2 with x1 in registers (exact products)
+        const int rc = launch_mxfp8_decode(a, st, sk);
+        if (rc != OPSNN_NOT_TAKEN) return rc;
+        if (a.M * a.N < 64 * 64) return OPSNN_NOT_TAKEN;
+        sk = SplitK{};   // (the partial sums were laid out for the kernel above; the tile kernels run unsplit)
+    }
     // MXFP8 runs on the block kernel of qmm_fp8_block.hip in MX mode (16x16x128 instructions, 64 x 128 per wave, the
     // pipeline tuned for the fp8 block-scale path); the 32x32x64 tile kernel stays available on request
     // (OPSNN_VARIANT_MX_FP8_MFMA) for comparison.  The 8-bit forms of the matrix instruction sum their products with a

@@ -276,6 +276,39 @@ def test_mxfp8_exact_window(gpu, exp_range, batch):
         check_close(got, want, orc.BF16, "mxfp8 beyond the window", fp8_mfma=True, abs_sum=abs_sum)
 
 
+@pytest.mark.parametrize("M,K,N,exp_range,out", [
+    # up to 32 rows of x1 against a K-contiguous x2: K shared by 16 waves (4096, 8192) or by 8 (3072, 7168), ragged columns, two
+    # passes; a K that one workgroup's waves do not share exactly (28 blocks: idle waves; 86, 144, 148: K segments with fp32
+    # partial sums); one row and fewer than 64 x 64 outputs; scale exponents over +-30 binades (no window as on the tiles)
+    (1, 4096, 512, 4, "bf16"), (16, 7168, 1000, 4, "bf16"), (9, 8192, 264, 4, "f16"), (32, 3072, 256, 4, "bf16"),
+    # (the long sums with fp16 output: fp32 sums in another order than the oracle's flip one bf16 result in a thousand by an
+    # ulp, which is four times the 1e-3 the bar allows)
+    (16, 3584, 256, 4, "f32"), (16, 11008, 264, 4, "f16"), (20, 18432, 256, 4, "f16"), (1, 18944, 384, 4, "f16"),
+    (16, 2048, 320, 30, "f32"), (12, 4096, 256, 14, "bf16"),
+])
+def test_mxfp8_few_rows(gpu, M, K, N, exp_range, out):
+    """MXFP8 with up to 32 rows: x1 in registers and x2 streamed once per 16 rows, both widened to bf16 with their block's
+    scale folded in (exact), fp32 sums in the matrix instruction -- the stated bar, with the plain kernel bit-identical."""
+    m = gpu
+    dt = {"bf16": m.ACL_BF16, "f16": m.ACL_FLOAT16, "f32": m.ACL_FLOAT}[out]
+    print(f"case mxfp8 few rows M={M} K={K} N={N} exp_range={exp_range} out={out}", flush=True)
+    inp = cases.make_mx_inputs(m, M, K, N, K + N + M, True, False, exp_range=exp_range)
+    bias = np.random.default_rng(1).normal(0, 1, N).astype(np.float32) if M % 2 == 0 else None
+    want = cases.oracle_mx(m, inp, M, K, N, True, dt, bias)
+    plain(False)
+    got = cases.run_mx_aclnn(m, inp, M, K, N, True, dt, bias)
+    if out == "f32":
+        assert np.isfinite(got).all()
+        pos = dict(inp, x1=inp["x1"] & 0x7F, x2=inp["x2"] & 0x7F)
+        abs_sum = cases.oracle_mx(m, pos, M, K, N, True, dt).astype(np.float64) + (np.abs(bias) if bias is not None else 0.0)
+        err = np.abs(got.astype(np.float64) - want.astype(np.float64))
+        assert (err <= 2.0 ** -18 * abs_sum + 1e-30).all(), f"worst error / sum of magnitudes: {float((err / (abs_sum + 1e-30)).max()):.3e}"
+    else:
+        check_close(got, want, orc.BF16 if out == "bf16" else orc.F16, "mxfp8 few rows")
+    plain(True)
+    assert np.array_equal(cases.run_mx_aclnn(m, inp, M, K, N, True, dt, bias), want)
+
+
 @pytest.mark.parametrize("M,K,N,tB,fp4,bias", [(256, 1024, 384, True, True, True), (300, 512, 262, True, True, False), (128, 512, 256, False, True, True),
                                                (200, 960, 264, True, True, False), (256, 1024, 384, True, False, True), (130, 256, 200, True, False, False)])
 def test_mx_fp32_output(gpu, M, K, N, tB, fp4, bias):
