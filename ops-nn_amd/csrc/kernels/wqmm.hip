@@ -333,7 +333,7 @@ static bool stream_eligible(WqParams& p, WqStreamOpts& o)
     int xsplits = 1;
     bool xexact = true;
     o.xreg = p.M <= 16 && xreg_shape(WBITS, p.K, xreg_nw, xnw, xnch, p.M, p.part != nullptr, &xsplits, &xexact) && (p.M >= xreg_min || (xsplits > 1 && !o.resx));
-    o.xreg_vscale = o.xreg && xexact && p.group == KC && p.s_rs == 1 && p.s_cs % 8 == 0 &&
+    o.xreg_vscale = o.xreg && p.group == KC && p.s_rs == 1 && p.s_cs % 8 == 0 && p.s_cs >= nch &&
                     (uintptr_t)p.scale % 16 == 0 && (!p.offset || (uintptr_t)p.offset % 16 == 0);
     // more than 32 rows: two weight blocks per wave share every x fragment, up to 128 rows per pass over the weights
     // (needs whole groups of chunks in flight and whole wave tiles of columns)
@@ -374,7 +374,7 @@ static int launch_slabs_float(WqParams p, hipStream_t st)
     // up to 16 rows: x in registers (mxfp4: e2m1 codes with a row's e8m0 bytes contiguous; e4m3 codes with per-channel scales)
     if (p.M <= 16 && !p.offset) {
         bool ok;
-        if (WBITS == 4) ok = p.scale_e8m0 && p.group == 32 && p.s_rs == 1 && p.s_cs % 16 == 0 && (uintptr_t)p.scale % 16 == 0;
+        if (WBITS == 4) ok = p.scale_e8m0 && p.group == 32 && p.s_rs == 1 && p.s_cs % 16 == 0 && p.s_cs >= p.K / 32 && (uintptr_t)p.scale % 16 == 0;
         else ok = !p.scale_e8m0 && p.group >= p.K;
         if (ok) {
             p.m_base = 0; p.m_rows = p.M; p.cpg_shift = 31;

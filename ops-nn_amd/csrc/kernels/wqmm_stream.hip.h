@@ -1208,31 +1208,35 @@ __global__ __launch_bounds__(NW * 64) void wqmm_xreg_kernel(WqParams p)
     // dword c belongs to lane group g); fetched one row block ahead
     constexpr int SW = MXS ? NCH : NCH / 2;
     uint32_t sv[SW], ov[SW], svn[SW], ovn[SW];
+    // (A wave with no live chunk fetches the row's first scales instead: nothing uses them.  A wave with some idle chunks
+    // reads past the row's last scale, but not past its pitch: these loads are chosen only for rows whose pitch is a whole
+    // number of 16-byte pieces.)
+    const int cbs = nlive > 0 ? cbase : 0;
     auto load_scales = [&](const uint16_t* sr, const uint16_t* orw, uint32_t (&sd)[SW], uint32_t (&od)[SW]) {
         if constexpr (MXS) {
 #pragma unroll
             for (int h = 0; h < NCH / 4; h++) {
-                const v4i t = *(const v4i*)((const uint8_t*)sr + cbase * 4 + 16 * h);
+                const v4i t = *(const v4i*)((const uint8_t*)sr + cbs * 4 + 16 * h);
 #pragma unroll
                 for (int e = 0; e < 4; e++) sd[4 * h + e] = (uint32_t)t[e];
             }
         } else if constexpr (NCH % 8 == 0) {
 #pragma unroll
             for (int h = 0; h < NCH / 8; h++) {
-                const v4i t = *(const v4i*)(sr + cbase + 8 * h);
+                const v4i t = *(const v4i*)(sr + cbs + 8 * h);
 #pragma unroll
                 for (int e = 0; e < 4; e++) sd[4 * h + e] = (uint32_t)t[e];
                 if constexpr (HAS_OFF) {
-                    const v4i u = *(const v4i*)(orw + cbase + 8 * h);
+                    const v4i u = *(const v4i*)(orw + cbs + 8 * h);
 #pragma unroll
                     for (int e = 0; e < 4; e++) od[4 * h + e] = (uint32_t)u[e];
                 }
             }
         } else {
-            const v2i t = *(const v2i*)(sr + cbase);
+            const v2i t = *(const v2i*)(sr + cbs);
             sd[0] = (uint32_t)t[0]; sd[1] = (uint32_t)t[1];
             if constexpr (HAS_OFF) {
-                const v2i u = *(const v2i*)(orw + cbase);
+                const v2i u = *(const v2i*)(orw + cbs);
                 od[0] = (uint32_t)u[0]; od[1] = (uint32_t)u[1];
             }
         }
@@ -1462,10 +1466,12 @@ static int launch_xreg_one(const WqParams& p, hipStream_t st, int splits = 1)
     }
     const int64_t nblocks = (p.N + 15) / 16;
     if (splits < 1 || splits > 16 || (splits > 1 && (!p.part || p.m_base != 0 || p.m_rows != p.M))) return -1;
-    {   // the segments cover K, the last one with idle chunks worth at most a sixth of K; vector scale loads only for whole segments
+    {   // the segments cover K, the last one with idle chunks worth at most a sixth of K; with idle chunks the vector scale
+        // loads of a wave's last piece may reach past the row's last scale: the row's pitch must hold whole pieces
         const int64_t kc = 4 * (128 / WBITS), nch = p.K / kc, cover = (int64_t)splits * NW * NCH;
         if (p.K % 128 != 0 || cover < nch || (cover - nch) * 6 > nch || cover - nch >= (int64_t)NW * NCH) return -1;
-        if (cover != nch && SCM != 0) return -1;
+        if (cover != nch && SCM == 1 && (p.s_cs % 8 != 0 || p.s_cs < nch)) return -1;
+        if (cover != nch && SCM == 2 && (p.s_cs % 16 != 0 || p.s_cs < nch * 4)) return -1;
     }
     const int64_t g = ((int64_t)resx_grid(1ll << 40) / (TWO ? 1 : 2) + splits - 1) / splits;   // (resx_grid: two per CU)
     constexpr int STEPS = (4 * (128 / WBITS)) / 32;
@@ -1517,7 +1523,6 @@ static int launch_xreg(const WqParams& p, bool has_off, bool vscale, int force_n
     int nw = 0, nch = 0, splits = 1;
     bool exact = true;
     if (!xreg_shape(WBITS, p.K, force_nw, nw, nch, p.M, p.part != nullptr, &splits, &exact)) return OPSNN_NOT_TAKEN;
-    if (!exact) vscale = false;   // (vector scale loads would read past the row's last scale)
     if (nw == 16 && nch == 4) return launch_xreg_nch<XDT, WBITS, 16, 4>(p, has_off, vscale, st, splits);
     if constexpr (WBITS == 8) {
         if (nw == 16 && nch == 8) return launch_xreg_nch<XDT, WBITS, 16, 8>(p, has_off, vscale, st);
@@ -1533,7 +1538,8 @@ template <int XDT, int WBITS>
 static int launch_xreg_float(const WqParams& p, hipStream_t st)
 {
     int nw = 0, nch = 0, splits = 1;
-    if (!xreg_shape(WBITS, p.K, 0, nw, nch, p.M, p.part != nullptr, &splits)) return OPSNN_NOT_TAKEN;
+    bool exact = true;
+    if (!xreg_shape(WBITS, p.K, 0, nw, nch, p.M, p.part != nullptr, &splits, &exact)) return OPSNN_NOT_TAKEN;
     constexpr int SCM = WBITS == 4 ? 2 : 0;
     if (nw == 16 && nch == 4) return launch_xreg_one<XDT, WBITS, 16, 4, false, SCM, true>(p, st, splits);
     if constexpr (WBITS == 8) {
