@@ -22,6 +22,7 @@ int blockscale_rows_ksplit(const OpsnnQmmArgs& a);
 uint64_t rowcol_rows_workspace(const OpsnnQmmArgs& a);
 int launch_rowcol_rows(const OpsnnQmmArgs& a, hipStream_t st, SplitK sk);
 int rowcol_rows_ksplit(const OpsnnQmmArgs& a);
+int mxfp8_rows_ksplit(const OpsnnQmmArgs& a);
 int launch_tcg_mfma(const OpsnnQmmArgs& a, hipStream_t st);
 uint64_t tcg_workspace_bytes(const OpsnnQmmArgs& a);
 int launch_kg_mfma(const OpsnnQmmArgs& a, hipStream_t st);   // qmm_i4_kg.hip
@@ -204,6 +205,10 @@ static int splitk_for(const OpsnnQmmArgs& a, int mode)
     // 33 .. 128 rows of fp8 with block scales or row / column scales on the many-rows kernel
     if ((mode == 1 || mode == 3) && f8 && a.M <= 128) {
         if (const int sr = mode == 1 ? blockscale_rows_ksplit(a) : rowcol_rows_ksplit(a); sr > 1) return sr;
+    }
+    // 33 .. 256 rows of MXFP8 on the many-rows kernel (exact products: not when the 8-bit instruction was asked for)
+    if (mode == 2 && f8 && a.M <= 256 && !opsnnGetFp8Fast()) {
+        if (const int sr = mxfp8_rows_ksplit(a); sr > 1) return sr;
     }
     // (fewer than 64 x 64 outputs are the plain kernels' -- except int8 with few outputs against a long K, qmm_int8.hip)
     const bool tiny = a.M * a.N < 64 * 64;

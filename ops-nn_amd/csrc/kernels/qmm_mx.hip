@@ -244,10 +244,18 @@ static uint64_t mx_rest_bytes(const OpsnnQmmArgs& a0)
 
 // Workspace of an MX call: in front, what the exact route of MXFP8 needs (nothing for the other operand pairs), then the
 // re-laid-out and padded operand copies.
+uint64_t mxfp8_rows_workspace(const OpsnnQmmArgs& a);   // qmm_fp8_rows.hip
+int launch_mxfp8_rows(const OpsnnQmmArgs& a, void* region, hipStream_t st, SplitK sk);
+// (in front of that: the bf16 copy of x1 for MXFP8 with 33 .. 256 rows on the many-rows kernel)
+static uint64_t mx_rows_bytes(const OpsnnQmmArgs& a)
+{
+    if (a.force_variant == OPSNN_VARIANT_PLAIN || opsnn_force_plain() || opsnnGetFp8Fast() || !mx_call_ok(a)) return 0;
+    return align_up(mxfp8_rows_workspace(a), 256);
+}
 uint64_t mx_workspace_bytes(const OpsnnQmmArgs& a)
 {
     const bool matrix_cores = a.force_variant != OPSNN_VARIANT_PLAIN && !opsnn_force_plain();
-    return (matrix_cores ? mx_exact_bytes(a) : 0) + mx_rest_bytes(a);
+    return mx_rows_bytes(a) + (matrix_cores ? mx_exact_bytes(a) : 0) + mx_rest_bytes(a);
 }
 
 void* weight_cache_blob(const void* src, const void* src2, int64_t K, int64_t N, int bits, int64_t nb, uint64_t bytes, hipStream_t st, bool* fresh);
@@ -268,6 +276,11 @@ int launch_mx_mfma(const OpsnnQmmArgs& a0, hipStream_t st, SplitK sk)
     // one ulp off and the largest relative error above 2^-7); opsnnSetFp8Fast(1) asks for the 8-bit instruction.  The exact
     // route's tables sit in front of the workspace.  With a 4-bit x2 the same instruction is as close to the fp32 sums as
     // exact products are (measured on the same shapes), so that mode keeps it.
+    char* rows_region = nullptr;
+    if (const uint64_t rb = mx_rows_bytes(a0); rb && a.workspace) {
+        rows_region = (char*)a.workspace;
+        a.workspace = rows_region + rb;
+    }
     char* mxx = nullptr;
     if (const uint64_t front = mx_exact_bytes(a0); front && a.workspace) {
         mxx = (char*)a.workspace;
@@ -313,6 +326,10 @@ int launch_mx_mfma(const OpsnnQmmArgs& a0, hipStream_t st, SplitK sk)
         if (rc != 0) return rc;
     }
     if (a.x1_dtype == DT_E4M3 && a.x2_dtype == DT_E2M1) return launch_mx_a8w4_mfma(a, st, sk);   // fp8 x fp4: qmm_fp8_block.hip
+    if (fp8 && rows_region) {   // MXFP8 with 33 .. 256 rows: the many-rows streaming kernel on bf16 operands (exact products)
+        const int rc = launch_mxfp8_rows(a, rows_region, st, sk);
+        if (rc != OPSNN_NOT_TAKEN) return rc;
+    }
     if (fp8 && a.M <= 32) {   // MXFP8 with up to 32 rows: the stream over x2 with x1 in registers (exact products)
         const int rc = launch_mxfp8_decode(a, st, sk);
         if (rc != OPSNN_NOT_TAKEN) return rc;

@@ -387,8 +387,11 @@ static int launch_slabs_float(WqParams p, hipStream_t st)
         constexpr int64_t KC = 4 * (128 / WBITS);
         constexpr int rows_min = 17;
         bool ok = !p.offset && p.M >= rows_min && p.K % KC == 0 && (p.K / KC) % 2 == 0 && p.N % 32 == 0 && p.N >= 256 && p.K < (1ll << 23);
-        if (WBITS == 4) ok = ok && p.scale_e8m0 && p.group == 32 && p.s_rs == 1;
+        const bool mx8 = WBITS == 8 && p.scale_e8m0;   // e4m3 codes with e8m0 scales per 32 (MXFP8's x2: launch_wq_mx8_rows)
+        if (WBITS == 4 || mx8) ok = ok && p.scale_e8m0 && p.group == 32 && p.s_rs == 1;
         else ok = ok && !p.scale_e8m0 && p.group >= p.K;
+        // (the kernel's scale table counts in words of four e8m0 bytes = 128 k: one chunk of e2m1 codes, two of e4m3 codes)
+        const int cpg = WBITS == 4 ? 0 : mx8 ? 1 : 31;
         // (the 192- / 256-row instances want K in whole rounds of four x slabs)
         const int64_t nslab = narrow_n_slab(p.M, p.N);
         if (ok && (p.K / KC) % 8 != 0 && (nslab ? nslab : p.M) > 128) ok = false;
@@ -399,15 +402,15 @@ static int launch_slabs_float(WqParams p, hipStream_t st)
             p.ksplit = ks > 1 ? ks : 0;
             p.kunit = kunit;
             if (const int64_t slab = narrow_n_slab(p.M, p.N)) {   // narrow N: all row slabs in one launch
-                p.cpg_shift = WBITS == 4 ? 0 : 31;
+                p.cpg_shift = cpg;
                 p.m_base = 0; p.m_rows = slab; p.m_slab = slab; p.m_end = p.M;
-                p.cols64 = ks > 1 ? 0 : use_cols64<WBITS>(slab, (p.M + slab - 1) / slab, p.N, p.K);
+                p.cols64 = ks > 1 || mx8 ? 0 : use_cols64<WBITS>(slab, (p.M + slab - 1) / slab, p.N, p.K);
                 return launch_wq_rows_float<XDT, WBITS>(p, st);
             }
-            p.cols64 = ks > 1 ? 0 : use_cols64<WBITS>(p.M, 1, p.N, p.K);
+            p.cols64 = ks > 1 || mx8 ? 0 : use_cols64<WBITS>(p.M, 1, p.N, p.K);
             // up to 128 rows one pass; more: whole passes of 256 rows and the rest in one (as for integer codes below)
             const int64_t slab = p.M <= 128 ? 128 : 256;
-            p.cpg_shift = WBITS == 4 ? 0 : 31;   // (e2m1: the kernel's scale table counts in words of four e8m0 bytes, one per 128 k chunk)
+            p.cpg_shift = cpg;
             for (int64_t m0 = 0; m0 < p.M; m0 += slab) {
                 p.m_base = m0;
                 p.m_rows = (p.M - m0) < slab ? (p.M - m0) : slab;
@@ -532,6 +535,20 @@ static int launch_slabs(WqParams p, hipStream_t st)
         if (rc != 0) return rc;
     }
     return 0;
+}
+
+// MXFP8 with 33 rows of x1 and more on the many-rows kernel: p.x is x1 widened to bf16 with its block scales folded in, p.w
+// x2's e4m3 codes (K-contiguous), p.scale x2's e8m0 bytes (a row's bytes contiguous), p.y bf16.  The caller has checked the
+// shape (the conditions of launch_slabs_float's many-rows branch); OPSNN_NOT_TAKEN if the kernel declines.
+int launch_wq_mx8_rows(const WqParams& p0, hipStream_t st)
+{
+    WqParams p = p0;
+    p.w_float = 1; p.scale_e8m0 = 1; p.group = 32; p.group_shift = 5; p.s_rs = 1; p.offset = nullptr;
+    constexpr int64_t KC = 64;
+    if (p.M < 17 || p.K % (2 * KC) != 0 || p.N % 32 != 0 || p.N < 256 || p.K >= (1ll << 23)) return OPSNN_NOT_TAKEN;
+    const int64_t nslab = narrow_n_slab(p.M, p.N);
+    if ((p.K / KC) % 8 != 0 && (nslab ? nslab : p.M) > 128) return OPSNN_NOT_TAKEN;
+    return launch_slabs_float<DT_BF16, 8>(p, st);
 }
 
 int launch_wqmm_mfma(const OpsnnWqmmArgs& a0, hipStream_t st)

@@ -433,7 +433,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void w
     static_assert(WN * WK == 8, "eight waves");
     static_assert(!SLDS || WF == 0 || WF == 2, "the scale table serves the integer forms and the e8m0 bytes of e2m1 codes");
     static_assert(WF == 0 || !HAS_OFF, "floating-point weight codes have no offset");
-    static_assert(WF != 2 || WBITS == 4, "e8m0 group scales go with e2m1 codes");
+    static_assert(WF != 2 || WBITS == 4 || (WBITS == 8 && WK == 2), "e8m0 group scales: e2m1 codes, or e4m3 codes on the instances with two K waves");
     static_assert(WF != 3 || (WBITS == 8 && XDT == DT_F16 && WK == 2 && NB == 2), "the block-scale form: fp16 x, e4m3 w, a slab per 128-block");
     static_assert(WF != 4 || (WBITS == 8 && XDT == DT_F16 && !HAS_OFF), "the row / column scale form: fp16 x, e4m3 w");
     constexpr int NT = 512;
@@ -464,6 +464,9 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void w
     static_assert((16 * MB * XPR) % NT == 0 && XPR >= 16 && PF >= 2 && PPH >= 1 && STEPS == PPH * XH, "staging and prefetch shape");
     static_assert(MB <= 8 || (WF == 0 && SLDS) || WF == 1 || WF == 2, "the 192- / 256-row instances: integer codes with the scale table in LDS, or floating-point codes");
     static_assert(!(SLDS && WF == 2 && MB > 8) || WK == 2, "8-byte pieces: byte position of a lane's e8m0 scale inside the table word");
+    // a lane's piece holds half a group of 32 codes (8-byte pieces of e2m1 codes, 16-byte pieces of e4m3 codes): two lane
+    // groups share an e8m0 byte, a chunk of the wave holds two bytes and the table word of 128 k serves the chunks of both K waves
+    constexpr bool E8H = (MB > 8 && WBITS == 4) || (WF == 2 && WBITS == 8);
     // K in segments: this workgroup's is number blockIdx.z.  Segments are whole units of p.kunit k (whole slabs of x and
     // whole groups), as equal as that allows, the longer ones first.  From here on p.K is the segment's length and x, w, the scales and
     // offsets start at the segment; a row of x keeps its pitch ldx.
@@ -508,7 +511,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void w
     const uint16_t* orow = HAS_OFF ? p.offset + (n0 + nrow) * p.s_cs : nullptr;
     const int64_t sblk = 16 * p.s_cs;
     // WF 2: the byte of this lane's group in chunk 0 (8-byte pieces: a lane's 16 weights are half a group, two lanes share a byte)
-    const uint8_t* srow8 = (const uint8_t*)p.scale + (n0 + nrow) * p.s_cs + (HP ? g >> 1 : g);
+    const uint8_t* srow8 = (const uint8_t*)p.scale + (n0 + nrow) * p.s_cs + (E8H ? g >> 1 : g);
 
     // x copies: instruction `it` of this thread fills LDS piece it*NT + tid of the buffer, i.e. position
     // (it*NT + tid) % XPR of row (it*NT + tid) / XPR, with the row's piece position ^ (row % 16)
@@ -635,7 +638,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void w
     // WF 1: one scale per channel, read once.  WF 2 with the table: a table word holds the e8m0 bytes of 128 k; this lane's
     // 32 (8-byte pieces: 16) codes of a chunk belong to byte g of the chunk's word (g / 2 of the half that the chunk is)
     uint16_t sch[NB];
-    const int e8sh = 8 * (HP ? 2 * wk + (g >> 1) : g);
+    const int e8sh = 8 * (E8H ? 2 * wk + (g >> 1) : g);
     (void)sch; (void)e8sh;
     if constexpr (WF == 1) {
 #pragma unroll
@@ -1605,7 +1608,8 @@ static int launch_rows_one(const WqParams& p, hipStream_t st)
         // beside the x buffers (e2m1 codes: one word per 128 k, the four e8m0 bytes of a row read as a word; the caller
         // passes cpg_shift 0)
         const size_t red = (size_t)WN * (WK - 1) * NB * MB * 4 * 64 * 4;
-        const bool rows_ok = WF == 2 ? (p.s_cs % 4 == 0 && (uintptr_t)p.scale % 4 == 0 && p.cpg_shift == 0) : (p.s_rs == 1 || G == 1);
+        // (the caller counts a table word of 128 k in chunks: one of e2m1 codes, two of e4m3 codes)
+        const bool rows_ok = WF == 2 ? (p.s_cs % 4 == 0 && (uintptr_t)p.scale % 4 == 0 && p.cpg_shift == (WBITS == 8 ? 1 : 0)) : (p.s_rs == 1 || G == 1);
         if (rows_ok && (lds_x > red ? lds_x : red) + (size_t)(16 * NB * WN) * GP * 4 <= 160 * 1024)
             return launch_rows_one<XDT, WBITS, MB, NB, WN, WK, HAS_OFF, WF, true, KSP>(p, st);
     }
@@ -1676,6 +1680,14 @@ int launch_wq_rows_float(const WqParams& p, hipStream_t st);
     int launch_wq_rows_float<XDT, WBITS>(const WqParams& p, hipStream_t st)                                         \
     {                                                                                                               \
         constexpr int WF = WBITS == 4 ? 2 : 1;                                                                      \
+        if constexpr (WBITS == 8) {   /* e4m3 codes with e8m0 scales per 32 (no 64-column instance) */                 \
+            if (p.scale_e8m0) {                                                                                     \
+                if (p.m_rows > 192) return launch_rows_one<XDT, WBITS, 16, 2, 4, 2, false, 2>(p, st);               \
+                if (p.m_rows > 128) return launch_rows_one<XDT, WBITS, 12, 2, 4, 2, false, 2>(p, st);               \
+                return p.m_rows > 64 ? launch_rows_one<XDT, WBITS, 8, 2, 4, 2, false, 2>(p, st)                     \
+                                     : launch_rows_one<XDT, WBITS, 4, 2, 4, 2, false, 2>(p, st);                    \
+            }                                                                                                       \
+        }                                                                                                           \
         if (p.m_rows > 192) return launch_rows_one<XDT, WBITS, 16, 2, 4, 2, false, WF>(p, st);                      \
         if (p.m_rows > 128) return launch_rows_one<XDT, WBITS, 12, 2, 4, 2, false, WF>(p, st);                      \
         if (p.cols64 && p.m_rows <= 64) return launch_rows_one<XDT, WBITS, 4, 2, 2, 4, false, WF>(p, st);           \

@@ -309,6 +309,30 @@ def test_mxfp8_few_rows(gpu, M, K, N, exp_range, out):
     assert np.array_equal(cases.run_mx_aclnn(m, inp, M, K, N, True, dt, bias), want)
 
 
+@pytest.mark.parametrize("M,K,N,exp_range", [
+    # 33 .. 256 rows, bf16 output, K-contiguous x2: the 64- and 128-row instances, row slabs against a narrow x2 (N = 320: three
+    # workgroups), a last workgroup of 32 columns, a K of whole 128-element slabs that is no whole round (1664, 11008), K
+    # segments with partial sums (18432 against 256 columns), the 192- and 256-row instances against more than 128 workgroups,
+    # scale exponents over +-30 binades
+    (33, 1024, 256, 4), (64, 7168, 1024, 4), (100, 4096, 288, 4), (128, 1664, 512, 4), (200, 2048, 320, 4),
+    (96, 11008, 512, 4), (64, 18432, 256, 4), (192, 1536, 16640, 4), (256, 1024, 16640, 4), (48, 2048, 512, 30),
+    (130, 640, 16640, 4),       # (more than 128 rows per workgroup with a K that is no whole round of the 256-row instance: the tiles)
+])
+def test_mxfp8_many_rows(gpu, M, K, N, exp_range):
+    """MXFP8 with 33 .. 256 rows: x1 widened to bf16 with its block scales into the workspace, then the many-rows streaming
+    kernel on e4m3 codes with e8m0 group scales (exact products, fp32 sums) -- the stated bar; the plain kernel bit-identical."""
+    m = gpu
+    print(f"case mxfp8 many rows M={M} K={K} N={N} exp_range={exp_range}", flush=True)
+    inp = cases.make_mx_inputs(m, M, K, N, K + N + M, True, False, exp_range=exp_range)
+    bias = np.random.default_rng(1).normal(0, 1, N).astype(np.float32) if M % 2 == 0 else None
+    want = cases.oracle_mx(m, inp, M, K, N, True, m.ACL_BF16, bias)
+    plain(False)
+    got = cases.run_mx_aclnn(m, inp, M, K, N, True, m.ACL_BF16, bias)
+    check_close(got, want, orc.BF16, "mxfp8 many rows")
+    plain(True)
+    assert np.array_equal(cases.run_mx_aclnn(m, inp, M, K, N, True, m.ACL_BF16, bias), want)
+
+
 @pytest.mark.parametrize("M,K,N,tB,fp4,bias", [(256, 1024, 384, True, True, True), (300, 512, 262, True, True, False), (128, 512, 256, False, True, True),
                                                (200, 960, 264, True, True, False), (256, 1024, 384, True, False, True), (130, 256, 200, True, False, False)])
 def test_mx_fp32_output(gpu, M, K, N, tB, fp4, bias):
