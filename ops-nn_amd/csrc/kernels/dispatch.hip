@@ -206,8 +206,8 @@ static int splitk_for(const OpsnnQmmArgs& a, int mode)
     if ((mode == 1 || mode == 3) && f8 && a.M <= 128) {
         if (const int sr = mode == 1 ? blockscale_rows_ksplit(a) : rowcol_rows_ksplit(a); sr > 1) return sr;
     }
-    // 33 .. 256 rows of MXFP8 on the many-rows kernel (exact products: not when the 8-bit instruction was asked for)
-    if (mode == 2 && f8 && a.M <= 256 && !opsnnGetFp8Fast()) {
+    // 33 .. 256 rows of MXFP8 on the many-rows kernel
+    if (mode == 2 && f8 && a.M <= 256) {
         if (const int sr = mxfp8_rows_ksplit(a); sr > 1) return sr;
     }
     // (fewer than 64 x 64 outputs are the plain kernels' -- except int8 with few outputs against a long K, qmm_int8.hip)

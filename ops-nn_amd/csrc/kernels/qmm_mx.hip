@@ -249,7 +249,8 @@ int launch_mxfp8_rows(const OpsnnQmmArgs& a, void* region, hipStream_t st, Split
 // (in front of that: the bf16 copy of x1 for MXFP8 with 33 .. 256 rows on the many-rows kernel)
 static uint64_t mx_rows_bytes(const OpsnnQmmArgs& a)
 {
-    if (a.force_variant == OPSNN_VARIANT_PLAIN || opsnn_force_plain() || opsnnGetFp8Fast() || !mx_call_ok(a)) return 0;
+    // (whether or not opsnnSetFp8Fast is on: a workspace must not depend on a switch that may change between the two phases)
+    if (a.force_variant == OPSNN_VARIANT_PLAIN || opsnn_force_plain() || !mx_call_ok(a)) return 0;
     return align_up(mxfp8_rows_workspace(a), 256);
 }
 uint64_t mx_workspace_bytes(const OpsnnQmmArgs& a)
@@ -327,8 +328,11 @@ int launch_mx_mfma(const OpsnnQmmArgs& a0, hipStream_t st, SplitK sk)
     }
     if (a.x1_dtype == DT_E4M3 && a.x2_dtype == DT_E2M1) return launch_mx_a8w4_mfma(a, st, sk);   // fp8 x fp4: qmm_fp8_block.hip
     if (fp8 && rows_region) {   // MXFP8 with 33 .. 256 rows: the many-rows streaming kernel on bf16 operands (exact products)
-        const int rc = launch_mxfp8_rows(a, rows_region, st, sk);
-        if (rc != OPSNN_NOT_TAKEN) return rc;
+        if (!opsnnGetFp8Fast()) {
+            const int rc = launch_mxfp8_rows(a, rows_region, st, sk);
+            if (rc != OPSNN_NOT_TAKEN) return rc;
+        }
+        sk = SplitK{};   // (any partial sums were laid out for the kernel above; the tile kernels run unsplit)
     }
     if (fp8 && a.M <= 32) {   // MXFP8 with up to 32 rows: the stream over x2 with x1 in registers (exact products)
         const int rc = launch_mxfp8_decode(a, st, sk);
