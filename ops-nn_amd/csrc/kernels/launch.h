@@ -72,7 +72,7 @@ inline int splitk_factor(int64_t tiles, int64_t ktiles, double tile_us, int64_t 
 // (of 64 weight bytes): 16 x 4, 8-bit weights also 16 x 8, or 8 x 4 / 8 x 8.  A K that is exactly one such shape runs on
 // one workgroup per row block range; any other K of whole 128-element units goes in `splits` segments of 16 x 4 chunks
 // (else of 8 x 4), one workgroup column per segment, the last one with idle chunks past the end of K (`exact` false) when
-// that wastes at most a sixth of K's chunks; with more than one segment the columns leave fp32 partial sums
+// that wastes at most a fifth of K's chunks; with more than one segment the columns leave fp32 partial sums
 // [splits][M][N] at the front of the workspace.  False: the kernel does not take this K.
 struct WqXregPlan {
     int nw, nch, splits;
@@ -87,9 +87,9 @@ inline bool wq_xreg_plan(int wbits, int64_t M, int64_t K, WqXregPlan& pl)
     if (wbits == 8 && nch == 128) { pl = {16, 8, 1, true}; return true; }
     if (nch == 32) { pl = {8, 4, 1, true}; return true; }
     const int64_t s64 = (nch + 63) / 64, w64 = s64 * 64 - nch, s32 = (nch + 31) / 32, w32 = s32 * 32 - nch;
-    if (s64 == 1 && w64 * 6 <= nch) { pl = {16, 4, 1, false}; return true; }   // one workgroup, its last waves idle
-    if (s32 <= 16 && w32 * 6 <= nch) { pl = {8, 4, (int)s32, w32 == 0}; return true; }
-    if (s64 <= 16 && w64 * 6 <= nch) { pl = {16, 4, (int)s64, w64 == 0}; return true; }
+    if (s64 == 1 && w64 * 5 <= nch) { pl = {16, 4, 1, false}; return true; }   // one workgroup, its last waves idle
+    if (s32 <= 16 && w32 * 5 <= nch) { pl = {8, 4, (int)s32, w32 == 0}; return true; }
+    if (s64 <= 16 && w64 * 5 <= nch) { pl = {16, 4, (int)s64, w64 == 0}; return true; }
     return false;
 }
 // the count of partial-sum slices that plan needs (0: none)

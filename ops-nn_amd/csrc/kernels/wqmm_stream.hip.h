@@ -1469,10 +1469,10 @@ static int launch_xreg_one(const WqParams& p, hipStream_t st, int splits = 1)
     }
     const int64_t nblocks = (p.N + 15) / 16;
     if (splits < 1 || splits > 16 || (splits > 1 && (!p.part || p.m_base != 0 || p.m_rows != p.M))) return -1;
-    {   // the segments cover K, the last one with idle chunks worth at most a sixth of K; with idle chunks the vector scale
+    {   // the segments cover K, the last one with idle chunks worth at most a fifth of K; with idle chunks the vector scale
         // loads of a wave's last piece may reach past the row's last scale: the row's pitch must hold whole pieces
         const int64_t kc = 4 * (128 / WBITS), nch = p.K / kc, cover = (int64_t)splits * NW * NCH;
-        if (p.K % 128 != 0 || cover < nch || (cover - nch) * 6 > nch || cover - nch >= (int64_t)NW * NCH) return -1;
+        if (p.K % 128 != 0 || cover < nch || (cover - nch) * 5 > nch || cover - nch >= (int64_t)NW * NCH) return -1;
         if (cover != nch && SCM == 1 && (p.s_cs % 8 != 0 || p.s_cs < nch)) return -1;
         if (cover != nch && SCM == 2 && (p.s_cs % 16 != 0 || p.s_cs < nch * 4)) return -1;
     }

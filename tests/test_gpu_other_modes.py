@@ -716,6 +716,8 @@ def test_weight_only_rows_k_segments(gpu, M, K, N, x_dt, w_dt, group, off, bias)
     (4, 14336, 48, "f16", "i4", 0, True, False, None),
     (2, 14336, 72, "f16", "i4", 256, False, True, None),
     (16, 18432, 256, "f16", "i4", 128, True, True, None),      # 144 chunks in five segments of 32, vector scale loads
+    (16, 13824, 256, "f16", "i4", 128, True, True, None),      # 108 chunks in four segments of 32: 20 idle, the most the plan takes
+    (6, 13824, 264, "bf16", "fp4", 32, True, False, None),
     # ... floating-point codes: mxfp4 7168 = 8192 - 1024 in one workgroup, 18432 in five segments (a row's e8m0 bytes a whole
     # number of 16-byte pieces); e4m3 7168 = 4 x 2048 - 1024
     (16, 7168, 512, "f16", "fp4", 32, True, False, None),
