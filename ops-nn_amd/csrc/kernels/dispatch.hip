@@ -193,13 +193,14 @@ static int splitk_for(const OpsnnQmmArgs& a, int mode)
     const bool f8 = a.x1_dtype == DT_E4M3 && a.x2_dtype == DT_E4M3;
     // up to 32 rows of fp8 with block scales or row / column scales, or of int8 per-tile: the decode kernel's K segments
     const bool a8w4 = mode == 2 && a.x1_dtype == DT_E4M3 && a.x2_dtype == DT_E2M1;
-    if (a.M <= 32 && a.batch == 1 && a.N >= 256 &&
-        ((mode == 1 && (f8 || (a.x1_dtype == DT_I8 && a.x2_dtype == DT_I8)) && a.gsK == 128 && a.gsN == 128) ||
+    const bool i8pt = mode == 1 && a.x1_dtype == DT_I8 && a.x2_dtype == DT_I8;
+    if (a.M <= ((i8pt || a8w4) ? 16 : 32) && a.batch == 1 && a.N >= 256 &&
+        ((mode == 1 && (f8 || i8pt) && a.gsK == 128 && a.gsN == 128) ||
          (mode == 3 && f8 && a.x1_scale && a.x2_scale) || (a8w4 && out16) || (mode == 2 && f8))) {
         QmmDecodePlan pl;
         const int sd = qmm_decode_plan(a.K, true, pl, a8w4) ? pl.splits : 1;
         // (17 .. 32 rows of fp8 with block scales may also run on the many-rows kernel, with its own segments: room for either)
-        const int sr = mode == 1 && f8 ? blockscale_rows_ksplit(a) : mode == 3 && f8 ? rowcol_rows_ksplit(a) : 1;
+        const int sr = mode == 1 && f8 ? blockscale_rows_ksplit(a) : mode == 3 && f8 ? rowcol_rows_ksplit(a) : mode == 2 && f8 ? mxfp8_rows_ksplit(a) : 1;
         return sd > sr ? sd : sr;
     }
     // 33 .. 128 rows of fp8 with block scales or row / column scales on the many-rows kernel
@@ -232,7 +233,7 @@ static int splitk_for(const OpsnnQmmArgs& a, int mode)
         kunit = 256;
         tile_us = bm == 128 ? 0.6 : 1.3; bytes_per_us = 2.4e6;
     }
-    else if (a.M <= 32) return 1;   // (up to 32 rows the streaming kernels take the modes below)
+    else if (a.M <= 16) return 1;   // (up to 16 rows the streaming kernels take the modes below)
     else if (mode == 2 && a.x1_dtype == DT_E4M3 && a.x2_dtype == DT_E2M1 && out16) { bm = 256; tile_us = 1.8; }
     else if (mode == 1 && a.x1_dtype == DT_I8 && a.x2_dtype == DT_I8 && a.gsK == 128 && a.gsN == 128 && out16) { bm = a.M >= 512 ? 256 : 128; tile_us = 1.8; }
     else if (mode == 1 && f8 && a.gsK == 128 && a.gsN == 128 && !a.bias && a.M > 128 && (out16 || a.out_dtype == DT_F32)) { bm = 256; bn = 128; tile_us = 1.4; }

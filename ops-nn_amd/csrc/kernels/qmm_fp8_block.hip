@@ -611,7 +611,7 @@ int launch_mx_a8w4_mfma(const OpsnnQmmArgs& a, hipStream_t st, SplitK sk)
     {   // up to 32 rows: the stream over x2 with x1 in registers
         const int rc = launch_mx_a8w4_decode(a, st, sk);
         if (rc != OPSNN_NOT_TAKEN) return rc;
-        if (a.M <= 32) sk = SplitK{};   // (the partial sums were laid out for the kernel above; the tile kernel runs unsplit)
+        if (a.M <= 16) sk = SplitK{};   // (the partial sums were laid out for the kernel above; the tile kernel runs unsplit)
     }
     if (a.out_dtype != DT_BF16 && a.out_dtype != DT_F16) return OPSNN_NOT_TAKEN;
     if (a.K % 128 != 0 || a.M * a.N < 64 * 64 || a.x1.col_stride != 1 || a.x2.row_stride != 1) return OPSNN_NOT_TAKEN;
@@ -737,7 +737,7 @@ int launch_blockscale_mfma(const OpsnnQmmArgs& a0, hipStream_t st, SplitK sk)
         if (rc != OPSNN_NOT_TAKEN) return rc;
     }
     if (tiny) return OPSNN_NOT_TAKEN;
-    if (a.M <= 32) sk = SplitK{};   // (with so few rows the partial sums were laid out for the kernel above; the tile kernels run unsplit)
+    if (a.M <= (i8 ? 16 : 32)) sk = SplitK{};   // (with so few rows the partial sums were laid out for the kernel above; the tile kernels run unsplit)
     if (!i8 && (!opsnnGetFp8Fast() || out32)) {   // exact products and sums unless the caller asked for the 8-bit matrix instruction
         const int rc = launch_blockscale_exact(a, st, sk);
         if (rc != OPSNN_NOT_TAKEN || out32) return rc;

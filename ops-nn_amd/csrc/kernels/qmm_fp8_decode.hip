@@ -613,7 +613,8 @@ int launch_blockscale_decode(const OpsnnQmmArgs& a, hipStream_t st, SplitK sk)
     if ((!i8 && (a.x1_dtype != DT_E4M3 || a.x2_dtype != DT_E4M3)) || a.batch != 1) return OPSNN_NOT_TAKEN;
     if (a.out_dtype != DT_BF16 && a.out_dtype != DT_F16 && !(a.out_dtype == DT_F32 && !i8)) return OPSNN_NOT_TAKEN;
     if (a.bias && !(i8 && a.bias_dtype == DT_F32)) return OPSNN_NOT_TAKEN;
-    if (a.M > 32 || a.N < 256) return OPSNN_NOT_TAKEN;
+    // (int8: 17 .. 32 rows are one pass of the tile kernel with K split, ahead of two passes here: 32 x 18432 x 7168 66 us here, 42 there)
+    if (a.M > (i8 ? 16 : 32) || a.N < 256) return OPSNN_NOT_TAKEN;
     if (a.gsK != 128 || a.gsN != 128 || (a.gsM != 1 && a.gsM != 128)) return OPSNN_NOT_TAKEN;
     if (a.K % 128 != 0 || a.x1.col_stride != 1 || a.x2.row_stride != 1) return OPSNN_NOT_TAKEN;
     if (((uintptr_t)a.x1.ptr | (uintptr_t)a.x2.ptr | (uint64_t)a.x1.row_stride | (uint64_t)a.x2.col_stride) % 16) return OPSNN_NOT_TAKEN;
@@ -676,7 +677,8 @@ int launch_mx_a8w4_decode(const OpsnnQmmArgs& a, hipStream_t st, SplitK sk)
 {
     if (a.x1_dtype != DT_E4M3 || a.x2_dtype != DT_E2M1 || a.batch != 1) return OPSNN_NOT_TAKEN;
     if (a.out_dtype != DT_BF16 && a.out_dtype != DT_F16) return OPSNN_NOT_TAKEN;
-    if (a.M > 32 || a.N < 256 || a.K % 128 != 0 || a.x1.col_stride != 1 || a.x2.row_stride != 1 || a.x2.col_stride % 2) return OPSNN_NOT_TAKEN;
+    // (17 rows and more: one pass of the tile kernel with K split, ahead of two passes here)
+    if (a.M > 16 || a.N < 256 || a.K % 128 != 0 || a.x1.col_stride != 1 || a.x2.row_stride != 1 || a.x2.col_stride % 2) return OPSNN_NOT_TAKEN;
     if (a.x1_scale_mat.col_stride != 2 || a.x2_scale_mat.col_stride != 2) return OPSNN_NOT_TAKEN;   // [rows, K / 64, 2]: a row's bytes contiguous
     if (a.bias && a.bias_dtype != DT_F32 && a.bias_dtype != DT_BF16 && a.bias_dtype != DT_F16) return OPSNN_NOT_TAKEN;
     const int64_t ldb = a.x2.col_stride / 2;

@@ -144,7 +144,7 @@ int launch_rowcol_rows(const OpsnnQmmArgs& a, hipStream_t st, SplitK sk)
     return a.M > 64 ? launch_rows_one<DT_F16, 8, 8, 2, 4, 2, false, 4>(p, st) : launch_rows_one<DT_F16, 8, 4, 2, 4, 2, false, 4>(p, st);
 }
 
-// ---- MXFP8 (e8m0 scales per 32 elements of K on both operands) with 33 .. 256 rows of x1 ----
+// ---- MXFP8 (e8m0 scales per 32 elements of K on both operands) with 17 .. 256 rows of x1 ----
 // The many-rows kernel in its weight-only form for e4m3 codes with e8m0 group scales and bf16 activations: a pre-step widens
 // x1 to bf16 with its block scales folded in (an e4m3 value times a power of two is a bf16 value wherever fp32 would hold
 // it: M * K * 2 bytes of workspace), the kernel widens x2's codes the same way (T(w * s) is exact) and
@@ -179,7 +179,7 @@ bool mx8_rows_eligible(const OpsnnQmmArgs& a)
 {
     if (a.x1_dtype != DT_E4M3 || a.x2_dtype != DT_E4M3 || a.batch != 1 || a.out_dtype != DT_BF16) return false;
     if (a.force_variant != 0 || (a.bias && a.bias_dtype != DT_F32)) return false;
-    if (a.M <= 32 || a.M > 256 || a.N % 32 != 0 || a.N < 256 || a.K % 128 != 0 || a.K >= (1ll << 23)) return false;
+    if (a.M <= 16 || a.M > 256 || a.N % 32 != 0 || a.N < 256 || a.K % 128 != 0 || a.K >= (1ll << 23)) return false;
     if (a.x1.col_stride != 1 || a.x2.row_stride != 1 || a.x1.row_stride < a.K || a.x2.col_stride < a.K) return false;
     if (((uintptr_t)a.x1.ptr | (uintptr_t)a.x2.ptr | (uint64_t)a.x1.row_stride | (uint64_t)a.x2.col_stride) % 16 || (uintptr_t)a.out % 16) return false;
     if (a.x1_scale_mat.col_stride != 2 || a.x2_scale_mat.col_stride != 2) return false;   // [rows, K / 64, 2]: a row's bytes contiguous

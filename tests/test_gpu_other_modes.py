@@ -310,16 +310,17 @@ def test_mxfp8_few_rows(gpu, M, K, N, exp_range, out):
 
 
 @pytest.mark.parametrize("M,K,N,exp_range", [
-    # 33 .. 256 rows, bf16 output, K-contiguous x2: the 64- and 128-row instances, row slabs against a narrow x2 (N = 320: three
+    # 17 .. 256 rows, bf16 output, K-contiguous x2: the 64- and 128-row instances, row slabs against a narrow x2 (N = 320: three
     # workgroups), a last workgroup of 32 columns, a K of whole 128-element slabs that is no whole round (1664, 11008), K
     # segments with partial sums (18432 against 256 columns), the 192- and 256-row instances against more than 128 workgroups,
     # scale exponents over +-30 binades
+    (17, 2048, 256, 4), (24, 8192, 512, 4),
     (33, 1024, 256, 4), (64, 7168, 1024, 4), (100, 4096, 288, 4), (128, 1664, 512, 4), (200, 2048, 320, 4),
     (96, 11008, 512, 4), (64, 18432, 256, 4), (192, 1536, 16640, 4), (256, 1024, 16640, 4), (48, 2048, 512, 30),
     (130, 640, 16640, 4),       # (more than 128 rows per workgroup with a K that is no whole round of the 256-row instance: the tiles)
 ])
 def test_mxfp8_many_rows(gpu, M, K, N, exp_range):
-    """MXFP8 with 33 .. 256 rows: x1 widened to bf16 with its block scales into the workspace, then the many-rows streaming
+    """MXFP8 with 17 .. 256 rows: x1 widened to bf16 with its block scales into the workspace, then the many-rows streaming
     kernel on e4m3 codes with e8m0 group scales (exact products, fp32 sums) -- the stated bar; the plain kernel bit-identical."""
     m = gpu
     print(f"case mxfp8 many rows M={M} K={K} N={N} exp_range={exp_range}", flush=True)

@@ -144,7 +144,9 @@ def test_gpu_a8w4_mx(gpu, M, K, N, tB):
                                    (16, 2048, 256),
                                    # ... a K that one workgroup's waves do not share exactly: one segment with idle waves (28
                                    # chunks), K segments with fp32 partial sums (86, 144, 19 chunks; two passes; one row)
-                                   (16, 3584, 256), (16, 11008, 264), (32, 18432, 256), (7, 2432, 512), (1, 18944, 384),
+                                   (16, 3584, 256), (16, 11008, 264), (7, 2432, 512), (1, 18944, 384),
+                                   # 17 .. 32 rows: the tile kernel, with K split where the tiles are few
+                                   (32, 18432, 256), (24, 4096, 512), (17, 11008, 264),
                                    # few tiles against a long K: K split over 2 .. 16 workgroups per tile, fp32 partial sums in the
                                    # workspace, summed in split order (also (512, 2048, 520), (100, 1024, 1000) and
                                    # (1024, 4096, 1024) above); a column count that is no multiple of 4
