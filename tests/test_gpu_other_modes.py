@@ -151,7 +151,7 @@ def _rows_ksplit(wbits, M, N, K, group):
     # segments over workgroup columns with fp32 partial sums and a second kernel (86 blocks: three segments of 16 x 2; 144:
     # three of 8 x 6; 108: seven of 16 x 1; 19: three of 8 x 1; 148 in two passes: five of 16 x 2)
     (5, 3584, 264, 1, "f16"), (16, 11008, 512, 1, "bf16"), (16, 18432, 256, 1, "bf16"), (12, 13824, 384, 128, "f32"),
-    (16, 2432, 256, 1, "f16"), (32, 18944, 264, 1, "bf16"),
+    (16, 2432, 256, 1, "f16"), (32, 18944, 264, 1, "bf16"), (4, 128, 256, 1, "bf16"), (16, 640, 272, 1, "f32"),
     # 17 .. 32 rows where the many-rows kernel does not apply (N % 128, K % 512): two passes; one scale row for all of x1 (B-B)
     (17, 2048, 520, 1, "bf16"), (32, 7168, 520, 128, "f16"), (24, 1024, 256, 1, "f32"), (20, 4096, 256, 1, "f32"),
     # 17 .. 64 rows (N % 128 == 0, K % 512 == 0): x1 widened into the workspace, the many-rows streaming kernel
@@ -284,7 +284,7 @@ def test_mxfp8_exact_window(gpu, exp_range, batch):
     # (the long sums with fp16 output: fp32 sums in another order than the oracle's flip one bf16 result in a thousand by an
     # ulp, which is four times the 1e-3 the bar allows)
     (16, 3584, 256, 4, "f32"), (16, 11008, 264, 4, "f16"), (20, 18432, 256, 4, "f16"), (1, 18944, 384, 4, "f16"),
-    (16, 2048, 320, 30, "f32"), (12, 4096, 256, 14, "bf16"),
+    (16, 2048, 320, 30, "f32"), (12, 4096, 256, 14, "bf16"), (2, 128, 256, 4, "bf16"), (16, 384, 264, 4, "f16"),
 ])
 def test_mxfp8_few_rows(gpu, M, K, N, exp_range, out):
     """MXFP8 with up to 32 rows: x1 in registers and x2 streamed once per 16 rows, both widened to bf16 with their block's

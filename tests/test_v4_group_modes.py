@@ -144,7 +144,7 @@ def test_gpu_a8w4_mx(gpu, M, K, N, tB):
                                    (16, 2048, 256),
                                    # ... a K that one workgroup's waves do not share exactly: one segment with idle waves (28
                                    # chunks), K segments with fp32 partial sums (86, 144, 19 chunks; two passes; one row)
-                                   (16, 3584, 256), (16, 11008, 264), (7, 2432, 512), (1, 18944, 384),
+                                   (16, 3584, 256), (16, 11008, 264), (7, 2432, 512), (1, 18944, 384), (3, 128, 256), (16, 640, 264),
                                    # 17 .. 32 rows: the tile kernel, with K split where the tiles are few
                                    (32, 18432, 256), (24, 4096, 512), (17, 11008, 264),
                                    # few tiles against a long K: K split over 2 .. 16 workgroups per tile, fp32 partial sums in the
@@ -258,7 +258,7 @@ def test_gpu_pertile_i8(gpu, M, K, N, tB):
                                       (16, 4096, 512, True), (9, 2048, 264, True), (24, 1024, 520, True), (16, 1024, 256, False),
                                       (1, 7168, 384, True),
                                       # ... a K that one workgroup's waves do not share exactly: idle waves, K segments
-                                      (16, 3584, 256, True), (16, 11008, 264, True), (20, 18432, 256, True),
+                                      (16, 3584, 256, True), (16, 11008, 264, True), (20, 18432, 256, True), (5, 128, 256, True),
                                       # few tiles against a long K: the K split ((640, 1024, 520) above: with the re-layout of
                                       # an N-contiguous x2 behind the partial sums in the workspace)
                                       (128, 4096, 4096, True), (40, 8192, 256, True), (96, 1024, 258, True), (200, 2048, 1000, False)])
