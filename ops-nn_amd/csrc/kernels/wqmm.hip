@@ -387,7 +387,7 @@ static int launch_slabs_float(WqParams p, hipStream_t st)
         constexpr int64_t KC = 4 * (128 / WBITS);
         constexpr int rows_min = 17;
         bool ok = !p.offset && p.M >= rows_min && p.K % KC == 0 && (p.K / KC) % 2 == 0 && p.N % 32 == 0 && p.N >= 256 && p.K < (1ll << 23);
-        const bool mx8 = WBITS == 8 && p.scale_e8m0;   // e4m3 codes with e8m0 scales per 32 (MXFP8's x2: launch_wq_mx8_rows)
+        const bool mx8 = WBITS == 8 && p.scale_e8m0 && p.mx8_rows;   // e4m3 codes with e8m0 scales per 32 (MXFP8's x2: launch_wq_mx8_rows)
         if (WBITS == 4 || mx8) ok = ok && p.scale_e8m0 && p.group == 32 && p.s_rs == 1;
         else ok = ok && !p.scale_e8m0 && p.group >= p.K;
         // (the kernel's scale table counts in words of four e8m0 bytes = 128 k: one chunk of e2m1 codes, two of e4m3 codes)
@@ -543,7 +543,7 @@ static int launch_slabs(WqParams p, hipStream_t st)
 int launch_wq_mx8_rows(const WqParams& p0, hipStream_t st)
 {
     WqParams p = p0;
-    p.w_float = 1; p.scale_e8m0 = 1; p.group = 32; p.group_shift = 5; p.s_rs = 1; p.offset = nullptr;
+    p.w_float = 1; p.scale_e8m0 = 1; p.mx8_rows = 1; p.group = 32; p.group_shift = 5; p.s_rs = 1; p.offset = nullptr;
     constexpr int64_t KC = 64;
     if (p.M < 17 || p.K % (2 * KC) != 0 || p.N % 32 != 0 || p.N < 256 || p.K >= (1ll << 23)) return OPSNN_NOT_TAKEN;
     const int64_t nslab = narrow_n_slab(p.M, p.N);

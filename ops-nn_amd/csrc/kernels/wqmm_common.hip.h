@@ -33,6 +33,7 @@ struct WqParams {
     int cols64;              // launcher hint: up to 64 rows on the instance whose workgroups take 64 columns (K split over four waves)
     int w_float;             // weights are floating-point codes (4 bits: e2m1, 8 bits: e4m3), not two's-complement integers
     int scale_e8m0;          // scale is one e8m0 byte per element (MX), not a 16-bit value of x's dtype
+    int mx8_rows;            // set by launch_wq_mx8_rows only: e4m3 codes with e8m0 scales per 32 on the many-rows kernel (MXFP8's x2)
     // fp8 block-scale form of the many-rows kernel (x is x1 widened to fp16, w is x2 in e4m3): fp32 scales per 128 x 128
     // block of w (bs2) and per row group and 128-block of x (bs1), output type of the call
     const float* bs1; const float* bs2;
