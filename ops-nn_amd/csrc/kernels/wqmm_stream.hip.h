@@ -609,7 +609,8 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void w
     // two at or above the groups per row; the swizzle (4 * (rw % 16), kept below P) spreads the 16 rows that one read touches
     // over the banks.  The table is complete behind the loop's first barrier.
     uint32_t* stab = (uint32_t*)(sx + LDS_MAIN);
-    const int sG = p.cpg_shift >= 31 ? 1 : (int)((p.K / KCH) >> p.cpg_shift);   // groups of this workgroup's K
+    // groups of this workgroup's K (the last one may be short)
+    const int sG = p.cpg_shift >= 31 ? 1 : (int)(((p.K / KCH) + (1ll << p.cpg_shift) - 1) >> p.cpg_shift);
     const int sP = sG <= 1 ? 1 : 1 << (32 - __builtin_clz((unsigned)(sG - 1)));    // a table row's pitch: the power of two at or above
     const int cpg_shift = p.cpg_shift >= 31 ? 31 : p.cpg_shift + (HP ? 1 : 0);   // chunks of this kernel per group
     int stab_row[NB], stab_sw[NB];
@@ -1600,7 +1601,7 @@ static int launch_rows_one(const WqParams& p, hipStream_t st)
         kseg = (p.K / p.kunit + p.ksplit - 1) / p.ksplit * p.kunit;
     }
     // groups of that K, and the pitch of a scale table row: the power of two at or above
-    const int64_t G = p.cpg_shift >= 31 ? 1 : ((kseg / KC) >> p.cpg_shift);
+    const int64_t G = p.cpg_shift >= 31 ? 1 : (((kseg / KC) + (1ll << p.cpg_shift) - 1) >> p.cpg_shift);   // (the last group may be short)
     int64_t GP = 1;
     while (GP < G) GP *= 2;
     if constexpr ((WF == 0 || WF == 2) && !SLDS) {

@@ -587,6 +587,9 @@ def test_weight_only_256_row_instance(gpu, M, K, N, x_dt, w_dt, group, tW, off, 
     # K in whole x slabs (two chunks on 128-column workgroups, four on 64-column ones) but no whole rounds of the chunk
     # pipeline: a shorter last round behind the loop, on the 64- and 128-row instances; the 192- / 256-row ones decline
     (64, 1280, 256, "f16", "i4", 128, True, None),            # five slabs on 128-column workgroups
+    (64, 2816, 256, "f16", "i4", 512, True, None),            # ... and a short last group (5.5 groups): six table entries per row
+    (100, 3072, 288, "bf16", "i4", 2048, True, "bf16"),       # one and a half groups
+    (64, 1408, 256, "bf16", "i8", 256, True, None),
     (64, 1536, 288, "bf16", "i4", 128, False, "bf16"),        # three slabs on 64-column workgroups, six on 128-column ones
     (128, 3584, 256, "f16", "i4", 128, True, None),           # seven / fourteen slabs; one pass: the 128-row instance
     (100, 640, 320, "bf16", "i8", 64, True, None),
