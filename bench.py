@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the quantized-matmul hot path on one MI355X.
 
-  python bench.py [--gpus 1] [--steps K] [--warmup W] [--config 1..14] [--shape M,K,N] [--m M] [--cold] [--fp8-fast] [--no-cpu] [--calib-copy] [--layout packed|nd] [--weight-cache MB]
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--config 1..15] [--shape M,K,N] [--m M] [--cold] [--fp8-fast] [--no-cpu] [--calib-copy] [--layout packed|nd] [--weight-cache MB]
 
 A step is one pass of the operator (both aclnn phases) over one batch of synthetic, seeded input that is already
 resident in HBM.  One JSON line is printed.
@@ -94,8 +94,8 @@ def main():
                     help="0 (default): every BASELINE config, headline config 2; 1-5: that BASELINE config only; 6-9: the "
                          "pre-pack / quantizer operators that prepare their tensors; 10: the int4 x int4 K-G mode at 4096^3; "
                          "11: config 3's shape with mxfp4 weights; 12: config 4's operator with the --m rows of a decode step; "
-                         "13 / 14: the fp8 x fp4 MX mode / the int8 per-tile mode at config 3's K and N with the --m rows of a decode step")
-    ap.add_argument("--m", type=int, default=None, help="M for config 3 (1, 16, 64 or 256) and configs 11 to 14 (default 16)")
+                         "13 / 14 / 15: the fp8 x fp4 MX mode / the int8 per-tile mode / MXFP8 at config 3's K and N with the --m rows of a decode step")
+    ap.add_argument("--m", type=int, default=None, help="M for config 3 (1, 16, 64 or 256) and configs 11 to 15 (default 16)")
     ap.add_argument("--shape", default=None, metavar="M,K,N",
                     help="configs 2, 4 and 5 (one batch) at another shape, e.g. --config 4 --shape 512,7168,2048: the mid-size "
                          "calls whose few tiles split K (not a BASELINE workload; the record says so)")

@@ -320,6 +320,58 @@ class ConfigPerTileRows(Workload):
                 "sample": f"first {rows} of {self.M} rows of x1 against the full x2 (oracle/liboracle.so, OpenMP), {t:.2f} s"}
 
 
+class ConfigMxfp8Rows(Workload):
+    """Not a BASELINE config: MXFP8 (e4m3 x e4m3, e8m0 scales per 32 elements of K on both operands) at config 3's K and N with
+    the few rows of x1 of a decode step (--m, default 16): a stream over x2 against the HBM roofline."""
+    metric = "quant_gemm_stream_bandwidth"
+    bound = "hbm"
+    peak_key = "fp8"
+    dtype = "fp8_e4m3 x fp8_e4m3, both widened to bf16 with their e8m0 block scales (exact), fp32 sums"
+    kernel = "mx8_decode_kernel (v_mfma_f32_16x16x32_bf16); from 17 rows wqmm_rows_kernel on e4m3 codes with e8m0 scales"
+
+    def __init__(self, m, args, K=8192, N=28672):
+        M = args.m or 16
+        self.m, self.M, self.K, self.N = m, M, K, N
+        self.inp = cases.make_mx_inputs(m, M, K, N, 0, True, False)
+        self.d = {k: m.DeviceBuffer(host=v) for k, v in self.inp.items() if isinstance(v, np.ndarray)}
+        self.d_out = m.DeviceBuffer(M * N * 2)
+        KS = K // 64
+        self.t_x1 = m.Tensor((M, K), m.ACL_FLOAT8_E4M3FN, self.d["x1"])
+        self.t_x2 = m.Tensor((N, K), m.ACL_FLOAT8_E4M3FN, self.d["x2"])
+        self.t_s1 = m.Tensor((M, KS, 2), m.ACL_FLOAT8_E8M0, self.d["s1"])
+        self.t_s2 = m.Tensor((N, KS, 2), m.ACL_FLOAT8_E8M0, self.d["s2"])
+        self.t_out = m.Tensor((M, N), m.ACL_BF16, self.d_out)
+        self.gs = (1 << 32) | (1 << 16) | 32
+        rc, ws, ex = self._phase1()
+        m.lib().aclDestroyAclOpExecutor(ex)
+        self.ws = m.DeviceBuffer(ws) if ws else None
+        self.ws_size = ws
+        self.flop = 2 * M * N * K
+        self.bytes = M * K + N * K + M * K // 32 + N * K // 32 + 2 * M * N
+        self.config = {"workload": "aclnnQuantMatmulV5 MXFP8 (e8m0 scales per 32 K), bf16 out, decode rows", "M": M, "K": K, "N": N,
+                       "x2_layout": "K-contiguous (transposeX2)"}
+
+    def _phase1(self):
+        m = self.m
+        rc, ws, ex = m.quant_matmul_v5_get_workspace(self.t_x1, self.t_x2, self.t_s1, self.t_s2, self.t_out, transpose_x2=True, group_size=self.gs)
+        m.check(rc, "phase 1")
+        return rc, ws, ex
+
+    def step(self, stream):
+        m = self.m
+        rc, ws, ex = self._phase1()
+        m.check(m.lib().aclnnQuantMatmulV5(self.ws.ptr if self.ws else None, self.ws_size, ex, stream.ptr), "phase 2")
+
+    def cpu_baseline(self):
+        rows = min(self.M, 16)
+        t0 = time.perf_counter()
+        orc.qmm_mx(np.ascontiguousarray(self.inp["x1"][0][:rows]), self.inp["x2"][0], orc.E4M3, orc.E4M3, rows, self.K, self.N, False, True,
+                   np.ascontiguousarray(self.inp["s1"][0][:rows]), np.ascontiguousarray(self.inp["s2"][0]), None, orc.BF16)
+        t = time.perf_counter() - t0
+        return {"value": self.bytes * rows / self.M / t / 1e9, "unit": "GB/s", "cores": _cores(), "kind": "port",
+                "sample": f"first {rows} of {self.M} rows of x1 against the full x2 (oracle/liboracle.so, OpenMP), {t:.2f} s"}
+
+
 class Config5(Workload):
     """aclnnQuantMatmulV5, MXFP4 (e2m1 with e8m0 scale per 32 K), batch 8, bf16 output."""
     peak_key, dtype = "fp4", "fp4_e2m1"
@@ -610,6 +662,8 @@ def make_workload(m, config, args):
         return ConfigA8W4Rows(m, args)
     if config == 14:
         return ConfigPerTileRows(m, args)
+    if config == 15:
+        return ConfigMxfp8Rows(m, args)
     if config == 5:
         return Config5(m, args)
     raise SystemExit(f"bench.py: config {config} is not wired up yet")
