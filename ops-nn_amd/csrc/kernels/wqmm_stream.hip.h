@@ -1101,11 +1101,12 @@ __global__ __launch_bounds__(256, 2) void wqmm_resx_kernel(WqParams p)
                     }
                 }
                 if constexpr (LAST) {
-                    // slot j next holds chunk cw + PF of this row block, or, past its end, a chunk of the next one
-                    // (clamped when the stream ends: the value is then never used)
+                    // slot j next holds chunk cw + PF of this row block, or, past its end, the chunk of the next row block
+                    // that the slot serves first: chunk j of its first super-step (not cw + PF - NCW: that is the same only
+                    // when a row block is a whole number of super-steps)
                     const int nx = cw + PF;
                     if (nx < NCW) fetch(j, wptr, srow, orow, nx);
-                    else fetch(j, wptr_n, srow_n, orow_n, (nx - NCW) < NCW ? (nx - NCW) : NCW - 1);
+                    else fetch(j, wptr_n, srow_n, orow_n, j < NCW ? j : NCW - 1);
                 } else {
                     fetch(j, wptr, srow, orow, cw + PF);
                 }

@@ -458,6 +458,11 @@ def test_mx_batched(gpu, M, K, N, batch):
     (16, 1152, 8208, "f16", "i4", 128, True, True, None),       # 9 groups: not a multiple of 8; 513 row blocks
     (9, 640, 96, "bf16", "i8", 128, True, True, "bf16"),
     (64, 1024, 320, "bf16", "i8", 0, True, False, None),
+    # ... x whole in LDS with more row blocks than workgroups (513 on 512) and a row block that is no whole number of
+    # eight-chunk super-steps (4, 3 and 4 chunks per wave): the refills that run into the next row block
+    (3, 2048, 8208, "f16", "i4", 128, True, True, None),
+    (16, 1536, 8240, "bf16", "i4", 0, True, False, "bf16"),
+    (9, 1024, 8208, "f16", "i8", 64, True, True, None),
     # ... K split between the waves of a workgroup (narrow N, M <= 16)
     (16, 4096, 256, "bf16", "i8", 0, True, False, None),
     (1, 4096, 200, "f16", "i4", 128, True, True, "f16"),

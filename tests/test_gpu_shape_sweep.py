@@ -1,0 +1,129 @@
+"""Seeded sweeps over (M, K, N) for the modes whose kernel choice depends on the shape: few rows against many, a K that is or
+is not a whole number of a kernel's units, a narrow or a wide right operand.  The single shapes of the other test files name
+the case each of them is there for; these sweeps look for the combinations between them (a selector's thresholds, the K
+segments, idle waves, row slabs, short last rounds).  Every case is compared with the oracle at the mode's own bar; the
+shapes are small enough for the whole file to run in well under a minute.
+"""
+import numpy as np
+import pytest
+
+import cases
+import oracle_api as orc
+from test_gpu_other_modes import check_close, plain
+
+pytestmark = pytest.mark.gpu
+
+
+def _shapes(seed, count, m_max, k_unit, k_max, n_unit, n_lo, n_hi):
+    """`count` shapes: M from the few-rows, many-rows and tile ranges, K in whole units, N in whole units."""
+    rng = np.random.default_rng(seed)
+    out = []
+    for i in range(count):
+        lo, hi = ((1, 17), (17, 65), (65, 257), (257, m_max + 1))[i % 4]
+        hi = min(hi, m_max + 1)
+        M = int(rng.integers(lo, hi)) if lo < hi else int(rng.integers(1, m_max + 1))
+        K = int(rng.integers(1, k_max // k_unit + 1)) * k_unit
+        N = int(rng.integers(n_lo // n_unit, n_hi // n_unit + 1)) * n_unit
+        out.append((M, K, N))
+    return out
+
+
+def _b16_bar(got, want, code, what, K=0):
+    g, w = orc.b16_to_f32(got, code), orc.b16_to_f32(want, code)
+    assert np.isfinite(g).all(), what
+    mx, mean = orc.rel_err_stats(g, w)
+    assert mx <= 2.0 ** -7 and mean <= 2.0 ** -10, f"{what}: max rel {mx:.3e} mean rel {mean:.3e}"
+    # 99.9 % within rtol = atol = 1e-3.  Two allowances that the single-shape tests do not need: with a few hundred outputs one
+    # bf16 result an ulp off is already more than a thousandth of them; and beyond K = 8192 fp32 sums in another order than the
+    # oracle's flip one bf16 result in a thousand by an ulp (four times the 1e-3), so bf16 outputs get 3e-3 there.
+    allow = max(3e-3 if (K > 8192 and code == orc.BF16) else 1e-3, 2.0 / g.size)
+    frac = orc.isclose_fraction(g, w)
+    assert frac <= allow, f"{what}: {frac:.2e} of elements outside rtol=atol=1e-3"
+
+
+# (the last six of each list: more than 128 workgroups of 128 columns, where the 192- / 256-row instances and the tiles take over)
+@pytest.mark.parametrize("M,K,N", _shapes(11, 40, 400, 128, 6144, 32, 256, 1024) + _shapes(31, 6, 300, 128, 1536, 32, 16512, 20480))
+@pytest.mark.parametrize("w_dt,group", [("i4", 128), ("i8", 0), ("i4", 512), ("fp4", 32)])
+def test_weight_only_shapes(gpu, M, K, N, w_dt, group):
+    m = gpu
+    if w_dt == "i4" and K % 256:
+        K += 128   # (int4 rows of whole 16-byte pieces per chunk pair keep the case on the streamlined kernels)
+    if group and K <= group:
+        group = 0 if w_dt != "fp4" else 32
+    dt = {"i8": m.ACL_INT8, "i4": m.ACL_INT4, "fp4": m.ACL_FLOAT4_E2M1}
+    x_dt = m.ACL_FLOAT16 if (M + N) % 2 else m.ACL_BF16
+    print(f"case sweep weight-only M={M} K={K} N={N} w={w_dt} g={group}", flush=True)
+    inp = cases.make_wq_inputs(m, M, K, N, M + K + N, x_dt, dt[w_dt], group, True, w_dt != "fp4", None)
+    want = cases.oracle_wq(m, inp, M, K, N)
+    plain(False)
+    check_close(cases.run_wq_aclnn(m, inp, M, K, N), want, x_dt, "weight-only sweep")
+
+
+@pytest.mark.parametrize("M,K,N", _shapes(12, 32, 300, 128, 4096, 128, 256, 1024) + _shapes(13, 8, 64, 128, 20480, 8, 256, 520) +
+                         _shapes(32, 6, 300, 128, 1536, 128, 16512, 20480))
+def test_fp8_block_scale_shapes(gpu, M, K, N):
+    m = gpu
+    gsM = 128 if (M + K) % 3 == 0 else 1
+    out = (m.ACL_BF16, m.ACL_FLOAT16, m.ACL_FLOAT)[(M + N) % 3]
+    print(f"case sweep fp8 block M={M} K={K} N={N} gsM={gsM} out={out}", flush=True)
+    inp = cases.make_blockscale_inputs(m, M, K, N, M + N + K, True, gsM)
+    want = cases.oracle_blockscale(m, inp, M, K, N, True, out)
+    got = cases.run_blockscale_aclnn(m, inp, M, K, N, True, out)
+    if out == m.ACL_FLOAT:
+        assert np.isfinite(got).all()
+        mx, mean = orc.rel_err_stats(got, want)
+        assert mean <= 2.0 ** -16 and orc.isclose_fraction(got, want) == 0.0, f"max rel {mx:.3e} mean rel {mean:.3e}"
+    else:
+        _b16_bar(got, want, orc.BF16 if out == m.ACL_BF16 else orc.F16, "fp8 block sweep", K)
+
+
+@pytest.mark.parametrize("M,K,N", _shapes(14, 24, 300, 128, 4096, 32, 256, 1024) + _shapes(15, 8, 64, 128, 20480, 8, 256, 520) +
+                         _shapes(33, 6, 300, 128, 1536, 32, 16512, 20480))
+def test_fp8_row_column_scale_shapes(gpu, M, K, N):
+    m = gpu
+    out = m.ACL_BF16 if (M + N) % 2 else m.ACL_FLOAT16
+    print(f"case sweep fp8 K-C M={M} K={K} N={N}", flush=True)
+    inp = cases.make_tc_inputs(m, M, K, N, M + N, m.ACL_FLOAT8_E4M3FN, m.ACL_FLOAT, N, m.ACL_FLOAT if K % 256 else None, True, pertoken="M")
+    want = cases.oracle_tc(m, inp, M, K, N, out)
+    _b16_bar(cases.run_tc_aclnn(m, inp, M, K, N, out), want, orc.BF16 if out == m.ACL_BF16 else orc.F16, "fp8 K-C sweep", K)
+
+
+@pytest.mark.parametrize("M,K,N", _shapes(16, 24, 300, 128, 4096, 8, 256, 1024) + _shapes(17, 8, 64, 128, 20480, 8, 256, 520))
+def test_int8_per_tile_shapes(gpu, M, K, N):
+    m = gpu
+    print(f"case sweep int8 per-tile M={M} K={K} N={N}", flush=True)
+    inp = cases.make_pertile_i8_inputs(m, M, K, N, M + N, True)
+    want = cases.oracle_pertile_i8(m, inp, M, K, N, True, m.ACL_BF16)
+    _b16_bar(cases.run_pertile_i8_aclnn(m, inp, M, K, N, True, m.ACL_BF16), want, orc.BF16, "int8 per-tile sweep", K)
+
+
+@pytest.mark.parametrize("M,K,N", _shapes(18, 24, 300, 128, 4096, 8, 256, 1024) + _shapes(19, 8, 64, 128, 20480, 8, 256, 520))
+def test_fp8_fp4_mx_shapes(gpu, M, K, N):
+    m = gpu
+    print(f"case sweep fp8 x fp4 MX M={M} K={K} N={N}", flush=True)
+    inp = cases.make_a8w4_mx_inputs(m, M, K, N, M + N, True)
+    want = cases.oracle_a8w4_mx(m, inp, M, K, N, True, m.ACL_FLOAT16)
+    _b16_bar(cases.run_a8w4_mx_aclnn(m, inp, M, K, N, True, m.ACL_FLOAT16), want, orc.F16, "fp8 x fp4 MX sweep", K)
+
+
+@pytest.mark.parametrize("M,K,N", _shapes(20, 32, 300, 128, 4096, 32, 256, 1024) + _shapes(21, 8, 64, 128, 20480, 8, 256, 520) +
+                         _shapes(34, 6, 300, 128, 1536, 32, 16512, 20480))
+@pytest.mark.parametrize("fp4", [False, True])
+def test_mx_shapes(gpu, M, K, N, fp4):
+    m = gpu
+    out = m.ACL_BF16 if (fp4 or (M + K // 128) % 2) else m.ACL_FLOAT16   # (sums of e2m1 products with these scales leave the fp16 range)
+    print(f"case sweep mx M={M} K={K} N={N} fp4={fp4} out={out}", flush=True)
+    inp = cases.make_mx_inputs(m, M, K, N, K + N + M, True, fp4)
+    bias = np.random.default_rng(M).normal(0, 1, N).astype(np.float32) if N % 64 == 0 else None
+    want = cases.oracle_mx(m, inp, M, K, N, True, out, bias)
+    plain(False)
+    _b16_bar(cases.run_mx_aclnn(m, inp, M, K, N, True, out, bias), want, orc.BF16 if out == m.ACL_BF16 else orc.F16, "mx sweep", K)
+
+
+@pytest.mark.parametrize("M,K,N", _shapes(22, 24, 300, 16, 4096, 8, 64, 1024) + _shapes(23, 8, 16, 128, 20480, 8, 256, 520))
+def test_int8_shapes_are_bit_identical(gpu, M, K, N):
+    m = gpu
+    print(f"case sweep int8 K-C M={M} K={K} N={N}", flush=True)
+    got, want, _ = cases.run_qmm_int8_case(m, orc, M, K, N, seed=M * 31 + N, out_dtype=m.ACL_BF16, bias_dtype=m.ACL_BF16 if K % 32 else None,
+                                           transpose_x2=True)
+    assert np.array_equal(got, want), f"{int((got != want).sum())} of {got.size} outputs differ"
