@@ -127,3 +127,74 @@ def test_int8_shapes_are_bit_identical(gpu, M, K, N):
     got, want, _ = cases.run_qmm_int8_case(m, orc, M, K, N, seed=M * 31 + N, out_dtype=m.ACL_BF16, bias_dtype=m.ACL_BF16 if K % 32 else None,
                                            transpose_x2=True)
     assert np.array_equal(got, want), f"{int((got != want).sum())} of {got.size} outputs differ"
+
+
+# ---- few rows against a wide right operand: every stream kernel's workgroups walk several column blocks ----
+def _few_rows_wide(seed, count, m_max, k_unit, k_max, n_unit):
+    rng = np.random.default_rng(seed)
+    return [(int(rng.integers(1, m_max + 1)), int(rng.integers(1, k_max // k_unit + 1)) * k_unit,
+             int(rng.integers(8192 // n_unit, 30000 // n_unit)) * n_unit) for _ in range(count)]
+
+
+@pytest.mark.parametrize("M,K,N", _few_rows_wide(41, 16, 16, 128, 8192, 16))
+@pytest.mark.parametrize("w_dt,group", [("i4", 128), ("i8", 0), ("i8", 64), ("fp4", 32)])
+def test_weight_only_few_rows_wide(gpu, M, K, N, w_dt, group):
+    m = gpu
+    if group and K <= group:
+        group = 0 if w_dt != "fp4" else 32
+    dt = {"i8": m.ACL_INT8, "i4": m.ACL_INT4, "fp4": m.ACL_FLOAT4_E2M1}
+    x_dt = m.ACL_FLOAT16 if (M + N // 16) % 2 else m.ACL_BF16
+    print(f"case sweep weight-only wide M={M} K={K} N={N} w={w_dt} g={group}", flush=True)
+    inp = cases.make_wq_inputs(m, M, K, N, M + K + N, x_dt, dt[w_dt], group, True, w_dt != "fp4", None)
+    want = cases.oracle_wq(m, inp, M, K, N)
+    plain(False)
+    check_close(cases.run_wq_aclnn(m, inp, M, K, N), want, x_dt, "weight-only sweep, wide")
+
+
+@pytest.mark.parametrize("M,K,N", _few_rows_wide(42, 10, 32, 128, 8192, 128))
+def test_fp8_block_scale_few_rows_wide(gpu, M, K, N):
+    m = gpu
+    print(f"case sweep fp8 block wide M={M} K={K} N={N}", flush=True)
+    inp = cases.make_blockscale_inputs(m, M, K, N, M + N + K, True, 1)
+    want = cases.oracle_blockscale(m, inp, M, K, N, True, m.ACL_FLOAT16)
+    _b16_bar(cases.run_blockscale_aclnn(m, inp, M, K, N, True, m.ACL_FLOAT16), want, orc.F16, "fp8 block sweep, wide", K)
+
+
+@pytest.mark.parametrize("M,K,N", _few_rows_wide(43, 10, 32, 128, 8192, 8))
+@pytest.mark.parametrize("mode", ["kc", "pertile", "a8w4", "mxfp8", "mxfp4"])
+def test_quant_modes_few_rows_wide(gpu, M, K, N, mode):
+    m = gpu
+    print(f"case sweep {mode} wide M={M} K={K} N={N}", flush=True)
+    plain(False)
+    if mode == "kc":
+        inp = cases.make_tc_inputs(m, M, K, N, M + N, m.ACL_FLOAT8_E4M3FN, m.ACL_FLOAT, N, m.ACL_FLOAT, True, pertoken="M")
+        want = cases.oracle_tc(m, inp, M, K, N, m.ACL_FLOAT16)
+        _b16_bar(cases.run_tc_aclnn(m, inp, M, K, N, m.ACL_FLOAT16), want, orc.F16, "fp8 K-C sweep, wide", K)
+    elif mode == "pertile":
+        inp = cases.make_pertile_i8_inputs(m, M, K, N, M + N, True)
+        want = cases.oracle_pertile_i8(m, inp, M, K, N, True, m.ACL_BF16)
+        _b16_bar(cases.run_pertile_i8_aclnn(m, inp, M, K, N, True, m.ACL_BF16), want, orc.BF16, "int8 per-tile sweep, wide", K)
+    elif mode == "a8w4":
+        inp = cases.make_a8w4_mx_inputs(m, M, K, N, M + N, True)
+        want = cases.oracle_a8w4_mx(m, inp, M, K, N, True, m.ACL_FLOAT16)
+        _b16_bar(cases.run_a8w4_mx_aclnn(m, inp, M, K, N, True, m.ACL_FLOAT16), want, orc.F16, "fp8 x fp4 MX sweep, wide", K)
+    else:
+        fp4 = mode == "mxfp4"
+        inp = cases.make_mx_inputs(m, M, K, N, K + N + M, True, fp4)
+        want = cases.oracle_mx(m, inp, M, K, N, True, m.ACL_BF16)
+        _b16_bar(cases.run_mx_aclnn(m, inp, M, K, N, True, m.ACL_BF16), want, orc.BF16, "mx sweep, wide", K)
+
+
+# ---- an N-contiguous right operand (re-laid out into the workspace first) ----
+@pytest.mark.parametrize("M,K,N", _shapes(44, 12, 300, 128, 3072, 32, 256, 1024))
+@pytest.mark.parametrize("w_dt,group", [("i4", 128), ("i8", 0)])
+def test_weight_only_n_contiguous_shapes(gpu, M, K, N, w_dt, group):
+    m = gpu
+    dt = {"i8": m.ACL_INT8, "i4": m.ACL_INT4}
+    if group and K <= group:
+        group = 0
+    print(f"case sweep weight-only N-contiguous M={M} K={K} N={N} w={w_dt} g={group}", flush=True)
+    inp = cases.make_wq_inputs(m, M, K, N, M + K + N, m.ACL_BF16, dt[w_dt], group, False, True, m.ACL_BF16)
+    want = cases.oracle_wq(m, inp, M, K, N)
+    plain(False)
+    check_close(cases.run_wq_aclnn(m, inp, M, K, N), want, m.ACL_BF16, "weight-only sweep, N-contiguous")
