@@ -198,3 +198,64 @@ def test_weight_only_n_contiguous_shapes(gpu, M, K, N, w_dt, group):
     want = cases.oracle_wq(m, inp, M, K, N)
     plain(False)
     check_close(cases.run_wq_aclnn(m, inp, M, K, N), want, m.ACL_BF16, "weight-only sweep, N-contiguous")
+
+
+# ---- the quantizers that prepare the operands: bit-exact, any row count and row length ----
+def _mats(seed, count, rows_max, col_unit, cols_max):
+    rng = np.random.default_rng(seed)
+    return [(int(rng.integers(1, rows_max + 1)), int(rng.integers(1, cols_max // col_unit + 1)) * col_unit) for _ in range(count)]
+
+
+@pytest.mark.parametrize("rows,cols", _mats(51, 24, 700, 2, 9000))
+@pytest.mark.parametrize("y_name,symmetric", [("i8", True), ("i8", False), ("i4", True), ("e4m3", True)])
+def test_dynamic_quant_shapes(gpu, rows, cols, y_name, symmetric):
+    from test_dynamic_quant import _run
+    m = gpu
+    y_dt = {"i8": orc.I8, "i4": orc.I4, "e4m3": orc.E4M3}[y_name]
+    x_dt = orc.BF16 if (rows + cols) % 2 else orc.F16
+    print(f"case sweep dynamic quant {rows}x{cols} y={y_name} symmetric={symmetric}", flush=True)
+    rng = np.random.default_rng(rows * 7 + cols)
+    xb = orc.f32_to_b16(rng.normal(0, 2, size=(rows, cols)).astype(np.float32), x_dt)
+    smb = orc.f32_to_b16(rng.uniform(0.5, 2.0, cols).astype(np.float32), x_dt) if cols % 4 == 0 else None
+    want = orc.dynamic_quant(xb, x_dt, y_dt, smooth=smb, symmetric=symmetric)
+    gy, gs, go = _run(m, xb, x_dt, y_dt, smb, symmetric)
+    assert np.array_equal(gs.view(np.uint32), want[1].reshape(-1).view(np.uint32)), "scale differs"
+    if not symmetric:
+        assert np.array_equal(go.view(np.uint32), want[2].reshape(-1).view(np.uint32)), "offset differs"
+    wy = want[0].reshape(-1)
+    z = ((gy | wy) & 0x7f) == 0 if y_dt == orc.E4M3 else np.zeros(gy.shape, bool)   # the sign of a zero result is not pinned
+    assert np.array_equal(gy[~z], wy[~z]), f"{int((gy[~z] != wy[~z]).sum())} outputs differ"
+
+
+@pytest.mark.parametrize("rows,cols", _mats(52, 20, 700, 1, 3000))
+@pytest.mark.parametrize("rb,cb", [(1, 128), (128, 128), (64, 192)])
+def test_dynamic_block_quant_shapes(gpu, rows, cols, rb, cb):
+    from test_dynamic_block_quant import _run
+    m = gpu
+    x_dt = orc.BF16 if (rows + cols) % 2 else orc.F16
+    print(f"case sweep block quant {rows}x{cols} {rb}x{cb}", flush=True)
+    rng = np.random.default_rng(rows * 5 + cols)
+    xf = (rng.normal(0, 1, size=(rows, cols)) * 10.0 ** rng.integers(-3, 3, size=(rows, cols))).astype(np.float32)
+    xb = orc.f32_to_b16(xf, x_dt)
+    want_y, want_s = orc.dynamic_block_quant(xb, x_dt, orc.E4M3, rb, cb, 0.0)
+    gy, gs = _run(m, xb, x_dt, orc.E4M3, rb, cb, 0.0)
+    assert np.array_equal(gs.view(np.uint32), want_s.view(np.uint32)), "scale differs"
+    z = ((gy | want_y) & 0x7f) == 0
+    assert np.array_equal(gy[~z], want_y[~z]), f"{int((gy[~z] != want_y[~z]).sum())} of {want_y.size} outputs differ"
+
+
+@pytest.mark.parametrize("rows,cols", _mats(53, 24, 700, 2, 9000))
+@pytest.mark.parametrize("y_name", ["e2m1", "e4m3"])
+def test_dynamic_mx_quant_shapes(gpu, rows, cols, y_name):
+    from test_dynamic_mx_quant import _run, _codes, _same_but_zero_sign
+    m = gpu
+    y_dt = orc.E2M1 if y_name == "e2m1" else orc.E4M3
+    x_dt = orc.BF16 if (rows + cols) % 2 else orc.F16
+    print(f"case sweep mx quant {rows}x{cols} y={y_name}", flush=True)
+    rng = np.random.default_rng(rows * 3 + cols)
+    xf = (rng.normal(0, 1, size=(rows, cols)) * 2.0 ** rng.integers(-14, 14, size=(rows, 1))).astype(np.float32)
+    xb = orc.f32_to_b16(xf, x_dt)
+    want_y, want_s = orc.dynamic_mx_quant(xb, x_dt, y_dt)
+    gy, gs = _run(m, xb, x_dt, y_dt)
+    assert np.array_equal(gs, want_s), "scale bytes differ"
+    assert _same_but_zero_sign(_codes(gy, y_dt), _codes(want_y.reshape(-1), y_dt), y_dt)
