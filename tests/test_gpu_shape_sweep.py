@@ -259,3 +259,53 @@ def test_dynamic_mx_quant_shapes(gpu, rows, cols, y_name):
     gy, gs = _run(m, xb, x_dt, y_dt)
     assert np.array_equal(gs, want_s), "scale bytes differ"
     assert _same_but_zero_sign(_codes(gy, y_dt), _codes(want_y.reshape(-1), y_dt), y_dt)
+
+
+# ---- K tails: a K that is no whole number of 128-element tiles (padding pre-steps) or of 16 (int8) ----
+def _tails(seed, count, m_max, k_unit, k_max, n_unit, n_hi):
+    rng = np.random.default_rng(seed)
+    out = []
+    while len(out) < count:
+        M, K, N = int(rng.integers(1, m_max + 1)), int(rng.integers(1, k_max // k_unit + 1)) * k_unit, int(rng.integers(64 // n_unit, n_hi // n_unit + 1)) * n_unit
+        if K % 128:
+            out.append((M, K, N))
+    return out
+
+
+@pytest.mark.parametrize("M,K,N", _tails(61, 16, 300, 1, 3000, 1, 600))
+def test_int8_k_tail_shapes_are_bit_identical(gpu, M, K, N):
+    m = gpu
+    print(f"case sweep int8 K tail M={M} K={K} N={N}", flush=True)
+    got, want, _ = cases.run_qmm_int8_case(m, orc, M, K, N, seed=M * 31 + N, out_dtype=m.ACL_FLOAT16, bias_dtype=m.ACL_FLOAT if K % 2 else None,
+                                           transpose_x2=(M + K) % 3 != 0)
+    assert np.array_equal(got, want), f"{int((got != want).sum())} of {got.size} outputs differ"
+
+
+@pytest.mark.parametrize("M,K,N", _tails(62, 12, 300, 8, 3000, 8, 600))
+def test_fp8_block_scale_k_tail_shapes(gpu, M, K, N):
+    m = gpu
+    tB = (M + N) % 4 != 0
+    print(f"case sweep fp8 block K tail M={M} K={K} N={N} tB={tB}", flush=True)
+    inp = cases.make_blockscale_inputs(m, M, K, N, M + N + K, tB, 1)
+    want = cases.oracle_blockscale(m, inp, M, K, N, tB, m.ACL_FLOAT16)
+    _b16_bar(cases.run_blockscale_aclnn(m, inp, M, K, N, tB, m.ACL_FLOAT16), want, orc.F16, "fp8 block K tail sweep", K)
+
+
+@pytest.mark.parametrize("M,K,N", _tails(63, 12, 300, 32, 3000, 2, 600))
+@pytest.mark.parametrize("fp4", [False, True])
+def test_mx_k_tail_shapes(gpu, M, K, N, fp4):
+    m = gpu
+    print(f"case sweep mx K tail M={M} K={K} N={N} fp4={fp4}", flush=True)
+    inp = cases.make_mx_inputs(m, M, K, N, K + N + M, True, fp4)
+    want = cases.oracle_mx(m, inp, M, K, N, True, m.ACL_BF16)
+    plain(False)
+    _b16_bar(cases.run_mx_aclnn(m, inp, M, K, N, True, m.ACL_BF16), want, orc.BF16, "mx K tail sweep", K)
+
+
+@pytest.mark.parametrize("M,K,N", _tails(64, 10, 300, 32, 3000, 2, 600))
+def test_fp8_fp4_mx_k_tail_shapes(gpu, M, K, N):
+    m = gpu
+    print(f"case sweep fp8 x fp4 MX K tail M={M} K={K} N={N}", flush=True)
+    inp = cases.make_a8w4_mx_inputs(m, M, K, N, M + N, True)
+    want = cases.oracle_a8w4_mx(m, inp, M, K, N, True, m.ACL_FLOAT16)
+    _b16_bar(cases.run_a8w4_mx_aclnn(m, inp, M, K, N, True, m.ACL_FLOAT16), want, orc.F16, "fp8 x fp4 MX K tail sweep", K)
