@@ -309,3 +309,52 @@ def test_fp8_fp4_mx_k_tail_shapes(gpu, M, K, N):
     inp = cases.make_a8w4_mx_inputs(m, M, K, N, M + N, True)
     want = cases.oracle_a8w4_mx(m, inp, M, K, N, True, m.ACL_FLOAT16)
     _b16_bar(cases.run_a8w4_mx_aclnn(m, inp, M, K, N, True, m.ACL_FLOAT16), want, orc.F16, "fp8 x fp4 MX K tail sweep", K)
+
+
+# ---- batched operands: every batch has its own x1 and x2; the scales, the bias and the kernel choice are shared ----
+@pytest.mark.parametrize("M,K,N", _shapes(71, 12, 300, 16, 2048, 8, 64, 600) + _shapes(72, 4, 16, 128, 12288, 8, 256, 520))
+def test_int8_batched_shapes_are_bit_identical(gpu, M, K, N):
+    m = gpu
+    batch = 2 + (M + N) % 3
+    print(f"case sweep int8 batched M={M} K={K} N={N} batch={batch}", flush=True)
+    got, want, _ = cases.run_qmm_int8_case(m, orc, M, K, N, seed=M * 31 + N, out_dtype=m.ACL_BF16, bias_dtype=m.ACL_FLOAT if K % 32 else None,
+                                           transpose_x2=(M + K) % 3 != 0, batch=batch)
+    assert np.array_equal(got, want), f"{int((got != want).sum())} of {got.size} outputs differ"
+
+
+@pytest.mark.parametrize("M,K,N", _shapes(73, 12, 300, 128, 2048, 8, 64, 600) + _shapes(74, 4, 32, 128, 12288, 8, 256, 520))
+@pytest.mark.parametrize("fp4", [False, True])
+def test_mx_batched_shapes(gpu, M, K, N, fp4):
+    m = gpu
+    batch = 2 + (M + N) % 3
+    print(f"case sweep mx batched M={M} K={K} N={N} fp4={fp4} batch={batch}", flush=True)
+    inp = cases.make_mx_inputs(m, M, K, N, K + N + M, True, fp4, batch=batch)
+    want = cases.oracle_mx(m, inp, M, K, N, True, m.ACL_BF16)
+    plain(False)
+    _b16_bar(cases.run_mx_aclnn(m, inp, M, K, N, True, m.ACL_BF16), want, orc.BF16, "mx batched sweep", K)
+
+
+# ---- the two group modes whose right operand is always stored [N, K] ----
+@pytest.mark.parametrize("M,K,N", _shapes(75, 20, 300, 32, 3072, 8, 64, 600) + _shapes(76, 6, 64, 128, 12288, 8, 256, 520))
+def test_fp8_fp4_group_scale_shapes(gpu, M, K, N):
+    """fp8 x fp4 with 16-bit scales per 32 elements of K and a packed output scale per column."""
+    m = gpu
+    K = max(K, 64)   # (the mode needs more than one group)
+    s_dt, out = (m.ACL_BF16, m.ACL_BF16) if (M + N) % 2 else (m.ACL_FLOAT16, m.ACL_FLOAT16)
+    print(f"case sweep fp8 x fp4 group scale M={M} K={K} N={N} scale={s_dt}", flush=True)
+    inp = cases.make_tcg_inputs(m, M, K, N, M + N, s_dt)
+    inp["s2"] = inp["s2"] ^ ((np.arange(inp["s2"].size, dtype=np.uint32).reshape(inp["s2"].shape) % 3 == 0).astype(np.uint16) << 15)
+    want = cases.oracle_tcg(m, inp, M, K, N, out)
+    _b16_bar(cases.run_tcg_aclnn(m, inp, M, K, N, out), want, orc.BF16 if out == m.ACL_BF16 else orc.F16, "fp8 x fp4 group scale sweep", K)
+
+
+@pytest.mark.parametrize("M,K,N", _shapes(77, 16, 300, 1024, 8192, 256, 256, 1536))
+def test_int4_group_offset_shapes_are_bit_identical(gpu, M, K, N):
+    """int4 x int4 with scales and offsets per 256 elements of K."""
+    m = gpu
+    out = m.ACL_BF16 if (M + N // 256) % 2 else m.ACL_FLOAT16
+    print(f"case sweep int4 K-G M={M} K={K} N={N} out={out}", flush=True)
+    inp = cases.make_i4_asym_inputs(m, M, K, N, M + N)
+    want = cases.oracle_i4_asym(m, inp, M, K, N, out)
+    got = cases.run_i4_asym_aclnn(m, inp, M, K, N, out)
+    assert np.array_equal(got, want), f"{int((got != want).sum())} of {got.size} outputs differ"
