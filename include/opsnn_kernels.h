@@ -113,6 +113,9 @@ OPSNN_API void opsnnSetForcePlain(int on);
 OPSNN_API void opsnnSetMx8Wide(int n);
 OPSNN_API void opsnnSetWqTileMin(int m);
 OPSNN_API void opsnnSetWqNarrowSlabs(int on);
+/* Another hook of the parity tests: fills the LDS of every compute unit with all-ones bytes (NaN in every floating-point
+ * format used here) on `stream`, so that the next kernel shows if it reads LDS that it has not written.  0 or a HIP status. */
+OPSNN_API int opsnnDebugFillLds(void* stream);
 /* Opt-in cache of re-laid-out right operands.  The matrix-core kernels stream a K-contiguous right operand; x2 / weight
  * stored [K, N] with N contiguous is re-laid out inside every call (into the caller's workspace) unless this cache is on:
  * then opsnnQmmInt8, opsnnQmmBlockScale, opsnnQmmMx (data and scales) and opsnnWqmm keep the K-contiguous copy in device memory of the library's own, keyed

@@ -58,6 +58,29 @@ extern "C" void opsnnSetMx8Wide(int n) { __atomic_store_n(&g_mx8_wide, n, __ATOM
 extern "C" __attribute__((visibility("hidden"))) bool opsnn_force_plain() { return __atomic_load_n(&g_force_plain, __ATOMIC_RELAXED) != 0; }
 extern "C" __attribute__((visibility("hidden"))) int opsnn_mx8_wide() { return __atomic_load_n(&g_mx8_wide, __ATOMIC_RELAXED); }
 
+// A hook of the parity tests: fills the LDS of every compute unit with all-ones bytes (NaN as fp32, fp16, bf16 and e4m3), so
+// that a kernel launched next which reads LDS it has not written gives results the tests can tell from correct ones.  One
+// workgroup fits a compute unit at a time (the whole 160 KiB); each stays a few tens of microseconds, so a launch of four
+// per unit reaches them all.
+__global__ __launch_bounds__(1024) void lds_fill_kernel(int spins)
+{
+    extern __shared__ uint32_t lds_all[];
+    volatile uint32_t* v = lds_all;
+    for (int i = threadIdx.x; i < 163840 / 4; i += 1024) v[i] = 0xffffffffu;
+    for (int i = 0; i < spins; i++) __builtin_amdgcn_s_sleep(16);
+}
+extern "C" int opsnnDebugFillLds(void* stream)
+{
+    static std::atomic<uint64_t> attr_set{0};
+    if (!opsnn::device_flag_test(attr_set)) {
+        hipError_t e = hipFuncSetAttribute((const void*)lds_fill_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 163840);
+        if (e != hipSuccess) return (int)e;
+        opsnn::device_flag_set(attr_set);
+    }
+    hipLaunchKernelGGL(lds_fill_kernel, dim3(1024), dim3(1024), 163840, (hipStream_t)stream, 64);
+    return (int)hipGetLastError();
+}
+
 // fp8 x fp8 arithmetic of the block-scale and row/column-scale modes: 0 (default) exact products and sums on the fp16
 // matrix instruction, 1 the 8-bit matrix instruction (about 1.5x faster, sums aligned in a narrower window).  The
 // initial value comes from OPSNN_FP8_FAST, read once.

@@ -149,6 +149,9 @@ __global__ __launch_bounds__(256, 2) void wqmm_decode_kernel(WqParams p)
                 if (slab + 1 < NSLAB) store_x((slab + 1) & 1);
                 if (slab + 2 < NSLAB) load_x(slab + 2);
             }
+            // chunks past the end of K: their weights count as zero, but the x slab they would read may never have been
+            // written (one slab only), and 0 x NaN from stale LDS is NaN
+            if (c >= NCHUNK) continue;
             if (WK > 1 && (i % WK) != wk) continue;
             const int slab = c / CPS;
             const char* xs = sx + (slab & 1) * XSLAB;

@@ -26,3 +26,13 @@ def gpu(opsnn):
     opsnn.check(opsnn.lib().aclInit(None), "aclInit")
     opsnn.check(opsnn.lib().aclrtSetDevice(0), "aclrtSetDevice")
     return opsnn
+
+
+@pytest.fixture(autouse=True)
+def _stale_lds(request):
+    """Before every GPU test the LDS of all compute units is filled with NaN patterns: a kernel that multiplies LDS it never
+    wrote by zero weights would pass on clean LDS and fail only after certain other kernels."""
+    if "gpu" in request.fixturenames:
+        m = request.getfixturevalue("gpu")
+        m.check(m.lib().opsnnDebugFillLds(None), "opsnnDebugFillLds")
+    yield

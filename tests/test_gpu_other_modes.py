@@ -28,7 +28,9 @@ def check_close(got_bits, want_bits, dt, what, exact=False, fp8_mfma=False, abs_
             raise AssertionError(f"{what}: {len(bad)} of {got_bits.size} differ, first at {bad[0]}")
         return
     got, want = orc.b16_to_f32(got_bits, dt), orc.b16_to_f32(want_bits, dt)
-    assert np.isfinite(got).all(), f"{what}: non-finite output"
+    if not np.isfinite(got).all():
+        bad = np.argwhere(~np.isfinite(got))
+        raise AssertionError(f"{what}: {len(bad)} non-finite outputs of {got.size}, first at {bad[0]}, last at {bad[-1]}")
     mx, mean = orc.rel_err_stats(got, want)
     frac = orc.isclose_fraction(got, want)
     if abs_sum is not None:

@@ -358,3 +358,53 @@ def test_int4_group_offset_shapes_are_bit_identical(gpu, M, K, N):
     want = cases.oracle_i4_asym(m, inp, M, K, N, out)
     got = cases.run_i4_asym_aclnn(m, inp, M, K, N, out)
     assert np.array_equal(got, want), f"{int((got != want).sum())} of {got.size} outputs differ"
+
+
+# ---- FRACTAL_NZ right operands: the NZ entry points give bit for bit what the ND ones give on the same matrix ----
+@pytest.mark.parametrize("M,K,N", _shapes(81, 16, 300, 64, 3072, 8, 64, 1024))
+@pytest.mark.parametrize("w_dt,group,c0e", [("i4", 128, 16), ("i4", 0, 32), ("i8", 0, 32)])
+def test_weight_only_nz_shapes_equal_nd(gpu, M, K, N, w_dt, group, c0e):
+    from test_nz_entry_points import nd_to_nz
+    m = gpu
+    if group and K % group:
+        K += group - K % group
+    tW = w_dt == "i8" and (M + N) % 2 == 1
+    dt = {"i8": m.ACL_INT8, "i4": m.ACL_INT4}
+    x_dt = m.ACL_FLOAT16 if (M + N) % 4 < 2 else m.ACL_BF16
+    print(f"case sweep weight-only NZ M={M} K={K} N={N} w={w_dt} g={group} tW={tW} c0={c0e}", flush=True)
+    inp = cases.make_wq_inputs(m, M, K, N, M + N, x_dt, dt[w_dt], group, tW, True, None)
+    plain(False)
+    want = cases.run_wq_aclnn(m, inp, M, K, N)
+    check_close(want, cases.oracle_wq(m, inp, M, K, N), x_dt, "weight-only NZ sweep, ND call")
+    nz = nd_to_nz(inp["w"].reshape(N if tW else K, -1).view(np.uint8), c0e if w_dt == "i8" else c0e // 2)
+    got = cases.run_wq_aclnn(m, dict(inp, w=nz), M, K, N, nz_storage=(nz.shape[0], nz.shape[1], 16, c0e))
+    assert np.array_equal(got, want), f"{int((got != want).sum())} of {got.size} outputs differ from the ND entry point"
+
+
+@pytest.mark.parametrize("M,K,N", _shapes(82, 16, 300, 4, 3072, 4, 64, 1024))
+def test_int8_nz_shapes_equal_nd(gpu, M, K, N):
+    from test_nz_entry_points import nd_to_nz
+    m = gpu
+    tB = (M + K) % 2 == 1
+    print(f"case sweep int8 NZ M={M} K={K} N={N} tB={tB}", flush=True)
+    inp = cases.make_qmm_int8_inputs(m, M, K, N, M + K, m.ACL_BF16, tB)
+    want, _ = cases.oracle_qmm_int8(m, inp, M, K, N, tB, m.ACL_BF16)
+    nz = nd_to_nz(inp["x2"][0].view(np.uint8), 32)
+    got = cases.run_qmm_int8_aclnn(m, dict(inp, x2=nz[None]), M, K, N, tB, m.ACL_BF16, nz_storage=(nz.shape[0], nz.shape[1], 16, 32))
+    assert np.array_equal(got, want), f"{int((got != want).sum())} of {got.size} outputs differ"
+
+
+# ---- a K of one x slab on the first-generation weight-only kernel (N no multiple of 32 keeps the call there): the chunks
+# past the end of K must not be multiplied at all -- their x slab in LDS was never written (found as NaN results that
+# depended on the kernel that had run before; conftest fills the LDS with NaN patterns before every GPU test) ----
+@pytest.mark.parametrize("M,K,N,w_dt", [(244, 192, 144, "i4"), (60, 64, 48, "i4"), (16, 512, 40, "i4"), (30, 256, 72, "i4"), (9, 96, 24, "i8"),
+                                        (50, 64, 80, "i8"), (32, 208, 56, "i8"), (128, 128, 16, "i8")])
+def test_weight_only_one_slab_of_k(gpu, M, K, N, w_dt):
+    m = gpu
+    dt = {"i8": m.ACL_INT8, "i4": m.ACL_INT4}
+    for x_dt in (m.ACL_FLOAT16, m.ACL_BF16):
+        print(f"case weight-only one slab M={M} K={K} N={N} w={w_dt} x={x_dt}", flush=True)
+        inp = cases.make_wq_inputs(m, M, K, N, M + N, x_dt, dt[w_dt], 0, True, True, None)
+        plain(False)
+        m.check(m.lib().opsnnDebugFillLds(None), "opsnnDebugFillLds")
+        check_close(cases.run_wq_aclnn(m, inp, M, K, N), cases.oracle_wq(m, inp, M, K, N), x_dt, "weight-only, one slab of K")
