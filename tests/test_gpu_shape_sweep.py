@@ -408,3 +408,49 @@ def test_weight_only_one_slab_of_k(gpu, M, K, N, w_dt):
         plain(False)
         m.check(m.lib().opsnnDebugFillLds(None), "opsnnDebugFillLds")
         check_close(cases.run_wq_aclnn(m, inp, M, K, N), cases.oracle_wq(m, inp, M, K, N), x_dt, "weight-only, one slab of K")
+
+
+# ---- int8 epilogues: output, bias and x2-scale forms picked per shape ----
+_EPILOGUES = [("bf16", "bf16", "f32", None), ("bf16", None, "f32", 1), ("f16", "f32", "f32", None), ("bf16", "i32", "bf16", None),
+              ("f16", "f16", "f32", 1), ("bf16", "bf16", "bf16", None)]
+
+
+@pytest.mark.parametrize("M,K,N", _shapes(91, 36, 400, 8, 4096, 1, 32, 1100) + _shapes(92, 6, 32, 64, 16384, 4, 128, 600))
+def test_int8_epilogue_forms_are_bit_identical(gpu, M, K, N):
+    m = gpu
+    dt = {"bf16": m.ACL_BF16, "f16": m.ACL_FLOAT16, "f32": m.ACL_FLOAT, "i32": m.ACL_INT32, None: None}
+    out_dt, bias_dt, s2_dt, s2_len = _EPILOGUES[(M + K + N) % len(_EPILOGUES)]
+    tB = (M + N) % 3 != 0
+    print(f"case sweep int8 epilogue M={M} K={K} N={N} tB={tB} out={out_dt} bias={bias_dt} s2={s2_dt} x{s2_len}", flush=True)
+    got, want, _ = cases.run_qmm_int8_case(m, orc, M, K, N, seed=M * 31 + N, out_dtype=dt[out_dt], bias_dtype=dt[bias_dt], transpose_x2=tB,
+                                           x2s_len=s2_len, x2s_dtype=dt[s2_dt])
+    assert np.array_equal(got, want), f"{int((got != want).sum())} of {got.size} outputs differ"
+
+
+# ---- weight-only forms: bias (x's dtype or fp32), no offset, one scale for the whole weight, the V3 entry point, e4m3 weights ----
+_WQ_FORMS = [dict(w="i4", group=128, off=True, bias="x", pt=False, v3=False), dict(w="i8", group=0, off=False, bias="f32", pt=False, v3=False),
+             dict(w="i4", group=0, off=False, bias=None, pt=True, v3=False), dict(w="i8", group=0, off=True, bias="x", pt=True, v3=True),
+             dict(w="i8", group=128, off=True, bias="f32", pt=False, v3=True), dict(w="i4", group=64, off=False, bias="x", pt=False, v3=False),
+             dict(w="e4m3", group=0, off=False, bias=None, pt=False, v3=False)]
+
+
+@pytest.mark.parametrize("M,K,N", _shapes(93, 44, 400, 128, 6144, 32, 256, 1024) + _shapes(94, 12, 64, 128, 16384, 8, 64, 520))
+def test_weight_only_forms(gpu, M, K, N):
+    m = gpu
+    f = _WQ_FORMS[(M + K // 128 + N // 8) % len(_WQ_FORMS)]
+    if f["w"] == "i4" and K % 256:
+        K += 128
+    x_dt = m.ACL_FLOAT16 if (M + N) % 2 else m.ACL_BF16
+    if f["w"] == "e4m3":
+        x_dt = m.ACL_BF16 if K > 4096 else x_dt
+    group = f["group"] if K > f["group"] else 0
+    w_dt = {"i8": m.ACL_INT8, "i4": m.ACL_INT4, "e4m3": m.ACL_FLOAT8_E4M3FN}[f["w"]]
+    bias_dt = {"x": x_dt, "f32": m.ACL_FLOAT, None: None}[f["bias"]]
+    if bias_dt == m.ACL_FLOAT and x_dt != m.ACL_BF16:
+        bias_dt = x_dt   # (an fp32 bias goes with bf16 x)
+    tW = (M + K // 128) % 3 != 0
+    print(f"case sweep weight-only forms M={M} K={K} N={N} tW={tW} x={x_dt} {f}", flush=True)
+    inp = cases.make_wq_inputs(m, M, K, N, M + K + N, x_dt, w_dt, group, tW, f["off"], bias_dt, per_tensor=f["pt"] and group == 0)
+    want = cases.oracle_wq(m, inp, M, K, N)
+    plain(False)
+    check_close(cases.run_wq_aclnn(m, inp, M, K, N, v3=f["v3"]), want, x_dt, "weight-only forms sweep")
