@@ -454,3 +454,41 @@ def test_weight_only_forms(gpu, M, K, N):
     want = cases.oracle_wq(m, inp, M, K, N)
     plain(False)
     check_close(cases.run_wq_aclnn(m, inp, M, K, N, v3=f["v3"]), want, x_dt, "weight-only forms sweep")
+
+
+# ---- int8 without a per-token scale: packed, fp32 and bf16 scales, int8 / int32 / 16-bit outputs, offsets ----
+_TC_FORMS = [("u64", "N", "i32", "f16", 0), ("u64", 1, "i32", "i8", 1), ("u64", "N", "i32", "i8", "N"), ("u64", "N", None, "i8", 0),
+             ("f32", 1, "i32", "bf16", 0), ("f32", 1, "f32", "bf16", 0), ("bf16", 1, None, "bf16", 0), ("f32", "N", "i32", "i32", 0),
+             ("bf16", "N", "bf16", "bf16", 0)]
+
+
+@pytest.mark.parametrize("M,K,N", _shapes(95, 36, 400, 8, 4096, 1, 32, 1100) + _shapes(96, 9, 32, 64, 16384, 4, 128, 600))
+def test_int8_static_forms_are_bit_identical(gpu, M, K, N):
+    m = gpu
+    dt = {"u64": m.ACL_UINT64, "f32": m.ACL_FLOAT, "bf16": m.ACL_BF16, "f16": m.ACL_FLOAT16, "i32": m.ACL_INT32, "i8": m.ACL_INT8, None: None}
+    s_dt, s_len, bias_dt, out_dt, off_len = _TC_FORMS[(M + K + N) % len(_TC_FORMS)]
+    tB = (M + N) % 3 != 0
+    print(f"case sweep int8 static M={M} K={K} N={N} tB={tB} scale={s_dt}/{s_len} bias={bias_dt} out={out_dt} off={off_len}", flush=True)
+    inp = cases.make_tc_inputs(m, M, K, N, M + N, m.ACL_INT8, dt[s_dt], 1 if s_len == 1 else N, dt[bias_dt], tB, pertoken=False,
+                               offset_len=N if off_len == "N" else off_len)
+    want = cases.oracle_tc(m, inp, M, K, N, dt[out_dt])
+    got = cases.run_tc_aclnn(m, inp, M, K, N, dt[out_dt])
+    assert np.array_equal(got, want), f"{int((got != want).sum())} of {got.size} outputs differ"
+
+
+# ---- fp8 with per-row, one-element or no x1 scale; e4m3 and e5m2; fp32 and packed x2 scales; K tails and N-contiguous x2 ----
+_F8_FORMS = [("e4m3", "f32", "N", "f32", "M"), ("e5m2", "f32", "N", "f32", True), ("e4m3", "u64", "N", None, False), ("e4m3", "u64", 1, "f32", False),
+             ("e4m3", "f32", 1, None, "M"), ("e4m3", "f32", 1, None, True), ("e5m2", "f32", "N", None, "M")]
+
+
+@pytest.mark.parametrize("M,K,N", _shapes(97, 35, 400, 8, 4096, 8, 64, 1100) + _shapes(98, 7, 32, 128, 16384, 8, 128, 600))
+def test_fp8_scale_forms(gpu, M, K, N):
+    m = gpu
+    dt = {"e4m3": m.ACL_FLOAT8_E4M3FN, "e5m2": m.ACL_FLOAT8_E5M2, "u64": m.ACL_UINT64, "f32": m.ACL_FLOAT, None: None}
+    in_dt, s_dt, s_len, bias_dt, pt = _F8_FORMS[(M + K // 8 + N // 8) % len(_F8_FORMS)]
+    out = m.ACL_BF16 if (M + N) % 2 else m.ACL_FLOAT16
+    tB = (M + N) % 3 != 0
+    print(f"case sweep fp8 forms M={M} K={K} N={N} tB={tB} in={in_dt} scale={s_dt}/{s_len} bias={bias_dt} pt={pt}", flush=True)
+    inp = cases.make_tc_inputs(m, M, K, N, M + N, dt[in_dt], dt[s_dt], 1 if s_len == 1 else N, dt[bias_dt], tB, pertoken=pt, e5m2=in_dt == "e5m2")
+    want = cases.oracle_tc(m, inp, M, K, N, out)
+    _b16_bar(cases.run_tc_aclnn(m, inp, M, K, N, out), want, orc.BF16 if out == m.ACL_BF16 else orc.F16, "fp8 forms sweep", K)
