@@ -31,8 +31,13 @@ def _shapes(seed, count, m_max, k_unit, k_max, n_unit, n_lo, n_hi):
 def _b16_bar(got, want, code, what, K=0):
     g, w = orc.b16_to_f32(got, code), orc.b16_to_f32(want, code)
     assert np.isfinite(g).all(), what
-    mx, mean = orc.rel_err_stats(g, w)
-    assert mx <= 2.0 ** -7 and mean <= 2.0 ** -10, f"{what}: max rel {mx:.3e} mean rel {mean:.3e}"
+    # (the relative error's denominator has a floor of a hundredth of the mean |want|; for fp16 outputs at least 128 steps of the
+    # subnormal range, 2^-17, so that one such step on a small result is not counted as more than 2^-7)
+    floor = max(float(np.mean(np.abs(w))) * 1e-2, 2.0 ** -17 if code == orc.F16 else 1e-30)
+    mx, mean = orc.rel_err_stats(g, w, floor)
+    if not (mx <= 2.0 ** -7 and mean <= 2.0 ** -10):
+        i = np.unravel_index(np.argmax(np.abs(g - w) / np.maximum(np.abs(w), 1e-30)), g.shape)
+        raise AssertionError(f"{what}: max rel {mx:.3e} mean rel {mean:.3e}; worst at {i}: got {g[i]!r} want {w[i]!r}, median |want| {np.median(np.abs(w)):.3e}")
     # 99.9 % within rtol = atol = 1e-3.  Two allowances that the single-shape tests do not need: with a few hundred outputs one
     # bf16 result an ulp off is already more than a thousandth of them; and beyond K = 8192 fp32 sums in another order than the
     # oracle's flip one bf16 result in a thousand by an ulp (four times the 1e-3), so bf16 outputs get 3e-3 there.
@@ -492,3 +497,25 @@ def test_fp8_scale_forms(gpu, M, K, N):
     inp = cases.make_tc_inputs(m, M, K, N, M + N, dt[in_dt], dt[s_dt], 1 if s_len == 1 else N, dt[bias_dt], tB, pertoken=pt, e5m2=in_dt == "e5m2")
     want = cases.oracle_tc(m, inp, M, K, N, out)
     _b16_bar(cases.run_tc_aclnn(m, inp, M, K, N, out), want, orc.BF16 if out == m.ACL_BF16 else orc.F16, "fp8 forms sweep", K)
+
+
+# ---- fp8 block scales with N-contiguous and batched operands, int8 per-tile with N-contiguous x2 ----
+@pytest.mark.parametrize("M,K,N", _shapes(99, 20, 300, 128, 4096, 128, 128, 1024) + _shapes(100, 4, 32, 128, 12288, 128, 256, 640))
+def test_fp8_block_scale_n_contiguous_and_batched(gpu, M, K, N):
+    m = gpu
+    batch, tB = 1 + (M + N // 128) % 3, (M + K // 128) % 2 == 0
+    gsM = 128 if (M + K) % 3 == 0 else 1
+    out = m.ACL_BF16 if (M + N // 128) % 2 else m.ACL_FLOAT16
+    print(f"case sweep fp8 block M={M} K={K} N={N} tB={tB} batch={batch} gsM={gsM}", flush=True)
+    inp = cases.make_blockscale_inputs(m, M, K, N, M + N + K, tB, gsM, batch=batch)
+    want = cases.oracle_blockscale(m, inp, M, K, N, tB, out)
+    _b16_bar(cases.run_blockscale_aclnn(m, inp, M, K, N, tB, out), want, orc.BF16 if out == m.ACL_BF16 else orc.F16, "fp8 block sweep, layouts", K)
+
+
+@pytest.mark.parametrize("M,K,N", _shapes(101, 16, 300, 128, 4096, 8, 128, 1024))
+def test_int8_per_tile_n_contiguous(gpu, M, K, N):
+    m = gpu
+    print(f"case sweep int8 per-tile N-contiguous M={M} K={K} N={N}", flush=True)
+    inp = cases.make_pertile_i8_inputs(m, M, K, N, M + N, False)
+    want = cases.oracle_pertile_i8(m, inp, M, K, N, False, m.ACL_BF16)
+    _b16_bar(cases.run_pertile_i8_aclnn(m, inp, M, K, N, False, m.ACL_BF16), want, orc.BF16, "int8 per-tile N-contiguous sweep", K)
