@@ -363,11 +363,26 @@ def quant_matmul_v5_get_workspace(x1, x2, x1_scale, x2_scale, out, *, y_scale=No
     return rc, ws.value, ex.value
 
 
+# A byte (0 .. 255) to fill every workspace with that the two-phase helpers below allocate, or None.  The parity tests set 0xFF
+# (NaN in every floating-point format used here): a kernel that reads workspace bytes no kernel of the call has written then
+# shows in the results.
+FILL_NEW_WORKSPACE = None
+
+
+def _new_workspace(nbytes):
+    if not nbytes:
+        return None
+    buf = DeviceBuffer(nbytes)
+    if FILL_NEW_WORKSPACE is not None:
+        buf.fill(FILL_NEW_WORKSPACE)
+    return buf
+
+
 def quant_matmul_v5(x1, x2, x1_scale, x2_scale, out, stream=None, **kw):
     """Both phases; allocates the workspace the first phase asks for.  Asynchronous on `stream`."""
     rc, ws, ex = quant_matmul_v5_get_workspace(x1, x2, x1_scale, x2_scale, out, **kw)
     check(rc, "aclnnQuantMatmulV5GetWorkspaceSize")
-    wbuf = DeviceBuffer(ws) if ws else None
+    wbuf = _new_workspace(ws)
     run = lib().aclnnQuantMatmulWeightNz if kw.get("weight_nz") else lib().aclnnQuantMatmulV5
     check(run(wbuf.ptr if wbuf else None, ws, ex, stream.ptr if stream else None), "aclnnQuantMatmulV5")
     return wbuf  # keep alive until the stream has been synchronised
@@ -379,7 +394,7 @@ def prepack_matmul_weight(weight, packed, scale=None, scale_packed=None, stream=
     rc = lib().aclnnPrepackMatmulWeightGetWorkspaceSize(_h(weight), _h(scale), _h(packed), _h(scale_packed), C.byref(ws), C.byref(ex))
     if rc != 0:
         return rc, None
-    wbuf = DeviceBuffer(ws.value) if ws.value else None
+    wbuf = _new_workspace(ws.value)
     check(lib().aclnnPrepackMatmulWeight(wbuf.ptr if wbuf else None, ws.value, ex, stream.ptr if stream else None), "aclnnPrepackMatmulWeight")
     return 0, wbuf
 
@@ -406,7 +421,7 @@ def weight_quant_batch_matmul(x, weight, scale, y, stream=None, **kw):
     v3 = kw.get("inner_precise") is not None
     rc, ws, ex = weight_quant_batch_matmul_get_workspace(x, weight, scale, y, **kw)
     check(rc, "aclnnWeightQuantBatchMatmulGetWorkspaceSize")
-    wbuf = DeviceBuffer(ws) if ws else None
+    wbuf = _new_workspace(ws)
     run = lib().aclnnWeightQuantBatchMatmulV3 if v3 else lib().aclnnWeightQuantBatchMatmulV2
     if kw.get("weight_nz"):
         run = lib().aclnnWeightQuantBatchMatmulNz

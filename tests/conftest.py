@@ -25,6 +25,9 @@ def gpu(opsnn):
         pytest.fail("this test is marked gpu but no HIP device is visible")
     opsnn.check(opsnn.lib().aclInit(None), "aclInit")
     opsnn.check(opsnn.lib().aclrtSetDevice(0), "aclrtSetDevice")
+    # every workspace the two-phase helpers allocate starts as NaN patterns: reading a part that the call has not written shows
+    import opsnn.binding
+    opsnn.binding.FILL_NEW_WORKSPACE = 0xFF
     return opsnn
 
 
