@@ -39,6 +39,36 @@ def as_f32(arr, dt, m):
     return np.asarray(arr, np.float32)
 
 
+GUARD = 4096
+
+
+def guarded_out(m, nbytes, fill=0xFF):
+    """An output allocation with GUARD bytes in front of and behind the nbytes the call may write, all filled with `fill`;
+    to_host checks that both guards still hold the fill (a store outside the output would otherwise land in whatever the
+    allocator has placed next to it, unseen)."""
+    class _Guarded(m.DeviceBuffer):
+        def __init__(self):
+            self.whole = m.DeviceBuffer(nbytes + 2 * GUARD)
+            self.whole.fill(fill)
+            self.nbytes, self.ptr = int(nbytes), self.whole.ptr + GUARD
+
+        def fill(self, byte):
+            pass   # (already filled; the guards must keep their byte)
+
+        def free(self):
+            self.ptr = None
+
+        def to_host(self, dtype, shape):
+            raw = self.whole.to_host(np.uint8, (self.nbytes + 2 * GUARD,))
+            front, back = raw[:GUARD], raw[GUARD + self.nbytes:]
+            assert (front == fill).all(), f"{int((front != fill).sum())} bytes written in front of the output"
+            assert (back == fill).all(), f"{int((back != fill).sum())} bytes written behind the output, first at +{int(np.argmax(back != fill))}"
+            out = np.empty(shape, dtype=dtype)
+            assert out.nbytes <= self.nbytes
+            return raw[GUARD:GUARD + out.nbytes].view(out.dtype).reshape(shape).copy()
+    return _Guarded()
+
+
 def make_qmm_int8_inputs(m, M, K, N, seed, bias_dtype, transpose_x2, x2s_dtype=None, x2s_len=None, batch=1, x1s=True):
     rng = np.random.default_rng(seed)
     x1 = gen_int8(rng, (batch, M, K))
@@ -76,8 +106,7 @@ def run_qmm_int8_aclnn(m, inp, M, K, N, transpose_x2, out_dtype, x2_as_view=Fals
     bshape = (batch,) if batch > 1 else ()
     d = {k: m.DeviceBuffer(host=v) for k, v in inp.items() if isinstance(v, np.ndarray)}
     out_np = orc.out_array((batch, M, N), out_dtype)
-    d_out = m.DeviceBuffer(out_np.nbytes)
-    d_out.fill(0xFF)
+    d_out = guarded_out(m, out_np.nbytes)
     x1 = m.Tensor(bshape + (M, K), m.ACL_INT8, d["x1"])
     if transpose_x2 and x2_as_view:
         assert batch == 1
@@ -161,8 +190,7 @@ def run_blockscale_aclnn(m, inp, M, K, N, tB, out_dtype, group_size=None):
     bshape = (batch,) if batch > 1 else ()
     d = {k: m.DeviceBuffer(host=v) for k, v in inp.items() if isinstance(v, np.ndarray)}
     out_np = orc.out_array((batch, M, N), out_dtype)
-    d_out = m.DeviceBuffer(out_np.nbytes)
-    d_out.fill(0xFF)
+    d_out = guarded_out(m, out_np.nbytes)
     x1 = m.Tensor(bshape + (M, K), m.ACL_FLOAT8_E4M3FN, d["x1"])
     x2 = m.Tensor(bshape + ((N, K) if tB else (K, N)), m.ACL_FLOAT8_E4M3FN, d["x2"])
     s1 = m.Tensor(bshape + inp["s1"].shape[1:], m.ACL_FLOAT, d["s1"])
@@ -214,8 +242,7 @@ def oracle_tc(m, inp, M, K, N, out_dt):
 def run_tc_aclnn(m, inp, M, K, N, out_dt):
     d = {k: m.DeviceBuffer(host=v) for k, v in inp.items() if isinstance(v, np.ndarray)}
     out_np = orc.out_array((M, N), out_dt)
-    d_out = m.DeviceBuffer(out_np.nbytes)
-    d_out.fill(0x7F)
+    d_out = guarded_out(m, out_np.nbytes, 0x7F)
     tB = inp["tB"]
     x1 = m.Tensor((M, K), inp["in_dt"], d["x1"])
     x2 = m.Tensor((N, K) if tB else (K, N), inp["x2_dt"], d["x2"])
@@ -265,8 +292,7 @@ def run_mx_aclnn(m, inp, M, K, N, tB, out_dtype, bias=None, nz_storage=None):
     adt = m.ACL_FLOAT4_E2M1 if inp["fp4"] else m.ACL_FLOAT8_E4M3FN
     d = {k: m.DeviceBuffer(host=v) for k, v in inp.items() if isinstance(v, np.ndarray)}
     out_np = orc.out_array((batch, M, N), out_dtype)
-    d_out = m.DeviceBuffer(out_np.nbytes)
-    d_out.fill(0xFF)
+    d_out = guarded_out(m, out_np.nbytes)
     x1 = m.Tensor(bshape + (M, K), adt, d["x1"])
     x2 = m.Tensor(bshape + ((N, K) if tB else (K, N)), adt, d["x2"], fmt=29 if nz_storage else m.ACL_FORMAT_ND, storage_shape=nz_storage)
     s1 = m.Tensor(bshape + inp["s1"].shape[1:], m.ACL_FLOAT8_E8M0, d["s1"])
@@ -323,8 +349,7 @@ def oracle_wq(m, inp, M, K, N, rows=None):
 
 def run_wq_aclnn(m, inp, M, K, N, v3=False, scale_2d=None, nz_storage=None):
     d = {k: m.DeviceBuffer(host=v) for k, v in inp.items() if isinstance(v, np.ndarray)}
-    d_y = m.DeviceBuffer(M * N * 2)
-    d_y.fill(0xFF)
+    d_y = guarded_out(m, M * N * 2)
     tW, group = inp["tW"], inp["group"]
     G = -(-K // group) if group > 0 else 1
     x = m.Tensor((M, K), inp["x_dt"], d["x"])
@@ -376,7 +401,7 @@ def oracle_a8w4_mx(m, inp, M, K, N, tB, out_dt, bias_dt=None):
 def run_a8w4_mx_aclnn(m, inp, M, K, N, tB, out_dt, bias_dt=None):
     d = {k: m.DeviceBuffer(host=v) for k, v in inp.items()}
     out_np = orc.out_array((M, N), out_dt)
-    d_out = m.DeviceBuffer(out_np.nbytes); d_out.fill(0xFF)
+    d_out = guarded_out(m, out_np.nbytes)
     x1 = m.Tensor((M, K), m.ACL_FLOAT8_E4M3FN, d["x1"])
     x2 = m.Tensor((N, K) if tB else (K, N), m.ACL_FLOAT4_E2M1, d["x2"])
     s1 = m.Tensor(inp["s1"].shape, m.ACL_FLOAT8_E8M0, d["s1"])
@@ -408,7 +433,7 @@ def oracle_tcg(m, inp, M, K, N, out_dt):
 def run_tcg_aclnn(m, inp, M, K, N, out_dt, ys_dt=None):
     d = {k: m.DeviceBuffer(host=v) for k, v in inp.items() if isinstance(v, np.ndarray)}
     out_np = orc.out_array((M, N), out_dt)
-    d_out = m.DeviceBuffer(out_np.nbytes); d_out.fill(0xFF)
+    d_out = guarded_out(m, out_np.nbytes)
     x1 = m.Tensor((M, K), m.ACL_FLOAT8_E4M3FN, d["x1"])
     x2 = m.Tensor((N, K), m.ACL_FLOAT4_E2M1, d["x2"])
     s2 = m.Tensor((N, K // 32), inp["s_dt"], d["s2"])
@@ -437,7 +462,7 @@ def oracle_pertile_i8(m, inp, M, K, N, tB, out_dt):
 def run_pertile_i8_aclnn(m, inp, M, K, N, tB, out_dt):
     d = {k: m.DeviceBuffer(host=v) for k, v in inp.items()}
     out_np = orc.out_array((M, N), out_dt)
-    d_out = m.DeviceBuffer(out_np.nbytes); d_out.fill(0xFF)
+    d_out = guarded_out(m, out_np.nbytes)
     x1 = m.Tensor((M, K), m.ACL_INT8, d["x1"])
     x2 = m.Tensor((N, K) if tB else (K, N), m.ACL_INT8, d["x2"])
     s1 = m.Tensor(inp["s1"].shape, m.ACL_FLOAT, d["s1"])
@@ -469,7 +494,7 @@ def oracle_i4_asym(m, inp, M, K, N, out_dt):
 def run_i4_asym_aclnn(m, inp, M, K, N, out_dt):
     d = {k: m.DeviceBuffer(host=v) for k, v in inp.items()}
     out_np = orc.out_array((M, N), out_dt)
-    d_out = m.DeviceBuffer(out_np.nbytes); d_out.fill(0xFF)
+    d_out = guarded_out(m, out_np.nbytes)
     x1 = m.Tensor((M, K), m.ACL_INT4, d["x1"])
     x2 = m.Tensor((N, K), m.ACL_INT4, d["x2"])
     s1 = m.Tensor(inp["s1"].shape, m.ACL_FLOAT, d["s1"])
