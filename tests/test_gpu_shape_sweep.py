@@ -519,3 +519,23 @@ def test_int8_per_tile_n_contiguous(gpu, M, K, N):
     inp = cases.make_pertile_i8_inputs(m, M, K, N, M + N, False)
     want = cases.oracle_pertile_i8(m, inp, M, K, N, False, m.ACL_BF16)
     _b16_bar(cases.run_pertile_i8_aclnn(m, inp, M, K, N, False, m.ACL_BF16), want, orc.BF16, "int8 per-tile N-contiguous sweep", K)
+
+
+# ---- weight-only with any N and a short or ragged K: the first-generation kernel and the plain one behind the streamlined ones ----
+@pytest.mark.parametrize("M,K,N", _shapes(102, 40, 300, 8, 2048, 1, 8, 700))
+@pytest.mark.parametrize("w_dt", ["i4", "i8"])
+def test_weight_only_ragged_shapes(gpu, M, K, N, w_dt):
+    m = gpu
+    dt = {"i8": m.ACL_INT8, "i4": m.ACL_INT4}
+    x_dt = m.ACL_FLOAT16 if (M + N) % 2 else m.ACL_BF16
+    group = (0, 32, 64, 128)[(M + K // 8) % 4]
+    if group and (K % group or K <= group):
+        group = 0
+    tW = (M + N + K // 8) % 3 != 0
+    if w_dt == "i4" and not tW and N % 2:
+        N += 1   # (packed nibbles: whole bytes per stored row)
+    print(f"case sweep weight-only ragged M={M} K={K} N={N} w={w_dt} g={group} tW={tW}", flush=True)
+    inp = cases.make_wq_inputs(m, M, K, N, M + K + N, x_dt, dt[w_dt], group, tW, (M + N) % 4 != 0, x_dt if N % 3 == 0 else None)
+    want = cases.oracle_wq(m, inp, M, K, N)
+    plain(False)
+    check_close(cases.run_wq_aclnn(m, inp, M, K, N), want, x_dt, "weight-only ragged sweep")
