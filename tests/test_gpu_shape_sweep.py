@@ -539,3 +539,31 @@ def test_weight_only_ragged_shapes(gpu, M, K, N, w_dt):
     want = cases.oracle_wq(m, inp, M, K, N)
     plain(False)
     check_close(cases.run_wq_aclnn(m, inp, M, K, N), want, x_dt, "weight-only ragged sweep")
+
+
+# ---- the re-layout behind N-contiguous right operands (aclnnPrepackMatmulWeight), bytes and nibbles, any K and N ----
+@pytest.mark.parametrize("K,N", _mats(110, 30, 3000, 1, 3000) + [(1, 1), (2, 4097), (4097, 2), (64, 64), (33, 31)])
+@pytest.mark.parametrize("bits", [8, 4])
+def test_prepack_shapes(gpu, K, N, bits):
+    m = gpu
+    if bits == 4:
+        K, N = K + K % 2, N + N % 2   # whole bytes per row on both sides
+    B = 1 + (K + N) % 2
+    print(f"case sweep prepack K={K} N={N} bits={bits} batch={B}", flush=True)
+    rng = np.random.default_rng(K * 7 + N)
+    if bits == 8:
+        src = rng.integers(-128, 128, size=(B, K, N), dtype=np.int8)
+        want = np.ascontiguousarray(src.transpose(0, 2, 1)).view(np.uint8)
+        adt = m.ACL_INT8
+    else:
+        codes = rng.integers(0, 16, size=(B, K, N), dtype=np.uint8)
+        src = orc.pack_nibbles(codes)
+        want = orc.pack_nibbles(np.ascontiguousarray(codes.transpose(0, 2, 1)))
+        adt = m.ACL_INT4
+    d_src = m.DeviceBuffer(host=src)
+    d_dst = cases.guarded_out(m, want.nbytes, 0xEE)
+    rc, ws = m.prepack_matmul_weight(m.Tensor((B, K, N), adt, d_src), m.Tensor((B, N, K), adt, d_dst))
+    assert rc == 0, m.err_msg()
+    m.check(m.lib().aclrtSynchronizeDevice(), "sync")
+    got = d_dst.to_host(np.uint8, want.shape)
+    assert np.array_equal(got, want), f"{int((got != want).sum())} of {want.size} bytes differ"
