@@ -567,3 +567,68 @@ def test_prepack_shapes(gpu, K, N, bits):
     m.check(m.lib().aclrtSynchronizeDevice(), "sync")
     got = d_dst.to_host(np.uint8, want.shape)
     assert np.array_equal(got, want), f"{int((got != want).sum())} of {want.size} bytes differ"
+
+
+# ---- operands at element offsets inside their storage: pointers that are not 16-byte (or even 4-byte) aligned ----
+def _at_offset(m, shape, dtype, host, off, elem_bytes, strides=None, storage_cols=None):
+    """A tensor whose data starts `off` elements into its storage (junk in front); returns (tensor, buffer).  storage_cols: the
+    storage is declared as rows of that many elements (for operands whose storage must have two dimensions)."""
+    raw = np.ascontiguousarray(host).view(np.uint8).reshape(-1)
+    n = off + raw.size // elem_bytes
+    if storage_cols:
+        rows = -(-n // storage_cols)
+        sshape, tail = (rows, storage_cols), (rows * storage_cols - n) * elem_bytes
+    else:
+        sshape, tail = (n,), 0
+    buf = m.DeviceBuffer(host=np.concatenate([np.full(off * elem_bytes, 0x5A, np.uint8), raw, np.full(tail, 0x5A, np.uint8)]))
+    return m.Tensor(shape, dtype, buf, strides=strides, offset=off, storage_shape=sshape), buf
+
+
+@pytest.mark.parametrize("M,K,N", _shapes(120, 24, 400, 16, 4096, 8, 64, 1100))
+def test_int8_operands_at_odd_offsets_are_bit_identical(gpu, M, K, N):
+    m = gpu
+    tB = (M + N) % 3 != 0
+    o = [(1, 3, 1, 1, 1, 1), (4, 8, 2, 0, 1, 2), (16, 1, 0, 1, 0, 4), (0, 16, 1, 1, 1, 0), (5, 0, 0, 0, 0, 1)][(M + K + N) % 5]
+    print(f"case sweep int8 offsets M={M} K={K} N={N} tB={tB} offsets={o}", flush=True)
+    inp = cases.make_qmm_int8_inputs(m, M, K, N, M * 31 + N, m.ACL_BF16, tB)
+    want, _ = cases.oracle_qmm_int8(m, inp, M, K, N, tB, m.ACL_BF16)
+    x1, b1 = _at_offset(m, (M, K), m.ACL_INT8, inp["x1"][0], o[0], 1)
+    x2, b2 = _at_offset(m, (N, K) if tB else (K, N), m.ACL_INT8, inp["x2"][0], o[1], 1, storage_cols=K if tB else N)
+    s1, b3 = _at_offset(m, (M,), m.ACL_FLOAT, inp["s1"], o[2], 4)
+    s2, b4 = _at_offset(m, (N,), m.ACL_FLOAT, inp["s2"], o[3], 4)
+    bias, b5 = _at_offset(m, (N,), m.ACL_BF16, inp["bias"], o[4], 2)
+    d_out = cases.guarded_out(m, (M * N + o[5]) * 2)
+    out = m.Tensor((M, N), m.ACL_BF16, d_out, offset=o[5], storage_shape=(M * N + o[5],))
+    ws = m.quant_matmul_v5(x1, x2, s1, s2, out, bias=bias, transpose_x2=tB)
+    m.check(m.lib().aclrtSynchronizeDevice(), "sync")
+    del ws
+    got = d_out.to_host(np.uint16, (M * N + o[5],))
+    assert (got[:o[5]] == 0xFFFF).all(), "wrote in front of the output view"
+    got = got[o[5]:].reshape(M, N)
+    assert np.array_equal(got, want[0]), f"{int((got != want[0]).sum())} of {got.size} outputs differ"
+
+
+@pytest.mark.parametrize("M,K,N", _shapes(121, 24, 300, 128, 4096, 32, 256, 1024))
+def test_weight_only_operands_at_odd_offsets(gpu, M, K, N):
+    m = gpu
+    o = [(1, 1, 1, 1), (8, 16, 0, 2), (3, 0, 1, 0), (0, 4, 2, 4), (2, 3, 1, 1)][(M + K // 128 + N // 32) % 5]
+    x_dt = m.ACL_FLOAT16 if (M + N) % 2 else m.ACL_BF16
+    group = 128 if (M + K // 128) % 2 and K > 128 else 0
+    G = K // group if group else 1
+    print(f"case sweep weight-only offsets M={M} K={K} N={N} g={group} offsets={o}", flush=True)
+    inp = cases.make_wq_inputs(m, M, K, N, M + K + N, x_dt, m.ACL_INT8, group, True, True, None)
+    want = cases.oracle_wq(m, inp, M, K, N)
+    x, b1 = _at_offset(m, (M, K), x_dt, inp["x"], o[0], 2)
+    w, b2 = _at_offset(m, (K, N), m.ACL_INT8, inp["w"], o[1], 1, strides=(1, K))
+    sshape, sst = ((G, N), (1, G)) if group else ((N,), None)
+    sc, b3 = _at_offset(m, sshape, x_dt, inp["scale"], o[2], 2, strides=sst)
+    off, b4 = _at_offset(m, sshape, x_dt, inp["offset"], o[2], 2, strides=sst)
+    d_y = cases.guarded_out(m, (M * N + o[3]) * 2)
+    y = m.Tensor((M, N), x_dt, d_y, offset=o[3], storage_shape=(M * N + o[3],))
+    plain(False)
+    ws = m.weight_quant_batch_matmul(x, w, sc, y, offset=off, group_size=group)
+    m.check(m.lib().aclrtSynchronizeDevice(), "sync")
+    del ws
+    got = d_y.to_host(np.uint16, (M * N + o[3],))
+    assert (got[:o[3]] == 0xFFFF).all(), "wrote in front of the output view"
+    check_close(got[o[3]:].reshape(M, N), want, x_dt, "weight-only at odd offsets")
