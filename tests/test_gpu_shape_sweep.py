@@ -632,3 +632,32 @@ def test_weight_only_operands_at_odd_offsets(gpu, M, K, N):
     got = d_y.to_host(np.uint16, (M * N + o[3],))
     assert (got[:o[3]] == 0xFFFF).all(), "wrote in front of the output view"
     check_close(got[o[3]:].reshape(M, N), want, x_dt, "weight-only at odd offsets")
+
+
+@pytest.mark.parametrize("M,K,N", _shapes(122, 20, 300, 128, 4096, 128, 128, 1024))
+@pytest.mark.parametrize("mode", ["block", "mxfp8"])
+def test_fp8_operands_at_odd_offsets(gpu, M, K, N, mode):
+    m = gpu
+    o = [(1, 3, 1, 1, 1), (4, 8, 2, 0, 2), (16, 1, 0, 1, 4), (0, 16, 1, 1, 0), (5, 0, 0, 0, 1)][(M + K // 128 + N // 128) % 5]
+    print(f"case sweep fp8 offsets {mode} M={M} K={K} N={N} offsets={o}", flush=True)
+    if mode == "block":
+        inp = cases.make_blockscale_inputs(m, M, K, N, M + N + K, True, 1)
+        want = cases.oracle_blockscale(m, inp, M, K, N, True, m.ACL_BF16)[0]
+        sdt, sb, gs = m.ACL_FLOAT, 4, (1 << 32) | (128 << 16) | 128
+    else:
+        inp = cases.make_mx_inputs(m, M, K, N, M + N + K, True, False)
+        want = cases.oracle_mx(m, inp, M, K, N, True, m.ACL_BF16)[0]
+        sdt, sb, gs = m.ACL_FLOAT8_E8M0, 1, (1 << 32) | (1 << 16) | 32
+    x1, b1 = _at_offset(m, (M, K), m.ACL_FLOAT8_E4M3FN, inp["x1"][0], o[0], 1)
+    x2, b2 = _at_offset(m, (N, K), m.ACL_FLOAT8_E4M3FN, inp["x2"][0], o[1], 1, storage_cols=K)
+    s1, b3 = _at_offset(m, inp["s1"].shape[1:], sdt, inp["s1"][0], o[2], sb, storage_cols=inp["s1"].shape[-1] * (inp["s1"].shape[-2] if mode != "block" else 1))
+    s2, b4 = _at_offset(m, inp["s2"].shape[1:], sdt, inp["s2"][0], o[3], sb, storage_cols=inp["s2"].shape[-1] * (inp["s2"].shape[-2] if mode != "block" else 1))
+    d_out = cases.guarded_out(m, (M * N + o[4]) * 2)
+    out = m.Tensor((M, N), m.ACL_BF16, d_out, offset=o[4], storage_shape=(M * N + o[4],))
+    plain(False)
+    ws = m.quant_matmul_v5(x1, x2, s1, s2, out, transpose_x2=True, group_size=gs)
+    m.check(m.lib().aclrtSynchronizeDevice(), "sync")
+    del ws
+    got = d_out.to_host(np.uint16, (M * N + o[4],))
+    assert (got[:o[4]] == 0xFFFF).all(), "wrote in front of the output view"
+    _b16_bar(got[o[4]:].reshape(M, N), want, orc.BF16, f"fp8 {mode} at odd offsets", K)
