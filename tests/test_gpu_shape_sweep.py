@@ -661,3 +661,82 @@ def test_fp8_operands_at_odd_offsets(gpu, M, K, N, mode):
     got = d_out.to_host(np.uint16, (M * N + o[4],))
     assert (got[:o[4]] == 0xFFFF).all(), "wrote in front of the output view"
     _b16_bar(got[o[4]:].reshape(M, N), want, orc.BF16, f"fp8 {mode} at odd offsets", K)
+
+
+# ---- a NaN row of x stays in its row: no kernel may multiply another row's x (a K tail read from the next row, a padded row
+# block) into a result, not even with a zero weight ----
+@pytest.mark.parametrize("M,K,N", _shapes(130, 28, 300, 8, 4096, 8, 64, 1024) + _shapes(131, 8, 300, 128, 8192, 32, 256, 1024))
+@pytest.mark.parametrize("w_dt", ["i4", "i8"])
+def test_weight_only_nan_row_stays_in_its_row(gpu, M, K, N, w_dt):
+    m = gpu
+    if M < 2:
+        M = 2
+    if w_dt == "i4":
+        K += K % 2
+    dt = {"i8": m.ACL_INT8, "i4": m.ACL_INT4}
+    x_dt = m.ACL_FLOAT16 if (M + N) % 2 else m.ACL_BF16
+    group = 128 if (M + K // 8) % 2 and K % 128 == 0 and K > 128 else 0
+    print(f"case sweep weight-only NaN row M={M} K={K} N={N} w={w_dt} g={group}", flush=True)
+    inp = cases.make_wq_inputs(m, M, K, N, M + K + N, x_dt, dt[w_dt], group, True, True, None)
+    bad = sorted({M // 2, M - 1})
+    clean = [r for r in range(M) if r not in bad]
+    inp["x"][bad] = 0x7E00 if x_dt == m.ACL_FLOAT16 else 0x7FC0
+    plain(False)
+    got = cases.run_wq_aclnn(m, inp, M, K, N)
+    g = orc.b16_to_f32(got, x_dt)
+    assert np.isnan(g[bad]).all(), "a NaN row of x gave finite results"
+    if clean:
+        want = cases.oracle_wq(m, inp, M, K, N, rows=clean)
+        check_close(got[clean], want, x_dt, "rows next to a NaN row")
+
+
+@pytest.mark.parametrize("M,K,N", _shapes(132, 24, 300, 32, 4096, 8, 64, 1024) + _shapes(133, 6, 64, 128, 16384, 8, 256, 520))
+@pytest.mark.parametrize("mode", ["block", "mxfp8", "mxfp4"])
+def test_quant_modes_nan_row_stays_in_its_row(gpu, M, K, N, mode):
+    m = gpu
+    M = max(M, 2)
+    bad = sorted({M // 2, M - 1})
+    clean = [r for r in range(M) if r not in bad]
+    print(f"case sweep {mode} NaN row M={M} K={K} N={N}", flush=True)
+    plain(False)
+    if mode == "block":
+        inp = cases.make_blockscale_inputs(m, M, K, N, M + N + K, True, 1)
+        inp["x1"][0, bad] = 0x7F   # e4m3 NaN
+        got = cases.run_blockscale_aclnn(m, inp, M, K, N, True, m.ACL_BF16)[0]
+        want = cases.oracle_blockscale(m, inp, M, K, N, True, m.ACL_BF16, rows=clean)[0] if clean else None
+    else:
+        inp = cases.make_mx_inputs(m, M, K, N, M + N + K, True, mode == "mxfp4")
+        # MXFP4: an e8m0 NaN scale makes the whole block NaN (e2m1 has no NaN code of its own).  MXFP8: NaN elements (a NaN
+        # scale would also send the whole call from the exact products to the scaled 8-bit instruction, whose bar is another)
+        if mode == "mxfp4":
+            inp["s1"][0, bad] = 0xFF
+        else:
+            inp["x1"][0, bad] = 0x7F
+        got = cases.run_mx_aclnn(m, inp, M, K, N, True, m.ACL_BF16)[0]
+        want = cases.oracle_mx(m, inp, M, K, N, True, m.ACL_BF16, rows=clean)[0] if clean else None
+    g = orc.b16_to_f32(got, orc.BF16)
+    assert np.isnan(g[bad]).all(), "a NaN row of x1 gave finite results"
+    if clean:
+        _b16_bar(got[clean], want, orc.BF16, f"{mode}: rows next to a NaN row", K)
+
+
+@pytest.mark.parametrize("M,K,N", _shapes(134, 24, 300, 8, 4096, 8, 64, 1024) + _shapes(135, 8, 300, 128, 8192, 32, 256, 1024))
+def test_weight_only_nan_scale_stays_in_its_column(gpu, M, K, N):
+    """A NaN scale of one output column (all its groups) makes that column NaN and no other."""
+    m = gpu
+    x_dt = m.ACL_FLOAT16 if (M + N) % 2 else m.ACL_BF16
+    w_dt = m.ACL_INT8 if (M + K // 8) % 2 else m.ACL_INT4
+    if w_dt == m.ACL_INT4:
+        K += K % 2
+    group = 128 if (M + N // 8) % 2 and K % 128 == 0 and K > 128 else 0
+    print(f"case sweep weight-only NaN scale column M={M} K={K} N={N} w={w_dt} g={group}", flush=True)
+    inp = cases.make_wq_inputs(m, M, K, N, M + K + N, x_dt, w_dt, group, True, True, None)
+    want = cases.oracle_wq(m, inp, M, K, N)
+    bad = sorted({0, N // 3, N - 1})
+    inp["scale"][bad] = 0x7E00 if x_dt == m.ACL_FLOAT16 else 0x7FC0
+    plain(False)
+    got = cases.run_wq_aclnn(m, inp, M, K, N)
+    g = orc.b16_to_f32(got, x_dt)
+    assert np.isnan(g[:, bad]).all(), "a NaN scale column gave finite results"
+    keep = np.ones(N, bool); keep[bad] = False
+    check_close(np.ascontiguousarray(got[:, keep]), np.ascontiguousarray(want[:, keep]), x_dt, "columns next to a NaN scale column")
