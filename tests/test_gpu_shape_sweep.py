@@ -740,3 +740,41 @@ def test_weight_only_nan_scale_stays_in_its_column(gpu, M, K, N):
     assert np.isnan(g[:, bad]).all(), "a NaN scale column gave finite results"
     keep = np.ones(N, bool); keep[bad] = False
     check_close(np.ascontiguousarray(got[:, keep]), np.ascontiguousarray(want[:, keep]), x_dt, "columns next to a NaN scale column")
+
+
+@pytest.mark.parametrize("M,K,N", _shapes(136, 20, 300, 128, 4096, 8, 64, 1024) + _shapes(137, 6, 64, 128, 16384, 8, 256, 520))
+@pytest.mark.parametrize("mode", ["int8", "fp8_kc", "pertile", "a8w4"])
+def test_scaled_modes_nan_row_scale_stays_in_its_row(gpu, M, K, N, mode):
+    """A NaN x1 scale of one row (a NaN x1 element for fp8 x fp4) makes that output row NaN and no other."""
+    m = gpu
+    M = max(M, 2)
+    bad = sorted({M // 2, M - 1})
+    clean = [r for r in range(M) if r not in bad]
+    print(f"case sweep {mode} NaN row scale M={M} K={K} N={N}", flush=True)
+    if mode == "int8":
+        inp = cases.make_qmm_int8_inputs(m, M, K, N, M * 31 + N, m.ACL_BF16, True)
+        inp["s1"][bad] = np.nan
+        got = cases.run_qmm_int8_aclnn(m, inp, M, K, N, True, m.ACL_BF16)[0]
+        want = cases.oracle_qmm_int8(m, inp, M, K, N, True, m.ACL_BF16)[0][0]
+    elif mode == "fp8_kc":
+        inp = cases.make_tc_inputs(m, M, K, N, M + N, m.ACL_FLOAT8_E4M3FN, m.ACL_FLOAT, N, m.ACL_FLOAT, True, pertoken="M")
+        inp["pt"][bad] = np.nan
+        got = cases.run_tc_aclnn(m, inp, M, K, N, m.ACL_BF16)
+        want = cases.oracle_tc(m, inp, M, K, N, m.ACL_BF16)
+    elif mode == "pertile":
+        inp = cases.make_pertile_i8_inputs(m, M, K, N, M + N, True)
+        inp["s1"][bad] = np.nan
+        got = cases.run_pertile_i8_aclnn(m, inp, M, K, N, True, m.ACL_BF16)
+        want = cases.oracle_pertile_i8(m, inp, M, K, N, True, m.ACL_BF16)
+    else:
+        inp = cases.make_a8w4_mx_inputs(m, M, K, N, M + N, True)
+        inp["x1"][bad] = 0x7F
+        got = cases.run_a8w4_mx_aclnn(m, inp, M, K, N, True, m.ACL_BF16, bias_dt=orc.BF16)
+        want = cases.oracle_a8w4_mx(m, inp, M, K, N, True, m.ACL_BF16, bias_dt=orc.BF16)
+    g = orc.b16_to_f32(got, orc.BF16)
+    assert np.isnan(g[bad]).all(), "a NaN row gave finite results"
+    assert np.isnan(orc.b16_to_f32(want, orc.BF16)[bad]).all()
+    if mode == "int8":
+        assert np.array_equal(got[clean], want[clean]), f"{int((got[clean] != want[clean]).sum())} outputs of the other rows differ"
+    else:
+        _b16_bar(np.ascontiguousarray(got[clean]), np.ascontiguousarray(want[clean]), orc.BF16, f"{mode}: rows next to a NaN row", K)
