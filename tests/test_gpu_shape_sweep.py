@@ -778,3 +778,43 @@ def test_scaled_modes_nan_row_scale_stays_in_its_row(gpu, M, K, N, mode):
         assert np.array_equal(got[clean], want[clean]), f"{int((got[clean] != want[clean]).sum())} outputs of the other rows differ"
     else:
         _b16_bar(np.ascontiguousarray(got[clean]), np.ascontiguousarray(want[clean]), orc.BF16, f"{mode}: rows next to a NaN row", K)
+
+
+# ---- the same call three times gives the same bits: partial sums are added in a fixed order, and a race (a missing barrier or
+# wait) would show as a result that changes between runs while staying inside the tolerance of the comparisons above ----
+@pytest.mark.parametrize("M,K,N", _shapes(140, 16, 300, 128, 4096, 32, 256, 1024) + _shapes(141, 8, 64, 128, 20480, 32, 256, 1024) +
+                         _shapes(142, 4, 300, 128, 1536, 128, 16512, 20480))
+@pytest.mark.parametrize("mode", ["wq_i4", "wq_i8", "wq_fp4", "block", "fp8_kc", "pertile", "a8w4", "mxfp8", "mxfp4", "tcg"])
+def test_repeated_calls_are_bit_identical(gpu, M, K, N, mode):
+    m = gpu
+    print(f"case sweep repeat {mode} M={M} K={K} N={N}", flush=True)
+    plain(False)
+    if mode.startswith("wq_"):
+        w_dt, group, off = {"wq_i4": (m.ACL_INT4, 128, True), "wq_i8": (m.ACL_INT8, 0, True), "wq_fp4": (m.ACL_FLOAT4_E2M1, 32, False)}[mode]
+        if mode == "wq_i4" and K % 256:
+            K += 128
+        inp = cases.make_wq_inputs(m, M, K, N, M + K + N, m.ACL_BF16 if (M + N) % 2 else m.ACL_FLOAT16, w_dt, group if K > group else 0, True, off, None)
+        run = lambda: cases.run_wq_aclnn(m, inp, M, K, N)
+    elif mode == "block":
+        inp = cases.make_blockscale_inputs(m, M, K, N, M + N + K, True, 1)
+        run = lambda: cases.run_blockscale_aclnn(m, inp, M, K, N, True, m.ACL_BF16)
+    elif mode == "fp8_kc":
+        inp = cases.make_tc_inputs(m, M, K, N, M + N, m.ACL_FLOAT8_E4M3FN, m.ACL_FLOAT, N, m.ACL_FLOAT, True, pertoken="M")
+        run = lambda: cases.run_tc_aclnn(m, inp, M, K, N, m.ACL_BF16)
+    elif mode == "pertile":
+        inp = cases.make_pertile_i8_inputs(m, M, K, N, M + N, True)
+        run = lambda: cases.run_pertile_i8_aclnn(m, inp, M, K, N, True, m.ACL_BF16)
+    elif mode == "a8w4":
+        inp = cases.make_a8w4_mx_inputs(m, M, K, N, M + N, True)
+        run = lambda: cases.run_a8w4_mx_aclnn(m, inp, M, K, N, True, m.ACL_FLOAT16)
+    elif mode == "tcg":
+        inp = cases.make_tcg_inputs(m, M, K, N, M + N, m.ACL_BF16)
+        run = lambda: cases.run_tcg_aclnn(m, inp, M, K, N, m.ACL_BF16)
+    else:
+        inp = cases.make_mx_inputs(m, M, K, N, K + N + M, True, mode == "mxfp4")
+        run = lambda: cases.run_mx_aclnn(m, inp, M, K, N, True, m.ACL_BF16)
+    first = run()
+    for rep in (1, 2):
+        m.check(m.lib().opsnnDebugFillLds(None), "opsnnDebugFillLds")
+        again = run()
+        assert np.array_equal(first.view(np.uint16), again.view(np.uint16)), f"run {rep + 1}: {int((first.view(np.uint16) != again.view(np.uint16)).sum())} of {first.size} outputs differ from the first run"
